@@ -1,0 +1,185 @@
+/*
+ * shv_hip.h — C ABI of the MI355X (gfx950) backend for strix-halo-vulkan's language-model
+ * token loop.  It takes the place of the reference's Vulkan shim (vk/shim.h) underneath the
+ * Go-side op surface (llm/gpu_*.go): a host binding (cgo, ctypes, C++) sees opaque handles,
+ * device addresses, plain sizes and POD argument blocks, and nothing else.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a negative SHV_E_* code otherwise;
+ *     shv_last_error() gives the message for the calling thread (vk.Error{Op,Result},
+ *     vk/engine.go:21-36, carries the same two facts).
+ *   - a context owns ONE in-order HIP stream: consecutive ops are ordered as the reference's
+ *     dispatches are by the barrier it records between them (vk/engine.go:853-859).
+ *   - the context is not internally synchronised: one host thread at a time, as
+ *     backend.Device.Do serialises every caller of the reference (backend/device.go:24-36).
+ *   - device memory is not host-mapped on a discrete GPU, so Buffer.Write* / Read*
+ *     (vk/engine.go:319-634) become shv_upload / shv_download on device addresses.
+ *   - an op is {kind, flags, 248-byte POD block}: the analogue of MultiDispatch{Pipeline,
+ *     GroupsX, GroupsY, PushConstants} with its 256-byte push block (vk/engine.go:848-860,
+ *     llm/gpu.go:60-109).  Grid shapes are chosen inside the library.
+ *   - values that change from token to token (sequence position, token id) are read by the
+ *     kernels from device memory, so a recorded sequence is byte-identical between tokens
+ *     and can be replayed (vk/engine.go:997-1081).
+ */
+#ifndef SHV_HIP_H
+#define SHV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SHV_OK 0
+#define SHV_E_INVALID (-1)   /* bad argument or shape the kernels do not cover */
+#define SHV_E_HIP (-2)       /* a HIP runtime call failed                     */
+#define SHV_E_NOMEM (-3)
+#define SHV_E_STATE (-4)     /* call not valid in the context's current state */
+
+#define SHV_Q4K_BLOCK 256    /* weights per GGUF Q4_K super-block */
+#define SHV_Q4K_BYTES 144    /* bytes per super-block: f16 d, f16 dmin, 12 B scales, 128 B nibbles */
+
+typedef struct shv_ctx shv_ctx;
+typedef struct shv_prerecorded shv_prerecorded;
+
+typedef struct {
+    char name[128];
+    char arch[32];
+    int32_t compute_units;
+    int32_t wave_size;
+    int32_t lds_bytes_per_cu;
+    int32_t clock_mhz;
+    uint64_t hbm_bytes;
+} shv_props;
+
+/* ---- device, replaces shim_create_instance .. shim_create_device (vk/shim.h:84-114) ---- */
+const char *shv_last_error(void);
+int shv_device_count(int *out);
+int shv_init(int device, shv_ctx **out);
+void shv_destroy(shv_ctx *ctx);
+int shv_device_props(shv_ctx *ctx, shv_props *out);   /* vk/engine.go:144-253 PhysicalDevice */
+int shv_sync(shv_ctx *ctx);                           /* shim_device_wait_idle, vk/shim.h:115 */
+int shv_submits(shv_ctx *ctx, uint64_t *out);         /* Device.Submits, vk/engine.go:303-308 */
+
+/* ---- buffers, replaces shim_create_storage_buffer / shim_destroy_buffer (vk/shim.h:120-131)
+ *      and the Buffer read/write family (vk/engine.go:319-634).  Upload/download block. ---- */
+int shv_alloc(shv_ctx *ctx, size_t bytes, void **dptr);
+int shv_free(shv_ctx *ctx, void *dptr);
+int shv_upload(shv_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int shv_download(shv_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+int shv_copy(shv_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);  /* async, in order */
+int shv_zero(shv_ctx *ctx, void *dst_dev, size_t bytes);                       /* Buffer.Zero*, async */
+int shv_host_alloc(shv_ctx *ctx, size_t bytes, void **hptr);  /* pinned staging */
+int shv_host_free(shv_ctx *ctx, void *hptr);
+
+/* ---- op argument blocks ---------------------------------------------------------------- */
+
+enum {
+    SHV_OP_GEMV_Q4K = 1,
+    SHV_OP_DEQUANT_Q4K = 2,
+    SHV_OP_QUANTIZE_Q4K = 3,
+    SHV_OP_FILL_NORMAL = 4,
+    SHV_OP_MOE_ROUTER = 5,
+    SHV_OP_MOE_UP = 6,
+    SHV_OP_MOE_DOWN = 7,
+    SHV_OP_DN_STEP = 8,
+    SHV_OP_ATTN_DECODE = 9,
+    SHV_OP_EMBED = 10,
+    SHV_OP_ARGMAX = 11,
+    SHV_OP_RMSNORM = 12,
+    SHV_OP_COPY_F32 = 13,
+    SHV_OP__COUNT
+};
+
+/* prologues a Q4_K GEMV can apply to its input vector while staging it */
+enum {
+    SHV_PRO_NONE = 0,
+    SHV_PRO_RMSNORM = 1,     /* x * rsqrt(mean(x^2)+eps) * gamma            (llm/hc.go:176-190)       */
+    SHV_PRO_GATED_NORM = 2,  /* per head of head_dim: rms * gamma[head_dim] * sigmoid(z)
+                                                                            (llm/deltanet.go:329-341) */
+    SHV_PRO_MUL_SIGMOID = 3  /* x * sigmoid(z)                              (llm/attn.go:198-205)     */
+};
+
+/* y[t][r] = sum_i W[r][i] * pro(x[t])[i] (+ residual[t][r]); W is GGUF Q4_K, row-major, k%256==0.
+ * The reference's CPU form is matvec over Tensor.DequantizeRow (llm/hc.go:255-264,
+ * gguf/dequant.go:119-124); its GPU forms are llm_gemv.comp and llm_moe_gemv.comp.
+ * ring_slots>0: row t is written at y + ((pos[0]+t) % ring_slots)*ring_stride instead of
+ * y + t*y_stride (the DeltaNet projection ring, shaders/llm_dn_conv.comp:36-49). */
+typedef struct {
+    const void *w;
+    const float *x;
+    float *y;
+    const float *residual;
+    const float *gamma;
+    const float *z;
+    const int32_t *pos;
+    int32_t n, k, n_tok;
+    int32_t prologue;
+    int32_t head_dim;
+    float eps;
+    int32_t x_stride, y_stride, z_stride;
+    int32_t ring_slots, ring_stride;
+} shv_gemv_q4k_args;
+
+/* dst[i] = d*sc*q - dmin*m for every weight of `rows` rows, the reference's dequantQ4_K
+ * expression term for term (gguf/dequant.go:252-276); bit-exact. */
+typedef struct {
+    const void *w;
+    float *dst;
+    int64_t rows;
+    int32_t k;
+} shv_dequant_q4k_args;
+
+/* src float32 [rows][k] -> GGUF Q4_K rows, the reference's round-to-nearest quantiser
+ * (llm/quantk.go:115-179, llm/sim.go:982-1060, llm/moebank.go:489-532); bit-exact. */
+typedef struct {
+    const float *src;
+    void *dst;
+    int64_t rows;
+    int32_t k;
+} shv_quantize_q4k_args;
+
+/* dst[i] = mean + std * N(0,1), counter-based (seed, i): synthetic weights made in HBM. */
+typedef struct {
+    float *dst;
+    int64_t n;
+    uint64_t seed;
+    float mean, std;
+} shv_fill_normal_args;
+
+typedef struct {
+    uint32_t kind;
+    uint32_t flags;          /* bit 0: may overlap the previous op (MultiDispatch.Overlap) */
+    uint8_t args[248];
+} shv_op;
+
+/* ---- running ops ------------------------------------------------------------------------- */
+
+/* Enqueue one op on the context's stream and return without waiting. */
+int shv_enqueue(shv_ctx *ctx, uint32_t kind, const void *args, size_t args_bytes);
+
+/* DispatchMultiTimed / DispatchMultiMarked (vk/engine.go:893-935): run the sequence `iters`
+ * times, block until done, return GPU time for the whole run in total_ns and, if per_op_ns is
+ * not NULL (one slot per op, iters must be 1), the GPU time of each op. */
+int shv_dispatch_multi(shv_ctx *ctx, const shv_op *ops, int n_ops, int iters,
+                       uint64_t *total_ns, uint64_t *per_op_ns);
+
+/* NewPrerecorded / Submit / Count / Destroy (vk/engine.go:997-1086): the sequence is recorded
+ * once (a HIP graph) and replayed.  submit blocks and returns GPU time; launch does not block. */
+int shv_prerecord(shv_ctx *ctx, const shv_op *ops, int n_ops, shv_prerecorded **out);
+int shv_prerecorded_submit(shv_ctx *ctx, shv_prerecorded *p, int iters, uint64_t *total_ns);
+int shv_prerecorded_launch(shv_ctx *ctx, shv_prerecorded *p);
+int shv_prerecorded_count(const shv_prerecorded *p);
+void shv_prerecorded_destroy(shv_ctx *ctx, shv_prerecorded *p);
+
+/* Convenience entry points: one op each, enqueued without waiting. */
+int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
+int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
+int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
+int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,245 @@
+// Q4_K dequant-fused GEMV for batch-1..4 decode: y[t] = W * pro(x[t]) (+ residual[t]).
+//
+// HBM-bound: every weight byte is read once with 128-bit loads and nothing else of size moves.
+// Work split (wave64): a lane owns one 64-weight group of a row — 32 contiguous payload bytes
+// (two 16-byte loads) plus the row's 16-byte super-block header — and keeps the 64 activations of
+// those columns in registers for every row it visits.  K/64 lanes cover a row, so a wave covers
+// 64/(K/64) rows per pass and reduces each row across its lanes with DPP.  Passes of a wave are
+// unrolled so all of its loads are in flight before the first is consumed.
+//
+// The input vector is staged once per 256-thread block through LDS, where the optional prologue
+// (RMSNorm, DeltaNet's gated per-head norm, or attention's sigmoid gate) is applied.
+#include "shv_device.hpp"
+#include "shv_internal.hpp"
+
+namespace {
+
+using namespace shv;
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kMaxTok = 4;
+
+// LDS layout of the staged vector: each 64-float slice is followed by 4 floats of padding so
+// that the lanes of a wave, which read slices 256 bytes apart, fall on different banks.
+__device__ __forceinline__ int lds_slot(int i) { return i + (i >> 6) * 4; }
+
+// U consecutive passes of one wave: issue every load, then consume.
+template <int K, int NT, int U>
+__device__ __forceinline__ void gemv_passes(const shv_gemv_q4k_args &a, const char *wbase, int g, int lane, int rsub,
+                                            long long pass, int n, const float (*xr)[64], const float *xs_lo,
+                                            const float *xs_hi, const size_t *y_off) {
+    constexpr int LPR = K / 64;
+    constexpr int RPP = 64 / LPR;
+    constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+    uint4 hdr[U], q0[U], q1[U];
+    int row[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const long long r = (pass + u) * RPP + rsub;
+        row[u] = r < n ? static_cast<int>(r) : -1;
+        const char *rp = wbase + static_cast<size_t>(row[u] < 0 ? 0 : row[u]) * ROWB;
+        hdr[u] = load_stream16(rp);
+        q0[u] = load_stream16(rp + 16 + g * 32);
+        q1[u] = load_stream16(rp + 32 + g * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float acc = q4k_group_dot(hdr[u], q0[u], q1[u], g, xr[t], xs_lo[t], xs_hi[t]);
+            acc = group_sum<LPR>(acc);
+            if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
+                float r = acc;
+                if (a.residual) r += a.residual[static_cast<size_t>(t) * a.y_stride + row[u]];
+                a.y[y_off[t] + row[u]] = r;
+            }
+        }
+    }
+}
+
+template <int K, int NT>
+__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int passes_per_wave) {
+    constexpr int LPR = K / 64;   // lanes per row
+    constexpr int XPAD = K + K / 64 * 4;
+    extern __shared__ float smem[];
+    float(*xs)[XPAD] = reinterpret_cast<float(*)[XPAD]>(smem);
+    __shared__ float red[4];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // ---- stage pro(x) in LDS ----
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const float *x = a.x + static_cast<size_t>(t) * a.x_stride;
+        if (a.prologue == SHV_PRO_RMSNORM) {
+            float v[K / kBlock];
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < K / kBlock; i++) {
+                v[i] = x[tid + i * kBlock];
+                ss = fmaf(v[i], v[i], ss);
+            }
+            ss = block_sum_256(ss, red);
+            const float scale = 1.f / sqrtf(ss / static_cast<float>(K) + a.eps);
+#pragma unroll
+            for (int i = 0; i < K / kBlock; i++) {
+                const int c = tid + i * kBlock;
+                xs[t][lds_slot(c)] = v[i] * scale * a.gamma[c];
+            }
+        } else if (a.prologue == SHV_PRO_GATED_NORM) {
+            // thread owns K/256 consecutive columns; a head of head_dim columns spans
+            // head_dim/(K/256) consecutive threads (a power of two <= 64).
+            constexpr int PER = K / kBlock;
+            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+            float v[PER];
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < PER; i++) {
+                v[i] = x[tid * PER + i];
+                ss = fmaf(v[i], v[i], ss);
+            }
+            const int span = a.head_dim / PER;
+            for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
+            const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
+#pragma unroll
+            for (int i = 0; i < PER; i++) {
+                const int c = tid * PER + i;
+                const float g = 1.f / (1.f + expf(-z[c]));
+                xs[t][lds_slot(c)] = v[i] * scale * a.gamma[c % a.head_dim] * g;
+            }
+        } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
+            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+#pragma unroll
+            for (int i = 0; i < K / kBlock; i++) {
+                const int c = tid + i * kBlock;
+                xs[t][lds_slot(c)] = x[c] * (1.f / (1.f + expf(-z[c])));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < K / kBlock; i++) {
+                const int c = tid + i * kBlock;
+                xs[t][lds_slot(c)] = x[c];
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- this lane's 64 activations per token ----
+    const int gi = lane % LPR;   // 64-weight group of the row
+    const int rsub = lane / LPR; // which of the pass's rows
+    float xr[NT][64];
+    float xs_lo[NT], xs_hi[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const float4 *src = reinterpret_cast<const float4 *>(&xs[t][gi * 68]);
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float4 f = src[i];
+            xr[t][4 * i + 0] = f.x;
+            xr[t][4 * i + 1] = f.y;
+            xr[t][4 * i + 2] = f.z;
+            xr[t][4 * i + 3] = f.w;
+            const float s = (f.x + f.y) + (f.z + f.w);
+            if (i < 8) lo += s; else hi += s;
+        }
+        xs_lo[t] = lo;
+        xs_hi[t] = hi;
+    }
+
+    const int sb = gi >> 2, g = gi & 3;
+    const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
+    const int n = a.n;
+    const long long first_pass = (static_cast<long long>(blockIdx.x) * kWavesPerBlock + wave) * passes_per_wave;
+
+    size_t y_off[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        if (a.ring_slots > 0) {
+            const int p = a.pos ? a.pos[0] : 0;
+            y_off[t] = static_cast<size_t>((p + t) % a.ring_slots) * a.ring_stride;
+        } else {
+            y_off[t] = static_cast<size_t>(t) * a.y_stride;
+        }
+    }
+
+    int p0 = 0;
+    for (; p0 + 4 <= passes_per_wave; p0 += 4)
+        gemv_passes<K, NT, 4>(a, wbase, g, lane, rsub, first_pass + p0, n, xr, xs_lo, xs_hi, y_off);
+    if (p0 + 2 <= passes_per_wave) {
+        gemv_passes<K, NT, 2>(a, wbase, g, lane, rsub, first_pass + p0, n, xr, xs_lo, xs_hi, y_off);
+        p0 += 2;
+    }
+    if (p0 < passes_per_wave)
+        gemv_passes<K, NT, 1>(a, wbase, g, lane, rsub, first_pass + p0, n, xr, xs_lo, xs_hi, y_off);
+}
+
+template <int K, int NT>
+int launch_nt(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw) {
+    if (lds > 48 * 1024) {
+        // above the default dynamic-LDS allowance the limit has to be raised once per kernel
+        static bool raised = false;
+        if (!raised) {
+            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_kernel<K, NT>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((gemv_q4k_kernel<K, NT>), grid, block, lds, ctx->stream, a, ppw);
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}
+
+template <int K>
+int launch_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    constexpr int RPP = 64 / (K / 64);
+    const long long passes = (static_cast<long long>(a.n) + RPP - 1) / RPP;
+    // Enough waves to have every load of a small matrix in flight at once; large matrices get
+    // several passes per wave so the staging of x is amortised.
+    const long long target_waves = static_cast<long long>(ctx->prop.multiProcessorCount) * 4 * 4;
+    long long ppw = (passes + target_waves - 1) / target_waves;
+    if (ppw < 1) ppw = 1;
+    const long long waves = (passes + ppw - 1) / ppw;
+    const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+    SHV_REQUIRE(blocks > 0 && blocks < (1ll << 31), "gemv_q4k: grid of %lld blocks", blocks);
+    dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
+    const size_t lds = static_cast<size_t>(a.n_tok) * (K + K / 64 * 4) * sizeof(float);
+    switch (a.n_tok) {
+        case 1: return launch_nt<K, 1>(ctx, a, grid, block, lds, static_cast<int>(ppw));
+        case 2: return launch_nt<K, 2>(ctx, a, grid, block, lds, static_cast<int>(ppw));
+        case 3: return launch_nt<K, 3>(ctx, a, grid, block, lds, static_cast<int>(ppw));
+        case 4: return launch_nt<K, 4>(ctx, a, grid, block, lds, static_cast<int>(ppw));
+        default: return shv_set_error(SHV_E_INVALID, "gemv_q4k: n_tok %d, the GEMV covers 1..%d rows", a.n_tok, kMaxTok);
+    }
+}
+
+}  // namespace
+
+int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
+    const shv_gemv_q4k_args &a = *pa;
+    SHV_REQUIRE(a.w && a.x && a.y, "gemv_q4k: NULL w, x or y");
+    SHV_REQUIRE(a.n > 0, "gemv_q4k: n = %d", a.n);
+    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= kMaxTok, "gemv_q4k: n_tok %d, the GEMV covers 1..%d rows", a.n_tok, kMaxTok);
+    SHV_REQUIRE(shv_aligned16(a.w), "gemv_q4k: w must be 16-byte aligned");
+    SHV_REQUIRE(a.x_stride >= a.k || a.n_tok == 1, "gemv_q4k: x_stride %d < k %d", a.x_stride, a.k);
+    SHV_REQUIRE(a.y_stride >= a.n || a.n_tok == 1 || a.ring_slots > 0, "gemv_q4k: y_stride %d < n %d", a.y_stride, a.n);
+    SHV_REQUIRE(a.prologue >= SHV_PRO_NONE && a.prologue <= SHV_PRO_MUL_SIGMOID, "gemv_q4k: prologue %d", a.prologue);
+    if (a.prologue == SHV_PRO_RMSNORM) SHV_REQUIRE(a.gamma, "gemv_q4k: RMSNorm prologue without gamma");
+    if (a.prologue == SHV_PRO_GATED_NORM) {
+        SHV_REQUIRE(a.gamma && a.z, "gemv_q4k: gated-norm prologue without gamma or z");
+        const int per = a.k / kBlock;
+        SHV_REQUIRE(a.head_dim > 0 && a.k % a.head_dim == 0 && per > 0 && a.head_dim % per == 0 &&
+                        a.head_dim / per <= 64 && ((a.head_dim / per) & (a.head_dim / per - 1)) == 0,
+                    "gemv_q4k: gated-norm head_dim %d does not tile k %d", a.head_dim, a.k);
+    }
+    if (a.prologue == SHV_PRO_MUL_SIGMOID) SHV_REQUIRE(a.z, "gemv_q4k: sigmoid-gate prologue without z");
+    if (a.ring_slots > 0) SHV_REQUIRE(a.ring_stride >= a.n && a.n_tok <= a.ring_slots, "gemv_q4k: ring of %d slots, stride %d", a.ring_slots, a.ring_stride);
+    switch (a.k) {
+        case 512: return launch_k<512>(ctx, a);
+        case 1024: return launch_k<1024>(ctx, a);
+        case 2048: return launch_k<2048>(ctx, a);
+        case 4096: return launch_k<4096>(ctx, a);
+        default: return shv_set_error(SHV_E_INVALID, "gemv_q4k: k = %d; built for 512, 1024, 2048 and 4096", a.k);
+    }
+}

@@ -1,0 +1,304 @@
+// C-ABI layer: context, buffers, op dispatch, timed sequences and prerecorded (HIP graph) replay.
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "shv_internal.hpp"
+
+static thread_local char g_err[512] = "";
+
+int shv_set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+extern "C" {
+
+const char *shv_last_error(void) { return g_err; }
+
+int shv_device_count(int *out) {
+    SHV_REQUIRE(out != nullptr, "shv_device_count: out is NULL");
+    int n = 0;
+    SHV_HIP_CHECK(hipGetDeviceCount(&n));
+    *out = n;
+    return SHV_OK;
+}
+
+int shv_init(int device, shv_ctx **out) {
+    SHV_REQUIRE(out != nullptr, "shv_init: out is NULL");
+    *out = nullptr;
+    int n = 0;
+    SHV_HIP_CHECK(hipGetDeviceCount(&n));
+    SHV_REQUIRE(device >= 0 && device < n, "shv_init: device %d of %d", device, n);
+    SHV_HIP_CHECK(hipSetDevice(device));
+    shv_ctx *ctx = new (std::nothrow) shv_ctx();
+    if (!ctx) return shv_set_error(SHV_E_NOMEM, "shv_init: out of host memory");
+    ctx->device = device;
+    hipError_t e = hipGetDeviceProperties(&ctx->prop, device);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev_begin);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev_end);
+    ctx->n_counters = 4096;
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->counters), ctx->n_counters * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int32_t));
+    if (e != hipSuccess) {
+        shv_destroy(ctx);
+        return shv_set_error(SHV_E_HIP, "shv_init: %s", hipGetErrorString(e));
+    }
+    if (std::strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0) {
+        char arch[64];
+        std::snprintf(arch, sizeof(arch), "%s", ctx->prop.gcnArchName);
+        shv_destroy(ctx);
+        return shv_set_error(SHV_E_INVALID, "shv_init: device %d is %s; this library holds gfx950 code only", device, arch);
+    }
+    *out = ctx;
+    return SHV_OK;
+}
+
+void shv_destroy(shv_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
+    if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+int shv_device_props(shv_ctx *ctx, shv_props *out) {
+    SHV_REQUIRE(ctx && out, "shv_device_props: NULL argument");
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "%s", ctx->prop.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", ctx->prop.gcnArchName);
+    out->compute_units = ctx->prop.multiProcessorCount;
+    out->wave_size = ctx->prop.warpSize;
+    out->lds_bytes_per_cu = static_cast<int32_t>(ctx->prop.maxSharedMemoryPerMultiProcessor);
+    out->clock_mhz = ctx->prop.clockRate / 1000;
+    out->hbm_bytes = ctx->prop.totalGlobalMem;
+    return SHV_OK;
+}
+
+int shv_sync(shv_ctx *ctx) {
+    SHV_REQUIRE(ctx, "shv_sync: NULL context");
+    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    return SHV_OK;
+}
+
+int shv_submits(shv_ctx *ctx, uint64_t *out) {
+    SHV_REQUIRE(ctx && out, "shv_submits: NULL argument");
+    *out = ctx->submits;
+    return SHV_OK;
+}
+
+int shv_alloc(shv_ctx *ctx, size_t bytes, void **dptr) {
+    SHV_REQUIRE(ctx && dptr, "shv_alloc: NULL argument");
+    SHV_REQUIRE(bytes > 0, "shv_alloc: zero bytes");
+    *dptr = nullptr;
+    hipError_t e = hipMalloc(dptr, bytes);
+    if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError();
+        return shv_set_error(SHV_E_NOMEM, "shv_alloc: %zu bytes do not fit in device memory", bytes);
+    }
+    SHV_HIP_CHECK(e);
+    return SHV_OK;
+}
+
+int shv_free(shv_ctx *ctx, void *dptr) {
+    SHV_REQUIRE(ctx, "shv_free: NULL context");
+    if (!dptr) return SHV_OK;
+    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(hipFree(dptr));
+    return SHV_OK;
+}
+
+int shv_upload(shv_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    SHV_REQUIRE(ctx && dst && src, "shv_upload: NULL argument");
+    SHV_REQUIRE(!ctx->capturing, "shv_upload: not valid while recording");
+    if (bytes == 0) return SHV_OK;
+    SHV_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    return SHV_OK;
+}
+
+int shv_download(shv_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    SHV_REQUIRE(ctx && dst && src, "shv_download: NULL argument");
+    SHV_REQUIRE(!ctx->capturing, "shv_download: not valid while recording");
+    if (bytes == 0) return SHV_OK;
+    SHV_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    return SHV_OK;
+}
+
+int shv_copy(shv_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    SHV_REQUIRE(ctx && dst && src, "shv_copy: NULL argument");
+    if (bytes == 0) return SHV_OK;
+    SHV_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return SHV_OK;
+}
+
+int shv_host_alloc(shv_ctx *ctx, size_t bytes, void **hptr) {
+    SHV_REQUIRE(ctx && hptr && bytes > 0, "shv_host_alloc: bad argument");
+    SHV_HIP_CHECK(hipHostMalloc(hptr, bytes, hipHostMallocDefault));
+    return SHV_OK;
+}
+
+int shv_host_free(shv_ctx *ctx, void *hptr) {
+    SHV_REQUIRE(ctx, "shv_host_free: NULL context");
+    if (hptr) SHV_HIP_CHECK(hipHostFree(hptr));
+    return SHV_OK;
+}
+
+}  // extern "C"
+
+// ---- op dispatch ----------------------------------------------------------------------------
+
+template <typename T>
+static int run_as(shv_ctx *ctx, const void *args, size_t bytes, int (*fn)(shv_ctx *, const T *), const char *name) {
+    static_assert(sizeof(T) <= sizeof(shv_op::args), "argument block exceeds the op record");
+    SHV_REQUIRE(bytes >= sizeof(T), "%s: argument block is %zu bytes, need %zu", name, bytes, sizeof(T));
+    T a;
+    std::memcpy(&a, args, sizeof(T));
+    return fn(ctx, &a);
+}
+
+static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t bytes) {
+    SHV_REQUIRE(ctx && args, "shv_enqueue: NULL argument");
+    switch (kind) {
+        case SHV_OP_GEMV_Q4K: return run_as<shv_gemv_q4k_args>(ctx, args, bytes, shv_launch_gemv_q4k, "gemv_q4k");
+        case SHV_OP_DEQUANT_Q4K: return run_as<shv_dequant_q4k_args>(ctx, args, bytes, shv_launch_dequant_q4k, "dequant_q4k");
+        case SHV_OP_QUANTIZE_Q4K: return run_as<shv_quantize_q4k_args>(ctx, args, bytes, shv_launch_quantize_q4k, "quantize_q4k");
+        case SHV_OP_FILL_NORMAL: return run_as<shv_fill_normal_args>(ctx, args, bytes, shv_launch_fill_normal, "fill_normal");
+        default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
+    }
+}
+
+extern "C" {
+
+int shv_enqueue(shv_ctx *ctx, uint32_t kind, const void *args, size_t args_bytes) {
+    return dispatch_one(ctx, kind, args, args_bytes);
+}
+
+int shv_zero(shv_ctx *ctx, void *dst, size_t bytes) {
+    SHV_REQUIRE(ctx && dst, "shv_zero: NULL argument");
+    SHV_REQUIRE(!ctx->capturing, "shv_zero: not valid while recording");
+    if (bytes == 0) return SHV_OK;
+    SHV_HIP_CHECK(hipMemsetAsync(dst, 0, bytes, ctx->stream));
+    return SHV_OK;
+}
+
+int shv_dispatch_multi(shv_ctx *ctx, const shv_op *ops, int n_ops, int iters, uint64_t *total_ns,
+                       uint64_t *per_op_ns) {
+    SHV_REQUIRE(ctx && ops, "shv_dispatch_multi: NULL argument");
+    SHV_REQUIRE(n_ops > 0, "shv_dispatch_multi: empty op sequence");
+    SHV_REQUIRE(iters >= 1, "shv_dispatch_multi: iters %d", iters);
+    SHV_REQUIRE(!ctx->capturing, "shv_dispatch_multi: not valid while recording");
+    SHV_REQUIRE(per_op_ns == nullptr || iters == 1, "shv_dispatch_multi: per-op times need iters == 1");
+    std::vector<hipEvent_t> marks;
+    if (per_op_ns) {
+        marks.resize(n_ops + 1);
+        for (auto &m : marks) SHV_HIP_CHECK(hipEventCreate(&m));
+    }
+    int rc = SHV_OK;
+    hipError_t e = hipEventRecord(ctx->ev_begin, ctx->stream);
+    if (per_op_ns && e == hipSuccess) e = hipEventRecord(marks[0], ctx->stream);
+    for (int it = 0; it < iters && rc == SHV_OK && e == hipSuccess; it++)
+        for (int i = 0; i < n_ops && rc == SHV_OK && e == hipSuccess; i++) {
+            rc = dispatch_one(ctx, ops[i].kind, ops[i].args, sizeof(ops[i].args));
+            if (per_op_ns && rc == SHV_OK) e = hipEventRecord(marks[i + 1], ctx->stream);
+        }
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev_end, ctx->stream);
+    hipError_t es = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) e = es;
+    ctx->submits++;
+    if (rc == SHV_OK && e == hipSuccess) {
+        float ms = 0;
+        e = hipEventElapsedTime(&ms, ctx->ev_begin, ctx->ev_end);
+        if (total_ns) *total_ns = static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+        for (int i = 0; per_op_ns && i < n_ops && e == hipSuccess; i++) {
+            e = hipEventElapsedTime(&ms, marks[i], marks[i + 1]);
+            per_op_ns[i] = static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+        }
+    }
+    for (auto &m : marks) (void)hipEventDestroy(m);
+    if (rc != SHV_OK) return rc;
+    if (e != hipSuccess) return shv_set_error(SHV_E_HIP, "shv_dispatch_multi: %s", hipGetErrorString(e));
+    return SHV_OK;
+}
+
+int shv_prerecord(shv_ctx *ctx, const shv_op *ops, int n_ops, shv_prerecorded **out) {
+    SHV_REQUIRE(ctx && ops && out, "shv_prerecord: NULL argument");
+    SHV_REQUIRE(n_ops > 0, "shv_prerecord: empty op sequence");
+    SHV_REQUIRE(!ctx->capturing, "shv_prerecord: already recording");
+    *out = nullptr;
+    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    int rc = SHV_OK;
+    for (int i = 0; i < n_ops && rc == SHV_OK; i++)
+        rc = dispatch_one(ctx, ops[i].kind, ops[i].args, sizeof(ops[i].args));
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    ctx->capturing = false;
+    if (rc != SHV_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (e != hipSuccess) return shv_set_error(SHV_E_HIP, "shv_prerecord: end capture: %s", hipGetErrorString(e));
+    shv_prerecorded *p = new (std::nothrow) shv_prerecorded();
+    if (!p) {
+        (void)hipGraphDestroy(graph);
+        return shv_set_error(SHV_E_NOMEM, "shv_prerecord: out of host memory");
+    }
+    p->graph = graph;
+    p->count = n_ops;
+    e = hipGraphInstantiate(&p->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        delete p;
+        return shv_set_error(SHV_E_HIP, "shv_prerecord: instantiate: %s", hipGetErrorString(e));
+    }
+    *out = p;
+    return SHV_OK;
+}
+
+int shv_prerecorded_launch(shv_ctx *ctx, shv_prerecorded *p) {
+    SHV_REQUIRE(ctx && p && p->exec, "shv_prerecorded_launch: NULL argument");
+    SHV_HIP_CHECK(hipGraphLaunch(p->exec, ctx->stream));
+    ctx->submits++;
+    return SHV_OK;
+}
+
+int shv_prerecorded_submit(shv_ctx *ctx, shv_prerecorded *p, int iters, uint64_t *total_ns) {
+    SHV_REQUIRE(ctx && p && p->exec, "shv_prerecorded_submit: NULL argument");
+    SHV_REQUIRE(iters >= 1, "shv_prerecorded_submit: iters %d", iters);
+    SHV_HIP_CHECK(hipEventRecord(ctx->ev_begin, ctx->stream));
+    for (int i = 0; i < iters; i++) SHV_HIP_CHECK(hipGraphLaunch(p->exec, ctx->stream));
+    SHV_HIP_CHECK(hipEventRecord(ctx->ev_end, ctx->stream));
+    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    ctx->submits += static_cast<uint64_t>(iters);
+    float ms = 0;
+    SHV_HIP_CHECK(hipEventElapsedTime(&ms, ctx->ev_begin, ctx->ev_end));
+    if (total_ns) *total_ns = static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+    return SHV_OK;
+}
+
+int shv_prerecorded_count(const shv_prerecorded *p) { return p ? p->count : 0; }
+
+void shv_prerecorded_destroy(shv_ctx *ctx, shv_prerecorded *p) {
+    if (!p) return;
+    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (p->exec) (void)hipGraphExecDestroy(p->exec);
+    if (p->graph) (void)hipGraphDestroy(p->graph);
+    delete p;
+}
+
+int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a) { return dispatch_one(ctx, SHV_OP_GEMV_Q4K, a, sizeof(*a)); }
+int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a) { return dispatch_one(ctx, SHV_OP_DEQUANT_Q4K, a, sizeof(*a)); }
+int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a) { return dispatch_one(ctx, SHV_OP_QUANTIZE_Q4K, a, sizeof(*a)); }
+int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a) { return dispatch_one(ctx, SHV_OP_FILL_NORMAL, a, sizeof(*a)); }
+
+}  // extern "C"

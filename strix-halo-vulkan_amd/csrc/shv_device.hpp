@@ -1,0 +1,140 @@
+// Device-side helpers shared by the kernels: wave64 reductions over DPP, Q4_K header decode,
+// nibble unpacking.  Written for gfx950 (CDNA4, 64-wide wavefronts) only.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace shv {
+
+constexpr int kWave = 64;
+
+// ---- DPP lane exchange ----------------------------------------------------------------------
+// update_dpp(old, src, ctrl, row_mask, bank_mask, bound_ctrl): lanes of disabled rows keep `old`.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_f32(float v) {
+    int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
+    return __int_as_float(r);
+}
+
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i within 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15-i within 16
+constexpr int kDppBcast15 = 0x142;    // lane 15 of each row of 16 -> the next row
+constexpr int kDppBcast31 = 0x143;    // lane 31 -> lanes 32..63
+
+// Sum over aligned groups of W consecutive lanes.  For W <= 16 every lane of the group ends up
+// with the group's sum; for W = 32 and 64 only the LAST 16 lanes of the group hold it.
+template <int W>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(W == 1 || W == 2 || W == 4 || W == 8 || W == 16 || W == 32 || W == 64, "group width");
+    if (W >= 2) v += dpp_f32<kDppXor1>(v);
+    if (W >= 4) v += dpp_f32<kDppXor2>(v);
+    if (W >= 8) v += dpp_f32<kDppHalfMirror>(v);
+    if (W >= 16) v += dpp_f32<kDppMirror>(v);
+    if (W >= 32) v += dpp_f32<kDppBcast15, 0xA>(v);
+    if (W >= 64) v += dpp_f32<kDppBcast31, 0xC>(v);
+    return v;
+}
+
+// The lane of a W-group that is guaranteed to hold group_sum's result.
+template <int W>
+__device__ __forceinline__ bool group_sum_owner(int lane) {
+    return (lane & (W - 1)) == (W - 1);
+}
+
+// Sum over the whole wave, delivered to every lane.
+__device__ __forceinline__ float wave_sum_all(float v) {
+    v = group_sum<64>(v);
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+__device__ __forceinline__ float wave_max_all(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Sum over a 256-thread block; `red` is 4 floats of LDS.  Every thread gets the result.
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+    v = wave_sum_all(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = red[0] + red[1] + red[2] + red[3];
+    __syncthreads();
+    return r;
+}
+
+// ---- Q4_K -----------------------------------------------------------------------------------
+// Super-block: f16 d @0, f16 dmin @2, 12 bytes of packed 6-bit (scale, min) pairs @4, 128 bytes of
+// nibbles @16.  Within each group of 64 weights the low nibbles of 32 bytes come first, then the
+// high nibbles.  The header is read as one 16-byte word: x = d | dmin<<16, y,z,w = scale bytes.
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(h & 0xffffu)));
+}
+
+// Scales and mins of sub-blocks 2g and 2g+1 (the two halves of 64-weight group g), as packed
+// bytes sc = sc0 | sc1<<8, mn = m0 | m1<<8.  Integer-exact get_scale_min_k4.
+__device__ __forceinline__ void q4k_group_scale_min(const uint4 &hdr, int g, uint32_t &sc, uint32_t &mn) {
+    const uint32_t sh = (g & 1) * 16;
+    const uint32_t a = hdr.y >> sh, b = hdr.z >> sh, c = hdr.w >> sh;
+    const uint32_t sc_lo = a & 0x3F3Fu, mn_lo = b & 0x3F3Fu;
+    const uint32_t sc_hi = (c & 0x0F0Fu) | ((a >> 2) & 0x3030u);
+    const uint32_t mn_hi = ((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);
+    sc = g >= 2 ? sc_hi : sc_lo;
+    mn = g >= 2 ? mn_hi : mn_lo;
+}
+
+// Dot product of the 8 weights in one payload dword with x: low nibbles of the four bytes meet
+// xlo[0..3], high nibbles meet xhi[0..3].
+__device__ __forceinline__ void q4k_dot8(uint32_t q, const float *xlo, const float *xhi, float &acc_lo, float &acc_hi) {
+    const uint32_t lo = q & 0x0F0F0F0Fu;
+    const uint32_t hi = (q >> 4) & 0x0F0F0F0Fu;
+    acc_lo = fmaf(static_cast<float>(lo & 0xFFu), xlo[0], acc_lo);
+    acc_lo = fmaf(static_cast<float>((lo >> 8) & 0xFFu), xlo[1], acc_lo);
+    acc_lo = fmaf(static_cast<float>((lo >> 16) & 0xFFu), xlo[2], acc_lo);
+    acc_lo = fmaf(static_cast<float>(lo >> 24), xlo[3], acc_lo);
+    acc_hi = fmaf(static_cast<float>(hi & 0xFFu), xhi[0], acc_hi);
+    acc_hi = fmaf(static_cast<float>((hi >> 8) & 0xFFu), xhi[1], acc_hi);
+    acc_hi = fmaf(static_cast<float>((hi >> 16) & 0xFFu), xhi[2], acc_hi);
+    acc_hi = fmaf(static_cast<float>(hi >> 24), xhi[3], acc_hi);
+}
+
+// One lane's share of one row: a 64-weight group (32 payload bytes in p0,p1) against the 64
+// activations xr[0..63] of the same columns.  xs_lo / xs_hi are the sums of xr[0..31] / xr[32..63].
+__device__ __forceinline__ float q4k_group_dot(const uint4 &hdr, const uint4 &p0, const uint4 &p1, int g,
+                                               const float *xr, float xs_lo, float xs_hi) {
+    uint32_t sc, mn;
+    q4k_group_scale_min(hdr, g, sc, mn);
+    const float d = f16_bits_to_f32(hdr.x), dmin = f16_bits_to_f32(hdr.x >> 16);
+    float lo = 0.f, hi = 0.f;
+    q4k_dot8(p0.x, xr + 0, xr + 32, lo, hi);
+    q4k_dot8(p0.y, xr + 4, xr + 36, lo, hi);
+    q4k_dot8(p0.z, xr + 8, xr + 40, lo, hi);
+    q4k_dot8(p0.w, xr + 12, xr + 44, lo, hi);
+    q4k_dot8(p1.x, xr + 16, xr + 48, lo, hi);
+    q4k_dot8(p1.y, xr + 20, xr + 52, lo, hi);
+    q4k_dot8(p1.z, xr + 24, xr + 56, lo, hi);
+    q4k_dot8(p1.w, xr + 28, xr + 60, lo, hi);
+    const float ds0 = d * static_cast<float>(sc & 0xFFu), ds1 = d * static_cast<float>(sc >> 8);
+    const float dm0 = dmin * static_cast<float>(mn & 0xFFu), dm1 = dmin * static_cast<float>(mn >> 8);
+    return ds0 * lo - dm0 * xs_lo + ds1 * hi - dm1 * xs_hi;
+}
+
+typedef uint32_t u32x4_native __attribute__((ext_vector_type(4)));
+
+// 128-bit streaming load: weights are read once per token and should not displace the
+// activations and partial results that later kernels find in L2.
+__device__ __forceinline__ uint4 load_stream16(const void *p) {
+    const u32x4_native v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_native *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+__device__ __forceinline__ float sigmoidf_dev(float x) { return 1.f / (1.f + __expf(-x)); }
+__device__ __forceinline__ float siluf_dev(float x) { return x * sigmoidf_dev(x); }
+
+}  // namespace shv

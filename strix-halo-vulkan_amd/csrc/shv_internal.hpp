@@ -1,0 +1,51 @@
+// Internal declarations shared by the C-ABI layer and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "shv_hip.h"
+
+struct shv_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t prop{};
+    uint64_t submits = 0;
+    bool capturing = false;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    // scratch the library's own kernels need (arrival counters for last-block epilogues)
+    int32_t *counters = nullptr;
+    int n_counters = 0;
+};
+
+struct shv_prerecorded {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int count = 0;
+};
+
+int shv_set_error(int code, const char *fmt, ...);
+
+#define SHV_HIP_CHECK(expr)                                                                    \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess)                                                                  \
+            return shv_set_error(SHV_E_HIP, "%s: %s (%s:%d)", #expr, hipGetErrorString(e_),    \
+                                 __FILE__, __LINE__);                                          \
+    } while (0)
+
+#define SHV_REQUIRE(cond, ...)                                                                 \
+    do {                                                                                       \
+        if (!(cond)) return shv_set_error(SHV_E_INVALID, __VA_ARGS__);                         \
+    } while (0)
+
+static inline bool shv_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// one launcher per op kind; each validates its argument block on the host before launching
+int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
+int shv_launch_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
+int shv_launch_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
+int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);

@@ -1,0 +1,264 @@
+"""ctypes binding of include/shv_hip.h.  Mirrors the header one to one; no arithmetic lives here."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+Q4K_BLOCK = 256
+Q4K_BYTES = 144
+
+OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
+OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
+OP_EMBED, OP_ARGMAX, OP_RMSNORM, OP_COPY_F32 = 10, 11, 12, 13
+PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID = 0, 1, 2, 3
+
+
+class ShvError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("shv error %d: %s" % (code, msg))
+        self.code = code
+
+
+def lib_path():
+    return os.path.join(HERE, "libshv_hip.so")
+
+
+class Props(C.Structure):
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 32), ("compute_units", C.c_int32),
+                ("wave_size", C.c_int32), ("lds_bytes_per_cu", C.c_int32), ("clock_mhz", C.c_int32),
+                ("hbm_bytes", C.c_uint64)]
+
+
+class GemvQ4KArgs(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("x", C.c_void_p), ("y", C.c_void_p), ("residual", C.c_void_p),
+                ("gamma", C.c_void_p), ("z", C.c_void_p), ("pos", C.c_void_p),
+                ("n", C.c_int32), ("k", C.c_int32), ("n_tok", C.c_int32), ("prologue", C.c_int32),
+                ("head_dim", C.c_int32), ("eps", C.c_float), ("x_stride", C.c_int32),
+                ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("ring_slots", C.c_int32),
+                ("ring_stride", C.c_int32)]
+
+
+class DequantQ4KArgs(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("dst", C.c_void_p), ("rows", C.c_int64), ("k", C.c_int32)]
+
+
+class QuantizeQ4KArgs(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("rows", C.c_int64), ("k", C.c_int32)]
+
+
+class FillNormalArgs(C.Structure):
+    _fields_ = [("dst", C.c_void_p), ("n", C.c_int64), ("seed", C.c_uint64), ("mean", C.c_float),
+                ("std", C.c_float)]
+
+
+class Op(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("flags", C.c_uint32), ("args", C.c_uint8 * 248)]
+
+
+def make_op(kind, args, flags=0):
+    op = Op()
+    op.kind, op.flags = kind, flags
+    n = C.sizeof(args)
+    assert n <= 248, n
+    C.memmove(op.args, C.byref(args), n)
+    return op
+
+
+# every symbol include/shv_hip.h declares; the CPU test suite checks the library exports them all
+SYMBOLS = [
+    "shv_last_error", "shv_device_count", "shv_init", "shv_destroy", "shv_device_props", "shv_sync",
+    "shv_submits", "shv_alloc", "shv_free", "shv_upload", "shv_download", "shv_copy", "shv_zero",
+    "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
+    "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
+    "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_quantize_q4k",
+    "shv_fill_normal",
+]
+
+_lib = None
+
+
+def load():
+    """Load libshv_hip.so.  Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    p = lib_path()
+    if not os.path.exists(p):
+        raise ShvError(-4, "%s is missing: build it with `python strix-halo-vulkan_amd/build.py`" % p)
+    L = C.CDLL(p)
+    vp, vpp = C.c_void_p, C.POINTER(C.c_void_p)
+    L.shv_last_error.restype = C.c_char_p
+    L.shv_device_count.argtypes = [C.POINTER(C.c_int)]
+    L.shv_init.argtypes = [C.c_int, vpp]
+    L.shv_destroy.argtypes = [vp]
+    L.shv_destroy.restype = None
+    L.shv_device_props.argtypes = [vp, C.POINTER(Props)]
+    L.shv_sync.argtypes = [vp]
+    L.shv_submits.argtypes = [vp, C.POINTER(C.c_uint64)]
+    L.shv_alloc.argtypes = [vp, C.c_size_t, vpp]
+    L.shv_free.argtypes = [vp, vp]
+    L.shv_upload.argtypes = [vp, vp, vp, C.c_size_t]
+    L.shv_download.argtypes = [vp, vp, vp, C.c_size_t]
+    L.shv_copy.argtypes = [vp, vp, vp, C.c_size_t]
+    L.shv_zero.argtypes = [vp, vp, C.c_size_t]
+    L.shv_host_alloc.argtypes = [vp, C.c_size_t, vpp]
+    L.shv_host_free.argtypes = [vp, vp]
+    L.shv_enqueue.argtypes = [vp, C.c_uint32, vp, C.c_size_t]
+    L.shv_dispatch_multi.argtypes = [vp, C.POINTER(Op), C.c_int, C.c_int, C.POINTER(C.c_uint64),
+                                     C.POINTER(C.c_uint64)]
+    L.shv_prerecord.argtypes = [vp, C.POINTER(Op), C.c_int, vpp]
+    L.shv_prerecorded_submit.argtypes = [vp, vp, C.c_int, C.POINTER(C.c_uint64)]
+    L.shv_prerecorded_launch.argtypes = [vp, vp]
+    L.shv_prerecorded_count.argtypes = [vp]
+    L.shv_prerecorded_destroy.argtypes = [vp, vp]
+    L.shv_prerecorded_destroy.restype = None
+    L.shv_gemv_q4k.argtypes = [vp, C.POINTER(GemvQ4KArgs)]
+    L.shv_dequant_q4k.argtypes = [vp, C.POINTER(DequantQ4KArgs)]
+    L.shv_quantize_q4k.argtypes = [vp, C.POINTER(QuantizeQ4KArgs)]
+    L.shv_fill_normal.argtypes = [vp, C.POINTER(FillNormalArgs)]
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != 0:
+        raise ShvError(rc, load().shv_last_error().decode("utf-8", "replace"))
+
+
+class DeviceBuffer:
+    """A device allocation owned by a Context (vk.Buffer's role, vk/engine.go:319-634)."""
+
+    def __init__(self, ctx, nbytes):
+        self.ctx, self.nbytes = ctx, int(nbytes)
+        p = C.c_void_p()
+        check(ctx.L.shv_alloc(ctx.h, self.nbytes, C.byref(p)))
+        self.ptr = p.value
+
+    def at(self, byte_offset):
+        assert 0 <= byte_offset <= self.nbytes
+        return self.ptr + byte_offset
+
+    def write(self, arr, byte_offset=0):
+        arr = np.ascontiguousarray(arr)
+        assert byte_offset + arr.nbytes <= self.nbytes, (byte_offset, arr.nbytes, self.nbytes)
+        check(self.ctx.L.shv_upload(self.ctx.h, self.ptr + byte_offset, arr.ctypes.data, arr.nbytes))
+        return self
+
+    def read(self, dtype, count, byte_offset=0):
+        out = np.empty(count, dtype=dtype)
+        assert byte_offset + out.nbytes <= self.nbytes, (byte_offset, out.nbytes, self.nbytes)
+        check(self.ctx.L.shv_download(self.ctx.h, out.ctypes.data, self.ptr + byte_offset, out.nbytes))
+        return out
+
+    def zero(self):
+        check(self.ctx.L.shv_zero(self.ctx.h, self.ptr, self.nbytes))
+        return self
+
+    def free(self):
+        if self.ptr:
+            check(self.ctx.L.shv_free(self.ctx.h, self.ptr))
+            self.ptr = None
+
+
+class Prerecorded:
+    def __init__(self, ctx, ops):
+        self.ctx = ctx
+        arr = (Op * len(ops))(*ops)
+        p = C.c_void_p()
+        check(ctx.L.shv_prerecord(ctx.h, arr, len(ops), C.byref(p)))
+        self.h = p
+
+    def submit(self, iters=1):
+        ns = C.c_uint64()
+        check(self.ctx.L.shv_prerecorded_submit(self.ctx.h, self.h, iters, C.byref(ns)))
+        return ns.value
+
+    def launch(self):
+        check(self.ctx.L.shv_prerecorded_launch(self.ctx.h, self.h))
+
+    def count(self):
+        return self.ctx.L.shv_prerecorded_count(self.h)
+
+    def destroy(self):
+        if self.h:
+            self.ctx.L.shv_prerecorded_destroy(self.ctx.h, self.h)
+            self.h = None
+
+
+class Context:
+    """One device, one in-order stream (vk.Device's role, vk/engine.go:266-311)."""
+
+    def __init__(self, device=0):
+        self.L = load()
+        h = C.c_void_p()
+        check(self.L.shv_init(device, C.byref(h)))
+        self.h = h
+        self._bufs = []
+
+    def props(self):
+        p = Props()
+        check(self.L.shv_device_props(self.h, C.byref(p)))
+        return p
+
+    def alloc(self, nbytes):
+        b = DeviceBuffer(self, max(int(nbytes), 16))
+        self._bufs.append(b)
+        return b
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        return self.alloc(arr.nbytes).write(arr)
+
+    def sync(self):
+        check(self.L.shv_sync(self.h))
+
+    def enqueue(self, kind, args):
+        check(self.L.shv_enqueue(self.h, kind, C.byref(args), C.sizeof(args)))
+
+    def dispatch_multi(self, ops, iters=1, per_op=False):
+        arr = (Op * len(ops))(*ops)
+        total = C.c_uint64()
+        per = (C.c_uint64 * len(ops))() if per_op else None
+        check(self.L.shv_dispatch_multi(self.h, arr, len(ops), iters, C.byref(total), per))
+        return (total.value, list(per)) if per_op else total.value
+
+    def prerecord(self, ops):
+        return Prerecorded(self, ops)
+
+    def destroy(self):
+        if self.h:
+            for b in self._bufs:
+                if b.ptr:
+                    b.free()
+            self._bufs = []
+            self.L.shv_destroy(self.h)
+            self.h = None
+
+    # ---- convenience wrappers over single ops ----
+    def gemv_q4k(self, w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None,
+                 eps=1e-6, head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None,
+                 ring_slots=0, ring_stride=0):
+        a = gemv_args(w, x, y, n, k, n_tok, prologue, gamma, z, residual, eps, head_dim, x_stride,
+                      y_stride, z_stride, pos, ring_slots, ring_stride)
+        check(self.L.shv_gemv_q4k(self.h, C.byref(a)))
+
+
+def _ptr(b):
+    if b is None:
+        return None
+    return b.ptr if isinstance(b, DeviceBuffer) else int(b)
+
+
+def gemv_args(w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None, eps=1e-6,
+              head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None, ring_slots=0,
+              ring_stride=0):
+    a = GemvQ4KArgs()
+    a.w, a.x, a.y = _ptr(w), _ptr(x), _ptr(y)
+    a.residual, a.gamma, a.z, a.pos = _ptr(residual), _ptr(gamma), _ptr(z), _ptr(pos)
+    a.n, a.k, a.n_tok, a.prologue, a.head_dim, a.eps = n, k, n_tok, prologue, head_dim, eps
+    a.x_stride = k if x_stride is None else x_stride
+    a.y_stride = n if y_stride is None else y_stride
+    a.z_stride = k if z_stride is None else z_stride
+    a.ring_slots, a.ring_stride = ring_slots, ring_stride
+    return a

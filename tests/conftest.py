@@ -17,3 +17,12 @@ GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 @pytest.fixture(scope="session")
 def golden_dir():
     return GOLDEN
+
+
+@pytest.fixture(scope="session")
+def ctx():
+    """One device context for the whole GPU session (the reference's tests share one vk.Device)."""
+    import shv
+    c = shv.pkg.Context(0)
+    yield c
+    c.destroy()
