@@ -148,6 +148,52 @@ typedef struct {
     float mean, std;
 } shv_fill_normal_args;
 
+/* MoE router (MoETrace.Route, llm/moe.go:219-274; shaders llm_moe_router/route.comp): per token
+ * xn = RMSNorm(h)*gamma (gamma NULL: h is used as it is), logits = router*xn in float32, softmax,
+ * the n_used largest probabilities in descending order (ties to the lower index), their sum
+ * clamped at 2^-14, the normalised weights; weights[t][n_used] = sigmoid(shared_gate . xn)
+ * (llm/moe.go:396-402).  logits is [T][n_expert+1], the last column the shared-gate logit. */
+typedef struct {
+    const float *h;
+    const float *gamma;
+    const float *router;
+    const float *shared_gate;
+    float *xn;
+    float *logits;
+    int32_t *topk;
+    float *weights;
+    int32_t n_tok, n_embd, n_expert, n_used;
+    float eps;
+    int32_t h_stride;
+} shv_moe_router_args;
+
+/* Expert-gathered gate/up GEMV with SwiGLU (MoETrace.Experts/Shared, llm/moe.go:289-409;
+ * llm_moe_gemv.comp MODE 0): act[t][s] = silu(Wg_e xn[t]) * (Wu_e xn[t]) for e = topk[t][s],
+ * s < n_used, and for the shared expert in slot n_used.  Only the selected experts' rows are
+ * read.  Banks are GGUF Q4_K: expert e's row j is row e*ffn + j, n_embd long. */
+typedef struct {
+    const float *xn;
+    const int32_t *topk;
+    const void *gate_exps, *up_exps;
+    const void *gate_sh, *up_sh;
+    float *act;
+    int32_t n_tok, n_embd, n_used, ffn;
+} shv_moe_up_args;
+
+/* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +
+ * llm_moe_combine.comp): out[t] = residual[t] + sum_s weights[t][s] * (Wd_e act[t][s])
+ * + weights[t][n_used] * (Wd_shared act[t][n_used]).  residual may be NULL. */
+typedef struct {
+    const float *act;
+    const int32_t *topk;
+    const float *weights;
+    const void *down_exps, *down_sh;
+    const float *residual;
+    float *out;
+    int32_t n_tok, n_embd, n_used, ffn;
+    int32_t res_stride, out_stride;
+} shv_moe_down_args;
+
 typedef struct {
     uint32_t kind;
     uint32_t flags;          /* bit 0: may overlap the previous op (MultiDispatch.Overlap) */
@@ -178,6 +224,9 @@ int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
 int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
 int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
 int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
+int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
+int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
+int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 
 #ifdef __cplusplus
 }

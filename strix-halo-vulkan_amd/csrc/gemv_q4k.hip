@@ -20,43 +20,47 @@ constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kMaxTok = 4;
 
-// LDS layout of the staged vector: each 64-float slice is followed by 4 floats of padding so
-// that the lanes of a wave, which read slices 256 bytes apart, fall on different banks.
-__device__ __forceinline__ int lds_slot(int i) { return i + (i >> 6) * 4; }
-
-// U consecutive passes of one wave: issue every load, then consume.
+// U consecutive passes of one wave.  load() issues every 128-bit load of the batch; compute()
+// consumes them.  The kernel keeps two batches alive so that the loads of the next one are in
+// flight while the current one is being multiplied.
 template <int K, int NT, int U>
-__device__ __forceinline__ void gemv_passes(const shv_gemv_q4k_args &a, const char *wbase, int g, int lane, int rsub,
-                                            long long pass, int n, const float (*xr)[64], const float *xs_lo,
-                                            const float *xs_hi, const size_t *y_off) {
-    constexpr int LPR = K / 64;
-    constexpr int RPP = 64 / LPR;
-    constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+struct GemvBatch {
+    static constexpr int LPR = K / 64;
+    static constexpr int RPP = 64 / LPR;
+    static constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     uint4 hdr[U], q0[U], q1[U];
     int row[U];
+
+    __device__ __forceinline__ void load(const char *wbase, int g, int rsub, long long pass, int n) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        const long long r = (pass + u) * RPP + rsub;
-        row[u] = r < n ? static_cast<int>(r) : -1;
-        const char *rp = wbase + static_cast<size_t>(row[u] < 0 ? 0 : row[u]) * ROWB;
-        hdr[u] = load_stream16(rp);
-        q0[u] = load_stream16(rp + 16 + g * 32);
-        q1[u] = load_stream16(rp + 32 + g * 32);
+        for (int u = 0; u < U; u++) {
+            const long long r = (pass + u) * RPP + rsub;
+            row[u] = r < n ? static_cast<int>(r) : -1;
+            const char *rp = wbase + static_cast<size_t>(row[u] < 0 ? 0 : row[u]) * ROWB;
+            hdr[u] = load_stream16(rp);
+            q0[u] = load_stream16(rp + 16 + g * 32);
+            q1[u] = load_stream16(rp + 32 + g * 32);
+        }
     }
+
+    __device__ __forceinline__ void compute(const shv_gemv_q4k_args &a, int g, int lane, const NibbleConsts &nc,
+                                            const float (*xr)[64], const float *xs_lo, const float *xs_hi,
+                                            const size_t *y_off) const {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
+        for (int u = 0; u < U; u++) {
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            float acc = q4k_group_dot(hdr[u], q0[u], q1[u], g, xr[t], xs_lo[t], xs_hi[t]);
-            acc = group_sum<LPR>(acc);
-            if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
-                float r = acc;
-                if (a.residual) r += a.residual[static_cast<size_t>(t) * a.y_stride + row[u]];
-                a.y[y_off[t] + row[u]] = r;
+            for (int t = 0; t < NT; t++) {
+                float acc = q4k_group_dot(hdr[u], q0[u], q1[u], g, nc, xr[t], xs_lo[t], xs_hi[t]);
+                acc = group_sum<LPR>(acc);
+                if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
+                    float r = acc;
+                    if (a.residual) r += a.residual[static_cast<size_t>(t) * a.y_stride + row[u]];
+                    a.y[y_off[t] + row[u]] = r;
+                }
             }
         }
     }
-}
+};
 
 template <int K, int NT>
 __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int passes_per_wave) {
@@ -131,22 +135,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     float xr[NT][64];
     float xs_lo[NT], xs_hi[NT];
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const float4 *src = reinterpret_cast<const float4 *>(&xs[t][gi * 68]);
-        float lo = 0.f, hi = 0.f;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const float4 f = src[i];
-            xr[t][4 * i + 0] = f.x;
-            xr[t][4 * i + 1] = f.y;
-            xr[t][4 * i + 2] = f.z;
-            xr[t][4 * i + 3] = f.w;
-            const float s = (f.x + f.y) + (f.z + f.w);
-            if (i < 8) lo += s; else hi += s;
-        }
-        xs_lo[t] = lo;
-        xs_hi[t] = hi;
-    }
+    for (int t = 0; t < NT; t++) load_x_slice(xs[t], gi, xr[t], xs_lo[t], xs_hi[t]);
 
     const int sb = gi >> 2, g = gi & 3;
     const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
@@ -164,15 +153,34 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
         }
     }
 
-    int p0 = 0;
-    for (; p0 + 4 <= passes_per_wave; p0 += 4)
-        gemv_passes<K, NT, 4>(a, wbase, g, lane, rsub, first_pass + p0, n, xr, xs_lo, xs_hi, y_off);
+    const NibbleConsts nc = nibble_consts();
+    constexpr int U = 4;
+    const int nb = passes_per_wave / U;  // full batches, double-buffered
+    if (nb > 0) {
+        GemvBatch<K, NT, U> A, B;
+        A.load(wbase, g, rsub, first_pass, n);
+        for (int b = 0; b < nb; b += 2) {
+            const bool has_b = b + 1 < nb;
+            if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U, n);
+            A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+            if (has_b) {
+                if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U, n);
+                B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+            }
+        }
+    }
+    int p0 = nb * U;
     if (p0 + 2 <= passes_per_wave) {
-        gemv_passes<K, NT, 2>(a, wbase, g, lane, rsub, first_pass + p0, n, xr, xs_lo, xs_hi, y_off);
+        GemvBatch<K, NT, 2> T2;
+        T2.load(wbase, g, rsub, first_pass + p0, n);
+        T2.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
         p0 += 2;
     }
-    if (p0 < passes_per_wave)
-        gemv_passes<K, NT, 1>(a, wbase, g, lane, rsub, first_pass + p0, n, xr, xs_lo, xs_hi, y_off);
+    if (p0 < passes_per_wave) {
+        GemvBatch<K, NT, 1> T1;
+        T1.load(wbase, g, rsub, first_pass + p0, n);
+        T1.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+    }
 }
 
 template <int K, int NT>

@@ -1,0 +1,353 @@
+// MoE FFN decode step: router (+softmax/top-k in the last block to finish), expert-gathered
+// gate/up GEMV with SwiGLU, down GEMV with weighting and combine.  Only the rows of the selected
+// experts (and the shared one) are read from HBM.
+#include "shv_device.hpp"
+#include "shv_internal.hpp"
+
+namespace {
+
+using namespace shv;
+
+constexpr int kBlock = 256;
+constexpr int kMaxUsed = 16;
+constexpr float kWeightsSumFloor = 6.103515625e-5f;  // 2^-14
+
+// ---------------------------------------------------------------------------- router ---------
+
+// Descending order on (probability, lower index first) as one 64-bit key.
+__device__ __forceinline__ unsigned long long route_key(float p, int idx) {
+    return (static_cast<unsigned long long>(__float_as_uint(p)) << 32) | static_cast<unsigned int>(0x7FFFFFFF - idx);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const unsigned long long o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// One wave routes one token: softmax over n_expert logits (n_expert <= 64*8), then n_used rounds of
+// arg-max.  Probabilities are formed as the reference forms them (exp, sequential float32 sum in
+// index order, multiply by the reciprocal) so that equal logits stay equal probabilities.
+template <int PER>
+__device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *probs_lds) {
+    const int lane = threadIdx.x & 63;
+    float l[PER];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        l[i] = e < n_expert ? logits[e] : -INFINITY;
+        mx = fmaxf(mx, l[i]);
+    }
+    mx = wave_max_all(mx);
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        if (e < n_expert) probs_lds[e] = expf(l[i] - mx);
+    }
+    __builtin_amdgcn_wave_barrier();
+    // the reference's sum runs over the experts in index order in float32; one lane repeats it
+    float sum = 0.f;
+    if (lane == 0)
+        for (int e = 0; e < n_expert; e++) sum += probs_lds[e];
+    sum = __shfl(sum, 0, 64);
+    const float inv = 1.f / sum;
+    unsigned long long key[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        key[i] = e < n_expert ? route_key(probs_lds[e] * inv, e) : 0ull;
+    }
+    // lane k keeps the k-th pick; the running sum is uniform across the wave
+    float my_w = 0.f, wsum = 0.f;
+    int my_e = 0;
+#pragma unroll 1
+    for (int k = 0; k < n_used; k++) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int i = 0; i < PER; i++) best = key[i] > best ? key[i] : best;
+        best = wave_max_u64(best);
+#pragma unroll
+        for (int i = 0; i < PER; i++)
+            if (key[i] == best) key[i] = 0ull;
+        const float w = __uint_as_float(static_cast<unsigned int>(best >> 32));
+        if (lane == k) {
+            my_e = 0x7FFFFFFF - static_cast<int>(best & 0xFFFFFFFFull);
+            my_w = w;
+        }
+        wsum += w;  // slot order, float32: the reference's sum
+    }
+    if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
+    if (lane < n_used) {
+        topk[lane] = my_e;
+        weights[lane] = my_w / wsum;
+    }
+}
+
+// grid: ceil((n_expert+1)/4) blocks of 4 waves, one float32 router row per wave.
+template <int H>
+__global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args a, int32_t *counter) {
+    __shared__ float xs[H];
+    __shared__ float red[4];
+    __shared__ float probs[4][512];
+    __shared__ int is_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = blockIdx.x * 4 + wave;  // n_expert = the shared-gate row
+    for (int t = 0; t < a.n_tok; t++) {
+        const float *h = a.h + static_cast<size_t>(t) * a.h_stride;
+        float v[H / kBlock];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < H / kBlock; i++) {
+            v[i] = h[tid + i * kBlock];
+            ss = fmaf(v[i], v[i], ss);
+        }
+        float scale = 1.f;
+        if (a.gamma) {
+            ss = block_sum_256(ss, red);
+            scale = 1.f / sqrtf(ss / static_cast<float>(H) + a.eps);
+        }
+#pragma unroll
+        for (int i = 0; i < H / kBlock; i++) {
+            const int c = tid + i * kBlock;
+            const float x = a.gamma ? v[i] * scale * a.gamma[c] : v[i];
+            xs[c] = x;
+            if (blockIdx.x == 0 && a.xn) a.xn[static_cast<size_t>(t) * H + c] = x;
+        }
+        __syncthreads();
+        if (row <= a.n_expert && (row < a.n_expert || a.shared_gate)) {
+            const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < H / 256; i++) {
+                const int c = (i * 64 + lane) * 4;
+                const float4 wv = *reinterpret_cast<const float4 *>(w + c);
+                const float4 xv = *reinterpret_cast<const float4 *>(xs + c);
+                acc = fmaf(wv.x, xv.x, acc);
+                acc = fmaf(wv.y, xv.y, acc);
+                acc = fmaf(wv.z, xv.z, acc);
+                acc = fmaf(wv.w, xv.w, acc);
+            }
+            acc = wave_sum_all(acc);
+            if (lane == 0) a.logits[static_cast<size_t>(t) * (a.n_expert + 1) + row] = acc;
+        }
+        __syncthreads();
+    }
+    // ---- the last block to arrive routes every token ----
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const int prev = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = prev == static_cast<int>(gridDim.x) - 1;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int t = wave; t < a.n_tok; t += 4) {
+        const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
+        float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
+        route_token<8>(lg, a.n_expert, a.n_used, a.topk + static_cast<size_t>(t) * a.n_used, wt, probs[wave]);
+        if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(lg[a.n_expert]) : 0.f;
+    }
+}
+
+// ------------------------------------------------------------------------------- up ----------
+
+// grid: (ffn/RPP/4 row groups, n_used+1 slots, n_tok).  One pass per wave: RPP gate rows and the
+// same RPP up rows of one expert, six 16-byte loads per lane in flight together.
+template <int K>
+__global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
+    constexpr int LPR = K / 64, RPP = 64 / LPR;
+    constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+    __shared__ float xs[lds_padded(K)];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int slot = blockIdx.y, t = blockIdx.z;
+    const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
+    const int row = (blockIdx.x * 4 + wave) * RPP + rsub;  // row within the expert
+    const bool live = row < a.ffn;
+
+    // issue the weight loads first: they do not depend on the staged vector
+    const char *gbase, *ubase;
+    if (slot < a.n_used) {
+        const int e = a.topk[static_cast<size_t>(t) * a.n_used + slot];
+        gbase = static_cast<const char *>(a.gate_exps) + static_cast<size_t>(e) * a.ffn * ROWB;
+        ubase = static_cast<const char *>(a.up_exps) + static_cast<size_t>(e) * a.ffn * ROWB;
+    } else {
+        gbase = static_cast<const char *>(a.gate_sh);
+        ubase = static_cast<const char *>(a.up_sh);
+    }
+    const size_t roff = static_cast<size_t>(live ? row : 0) * ROWB + sb * SHV_Q4K_BYTES;
+    Q4kLane wg, wu;
+    wg.load(gbase + roff, g);
+    wu.load(ubase + roff, g);
+
+    const float *x = a.xn + static_cast<size_t>(t) * K;
+#pragma unroll
+    for (int i = 0; i < K / kBlock; i++) {
+        const int c = tid + i * kBlock;
+        xs[lds_slot(c)] = x[c];
+    }
+    __syncthreads();
+    float xr[64], xs_lo, xs_hi;
+    load_x_slice(xs, gi, xr, xs_lo, xs_hi);
+    const NibbleConsts nc = nibble_consts();
+    float gv = wg.dot(g, nc, xr, xs_lo, xs_hi);
+    float uv = wu.dot(g, nc, xr, xs_lo, xs_hi);
+    gv = group_sum<LPR>(gv);
+    uv = group_sum<LPR>(uv);
+    if (live && group_sum_owner<LPR>(lane)) {
+        const float s = gv * sigmoid_exact(gv);
+        a.act[(static_cast<size_t>(t) * (a.n_used + 1) + slot) * a.ffn + row] = s * uv;
+    }
+}
+
+// ------------------------------------------------------------------------------ down ---------
+
+// grid: (n_embd/RPP row groups, n_tok).  A block owns RPP output rows of one token; its four
+// waves split the n_used+1 slots, each lane scales its partial dot by the slot's weight, and the
+// block adds the four waves' sums (and the residual) at the end.
+template <int K, int MAXS>
+__global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
+    constexpr int LPR = K / 64, RPP = 64 / LPR;
+    constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+    constexpr int SPW = (MAXS + 3) / 4;  // slots per wave
+    __shared__ float xs[MAXS][lds_padded(K)];
+    __shared__ float part[4][RPP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.y;
+    const int ns = a.n_used + 1;
+    const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
+    const int row = blockIdx.x * RPP + rsub;
+    const bool live = row < a.n_embd;
+    const size_t roff = static_cast<size_t>(live ? row : 0) * ROWB + sb * SHV_Q4K_BYTES;
+
+    Q4kLane w[SPW];
+    float wt[SPW];
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+        const int s = wave + 4 * i;
+        wt[i] = 0.f;
+        if (s < ns) {
+            const char *base;
+            if (s < a.n_used) {
+                const int e = a.topk[static_cast<size_t>(t) * a.n_used + s];
+                base = static_cast<const char *>(a.down_exps) + static_cast<size_t>(e) * a.n_embd * ROWB;
+            } else {
+                base = static_cast<const char *>(a.down_sh);
+            }
+            w[i].load(base + roff, g);
+            wt[i] = a.weights[static_cast<size_t>(t) * ns + s];
+        }
+    }
+    const float *act = a.act + static_cast<size_t>(t) * ns * K;
+    for (int c = tid; c < ns * K; c += kBlock) xs[c / K][lds_slot(c % K)] = act[c];
+    __syncthreads();
+
+    const NibbleConsts nc = nibble_consts();
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+        const int s = wave + 4 * i;
+        if (s < ns) {
+            float xr[64], xs_lo, xs_hi;
+            load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
+            acc = fmaf(wt[i], w[i].dot(g, nc, xr, xs_lo, xs_hi), acc);
+        }
+    }
+    acc = group_sum<LPR>(acc);
+    if (group_sum_owner<LPR>(lane)) part[wave][rsub] = acc;
+    __syncthreads();
+    if (tid < RPP) {
+        const int r = blockIdx.x * RPP + tid;
+        if (r < a.n_embd) {
+            float v = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
+            if (a.residual) v += a.residual[static_cast<size_t>(t) * a.res_stride + r];
+            a.out[static_cast<size_t>(t) * a.out_stride + r] = v;
+        }
+    }
+}
+
+}  // namespace
+
+int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
+    const shv_moe_router_args &a = *pa;
+    SHV_REQUIRE(a.h && a.router && a.logits && a.topk && a.weights, "moe_router: NULL h, router, logits, topk or weights");
+    SHV_REQUIRE(a.n_tok >= 1, "moe_router: n_tok %d", a.n_tok);
+    SHV_REQUIRE(a.n_expert >= 1 && a.n_expert <= 512, "moe_router: n_expert %d, the routing wave covers up to 512", a.n_expert);
+    SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed && a.n_used <= a.n_expert, "moe_router: n_used %d of %d (at most %d)", a.n_used, a.n_expert, kMaxUsed);
+    SHV_REQUIRE(a.h_stride >= a.n_embd, "moe_router: h_stride %d < n_embd %d", a.h_stride, a.n_embd);
+    SHV_REQUIRE(shv_aligned16(a.router) && shv_aligned16(a.shared_gate), "moe_router: router and shared_gate must be 16-byte aligned");
+    const unsigned blocks = static_cast<unsigned>((a.n_expert + 1 + 3) / 4);
+    int32_t *counter = ctx->counters + shv_ctx::kCounterRouter;
+    switch (a.n_embd) {
+        case 2048: hipLaunchKernelGGL(moe_router_kernel<2048>, dim3(blocks), dim3(kBlock), 0, ctx->stream, a, counter); break;
+        case 1024: hipLaunchKernelGGL(moe_router_kernel<1024>, dim3(blocks), dim3(kBlock), 0, ctx->stream, a, counter); break;
+        case 512: hipLaunchKernelGGL(moe_router_kernel<512>, dim3(blocks), dim3(kBlock), 0, ctx->stream, a, counter); break;
+        default: return shv_set_error(SHV_E_INVALID, "moe_router: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
+    }
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}
+
+int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
+    const shv_moe_up_args &a = *pa;
+    SHV_REQUIRE(a.xn && a.topk && a.gate_exps && a.up_exps && a.gate_sh && a.up_sh && a.act, "moe_up: NULL argument");
+    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
+    SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
+    SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
+    SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
+                "moe_up: weight banks must be 16-byte aligned");
+    dim3 block(kBlock);
+    switch (a.n_embd) {
+        case 2048: {
+            constexpr int RPP = 64 / (2048 / 64);
+            dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
+            hipLaunchKernelGGL(moe_up_kernel<2048>, grid, block, 0, ctx->stream, a);
+            break;
+        }
+        case 1024: {
+            constexpr int RPP = 64 / (1024 / 64);
+            dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
+            hipLaunchKernelGGL(moe_up_kernel<1024>, grid, block, 0, ctx->stream, a);
+            break;
+        }
+        case 512: {
+            constexpr int RPP = 64 / (512 / 64);
+            dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
+            hipLaunchKernelGGL(moe_up_kernel<512>, grid, block, 0, ctx->stream, a);
+            break;
+        }
+        default: return shv_set_error(SHV_E_INVALID, "moe_up: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
+    }
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}
+
+int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
+    const shv_moe_down_args &a = *pa;
+    SHV_REQUIRE(a.act && a.topk && a.weights && a.down_exps && a.down_sh && a.out, "moe_down: NULL argument");
+    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_down: n_tok %d", a.n_tok);
+    SHV_REQUIRE(a.n_used >= 1 && a.n_used + 1 <= 12, "moe_down: n_used %d; built for up to 11 routed experts", a.n_used);
+    SHV_REQUIRE(a.n_embd >= 1 && a.out_stride >= a.n_embd && (!a.residual || a.res_stride >= a.n_embd), "moe_down: strides");
+    SHV_REQUIRE(shv_aligned16(a.down_exps) && shv_aligned16(a.down_sh), "moe_down: weight banks must be 16-byte aligned");
+    dim3 block(kBlock);
+    switch (a.ffn) {
+        case 512: {
+            constexpr int RPP = 64 / (512 / 64);
+            hipLaunchKernelGGL((moe_down_kernel<512, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, ctx->stream, a);
+            break;
+        }
+        case 256: {
+            constexpr int RPP = 64 / (256 / 64);
+            hipLaunchKernelGGL((moe_down_kernel<256, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, ctx->stream, a);
+            break;
+        }
+        default: return shv_set_error(SHV_E_INVALID, "moe_down: ffn = %d; built for 256 and 512", a.ffn);
+    }
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}

@@ -172,6 +172,9 @@ static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t by
         case SHV_OP_DEQUANT_Q4K: return run_as<shv_dequant_q4k_args>(ctx, args, bytes, shv_launch_dequant_q4k, "dequant_q4k");
         case SHV_OP_QUANTIZE_Q4K: return run_as<shv_quantize_q4k_args>(ctx, args, bytes, shv_launch_quantize_q4k, "quantize_q4k");
         case SHV_OP_FILL_NORMAL: return run_as<shv_fill_normal_args>(ctx, args, bytes, shv_launch_fill_normal, "fill_normal");
+        case SHV_OP_MOE_ROUTER: return run_as<shv_moe_router_args>(ctx, args, bytes, shv_launch_moe_router, "moe_router");
+        case SHV_OP_MOE_UP: return run_as<shv_moe_up_args>(ctx, args, bytes, shv_launch_moe_up, "moe_up");
+        case SHV_OP_MOE_DOWN: return run_as<shv_moe_down_args>(ctx, args, bytes, shv_launch_moe_down, "moe_down");
         default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
     }
 }
@@ -300,5 +303,8 @@ int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a) { return dispatch_one
 int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a) { return dispatch_one(ctx, SHV_OP_DEQUANT_Q4K, a, sizeof(*a)); }
 int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a) { return dispatch_one(ctx, SHV_OP_QUANTIZE_Q4K, a, sizeof(*a)); }
 int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a) { return dispatch_one(ctx, SHV_OP_FILL_NORMAL, a, sizeof(*a)); }
+int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a) { return dispatch_one(ctx, SHV_OP_MOE_ROUTER, a, sizeof(*a)); }
+int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a) { return dispatch_one(ctx, SHV_OP_MOE_UP, a, sizeof(*a)); }
+int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a) { return dispatch_one(ctx, SHV_OP_MOE_DOWN, a, sizeof(*a)); }
 
 }  // extern "C"

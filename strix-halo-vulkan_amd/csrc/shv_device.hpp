@@ -89,37 +89,64 @@ __device__ __forceinline__ void q4k_group_scale_min(const uint4 &hdr, int g, uin
     mn = g >= 2 ? mn_hi : mn_lo;
 }
 
-// Dot product of the 8 weights in one payload dword with x: low nibbles of the four bytes meet
-// xlo[0..3], high nibbles meet xhi[0..3].
-__device__ __forceinline__ void q4k_dot8(uint32_t q, const float *xlo, const float *xhi, float &acc_lo, float &acc_hi) {
-    const uint32_t lo = q & 0x0F0F0F0Fu;
-    const uint32_t hi = (q >> 4) & 0x0F0F0F0Fu;
-    acc_lo = fmaf(static_cast<float>(lo & 0xFFu), xlo[0], acc_lo);
-    acc_lo = fmaf(static_cast<float>((lo >> 8) & 0xFFu), xlo[1], acc_lo);
-    acc_lo = fmaf(static_cast<float>((lo >> 16) & 0xFFu), xlo[2], acc_lo);
-    acc_lo = fmaf(static_cast<float>(lo >> 24), xlo[3], acc_lo);
-    acc_hi = fmaf(static_cast<float>(hi & 0xFFu), xhi[0], acc_hi);
-    acc_hi = fmaf(static_cast<float>((hi >> 8) & 0xFFu), xhi[1], acc_hi);
-    acc_hi = fmaf(static_cast<float>((hi >> 16) & 0xFFu), xhi[2], acc_hi);
-    acc_hi = fmaf(static_cast<float>(hi >> 24), xhi[3], acc_hi);
+typedef _Float16 f16x2_native __attribute__((ext_vector_type(2)));
+
+// Constants of the nibble-to-half trick, made opaque to the optimiser so that they live in
+// registers and (q & mask) | one becomes a single v_and_or_b32.
+struct NibbleConsts {
+    uint32_t mask;  // 0x00F000F0: bits 4..7 of both halves
+    uint32_t one;   // 0x54005400: the half 64.0 in both halves
+};
+__device__ __forceinline__ NibbleConsts nibble_consts() {
+    NibbleConsts c;
+    c.mask = 0x00F000F0u;
+    c.one = 0x54005400u;
+    asm volatile("" : "+s"(c.mask));
+    asm volatile("" : "+v"(c.one));
+    return c;
+}
+
+// A 4-bit level n placed in mantissa bits 4..7 of the half 64.0 reads as exactly 64 + n, and
+// v_fma_mix_f32 widens a half operand for free, so each weight costs one FMA and half of a
+// bit-field op.  The accumulators therefore carry 64*sum(x) on top of sum(n*x); the caller
+// takes it off again with the same sums of x it needs for the Q4_K min term.
+//
+// One payload dword holds 8 weights: the low nibbles of its four bytes meet xlo[0..3] and the
+// high nibbles meet xhi[0..3].
+__device__ __forceinline__ void q4k_dot8(uint32_t q, const NibbleConsts &c, const float *xlo, const float *xhi,
+                                         float &acc_lo, float &acc_hi) {
+    const f16x2_native t1 = __builtin_bit_cast(f16x2_native, (q & c.mask) | c.one);         // high nibbles of bytes 0,2
+    const f16x2_native t3 = __builtin_bit_cast(f16x2_native, ((q >> 8) & c.mask) | c.one);  // high nibbles of bytes 1,3
+    const f16x2_native t0 = __builtin_bit_cast(f16x2_native, ((q << 4) & c.mask) | c.one);  // low nibbles of bytes 0,2
+    const f16x2_native t2 = __builtin_bit_cast(f16x2_native, ((q >> 4) & c.mask) | c.one);  // low nibbles of bytes 1,3
+    acc_lo = fmaf(static_cast<float>(t0.x), xlo[0], acc_lo);
+    acc_lo = fmaf(static_cast<float>(t2.x), xlo[1], acc_lo);
+    acc_lo = fmaf(static_cast<float>(t0.y), xlo[2], acc_lo);
+    acc_lo = fmaf(static_cast<float>(t2.y), xlo[3], acc_lo);
+    acc_hi = fmaf(static_cast<float>(t1.x), xhi[0], acc_hi);
+    acc_hi = fmaf(static_cast<float>(t3.x), xhi[1], acc_hi);
+    acc_hi = fmaf(static_cast<float>(t1.y), xhi[2], acc_hi);
+    acc_hi = fmaf(static_cast<float>(t3.y), xhi[3], acc_hi);
 }
 
 // One lane's share of one row: a 64-weight group (32 payload bytes in p0,p1) against the 64
 // activations xr[0..63] of the same columns.  xs_lo / xs_hi are the sums of xr[0..31] / xr[32..63].
 __device__ __forceinline__ float q4k_group_dot(const uint4 &hdr, const uint4 &p0, const uint4 &p1, int g,
-                                               const float *xr, float xs_lo, float xs_hi) {
+                                               const NibbleConsts &c, const float *xr, float xs_lo, float xs_hi) {
     uint32_t sc, mn;
     q4k_group_scale_min(hdr, g, sc, mn);
     const float d = f16_bits_to_f32(hdr.x), dmin = f16_bits_to_f32(hdr.x >> 16);
     float lo = 0.f, hi = 0.f;
-    q4k_dot8(p0.x, xr + 0, xr + 32, lo, hi);
-    q4k_dot8(p0.y, xr + 4, xr + 36, lo, hi);
-    q4k_dot8(p0.z, xr + 8, xr + 40, lo, hi);
-    q4k_dot8(p0.w, xr + 12, xr + 44, lo, hi);
-    q4k_dot8(p1.x, xr + 16, xr + 48, lo, hi);
-    q4k_dot8(p1.y, xr + 20, xr + 52, lo, hi);
-    q4k_dot8(p1.z, xr + 24, xr + 56, lo, hi);
-    q4k_dot8(p1.w, xr + 28, xr + 60, lo, hi);
+    q4k_dot8(p0.x, c, xr + 0, xr + 32, lo, hi);
+    q4k_dot8(p0.y, c, xr + 4, xr + 36, lo, hi);
+    q4k_dot8(p0.z, c, xr + 8, xr + 40, lo, hi);
+    q4k_dot8(p0.w, c, xr + 12, xr + 44, lo, hi);
+    q4k_dot8(p1.x, c, xr + 16, xr + 48, lo, hi);
+    q4k_dot8(p1.y, c, xr + 20, xr + 52, lo, hi);
+    q4k_dot8(p1.z, c, xr + 24, xr + 56, lo, hi);
+    q4k_dot8(p1.w, c, xr + 28, xr + 60, lo, hi);
+    lo = fmaf(-64.f, xs_lo, lo);
+    hi = fmaf(-64.f, xs_hi, hi);
     const float ds0 = d * static_cast<float>(sc & 0xFFu), ds1 = d * static_cast<float>(sc >> 8);
     const float dm0 = dmin * static_cast<float>(mn & 0xFFu), dm1 = dmin * static_cast<float>(mn >> 8);
     return ds0 * lo - dm0 * xs_lo + ds1 * hi - dm1 * xs_hi;
@@ -133,6 +160,46 @@ __device__ __forceinline__ uint4 load_stream16(const void *p) {
     const u32x4_native v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_native *>(p));
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+
+// ---- staging an activation vector for the Q4_K row kernels -----------------------------------
+// LDS layout: each 64-float slice is followed by 4 floats of padding so that the lanes of a wave,
+// which read slices 256 bytes apart, fall on different banks.
+__device__ __forceinline__ int lds_slot(int i) { return i + (i >> 6) * 4; }
+__host__ __device__ constexpr int lds_padded(int k) { return k + (k >> 6) * 4; }
+
+// The 64 activations of 64-weight group `gi`, from a vector staged with lds_slot(), plus the sums
+// of their first and second 32 (the columns the low and the high nibbles of the group meet).
+__device__ __forceinline__ void load_x_slice(const float *xs, int gi, float *xr, float &xs_lo, float &xs_hi) {
+    const float4 *src = reinterpret_cast<const float4 *>(xs + gi * 68);
+    float lo = 0.f, hi = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float4 f = src[i];
+        xr[4 * i + 0] = f.x;
+        xr[4 * i + 1] = f.y;
+        xr[4 * i + 2] = f.z;
+        xr[4 * i + 3] = f.w;
+        const float s = (f.x + f.y) + (f.z + f.w);
+        if (i < 8) lo += s; else hi += s;
+    }
+    xs_lo = lo;
+    xs_hi = hi;
+}
+
+// One lane's loads for one row: the super-block header and the 32 payload bytes of its group.
+struct Q4kLane {
+    uint4 hdr, q0, q1;
+    __device__ __forceinline__ void load(const char *row_sb, int g) {
+        hdr = load_stream16(row_sb);
+        q0 = load_stream16(row_sb + 16 + g * 32);
+        q1 = load_stream16(row_sb + 32 + g * 32);
+    }
+    __device__ __forceinline__ float dot(int g, const NibbleConsts &c, const float *xr, float xs_lo, float xs_hi) const {
+        return q4k_group_dot(hdr, q0, q1, g, c, xr, xs_lo, xs_hi);
+    }
+};
+
+__device__ __forceinline__ float sigmoid_exact(float x) { return 1.f / (1.f + expf(-x)); }
 
 __device__ __forceinline__ float sigmoidf_dev(float x) { return 1.f / (1.f + __expf(-x)); }
 __device__ __forceinline__ float siluf_dev(float x) { return x * sigmoidf_dev(x); }

@@ -19,6 +19,7 @@ struct shv_ctx {
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
     int32_t *counters = nullptr;
     int n_counters = 0;
+    enum { kCounterRouter = 0, kCounterArgmax = 1, kCounterAttn = 16 };
 };
 
 struct shv_prerecorded {
@@ -49,3 +50,6 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
 int shv_launch_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
 int shv_launch_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
 int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
+int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
+int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
+int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);

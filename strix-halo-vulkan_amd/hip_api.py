@@ -52,6 +52,29 @@ class FillNormalArgs(C.Structure):
                 ("std", C.c_float)]
 
 
+class MoeRouterArgs(C.Structure):
+    _fields_ = [("h", C.c_void_p), ("gamma", C.c_void_p), ("router", C.c_void_p),
+                ("shared_gate", C.c_void_p), ("xn", C.c_void_p), ("logits", C.c_void_p),
+                ("topk", C.c_void_p), ("weights", C.c_void_p), ("n_tok", C.c_int32),
+                ("n_embd", C.c_int32), ("n_expert", C.c_int32), ("n_used", C.c_int32),
+                ("eps", C.c_float), ("h_stride", C.c_int32)]
+
+
+class MoeUpArgs(C.Structure):
+    _fields_ = [("xn", C.c_void_p), ("topk", C.c_void_p), ("gate_exps", C.c_void_p),
+                ("up_exps", C.c_void_p), ("gate_sh", C.c_void_p), ("up_sh", C.c_void_p),
+                ("act", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
+                ("n_used", C.c_int32), ("ffn", C.c_int32)]
+
+
+class MoeDownArgs(C.Structure):
+    _fields_ = [("act", C.c_void_p), ("topk", C.c_void_p), ("weights", C.c_void_p),
+                ("down_exps", C.c_void_p), ("down_sh", C.c_void_p), ("residual", C.c_void_p),
+                ("out", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
+                ("n_used", C.c_int32), ("ffn", C.c_int32), ("res_stride", C.c_int32),
+                ("out_stride", C.c_int32)]
+
+
 class Op(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("flags", C.c_uint32), ("args", C.c_uint8 * 248)]
 
@@ -72,7 +95,7 @@ SYMBOLS = [
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_quantize_q4k",
-    "shv_fill_normal",
+    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down",
 ]
 
 _lib = None
@@ -117,6 +140,9 @@ def load():
     L.shv_dequant_q4k.argtypes = [vp, C.POINTER(DequantQ4KArgs)]
     L.shv_quantize_q4k.argtypes = [vp, C.POINTER(QuantizeQ4KArgs)]
     L.shv_fill_normal.argtypes = [vp, C.POINTER(FillNormalArgs)]
+    L.shv_moe_router.argtypes = [vp, C.POINTER(MoeRouterArgs)]
+    L.shv_moe_up.argtypes = [vp, C.POINTER(MoeUpArgs)]
+    L.shv_moe_down.argtypes = [vp, C.POINTER(MoeDownArgs)]
     _lib = L
     return L
 
@@ -242,6 +268,11 @@ class Context:
         a = gemv_args(w, x, y, n, k, n_tok, prologue, gamma, z, residual, eps, head_dim, x_stride,
                       y_stride, z_stride, pos, ring_slots, ring_stride)
         check(self.L.shv_gemv_q4k(self.h, C.byref(a)))
+
+
+def ptr(b):
+    """Device address of a DeviceBuffer, an int, or None."""
+    return _ptr(b)
 
 
 def _ptr(b):
