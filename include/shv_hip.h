@@ -104,8 +104,11 @@ enum {
 /* y[t][r] = sum_i W[r][i] * pro(x[t])[i] (+ residual[t][r]); W is GGUF Q4_K, row-major, k%256==0.
  * The reference's CPU form is matvec over Tensor.DequantizeRow (llm/hc.go:255-264,
  * gguf/dequant.go:119-124); its GPU forms are llm_gemv.comp and llm_moe_gemv.comp.
- * ring_slots>0: row t is written at y + ((pos[0]+t) % ring_slots)*ring_stride instead of
- * y + t*y_stride (the DeltaNet projection ring, shaders/llm_dn_conv.comp:36-49). */
+ * Rows are grouped into sequences of seq_len consecutive tokens (seq_len 0 means one sequence
+ * of n_tok).  ring_slots>0 selects ring output, the DeltaNet projection ring of
+ * shaders/llm_dn_conv.comp:36-49 and llm_seq_hist.comp:17-26: row i of sequence s is written at
+ * y + (slot[s]*ring_slots + (pos[s]+i) % ring_slots) * ring_stride, slot[s] = s when slot is NULL,
+ * instead of y + t*y_stride. */
 typedef struct {
     const void *w;
     const float *x;
@@ -114,12 +117,13 @@ typedef struct {
     const float *gamma;
     const float *z;
     const int32_t *pos;
+    const int32_t *slot;
     int32_t n, k, n_tok;
     int32_t prologue;
     int32_t head_dim;
     float eps;
     int32_t x_stride, y_stride, z_stride;
-    int32_t ring_slots, ring_stride;
+    int32_t seq_len, ring_slots, ring_stride;
 } shv_gemv_q4k_args;
 
 /* dst[i] = d*sc*q - dmin*m for every weight of `rows` rows, the reference's dequantQ4_K
@@ -194,6 +198,33 @@ typedef struct {
     int32_t res_stride, out_stride;
 } shv_moe_down_args;
 
+/* Gated DeltaNet step(s) after the fused projection (DeltaNetLayer, llm/deltanet.go:266-327 and
+ * deltaRule :365-403; shaders llm_dn_conv.comp + llm_dn_scan.comp): for each of n_seq sequences,
+ * seq_len consecutive tokens starting at pos[s] on state slot[s] (s itself when slot is NULL):
+ * depthwise causal conv (kernel 4) over the ring of fused projection rows, SiLU, L2-normalised
+ * q and k per key head, g = exp(softplus(alpha+dt_bias)*A), beta = sigmoid(b), then
+ * S *= g; delta = (v - S^T k)*beta; S += k delta^T; o = S^T q / sqrt(d).
+ * A ring row is [q (hk*d) | k (hk*d) | v (hv*d) | z (hv*d) | alpha (hv) | beta (hv)]; positions
+ * before the start of a sequence read as zero.  state is [n_slots][hv][d][d] float32 holding
+ * S[i][j] at [j*d+i] (the reference's transposed layout), updated in place; out is the raw
+ * attention output [n_seq*seq_len][hv*d] that the gated norm of the out projection consumes.
+ * v-head h reads key head h % hk (kHeadOfV, llm/deltanet.go:412-418). */
+typedef struct {
+    const float *ring;
+    const float *conv1d;
+    const float *a;
+    const float *dt_bias;
+    float *state;
+    float *out;
+    const int32_t *pos;
+    const int32_t *slot;
+    int32_t n_seq, seq_len;
+    int32_t n_head_k, n_head_v, head_dim, conv;
+    int32_t ring_slots, ring_stride;
+    float eps;
+    int32_t qk_norm_max;
+} shv_dn_step_args;
+
 typedef struct {
     uint32_t kind;
     uint32_t flags;          /* bit 0: may overlap the previous op (MultiDispatch.Overlap) */
@@ -227,6 +258,7 @@ int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
 int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
 int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
+int shv_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,137 @@
+// Gated DeltaNet decode step: causal conv1d + SiLU + L2 norm of q/k, decay and write strength,
+// and the delta-rule update of the 128x128 float32 state of each value head.
+//
+// HBM-bound on the state (read once, written once per call).  A 256-thread block owns 8 of a
+// head's 128 state rows (row j holds column j of S, contiguous over the key axis): a wave holds
+// two rows, 32 lanes x float4 each, in registers across all tokens of the call, and reduces the
+// two dot products of the rule (against k, then against q) over those 32 lanes with DPP.  The
+// cheap per-head prologue (conv, norm, gate) is recomputed by every block of the head so that no
+// grid-wide hand-over is needed.
+#include "shv_device.hpp"
+#include "shv_internal.hpp"
+
+namespace {
+
+using namespace shv;
+
+constexpr int kBlock = 256;
+constexpr int kD = 128;       // head dimension the kernel is built for
+constexpr int kRowsPerBlock = 8;
+
+// Sum over aligned groups of 32 lanes, result in every lane of the group.
+__device__ __forceinline__ float sum32_all(float v) {
+    v += dpp_f32<kDppXor1>(v);
+    v += dpp_f32<kDppXor2>(v);
+    v += dpp_f32<kDppHalfMirror>(v);
+    v += dpp_f32<kDppMirror>(v);
+    v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
+__device__ __forceinline__ float softplus_ref(float x) {
+    // the add inside the log is float32 on purpose: below about -16.6 it returns exactly 0
+    return x > 20.f ? x : logf(1.f + expf(x));
+}
+
+// Causal depthwise conv of kernel 4 for channel ch at position p: taps 0..3 meet positions
+// p-3..p; rows before the sequence start are zero.
+__device__ __forceinline__ float conv4(const float *ring, int ring_slots, int ring_stride, const float *taps, int ch, int p) {
+    const float4 k = *reinterpret_cast<const float4 *>(taps + static_cast<size_t>(ch) * 4);
+    const float kk[4] = {k.x, k.y, k.z, k.w};
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int pp = p + j - 3;
+        const float x = pp < 0 ? 0.f : ring[static_cast<size_t>(pp % ring_slots) * ring_stride + ch];
+        s += x * kk[j];
+    }
+    return s;
+}
+
+// grid: (128/8 row chunks, n_head_v, n_seq)
+__global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
+    __shared__ __align__(16) float qs[kD];
+    __shared__ __align__(16) float ks[kD];
+    __shared__ float vs[kRowsPerBlock];
+    __shared__ float red[4];
+    __shared__ float gb[2];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int chunk = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
+    const int slot = a.slot ? a.slot[seq] : seq;
+    const int pos0 = a.pos ? a.pos[seq] : 0;
+    const int hk = h % a.n_head_k;
+    const int qk = a.n_head_k * kD, vw = a.n_head_v * kD;
+    const int alpha_off = 2 * qk + 2 * vw, beta_off = alpha_off + a.n_head_v;
+    const int rsub = lane >> 5, li = lane & 31;
+    const int jl = wave * 2 + rsub;           // row within the block
+    const int j = chunk * kRowsPerBlock + jl; // row of the head's state
+    float *srow = a.state + ((static_cast<size_t>(slot) * a.n_head_v + h) * kD + j) * kD + li * 4;
+    float4 s = *reinterpret_cast<const float4 *>(srow);  // in flight while the prologue runs
+
+    const float *ring = a.ring + static_cast<size_t>(slot) * a.ring_slots * a.ring_stride;
+    const float scale = 1.f / sqrtf(static_cast<float>(kD));
+
+    for (int i = 0; i < a.seq_len; i++) {
+        const int p = pos0 + i;
+        // q (threads 0..127) and k (128..255) channels of key head hk
+        const int ch = tid < kD ? hk * kD + tid : qk + hk * kD + (tid - kD);
+        const float c = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, ch, p);
+        const float act = c * sigmoid_exact(c);
+        const float ss = wave_sum_all(act * act);
+        if (lane == 0) red[wave] = ss;
+        if (tid < kRowsPerBlock) {
+            const int vch = 2 * qk + h * kD + chunk * kRowsPerBlock + tid;
+            const float cv = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, vch, p);
+            vs[tid] = cv * sigmoid_exact(cv);
+        }
+        if (tid == 64) {
+            const float *row = ring + static_cast<size_t>(p % a.ring_slots) * a.ring_stride;
+            const float asp = softplus_ref(row[alpha_off + h] + a.dt_bias[h]);
+            gb[0] = expf(asp * a.a[h]);
+            gb[1] = sigmoid_exact(row[beta_off + h]);
+        }
+        __syncthreads();
+        {
+            const float ssq = tid < kD ? red[0] + red[1] : red[2] + red[3];
+            const float nrm = a.qk_norm_max ? 1.f / fmaxf(sqrtf(ssq), a.eps) : 1.f / sqrtf(ssq + a.eps);
+            if (tid < kD) qs[tid] = act * nrm; else ks[tid - kD] = act * nrm;
+        }
+        __syncthreads();
+        const float4 k4 = *reinterpret_cast<const float4 *>(ks + li * 4);
+        const float4 q4 = *reinterpret_cast<const float4 *>(qs + li * 4);
+        const float g = gb[0], beta = gb[1], vj = vs[jl];
+        s.x *= g; s.y *= g; s.z *= g; s.w *= g;
+        const float dk = sum32_all(fmaf(s.x, k4.x, fmaf(s.y, k4.y, fmaf(s.z, k4.z, s.w * k4.w))));
+        const float delta = (vj - dk) * beta;
+        s.x = fmaf(delta, k4.x, s.x);
+        s.y = fmaf(delta, k4.y, s.y);
+        s.z = fmaf(delta, k4.z, s.z);
+        s.w = fmaf(delta, k4.w, s.w);
+        const float oq = sum32_all(fmaf(s.x, q4.x, fmaf(s.y, q4.y, fmaf(s.z, q4.z, s.w * q4.w))));
+        if (li == 0)
+            a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j] = oq * scale;
+        __syncthreads();
+    }
+    *reinterpret_cast<float4 *>(srow) = s;
+}
+
+}  // namespace
+
+int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
+    const shv_dn_step_args &a = *pa;
+    SHV_REQUIRE(a.ring && a.conv1d && a.a && a.dt_bias && a.state && a.out, "dn_step: NULL argument");
+    SHV_REQUIRE(a.head_dim == kD, "dn_step: head_dim %d; built for %d", a.head_dim, kD);
+    SHV_REQUIRE(a.conv == 4, "dn_step: conv kernel %d; built for 4", a.conv);
+    SHV_REQUIRE(a.n_head_k >= 1 && a.n_head_v >= a.n_head_k && a.n_head_v <= 65535, "dn_step: heads %d/%d", a.n_head_k, a.n_head_v);
+    SHV_REQUIRE(a.n_seq >= 1 && a.n_seq <= 65535 && a.seq_len >= 1, "dn_step: %d sequences of %d", a.n_seq, a.seq_len);
+    const int width = 2 * a.n_head_k * kD + 2 * a.n_head_v * kD + 2 * a.n_head_v;
+    SHV_REQUIRE(a.ring_stride >= width, "dn_step: ring_stride %d < row width %d", a.ring_stride, width);
+    SHV_REQUIRE(a.ring_slots >= a.seq_len + a.conv - 1, "dn_step: a ring of %d slots cannot hold %d tokens and %d of history",
+                a.ring_slots, a.seq_len, a.conv - 1);
+    SHV_REQUIRE(shv_aligned16(a.state) && shv_aligned16(a.conv1d), "dn_step: state and conv1d must be 16-byte aligned");
+    dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
+    hipLaunchKernelGGL(dn_step_kernel, grid, dim3(kBlock), 0, ctx->stream, a);
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}

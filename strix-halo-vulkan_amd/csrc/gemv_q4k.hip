@@ -45,7 +45,7 @@ struct GemvBatch {
 
     __device__ __forceinline__ void compute(const shv_gemv_q4k_args &a, int g, int lane, const NibbleConsts &nc,
                                             const float (*xr)[64], const float *xs_lo, const float *xs_hi,
-                                            const size_t *y_off) const {
+                                            const size_t *y_off, int t0) const {
 #pragma unroll
         for (int u = 0; u < U; u++) {
 #pragma unroll
@@ -54,7 +54,7 @@ struct GemvBatch {
                 acc = group_sum<LPR>(acc);
                 if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
                     float r = acc;
-                    if (a.residual) r += a.residual[static_cast<size_t>(t) * a.y_stride + row[u]];
+                    if (a.residual) r += a.residual[static_cast<size_t>(t0 + t) * a.y_stride + row[u]];
                     a.y[y_off[t] + row[u]] = r;
                 }
             }
@@ -63,7 +63,7 @@ struct GemvBatch {
 };
 
 template <int K, int NT>
-__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int passes_per_wave) {
+__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int passes_per_wave, int t0) {
     constexpr int LPR = K / 64;   // lanes per row
     constexpr int XPAD = K + K / 64 * 4;
     extern __shared__ float smem[];
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     // ---- stage pro(x) in LDS ----
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        const float *x = a.x + static_cast<size_t>(t) * a.x_stride;
+        const float *x = a.x + static_cast<size_t>(t0 + t) * a.x_stride;
         if (a.prologue == SHV_PRO_RMSNORM) {
             float v[K / kBlock];
             float ss = 0.f;
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
             // thread owns K/256 consecutive columns; a head of head_dim columns spans
             // head_dim/(K/256) consecutive threads (a power of two <= 64).
             constexpr int PER = K / kBlock;
-            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+            const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
             float v[PER];
             float ss = 0.f;
 #pragma unroll
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
                 xs[t][lds_slot(c)] = v[i] * scale * a.gamma[c % a.head_dim] * g;
             }
         } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
-            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+            const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
 #pragma unroll
             for (int i = 0; i < K / kBlock; i++) {
                 const int c = tid + i * kBlock;
@@ -146,10 +146,13 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         if (a.ring_slots > 0) {
-            const int p = a.pos ? a.pos[0] : 0;
-            y_off[t] = static_cast<size_t>((p + t) % a.ring_slots) * a.ring_stride;
+            const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+            const int s = (t0 + t) / sl, i = (t0 + t) % sl;
+            const int p = a.pos ? a.pos[s] : 0;
+            const int slot = a.slot ? a.slot[s] : s;
+            y_off[t] = (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
         } else {
-            y_off[t] = static_cast<size_t>(t) * a.y_stride;
+            y_off[t] = static_cast<size_t>(t0 + t) * a.y_stride;
         }
     }
 
@@ -162,10 +165,10 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
         for (int b = 0; b < nb; b += 2) {
             const bool has_b = b + 1 < nb;
             if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U, n);
-            A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+            A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
             if (has_b) {
                 if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U, n);
-                B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+                B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
             }
         }
     }
@@ -173,18 +176,18 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     if (p0 + 2 <= passes_per_wave) {
         GemvBatch<K, NT, 2> T2;
         T2.load(wbase, g, rsub, first_pass + p0, n);
-        T2.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+        T2.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
         p0 += 2;
     }
     if (p0 < passes_per_wave) {
         GemvBatch<K, NT, 1> T1;
         T1.load(wbase, g, rsub, first_pass + p0, n);
-        T1.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off);
+        T1.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
     }
 }
 
 template <int K, int NT>
-int launch_nt(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw) {
+int launch_nt(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw, int t0) {
     if (lds > 48 * 1024) {
         // above the default dynamic-LDS allowance the limit has to be raised once per kernel
         static bool raised = false;
@@ -194,7 +197,7 @@ int launch_nt(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, s
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_q4k_kernel<K, NT>), grid, block, lds, ctx->stream, a, ppw);
+    hipLaunchKernelGGL((gemv_q4k_kernel<K, NT>), grid, block, lds, ctx->stream, a, ppw, t0);
     SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
@@ -212,14 +215,20 @@ int launch_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     SHV_REQUIRE(blocks > 0 && blocks < (1ll << 31), "gemv_q4k: grid of %lld blocks", blocks);
     dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
-    const size_t lds = static_cast<size_t>(a.n_tok) * (K + K / 64 * 4) * sizeof(float);
-    switch (a.n_tok) {
-        case 1: return launch_nt<K, 1>(ctx, a, grid, block, lds, static_cast<int>(ppw));
-        case 2: return launch_nt<K, 2>(ctx, a, grid, block, lds, static_cast<int>(ppw));
-        case 3: return launch_nt<K, 3>(ctx, a, grid, block, lds, static_cast<int>(ppw));
-        case 4: return launch_nt<K, 4>(ctx, a, grid, block, lds, static_cast<int>(ppw));
-        default: return shv_set_error(SHV_E_INVALID, "gemv_q4k: n_tok %d, the GEMV covers 1..%d rows", a.n_tok, kMaxTok);
+    // more than kMaxTok rows: several launches of up to kMaxTok rows each over the same weights
+    for (int t0 = 0; t0 < a.n_tok; t0 += kMaxTok) {
+        const int nt = a.n_tok - t0 < kMaxTok ? a.n_tok - t0 : kMaxTok;
+        const size_t lds = static_cast<size_t>(nt) * (K + K / 64 * 4) * sizeof(float);
+        int rc;
+        switch (nt) {
+            case 1: rc = launch_nt<K, 1>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
+            case 2: rc = launch_nt<K, 2>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
+            case 3: rc = launch_nt<K, 3>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
+            default: rc = launch_nt<K, 4>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
+        }
+        if (rc != SHV_OK) return rc;
     }
+    return SHV_OK;
 }
 
 }  // namespace
@@ -228,7 +237,7 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
     const shv_gemv_q4k_args &a = *pa;
     SHV_REQUIRE(a.w && a.x && a.y, "gemv_q4k: NULL w, x or y");
     SHV_REQUIRE(a.n > 0, "gemv_q4k: n = %d", a.n);
-    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= kMaxTok, "gemv_q4k: n_tok %d, the GEMV covers 1..%d rows", a.n_tok, kMaxTok);
+    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 64, "gemv_q4k: n_tok %d, the GEMV covers 1..64 rows", a.n_tok);
     SHV_REQUIRE(shv_aligned16(a.w), "gemv_q4k: w must be 16-byte aligned");
     SHV_REQUIRE(a.x_stride >= a.k || a.n_tok == 1, "gemv_q4k: x_stride %d < k %d", a.x_stride, a.k);
     SHV_REQUIRE(a.y_stride >= a.n || a.n_tok == 1 || a.ring_slots > 0, "gemv_q4k: y_stride %d < n %d", a.y_stride, a.n);
@@ -242,7 +251,11 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
                     "gemv_q4k: gated-norm head_dim %d does not tile k %d", a.head_dim, a.k);
     }
     if (a.prologue == SHV_PRO_MUL_SIGMOID) SHV_REQUIRE(a.z, "gemv_q4k: sigmoid-gate prologue without z");
-    if (a.ring_slots > 0) SHV_REQUIRE(a.ring_stride >= a.n && a.n_tok <= a.ring_slots, "gemv_q4k: ring of %d slots, stride %d", a.ring_slots, a.ring_stride);
+    if (a.ring_slots > 0) {
+        const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+        SHV_REQUIRE(a.ring_stride >= a.n && sl <= a.ring_slots && a.n_tok % sl == 0 && !a.residual,
+                    "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
+    }
     switch (a.k) {
         case 512: return launch_k<512>(ctx, a);
         case 1024: return launch_k<1024>(ctx, a);

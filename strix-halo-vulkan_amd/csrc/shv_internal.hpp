@@ -53,3 +53,4 @@ int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
 int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
 int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
+int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);

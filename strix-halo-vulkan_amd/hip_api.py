@@ -32,11 +32,11 @@ class Props(C.Structure):
 
 class GemvQ4KArgs(C.Structure):
     _fields_ = [("w", C.c_void_p), ("x", C.c_void_p), ("y", C.c_void_p), ("residual", C.c_void_p),
-                ("gamma", C.c_void_p), ("z", C.c_void_p), ("pos", C.c_void_p),
+                ("gamma", C.c_void_p), ("z", C.c_void_p), ("pos", C.c_void_p), ("slot", C.c_void_p),
                 ("n", C.c_int32), ("k", C.c_int32), ("n_tok", C.c_int32), ("prologue", C.c_int32),
                 ("head_dim", C.c_int32), ("eps", C.c_float), ("x_stride", C.c_int32),
-                ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("ring_slots", C.c_int32),
-                ("ring_stride", C.c_int32)]
+                ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("seq_len", C.c_int32),
+                ("ring_slots", C.c_int32), ("ring_stride", C.c_int32)]
 
 
 class DequantQ4KArgs(C.Structure):
@@ -75,6 +75,15 @@ class MoeDownArgs(C.Structure):
                 ("out_stride", C.c_int32)]
 
 
+class DnStepArgs(C.Structure):
+    _fields_ = [("ring", C.c_void_p), ("conv1d", C.c_void_p), ("a", C.c_void_p),
+                ("dt_bias", C.c_void_p), ("state", C.c_void_p), ("out", C.c_void_p),
+                ("pos", C.c_void_p), ("slot", C.c_void_p), ("n_seq", C.c_int32),
+                ("seq_len", C.c_int32), ("n_head_k", C.c_int32), ("n_head_v", C.c_int32),
+                ("head_dim", C.c_int32), ("conv", C.c_int32), ("ring_slots", C.c_int32),
+                ("ring_stride", C.c_int32), ("eps", C.c_float), ("qk_norm_max", C.c_int32)]
+
+
 class Op(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("flags", C.c_uint32), ("args", C.c_uint8 * 248)]
 
@@ -95,7 +104,7 @@ SYMBOLS = [
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_quantize_q4k",
-    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down",
+    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step",
 ]
 
 _lib = None
@@ -143,6 +152,7 @@ def load():
     L.shv_moe_router.argtypes = [vp, C.POINTER(MoeRouterArgs)]
     L.shv_moe_up.argtypes = [vp, C.POINTER(MoeUpArgs)]
     L.shv_moe_down.argtypes = [vp, C.POINTER(MoeDownArgs)]
+    L.shv_dn_step.argtypes = [vp, C.POINTER(DnStepArgs)]
     _lib = L
     return L
 
@@ -264,9 +274,9 @@ class Context:
     # ---- convenience wrappers over single ops ----
     def gemv_q4k(self, w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None,
                  eps=1e-6, head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None,
-                 ring_slots=0, ring_stride=0):
+                 ring_slots=0, ring_stride=0, slot=None, seq_len=0):
         a = gemv_args(w, x, y, n, k, n_tok, prologue, gamma, z, residual, eps, head_dim, x_stride,
-                      y_stride, z_stride, pos, ring_slots, ring_stride)
+                      y_stride, z_stride, pos, ring_slots, ring_stride, slot, seq_len)
         check(self.L.shv_gemv_q4k(self.h, C.byref(a)))
 
 
@@ -283,7 +293,7 @@ def _ptr(b):
 
 def gemv_args(w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None, eps=1e-6,
               head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None, ring_slots=0,
-              ring_stride=0):
+              ring_stride=0, slot=None, seq_len=0):
     a = GemvQ4KArgs()
     a.w, a.x, a.y = _ptr(w), _ptr(x), _ptr(y)
     a.residual, a.gamma, a.z, a.pos = _ptr(residual), _ptr(gamma), _ptr(z), _ptr(pos)
@@ -291,5 +301,5 @@ def gemv_args(w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, res
     a.x_stride = k if x_stride is None else x_stride
     a.y_stride = n if y_stride is None else y_stride
     a.z_stride = k if z_stride is None else z_stride
-    a.ring_slots, a.ring_stride = ring_slots, ring_stride
+    a.ring_slots, a.ring_stride, a.slot, a.seq_len = ring_slots, ring_stride, _ptr(slot), seq_len
     return a

@@ -1,0 +1,169 @@
+"""Gated DeltaNet layer on the GPU (fused projection GEMV -> dn_step -> out projection with the
+gated norm as its prologue) against the oracle's DeltaNetLayer (llm/deltanet.go:212-403)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import shv
+
+pytestmark = pytest.mark.gpu
+A = shv.api
+TOL = 1e-3
+EPS = 1e-6
+
+
+class DnCase:
+    def __init__(self, ctx, seed, H=2048, hk=16, hv=32, d=128, conv=4):
+        rng = np.random.default_rng(seed)
+        self.ctx, self.H, self.hk, self.hv, self.d, self.conv = ctx, H, hk, hv, d, conv
+        self.qk, self.vw = hk * d, hv * d
+        self.cw = 2 * self.qk + self.vw
+        self.width = self.cw + self.vw + 2 * hv  # fused projection rows: qkv | z | alpha | beta
+        q = lambda rows, k: O.quantize_q4k((rng.standard_normal((rows, k)) * 0.02).astype(np.float32))
+        self.qkv, self.z, self.alpha, self.beta = q(self.cw, H), q(self.vw, H), q(hv, H), q(hv, H)
+        self.out = q(H, self.vw)
+        self.conv1d = (rng.standard_normal((self.cw, conv)) * 0.3).astype(np.float32)
+        self.a = (-np.exp(rng.standard_normal(hv))).astype(np.float32)
+        self.dt_bias = rng.standard_normal(hv).astype(np.float32)
+        self.norm = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+        self.rng = rng
+        self.fused = np.concatenate([self.qkv, self.z, self.alpha, self.beta], axis=0)
+
+    def cfg(self):
+        return O.DnCfg(self.H, self.d, self.hk, self.hv, self.conv, EPS, 0)
+
+    def w(self):
+        return O.DnW(O.B(self.qkv), O.B(self.z), O.B(self.alpha), O.B(self.beta), O.B(self.out),
+                     O.F(self.conv1d), O.F(self.a), O.F(self.dt_bias), O.F(self.norm))
+
+    def oracle(self, xn, conv_state, s_state):
+        T = xn.shape[0]
+        res = np.empty((T, self.H), np.float32)
+        attn = np.empty((T, self.vw), np.float32)
+        cfg, w = self.cfg(), self.w()
+        O.lib().shv_ref_deltanet_layer(O.C.byref(cfg), O.C.byref(w), O.F(xn), T, O.F(conv_state),
+                                       O.F(s_state), O.F(res), None, None, None, None, None,
+                                       O.F(attn), None, 0, 8)
+        return res, attn
+
+    def upload(self):
+        c = self.ctx
+        self.d_fused, self.d_out = c.upload(self.fused), c.upload(self.out)
+        self.d_conv, self.d_a, self.d_dt = c.upload(self.conv1d), c.upload(self.a), c.upload(self.dt_bias)
+        self.d_norm = c.upload(self.norm)
+
+    def step_ops(self, d_x, d_ring, d_state, d_attn, d_res, d_pos, d_slot, n_seq, seq_len, ring_slots):
+        n_tok = n_seq * seq_len
+        return [
+            A.make_op(A.OP_GEMV_Q4K, A.gemv_args(self.d_fused, d_x, d_ring, self.width, self.H, n_tok,
+                                                 pos=d_pos, slot=d_slot, seq_len=seq_len,
+                                                 ring_slots=ring_slots, ring_stride=self.width)),
+            A.make_op(A.OP_DN_STEP, A.DnStepArgs(d_ring.ptr, self.d_conv.ptr, self.d_a.ptr, self.d_dt.ptr,
+                                                 d_state.ptr, d_attn.ptr, d_pos.ptr,
+                                                 A.ptr(d_slot), n_seq, seq_len, self.hk, self.hv,
+                                                 self.d, self.conv, ring_slots, self.width, EPS, 0)),
+            A.make_op(A.OP_GEMV_Q4K, A.gemv_args(self.d_out, d_attn, d_res, self.H, self.vw, n_tok,
+                                                 prologue=A.PRO_GATED_NORM, gamma=self.d_norm,
+                                                 z=d_ring.at(0), head_dim=self.d, eps=EPS)),
+        ]
+
+
+def test_decode_steps_from_a_fresh_state(ctx):
+    """Seven tokens one at a time on the GPU against seven tokens in one oracle call."""
+    case = DnCase(ctx, seed=1)
+    case.upload()
+    T = 7
+    xn = case.rng.standard_normal((T, case.H)).astype(np.float32)
+    conv_state = np.zeros((case.cw, 3), np.float32)
+    s_state = np.zeros((case.hv, case.d, case.d), np.float32)
+    want_res, want_attn = case.oracle(xn, conv_state, s_state)
+
+    c = ctx
+    slots = 4
+    d_ring = c.alloc(slots * case.width * 4).zero()
+    d_state = c.alloc(s_state.nbytes).zero()
+    d_attn, d_res = c.alloc(case.vw * 4), c.alloc(case.H * 4)
+    d_pos, d_x = c.alloc(4), c.alloc(case.H * 4)
+    got_res, got_attn = [], []
+    for t in range(T):
+        d_pos.write(np.array([t], np.int32))
+        d_x.write(xn[t])
+        ops = case.step_ops(d_x, d_ring, d_state, d_attn, d_res, d_pos, None, 1, 1, slots)
+        # the out projection reads z from the ring row of this position
+        ga = A.gemv_args(case.d_out, d_attn, d_res, case.H, case.vw, 1, prologue=A.PRO_GATED_NORM,
+                         gamma=case.d_norm, z=d_ring.at(((t % slots) * case.width + case.cw) * 4),
+                         head_dim=case.d, eps=EPS)
+        ops[2] = A.make_op(A.OP_GEMV_Q4K, ga)
+        c.dispatch_multi(ops)
+        got_res.append(d_res.read(np.float32, case.H))
+        got_attn.append(d_attn.read(np.float32, case.vw))
+    got_res, got_attn = np.array(got_res), np.array(got_attn)
+    e_attn, e_res = O.rel_l2(got_attn, want_attn), O.rel_l2(got_res, want_res)
+    e_state = O.rel_l2(d_state.read(np.float32, s_state.size), s_state)
+    print(f"deltanet decode x{T}: attn {e_attn:.3e} result {e_res:.3e} state {e_state:.3e}")
+    assert e_attn <= TOL and e_res <= TOL and e_state <= TOL
+    for t in range(T):
+        assert O.rel_l2(got_res[t], want_res[t]) <= TOL, t
+
+
+@pytest.mark.parametrize("B", [1, 8])
+def test_decode_step_with_random_state(ctx, B):
+    """BASELINE config 3, decode mode: batch 1 and 8 sequences, each with its own state ~N(0,0.1)
+    and its own three rows of conv history, at different positions."""
+    case = DnCase(ctx, seed=10 + B)
+    case.upload()
+    rng = case.rng
+    slots = 4
+    xn = rng.standard_normal((B, case.H)).astype(np.float32)
+    s0 = (rng.standard_normal((B, case.hv, case.d, case.d)) * 0.1).astype(np.float32)
+    hist = rng.standard_normal((B, 3, case.width)).astype(np.float32)  # rows at positions p-3..p-1
+    pos = (3 + 5 * np.arange(B)).astype(np.int32)
+    ring = np.zeros((B, slots, case.width), np.float32)
+    for b in range(B):
+        for i in range(3):
+            ring[b, (pos[b] - 3 + i) % slots] = hist[b, i]
+    c = ctx
+    d_ring, d_state = c.upload(ring), c.upload(s0)
+    d_attn, d_res = c.alloc(B * case.vw * 4), c.alloc(B * case.H * 4)
+    d_pos, d_x = c.upload(pos), c.upload(xn)
+    ops = case.step_ops(d_x, d_ring, d_state, d_attn, d_res, d_pos, None, B, 1, slots)[:2]
+    c.dispatch_multi(ops)
+    got_attn = d_attn.read(np.float32, B * case.vw).reshape(B, case.vw)
+    got_state = d_state.read(np.float32, s0.size).reshape(s0.shape)
+    for b in range(B):
+        conv_state = np.ascontiguousarray(hist[b, :, :case.cw].T)  # [cw][3], column 0 oldest
+        s_state = s0[b].copy()
+        _, want_attn = case.oracle(xn[b:b + 1], conv_state, s_state)
+        assert O.rel_l2(got_attn[b], want_attn[0]) <= TOL, b
+        assert O.rel_l2(got_state[b], s_state) <= TOL, b
+
+
+def test_three_rows_in_one_call_equal_three_calls(ctx):
+    """A multi-row pass over one sequence (the verify pass's shape) must walk the rows in order on
+    one state: same answer as three single steps."""
+    case = DnCase(ctx, seed=21)
+    case.upload()
+    T, slots = 3, 8
+    xn = case.rng.standard_normal((T, case.H)).astype(np.float32)
+    conv_state = np.zeros((case.cw, 3), np.float32)
+    s_state = np.zeros((case.hv, case.d, case.d), np.float32)
+    _, want_attn = case.oracle(xn, conv_state, s_state)
+    c = ctx
+    d_ring = c.alloc(slots * case.width * 4).zero()
+    d_state = c.alloc(s_state.nbytes).zero()
+    d_attn, d_res = c.alloc(T * case.vw * 4), c.alloc(T * case.H * 4)
+    ops = case.step_ops(c.upload(xn), d_ring, d_state, d_attn, d_res, c.upload(np.array([0], np.int32)),
+                        None, 1, T, slots)[:2]
+    c.dispatch_multi(ops)
+    assert O.rel_l2(d_attn.read(np.float32, T * case.vw).reshape(T, -1), want_attn) <= TOL
+    assert O.rel_l2(d_state.read(np.float32, s_state.size), s_state) <= TOL
+
+
+def test_dn_step_refuses_unsupported_shapes(ctx):
+    d = ctx.alloc(1 << 16)
+    with pytest.raises(shv.pkg.ShvError):
+        ctx.enqueue(A.OP_DN_STEP, A.DnStepArgs(d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 1,
+                                               16, 32, 64, 4, 4, 12352, EPS, 0))
+    with pytest.raises(shv.pkg.ShvError):
+        ctx.enqueue(A.OP_DN_STEP, A.DnStepArgs(d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, None, 1, 4,
+                                               16, 32, 128, 4, 4, 12352, EPS, 0))

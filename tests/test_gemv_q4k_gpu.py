@@ -53,7 +53,7 @@ def test_config1_exact_shape_and_seeded_inputs(ctx):
     assert O.rel_l2(dy3.read(np.float32, n), lin) <= 1e-5
 
 
-@pytest.mark.parametrize("n_tok", [2, 3, 4])
+@pytest.mark.parametrize("n_tok", [2, 3, 4, 8, 13])
 def test_gemv_rows_share_one_weight_pass(ctx, n_tok):
     rng = np.random.default_rng(7 + n_tok)
     n, k = 1024, 2048
@@ -119,7 +119,7 @@ def test_gemv_refuses_shapes_it_does_not_cover(ctx):
     with pytest.raises(shv.pkg.ShvError):
         ctx.gemv_q4k(d, d, d, 16, 768)
     with pytest.raises(shv.pkg.ShvError):
-        ctx.gemv_q4k(d, d, d, 16, 2048, n_tok=5)
+        ctx.gemv_q4k(d, d, d, 16, 2048, n_tok=65)
     with pytest.raises(shv.pkg.ShvError):
         ctx.gemv_q4k(d.at(4), d, d, 16, 2048)
 
