@@ -98,7 +98,8 @@ enum {
     SHV_PRO_RMSNORM = 1,     /* x * rsqrt(mean(x^2)+eps) * gamma            (llm/hc.go:176-190)       */
     SHV_PRO_GATED_NORM = 2,  /* per head of head_dim: rms * gamma[head_dim] * sigmoid(z)
                                                                             (llm/deltanet.go:329-341) */
-    SHV_PRO_MUL_SIGMOID = 3  /* x * sigmoid(z)                              (llm/attn.go:198-205)     */
+    SHV_PRO_MUL_SIGMOID = 3  /* x * sigmoid(z); with head_dim > 0, z holds [q | gate] per head and
+                                the gate half is read                      (llm/attn.go:162-166,198-205) */
 };
 
 /* y[t][r] = sum_i W[r][i] * pro(x[t])[i] (+ residual[t][r]); W is GGUF Q4_K, row-major, k%256==0.
@@ -225,6 +226,35 @@ typedef struct {
     int32_t qk_norm_max;
 } shv_dn_step_args;
 
+/* Gated full-attention decode over an fp16 KV cache (AttnLayerAt, llm/attn.go:162-205, and
+ * attention :444-496; shaders llm_attn_pack.comp + llm_attn_wmma.comp -DSPLITK +
+ * llm_attn_combine.comp).  Input is the fused projection row
+ *   [ per head: q (d) | gate (d) ] x n_head, then k (n_head_kv*d), then v (n_head_kv*d).
+ * For each of n_seq sequences, seq_len consecutive rows at positions pos[s]+i on cache slot
+ * slot[s] (s itself when NULL): per-head RMS norm of q and k with one gamma each, NeoX rotary on
+ * the first rope_dims dims from the host-built table (row p: cos[rope_dims/2] then
+ * sin[rope_dims/2]; llm/gpu_attn.go:1452-1476), K and V rounded to binary16 into cell p of the
+ * cache, then causal GQA softmax attention of the row over cells 0..p, split n_splits ways over
+ * the cells and merged.  out is [rows][n_head*d] BEFORE the sigmoid gate, which the output
+ * projection applies as its prologue.  kcache / vcache are [n_slots][max_cells][n_head_kv][d]
+ * binary16; partial is scratch of n_seq*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2) floats. */
+typedef struct {
+    const float *qkv;
+    const float *q_norm;
+    const float *k_norm;
+    const float *rope;
+    void *kcache;
+    void *vcache;
+    float *partial;
+    float *out;
+    const int32_t *pos;
+    const int32_t *slot;
+    int32_t n_seq, seq_len;
+    int32_t n_head, n_head_kv, head_dim, rope_dims;
+    int32_t max_cells, qkv_stride, n_splits;
+    float eps;
+} shv_attn_decode_args;
+
 typedef struct {
     uint32_t kind;
     uint32_t flags;          /* bit 0: may overlap the previous op (MultiDispatch.Overlap) */
@@ -259,6 +289,7 @@ int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
 int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
+int shv_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
 
 #ifdef __cplusplus
 }

@@ -117,7 +117,10 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 #pragma unroll
             for (int i = 0; i < K / kBlock; i++) {
                 const int c = tid + i * kBlock;
-                xs[t][lds_slot(c)] = x[c] * (1.f / (1.f + expf(-z[c])));
+                // head_dim > 0: z rows are [q (head_dim) | gate (head_dim)] per head and the gate
+                // half is the one wanted (the fused query projection, llm/attn.go:162-166)
+                const int zi = a.head_dim > 0 ? (c / a.head_dim) * 2 * a.head_dim + a.head_dim + c % a.head_dim : c;
+                xs[t][lds_slot(c)] = x[c] * (1.f / (1.f + expf(-z[zi])));
             }
         } else {
 #pragma unroll

@@ -176,6 +176,7 @@ static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t by
         case SHV_OP_MOE_UP: return run_as<shv_moe_up_args>(ctx, args, bytes, shv_launch_moe_up, "moe_up");
         case SHV_OP_MOE_DOWN: return run_as<shv_moe_down_args>(ctx, args, bytes, shv_launch_moe_down, "moe_down");
         case SHV_OP_DN_STEP: return run_as<shv_dn_step_args>(ctx, args, bytes, shv_launch_dn_step, "dn_step");
+        case SHV_OP_ATTN_DECODE: return run_as<shv_attn_decode_args>(ctx, args, bytes, shv_launch_attn_decode, "attn_decode");
         default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
     }
 }
@@ -308,5 +309,6 @@ int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a) { return dispatch
 int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a) { return dispatch_one(ctx, SHV_OP_MOE_UP, a, sizeof(*a)); }
 int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a) { return dispatch_one(ctx, SHV_OP_MOE_DOWN, a, sizeof(*a)); }
 int shv_dn_step(shv_ctx *ctx, const shv_dn_step_args *a) { return dispatch_one(ctx, SHV_OP_DN_STEP, a, sizeof(*a)); }
+int shv_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a) { return dispatch_one(ctx, SHV_OP_ATTN_DECODE, a, sizeof(*a)); }
 
 }  // extern "C"

@@ -54,3 +54,4 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
 int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
+int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);

@@ -84,6 +84,16 @@ class DnStepArgs(C.Structure):
                 ("ring_stride", C.c_int32), ("eps", C.c_float), ("qk_norm_max", C.c_int32)]
 
 
+class AttnDecodeArgs(C.Structure):
+    _fields_ = [("qkv", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
+                ("rope", C.c_void_p), ("kcache", C.c_void_p), ("vcache", C.c_void_p),
+                ("partial", C.c_void_p), ("out", C.c_void_p), ("pos", C.c_void_p),
+                ("slot", C.c_void_p), ("n_seq", C.c_int32), ("seq_len", C.c_int32),
+                ("n_head", C.c_int32), ("n_head_kv", C.c_int32), ("head_dim", C.c_int32),
+                ("rope_dims", C.c_int32), ("max_cells", C.c_int32), ("qkv_stride", C.c_int32),
+                ("n_splits", C.c_int32), ("eps", C.c_float)]
+
+
 class Op(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("flags", C.c_uint32), ("args", C.c_uint8 * 248)]
 
@@ -104,7 +114,7 @@ SYMBOLS = [
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_quantize_q4k",
-    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step",
+    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode",
 ]
 
 _lib = None
@@ -153,6 +163,7 @@ def load():
     L.shv_moe_up.argtypes = [vp, C.POINTER(MoeUpArgs)]
     L.shv_moe_down.argtypes = [vp, C.POINTER(MoeDownArgs)]
     L.shv_dn_step.argtypes = [vp, C.POINTER(DnStepArgs)]
+    L.shv_attn_decode.argtypes = [vp, C.POINTER(AttnDecodeArgs)]
     _lib = L
     return L
 
