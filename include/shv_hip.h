@@ -87,8 +87,7 @@ enum {
     SHV_OP_ATTN_DECODE = 9,
     SHV_OP_EMBED = 10,
     SHV_OP_ARGMAX = 11,
-    SHV_OP_RMSNORM = 12,
-    SHV_OP_COPY_F32 = 13,
+    SHV_OP_ADVANCE = 12,
     SHV_OP__COUNT
 };
 
@@ -109,7 +108,9 @@ enum {
  * of n_tok).  ring_slots>0 selects ring output, the DeltaNet projection ring of
  * shaders/llm_dn_conv.comp:36-49 and llm_seq_hist.comp:17-26: row i of sequence s is written at
  * y + (slot[s]*ring_slots + (pos[s]+i) % ring_slots) * ring_stride, slot[s] = s when slot is NULL,
- * instead of y + t*y_stride. */
+ * instead of y + t*y_stride.  z_ring != 0 reads the prologue's z row from the same ring
+ * geometry instead (z + (slot*ring_slots + (pos+i) % ring_slots) * ring_stride) and leaves y
+ * plain: the DeltaNet output projection takes its gate z from the projection ring. */
 typedef struct {
     const void *w;
     const float *x;
@@ -125,6 +126,7 @@ typedef struct {
     float eps;
     int32_t x_stride, y_stride, z_stride;
     int32_t seq_len, ring_slots, ring_stride;
+    int32_t z_ring;
 } shv_gemv_q4k_args;
 
 /* dst[i] = d*sc*q - dmin*m for every weight of `rows` rows, the reference's dequantQ4_K
@@ -255,6 +257,35 @@ typedef struct {
     float eps;
 } shv_attn_decode_args;
 
+/* Token embedding gather (Model.Embeddings, llm/model.go:134; hc.UploadInit, llm/graph.go:1815):
+ * x[t] = float32(table[id_t]) for n_tok rows, id_t = ids[pos[0]+t] when pos is given, else ids[t].
+ * table is binary16 [vocab][n_embd].  An id outside [0, vocab) yields a row of NaN. */
+typedef struct {
+    const void *table;
+    const int32_t *ids;
+    const int32_t *pos;
+    float *x;
+    int32_t n_tok, n_embd, vocab, x_stride;
+} shv_embed_args;
+
+/* Greedy sampler (Argmax, llm/sample.go:359-367): the index of the first maximum of each row of
+ * logits [n_rows][n]; NaN never wins.  best[r] receives the index.  When ids and pos are given
+ * (n_rows must be 1) the index is also stored as the next token, ids[pos[0]+1], and pos[0] is
+ * advanced by one, so a recorded decode step can be replayed back to back without the host. */
+typedef struct {
+    const float *logits;
+    int32_t *best;
+    int32_t *ids;
+    int32_t *pos;
+    int32_t n_rows, n, logits_stride;
+} shv_argmax_args;
+
+/* pos[s] += delta for s < n_seq: the step of a recorded pass that does not sample. */
+typedef struct {
+    int32_t *pos;
+    int32_t n_seq, delta;
+} shv_advance_args;
+
 typedef struct {
     uint32_t kind;
     uint32_t flags;          /* bit 0: may overlap the previous op (MultiDispatch.Overlap) */
@@ -290,6 +321,9 @@ int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
 int shv_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
+int shv_embed(shv_ctx *ctx, const shv_embed_args *a);
+int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a);
+int shv_advance(shv_ctx *ctx, const shv_advance_args *a);
 
 #ifdef __cplusplus
 }

@@ -96,6 +96,13 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
             // head_dim/(K/256) consecutive threads (a power of two <= 64).
             constexpr int PER = K / kBlock;
             const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
+            if (a.z_ring) {
+                const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+                const int s = (t0 + t) / sl, i = (t0 + t) % sl;
+                const int p = a.pos ? a.pos[s] : 0;
+                const int slot = a.slot ? a.slot[s] : s;
+                z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
+            }
             float v[PER];
             float ss = 0.f;
 #pragma unroll
@@ -148,7 +155,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     size_t y_off[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        if (a.ring_slots > 0) {
+        if (a.ring_slots > 0 && !a.z_ring) {
             const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
             const int s = (t0 + t) / sl, i = (t0 + t) % sl;
             const int p = a.pos ? a.pos[s] : 0;
@@ -254,9 +261,10 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
                     "gemv_q4k: gated-norm head_dim %d does not tile k %d", a.head_dim, a.k);
     }
     if (a.prologue == SHV_PRO_MUL_SIGMOID) SHV_REQUIRE(a.z, "gemv_q4k: sigmoid-gate prologue without z");
+    if (a.z_ring) SHV_REQUIRE(a.prologue == SHV_PRO_GATED_NORM && a.ring_slots > 0, "gemv_q4k: z_ring needs the gated-norm prologue and a ring");
     if (a.ring_slots > 0) {
         const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
-        SHV_REQUIRE(a.ring_stride >= a.n && sl <= a.ring_slots && a.n_tok % sl == 0 && !a.residual,
+        SHV_REQUIRE((a.z_ring || (a.ring_stride >= a.n && !a.residual)) && sl <= a.ring_slots && a.n_tok % sl == 0,
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
     switch (a.k) {

@@ -79,3 +79,127 @@ int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a) {
     SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
+
+// ---- token-loop glue: embedding gather, greedy arg-max, position advance ------------------------
+
+namespace {
+
+__global__ __launch_bounds__(256) void embed_kernel(shv_embed_args a) {
+    const int t = blockIdx.y;
+    const int id = a.ids[(a.pos ? a.pos[0] : 0) + t];
+    const bool ok = id >= 0 && id < a.vocab;
+    const uint16_t *row = static_cast<const uint16_t *>(a.table) + static_cast<size_t>(ok ? id : 0) * a.n_embd;
+    float *x = a.x + static_cast<size_t>(t) * a.x_stride;
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < a.n_embd; c += gridDim.x * blockDim.x)
+        x[c] = ok ? __half2float(__ushort_as_half(row[c])) : __int_as_float(0x7fc00000);
+}
+
+// (value, index) ordered so that the larger value wins and, between equal values, the lower index.
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+__device__ __forceinline__ void wave_best(float &v, int &i) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(v, off, 64);
+        const int oi = __shfl_xor(i, off, 64);
+        if (better(ov, oi, v, i)) { v = ov; i = oi; }
+    }
+}
+
+// grid: (blocks, n_rows).  Each block scans a contiguous chunk of one row; the last block of the
+// row to arrive reduces the per-block winners.
+__global__ __launch_bounds__(256) void argmax_kernel(shv_argmax_args a, float *pval, int32_t *pidx, int32_t *counters) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    __shared__ int is_last;
+    const int r = blockIdx.y, nb = gridDim.x;
+    const float *lg = a.logits + static_cast<size_t>(r) * a.logits_stride;
+    const int chunk = (a.n + nb - 1) / nb;
+    const int lo = blockIdx.x * chunk, hi = lo + chunk < a.n ? lo + chunk : a.n;
+    // "no candidate" is (-inf, n): any real element beats it, including -inf at a lower index
+    float bv = -INFINITY;
+    int bi = a.n;
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        const float v = lg[i];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+    wave_best(bv, bi);
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++)
+            if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+        pval[r * nb + blockIdx.x] = bv;
+        pidx[r * nb + blockIdx.x] = bi;
+        __threadfence();
+        const int prev = __hip_atomic_fetch_add(counters + r, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = prev == nb - 1;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    bv = -INFINITY;
+    bi = a.n;
+    for (int b = threadIdx.x; b < nb; b += blockDim.x) {
+        const float v = pval[r * nb + b];
+        const int i = pidx[r * nb + b];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+    wave_best(bv, bi);
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++)
+            if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+        // a row of NaN (or -inf only at the top) has no element that is `>` -inf: the reference
+        // returns 0 there
+        if (bi >= a.n) bi = 0;
+        a.best[r] = bi;
+        if (a.ids && a.pos) {
+            const int p = a.pos[0];
+            a.ids[p + 1] = bi;
+            a.pos[0] = p + 1;
+        }
+        __hip_atomic_store(counters + r, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+__global__ void advance_kernel(shv_advance_args a) {
+    const int s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s < a.n_seq) a.pos[s] += a.delta;
+}
+
+}  // namespace
+
+int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a) {
+    SHV_REQUIRE(a->table && a->ids && a->x, "embed: NULL argument");
+    SHV_REQUIRE(a->n_tok >= 1 && a->n_tok <= 65535 && a->n_embd >= 1 && a->vocab >= 1 && a->x_stride >= a->n_embd,
+                "embed: n_tok %d, n_embd %d, vocab %d, x_stride %d", a->n_tok, a->n_embd, a->vocab, a->x_stride);
+    const int bx = (a->n_embd + 255) / 256;
+    hipLaunchKernelGGL(embed_kernel, dim3(bx < 8 ? bx : 8, a->n_tok), dim3(256), 0, ctx->stream, *a);
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}
+
+int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a) {
+    SHV_REQUIRE(a->logits && a->best, "argmax: NULL logits or best");
+    SHV_REQUIRE(a->n_rows >= 1 && a->n >= 1 && a->logits_stride >= a->n, "argmax: %d rows of %d, stride %d", a->n_rows, a->n, a->logits_stride);
+    SHV_REQUIRE((a->ids == nullptr) == (a->pos == nullptr), "argmax: ids and pos go together");
+    SHV_REQUIRE(!a->ids || a->n_rows == 1, "argmax: storing the next token needs exactly one row");
+    int nb = (a->n + 1023) / 1024;
+    const int cap = shv_ctx::kArgmaxBlocks / a->n_rows;
+    SHV_REQUIRE(cap >= 1 && a->n_rows <= 14, "argmax: %d rows is more than one launch covers", a->n_rows);
+    if (nb > cap) nb = cap;
+    if (nb > 256) nb = 256;
+    hipLaunchKernelGGL(argmax_kernel, dim3(nb, a->n_rows), dim3(256), 0, ctx->stream, *a, ctx->argmax_val, ctx->argmax_idx,
+                       ctx->counters + shv_ctx::kCounterArgmax);
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}
+
+int shv_launch_advance(shv_ctx *ctx, const shv_advance_args *a) {
+    SHV_REQUIRE(a->pos && a->n_seq >= 1, "advance: NULL pos or n_seq %d", a->n_seq);
+    hipLaunchKernelGGL(advance_kernel, dim3((a->n_seq + 63) / 64), dim3(64), 0, ctx->stream, *a);
+    SHV_HIP_CHECK(hipGetLastError());
+    return SHV_OK;
+}

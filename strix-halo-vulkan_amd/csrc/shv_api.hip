@@ -44,6 +44,8 @@ int shv_init(int device, shv_ctx **out) {
     ctx->n_counters = 4096;
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->counters), ctx->n_counters * sizeof(int32_t));
     if (e == hipSuccess) e = hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_val), shv_ctx::kArgmaxBlocks * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_idx), shv_ctx::kArgmaxBlocks * sizeof(int32_t));
     if (e != hipSuccess) {
         shv_destroy(ctx);
         return shv_set_error(SHV_E_HIP, "shv_init: %s", hipGetErrorString(e));
@@ -63,6 +65,8 @@ void shv_destroy(shv_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->argmax_val) (void)hipFree(ctx->argmax_val);
+    if (ctx->argmax_idx) (void)hipFree(ctx->argmax_idx);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -177,6 +181,9 @@ static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t by
         case SHV_OP_MOE_DOWN: return run_as<shv_moe_down_args>(ctx, args, bytes, shv_launch_moe_down, "moe_down");
         case SHV_OP_DN_STEP: return run_as<shv_dn_step_args>(ctx, args, bytes, shv_launch_dn_step, "dn_step");
         case SHV_OP_ATTN_DECODE: return run_as<shv_attn_decode_args>(ctx, args, bytes, shv_launch_attn_decode, "attn_decode");
+        case SHV_OP_EMBED: return run_as<shv_embed_args>(ctx, args, bytes, shv_launch_embed, "embed");
+        case SHV_OP_ARGMAX: return run_as<shv_argmax_args>(ctx, args, bytes, shv_launch_argmax, "argmax");
+        case SHV_OP_ADVANCE: return run_as<shv_advance_args>(ctx, args, bytes, shv_launch_advance, "advance");
         default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
     }
 }
@@ -310,5 +317,8 @@ int shv_moe_up(shv_ctx *ctx, const shv_moe_up_args *a) { return dispatch_one(ctx
 int shv_moe_down(shv_ctx *ctx, const shv_moe_down_args *a) { return dispatch_one(ctx, SHV_OP_MOE_DOWN, a, sizeof(*a)); }
 int shv_dn_step(shv_ctx *ctx, const shv_dn_step_args *a) { return dispatch_one(ctx, SHV_OP_DN_STEP, a, sizeof(*a)); }
 int shv_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a) { return dispatch_one(ctx, SHV_OP_ATTN_DECODE, a, sizeof(*a)); }
+int shv_embed(shv_ctx *ctx, const shv_embed_args *a) { return dispatch_one(ctx, SHV_OP_EMBED, a, sizeof(*a)); }
+int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a) { return dispatch_one(ctx, SHV_OP_ARGMAX, a, sizeof(*a)); }
+int shv_advance(shv_ctx *ctx, const shv_advance_args *a) { return dispatch_one(ctx, SHV_OP_ADVANCE, a, sizeof(*a)); }
 
 }  // extern "C"

@@ -19,6 +19,10 @@ struct shv_ctx {
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
     int32_t *counters = nullptr;
     int n_counters = 0;
+    // per-block partial results of the arg-max reduction: (value, index) pairs
+    float *argmax_val = nullptr;
+    int32_t *argmax_idx = nullptr;
+    enum { kArgmaxBlocks = 512 };
     enum { kCounterRouter = 0, kCounterArgmax = 1, kCounterAttn = 16 };
 };
 
@@ -55,3 +59,6 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
 int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
+int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a);
+int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a);
+int shv_launch_advance(shv_ctx *ctx, const shv_advance_args *a);

@@ -10,7 +10,7 @@ Q4K_BYTES = 144
 
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
-OP_EMBED, OP_ARGMAX, OP_RMSNORM, OP_COPY_F32 = 10, 11, 12, 13
+OP_EMBED, OP_ARGMAX, OP_ADVANCE = 10, 11, 12
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID = 0, 1, 2, 3
 
 
@@ -36,7 +36,7 @@ class GemvQ4KArgs(C.Structure):
                 ("n", C.c_int32), ("k", C.c_int32), ("n_tok", C.c_int32), ("prologue", C.c_int32),
                 ("head_dim", C.c_int32), ("eps", C.c_float), ("x_stride", C.c_int32),
                 ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("seq_len", C.c_int32),
-                ("ring_slots", C.c_int32), ("ring_stride", C.c_int32)]
+                ("ring_slots", C.c_int32), ("ring_stride", C.c_int32), ("z_ring", C.c_int32)]
 
 
 class DequantQ4KArgs(C.Structure):
@@ -94,6 +94,22 @@ class AttnDecodeArgs(C.Structure):
                 ("n_splits", C.c_int32), ("eps", C.c_float)]
 
 
+class EmbedArgs(C.Structure):
+    _fields_ = [("table", C.c_void_p), ("ids", C.c_void_p), ("pos", C.c_void_p), ("x", C.c_void_p),
+                ("n_tok", C.c_int32), ("n_embd", C.c_int32), ("vocab", C.c_int32),
+                ("x_stride", C.c_int32)]
+
+
+class ArgmaxArgs(C.Structure):
+    _fields_ = [("logits", C.c_void_p), ("best", C.c_void_p), ("ids", C.c_void_p),
+                ("pos", C.c_void_p), ("n_rows", C.c_int32), ("n", C.c_int32),
+                ("logits_stride", C.c_int32)]
+
+
+class AdvanceArgs(C.Structure):
+    _fields_ = [("pos", C.c_void_p), ("n_seq", C.c_int32), ("delta", C.c_int32)]
+
+
 class Op(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("flags", C.c_uint32), ("args", C.c_uint8 * 248)]
 
@@ -114,7 +130,7 @@ SYMBOLS = [
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_quantize_q4k",
-    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode",
+    "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
 ]
 
 _lib = None
@@ -164,6 +180,9 @@ def load():
     L.shv_moe_down.argtypes = [vp, C.POINTER(MoeDownArgs)]
     L.shv_dn_step.argtypes = [vp, C.POINTER(DnStepArgs)]
     L.shv_attn_decode.argtypes = [vp, C.POINTER(AttnDecodeArgs)]
+    L.shv_embed.argtypes = [vp, C.POINTER(EmbedArgs)]
+    L.shv_argmax.argtypes = [vp, C.POINTER(ArgmaxArgs)]
+    L.shv_advance.argtypes = [vp, C.POINTER(AdvanceArgs)]
     _lib = L
     return L
 
@@ -285,9 +304,9 @@ class Context:
     # ---- convenience wrappers over single ops ----
     def gemv_q4k(self, w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None,
                  eps=1e-6, head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None,
-                 ring_slots=0, ring_stride=0, slot=None, seq_len=0):
+                 ring_slots=0, ring_stride=0, slot=None, seq_len=0, z_ring=0):
         a = gemv_args(w, x, y, n, k, n_tok, prologue, gamma, z, residual, eps, head_dim, x_stride,
-                      y_stride, z_stride, pos, ring_slots, ring_stride, slot, seq_len)
+                      y_stride, z_stride, pos, ring_slots, ring_stride, slot, seq_len, z_ring)
         check(self.L.shv_gemv_q4k(self.h, C.byref(a)))
 
 
@@ -304,7 +323,7 @@ def _ptr(b):
 
 def gemv_args(w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None, eps=1e-6,
               head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None, ring_slots=0,
-              ring_stride=0, slot=None, seq_len=0):
+              ring_stride=0, slot=None, seq_len=0, z_ring=0):
     a = GemvQ4KArgs()
     a.w, a.x, a.y = _ptr(w), _ptr(x), _ptr(y)
     a.residual, a.gamma, a.z, a.pos = _ptr(residual), _ptr(gamma), _ptr(z), _ptr(pos)
@@ -313,4 +332,5 @@ def gemv_args(w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, res
     a.y_stride = n if y_stride is None else y_stride
     a.z_stride = k if z_stride is None else z_stride
     a.ring_slots, a.ring_stride, a.slot, a.seq_len = ring_slots, ring_stride, _ptr(slot), seq_len
+    a.z_ring = z_ring
     return a

@@ -1,0 +1,69 @@
+"""Token-loop glue ops: embedding gather, greedy arg-max (llm/sample.go:359-367), advance."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import shv
+
+pytestmark = pytest.mark.gpu
+A = shv.api
+
+
+def _argmax(ctx, logits):
+    logits = np.ascontiguousarray(logits, np.float32)
+    rows, n = logits.shape
+    best = ctx.alloc(rows * 4)
+    ctx.enqueue(A.OP_ARGMAX, A.ArgmaxArgs(ctx.upload(logits).ptr, best.ptr, None, None, rows, n, n))
+    return best.read(np.int32, rows)
+
+
+def test_argmax_first_maximum_wins(ctx):
+    rng = np.random.default_rng(1)
+    L = O.lib()
+    for n in (1, 7, 1000, 151936):
+        x = rng.standard_normal((3, n)).astype(np.float32)
+        want = [L.shv_ref_argmax(O.F(np.ascontiguousarray(r)), n) for r in x]
+        assert list(_argmax(ctx, x)) == want == list(np.argmax(x, axis=1))
+    # ties go to the lowest id (llm/sample_test.go:17), wherever the block boundaries fall
+    x = np.zeros((1, 151936), np.float32)
+    x[0, [5, 700, 1024, 151935]] = 3.0
+    assert _argmax(ctx, x)[0] == 5
+    x[0, 5] = 0.0
+    assert _argmax(ctx, x)[0] == 700
+    # NaN never wins; a row with nothing above -inf returns 0
+    x = np.full((2, 4096), -np.inf, np.float32)
+    x[0, 100] = np.nan
+    x[0, 200] = -1e30
+    assert list(_argmax(ctx, x)) == [200, 0]
+    assert _argmax(ctx, np.full((1, 300), np.nan, np.float32))[0] == 0
+
+
+def test_argmax_feeds_the_next_step(ctx):
+    logits = np.zeros((1, 5000), np.float32)
+    logits[0, 4321] = 1.0
+    ids = ctx.upload(np.array([11, 22, 33, -1, -1], np.int32))
+    pos = ctx.upload(np.array([2], np.int32))
+    best = ctx.alloc(4)
+    ctx.enqueue(A.OP_ARGMAX, A.ArgmaxArgs(ctx.upload(logits).ptr, best.ptr, ids.ptr, pos.ptr, 1, 5000, 5000))
+    assert best.read(np.int32, 1)[0] == 4321
+    assert list(ids.read(np.int32, 5)) == [11, 22, 33, 4321, -1]
+    assert pos.read(np.int32, 1)[0] == 3
+    ctx.enqueue(A.OP_ADVANCE, A.AdvanceArgs(pos.ptr, 1, 4))
+    assert pos.read(np.int32, 1)[0] == 7
+
+
+def test_embedding_gather(ctx):
+    rng = np.random.default_rng(2)
+    vocab, H = 1000, 2048
+    table = rng.standard_normal((vocab, H)).astype(np.float16)
+    ids = np.array([3, 999, 0, 17, 5000], np.int32)
+    d_x = ctx.alloc(4 * H * 4)
+    d_t, d_ids = ctx.upload(table), ctx.upload(ids)
+    ctx.enqueue(A.OP_EMBED, A.EmbedArgs(d_t.ptr, d_ids.ptr, None, d_x.ptr, 4, H, vocab, H))
+    got = d_x.read(np.float32, 4 * H).reshape(4, H)
+    assert np.array_equal(got, table[ids[:4]].astype(np.float32))
+    # position-relative read, and an id outside the vocabulary is NaN rather than a wild read
+    ctx.enqueue(A.OP_EMBED, A.EmbedArgs(d_t.ptr, d_ids.ptr, ctx.upload(np.array([3], np.int32)).ptr, d_x.ptr,
+                                        2, H, vocab, H))
+    got = d_x.read(np.float32, 2 * H).reshape(2, H)
+    assert np.array_equal(got[0], table[17].astype(np.float32)) and np.isnan(got[1]).all()
