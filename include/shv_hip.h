@@ -147,12 +147,14 @@ typedef struct {
     int32_t k;
 } shv_quantize_q4k_args;
 
-/* dst[i] = mean + std * N(0,1), counter-based (seed, i): synthetic weights made in HBM. */
+/* dst[i] = mean + std * N(0,1), counter-based (seed, i): synthetic weights made in HBM.
+ * half != 0 stores binary16 (round to nearest even) instead of float32. */
 typedef struct {
-    float *dst;
+    void *dst;
     int64_t n;
     uint64_t seed;
     float mean, std;
+    int32_t half;
 } shv_fill_normal_args;
 
 /* MoE router (MoETrace.Route, llm/moe.go:219-274; shaders llm_moe_router/route.comp): per token

@@ -761,3 +761,37 @@ void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, cons
         shv_ref_gemv_q4k(out + (size_t)i * H, w->o, pre + (size_t)i * gw, H, gw, threads);
     free(pre); free(pos); free(V); free(K); free(G); free(Q); free(qfull);
 }
+
+/* ------------------------------------------------------------- token loop --- */
+
+void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
+                          const int32_t *ids, int n_tok, float *logits, float *hidden, int threads) {
+    int H = c->n_embd;
+    size_t T = (size_t)n_tok;
+    float *x = (float *)malloc(sizeof(float) * T * H);
+    float *xn = (float *)malloc(sizeof(float) * T * H);
+    float *y = (float *)malloc(sizeof(float) * T * H);
+    for (int t = 0; t < n_tok; t++)
+        for (int i = 0; i < H; i++) x[(size_t)t * H + i] = shv_ref_f16_to_f32(w->embd[(size_t)ids[t] * H + i]);
+    for (int l = 0; l < c->n_layer; l++) {
+        const shv_ref_layer_w *lw = &w->layers[l];
+        for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->attn_norm, H, c->eps);
+        if ((l + 1) % c->attn_every == 0)
+            shv_ref_attn_layer(&c->attn, &lw->attn, xn, n_tok, st->past, st->kcache[l], st->vcache[l], y, NULL, NULL, threads);
+        else
+            shv_ref_deltanet_layer(&c->dn, &lw->dn, xn, n_tok, st->dn_conv[l], st->dn_s[l], y, NULL, NULL, NULL,
+                                   NULL, NULL, NULL, NULL, 0, threads);
+        for (size_t i = 0; i < T * H; i++) x[i] += y[i];
+        for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->ffn_norm, H, c->eps);
+        shv_ref_moe_block(&c->moe, &lw->moe, xn, n_tok, y, NULL, NULL, NULL, NULL, NULL, NULL, threads);
+        for (size_t i = 0; i < T * H; i++) x[i] += y[i];
+    }
+    st->past += n_tok;
+    const float *last = x + (T - 1) * H;
+    if (hidden) memcpy(hidden, last, sizeof(float) * H);
+    if (logits) {
+        shv_ref_rmsnorm(xn, last, w->out_norm, H, c->eps);
+        shv_ref_gemv_q4k(logits, w->lm_head, xn, c->vocab, H, threads);
+    }
+    free(y); free(xn); free(x);
+}

@@ -159,6 +159,56 @@ void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, cons
                         int n_tok, int past, uint16_t *kcache, uint16_t *vcache, float *out,
                         float *q_rot, float *pregate, int threads);
 
+/* ---- the token loop over the synthetic Qwen3-Next-shape model ----
+ * The reference's loop body is llm/graph.go:2330-2466 (per layer: mix -> DeltaNet or attention ->
+ * combine -> mix -> MoE -> combine; then the head, :1762) and its driver cmd/llm/generate.go:121-165
+ * (prefill, Argmax, extend).  BASELINE's model has no hyper-connection streams, so "mix" is a plain
+ * RMSNorm (llm/hc.go:176-190 with hc=1) and "combine" a residual add:
+ *     x = float32(embd[id])
+ *     x += Block_l(RMSNorm(x, attn_norm_l))     Block = DeltaNet, or attention on every attn_every-th layer
+ *     x += MoE_l(RMSNorm(x, ffn_norm_l))
+ *     logits = lm_head * RMSNorm(x, out_norm)
+ * The composition is this repository's reading of that shape: "parity unpinned" against any
+ * reference-held vector, like the blocks it is made of. */
+typedef struct {
+    int n_layer, n_embd, vocab;
+    int attn_every;      /* layer l is full attention when (l+1) % attn_every == 0 */
+    float eps;
+    int max_cells;       /* KV cache capacity per attention layer */
+    shv_ref_moe_cfg moe;
+    shv_ref_dn_cfg dn;
+    shv_ref_attn_cfg attn;
+} shv_ref_model_cfg;
+
+typedef struct {
+    const float *attn_norm;  /* [n_embd] */
+    const float *ffn_norm;   /* [n_embd] */
+    shv_ref_dn_w dn;         /* used on DeltaNet layers   */
+    shv_ref_attn_w attn;     /* used on attention layers  */
+    shv_ref_moe_w moe;
+} shv_ref_layer_w;
+
+typedef struct {
+    const uint16_t *embd;    /* binary16 [vocab][n_embd] */
+    const float *out_norm;   /* [n_embd] */
+    const uint8_t *lm_head;  /* Q4_K [vocab][n_embd] */
+    const shv_ref_layer_w *layers;
+} shv_ref_model_w;
+
+/* Per-layer state; entries of the other kind of layer are NULL. */
+typedef struct {
+    float **dn_conv;      /* [n_layer] -> [conv_width][conv-1] */
+    float **dn_s;         /* [n_layer] -> [hv][d][d] */
+    uint16_t **kcache;    /* [n_layer] -> [max_cells][n_head_kv][head_dim] */
+    uint16_t **vcache;
+    int past;             /* tokens already in the sequence */
+} shv_ref_model_state;
+
+/* Extend the sequence by n_tok tokens (Graph.Extend, llm/graph.go:1709-1777): logits [vocab] and
+ * hidden [n_embd] (the residual stream before the final norm) of the LAST row; either may be NULL. */
+void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
+                          const int32_t *ids, int n_tok, float *logits, float *hidden, int threads);
+
 #ifdef __cplusplus
 }
 #endif

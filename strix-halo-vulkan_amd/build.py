@@ -18,6 +18,9 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libshv_hip.so")
+HOST = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(HERE, "libshv_llm.so")
+CXX = os.environ.get("CXX", "g++")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
@@ -69,7 +72,24 @@ def build(jobs=8, force=False):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr))
+    build_host(force)
     return LIB
+
+
+def build_host(force=False):
+    """The C++ host layer (host/*.cpp) above the C ABI: plain g++, linked against libshv_hip.so."""
+    srcs = sorted(os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".cpp"))
+    deps = srcs + [os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith((".hpp", ".h"))]
+    deps += [os.path.join(ROOT, "include", "shv_hip.h"), LIB]
+    if force or _stale(HOST_LIB, deps):
+        cmd = [CXX, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"),
+               "-I" + HOST, "-o", HOST_LIB] + srcs + ["-L" + HERE, "-lshv_hip", "-Wl,-rpath,$ORIGIN"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host build failed:\n%s\n%s" % (" ".join(cmd), r.stderr))
+        if r.stderr.strip():
+            sys.stderr.write(r.stderr)
+    return HOST_LIB
 
 
 if __name__ == "__main__":

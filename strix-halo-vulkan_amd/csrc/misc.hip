@@ -43,14 +43,17 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
 }
 
 // dst[i] = mean + std * z_i, z_i from Box-Muller on the two halves of splitmix64(seed, i).
-__global__ __launch_bounds__(256) void fill_normal_kernel(float *dst, long long n, uint64_t seed, float mean, float std) {
+__global__ __launch_bounds__(256) void fill_normal_kernel(void *dstv, long long n, uint64_t seed, float mean, float std, int half) {
+    float *dst = static_cast<float *>(dstv);
+    uint16_t *dsth = static_cast<uint16_t *>(dstv);
     const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
     for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
         const uint64_t r = splitmix64(seed * 0xD1342543DE82EF95ull + static_cast<uint64_t>(i));
         const float u1 = (static_cast<float>(static_cast<uint32_t>(r >> 40)) + 1.0f) * (1.0f / 16777216.0f);
         const float u2 = static_cast<float>(static_cast<uint32_t>(r) >> 8) * (1.0f / 16777216.0f);
         const float rad = sqrtf(-2.0f * logf(u1));
-        dst[i] = mean + std * rad * cosf(6.28318530717958647692f * u2);
+        const float v = mean + std * rad * cosf(6.28318530717958647692f * u2);
+        if (half) dsth[i] = __half_as_ushort(__float2half_rn(v)); else dst[i] = v;
     }
 }
 
@@ -75,7 +78,7 @@ int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a) {
     const long long cap = static_cast<long long>(ctx->prop.multiProcessorCount) * 32;
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL(fill_normal_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx->stream, a->dst,
-                       static_cast<long long>(a->n), a->seed, a->mean, a->std);
+                       static_cast<long long>(a->n), a->seed, a->mean, a->std, a->half);
     SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }

@@ -49,7 +49,7 @@ class QuantizeQ4KArgs(C.Structure):
 
 class FillNormalArgs(C.Structure):
     _fields_ = [("dst", C.c_void_p), ("n", C.c_int64), ("seed", C.c_uint64), ("mean", C.c_float),
-                ("std", C.c_float)]
+                ("std", C.c_float), ("half", C.c_int32)]
 
 
 class MoeRouterArgs(C.Structure):

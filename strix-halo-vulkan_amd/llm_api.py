@@ -1,0 +1,184 @@
+"""ctypes binding of host/shv_llm.h: the C++ host layer (llm::Graph and its blocks) for the tests
+and the benchmark.  No arithmetic lives here."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import hip_api
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+class Config(C.Structure):
+    """shvllm_config; defaults are the synthetic Qwen3-Next-shape model."""
+    _fields_ = [("n_layer", C.c_int32), ("n_embd", C.c_int32), ("n_head", C.c_int32),
+                ("n_head_kv", C.c_int32), ("head_dim", C.c_int32), ("rope_dims", C.c_int32),
+                ("rope_base", C.c_float), ("n_expert", C.c_int32), ("n_expert_used", C.c_int32),
+                ("ffn_expert", C.c_int32), ("vocab", C.c_int32), ("rms_eps", C.c_float),
+                ("ssm_head_dim", C.c_int32), ("ssm_head_k", C.c_int32), ("ssm_head_v", C.c_int32),
+                ("ssm_conv", C.c_int32), ("attn_every", C.c_int32), ("nkv", C.c_int32),
+                ("layers", C.c_int32), ("no_head", C.c_int32), ("attn_splits", C.c_int32)]
+
+    def __init__(self, **kw):
+        d = dict(n_layer=48, n_embd=2048, n_head=16, n_head_kv=2, head_dim=256, rope_dims=64,
+                 rope_base=1e7, n_expert=512, n_expert_used=10, ffn_expert=512, vocab=151936,
+                 rms_eps=1e-6, ssm_head_dim=128, ssm_head_k=16, ssm_head_v=32, ssm_conv=4,
+                 attn_every=4, nkv=4096, layers=0, no_head=0, attn_splits=0)
+        d.update(kw)
+        super().__init__(**d)
+
+
+_lib = None
+
+
+def lib_path():
+    return os.path.join(HERE, "libshv_llm.so")
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    hip_api.load()
+    p = lib_path()
+    if not os.path.exists(p):
+        raise hip_api.ShvError(-4, "%s is missing: build it with `python strix-halo-vulkan_amd/build.py`" % p)
+    L = C.CDLL(p)
+    vp = C.c_void_p
+    L.shvllm_last_error.restype = C.c_char_p
+    L.shvllm_open.argtypes = [C.c_int, C.POINTER(Config), C.POINTER(vp)]
+    L.shvllm_close.argtypes = [vp]
+    L.shvllm_close.restype = None
+    L.shvllm_ctx.argtypes = [vp]
+    L.shvllm_ctx.restype = vp
+    L.shvllm_init_synthetic.argtypes = [vp, C.c_uint64]
+    L.shvllm_tensor_count.argtypes = [vp]
+    L.shvllm_tensor_at.argtypes = [vp, C.c_int, C.POINTER(C.c_char_p), C.POINTER(vp), C.POINTER(C.c_uint64),
+                                   C.POINTER(C.c_int32), C.POINTER(C.c_int64), C.POINTER(C.c_int64),
+                                   C.POINTER(C.c_int32)]
+    L.shvllm_tensor.argtypes = [vp, C.c_char_p, C.POINTER(vp), C.POINTER(C.c_uint64)]
+    L.shvllm_weight_bytes.argtypes = [vp]
+    L.shvllm_weight_bytes.restype = C.c_uint64
+    L.shvllm_stage.argtypes = [vp]
+    L.shvllm_reset.argtypes = [vp]
+    L.shvllm_extend.argtypes = [vp, C.POINTER(C.c_int32), C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    L.shvllm_generate.argtypes = [vp, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_uint64)]
+    L.shvllm_past.argtypes = [vp]
+    L.shvllm_dispatches.argtypes = [vp]
+    L.shvllm_profile_step.argtypes = [vp, C.POINTER(C.c_char * 32), C.POINTER(C.c_uint64), C.c_int,
+                                      C.POINTER(C.c_int)]
+    L.shvllm_dn_state.argtypes = [vp, C.c_int, C.POINTER(C.c_float)]
+    L.shvllm_kv.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_uint16), C.POINTER(C.c_uint16)]
+    L.shvllm_gpu_nanos.argtypes = [vp]
+    L.shvllm_gpu_nanos.restype = C.c_uint64
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise hip_api.ShvError(rc, load().shvllm_last_error().decode("utf-8", "replace"))
+
+
+KIND_DTYPE = {0: np.float32, 1: np.uint16, 2: np.uint8}  # F32, F16 (bit patterns), Q4K (bytes)
+
+
+class LLM:
+    """llm.Model + llm.Graph behind one handle."""
+
+    def __init__(self, cfg, device=0):
+        self.L = load()
+        self.H = hip_api.load()
+        self.cfg = cfg
+        h = C.c_void_p()
+        _check(self.L.shvllm_open(device, C.byref(cfg), C.byref(h)))
+        self.h = h
+        self.ctx = self.L.shvllm_ctx(h)
+
+    def close(self):
+        if self.h:
+            self.L.shvllm_close(self.h)
+            self.h = None
+
+    def init_synthetic(self, seed):
+        _check(self.L.shvllm_init_synthetic(self.h, seed))
+
+    def tensors(self):
+        """[(name, device pointer, bytes, kind, rows, cols, is_alias)]"""
+        out = []
+        for i in range(self.L.shvllm_tensor_count(self.h)):
+            name, ptr, nb = C.c_char_p(), C.c_void_p(), C.c_uint64()
+            kind, rows, cols, al = C.c_int32(), C.c_int64(), C.c_int64(), C.c_int32()
+            _check(self.L.shvllm_tensor_at(self.h, i, C.byref(name), C.byref(ptr), C.byref(nb), C.byref(kind),
+                                           C.byref(rows), C.byref(cols), C.byref(al)))
+            out.append((name.value.decode(), ptr.value, nb.value, kind.value, rows.value, cols.value, bool(al.value)))
+        return out
+
+    def download(self, name):
+        ptr, nb = C.c_void_p(), C.c_uint64()
+        _check(self.L.shvllm_tensor(self.h, name.encode(), C.byref(ptr), C.byref(nb)))
+        kind = next(t[3] for t in self.tensors() if t[0] == name)
+        dt = np.dtype(KIND_DTYPE[kind])
+        a = np.empty(nb.value // dt.itemsize, dtype=dt)
+        hip_api.check(self.H.shv_download(self.ctx, a.ctypes.data, ptr, nb.value))
+        return a
+
+    def upload(self, name, arr):
+        ptr, nb = C.c_void_p(), C.c_uint64()
+        _check(self.L.shvllm_tensor(self.h, name.encode(), C.byref(ptr), C.byref(nb)))
+        arr = np.ascontiguousarray(arr)
+        assert arr.nbytes == nb.value, (name, arr.nbytes, nb.value)
+        hip_api.check(self.H.shv_upload(self.ctx, ptr, arr.ctypes.data, arr.nbytes))
+
+    def weight_bytes(self):
+        return self.L.shvllm_weight_bytes(self.h)
+
+    def stage(self):
+        _check(self.L.shvllm_stage(self.h))
+
+    def reset(self):
+        _check(self.L.shvllm_reset(self.h))
+
+    def extend(self, ids, want_logits=True, want_hidden=False):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        lg = np.empty(self.cfg.vocab, np.float32) if want_logits else None
+        hd = np.empty(self.cfg.n_embd, np.float32) if want_hidden else None
+        fp = C.POINTER(C.c_float)
+        _check(self.L.shvllm_extend(self.h, ids.ctypes.data_as(C.POINTER(C.c_int32)), len(ids),
+                                    lg.ctypes.data_as(fp) if lg is not None else None,
+                                    hd.ctypes.data_as(fp) if hd is not None else None))
+        return lg, hd
+
+    def generate(self, n):
+        out = np.empty(n, np.int32)
+        ns = C.c_uint64()
+        _check(self.L.shvllm_generate(self.h, n, out.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(ns)))
+        return out, ns.value
+
+    def past(self):
+        return self.L.shvllm_past(self.h)
+
+    def dispatches(self):
+        return self.L.shvllm_dispatches(self.h)
+
+    def profile_step(self):
+        labels = (C.c_char * 32 * 64)()
+        ns = (C.c_uint64 * 64)()
+        n = C.c_int()
+        _check(self.L.shvllm_profile_step(self.h, labels, ns, 64, C.byref(n)))
+        return [(labels[i].value.decode(), ns[i]) for i in range(n.value)]
+
+    def dn_state(self, layer):
+        c = self.cfg
+        out = np.empty((c.ssm_head_v, c.ssm_head_dim, c.ssm_head_dim), np.float32)
+        _check(self.L.shvllm_dn_state(self.h, layer, out.ctypes.data_as(C.POINTER(C.c_float))))
+        return out
+
+    def kv(self, layer, cells):
+        c = self.cfg
+        k = np.empty((cells, c.n_head_kv, c.head_dim), np.uint16)
+        v = np.empty_like(k)
+        u16 = C.POINTER(C.c_uint16)
+        _check(self.L.shvllm_kv(self.h, layer, cells, k.ctypes.data_as(u16), v.ctypes.data_as(u16)))
+        return k, v

@@ -58,6 +58,24 @@ class AttnW(C.Structure):
     _fields_ = [("q", u8p), ("k", u8p), ("v", u8p), ("o", u8p), ("q_norm", f32p), ("k_norm", f32p)]
 
 
+class ModelCfg(C.Structure):
+    _fields_ = [("n_layer", C.c_int), ("n_embd", C.c_int), ("vocab", C.c_int), ("attn_every", C.c_int),
+                ("eps", C.c_float), ("max_cells", C.c_int), ("moe", MoeCfg), ("dn", DnCfg), ("attn", AttnCfg)]
+
+
+class LayerW(C.Structure):
+    _fields_ = [("attn_norm", f32p), ("ffn_norm", f32p), ("dn", DnW), ("attn", AttnW), ("moe", MoeW)]
+
+
+class ModelW(C.Structure):
+    _fields_ = [("embd", u16p), ("out_norm", f32p), ("lm_head", u8p), ("layers", C.POINTER(LayerW))]
+
+
+class ModelState(C.Structure):
+    _fields_ = [("dn_conv", C.POINTER(f32p)), ("dn_s", C.POINTER(f32p)), ("kcache", C.POINTER(u16p)),
+                ("vcache", C.POINTER(u16p)), ("past", C.c_int)]
+
+
 _lib = None
 
 
@@ -103,6 +121,8 @@ def lib():
     L.shv_ref_rope.argtypes = [C.POINTER(AttnCfg), f32p, i32p, C.c_int, C.c_int, C.c_int]
     L.shv_ref_attn_layer.argtypes = [C.POINTER(AttnCfg), C.POINTER(AttnW), f32p, C.c_int, C.c_int,
                                      u16p, u16p, f32p, f32p, f32p, C.c_int]
+    L.shv_ref_model_extend.argtypes = [C.POINTER(ModelCfg), C.POINTER(ModelW), C.POINTER(ModelState), i32p,
+                                       C.c_int, f32p, f32p, C.c_int]
     _lib = L
     return L
 
@@ -175,3 +195,68 @@ def rel_l2(got, want):
     want = np.asarray(want, dtype=np.float64).ravel()
     den = np.linalg.norm(want)
     return float(np.linalg.norm(got - want) / (den if den > 0 else 1.0))
+
+
+class OracleModel:
+    """The CPU token loop over a model whose tensors are given by GGUF-style name (numpy arrays):
+    Q4_K tensors as bytes, the embedding as binary16 bit patterns, the rest float32."""
+
+    def __init__(self, cfg, tensors, max_cells, sections=(11, 11, 10, 0)):
+        """cfg: any object with the fields of the host layer's config."""
+        self.cfg, self.t, self.keep = cfg, tensors, []
+        ne, d = cfg.n_embd, cfg.ssm_head_dim
+        self.mcfg = ModelCfg(
+            cfg.n_layer, ne, cfg.vocab, cfg.attn_every, cfg.rms_eps, max_cells,
+            MoeCfg(ne, cfg.n_expert, cfg.n_expert_used, cfg.ffn_expert, cfg.ffn_expert),
+            DnCfg(ne, d, cfg.ssm_head_k, cfg.ssm_head_v, cfg.ssm_conv, cfg.rms_eps, 0),
+            AttnCfg(ne, cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.rope_dims, cfg.rope_base,
+                    (C.c_int * 4)(*sections), cfg.rms_eps))
+        blk = lambda l, n: tensors["blk.%d.%s.weight" % (l, n)]
+        layers = (LayerW * cfg.n_layer)()
+        for l in range(cfg.n_layer):
+            lw = layers[l]
+            lw.attn_norm, lw.ffn_norm = F(blk(l, "attn_norm")), F(blk(l, "post_attention_norm"))
+            if (l + 1) % cfg.attn_every == 0:
+                lw.attn = AttnW(B(blk(l, "attn_q")), B(blk(l, "attn_k")), B(blk(l, "attn_v")),
+                                B(blk(l, "attn_output")), F(blk(l, "attn_q_norm")), F(blk(l, "attn_k_norm")))
+            else:
+                lw.dn = DnW(B(blk(l, "attn_qkv")), B(blk(l, "attn_gate")), B(blk(l, "ssm_alpha")),
+                            B(blk(l, "ssm_beta")), B(blk(l, "ssm_out")), F(blk(l, "ssm_conv1d")),
+                            F(blk(l, "ssm_a")), F(blk(l, "ssm_dt")), F(blk(l, "ssm_norm")))
+            lw.moe = MoeW(F(blk(l, "ffn_gate_inp")), F(blk(l, "ffn_gate_inp_shexp")), B(blk(l, "ffn_gate_exps")),
+                          B(blk(l, "ffn_up_exps")), B(blk(l, "ffn_down_exps")), B(blk(l, "ffn_gate_shexp")),
+                          B(blk(l, "ffn_up_shexp")), B(blk(l, "ffn_down_shexp")))
+        self.layers = layers
+        self.w = ModelW(H(tensors["token_embd.weight"]), F(tensors["output_norm.weight"]),
+                        B(tensors["output.weight"]), layers)
+        self.max_cells = max_cells
+        self.reset()
+
+    def reset(self):
+        c, n = self.cfg, self.cfg.n_layer
+        cw = 2 * c.ssm_head_k * c.ssm_head_dim + c.ssm_head_v * c.ssm_head_dim
+        self.dn_conv, self.dn_s, self.kc, self.vc = [None] * n, [None] * n, [None] * n, [None] * n
+        a_conv, a_s, a_k, a_v = (f32p * n)(), (f32p * n)(), (u16p * n)(), (u16p * n)()
+        for l in range(n):
+            if (l + 1) % c.attn_every == 0:
+                self.kc[l] = np.zeros((self.max_cells, c.n_head_kv, c.head_dim), np.uint16)
+                self.vc[l] = np.zeros_like(self.kc[l])
+                a_k[l], a_v[l] = H(self.kc[l]), H(self.vc[l])
+            else:
+                self.dn_conv[l] = np.zeros((cw, c.ssm_conv - 1), np.float32)
+                self.dn_s[l] = np.zeros((c.ssm_head_v, c.ssm_head_dim, c.ssm_head_dim), np.float32)
+                a_conv[l], a_s[l] = F(self.dn_conv[l]), F(self.dn_s[l])
+        self.arrays = (a_conv, a_s, a_k, a_v)
+        self.state = ModelState(a_conv, a_s, a_k, a_v, 0)
+
+    def extend(self, ids, threads=8):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        logits = np.empty(self.cfg.vocab, np.float32)
+        hidden = np.empty(self.cfg.n_embd, np.float32)
+        lib().shv_ref_model_extend(C.byref(self.mcfg), C.byref(self.w), C.byref(self.state), I(ids), len(ids),
+                                   F(logits), F(hidden), threads)
+        return logits, hidden
+
+    @property
+    def past(self):
+        return self.state.past
