@@ -62,7 +62,8 @@ struct GemvBatch {
     }
 };
 
-template <int K, int NT>
+// U is the number of passes a wave loads together; passes_per_wave is a multiple of it.
+template <int K, int NT, int U>
 __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int passes_per_wave, int t0) {
     constexpr int LPR = K / 64;   // lanes per row
     constexpr int XPAD = K + K / 64 * 4;
@@ -71,6 +72,17 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     __shared__ float red[4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int gi = lane % LPR;   // 64-weight group of the row
+    const int rsub = lane / LPR; // which of the pass's rows
+    const int sb = gi >> 2, g = gi & 3;
+    const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
+    const int n = a.n;
+    const long long first_pass = (static_cast<long long>(blockIdx.x) * kWavesPerBlock + wave) * passes_per_wave;
+
+    // The first batch of weights does not depend on the activations: its loads go out before
+    // the prologue so that HBM latency and the staging of x overlap.
+    GemvBatch<K, NT, U> A, B;
+    A.load(wbase, g, rsub, first_pass, n);
 
     // ---- stage pro(x) in LDS ----
 #pragma unroll
@@ -140,17 +152,10 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     __syncthreads();
 
     // ---- this lane's 64 activations per token ----
-    const int gi = lane % LPR;   // 64-weight group of the row
-    const int rsub = lane / LPR; // which of the pass's rows
     float xr[NT][64];
     float xs_lo[NT], xs_hi[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) load_x_slice(xs[t], gi, xr[t], xs_lo[t], xs_hi[t]);
-
-    const int sb = gi >> 2, g = gi & 3;
-    const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
-    const int n = a.n;
-    const long long first_pass = (static_cast<long long>(blockIdx.x) * kWavesPerBlock + wave) * passes_per_wave;
 
     size_t y_off[NT];
 #pragma unroll
@@ -167,60 +172,59 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     }
 
     const NibbleConsts nc = nibble_consts();
-    constexpr int U = 4;
-    const int nb = passes_per_wave / U;  // full batches, double-buffered
-    if (nb > 0) {
-        GemvBatch<K, NT, U> A, B;
-        A.load(wbase, g, rsub, first_pass, n);
-        for (int b = 0; b < nb; b += 2) {
-            const bool has_b = b + 1 < nb;
-            if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U, n);
-            A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
-            if (has_b) {
-                if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U, n);
-                B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
-            }
+    const int nb = passes_per_wave / U;  // batches, double-buffered
+    for (int b = 0; b < nb; b += 2) {
+        const bool has_b = b + 1 < nb;
+        if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U, n);
+        A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
+        if (has_b) {
+            if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U, n);
+            B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
         }
-    }
-    int p0 = nb * U;
-    if (p0 + 2 <= passes_per_wave) {
-        GemvBatch<K, NT, 2> T2;
-        T2.load(wbase, g, rsub, first_pass + p0, n);
-        T2.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
-        p0 += 2;
-    }
-    if (p0 < passes_per_wave) {
-        GemvBatch<K, NT, 1> T1;
-        T1.load(wbase, g, rsub, first_pass + p0, n);
-        T1.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
     }
 }
 
-template <int K, int NT>
-int launch_nt(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw, int t0) {
+template <int K, int NT, int U>
+int launch_ntu(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw, int t0) {
     if (lds > 48 * 1024) {
         // above the default dynamic-LDS allowance the limit has to be raised once per kernel
         static bool raised = false;
         if (!raised) {
-            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_kernel<K, NT>),
+            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_kernel<K, NT, U>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_q4k_kernel<K, NT>), grid, block, lds, ctx->stream, a, ppw, t0);
+    hipLaunchKernelGGL((gemv_q4k_kernel<K, NT, U>), grid, block, lds, ctx->stream, a, ppw, t0);
     SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
+}
+
+template <int K, int NT>
+int launch_nt(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw, int u, int t0) {
+    switch (u) {
+        case 1: return launch_ntu<K, NT, 1>(ctx, a, grid, block, lds, ppw, t0);
+        case 2: return launch_ntu<K, NT, 2>(ctx, a, grid, block, lds, ppw, t0);
+        case 3: return launch_ntu<K, NT, 3>(ctx, a, grid, block, lds, ppw, t0);
+        default: return launch_ntu<K, NT, 4>(ctx, a, grid, block, lds, ppw, t0);
+    }
 }
 
 template <int K>
 int launch_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     constexpr int RPP = 64 / (K / 64);
     const long long passes = (static_cast<long long>(a.n) + RPP - 1) / RPP;
-    // Enough waves to have every load of a small matrix in flight at once; large matrices get
-    // several passes per wave so the staging of x is amortised.
-    const long long target_waves = static_cast<long long>(ctx->prop.multiProcessorCount) * 4 * 4;
-    long long ppw = (passes + target_waves - 1) / target_waves;
+    // One round of resident waves (two per SIMD at this kernel's register count): every wave of
+    // the grid is on the chip at once and streams its share of the rows.  Up to four passes are
+    // loaded together; longer shares run as double-buffered batches of four.
+    const long long resident = static_cast<long long>(ctx->prop.multiProcessorCount) * 4 * 2;
+    long long ppw = (passes + resident - 1) / resident;
     if (ppw < 1) ppw = 1;
+    int u = static_cast<int>(ppw);
+    if (ppw > 4) {
+        ppw = (ppw + 3) / 4 * 4;
+        u = 4;
+    }
     const long long waves = (passes + ppw - 1) / ppw;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     SHV_REQUIRE(blocks > 0 && blocks < (1ll << 31), "gemv_q4k: grid of %lld blocks", blocks);
@@ -231,10 +235,10 @@ int launch_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
         const size_t lds = static_cast<size_t>(nt) * (K + K / 64 * 4) * sizeof(float);
         int rc;
         switch (nt) {
-            case 1: rc = launch_nt<K, 1>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
-            case 2: rc = launch_nt<K, 2>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
-            case 3: rc = launch_nt<K, 3>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
-            default: rc = launch_nt<K, 4>(ctx, a, grid, block, lds, static_cast<int>(ppw), t0); break;
+            case 1: rc = launch_nt<K, 1>(ctx, a, grid, block, lds, static_cast<int>(ppw), u, t0); break;
+            case 2: rc = launch_nt<K, 2>(ctx, a, grid, block, lds, static_cast<int>(ppw), u, t0); break;
+            case 3: rc = launch_nt<K, 3>(ctx, a, grid, block, lds, static_cast<int>(ppw), u, t0); break;
+            default: rc = launch_nt<K, 4>(ctx, a, grid, block, lds, static_cast<int>(ppw), u, t0); break;
         }
         if (rc != SHV_OK) return rc;
     }

@@ -132,20 +132,15 @@ __global__ __launch_bounds__(256) void argmax_kernel(shv_argmax_args a, float *p
     if (threadIdx.x == 0) {
         for (int w = 1; w < 4; w++)
             if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
-        pval[r * nb + blockIdx.x] = bv;
-        pidx[r * nb + blockIdx.x] = bi;
-        __threadfence();
-        const int prev = __hip_atomic_fetch_add(counters + r, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = prev == nb - 1;
+        shv::store_agent(pval + r * nb + blockIdx.x, bv);
+        shv::store_agent(pidx + r * nb + blockIdx.x, bi);
     }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
+    if (!shv::arrive_last(counters + r, nb, &is_last)) return;
     bv = -INFINITY;
     bi = a.n;
     for (int b = threadIdx.x; b < nb; b += blockDim.x) {
-        const float v = pval[r * nb + b];
-        const int i = pidx[r * nb + b];
+        const float v = shv::load_agent(pval + r * nb + b);
+        const int i = shv::load_agent(pidx + r * nb + b);
         if (better(v, i, bv, bi)) { bv = v; bi = i; }
     }
     wave_best(bv, bi);
@@ -163,7 +158,6 @@ __global__ __launch_bounds__(256) void argmax_kernel(shv_argmax_args a, float *p
             a.ids[p + 1] = bi;
             a.pos[0] = p + 1;
         }
-        __hip_atomic_store(counters + r, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 

@@ -14,23 +14,45 @@ constexpr float kWeightsSumFloor = 6.103515625e-5f;  // 2^-14
 
 // ---------------------------------------------------------------------------- router ---------
 
-// Descending order on (probability, lower index first) as one 64-bit key.
-__device__ __forceinline__ unsigned long long route_key(float p, int idx) {
-    return (static_cast<unsigned long long>(__float_as_uint(p)) << 32) | static_cast<unsigned int>(0x7FFFFFFF - idx);
+// Candidates are ordered by (probability, lower index first): the pair (bits of p, 0x7FFFFFFF-idx)
+// compared lexicographically.  Probabilities are positive, so their bit patterns order as they do.
+__device__ __forceinline__ bool pair_gt(uint32_t ah, uint32_t al, uint32_t bh, uint32_t bl) {
+    return ah > bh || (ah == bh && al > bl);
 }
 
-__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+template <int CTRL>
+__device__ __forceinline__ void pair_max_step(uint32_t &hi, uint32_t &lo) {
+    const uint32_t oh = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(hi), CTRL, 0xF, 0xF, false));
+    const uint32_t ol = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(lo), CTRL, 0xF, 0xF, false));
+    const bool take = pair_gt(oh, ol, hi, lo);
+    hi = take ? oh : hi;
+    lo = take ? ol : lo;
+}
+
+// Maximum pair over the wave, in every lane: DPP within the rows of 16, then the four row
+// winners are read out as scalars.
+__device__ __forceinline__ void wave_pair_max(uint32_t &hi, uint32_t &lo) {
+    pair_max_step<kDppXor1>(hi, lo);
+    pair_max_step<kDppXor2>(hi, lo);
+    pair_max_step<kDppHalfMirror>(hi, lo);
+    pair_max_step<kDppMirror>(hi, lo);
+    uint32_t bh = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 0));
+    uint32_t bl = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 0));
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        const unsigned long long o = __shfl_xor(v, off, 64);
-        v = o > v ? o : v;
+    for (int r = 16; r < 64; r += 16) {
+        const uint32_t oh = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), r));
+        const uint32_t ol = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), r));
+        const bool take = pair_gt(oh, ol, bh, bl);
+        bh = take ? oh : bh;
+        bl = take ? ol : bl;
     }
-    return v;
+    hi = bh;
+    lo = bl;
 }
 
 // One wave routes one token: softmax over n_expert logits (n_expert <= 64*8), then n_used rounds of
-// arg-max.  Probabilities are formed as the reference forms them (exp, sequential float32 sum in
-// index order, multiply by the reciprocal) so that equal logits stay equal probabilities.
+// arg-max.  Probabilities are formed as the reference forms them (exp of the logit minus the
+// maximum, times the reciprocal of their sum) so that equal logits stay equal probabilities.
 template <int PER>
 __device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *probs_lds) {
     const int lane = threadIdx.x & 63;
@@ -39,7 +61,7 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int e = lane + i * 64;
-        l[i] = e < n_expert ? logits[e] : -INFINITY;
+        l[i] = e < n_expert ? load_agent(logits + e) : -INFINITY;
         mx = fmaxf(mx, l[i]);
     }
     mx = wave_max_all(mx);
@@ -49,33 +71,43 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         if (e < n_expert) probs_lds[e] = expf(l[i] - mx);
     }
     __builtin_amdgcn_wave_barrier();
-    // the reference's sum runs over the experts in index order in float32; one lane repeats it
+    // The reference adds the exponentials one after another in index order; a tree over the wave
+    // differs from that in the last bits of the sum only, and the sum scales every probability
+    // alike, so neither the order of the experts nor the normalised weights move with it.
     float sum = 0.f;
-    if (lane == 0)
-        for (int e = 0; e < n_expert; e++) sum += probs_lds[e];
-    sum = __shfl(sum, 0, 64);
-    const float inv = 1.f / sum;
-    unsigned long long key[PER];
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int e = lane + i * 64;
-        key[i] = e < n_expert ? route_key(probs_lds[e] * inv, e) : 0ull;
+        if (e < n_expert) sum += probs_lds[e];
+    }
+    sum = wave_sum_all(sum);
+    const float inv = 1.f / sum;
+    uint32_t kh[PER], kl[PER];  // (0, 0) marks an empty or already taken candidate
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        kh[i] = e < n_expert ? __float_as_uint(probs_lds[e] * inv) : 0u;
+        kl[i] = e < n_expert ? static_cast<uint32_t>(0x7FFFFFFF - e) : 0u;
     }
     // lane k keeps the k-th pick; the running sum is uniform across the wave
     float my_w = 0.f, wsum = 0.f;
     int my_e = 0;
 #pragma unroll 1
     for (int k = 0; k < n_used; k++) {
-        unsigned long long best = 0ull;
+        uint32_t bh = 0u, bl = 0u;
 #pragma unroll
-        for (int i = 0; i < PER; i++) best = key[i] > best ? key[i] : best;
-        best = wave_max_u64(best);
+        for (int i = 0; i < PER; i++) {
+            const bool take = pair_gt(kh[i], kl[i], bh, bl);
+            bh = take ? kh[i] : bh;
+            bl = take ? kl[i] : bl;
+        }
+        wave_pair_max(bh, bl);
 #pragma unroll
         for (int i = 0; i < PER; i++)
-            if (key[i] == best) key[i] = 0ull;
-        const float w = __uint_as_float(static_cast<unsigned int>(best >> 32));
+            if (kh[i] == bh && kl[i] == bl) kh[i] = kl[i] = 0u;
+        const float w = __uint_as_float(bh);
         if (lane == k) {
-            my_e = 0x7FFFFFFF - static_cast<int>(best & 0xFFFFFFFFull);
+            my_e = 0x7FFFFFFF - static_cast<int>(bl);
             my_w = w;
         }
         wsum += w;  // slot order, float32: the reference's sum
@@ -96,6 +128,16 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
     __shared__ int is_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = blockIdx.x * 4 + wave;  // n_expert = the shared-gate row
+    const bool has_row = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
+    // the wave's router row is in flight while the first token is being normalised, and stays in
+    // registers for every token
+    float4 wrow[H / 256];
+    {
+        const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
+#pragma unroll
+        for (int i = 0; i < H / 256; i++)
+            wrow[i] = has_row ? *reinterpret_cast<const float4 *>(w + (i * 64 + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     for (int t = 0; t < a.n_tok; t++) {
         const float *h = a.h + static_cast<size_t>(t) * a.h_stride;
         float v[H / kBlock];
@@ -118,13 +160,12 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
             if (blockIdx.x == 0 && a.xn) a.xn[static_cast<size_t>(t) * H + c] = x;
         }
         __syncthreads();
-        if (row <= a.n_expert && (row < a.n_expert || a.shared_gate)) {
-            const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
+        if (has_row) {
             float acc = 0.f;
 #pragma unroll
             for (int i = 0; i < H / 256; i++) {
                 const int c = (i * 64 + lane) * 4;
-                const float4 wv = *reinterpret_cast<const float4 *>(w + c);
+                const float4 wv = wrow[i];
                 const float4 xv = *reinterpret_cast<const float4 *>(xs + c);
                 acc = fmaf(wv.x, xv.x, acc);
                 acc = fmaf(wv.y, xv.y, acc);
@@ -132,26 +173,17 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
                 acc = fmaf(wv.w, xv.w, acc);
             }
             acc = wave_sum_all(acc);
-            if (lane == 0) a.logits[static_cast<size_t>(t) * (a.n_expert + 1) + row] = acc;
+            if (lane == 0) store_agent(a.logits + static_cast<size_t>(t) * (a.n_expert + 1) + row, acc);
         }
         __syncthreads();
     }
     // ---- the last block to arrive routes every token ----
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const int prev = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = prev == static_cast<int>(gridDim.x) - 1;
-    }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
-    if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!arrive_last(counter, static_cast<int>(gridDim.x), &is_last)) return;
     for (int t = wave; t < a.n_tok; t += 4) {
         const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
         float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
         route_token<8>(lg, a.n_expert, a.n_used, a.topk + static_cast<size_t>(t) * a.n_used, wt, probs[wave]);
-        if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(lg[a.n_expert]) : 0.f;
+        if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(load_agent(lg + a.n_expert)) : 0.f;
     }
 }
 
@@ -215,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int SPW = (MAXS + 3) / 4;  // slots per wave
-    __shared__ float xs[MAXS][lds_padded(K)];
+    __shared__ __align__(16) float xs[MAXS][lds_padded(K)];
     __shared__ float part[4][RPP];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t = blockIdx.y;
@@ -243,9 +275,31 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
             wt[i] = a.weights[static_cast<size_t>(t) * ns + s];
         }
     }
+    // each wave stages the activations of its own slots only, so no block-wide hand-over is
+    // needed before the dot products: all loads first, then the LDS writes
     const float *act = a.act + static_cast<size_t>(t) * ns * K;
-    for (int c = tid; c < ns * K; c += kBlock) xs[c / K][lds_slot(c % K)] = act[c];
-    __syncthreads();
+    constexpr int F4 = K / 4 / 64;  // float4 per lane per slot
+    float4 stage[SPW][F4];
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+        const int s = wave + 4 * i;
+#pragma unroll
+        for (int j = 0; j < F4; j++)
+            stage[i][j] = s < ns ? *reinterpret_cast<const float4 *>(act + static_cast<size_t>(s) * K + (j * 64 + lane) * 4)
+                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < SPW; i++) {
+        const int s = wave + 4 * i;
+        if (s < ns) {
+#pragma unroll
+            for (int j = 0; j < F4; j++) {
+                const int c = (j * 64 + lane) * 4;  // four consecutive columns never straddle a 64-slice
+                *reinterpret_cast<float4 *>(&xs[s][lds_slot(c)]) = stage[i][j];
+            }
+        }
+    }
+    __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
 
     const NibbleConsts nc = nibble_consts();
     float acc = 0.f;

@@ -199,6 +199,42 @@ struct Q4kLane {
     }
 };
 
+// ---- handing results from many blocks to the last one to finish ---------------------------------
+// The L2 caches of the chip's eight dies are not coherent with one another, and a device-scope
+// release or acquire fence pays for that by writing back and invalidating a whole L2 — tens of
+// microseconds when every block of a grid does it.  Instead, the few values that cross between
+// blocks inside one kernel are written and read with device-scope atomic accesses, which go
+// through to the coherence point on their own; the arrival counter is a relaxed device-scope
+// atomic, ordered after the block's stores by waiting for them to complete.
+__device__ __forceinline__ void store_agent(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_agent(int32_t *p, int32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float load_agent(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int32_t load_agent(const int32_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_agent2(float *p, float a, float b) {
+    const unsigned long long v = static_cast<unsigned long long>(__float_as_uint(a)) | (static_cast<unsigned long long>(__float_as_uint(b)) << 32);
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 load_agent2(const float *p) {
+    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(__uint_as_float(static_cast<unsigned int>(v)), __uint_as_float(static_cast<unsigned int>(v >> 32)));
+}
+
+// Block-wide: every thread's earlier device-scope stores have completed, then one thread counts
+// the block in.  Returns true in every thread of the block that arrived last; that block also
+// re-arms the counter for the next launch.
+__device__ __forceinline__ bool arrive_last(int32_t *counter, int expected, int *lds_flag) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int prev = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev == expected - 1;
+        if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *lds_flag = last;
+    }
+    __syncthreads();
+    return *lds_flag != 0;
+}
+
 __device__ __forceinline__ float sigmoid_exact(float x) { return 1.f / (1.f + expf(-x)); }
 
 __device__ __forceinline__ float sigmoidf_dev(float x) { return 1.f / (1.f + __expf(-x)); }

@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <random>
 
@@ -448,8 +449,7 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     qkv_ = static_cast<float *>(dev.alloc(T * c_.AttnFusedRows() * 4));
     ctx_ = static_cast<float *>(dev.alloc(T * c_.NHead * c_.HeadDim * 4));
-    const int max_splits = std::max(256, (nKV + 1023) / 1024);
-    partial_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.NHeadKV) * max_splits * 8 * (c_.HeadDim + 2) * 4));
+    partial_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.NHeadKV) * kMaxSplits * 8 * (c_.HeadDim + 2) * 4));
     const std::vector<float> rt = rope_table(nKV, c_.RopeDims, c_.RopeBase);
     rope_ = static_cast<float *>(dev.alloc(rt.size() * 4));
     dev.upload(rope_, rt.data(), rt.size() * 4);
@@ -465,11 +465,10 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
 }
 
 void AttnGPU::SetSplits(int n) {
-    // enough slices to spread a long cache over the chip, few enough that a short one is not all
-    // merge: about 64 cells a slice at the capacity, at least what a block's LDS can score
-    if (n <= 0) n = std::min(256, std::max(8, n_kv_ / 64));
-    n = std::max(n, (n_kv_ + 1023) / 1024);
-    if (n > std::max(256, (n_kv_ + 1023) / 1024)) throw Error("llm: AttnGPU.SetSplits: too many slices");
+    // slices for the cache's capacity: about 128 cells each up to 256 slices (the kernel engages
+    // only as many as the sequence's current length fills)
+    if (n <= 0) n = std::min(256, std::max(8, (n_kv_ + 127) / 128));
+    if (n > kMaxSplits) throw Error("llm: AttnGPU.SetSplits: at most " + std::to_string(kMaxSplits) + " slices");
     splits_ = n;
 }
 
@@ -602,6 +601,21 @@ std::vector<float> HeadGPU::Logits() const { return read_back<float>(dev_, logit
 
 // -------------------------------------------------------------------------------- Graph -------
 
+// LLM_NO_PRERECORD=1 replays nothing: every pass is dispatched op by op, as the reference's
+// knob of the same name does (llm/graph.go:306).  Profilers that cannot follow a graph launch
+// see every kernel this way.
+static bool no_prerecord() {
+    const char *e = std::getenv("LLM_NO_PRERECORD");
+    return e && e[0] == '1';
+}
+
+static void submit(Device &dev, shv_prerecorded *rec, const std::vector<shv_op> &ops, int iters, uint64_t *ns, const char *what) {
+    if (no_prerecord())
+        check(shv_dispatch_multi(dev.ctx(), ops.data(), static_cast<int>(ops.size()), iters, ns, nullptr), what);
+    else
+        check(shv_prerecorded_submit(dev.ctx(), rec, iters, ns), what);
+}
+
 Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_(m), c_(m.config()), o_(opts) {
     layers_ = opts.Layers > 0 ? opts.Layers : c_.NLayer;
     if (layers_ > c_.NLayer) throw Error("llm: NewGraph: " + std::to_string(layers_) + " layers of a " + std::to_string(c_.NLayer) + "-layer model");
@@ -698,13 +712,13 @@ void Graph::Extend(const std::vector<int32_t> &ids, std::vector<float> *logits, 
     dev_.upload(pos_, &p, 4);
     // every row but the last goes through the headless step; the last one samples
     uint64_t ns = 0;
-    if (n > 1) check(shv_prerecorded_submit(dev_.ctx(), prefill_, n - 1, &ns), "prefill");
+    if (n > 1) submit(dev_, prefill_, prefill_ops_, n - 1, &ns, "prefill");
     Stats.GPUNanos += ns;
     if (head_) {
-        check(shv_prerecorded_submit(dev_.ctx(), step_, 1, &ns), "decode step");
+        submit(dev_, step_, step_ops_, 1, &ns, "decode step");
         Stats.Dispatches = static_cast<int>(step_ops_.size());
     } else {
-        check(shv_prerecorded_submit(dev_.ctx(), prefill_, 1, &ns), "last row");
+        submit(dev_, prefill_, prefill_ops_, 1, &ns, "last row");
         Stats.Dispatches = static_cast<int>(prefill_ops_.size());
     }
     Stats.GPUNanos += ns;
@@ -728,7 +742,7 @@ std::vector<int32_t> Graph::Generate(int n, uint64_t *gpu_nanos) {
     // the last Extend already sampled the token at position past_: it sits in ids[past_], and
     // every replay consumes ids[pos] and appends ids[pos+1]
     uint64_t ns = 0;
-    if (n > 1) check(shv_prerecorded_submit(dev_.ctx(), step_, n - 1, &ns), "generate");
+    if (n > 1) submit(dev_, step_, step_ops_, n - 1, &ns, "generate");
     if (gpu_nanos) *gpu_nanos = ns;
     std::vector<int32_t> out(n);
     dev_.download(out.data(), ids_ + past_, static_cast<size_t>(n) * 4);

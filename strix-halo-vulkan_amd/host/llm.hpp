@@ -193,6 +193,7 @@ public:
     void Upload(const std::vector<float> &x, int nTok);
     void Resize(int nTok);
     void Run(int layer);
+    static constexpr int kMaxSplits = 512;  // what the decode kernel's merge has room for
     void SetSplits(int n);
     int Splits() const { return splits_; }
     std::vector<shv_op> Dispatches(int layer, const float *in, float *out, int nTok, std::vector<std::string> *labels) const;

@@ -168,6 +168,6 @@ def test_attn_refuses_unsupported_shapes(ctx):
                                                  n_seq=1, seq_len=1, n_head=16, n_head_kv=2, head_dim=256,
                                                  rope_dims=64, max_cells=64, qkv_stride=9216, n_splits=4,
                                                  eps=EPS), **kw})
-    for bad in (dict(head_dim=128), dict(n_head=24), dict(n_splits=1, max_cells=5000), dict(qkv_stride=100)):
+    for bad in (dict(head_dim=128), dict(n_head=24), dict(n_splits=1000), dict(qkv_stride=100)):
         with pytest.raises(shv.pkg.ShvError):
             ctx.enqueue(A.OP_ATTN_DECODE, mk(**bad))
