@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the token loop on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one batch-1 greedy decode token of the synthetic Qwen3-Next-shape model (48 layers, 3
+gated-DeltaNet + 1 gated-attention repeating, 512-expert top-10 Q4_K MoE on every layer, vocab
+151 936): the prompt of 2048 random ids is prefilled first (untimed), W tokens are decoded untimed,
+then exactly K tokens are timed between two synchronisations.  Everything the timed region reads is
+resident in HBM before it starts.  Prints ONE JSON line.
+
+Beside the headline it reports
+  roofline      the dominant kernel of the step (the expert-gathered gate/up GEMV, 48 launches a
+                token): algorithmic bytes per launch over the kernel's own measured duration
+                (timestamps on the kernel's dispatch, taken live), against 8 TB/s
+  cpu_baseline  the CPU restatement of the reference's Go path (oracle/), timed on this host on a
+                bounded sample of the same model: layers 0..3 (one DeltaNet x3 + attention period)
+                plus the head, a few decode tokens, scaled by 12 periods to a 48-layer token
+  gemv          the single Q4_K GEMV of BASELINE config 1 (4096x2048) over a rotating set of
+                distinct weight matrices larger than the 256 MB Infinity Cache, and the 175 MB
+                lm_head GEMV, in GB/s and as a fraction of 8 TB/s
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X
+Q4K_ROW = lambda k: k // 256 * 144
+
+
+def moe_up_bytes(cfg):
+    """Algorithmic bytes of one moe.up launch at batch 1: gate and up rows of the routed experts
+    and the shared one, the normalised activation in, the SwiGLU activations out."""
+    experts = cfg.n_expert_used + 1
+    w = experts * 2 * cfg.ffn_expert * Q4K_ROW(cfg.n_embd)
+    return w + cfg.n_embd * 4 + experts * cfg.ffn_expert * 4 + cfg.n_expert_used * 4
+
+
+def token_bytes(cfg, ctx_len):
+    """Algorithmic bytes one decode token touches (each weight, state and cache byte once)."""
+    H, E, U, F = cfg.n_embd, cfg.n_expert, cfg.n_expert_used, cfg.ffn_expert
+    qk, vw = cfg.ssm_head_k * cfg.ssm_head_dim, cfg.ssm_head_v * cfg.ssm_head_dim
+    dn_rows = 2 * qk + 2 * vw + 2 * cfg.ssm_head_v
+    dn = dn_rows * Q4K_ROW(H) + H * Q4K_ROW(vw) + 2 * cfg.ssm_head_v * cfg.ssm_head_dim ** 2 * 4 + (2 * qk + vw) * 16
+    at_rows = cfg.n_head * 2 * cfg.head_dim + 2 * cfg.n_head_kv * cfg.head_dim
+    at = at_rows * Q4K_ROW(H) + H * Q4K_ROW(cfg.n_head * cfg.head_dim) + ctx_len * cfg.n_head_kv * cfg.head_dim * 2 * 2
+    moe = E * H * 4 + H * 4 + (U + 1) * (2 * F * Q4K_ROW(H) + H * Q4K_ROW(F))
+    n_attn = cfg.n_layer // cfg.attn_every
+    head = cfg.vocab * Q4K_ROW(H) + H * 2
+    return (cfg.n_layer - n_attn) * dn + n_attn * at + cfg.n_layer * moe + head
+
+
+def cpu_baseline(m, cfg, LA, n_tokens):
+    """Time the oracle's token loop on a 4-layer slice of the same weights."""
+    import oracle_lib as O
+    per = cfg.attn_every
+    sub = LA.Config(**{f: getattr(cfg, f) for f, _ in cfg._fields_})
+    sub.n_layer = per
+    names = [t[0] for t in m.tensors()]
+    keep = [n for n in names if not n.startswith("blk.") or int(n.split(".")[1]) < per]
+    tensors = {n: m.download(n) for n in keep}
+    cores = min(os.cpu_count() or 1, 16)
+    om = O.OracleModel(sub, tensors, max_cells=64)
+    rng = np.random.default_rng(1)
+    om.extend(rng.integers(0, cfg.vocab, size=1).astype(np.int32), threads=cores)  # touch everything once
+    t0 = time.perf_counter()
+    head_s = 0.0
+    for _ in range(n_tokens):
+        om.extend(rng.integers(0, cfg.vocab, size=1).astype(np.int32), threads=cores)
+    dt = (time.perf_counter() - t0) / n_tokens
+    # the head runs once per token, the 4-layer period 12 times: time the head alone to split them
+    x = rng.standard_normal(cfg.n_embd).astype(np.float32)
+    t0 = time.perf_counter()
+    O.gemv_q4k(tensors["output.weight"], x, cfg.vocab, cfg.n_embd, threads=cores)
+    head_s = time.perf_counter() - t0
+    periods = cfg.n_layer // per
+    per_token = (dt - head_s) * periods + head_s
+    return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "sample": "C restatement of the reference's Go CPU path (oracle/), layers 0-%d + lm_head of the same "
+                      "weights, %d decode tokens at context <= %d; period time x%d + head time; rows of each matvec "
+                      "split over %d threads" % (per - 1, n_tokens, n_tokens + 1, periods, cores)}
+
+
+def gemv_rates(m, cfg, A, LA):
+    """Config 1's GEMV over rotating weights, and the lm_head GEMV, timed by GPU events."""
+    pkg = importlib.import_module("strix-halo-vulkan_amd")
+    H = pkg.hip_api.load()
+    import ctypes as C
+    ctx = m.ctx
+    out = {}
+
+    def alloc(n):
+        p = C.c_void_p()
+        A.check(H.shv_alloc(ctx, n, C.byref(p)))
+        return p.value
+
+    n, k = 4096, cfg.n_embd
+    bank = next(t for t in m.tensors() if t[0] == "blk.0.ffn_gate_exps.weight")
+    mat_bytes = n * Q4K_ROW(k)
+    copies = min(bank[2] // mat_bytes, 128)
+    dx, dy = alloc(k * 4), alloc(max(n, cfg.vocab) * 4)
+    x = np.random.default_rng(2).standard_normal(k).astype(np.float32)
+    A.check(H.shv_upload(ctx, dx, x.ctypes.data, x.nbytes))
+    ops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(bank[1] + i * mat_bytes, dx, dy, n, k)) for i in range(copies)]
+    arr = (A.Op * len(ops))(*ops)
+    pre = C.c_void_p()
+    A.check(H.shv_prerecord(ctx, arr, len(ops), C.byref(pre)))
+    ns = C.c_uint64()
+    A.check(H.shv_prerecorded_submit(ctx, pre, 2, C.byref(ns)))
+    A.check(H.shv_prerecorded_submit(ctx, pre, 10, C.byref(ns)))
+    per = ns.value / (10 * copies) / 1e9
+    alg = mat_bytes + k * 4 + n * 4
+    out["config1_4096x2048"] = {"us": round(per * 1e6, 3), "GBps": round(alg / per / 1e9, 1),
+                                "frac_hbm_peak": round(alg / per / HBM_PEAK, 4),
+                                "distinct_matrices": int(copies), "rotating_MB": round(copies * mat_bytes / 1e6, 1)}
+    H.shv_prerecorded_destroy(ctx, pre)
+    head = next(t for t in m.tensors() if t[0] == "output.weight")
+    ops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(head[1], dx, dy, cfg.vocab, k))]
+    arr = (A.Op * 1)(*ops)
+    A.check(H.shv_dispatch_multi(ctx, arr, 1, 3, C.byref(ns), None))
+    A.check(H.shv_dispatch_multi(ctx, arr, 1, 20, C.byref(ns), None))
+    per = ns.value / 20 / 1e9
+    alg = head[2] + k * 4 + cfg.vocab * 4
+    out["lm_head_151936x2048"] = {"us": round(per * 1e6, 2), "GBps": round(alg / per / 1e9, 1),
+                                  "frac_hbm_peak": round(alg / per / HBM_PEAK, 4)}
+    for p in (dx, dy):
+        H.shv_free(ctx, p)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=48)
+    ap.add_argument("--cpu-tokens", type=int, default=4)
+    ap.add_argument("--no-cpu", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs the token loop on ONE GPU (one process, one stream); "
+                 "--gpus %d is not supported. How the path would shard is described in DESIGN.md." % a.gpus)
+    if a.steps < 1 or a.warmup < 1:
+        sys.exit("bench.py: --steps and --warmup must be at least 1")
+    pkg = importlib.import_module("strix-halo-vulkan_amd")
+    LA, A = pkg.llm_api, pkg.hip_api
+    nkv = a.prompt + a.warmup + a.steps + 64
+    cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128)
+    m = LA.LLM(cfg)
+    m.init_synthetic(20260101)
+    m.stage()
+    rng = np.random.default_rng(0)
+    prompt = rng.integers(0, cfg.vocab, size=a.prompt).astype(np.int32)
+    t0 = time.perf_counter()
+    m.extend(prompt, want_logits=False)
+    prefill_s = time.perf_counter() - t0
+    m.generate(a.warmup + 1)              # W untimed decode steps
+    t0 = time.perf_counter()              # generate() returns only after the stream has drained
+    ids, gpu_ns = m.generate(a.steps + 1)  # exactly K replays of the recorded decode step
+    wall = time.perf_counter() - t0
+    ctx_len = m.past()
+    tok_s = a.steps / wall
+
+    # the dominant kernel, timed live from its own dispatch timestamps over a few real steps
+    acc, n_prof = {}, 8
+    for _ in range(n_prof):
+        for k, v in m.profile_step():
+            acc[k] = acc.get(k, 0.0) + v / n_prof
+    up_ns = acc["moe.up"] / cfg.n_layer
+    up_bytes = moe_up_bytes(cfg)
+    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048> (expert-gathered Q4_K gate/up GEMV + SwiGLU)",
+            "achieved": round(up_bytes / (up_ns / 1e9) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": round(up_bytes / (up_ns / 1e9) / HBM_PEAK, 4), "traffic": None,
+            "bytes_per_launch": up_bytes, "avg_launch_us": round(up_ns / 1e3, 3), "launches_per_step": cfg.n_layer}
+    tb = token_bytes(cfg, ctx_len)
+    rec = {
+        "metric": "batch-1 decode tok/s (Q4_K MoE+DeltaNet)", "value": round(tok_s, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(wall / a.steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE config 5: synthetic random-init Qwen3-Next-shape model, %d layers "
+                               "(3 gated-DeltaNet + 1 gated-attention), 512 experts top-10 + shared, Q4_K weights "
+                               "drawn N(0,0.02) and quantised on the device by the reference's quantiser, fp16 KV "
+                               "cache, vocab 151936; prompt %d random ids then greedy decode at batch 1"
+                               % (cfg.n_layer, a.prompt),
+                   "context_at_end": ctx_len, "prefill": "token by token through the recorded step (%.1f tok/s, untimed)"
+                                                          % (a.prompt / prefill_s),
+                   "weights_GB": round(m.weight_bytes() / 1e9, 2), "dispatches_per_step": m.dispatches()},
+        "gpu_ms_per_step": round(gpu_ns / a.steps / 1e6, 4),
+        "token_bytes": tb, "token_roofline_tok_s": round(HBM_PEAK / tb, 1), "frac_of_token_roofline": round(tok_s * tb / HBM_PEAK, 4),
+        "step_kernel_us": {k: round(v / 1e3, 1) for k, v in sorted(acc.items(), key=lambda kv: -kv[1])},
+        "roofline": roof,
+        "gemv": gemv_rates(m, cfg, A, LA),
+    }
+    if not a.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline(m, cfg, LA, a.cpu_tokens)
+    m.close()
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

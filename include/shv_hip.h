@@ -300,8 +300,9 @@ typedef struct {
 int shv_enqueue(shv_ctx *ctx, uint32_t kind, const void *args, size_t args_bytes);
 
 /* DispatchMultiTimed / DispatchMultiMarked (vk/engine.go:893-935): run the sequence `iters`
- * times, block until done, return GPU time for the whole run in total_ns and, if per_op_ns is
- * not NULL (one slot per op, iters must be 1), the GPU time of each op. */
+ * times, block until done, return GPU time for the whole run in total_ns (first launch to last
+ * completion, gaps included) and, if per_op_ns is not NULL (one slot per op, iters must be 1),
+ * the time each op's kernels ran, from timestamps on the kernels themselves. */
 int shv_dispatch_multi(shv_ctx *ctx, const shv_op *ops, int n_ops, int iters,
                        uint64_t *total_ns, uint64_t *per_op_ns);
 

@@ -382,8 +382,7 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
                 "attn_decode: qkv, caches, norms, partial and out must be 16-byte aligned");
     dim3 grid(a.n_splits, a.n_head_kv, a.n_seq);
     for (int i = 0; i < a.seq_len; i++) {
-        hipLaunchKernelGGL(attn_decode_kernel, grid, dim3(kBlock), 0, ctx->stream, a, i, ctx->counters + shv_ctx::kCounterAttn);
-        SHV_HIP_CHECK(hipGetLastError());
+        SHV_LAUNCH(ctx, attn_decode_kernel, grid, dim3(kBlock), 0, a, i, ctx->counters + shv_ctx::kCounterAttn);
     }
     return SHV_OK;
 }

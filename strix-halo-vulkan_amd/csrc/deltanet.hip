@@ -131,7 +131,6 @@ int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
                 a.ring_slots, a.seq_len, a.conv - 1);
     SHV_REQUIRE(shv_aligned16(a.state) && shv_aligned16(a.conv1d), "dn_step: state and conv1d must be 16-byte aligned");
     dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
-    hipLaunchKernelGGL(dn_step_kernel, grid, dim3(kBlock), 0, ctx->stream, a);
-    SHV_HIP_CHECK(hipGetLastError());
+    SHV_LAUNCH(ctx, dn_step_kernel, grid, dim3(kBlock), 0, a);
     return SHV_OK;
 }

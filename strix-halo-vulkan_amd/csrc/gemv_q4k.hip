@@ -195,8 +195,7 @@ int launch_ntu(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, 
             raised = true;
         }
     }
-    hipLaunchKernelGGL((gemv_q4k_kernel<K, NT, U>), grid, block, lds, ctx->stream, a, ppw, t0);
-    SHV_HIP_CHECK(hipGetLastError());
+    SHV_LAUNCH(ctx, (gemv_q4k_kernel<K, NT, U>), grid, block, lds, a, ppw, t0);
     return SHV_OK;
 }
 

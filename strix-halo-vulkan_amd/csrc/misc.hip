@@ -66,9 +66,8 @@ int shv_launch_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a) {
     const long long groups = a->rows * (a->k / 64);
     const long long blocks = (groups + 255) / 256;
     SHV_REQUIRE(blocks < (1ll << 31), "dequant_q4k: %lld groups is too many for one launch", groups);
-    hipLaunchKernelGGL(dequant_q4k_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx->stream,
+    SHV_LAUNCH(ctx, dequant_q4k_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
                        static_cast<const uint8_t *>(a->w), a->dst, groups);
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
 
@@ -77,9 +76,8 @@ int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a) {
     long long blocks = (a->n + 255) / 256;
     const long long cap = static_cast<long long>(ctx->prop.multiProcessorCount) * 32;
     if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(fill_normal_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx->stream, a->dst,
+    SHV_LAUNCH(ctx, fill_normal_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, a->dst,
                        static_cast<long long>(a->n), a->seed, a->mean, a->std, a->half);
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
 
@@ -173,8 +171,7 @@ int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a) {
     SHV_REQUIRE(a->n_tok >= 1 && a->n_tok <= 65535 && a->n_embd >= 1 && a->vocab >= 1 && a->x_stride >= a->n_embd,
                 "embed: n_tok %d, n_embd %d, vocab %d, x_stride %d", a->n_tok, a->n_embd, a->vocab, a->x_stride);
     const int bx = (a->n_embd + 255) / 256;
-    hipLaunchKernelGGL(embed_kernel, dim3(bx < 8 ? bx : 8, a->n_tok), dim3(256), 0, ctx->stream, *a);
-    SHV_HIP_CHECK(hipGetLastError());
+    SHV_LAUNCH(ctx, embed_kernel, dim3(bx < 8 ? bx : 8, a->n_tok), dim3(256), 0, *a);
     return SHV_OK;
 }
 
@@ -188,15 +185,13 @@ int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a) {
     SHV_REQUIRE(cap >= 1 && a->n_rows <= 14, "argmax: %d rows is more than one launch covers", a->n_rows);
     if (nb > cap) nb = cap;
     if (nb > 256) nb = 256;
-    hipLaunchKernelGGL(argmax_kernel, dim3(nb, a->n_rows), dim3(256), 0, ctx->stream, *a, ctx->argmax_val, ctx->argmax_idx,
+    SHV_LAUNCH(ctx, argmax_kernel, dim3(nb, a->n_rows), dim3(256), 0, *a, ctx->argmax_val, ctx->argmax_idx,
                        ctx->counters + shv_ctx::kCounterArgmax);
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
 
 int shv_launch_advance(shv_ctx *ctx, const shv_advance_args *a) {
     SHV_REQUIRE(a->pos && a->n_seq >= 1, "advance: NULL pos or n_seq %d", a->n_seq);
-    hipLaunchKernelGGL(advance_kernel, dim3((a->n_seq + 63) / 64), dim3(64), 0, ctx->stream, *a);
-    SHV_HIP_CHECK(hipGetLastError());
+    SHV_LAUNCH(ctx, advance_kernel, dim3((a->n_seq + 63) / 64), dim3(64), 0, *a);
     return SHV_OK;
 }

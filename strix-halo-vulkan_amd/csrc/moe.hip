@@ -338,12 +338,11 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     const unsigned blocks = static_cast<unsigned>((a.n_expert + 1 + 3) / 4);
     int32_t *counter = ctx->counters + shv_ctx::kCounterRouter;
     switch (a.n_embd) {
-        case 2048: hipLaunchKernelGGL(moe_router_kernel<2048>, dim3(blocks), dim3(kBlock), 0, ctx->stream, a, counter); break;
-        case 1024: hipLaunchKernelGGL(moe_router_kernel<1024>, dim3(blocks), dim3(kBlock), 0, ctx->stream, a, counter); break;
-        case 512: hipLaunchKernelGGL(moe_router_kernel<512>, dim3(blocks), dim3(kBlock), 0, ctx->stream, a, counter); break;
+        case 2048: SHV_LAUNCH(ctx, moe_router_kernel<2048>, dim3(blocks), dim3(kBlock), 0, a, counter); break;
+        case 1024: SHV_LAUNCH(ctx, moe_router_kernel<1024>, dim3(blocks), dim3(kBlock), 0, a, counter); break;
+        case 512: SHV_LAUNCH(ctx, moe_router_kernel<512>, dim3(blocks), dim3(kBlock), 0, a, counter); break;
         default: return shv_set_error(SHV_E_INVALID, "moe_router: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
     }
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
 
@@ -360,24 +359,23 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
         case 2048: {
             constexpr int RPP = 64 / (2048 / 64);
             dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            hipLaunchKernelGGL(moe_up_kernel<2048>, grid, block, 0, ctx->stream, a);
+            SHV_LAUNCH(ctx, moe_up_kernel<2048>, grid, block, 0, a);
             break;
         }
         case 1024: {
             constexpr int RPP = 64 / (1024 / 64);
             dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            hipLaunchKernelGGL(moe_up_kernel<1024>, grid, block, 0, ctx->stream, a);
+            SHV_LAUNCH(ctx, moe_up_kernel<1024>, grid, block, 0, a);
             break;
         }
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
             dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            hipLaunchKernelGGL(moe_up_kernel<512>, grid, block, 0, ctx->stream, a);
+            SHV_LAUNCH(ctx, moe_up_kernel<512>, grid, block, 0, a);
             break;
         }
         default: return shv_set_error(SHV_E_INVALID, "moe_up: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
     }
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }
 
@@ -392,16 +390,15 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     switch (a.ffn) {
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
-            hipLaunchKernelGGL((moe_down_kernel<512, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, ctx->stream, a);
+            SHV_LAUNCH(ctx, (moe_down_kernel<512, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
             break;
         }
         case 256: {
             constexpr int RPP = 64 / (256 / 64);
-            hipLaunchKernelGGL((moe_down_kernel<256, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, ctx->stream, a);
+            SHV_LAUNCH(ctx, (moe_down_kernel<256, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
             break;
         }
         default: return shv_set_error(SHV_E_INVALID, "moe_down: ffn = %d; built for 256 and 512", a.ffn);
     }
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }

@@ -179,8 +179,7 @@ int shv_launch_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a) {
     const long long n_blocks = a->rows * (a->k / SHV_Q4K_BLOCK);
     const long long grid = (n_blocks + 31) / 32;
     SHV_REQUIRE(grid < (1ll << 31), "quantize_q4k: %lld super-blocks is too many for one launch", n_blocks);
-    hipLaunchKernelGGL(quantize_q4k_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, ctx->stream, a->src,
+    SHV_LAUNCH(ctx, quantize_q4k_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, a->src,
                        static_cast<uint8_t *>(a->dst), n_blocks);
-    SHV_HIP_CHECK(hipGetLastError());
     return SHV_OK;
 }

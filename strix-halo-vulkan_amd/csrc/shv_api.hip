@@ -67,6 +67,7 @@ void shv_destroy(shv_ctx *ctx) {
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->argmax_val) (void)hipFree(ctx->argmax_val);
     if (ctx->argmax_idx) (void)hipFree(ctx->argmax_idx);
+    for (hipEvent_t ev : ctx->mark_pool) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -209,33 +210,35 @@ int shv_dispatch_multi(shv_ctx *ctx, const shv_op *ops, int n_ops, int iters, ui
     SHV_REQUIRE(iters >= 1, "shv_dispatch_multi: iters %d", iters);
     SHV_REQUIRE(!ctx->capturing, "shv_dispatch_multi: not valid while recording");
     SHV_REQUIRE(per_op_ns == nullptr || iters == 1, "shv_dispatch_multi: per-op times need iters == 1");
-    std::vector<hipEvent_t> marks;
-    if (per_op_ns) {
-        marks.resize(n_ops + 1);
-        for (auto &m : marks) SHV_HIP_CHECK(hipEventCreate(&m));
-    }
+    // per-op times come from timestamps on the kernels themselves, so they hold no launch gap
+    ctx->marks.clear();
+    ctx->marking = per_op_ns != nullptr;
     int rc = SHV_OK;
     hipError_t e = hipEventRecord(ctx->ev_begin, ctx->stream);
-    if (per_op_ns && e == hipSuccess) e = hipEventRecord(marks[0], ctx->stream);
     for (int it = 0; it < iters && rc == SHV_OK && e == hipSuccess; it++)
-        for (int i = 0; i < n_ops && rc == SHV_OK && e == hipSuccess; i++) {
+        for (int i = 0; i < n_ops && rc == SHV_OK; i++) {
+            ctx->mark_op = i;
             rc = dispatch_one(ctx, ops[i].kind, ops[i].args, sizeof(ops[i].args));
-            if (per_op_ns && rc == SHV_OK) e = hipEventRecord(marks[i + 1], ctx->stream);
         }
+    ctx->marking = false;
     if (e == hipSuccess) e = hipEventRecord(ctx->ev_end, ctx->stream);
-    hipError_t es = hipStreamSynchronize(ctx->stream);
+    const hipError_t es = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess) e = es;
     ctx->submits++;
     if (rc == SHV_OK && e == hipSuccess) {
         float ms = 0;
         e = hipEventElapsedTime(&ms, ctx->ev_begin, ctx->ev_end);
         if (total_ns) *total_ns = static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
-        for (int i = 0; per_op_ns && i < n_ops && e == hipSuccess; i++) {
-            e = hipEventElapsedTime(&ms, marks[i], marks[i + 1]);
-            per_op_ns[i] = static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+        if (per_op_ns) {
+            for (int i = 0; i < n_ops; i++) per_op_ns[i] = 0;
+            for (const auto &m : ctx->marks) {
+                if (e != hipSuccess) break;
+                e = hipEventElapsedTime(&ms, ctx->mark_pool[m.start], ctx->mark_pool[m.stop]);
+                per_op_ns[m.op] += static_cast<uint64_t>(static_cast<double>(ms) * 1e6);
+            }
         }
     }
-    for (auto &m : marks) (void)hipEventDestroy(m);
+    ctx->marks.clear();
     if (rc != SHV_OK) return rc;
     if (e != hipSuccess) return shv_set_error(SHV_E_HIP, "shv_dispatch_multi: %s", hipGetErrorString(e));
     return SHV_OK;

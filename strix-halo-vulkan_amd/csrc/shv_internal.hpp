@@ -1,11 +1,13 @@
 // Internal declarations shared by the C-ABI layer and the kernel launchers.
 #pragma once
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <vector>
 
 #include "shv_hip.h"
 
@@ -23,6 +25,28 @@ struct shv_ctx {
     float *argmax_val = nullptr;
     int32_t *argmax_idx = nullptr;
     enum { kArgmaxBlocks = 512 };
+    // Per-kernel GPU timestamps for a marked dispatch: while `marking` is set every launch is
+    // bracketed by a pair of events taken from the dispatch packet itself, so an op's time is the
+    // time its kernels ran and holds no launch gap.
+    bool marking = false;
+    int mark_op = 0;
+    std::vector<hipEvent_t> mark_pool;
+    struct Mark { int op, start, stop; };
+    std::vector<Mark> marks;
+    hipError_t next_marks(hipEvent_t *s, hipEvent_t *e) {
+        const size_t need = marks.size() * 2 + 2;
+        while (mark_pool.size() < need) {
+            hipEvent_t ev;
+            const hipError_t rc = hipEventCreate(&ev);
+            if (rc != hipSuccess) return rc;
+            mark_pool.push_back(ev);
+        }
+        const int i = static_cast<int>(marks.size()) * 2;
+        marks.push_back({mark_op, i, i + 1});
+        *s = mark_pool[i];
+        *e = mark_pool[i + 1];
+        return hipSuccess;
+    }
     enum { kCounterRouter = 0, kCounterArgmax = 1, kCounterAttn = 16 };
 };
 
@@ -45,6 +69,19 @@ int shv_set_error(int code, const char *fmt, ...);
 #define SHV_REQUIRE(cond, ...)                                                                 \
     do {                                                                                       \
         if (!(cond)) return shv_set_error(SHV_E_INVALID, __VA_ARGS__);                         \
+    } while (0)
+
+// Every kernel launch of the library goes through here.
+#define SHV_LAUNCH(ctx, kern, grid, block, lds, ...)                                           \
+    do {                                                                                       \
+        if ((ctx)->marking) {                                                                  \
+            hipEvent_t ms_, me_;                                                               \
+            SHV_HIP_CHECK((ctx)->next_marks(&ms_, &me_));                                      \
+            hipExtLaunchKernelGGL(kern, grid, block, lds, (ctx)->stream, ms_, me_, 0, __VA_ARGS__); \
+        } else {                                                                               \
+            hipLaunchKernelGGL(kern, grid, block, lds, (ctx)->stream, __VA_ARGS__);            \
+        }                                                                                      \
+        SHV_HIP_CHECK(hipGetLastError());                                                      \
     } while (0)
 
 static inline bool shv_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
