@@ -161,7 +161,9 @@ typedef struct {
  * xn = RMSNorm(h)*gamma (gamma NULL: h is used as it is), logits = router*xn in float32, softmax,
  * the n_used largest probabilities in descending order (ties to the lower index), their sum
  * clamped at 2^-14, the normalised weights; weights[t][n_used] = sigmoid(shared_gate . xn)
- * (llm/moe.go:396-402).  logits is [T][n_expert+1], the last column the shared-gate logit. */
+ * (llm/moe.go:396-402).  logits is [T][n_expert+1], the last column the shared-gate logit.
+ * defer_route != 0 stops after the logits (topk and weights may then be NULL): the selection is
+ * left to shv_moe_up, which saves the router a cross-block hand-over inside the kernel. */
 typedef struct {
     const float *h;
     const float *gamma;
@@ -174,19 +176,26 @@ typedef struct {
     int32_t n_tok, n_embd, n_expert, n_used;
     float eps;
     int32_t h_stride;
+    int32_t defer_route;
 } shv_moe_router_args;
 
 /* Expert-gathered gate/up GEMV with SwiGLU (MoETrace.Experts/Shared, llm/moe.go:289-409;
  * llm_moe_gemv.comp MODE 0): act[t][s] = silu(Wg_e xn[t]) * (Wu_e xn[t]) for e = topk[t][s],
  * s < n_used, and for the shared expert in slot n_used.  Only the selected experts' rows are
- * read.  Banks are GGUF Q4_K: expert e's row j is row e*ffn + j, n_embd long. */
+ * read.  Banks are GGUF Q4_K: expert e's row j is row e*ffn + j, n_embd long.
+ * When logits is given ([T][n_expert+1] from a router run with defer_route) every block first
+ * routes its token from them exactly as the router would, and the selection is also stored to
+ * topk [T][n_used] and weights [T][n_used+1] for the down projection; otherwise topk is read. */
 typedef struct {
     const float *xn;
-    const int32_t *topk;
+    int32_t *topk;
     const void *gate_exps, *up_exps;
     const void *gate_sh, *up_sh;
     float *act;
     int32_t n_tok, n_embd, n_used, ffn;
+    const float *logits;
+    float *weights;
+    int32_t n_expert;
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +

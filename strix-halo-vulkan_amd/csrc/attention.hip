@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_arg
     {
         const int hh = tid >> 5, d0 = (tid & 31) * 8;
         float num[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        constexpr int MB = 8;
+        constexpr int MB = 16;
         for (int s0 = 0; s0 < n_active; s0 += MB) {
             float4 r0[MB], r1[MB];
 #pragma unroll

@@ -53,7 +53,9 @@ __device__ __forceinline__ void wave_pair_max(uint32_t &hi, uint32_t &lo) {
 // One wave routes one token: softmax over n_expert logits (n_expert <= 64*8), then n_used rounds of
 // arg-max.  Probabilities are formed as the reference forms them (exp of the logit minus the
 // maximum, times the reciprocal of their sum) so that equal logits stay equal probabilities.
-template <int PER>
+// AGENT: the logits were written earlier in this same kernel by other blocks and must be read
+// with device-scope loads; otherwise they come from an earlier kernel and plain loads do.
+template <int PER, bool AGENT>
 __device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *probs_lds) {
     const int lane = threadIdx.x & 63;
     float l[PER];
@@ -61,7 +63,7 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int e = lane + i * 64;
-        l[i] = e < n_expert ? load_agent(logits + e) : -INFINITY;
+        l[i] = e < n_expert ? (AGENT ? load_agent(logits + e) : logits[e]) : -INFINITY;
         mx = fmaxf(mx, l[i]);
     }
     mx = wave_max_all(mx);
@@ -173,16 +175,20 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
                 acc = fmaf(wv.w, xv.w, acc);
             }
             acc = wave_sum_all(acc);
-            if (lane == 0) store_agent(a.logits + static_cast<size_t>(t) * (a.n_expert + 1) + row, acc);
+            if (lane == 0) {
+                float *dst = a.logits + static_cast<size_t>(t) * (a.n_expert + 1) + row;
+                if (a.defer_route) *dst = acc; else store_agent(dst, acc);
+            }
         }
         __syncthreads();
     }
+    if (a.defer_route) return;  // the expert kernel routes from the logits
     // ---- the last block to arrive routes every token ----
     if (!arrive_last(counter, static_cast<int>(gridDim.x), &is_last)) return;
     for (int t = wave; t < a.n_tok; t += 4) {
         const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
         float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
-        route_token<8>(lg, a.n_expert, a.n_used, a.topk + static_cast<size_t>(t) * a.n_used, wt, probs[wave]);
+        route_token<8, true>(lg, a.n_expert, a.n_used, a.topk + static_cast<size_t>(t) * a.n_used, wt, probs[wave]);
         if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(load_agent(lg + a.n_expert)) : 0.f;
     }
 }
@@ -196,16 +202,39 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     __shared__ float xs[lds_padded(K)];
+    __shared__ float probs[512];
+    __shared__ int32_t s_topk[kMaxUsed];
+    __shared__ float s_w[kMaxUsed + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int slot = blockIdx.y, t = blockIdx.z;
     const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
     const int row = (blockIdx.x * 4 + wave) * RPP + rsub;  // row within the expert
     const bool live = row < a.ffn;
 
-    // issue the weight loads first: they do not depend on the staged vector
+    // the activation row is requested before anything else and staged further down
+    const float *x = a.xn + static_cast<size_t>(t) * K;
+    float xv[K / kBlock];
+#pragma unroll
+    for (int i = 0; i < K / kBlock; i++) xv[i] = x[tid + i * kBlock];
+
+    if (a.logits) {
+        // route this block's token from the router's logits (one wave), share the result
+        if (wave == 0) {
+            const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
+            route_token<8, false>(lg, a.n_expert, a.n_used, s_topk, s_w, probs);
+            if (lane == 0) s_w[a.n_used] = sigmoid_exact(lg[a.n_expert]);
+        }
+        __syncthreads();
+        if (blockIdx.x == 0 && blockIdx.y == 0) {
+            if (tid < a.n_used) a.topk[static_cast<size_t>(t) * a.n_used + tid] = s_topk[tid];
+            if (tid <= a.n_used) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + tid] = s_w[tid];
+        }
+    }
+
+    // the weight loads go out next: they do not depend on the staged vector
     const char *gbase, *ubase;
     if (slot < a.n_used) {
-        const int e = a.topk[static_cast<size_t>(t) * a.n_used + slot];
+        const int e = a.logits ? s_topk[slot] : a.topk[static_cast<size_t>(t) * a.n_used + slot];
         gbase = static_cast<const char *>(a.gate_exps) + static_cast<size_t>(e) * a.ffn * ROWB;
         ubase = static_cast<const char *>(a.up_exps) + static_cast<size_t>(e) * a.ffn * ROWB;
     } else {
@@ -217,12 +246,8 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     wg.load(gbase + roff, g);
     wu.load(ubase + roff, g);
 
-    const float *x = a.xn + static_cast<size_t>(t) * K;
 #pragma unroll
-    for (int i = 0; i < K / kBlock; i++) {
-        const int c = tid + i * kBlock;
-        xs[lds_slot(c)] = x[c];
-    }
+    for (int i = 0; i < K / kBlock; i++) xs[lds_slot(tid + i * kBlock)] = xv[i];
     __syncthreads();
     float xr[64], xs_lo, xs_hi;
     load_x_slice(xs, gi, xr, xs_lo, xs_hi);
@@ -329,7 +354,8 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
 
 int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     const shv_moe_router_args &a = *pa;
-    SHV_REQUIRE(a.h && a.router && a.logits && a.topk && a.weights, "moe_router: NULL h, router, logits, topk or weights");
+    SHV_REQUIRE(a.h && a.router && a.logits, "moe_router: NULL h, router or logits");
+    SHV_REQUIRE(a.defer_route || (a.topk && a.weights), "moe_router: NULL topk or weights");
     SHV_REQUIRE(a.n_tok >= 1, "moe_router: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_expert >= 1 && a.n_expert <= 512, "moe_router: n_expert %d, the routing wave covers up to 512", a.n_expert);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed && a.n_used <= a.n_expert, "moe_router: n_used %d of %d (at most %d)", a.n_used, a.n_expert, kMaxUsed);
@@ -349,6 +375,10 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
 int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     const shv_moe_up_args &a = *pa;
     SHV_REQUIRE(a.xn && a.topk && a.gate_exps && a.up_exps && a.gate_sh && a.up_sh && a.act, "moe_up: NULL argument");
+    if (a.logits) {
+        SHV_REQUIRE(a.weights, "moe_up: routing from logits needs somewhere to store the weights");
+        SHV_REQUIRE(a.n_expert >= 1 && a.n_expert <= 512 && a.n_used <= a.n_expert, "moe_up: n_expert %d, n_used %d", a.n_expert, a.n_used);
+    }
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);

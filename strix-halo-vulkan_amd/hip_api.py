@@ -57,14 +57,15 @@ class MoeRouterArgs(C.Structure):
                 ("shared_gate", C.c_void_p), ("xn", C.c_void_p), ("logits", C.c_void_p),
                 ("topk", C.c_void_p), ("weights", C.c_void_p), ("n_tok", C.c_int32),
                 ("n_embd", C.c_int32), ("n_expert", C.c_int32), ("n_used", C.c_int32),
-                ("eps", C.c_float), ("h_stride", C.c_int32)]
+                ("eps", C.c_float), ("h_stride", C.c_int32), ("defer_route", C.c_int32)]
 
 
 class MoeUpArgs(C.Structure):
     _fields_ = [("xn", C.c_void_p), ("topk", C.c_void_p), ("gate_exps", C.c_void_p),
                 ("up_exps", C.c_void_p), ("gate_sh", C.c_void_p), ("up_sh", C.c_void_p),
                 ("act", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
-                ("n_used", C.c_int32), ("ffn", C.c_int32)]
+                ("n_used", C.c_int32), ("ffn", C.c_int32), ("logits", C.c_void_p),
+                ("weights", C.c_void_p), ("n_expert", C.c_int32)]
 
 
 class MoeDownArgs(C.Structure):

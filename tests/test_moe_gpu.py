@@ -46,7 +46,7 @@ class MoeCase:
         r["xn"] = xn
         return r
 
-    def gpu(self, residual=False):
+    def gpu(self, residual=False, defer=False):
         c, T, H, E, used, ffn = self.ctx, self.T, self.H, self.E, self.used, self.ffn
         d = {k: c.upload(getattr(self, k)) for k in
              ("router", "shared_gate", "gate_exps", "up_exps", "down_exps", "gate_sh", "up_sh",
@@ -55,9 +55,10 @@ class MoeCase:
         topk, weights = c.alloc(T * used * 4), c.alloc(T * (used + 1) * 4)
         act, out = c.alloc(T * (used + 1) * ffn * 4), c.alloc(T * H * 4)
         ra = A.MoeRouterArgs(d["h"].ptr, d["gamma"].ptr, d["router"].ptr, d["shared_gate"].ptr, xn.ptr,
-                             logits.ptr, topk.ptr, weights.ptr, T, H, E, used, EPS, H)
+                             logits.ptr, topk.ptr, weights.ptr, T, H, E, used, EPS, H, 1 if defer else 0)
         ua = A.MoeUpArgs(xn.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr,
-                         d["up_sh"].ptr, act.ptr, T, H, used, ffn)
+                         d["up_sh"].ptr, act.ptr, T, H, used, ffn, logits.ptr if defer else None,
+                         weights.ptr if defer else None, E)
         da = A.MoeDownArgs(act.ptr, topk.ptr, weights.ptr, d["down_exps"].ptr, d["down_sh"].ptr,
                            d["res"].ptr if residual else None, out.ptr, T, H, used, ffn, H, H)
         ops = [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
@@ -75,8 +76,8 @@ def _margin(probs_row, used):
     return float(np.min((s[:-1] - s[1:]) / s[:-1]))
 
 
-def _check(case, residual=False):
-    want, got = case.oracle(), case.gpu(residual)
+def _check(case, residual=False, defer=False):
+    want, got = case.oracle(), case.gpu(residual, defer)
     assert O.rel_l2(got["xn"], want["xn"]) <= 1e-5
     assert O.rel_l2(got["logits"][:, :case.E], want["logits"]) <= 1e-4
     # top-k ids are demanded bit-exact; the inputs must not sit on a near-tie for that to be a
@@ -96,9 +97,12 @@ def _check(case, residual=False):
     return got
 
 
+@pytest.mark.parametrize("defer", [False, True])
 @pytest.mark.parametrize("T", [1, 4, 16])
-def test_moe_block_matches_oracle(ctx, T):
-    _check(MoeCase(ctx, seed=100 + T, E=64, used=10, T=T))
+def test_moe_block_matches_oracle(ctx, T, defer):
+    """defer: the selection is made by the expert kernel from the router's logits instead of by
+    the router's last block; both must give the reference's selection."""
+    _check(MoeCase(ctx, seed=100 + T, E=64, used=10, T=T), defer=defer)
 
 
 def test_moe_block_with_residual_and_few_experts(ctx):
@@ -109,9 +113,10 @@ def test_route_ties_go_to_the_lower_index(ctx):
     """Equal logits must select experts 0..used-1 in order (sort.SliceStable, llm/moe.go:249-252)
     with equal weights 1/used."""
     case = MoeCase(ctx, seed=9, E=64, used=10, T=3, tie_router=True)
-    got = case.gpu()
-    assert np.array_equal(got["topk"], np.tile(np.arange(10, dtype=np.int32), (3, 1)))
-    assert np.allclose(got["weights"][:, :10], 0.1, rtol=1e-6)
+    for defer in (False, True):
+        got = case.gpu(defer=defer)
+        assert np.array_equal(got["topk"], np.tile(np.arange(10, dtype=np.int32), (3, 1)))
+        assert np.allclose(got["weights"][:, :10], 0.1, rtol=1e-6)
     want = case.oracle()
     assert np.array_equal(want["topk"], got["topk"])
 
@@ -129,7 +134,7 @@ def test_moe_refuses_unsupported_shapes(ctx):
     d = ctx.alloc(1 << 16)
     with pytest.raises(shv.pkg.ShvError):
         ctx.enqueue(A.OP_MOE_ROUTER, A.MoeRouterArgs(d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr,
-                                                     d.ptr, 1, 2048, 1024, 10, EPS, 2048))
+                                                     d.ptr, 1, 2048, 1024, 10, EPS, 2048, 0))
     with pytest.raises(shv.pkg.ShvError):
         ctx.enqueue(A.OP_MOE_DOWN, A.MoeDownArgs(d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, None, d.ptr, 1,
                                                  2048, 10, 640, 2048, 2048))
@@ -166,4 +171,4 @@ def test_moe_full_config_bank(ctx):
     case.res = rng.standard_normal((T, H)).astype(np.float32)
     for b in dev.values():
         b.free()
-    _check(case, residual=True)
+    _check(case, residual=True, defer=True)

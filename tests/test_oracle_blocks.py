@@ -1,0 +1,465 @@
+"""Pins the oracle's block-level functions by what the mathematics fixes, since the reference
+holds no vector for them that can be used without its checkpoint: float64 re-derivations written
+independently in numpy, closed forms, invariants the reference's own tests state
+(llm/deltanet_test.go:234-320, llm/attn_test.go:87-129, llm/sample_test.go:17, llm/moe_test.go),
+and constructed edge cases.  Each check is chosen so that a plausible slip (a dropped term, a
+transposed state, a wrong head map, the wrong nibble order) fails it."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+EPS = 1e-6
+L = O.lib()
+
+
+def q4(rng, rows, k, std=0.02):
+    return O.quantize_q4k((rng.standard_normal((rows, k)) * std).astype(np.float32))
+
+
+def deq(q, k):
+    return O.dequant_q4k(q, k).astype(np.float64)
+
+
+# ------------------------------------------------------------------ dense helpers ----------------
+
+def test_gemv_is_dequant_then_dot():
+    rng = np.random.default_rng(1)
+    n, k = 96, 1024
+    wq = q4(rng, n, k)
+    x = rng.standard_normal(k).astype(np.float32)
+    want = deq(wq, k) @ x.astype(np.float64)
+    for threads in (1, 5):
+        got = O.gemv_q4k(wq, x, n, k, threads)
+        assert O.rel_l2(got, want) < 2e-6
+    assert np.array_equal(O.gemv_q4k(wq, x, n, k, 1), O.gemv_q4k(wq, x, n, k, 7))  # threads change no value
+    # sequential float32 accumulation, not pairwise and not float64: reproduce it exactly
+    w32 = O.dequant_q4k(wq, k)
+    s = np.float32(0)
+    for i in range(k):
+        s = np.float32(s + np.float32(w32[3, i] * x[i]))
+    assert O.gemv_q4k(wq, x, n, k, 1)[3] == s
+
+
+def test_rmsnorm_and_head_norm_against_float64():
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((5, 2048)) * 3).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(2048)).astype(np.float32)
+    want = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + EPS) * g
+    assert O.rel_l2(O.rmsnorm(x, g, EPS), want) < 1e-6
+    h = x.reshape(-1, 256).copy()
+    gh = g[:256].copy()
+    wanth = h.astype(np.float64) / np.sqrt((h.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + EPS) * gh
+    L.shv_ref_head_norm(O.F(h), O.F(gh), 256, h.shape[0], EPS)
+    assert O.rel_l2(h, wanth) < 1e-6
+    z = np.zeros((1, 64), np.float32)
+    assert np.array_equal(O.rmsnorm(z, np.ones(64, np.float32), EPS), z)  # eps keeps a zero row finite
+
+
+def test_scalar_activations():
+    for v in (-30.0, -3.5, 0.0, 0.7, 12.0):
+        assert abs(L.shv_ref_sigmoid(v) - 1 / (1 + np.exp(-v))) < 1e-7
+        assert abs(L.shv_ref_silu(v) - v / (1 + np.exp(-v))) < 1e-6 * max(1, abs(v))
+    # softplus: the reference's two documented edges (llm/deltanet.go:445-455)
+    assert L.shv_ref_softplus(20.5) == np.float32(20.5)          # identity above 20
+    assert L.shv_ref_softplus(-17.0) == 0.0                      # float32 add flushes to exactly 0
+    assert L.shv_ref_softplus(-16.0) > 0.0
+    for v in (-5.0, 0.0, 3.0, 19.9):
+        assert abs(L.shv_ref_softplus(v) - np.log1p(np.exp(v))) < 2e-7 * max(1, abs(v)) + 6e-8
+
+
+def test_argmax_first_maximum():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(5000).astype(np.float32)
+    assert L.shv_ref_argmax(O.F(x), x.size) == int(np.argmax(x))
+    x[[40, 4000]] = 9.0
+    assert L.shv_ref_argmax(O.F(x), x.size) == 40                 # ties go to the lowest id
+    n = np.full(10, np.nan, np.float32)
+    assert L.shv_ref_argmax(O.F(n), 10) == 0                      # NaN never wins
+
+
+# --------------------------------------------------------------------------- MoE ---------------
+
+def moe_setup(rng, H=512, E=16, used=4, ffn=256, T=3):
+    w = dict(router=(rng.standard_normal((E, H)) * 0.05).astype(np.float32),
+             shared_gate=(rng.standard_normal(H) * 0.05).astype(np.float32),
+             gate_exps=q4(rng, E * ffn, H), up_exps=q4(rng, E * ffn, H), down_exps=q4(rng, E * H, ffn),
+             gate_sh=q4(rng, ffn, H), up_sh=q4(rng, ffn, H), down_sh=q4(rng, H, ffn))
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    cfg = O.MoeCfg(H, E, used, ffn, ffn)
+    mw = O.MoeW(O.F(w["router"]), O.F(w["shared_gate"]), O.B(w["gate_exps"]), O.B(w["up_exps"]),
+                O.B(w["down_exps"]), O.B(w["gate_sh"]), O.B(w["up_sh"]), O.B(w["down_sh"]))
+    return cfg, mw, w, x
+
+
+def run_moe(cfg, mw, x):
+    T = x.shape[0]
+    r = dict(out=np.empty((T, cfg.n_embd), np.float32), logits=np.empty((T, cfg.n_expert), np.float32),
+             topk=np.empty((T, cfg.n_used), np.int32), weights=np.empty((T, cfg.n_used), np.float32),
+             moe_out=np.empty((T, cfg.n_embd), np.float32), sig=np.empty(T, np.float32))
+    L.shv_ref_moe_block(O.C.byref(cfg), O.C.byref(mw), O.F(x), T, O.F(r["out"]), O.F(r["logits"]), O.I(r["topk"]),
+                        O.F(r["weights"]), None, O.F(r["moe_out"]), O.F(r["sig"]), 1)
+    return r
+
+
+def test_route_against_numpy():
+    rng = np.random.default_rng(4)
+    cfg, mw, w, x = moe_setup(rng)
+    r = run_moe(cfg, mw, x)
+    lg = x.astype(np.float64) @ w["router"].astype(np.float64).T
+    assert O.rel_l2(r["logits"], lg) < 1e-6
+    p = np.exp(lg - lg.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    order = np.argsort(-p, axis=1, kind="stable")[:, :cfg.n_used]
+    assert np.array_equal(r["topk"], order)                       # descending, tie-free input
+    sel = np.take_along_axis(p, order, axis=1)
+    assert np.allclose(r["weights"], sel / sel.sum(axis=1, keepdims=True), rtol=1e-5)
+    assert np.allclose(r["weights"].sum(axis=1), 1, atol=1e-6)
+    assert (np.diff(r["weights"], axis=1) <= 0).all()
+
+
+def test_route_ties_clamp_and_softmax():
+    rng = np.random.default_rng(5)
+    cfg, mw, w, x = moe_setup(rng)
+    w["router"][:] = w["router"][0]                               # every logit equal
+    r = run_moe(cfg, mw, x)
+    assert np.array_equal(r["topk"], np.tile(np.arange(cfg.n_used, dtype=np.int32), (x.shape[0], 1)))
+    assert np.allclose(r["weights"], 1 / cfg.n_used)
+    # ties inside the selection keep ascending index order (sort.SliceStable, llm/moe.go:249-252)
+    w["router"][:] = 0
+    w["router"][[9, 2, 11], 0] = 1.0
+    xx = np.zeros_like(x)
+    xx[:, 0] = 2.0
+    rr = run_moe(cfg, mw, xx)
+    assert list(rr["topk"][0][:3]) == [2, 9, 11]
+    # softmax alone: sums to one, shift invariant
+    src = rng.standard_normal(64).astype(np.float32)
+    a, b = np.empty(64, np.float32), np.empty(64, np.float32)
+    L.shv_ref_softmax(O.F(a), O.F(src), 64)
+    L.shv_ref_softmax(O.F(b), O.F((src + 5).astype(np.float32)), 64)
+    assert abs(a.sum() - 1) < 1e-6 and np.allclose(a, b, atol=1e-7)
+    # the clamp at 2^-14 is inert unless the selected mass is below it: force it with many experts
+    # holding nearly all the mass outside the selection
+    cfg2 = O.MoeCfg(cfg.n_embd, cfg.n_expert, 1, cfg.ffn_expert, cfg.ffn_shared)
+    logits = np.empty((1, cfg.n_expert), np.float32)
+    probs = np.empty_like(logits)
+    topk = np.empty((1, 1), np.int32)
+    wn = np.empty((1, 1), np.float32)
+    L.shv_ref_moe_route(O.C.byref(cfg2), O.C.byref(mw), O.F(xx[:1]), 1, O.F(logits), O.F(probs), O.I(topk), O.F(wn))
+    assert abs(wn[0, 0] - 1.0) < 1e-6                             # one expert: weight is p/p = 1
+
+
+def test_moe_block_against_dense_float64():
+    """Brute force: dequantise every expert, mask by the selection, compare."""
+    rng = np.random.default_rng(6)
+    cfg, mw, w, x = moe_setup(rng)
+    r = run_moe(cfg, mw, x)
+    H, E, ffn = cfg.n_embd, cfg.n_expert, cfg.ffn_expert
+    G, U, D = deq(w["gate_exps"], H).reshape(E, ffn, H), deq(w["up_exps"], H).reshape(E, ffn, H), deq(w["down_exps"], ffn).reshape(E, H, ffn)
+    silu = lambda v: v / (1 + np.exp(-v))
+    for t in range(x.shape[0]):
+        xt = x[t].astype(np.float64)
+        routed = np.zeros(H)
+        for k in range(cfg.n_used):
+            e = r["topk"][t, k]
+            routed += r["weights"][t, k] * (D[e] @ (silu(G[e] @ xt) * (U[e] @ xt)))
+        assert O.rel_l2(r["moe_out"][t], routed) < 1e-5
+        sh = deq(w["down_sh"], ffn) @ (silu(deq(w["gate_sh"], H) @ xt) * (deq(w["up_sh"], H) @ xt))
+        gate = 1 / (1 + np.exp(-(w["shared_gate"].astype(np.float64) @ xt)))
+        assert abs(r["sig"][t] - gate) < 1e-6
+        assert O.rel_l2(r["out"][t], routed + gate * sh) < 1e-5
+
+
+# ---------------------------------------------------------------------- DeltaNet ---------------
+
+def dn_setup(rng, H=512, hk=2, hv=4, d=128):
+    qk, vw = hk * d, hv * d
+    cw = 2 * qk + vw
+    w = dict(qkv=q4(rng, cw, H, 0.05), z=q4(rng, vw, H, 0.05), alpha=q4(rng, hv, H, 0.05), beta=q4(rng, hv, H, 0.05),
+             out=q4(rng, H, vw), conv1d=(rng.standard_normal((cw, 4)) * 0.3).astype(np.float32),
+             a=(-np.exp(rng.standard_normal(hv))).astype(np.float32), dt=rng.standard_normal(hv).astype(np.float32),
+             norm=(1 + 0.1 * rng.standard_normal(d)).astype(np.float32))
+    cfg = O.DnCfg(H, d, hk, hv, 4, EPS, 0)
+    dw = O.DnW(O.B(w["qkv"]), O.B(w["z"]), O.B(w["alpha"]), O.B(w["beta"]), O.B(w["out"]), O.F(w["conv1d"]),
+               O.F(w["a"]), O.F(w["dt"]), O.F(w["norm"]))
+    return cfg, dw, w, (qk, vw, cw)
+
+
+def run_dn(cfg, dw, x, conv, S, divide=0, traces=False):
+    T = x.shape[0]
+    hv, hk, d = cfg.n_head_v, cfg.n_head_k, cfg.head_dim
+    res = np.empty((T, cfg.n_embd), np.float32)
+    tr = dict(qkv=np.empty((T, 2 * hk * d + hv * d), np.float32), qn=np.empty((T, hk, d), np.float32),
+              kn=np.empty((T, hk, d), np.float32), gate=np.empty((T, hv), np.float32),
+              bsig=np.empty((T, hv), np.float32), attn=np.empty((T, hv, d), np.float32),
+              final=np.empty((T, hv * d), np.float32))
+    L.shv_ref_deltanet_layer(O.C.byref(cfg), O.C.byref(dw), O.F(x), T, O.F(conv), O.F(S), O.F(res), O.F(tr["qkv"]),
+                             O.F(tr["qn"]), O.F(tr["kn"]), O.F(tr["gate"]), O.F(tr["bsig"]), O.F(tr["attn"]),
+                             O.F(tr["final"]), divide, 1)
+    return (res, tr) if traces else res
+
+
+def test_deltanet_chunk_split_is_bit_identical():
+    """llm/deltanet_test.go:280-320: 3 + 4 tokens == 7 tokens, output and state, bit for bit; and
+    the negative control: dropping the carried state must change the answer."""
+    rng = np.random.default_rng(7)
+    cfg, dw, w, (qk, vw, cw) = dn_setup(rng)
+    x = rng.standard_normal((7, cfg.n_embd)).astype(np.float32)
+    z = lambda: (np.zeros((cw, 3), np.float32), np.zeros((cfg.n_head_v, 128, 128), np.float32))
+    c1, s1 = z()
+    whole = run_dn(cfg, dw, x, c1, s1)
+    c2, s2 = z()
+    a = run_dn(cfg, dw, x[:3], c2, s2)
+    b = run_dn(cfg, dw, x[3:], c2, s2)
+    assert np.array_equal(np.concatenate([a, b]), whole)
+    assert np.array_equal(s1, s2) and np.array_equal(c1, c2)
+    c3, s3 = z()
+    fresh = run_dn(cfg, dw, x[3:], c3, s3)
+    assert not np.allclose(fresh, whole[3:], rtol=1e-3)
+
+
+def test_deltanet_against_independent_float64_recurrence():
+    """The layer re-derived in numpy float64 from the paper's form S <- S*g + k (beta (v - S^T k))^T,
+    o = S^T q / sqrt(d), with the state held UNtransposed: catches a transposed state, a wrong
+    head map, a conv window slip, a missing beta or decay."""
+    rng = np.random.default_rng(8)
+    cfg, dw, w, (qk, vw, cw) = dn_setup(rng)
+    hk, hv, d, H = cfg.n_head_k, cfg.n_head_v, cfg.head_dim, cfg.n_embd
+    T = 6
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    conv, S = np.zeros((cw, 3), np.float32), np.zeros((hv, d, d), np.float32)
+    res, tr = run_dn(cfg, dw, x, conv, S, traces=True)
+    X = x.astype(np.float64)
+    mixed = X @ deq(w["qkv"], H).T
+    zz = X @ deq(w["z"], H).T
+    al = X @ deq(w["alpha"], H).T
+    be = X @ deq(w["beta"], H).T
+    softplus = lambda v: np.where(v > 20, v, np.log1p(np.exp(np.minimum(v, 20))))
+    gate = softplus(al + w["dt"]) * w["a"]
+    bsig = 1 / (1 + np.exp(-be))
+    pad = np.concatenate([np.zeros((3, cw)), mixed])
+    convd = sum(pad[j:j + T] * w["conv1d"][:, j].astype(np.float64) for j in range(4))
+    act = convd / (1 + np.exp(-convd))
+    q, k, v = act[:, :qk].reshape(T, hk, d), act[:, qk:2 * qk].reshape(T, hk, d), act[:, 2 * qk:].reshape(T, hv, d)
+    qn = q / np.sqrt((q ** 2).sum(-1, keepdims=True) + EPS)
+    kn = k / np.sqrt((k ** 2).sum(-1, keepdims=True) + EPS)
+    Sm = np.zeros((hv, d, d))          # S[i][j]: key axis i, value axis j
+    out = np.zeros((T, hv, d))
+    for t in range(T):
+        for h in range(hv):
+            kk, qq = kn[t, h % hk], qn[t, h % hk]
+            Sm[h] *= np.exp(gate[t, h])
+            delta = (v[t, h] - Sm[h].T @ kk) * bsig[t, h]
+            Sm[h] += np.outer(kk, delta)
+            out[t, h] = Sm[h].T @ qq / np.sqrt(d)
+    assert O.rel_l2(tr["qkv"], mixed) < 1e-5
+    assert O.rel_l2(tr["gate"], gate) < 1e-5 and O.rel_l2(tr["bsig"], bsig) < 1e-6
+    assert O.rel_l2(tr["qn"], qn) < 1e-5 and O.rel_l2(tr["kn"], kn) < 1e-5
+    assert O.rel_l2(tr["attn"], out) < 1e-4
+    assert O.rel_l2(S, Sm.transpose(0, 2, 1)) < 1e-4              # the oracle stores S transposed
+    fin = out / np.sqrt((out ** 2).mean(-1, keepdims=True) + EPS) * w["norm"] * (1 / (1 + np.exp(-zz))).reshape(T, hv, d)
+    assert O.rel_l2(tr["final"], fin.reshape(T, -1)) < 1e-4
+    assert O.rel_l2(res, fin.reshape(T, -1) @ deq(w["out"], vw).T) < 1e-4
+    assert np.array_equal(conv, np.ascontiguousarray(tr["qkv"][-3:].T))  # history = last 3 rows, oldest first
+
+
+def test_delta_rule_closed_form_and_head_map():
+    """g = 0 (no decay), beta = 1, orthonormal keys: after T tokens S = sum_t k_t v_t^T and the
+    read-out of a stored key returns its value.  And the modulo head map against the divide map
+    (llm/deltanet_test.go:234-268): they must disagree when hv != hk."""
+    d, hk, hv, T = 128, 2, 4, 5
+    rng = np.random.default_rng(9)
+    Q, _ = np.linalg.qr(rng.standard_normal((d, d)))
+    kn = np.zeros((T, hk, d), np.float32)
+    for t in range(T):
+        kn[t, 0], kn[t, 1] = Q[:, t], Q[:, 10 + t]
+    v = rng.standard_normal((T, hv, d)).astype(np.float32)
+    gate = np.zeros((T, hv), np.float32)
+    beta = np.ones((T, hv), np.float32)
+    S = np.zeros((hv, d, d), np.float32)
+    out = np.empty((T, hv, d), np.float32)
+    k_of = np.array([h % hk for h in range(hv)], np.int32)
+    L.shv_ref_delta_rule(d, hk, hv, T, O.F(kn), O.F(kn), O.F(v), O.F(gate), O.F(beta), O.F(S), O.F(out), O.I(k_of))
+    for h in range(hv):
+        want = sum(np.outer(kn[t, h % hk].astype(np.float64), v[t, h].astype(np.float64)) for t in range(T))
+        assert np.allclose(S[h].T, want, atol=1e-5)               # S[i][j] lives at [j][i]
+        for t in range(T):
+            assert np.allclose(out[t, h] * np.sqrt(d), v[t, h], atol=1e-4)   # q = k_t reads v_t back
+    cfg, dw, w, (qk, vw, cw) = dn_setup(rng)
+    x = rng.standard_normal((3, cfg.n_embd)).astype(np.float32)
+    z = lambda: (np.zeros((cw, 3), np.float32), np.zeros((cfg.n_head_v, 128, 128), np.float32))
+    a = run_dn(cfg, dw, x, *z(), divide=0)
+    b = run_dn(cfg, dw, x, *z(), divide=1)
+    assert O.rel_l2(a, b) > 1e-2
+
+
+# --------------------------------------------------------------------- attention ---------------
+
+def attn_cfg(H=512, nh=4, nkv=2, d=64, rope=32):
+    return O.AttnCfg(H, nh, nkv, d, rope, 1e7, (O.C.c_int * 4)(6, 5, 5, 0), EPS)
+
+
+def test_rope_is_neox_on_the_first_dims_only():
+    """llm/attn_test.go:87,129: pairs (i, i + n_rot/2), dims past n_rot untouched, identity at
+    position 0, norm preserved; angles pos * base^(-2i/n_rot)."""
+    cfg = attn_cfg()
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((3, 4, 64)).astype(np.float32)
+    pos = np.array([0, 5, 1000], np.int32)
+    y = x.copy()
+    L.shv_ref_rope(O.C.byref(cfg), O.F(y), O.I(pos), 4, 64, 3)
+    assert np.array_equal(y[0], x[0])                              # position 0
+    assert np.array_equal(y[:, :, 32:], x[:, :, 32:])              # dims >= n_rot
+    assert np.allclose(np.linalg.norm(y, axis=-1), np.linalg.norm(x, axis=-1), rtol=1e-5)
+    half = 16
+    for t in (1, 2):
+        for i in range(half):
+            th = float(pos[t]) * (1e7 ** (-2.0 * i / 32))
+            c, s = np.cos(th), np.sin(th)
+            assert np.allclose(y[t, :, i], x[t, :, i] * c - x[t, :, i + half] * s, atol=2e-5)
+            assert np.allclose(y[t, :, i + half], x[t, :, i] * s + x[t, :, i + half] * c, atol=2e-5)
+
+
+def attn_setup(rng, cfg):
+    H, nh, nkv, d = cfg.n_embd, cfg.n_head, cfg.n_head_kv, cfg.head_dim
+    w = dict(q=q4(rng, nh * 2 * d, H, 0.05), k=q4(rng, nkv * d, H, 0.05), v=q4(rng, nkv * d, H, 0.05),
+             o=q4(rng, H, nh * d), qn=(1 + 0.1 * rng.standard_normal(d)).astype(np.float32),
+             kn=(1 + 0.1 * rng.standard_normal(d)).astype(np.float32))
+    aw = O.AttnW(O.B(w["q"]), O.B(w["k"]), O.B(w["v"]), O.B(w["o"]), O.F(w["qn"]), O.F(w["kn"]))
+    return aw, w
+
+
+def run_attn(cfg, aw, x, past, kc, vc):
+    T = x.shape[0]
+    out = np.empty((T, cfg.n_embd), np.float32)
+    pre = np.empty((T, cfg.n_head * cfg.head_dim), np.float32)
+    L.shv_ref_attn_layer(O.C.byref(cfg), O.C.byref(aw), O.F(x), T, past, O.H(kc), O.H(vc), O.F(out), None, O.F(pre), 1)
+    return out, pre
+
+
+def test_attention_against_independent_float64():
+    """Causal GQA with a query gate, re-derived in numpy float64 on the half-rounded K and V."""
+    cfg = attn_cfg()
+    rng = np.random.default_rng(11)
+    aw, w = attn_setup(rng, cfg)
+    H, nh, nkv, d, T = cfg.n_embd, cfg.n_head, cfg.n_head_kv, cfg.head_dim, 7
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    kc, vc = np.zeros((16, nkv, d), np.uint16), np.zeros((16, nkv, d), np.uint16)
+    out, pre = run_attn(cfg, aw, x, 0, kc, vc)
+    X = x.astype(np.float64)
+    qg = (X @ deq(w["q"], H).T).reshape(T, nh, 2, d)
+    q, gate = qg[:, :, 0], qg[:, :, 1]
+    k = (X @ deq(w["k"], H).T).reshape(T, nkv, d)
+    v = (X @ deq(w["v"], H).T).reshape(T, nkv, d)
+    hn = lambda a, g: a / np.sqrt((a ** 2).mean(-1, keepdims=True) + EPS) * g
+
+    def rope(a):
+        a = a.copy()
+        for t in range(T):
+            for i in range(16):
+                th = t * (1e7 ** (-2.0 * i / 32))
+                x0, x1 = a[t, :, i].copy(), a[t, :, i + 16].copy()
+                a[t, :, i], a[t, :, i + 16] = x0 * np.cos(th) - x1 * np.sin(th), x0 * np.sin(th) + x1 * np.cos(th)
+        return a
+
+    q, k = rope(hn(q, w["qn"])), rope(hn(k, w["kn"]))
+    k16 = k.astype(np.float16).astype(np.float64)
+    v16 = v.astype(np.float16).astype(np.float64)
+    want = np.zeros((T, nh, d))
+    for t in range(T):
+        for h in range(nh):
+            s = k16[:t + 1, h // (nh // nkv)] @ q[t, h] / np.sqrt(d)
+            p = np.exp(s - s.max())
+            want[t, h] = (p / p.sum()) @ v16[:t + 1, h // (nh // nkv)]
+    assert O.rel_l2(pre, want.reshape(T, -1)) < 5e-4               # halves of K,V may round apart
+    gated = want * (1 / (1 + np.exp(-gate)))
+    assert O.rel_l2(out, gated.reshape(T, -1) @ deq(w["o"], nh * d).T) < 5e-4
+    assert np.array_equal(vc[:T].view(np.float16), v.astype(np.float32).astype(np.float16)) or \
+        np.count_nonzero(vc[:T].view(np.float16) != v.astype(np.float32).astype(np.float16)) < vc[:T].size // 50
+
+
+def test_attention_cache_steps_equal_one_pass():
+    """Seven tokens at once == 4 then 3 over the carried cache, bit for bit: the generalisation to a
+    non-empty cache changes nothing about the reference's whole-prompt function."""
+    cfg = attn_cfg()
+    rng = np.random.default_rng(12)
+    aw, w = attn_setup(rng, cfg)
+    x = rng.standard_normal((7, cfg.n_embd)).astype(np.float32)
+    mk = lambda: (np.zeros((16, cfg.n_head_kv, cfg.head_dim), np.uint16), np.zeros((16, cfg.n_head_kv, cfg.head_dim), np.uint16))
+    kc, vc = mk()
+    whole, _ = run_attn(cfg, aw, x, 0, kc, vc)
+    kc2, vc2 = mk()
+    a, _ = run_attn(cfg, aw, x[:4], 0, kc2, vc2)
+    b, _ = run_attn(cfg, aw, x[4:], 4, kc2, vc2)
+    assert np.array_equal(np.concatenate([a, b]), whole)
+    assert np.array_equal(kc, kc2) and np.array_equal(vc, vc2)
+
+
+# ------------------------------------------------------------------- token loop ----------------
+
+def test_model_loop_chunk_split_and_composition():
+    """Pre-norm residual composition (attn every 2nd layer here): the loop in pieces equals the loop
+    at once, and the hidden state equals the layers applied by hand."""
+    rng = np.random.default_rng(13)
+
+    class Cfg:
+        n_layer, n_embd, vocab, attn_every, rms_eps = 2, 512, 300, 2, EPS
+        n_expert, n_expert_used, ffn_expert = 8, 2, 256
+        ssm_head_dim, ssm_head_k, ssm_head_v, ssm_conv = 128, 2, 4, 4
+        n_head, n_head_kv, head_dim, rope_dims, rope_base = 4, 2, 64, 32, 1e7
+
+    c = Cfg
+    H, d = c.n_embd, c.ssm_head_dim
+    qk, vw = c.ssm_head_k * d, c.ssm_head_v * d
+    t = {"token_embd.weight": rng.standard_normal((c.vocab, H)).astype(np.float16).view(np.uint16),
+         "output_norm.weight": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32),
+         "output.weight": q4(rng, c.vocab, H)}
+    for l in range(c.n_layer):
+        b = lambda n: "blk.%d.%s.weight" % (l, n)
+        t[b("attn_norm")] = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+        t[b("post_attention_norm")] = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+        if (l + 1) % c.attn_every == 0:
+            t[b("attn_q")], t[b("attn_k")], t[b("attn_v")] = q4(rng, c.n_head * 2 * c.head_dim, H), q4(rng, c.n_head_kv * c.head_dim, H), q4(rng, c.n_head_kv * c.head_dim, H)
+            t[b("attn_output")] = q4(rng, H, c.n_head * c.head_dim)
+            t[b("attn_q_norm")] = np.ones(c.head_dim, np.float32)
+            t[b("attn_k_norm")] = np.ones(c.head_dim, np.float32)
+        else:
+            t[b("attn_qkv")], t[b("attn_gate")] = q4(rng, 2 * qk + vw, H), q4(rng, vw, H)
+            t[b("ssm_alpha")], t[b("ssm_beta")], t[b("ssm_out")] = q4(rng, c.ssm_head_v, H), q4(rng, c.ssm_head_v, H), q4(rng, H, vw)
+            t[b("ssm_conv1d")] = (rng.standard_normal((2 * qk + vw, 4)) * 0.3).astype(np.float32)
+            t[b("ssm_a")] = (-np.exp(rng.standard_normal(c.ssm_head_v))).astype(np.float32)
+            t[b("ssm_dt")] = rng.standard_normal(c.ssm_head_v).astype(np.float32)
+            t[b("ssm_norm")] = np.ones(d, np.float32)
+        t[b("ffn_gate_inp")] = (rng.standard_normal((c.n_expert, H)) * 0.05).astype(np.float32)
+        t[b("ffn_gate_inp_shexp")] = (rng.standard_normal(H) * 0.05).astype(np.float32)
+        t[b("ffn_gate_exps")], t[b("ffn_up_exps")] = q4(rng, c.n_expert * c.ffn_expert, H), q4(rng, c.n_expert * c.ffn_expert, H)
+        t[b("ffn_down_exps")] = q4(rng, c.n_expert * H, c.ffn_expert)
+        t[b("ffn_gate_shexp")], t[b("ffn_up_shexp")], t[b("ffn_down_shexp")] = q4(rng, c.ffn_expert, H), q4(rng, c.ffn_expert, H), q4(rng, H, c.ffn_expert)
+    ids = rng.integers(0, c.vocab, size=6).astype(np.int32)
+    m1 = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
+    lg1, hd1 = m1.extend(ids, threads=1)
+    m2 = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
+    m2.extend(ids[:2], threads=1)
+    lg2, hd2 = m2.extend(ids[2:], threads=1)
+    assert np.array_equal(lg1, lg2) and np.array_equal(hd1, hd2) and m1.past == m2.past == 6
+    # by hand, one token from an empty state: x + dn(norm x); + moe(norm .); then attention layer
+    m3 = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
+    _, hd3 = m3.extend(ids[:1], threads=1)
+    x = t["token_embd.weight"][ids[0]].view(np.float16).astype(np.float32)[None]
+    for l in range(c.n_layer):
+        lw = m3.layers[l]
+        b = lambda n: t["blk.%d.%s.weight" % (l, n)]
+        xn = O.rmsnorm(x, b("attn_norm"), EPS)
+        y = np.empty_like(x)
+        if (l + 1) % c.attn_every == 0:
+            kc, vc = np.zeros((16, c.n_head_kv, c.head_dim), np.uint16), np.zeros((16, c.n_head_kv, c.head_dim), np.uint16)
+            L.shv_ref_attn_layer(O.C.byref(m3.mcfg.attn), O.C.byref(lw.attn), O.F(xn), 1, 0, O.H(kc), O.H(vc), O.F(y), None, None, 1)
+        else:
+            conv, S = np.zeros((2 * qk + vw, 3), np.float32), np.zeros((c.ssm_head_v, d, d), np.float32)
+            L.shv_ref_deltanet_layer(O.C.byref(m3.mcfg.dn), O.C.byref(lw.dn), O.F(xn), 1, O.F(conv), O.F(S), O.F(y),
+                                     None, None, None, None, None, None, None, 0, 1)
+        x = x + y
+        xn = O.rmsnorm(x, b("post_attention_norm"), EPS)
+        L.shv_ref_moe_block(O.C.byref(m3.mcfg.moe), O.C.byref(lw.moe), O.F(xn), 1, O.F(y), None, None, None, None, None, None, 1)
+        x = x + y
+    assert np.array_equal(x[0], hd3)
