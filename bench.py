@@ -146,6 +146,9 @@ def main():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--cpu-tokens", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy, the known-size kernel that "
+                         "hardware-counter readings of HBM traffic are scaled by")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs the token loop on ONE GPU (one process, one stream); "
@@ -201,6 +204,17 @@ def main():
         "roofline": roof,
         "gemv": gemv_rates(m, cfg, A, LA),
     }
+    if a.pmc_copy:
+        import ctypes as C
+        H = A.load()
+        n = 256 << 20
+        src, dst = C.c_void_p(), C.c_void_p()
+        A.check(H.shv_alloc(m.ctx, n, C.byref(src)))
+        A.check(H.shv_alloc(m.ctx, n, C.byref(dst)))
+        A.check(H.shv_zero(m.ctx, src, n))
+        A.check(H.shv_copy(m.ctx, dst, src, n))
+        A.check(H.shv_sync(m.ctx))
+        rec["pmc_copy_bytes"] = n
     if not a.no_cpu:
         rec["cpu_baseline"] = cpu_baseline(m, cfg, LA, a.cpu_tokens)
     m.close()

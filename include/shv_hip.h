@@ -162,8 +162,8 @@ typedef struct {
  * the n_used largest probabilities in descending order (ties to the lower index), their sum
  * clamped at 2^-14, the normalised weights; weights[t][n_used] = sigmoid(shared_gate . xn)
  * (llm/moe.go:396-402).  logits is [T][n_expert+1], the last column the shared-gate logit.
- * defer_route != 0 stops after the logits (topk and weights may then be NULL): the selection is
- * left to shv_moe_up, which saves the router a cross-block hand-over inside the kernel. */
+ * defer_route != 0 stops after the logits (topk and weights may then be NULL) and leaves the
+ * selection to shv_moe_up, which can make it from the logits in its own prologue. */
 typedef struct {
     const float *h;
     const float *gamma;

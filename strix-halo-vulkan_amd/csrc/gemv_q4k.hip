@@ -31,10 +31,11 @@ struct GemvBatch {
     uint4 hdr[U], q0[U], q1[U];
     int row[U];
 
-    __device__ __forceinline__ void load(const char *wbase, int g, int rsub, long long pass, int n) {
+    // the batch's passes are `stride` apart: pass, pass + stride, ...
+    __device__ __forceinline__ void load(const char *wbase, int g, int rsub, long long pass, long long stride, int n) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const long long r = (pass + u) * RPP + rsub;
+            const long long r = (pass + u * stride) * RPP + rsub;
             row[u] = r < n ? static_cast<int>(r) : -1;
             const char *rp = wbase + static_cast<size_t>(row[u] < 0 ? 0 : row[u]) * ROWB;
             hdr[u] = load_stream16(rp);
@@ -62,9 +63,11 @@ struct GemvBatch {
     }
 };
 
-// U is the number of passes a wave loads together; passes_per_wave is a multiple of it.
+// The grid's waves share the passes round-robin: wave w takes passes w, w + W, w + 2W, ... (W waves
+// in the grid), so at any moment the chip streams one contiguous window of rows and no wave has
+// more than one pass more than another.  U passes are loaded together; n_batches batches a wave.
 template <int K, int NT, int U>
-__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int passes_per_wave, int t0) {
+__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int n_batches, int t0) {
     constexpr int LPR = K / 64;   // lanes per row
     constexpr int XPAD = K + K / 64 * 4;
     extern __shared__ float smem[];
@@ -77,12 +80,13 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     const int sb = gi >> 2, g = gi & 3;
     const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
     const int n = a.n;
-    const long long first_pass = (static_cast<long long>(blockIdx.x) * kWavesPerBlock + wave) * passes_per_wave;
+    const long long first_pass = static_cast<long long>(blockIdx.x) * kWavesPerBlock + wave;
+    const long long stride = static_cast<long long>(gridDim.x) * kWavesPerBlock;
 
     // The first batch of weights does not depend on the activations: its loads go out before
     // the prologue so that HBM latency and the staging of x overlap.
     GemvBatch<K, NT, U> A, B;
-    A.load(wbase, g, rsub, first_pass, n);
+    A.load(wbase, g, rsub, first_pass, stride, n);
 
     // ---- stage pro(x) in LDS ----
 #pragma unroll
@@ -172,13 +176,13 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     }
 
     const NibbleConsts nc = nibble_consts();
-    const int nb = passes_per_wave / U;  // batches, double-buffered
+    const int nb = n_batches;  // double-buffered
     for (int b = 0; b < nb; b += 2) {
         const bool has_b = b + 1 < nb;
-        if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U, n);
+        if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U * stride, stride, n);
         A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
         if (has_b) {
-            if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U, n);
+            if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U * stride, stride, n);
             B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
         }
     }
@@ -213,20 +217,17 @@ template <int K>
 int launch_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     constexpr int RPP = 64 / (K / 64);
     const long long passes = (static_cast<long long>(a.n) + RPP - 1) / RPP;
-    // One round of resident waves (two per SIMD at this kernel's register count): every wave of
-    // the grid is on the chip at once and streams its share of the rows.  Up to four passes are
-    // loaded together; longer shares run as double-buffered batches of four.
-    const long long resident = static_cast<long long>(ctx->prop.multiProcessorCount) * 4 * 2;
-    long long ppw = (passes + resident - 1) / resident;
-    if (ppw < 1) ppw = 1;
-    int u = static_cast<int>(ppw);
-    if (ppw > 4) {
-        ppw = (ppw + 3) / 4 * 4;
-        u = 4;
-    }
-    const long long waves = (passes + ppw - 1) / ppw;
-    const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-    SHV_REQUIRE(blocks > 0 && blocks < (1ll << 31), "gemv_q4k: grid of %lld blocks", blocks);
+    // One round of resident blocks (two waves per SIMD at this kernel's register count, i.e. two
+    // blocks per CU): every wave of the grid is on the chip at once.  Up to four passes of a wave
+    // are loaded together; longer shares run as double-buffered batches of four.
+    const long long resident = static_cast<long long>(ctx->prop.multiProcessorCount) * 2;
+    long long blocks = (passes + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > resident) blocks = resident;
+    const long long waves = blocks * kWavesPerBlock;
+    const long long iters = (passes + waves - 1) / waves;
+    const int u = iters < 4 ? static_cast<int>(iters) : 4;
+    const long long ppw = (iters + u - 1) / u;  // batches per wave
+    SHV_REQUIRE(blocks > 0 && ppw < (1ll << 31), "gemv_q4k: grid of %lld blocks", blocks);
     dim3 grid(static_cast<unsigned>(blocks)), block(kBlock);
     // more than kMaxTok rows: several launches of up to kMaxTok rows each over the same weights
     for (int t0 = 0; t0 < a.n_tok; t0 += kMaxTok) {

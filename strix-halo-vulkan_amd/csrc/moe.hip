@@ -1,4 +1,4 @@
-// MoE FFN decode step: router (+softmax/top-k in the last block to finish), expert-gathered
+// MoE FFN decode step: router logits, softmax/top-k selection, expert-gathered
 // gate/up GEMV with SwiGLU, down GEMV with weighting and combine.  Only the rows of the selected
 // experts (and the shared one) are read from HBM.
 #include "shv_device.hpp"
@@ -50,50 +50,11 @@ __device__ __forceinline__ void wave_pair_max(uint32_t &hi, uint32_t &lo) {
     lo = bl;
 }
 
-// One wave routes one token: softmax over n_expert logits (n_expert <= 64*8), then n_used rounds of
-// arg-max.  Probabilities are formed as the reference forms them (exp of the logit minus the
-// maximum, times the reciprocal of their sum) so that equal logits stay equal probabilities.
-// AGENT: the logits were written earlier in this same kernel by other blocks and must be read
-// with device-scope loads; otherwise they come from an earlier kernel and plain loads do.
-template <int PER, bool AGENT>
-__device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *probs_lds) {
+// n_used rounds of arg-max over the wave's candidates: the general selection, used when ties make
+// the shortcut below ambiguous.  kh/kl hold (bits of p, 0x7FFFFFFF - index); (0, 0) is empty.
+template <int PER>
+__device__ void select_by_rounds(uint32_t *kh, uint32_t *kl, int n_used, int32_t *sel_e, float *sel_w) {
     const int lane = threadIdx.x & 63;
-    float l[PER];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int e = lane + i * 64;
-        l[i] = e < n_expert ? (AGENT ? load_agent(logits + e) : logits[e]) : -INFINITY;
-        mx = fmaxf(mx, l[i]);
-    }
-    mx = wave_max_all(mx);
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int e = lane + i * 64;
-        if (e < n_expert) probs_lds[e] = expf(l[i] - mx);
-    }
-    __builtin_amdgcn_wave_barrier();
-    // The reference adds the exponentials one after another in index order; a tree over the wave
-    // differs from that in the last bits of the sum only, and the sum scales every probability
-    // alike, so neither the order of the experts nor the normalised weights move with it.
-    float sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int e = lane + i * 64;
-        if (e < n_expert) sum += probs_lds[e];
-    }
-    sum = wave_sum_all(sum);
-    const float inv = 1.f / sum;
-    uint32_t kh[PER], kl[PER];  // (0, 0) marks an empty or already taken candidate
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int e = lane + i * 64;
-        kh[i] = e < n_expert ? __float_as_uint(probs_lds[e] * inv) : 0u;
-        kl[i] = e < n_expert ? static_cast<uint32_t>(0x7FFFFFFF - e) : 0u;
-    }
-    // lane k keeps the k-th pick; the running sum is uniform across the wave
-    float my_w = 0.f, wsum = 0.f;
-    int my_e = 0;
 #pragma unroll 1
     for (int k = 0; k < n_used; k++) {
         uint32_t bh = 0u, bl = 0u;
@@ -107,27 +68,113 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
 #pragma unroll
         for (int i = 0; i < PER; i++)
             if (kh[i] == bh && kl[i] == bl) kh[i] = kl[i] = 0u;
-        const float w = __uint_as_float(bh);
-        if (lane == k) {
-            my_e = 0x7FFFFFFF - static_cast<int>(bl);
-            my_w = w;
+        if (lane == 0) {
+            sel_e[k] = 0x7FFFFFFF - static_cast<int>(bl);
+            sel_w[k] = __uint_as_float(bh);
         }
-        wsum += w;  // slot order, float32: the reference's sum
     }
+}
+
+// One wave routes one token: softmax over n_expert logits (n_expert <= 64*PER), the n_used largest
+// probabilities in descending order with ties to the lower index, their sum in slot order clamped
+// at 2^-14, the normalised weights.  Probabilities are formed as the reference forms them (exp of
+// the logit minus the maximum, times the reciprocal of their sum) so equal logits stay equal
+// probabilities; the reference adds the exponentials one after another where a tree is used
+// here, which moves only the last bits of a factor common to every probability.
+//
+// Selection: the n_used-th largest of the 64 per-lane maxima bounds the n_used-th largest key from
+// below, so only keys at or above it can be selected.  Those few candidates (found by a bitwise
+// search with wave ballots) are compacted into LDS and ranked against each other.
+// lds: scratch of at least 192 floats.
+template <int PER, bool AGENT>
+__device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *lds) {
+    const int lane = threadIdx.x & 63;
+    uint32_t *cand_p = reinterpret_cast<uint32_t *>(lds);       // [64]
+    int32_t *cand_e = reinterpret_cast<int32_t *>(lds + 64);    // [64]
+    int32_t *sel_e = reinterpret_cast<int32_t *>(lds + 128);    // [kMaxUsed]
+    float *sel_w = lds + 128 + kMaxUsed;                        // [kMaxUsed]
+    float l[PER];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        l[i] = e < n_expert ? (AGENT ? load_agent(logits + e) : logits[e]) : -INFINITY;
+        mx = fmaxf(mx, l[i]);
+    }
+    mx = wave_max_all(mx);
+    float ex[PER];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        ex[i] = e < n_expert ? expf(l[i] - mx) : 0.f;
+        sum += ex[i];
+    }
+    sum = wave_sum_all(sum);
+    const float inv = 1.f / sum;
+    uint32_t kh[PER], kl[PER];
+    uint32_t lane_max = 0u;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int e = lane + i * 64;
+        kh[i] = e < n_expert ? __float_as_uint(ex[i] * inv) : 0u;
+        kl[i] = e < n_expert ? static_cast<uint32_t>(0x7FFFFFFF - e) : 0u;
+        lane_max = kh[i] > lane_max ? kh[i] : lane_max;
+    }
+    // thr = the n_used-th largest lane maximum: the largest v with at least n_used lanes >= v
+    uint32_t thr = 0u;
+#pragma unroll 1
+    for (int b = 30; b >= 0; b--) {
+        const uint32_t c = thr | (1u << b);
+        if (__popcll(__ballot(lane_max >= c)) >= n_used) thr = c;
+    }
+    // compact the keys at or above it
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const bool pred = kl[i] != 0u && kh[i] >= thr;
+        const unsigned long long mask = __ballot(pred);
+        const int pos = total + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                                 __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)));
+        if (pred && pos < 64) {
+            cand_p[pos] = kh[i];
+            cand_e[pos] = lane + i * 64;
+        }
+        total += __popcll(mask);
+    }
+    if (total > 64 || n_expert < 64) {
+        // many equal probabilities (or fewer experts than lanes): take the general road
+        select_by_rounds<PER>(kh, kl, n_used, sel_e, sel_w);
+    } else {
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t my_p = lane < total ? cand_p[lane] : 0u;
+        const int my_e = lane < total ? cand_e[lane] : 0x7FFFFFFF;
+        int rank = 0;
+        for (int j = 0; j < total; j++) {
+            const uint32_t op = cand_p[j];
+            const int oe = cand_e[j];
+            rank += (op > my_p || (op == my_p && oe < my_e)) ? 1 : 0;
+        }
+        if (lane < total && rank < n_used) {
+            sel_e[rank] = my_e;
+            sel_w[rank] = __uint_as_float(my_p);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    float wsum = 0.f;
+    for (int k = 0; k < n_used; k++) wsum += sel_w[k];  // slot order, float32: the reference's sum
     if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
     if (lane < n_used) {
-        topk[lane] = my_e;
-        weights[lane] = my_w / wsum;
+        topk[lane] = sel_e[lane];
+        weights[lane] = sel_w[lane] / wsum;
     }
 }
 
 // grid: ceil((n_expert+1)/4) blocks of 4 waves, one float32 router row per wave.
 template <int H>
-__global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args a, int32_t *counter) {
+__global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args a) {
     __shared__ float xs[H];
     __shared__ float red[4];
-    __shared__ float probs[4][512];
-    __shared__ int is_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = blockIdx.x * 4 + wave;  // n_expert = the shared-gate row
     const bool has_row = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
@@ -175,22 +222,20 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
                 acc = fmaf(wv.w, xv.w, acc);
             }
             acc = wave_sum_all(acc);
-            if (lane == 0) {
-                float *dst = a.logits + static_cast<size_t>(t) * (a.n_expert + 1) + row;
-                if (a.defer_route) *dst = acc; else store_agent(dst, acc);
-            }
+            if (lane == 0) a.logits[static_cast<size_t>(t) * (a.n_expert + 1) + row] = acc;
         }
         __syncthreads();
     }
-    if (a.defer_route) return;  // the expert kernel routes from the logits
-    // ---- the last block to arrive routes every token ----
-    if (!arrive_last(counter, static_cast<int>(gridDim.x), &is_last)) return;
-    for (int t = wave; t < a.n_tok; t += 4) {
-        const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
-        float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
-        route_token<8, true>(lg, a.n_expert, a.n_used, a.topk + static_cast<size_t>(t) * a.n_used, wt, probs[wave]);
-        if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(load_agent(lg + a.n_expert)) : 0.f;
-    }
+}
+
+// grid: n_tok blocks of one wave: the selection for one token from its finished logits.
+__global__ __launch_bounds__(64) void moe_route_kernel(shv_moe_router_args a) {
+    __shared__ float probs[192];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
+    float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
+    route_token<8, false>(lg, a.n_expert, a.n_used, a.topk + static_cast<size_t>(t) * a.n_used, wt, probs);
+    if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(lg[a.n_expert]) : 0.f;
 }
 
 // ------------------------------------------------------------------------------- up ----------
@@ -202,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     __shared__ float xs[lds_padded(K)];
-    __shared__ float probs[512];
+    __shared__ float probs[192];
     __shared__ int32_t s_topk[kMaxUsed];
     __shared__ float s_w[kMaxUsed + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -362,13 +407,15 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     SHV_REQUIRE(a.h_stride >= a.n_embd, "moe_router: h_stride %d < n_embd %d", a.h_stride, a.n_embd);
     SHV_REQUIRE(shv_aligned16(a.router) && shv_aligned16(a.shared_gate), "moe_router: router and shared_gate must be 16-byte aligned");
     const unsigned blocks = static_cast<unsigned>((a.n_expert + 1 + 3) / 4);
-    int32_t *counter = ctx->counters + shv_ctx::kCounterRouter;
     switch (a.n_embd) {
-        case 2048: SHV_LAUNCH(ctx, moe_router_kernel<2048>, dim3(blocks), dim3(kBlock), 0, a, counter); break;
-        case 1024: SHV_LAUNCH(ctx, moe_router_kernel<1024>, dim3(blocks), dim3(kBlock), 0, a, counter); break;
-        case 512: SHV_LAUNCH(ctx, moe_router_kernel<512>, dim3(blocks), dim3(kBlock), 0, a, counter); break;
+        case 2048: SHV_LAUNCH(ctx, moe_router_kernel<2048>, dim3(blocks), dim3(kBlock), 0, a); break;
+        case 1024: SHV_LAUNCH(ctx, moe_router_kernel<1024>, dim3(blocks), dim3(kBlock), 0, a); break;
+        case 512: SHV_LAUNCH(ctx, moe_router_kernel<512>, dim3(blocks), dim3(kBlock), 0, a); break;
         default: return shv_set_error(SHV_E_INVALID, "moe_router: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
     }
+    // the selection needs every logit of the token, i.e. the whole grid above: a second, tiny
+    // launch is cheaper than handing the logits to one block inside the first
+    if (!a.defer_route) SHV_LAUNCH(ctx, moe_route_kernel, dim3(a.n_tok), dim3(64), 0, a);
     return SHV_OK;
 }
 

@@ -226,7 +226,6 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     r.n_used = c_.NExpertUsed;
     r.eps = c_.RMSEps;
     r.h_stride = c_.NEmbd;
-    r.defer_route = 1;  // the expert kernel selects from the logits; no hand-over inside the router
     shv_moe_up_args u{};
     u.xn = xn_;
     u.topk = topk_;
@@ -239,9 +238,6 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     u.n_embd = c_.NEmbd;
     u.n_used = c_.NExpertUsed;
     u.ffn = c_.FFNExpert;
-    u.logits = logits_;
-    u.weights = weights_;
-    u.n_expert = c_.NExpert;
     shv_moe_down_args d{};
     d.act = act_;
     d.topk = topk_;
