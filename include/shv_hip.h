@@ -97,8 +97,11 @@ enum {
     SHV_PRO_RMSNORM = 1,     /* x * rsqrt(mean(x^2)+eps) * gamma            (llm/hc.go:176-190)       */
     SHV_PRO_GATED_NORM = 2,  /* per head of head_dim: rms * gamma[head_dim] * sigmoid(z)
                                                                             (llm/deltanet.go:329-341) */
-    SHV_PRO_MUL_SIGMOID = 3  /* x * sigmoid(z); with head_dim > 0, z holds [q | gate] per head and
+    SHV_PRO_MUL_SIGMOID = 3, /* x * sigmoid(z); with head_dim > 0, z holds [q | gate] per head and
                                 the gate half is read                      (llm/attn.go:162-166,198-205) */
+    SHV_PRO_RMSNORM_PAIR = 4 /* the draft head's input (llm/mtp.go:44-46): the k-wide vector is
+                                [RMSNorm(x)*gamma[0..k/2) | RMSNorm(z)*gamma[k/2..k)], x and z each
+                                k/2 wide with strides x_stride and z_stride                        */
 };
 
 /* y[t][r] = sum_i W[r][i] * pro(x[t])[i] (+ residual[t][r]); W is GGUF Q4_K, row-major, k%256==0.
@@ -222,7 +225,14 @@ typedef struct {
  * before the start of a sequence read as zero.  state is [n_slots][hv][d][d] float32 holding
  * S[i][j] at [j*d+i] (the reference's transposed layout), updated in place; out is the raw
  * attention output [n_seq*seq_len][hv*d] that the gated norm of the out projection consumes.
- * v-head h reads key head h % hk (kHeadOfV, llm/deltanet.go:412-418). */
+ * v-head h reads key head h % hk (kHeadOfV, llm/deltanet.go:412-418).
+ * Rewindable passes (DeltaNetGPU.Speculate / KeepSlot, llm/gpu_deltanet.go:1091-1133): with
+ * n_planes > 1 a state slot holds n_planes copies of S, state is [n_slots][n_planes][hv][d][d],
+ * and plane[slot] names the committed one, which is the one read.  spec == 0 updates it in place.
+ * spec != 0 leaves it untouched and stores the state after row i of the pass into plane
+ * (plane[slot] + 1 + i) % n_planes, so that accepting the first k rows of the pass is
+ * plane[slot] = (plane[slot] + k) % n_planes and discarding it is doing nothing; seq_len must then
+ * be below n_planes.  plane NULL reads plane 0. */
 typedef struct {
     const float *ring;
     const float *conv1d;
@@ -237,6 +247,8 @@ typedef struct {
     int32_t ring_slots, ring_stride;
     float eps;
     int32_t qk_norm_max;
+    const int32_t *plane;
+    int32_t n_planes, spec;
 } shv_dn_step_args;
 
 /* Gated full-attention decode over an fp16 KV cache (AttnLayerAt, llm/attn.go:162-205, and
@@ -281,14 +293,16 @@ typedef struct {
 
 /* Greedy sampler (Argmax, llm/sample.go:359-367): the index of the first maximum of each row of
  * logits [n_rows][n]; NaN never wins.  best[r] receives the index.  When ids and pos are given
- * (n_rows must be 1) the index is also stored as the next token, ids[pos[0]+1], and pos[0] is
- * advanced by one, so a recorded decode step can be replayed back to back without the host. */
+ * (n_rows must be 1) the index is also stored as the next token, ids[pos[0]+advance], and pos[0]
+ * is advanced by `advance` (0 means 1: the rows the pass carried), so a recorded decode step can be
+ * replayed back to back without the host. */
 typedef struct {
     const float *logits;
     int32_t *best;
     int32_t *ids;
     int32_t *pos;
     int32_t n_rows, n, logits_stride;
+    int32_t advance;
 } shv_argmax_args;
 
 /* pos[s] += delta for s < n_seq: the step of a recorded pass that does not sample. */

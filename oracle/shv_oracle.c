@@ -764,8 +764,8 @@ void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, cons
 
 /* ------------------------------------------------------------- token loop --- */
 
-void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
-                          const int32_t *ids, int n_tok, float *logits, float *hidden, int threads) {
+void shv_ref_model_extend_rows(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
+                               const int32_t *ids, int n_tok, float *logits_rows, float *hidden_rows, int threads) {
     int H = c->n_embd;
     size_t T = (size_t)n_tok;
     float *x = (float *)malloc(sizeof(float) * T * H);
@@ -787,11 +787,61 @@ void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, 
         for (size_t i = 0; i < T * H; i++) x[i] += y[i];
     }
     st->past += n_tok;
-    const float *last = x + (T - 1) * H;
-    if (hidden) memcpy(hidden, last, sizeof(float) * H);
-    if (logits) {
-        shv_ref_rmsnorm(xn, last, w->out_norm, H, c->eps);
-        shv_ref_gemv_q4k(logits, w->lm_head, xn, c->vocab, H, threads);
+    if (hidden_rows) memcpy(hidden_rows, x, sizeof(float) * T * H);
+    if (logits_rows) {
+        for (int t = 0; t < n_tok; t++) {
+            shv_ref_rmsnorm(xn, x + (size_t)t * H, w->out_norm, H, c->eps);
+            shv_ref_gemv_q4k(logits_rows + (size_t)t * c->vocab, w->lm_head, xn, c->vocab, H, threads);
+        }
     }
     free(y); free(xn); free(x);
+}
+
+void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
+                          const int32_t *ids, int n_tok, float *logits, float *hidden, int threads) {
+    int H = c->n_embd;
+    float *rows = (float *)malloc(sizeof(float) * (size_t)n_tok * H);
+    shv_ref_model_extend_rows(c, w, st, ids, n_tok, NULL, rows, threads);
+    const float *last = rows + (size_t)(n_tok - 1) * H;
+    if (hidden) memcpy(hidden, last, sizeof(float) * H);
+    if (logits) {
+        float *xn = (float *)malloc(sizeof(float) * H);
+        shv_ref_rmsnorm(xn, last, w->out_norm, H, c->eps);
+        shv_ref_gemv_q4k(logits, w->lm_head, xn, c->vocab, H, threads);
+        free(xn);
+    }
+    free(rows);
+}
+
+/* llm/mtp.go:31-53 without hyper-connection streams; the block itself is the trunk's attention
+ * layer and MoE (llm/mtp.go:47-49). */
+void shv_ref_mtp_rows(const shv_ref_model_cfg *c, const shv_ref_model_w *w, const shv_ref_mtp_w *mw,
+                      uint16_t *kcache, uint16_t *vcache, const float *hs, const int32_t *ids, int n_tok,
+                      int pos, float *logits, float *res, int threads) {
+    int H = c->n_embd;
+    size_t T = (size_t)n_tok;
+    float *x = (float *)malloc(sizeof(float) * T * H);
+    float *xn = (float *)malloc(sizeof(float) * T * H);
+    float *y = (float *)malloc(sizeof(float) * T * H);
+    float *cat = (float *)malloc(sizeof(float) * 2 * H);
+    float *e = (float *)malloc(sizeof(float) * H);
+    for (int t = 0; t < n_tok; t++) {
+        for (int i = 0; i < H; i++) e[i] = shv_ref_f16_to_f32(w->embd[(size_t)ids[t] * H + i]);
+        shv_ref_rmsnorm(cat, e, mw->enorm, H, c->eps);
+        shv_ref_rmsnorm(cat + H, hs + (size_t)t * H, mw->hnorm, H, c->eps);
+        shv_ref_gemv_q4k(x + (size_t)t * H, mw->eh_proj, cat, H, 2 * H, threads);
+    }
+    const shv_ref_layer_w *lw = &mw->layer;
+    for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->attn_norm, H, c->eps);
+    shv_ref_attn_layer(&c->attn, &lw->attn, xn, n_tok, pos, kcache, vcache, y, NULL, NULL, threads);
+    for (size_t i = 0; i < T * H; i++) x[i] += y[i];
+    for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->ffn_norm, H, c->eps);
+    shv_ref_moe_block(&c->moe, &lw->moe, xn, n_tok, y, NULL, NULL, NULL, NULL, NULL, NULL, threads);
+    for (size_t i = 0; i < T * H; i++) x[i] += y[i];
+    if (res) memcpy(res, x, sizeof(float) * T * H);
+    if (logits) {
+        shv_ref_rmsnorm(xn, x + (T - 1) * H, mw->head_norm, H, c->eps);
+        shv_ref_gemv_q4k(logits, w->lm_head, xn, c->vocab, H, threads);
+    }
+    free(e); free(cat); free(y); free(xn); free(x);
 }

@@ -208,6 +208,31 @@ typedef struct {
  * hidden [n_embd] (the residual stream before the final norm) of the LAST row; either may be NULL. */
 void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
                           const int32_t *ids, int n_tok, float *logits, float *hidden, int threads);
+/* The same pass with EVERY row's logits [n_tok][vocab] and residual [n_tok][n_embd] (Graph.ExtendRows,
+ * llm/graph.go:1383-1429: the verification pass of the speculative loop); either may be NULL. */
+void shv_ref_model_extend_rows(const shv_ref_model_cfg *c, const shv_ref_model_w *w, shv_ref_model_state *st,
+                               const int32_t *ids, int n_tok, float *logits_rows, float *hidden_rows, int threads);
+
+/* ---- the draft head (MTPHead.Rows, llm/mtp.go:31-53,542-673) for a model without hyper-connection
+ * streams, which is qwen3next's wiring as llm/mtp.go:31-33 names it:
+ *     x   = eh_proj . concat(RMSNorm(embd(id), enorm), RMSNorm(h, hnorm))
+ *     x  += Attn(RMSNorm(x, attn_norm))        one full-attention block with a KV cache of its own
+ *     x  += MoE(RMSNorm(x, ffn_norm))
+ *     logits = lm_head . RMSNorm(x, shared_head_norm)      (the trunk's lm_head)
+ * hs is [n_tok][n_embd], the residual behind each row; rows sit at positions pos..pos+n_tok-1 of the
+ * draft's own cache.  res receives every row's x, logits the LAST row's.  "parity unpinned": the
+ * reference's own wiring is for its four-stream model and has no numerical oracle either
+ * (llm/mtp.go:23-29); this composition is pinned only through the blocks it is made of. */
+typedef struct {
+    const float *enorm, *hnorm;   /* [n_embd] */
+    const uint8_t *eh_proj;       /* Q4_K [n_embd][2*n_embd] */
+    const float *head_norm;       /* [n_embd] */
+    shv_ref_layer_w layer;        /* attention weights, norms and MoE of the draft block */
+} shv_ref_mtp_w;
+
+void shv_ref_mtp_rows(const shv_ref_model_cfg *c, const shv_ref_model_w *w, const shv_ref_mtp_w *mw,
+                      uint16_t *kcache, uint16_t *vcache, const float *hs, const int32_t *ids, int n_tok,
+                      int pos, float *logits, float *res, int threads);
 
 #ifdef __cplusplus
 }

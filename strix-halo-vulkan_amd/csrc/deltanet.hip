@@ -66,7 +66,12 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
     const int rsub = lane >> 5, li = lane & 31;
     const int jl = wave * 2 + rsub;           // row within the block
     const int j = chunk * kRowsPerBlock + jl; // row of the head's state
-    float *srow = a.state + ((static_cast<size_t>(slot) * a.n_head_v + h) * kD + j) * kD + li * 4;
+    // a slot holds n_planes copies of the state; the committed one is read
+    const int planes = a.n_planes > 1 ? a.n_planes : 1;
+    const int cur = a.plane ? static_cast<int>(static_cast<unsigned>(a.plane[slot]) % static_cast<unsigned>(planes)) : 0;
+    const size_t plane_floats = static_cast<size_t>(a.n_head_v) * kD * kD;
+    float *sslot = a.state + static_cast<size_t>(slot) * planes * plane_floats + (static_cast<size_t>(h) * kD + j) * kD + li * 4;
+    float *srow = sslot + cur * plane_floats;
     float4 s = *reinterpret_cast<const float4 *>(srow);  // in flight while the prologue runs
 
     const float *ring = a.ring + static_cast<size_t>(slot) * a.ring_slots * a.ring_stride;
@@ -111,9 +116,11 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
         const float oq = sum32_all(fmaf(s.x, q4.x, fmaf(s.y, q4.y, fmaf(s.z, q4.z, s.w * q4.w))));
         if (li == 0)
             a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j] = oq * scale;
+        // a rewindable pass keeps every prefix: the state after row i goes to its own plane
+        if (a.spec) *reinterpret_cast<float4 *>(sslot + ((cur + 1 + i) % planes) * plane_floats) = s;
         __syncthreads();
     }
-    *reinterpret_cast<float4 *>(srow) = s;
+    if (!a.spec) *reinterpret_cast<float4 *>(srow) = s;
 }
 
 }  // namespace
@@ -130,6 +137,9 @@ int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
     SHV_REQUIRE(a.ring_slots >= a.seq_len + a.conv - 1, "dn_step: a ring of %d slots cannot hold %d tokens and %d of history",
                 a.ring_slots, a.seq_len, a.conv - 1);
     SHV_REQUIRE(shv_aligned16(a.state) && shv_aligned16(a.conv1d), "dn_step: state and conv1d must be 16-byte aligned");
+    SHV_REQUIRE(a.n_planes >= 0 && a.n_planes <= 64, "dn_step: %d state planes", a.n_planes);
+    SHV_REQUIRE(!a.spec || (a.n_planes > 1 && a.seq_len < a.n_planes), "dn_step: a rewindable pass of %d rows needs more than %d state planes",
+                a.seq_len, a.n_planes);
     dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
     SHV_LAUNCH(ctx, dn_step_kernel, grid, dim3(kBlock), 0, a);
     return SHV_OK;

@@ -135,6 +135,30 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
                 const float g = 1.f / (1.f + expf(-z[c]));
                 xs[t][lds_slot(c)] = v[i] * scale * a.gamma[c % a.head_dim] * g;
             }
+        } else if (a.prologue == SHV_PRO_RMSNORM_PAIR) {
+            // two K/2-wide vectors, each with its own RMS, side by side
+            if constexpr (K >= 2 * kBlock) {
+                constexpr int HALF = K / kBlock / 2;
+                const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
+                float v[2 * HALF];
+                float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                for (int i = 0; i < HALF; i++) {
+                    v[i] = x[tid + i * kBlock];
+                    v[HALF + i] = z[tid + i * kBlock];
+                    s0 = fmaf(v[i], v[i], s0);
+                    s1 = fmaf(v[HALF + i], v[HALF + i], s1);
+                }
+                s0 = block_sum_256(s0, red);
+                s1 = block_sum_256(s1, red);
+                const float sc0 = 1.f / sqrtf(s0 / static_cast<float>(K / 2) + a.eps);
+                const float sc1 = 1.f / sqrtf(s1 / static_cast<float>(K / 2) + a.eps);
+#pragma unroll
+                for (int i = 0; i < 2 * HALF; i++) {
+                    const int c = tid + i * kBlock;
+                    xs[t][lds_slot(c)] = v[i] * (i < HALF ? sc0 : sc1) * a.gamma[c];
+                }
+            }
         } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
             const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
 #pragma unroll
@@ -253,9 +277,12 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
     SHV_REQUIRE(a.n > 0, "gemv_q4k: n = %d", a.n);
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 64, "gemv_q4k: n_tok %d, the GEMV covers 1..64 rows", a.n_tok);
     SHV_REQUIRE(shv_aligned16(a.w), "gemv_q4k: w must be 16-byte aligned");
-    SHV_REQUIRE(a.x_stride >= a.k || a.n_tok == 1, "gemv_q4k: x_stride %d < k %d", a.x_stride, a.k);
+    const int x_width = a.prologue == SHV_PRO_RMSNORM_PAIR ? a.k / 2 : a.k;
+    SHV_REQUIRE(a.x_stride >= x_width || a.n_tok == 1, "gemv_q4k: x_stride %d < %d", a.x_stride, x_width);
     SHV_REQUIRE(a.y_stride >= a.n || a.n_tok == 1 || a.ring_slots > 0, "gemv_q4k: y_stride %d < n %d", a.y_stride, a.n);
-    SHV_REQUIRE(a.prologue >= SHV_PRO_NONE && a.prologue <= SHV_PRO_MUL_SIGMOID, "gemv_q4k: prologue %d", a.prologue);
+    SHV_REQUIRE(a.prologue >= SHV_PRO_NONE && a.prologue <= SHV_PRO_RMSNORM_PAIR, "gemv_q4k: prologue %d", a.prologue);
+    if (a.prologue == SHV_PRO_RMSNORM_PAIR)
+        SHV_REQUIRE(a.gamma && a.z && a.k >= 512 && (a.z_stride >= a.k / 2 || a.n_tok == 1), "gemv_q4k: pair-norm prologue needs gamma, z and k >= 512");
     if (a.prologue == SHV_PRO_RMSNORM) SHV_REQUIRE(a.gamma, "gemv_q4k: RMSNorm prologue without gamma");
     if (a.prologue == SHV_PRO_GATED_NORM) {
         SHV_REQUIRE(a.gamma && a.z, "gemv_q4k: gated-norm prologue without gamma or z");

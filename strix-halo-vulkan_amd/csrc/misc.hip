@@ -152,9 +152,9 @@ __global__ __launch_bounds__(256) void argmax_kernel(shv_argmax_args a, float *p
         if (bi >= a.n) bi = 0;
         a.best[r] = bi;
         if (a.ids && a.pos) {
-            const int p = a.pos[0];
-            a.ids[p + 1] = bi;
-            a.pos[0] = p + 1;
+            const int p = a.pos[0] + (a.advance > 0 ? a.advance : 1);
+            a.ids[p] = bi;
+            a.pos[0] = p;
         }
     }
 }
@@ -180,6 +180,7 @@ int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a) {
     SHV_REQUIRE(a->n_rows >= 1 && a->n >= 1 && a->logits_stride >= a->n, "argmax: %d rows of %d, stride %d", a->n_rows, a->n, a->logits_stride);
     SHV_REQUIRE((a->ids == nullptr) == (a->pos == nullptr), "argmax: ids and pos go together");
     SHV_REQUIRE(!a->ids || a->n_rows == 1, "argmax: storing the next token needs exactly one row");
+    SHV_REQUIRE(a->advance >= 0, "argmax: advance %d", a->advance);
     int nb = (a->n + 1023) / 1024;
     const int cap = shv_ctx::kArgmaxBlocks / a->n_rows;
     SHV_REQUIRE(cap >= 1 && a->n_rows <= 14, "argmax: %d rows is more than one launch covers", a->n_rows);

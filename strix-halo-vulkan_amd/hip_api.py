@@ -11,7 +11,7 @@ Q4K_BYTES = 144
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
 OP_EMBED, OP_ARGMAX, OP_ADVANCE = 10, 11, 12
-PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID = 0, 1, 2, 3
+PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 
 class ShvError(RuntimeError):
@@ -82,7 +82,8 @@ class DnStepArgs(C.Structure):
                 ("pos", C.c_void_p), ("slot", C.c_void_p), ("n_seq", C.c_int32),
                 ("seq_len", C.c_int32), ("n_head_k", C.c_int32), ("n_head_v", C.c_int32),
                 ("head_dim", C.c_int32), ("conv", C.c_int32), ("ring_slots", C.c_int32),
-                ("ring_stride", C.c_int32), ("eps", C.c_float), ("qk_norm_max", C.c_int32)]
+                ("ring_stride", C.c_int32), ("eps", C.c_float), ("qk_norm_max", C.c_int32),
+                ("plane", C.c_void_p), ("n_planes", C.c_int32), ("spec", C.c_int32)]
 
 
 class AttnDecodeArgs(C.Structure):
@@ -104,7 +105,7 @@ class EmbedArgs(C.Structure):
 class ArgmaxArgs(C.Structure):
     _fields_ = [("logits", C.c_void_p), ("best", C.c_void_p), ("ids", C.c_void_p),
                 ("pos", C.c_void_p), ("n_rows", C.c_int32), ("n", C.c_int32),
-                ("logits_stride", C.c_int32)]
+                ("logits_stride", C.c_int32), ("advance", C.c_int32)]
 
 
 class AdvanceArgs(C.Structure):

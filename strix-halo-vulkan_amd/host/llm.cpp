@@ -97,7 +97,17 @@ Model::Model(Device &dev, const Config &cfg) : dev_(dev), cfg_(cfg) {
     add("token_embd.weight", TensorView::F16, c.VocabSize, c.NEmbd, 0.f, 1.f);
     add("output_norm.weight", TensorView::F32, 1, c.NEmbd, 1.f, 0.1f);
     add("output.weight", TensorView::Q4K, c.VocabSize, c.NEmbd, 0.f, 0.02f);
-    for (int l = 0; l < c.NLayer; l++) {
+    if (c.NextN < 0 || c.NextN > 1) throw Error("llm: nextn_predict_layers " + std::to_string(c.NextN) + "; one draft block at most");
+    for (int l = 0; l < c.Blocks(); l++) {
+        if (l >= c.NLayer) {
+            // the draft block's own tensors (llm/mtp.go:36-53): the two input norms side by side
+            // so that one projection prologue reads them, eh_proj [NEmbd][2*NEmbd], the head norm
+            add(Blk(l, "nextn.ehnorm_fused"), TensorView::F32, 2, c.NEmbd, 1.f, 0.1f);
+            alias(Blk(l, "nextn.enorm"), Blk(l, "nextn.ehnorm_fused"), 0, 1);
+            alias(Blk(l, "nextn.hnorm"), Blk(l, "nextn.ehnorm_fused"), 1, 1);
+            add(Blk(l, "nextn.eh_proj"), TensorView::Q4K, c.NEmbd, 2 * c.NEmbd, 0.f, 0.02f);
+            add(Blk(l, "nextn.shared_head_norm"), TensorView::F32, 1, c.NEmbd, 1.f, 0.1f);
+        }
         add(Blk(l, "attn_norm"), TensorView::F32, 1, c.NEmbd, 1.f, 0.1f);
         add(Blk(l, "post_attention_norm"), TensorView::F32, 1, c.NEmbd, 1.f, 0.1f);
         if (c.IsAttn(l)) {
@@ -293,21 +303,24 @@ std::vector<float> MoEGPU::Out() const { return read_back<float>(dev_, out_, sta
 
 // ----------------------------------------------------------------------------- DeltaNet -------
 
-DeltaNetGPU::DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, int32_t *pos)
-    : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens), slots_(slots), pos_(pos) {
+DeltaNetGPU::DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, int32_t *pos, int planes, int32_t *plane)
+    : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens), slots_(slots), planes_(planes), pos_(pos), plane_(plane) {
     // refusals at construction, never at run (llm/gpu_deltanet.go:423-447)
     if (c_.SSMHeadDim != 128) throw Error("llm: DeltaNetGPU: head dimension " + std::to_string(c_.SSMHeadDim) + ", the step kernel is built for 128");
     if (c_.SSMConv != 4) throw Error("llm: DeltaNetGPU: conv kernel " + std::to_string(c_.SSMConv) + ", built for 4");
-    if (maxTokens < 1 || maxTokens + c_.SSMConv - 1 > kRing) throw Error("llm: DeltaNetGPU: a pass of " + std::to_string(maxTokens) + " rows does not fit the projection ring");
+    if (maxTokens < 1 || maxTokens > 64) throw Error("llm: DeltaNetGPU: a pass of " + std::to_string(maxTokens) + " rows; 1..64");
     if (slots < 1) throw Error("llm: DeltaNetGPU: no slots");
+    if (planes < 1 || planes > 64 || (planes > 1 && !plane)) throw Error("llm: DeltaNetGPU: " + std::to_string(planes) + " state planes");
+    // the ring holds a pass's rows and the conv's history behind them
+    ring_slots_ = std::max(kRing, maxTokens + c_.SSMConv - 1);
     const size_t T = maxTokens;
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     attn_ = static_cast<float *>(dev.alloc(T * c_.VWidth() * 4));
     ring_.assign(c_.NLayer, nullptr);
     state_.assign(c_.NLayer, nullptr);
-    const size_t ring_bytes = static_cast<size_t>(slots) * kRing * c_.DNFusedRows() * 4;
-    const size_t st_bytes = static_cast<size_t>(slots) * c_.SSMHeadV * c_.SSMHeadDim * c_.SSMHeadDim * 4;
+    const size_t ring_bytes = static_cast<size_t>(slots) * ring_slots_ * c_.DNFusedRows() * 4;
+    const size_t st_bytes = static_cast<size_t>(slots) * planes * c_.SSMHeadV * c_.SSMHeadDim * c_.SSMHeadDim * 4;
     for (int l = 0; l < c_.NLayer; l++) {
         if (c_.IsAttn(l)) continue;
         ring_[l] = static_cast<float *>(dev.alloc_zero(ring_bytes));
@@ -329,8 +342,8 @@ void DeltaNetGPU::Upload(const std::vector<float> &x, int nTok) {
 
 void DeltaNetGPU::Reset(int l) {
     if (l < 0 || l >= c_.NLayer || !state_[l]) throw Error("llm: DeltaNetGPU.Reset: layer " + std::to_string(l) + " is not a DeltaNet layer");
-    dev_.zero(ring_[l], static_cast<size_t>(slots_) * kRing * c_.DNFusedRows() * 4);
-    dev_.zero(state_[l], static_cast<size_t>(slots_) * c_.SSMHeadV * c_.SSMHeadDim * c_.SSMHeadDim * 4);
+    dev_.zero(ring_[l], static_cast<size_t>(slots_) * ring_slots_ * c_.DNFusedRows() * 4);
+    dev_.zero(state_[l], static_cast<size_t>(slots_) * planes_ * c_.SSMHeadV * c_.SSMHeadDim * c_.SSMHeadDim * 4);
 }
 
 void DeltaNetGPU::ResetAll() {
@@ -338,15 +351,41 @@ void DeltaNetGPU::ResetAll() {
         if (state_[l]) Reset(l);
 }
 
+// One slot's carried history back to an empty sequence's: every plane of its state and its ring.
+void DeltaNetGPU::ResetSlot(int slot) {
+    if (slot < 0 || slot >= slots_) throw Error("llm: DeltaNetGPU.ResetSlot: slot " + std::to_string(slot) + " of " + std::to_string(slots_));
+    const size_t ring_floats = static_cast<size_t>(ring_slots_) * c_.DNFusedRows();
+    const size_t st_floats = static_cast<size_t>(planes_) * c_.SSMHeadV * c_.SSMHeadDim * c_.SSMHeadDim;
+    for (int l = 0; l < c_.NLayer; l++) {
+        if (!state_[l]) continue;
+        dev_.zero(ring_[l] + slot * ring_floats, ring_floats * 4);
+        dev_.zero(state_[l] + slot * st_floats, st_floats * 4);
+    }
+}
+
 std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, int nTok, std::vector<std::string> *labels) const {
-    if (!state_[l]) throw Error("llm: DeltaNetGPU: layer " + std::to_string(l) + " is not a DeltaNet layer");
+    PassRows r;
+    r.pos = pos_;
+    r.seq_len = nTok;
+    return Dispatches(l, in, out, r, labels);
+}
+
+std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, const PassRows &r, std::vector<std::string> *labels) const {
+    if (l < 0 || l >= c_.NLayer || !state_[l]) throw Error("llm: DeltaNetGPU: layer " + std::to_string(l) + " is not a DeltaNet layer");
+    const int nTok = r.rows();
+    if (nTok < 1 || nTok > max_tok_) throw Error("llm: DeltaNetGPU: " + std::to_string(nTok) + " rows, staged for " + std::to_string(max_tok_));
+    if (r.n_seq > slots_) throw Error("llm: DeltaNetGPU: this block was staged with " + std::to_string(slots_) + " sequence slot(s) (GraphOpts.Slots)");
+    if (r.spec && r.seq_len >= planes_)
+        throw Error("llm: DeltaNetGPU: a rewindable pass of " + std::to_string(r.seq_len) + " rows needs " + std::to_string(r.seq_len + 1) +
+                    " state planes, " + std::to_string(planes_) + " are staged (GraphOpts.Speculative, SpecRows)");
     const int width = c_.DNFusedRows();
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor(Model::Blk(l, "ssm_in_fused")).ptr;
     p.x = in;
     p.y = ring_[l];
     p.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "attn_norm")).ptr);
-    p.pos = pos_;
+    p.pos = r.pos;
+    p.slot = r.slot;
     p.n = width;
     p.k = c_.NEmbd;
     p.n_tok = nTok;
@@ -354,8 +393,8 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     p.eps = c_.RMSEps;
     p.x_stride = c_.NEmbd;
     p.y_stride = width;
-    p.seq_len = nTok;
-    p.ring_slots = kRing;
+    p.seq_len = r.seq_len;
+    p.ring_slots = ring_slots_;
     p.ring_stride = width;
     shv_dn_step_args s{};
     s.ring = ring_[l];
@@ -364,14 +403,18 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     s.dt_bias = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ssm_dt")).ptr);
     s.state = state_[l];
     s.out = attn_;
-    s.pos = pos_;
-    s.n_seq = 1;
-    s.seq_len = nTok;
+    s.pos = r.pos;
+    s.slot = r.slot;
+    s.n_seq = r.n_seq;
+    s.seq_len = r.seq_len;
+    s.plane = plane_;
+    s.n_planes = planes_;
+    s.spec = r.spec ? 1 : 0;
     s.n_head_k = c_.SSMHeadK;
     s.n_head_v = c_.SSMHeadV;
     s.head_dim = c_.SSMHeadDim;
     s.conv = c_.SSMConv;
-    s.ring_slots = kRing;
+    s.ring_slots = ring_slots_;
     s.ring_stride = width;
     s.eps = c_.RMSEps;
     shv_gemv_q4k_args o{};
@@ -381,7 +424,8 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     o.residual = in;
     o.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ssm_norm")).ptr);
     o.z = ring_[l] + c_.ConvWidth();  // the z columns of a projection row
-    o.pos = pos_;
+    o.pos = r.pos;
+    o.slot = r.slot;
     o.n = c_.NEmbd;
     o.k = c_.VWidth();
     o.n_tok = nTok;
@@ -390,8 +434,8 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     o.eps = c_.RMSEps;
     o.x_stride = c_.VWidth();
     o.y_stride = c_.NEmbd;
-    o.seq_len = nTok;
-    o.ring_slots = kRing;
+    o.seq_len = r.seq_len;
+    o.ring_slots = ring_slots_;
     o.ring_stride = width;
     o.z_ring = 1;
     if (labels) labels->insert(labels->end(), {"dn.qkv", "dn.step", "dn.out"});
@@ -403,16 +447,18 @@ void DeltaNetGPU::Run(int layer) {
     dev_.run(Dispatches(layer, in_, out_, n_tok_, nullptr));
 }
 
-std::vector<float> DeltaNetGPU::State(int l, int slot) const {
-    if (!state_[l] || slot < 0 || slot >= slots_) throw Error("llm: DeltaNetGPU.State: no such layer or slot");
+std::vector<float> DeltaNetGPU::State(int l, int slot, int plane) const {
+    if (l < 0 || l >= c_.NLayer || !state_[l] || slot < 0 || slot >= slots_ || plane < 0 || plane >= planes_)
+        throw Error("llm: DeltaNetGPU.State: no such layer, slot or plane");
     const size_t n = static_cast<size_t>(c_.SSMHeadV) * c_.SSMHeadDim * c_.SSMHeadDim;
-    return read_back<float>(dev_, state_[l] + slot * n, n);
+    return read_back<float>(dev_, state_[l] + (static_cast<size_t>(slot) * planes_ + plane) * n, n);
 }
 
-void DeltaNetGPU::SetState(int l, const std::vector<float> &s, int slot) {
+void DeltaNetGPU::SetState(int l, const std::vector<float> &s, int slot, int plane) {
     const size_t n = static_cast<size_t>(c_.SSMHeadV) * c_.SSMHeadDim * c_.SSMHeadDim;
-    if (!state_[l] || slot < 0 || slot >= slots_ || s.size() != n) throw Error("llm: DeltaNetGPU.SetState: no such layer or slot, or wrong length");
-    dev_.upload(state_[l] + slot * n, s.data(), n * 4);
+    if (l < 0 || l >= c_.NLayer || !state_[l] || slot < 0 || slot >= slots_ || plane < 0 || plane >= planes_ || s.size() != n)
+        throw Error("llm: DeltaNetGPU.SetState: no such layer, slot or plane, or wrong length");
+    dev_.upload(state_[l] + (static_cast<size_t>(slot) * planes_ + plane) * n, s.data(), n * 4);
 }
 
 std::vector<float> DeltaNetGPU::Result() const { return read_back<float>(dev_, attn_, static_cast<size_t>(n_tok_) * c_.VWidth()); }
@@ -438,7 +484,7 @@ static std::vector<float> rope_table(int cells, int rope_dims, float base) {
     return t;
 }
 
-AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots, int32_t *pos)
+AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots, int32_t *pos, int only_layer)
     : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens), n_kv_(nKV), slots_(slots), pos_(pos) {
     if (c_.HeadDim != 256) throw Error("llm: AttnGPU: head dimension " + std::to_string(c_.HeadDim) + ", the decode kernel is built for 256");
     if (c_.NHead != 8 * c_.NHeadKV) throw Error("llm: AttnGPU: the decode kernel is built for 8 query heads per KV head");
@@ -449,15 +495,17 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     qkv_ = static_cast<float *>(dev.alloc(T * c_.AttnFusedRows() * 4));
     ctx_ = static_cast<float *>(dev.alloc(T * c_.NHead * c_.HeadDim * 4));
-    partial_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.NHeadKV) * kMaxSplits * 8 * (c_.HeadDim + 2) * 4));
+    // one set of slice records per sequence of a batched pass (an ordinary pass is one sequence)
+    partial_ = static_cast<float *>(dev.alloc(T * c_.NHeadKV * kMaxSplits * 8 * (c_.HeadDim + 2) * 4));
     const std::vector<float> rt = rope_table(nKV, c_.RopeDims, c_.RopeBase);
     rope_ = static_cast<float *>(dev.alloc(rt.size() * 4));
     dev.upload(rope_, rt.data(), rt.size() * 4);
-    kc_.assign(c_.NLayer, nullptr);
-    vc_.assign(c_.NLayer, nullptr);
+    kc_.assign(c_.Blocks(), nullptr);
+    vc_.assign(c_.Blocks(), nullptr);
+    if (only_layer >= c_.Blocks()) throw Error("llm: AttnGPU: block " + std::to_string(only_layer) + " of " + std::to_string(c_.Blocks()));
     const size_t cb = static_cast<size_t>(slots) * nKV * c_.NHeadKV * c_.HeadDim * 2;
-    for (int l = 0; l < c_.NLayer; l++) {
-        if (!c_.IsAttn(l)) continue;
+    for (int l = 0; l < c_.Blocks(); l++) {
+        if (only_layer >= 0 ? l != only_layer : (l >= c_.NLayer || !c_.IsAttn(l))) continue;
         kc_[l] = dev.alloc(cb);
         vc_[l] = dev.alloc(cb);
         cache_bytes_ += 2 * cb;
@@ -484,7 +532,17 @@ void AttnGPU::Upload(const std::vector<float> &x, int nTok) {
 }
 
 std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, int nTok, std::vector<std::string> *labels) const {
-    if (!kc_[l]) throw Error("llm: AttnGPU: layer " + std::to_string(l) + " is not an attention layer");
+    PassRows r;
+    r.pos = pos_;
+    r.seq_len = nTok;
+    return Dispatches(l, in, out, r, labels);
+}
+
+std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, const PassRows &r, std::vector<std::string> *labels) const {
+    if (l < 0 || l >= c_.Blocks() || !kc_[l]) throw Error("llm: AttnGPU: layer " + std::to_string(l) + " is not an attention layer staged here");
+    const int nTok = r.rows();
+    if (nTok < 1 || nTok > max_tok_) throw Error("llm: AttnGPU: " + std::to_string(nTok) + " rows, staged for " + std::to_string(max_tok_));
+    if (r.n_seq > slots_) throw Error("llm: AttnGPU: this block was staged with " + std::to_string(slots_) + " sequence slot(s) (GraphOpts.Slots)");
     const int width = c_.AttnFusedRows();
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor(Model::Blk(l, "attn_qkv_fused")).ptr;
@@ -507,9 +565,10 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, int 
     a.vcache = vc_[l];
     a.partial = partial_;
     a.out = ctx_;
-    a.pos = pos_;
-    a.n_seq = 1;
-    a.seq_len = nTok;
+    a.pos = r.pos;
+    a.slot = r.slot;
+    a.n_seq = r.n_seq;
+    a.seq_len = r.seq_len;
     a.n_head = c_.NHead;
     a.n_head_kv = c_.NHeadKV;
     a.head_dim = c_.HeadDim;
@@ -545,15 +604,15 @@ std::vector<float> AttnGPU::Context() const { return read_back<float>(dev_, ctx_
 std::vector<float> AttnGPU::Out() const { return read_back<float>(dev_, out_, static_cast<size_t>(n_tok_) * c_.NEmbd); }
 
 std::vector<uint16_t> AttnGPU::K(int l, int cells, int slot) const {
-    if (!kc_[l] || cells > n_kv_ || slot >= slots_) throw Error("llm: AttnGPU.K: no such layer, cell or slot");
+    if (l < 0 || l >= c_.Blocks() || !kc_[l] || cells > n_kv_ || slot < 0 || slot >= slots_) throw Error("llm: AttnGPU.K: no such layer, cell or slot");
     const size_t per = static_cast<size_t>(c_.NHeadKV) * c_.HeadDim;
-    return read_back<uint16_t>(dev_, static_cast<uint16_t *>(kc_[l]) + slot * n_kv_ * per, cells * per);
+    return read_back<uint16_t>(dev_, static_cast<uint16_t *>(kc_[l]) + static_cast<size_t>(slot) * n_kv_ * per, cells * per);
 }
 
 std::vector<uint16_t> AttnGPU::V(int l, int cells, int slot) const {
-    if (!vc_[l] || cells > n_kv_ || slot >= slots_) throw Error("llm: AttnGPU.V: no such layer, cell or slot");
+    if (l < 0 || l >= c_.Blocks() || !vc_[l] || cells > n_kv_ || slot < 0 || slot >= slots_) throw Error("llm: AttnGPU.V: no such layer, cell or slot");
     const size_t per = static_cast<size_t>(c_.NHeadKV) * c_.HeadDim;
-    return read_back<uint16_t>(dev_, static_cast<uint16_t *>(vc_[l]) + slot * n_kv_ * per, cells * per);
+    return read_back<uint16_t>(dev_, static_cast<uint16_t *>(vc_[l]) + static_cast<size_t>(slot) * n_kv_ * per, cells * per);
 }
 
 // --------------------------------------------------------------------------------- Head -------
@@ -576,12 +635,18 @@ void HeadGPU::Upload(const std::vector<float> &x, int rows) {
 }
 
 std::vector<shv_op> HeadGPU::Dispatches(const float *in, int rows, std::vector<std::string> *labels) const {
+    return DispatchesTo(in, rows, static_cast<const float *>(m_.Tensor("output_norm.weight").ptr), logits_, c_.VocabSize, labels);
+}
+
+std::vector<shv_op> HeadGPU::DispatchesTo(const float *in, int rows, const float *gamma, float *logits, int cols,
+                                          std::vector<std::string> *labels) const {
+    if (rows < 1 || cols < 1 || cols > c_.VocabSize) throw Error("llm: HeadGPU: " + std::to_string(rows) + " rows over " + std::to_string(cols) + " columns");
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor("output.weight").ptr;
     p.x = in;
-    p.y = logits_;
-    p.gamma = static_cast<const float *>(m_.Tensor("output_norm.weight").ptr);
-    p.n = c_.VocabSize;
+    p.y = logits;
+    p.gamma = gamma;
+    p.n = cols;
     p.k = c_.NEmbd;
     p.n_tok = rows;
     p.prologue = SHV_PRO_RMSNORM;
@@ -609,34 +674,62 @@ static bool no_prerecord() {
     return e && e[0] == '1';
 }
 
-static void submit(Device &dev, shv_prerecorded *rec, const std::vector<shv_op> &ops, int iters, uint64_t *ns, const char *what) {
-    if (no_prerecord())
-        check(shv_dispatch_multi(dev.ctx(), ops.data(), static_cast<int>(ops.size()), iters, ns, nullptr), what);
-    else
-        check(shv_prerecorded_submit(dev.ctx(), rec, iters, ns), what);
+static uint64_t submit_pass(Device &dev, Pass &p, int iters, const char *what) {
+    uint64_t ns = 0;
+    if (no_prerecord()) {
+        check(shv_dispatch_multi(dev.ctx(), p.ops.data(), static_cast<int>(p.ops.size()), iters, &ns, nullptr), what);
+    } else {
+        if (!p.rec) check(shv_prerecord(dev.ctx(), p.ops.data(), static_cast<int>(p.ops.size()), &p.rec), what);
+        check(shv_prerecorded_submit(dev.ctx(), p.rec, iters, &ns), what);
+    }
+    return ns;
+}
+
+static void drop_passes(Device &dev, std::map<std::vector<int>, Pass> &passes) {
+    for (auto &kv : passes)
+        if (kv.second.rec) shv_prerecorded_destroy(dev.ctx(), kv.second.rec);
+    passes.clear();
 }
 
 Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_(m), c_(m.config()), o_(opts) {
     layers_ = opts.Layers > 0 ? opts.Layers : c_.NLayer;
     if (layers_ > c_.NLayer) throw Error("llm: NewGraph: " + std::to_string(layers_) + " layers of a " + std::to_string(c_.NLayer) + "-layer model");
-    if (o_.MaxTokens != 1) throw Error("llm: NewGraph: this build records one-row passes only (MaxTokens 1)");
-    if (o_.Slots != 1) throw Error("llm: NewGraph: this build stages one sequence (Slots 1)");
+    if (o_.MaxTokens < 1 || o_.MaxTokens > 64) throw Error("llm: NewGraph: MaxTokens " + std::to_string(o_.MaxTokens) + "; a pass carries 1..64 rows");
+    if (o_.Slots < 1 || o_.Slots > 32) throw Error("llm: NewGraph: Slots " + std::to_string(o_.Slots) + "; 1..32");
     if (o_.NKV < 2) throw Error("llm: NewGraph: NKV " + std::to_string(o_.NKV));
-    x_ = static_cast<float *>(dev.alloc(static_cast<size_t>(o_.MaxTokens) * c_.NEmbd * 4));
-    ids_ = static_cast<int32_t *>(dev.alloc_zero((static_cast<size_t>(o_.NKV) + 2) * 4));
-    pos_ = static_cast<int32_t *>(dev.alloc_zero(static_cast<size_t>(o_.Slots) * 4));
-    best_ = static_cast<int32_t *>(dev.alloc_zero(64));
-    moe_ = new MoEGPU(dev, m, o_.MaxTokens);
-    dn_ = new DeltaNetGPU(dev, m, o_.MaxTokens, o_.Slots, pos_);
-    attn_ = new AttnGPU(dev, m, o_.MaxTokens, o_.NKV, o_.Slots, pos_);
+    if (o_.Speculative && (o_.SpecRows < 2 || o_.SpecRows > 8)) throw Error("llm: NewGraph: SpecRows " + std::to_string(o_.SpecRows) + "; 2..8");
+    if (o_.HeadRows < 0 || o_.HeadRows > 14) throw Error("llm: NewGraph: HeadRows " + std::to_string(o_.HeadRows) + "; the sampler covers 14 rows a pass");
+    // the widest pass anything here may ask for
+    rows_max_ = std::max(o_.MaxTokens, std::max(o_.HeadRows, o_.Speculative ? o_.SpecRows : 1));
+    const int planes = o_.Speculative ? o_.SpecRows + 1 : 1;
+    const int head_rows = std::min(14, o_.HeadRows > 0 ? std::max(o_.HeadRows, o_.Speculative ? o_.SpecRows : 1) : rows_max_);
+    seq_.assign(o_.Slots, Seq());
+    x_ = static_cast<float *>(dev.alloc(static_cast<size_t>(rows_max_) * c_.NEmbd * 4));
+    ids_stride_ = static_cast<size_t>(o_.NKV) + 2;
+    ids_ = static_cast<int32_t *>(dev.alloc_zero(ids_stride_ * o_.Slots * 4));
+    const size_t S = o_.Slots, R = rows_max_;
+    ctl_ = static_cast<int32_t *>(dev.alloc_zero((3 * S + 3 * R) * 4));
+    pos_ = ctl_;
+    plane_ = ctl_ + S;
+    slot_ix_ = ctl_ + 2 * S;
+    row_pos_ = ctl_ + 3 * S;
+    row_slot_ = row_pos_ + R;
+    row_ids_ = row_slot_ + R;
+    std::vector<int32_t> ix(S);
+    for (size_t i = 0; i < S; i++) ix[i] = static_cast<int32_t>(i);
+    dev.upload(slot_ix_, ix.data(), S * 4);
+    best_ = static_cast<int32_t *>(dev.alloc_zero(64 * 4));
+    moe_ = new MoEGPU(dev, m, rows_max_);
+    dn_ = new DeltaNetGPU(dev, m, rows_max_, o_.Slots, pos_, planes, plane_);
+    attn_ = new AttnGPU(dev, m, rows_max_, o_.NKV, o_.Slots, pos_);
     if (o_.AttnSplits > 0) attn_->SetSplits(o_.AttnSplits);
-    if (!o_.NoHead) head_ = new HeadGPU(dev, m, 1);
-    record();
+    if (!o_.NoHead) head_ = new HeadGPU(dev, m, head_rows);
+    // the decode step of slot 0 is recorded up front, as NewGraph does (llm/graph.go:609)
+    pass(0, 1, head_ ? kSample : kPrefill, false);
 }
 
 Graph::~Graph() {
-    if (step_) shv_prerecorded_destroy(dev_.ctx(), step_);
-    if (prefill_) shv_prerecorded_destroy(dev_.ctx(), prefill_);
+    drop_passes(dev_, passes_);
     delete moe_;
     delete dn_;
     delete attn_;
@@ -645,55 +738,128 @@ Graph::~Graph() {
 
 // The loop body of llm/graph.go:2330-2466 for a model without hyper-connection streams: the
 // residual stream stays in one buffer, every block reads it through its RMSNorm prologue and
-// adds its output back in place.
-void Graph::record() {
-    std::vector<shv_op> ops;
-    std::vector<std::string> labels;
+// adds its output back in place.  What follows the layers depends on the kind of pass:
+//   kPrefill  nothing; the position moves on by the pass's rows
+//   kSample   the head on the last row; its arg-max becomes the next token and the position moves
+//   kRows     the head and arg-max on every row (ExtendRows); the position moves
+//   kBatch    one row per sequence, positions and slots from the row tables (DecodeRows)
+Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
+    const std::vector<int> key{slot, rows, static_cast<int>(kind), spec ? 1 : 0};
+    auto it = passes_.find(key);
+    if (it != passes_.end()) return it->second;
+    if (rows < 1 || rows > rows_max_) throw Error("llm: a pass of " + std::to_string(rows) + " rows, the arenas hold " + std::to_string(rows_max_) + " — GraphOpts.MaxTokens");
+    if ((kind == kRows || kind == kBatch) && (!head_ || rows > head_->MaxRows()))
+        throw Error("llm: " + std::to_string(rows) + " rows, the head arena holds " + std::to_string(head_ ? head_->MaxRows() : 0) + " — GraphOpts.HeadRows");
+    Pass p;
+    PassRows r;
+    r.spec = spec;
     shv_embed_args e{};
     e.table = m_.Tensor("token_embd.weight").ptr;
-    e.ids = ids_;
-    e.pos = pos_;
     e.x = x_;
-    e.n_tok = 1;
+    e.n_tok = rows;
     e.n_embd = c_.NEmbd;
     e.vocab = c_.VocabSize;
     e.x_stride = c_.NEmbd;
-    ops.push_back(make_op(SHV_OP_EMBED, e));
-    labels.push_back("embed");
-    for (int l = 0; l < layers_; l++) {
-        auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, 1, &labels) : dn_->Dispatches(l, x_, x_, 1, &labels);
-        ops.insert(ops.end(), sub.begin(), sub.end());
-        auto ffn = moe_->Dispatches(l, x_, x_, 1, &labels);
-        ops.insert(ops.end(), ffn.begin(), ffn.end());
+    if (kind == kBatch) {
+        r.pos = row_pos_;
+        r.slot = row_slot_;
+        r.n_seq = rows;
+        r.seq_len = 1;
+        e.ids = row_ids_;
+    } else {
+        r.pos = pos_ + slot;
+        r.slot = slot_ix_ + slot;
+        r.n_seq = 1;
+        r.seq_len = rows;
+        e.ids = ids_ + slot * ids_stride_;
+        e.pos = pos_ + slot;
     }
-    prefill_ops_ = ops;
-    shv_advance_args adv{pos_, 1, 1};
-    prefill_ops_.push_back(make_op(SHV_OP_ADVANCE, adv));
-    check(shv_prerecord(dev_.ctx(), prefill_ops_.data(), static_cast<int>(prefill_ops_.size()), &prefill_), "record prefill step");
+    p.ops.push_back(make_op(SHV_OP_EMBED, e));
+    p.labels.push_back("embed");
+    for (int l = 0; l < layers_; l++) {
+        auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, r, &p.labels) : dn_->Dispatches(l, x_, x_, r, &p.labels);
+        p.ops.insert(p.ops.end(), sub.begin(), sub.end());
+        auto ffn = moe_->Dispatches(l, x_, x_, rows, &p.labels);
+        p.ops.insert(p.ops.end(), ffn.begin(), ffn.end());
+    }
+    shv_argmax_args am{};
     if (head_) {
-        auto h = head_->Dispatches(x_, 1, &labels);
-        ops.insert(ops.end(), h.begin(), h.end());
-        shv_argmax_args am{};
         am.logits = head_->LogitsPort();
         am.best = best_;
-        am.ids = ids_;
-        am.pos = pos_;
-        am.n_rows = 1;
         am.n = c_.VocabSize;
         am.logits_stride = c_.VocabSize;
-        ops.push_back(make_op(SHV_OP_ARGMAX, am));
-        labels.push_back("argmax");
-        step_ops_ = ops;
-        step_labels_ = labels;
-        check(shv_prerecord(dev_.ctx(), step_ops_.data(), static_cast<int>(step_ops_.size()), &step_), "record decode step");
     }
+    shv_advance_args adv{pos_ + (slot < 0 ? 0 : slot), 1, rows};
+    switch (kind) {
+        case kPrefill:
+            p.ops.push_back(make_op(SHV_OP_ADVANCE, adv));
+            p.labels.push_back("advance");
+            break;
+        case kSample: {
+            if (!head_) throw Error("llm: this graph was staged without a head");
+            auto h = head_->Dispatches(x_ + static_cast<size_t>(rows - 1) * c_.NEmbd, 1, &p.labels);
+            p.ops.insert(p.ops.end(), h.begin(), h.end());
+            am.ids = ids_ + slot * ids_stride_;
+            am.pos = pos_ + slot;
+            am.n_rows = 1;
+            am.advance = rows;
+            p.ops.push_back(make_op(SHV_OP_ARGMAX, am));
+            p.labels.push_back("argmax");
+            break;
+        }
+        case kRows:
+        case kBatch: {
+            auto h = head_->Dispatches(x_, rows, &p.labels);
+            p.ops.insert(p.ops.end(), h.begin(), h.end());
+            am.n_rows = rows;
+            p.ops.push_back(make_op(SHV_OP_ARGMAX, am));
+            p.labels.push_back("argmax");
+            if (kind == kRows) {
+                p.ops.push_back(make_op(SHV_OP_ADVANCE, adv));
+                p.labels.push_back("advance");
+            }
+            break;
+        }
+    }
+    return passes_[key] = std::move(p);
+}
+
+uint64_t Graph::submit(Pass &p, int iters, const char *what) {
+    const uint64_t ns = submit_pass(dev_, p, iters, what);
+    Stats.GPUNanos += ns;
+    Stats.Dispatches = static_cast<int>(p.ops.size());
+    return ns;
+}
+
+int Graph::Dispatches() { return static_cast<int>(pass(slot_, 1, head_ ? kSample : kPrefill, false).ops.size()); }
+
+// The host is the authority on where each sequence stands between calls; the recorded passes
+// move the device copy themselves while they replay.
+void Graph::put_pos() {
+    std::vector<int32_t> v(2 * o_.Slots);
+    for (int s = 0; s < o_.Slots; s++) {
+        v[s] = seq_[s].past;
+        v[o_.Slots + s] = seq_[s].plane;
+    }
+    dev_.upload(ctl_, v.data(), v.size() * 4);
 }
 
 void Graph::Reset() {
-    dn_->ResetAll();
-    const int32_t zero = 0;
-    dev_.upload(pos_, &zero, 4);
-    past_ = 0;
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    dn_->ResetSlot(slot_);
+    seq_[slot_] = Seq();
+    put_pos();
+}
+
+void Graph::UseSlot(int s) {
+    if (s < 0 || s >= o_.Slots) throw Error("llm: sequence slot " + std::to_string(s) + " of " + std::to_string(o_.Slots));
+    if (spec_armed_ && s != slot_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    slot_ = s;
+}
+
+void Graph::check_ids(const std::vector<int32_t> &ids) const {
+    for (int32_t id : ids)
+        if (id < 0 || id >= c_.VocabSize) throw Error("llm: token " + std::to_string(id) + " is outside the vocabulary");
 }
 
 void Graph::Forward(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *hidden) {
@@ -701,77 +867,485 @@ void Graph::Forward(const std::vector<int32_t> &ids, std::vector<float> *logits,
     Extend(ids, logits, hidden);
 }
 
-void Graph::Extend(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *hidden) {
+// The rows go through in chunks of MaxTokens; every chunk but the last is headless, the last one
+// samples.  res_all, when given, receives every row's residual.
+void Graph::extend(const std::vector<int32_t> &ids, float *res_all) {
     const int n = static_cast<int>(ids.size());
+    Seq &q = seq_[slot_];
     if (n < 1) throw Error("llm: Graph.Extend: no tokens");
-    if (past_ + n + 1 > o_.NKV) throw Error("llm: Graph.Extend: " + std::to_string(past_ + n) + " tokens do not fit " + std::to_string(o_.NKV) + " cells");
-    for (int32_t id : ids)
-        if (id < 0 || id >= c_.VocabSize) throw Error("llm: Graph.Extend: token " + std::to_string(id) + " is outside the vocabulary");
-    dev_.upload(ids_ + past_, ids.data(), static_cast<size_t>(n) * 4);
-    const int32_t p = past_;
-    dev_.upload(pos_, &p, 4);
-    // every row but the last goes through the headless step; the last one samples
-    uint64_t ns = 0;
-    if (n > 1) submit(dev_, prefill_, prefill_ops_, n - 1, &ns, "prefill");
-    Stats.GPUNanos += ns;
-    if (head_) {
-        submit(dev_, step_, step_ops_, 1, &ns, "decode step");
-        Stats.Dispatches = static_cast<int>(step_ops_.size());
-    } else {
-        submit(dev_, prefill_, prefill_ops_, 1, &ns, "last row");
-        Stats.Dispatches = static_cast<int>(prefill_ops_.size());
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past + n + 1 > o_.NKV) throw Error("llm: Graph.Extend: " + std::to_string(q.past + n) + " tokens do not fit " + std::to_string(o_.NKV) + " cells");
+    check_ids(ids);
+    dev_.upload(ids_ + slot_ * ids_stride_ + q.past, ids.data(), static_cast<size_t>(n) * 4);
+    put_pos();
+    const int M = o_.MaxTokens;
+    const int last = n % M == 0 ? M : n % M;
+    const int full = (n - last) / M;
+    const size_t row_bytes = static_cast<size_t>(c_.NEmbd) * 4;
+    if (full > 0) {
+        Pass &p = pass(slot_, M, kPrefill, false);
+        if (res_all) {
+            for (int i = 0; i < full; i++) {
+                submit(p, 1, "prefill");
+                check(shv_copy(dev_.ctx(), res_all + static_cast<size_t>(i) * M * c_.NEmbd, x_, M * row_bytes), "keep residual");
+            }
+        } else {
+            submit(p, full, "prefill");
+        }
     }
-    Stats.GPUNanos += ns;
+    submit(pass(slot_, last, head_ ? kSample : kPrefill, false), 1, "last rows");
+    if (res_all) check(shv_copy(dev_.ctx(), res_all + static_cast<size_t>(full) * M * c_.NEmbd, x_, last * row_bytes), "keep residual");
     Stats.Runs++;
-    past_ += n;
+    q.past += n;
+    last_rows_ = last;
+}
+
+void Graph::Extend(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *hidden) {
+    if (logits && !head_) throw Error("llm: Graph.Extend: the graph was staged without a head");
+    extend(ids, nullptr);
     if (logits) {
-        if (!head_) throw Error("llm: Graph.Extend: the graph was staged without a head");
         logits->resize(c_.VocabSize);
         dev_.download(logits->data(), head_->LogitsPort(), static_cast<size_t>(c_.VocabSize) * 4);
     }
     if (hidden) {
         hidden->resize(c_.NEmbd);
-        dev_.download(hidden->data(), x_, static_cast<size_t>(c_.NEmbd) * 4);
+        dev_.download(hidden->data(), x_ + static_cast<size_t>(last_rows_ - 1) * c_.NEmbd, static_cast<size_t>(c_.NEmbd) * 4);
     }
 }
 
+const float *Graph::ForwardResidual(const std::vector<int32_t> &ids, std::vector<float> *logits) {
+    if (logits && !head_) throw Error("llm: Graph.ForwardResidual: the graph was staged without a head");
+    Reset();
+    if (ids.size() > res_all_rows_) {
+        // grown, never shrunk: the device's allocations live as long as the device
+        res_all_rows_ = std::max<size_t>(ids.size(), 256);
+        res_all_ = static_cast<float *>(dev_.alloc(res_all_rows_ * c_.NEmbd * 4));
+    }
+    extend(ids, res_all_);
+    if (logits) {
+        logits->resize(c_.VocabSize);
+        dev_.download(logits->data(), head_->LogitsPort(), static_cast<size_t>(c_.VocabSize) * 4);
+    }
+    return res_all_;
+}
+
+void Graph::ExtendRows(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *res) {
+    if (!head_) throw Error("llm: this graph was staged without a head");
+    const int n = static_cast<int>(ids.size());
+    Seq &q = seq_[slot_];
+    if (n <= 0 || n > head_->MaxRows()) throw Error("llm: " + std::to_string(n) + " rows, the head arena holds " + std::to_string(head_->MaxRows()) + " — GraphOpts.HeadRows");
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past + n + 1 > o_.NKV) throw Error("llm: Graph.ExtendRows: " + std::to_string(q.past + n) + " tokens do not fit " + std::to_string(o_.NKV) + " cells");
+    check_ids(ids);
+    Pass &p = pass(slot_, n, kRows, spec_);
+    dev_.upload(ids_ + slot_ * ids_stride_ + q.past, ids.data(), static_cast<size_t>(n) * 4);
+    put_pos();
+    submit(p, 1, "rows");
+    Stats.Runs++;
+    if (spec_) {
+        spec_armed_ = true;
+        spec_past_ = q.past;
+        spec_rows_ = n;
+    }
+    q.past += n;
+    last_rows_ = n;
+    if (logits) {
+        logits->resize(static_cast<size_t>(n) * c_.VocabSize);
+        dev_.download(logits->data(), head_->LogitsPort(), logits->size() * 4);
+    }
+    if (res) {
+        res->resize(static_cast<size_t>(n) * c_.NEmbd);
+        dev_.download(res->data(), x_, res->size() * 4);
+    }
+}
+
+void Graph::DecodeRows(const std::vector<int> &slots, const std::vector<int32_t> &ids, std::vector<float> *logits) {
+    const int n = static_cast<int>(slots.size());
+    if (n == 0 || n != static_cast<int>(ids.size())) throw Error("llm: " + std::to_string(n) + " slots and " + std::to_string(ids.size()) + " tokens");
+    if (!head_) throw Error("llm: this graph was staged without a head");
+    if (n > head_->MaxRows()) throw Error("llm: " + std::to_string(n) + " rows, the head arena holds " + std::to_string(head_->MaxRows()) + " — GraphOpts.HeadRows");
+    if (spec_) throw Error("llm: a speculating graph cannot batch sequences");
+    check_ids(ids);
+    // checkBatch (llm/batch.go:45-63): a slot out of range or named twice, a position past the cache
+    std::vector<int32_t> rows(3 * static_cast<size_t>(rows_max_), 0);
+    std::vector<bool> seen(o_.Slots, false);
+    for (int r = 0; r < n; r++) {
+        const int s = slots[r];
+        if (s < 0 || s >= o_.Slots) throw Error("llm: batch row on slot " + std::to_string(s) + " of " + std::to_string(o_.Slots));
+        if (seen[s]) throw Error("llm: slot " + std::to_string(s) + " twice in one batch");
+        seen[s] = true;
+        if (seq_[s].past + 2 > o_.NKV) throw Error("llm: a token at position " + std::to_string(seq_[s].past) + " of a " + std::to_string(o_.NKV) + "-cell context");
+        rows[r] = seq_[s].past;
+        rows[rows_max_ + r] = s;
+        rows[2 * rows_max_ + r] = ids[r];
+    }
+    Pass &p = pass(-1, n, kBatch, false);
+    put_pos();
+    dev_.upload(row_pos_, rows.data(), rows.size() * 4);
+    for (int r = 0; r < n; r++) dev_.upload(ids_ + slots[r] * ids_stride_ + seq_[slots[r]].past, &ids[r], 4);
+    submit(p, 1, "batched rows");
+    Stats.Runs++;
+    for (int r = 0; r < n; r++) seq_[slots[r]].past++;
+    put_pos();
+    last_rows_ = n;
+    if (logits) {
+        logits->resize(static_cast<size_t>(n) * c_.VocabSize);
+        dev_.download(logits->data(), head_->LogitsPort(), logits->size() * 4);
+    }
+}
+
+std::vector<int32_t> Graph::Argmaxes() const { return read_back<int32_t>(dev_, best_, last_rows_ > 0 ? last_rows_ : 1); }
+
 std::vector<int32_t> Graph::Generate(int n, uint64_t *gpu_nanos) {
+    Seq &q = seq_[slot_];
     if (!head_) throw Error("llm: Graph.Generate: the graph was staged without a head");
-    if (past_ < 1) throw Error("llm: Graph.Generate before a prompt");
-    if (n < 1 || past_ + n + 1 > o_.NKV) throw Error("llm: Graph.Generate: " + std::to_string(n) + " more tokens do not fit the cache");
-    // the last Extend already sampled the token at position past_: it sits in ids[past_], and
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past < 1) throw Error("llm: Graph.Generate before a prompt");
+    if (n < 1 || q.past + n + 1 > o_.NKV) throw Error("llm: Graph.Generate: " + std::to_string(n) + " more tokens do not fit the cache");
+    // the last Extend already sampled the token at position past: it sits in ids[past], and
     // every replay consumes ids[pos] and appends ids[pos+1]
     uint64_t ns = 0;
-    if (n > 1) submit(dev_, step_, step_ops_, n - 1, &ns, "generate");
+    if (n > 1) {
+        put_pos();
+        ns = submit(pass(slot_, 1, kSample, false), n - 1, "generate");
+    }
     if (gpu_nanos) *gpu_nanos = ns;
     std::vector<int32_t> out(n);
-    dev_.download(out.data(), ids_ + past_, static_cast<size_t>(n) * 4);
-    past_ += n - 1;
-    Stats.GPUNanos += ns;
+    dev_.download(out.data(), ids_ + slot_ * ids_stride_ + q.past, static_cast<size_t>(n) * 4);
+    q.past += n - 1;
+    last_rows_ = 1;
     return out;
 }
 
-std::vector<int32_t> Graph::Ids() const { return read_back<int32_t>(dev_, ids_, past_); }
+std::vector<int32_t> Graph::Ids() const { return read_back<int32_t>(dev_, ids_ + slot_ * ids_stride_, seq_[slot_].past); }
+
+// ---- rewindable passes (llm/graph.go:1122-1267) ----
+// The DeltaNet state is the only thing a pass changes that a shorter sequence would still see:
+// a cache cell or a projection-ring row past the end of the sequence is never read.  A rewindable
+// pass therefore leaves the committed state plane alone and stores the state after each of its
+// rows in the planes that follow it, and ending the pass is moving two integers.
+
+void Graph::Speculate(bool on) {
+    if (on == spec_) return;
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (on && dn_->Planes() < 2)
+        throw Error("llm: this block was staged with one state slot; a rewindable pass needs two (GraphOpts.Speculative)");
+    spec_ = on;
+}
+
+void Graph::SpeculateFirst(bool on) {
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    spec_first_ = on;
+}
+
+void Graph::Keep(int k) {
+    if (!spec_armed_) throw Error("llm: nothing to keep; no speculative pass has run");
+    if (!spec_first_) throw Error("llm: this pass did not store its prefixes apart (SpeculateFirst)");
+    if (k < 1 || k > spec_rows_) throw Error("llm: keeping " + std::to_string(k) + " rows of a " + std::to_string(spec_rows_) + "-row pass");
+    if (k == spec_rows_) return Commit();
+    Seq &q = seq_[slot_];
+    q.plane = (q.plane + k) % dn_->Planes();
+    q.past = spec_past_ + k;
+    put_pos();
+    spec_armed_ = false;
+}
+
+void Graph::Commit() {
+    if (!spec_armed_) throw Error("llm: nothing to commit; no speculative pass has run");
+    Seq &q = seq_[slot_];
+    q.plane = (q.plane + spec_rows_) % dn_->Planes();
+    put_pos();
+    spec_armed_ = false;
+}
+
+void Graph::Rewind() {
+    if (!spec_armed_) throw Error("llm: nothing to rewind; no speculative pass has run");
+    if (spec_first_) throw Error("llm: a keep-first pass is ended by KeepFirst or Commit");
+    seq_[slot_].past = spec_past_;
+    put_pos();
+    spec_armed_ = false;
+}
 
 // One real decode step (the sequence advances by one token, as after Generate(1)), dispatched op
 // by op so that every op has its own GPU time.
-std::vector<Stage> Graph::ProfileStep() {
-    if (!head_) throw Error("llm: Graph.ProfileStep: the graph was staged without a head");
-    if (past_ < 1 || past_ + 2 > o_.NKV) throw Error("llm: Graph.ProfileStep: needs a prompt and a free cell");
-    std::vector<uint64_t> per(step_ops_.size());
-    uint64_t total = 0;
-    check(shv_dispatch_multi(dev_.ctx(), step_ops_.data(), static_cast<int>(step_ops_.size()), 1, &total, per.data()), "profile step");
-    past_ += 1;
+static std::vector<Stage> fold_stages(const Pass &p, const std::vector<uint64_t> &per, uint64_t total, std::map<std::string, uint64_t> *kinds_out) {
     std::map<std::string, uint64_t> kinds;
     std::vector<std::string> order;
     for (size_t i = 0; i < per.size(); i++) {
-        if (!kinds.count(step_labels_[i])) order.push_back(step_labels_[i]);
-        kinds[step_labels_[i]] += per[i];
+        if (!kinds.count(p.labels[i])) order.push_back(p.labels[i]);
+        kinds[p.labels[i]] += per[i];
     }
-    Stats.Kinds = kinds;
     std::vector<Stage> out;
     for (const auto &k : order) out.push_back({k, kinds[k]});
     out.push_back({"total", total});
+    if (kinds_out) *kinds_out = kinds;
+    return out;
+}
+
+std::vector<Stage> Graph::ProfileStep() {
+    Seq &q = seq_[slot_];
+    if (!head_) throw Error("llm: Graph.ProfileStep: the graph was staged without a head");
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past < 1 || q.past + 2 > o_.NKV) throw Error("llm: Graph.ProfileStep: needs a prompt and a free cell");
+    Pass &p = pass(slot_, 1, kSample, false);
+    put_pos();
+    std::vector<uint64_t> per(p.ops.size());
+    uint64_t total = 0;
+    check(shv_dispatch_multi(dev_.ctx(), p.ops.data(), static_cast<int>(p.ops.size()), 1, &total, per.data()), "profile step");
+    q.past += 1;
+    return fold_stages(p, per, total, &Stats.Kinds);
+}
+
+// A `rows`-row verification pass timed op by op and then discarded: the sequence is where it was.
+std::vector<Stage> Graph::ProfileRows(int rows) {
+    Seq &q = seq_[slot_];
+    if (!head_) throw Error("llm: Graph.ProfileRows: the graph was staged without a head");
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (dn_->Planes() <= rows) throw Error("llm: Graph.ProfileRows: a discarded pass of " + std::to_string(rows) + " rows needs GraphOpts.Speculative with SpecRows >= " + std::to_string(rows));
+    if (q.past < 1 || q.past + rows + 1 > o_.NKV) throw Error("llm: Graph.ProfileRows: needs a prompt and free cells");
+    Pass &p = pass(slot_, rows, kRows, true);
+    // the rows re-run the sequence's own next token `rows` times over: values do not matter here
+    std::vector<int32_t> next(1);
+    dev_.download(next.data(), ids_ + slot_ * ids_stride_ + q.past, 4);
+    std::vector<int32_t> ids(rows, next[0]);
+    put_pos();
+    dev_.upload(ids_ + slot_ * ids_stride_ + q.past, ids.data(), ids.size() * 4);
+    std::vector<uint64_t> per(p.ops.size());
+    uint64_t total = 0;
+    check(shv_dispatch_multi(dev_.ctx(), p.ops.data(), static_cast<int>(p.ops.size()), 1, &total, per.data()), "profile rows");
+    put_pos();  // discarded: the position goes back, the committed plane never moved
+    return fold_stages(p, per, total, nullptr);
+}
+
+// ------------------------------------------------------------------------------ MTPHead -------
+
+MTPHead::MTPHead(Device &dev, const Model &m, HeadGPU &head, int maxTok, int nKV, int slots)
+    : dev_(dev), m_(m), c_(m.config()), head_(head), max_tok_(maxTok), n_kv_(nKV), layer_(m.config().NLayer) {
+    if (c_.NextN != 1) throw Error("llm: the model carries no draft block (nextn_predict_layers is " + std::to_string(c_.NextN) + ")");
+    if (maxTok < 1 || maxTok > 64) throw Error("llm: MTPHead: " + std::to_string(maxTok) + " rows a call; 1..64");
+    if (slots < 1) throw Error("llm: MTPHead: no slots");
+    pasts_.assign(slots, 0);
+    const size_t T = maxTok, E = c_.NEmbd;
+    x_ = static_cast<float *>(dev.alloc(T * E * 4));
+    h_ = static_cast<float *>(dev.alloc(T * E * 4));
+    e_ = static_cast<float *>(dev.alloc(T * E * 4));
+    logits_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.VocabSize) * 4));
+    const size_t S = slots;
+    ctl_ = static_cast<int32_t *>(dev.alloc_zero((2 * S + T + 16) * 4));
+    pos_ = ctl_;
+    slot_ix_ = ctl_ + S;
+    ids_ = ctl_ + 2 * S;
+    best_ = ids_ + T;
+    std::vector<int32_t> ix(S);
+    for (size_t i = 0; i < S; i++) ix[i] = static_cast<int32_t>(i);
+    dev.upload(slot_ix_, ix.data(), S * 4);
+    attn_ = new AttnGPU(dev, m, maxTok, nKV, slots, pos_, layer_);
+    moe_ = new MoEGPU(dev, m, maxTok);
+}
+
+MTPHead::~MTPHead() {
+    drop_passes(dev_, passes_);
+    delete attn_;
+    delete moe_;
+}
+
+void MTPHead::Rewind(int n) {
+    if (n < 0 || n > pasts_[slot_]) throw Error("llm: rewind to " + std::to_string(n) + " of " + std::to_string(pasts_[slot_]));
+    pasts_[slot_] = n;
+}
+
+void MTPHead::UseSlot(int s) {
+    if (s < 0 || s >= static_cast<int>(pasts_.size())) throw Error("llm: draft cache slot " + std::to_string(s) + " of " + std::to_string(pasts_.size()));
+    slot_ = s;
+}
+
+void MTPHead::SetVocab(int k) {
+    if (k < 0 || k > c_.VocabSize) throw Error("llm: a draft vocabulary of " + std::to_string(k) + " of " + std::to_string(c_.VocabSize));
+    if (k != vocab_) drop_passes(dev_, passes_);
+    vocab_ = k;
+}
+
+int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos, bool head) {
+    const int n = static_cast<int>(ids.size());
+    if (!hs || n < 1 || n > max_tok_) throw Error("llm: MTPHead.Rows: " + std::to_string(n) + " rows, staged for " + std::to_string(max_tok_));
+    if (pos < 0 || pos > pasts_[slot_]) throw Error("llm: MTPHead.Rows: position " + std::to_string(pos) + " leaves a gap after the draft cache's " + std::to_string(pasts_[slot_]) + " cells");
+    if (pos + n + 1 > n_kv_) throw Error("llm: MTPHead.Rows: " + std::to_string(pos + n) + " cells do not fit " + std::to_string(n_kv_));
+    for (int32_t id : ids)
+        if (id < 0 || id >= c_.VocabSize) throw Error("llm: token " + std::to_string(id) + " is outside the vocabulary");
+    const std::vector<int> key{slot_, n, head ? 1 : 0};
+    auto it = passes_.find(key);
+    if (it == passes_.end()) {
+        Pass p;
+        const int E = c_.NEmbd;
+        shv_embed_args e{};
+        e.table = m_.Tensor("token_embd.weight").ptr;
+        e.ids = ids_;
+        e.x = e_;
+        e.n_tok = n;
+        e.n_embd = E;
+        e.vocab = c_.VocabSize;
+        e.x_stride = E;
+        p.ops.push_back(make_op(SHV_OP_EMBED, e));
+        p.labels.push_back("embed");
+        shv_gemv_q4k_args g{};
+        g.w = m_.Tensor(Model::Blk(layer_, "nextn.eh_proj")).ptr;
+        g.x = e_;
+        g.z = h_;
+        g.y = x_;
+        g.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(layer_, "nextn.ehnorm_fused")).ptr);
+        g.n = E;
+        g.k = 2 * E;
+        g.n_tok = n;
+        g.prologue = SHV_PRO_RMSNORM_PAIR;
+        g.eps = c_.RMSEps;
+        g.x_stride = g.z_stride = g.y_stride = E;
+        p.ops.push_back(make_op(SHV_OP_GEMV_Q4K, g));
+        p.labels.push_back("mtp.eh_proj");
+        PassRows r;
+        r.pos = pos_ + slot_;
+        r.slot = slot_ix_ + slot_;
+        r.seq_len = n;
+        auto a = attn_->Dispatches(layer_, x_, x_, r, &p.labels);
+        p.ops.insert(p.ops.end(), a.begin(), a.end());
+        auto f = moe_->Dispatches(layer_, x_, x_, n, &p.labels);
+        p.ops.insert(p.ops.end(), f.begin(), f.end());
+        if (head) {
+            const int cols = vocab_ > 0 ? vocab_ : c_.VocabSize;
+            auto h = head_.DispatchesTo(x_ + static_cast<size_t>(n - 1) * E, 1,
+                                        static_cast<const float *>(m_.Tensor(Model::Blk(layer_, "nextn.shared_head_norm")).ptr), logits_, cols, &p.labels);
+            p.ops.insert(p.ops.end(), h.begin(), h.end());
+            shv_argmax_args am{};
+            am.logits = logits_;
+            am.best = best_;
+            am.n_rows = 1;
+            am.n = cols;
+            am.logits_stride = c_.VocabSize;
+            p.ops.push_back(make_op(SHV_OP_ARGMAX, am));
+            p.labels.push_back("argmax");
+        }
+        it = passes_.emplace(key, std::move(p)).first;
+    }
+    // the block's input h may be this block's own output rows: it is copied aside first
+    check(shv_copy(dev_.ctx(), h_, hs, static_cast<size_t>(n) * c_.NEmbd * 4), "draft input");
+    dev_.upload(ids_, ids.data(), static_cast<size_t>(n) * 4);
+    const int32_t p32 = pos;
+    dev_.upload(pos_ + slot_, &p32, 4);
+    GPUNanos += submit_pass(dev_, it->second, 1, "draft");
+    Steps++;
+    pasts_[slot_] = pos + n;
+    if (!head) return -1;
+    int32_t best = -1;
+    dev_.download(&best, best_, 4);
+    return best;
+}
+
+void MTPHead::RowsHost(const std::vector<float> &hs, const std::vector<int32_t> &ids, int pos, bool head, std::vector<float> *logits,
+                       std::vector<float> *res) {
+    const size_t n = ids.size(), E = c_.NEmbd;
+    if (n < 1 || n > static_cast<size_t>(max_tok_) || hs.size() != n * E) throw Error("llm: the hidden state is " + std::to_string(hs.size()) + " values, want " + std::to_string(n * E));
+    // staged through the embedding arena, which the pass overwrites only after h has been copied aside
+    dev_.upload(e_, hs.data(), hs.size() * 4);
+    Rows(e_, ids, pos, head);
+    if (logits && head) {
+        logits->resize(vocab_ > 0 ? vocab_ : c_.VocabSize);
+        dev_.download(logits->data(), logits_, logits->size() * 4);
+    }
+    if (res) {
+        res->resize(n * E);
+        dev_.download(res->data(), x_, res->size() * 4);
+    }
+}
+
+// --------------------------------------------------------------------------- Speculator -------
+
+Speculator::Speculator(Graph &g, MTPHead &d, int depth) : Depth(depth), g_(g), d_(d) {
+    if (depth < 1 || depth + 1 > g.MaxRows()) throw Error("llm: a draft depth of " + std::to_string(depth) + " needs passes of " + std::to_string(depth + 1) + " rows — GraphOpts.SpecRows");
+    if (d.MaxRows() < depth + 1) throw Error("llm: the draft head is staged for " + std::to_string(d.MaxRows()) + " rows; a round owes up to " + std::to_string(depth + 1));
+    h_ = static_cast<float *>(g.Dev().alloc(static_cast<size_t>(depth + 1) * g.GetModel().config().NEmbd * 4));
+    g.Speculate(true);
+    g.SpeculateFirst(true);
+}
+
+int32_t Speculator::Start(const std::vector<int32_t> &prompt) {
+    const int T = static_cast<int>(prompt.size());
+    if (T < 1) throw Error("llm: Speculator.Start: no prompt");
+    const size_t E = g_.GetModel().config().NEmbd;
+    g_.Speculate(false);  // the prompt is committed as it runs
+    const float *res = g_.ForwardResidual(prompt, nullptr);
+    // Prime (llm/spec.go:286-326): the draft's cell at position p is written from the trunk's
+    // residual at p-1 and the token at p; cell 0 has nothing behind it and takes a zero residual.
+    d_.Reset();
+    g_.Dev().zero(h_, E * 4);
+    d_.Rows(h_, {prompt[0]}, 0, false);
+    const int M = d_.MaxRows();
+    for (int a = 1; a < T; a += M) {
+        const int n = std::min(M, T - a);
+        d_.Rows(res + static_cast<size_t>(a - 1) * E, std::vector<int32_t>(prompt.begin() + a, prompt.begin() + a + n), a, false);
+    }
+    // the trunk's residual after the last prompt row seeds the first round
+    check(shv_copy(g_.Dev().ctx(), h_, res + static_cast<size_t>(T - 1) * E, E * 4), "seed");
+    owe_x_.clear();
+    // the token the prompt's last row sampled sits one past the sequence's end
+    pend_ = g_.Generate(1, nullptr)[0];
+    g_.Speculate(true);
+    g_.SpeculateFirst(true);
+    Stats = SpecStats();
+    Stats.Tokens = 1;
+    return pend_;
+}
+
+std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced) {
+    if (pend_ < 0) throw Error("llm: Speculator.Round before Start");
+    const size_t E = g_.GetModel().config().NEmbd;
+    const int at = g_.Past();
+    const int owed = static_cast<int>(owe_x_.size());
+    // 1. the drafts: the owed rows and the first draft in one call, then each further draft from
+    //    the draft's own residual
+    const uint64_t d0 = d_.GPUNanos;
+    std::vector<int32_t> rows{pend_};
+    std::vector<int32_t> xs(owe_x_);
+    xs.push_back(pend_);
+    int32_t dtok = d_.Rows(h_, xs, at - owed, true);
+    for (int k = 0; k < Depth; k++) {
+        if (k > 0) {
+            std::vector<int32_t> one{rows[k]};
+            // the last row of the previous call is the residual this one chains on
+            dtok = d_.Rows(d_.ResPort() + (k == 1 ? static_cast<size_t>(owed) * E : 0), one, at + k, true);
+        }
+        rows.push_back(k < static_cast<int>(forced.size()) ? forced[k] : dtok);
+    }
+    Stats.DraftNanos += d_.GPUNanos - d0;
+
+    // 2. the verification pass
+    const uint64_t v0 = g_.Stats.GPUNanos;
+    g_.ExtendRows(rows, nullptr, nullptr);
+    Stats.VerifyNanos += g_.Stats.GPUNanos - v0;
+    const std::vector<int32_t> best = g_.Argmaxes();
+    const int n = static_cast<int>(rows.size());
+    Stats.Passes[std::min(n, 4)]++;
+    Stats.Rounds++;
+    if (n > 1) Stats.Drafted++;
+
+    // 3. row i's arg-max is the trunk's token at at+i+1; the pass is the sequence up to the first
+    //    draft it disagrees with
+    std::vector<int32_t> out;
+    for (int i = 0; i < n; i++) {
+        out.push_back(best[i]);
+        if (i + 1 == n) break;
+        Stats.DraftedAt[std::min(i, 3)]++;
+        if (rows[i + 1] != best[i]) break;
+        Stats.AcceptedAt[std::min(i, 3)]++;
+    }
+    const int keep = static_cast<int>(out.size());
+    if (keep > 1) Stats.Accepted++;
+    g_.Keep(keep);
+    // the rows the draft's cache has not seen from the trunk's side (CatchUp, llm/spec.go:838-843),
+    // then the residual the next draft is seeded from
+    check(shv_copy(g_.Dev().ctx(), h_, g_.ResPort(), static_cast<size_t>(keep) * E * 4), "seed");
+    owe_x_.assign(rows.begin() + 1, rows.begin() + keep);
+    d_.Rewind(std::min(d_.Past(), at + 1));
+    pend_ = out[keep - 1];
+    Stats.Tokens += keep;
     return out;
 }
 

@@ -10,6 +10,7 @@
 #pragma once
 
 #include <cstdint>
+#include <functional>
 #include <map>
 #include <stdexcept>
 #include <string>
@@ -77,8 +78,11 @@ struct Config {
     int SSMHeadV = 32;     // ssm.time_step_rank
     int SSMConv = 4;       // ssm.conv_kernel
     int AttnEvery = 4;     // every 4th layer is full attention, the rest gated DeltaNet
+    int NextN = 0;         // nextn_predict_layers: 1 adds the draft head as block NLayer (llm/mtp.go:137)
 
-    bool IsAttn(int layer) const { return (layer + 1) % AttnEvery == 0; }
+    // The draft block is a full-attention layer (llm/mtp.go:17-21).
+    bool IsAttn(int layer) const { return layer >= NLayer || (layer + 1) % AttnEvery == 0; }
+    int Blocks() const { return NLayer + NextN; }
     int QKWidth() const { return SSMHeadK * SSMHeadDim; }
     int VWidth() const { return SSMHeadV * SSMHeadDim; }
     int ConvWidth() const { return 2 * QKWidth() + VWidth(); }
@@ -123,6 +127,18 @@ struct Stage {
     uint64_t GPUNanos = 0;
 };
 
+// How the rows of a pass map to sequences (llm/batch.go:33-72): n_seq sequences of seq_len
+// consecutive rows each; sequence s starts at position pos[s] on slot slot[s].  An ordinary pass
+// is one sequence of nTok rows; a batched decode pass is nTok sequences of one row.  Both arrays
+// live on the device, so a recorded pass follows the sequence without being re-recorded.
+struct PassRows {
+    const int32_t *pos = nullptr;
+    const int32_t *slot = nullptr;  // nullptr: sequence s is slot s
+    int n_seq = 1, seq_len = 1;
+    bool spec = false;              // DeltaNet: a rewindable pass (state goes to the other planes)
+    int rows() const { return n_seq * seq_len; }
+};
+
 // ---- blocks ------------------------------------------------------------------------------------
 // Each block mirrors its Go namesake: it owns its activation buffers, takes [nTok][NEmbd] float32
 // through Upload, runs one layer with Run, and hands tensors back in the CPU reference's layouts.
@@ -159,16 +175,22 @@ private:
 // llm.DeltaNetGPU (llm/gpu_deltanet.go:207-322, NewDeltaNetGPUBank :421)
 class DeltaNetGPU {
 public:
-    static constexpr int kRing = 8;  // projection rows kept per slot: up to 5 rows a pass + 3 of history
-    DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, int32_t *pos);
+    static constexpr int kRing = 8;  // least projection rows kept per slot: up to 5 rows a pass + 3 of history
+    // planes > 1 stages the state copies a rewindable pass needs (WithDNSpecSlots,
+    // llm/gpu_deltanet.go:380); plane is the device array naming each slot's committed copy.
+    DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, int32_t *pos, int planes = 1, int32_t *plane = nullptr);
     void Upload(const std::vector<float> &x, int nTok);
     void Resize(int nTok);
     void Run(int layer);
     void Reset(int layer);
     void ResetAll();
+    void ResetSlot(int slot);
     std::vector<shv_op> Dispatches(int layer, const float *in, float *out, int nTok, std::vector<std::string> *labels) const;
-    std::vector<float> State(int layer, int slot = 0) const;  // S, [hv][d][d]
-    void SetState(int layer, const std::vector<float> &s, int slot = 0);
+    std::vector<shv_op> Dispatches(int layer, const float *in, float *out, const PassRows &rows, std::vector<std::string> *labels) const;
+    std::vector<float> State(int layer, int slot = 0, int plane = 0) const;  // S, [hv][d][d]
+    void SetState(int layer, const std::vector<float> &s, int slot = 0, int plane = 0);
+    int Planes() const { return planes_; }
+    int RingSlots() const { return ring_slots_; }
     std::vector<float> Result() const;  // [T][hv*d] attention output before the gated norm
     std::vector<float> Out() const;     // [T][NEmbd]
     float *InPort() const { return in_; }
@@ -179,8 +201,8 @@ private:
     Device &dev_;
     const Model &m_;
     Config c_;
-    int max_tok_, slots_, n_tok_ = 0;
-    int32_t *pos_;
+    int max_tok_, slots_, planes_, ring_slots_, n_tok_ = 0;
+    int32_t *pos_, *plane_;
     float *in_, *out_, *attn_;
     std::vector<float *> ring_, state_;  // per layer (nullptr on attention layers)
     uint64_t state_bytes_ = 0;
@@ -189,7 +211,8 @@ private:
 // llm.AttnGPU (llm/gpu_attn.go:403-539, NewAttnGPUBank :779)
 class AttnGPU {
 public:
-    AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots, int32_t *pos);
+    // only_layer >= 0 stages that one block alone (the draft head's, llm/mtp.go:176-275)
+    AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots, int32_t *pos, int only_layer = -1);
     void Upload(const std::vector<float> &x, int nTok);
     void Resize(int nTok);
     void Run(int layer);
@@ -197,6 +220,7 @@ public:
     void SetSplits(int n);
     int Splits() const { return splits_; }
     std::vector<shv_op> Dispatches(int layer, const float *in, float *out, int nTok, std::vector<std::string> *labels) const;
+    std::vector<shv_op> Dispatches(int layer, const float *in, float *out, const PassRows &rows, std::vector<std::string> *labels) const;
     std::vector<float> Context() const;  // [T][NHead*HeadDim] before the gate
     std::vector<float> Out() const;
     std::vector<uint16_t> K(int layer, int cells, int slot = 0) const;  // fp16 bits, [cells][nkv][d]
@@ -224,6 +248,10 @@ public:
     void Resize(int rows);
     void Run();
     std::vector<shv_op> Dispatches(const float *in, int rows, std::vector<std::string> *labels) const;
+    // the same projection through another norm and into another arena, over the first `cols`
+    // vocabulary entries (RunCols, llm/gpu_head.go:499): what the draft head borrows
+    std::vector<shv_op> DispatchesTo(const float *in, int rows, const float *gamma, float *logits, int cols,
+                                     std::vector<std::string> *labels) const;
     std::vector<float> Logits() const;  // [rows][vocab]
     int Vocab() const { return c_.VocabSize; }
     int MaxRows() const { return max_rows_; }
@@ -240,12 +268,15 @@ private:
 
 // llm.GraphOpts (llm/graph.go:58-126), the fields that apply here.
 struct GraphOpts {
-    int MaxTokens = 1;  // rows a pass may carry
+    int MaxTokens = 1;  // rows a pass may carry (a longer prompt goes through in chunks of this)
     int NKV = 4096;     // attention cache cells per slot
     int Layers = 0;     // 0: all of the model's layers
     bool NoHead = false;
-    int Slots = 1;
-    int AttnSplits = 0;  // 0: chosen from NKV
+    int Slots = 1;            // sequences held side by side (UseSlot, DecodeRows)
+    int AttnSplits = 0;       // 0: chosen from NKV
+    int HeadRows = 0;         // rows ExtendRows / DecodeRows may carry; 0: MaxTokens
+    bool Speculative = false; // stage the DeltaNet state planes rewindable passes need
+    int SpecRows = 2;         // rows of a verification pass: draft depth + 1
 };
 
 // llm.GraphStats (llm/graph.go:536-566)
@@ -256,7 +287,15 @@ struct GraphStats {
     std::map<std::string, uint64_t> Kinds;  // GPU time by dispatch label
 };
 
-// llm.Graph (llm/graph.go:184-289, NewGraph :609): the whole model as one recorded op sequence.
+// A recorded op sequence and its replayable form.
+struct Pass {
+    std::vector<shv_op> ops;
+    std::vector<std::string> labels;
+    shv_prerecorded *rec = nullptr;
+};
+
+// llm.Graph (llm/graph.go:184-289, NewGraph :609): the whole model as recorded op sequences, one
+// per (slot, row count, kind of pass), recorded the first time each is needed.
 class Graph {
 public:
     Graph(Device &dev, const Model &m, const GraphOpts &opts);
@@ -265,41 +304,165 @@ public:
     void Forward(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *hidden);
     // Extend appends ids to the sequence and returns the LAST row's logits (llm/graph.go:1709).
     void Extend(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *hidden);
+    // ForwardResidual is Forward that also keeps the residual of EVERY prompt row on the device,
+    // [T][NEmbd], which is what primes the draft head (llm/graph.go:1441-1450).
+    const float *ForwardResidual(const std::vector<int32_t> &ids, std::vector<float> *logits);
+    // ExtendRows appends ids and computes every row's logits: the verification pass
+    // (llm/graph.go:1383-1429).  logits [n][vocab] and res [n][NEmbd] (the residual before the
+    // final norm) are copied out when asked for; Argmaxes() and ResPort() serve a caller that
+    // needs only the greedy tokens and leaves the residual on the device.
+    void ExtendRows(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *res);
+    // DecodeRows advances n sequences by one token each in one pass (llm/graph.go:1527-1666).
+    void DecodeRows(const std::vector<int> &slots, const std::vector<int32_t> &ids, std::vector<float> *logits);
+    std::vector<int32_t> Argmaxes() const;     // the greedy token of each row of the last ExtendRows / DecodeRows
+    const float *ResPort() const { return x_; }  // residual rows of the last pass, on the device
     // Greedy continuation (cmd/llm/generate.go:121-165): n replays of the recorded decode step with
     // the arg-max feeding the next step on the device; returns the n tokens and GPU time.
     std::vector<int32_t> Generate(int n, uint64_t *gpu_nanos);
-    void Reset();
-    int Past() const { return past_; }
+    void Reset();  // the live slot's sequence
+    void UseSlot(int s);
+    int Slots() const { return o_.Slots; }
+    int Slot() const { return slot_; }
+    int Past() const { return seq_[slot_].past; }
+    int Plane() const { return seq_[slot_].plane; }  // the live slot's committed DeltaNet state plane
+    int NKV() const { return o_.NKV; }
+    int MaxRows() const { return rows_max_; }
     std::vector<int32_t> Ids() const;
+    // Rewindable passes (llm/graph.go:1122-1267).  While Speculate is on, ExtendRows leaves the
+    // committed DeltaNet state alone and stores the state after each of its rows apart; exactly
+    // one such pass may be in flight, ended by Commit (all rows), Keep(k) (the first k; needs
+    // SpeculateFirst) or Rewind (none; refused under SpeculateFirst, as in the reference).
+    void Speculate(bool on);
+    bool Speculating() const { return spec_; }
+    void SpeculateFirst(bool on);
+    void Keep(int k);
+    void KeepFirst() { Keep(1); }
+    void Commit();
+    void Rewind();
     // One decode step dispatched op by op with a GPU time per op, folded by label
     // (DispatchMultiMarked + recorder.submit, vk/engine.go:913, llm/record.go:217-232).
     std::vector<Stage> ProfileStep();
+    // GPU time of one `rows`-row verification pass relative to nothing: nanoseconds per op label.
+    std::vector<Stage> ProfileRows(int rows);
     GraphStats Stats;
     void ResetStats() { Stats = GraphStats(); }
-    int Dispatches() const { return static_cast<int>(step_ops_.size()); }
+    int Dispatches();
     MoEGPU &MoE() { return *moe_; }
     DeltaNetGPU &DeltaNet() { return *dn_; }
     AttnGPU &Attn() { return *attn_; }
     HeadGPU &Head() { return *head_; }
+    Device &Dev() { return dev_; }
+    const Model &GetModel() const { return m_; }
 
 private:
-    void record();
+    enum Kind { kPrefill = 0, kSample = 1, kRows = 2, kBatch = 3 };
+    struct Seq {
+        int past = 0;
+        int plane = 0;
+    };
+    Pass &pass(int slot, int rows, Kind kind, bool spec);
+    uint64_t submit(Pass &p, int iters, const char *what);
+    void put_pos();
+    void check_ids(const std::vector<int32_t> &ids) const;
+    void extend(const std::vector<int32_t> &ids, float *res_all);
     Device &dev_;
     const Model &m_;
     Config c_;
     GraphOpts o_;
-    int layers_, past_ = 0;
-    float *x_ = nullptr;     // residual stream, [MaxTokens][NEmbd]
-    int32_t *ids_ = nullptr; // the sequence's tokens by position
-    int32_t *pos_ = nullptr; // [Slots] position of each slot's next row
+    int layers_, rows_max_, slot_ = 0;
+    std::vector<Seq> seq_;
+    bool spec_ = false, spec_first_ = false, spec_armed_ = false;
+    int spec_past_ = 0, spec_rows_ = 0;
+    int last_rows_ = 0;
+    float *x_ = nullptr;       // residual stream, [rows_max][NEmbd]
+    float *res_all_ = nullptr; // ForwardResidual's rows
+    size_t res_all_rows_ = 0;
+    int32_t *ids_ = nullptr;   // [Slots][NKV+2] the sequences' tokens by position
+    int32_t *ctl_ = nullptr;   // pos[Slots] | plane[Slots] | slot index[Slots] | row pos[rows] | row slot[rows] | row ids[rows]
+    int32_t *pos_ = nullptr, *plane_ = nullptr, *slot_ix_ = nullptr, *row_pos_ = nullptr, *row_slot_ = nullptr, *row_ids_ = nullptr;
     int32_t *best_ = nullptr;
+    size_t ids_stride_ = 0;
     MoEGPU *moe_ = nullptr;
     DeltaNetGPU *dn_ = nullptr;
     AttnGPU *attn_ = nullptr;
     HeadGPU *head_ = nullptr;
-    std::vector<shv_op> step_ops_, prefill_ops_;  // one token with the head + arg-max / without
-    std::vector<std::string> step_labels_;
-    shv_prerecorded *step_ = nullptr, *prefill_ = nullptr;
+    std::map<std::vector<int>, Pass> passes_;
+};
+
+// llm.MTPHead (llm/mtp.go:84-134, NewMTPHeadSlots :151): the draft block staged beside the trunk.
+// For a model without hyper-connection streams the wiring is qwen3next's (llm/mtp.go:31-33):
+//     x   = eh_proj . concat(RMSNorm(embd(token), enorm), RMSNorm(h, hnorm))
+//     x  += Attn(RMSNorm(x, attn_norm));  x += MoE(RMSNorm(x, ffn_norm))
+//     logits = lm_head . RMSNorm(x, shared_head_norm)           (the trunk's lm_head, borrowed)
+// h is the trunk's residual after the previous token, or this block's own x when drafts chain.
+// Its only carried state is a one-layer KV cache per slot, which Rewind moves for free.
+class MTPHead {
+public:
+    MTPHead(Device &dev, const Model &m, HeadGPU &head, int maxTok, int nKV, int slots);
+    ~MTPHead();
+    // n rows at positions pos..pos+n-1: hs is [n][NEmbd] ON THE DEVICE (the trunk's ResPort() or
+    // ResPort() of this head), ids the token at each position.  With head, the last row's logits
+    // are computed and its greedy token returned (-1 otherwise).  (MTPHead.Rows, llm/mtp.go:542)
+    int32_t Rows(const float *hs, const std::vector<int32_t> &ids, int pos, bool head);
+    // the reference's host-side signature: hs from host memory, logits and residual copied back
+    void RowsHost(const std::vector<float> &hs, const std::vector<int32_t> &ids, int pos, bool head,
+                  std::vector<float> *logits, std::vector<float> *res);
+    const float *ResPort() const { return x_; }  // [n][NEmbd] of the last call
+    int Past() const { return pasts_[slot_]; }
+    void Rewind(int n);
+    void Reset() { pasts_[slot_] = 0; }
+    int Slots() const { return static_cast<int>(pasts_.size()); }
+    void UseSlot(int s);
+    int MaxRows() const { return max_tok_; }
+    void SetVocab(int k);  // draft over a prefix of the vocabulary (llm/mtp.go:675); 0: all of it
+    int Steps = 0;
+    uint64_t GPUNanos = 0;
+
+private:
+    Device &dev_;
+    const Model &m_;
+    Config c_;
+    HeadGPU &head_;
+    int max_tok_, n_kv_, layer_, slot_ = 0, vocab_ = 0;
+    std::vector<int> pasts_;
+    AttnGPU *attn_ = nullptr;
+    MoEGPU *moe_ = nullptr;
+    float *x_, *h_, *e_, *logits_;
+    int32_t *ctl_, *pos_, *slot_ix_, *ids_, *best_;
+    std::map<std::vector<int>, Pass> passes_;
+};
+
+// llm.SpecStats (llm/spec.go:67-112), the counters that exist without a sampler.
+struct SpecStats {
+    int Rounds = 0, Drafted = 0, Accepted = 0, Tokens = 0;
+    int Passes[5] = {0, 0, 0, 0, 0};
+    int DraftedAt[4] = {0, 0, 0, 0}, AcceptedAt[4] = {0, 0, 0, 0};
+    uint64_t DraftNanos = 0, VerifyNanos = 0;
+};
+
+// llm.Speculator (llm/spec.go:221-857), greedy: the draft head proposes Depth tokens, one
+// verification pass of Depth+1 rows checks them, the longest agreeing prefix is kept.  Every token
+// it emits is the trunk's own arg-max over the trunk's own sequence.
+class Speculator {
+public:
+    Speculator(Graph &g, MTPHead &d, int depth);
+    // Prefill the prompt through the trunk and the draft (Start + Prime, llm/spec.go:300-420);
+    // returns the first generated token.
+    int32_t Start(const std::vector<int32_t> &prompt);
+    // One round (llm/spec.go:703-857): the tokens it emitted, 1..Depth+1 of them.  `forced`, when
+    // not empty, replaces the draft head's proposals (the draft still runs): the reference's
+    // `propose` hook, which tests use to drive every acceptance length.
+    std::vector<int32_t> Round(const std::vector<int32_t> &forced = {});
+    void Stop() { g_.Speculate(false); }
+    SpecStats Stats;
+    int Depth;
+
+private:
+    Graph &g_;
+    MTPHead &d_;
+    int32_t pend_ = -1;
+    float *h_ = nullptr;  // [Depth+1][NEmbd]: the owed rows' residuals, then the trunk's last one
+    std::vector<int32_t> owe_x_;
 };
 
 }  // namespace llm

@@ -11,6 +11,8 @@ struct shvllm {
     std::unique_ptr<llm::Device> dev;
     std::unique_ptr<llm::Model> model;
     std::unique_ptr<llm::Graph> graph;
+    std::unique_ptr<llm::MTPHead> mtp;
+    std::unique_ptr<llm::Speculator> spec;
     llm::GraphOpts opts;
     std::vector<std::string> names;
 };
@@ -60,10 +62,16 @@ int shvllm_open(int device, const shvllm_config *c, shvllm **out) {
         cfg.SSMHeadV = c->ssm_head_v;
         cfg.SSMConv = c->ssm_conv;
         cfg.AttnEvery = c->attn_every;
+        cfg.NextN = c->nextn;
         h->opts.NKV = c->nkv;
         h->opts.Layers = c->layers;
         h->opts.NoHead = c->no_head != 0;
         h->opts.AttnSplits = c->attn_splits;
+        h->opts.MaxTokens = c->max_tokens > 0 ? c->max_tokens : 1;
+        h->opts.Slots = c->slots > 0 ? c->slots : 1;
+        h->opts.HeadRows = c->head_rows;
+        h->opts.Speculative = c->speculative != 0;
+        if (c->spec_rows > 0) h->opts.SpecRows = c->spec_rows;
         h->model = std::make_unique<llm::Model>(*h->dev, cfg);
         for (const auto &kv : h->model->Tensors()) h->names.push_back(kv.first);
         *out = h.release();
@@ -72,6 +80,8 @@ int shvllm_open(int device, const shvllm_config *c, shvllm **out) {
 
 void shvllm_close(shvllm *h) {
     if (!h) return;
+    h->spec.reset();
+    h->mtp.reset();
     h->graph.reset();
     h->model.reset();
     h->dev.reset();
@@ -112,7 +122,11 @@ int shvllm_tensor(shvllm *h, const char *name, void **dptr, uint64_t *bytes) {
 uint64_t shvllm_weight_bytes(shvllm *h) { return h && h->model ? h->model->WeightBytes() : 0; }
 
 int shvllm_stage(shvllm *h) {
-    return guard([&] { h->graph = std::make_unique<llm::Graph>(*h->dev, *h->model, h->opts); });
+    return guard([&] {
+        h->spec.reset();
+        h->mtp.reset();
+        h->graph = std::make_unique<llm::Graph>(*h->dev, *h->model, h->opts);
+    });
 }
 
 int shvllm_reset(shvllm *h) {
@@ -171,5 +185,172 @@ int shvllm_kv(shvllm *h, int layer, int cells, uint16_t *k, uint16_t *v) {
 }
 
 uint64_t shvllm_gpu_nanos(shvllm *h) { return h && h->graph ? h->graph->Stats.GPUNanos : 0; }
+
+static void stages_out(const std::vector<llm::Stage> &st, char (*labels)[32], uint64_t *nanos, int max, int *n) {
+    int k = 0;
+    for (const auto &s : st) {
+        if (k >= max) break;
+        std::snprintf(labels[k], 32, "%s", s.Kind.c_str());
+        nanos[k] = s.GPUNanos;
+        k++;
+    }
+    if (n) *n = k;
+}
+
+int shvllm_extend_rows(shvllm *h, const int32_t *ids, int n, float *logits, float *res, int32_t *best) {
+    return guard([&] {
+        if (!ids || n < 1) throw llm::Error("llm: shvllm_extend_rows: no tokens");
+        std::vector<float> lg, rs;
+        graph_of(h).ExtendRows(std::vector<int32_t>(ids, ids + n), logits ? &lg : nullptr, res ? &rs : nullptr);
+        if (logits) std::memcpy(logits, lg.data(), lg.size() * 4);
+        if (res) std::memcpy(res, rs.data(), rs.size() * 4);
+        if (best) {
+            auto b = graph_of(h).Argmaxes();
+            std::memcpy(best, b.data(), b.size() * 4);
+        }
+    });
+}
+
+int shvllm_decode_rows(shvllm *h, const int32_t *slots, const int32_t *ids, int n, float *logits, int32_t *best) {
+    return guard([&] {
+        if (!ids || !slots || n < 1) throw llm::Error("llm: shvllm_decode_rows: no rows");
+        std::vector<float> lg;
+        const bool single = n == 1;
+        graph_of(h).DecodeRows(std::vector<int>(slots, slots + n), std::vector<int32_t>(ids, ids + n), logits ? &lg : nullptr);
+        if (logits) std::memcpy(logits, lg.data(), lg.size() * 4);
+        if (best) {
+            auto b = graph_of(h).Argmaxes();
+            std::memcpy(best, b.data(), (single ? 1 : b.size()) * 4);
+        }
+    });
+}
+
+int shvllm_use_slot(shvllm *h, int slot) {
+    return guard([&] { graph_of(h).UseSlot(slot); });
+}
+int shvllm_speculate(shvllm *h, int on) {
+    return guard([&] { graph_of(h).Speculate(on != 0); });
+}
+int shvllm_speculate_first(shvllm *h, int on) {
+    return guard([&] { graph_of(h).SpeculateFirst(on != 0); });
+}
+int shvllm_keep(shvllm *h, int k) {
+    return guard([&] { graph_of(h).Keep(k); });
+}
+int shvllm_commit(shvllm *h) {
+    return guard([&] { graph_of(h).Commit(); });
+}
+int shvllm_rewind(shvllm *h) {
+    return guard([&] { graph_of(h).Rewind(); });
+}
+int shvllm_plane(shvllm *h) { return h && h->graph ? h->graph->Plane() : -1; }
+
+int shvllm_ids(shvllm *h, int32_t *dst, int max, int *n) {
+    return guard([&] {
+        auto v = graph_of(h).Ids();
+        const int k = static_cast<int>(v.size()) < max ? static_cast<int>(v.size()) : max;
+        if (dst && k > 0) std::memcpy(dst, v.data(), static_cast<size_t>(k) * 4);
+        if (n) *n = static_cast<int>(v.size());
+    });
+}
+
+int shvllm_dn_state_at(shvllm *h, int layer, int slot, int plane, float *dst) {
+    return guard([&] {
+        auto s = graph_of(h).DeltaNet().State(layer, slot, plane);
+        std::memcpy(dst, s.data(), s.size() * 4);
+    });
+}
+
+int shvllm_kv_at(shvllm *h, int layer, int slot, int cells, uint16_t *k, uint16_t *v) {
+    return guard([&] {
+        auto kk = graph_of(h).Attn().K(layer, cells, slot);
+        auto vv = graph_of(h).Attn().V(layer, cells, slot);
+        if (k) std::memcpy(k, kk.data(), kk.size() * 2);
+        if (v) std::memcpy(v, vv.data(), vv.size() * 2);
+    });
+}
+
+int shvllm_profile_rows(shvllm *h, int rows, char (*labels)[32], uint64_t *nanos, int max, int *n) {
+    return guard([&] { stages_out(graph_of(h).ProfileRows(rows), labels, nanos, max, n); });
+}
+
+static llm::MTPHead &mtp_of(shvllm *h) {
+    if (!h || !h->mtp) throw llm::Error("llm: the draft head has not been staged");
+    return *h->mtp;
+}
+
+static llm::Speculator &spec_of(shvllm *h) {
+    if (!h || !h->spec) throw llm::Error("llm: no speculator has been opened");
+    return *h->spec;
+}
+
+int shvllm_mtp_stage(shvllm *h, int max_tok, int vocab_prefix) {
+    return guard([&] {
+        llm::Graph &g = graph_of(h);
+        h->spec.reset();
+        h->mtp = std::make_unique<llm::MTPHead>(*h->dev, *h->model, g.Head(), max_tok, g.NKV(), g.Slots());
+        h->mtp->SetVocab(vocab_prefix);
+    });
+}
+
+int shvllm_mtp_rows(shvllm *h, const float *hs, const int32_t *ids, int n, int pos, int head, float *logits, float *res) {
+    return guard([&] {
+        if (!hs || !ids || n < 1) throw llm::Error("llm: shvllm_mtp_rows: no rows");
+        const size_t E = h->model->config().NEmbd;
+        std::vector<float> lg, rs;
+        mtp_of(h).RowsHost(std::vector<float>(hs, hs + n * E), std::vector<int32_t>(ids, ids + n), pos, head != 0,
+                           logits ? &lg : nullptr, res ? &rs : nullptr);
+        if (logits && !lg.empty()) std::memcpy(logits, lg.data(), lg.size() * 4);
+        if (res) std::memcpy(res, rs.data(), rs.size() * 4);
+    });
+}
+
+int shvllm_mtp_rewind(shvllm *h, int n) {
+    return guard([&] { mtp_of(h).Rewind(n); });
+}
+int shvllm_mtp_past(shvllm *h) { return h && h->mtp ? h->mtp->Past() : -1; }
+
+int shvllm_spec_open(shvllm *h, int depth) {
+    return guard([&] { h->spec = std::make_unique<llm::Speculator>(graph_of(h), mtp_of(h), depth); });
+}
+
+int shvllm_spec_start(shvllm *h, const int32_t *prompt, int n, int32_t *first) {
+    return guard([&] {
+        if (!prompt || n < 1) throw llm::Error("llm: shvllm_spec_start: no prompt");
+        const int32_t t = spec_of(h).Start(std::vector<int32_t>(prompt, prompt + n));
+        if (first) *first = t;
+    });
+}
+
+int shvllm_spec_round(shvllm *h, const int32_t *forced, int n_forced, int32_t *out, int max, int *n_out) {
+    return guard([&] {
+        std::vector<int32_t> f;
+        if (forced && n_forced > 0) f.assign(forced, forced + n_forced);
+        auto v = spec_of(h).Round(f);
+        if (static_cast<int>(v.size()) > max) throw llm::Error("llm: shvllm_spec_round: the round emitted more tokens than the caller has room for");
+        if (out) std::memcpy(out, v.data(), v.size() * 4);
+        if (n_out) *n_out = static_cast<int>(v.size());
+    });
+}
+
+int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos) {
+    return guard([&] {
+        const llm::SpecStats &s = spec_of(h).Stats;
+        if (counts) {
+            int k = 0;
+            counts[k++] = s.Rounds;
+            counts[k++] = s.Drafted;
+            counts[k++] = s.Accepted;
+            counts[k++] = s.Tokens;
+            for (int i = 0; i < 5; i++) counts[k++] = s.Passes[i];
+            for (int i = 0; i < 4; i++) counts[k++] = s.DraftedAt[i];
+            for (int i = 0; i < 4; i++) counts[k++] = s.AcceptedAt[i];
+        }
+        if (nanos) {
+            nanos[0] = s.DraftNanos;
+            nanos[1] = s.VerifyNanos;
+        }
+    });
+}
 
 }  // extern "C"

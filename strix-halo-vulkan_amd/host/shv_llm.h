@@ -24,6 +24,9 @@ typedef struct {
     float rms_eps;
     int32_t ssm_head_dim, ssm_head_k, ssm_head_v, ssm_conv, attn_every;
     int32_t nkv, layers, no_head, attn_splits;   /* GraphOpts: cells, layer truncation, head, slices */
+    int32_t max_tokens, slots, head_rows;        /* GraphOpts: rows a pass, sequences, rows with logits */
+    int32_t speculative, spec_rows;              /* GraphOpts: rewindable passes and their width */
+    int32_t nextn;                               /* 1: the model carries the draft block */
 } shvllm_config;
 
 const char *shvllm_last_error(void);
@@ -48,6 +51,35 @@ int shvllm_profile_step(shvllm *h, char (*labels)[32], uint64_t *nanos, int max,
 int shvllm_dn_state(shvllm *h, int layer, float *dst);                   /* [hv][d][d] */
 int shvllm_kv(shvllm *h, int layer, int cells, uint16_t *k, uint16_t *v); /* [cells][nkv][d] halves */
 uint64_t shvllm_gpu_nanos(shvllm *h);
+
+/* multi-row passes, sequence slots and rewindable passes (Graph.ExtendRows / DecodeRows / UseSlot /
+ * Speculate / SpeculateFirst / Keep / Commit / Rewind).  Output pointers may be NULL. */
+int shvllm_extend_rows(shvllm *h, const int32_t *ids, int n, float *logits, float *res, int32_t *best);
+int shvllm_decode_rows(shvllm *h, const int32_t *slots, const int32_t *ids, int n, float *logits, int32_t *best);
+int shvllm_use_slot(shvllm *h, int slot);
+int shvllm_speculate(shvllm *h, int on);
+int shvllm_speculate_first(shvllm *h, int on);
+int shvllm_keep(shvllm *h, int k);
+int shvllm_commit(shvllm *h);
+int shvllm_rewind(shvllm *h);
+int shvllm_plane(shvllm *h);
+int shvllm_ids(shvllm *h, int32_t *dst, int max, int *n);
+int shvllm_dn_state_at(shvllm *h, int layer, int slot, int plane, float *dst);
+int shvllm_kv_at(shvllm *h, int layer, int slot, int cells, uint16_t *k, uint16_t *v);
+int shvllm_profile_rows(shvllm *h, int rows, char (*labels)[32], uint64_t *nanos, int max, int *n);
+
+/* the draft head (MTPHead) and the greedy speculative loop (Speculator) over the staged graph */
+int shvllm_mtp_stage(shvllm *h, int max_tok, int vocab_prefix);
+int shvllm_mtp_rows(shvllm *h, const float *hs, const int32_t *ids, int n, int pos, int head, float *logits, float *res);
+int shvllm_mtp_rewind(shvllm *h, int n);
+int shvllm_mtp_past(shvllm *h);
+int shvllm_spec_open(shvllm *h, int depth);
+int shvllm_spec_start(shvllm *h, const int32_t *prompt, int n, int32_t *first);
+/* one round; forced (n_forced of them, may be 0) replaces the draft head's proposals */
+int shvllm_spec_round(shvllm *h, const int32_t *forced, int n_forced, int32_t *out, int max, int *n_out);
+/* counts: rounds, drafted, accepted, tokens, passes[5], drafted_at[4], accepted_at[4] (17 values);
+ * nanos: draft, verify */
+int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos);
 
 #ifdef __cplusplus
 }

@@ -18,13 +18,16 @@ class Config(C.Structure):
                 ("ffn_expert", C.c_int32), ("vocab", C.c_int32), ("rms_eps", C.c_float),
                 ("ssm_head_dim", C.c_int32), ("ssm_head_k", C.c_int32), ("ssm_head_v", C.c_int32),
                 ("ssm_conv", C.c_int32), ("attn_every", C.c_int32), ("nkv", C.c_int32),
-                ("layers", C.c_int32), ("no_head", C.c_int32), ("attn_splits", C.c_int32)]
+                ("layers", C.c_int32), ("no_head", C.c_int32), ("attn_splits", C.c_int32),
+                ("max_tokens", C.c_int32), ("slots", C.c_int32), ("head_rows", C.c_int32),
+                ("speculative", C.c_int32), ("spec_rows", C.c_int32), ("nextn", C.c_int32)]
 
     def __init__(self, **kw):
         d = dict(n_layer=48, n_embd=2048, n_head=16, n_head_kv=2, head_dim=256, rope_dims=64,
                  rope_base=1e7, n_expert=512, n_expert_used=10, ffn_expert=512, vocab=151936,
                  rms_eps=1e-6, ssm_head_dim=128, ssm_head_k=16, ssm_head_v=32, ssm_conv=4,
-                 attn_every=4, nkv=4096, layers=0, no_head=0, attn_splits=0)
+                 attn_every=4, nkv=4096, layers=0, no_head=0, attn_splits=0, max_tokens=1, slots=1,
+                 head_rows=0, speculative=0, spec_rows=2, nextn=0)
         d.update(kw)
         super().__init__(**d)
 
@@ -72,6 +75,23 @@ def load():
     L.shvllm_kv.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_uint16), C.POINTER(C.c_uint16)]
     L.shvllm_gpu_nanos.argtypes = [vp]
     L.shvllm_gpu_nanos.restype = C.c_uint64
+    i32p, f32p, u16p = C.POINTER(C.c_int32), C.POINTER(C.c_float), C.POINTER(C.c_uint16)
+    L.shvllm_extend_rows.argtypes = [vp, i32p, C.c_int, f32p, f32p, i32p]
+    L.shvllm_decode_rows.argtypes = [vp, i32p, i32p, C.c_int, f32p, i32p]
+    for name in ("use_slot", "speculate", "speculate_first", "keep", "mtp_rewind", "spec_open"):
+        getattr(L, "shvllm_" + name).argtypes = [vp, C.c_int]
+    for name in ("commit", "rewind", "plane", "mtp_past"):
+        getattr(L, "shvllm_" + name).argtypes = [vp]
+    L.shvllm_ids.argtypes = [vp, i32p, C.c_int, C.POINTER(C.c_int)]
+    L.shvllm_dn_state_at.argtypes = [vp, C.c_int, C.c_int, C.c_int, f32p]
+    L.shvllm_kv_at.argtypes = [vp, C.c_int, C.c_int, C.c_int, u16p, u16p]
+    L.shvllm_profile_rows.argtypes = [vp, C.c_int, C.POINTER(C.c_char * 32), C.POINTER(C.c_uint64), C.c_int,
+                                      C.POINTER(C.c_int)]
+    L.shvllm_mtp_stage.argtypes = [vp, C.c_int, C.c_int]
+    L.shvllm_mtp_rows.argtypes = [vp, f32p, i32p, C.c_int, C.c_int, C.c_int, f32p, f32p]
+    L.shvllm_spec_start.argtypes = [vp, i32p, C.c_int, i32p]
+    L.shvllm_spec_round.argtypes = [vp, i32p, C.c_int, i32p, C.c_int, C.POINTER(C.c_int)]
+    L.shvllm_spec_stats.argtypes = [vp, i32p, C.POINTER(C.c_uint64)]
     _lib = L
     return L
 
@@ -182,3 +202,129 @@ class LLM:
         u16 = C.POINTER(C.c_uint16)
         _check(self.L.shvllm_kv(self.h, layer, cells, k.ctypes.data_as(u16), v.ctypes.data_as(u16)))
         return k, v
+
+    # ---- multi-row passes, slots, rewindable passes ----
+
+    def extend_rows(self, ids, want_logits=False, want_res=False):
+        """Graph.ExtendRows: (greedy token per row, logits [n][vocab] or None, residual [n][n_embd] or None)"""
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        n = len(ids)
+        lg = np.empty((n, self.cfg.vocab), np.float32) if want_logits else None
+        rs = np.empty((n, self.cfg.n_embd), np.float32) if want_res else None
+        best = np.empty(n, np.int32)
+        fp, ip = C.POINTER(C.c_float), C.POINTER(C.c_int32)
+        _check(self.L.shvllm_extend_rows(self.h, ids.ctypes.data_as(ip), n,
+                                         lg.ctypes.data_as(fp) if lg is not None else None,
+                                         rs.ctypes.data_as(fp) if rs is not None else None, best.ctypes.data_as(ip)))
+        return best, lg, rs
+
+    def decode_rows(self, slots, ids, want_logits=False):
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        n = len(ids)
+        lg = np.empty((n, self.cfg.vocab), np.float32) if want_logits else None
+        best = np.empty(n, np.int32)
+        fp, ip = C.POINTER(C.c_float), C.POINTER(C.c_int32)
+        _check(self.L.shvllm_decode_rows(self.h, slots.ctypes.data_as(ip), ids.ctypes.data_as(ip), n,
+                                         lg.ctypes.data_as(fp) if lg is not None else None, best.ctypes.data_as(ip)))
+        return best, lg
+
+    def use_slot(self, s):
+        _check(self.L.shvllm_use_slot(self.h, s))
+
+    def speculate(self, on):
+        _check(self.L.shvllm_speculate(self.h, int(on)))
+
+    def speculate_first(self, on):
+        _check(self.L.shvllm_speculate_first(self.h, int(on)))
+
+    def keep(self, k):
+        _check(self.L.shvllm_keep(self.h, k))
+
+    def commit(self):
+        _check(self.L.shvllm_commit(self.h))
+
+    def rewind(self):
+        _check(self.L.shvllm_rewind(self.h))
+
+    def plane(self):
+        return self.L.shvllm_plane(self.h)
+
+    def ids(self):
+        n = C.c_int()
+        _check(self.L.shvllm_ids(self.h, None, 0, C.byref(n)))
+        out = np.empty(max(n.value, 1), np.int32)
+        _check(self.L.shvllm_ids(self.h, out.ctypes.data_as(C.POINTER(C.c_int32)), n.value, C.byref(n)))
+        return out[:n.value]
+
+    def dn_state_at(self, layer, slot=0, plane=0):
+        c = self.cfg
+        out = np.empty((c.ssm_head_v, c.ssm_head_dim, c.ssm_head_dim), np.float32)
+        _check(self.L.shvllm_dn_state_at(self.h, layer, slot, plane, out.ctypes.data_as(C.POINTER(C.c_float))))
+        return out
+
+    def kv_at(self, layer, slot, cells):
+        c = self.cfg
+        k = np.empty((cells, c.n_head_kv, c.head_dim), np.uint16)
+        v = np.empty_like(k)
+        u16 = C.POINTER(C.c_uint16)
+        _check(self.L.shvllm_kv_at(self.h, layer, slot, cells, k.ctypes.data_as(u16), v.ctypes.data_as(u16)))
+        return k, v
+
+    def profile_rows(self, rows):
+        labels = (C.c_char * 32 * 64)()
+        ns = (C.c_uint64 * 64)()
+        n = C.c_int()
+        _check(self.L.shvllm_profile_rows(self.h, rows, labels, ns, 64, C.byref(n)))
+        return [(labels[i].value.decode(), ns[i]) for i in range(n.value)]
+
+    # ---- draft head and speculative loop ----
+
+    def mtp_stage(self, max_tok=4, vocab_prefix=0):
+        _check(self.L.shvllm_mtp_stage(self.h, max_tok, vocab_prefix))
+
+    def mtp_rows(self, hs, ids, pos, head=True, want_res=True):
+        """MTPHead.Rows with host buffers: (last row's logits or None, residual rows or None)"""
+        hs = np.ascontiguousarray(hs, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        n = len(ids)
+        lg = np.empty(self.cfg.vocab, np.float32) if head else None
+        rs = np.empty((n, self.cfg.n_embd), np.float32) if want_res else None
+        fp, ip = C.POINTER(C.c_float), C.POINTER(C.c_int32)
+        _check(self.L.shvllm_mtp_rows(self.h, hs.ctypes.data_as(fp), ids.ctypes.data_as(ip), n, pos, int(head),
+                                      lg.ctypes.data_as(fp) if lg is not None else None,
+                                      rs.ctypes.data_as(fp) if rs is not None else None))
+        return lg, rs
+
+    def mtp_rewind(self, n):
+        _check(self.L.shvllm_mtp_rewind(self.h, n))
+
+    def mtp_past(self):
+        return self.L.shvllm_mtp_past(self.h)
+
+    def spec_open(self, depth):
+        _check(self.L.shvllm_spec_open(self.h, depth))
+
+    def spec_start(self, prompt):
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        first = C.c_int32()
+        _check(self.L.shvllm_spec_start(self.h, prompt.ctypes.data_as(C.POINTER(C.c_int32)), len(prompt), C.byref(first)))
+        return first.value
+
+    def spec_round(self, forced=()):
+        forced = np.ascontiguousarray(forced, dtype=np.int32)
+        out = np.empty(16, np.int32)
+        n = C.c_int()
+        ip = C.POINTER(C.c_int32)
+        _check(self.L.shvllm_spec_round(self.h, forced.ctypes.data_as(ip) if len(forced) else None, len(forced),
+                                        out.ctypes.data_as(ip), 16, C.byref(n)))
+        return out[:n.value].copy()
+
+    def spec_stats(self):
+        counts = np.zeros(17, np.int32)
+        nanos = np.zeros(2, np.uint64)
+        _check(self.L.shvllm_spec_stats(self.h, counts.ctypes.data_as(C.POINTER(C.c_int32)),
+                                        nanos.ctypes.data_as(C.POINTER(C.c_uint64))))
+        return dict(rounds=int(counts[0]), drafted=int(counts[1]), accepted=int(counts[2]), tokens=int(counts[3]),
+                    passes=counts[4:9].tolist(), drafted_at=counts[9:13].tolist(), accepted_at=counts[13:17].tolist(),
+                    draft_ns=int(nanos[0]), verify_ns=int(nanos[1]))

@@ -76,6 +76,10 @@ class ModelState(C.Structure):
                 ("vcache", C.POINTER(u16p)), ("past", C.c_int)]
 
 
+class MtpW(C.Structure):
+    _fields_ = [("enorm", f32p), ("hnorm", f32p), ("eh_proj", u8p), ("head_norm", f32p), ("layer", LayerW)]
+
+
 _lib = None
 
 
@@ -123,6 +127,9 @@ def lib():
                                      u16p, u16p, f32p, f32p, f32p, C.c_int]
     L.shv_ref_model_extend.argtypes = [C.POINTER(ModelCfg), C.POINTER(ModelW), C.POINTER(ModelState), i32p,
                                        C.c_int, f32p, f32p, C.c_int]
+    L.shv_ref_model_extend_rows.argtypes = L.shv_ref_model_extend.argtypes
+    L.shv_ref_mtp_rows.argtypes = [C.POINTER(ModelCfg), C.POINTER(ModelW), C.POINTER(MtpW), u16p, u16p, f32p, i32p,
+                                   C.c_int, C.c_int, f32p, f32p, C.c_int]
     _lib = L
     return L
 
@@ -260,3 +267,55 @@ class OracleModel:
     @property
     def past(self):
         return self.state.past
+
+    def extend_rows(self, ids, threads=8):
+        """every row's logits [n][vocab] and residual [n][n_embd] (the verification pass)"""
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        logits = np.empty((len(ids), self.cfg.vocab), np.float32)
+        hidden = np.empty((len(ids), self.cfg.n_embd), np.float32)
+        lib().shv_ref_model_extend_rows(C.byref(self.mcfg), C.byref(self.w), C.byref(self.state), I(ids), len(ids),
+                                        F(logits), F(hidden), threads)
+        return logits, hidden
+
+    def snapshot(self):
+        """the carried state, to come back to with restore()"""
+        cp = lambda xs: [None if a is None else a.copy() for a in xs]
+        return cp(self.dn_conv), cp(self.dn_s), cp(self.kc), cp(self.vc), self.state.past
+
+    def restore(self, snap):
+        for dst, src in zip((self.dn_conv, self.dn_s, self.kc, self.vc), snap[:4]):
+            for d, s_ in zip(dst, src):
+                if d is not None:
+                    d[...] = s_
+        self.state.past = snap[4]
+
+
+class OracleMTP:
+    """The draft head on the CPU over the draft block's tensors (block n_layer of the same model)."""
+
+    def __init__(self, om, max_cells):
+        cfg, t = om.cfg, om.t
+        self.om = om
+        blk = lambda n: t["blk.%d.%s.weight" % (cfg.n_layer, n)]
+        lw = LayerW()
+        lw.attn_norm, lw.ffn_norm = F(blk("attn_norm")), F(blk("post_attention_norm"))
+        lw.attn = AttnW(B(blk("attn_q")), B(blk("attn_k")), B(blk("attn_v")), B(blk("attn_output")),
+                        F(blk("attn_q_norm")), F(blk("attn_k_norm")))
+        lw.moe = MoeW(F(blk("ffn_gate_inp")), F(blk("ffn_gate_inp_shexp")), B(blk("ffn_gate_exps")),
+                      B(blk("ffn_up_exps")), B(blk("ffn_down_exps")), B(blk("ffn_gate_shexp")),
+                      B(blk("ffn_up_shexp")), B(blk("ffn_down_shexp")))
+        self.w = MtpW(F(blk("nextn.enorm")), F(blk("nextn.hnorm")), B(blk("nextn.eh_proj")),
+                      F(blk("nextn.shared_head_norm")), lw)
+        self.kc = np.zeros((max_cells, cfg.n_head_kv, cfg.head_dim), np.uint16)
+        self.vc = np.zeros_like(self.kc)
+
+    def rows(self, hs, ids, pos, threads=8):
+        cfg = self.om.cfg
+        hs = np.ascontiguousarray(hs, dtype=np.float32).reshape(-1, cfg.n_embd)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        assert hs.shape[0] == len(ids)
+        logits = np.empty(cfg.vocab, np.float32)
+        res = np.empty((len(ids), cfg.n_embd), np.float32)
+        lib().shv_ref_mtp_rows(C.byref(self.om.mcfg), C.byref(self.om.w), C.byref(self.w), H(self.kc), H(self.vc),
+                               F(hs), I(ids), len(ids), pos, F(logits), F(res), threads)
+        return logits, res

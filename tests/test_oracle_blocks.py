@@ -397,28 +397,28 @@ def test_attention_cache_steps_equal_one_pass():
 
 # ------------------------------------------------------------------- token loop ----------------
 
-def test_model_loop_chunk_split_and_composition():
-    """Pre-norm residual composition (attn every 2nd layer here): the loop in pieces equals the loop
-    at once, and the hidden state equals the layers applied by hand."""
-    rng = np.random.default_rng(13)
+class TinyCfg:
+    n_layer, n_embd, vocab, attn_every, rms_eps = 2, 512, 300, 2, EPS
+    n_expert, n_expert_used, ffn_expert = 8, 2, 256
+    ssm_head_dim, ssm_head_k, ssm_head_v, ssm_conv = 128, 2, 4, 4
+    n_head, n_head_kv, head_dim, rope_dims, rope_base = 4, 2, 64, 32, 1e7
 
-    class Cfg:
-        n_layer, n_embd, vocab, attn_every, rms_eps = 2, 512, 300, 2, EPS
-        n_expert, n_expert_used, ffn_expert = 8, 2, 256
-        ssm_head_dim, ssm_head_k, ssm_head_v, ssm_conv = 128, 2, 4, 4
-        n_head, n_head_kv, head_dim, rope_dims, rope_base = 4, 2, 64, 32, 1e7
 
-    c = Cfg
+def tiny_tensors(rng, c, draft=False):
+    """Random tensors of a two-layer model (DeltaNet, then attention) by GGUF name; with `draft`,
+    block n_layer is the draft head's attention block with its nextn tensors."""
     H, d = c.n_embd, c.ssm_head_dim
     qk, vw = c.ssm_head_k * d, c.ssm_head_v * d
+    gam = lambda n: (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
     t = {"token_embd.weight": rng.standard_normal((c.vocab, H)).astype(np.float16).view(np.uint16),
-         "output_norm.weight": (1 + 0.1 * rng.standard_normal(H)).astype(np.float32),
-         "output.weight": q4(rng, c.vocab, H)}
-    for l in range(c.n_layer):
+         "output_norm.weight": gam(H), "output.weight": q4(rng, c.vocab, H)}
+    for l in range(c.n_layer + (1 if draft else 0)):
         b = lambda n: "blk.%d.%s.weight" % (l, n)
-        t[b("attn_norm")] = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
-        t[b("post_attention_norm")] = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
-        if (l + 1) % c.attn_every == 0:
+        t[b("attn_norm")], t[b("post_attention_norm")] = gam(H), gam(H)
+        if l >= c.n_layer:
+            t[b("nextn.enorm")], t[b("nextn.hnorm")], t[b("nextn.shared_head_norm")] = gam(H), gam(H), gam(H)
+            t[b("nextn.eh_proj")] = q4(rng, H, 2 * H)
+        if l >= c.n_layer or (l + 1) % c.attn_every == 0:
             t[b("attn_q")], t[b("attn_k")], t[b("attn_v")] = q4(rng, c.n_head * 2 * c.head_dim, H), q4(rng, c.n_head_kv * c.head_dim, H), q4(rng, c.n_head_kv * c.head_dim, H)
             t[b("attn_output")] = q4(rng, H, c.n_head * c.head_dim)
             t[b("attn_q_norm")] = np.ones(c.head_dim, np.float32)
@@ -435,6 +435,18 @@ def test_model_loop_chunk_split_and_composition():
         t[b("ffn_gate_exps")], t[b("ffn_up_exps")] = q4(rng, c.n_expert * c.ffn_expert, H), q4(rng, c.n_expert * c.ffn_expert, H)
         t[b("ffn_down_exps")] = q4(rng, c.n_expert * H, c.ffn_expert)
         t[b("ffn_gate_shexp")], t[b("ffn_up_shexp")], t[b("ffn_down_shexp")] = q4(rng, c.ffn_expert, H), q4(rng, c.ffn_expert, H), q4(rng, H, c.ffn_expert)
+    return t
+
+
+def test_model_loop_chunk_split_and_composition():
+    """Pre-norm residual composition (attn every 2nd layer here): the loop in pieces equals the loop
+    at once, and the hidden state equals the layers applied by hand."""
+    rng = np.random.default_rng(13)
+
+    c = TinyCfg
+    H, d = c.n_embd, c.ssm_head_dim
+    qk, vw = c.ssm_head_k * d, c.ssm_head_v * d
+    t = tiny_tensors(rng, c)
     ids = rng.integers(0, c.vocab, size=6).astype(np.int32)
     m1 = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
     lg1, hd1 = m1.extend(ids, threads=1)
@@ -463,3 +475,76 @@ def test_model_loop_chunk_split_and_composition():
         L.shv_ref_moe_block(O.C.byref(m3.mcfg.moe), O.C.byref(lw.moe), O.F(xn), 1, O.F(y), None, None, None, None, None, None, 1)
         x = x + y
     assert np.array_equal(x[0], hd3)
+
+
+
+def test_extend_rows_is_extend_row_by_row():
+    """Every row of the verification pass carries the logits and residual that Extend returns for
+    the sequence cut after that row; the carried state afterwards is the same."""
+    rng = np.random.default_rng(21)
+    c = TinyCfg
+    t = tiny_tensors(rng, c)
+    ids = rng.integers(0, c.vocab, size=5).astype(np.int32)
+    a = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
+    a.extend(ids[:2], threads=1)
+    lg_rows, hd_rows = a.extend_rows(ids[2:], threads=1)
+    b = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
+    b.extend(ids[:2], threads=1)
+    for r in range(3):
+        lg, hd = b.extend(ids[2 + r:3 + r], threads=1)
+        assert np.array_equal(lg, lg_rows[r]) and np.array_equal(hd, hd_rows[r]), r
+    assert a.past == b.past == 5
+    assert np.array_equal(a.dn_s[0], b.dn_s[0]) and np.array_equal(a.kc[1], b.kc[1])
+    # snapshot / restore brings the sequence back to where it was
+    snap = a.snapshot()
+    a.extend(ids[:1], threads=1)
+    a.restore(snap)
+    assert a.past == 5 and np.array_equal(a.dn_s[0], b.dn_s[0]) and np.array_equal(a.kc[1], b.kc[1])
+
+
+def test_draft_head_wiring():
+    """The draft head from its parts: concat(norm(embedding), norm(h)) through eh_proj, one attention
+    block over the draft's own cache, the MoE, the head norm and the trunk's lm_head.  Swapping the
+    two input norms or the halves of the concatenation changes the result (negative controls), and
+    three rows at once equal one row then two."""
+    rng = np.random.default_rng(22)
+    c = TinyCfg
+    t = tiny_tensors(rng, c, draft=True)
+    H = c.n_embd
+    om = O.OracleModel(c, t, max_cells=16, sections=(6, 5, 5, 0))
+    hs = rng.standard_normal((3, H)).astype(np.float32)
+    ids = rng.integers(0, c.vocab, size=3).astype(np.int32)
+    d1 = O.OracleMTP(om, 16)
+    lg, res = d1.rows(hs, ids, 0, threads=1)
+    d2 = O.OracleMTP(om, 16)
+    d2.rows(hs[:1], ids[:1], 0, threads=1)
+    lg2, res2 = d2.rows(hs[1:], ids[1:], 1, threads=1)
+    assert np.array_equal(lg, lg2) and np.array_equal(res[1:], res2)
+    assert np.array_equal(d1.kc, d2.kc) and np.array_equal(d1.vc, d2.vc)
+
+    b = lambda n: t["blk.%d.%s.weight" % (c.n_layer, n)]
+
+    def by_hand(first_norm, second_norm, swap_halves):
+        e = t["token_embd.weight"][ids[:1]].view(np.float16).astype(np.float32)
+        parts = [O.rmsnorm(e, b(first_norm), EPS)[0], O.rmsnorm(hs[:1], b(second_norm), EPS)[0]]
+        cat = np.concatenate(parts[::-1] if swap_halves else parts)
+        x = O.gemv_q4k(b("nextn.eh_proj"), cat, H, 2 * H)[None]
+        lw = d1.w.layer
+        y = np.empty_like(x)
+        kc, vc = np.zeros((16, c.n_head_kv, c.head_dim), np.uint16), np.zeros((16, c.n_head_kv, c.head_dim), np.uint16)
+        xn = O.rmsnorm(x, b("attn_norm"), EPS)
+        L.shv_ref_attn_layer(O.C.byref(om.mcfg.attn), O.C.byref(lw.attn), O.F(xn), 1, 0, O.H(kc), O.H(vc), O.F(y), None, None, 1)
+        x = x + y
+        xn = O.rmsnorm(x, b("post_attention_norm"), EPS)
+        L.shv_ref_moe_block(O.C.byref(om.mcfg.moe), O.C.byref(lw.moe), O.F(xn), 1, O.F(y), None, None, None, None, None, None, 1)
+        x = x + y
+        logits = O.gemv_q4k(t["output.weight"], O.rmsnorm(x, b("nextn.shared_head_norm"), EPS)[0], c.vocab, H)
+        return x[0], logits
+
+    d3 = O.OracleMTP(om, 16)
+    lg1, res1 = d3.rows(hs[:1], ids[:1], 0, threads=1)
+    x, logits = by_hand("nextn.enorm", "nextn.hnorm", False)
+    assert np.array_equal(x, res1[0]) and np.array_equal(logits, lg1)
+    for args in (("nextn.hnorm", "nextn.enorm", False), ("nextn.enorm", "nextn.hnorm", True)):
+        x_bad, _ = by_hand(*args)
+        assert O.rel_l2(x_bad, res1[0]) > 1e-2

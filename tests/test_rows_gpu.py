@@ -1,0 +1,271 @@
+"""Multi-row passes, sequence slots, rewindable passes, the draft head and the speculative loop on
+the GPU against the CPU oracle.  The reference's gates of this kind: TestGraphIsAChunkSplit
+(llm/graph_cache_test.go:39), TestSpeculationRewindIsTheSequence and the keep-prefix tests of
+llm/graph_spec_test.go, TestDecodeRowsIsTheSequences (llm/batch_test.go), and the losslessness
+argument of llm/spec.go:49-56 (every emitted token is the trunk's own arg-max)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import shv
+
+pytestmark = pytest.mark.gpu
+LA = shv.pkg.llm_api
+ROWS = 4  # rows of the widest pass: draft depth 3 + 1
+
+
+def cfg_rows(**kw):
+    d = dict(n_layer=4, n_expert=16, n_expert_used=4, vocab=4096, nkv=128, max_tokens=ROWS, slots=3,
+             head_rows=ROWS, speculative=1, spec_rows=ROWS, nextn=1)
+    d.update(kw)
+    return LA.Config(**d)
+
+
+@pytest.fixture(scope="module")
+def rig():
+    cfg = cfg_rows()
+    m = LA.LLM(cfg)
+    m.init_synthetic(4321)
+    m.stage()
+    tensors = {t[0]: m.download(t[0]) for t in m.tensors()}
+    yield m, cfg, tensors
+    m.close()
+
+
+def fresh(m, slot=0):
+    m.speculate(False)
+    m.speculate_first(False)
+    m.use_slot(slot)
+    m.reset()
+
+
+def test_chunked_prompt_matches_the_cpu(rig):
+    """11 prompt rows go through as 4+4+3; the last row's logits and residual are the CPU's."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(11)
+    prompt = rng.integers(0, cfg.vocab, size=11).astype(np.int32)
+    om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+    fresh(m)
+    lg, hd = m.extend(prompt, want_hidden=True)
+    lg_cpu, hd_cpu = om.extend(prompt)
+    assert O.rel_l2(hd, hd_cpu) <= 1e-3 and O.rel_l2(lg, lg_cpu) <= 1e-3
+    assert m.past() == 11
+    # the same prompt in other pieces (5+6: passes of 4+1 and 4+2 rows)
+    fresh(m)
+    m.extend(prompt[:5])
+    lg2, _ = m.extend(prompt[5:])
+    assert O.rel_l2(lg2, lg) <= 1e-5
+    # the carried state agrees with the CPU's
+    assert O.rel_l2(m.dn_state(0), om.dn_s[0]) <= 1e-3
+    k, v = m.kv(3, 11)
+    kf = lambda a: a.view(np.float16).astype(np.float32)
+    assert O.rel_l2(kf(k), kf(om.kc[3][:11])) <= 2e-3 and O.rel_l2(kf(v), kf(om.vc[3][:11])) <= 2e-3
+
+
+def test_extend_rows_is_every_rows_logits(rig):
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(12)
+    prompt = rng.integers(0, cfg.vocab, size=6).astype(np.int32)
+    rows = rng.integers(0, cfg.vocab, size=ROWS).astype(np.int32)
+    om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+    om.extend(prompt)
+    lg_cpu, res_cpu = om.extend_rows(rows)
+    fresh(m)
+    m.extend(prompt)
+    best, lg, res = m.extend_rows(rows, want_logits=True, want_res=True)
+    assert m.past() == 6 + ROWS
+    for r in range(ROWS):
+        assert O.rel_l2(lg[r], lg_cpu[r]) <= 1e-3, r
+        assert O.rel_l2(res[r], res_cpu[r]) <= 1e-3, r
+        assert best[r] == int(O.lib().shv_ref_argmax(O.F(np.ascontiguousarray(lg[r])), cfg.vocab))
+    with pytest.raises(shv.pkg.ShvError):
+        m.extend_rows(np.zeros(ROWS + 1, np.int32))      # more rows than the head arena holds
+
+
+@pytest.mark.parametrize("keep", [1, 2, 3, 4])
+def test_keeping_a_prefix_is_the_shorter_sequence(rig, keep):
+    """A rewindable 4-row pass, then Keep(k): the sequence, the DeltaNet state and what the next
+    token sees are those of the prompt plus the first k rows alone."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(13)
+    prompt = rng.integers(0, cfg.vocab, size=7).astype(np.int32)
+    rows = rng.integers(0, cfg.vocab, size=ROWS).astype(np.int32)
+    probe = rng.integers(0, cfg.vocab, size=1).astype(np.int32)
+    om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+    om.extend(prompt)
+    om.extend(rows[:keep])
+    want_state = om.dn_s[0].copy()
+    lg_cpu, _ = om.extend(probe)
+
+    fresh(m)
+    m.extend(prompt)
+    plane0 = m.plane()
+    m.speculate(True)
+    m.speculate_first(True)
+    m.extend_rows(rows)
+    with pytest.raises(shv.pkg.ShvError):
+        m.extend_rows(rows)                               # one pass in flight at most
+    with pytest.raises(shv.pkg.ShvError):
+        m.rewind()                                        # a keep-first pass is kept or committed
+    m.keep(keep)
+    assert m.past() == 7 + keep
+    assert m.plane() == (plane0 + keep) % (ROWS + 1)
+    assert O.rel_l2(m.dn_state_at(0, 0, m.plane()), want_state) <= 1e-3
+    assert list(m.ids()) == list(prompt) + list(rows[:keep])
+    lg = m.extend_rows(probe, want_logits=True)[1]
+    m.commit()
+    assert O.rel_l2(lg[0], lg_cpu) <= 1e-3
+    # and the plain recorded decode step runs from the plane the passes left committed
+    m.speculate(False)
+    tok = np.array([int(np.argmax(lg_cpu))], np.int32)
+    lg_next, _ = m.extend(tok)
+    lg_next_cpu, _ = om.extend(tok)
+    assert O.rel_l2(lg_next, lg_next_cpu) <= 1e-3
+
+
+def test_rewind_discards_the_pass(rig):
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(14)
+    prompt = rng.integers(0, cfg.vocab, size=5).astype(np.int32)
+    rows = rng.integers(0, cfg.vocab, size=3).astype(np.int32)
+    probe = rng.integers(0, cfg.vocab, size=2).astype(np.int32)
+    fresh(m)
+    m.extend(prompt)
+    before = m.dn_state_at(0, 0, m.plane()).copy()
+    want, _ = m.extend(probe)            # the control: the probe straight after the prompt
+    fresh(m)
+    m.extend(prompt)
+    m.speculate(True)
+    m.extend_rows(rows)
+    assert m.past() == 8
+    with pytest.raises(shv.pkg.ShvError):
+        m.keep(1)                         # prefixes are kept only under SpeculateFirst
+    m.rewind()
+    assert m.past() == 5
+    assert np.array_equal(m.dn_state_at(0, 0, m.plane()), before)
+    m.speculate(False)
+    got, _ = m.extend(probe)
+    assert np.array_equal(got, want)
+    with pytest.raises(shv.pkg.ShvError):
+        m.commit()                        # nothing in flight
+
+
+def test_speculate_needs_the_planes():
+    cfg = cfg_rows(speculative=0, nextn=0, slots=1)
+    m = LA.LLM(cfg)
+    m.init_synthetic(1)
+    m.stage()
+    with pytest.raises(shv.pkg.ShvError):
+        m.speculate(True)
+    m.close()
+
+
+def test_decode_rows_advances_each_sequence(rig):
+    """Three sequences of different lengths take one token each in one pass; every row's logits are
+    those of its own sequence run alone on the CPU (llm/graph.go:1527-1666)."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(15)
+    prompts = [rng.integers(0, cfg.vocab, size=n).astype(np.int32) for n in (3, 9, 6)]
+    toks = rng.integers(0, cfg.vocab, size=3).astype(np.int32)
+    oms = [O.OracleModel(cfg, tensors, max_cells=cfg.nkv) for _ in prompts]
+    for s, p in enumerate(prompts):
+        fresh(m, s)
+        m.extend(p)
+        oms[s].extend(p)
+    order = [2, 0, 1]
+    best, lg = m.decode_rows(order, toks, want_logits=True)
+    for r, s in enumerate(order):
+        lg_cpu, _ = oms[s].extend(toks[r:r + 1])
+        assert O.rel_l2(lg[r], lg_cpu) <= 1e-3, (r, s)
+        assert best[r] == int(np.argmax(lg[r]))
+    for s, p in enumerate(prompts):
+        m.use_slot(s)
+        assert m.past() == len(p) + 1
+        assert m.ids()[-1] == toks[order.index(s)]
+    # a second batched step over two of them, then one alone through the same entry point
+    toks2 = rng.integers(0, cfg.vocab, size=2).astype(np.int32)
+    _, lg2 = m.decode_rows([1, 2], toks2, want_logits=True)
+    for r, s in enumerate([1, 2]):
+        lg_cpu, _ = oms[s].extend(toks2[r:r + 1])
+        assert O.rel_l2(lg2[r], lg_cpu) <= 1e-3
+    _, lg3 = m.decode_rows([0], toks2[:1], want_logits=True)
+    lg_cpu, _ = oms[0].extend(toks2[:1])
+    assert O.rel_l2(lg3[0], lg_cpu) <= 1e-3
+    with pytest.raises(shv.pkg.ShvError):
+        m.decode_rows([0, 0], toks2)                      # a slot twice in one batch
+    with pytest.raises(shv.pkg.ShvError):
+        m.decode_rows([0, 3], toks2)                      # a slot that does not exist
+    m.use_slot(0)
+
+
+def test_draft_head_rows_match_the_cpu(rig):
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(16)
+    om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+    dm = O.OracleMTP(om, cfg.nkv)
+    fresh(m)
+    m.extend(np.array([1, 2, 3], np.int32))               # the head borrows a staged graph
+    m.mtp_stage(max_tok=ROWS)
+    hs = rng.standard_normal((3, cfg.n_embd)).astype(np.float32)
+    ids = rng.integers(0, cfg.vocab, size=3).astype(np.int32)
+    lg, res = m.mtp_rows(hs, ids, 0)
+    lg_cpu, res_cpu = dm.rows(hs, ids, 0)
+    assert O.rel_l2(res, res_cpu) <= 1e-3 and O.rel_l2(lg, lg_cpu) <= 1e-3
+    # a chained step: the draft's own residual behind the next row, over the cells just written
+    one = rng.integers(0, cfg.vocab, size=1).astype(np.int32)
+    lg2, res2 = m.mtp_rows(res[-1:], one, 3)
+    lg2_cpu, res2_cpu = dm.rows(res_cpu[-1:], one, 3)
+    assert O.rel_l2(res2, res2_cpu) <= 1e-3 and O.rel_l2(lg2, lg2_cpu) <= 1e-3
+    assert m.mtp_past() == 4
+    # rewinding is the whole of the draft's rollback: position 2 again sees cells 0..1 only
+    m.mtp_rewind(2)
+    lg3, _ = m.mtp_rows(hs[2:], ids[2:], 2)
+    dm3 = O.OracleMTP(om, cfg.nkv)
+    dm3.rows(hs[:2], ids[:2], 0)
+    lg3_cpu, _ = dm3.rows(hs[2:], ids[2:], 2)
+    assert O.rel_l2(lg3, lg3_cpu) <= 1e-3
+    with pytest.raises(shv.pkg.ShvError):
+        m.mtp_rows(hs[:1], ids[:1], 7)                    # a gap in the draft's cache
+
+
+@pytest.mark.parametrize("mode", ["draft", "all-right", "first-right", "second-right"])
+def test_speculative_loop_emits_the_greedy_sequence(rig, mode):
+    """Whatever the drafts are — the draft head's own, all correct, or correct up to a point — the
+    loop emits exactly the tokens of plain greedy decoding, and keeps as many rows as agree."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(17)
+    prompt = rng.integers(0, cfg.vocab, size=10).astype(np.int32)
+    n_new = 24
+    fresh(m)
+    m.extend(prompt)
+    plain, _ = m.generate(n_new + ROWS)
+    plain = list(plain)
+
+    fresh(m)
+    m.mtp_stage(max_tok=ROWS)
+    depth = ROWS - 1
+    m.spec_open(depth)
+    out = [m.spec_start(prompt)]
+    assert out[0] == plain[0]
+    rounds = 0
+    while len(out) < n_new:
+        nxt = plain[len(out):len(out) + depth]            # the true continuation after the pending token
+        forced = {"draft": [], "all-right": nxt, "first-right": [nxt[0], (nxt[1] + 1) % cfg.vocab, nxt[2]],
+                  "second-right": [nxt[0], nxt[1], (nxt[2] + 1) % cfg.vocab]}[mode]
+        got = list(m.spec_round(forced))
+        want_keep = {"all-right": depth + 1, "first-right": 2, "second-right": 3}.get(mode)
+        if want_keep:
+            assert len(got) == want_keep, (mode, got)
+        out += got
+        rounds += 1
+    assert out[:n_new] == plain[:n_new], mode
+    st = m.spec_stats()
+    assert st["rounds"] == rounds and st["tokens"] == len(out)
+    assert st["passes"][min(depth + 1, 4)] == rounds
+    if mode == "all-right":
+        assert st["accepted_at"][:3] == [rounds] * 3
+    if mode == "first-right":
+        assert st["accepted_at"][0] == rounds and st["accepted_at"][1] == 0
+    # the trunk holds exactly the emitted tokens but the pending one
+    assert m.past() == len(prompt) + len(out) - 1
+    assert list(m.ids()) == list(prompt) + out[:-1]
