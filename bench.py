@@ -17,8 +17,13 @@ Beside the headline it reports
                 bounded sample of the same model: layers 0..3 (one DeltaNet x3 + attention period)
                 plus the head, a few decode tokens, scaled by 12 periods to a 48-layer token
   gemv          the single Q4_K GEMV of BASELINE config 1 (4096x2048) over a rotating set of
-                distinct weight matrices larger than the 256 MB Infinity Cache, and the 175 MB
-                lm_head GEMV, in GB/s and as a fraction of 8 TB/s
+                distinct weight matrices of more than 2 GiB in all (the Infinity Cache is 256 MB), and
+                the 175 MB lm_head GEMV, in GB/s and as a fraction of 8 TB/s
+  mtp           BASELINE config 5's second run: a one-block draft head at depth 2 and batched
+                3-row verification passes.  What a 2-row and a 3-row pass cost in decode steps, what
+                a draft costs, and the greedy speculative loop's rounds on this (random-init, so
+                never-agreeing) draft head; beside it the same rounds fed the true continuation as
+                drafts, which prices the mechanics when every draft is accepted
 """
 import argparse
 import importlib
@@ -104,13 +109,18 @@ def gemv_rates(m, cfg, A, LA):
         return p.value
 
     n, k = 4096, cfg.n_embd
-    bank = next(t for t in m.tensors() if t[0] == "blk.0.ffn_gate_exps.weight")
     mat_bytes = n * Q4K_ROW(k)
-    copies = min(bank[2] // mat_bytes, 128)
+    # distinct 4096x2048 matrices: windows of the experts' gate banks, layer after layer, until
+    # more than 2 GiB of weights rotate
+    mats = []
+    for t in m.tensors():
+        if t[0].endswith("ffn_gate_exps.weight") and len(mats) * mat_bytes < (2 << 30):
+            mats += [t[1] + i * mat_bytes for i in range(t[2] // mat_bytes)]
+    copies = len(mats)
     dx, dy = alloc(k * 4), alloc(max(n, cfg.vocab) * 4)
     x = np.random.default_rng(2).standard_normal(k).astype(np.float32)
     A.check(H.shv_upload(ctx, dx, x.ctypes.data, x.nbytes))
-    ops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(bank[1] + i * mat_bytes, dx, dy, n, k)) for i in range(copies)]
+    ops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(w, dx, dy, n, k)) for w in mats]
     arr = (A.Op * len(ops))(*ops)
     pre = C.c_void_p()
     A.check(H.shv_prerecord(ctx, arr, len(ops), C.byref(pre)))
@@ -137,6 +147,34 @@ def gemv_rates(m, cfg, A, LA):
     return out
 
 
+def mtp_run(m, cfg, prompt, plain, acc, rounds):
+    """Pass costs in decode steps and the speculative loop at depth 2 (3-row verification)."""
+    kernels = lambda st: sum(v for k, v in st if k != "total")
+    step_ns = sum(v for k, v in acc.items() if k != "total")
+    out = {"depth": 2, "draft_vocab": 65536}
+    for rows in (2, 3):
+        st = [m.profile_rows(rows) for _ in range(4)]
+        out["pass_%d_rows_in_steps" % rows] = round(sum(kernels(x) for x in st) / len(st) / step_ns, 3)
+    m.mtp_stage(max_tok=4, vocab_prefix=65536)
+    m.spec_open(2)
+    for mode in ("draft_head", "true_continuation_as_drafts"):
+        first = m.spec_start(prompt)       # prefills the trunk again and primes the draft over the prompt
+        toks = [first]
+        t0 = time.perf_counter()
+        for _ in range(rounds):
+            forced = plain[len(toks):len(toks) + 2] if mode != "draft_head" else []
+            toks += list(m.spec_round(forced))
+        dt = time.perf_counter() - t0
+        st = m.spec_stats()
+        out[mode] = {"rounds": st["rounds"], "tokens_per_round": round((st["tokens"] - 1) / st["rounds"], 3),
+                     "accepted_at": st["accepted_at"][:2], "drafted_at": st["drafted_at"][:2],
+                     "round_ms": round(dt / rounds * 1e3, 4), "tok_s": round((len(toks) - 1) / dt, 1),
+                     "draft_gpu_ms_per_round": round(st["draft_ns"] / st["rounds"] / 1e6, 4),
+                     "verify_gpu_ms_per_round": round(st["verify_ns"] / st["rounds"] / 1e6, 4),
+                     "emitted_equals_plain_greedy": toks == plain[:len(toks)]}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -146,6 +184,8 @@ def main():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--cpu-tokens", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-mtp", action="store_true")
+    ap.add_argument("--mtp-rounds", type=int, default=64)
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware-counter readings of HBM traffic are scaled by")
@@ -157,8 +197,11 @@ def main():
         sys.exit("bench.py: --steps and --warmup must be at least 1")
     pkg = importlib.import_module("strix-halo-vulkan_amd")
     LA, A = pkg.llm_api, pkg.hip_api
-    nkv = a.prompt + a.warmup + a.steps + 64
-    cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128)
+    nkv = a.prompt + a.warmup + a.steps + 3 * a.mtp_rounds + 64
+    # prompt rows go through four at a time; the draft block and the state planes of rewindable
+    # 3-row passes are staged for the speculative run and cost the plain decode step nothing
+    cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=4, head_rows=3, speculative=1,
+                    spec_rows=3, nextn=1)
     m = LA.LLM(cfg)
     m.init_synthetic(20260101)
     m.stage()
@@ -167,7 +210,7 @@ def main():
     t0 = time.perf_counter()
     m.extend(prompt, want_logits=False)
     prefill_s = time.perf_counter() - t0
-    m.generate(a.warmup + 1)              # W untimed decode steps
+    ids_w, _ = m.generate(a.warmup + 1)   # W untimed decode steps
     t0 = time.perf_counter()              # generate() returns only after the stream has drained
     ids, gpu_ns = m.generate(a.steps + 1)  # exactly K replays of the recorded decode step
     wall = time.perf_counter() - t0
@@ -201,7 +244,7 @@ def main():
                                "drawn N(0,0.02) and quantised on the device by the reference's quantiser, fp16 KV "
                                "cache, vocab 151936; prompt %d random ids then greedy decode at batch 1"
                                % (cfg.n_layer, a.prompt),
-                   "context_at_end": ctx_len, "prefill": "token by token through the recorded step (%.1f tok/s, untimed)"
+                   "context_at_end": ctx_len, "prefill": "four rows a pass through the decode kernels (%.1f tok/s, untimed)"
                                                           % (a.prompt / prefill_s),
                    "weights_GB": round(m.weight_bytes() / 1e9, 2), "dispatches_per_step": m.dispatches()},
         "gpu_ms_per_step": round(gpu_ns / a.steps / 1e6, 4),
@@ -221,6 +264,11 @@ def main():
         A.check(H.shv_copy(m.ctx, dst, src, n))
         A.check(H.shv_sync(m.ctx))
         rec["pmc_copy_bytes"] = n
+    if not a.no_mtp:
+        plain = [int(t) for t in ids_w] + [int(t) for t in ids[1:]]
+        rounds = min(a.mtp_rounds, (len(plain) - 4) // 3)
+        if rounds >= 1:
+            rec["mtp"] = mtp_run(m, cfg, prompt, plain, acc, rounds)
     if not a.no_cpu:
         rec["cpu_baseline"] = cpu_baseline(m, cfg, LA, a.cpu_tokens)
     m.close()
