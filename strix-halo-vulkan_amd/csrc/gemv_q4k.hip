@@ -298,6 +298,7 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
         SHV_REQUIRE((a.z_ring || (a.ring_stride >= a.n && !a.residual)) && sl <= a.ring_slots && a.n_tok % sl == 0,
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
+    if (a.n_tok >= ctx->mfma_min_rows && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
     switch (a.k) {
         case 512: return launch_k<512>(ctx, a);
         case 1024: return launch_k<1024>(ctx, a);

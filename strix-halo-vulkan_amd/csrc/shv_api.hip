@@ -1,4 +1,5 @@
 // C-ABI layer: context, buffers, op dispatch, timed sequences and prerecorded (HIP graph) replay.
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -37,6 +38,10 @@ int shv_init(int device, shv_ctx **out) {
     shv_ctx *ctx = new (std::nothrow) shv_ctx();
     if (!ctx) return shv_set_error(SHV_E_NOMEM, "shv_init: out of host memory");
     ctx->device = device;
+    if (const char *e = std::getenv("SHV_MFMA_MIN_ROWS")) {
+        const int v = std::atoi(e);
+        if (v >= 2) ctx->mfma_min_rows = v;
+    }
     hipError_t e = hipGetDeviceProperties(&ctx->prop, device);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev_begin);

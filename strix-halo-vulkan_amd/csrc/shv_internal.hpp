@@ -17,6 +17,9 @@ struct shv_ctx {
     hipDeviceProp_t prop{};
     uint64_t submits = 0;
     bool capturing = false;
+    // Q4_K projections of at least this many rows run on the matrix cores (SHV_MFMA_MIN_ROWS in
+    // the environment overrides it; a large value keeps every pass on the row kernel)
+    int mfma_min_rows = 3;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
     int32_t *counters = nullptr;
@@ -88,6 +91,9 @@ static inline bool shv_aligned16(const void *p) { return (reinterpret_cast<uintp
 
 // one launcher per op kind; each validates its argument block on the host before launching
 int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
+// the matrix-core kernel for passes of two rows and more (gemm_q4k.hip)
+bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a);
+int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a);
 int shv_launch_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
 int shv_launch_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
 int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);

@@ -1,0 +1,158 @@
+"""Q4_K projections of several rows run on the matrix cores (gemm_q4k.hip); these tests hold
+that kernel to the oracle's GEMV row by row (matvec over dequantised rows, llm/hc.go:255-264), to a
+float64 product, and to the one-row kernel it replaces, over the shapes, prologues and output
+layouts the token loop uses (verification passes, batched decode rows, prompt chunks)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import shv
+
+pytestmark = pytest.mark.gpu
+A = shv.api
+TOL = 1e-3      # the bar against the oracle (its own sequential float32 sums are ~1e-6 off)
+TOL64 = 1e-5    # against float64: the activations go in as two halves, the products are exact
+
+
+def _weights(rng, n, k, std=0.02):
+    return O.quantize_q4k((rng.standard_normal((n, k)) * std).astype(np.float32))
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    """A context that sends every pass of two rows and more to the matrix-core kernel (the
+    library's own threshold is tuned to where that kernel starts to win)."""
+    os.environ["SHV_MFMA_MIN_ROWS"] = "2"
+    try:
+        c = A.Context(0)
+    finally:
+        del os.environ["SHV_MFMA_MIN_ROWS"]
+    yield c
+    c.destroy()
+
+
+@pytest.fixture(scope="module")
+def row_ctx():
+    """A second context that keeps every pass on the row kernel, to compare the two."""
+    os.environ["SHV_MFMA_MIN_ROWS"] = "1000"
+    try:
+        c = A.Context(0)
+    finally:
+        del os.environ["SHV_MFMA_MIN_ROWS"]
+    yield c
+    c.destroy()
+
+
+@pytest.mark.parametrize("n,k,rows", [(1024, 2048, 2), (4096, 2048, 3), (2048, 4096, 4), (2048, 512, 16),
+                                      (48, 1024, 5), (7, 2048, 2), (33, 256, 9), (12352, 2048, 16),
+                                      (2048, 4096, 17), (512, 2048, 40)])
+def test_rows_match_oracle_and_float64(ctx, row_ctx, n, k, rows):
+    rng = np.random.default_rng(n + k + rows)
+    wq = _weights(rng, n, k)
+    x = (rng.standard_normal((rows, k)) * rng.uniform(0.01, 30.0, size=(rows, 1))).astype(np.float32)
+    w64 = O.dequant_q4k(wq, k).astype(np.float64)
+    dy = ctx.alloc(rows * n * 4)
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(x), dy, n, k, n_tok=rows)
+    got = dy.read(np.float32, rows * n).reshape(rows, n)
+    ref = None
+    if k >= 512:  # the row kernel's narrowest matrix
+        dy2 = row_ctx.alloc(rows * n * 4)
+        row_ctx.gemv_q4k(row_ctx.upload(wq), row_ctx.upload(x), dy2, n, k, n_tok=rows)
+        ref = dy2.read(np.float32, rows * n).reshape(rows, n)
+    worst = 0.0
+    for t in range(rows):
+        assert O.rel_l2(got[t], O.gemv_q4k(wq, x[t], n, k, threads=8)) <= TOL, t
+        e64 = O.rel_l2(got[t], w64 @ x[t].astype(np.float64))
+        worst = max(worst, e64)
+        assert e64 <= TOL64, (t, e64)
+        assert ref is None or O.rel_l2(got[t], ref[t]) <= TOL64, t
+    print(f"gemm {n}x{k} x{rows}: worst rel-L2 vs float64 {worst:.2e}")
+
+
+def test_rmsnorm_prologue_residual_in_place(ctx):
+    """The residual stream's own rows are the residual and the destination (dn.out, attn.out, the
+    MoE down projection write x in place)."""
+    rng = np.random.default_rng(31)
+    n, k, rows, eps = 2048, 2048, 3, 1e-6
+    wq = _weights(rng, n, k)
+    h = (rng.standard_normal((rows, k)) * 3).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    res = rng.standard_normal((rows, n)).astype(np.float32)
+    dy = ctx.upload(res)
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(h), dy, n, k, n_tok=rows, prologue=A.PRO_RMSNORM,
+                 gamma=ctx.upload(gamma), residual=dy, eps=eps)
+    got = dy.read(np.float32, rows * n).reshape(rows, n)
+    for t in range(rows):
+        want = O.gemv_q4k(wq, O.rmsnorm(h[t], gamma, eps), n, k, threads=8) + res[t]
+        assert O.rel_l2(got[t], want) <= TOL, t
+
+
+def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx):
+    """DeltaNet's output projection at its real shape: 4096 columns (two column ranges), per-head
+    norm, the gate z read from the projection ring at each row's position, residual in place."""
+    rng = np.random.default_rng(32)
+    n, k, d, eps, rows, slots = 2048, 4096, 128, 1e-6, 4, 8
+    ring_stride, z_col = 12352, 8192
+    wq = _weights(rng, n, k)
+    o = rng.standard_normal((rows, k)).astype(np.float32)
+    ring = rng.standard_normal((2, slots, ring_stride)).astype(np.float32)   # two sequence slots
+    gamma = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    res = rng.standard_normal((rows, n)).astype(np.float32)
+    pos, slot = 13, 1
+    L = O.lib()
+    dring, dy = ctx.upload(ring), ctx.upload(res)
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(o), dy, n, k, n_tok=rows, prologue=A.PRO_GATED_NORM,
+                 gamma=ctx.upload(gamma), z=dring.at(z_col * 4), head_dim=d, eps=eps, residual=dy,
+                 pos=ctx.upload(np.array([pos], np.int32)), slot=ctx.upload(np.array([slot], np.int32)),
+                 seq_len=rows, ring_slots=slots, ring_stride=ring_stride, z_ring=1)
+    got = dy.read(np.float32, rows * n).reshape(rows, n)
+    for t in range(rows):
+        z = ring[slot, (pos + t) % slots, z_col:z_col + k]
+        xn = O.rmsnorm(o[t].reshape(-1, d), gamma, eps).ravel()
+        sig = np.array([L.shv_ref_sigmoid(float(v)) for v in z], dtype=np.float32)
+        want = O.gemv_q4k(wq, (xn * sig).astype(np.float32), n, k, threads=8) + res[t]
+        assert O.rel_l2(got[t], want) <= TOL, t
+
+
+def test_sigmoid_gate_prologue_with_fused_query_rows(ctx):
+    """Attention's output projection: x * sigmoid(gate), the gate being the second half of each
+    head's [q | gate] rows in the fused projection (llm/attn.go:162-166,198-205)."""
+    rng = np.random.default_rng(33)
+    n, k, d, rows = 2048, 4096, 256, 3
+    heads, zw = k // d, 2 * k + 1024
+    wq = _weights(rng, n, k)
+    c = rng.standard_normal((rows, k)).astype(np.float32)
+    qkv = rng.standard_normal((rows, zw)).astype(np.float32)
+    L = O.lib()
+    dy = ctx.alloc(rows * n * 4)
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(c), dy, n, k, n_tok=rows, prologue=A.PRO_MUL_SIGMOID,
+                 z=ctx.upload(qkv), head_dim=d, z_stride=zw)
+    got = dy.read(np.float32, rows * n).reshape(rows, n)
+    for t in range(rows):
+        gate = np.concatenate([qkv[t, h * 2 * d + d:(h + 1) * 2 * d] for h in range(heads)])
+        sig = np.array([L.shv_ref_sigmoid(float(v)) for v in gate], dtype=np.float32)
+        want = O.gemv_q4k(wq, (c[t] * sig).astype(np.float32), n, k, threads=8)
+        assert O.rel_l2(got[t], want) <= TOL, t
+
+
+def test_ring_output_for_sequences_and_slots(ctx):
+    """The DeltaNet input projection writes each row into its sequence's ring at its position:
+    here two sequences of three rows each, on slots 2 and 0, wrapping around an 8-row ring."""
+    rng = np.random.default_rng(34)
+    n, k, slots, n_slots, seq_len = 528, 2048, 8, 3, 3
+    wq = _weights(rng, n, k)
+    x = rng.standard_normal((2 * seq_len, k)).astype(np.float32)
+    pos, slot = np.array([6, 17], np.int32), np.array([2, 0], np.int32)
+    ring = ctx.upload(np.full(n_slots * slots * n, -7.0, dtype=np.float32))
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(x), ring, n, k, n_tok=2 * seq_len, pos=ctx.upload(pos),
+                 slot=ctx.upload(slot), seq_len=seq_len, ring_slots=slots, ring_stride=n)
+    got = ring.read(np.float32, n_slots * slots * n).reshape(n_slots, slots, n)
+    written = np.zeros((n_slots, slots), bool)
+    for s in range(2):
+        for i in range(seq_len):
+            row = got[slot[s], (pos[s] + i) % slots]
+            assert O.rel_l2(row, O.gemv_q4k(wq, x[s * seq_len + i], n, k, threads=8)) <= TOL, (s, i)
+            written[slot[s], (pos[s] + i) % slots] = True
+    assert (got[~written] == -7.0).all()
