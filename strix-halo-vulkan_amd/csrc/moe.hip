@@ -121,12 +121,26 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         kl[i] = e < n_expert ? static_cast<uint32_t>(0x7FFFFFFF - e) : 0u;
         lane_max = kh[i] > lane_max ? kh[i] : lane_max;
     }
-    // thr = the n_used-th largest lane maximum: the largest v with at least n_used lanes >= v
+    // thr = the n_used-th largest lane maximum.  Every lane ranks its own maximum among the 64
+    // (ties by lane, so the ranks are distinct); the lane of rank n_used-1 holds the threshold.
     uint32_t thr = 0u;
-#pragma unroll 1
-    for (int b = 30; b >= 0; b--) {
-        const uint32_t c = thr | (1u << b);
-        if (__popcll(__ballot(lane_max >= c)) >= n_used) thr = c;
+    if (n_used <= 64) {
+        uint32_t *lm = cand_p;  // the candidate table is not in use yet
+        lm[lane] = lane_max;
+        __builtin_amdgcn_wave_barrier();
+        int rank = 0;
+#pragma unroll
+        for (int j4 = 0; j4 < 16; j4++) {
+            const uint4 o = *reinterpret_cast<const uint4 *>(lm + 4 * j4);
+            const uint32_t ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) rank += (ov[j] > lane_max || (ov[j] == lane_max && 4 * j4 + j < lane)) ? 1 : 0;
+        }
+        uint32_t *thr_slot = reinterpret_cast<uint32_t *>(sel_e);
+        if (rank == n_used - 1) *thr_slot = lane_max;
+        __builtin_amdgcn_wave_barrier();
+        thr = *thr_slot;
+        __builtin_amdgcn_wave_barrier();
     }
     // compact the keys at or above it
     int total = 0;

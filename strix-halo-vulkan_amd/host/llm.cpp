@@ -197,6 +197,7 @@ void Model::InitSynthetic(uint64_t seed) {
 MoEGPU::MoEGPU(Device &dev, const Model &m, int maxTokens) : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens) {
     if (maxTokens < 1) throw Error("llm: MoEGPU needs room for at least one token");
     if (c_.NExpertUsed > c_.NExpert) throw Error("llm: MoEGPU: more experts used than there are");
+    if (const char *e = std::getenv("LLM_MOE_ROUTE")) fused_route_ = std::strcmp(e, "kernel") != 0;
     const size_t T = maxTokens;
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
@@ -236,6 +237,7 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     r.n_used = c_.NExpertUsed;
     r.eps = c_.RMSEps;
     r.h_stride = c_.NEmbd;
+    r.defer_route = fused_route_ ? 1 : 0;
     shv_moe_up_args u{};
     u.xn = xn_;
     u.topk = topk_;
@@ -248,6 +250,11 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     u.n_embd = c_.NEmbd;
     u.n_used = c_.NExpertUsed;
     u.ffn = c_.FFNExpert;
+    if (fused_route_) {
+        u.logits = logits_;
+        u.weights = weights_;
+        u.n_expert = c_.NExpert;
+    }
     shv_moe_down_args d{};
     d.act = act_;
     d.topk = topk_;

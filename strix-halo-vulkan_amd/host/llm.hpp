@@ -161,6 +161,10 @@ public:
     float *InPort() const { return in_; }
     float *OutPort() const { return out_; }
     uint64_t ActivationBytes() const { return act_bytes_; }
+    // Where the top-k selection runs (MoEGPU.SetRouter, llm/gpu_moe.go:307): fused, in the prologue
+    // of the gate/up kernel from the router's logits, or as a dispatch of its own after the router.
+    void SetRouter(bool fused) { fused_route_ = fused; }
+    bool FusedRouter() const { return fused_route_; }
 
 private:
     Device &dev_;
@@ -170,6 +174,7 @@ private:
     float *in_, *out_, *xn_, *logits_, *weights_, *act_;
     int32_t *topk_;
     uint64_t act_bytes_ = 0;
+    bool fused_route_ = true;
 };
 
 // llm.DeltaNetGPU (llm/gpu_deltanet.go:207-322, NewDeltaNetGPUBank :421)

@@ -50,11 +50,12 @@ def test_chunked_prompt_matches_the_cpu(rig):
     lg_cpu, hd_cpu = om.extend(prompt)
     assert O.rel_l2(hd, hd_cpu) <= 1e-3 and O.rel_l2(lg, lg_cpu) <= 1e-3
     assert m.past() == 11
-    # the same prompt in other pieces (5+6: passes of 4+1 and 4+2 rows)
+    # the same prompt in other pieces (5+6: passes of 4+1 and 4+2 rows, which run through other
+    # kernels than 4+4+3 and add up in another order)
     fresh(m)
     m.extend(prompt[:5])
     lg2, _ = m.extend(prompt[5:])
-    assert O.rel_l2(lg2, lg) <= 1e-5
+    assert O.rel_l2(lg2, lg) <= 1e-4
     # the carried state agrees with the CPU's
     assert O.rel_l2(m.dn_state(0), om.dn_s[0]) <= 1e-3
     k, v = m.kv(3, 11)
