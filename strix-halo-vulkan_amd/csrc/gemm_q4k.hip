@@ -1,24 +1,23 @@
-// Q4_K dequant-fused GEMM for passes of 2..16 rows: Y[t] = W * pro(X[t]) (+ residual[t]) on the
+// Q4_K dequant-fused GEMM for passes of several rows: Y[t] = W * pro(X[t]) (+ residual[t]) on the
 // matrix cores, with the GEMV's arguments and results (verification passes, batched decode rows,
 // prompt chunks: llm/graph.go:1383-1429,1527-1666; the reference's form is llm_gemv.comp's
 // multi-row arm).
 //
 // Still HBM-bound on the weights, which are read once for all rows of the pass.  A 64-lane wave
-// multiplies a tile of 16 weight rows by up to 16 activation rows with v_mfma_f32_16x16x16_f16:
+// owns a tile of 16 weight rows and walks along them one 256-column super-block at a time,
+// multiplying by up to 16 activation rows with v_mfma_f32_16x16x16_f16:
 //   A (tokens x k)  the activations, split into two halves hi + lo (lo = x - hi) so that the
-//                   product keeps float32 accuracy; a wave keeps the fragments of its 256 columns
-//                   in registers for the whole kernel
+//                   product keeps float32 accuracy.  The block stages them once into LDS, already
+//                   in fragment order, and every wave reads them from there
 //   B (k x rows)    the 4-bit levels as exact halves 64+n (a level sits in mantissa bits 4..7 of
 //                   64.0); lane (row = lane%16, kb = lane/16) reads 8 payload bytes of each
 //                   64-weight group, whose low nibbles feed the group's first 32 columns and whose
 //                   high nibbles feed the other 32
 //   C (tokens x rows) one 32-column sub-block at a time, because each has its own scale and min;
 //                   the lane that loaded row n also holds C[.][n], so d*sc and dmin*m apply without
-//                   any exchange:  y += d*sc*(acc - 64*sum(x)) - dmin*m*sum(x).
-// The waves of a block share a row tile, each over its own super-block column, and add their tiles
-// through LDS.  Activation rows are staged four at a time through LDS, where the prologue runs.
-// A block covers up to 2048 columns at a time; a wider matrix is taken as column ranges one after
-// the other, each adding to what the one before left in y.
+//                   any exchange:  y += d*sc*acc - (64*d*sc + dmin*m)*sum(x).
+// Waves do not talk to one another while they stream, except that a matrix with few rows is also
+// split along its columns (KS waves a tile), whose partial tiles meet in LDS at the end.
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
 
@@ -30,16 +29,11 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kTileRows = 16;
-constexpr int kMaxRows = 16;   // activation rows one launch covers
-constexpr int kStage = 4;      // activation rows staged together
-constexpr int kSlice = 256;    // columns per wave: one super-block of each row
-constexpr int kSubs = kSlice / 32;
+constexpr int kDepth = 2;  // super-blocks of a tile requested ahead
 
-__host__ __device__ constexpr int xs_stride(int k) { return k + 8; }
-
-// One wave's loads for one row tile: the 16-byte header of the lane's row in the wave's
-// super-block column and 8 payload bytes of each of its four 64-weight groups.
-struct TileLoads {
+// One wave's loads for one super-block of its row tile: the 16-byte header of the lane's row and
+// 8 payload bytes of each of its four 64-weight groups.
+struct SbLoads {
     uint4 hdr;
     uint2 q[4];
     __device__ __forceinline__ void load(const char *sb, int kb) {
@@ -58,303 +52,286 @@ __device__ __forceinline__ half4_t levels(uint32_t even, uint32_t odd) {
     return __builtin_bit_cast(half4_t, v);
 }
 
-// K here is the width of the column range one launch covers (a.k, or a part of it).
-template <int K>
-struct Gemm {
-    static constexpr int NW = K / kSlice;
-    static constexpr int NTHR = NW * 64;
-    static constexpr int PER = 4;  // columns a thread stages per row: K / NTHR
-    static constexpr int XS = xs_stride(K);
-    static constexpr size_t lds_bytes() { return (static_cast<size_t>(kStage) * XS + K / 32 * 16 + NW * 256 + kStage * NW) * sizeof(float); }
+// LDS: the activation fragments, the per-sub-block sums of x, scratch for the staging's reductions
+// and for the column-split tiles.  TT is the pass's row capacity (4, 8 or 16).
+template <int TT>
+struct Lds {
+    // fragment (sub-block s, chunk c, part p) is 4*TT entries of 8 bytes: entry kb*TT + token
+    static __host__ __device__ constexpr size_t frag_bytes(int k) { return static_cast<size_t>(k / 32) * 4 * (4 * TT * 8); }
+    static __host__ __device__ constexpr size_t sx_bytes(int k) { return static_cast<size_t>(k / 32) * TT * 4; }
+    static __host__ __device__ constexpr size_t total(int k, int waves) {
+        return frag_bytes(k) + sx_bytes(k) + static_cast<size_t>(waves) * 64 * 16 /* tiles or reductions */ + TT * 8;
+    }
 };
 
-// Columns col0..col0+K of pro(x[t]) for gn <= 4 consecutive rows t_first.. into LDS rows of xs, by
-// all threads of the block; same prologues as the GEMV.  Every row's loads are issued before any
-// is used, so the rows cost one memory round trip together.  The RMSNorm needs the whole row and
-// runs only when the column range is the whole row.
-template <int K>
-__device__ __forceinline__ void stage_rows(const shv_gemv_q4k_args &a, int t_first, int gn, int col0, float *xs, float *red, int tid) {
-    using G = Gemm<K>;
-    const int lane = tid & 63, wave = tid >> 6;
-    // the gated norm reduces over a head, so its threads own consecutive columns; the others
-    // take columns NTHR apart, which coalesces better
-    const bool consec = a.prologue == SHV_PRO_GATED_NORM;
-    int col[G::PER];
-#pragma unroll
-    for (int i = 0; i < G::PER; i++) col[i] = consec ? tid * G::PER + i : tid + i * G::NTHR;
-    float v[kStage][G::PER], zv[kStage][G::PER];
+// Stage pro(x) of rows t0..t0+nt into fragment order.  A thread takes quads of four consecutive
+// columns of one row; quad q of the pass is row q / (K/4), columns 4*(q % (K/4)).., so a wave's quads
+// lie in one row and a 32-column sub-block is eight neighbouring lanes.
+template <int TT, int NTHR, int MAXQ>
+__device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt, char *frags, float *sxs, float *red) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.k, qpr = K / 4;              // quads per row
+    const int n_quads = nt * qpr;
+    float4 v[MAXQ], zv[MAXQ];  // MAXQ quads a thread at most: the launcher sizes the pass to fit
     const bool has_z = a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID;
-    // every row's gate pointer first: the positions they depend on are then fetched together
-    const float *zp[kStage];
+    const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
 #pragma unroll
-    for (int r = 0; r < kStage; r++) {
-        const int t = t_first + (r < gn ? r : 0);
-        zp[r] = a.z + static_cast<size_t>(t) * a.z_stride;
-        if (has_z && a.z_ring) {
-            const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
-            const int s = t / sl, k = t % sl;
-            const int p = a.pos ? a.pos[s] : 0;
-            const int slot = a.slot ? a.slot[s] : s;
-            zp[r] = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < kStage; r++) {
-        if (r >= gn) continue;
-        const float *x = a.x + static_cast<size_t>(t_first + r) * a.x_stride + col0;
-#pragma unroll
-        for (int i = 0; i < G::PER; i++) v[r][i] = x[col[i]];
+    for (int i = 0; i < MAXQ; i++) {
+        const int q = tid + i * NTHR;
+        if (q >= n_quads) continue;
+        const int t = t0 + q / qpr, c = 4 * (q % qpr);
+        v[i] = *reinterpret_cast<const float4 *>(a.x + static_cast<size_t>(t) * a.x_stride + c);
         if (has_z) {
-#pragma unroll
-            for (int i = 0; i < G::PER; i++) {
-                const int cg = col0 + col[i];
-                // sigmoid gate with head_dim: z rows are [q | gate] per head and the gate half is wanted
-                const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0
-                                   ? (cg / a.head_dim) * 2 * a.head_dim + a.head_dim + cg % a.head_dim : cg;
-                zv[r][i] = zp[r][zi];
+            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+            if (a.z_ring) {
+                const int s = t / sl, k = t % sl;
+                const int p = a.pos ? a.pos[s] : 0;
+                const int slot = a.slot ? a.slot[s] : s;
+                z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
             }
+            // sigmoid gate with head_dim: z rows are [q | gate] per head and the gate half is wanted
+            const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0 ? (c / a.head_dim) * 2 * a.head_dim + a.head_dim + c % a.head_dim : c;
+            zv[i] = *reinterpret_cast<const float4 *>(z + zi);
         }
     }
     if (a.prologue == SHV_PRO_RMSNORM) {
+        // all 64 quads of a wave lie in one row (K/4 is a multiple of 64): red[row][piece] takes
+        // the sum of squares of each 256-column piece, added up below in a fixed order
 #pragma unroll
-        for (int r = 0; r < kStage; r++) {
-            float ss = 0.f;
-#pragma unroll
-            for (int i = 0; i < G::PER; i++) ss = r < gn ? fmaf(v[r][i], v[r][i], ss) : ss;
+        for (int i = 0; i < MAXQ; i++) {
+            const int q = tid + i * NTHR;
+            float ss = q < n_quads ? fmaf(v[i].x, v[i].x, fmaf(v[i].y, v[i].y, fmaf(v[i].z, v[i].z, v[i].w * v[i].w))) : 0.f;
             ss = wave_sum_all(ss);
-            if (lane == 0) red[r * G::NW + wave] = ss;
+            const int q0 = wave * 64 + i * NTHR;
+            if (lane == 0 && q0 < n_quads) red[(q0 / qpr) * 16 + (q0 % qpr) / 64] = ss;
         }
         __syncthreads();
-#pragma unroll
-        for (int r = 0; r < kStage; r++) {
-            if (r >= gn) continue;
+        if (tid < nt) {
             float tot = 0.f;
-#pragma unroll
-            for (int w = 0; w < G::NW; w++) tot += red[r * G::NW + w];
-            const float scale = 1.f / sqrtf(tot / static_cast<float>(K) + a.eps);
-#pragma unroll
-            for (int i = 0; i < G::PER; i++) xs[r * G::XS + col[i]] = v[r][i] * scale * a.gamma[col[i]];
+            for (int pc = 0; pc < qpr / 64; pc++) tot += red[tid * 16 + pc];
+            red[TT * 16 + tid] = 1.f / sqrtf(tot / static_cast<float>(K) + a.eps);
         }
-    } else if (a.prologue == SHV_PRO_GATED_NORM) {
-        const int span = a.head_dim / G::PER;  // lanes a head spans
+        __syncthreads();
+    }
 #pragma unroll
-        for (int r = 0; r < kStage; r++) {
-            if (r >= gn) continue;
-            float ss = 0.f;
-#pragma unroll
-            for (int i = 0; i < G::PER; i++) ss = fmaf(v[r][i], v[r][i], ss);
+    for (int i = 0; i < MAXQ; i++) {
+        const int q = tid + i * NTHR;
+        const bool on = q < n_quads;
+        const int tl = on ? q / qpr : 0, c = on ? 4 * (q % qpr) : 0;
+        float x[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+        if (a.prologue == SHV_PRO_RMSNORM) {
+            const float scale = red[TT * 16 + tl];
+            const float4 g = *reinterpret_cast<const float4 *>(a.gamma + c);
+            x[0] *= scale * g.x; x[1] *= scale * g.y; x[2] *= scale * g.z; x[3] *= scale * g.w;
+        } else if (a.prologue == SHV_PRO_GATED_NORM) {
+            float ss = on ? fmaf(x[0], x[0], fmaf(x[1], x[1], fmaf(x[2], x[2], x[3] * x[3]))) : 0.f;
+            const int span = a.head_dim / 4;  // lanes a head spans
             for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
             const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
+            const float zz[4] = {zv[i].x, zv[i].y, zv[i].z, zv[i].w};
 #pragma unroll
-            for (int i = 0; i < G::PER; i++) {
-                const float g = 1.f / (1.f + expf(-zv[r][i]));
-                xs[r * G::XS + col[i]] = v[r][i] * scale * a.gamma[(col0 + col[i]) % a.head_dim] * g;
-            }
+            for (int j = 0; j < 4; j++) x[j] = x[j] * scale * a.gamma[(c + j) % a.head_dim] * (1.f / (1.f + expf(-zz[j])));
+        } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
+            const float zz[4] = {zv[i].x, zv[i].y, zv[i].z, zv[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) x[j] *= 1.f / (1.f + expf(-zz[j]));
         }
-    } else {
+        // the sub-block's sum of x: eight neighbouring lanes
+        float sum = on ? (x[0] + x[1]) + (x[2] + x[3]) : 0.f;
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        sum += __shfl_xor(sum, 4, 64);
+        if (on) {
+            const int sub = c >> 5, kb = (c & 31) >> 3, chunk = (c & 7) >> 2;
+            if ((c & 31) == 0) sxs[sub * TT + tl] = sum;
+            // k order of levels(): [x0, x2, x1, x3]
+            const float o[4] = {x[0], x[2], x[1], x[3]};
+            half4_t h, l;
 #pragma unroll
-        for (int r = 0; r < kStage; r++) {
-            if (r >= gn) continue;
-#pragma unroll
-            for (int i = 0; i < G::PER; i++) {
-                const float g = a.prologue == SHV_PRO_MUL_SIGMOID ? 1.f / (1.f + expf(-zv[r][i])) : 1.f;
-                xs[r * G::XS + col[i]] = v[r][i] * g;
+            for (int j = 0; j < 4; j++) {
+                const _Float16 hi = static_cast<_Float16>(o[j]);
+                h[j] = hi;
+                l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
             }
+            char *e = frags + (static_cast<size_t>((sub * 2 + chunk) * 2) * (4 * TT) + kb * TT + tl) * 8;
+            *reinterpret_cast<half4_t *>(e) = h;
+            *reinterpret_cast<half4_t *>(e + 4 * TT * 8) = l;
         }
     }
 }
 
-// grid: blocks take row tiles round-robin.  t0: first activation row of this launch, nt: how many.
-// A matrix wider than K runs as n_ranges column ranges one after the other; from the second on a
-// thread adds to the outputs it stored itself in the range before.
-template <int K>
-__global__ __launch_bounds__(Gemm<K>::NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int t0, int nt, int n_tiles, int n_ranges) {
-    using G = Gemm<K>;
-    extern __shared__ float smem[];
-    float *xs = smem;                             // [kStage][XS]
-    float *sxs = xs + kStage * G::XS;             // [K/32][16] sum of x per 32-column sub-block and row
-    float *tile = sxs + K / 32 * 16;              // [NW][256] the waves' partial tiles
-    float *red = tile + G::NW * 256;              // [kStage][NW]
+// grid: blocks of NTHR/64 waves.  KS consecutive waves share a row tile, each over 1/KS of the
+// columns.  t0: first activation row of this launch, nt: how many (<= TT).
+template <int TT, int NTHR, int MAXQ>
+__global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int t0, int nt, int n_tiles, int ks) {
+    extern __shared__ __align__(16) char smem[];
+    constexpr int NW = NTHR / 64;
+    char *frags = smem;
+    float *sxs = reinterpret_cast<float *>(smem + Lds<TT>::frag_bytes(a.k));
+    float *ytile = sxs + a.k / 32 * TT;                         // [NW][64] float4, also the staging's reductions
+    size_t *yoffs = reinterpret_cast<size_t *>(ytile + NW * 64 * 4);  // [TT]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n = lane & 15, kb = lane >> 4;      // B: weight row of the tile, k block; A: token n
-    const size_t row_bytes = static_cast<size_t>(a.k / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
+    const int n = lane & 15, kb = lane >> 4;  // B: weight row of the tile, k block; C: row n, tokens 4kb..4kb+3
+    const int sbs = a.k / SHV_Q4K_BLOCK;      // super-blocks a row
+    const size_t row_bytes = static_cast<size_t>(sbs) * SHV_Q4K_BYTES;
+    const int steps = sbs / ks, part = wave % ks;
+    const int tiles_per_block = NW / ks;
+    const char *wbase = static_cast<const char *>(a.w) + static_cast<size_t>(part * steps) * SHV_Q4K_BYTES;
+
+    // the first tile's first super-blocks do not depend on the activations
+    int tl = blockIdx.x * tiles_per_block + wave / ks;
+    SbLoads ld[kDepth];
+    {
+        const int r = tl * kTileRows + n;
+        const char *rp = wbase + static_cast<size_t>(r < a.n ? r : a.n - 1) * row_bytes;
+#pragma unroll
+        for (int d = 0; d < kDepth; d++)
+            if (d < steps && tl < n_tiles) ld[d].load(rp + d * SHV_Q4K_BYTES, kb);
+    }
 
     // where each activation row's outputs go (the DeltaNet projection ring, or plain rows)
-    const int o_tok = tid >> 4;  // the activation row of the output this thread adds up and stores, when tid < 256
-    size_t y_off = 0;
-    if (o_tok < nt) {
-        const int t = t0 + o_tok;
+    if (tid < nt) {
+        const int t = t0 + tid;
+        size_t off;
         if (a.ring_slots > 0 && !a.z_ring) {
             const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
             const int s = t / sl, i = t % sl;
             const int p = a.pos ? a.pos[s] : 0;
             const int slot = a.slot ? a.slot[s] : s;
-            y_off = (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
+            off = (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
         } else {
-            y_off = static_cast<size_t>(t) * a.y_stride;
+            off = static_cast<size_t>(t) * a.y_stride;
         }
+        yoffs[tid] = off;
     }
+    stage<TT, NTHR, MAXQ>(a, t0, nt, frags, sxs, ytile);
+    __syncthreads();
+
     const NibbleConsts nc = nibble_consts();
-    const float4 *sx4 = reinterpret_cast<const float4 *>(sxs) + wave * kSubs * 4 + kb;  // rows 4kb..4kb+3 of C
-
-    for (int rg = 0; rg < n_ranges; rg++) {
-    const int col0 = rg * K;
-    const float *residual = rg == 0 ? a.residual : a.y;
-    const char *wslice = static_cast<const char *>(a.w) + static_cast<size_t>(col0 / SHV_Q4K_BLOCK + wave) * SHV_Q4K_BYTES;
-
-    // the first tile's weights do not depend on the activations
-    TileLoads cur, nxt;
-    int tl = blockIdx.x;
-    {
+    // this lane's fragment entry and its four tokens' sums; rows beyond the capacity alias real ones
+    const char *my_frag = frags + (kb * TT + (n & (TT - 1))) * 8;
+    const float *my_sx = sxs + ((4 * kb) & (TT - 1));
+    constexpr int FRAG = 4 * TT * 8;  // bytes of one (sub-block, chunk, part) fragment
+    const int stride = gridDim.x * tiles_per_block;
+    const int iters = (n_tiles + stride - 1) / stride;
+    for (int it = 0; it < iters; it++, tl += stride) {
+        const bool live = tl < n_tiles;
         const int r = tl * kTileRows + n;
-        cur.load(wslice + static_cast<size_t>(r < a.n ? r : a.n - 1) * row_bytes, kb);
-    }
-
-    // ---- activations: this lane's token is n; its fragments cover the wave's 256 columns ----
-    half4_t xh[kSubs][2], xl[kSubs][2];
-#pragma unroll
-    for (int s = 0; s < kSubs; s++)
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            xh[s][c] = half4_t{0, 0, 0, 0};
-            xl[s][c] = half4_t{0, 0, 0, 0};
-        }
-    for (int g0 = 0; g0 < nt; g0 += kStage) {
-        const int gn = nt - g0 < kStage ? nt - g0 : kStage;
-        stage_rows<K>(a, t0 + g0, gn, col0, xs, red, tid);
-        __syncthreads();
-        if (n >= g0 && n < g0 + gn) {
-            const float *row = xs + (n - g0) * G::XS + wave * kSlice;
-#pragma unroll
-            for (int s = 0; s < kSubs; s++) {
-                // sub-block s of the slice: 64-weight group s/2, low (s even) or high nibbles
-                float sum = 0.f;
-#pragma unroll
-                for (int c = 0; c < 2; c++) {
-                    const float4 f = *reinterpret_cast<const float4 *>(row + s * 32 + kb * 8 + c * 4);
-                    const float v[4] = {f.x, f.z, f.y, f.w};  // the k order of levels()
-                    half4_t h, l;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const _Float16 hi = static_cast<_Float16>(v[j]);
-                        h[j] = hi;
-                        l[j] = static_cast<_Float16>(v[j] - static_cast<float>(hi));
-                    }
-                    xh[s][c] = h;
-                    xl[s][c] = l;
-                    sum += (f.x + f.y) + (f.z + f.w);
-                }
-                sum += __shfl_xor(sum, 16, 64);
-                sum += __shfl_xor(sum, 32, 64);
-                if (kb == 0) sxs[(wave * kSubs + s) * 16 + n] = sum;
-                __builtin_amdgcn_sched_barrier(0);  // one sub-block at a time: keeps the live set small
-            }
-        }
-        __syncthreads();
-    }
-    // rows of the pass beyond nt contribute nothing; their sums are never read
-
-    for (; tl < n_tiles; tl += gridDim.x) {
-        const int tn = tl + gridDim.x;
-        if (tn < n_tiles) {
-            const int r = tn * kTileRows + n;
-            nxt.load(wslice + static_cast<size_t>(r < a.n ? r : a.n - 1) * row_bytes, kb);
-        }
+        const char *rp = wbase + static_cast<size_t>(r < a.n ? r : a.n - 1) * row_bytes;
         float4_t y = {0.f, 0.f, 0.f, 0.f};
-        const float d = f16_bits_to_f32(cur.hdr.x), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+        if (live) {
+            // super-block j of a tile sits in slot j % depth; steps is a power of two, so is depth
+            const int depth = steps < kDepth ? steps : kDepth;
+            for (int st = 0; st < steps; st += depth) {
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            uint32_t sc, mn;
-            q4k_group_scale_min(cur.hdr, g, sc, mn);
-            const uint32_t q0 = cur.q[g].x, q1 = cur.q[g].y;
-#pragma unroll
-            for (int hi = 0; hi < 2; hi++) {
-                const int sub = g * 2 + hi;
-                half4_t b0, b1;
-                if (hi == 0) {
-                    b0 = levels(((q0 << 4) & nc.mask) | nc.one, ((q0 >> 4) & nc.mask) | nc.one);
-                    b1 = levels(((q1 << 4) & nc.mask) | nc.one, ((q1 >> 4) & nc.mask) | nc.one);
-                } else {
-                    b0 = levels((q0 & nc.mask) | nc.one, ((q0 >> 8) & nc.mask) | nc.one);
-                    b1 = levels((q1 & nc.mask) | nc.one, ((q1 >> 8) & nc.mask) | nc.one);
-                }
-                float4_t acc = {0.f, 0.f, 0.f, 0.f};
-                acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xh[sub][0], b0, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xh[sub][1], b1, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xl[sub][0], b0, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xl[sub][1], b1, acc, 0, 0, 0);
-                const float ds = d * static_cast<float>(hi ? sc >> 8 : sc & 0xFFu);
-                const float dm = dmin * static_cast<float>(hi ? mn >> 8 : mn & 0xFFu);
-                const float4 sx = sx4[sub * 4];
-                const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
-#pragma unroll
-                for (int j = 0; j < 4; j++) y[j] += ds * fmaf(-64.f, sxv[j], acc[j]) - dm * sxv[j];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // ---- add the waves' tiles and store: lane holds C[4kb+j][n] ----
-        float *mine = tile + wave * 256;
-#pragma unroll
-        for (int j = 0; j < 4; j++) mine[(4 * kb + j) * 16 + n] = y[j];
-        __syncthreads();
-        for (int o = tid; o < 256; o += G::NTHR) {
-            const int orow = o & 15, otok = o >> 4;
-            float v = 0.f;
-#pragma unroll
-            for (int w = 0; w < G::NW; w++) v += tile[w * 256 + o];
-            const int r = tl * kTileRows + orow;
-            if (otok < nt && r < a.n) {
-                // NTHR >= 256: o == tid and y_off is this thread's; smaller blocks recompute it
-                size_t off = y_off;
-                if (G::NTHR < 256) {
-                    const int t = t0 + otok;
-                    if (a.ring_slots > 0 && !a.z_ring) {
-                        const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
-                        const int s = t / sl, i = t % sl;
-                        const int p = a.pos ? a.pos[s] : 0;
-                        const int slot = a.slot ? a.slot[s] : s;
-                        off = (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
+                for (int d = 0; d < kDepth; d++) {
+                    if (d >= depth) break;
+                    const SbLoads cur = ld[d];
+                    // the same slot's next super-block, or the next tile's first ones
+                    if (st + d + depth < steps) {
+                        ld[d].load(rp + (st + d + depth) * SHV_Q4K_BYTES, kb);
                     } else {
-                        off = static_cast<size_t>(t) * a.y_stride;
+                        const int tn = tl + stride;
+                        const int dn = st + d + depth - steps;
+                        if (tn < n_tiles) {
+                            const int rn = tn * kTileRows + n;
+                            ld[d].load(wbase + static_cast<size_t>(rn < a.n ? rn : a.n - 1) * row_bytes + dn * SHV_Q4K_BYTES, kb);
+                        }
+                    }
+                    const int sb = part * steps + st + d;
+                    const float dd = f16_bits_to_f32(cur.hdr.x), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        uint32_t sc, mn;
+                        q4k_group_scale_min(cur.hdr, g, sc, mn);
+                        const uint32_t q0 = cur.q[g].x, q1 = cur.q[g].y;
+#pragma unroll
+                        for (int hi = 0; hi < 2; hi++) {
+                            const int sub = sb * 8 + g * 2 + hi;
+                            half4_t b0, b1;
+                            if (hi == 0) {
+                                b0 = levels(((q0 << 4) & nc.mask) | nc.one, ((q0 >> 4) & nc.mask) | nc.one);
+                                b1 = levels(((q1 << 4) & nc.mask) | nc.one, ((q1 >> 4) & nc.mask) | nc.one);
+                            } else {
+                                b0 = levels((q0 & nc.mask) | nc.one, ((q0 >> 8) & nc.mask) | nc.one);
+                                b1 = levels((q1 & nc.mask) | nc.one, ((q1 >> 8) & nc.mask) | nc.one);
+                            }
+                            const char *f = my_frag + static_cast<size_t>(sub) * 4 * FRAG;
+                            const half4_t xh0 = *reinterpret_cast<const half4_t *>(f);
+                            const half4_t xl0 = *reinterpret_cast<const half4_t *>(f + FRAG);
+                            const half4_t xh1 = *reinterpret_cast<const half4_t *>(f + 2 * FRAG);
+                            const half4_t xl1 = *reinterpret_cast<const half4_t *>(f + 3 * FRAG);
+                            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+                            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xh0, b0, acc, 0, 0, 0);
+                            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xh1, b1, acc, 0, 0, 0);
+                            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xl0, b0, acc, 0, 0, 0);
+                            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(xl1, b1, acc, 0, 0, 0);
+                            const float ds = dd * static_cast<float>(hi ? sc >> 8 : sc & 0xFFu);
+                            const float e = fmaf(64.f, ds, dmin * static_cast<float>(hi ? mn >> 8 : mn & 0xFFu));
+                            const float4 sx = *reinterpret_cast<const float4 *>(my_sx + sub * TT);
+                            const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
+#pragma unroll
+                            for (int j = 0; j < 4; j++) y[j] = fmaf(-e, sxv[j], fmaf(ds, acc[j], y[j]));
+                        }
                     }
                 }
-                if (residual) v += residual[static_cast<size_t>(t0 + otok) * a.y_stride + r];
-                a.y[off + r] = v;
             }
         }
-        __syncthreads();
-        cur = nxt;
+        // ---- the column parts of a tile meet in LDS; then C[4kb+j][n] goes out ----
+        if (ks > 1) {
+            *reinterpret_cast<float4_t *>(ytile + (wave * 64 + lane) * 4) = y;
+            __syncthreads();
+            if (part == 0) {
+                for (int p = 1; p < ks; p++) {
+                    const float4_t o = *reinterpret_cast<const float4_t *>(ytile + ((wave + p) * 64 + lane) * 4);
+                    y += o;
+                }
+            }
+        }
+        if (live && part == 0 && r < a.n) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int tok = 4 * kb + j;
+                if (tok < nt) {
+                    float v = y[j];
+                    if (a.residual) v += a.residual[static_cast<size_t>(t0 + tok) * a.y_stride + r];
+                    a.y[yoffs[tok] + r] = v;
+                }
+            }
+        }
+        if (ks > 1) __syncthreads();
     }
-    }  // column ranges
 }
 
-template <int K>
-int launch_gemm(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
-    using G = Gemm<K>;
+template <int TT, int NTHR, int MAXQ>
+int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt) {
+    constexpr int NW = NTHR / 64;
+    SHV_REQUIRE(nt * (a.k / 4) <= MAXQ * NTHR, "gemm_q4k: %d rows of %d columns are more than one block stages", nt, a.k);
     const int n_tiles = (a.n + kTileRows - 1) / kTileRows;
-    const size_t lds = G::lds_bytes();
-    static bool raised = false;
-    if (lds > 48 * 1024 && !raised) {
-        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_kernel<K>),
+    const size_t lds = Lds<TT>::total(a.k, NW);
+    static size_t raised = 0;
+    if (lds > 48 * 1024 && lds > raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_kernel<TT, NTHR, MAXQ>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = true;
+        raised = lds;
     }
-    // one round of resident blocks, so that the activations are staged once per block; the tiles
-    // are dealt evenly among them
-    static int per_cu = 0;
-    if (per_cu == 0) {
-        SHV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(&gemm_q4k_kernel<K>), G::NTHR, lds));
-        if (per_cu < 1) per_cu = 1;
-    }
+    int per_cu = 0;
+    SHV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(&gemm_q4k_kernel<TT, NTHR, MAXQ>), NTHR, lds));
+    SHV_REQUIRE(per_cu >= 1, "gemm_q4k: a block of %d threads with %zu bytes of LDS does not fit a compute unit", NTHR, lds);
+    // One round of resident blocks, so that the activations are staged once per block.  A matrix
+    // with too few row tiles to occupy the waves is also split along its columns.
+    const int slots = ctx->prop.multiProcessorCount * per_cu * NW;
+    const int sbs = a.k / SHV_Q4K_BLOCK;
+    int ks = 1;
+    while (ks < 4 && ks * 2 <= NW && sbs % (ks * 2) == 0 && n_tiles * ks * 2 <= slots) ks *= 2;
+    const int tiles_per_block = NW / ks;
     int blocks = ctx->prop.multiProcessorCount * per_cu;
-    if (blocks > n_tiles) blocks = n_tiles;
-    const int rounds = (n_tiles + blocks - 1) / blocks;
-    blocks = (n_tiles + rounds - 1) / rounds;
-    for (int t0 = 0; t0 < a.n_tok; t0 += kMaxRows) {
-        const int nt = a.n_tok - t0 < kMaxRows ? a.n_tok - t0 : kMaxRows;
-        SHV_LAUNCH(ctx, (gemm_q4k_kernel<K>), dim3(blocks), dim3(G::NTHR), lds, a, t0, nt, n_tiles, a.k / K);
-    }
+    const int need = (n_tiles + tiles_per_block - 1) / tiles_per_block;
+    if (blocks > need) blocks = need;
+    const int rounds = (need + blocks - 1) / blocks;
+    blocks = (need + rounds - 1) / rounds;
+    SHV_LAUNCH(ctx, (gemm_q4k_kernel<TT, NTHR, MAXQ>), dim3(blocks), dim3(NTHR), lds, a, t0, nt, n_tiles, ks);
     return SHV_OK;
 }
 
@@ -365,23 +342,30 @@ int launch_gemm(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
 bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a) {
     if (a.k != 256 && a.k != 512 && a.k != 1024 && a.k != 2048 && a.k != 4096) return false;
     if (a.prologue == SHV_PRO_RMSNORM_PAIR) return false;
-    if (a.k > 2048) {
-        // column ranges: no whole-row statistic, and plain rows to add into
-        if (a.prologue == SHV_PRO_RMSNORM || (a.ring_slots > 0 && !a.z_ring) || a.y_stride < a.n) return false;
-    }
     if (a.prologue == SHV_PRO_GATED_NORM) {
         const int span = a.head_dim / 4;
-        if (a.head_dim % 4 != 0 || span < 1 || span > 64 || (span & (span - 1)) != 0 || 2048 % a.head_dim != 0) return false;
+        if (a.head_dim % 4 != 0 || span < 1 || span > 64 || (span & (span - 1)) != 0) return false;
     }
-    // 8-byte loads of the payload and 16-byte loads of the staged rows
-    return a.x_stride % 4 == 0 && shv_aligned16(a.x);
+    if (a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim % 4 != 0) return false;
+    // 16-byte loads of the activation rows, their gates and the norm's gamma
+    if (a.x_stride % 4 != 0 || !shv_aligned16(a.x)) return false;
+    if (a.prologue == SHV_PRO_RMSNORM && !shv_aligned16(a.gamma)) return false;
+    if ((a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID) &&
+        (!shv_aligned16(a.z) || a.z_stride % 4 != 0 || (a.z_ring && a.ring_stride % 4 != 0)))
+        return false;
+    return true;
 }
 
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
-    switch (a.k) {
-        case 256: return launch_gemm<256>(ctx, a);
-        case 512: return launch_gemm<512>(ctx, a);
-        case 1024: return launch_gemm<1024>(ctx, a);
-        default: return launch_gemm<2048>(ctx, a);  // 2048, and 4096 as two column ranges
+    // the fragments of 16 rows of 4096 columns do not fit LDS: such a pass goes 8 rows at a time
+    const int cap = a.k > 2048 ? 8 : 16;
+    for (int t0 = 0; t0 < a.n_tok; t0 += cap) {
+        const int nt = a.n_tok - t0 < cap ? a.n_tok - t0 : cap;
+        int rc;
+        if (nt <= 4) rc = launch_tt<4, 512, 8>(ctx, a, t0, nt);
+        else if (nt <= 8) rc = launch_tt<8, 512, 16>(ctx, a, t0, nt);
+        else rc = launch_tt<16, 1024, 8>(ctx, a, t0, nt);
+        if (rc != SHV_OK) return rc;
     }
+    return SHV_OK;
 }

@@ -197,7 +197,8 @@ void Model::InitSynthetic(uint64_t seed) {
 MoEGPU::MoEGPU(Device &dev, const Model &m, int maxTokens) : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens) {
     if (maxTokens < 1) throw Error("llm: MoEGPU needs room for at least one token");
     if (c_.NExpertUsed > c_.NExpert) throw Error("llm: MoEGPU: more experts used than there are");
-    if (const char *e = std::getenv("LLM_MOE_ROUTE")) fused_route_ = std::strcmp(e, "kernel") != 0;
+    // the selection as a dispatch of its own measures the same at one row and better at several
+    if (const char *e = std::getenv("LLM_MOE_ROUTE")) fused_route_ = std::strcmp(e, "fused") == 0;
     const size_t T = maxTokens;
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));

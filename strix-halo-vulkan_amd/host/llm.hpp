@@ -174,7 +174,7 @@ private:
     float *in_, *out_, *xn_, *logits_, *weights_, *act_;
     int32_t *topk_;
     uint64_t act_bytes_ = 0;
-    bool fused_route_ = true;
+    bool fused_route_ = false;
 };
 
 // llm.DeltaNetGPU (llm/gpu_deltanet.go:207-322, NewDeltaNetGPUBank :421)
