@@ -262,7 +262,8 @@ typedef struct {
  * cache, then causal GQA softmax attention of the row over cells 0..p, split n_splits ways over
  * the cells and merged.  out is [rows][n_head*d] BEFORE the sigmoid gate, which the output
  * projection applies as its prologue.  kcache / vcache are [n_slots][max_cells][n_head_kv][d]
- * binary16; partial is scratch of n_seq*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2) floats. */
+ * binary16; partial is scratch of n_seq*min(seq_len,2)*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2)
+ * floats (the rows of a sequence are taken two at a time over one pass of the cache). */
 typedef struct {
     const float *qkv;
     const float *q_norm;

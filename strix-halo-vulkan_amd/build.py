@@ -50,7 +50,8 @@ def _compile(src, force):
     obj = os.path.join(OBJ, src[:-4] + ".o")
     path = os.path.join(CSRC, src)
     if force or _stale(obj, [path] + headers()):
-        cmd = [HIPCC] + COMMON + PER_FILE.get(src, []) + ["-c", path, "-o", obj]
+        # SHV_EXTRA_HIPCC_FLAGS: extra compiler flags for an experiment (e.g. a -D switch)
+        cmd = [HIPCC] + COMMON + PER_FILE.get(src, []) + os.environ.get("SHV_EXTRA_HIPCC_FLAGS", "").split() + ["-c", path, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("hipcc failed on %s:\n%s\n%s" % (src, " ".join(cmd), r.stderr))

@@ -1,16 +1,19 @@
-// Gated full-attention decode over an fp16 KV cache, GQA with 8 query heads per KV head.
+// Gated full-attention decode over an fp16 KV cache, GQA with 8 query heads per KV head, one or
+// two consecutive rows of a sequence per launch.
 //
 // HBM-bound on the cache: a block owns one KV head and one slice of the cells and serves all the
-// query heads of that KV head from a single pass over K and a single pass over V.
-//   prologue  per-head RMS norm + rotary of the block's query heads into LDS; the block that owns
-//             the new cell also normalises/rotates K, rounds K and V to binary16 and appends them
-//   per chunk of 128 cells (flash-decoding with a running max):
-//     (a) the chunk's V rows are requested, (b) scores: 32 lanes per cell (16-byte loads of K),
-//     eight partial dots per lane reduced with a transposing butterfly so every lane ends with
-//     one head's score, (c) running max and exponentials per head in LDS, (d) P*V: 64 lanes
-//     across the 256 dims of a V row, eight heads' accumulators per lane
-//   epilogue  the block's (max, sum, accumulator) goes to scratch; the last block of the KV head
-//             to arrive merges the slices
+// query heads of that KV head, for both rows, from a single pass over K and a single pass over V.
+//   start     the wave's first K and V rows are requested before anything else
+//   prologue  per-head RMS norm + rotary of the block's query heads into LDS; the block whose slice
+//             holds a new cell also normalises/rotates K, rounds K and V to binary16 and appends them
+//   per chunk of 64 cells, every wave on its own 16 cells with no block-wide synchronisation:
+//     scores (32 lanes a cell, 16-byte loads of K, eight partial dots a lane reduced with a
+//     transposing butterfly), a running max and sum per (row, head) kept by the wave, P*V with 64
+//     lanes across the 256 dims of a V row
+//   epilogue  the four waves' (max, sum, accumulator) are merged through LDS and go to scratch
+// A second, small kernel merges the slices: one block a (row, head), one thread a dim, every
+// slice's value requested at once.  (Merging in the last block to arrive instead costs more than
+// the launch: that block walks all the records alone, a few dependent round trips to memory.)
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
 
@@ -21,9 +24,13 @@ using namespace shv;
 constexpr int kBlock = 256;
 constexpr int kD = 256;        // head dimension the kernel is built for
 constexpr int kRep = 8;        // query heads per KV head
-constexpr int kChunk = 128;    // cells scored together; also what a slice is given while slices are to spare
-constexpr int kMaxSplits = 512; // slices the merge has LDS for
-constexpr int kPlane = kMaxSplits * kRep;
+#ifndef SHV_ATTN_WAVE_CELLS
+#define SHV_ATTN_WAVE_CELLS 16
+#endif
+constexpr int kWaveCells = SHV_ATTN_WAVE_CELLS; // cells a wave scores together
+constexpr int kChunk = 4 * kWaveCells;
+constexpr int kMaxSplits = 512;
+constexpr int kRec = kRep * (kD + 2);  // floats of one (slice, row) record: per head d values, max, sum
 
 // v[8] per lane -> the sum over the 32 lanes of an aligned half-wave of v[head], where
 // head = bit4(li)*4 + bit3(li)*2 + bit2(li); every lane of the half-wave gets one head's total.
@@ -79,23 +86,28 @@ __device__ __forceinline__ void norm_rope_head(const float *src, const float *ga
     __builtin_amdgcn_wave_barrier();
 }
 
-// grid: (n_splits, n_head_kv, n_seq); row_i is the row of each sequence this launch handles.
-__global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_args a, int row_i, int32_t *counters) {
-    __shared__ __align__(16) float qh[kRep][kD];         // 8 KB: normalised, rotated queries
-    __shared__ __align__(16) float sc[kChunk][kRep];     // 4 KB: scores, then probabilities, of a chunk
-    __shared__ __align__(16) float big[4 * kRep * kD];   // 32 KB: cross-wave sums, then the merge's weights
-    __shared__ __align__(16) float kv_tmp[kD];
-    __shared__ float red[4][kRep];
-    __shared__ float mrun[kRep], lrun[kRep], alpha[kRep];
-    __shared__ float stat[2][kRep];
-    __shared__ int is_last;
+// LDS of one block, R rows a launch.
+template <int R>
+struct Smem {
+    float qh[R][kRep][kD];                    // normalised, rotated queries
+    float sc[4][R][kWaveCells][kRep];         // per wave: scores, then probabilities, of its cells
+    float al[4][R][kRep];                     // per wave: the factor the running sums shrink by
+    float big[4][kRep][kD];                   // the waves' accumulators of one row, to be merged
+    float wm[4][kRep], wl[4][kRep];           // the waves' running max and sum of one row
+    float kv_tmp[R][kD];
+};
+
+// grid: (n_splits, n_head_kv, n_seq); rows row0..row0+R-1 of each sequence.
+template <int R>
+__global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_args a, int row0) {
+    extern __shared__ __align__(16) char smem_raw[];
+    Smem<R> &sm = *reinterpret_cast<Smem<R> *>(smem_raw);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
     const int slot = a.slot ? a.slot[seq] : seq;
-    const int p = (a.pos ? a.pos[seq] : 0) + row_i;
-    const int row = seq * a.seq_len + row_i;
-    const int n_cells = p + 1;
+    const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the launch's first row
+    const int n_cells = p_first + R;                       // cells the last row sees
     // The grid is sized for the cache's capacity; how many of its slices take part depends on how
     // many cells the sequence holds now: about kChunk cells a slice while there are slices to
     // spare, so that a short context is not mostly merge and a long one covers the whole chip.
@@ -107,91 +119,122 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_arg
     const int c0 = split * cps;
     const int c1 = c0 + cps < n_cells ? c0 + cps : n_cells;
     const int nc = c1 > c0 ? c1 - c0 : 0;
-    const bool owner = p >= c0 && p < c1;
 
-    const float *qkv = a.qkv + static_cast<size_t>(row) * a.qkv_stride;
-    const float *rope_row = a.rope + static_cast<size_t>(p) * a.rope_dims;
     const int kvw = a.n_head_kv * kD;
     uint16_t *kc = static_cast<uint16_t *>(a.kcache) + static_cast<size_t>(slot) * a.max_cells * kvw + kvh * kD;
     uint16_t *vc = static_cast<uint16_t *>(a.vcache) + static_cast<size_t>(slot) * a.max_cells * kvw + kvh * kD;
+    const int li = lane & 31, cg = lane >> 5;
+
+    // ---- the wave's first K and V rows: cells c0 + 16*wave + .. ; only cells that existed before
+    //      this launch may be read this early ----
+    uint4 kq[kWaveCells / 2];
+    uint2 vq[kWaveCells];
+    auto load_k = [&](int ch0, bool old_only) {
+#pragma unroll
+        for (int u = 0; u < kWaveCells / 2; u++) {
+            const int c = c0 + ch0 + wave * kWaveCells + 2 * u + cg;
+            if (c < c1 && (!old_only || c < p_first))
+                kq[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c) * kvw + 8 * li);
+            else if (!old_only || c >= c1)
+                kq[u] = make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    auto load_v = [&](int ch0, bool old_only) {
+#pragma unroll
+        for (int u = 0; u < kWaveCells; u++) {
+            const int c = c0 + ch0 + wave * kWaveCells + u;
+            if (c < c1 && (!old_only || c < p_first))
+                vq[u] = *reinterpret_cast<const uint2 *>(vc + static_cast<size_t>(c) * kvw + 4 * lane);
+            else if (!old_only || c >= c1)
+                vq[u] = make_uint2(0u, 0u);
+        }
+    };
+    load_k(0, true);
+    load_v(0, true);
 
     // ---- prologue ----
-    if (nc > 0) {
+    const float *qkv0 = a.qkv + static_cast<size_t>(seq * a.seq_len + row0) * a.qkv_stride;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int hh = wave * 2 + i;
-            const int head = kvh * kRep + hh;
-            norm_rope_head(qkv + static_cast<size_t>(head) * 2 * kD, a.q_norm, rope_row, a.rope_dims, a.eps, qh[hh], lane);
+    for (int j = 0; j < R; j++) {
+        const float *qkv = qkv0 + static_cast<size_t>(j) * a.qkv_stride;
+        const int p = p_first + j;
+        const float *rope_row = a.rope + static_cast<size_t>(p) * a.rope_dims;
+        if (nc > 0) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int hh = wave * 2 + i;
+                norm_rope_head(qkv + static_cast<size_t>(kvh * kRep + hh) * 2 * kD, a.q_norm, rope_row, a.rope_dims, a.eps, sm.qh[j][hh], lane);
+            }
+        }
+        if (p >= c0 && p < c1) {
+            // the new cell of row j lies in this slice: waves 2j and 2j+1 (mod 4) append its K and V
+            if (wave == ((2 * j) & 3)) {
+                const float *ksrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD;
+                norm_rope_head(ksrc, a.k_norm, rope_row, a.rope_dims, a.eps, sm.kv_tmp[j], lane);
+                uint16_t *dst = kc + static_cast<size_t>(p) * kvw;
+#pragma unroll
+                for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(sm.kv_tmp[j][4 * lane + i]));
+            } else if (wave == ((2 * j + 1) & 3)) {
+                const float *vsrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvw + kvh * kD;
+                uint16_t *dst = vc + static_cast<size_t>(p) * kvw;
+#pragma unroll
+                for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(vsrc[4 * lane + i]));
+            }
         }
     }
-    if (owner) {
-        if (wave == 0) {
-            const float *ksrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD;
-            norm_rope_head(ksrc, a.k_norm, rope_row, a.rope_dims, a.eps, kv_tmp, lane);
-            uint16_t *dst = kc + static_cast<size_t>(p) * kvw;
-#pragma unroll
-            for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(kv_tmp[4 * lane + i]));
-        } else if (wave == 1) {
-            const float *vsrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvw + kvh * kD;
-            uint16_t *dst = vc + static_cast<size_t>(p) * kvw;
-#pragma unroll
-            for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(vsrc[4 * lane + i]));
-        }
-        __threadfence_block();
-    }
-    if (tid < kRep) {
-        mrun[tid] = -INFINITY;
-        lrun[tid] = 0.f;
-    }
+    __threadfence_block();
     __syncthreads();
-
-    // The slice is walked in chunks of kChunk cells, flash-decoding style: the chunk's V rows are
-    // requested first and arrive while its scores are being formed.
-    float acc[kRep][4];
+    // the cells this launch appended can be read now
+    if (c1 > p_first) {
 #pragma unroll
-    for (int hh = 0; hh < kRep; hh++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc[hh][i] = 0.f;
-
-    const int li = lane & 31, cg = lane >> 5;
-    float qr[kRep][8];
-    if (nc > 0) {
-#pragma unroll
-        for (int hh = 0; hh < kRep; hh++) {
-            const float4 q0 = *reinterpret_cast<const float4 *>(&qh[hh][8 * li]);
-            const float4 q1 = *reinterpret_cast<const float4 *>(&qh[hh][8 * li + 4]);
-            qr[hh][0] = q0.x; qr[hh][1] = q0.y; qr[hh][2] = q0.z; qr[hh][3] = q0.w;
-            qr[hh][4] = q1.x; qr[hh][5] = q1.y; qr[hh][6] = q1.z; qr[hh][7] = q1.w;
+        for (int u = 0; u < kWaveCells / 2; u++) {
+            const int c = c0 + wave * kWaveCells + 2 * u + cg;
+            if (c >= p_first && c < c1) kq[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c) * kvw + 8 * li);
         }
+#pragma unroll
+        for (int u = 0; u < kWaveCells; u++) {
+            const int c = c0 + wave * kWaveCells + u;
+            if (c >= p_first && c < c1) vq[u] = *reinterpret_cast<const uint2 *>(vc + static_cast<size_t>(c) * kvw + 4 * lane);
+        }
+    }
+
+    // per lane: accumulators of 4 dims for every (row, head); the wave's running max and sum of
+    // (row, head = lane%8), the same in the eight lanes that share the head
+    float acc[R][kRep][4];
+    float m_run[R], l_run[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        m_run[j] = -INFINITY;
+        l_run[j] = 0.f;
+#pragma unroll
+        for (int hh = 0; hh < kRep; hh++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[j][hh][i] = 0.f;
     }
     const float scale = 1.f / sqrtf(static_cast<float>(kD));
     const int my_head = ((li >> 4) & 1) * 4 + ((li >> 3) & 1) * 2 + ((li >> 2) & 1);
 
     for (int ch0 = 0; ch0 < nc; ch0 += kChunk) {
-        const int cn = nc - ch0 < kChunk ? nc - ch0 : kChunk;
-        // (a) V rows of this wave's cells of the chunk: cells wave, wave+4, ... (4 dims a lane)
-        constexpr int VPW = kChunk / 4;
-        uint2 vq[VPW];
-#pragma unroll
-        for (int u = 0; u < VPW; u++) {
-            const int c = wave + 4 * u;
-            vq[u] = *reinterpret_cast<const uint2 *>(vc + static_cast<size_t>(c0 + ch0 + (c < cn ? c : 0)) * kvw + 4 * lane);
+        const int wc0 = c0 + ch0 + wave * kWaveCells;  // this wave's first cell of the chunk
+        if (ch0 > 0) {
+            load_k(ch0, false);
+            load_v(ch0, false);
         }
-        // (b) scores: 32 lanes a cell, 8 dims a lane, eight passes of the wave loaded together
-        constexpr int PB = 8;
+        if (wc0 < c1) {
 #pragma unroll
-        for (int half = 0; half < kChunk / (8 * PB); half++) {
-            const int cb0 = half * 8 * PB + wave * 2;
-            if (cb0 < cn) {
-                uint4 kq[PB];
+            for (int j = 0; j < R; j++) {
+                // (a) scores of row j: its queries come back from LDS, 8 dims of every head a lane
+                float qr[kRep][8];
 #pragma unroll
-                for (int u = 0; u < PB; u++) {
-                    const int c = cb0 + 8 * u + cg;
-                    kq[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c0 + ch0 + (c < cn ? c : 0)) * kvw + 8 * li);
+                for (int hh = 0; hh < kRep; hh++) {
+                    const float4 q0 = *reinterpret_cast<const float4 *>(&sm.qh[j][hh][8 * li]);
+                    const float4 q1 = *reinterpret_cast<const float4 *>(&sm.qh[j][hh][8 * li + 4]);
+                    qr[hh][0] = q0.x; qr[hh][1] = q0.y; qr[hh][2] = q0.z; qr[hh][3] = q0.w;
+                    qr[hh][4] = q1.x; qr[hh][5] = q1.y; qr[hh][6] = q1.z; qr[hh][7] = q1.w;
                 }
 #pragma unroll
-                for (int u = 0; u < PB; u++) {
-                    const int c = cb0 + 8 * u + cg;
+                for (int u = 0; u < kWaveCells / 2; u++) {
+                    const int cl = 2 * u + cg, c = wc0 + cl;
                     const float2 k01 = half2_bits_to_float2(kq[u].x), k23 = half2_bits_to_float2(kq[u].y);
                     const float2 k45 = half2_bits_to_float2(kq[u].z), k67 = half2_bits_to_float2(kq[u].w);
                     float part[kRep];
@@ -208,160 +251,147 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_arg
                         part[hh] = sdot;
                     }
                     const float tot = reduce8_over32(part, li);
-                    if (c < cn && (li & 3) == 0) sc[c][my_head] = tot * scale;
+                    // causal: row j sees cells up to its own position
+                    if ((li & 3) == 0) sm.sc[wave][j][cl][my_head] = (c < c1 && c <= p_first + j) ? tot * scale : -INFINITY;
                 }
+                __builtin_amdgcn_wave_barrier();
+                // (b) the wave's running max and sum: lane = (cell pair g, g+8 ; head)
+                {
+                    const int hh = lane & 7, g = lane >> 3;
+                    const float s0 = sm.sc[wave][j][g][hh], s1 = kWaveCells > 8 ? sm.sc[wave][j][(g + 8) % kWaveCells][hh] : -INFINITY;
+                    float mx = fmaxf(s0, s1);
+                    mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                    const float m_new = fmaxf(m_run[j], mx);
+                    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: all weights 0
+                    const float e0 = __expf(s0 - m_use), e1 = __expf(s1 - m_use);
+                    sm.sc[wave][j][g][hh] = e0;
+                    if (kWaveCells > 8) sm.sc[wave][j][(g + 8) % kWaveCells][hh] = e1;
+                    float sum = e0 + e1;
+                    sum += __shfl_xor(sum, 8, 64);
+                    sum += __shfl_xor(sum, 16, 64);
+                    sum += __shfl_xor(sum, 32, 64);
+                    const float alpha = __expf(m_run[j] - m_use);  // 0 while the old max is -inf
+                    l_run[j] = l_run[j] * alpha + sum;
+                    m_run[j] = m_new;
+                    if (g == 0) sm.al[wave][j][hh] = alpha;
+                }
+                __builtin_amdgcn_wave_barrier();
+                // (c) acc = acc*alpha + P*V over the wave's cells
+                {
+                    const float4 a0 = *reinterpret_cast<const float4 *>(&sm.al[wave][j][0]);
+                    const float4 a1 = *reinterpret_cast<const float4 *>(&sm.al[wave][j][4]);
+                    const float alv[kRep] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+                    for (int hh = 0; hh < kRep; hh++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc[j][hh][i] *= alv[hh];
+                }
+#pragma unroll
+                for (int u = 0; u < kWaveCells; u++) {
+                    const float2 v01 = half2_bits_to_float2(vq[u].x), v23 = half2_bits_to_float2(vq[u].y);
+                    const float4 p0 = *reinterpret_cast<const float4 *>(&sm.sc[wave][j][u][0]);
+                    const float4 p1 = *reinterpret_cast<const float4 *>(&sm.sc[wave][j][u][4]);
+                    const float pr[kRep] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+                    for (int hh = 0; hh < kRep; hh++) {
+                        acc[j][hh][0] = fmaf(pr[hh], v01.x, acc[j][hh][0]);
+                        acc[j][hh][1] = fmaf(pr[hh], v01.y, acc[j][hh][1]);
+                        acc[j][hh][2] = fmaf(pr[hh], v23.x, acc[j][hh][2]);
+                        acc[j][hh][3] = fmaf(pr[hh], v23.y, acc[j][hh][3]);
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
             }
         }
+    }
+    // ---- the four waves' results of each row are merged and go to scratch ----
+    float *part_base = a.partial + ((static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits + split) * R * kRec;
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        if (lane < kRep) {
+            sm.wm[wave][lane] = m_run[j];
+            sm.wl[wave][lane] = l_run[j];
+        }
+#pragma unroll
+        for (int hh = 0; hh < kRep; hh++)
+            *reinterpret_cast<float4 *>(&sm.big[wave][hh][4 * lane]) = make_float4(acc[j][hh][0], acc[j][hh][1], acc[j][hh][2], acc[j][hh][3]);
         __syncthreads();
-        // (c) running max, the chunk's exponentials and their sum, per head
         {
-            const int hh = tid & 7, stripe = tid >> 3;  // 32 stripes of cells
-            float mx = -INFINITY;
-            for (int c = stripe; c < cn; c += 32) mx = fmaxf(mx, sc[c][hh]);
-            mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            if (lane < kRep) red[wave][lane] = mx;
-            const float m_old = mrun[hh];
-            __syncthreads();
-            const float m_new = fmaxf(m_old, fmaxf(fmaxf(red[0][hh], red[1][hh]), fmaxf(red[2][hh], red[3][hh])));
-            __syncthreads();
-            float sum = 0.f;
-            for (int c = stripe; c < cn; c += 32) {
-                const float e = __expf(sc[c][hh] - m_new);
-                sc[c][hh] = e;
-                sum += e;
+            // thread = (head, 8 dims) here as in the merge below
+            const int hh = tid >> 5, d0 = (tid & 31) * 8;
+            float M = fmaxf(fmaxf(sm.wm[0][hh], sm.wm[1][hh]), fmaxf(sm.wm[2][hh], sm.wm[3][hh]));
+            float w[4], L = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                w[k] = sm.wm[k][hh] == -INFINITY ? 0.f : __expf(sm.wm[k][hh] - M);
+                L = fmaf(w[k], sm.wl[k][hh], L);
             }
-            sum += __shfl_xor(sum, 8, 64);
-            sum += __shfl_xor(sum, 16, 64);
-            sum += __shfl_xor(sum, 32, 64);
-            if (lane < kRep) red[wave][lane] = sum;
-            __syncthreads();
-            if (tid < kRep) {
-                const float al = __expf(m_old - m_new);  // 0 on the first chunk (m_old = -inf)
-                alpha[tid] = al;
-                lrun[tid] = lrun[tid] * al + ((red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]));
-                mrun[tid] = m_new;
-            }
-            __syncthreads();
-        }
-        // (d) acc = acc*alpha + P*V over this wave's cells of the chunk
+            float *rec = part_base + j * kRec + hh * (kD + 2);
 #pragma unroll
-        for (int hh = 0; hh < kRep; hh++) {
-            const float al = alpha[hh];
+            for (int i = 0; i < 8; i += 2) {
+                float v0 = 0.f, v1 = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[hh][i] *= al;
-        }
-#pragma unroll
-        for (int u = 0; u < VPW; u++) {
-            const int c = wave + 4 * u;
-            if (c < cn) {
-                const float2 v01 = half2_bits_to_float2(vq[u].x), v23 = half2_bits_to_float2(vq[u].y);
-                const float4 p0 = *reinterpret_cast<const float4 *>(&sc[c][0]);
-                const float4 p1 = *reinterpret_cast<const float4 *>(&sc[c][4]);
-                const float pr[kRep] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-#pragma unroll
-                for (int hh = 0; hh < kRep; hh++) {
-                    acc[hh][0] = fmaf(pr[hh], v01.x, acc[hh][0]);
-                    acc[hh][1] = fmaf(pr[hh], v01.y, acc[hh][1]);
-                    acc[hh][2] = fmaf(pr[hh], v23.x, acc[hh][2]);
-                    acc[hh][3] = fmaf(pr[hh], v23.y, acc[hh][3]);
+                for (int k = 0; k < 4; k++) {
+                    v0 = fmaf(w[k], sm.big[k][hh][d0 + i], v0);
+                    v1 = fmaf(w[k], sm.big[k][hh][d0 + i + 1], v1);
                 }
+                *reinterpret_cast<float2 *>(rec + d0 + i) = make_float2(v0, v1);
             }
+            if ((tid & 31) == 0) *reinterpret_cast<float2 *>(rec + kD) = make_float2(M, L);
         }
         __syncthreads();
     }
-    const float m_head = tid < kRep ? mrun[tid] : 0.f, l_head = tid < kRep ? lrun[tid] : 0.f;
-    // cross-wave sum through LDS: buf[wave][head][dim]
-    float *buf = big;
+}
+
+// grid: (n_head * 4, R, n_seq), one wave = 64 dims of one head.  The slices' records of that
+// (row, head) are combined with a running max; all of a batch's loads are in flight together.
+template <int R>
+__global__ __launch_bounds__(64) void attn_merge_kernel(shv_attn_decode_args a, int row0) {
+    const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + threadIdx.x, j = blockIdx.y, seq = blockIdx.z;
+    const int kvh = head / kRep, hh = head % kRep;
+    const int n_cells = (a.pos ? a.pos[seq] : 0) + row0 + R;
+    int n_active = (n_cells + kChunk - 1) / kChunk;
+    if (n_active > a.n_splits) n_active = a.n_splits;
+    const float *pin = a.partial + (static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
+    constexpr int MB = 64;
+    float num = 0.f, den = 0.f, M = -INFINITY;
+    for (int s0 = 0; s0 < n_active; s0 += MB) {
+        float v[MB];
+        float2 ml[MB];
 #pragma unroll
-    for (int hh = 0; hh < kRep; hh++)
-        *reinterpret_cast<float4 *>(buf + (wave * kRep + hh) * kD + 4 * lane) =
-            make_float4(acc[hh][0], acc[hh][1], acc[hh][2], acc[hh][3]);
-    if (tid < kRep) {
-        stat[0][tid] = m_head;
-        stat[1][tid] = l_head;
-    }
-    __syncthreads();
-    // partial record of this block: per head, d accumulators then (max, sum)
-    float *part_out = a.partial + ((static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits + split) * kRep * (kD + 2);
-    // thread = (head, 8 dims) here as in the merge below
-    {
-        const int hh = tid >> 5, d0 = (tid & 31) * 8;
-        float *rec = part_out + hh * (kD + 2) + d0;
+        for (int u = 0; u < MB; u++) {
+            const int sidx = s0 + u < n_active ? s0 + u : s0;
+            const float *rec = pin + static_cast<size_t>(sidx) * R * kRec;
+            v[u] = rec[d];
+            ml[u] = *reinterpret_cast<const float2 *>(rec + kD);
+        }
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) {
-            const float v0 = (buf[(0 * kRep + hh) * kD + d0 + i] + buf[(1 * kRep + hh) * kD + d0 + i]) +
-                             (buf[(2 * kRep + hh) * kD + d0 + i] + buf[(3 * kRep + hh) * kD + d0 + i]);
-            const float v1 = (buf[(0 * kRep + hh) * kD + d0 + i + 1] + buf[(1 * kRep + hh) * kD + d0 + i + 1]) +
-                             (buf[(2 * kRep + hh) * kD + d0 + i + 1] + buf[(3 * kRep + hh) * kD + d0 + i + 1]);
-            store_agent2(rec + i, v0, v1);
+        for (int u = 0; u < MB; u++) {
+            if (s0 + u >= n_active || ml[u].x == -INFINITY) continue;
+            const float Mn = fmaxf(M, ml[u].x);
+            const float shrink = __expf(M - Mn), w = __expf(ml[u].x - Mn);  // shrink is 0 while M is -inf
+            den = fmaf(den, shrink, w * ml[u].y);
+            num = fmaf(num, shrink, w * v[u]);
+            M = Mn;
         }
     }
-    if (tid < kRep) store_agent2(part_out + tid * (kD + 2) + kD, stat[0][tid], stat[1][tid]);
-    // ---- the last slice of this (sequence, KV head) to arrive merges them all ----
-    if (!arrive_last(counters + seq * a.n_head_kv + kvh, n_active, &is_last)) return;
-    const float *pin = a.partial + (static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits * kRep * (kD + 2);
-    // weights of the slices: w[s][h] = exp(m_s - M_h), and the merged denominator per head
-    float *wbuf = big;  // [n_active][kRep], and a second plane of the same size
-    for (int i = tid; i < n_active * kRep; i += kBlock) {
-        const int sidx = i / kRep, hh = i % kRep;
-        wbuf[i] = load_agent(pin + (static_cast<size_t>(sidx) * kRep + hh) * (kD + 2) + kD);
+    a.out[static_cast<size_t>(seq * a.seq_len + row0 + j) * a.n_head * kD + static_cast<size_t>(head) * kD + d] = num / den;
+}
+
+template <int R>
+int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0) {
+    static bool raised = false;
+    if (sizeof(Smem<R>) > 48 * 1024 && !raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_decode_kernel<R>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          static_cast<int>(sizeof(Smem<R>))));
+        raised = true;
     }
-    __syncthreads();
-    if (tid < kRep) {
-        float M = -INFINITY;
-        for (int sidx = 0; sidx < n_active; sidx++) M = fmaxf(M, wbuf[sidx * kRep + tid]);
-        stat[0][tid] = M;
-    }
-    __syncthreads();
-    for (int i = tid; i < n_active * kRep; i += kBlock) {
-        const int sidx = i / kRep, hh = i % kRep;
-        const float ms = wbuf[i];
-        const float w = ms == -INFINITY ? 0.f : __expf(ms - stat[0][hh]);
-        wbuf[i] = w;
-        // the slice's sum of exponentials, scaled, goes to a second plane
-        wbuf[kPlane + i] = w * load_agent(pin + (static_cast<size_t>(sidx) * kRep + hh) * (kD + 2) + kD + 1);
-    }
-    __syncthreads();
-    if (tid < kRep) {
-        float den = 0.f;
-        for (int sidx = 0; sidx < n_active; sidx++) den += wbuf[kPlane + sidx * kRep + tid];
-        stat[1][tid] = den;
-    }
-    __syncthreads();
-    // thread = (head, 8 dims): n_active records of two float4 each, eight slices in flight
-    {
-        const int hh = tid >> 5, d0 = (tid & 31) * 8;
-        float num[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        constexpr int MB = 16;
-        for (int s0 = 0; s0 < n_active; s0 += MB) {
-            float4 r0[MB], r1[MB];
-#pragma unroll
-            for (int u = 0; u < MB; u++) {
-                const int sidx = s0 + u < n_active ? s0 + u : s0;
-                const float *rec = pin + (static_cast<size_t>(sidx) * kRep + hh) * (kD + 2) + d0;
-                // records are 258 floats long, so only 8-byte alignment holds
-                const float2 a0 = load_agent2(rec), a1 = load_agent2(rec + 2);
-                const float2 a2 = load_agent2(rec + 4), a3 = load_agent2(rec + 6);
-                r0[u] = make_float4(a0.x, a0.y, a1.x, a1.y);
-                r1[u] = make_float4(a2.x, a2.y, a3.x, a3.y);
-            }
-#pragma unroll
-            for (int u = 0; u < MB; u++) {
-                if (s0 + u >= n_active) break;
-                const float w = wbuf[(s0 + u) * kRep + hh];
-                num[0] = fmaf(w, r0[u].x, num[0]); num[1] = fmaf(w, r0[u].y, num[1]);
-                num[2] = fmaf(w, r0[u].z, num[2]); num[3] = fmaf(w, r0[u].w, num[3]);
-                num[4] = fmaf(w, r1[u].x, num[4]); num[5] = fmaf(w, r1[u].y, num[5]);
-                num[6] = fmaf(w, r1[u].z, num[6]); num[7] = fmaf(w, r1[u].w, num[7]);
-            }
-        }
-        const float inv = 1.f / stat[1][hh];
-        float *o = a.out + static_cast<size_t>(row) * a.n_head * kD + static_cast<size_t>(kvh * kRep + hh) * kD + d0;
-        *reinterpret_cast<float4 *>(o) = make_float4(num[0] * inv, num[1] * inv, num[2] * inv, num[3] * inv);
-        *reinterpret_cast<float4 *>(o + 4) = make_float4(num[4] * inv, num[5] * inv, num[6] * inv, num[7] * inv);
-    }
+    dim3 grid(a.n_splits, a.n_head_kv, a.n_seq);
+    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), sizeof(Smem<R>), a, row0);
+    SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq), dim3(64), 0, a, row0);
+    return SHV_OK;
 }
 
 }  // namespace
@@ -374,15 +404,16 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
                 a.n_head, a.n_head_kv, kRep);
     SHV_REQUIRE(a.rope_dims >= 0 && a.rope_dims <= 128 && a.rope_dims % 2 == 0, "attn_decode: rope_dims %d", a.rope_dims);
     SHV_REQUIRE(a.n_seq >= 1 && a.seq_len >= 1, "attn_decode: %d sequences of %d rows", a.n_seq, a.seq_len);
-    SHV_REQUIRE(a.n_seq * a.n_head_kv <= ctx->n_counters - shv_ctx::kCounterAttn, "attn_decode: %d sequences is more than the library tracks", a.n_seq);
+    SHV_REQUIRE(a.n_seq <= 65535, "attn_decode: %d sequences", a.n_seq);
     SHV_REQUIRE(a.n_splits >= 1 && a.n_splits <= kMaxSplits, "attn_decode: %d slices; 1..%d", a.n_splits, kMaxSplits);
     SHV_REQUIRE(a.qkv_stride >= a.n_head * 2 * kD + 2 * a.n_head_kv * kD, "attn_decode: qkv_stride %d", a.qkv_stride);
     SHV_REQUIRE(shv_aligned16(a.qkv) && shv_aligned16(a.kcache) && shv_aligned16(a.vcache) && shv_aligned16(a.q_norm) &&
                     shv_aligned16(a.k_norm) && shv_aligned16(a.out) && shv_aligned16(a.partial) && a.qkv_stride % 4 == 0,
                 "attn_decode: qkv, caches, norms, partial and out must be 16-byte aligned");
-    dim3 grid(a.n_splits, a.n_head_kv, a.n_seq);
-    for (int i = 0; i < a.seq_len; i++) {
-        SHV_LAUNCH(ctx, attn_decode_kernel, grid, dim3(kBlock), 0, a, i, ctx->counters + shv_ctx::kCounterAttn);
+    // the rows of a sequence go two at a time: both see one pass over the cache
+    for (int i = 0; i < a.seq_len; i += 2) {
+        const int rc = a.seq_len - i >= 2 ? launch_rows<2>(ctx, a, i) : launch_rows<1>(ctx, a, i);
+        if (rc != SHV_OK) return rc;
     }
     return SHV_OK;
 }

@@ -521,9 +521,9 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
 }
 
 void AttnGPU::SetSplits(int n) {
-    // slices for the cache's capacity: about 128 cells each up to 256 slices (the kernel engages
-    // only as many as the sequence's current length fills)
-    if (n <= 0) n = std::min(256, std::max(8, (n_kv_ + 127) / 128));
+    // slices for the cache's capacity: about 64 cells each up to the kernel's limit (the kernel
+    // engages only as many as the sequence's current length fills)
+    if (n <= 0) n = std::min(kMaxSplits, std::max(8, (n_kv_ + 63) / 64));
     if (n > kMaxSplits) throw Error("llm: AttnGPU.SetSplits: at most " + std::to_string(kMaxSplits) + " slices");
     splits_ = n;
 }

@@ -76,8 +76,8 @@ class AttnCase:
         ]
 
 
-def _part_floats(n_seq, n_splits):
-    return n_seq * NKV * n_splits * (NH // NKV) * (D + 2)
+def _part_floats(n_seq, n_splits, seq_len=1):
+    return n_seq * min(seq_len, 2) * NKV * n_splits * (NH // NKV) * (D + 2)
 
 
 def test_decode_steps_from_an_empty_cache(ctx):
@@ -109,6 +109,36 @@ def test_decode_steps_from_an_empty_cache(ctx):
         g, w = got.view(np.float16).astype(np.float32), want.view(np.float16).astype(np.float32)
         assert (np.abs(g - w) <= np.abs(w) * 2.0 ** -10 + 1e-5).all()
         assert np.count_nonzero(got != want) <= got.size // 20
+
+
+@pytest.mark.parametrize("past,rows,n_splits", [(0, 2, 4), (0, 5, 4), (61, 4, 8), (300, 3, 16), (4000, 2, 64)])
+def test_rows_of_one_sequence_in_one_call(ctx, past, rows, n_splits):
+    """A verification pass or a prompt chunk: `rows` consecutive rows appended in one call, each
+    seeing the cells up to its own (the cache is walked once for two rows at a time), against the
+    oracle's layer over the same rows; the new cells may straddle a slice boundary."""
+    case = AttnCase(ctx, seed=5 + past)
+    max_cells = ((past + rows + 63) // 64) * 64
+    case.upload(max_cells)
+    rng = case.rng
+    kc = np.zeros((max_cells, NKV, D), np.uint16)
+    vc = np.zeros_like(kc)
+    kc[:past] = rng.standard_normal((past, NKV, D)).astype(np.float16).view(np.uint16)
+    vc[:past] = rng.standard_normal((past, NKV, D)).astype(np.float16).view(np.uint16)
+    xn = rng.standard_normal((rows, H)).astype(np.float32)
+    c = ctx
+    d_kc, d_vc = c.upload(kc), c.upload(vc)
+    want_out, want_pre = case.oracle(xn, past, kc, vc)
+    d_qkv, d_ctx, d_out = c.alloc(rows * case.width * 4), c.alloc(rows * NH * D * 4), c.alloc(rows * H * 4)
+    d_part = c.alloc(_part_floats(1, n_splits, rows) * 4)
+    c.dispatch_multi(case.ops(c.upload(xn), d_qkv, d_kc, d_vc, d_part, d_ctx, d_out,
+                              c.upload(np.array([past], np.int32)), 1, rows, max_cells, n_splits))
+    got_pre = d_ctx.read(np.float32, rows * NH * D).reshape(rows, -1)
+    got_out = d_out.read(np.float32, rows * H).reshape(rows, -1)
+    for t in range(rows):
+        assert O.rel_l2(got_pre[t], want_pre[t]) <= TOL and O.rel_l2(got_out[t], want_out[t]) <= TOL, t
+    got_k = d_kc.read(np.uint16, kc.size).reshape(kc.shape)[past:past + rows]
+    g, w = got_k.view(np.float16).astype(np.float32), kc[past:past + rows].view(np.float16).astype(np.float32)
+    assert (np.abs(g - w) <= np.abs(w) * 2.0 ** -10 + 1e-5).all()
 
 
 @pytest.mark.parametrize("past,n_seq,n_splits", [(4096, 1, 16), (4096, 3, 16), (32768, 1, 64),
