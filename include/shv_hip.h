@@ -261,8 +261,12 @@ typedef struct {
  * sin[rope_dims/2]; llm/gpu_attn.go:1452-1476), K and V rounded to binary16 into cell p of the
  * cache, then causal GQA softmax attention of the row over cells 0..p, split n_splits ways over
  * the cells and merged.  out is [rows][n_head*d] BEFORE the sigmoid gate, which the output
- * projection applies as its prologue.  kcache / vcache are [n_slots][max_cells][n_head_kv][d]
- * binary16; partial is scratch of n_seq*min(seq_len,2)*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2)
+ * projection applies as its prologue.  kcache is [n_slots][max_cells][n_head_kv][d] binary16;
+ * vcache holds V transposed in tiles of 32 cells, [n_slots][max_cells/32][n_head_kv][d][32] binary16
+ * (four cells of one dim are one operand of the second product, a tile of one KV head is 16
+ * contiguous KB).  max_cells is a multiple of 32 and both caches hold finite
+ * values in every cell (zeros before a cell is written): the last tile of a sequence reads a few
+ * cells past its end and weights them by zero. partial is scratch of n_seq*min(seq_len,2)*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2)
  * floats (the rows of a sequence are taken two at a time over one pass of the cache). */
 typedef struct {
     const float *qkv;

@@ -1,19 +1,26 @@
 // Gated full-attention decode over an fp16 KV cache, GQA with 8 query heads per KV head, one or
-// two consecutive rows of a sequence per launch.
+// two consecutive rows of a sequence per launch, on the matrix cores.
 //
 // HBM-bound on the cache: a block owns one KV head and one slice of the cells and serves all the
 // query heads of that KV head, for both rows, from a single pass over K and a single pass over V.
-//   start     the wave's first K and V rows are requested before anything else
-//   prologue  per-head RMS norm + rotary of the block's query heads into LDS; the block whose slice
-//             holds a new cell also normalises/rotates K, rounds K and V to binary16 and appends them
-//   per chunk of 64 cells, every wave on its own 16 cells with no block-wide synchronisation:
-//     scores (32 lanes a cell, 16-byte loads of K, eight partial dots a lane reduced with a
-//     transposing butterfly), a running max and sum per (row, head) kept by the wave, P*V with 64
-//     lanes across the 256 dims of a V row
-//   epilogue  the four waves' (max, sum, accumulator) are merged through LDS and go to scratch
-// A second, small kernel merges the slices: one block a (row, head), one thread a dim, every
-// slice's value requested at once.  (Merging in the last block to arrive instead costs more than
-// the launch: that block walks all the records alone, a few dependent round trips to memory.)
+// The 8 heads x 2 rows are the 16 rows of a v_mfma_f32_16x16x16_f16 tile:
+//   S^T = K Q^T   A = 16 cells x 16 dims of K straight from the cache (it is binary16 already),
+//                 B = the queries as hi + lo halves (so the product keeps float32 accuracy), kept
+//                 in LDS in operand order.  Computing the transpose leaves each lane with the
+//                 scores of one query row and four consecutive cells, which is exactly the A
+//                 operand of the second product: the probabilities never move between lanes
+//   O += P V      A = P as hi + lo halves, B = 16 cells x 16 dims of V.  V is cached transposed in
+//                 tiles of 32 cells, [cell/32][kv head][dim][cell%32], so that a lane's four cells of
+//                 one dim are 8 contiguous bytes and a wave's tile is 16 contiguous KB
+//   softmax       running max and sum per query row in the four lanes that share the row; the
+//                 accumulators are rescaled only when some row's maximum moved
+//   prologue      the wave's first tile of K and V is requested before anything else; per-head RMS
+//                 norm + rotary of the queries; the block whose slice holds a new cell normalises /
+//                 rotates K, rounds K and V to binary16 and appends them
+//   epilogue      the four waves' (max, sum, accumulator) are merged through LDS and go to scratch
+// A second, small kernel merges the slices: one wave a (row, head, 64 dims), every slice's value
+// requested at once.  (Merging in the last block to arrive instead costs more than the launch: that
+// block walks all the records alone, a few dependent round trips to memory.)
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
 
@@ -24,50 +31,15 @@ using namespace shv;
 constexpr int kBlock = 256;
 constexpr int kD = 256;        // head dimension the kernel is built for
 constexpr int kRep = 8;        // query heads per KV head
-#ifndef SHV_ATTN_WAVE_CELLS
-#define SHV_ATTN_WAVE_CELLS 16
-#endif
-constexpr int kWaveCells = SHV_ATTN_WAVE_CELLS; // cells a wave scores together
-constexpr int kChunk = 4 * kWaveCells;
+constexpr int kTile = 32;         // cells a wave takes at a time
+constexpr int kSliceCells = 128;  // cells a slice gets while there are slices to spare: one tile a wave
 constexpr int kMaxSplits = 512;
 constexpr int kRec = kRep * (kD + 2);  // floats of one (slice, row) record: per head d values, max, sum
 
-// v[8] per lane -> the sum over the 32 lanes of an aligned half-wave of v[head], where
-// head = bit4(li)*4 + bit3(li)*2 + bit2(li); every lane of the half-wave gets one head's total.
-__device__ __forceinline__ float reduce8_over32(const float *v, int li) {
-    const bool b4 = (li & 16) != 0, b3 = (li & 8) != 0, b2 = (li & 4) != 0;
-    float r[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float keep = b4 ? v[i + 4] : v[i];
-        const float send = b4 ? v[i] : v[i + 4];
-        r[i] = keep + __shfl_xor(send, 16, 64);
-    }
-    float r2[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const float keep = b3 ? r[i + 2] : r[i];
-        const float send = b3 ? r[i] : r[i + 2];
-        r2[i] = keep + __shfl_xor(send, 8, 64);
-    }
-    const float keep = b2 ? r2[1] : r2[0];
-    const float send = b2 ? r2[0] : r2[1];
-    float t = keep + __shfl_xor(send, 4, 64);
-    t += dpp_f32<kDppXor2>(t);
-    t += dpp_f32<kDppXor1>(t);
-    return t;
-}
-
-__device__ __forceinline__ float2 half2_bits_to_float2(uint32_t u) {
-    const f16x2_native h = __builtin_bit_cast(f16x2_native, u);
-    return make_float2(static_cast<float>(h.x), static_cast<float>(h.y));
-}
-
 // RMS norm over the 256 dims of one head by one wave (4 dims per lane), then NeoX rotary on the
 // first rope_dims dims through LDS.  dst is 256 floats of LDS.
-__device__ __forceinline__ void norm_rope_head(const float *src, const float *gamma, const float *rope_row, int rope_dims,
-                                               float eps, float *dst, int lane) {
-    const float4 v = *reinterpret_cast<const float4 *>(src + 4 * lane);
+__device__ __forceinline__ void norm_rope_loaded(const float4 v, const float *gamma, const float *rope_row, int rope_dims, float eps,
+                                                 float *dst, int lane) {
     const float ss = wave_sum_all(fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w))));
     const float sc = 1.f / sqrtf(ss / static_cast<float>(kD) + eps);
     const float4 g = *reinterpret_cast<const float4 *>(gamma + 4 * lane);
@@ -86,73 +58,104 @@ __device__ __forceinline__ void norm_rope_head(const float *src, const float *ga
     __builtin_amdgcn_wave_barrier();
 }
 
-// LDS of one block, R rows a launch.
-template <int R>
+__device__ __forceinline__ void norm_rope_head(const float *src, const float *gamma, const float *rope_row, int rope_dims,
+                                               float eps, float *dst, int lane) {
+    norm_rope_loaded(*reinterpret_cast<const float4 *>(src + 4 * lane), gamma, rope_row, rope_dims, eps, dst, lane);
+}
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ half4_t as_half4(uint32_t a, uint32_t b) {
+    u32x2_t v;
+    v.x = a;
+    v.y = b;
+    return __builtin_bit_cast(half4_t, v);
+}
+
+// x -> (hi, lo) halves with hi + lo = x to about 2^-22
+__device__ __forceinline__ void split4(const float *x, half4_t &h, half4_t &l) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const _Float16 hi = static_cast<_Float16>(x[t]);
+        h[t] = hi;
+        l[t] = static_cast<_Float16>(x[t] - static_cast<float>(hi));
+    }
+}
+
+// LDS of one block.  The queries are kept as matrix-core operands: entry [i][h][part][lane] is the
+// four dims 8*(kb + 4*i) + 4*h .. +3 of query row lane%16 (kb = lane/16), as hi or lo halves.
 struct Smem {
-    float qh[R][kRep][kD];                    // normalised, rotated queries
-    float sc[4][R][kWaveCells][kRep];         // per wave: scores, then probabilities, of its cells
-    float al[4][R][kRep];                     // per wave: the factor the running sums shrink by
-    float big[4][kRep][kD];                   // the waves' accumulators of one row, to be merged
-    float wm[4][kRep], wl[4][kRep];           // the waves' running max and sum of one row
-    float kv_tmp[R][kD];
+    half4_t qf[8][2][2][64];       // 16 KB
+    float big[4][kRep][kD];        // 32 KB: queries in float32 first; later the waves' accumulators of one row
+    float al[4][16];               // per wave: the factor each query row's running sums shrink by
+    float wm[4][16], wl[4][16];    // per wave: running max and sum of each query row
+    float kv_tmp[2][kD];
 };
 
-// grid: (n_splits, n_head_kv, n_seq); rows row0..row0+R-1 of each sequence.
+// grid: (n_splits, n_head_kv, n_seq); rows row0..row0+R-1 of each sequence.  Query row r of the
+// tile is head r%8 of sequence row r/8; with R = 1 rows 8..15 are padding.
 template <int R>
-__global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_args a, int row0) {
-    extern __shared__ __align__(16) char smem_raw[];
-    Smem<R> &sm = *reinterpret_cast<Smem<R> *>(smem_raw);
-
+__global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_args a, int row0) {
+    __shared__ Smem sm;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
     const int slot = a.slot ? a.slot[seq] : seq;
     const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the launch's first row
     const int n_cells = p_first + R;                       // cells the last row sees
     // The grid is sized for the cache's capacity; how many of its slices take part depends on how
-    // many cells the sequence holds now: about kChunk cells a slice while there are slices to
-    // spare, so that a short context is not mostly merge and a long one covers the whole chip.
-    int n_active = (n_cells + kChunk - 1) / kChunk;
+    // many cells the sequence holds now: about kSliceCells a slice while there are slices to spare.
+    int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
     if (n_active > a.n_splits) n_active = a.n_splits;
     if (split >= n_active) return;
     int cps = (n_cells + n_active - 1) / n_active;
-    cps = (cps + 7) & ~7;
+    cps = (cps + kTile - 1) & ~(kTile - 1);  // slices start on a tile of V
     const int c0 = split * cps;
     const int c1 = c0 + cps < n_cells ? c0 + cps : n_cells;
     const int nc = c1 > c0 ? c1 - c0 : 0;
 
     const int kvw = a.n_head_kv * kD;
+    // K is [cell][kv head][dim]; V is kept transposed in tiles of 32 cells,
+    // [cell/32][kv head][dim][cell%32], so that four cells of one dim are 8 contiguous bytes and a
+    // tile of one KV head is 16 contiguous KB
     uint16_t *kc = static_cast<uint16_t *>(a.kcache) + static_cast<size_t>(slot) * a.max_cells * kvw + kvh * kD;
-    uint16_t *vc = static_cast<uint16_t *>(a.vcache) + static_cast<size_t>(slot) * a.max_cells * kvw + kvh * kD;
-    const int li = lane & 31, cg = lane >> 5;
+    uint16_t *vt = static_cast<uint16_t *>(a.vcache) + static_cast<size_t>(slot) * a.max_cells * kvw + static_cast<size_t>(kvh) * kD * kTile;
+    const size_t vtile = static_cast<size_t>(kvw) * kTile;  // halves from one tile of V to the next
+    const int n = lane & 15, q = lane >> 4;
 
-    // ---- the wave's first K and V rows: cells c0 + 16*wave + .. ; only cells that existed before
-    //      this launch may be read this early ----
-    uint4 kq[kWaveCells / 2];
-    uint2 vq[kWaveCells];
-    auto load_k = [&](int ch0, bool old_only) {
-#pragma unroll
-        for (int u = 0; u < kWaveCells / 2; u++) {
-            const int c = c0 + ch0 + wave * kWaveCells + 2 * u + cg;
-            if (c < c1 && (!old_only || c < p_first))
-                kq[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c) * kvw + 8 * li);
-            else if (!old_only || c >= c1)
-                kq[u] = make_uint4(0u, 0u, 0u, 0u);
-        }
+    // One tile = 32 cells of this wave.  Score tile T (0,1), slot s (= lane%16 as the A row) is cell
+    // t0 + 8*(s/4) + 4*T + s%4, so that after the first product lane (row n, q) holds the scores of
+    // cells t0 + 8q + 4T + 0..3: the four consecutive cells its V operand covers.
+    struct Tile {
+        uint4 k[2][8], v[16];
     };
-    auto load_v = [&](int ch0, bool old_only) {
+    Tile ta;
+    auto load_tile = [&](Tile &tl, int t0) {
+        uint4(&kreg)[2][8] = tl.k;
+        uint4(&vreg)[16] = tl.v;
 #pragma unroll
-        for (int u = 0; u < kWaveCells; u++) {
-            const int c = c0 + ch0 + wave * kWaveCells + u;
-            if (c < c1 && (!old_only || c < p_first))
-                vq[u] = *reinterpret_cast<const uint2 *>(vc + static_cast<size_t>(c) * kvw + 4 * lane);
-            else if (!old_only || c >= c1)
-                vq[u] = make_uint2(0u, 0u);
+        for (int T = 0; T < 2; T++) {
+            int c = t0 + 8 * (n >> 2) + 4 * T + (n & 3);
+            c = c < c1 ? c : c1 - 1;
+            const uint16_t *row = kc + static_cast<size_t>(c) * kvw + 8 * q;
+#pragma unroll
+            for (int i = 0; i < 8; i++) kreg[T][i] = *reinterpret_cast<const uint4 *>(row + 32 * i);
         }
+        // this lane's eight cells of V.  The cache is whole tiles, so the cells of the last tile
+        // past the sequence's end exist; they hold finite values and get weight 0.
+#pragma unroll
+        for (int db = 0; db < 16; db++)
+            vreg[db] = *reinterpret_cast<const uint4 *>(vt + static_cast<size_t>(t0 / kTile) * vtile + (16 * db + n) * kTile + 8 * q);
     };
-    load_k(0, true);
-    load_v(0, true);
+    // the wave's first tile is requested before anything else, unless this launch is about to
+    // append cells inside it
+    const int t_first = c0 + kTile * wave;
+    const bool early = t_first < c1 && t_first + kTile <= p_first;
+    if (early) load_tile(ta, t_first);
 
-    // ---- prologue ----
+    // ---- prologue: queries (float32, into sm.big), new cells ----
+    float *qtmp = &sm.big[0][0][0];  // [8*R][kD]
     const float *qkv0 = a.qkv + static_cast<size_t>(seq * a.seq_len + row0) * a.qkv_stride;
 #pragma unroll
     for (int j = 0; j < R; j++) {
@@ -160,173 +163,183 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_arg
         const int p = p_first + j;
         const float *rope_row = a.rope + static_cast<size_t>(p) * a.rope_dims;
         if (nc > 0) {
+            // this wave's two heads: both rows of the fused projection are requested before either is used
+            float4 qv[2];
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const int hh = wave * 2 + i;
-                norm_rope_head(qkv + static_cast<size_t>(kvh * kRep + hh) * 2 * kD, a.q_norm, rope_row, a.rope_dims, a.eps, sm.qh[j][hh], lane);
-            }
+            for (int i = 0; i < 2; i++)
+                qv[i] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(kvh * kRep + wave * 2 + i) * 2 * kD + 4 * lane);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                norm_rope_loaded(qv[i], a.q_norm, rope_row, a.rope_dims, a.eps, qtmp + (8 * j + wave * 2 + i) * kD, lane);
         }
         if (p >= c0 && p < c1) {
-            // the new cell of row j lies in this slice: waves 2j and 2j+1 (mod 4) append its K and V
+            // the new cell of row j lies in this slice: one wave appends its K, all threads its V
             if (wave == ((2 * j) & 3)) {
                 const float *ksrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD;
                 norm_rope_head(ksrc, a.k_norm, rope_row, a.rope_dims, a.eps, sm.kv_tmp[j], lane);
                 uint16_t *dst = kc + static_cast<size_t>(p) * kvw;
 #pragma unroll
                 for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(sm.kv_tmp[j][4 * lane + i]));
-            } else if (wave == ((2 * j + 1) & 3)) {
-                const float *vsrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvw + kvh * kD;
-                uint16_t *dst = vc + static_cast<size_t>(p) * kvw;
-#pragma unroll
-                for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(vsrc[4 * lane + i]));
             }
+            const float *vsrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvw + kvh * kD;
+            vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vsrc[tid]));
         }
     }
     __threadfence_block();
     __syncthreads();
-    // the cells this launch appended can be read now
-    if (c1 > p_first) {
+    if (nc > 0) {
+        // queries as operands: 8*2*64 entries, four a thread; the score scale goes in here
+        const float scale = 1.f / sqrtf(static_cast<float>(kD));
 #pragma unroll
-        for (int u = 0; u < kWaveCells / 2; u++) {
-            const int c = c0 + wave * kWaveCells + 2 * u + cg;
-            if (c >= p_first && c < c1) kq[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c) * kvw + 8 * li);
-        }
-#pragma unroll
-        for (int u = 0; u < kWaveCells; u++) {
-            const int c = c0 + wave * kWaveCells + u;
-            if (c >= p_first && c < c1) vq[u] = *reinterpret_cast<const uint2 *>(vc + static_cast<size_t>(c) * kvw + 4 * lane);
-        }
-    }
-
-    // per lane: accumulators of 4 dims for every (row, head); the wave's running max and sum of
-    // (row, head = lane%8), the same in the eight lanes that share the head
-    float acc[R][kRep][4];
-    float m_run[R], l_run[R];
-#pragma unroll
-    for (int j = 0; j < R; j++) {
-        m_run[j] = -INFINITY;
-        l_run[j] = 0.f;
-#pragma unroll
-        for (int hh = 0; hh < kRep; hh++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) acc[j][hh][i] = 0.f;
-    }
-    const float scale = 1.f / sqrtf(static_cast<float>(kD));
-    const int my_head = ((li >> 4) & 1) * 4 + ((li >> 3) & 1) * 2 + ((li >> 2) & 1);
-
-    for (int ch0 = 0; ch0 < nc; ch0 += kChunk) {
-        const int wc0 = c0 + ch0 + wave * kWaveCells;  // this wave's first cell of the chunk
-        if (ch0 > 0) {
-            load_k(ch0, false);
-            load_v(ch0, false);
-        }
-        if (wc0 < c1) {
-#pragma unroll
-            for (int j = 0; j < R; j++) {
-                // (a) scores of row j: its queries come back from LDS, 8 dims of every head a lane
-                float qr[kRep][8];
-#pragma unroll
-                for (int hh = 0; hh < kRep; hh++) {
-                    const float4 q0 = *reinterpret_cast<const float4 *>(&sm.qh[j][hh][8 * li]);
-                    const float4 q1 = *reinterpret_cast<const float4 *>(&sm.qh[j][hh][8 * li + 4]);
-                    qr[hh][0] = q0.x; qr[hh][1] = q0.y; qr[hh][2] = q0.z; qr[hh][3] = q0.w;
-                    qr[hh][4] = q1.x; qr[hh][5] = q1.y; qr[hh][6] = q1.z; qr[hh][7] = q1.w;
-                }
-#pragma unroll
-                for (int u = 0; u < kWaveCells / 2; u++) {
-                    const int cl = 2 * u + cg, c = wc0 + cl;
-                    const float2 k01 = half2_bits_to_float2(kq[u].x), k23 = half2_bits_to_float2(kq[u].y);
-                    const float2 k45 = half2_bits_to_float2(kq[u].z), k67 = half2_bits_to_float2(kq[u].w);
-                    float part[kRep];
-#pragma unroll
-                    for (int hh = 0; hh < kRep; hh++) {
-                        float sdot = qr[hh][0] * k01.x;
-                        sdot = fmaf(qr[hh][1], k01.y, sdot);
-                        sdot = fmaf(qr[hh][2], k23.x, sdot);
-                        sdot = fmaf(qr[hh][3], k23.y, sdot);
-                        sdot = fmaf(qr[hh][4], k45.x, sdot);
-                        sdot = fmaf(qr[hh][5], k45.y, sdot);
-                        sdot = fmaf(qr[hh][6], k67.x, sdot);
-                        sdot = fmaf(qr[hh][7], k67.y, sdot);
-                        part[hh] = sdot;
-                    }
-                    const float tot = reduce8_over32(part, li);
-                    // causal: row j sees cells up to its own position
-                    if ((li & 3) == 0) sm.sc[wave][j][cl][my_head] = (c < c1 && c <= p_first + j) ? tot * scale : -INFINITY;
-                }
-                __builtin_amdgcn_wave_barrier();
-                // (b) the wave's running max and sum: lane = (cell pair g, g+8 ; head)
-                {
-                    const int hh = lane & 7, g = lane >> 3;
-                    const float s0 = sm.sc[wave][j][g][hh], s1 = kWaveCells > 8 ? sm.sc[wave][j][(g + 8) % kWaveCells][hh] : -INFINITY;
-                    float mx = fmaxf(s0, s1);
-                    mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
-                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                    const float m_new = fmaxf(m_run[j], mx);
-                    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: all weights 0
-                    const float e0 = __expf(s0 - m_use), e1 = __expf(s1 - m_use);
-                    sm.sc[wave][j][g][hh] = e0;
-                    if (kWaveCells > 8) sm.sc[wave][j][(g + 8) % kWaveCells][hh] = e1;
-                    float sum = e0 + e1;
-                    sum += __shfl_xor(sum, 8, 64);
-                    sum += __shfl_xor(sum, 16, 64);
-                    sum += __shfl_xor(sum, 32, 64);
-                    const float alpha = __expf(m_run[j] - m_use);  // 0 while the old max is -inf
-                    l_run[j] = l_run[j] * alpha + sum;
-                    m_run[j] = m_new;
-                    if (g == 0) sm.al[wave][j][hh] = alpha;
-                }
-                __builtin_amdgcn_wave_barrier();
-                // (c) acc = acc*alpha + P*V over the wave's cells
-                {
-                    const float4 a0 = *reinterpret_cast<const float4 *>(&sm.al[wave][j][0]);
-                    const float4 a1 = *reinterpret_cast<const float4 *>(&sm.al[wave][j][4]);
-                    const float alv[kRep] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-#pragma unroll
-                    for (int hh = 0; hh < kRep; hh++)
-#pragma unroll
-                        for (int i = 0; i < 4; i++) acc[j][hh][i] *= alv[hh];
-                }
-#pragma unroll
-                for (int u = 0; u < kWaveCells; u++) {
-                    const float2 v01 = half2_bits_to_float2(vq[u].x), v23 = half2_bits_to_float2(vq[u].y);
-                    const float4 p0 = *reinterpret_cast<const float4 *>(&sm.sc[wave][j][u][0]);
-                    const float4 p1 = *reinterpret_cast<const float4 *>(&sm.sc[wave][j][u][4]);
-                    const float pr[kRep] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-#pragma unroll
-                    for (int hh = 0; hh < kRep; hh++) {
-                        acc[j][hh][0] = fmaf(pr[hh], v01.x, acc[j][hh][0]);
-                        acc[j][hh][1] = fmaf(pr[hh], v01.y, acc[j][hh][1]);
-                        acc[j][hh][2] = fmaf(pr[hh], v23.x, acc[j][hh][2]);
-                        acc[j][hh][3] = fmaf(pr[hh], v23.y, acc[j][hh][3]);
-                    }
-                }
-                __builtin_amdgcn_wave_barrier();
+        for (int e = 0; e < 4; e++) {
+            const int idx = tid + e * kBlock;  // [i][h][lane]
+            const int ln = idx & 63, h = (idx >> 6) & 1, i = idx >> 7;
+            const int row = ln & 15, kb = ln >> 4;
+            float x[4] = {0.f, 0.f, 0.f, 0.f};
+            if (row < 8 * R) {
+                const float4 f = *reinterpret_cast<const float4 *>(qtmp + row * kD + 8 * (kb + 4 * i) + 4 * h);
+                x[0] = f.x * scale; x[1] = f.y * scale; x[2] = f.z * scale; x[3] = f.w * scale;
             }
+            half4_t hi, lo;
+            split4(x, hi, lo);
+            sm.qf[i][h][0][ln] = hi;
+            sm.qf[i][h][1][ln] = lo;
         }
     }
-    // ---- the four waves' results of each row are merged and go to scratch ----
+    __syncthreads();
+
+    // per lane: O[row 4q+i][dim 16*db + n] for the 16 dim blocks; the running max and sum of query
+    // row n (the same in the four lanes that share it)
+    float4_t o[16];
+#pragma unroll
+    for (int db = 0; db < 16; db++) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const int my_row_pos = p_first + (n >> 3);  // the last cell query row n may see
+
+    auto compute = [&](const Tile &tl, int t0) {
+        const uint4(&kreg)[2][8] = tl.k;
+        const uint4(&vreg)[16] = tl.v;
+        // ---- S^T = K Q^T: A = K (cells x dims), B = Q^T (dims x rows); four independent chains
+        //      of products (two score tiles, even and odd dim groups) keep the matrix pipe busy ----
+        float4_t st[2];
+        {
+            float4_t acc[2][2];
+#pragma unroll
+            for (int T = 0; T < 2; T++)
+#pragma unroll
+                for (int e = 0; e < 2; e++) acc[T][e] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                // the query operands come from LDS as they are used: held in registers for the
+                // whole loop they would push the tiles out to scratch
+                const half4_t qh0 = sm.qf[i][0][0][lane], qh1 = sm.qf[i][1][0][lane];
+                const half4_t ql0 = sm.qf[i][0][1][lane], ql1 = sm.qf[i][1][1][lane];
+#pragma unroll
+                for (int T = 0; T < 2; T++) {
+                    const half4_t k0 = as_half4(kreg[T][i].x, kreg[T][i].y), k1 = as_half4(kreg[T][i].z, kreg[T][i].w);
+                    float4_t c = acc[T][i & 1];
+                    c = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qh0, c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qh1, c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, ql0, c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, ql1, c, 0, 0, 0);
+                    acc[T][i & 1] = c;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            st[0] = acc[0][0] + acc[0][1];
+            st[1] = acc[1][0] + acc[1][1];
+        }
+        // ---- running softmax of query row n over this tile's 32 cells (8 here, 24 in the three
+        //      other lanes of the row); causal: row n sees cells up to its own position ----
+        float mx = -INFINITY;
+#pragma unroll
+        for (int T = 0; T < 2; T++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = t0 + 8 * q + 4 * T + i;
+                st[T][i] = (c < c1 && c <= my_row_pos) ? st[T][i] : -INFINITY;
+                mx = fmaxf(mx, st[T][i]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: all weights 0
+        float sum = 0.f;
+        half4_t ph[2], pl[2];
+#pragma unroll
+        for (int T = 0; T < 2; T++) {
+            float pv[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                pv[i] = __expf(st[T][i] - m_use);
+                sum += pv[i];
+            }
+            split4(pv, ph[T], pl[T]);
+        }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        const float alpha = __expf(m_run - m_use);  // 0 while the old max is -inf
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+        // the accumulators hold other rows than this lane's: the factors go through LDS, and are
+        // applied only when some row's maximum moved
+        if (__ballot(alpha != 1.f) != 0ull) {
+            if (q == 0) sm.al[wave][n] = alpha;
+            __builtin_amdgcn_wave_barrier();
+            const float4 af = *reinterpret_cast<const float4 *>(&sm.al[wave][4 * q]);
+            const float av[4] = {af.x, af.y, af.z, af.w};
+#pragma unroll
+            for (int db = 0; db < 16; db++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) o[db][i] *= av[i];
+            __builtin_amdgcn_wave_barrier();
+        }
+        // ---- O += P V: A = P (rows x cells), B = V (cells x dims) ----
+#pragma unroll
+        for (int db = 0; db < 16; db++) {
+            const uint4 v = vreg[db];
+            const half4_t v0 = as_half4(v.x, v.y), v1 = as_half4(v.z, v.w);
+            float4_t acc = o[db];
+            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(ph[0], v0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(pl[0], v0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(ph[1], v1, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x16f16(pl[1], v1, acc, 0, 0, 0);
+            o[db] = acc;
+        }
+    };
+    // the wave's tiles are 4*kTile cells apart; two blocks share a compute unit, one's loads
+    // overlap the other's products
+    constexpr int kStep = 4 * kTile;
+    for (int t0 = t_first; t0 < c1; t0 += kStep) {
+        if (!early || t0 != t_first) load_tile(ta, t0);
+        compute(ta, t0);
+    }
+    // ---- the four waves' results of each sequence row are merged and go to scratch ----
+    if (q == 0) {
+        sm.wm[wave][n] = m_run;
+        sm.wl[wave][n] = l_run;
+    }
+    __syncthreads();  // everyone is done with the queries in sm.qf / sm.big
     float *part_base = a.partial + ((static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits + split) * R * kRec;
 #pragma unroll
     for (int j = 0; j < R; j++) {
-        if (lane < kRep) {
-            sm.wm[wave][lane] = m_run[j];
-            sm.wl[wave][lane] = l_run[j];
-        }
+        // this lane's rows 4q..4q+3 belong to sequence row j when q/2 == j
+        if ((q >> 1) == j) {
 #pragma unroll
-        for (int hh = 0; hh < kRep; hh++)
-            *reinterpret_cast<float4 *>(&sm.big[wave][hh][4 * lane]) = make_float4(acc[j][hh][0], acc[j][hh][1], acc[j][hh][2], acc[j][hh][3]);
+            for (int db = 0; db < 16; db++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) sm.big[wave][(4 * q + i) & 7][16 * db + n] = o[db][i];
+        }
         __syncthreads();
         {
-            // thread = (head, 8 dims) here as in the merge below
-            const int hh = tid >> 5, d0 = (tid & 31) * 8;
-            float M = fmaxf(fmaxf(sm.wm[0][hh], sm.wm[1][hh]), fmaxf(sm.wm[2][hh], sm.wm[3][hh]));
+            // thread = (head, 8 dims)
+            const int hh = tid >> 5, d0 = (tid & 31) * 8, r = 8 * j + hh;
+            float M = fmaxf(fmaxf(sm.wm[0][r], sm.wm[1][r]), fmaxf(sm.wm[2][r], sm.wm[3][r]));
             float w[4], L = 0.f;
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                w[k] = sm.wm[k][hh] == -INFINITY ? 0.f : __expf(sm.wm[k][hh] - M);
-                L = fmaf(w[k], sm.wl[k][hh], L);
+                w[k] = sm.wm[k][r] == -INFINITY ? 0.f : __expf(sm.wm[k][r] - M);
+                L = fmaf(w[k], sm.wl[k][r], L);
             }
             float *rec = part_base + j * kRec + hh * (kD + 2);
 #pragma unroll
@@ -345,31 +358,35 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(shv_attn_decode_arg
     }
 }
 
-// grid: (n_head * 4, R, n_seq), one wave = 64 dims of one head.  The slices' records of that
-// (row, head) are combined with a running max; all of a batch's loads are in flight together.
+// grid: (n_head * 4, R, n_seq), one block = 64 dims of one head; its waves share the slices'
+// records of that (row, head), each folds its share with a running max (all of a batch's loads in
+// flight together), and the first wave folds their results.
+constexpr int kMergeWaves = 8;
 template <int R>
-__global__ __launch_bounds__(64) void attn_merge_kernel(shv_attn_decode_args a, int row0) {
-    const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + threadIdx.x, j = blockIdx.y, seq = blockIdx.z;
+__global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_decode_args a, int row0) {
+    __shared__ float red[3][kMergeWaves][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + lane, j = blockIdx.y, seq = blockIdx.z;
     const int kvh = head / kRep, hh = head % kRep;
     const int n_cells = (a.pos ? a.pos[seq] : 0) + row0 + R;
-    int n_active = (n_cells + kChunk - 1) / kChunk;
+    int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
     if (n_active > a.n_splits) n_active = a.n_splits;
     const float *pin = a.partial + (static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
-    constexpr int MB = 64;
+    constexpr int MB = 16, NW = kMergeWaves;
     float num = 0.f, den = 0.f, M = -INFINITY;
-    for (int s0 = 0; s0 < n_active; s0 += MB) {
+    for (int s0 = wave; s0 < n_active; s0 += NW * MB) {
         float v[MB];
         float2 ml[MB];
 #pragma unroll
         for (int u = 0; u < MB; u++) {
-            const int sidx = s0 + u < n_active ? s0 + u : s0;
+            const int sidx = s0 + NW * u < n_active ? s0 + NW * u : s0;
             const float *rec = pin + static_cast<size_t>(sidx) * R * kRec;
             v[u] = rec[d];
             ml[u] = *reinterpret_cast<const float2 *>(rec + kD);
         }
 #pragma unroll
         for (int u = 0; u < MB; u++) {
-            if (s0 + u >= n_active || ml[u].x == -INFINITY) continue;
+            if (s0 + NW * u >= n_active || ml[u].x == -INFINITY) continue;
             const float Mn = fmaxf(M, ml[u].x);
             const float shrink = __expf(M - Mn), w = __expf(ml[u].x - Mn);  // shrink is 0 while M is -inf
             den = fmaf(den, shrink, w * ml[u].y);
@@ -377,20 +394,30 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(shv_attn_decode_args a, 
             M = Mn;
         }
     }
-    a.out[static_cast<size_t>(seq * a.seq_len + row0 + j) * a.n_head * kD + static_cast<size_t>(head) * kD + d] = num / den;
+    red[0][wave][lane] = M;
+    red[1][wave][lane] = den;
+    red[2][wave][lane] = num;
+    __syncthreads();
+    if (wave != 0) return;
+    float Mt = red[0][0][lane];
+#pragma unroll
+    for (int k = 1; k < NW; k++) Mt = fmaxf(Mt, red[0][k][lane]);
+    float nt = 0.f, dt = 0.f;
+#pragma unroll
+    for (int k = 0; k < NW; k++) {
+        const float mk = red[0][k][lane];
+        const float w = mk == -INFINITY ? 0.f : __expf(mk - Mt);
+        dt = fmaf(w, red[1][k][lane], dt);
+        nt = fmaf(w, red[2][k][lane], nt);
+    }
+    a.out[static_cast<size_t>(seq * a.seq_len + row0 + j) * a.n_head * kD + static_cast<size_t>(head) * kD + d] = nt / dt;
 }
 
 template <int R>
 int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0) {
-    static bool raised = false;
-    if (sizeof(Smem<R>) > 48 * 1024 && !raised) {
-        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_decode_kernel<R>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          static_cast<int>(sizeof(Smem<R>))));
-        raised = true;
-    }
     dim3 grid(a.n_splits, a.n_head_kv, a.n_seq);
-    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), sizeof(Smem<R>), a, row0);
-    SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq), dim3(64), 0, a, row0);
+    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, a, row0);
+    SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq), dim3(64 * kMergeWaves), 0, a, row0);
     return SHV_OK;
 }
 
@@ -407,6 +434,7 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
     SHV_REQUIRE(a.n_seq <= 65535, "attn_decode: %d sequences", a.n_seq);
     SHV_REQUIRE(a.n_splits >= 1 && a.n_splits <= kMaxSplits, "attn_decode: %d slices; 1..%d", a.n_splits, kMaxSplits);
     SHV_REQUIRE(a.qkv_stride >= a.n_head * 2 * kD + 2 * a.n_head_kv * kD, "attn_decode: qkv_stride %d", a.qkv_stride);
+    SHV_REQUIRE(a.max_cells >= kTile && a.max_cells % kTile == 0, "attn_decode: max_cells %d; a multiple of %d", a.max_cells, kTile);
     SHV_REQUIRE(shv_aligned16(a.qkv) && shv_aligned16(a.kcache) && shv_aligned16(a.vcache) && shv_aligned16(a.q_norm) &&
                     shv_aligned16(a.k_norm) && shv_aligned16(a.out) && shv_aligned16(a.partial) && a.qkv_stride % 4 == 0,
                 "attn_decode: qkv, caches, norms, partial and out must be 16-byte aligned");

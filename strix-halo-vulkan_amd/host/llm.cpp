@@ -497,6 +497,8 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
     if (c_.HeadDim != 256) throw Error("llm: AttnGPU: head dimension " + std::to_string(c_.HeadDim) + ", the decode kernel is built for 256");
     if (c_.NHead != 8 * c_.NHeadKV) throw Error("llm: AttnGPU: the decode kernel is built for 8 query heads per KV head");
     if (maxTokens < 1 || nKV < maxTokens || slots < 1) throw Error("llm: AttnGPU: bad token, cell or slot count");
+    n_kv_ = (nKV + 31) & ~31;  // the decode kernel keeps V in tiles of 32 cells
+    nKV = n_kv_;
     SetSplits(0);
     const size_t T = maxTokens;
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
@@ -514,16 +516,17 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
     const size_t cb = static_cast<size_t>(slots) * nKV * c_.NHeadKV * c_.HeadDim * 2;
     for (int l = 0; l < c_.Blocks(); l++) {
         if (only_layer >= 0 ? l != only_layer : (l >= c_.NLayer || !c_.IsAttn(l))) continue;
-        kc_[l] = dev.alloc(cb);
-        vc_[l] = dev.alloc(cb);
+        // zeroed: cells beyond a sequence's end are read (and weighted by zero) with the last tile
+        kc_[l] = dev.alloc_zero(cb);
+        vc_[l] = dev.alloc_zero(cb);
         cache_bytes_ += 2 * cb;
     }
 }
 
 void AttnGPU::SetSplits(int n) {
-    // slices for the cache's capacity: about 64 cells each up to the kernel's limit (the kernel
-    // engages only as many as the sequence's current length fills)
-    if (n <= 0) n = std::min(kMaxSplits, std::max(8, (n_kv_ + 63) / 64));
+    // slices for the cache's capacity: 128 cells each, up to one block a compute unit over the KV
+    // heads (the kernel engages only as many as the sequence's current length fills)
+    if (n <= 0) n = std::min(128, std::max(8, (n_kv_ + 127) / 128));
     if (n > kMaxSplits) throw Error("llm: AttnGPU.SetSplits: at most " + std::to_string(kMaxSplits) + " slices");
     splits_ = n;
 }
@@ -619,8 +622,14 @@ std::vector<uint16_t> AttnGPU::K(int l, int cells, int slot) const {
 
 std::vector<uint16_t> AttnGPU::V(int l, int cells, int slot) const {
     if (l < 0 || l >= c_.Blocks() || !vc_[l] || cells > n_kv_ || slot < 0 || slot >= slots_) throw Error("llm: AttnGPU.V: no such layer, cell or slot");
+    // the device keeps V transposed in tiles of 32 cells, [cell/32][kv head][dim][cell%32]; callers
+    // get the reference's [cell][kv head][dim]
     const size_t per = static_cast<size_t>(c_.NHeadKV) * c_.HeadDim;
-    return read_back<uint16_t>(dev_, static_cast<uint16_t *>(vc_[l]) + static_cast<size_t>(slot) * n_kv_ * per, cells * per);
+    const std::vector<uint16_t> t = read_back<uint16_t>(dev_, static_cast<uint16_t *>(vc_[l]) + static_cast<size_t>(slot) * n_kv_ * per, n_kv_ * per);
+    std::vector<uint16_t> out(static_cast<size_t>(cells) * per);
+    for (int c = 0; c < cells; c++)
+        for (size_t hd = 0; hd < per; hd++) out[static_cast<size_t>(c) * per + hd] = t[(static_cast<size_t>(c / 32) * per + hd) * 32 + c % 32];
+    return out;
 }
 
 // --------------------------------------------------------------------------------- Head -------

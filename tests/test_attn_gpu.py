@@ -76,6 +76,20 @@ class AttnCase:
         ]
 
 
+def v_dev(vc):
+    """the device's V layout, tiles of 32 cells transposed: [..., cell/32, kv head, dim, cell%32] from
+    the reference's [..., cell, kv head, dim]"""
+    lead, (cells, nkv, d) = vc.shape[:-3], vc.shape[-3:]
+    t = vc.reshape(*lead, cells // 32, 32, nkv, d)
+    return np.ascontiguousarray(np.moveaxis(t, -3, -1))
+
+
+def v_host(vt):
+    """back to [..., cell, kv head, dim]"""
+    lead, (blocks, nkv, d, _) = vt.shape[:-4], vt.shape[-4:]
+    return np.ascontiguousarray(np.moveaxis(vt, -1, -3)).reshape(*lead, blocks * 32, nkv, d)
+
+
 def _part_floats(n_seq, n_splits, seq_len=1):
     return n_seq * min(seq_len, 2) * NKV * n_splits * (NH // NKV) * (D + 2)
 
@@ -102,7 +116,7 @@ def test_decode_steps_from_an_empty_cache(ctx):
         assert e_pre <= TOL and e_out <= TOL, (t, e_pre, e_out)
     # the cache the GPU wrote is the oracle's, half for half (norm, rope and rounding agree)
     got_k = d_kc.read(np.uint16, kc.size).reshape(kc.shape)[:T]
-    got_v = d_vc.read(np.uint16, vc.size).reshape(vc.shape)[:T]
+    got_v = v_host(d_vc.read(np.uint16, vc.size).reshape(max_cells // 32, NKV, D, 32))[:T]
     # float32 sums that differ in the last bits round to neighbouring halves now and then: never
     # more than one spacing of halves apart (or 1e-5 near zero), and only on a few percent of cells
     for got, want in ((got_k, kc[:T]), (got_v, vc[:T])):
@@ -126,7 +140,7 @@ def test_rows_of_one_sequence_in_one_call(ctx, past, rows, n_splits):
     vc[:past] = rng.standard_normal((past, NKV, D)).astype(np.float16).view(np.uint16)
     xn = rng.standard_normal((rows, H)).astype(np.float32)
     c = ctx
-    d_kc, d_vc = c.upload(kc), c.upload(vc)
+    d_kc, d_vc = c.upload(kc), c.upload(v_dev(vc))
     want_out, want_pre = case.oracle(xn, past, kc, vc)
     d_qkv, d_ctx, d_out = c.alloc(rows * case.width * 4), c.alloc(rows * NH * D * 4), c.alloc(rows * H * 4)
     d_part = c.alloc(_part_floats(1, n_splits, rows) * 4)
@@ -148,13 +162,13 @@ def test_decode_over_a_prefilled_cache(ctx, past, n_seq, n_splits):
     """BASELINE config 4: cache prefilled with N(0,1) halves; one decode row per slot."""
     case = AttnCase(ctx, seed=1000 + past + n_seq)
     rng = case.rng
-    max_cells = past + 1
+    max_cells = (past + 32) // 32 * 32   # room for the new cell, a multiple of 32
     case.upload(max_cells)
     c = ctx
     xn = rng.standard_normal((n_seq, H)).astype(np.float32)
     kcs = rng.standard_normal((n_seq, max_cells, NKV, D), dtype=np.float32).astype(np.float16).view(np.uint16)
     vcs = rng.standard_normal((n_seq, max_cells, NKV, D), dtype=np.float32).astype(np.float16).view(np.uint16)
-    d_kc, d_vc = c.upload(kcs), c.upload(vcs)
+    d_kc, d_vc = c.upload(kcs), c.upload(v_dev(vcs))
     d_qkv, d_ctx, d_out = c.alloc(n_seq * case.width * 4), c.alloc(n_seq * NH * D * 4), c.alloc(n_seq * H * 4)
     d_part = c.alloc(_part_floats(n_seq, n_splits) * 4)
     d_pos = c.upload(np.full(n_seq, past, np.int32))
@@ -175,7 +189,7 @@ def test_decode_over_a_prefilled_cache(ctx, past, n_seq, n_splits):
 def test_split_count_does_not_change_the_answer(ctx):
     """llm/gpu_attn_cache_test.go:395 (split vs unsplit within 1e-3); here 1e-5."""
     case = AttnCase(ctx, seed=5)
-    past, max_cells = 3000, 3001
+    past, max_cells = 3000, 3008 + 32 - 3008 % 32
     case.upload(max_cells)
     rng, c = case.rng, ctx
     xn = rng.standard_normal((1, H)).astype(np.float32)
@@ -183,7 +197,7 @@ def test_split_count_does_not_change_the_answer(ctx):
     vc = rng.standard_normal((max_cells, NKV, D), dtype=np.float32).astype(np.float16).view(np.uint16)
     outs = []
     for n_splits in (3, 16, 100):
-        d_kc, d_vc = c.upload(kc), c.upload(vc)
+        d_kc, d_vc = c.upload(kc), c.upload(v_dev(vc))
         d_qkv, d_ctx, d_out = c.alloc(case.width * 4), c.alloc(NH * D * 4), c.alloc(H * 4)
         c.dispatch_multi(case.ops(c.upload(xn), d_qkv, d_kc, d_vc, c.alloc(_part_floats(1, n_splits) * 4),
                                   d_ctx, d_out, c.upload(np.array([past], np.int32)), 1, 1, max_cells, n_splits))
