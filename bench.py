@@ -122,17 +122,22 @@ def gemv_rates(m, cfg, A, LA):
     A.check(H.shv_upload(ctx, dx, x.ctypes.data, x.nbytes))
     ops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(w, dx, dy, n, k)) for w in mats]
     arr = (A.Op * len(ops))(*ops)
-    pre = C.c_void_p()
-    A.check(H.shv_prerecord(ctx, arr, len(ops), C.byref(pre)))
     ns = C.c_uint64()
-    A.check(H.shv_prerecorded_submit(ctx, pre, 2, C.byref(ns)))
-    A.check(H.shv_prerecorded_submit(ctx, pre, 10, C.byref(ns)))
+    eager = os.environ.get("LLM_NO_PRERECORD", "")[:1] == "1"  # the profiler cannot follow a replay
+    if eager:
+        A.check(H.shv_dispatch_multi(ctx, arr, len(ops), 2, C.byref(ns), None))
+        A.check(H.shv_dispatch_multi(ctx, arr, len(ops), 10, C.byref(ns), None))
+    else:
+        pre = C.c_void_p()
+        A.check(H.shv_prerecord(ctx, arr, len(ops), C.byref(pre)))
+        A.check(H.shv_prerecorded_submit(ctx, pre, 2, C.byref(ns)))
+        A.check(H.shv_prerecorded_submit(ctx, pre, 10, C.byref(ns)))
+        H.shv_prerecorded_destroy(ctx, pre)
     per = ns.value / (10 * copies) / 1e9
     alg = mat_bytes + k * 4 + n * 4
     out["config1_4096x2048"] = {"us": round(per * 1e6, 3), "GBps": round(alg / per / 1e9, 1),
                                 "frac_hbm_peak": round(alg / per / HBM_PEAK, 4),
                                 "distinct_matrices": int(copies), "rotating_MB": round(copies * mat_bytes / 1e6, 1)}
-    H.shv_prerecorded_destroy(ctx, pre)
     head = next(t for t in m.tensors() if t[0] == "output.weight")
     ops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(head[1], dx, dy, cfg.vocab, k))]
     arr = (A.Op * 1)(*ops)
@@ -190,6 +195,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mtp", action="store_true")
     ap.add_argument("--mtp-rounds", type=int, default=64)
+    ap.add_argument("--prefill-rows", type=int, default=4,
+                    help="prompt rows per pass; 1 (with --no-mtp) sends the prompt through the one-row decode "
+                         "step itself, so that a kernel trace of the run holds decode launches only")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware-counter readings of HBM traffic are scaled by")
@@ -204,8 +212,13 @@ def main():
     nkv = a.prompt + a.warmup + a.steps + 3 * a.mtp_rounds + 64
     # prompt rows go through four at a time; the draft block and the state planes of rewindable
     # 3-row passes are staged for the speculative run and cost the plain decode step nothing
-    cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=4, head_rows=3, speculative=1,
-                    spec_rows=3, nextn=1)
+    if a.prefill_rows < 1 or (a.prefill_rows < 4 and not a.no_mtp):
+        sys.exit("bench.py: --prefill-rows below 4 needs --no-mtp (the speculative leg stages 3-row passes)")
+    if a.no_mtp:
+        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows)
+    else:
+        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows, head_rows=3,
+                        speculative=1, spec_rows=3, nextn=1)
     m = LA.LLM(cfg)
     m.init_synthetic(20260101)
     m.stage()
@@ -248,8 +261,7 @@ def main():
                                "drawn N(0,0.02) and quantised on the device by the reference's quantiser, fp16 KV "
                                "cache, vocab 151936; prompt %d random ids then greedy decode at batch 1"
                                % (cfg.n_layer, a.prompt),
-                   "context_at_end": ctx_len, "prefill": "four rows a pass through the decode kernels (%.1f tok/s, untimed)"
-                                                          % (a.prompt / prefill_s),
+                   "context_at_end": ctx_len, "prefill": "%d rows a pass (%.1f tok/s, untimed)" % (a.prefill_rows, a.prompt / prefill_s),
                    "weights_GB": round(m.weight_bytes() / 1e9, 2), "dispatches_per_step": m.dispatches()},
         "gpu_ms_per_step": round(gpu_ns / a.steps / 1e6, 4),
         "token_bytes": tb, "token_roofline_tok_s": round(HBM_PEAK / tb, 1), "frac_of_token_roofline": round(tok_s * tb / HBM_PEAK, 4),

@@ -82,7 +82,7 @@ __device__ void select_by_rounds(uint32_t *kh, uint32_t *kl, int n_used, int32_t
 // probabilities; the reference adds the exponentials one after another where a tree is used
 // here, which moves only the last bits of a factor common to every probability.
 //
-// Selection: the n_used-th largest of the 64 per-lane maxima bounds the n_used-th largest key from
+// Selection: the n_used-th largest of 16 group maxima bounds the n_used-th largest key from
 // below, so only keys at or above it can be selected.  Those few candidates (found by a bitwise
 // search with wave ballots) are compacted into LDS and ranked against each other.
 // lds: scratch of at least 192 floats.
@@ -121,23 +121,32 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         kl[i] = e < n_expert ? static_cast<uint32_t>(0x7FFFFFFF - e) : 0u;
         lane_max = kh[i] > lane_max ? kh[i] : lane_max;
     }
-    // thr = the n_used-th largest lane maximum.  Every lane ranks its own maximum among the 64
-    // (ties by lane, so the ranks are distinct); the lane of rank n_used-1 holds the threshold.
+    // thr = the n_used-th largest of the 16 maxima of four neighbouring lanes: n_used different
+    // groups hold a key at or above it, so the n_used largest keys all are.  Every lane ranks one
+    // group's maximum among the 16 (ties by group, so the ranks are distinct); the group of rank
+    // n_used-1 holds the threshold.
     uint32_t thr = 0u;
-    if (n_used <= 64) {
+    {
+        uint32_t gm = lane_max;
+        const uint32_t o1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppXor1, 0xF, 0xF, false));
+        gm = o1 > gm ? o1 : gm;
+        const uint32_t o2 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppXor2, 0xF, 0xF, false));
+        gm = o2 > gm ? o2 : gm;
         uint32_t *lm = cand_p;  // the candidate table is not in use yet
-        lm[lane] = lane_max;
+        if ((lane & 3) == 0) lm[lane >> 2] = gm;
         __builtin_amdgcn_wave_barrier();
+        const int grp = lane & 15;
+        const uint32_t mine = lm[grp];
         int rank = 0;
 #pragma unroll
-        for (int j4 = 0; j4 < 16; j4++) {
+        for (int j4 = 0; j4 < 4; j4++) {
             const uint4 o = *reinterpret_cast<const uint4 *>(lm + 4 * j4);
             const uint32_t ov[4] = {o.x, o.y, o.z, o.w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) rank += (ov[j] > lane_max || (ov[j] == lane_max && 4 * j4 + j < lane)) ? 1 : 0;
+            for (int j = 0; j < 4; j++) rank += (ov[j] > mine || (ov[j] == mine && 4 * j4 + j < grp)) ? 1 : 0;
         }
         uint32_t *thr_slot = reinterpret_cast<uint32_t *>(sel_e);
-        if (rank == n_used - 1) *thr_slot = lane_max;
+        if (lane < 16 && rank == n_used - 1) *thr_slot = mine;
         __builtin_amdgcn_wave_barrier();
         thr = *thr_slot;
         __builtin_amdgcn_wave_barrier();
@@ -164,10 +173,13 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         const uint32_t my_p = lane < total ? cand_p[lane] : 0u;
         const int my_e = lane < total ? cand_e[lane] : 0x7FFFFFFF;
         int rank = 0;
-        for (int j = 0; j < total; j++) {
-            const uint32_t op = cand_p[j];
-            const int oe = cand_e[j];
-            rank += (op > my_p || (op == my_p && oe < my_e)) ? 1 : 0;
+        for (int j0 = 0; j0 < total; j0 += 4) {  // four candidates a trip, their reads in flight together
+            const uint4 op4 = *reinterpret_cast<const uint4 *>(cand_p + j0);
+            const int4 oe4 = *reinterpret_cast<const int4 *>(cand_e + j0);
+            const uint32_t op[4] = {op4.x, op4.y, op4.z, op4.w};
+            const int oe[4] = {oe4.x, oe4.y, oe4.z, oe4.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) rank += (j0 + j < total && (op[j] > my_p || (op[j] == my_p && oe[j] < my_e))) ? 1 : 0;
         }
         if (lane < total && rank < n_used) {
             sel_e[rank] = my_e;
@@ -175,8 +187,18 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         }
     }
     __builtin_amdgcn_wave_barrier();
-    float wsum = 0.f;
-    for (int k = 0; k < n_used; k++) wsum += sel_w[k];  // slot order, float32: the reference's sum
+    float wsum = 0.f;  // slot order, float32: the reference's sum
+    {
+        float sw[kMaxUsed];
+#pragma unroll
+        for (int k4 = 0; k4 < kMaxUsed / 4; k4++) {
+            const float4 f = *reinterpret_cast<const float4 *>(sel_w + 4 * k4);
+            sw[4 * k4 + 0] = f.x; sw[4 * k4 + 1] = f.y; sw[4 * k4 + 2] = f.z; sw[4 * k4 + 3] = f.w;
+        }
+#pragma unroll
+        for (int k = 0; k < kMaxUsed; k++)
+            if (k < n_used) wsum += sw[k];
+    }
     if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
     if (lane < n_used) {
         topk[lane] = sel_e[lane];
@@ -244,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
 
 // grid: n_tok blocks of one wave: the selection for one token from its finished logits.
 __global__ __launch_bounds__(64) void moe_route_kernel(shv_moe_router_args a) {
-    __shared__ float probs[192];
+    __shared__ __align__(16) float probs[192];
     const int t = blockIdx.x, lane = threadIdx.x;
     const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
     float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
@@ -261,7 +283,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     __shared__ float xs[lds_padded(K)];
-    __shared__ float probs[192];
+    __shared__ __align__(16) float probs[192];
     __shared__ int32_t s_topk[kMaxUsed];
     __shared__ float s_w[kMaxUsed + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
