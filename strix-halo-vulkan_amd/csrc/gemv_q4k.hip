@@ -30,9 +30,11 @@ struct GemvBatch {
     static constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     uint4 hdr[U], q0[U], q1[U];
     int row[U];
+    float res[U][NT];  // the residual of the rows this lane writes, requested with the weights
 
     // the batch's passes are `stride` apart: pass, pass + stride, ...
-    __device__ __forceinline__ void load(const char *wbase, int g, int rsub, long long pass, long long stride, int n) {
+    __device__ __forceinline__ void load(const shv_gemv_q4k_args &a, const char *wbase, int g, int rsub, int lane, long long pass,
+                                         long long stride, int n, int t0) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const long long r = (pass + u * stride) * RPP + rsub;
@@ -41,6 +43,13 @@ struct GemvBatch {
             hdr[u] = load_stream16(rp);
             q0[u] = load_stream16(rp + 16 + g * 32);
             q1[u] = load_stream16(rp + 32 + g * 32);
+        }
+        if (a.residual) {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    res[u][t] = row[u] >= 0 && group_sum_owner<LPR>(lane) ? a.residual[static_cast<size_t>(t0 + t) * a.y_stride + row[u]] : 0.f;
         }
     }
 
@@ -55,7 +64,7 @@ struct GemvBatch {
                 acc = group_sum<LPR>(acc);
                 if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
                     float r = acc;
-                    if (a.residual) r += a.residual[static_cast<size_t>(t0 + t) * a.y_stride + row[u]];
+                    if (a.residual) r += res[u][t];
                     a.y[y_off[t] + row[u]] = r;
                 }
             }
@@ -86,66 +95,82 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     // The first batch of weights does not depend on the activations: its loads go out before
     // the prologue so that HBM latency and the staging of x overlap.
     GemvBatch<K, NT, U> A, B;
-    A.load(wbase, g, rsub, first_pass, stride, n);
+    A.load(a, wbase, g, rsub, lane, first_pass, stride, n, t0);
+
+    // where each row's ring slot is (its sequence's position and slot): asked for now, used by
+    // the gated-norm prologue or by the final store
+    int ring_row[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        ring_row[t] = 0;
+        if (a.ring_slots > 0) {
+            const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+            const int s = (t0 + t) / sl, i = (t0 + t) % sl;
+            const int p = a.pos ? a.pos[s] : 0;
+            const int slot = a.slot ? a.slot[s] : s;
+            ring_row[t] = slot * a.ring_slots + (p + i) % a.ring_slots;
+        }
+    }
 
     // ---- stage pro(x) in LDS ----
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const float *x = a.x + static_cast<size_t>(t0 + t) * a.x_stride;
         if (a.prologue == SHV_PRO_RMSNORM) {
-            float v[K / kBlock];
+            float v[K / kBlock], gm[K / kBlock];  // gamma is asked for before the block-wide sum, not after it
             float ss = 0.f;
 #pragma unroll
             for (int i = 0; i < K / kBlock; i++) {
                 v[i] = x[tid + i * kBlock];
-                ss = fmaf(v[i], v[i], ss);
+                gm[i] = a.gamma[tid + i * kBlock];
             }
+#pragma unroll
+            for (int i = 0; i < K / kBlock; i++) ss = fmaf(v[i], v[i], ss);
             ss = block_sum_256(ss, red);
             const float scale = 1.f / sqrtf(ss / static_cast<float>(K) + a.eps);
 #pragma unroll
-            for (int i = 0; i < K / kBlock; i++) {
-                const int c = tid + i * kBlock;
-                xs[t][lds_slot(c)] = v[i] * scale * a.gamma[c];
-            }
+            for (int i = 0; i < K / kBlock; i++) xs[t][lds_slot(tid + i * kBlock)] = v[i] * scale * gm[i];
         } else if (a.prologue == SHV_PRO_GATED_NORM) {
             // thread owns K/256 consecutive columns; a head of head_dim columns spans
             // head_dim/(K/256) consecutive threads (a power of two <= 64).
             constexpr int PER = K / kBlock;
             const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
-            if (a.z_ring) {
-                const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
-                const int s = (t0 + t) / sl, i = (t0 + t) % sl;
-                const int p = a.pos ? a.pos[s] : 0;
-                const int slot = a.slot ? a.slot[s] : s;
-                z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
-            }
-            float v[PER];
+            if (a.z_ring) z = a.z + static_cast<size_t>(ring_row[t]) * a.ring_stride;
+            float v[PER], zv[PER], gm[PER];
             float ss = 0.f;
 #pragma unroll
             for (int i = 0; i < PER; i++) {
                 v[i] = x[tid * PER + i];
-                ss = fmaf(v[i], v[i], ss);
+                zv[i] = z[tid * PER + i];
+                gm[i] = a.gamma[(tid * PER + i) % a.head_dim];
             }
+#pragma unroll
+            for (int i = 0; i < PER; i++) ss = fmaf(v[i], v[i], ss);
             const int span = a.head_dim / PER;
             for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
             const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
 #pragma unroll
             for (int i = 0; i < PER; i++) {
                 const int c = tid * PER + i;
-                const float g = 1.f / (1.f + expf(-z[c]));
-                xs[t][lds_slot(c)] = v[i] * scale * a.gamma[c % a.head_dim] * g;
+                const float g = 1.f / (1.f + expf(-zv[i]));
+                xs[t][lds_slot(c)] = v[i] * scale * gm[i] * g;
             }
         } else if (a.prologue == SHV_PRO_RMSNORM_PAIR) {
             // two K/2-wide vectors, each with its own RMS, side by side
             if constexpr (K >= 2 * kBlock) {
                 constexpr int HALF = K / kBlock / 2;
                 const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
-                float v[2 * HALF];
+                float v[2 * HALF], gm[2 * HALF];
                 float s0 = 0.f, s1 = 0.f;
 #pragma unroll
                 for (int i = 0; i < HALF; i++) {
                     v[i] = x[tid + i * kBlock];
                     v[HALF + i] = z[tid + i * kBlock];
+                }
+#pragma unroll
+                for (int i = 0; i < 2 * HALF; i++) gm[i] = a.gamma[tid + i * kBlock];
+#pragma unroll
+                for (int i = 0; i < HALF; i++) {
                     s0 = fmaf(v[i], v[i], s0);
                     s1 = fmaf(v[HALF + i], v[HALF + i], s1);
                 }
@@ -156,7 +181,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 #pragma unroll
                 for (int i = 0; i < 2 * HALF; i++) {
                     const int c = tid + i * kBlock;
-                    xs[t][lds_slot(c)] = v[i] * (i < HALF ? sc0 : sc1) * a.gamma[c];
+                    xs[t][lds_slot(c)] = v[i] * (i < HALF ? sc0 : sc1) * gm[i];
                 }
             }
         } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
@@ -189,11 +214,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         if (a.ring_slots > 0 && !a.z_ring) {
-            const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
-            const int s = (t0 + t) / sl, i = (t0 + t) % sl;
-            const int p = a.pos ? a.pos[s] : 0;
-            const int slot = a.slot ? a.slot[s] : s;
-            y_off[t] = (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
+            y_off[t] = static_cast<size_t>(ring_row[t]) * a.ring_stride;
         } else {
             y_off[t] = static_cast<size_t>(t0 + t) * a.y_stride;
         }
@@ -203,10 +224,10 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     const int nb = n_batches;  // double-buffered
     for (int b = 0; b < nb; b += 2) {
         const bool has_b = b + 1 < nb;
-        if (has_b) B.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 1) * U * stride, stride, n);
+        if (has_b) B.load(a, wbase, g, rsub, lane, first_pass + static_cast<long long>(b + 1) * U * stride, stride, n, t0);
         A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
         if (has_b) {
-            if (b + 2 < nb) A.load(wbase, g, rsub, first_pass + static_cast<long long>(b + 2) * U * stride, stride, n);
+            if (b + 2 < nb) A.load(a, wbase, g, rsub, lane, first_pass + static_cast<long long>(b + 2) * U * stride, stride, n, t0);
             B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
         }
     }

@@ -225,13 +225,15 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
     }
     for (int t = 0; t < a.n_tok; t++) {
         const float *h = a.h + static_cast<size_t>(t) * a.h_stride;
-        float v[H / kBlock];
+        float v[H / kBlock], gm[H / kBlock];  // gamma is asked for before the block-wide sum, not after it
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < H / kBlock; i++) {
             v[i] = h[tid + i * kBlock];
-            ss = fmaf(v[i], v[i], ss);
+            gm[i] = a.gamma ? a.gamma[tid + i * kBlock] : 1.f;
         }
+#pragma unroll
+        for (int i = 0; i < H / kBlock; i++) ss = fmaf(v[i], v[i], ss);
         float scale = 1.f;
         if (a.gamma) {
             ss = block_sum_256(ss, red);
@@ -240,7 +242,7 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
 #pragma unroll
         for (int i = 0; i < H / kBlock; i++) {
             const int c = tid + i * kBlock;
-            const float x = a.gamma ? v[i] * scale * a.gamma[c] : v[i];
+            const float x = a.gamma ? v[i] * scale * gm[i] : v[i];
             xs[c] = x;
             if (blockIdx.x == 0 && a.xn) a.xn[static_cast<size_t>(t) * H + c] = x;
         }
@@ -362,6 +364,9 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
     const int row = blockIdx.x * RPP + rsub;
     const bool live = row < a.n_embd;
     const size_t roff = static_cast<size_t>(live ? row : 0) * ROWB + sb * SHV_Q4K_BYTES;
+    // the residual of the row this thread will write at the end is asked for now
+    float res = 0.f;
+    if (a.residual && tid < RPP && blockIdx.x * RPP + tid < a.n_embd) res = a.residual[static_cast<size_t>(t) * a.res_stride + blockIdx.x * RPP + tid];
 
     Q4kLane w[SPW];
     float wt[SPW];
@@ -425,8 +430,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
         const int r = blockIdx.x * RPP + tid;
         if (r < a.n_embd) {
             float v = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
-            if (a.residual) v += a.residual[static_cast<size_t>(t) * a.res_stride + r];
-            a.out[static_cast<size_t>(t) * a.out_stride + r] = v;
+            a.out[static_cast<size_t>(t) * a.out_stride + r] = v + res;
         }
     }
 }
