@@ -691,6 +691,32 @@ static bool no_prerecord() {
     return e && e[0] == '1';
 }
 
+// In a pass of one or two rows the MoE up projection is told which down banks the op after it
+// will read for the same experts: workgroups added to its launch pull those rows into the L2 of
+// the die that will read them while the kernel's own workgroups compute (touch_down_exps in the
+// kernel interface).  The same hand-over from the down projection to the next block's input
+// projection was measured too and lost as much in the giver as it won in the taker.
+// LLM_TOUCH=0 turns it off, for measurements.
+static bool touch_on() {
+    const char *e = std::getenv("LLM_TOUCH");
+    return !(e && e[0] == '0');
+}
+
+static void wire_touches(std::vector<shv_op> &ops) {
+    if (!touch_on()) return;
+    for (size_t i = 0; i + 1 < ops.size(); i++) {
+        if (ops[i].kind != SHV_OP_MOE_UP || ops[i + 1].kind != SHV_OP_MOE_DOWN) continue;
+        shv_moe_up_args u;
+        shv_moe_down_args d;
+        std::memcpy(&u, ops[i].args, sizeof(u));
+        std::memcpy(&d, ops[i + 1].args, sizeof(d));
+        if (u.n_tok > 2) continue;
+        u.touch_down_exps = d.down_exps;
+        u.touch_down_sh = d.down_sh;
+        std::memcpy(ops[i].args, &u, sizeof(u));
+    }
+}
+
 static uint64_t submit_pass(Device &dev, Pass &p, int iters, const char *what) {
     uint64_t ns = 0;
     if (no_prerecord()) {
@@ -838,6 +864,7 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
             break;
         }
     }
+    wire_touches(p.ops);
     return passes_[key] = std::move(p);
 }
 
