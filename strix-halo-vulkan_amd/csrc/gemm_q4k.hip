@@ -130,11 +130,11 @@ __device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt
             const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
             const float zz[4] = {zv[i].x, zv[i].y, zv[i].z, zv[i].w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) x[j] = x[j] * scale * a.gamma[(c + j) % a.head_dim] * (1.f / (1.f + expf(-zz[j])));
+            for (int j = 0; j < 4; j++) x[j] = x[j] * scale * a.gamma[(c + j) % a.head_dim] * sigmoid_fast(zz[j]);
         } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
             const float zz[4] = {zv[i].x, zv[i].y, zv[i].z, zv[i].w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) x[j] *= 1.f / (1.f + expf(-zz[j]));
+            for (int j = 0; j < 4; j++) x[j] *= sigmoid_fast(zz[j]);
         }
         // the sub-block's sum of x: eight neighbouring lanes
         float sum = on ? (x[0] + x[1]) + (x[2] + x[3]) : 0.f;

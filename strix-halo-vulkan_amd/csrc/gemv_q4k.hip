@@ -138,11 +138,12 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
             if (a.z_ring) z = a.z + static_cast<size_t>(ring_row[t]) * a.ring_stride;
             float v[PER], zv[PER], gm[PER];
             float ss = 0.f;
+            const HeadSplit hs(a.head_dim);
 #pragma unroll
             for (int i = 0; i < PER; i++) {
                 v[i] = x[tid * PER + i];
                 zv[i] = z[tid * PER + i];
-                gm[i] = a.gamma[(tid * PER + i) % a.head_dim];
+                gm[i] = a.gamma[hs.dim(tid * PER + i)];
             }
 #pragma unroll
             for (int i = 0; i < PER; i++) ss = fmaf(v[i], v[i], ss);
@@ -152,8 +153,7 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 #pragma unroll
             for (int i = 0; i < PER; i++) {
                 const int c = tid * PER + i;
-                const float g = 1.f / (1.f + expf(-zv[i]));
-                xs[t][lds_slot(c)] = v[i] * scale * gm[i] * g;
+                xs[t][lds_slot(c)] = v[i] * scale * gm[i] * sigmoid_fast(zv[i]);
             }
         } else if (a.prologue == SHV_PRO_RMSNORM_PAIR) {
             // two K/2-wide vectors, each with its own RMS, side by side
@@ -186,14 +186,19 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
             }
         } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
             const float *z = a.z + static_cast<size_t>(t0 + t) * a.z_stride;
+            const HeadSplit hs(a.head_dim > 0 ? a.head_dim : 1);
+            float v[K / kBlock], zv[K / kBlock];
 #pragma unroll
             for (int i = 0; i < K / kBlock; i++) {
                 const int c = tid + i * kBlock;
                 // head_dim > 0: z rows are [q (head_dim) | gate (head_dim)] per head and the gate
                 // half is the one wanted (the fused query projection, llm/attn.go:162-166)
-                const int zi = a.head_dim > 0 ? (c / a.head_dim) * 2 * a.head_dim + a.head_dim + c % a.head_dim : c;
-                xs[t][lds_slot(c)] = x[c] * (1.f / (1.f + expf(-z[zi])));
+                const int zi = a.head_dim > 0 ? hs.head(c) * 2 * a.head_dim + a.head_dim + hs.dim(c) : c;
+                v[i] = x[c];
+                zv[i] = z[zi];
             }
+#pragma unroll
+            for (int i = 0; i < K / kBlock; i++) xs[t][lds_slot(tid + i * kBlock)] = v[i] * sigmoid_fast(zv[i]);
         } else {
 #pragma unroll
             for (int i = 0; i < K / kBlock; i++) {
@@ -312,7 +317,8 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
                         a.head_dim / per <= 64 && ((a.head_dim / per) & (a.head_dim / per - 1)) == 0,
                     "gemv_q4k: gated-norm head_dim %d does not tile k %d", a.head_dim, a.k);
     }
-    if (a.prologue == SHV_PRO_MUL_SIGMOID) SHV_REQUIRE(a.z, "gemv_q4k: sigmoid-gate prologue without z");
+    if (a.prologue == SHV_PRO_MUL_SIGMOID)
+        SHV_REQUIRE(a.z && a.head_dim >= 0 && (a.head_dim & (a.head_dim - 1)) == 0, "gemv_q4k: sigmoid-gate prologue needs z and a head_dim that is 0 or a power of two (%d)", a.head_dim);
     if (a.z_ring) SHV_REQUIRE(a.prologue == SHV_PRO_GATED_NORM && a.ring_slots > 0, "gemv_q4k: z_ring needs the gated-norm prologue and a ring");
     if (a.ring_slots > 0) {
         const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;

@@ -239,6 +239,20 @@ __device__ __forceinline__ bool arrive_last(int32_t *counter, int expected, int 
 
 __device__ __forceinline__ float sigmoid_exact(float x) { return 1.f / (1.f + expf(-x)); }
 
+// Sigmoid through the hardware exp2 and reciprocal, a few units in the last place from the exact
+// one: for the gates every workgroup of a projection applies to a whole activation vector, where
+// sixteen exact ones a thread were a visible part of the kernel.
+__device__ __forceinline__ float sigmoid_fast(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+
+// i / d and i % d for a head width d that is a power of two (the launchers check): a shift and a
+// mask, and no branch to keep the loads around them from being merged.
+struct HeadSplit {
+    int mask, shift;
+    __device__ __forceinline__ explicit HeadSplit(int head_dim) : mask(head_dim - 1), shift(__ffs(head_dim) - 1) {}
+    __device__ __forceinline__ int head(int i) const { return i >> shift; }
+    __device__ __forceinline__ int dim(int i) const { return i & mask; }
+};
+
 __device__ __forceinline__ float sigmoidf_dev(float x) { return 1.f / (1.f + __expf(-x)); }
 __device__ __forceinline__ float siluf_dev(float x) { return x * sigmoidf_dev(x); }
 
