@@ -199,16 +199,6 @@ typedef struct {
     const float *logits;
     float *weights;
     int32_t n_expert;
-    /* Hint, may be NULL: the down banks the following shv_moe_down will read for these same
-     * experts (n_embd rows of ffn each).  A batch-1 step is a chain of short kernels each waiting
-     * on its own first bytes; the chip's eight dies each have an L2 that keeps its lines from
-     * one kernel to the next, and workgroup i of a launch runs on die i % 8.  Given the banks,
-     * the launch carries one more layer of workgroups that only read one word of every 128-byte
-     * line of those rows, each on the die whose down workgroups will want them.  Results never
-     * depend on it; it is used when topk is an input (logits NULL) and the up grid's first
-     * dimension is a multiple of 8 (ffn 512 at n_embd 2048 is).  No counterpart in the
-     * reference, whose integrated GPU has one cache for everything. */
-    const void *touch_down_exps, *touch_down_sh;
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +

@@ -290,33 +290,6 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     __shared__ float s_w[kMaxUsed + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int slot = blockIdx.y, t = blockIdx.z;
-    if (t == a.n_tok) {
-        // An extra layer of workgroups (launched only with touch_down_exps, without routing from
-        // logits, and with a grid whose x is a multiple of 8, so that this one sits on die
-        // blockIdx.x % 8).  The down projection that follows reads, for this slot's expert,
-        // 64/(ffn/64) rows of n_embd per workgroup, workgroup b on die b % 8: this one pulls the
-        // rows of the b that share its die, the workgroups of one die splitting them, one
-        // 128-byte line a thread.
-        const int rowb_d = a.ffn / SHV_Q4K_BLOCK * SHV_Q4K_BYTES, rpp_d = 64 / (a.ffn / 64);
-        const int lines = rpp_d * rowb_d / 128;       // per down workgroup and slot
-        const int nb8 = (K + rpp_d - 1) / rpp_d / 8;  // down workgroups per die
-        const int per_die = gridDim.x / 8;            // of these workgroups, per slot and die
-        const int j = tid / lines, l = tid % lines;
-        const int m = (blockIdx.x >> 3) + per_die * j;
-        unsigned acc = 0u;
-        if (m < nb8) {
-            const int b = (blockIdx.x & 7) + 8 * m;
-            for (int tt = 0; tt < a.n_tok; tt++) {
-                const char *dbase = static_cast<const char *>(a.touch_down_sh);
-                if (slot < a.n_used)
-                    dbase = static_cast<const char *>(a.touch_down_exps) +
-                            static_cast<size_t>(a.topk[static_cast<size_t>(tt) * a.n_used + slot]) * K * rowb_d;
-                if (dbase) acc ^= *reinterpret_cast<const unsigned *>(dbase + static_cast<size_t>(b) * rpp_d * rowb_d + l * 128);
-            }
-        }
-        asm volatile("" ::"v"(acc));
-        return;
-    }
     const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
     const int row = (blockIdx.x * 4 + wave) * RPP + rsub;  // row within the expert
     const bool live = row < a.ffn;
@@ -499,29 +472,22 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
                 "moe_up: weight banks must be 16-byte aligned");
     dim3 block(kBlock);
-    // the down banks can be touched when their rows come in whole lines per workgroup of the down kernel
-    const bool touch = a.touch_down_exps && !a.logits && a.ffn >= 64 && a.ffn % SHV_Q4K_BLOCK == 0 &&
-                       (64 / (a.ffn / 64)) * (a.ffn / SHV_Q4K_BLOCK * SHV_Q4K_BYTES) % 128 == 0 &&
-                       (64 / (a.ffn / 64)) * (a.ffn / SHV_Q4K_BLOCK * SHV_Q4K_BYTES) / 128 <= kBlock;
     switch (a.n_embd) {
         case 2048: {
             constexpr int RPP = 64 / (2048 / 64);
             dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            if (touch && grid.x % 8 == 0) grid.z += 1;  // the workgroups that only touch the down banks
             SHV_LAUNCH(ctx, moe_up_kernel<2048>, grid, block, 0, a);
             break;
         }
         case 1024: {
             constexpr int RPP = 64 / (1024 / 64);
             dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            if (touch && grid.x % 8 == 0) grid.z += 1;  // the workgroups that only touch the down banks
             SHV_LAUNCH(ctx, moe_up_kernel<1024>, grid, block, 0, a);
             break;
         }
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
             dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            if (touch && grid.x % 8 == 0) grid.z += 1;  // the workgroups that only touch the down banks
             SHV_LAUNCH(ctx, moe_up_kernel<512>, grid, block, 0, a);
             break;
         }

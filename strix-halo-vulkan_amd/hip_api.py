@@ -65,8 +65,7 @@ class MoeUpArgs(C.Structure):
                 ("up_exps", C.c_void_p), ("gate_sh", C.c_void_p), ("up_sh", C.c_void_p),
                 ("act", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("logits", C.c_void_p),
-                ("weights", C.c_void_p), ("n_expert", C.c_int32),
-                ("touch_down_exps", C.c_void_p), ("touch_down_sh", C.c_void_p)]
+                ("weights", C.c_void_p), ("n_expert", C.c_int32)]
 
 
 class MoeDownArgs(C.Structure):

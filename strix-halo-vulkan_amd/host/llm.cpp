@@ -197,8 +197,8 @@ void Model::InitSynthetic(uint64_t seed) {
 MoEGPU::MoEGPU(Device &dev, const Model &m, int maxTokens) : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens) {
     if (maxTokens < 1) throw Error("llm: MoEGPU needs room for at least one token");
     if (c_.NExpertUsed > c_.NExpert) throw Error("llm: MoEGPU: more experts used than there are");
-    // the selection as a dispatch of its own measures the same at one row and better at several
-    if (const char *e = std::getenv("LLM_MOE_ROUTE")) fused_route_ = std::strcmp(e, "fused") == 0;
+    // LLM_MOE_ROUTE=fused|rows|kernel says where the selection runs (rows: fused in one-row passes only)
+    if (const char *e = std::getenv("LLM_MOE_ROUTE")) route_mode_ = std::strcmp(e, "fused") == 0 ? 1 : std::strcmp(e, "rows") == 0 ? 2 : 0;
     const size_t T = maxTokens;
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
@@ -238,7 +238,8 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     r.n_used = c_.NExpertUsed;
     r.eps = c_.RMSEps;
     r.h_stride = c_.NEmbd;
-    r.defer_route = fused_route_ ? 1 : 0;
+    const bool fused = FusedRouter(nTok);
+    r.defer_route = fused ? 1 : 0;
     shv_moe_up_args u{};
     u.xn = xn_;
     u.topk = topk_;
@@ -251,7 +252,7 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     u.n_embd = c_.NEmbd;
     u.n_used = c_.NExpertUsed;
     u.ffn = c_.FFNExpert;
-    if (fused_route_) {
+    if (fused) {
         u.logits = logits_;
         u.weights = weights_;
         u.n_expert = c_.NExpert;
@@ -691,32 +692,6 @@ static bool no_prerecord() {
     return e && e[0] == '1';
 }
 
-// In a pass of one or two rows the MoE up projection is told which down banks the op after it
-// will read for the same experts: workgroups added to its launch pull those rows into the L2 of
-// the die that will read them while the kernel's own workgroups compute (touch_down_exps in the
-// kernel interface).  The same hand-over from the down projection to the next block's input
-// projection was measured too and lost as much in the giver as it won in the taker.
-// LLM_TOUCH=0 turns it off, for measurements.
-static bool touch_on() {
-    const char *e = std::getenv("LLM_TOUCH");
-    return !(e && e[0] == '0');
-}
-
-static void wire_touches(std::vector<shv_op> &ops) {
-    if (!touch_on()) return;
-    for (size_t i = 0; i + 1 < ops.size(); i++) {
-        if (ops[i].kind != SHV_OP_MOE_UP || ops[i + 1].kind != SHV_OP_MOE_DOWN) continue;
-        shv_moe_up_args u;
-        shv_moe_down_args d;
-        std::memcpy(&u, ops[i].args, sizeof(u));
-        std::memcpy(&d, ops[i + 1].args, sizeof(d));
-        if (u.n_tok > 2) continue;
-        u.touch_down_exps = d.down_exps;
-        u.touch_down_sh = d.down_sh;
-        std::memcpy(ops[i].args, &u, sizeof(u));
-    }
-}
-
 static uint64_t submit_pass(Device &dev, Pass &p, int iters, const char *what) {
     uint64_t ns = 0;
     if (no_prerecord()) {
@@ -864,7 +839,6 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
             break;
         }
     }
-    wire_touches(p.ops);
     return passes_[key] = std::move(p);
 }
 
