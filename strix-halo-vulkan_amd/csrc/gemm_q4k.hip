@@ -90,7 +90,8 @@ __device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt
                 z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
             }
             // sigmoid gate with head_dim: z rows are [q | gate] per head and the gate half is wanted
-            const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0 ? (c / a.head_dim) * 2 * a.head_dim + a.head_dim + c % a.head_dim : c;
+            // (head_dim is 0 or a power of two: the launcher of the row kernel checks)
+            const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0 ? (c & ~(a.head_dim - 1)) * 2 + a.head_dim + (c & (a.head_dim - 1)) : c;
             zv[i] = *reinterpret_cast<const float4 *>(z + zi);
         }
     }
@@ -129,8 +130,11 @@ __device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt
             for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
             const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
             const float zz[4] = {zv[i].x, zv[i].y, zv[i].z, zv[i].w};
+            // head_dim is a power of two and a multiple of 4 here: the quad's four gammas are one load
+            const float4 g4 = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
+            const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) x[j] = x[j] * scale * a.gamma[(c + j) % a.head_dim] * sigmoid_fast(zz[j]);
+            for (int j = 0; j < 4; j++) x[j] = x[j] * scale * gg[j] * sigmoid_fast(zz[j]);
         } else if (a.prologue == SHV_PRO_MUL_SIGMOID) {
             const float zz[4] = {zv[i].x, zv[i].y, zv[i].z, zv[i].w};
 #pragma unroll
@@ -324,7 +328,7 @@ int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt) {
     const int slots = ctx->prop.multiProcessorCount * per_cu * NW;
     const int sbs = a.k / SHV_Q4K_BLOCK;
     int ks = 1;
-    while (ks < 4 && ks * 2 <= NW && sbs % (ks * 2) == 0 && n_tiles * ks * 2 <= slots) ks *= 2;
+    while (ks * 2 <= NW && sbs % (ks * 2) == 0 && n_tiles * ks * 2 <= slots) ks *= 2;
     const int tiles_per_block = NW / ks;
     int blocks = ctx->prop.multiProcessorCount * per_cu;
     const int need = (n_tiles + tiles_per_block - 1) / tiles_per_block;
@@ -344,7 +348,7 @@ bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a) {
     if (a.prologue == SHV_PRO_RMSNORM_PAIR) return false;
     if (a.prologue == SHV_PRO_GATED_NORM) {
         const int span = a.head_dim / 4;
-        if (a.head_dim % 4 != 0 || span < 1 || span > 64 || (span & (span - 1)) != 0) return false;
+        if (a.head_dim % 4 != 0 || span < 1 || span > 64 || (span & (span - 1)) != 0 || !shv_aligned16(a.gamma)) return false;
     }
     if (a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim % 4 != 0) return false;
     // 16-byte loads of the activation rows, their gates and the norm's gamma

@@ -273,6 +273,13 @@ int launch_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     const long long resident = static_cast<long long>(ctx->prop.multiProcessorCount) * 2;
     long long blocks = (passes + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > resident) blocks = resident;
+    // Every block stages (and for the gated prologues, transforms) the whole input row, which at
+    // 4096 columns is a visible part of a short kernel: there a wave takes two passes and the
+    // grid is half as many blocks.
+    if (K >= 4096) {
+        const long long half = (passes + 2 * kWavesPerBlock - 1) / (2 * kWavesPerBlock);
+        if (half < blocks) blocks = half;
+    }
     const long long waves = blocks * kWavesPerBlock;
     const long long iters = (passes + waves - 1) / waves;
     const int u = iters < 4 ? static_cast<int>(iters) : 4;
@@ -325,7 +332,7 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
         SHV_REQUIRE((a.z_ring || (a.ring_stride >= a.n && !a.residual)) && sl <= a.ring_slots && a.n_tok % sl == 0,
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
-    if (a.n_tok >= ctx->mfma_min_rows && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
+    if (a.n_tok >= (a.k > 2048 ? ctx->mfma_min_rows_wide : ctx->mfma_min_rows) && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
     switch (a.k) {
         case 512: return launch_k<512>(ctx, a);
         case 1024: return launch_k<1024>(ctx, a);

@@ -172,14 +172,14 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         __builtin_amdgcn_wave_barrier();
         const uint32_t my_p = lane < total ? cand_p[lane] : 0u;
         const int my_e = lane < total ? cand_e[lane] : 0x7FFFFFFF;
+        // rank of candidate j = how many candidates come before it: its key goes round as two
+        // scalars, every lane answers, and the answers are counted (no memory on the way)
         int rank = 0;
-        for (int j0 = 0; j0 < total; j0 += 4) {  // four candidates a trip, their reads in flight together
-            const uint4 op4 = *reinterpret_cast<const uint4 *>(cand_p + j0);
-            const int4 oe4 = *reinterpret_cast<const int4 *>(cand_e + j0);
-            const uint32_t op[4] = {op4.x, op4.y, op4.z, op4.w};
-            const int oe[4] = {oe4.x, oe4.y, oe4.z, oe4.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) rank += (j0 + j < total && (op[j] > my_p || (op[j] == my_p && oe[j] < my_e))) ? 1 : 0;
+        for (int j = 0; j < total; j++) {
+            const uint32_t pj = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_p), j));
+            const int ej = __builtin_amdgcn_readlane(my_e, j);
+            const int before = __popcll(__ballot(my_p > pj || (my_p == pj && my_e < ej)));
+            rank = lane == j ? before : rank;
         }
         if (lane < total && rank < n_used) {
             sel_e[rank] = my_e;
@@ -187,22 +187,15 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
         }
     }
     __builtin_amdgcn_wave_barrier();
-    float wsum = 0.f;  // slot order, float32: the reference's sum
-    {
-        float sw[kMaxUsed];
-#pragma unroll
-        for (int k4 = 0; k4 < kMaxUsed / 4; k4++) {
-            const float4 f = *reinterpret_cast<const float4 *>(sel_w + 4 * k4);
-            sw[4 * k4 + 0] = f.x; sw[4 * k4 + 1] = f.y; sw[4 * k4 + 2] = f.z; sw[4 * k4 + 3] = f.w;
-        }
-#pragma unroll
-        for (int k = 0; k < kMaxUsed; k++)
-            if (k < n_used) wsum += sw[k];
-    }
+    // lane k holds slot k; the sum runs over the slots in order, in float32: the reference's sum
+    const float w_mine = lane < n_used ? sel_w[lane] : 0.f;
+    const int32_t e_mine = lane < n_used ? sel_e[lane] : 0;
+    float wsum = 0.f;
+    for (int k = 0; k < n_used; k++) wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_mine), k));
     if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
     if (lane < n_used) {
-        topk[lane] = sel_e[lane];
-        weights[lane] = sel_w[lane] / wsum;
+        topk[lane] = e_mine;
+        weights[lane] = w_mine / wsum;
     }
 }
 

@@ -40,7 +40,7 @@ int shv_init(int device, shv_ctx **out) {
     ctx->device = device;
     if (const char *e = std::getenv("SHV_MFMA_MIN_ROWS")) {
         const int v = std::atoi(e);
-        if (v >= 2) ctx->mfma_min_rows = v;
+        if (v >= 2) ctx->mfma_min_rows = ctx->mfma_min_rows_wide = v;
     }
     hipError_t e = hipGetDeviceProperties(&ctx->prop, device);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);

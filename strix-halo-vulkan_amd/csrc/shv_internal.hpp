@@ -17,9 +17,12 @@ struct shv_ctx {
     hipDeviceProp_t prop{};
     uint64_t submits = 0;
     bool capturing = false;
-    // Q4_K projections of at least this many rows run on the matrix cores (SHV_MFMA_MIN_ROWS in
-    // the environment overrides it; a large value keeps every pass on the row kernel)
-    int mfma_min_rows = 3;
+    // Q4_K projections of at least this many rows run on the matrix cores: from 3 rows where the
+    // rows are up to 2048 columns, from 5 where they are wider (a 2048x4096 output projection is a
+    // few short launches' worth of bytes, and the row kernel's four rows cost less than staging
+    // operands).  SHV_MFMA_MIN_ROWS in the environment sets both; a large value keeps every pass
+    // on the row kernel.
+    int mfma_min_rows = 3, mfma_min_rows_wide = 5;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
     int32_t *counters = nullptr;
