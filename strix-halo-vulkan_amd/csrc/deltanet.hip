@@ -48,13 +48,19 @@ __device__ __forceinline__ float conv4(const float *ring, int ring_slots, int ri
     return s;
 }
 
-// grid: (128/8 row chunks, n_head_v, n_seq)
+constexpr int kPrep = 8;  // rows of a sequence whose conv, norms and gates are prepared together
+
+// grid: (128/8 row chunks, n_head_v, n_seq).  The rows of a call go in groups of kPrep: first
+// everything that does not depend on the state is worked out for the whole group, all threads
+// busy (a thread keeps the sliding window of its channel's ring values, so a row costs one load);
+// then the waves walk the group's rows with nothing between two rows but their own two
+// reductions.
 __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
-    __shared__ __align__(16) float qs[kD];
-    __shared__ __align__(16) float ks[kD];
-    __shared__ float vs[kRowsPerBlock];
-    __shared__ float red[4];
-    __shared__ float gb[2];
+    __shared__ __align__(16) float qs[kPrep][kD];
+    __shared__ __align__(16) float ks[kPrep][kD];
+    __shared__ float vs[kPrep][kRowsPerBlock];
+    __shared__ float red[kPrep][4];
+    __shared__ float gb[kPrep][2];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
@@ -72,53 +78,81 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
     const size_t plane_floats = static_cast<size_t>(a.n_head_v) * kD * kD;
     float *sslot = a.state + static_cast<size_t>(slot) * planes * plane_floats + (static_cast<size_t>(h) * kD + j) * kD + li * 4;
     float *srow = sslot + cur * plane_floats;
-    float4 s = *reinterpret_cast<const float4 *>(srow);  // in flight while the prologue runs
+    float4 s = *reinterpret_cast<const float4 *>(srow);  // in flight while the first group is prepared
 
     const float *ring = a.ring + static_cast<size_t>(slot) * a.ring_slots * a.ring_stride;
     const float scale = 1.f / sqrtf(static_cast<float>(kD));
+    // q (threads 0..127) and k (128..255) channels of key head hk
+    const int ch = tid < kD ? hk * kD + tid : qk + hk * kD + (tid - kD);
+    const float4 tp = *reinterpret_cast<const float4 *>(a.conv1d + static_cast<size_t>(ch) * 4);
 
-    for (int i = 0; i < a.seq_len; i++) {
-        const int p = pos0 + i;
-        // q (threads 0..127) and k (128..255) channels of key head hk
-        const int ch = tid < kD ? hk * kD + tid : qk + hk * kD + (tid - kD);
-        const float c = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, ch, p);
-        const float act = c * sigmoid_exact(c);
-        const float ss = wave_sum_all(act * act);
-        if (lane == 0) red[wave] = ss;
-        if (tid < kRowsPerBlock) {
-            const int vch = 2 * qk + h * kD + chunk * kRowsPerBlock + tid;
-            const float cv = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, vch, p);
-            vs[tid] = cv * sigmoid_exact(cv);
+    for (int i0 = 0; i0 < a.seq_len; i0 += kPrep) {
+        const int nr = a.seq_len - i0 < kPrep ? a.seq_len - i0 : kPrep;
+        const int p0 = pos0 + i0;
+        // ---- the group's q and k: causal depthwise conv (taps 0..3 meet positions p-3..p; rows
+        //      before the start of the sequence are zero), SiLU, sum of squares per key head ----
+        float x[kPrep + 3];
+        int rs = (p0 + a.ring_slots - 3) % a.ring_slots;  // ring row of position p0 - 3 (the ring holds more than 3 rows)
+#pragma unroll
+        for (int jj = 0; jj < kPrep + 3; jj++) {
+            x[jj] = (jj < nr + 3 && p0 + jj - 3 >= 0) ? ring[static_cast<size_t>(rs) * a.ring_stride + ch] : 0.f;
+            rs = rs + 1 == a.ring_slots ? 0 : rs + 1;
         }
-        if (tid == 64) {
-            const float *row = ring + static_cast<size_t>(p % a.ring_slots) * a.ring_stride;
+        float act[kPrep];
+#pragma unroll
+        for (int r = 0; r < kPrep; r++) {
+            if (r >= nr) break;
+            float c = 0.f;
+            c += x[r] * tp.x;
+            c += x[r + 1] * tp.y;
+            c += x[r + 2] * tp.z;
+            c += x[r + 3] * tp.w;
+            act[r] = c * sigmoid_exact(c);
+            const float ss = wave_sum_all(act[r] * act[r]);
+            if (lane == 0) red[r][wave] = ss;
+        }
+        // this block's eight v channels of each row, and each row's decay and write strength
+        if (tid < nr * kRowsPerBlock) {
+            const int r = tid / kRowsPerBlock, vr = tid % kRowsPerBlock;
+            const int vch = 2 * qk + h * kD + chunk * kRowsPerBlock + vr;
+            const float cv = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, vch, p0 + r);
+            vs[r][vr] = cv * sigmoid_exact(cv);
+        } else if (tid >= 64 && tid < 64 + nr) {
+            const int r = tid - 64;
+            const float *row = ring + static_cast<size_t>((p0 + r) % a.ring_slots) * a.ring_stride;
             const float asp = softplus_ref(row[alpha_off + h] + a.dt_bias[h]);
-            gb[0] = expf(asp * a.a[h]);
-            gb[1] = sigmoid_exact(row[beta_off + h]);
+            gb[r][0] = expf(asp * a.a[h]);
+            gb[r][1] = sigmoid_exact(row[beta_off + h]);
         }
         __syncthreads();
-        {
-            const float ssq = tid < kD ? red[0] + red[1] : red[2] + red[3];
+#pragma unroll
+        for (int r = 0; r < kPrep; r++) {
+            if (r >= nr) break;
+            const float ssq = tid < kD ? red[r][0] + red[r][1] : red[r][2] + red[r][3];
             const float nrm = a.qk_norm_max ? 1.f / fmaxf(sqrtf(ssq), a.eps) : 1.f / sqrtf(ssq + a.eps);
-            if (tid < kD) qs[tid] = act * nrm; else ks[tid - kD] = act * nrm;
+            if (tid < kD) qs[r][tid] = act[r] * nrm; else ks[r][tid - kD] = act[r] * nrm;
         }
         __syncthreads();
-        const float4 k4 = *reinterpret_cast<const float4 *>(ks + li * 4);
-        const float4 q4 = *reinterpret_cast<const float4 *>(qs + li * 4);
-        const float g = gb[0], beta = gb[1], vj = vs[jl];
-        s.x *= g; s.y *= g; s.z *= g; s.w *= g;
-        const float dk = sum32_all(fmaf(s.x, k4.x, fmaf(s.y, k4.y, fmaf(s.z, k4.z, s.w * k4.w))));
-        const float delta = (vj - dk) * beta;
-        s.x = fmaf(delta, k4.x, s.x);
-        s.y = fmaf(delta, k4.y, s.y);
-        s.z = fmaf(delta, k4.z, s.z);
-        s.w = fmaf(delta, k4.w, s.w);
-        const float oq = sum32_all(fmaf(s.x, q4.x, fmaf(s.y, q4.y, fmaf(s.z, q4.z, s.w * q4.w))));
-        if (li == 0)
-            a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j] = oq * scale;
-        // a rewindable pass keeps every prefix: the state after row i goes to its own plane
-        if (a.spec) *reinterpret_cast<float4 *>(sslot + ((cur + 1 + i) % planes) * plane_floats) = s;
-        __syncthreads();
+        // ---- the rule, row after row, the state in registers ----
+        for (int r = 0; r < nr; r++) {
+            const int i = i0 + r;
+            const float4 k4 = *reinterpret_cast<const float4 *>(&ks[r][li * 4]);
+            const float4 q4 = *reinterpret_cast<const float4 *>(&qs[r][li * 4]);
+            const float g = gb[r][0], beta = gb[r][1], vj = vs[r][jl];
+            s.x *= g; s.y *= g; s.z *= g; s.w *= g;
+            const float dk = sum32_all(fmaf(s.x, k4.x, fmaf(s.y, k4.y, fmaf(s.z, k4.z, s.w * k4.w))));
+            const float delta = (vj - dk) * beta;
+            s.x = fmaf(delta, k4.x, s.x);
+            s.y = fmaf(delta, k4.y, s.y);
+            s.z = fmaf(delta, k4.z, s.z);
+            s.w = fmaf(delta, k4.w, s.w);
+            const float oq = sum32_all(fmaf(s.x, q4.x, fmaf(s.y, q4.y, fmaf(s.z, q4.z, s.w * q4.w))));
+            if (li == 0)
+                a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j] = oq * scale;
+            // a rewindable pass keeps every prefix: the state after row i goes to its own plane
+            if (a.spec) *reinterpret_cast<float4 *>(sslot + ((cur + 1 + i) % planes) * plane_floats) = s;
+        }
+        if (i0 + kPrep < a.seq_len) __syncthreads();  // the next group overwrites what the waves just read
     }
     if (!a.spec) *reinterpret_cast<float4 *>(srow) = s;
 }

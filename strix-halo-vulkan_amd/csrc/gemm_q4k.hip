@@ -20,6 +20,7 @@
 // split along its columns (KS waves a tile), whose partial tiles meet in LDS at the end.
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
+#include <cstdlib>
 
 namespace {
 
@@ -366,7 +367,7 @@ int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     for (int t0 = 0; t0 < a.n_tok; t0 += cap) {
         const int nt = a.n_tok - t0 < cap ? a.n_tok - t0 : cap;
         int rc;
-        if (nt <= 4) rc = launch_tt<4, 512, 8>(ctx, a, t0, nt);
+        if (nt <= 4) rc = getenv("SHV_TT4_1024") ? launch_tt<4, 1024, 4>(ctx, a, t0, nt) : launch_tt<4, 512, 8>(ctx, a, t0, nt);
         else if (nt <= 8) rc = launch_tt<8, 512, 16>(ctx, a, t0, nt);
         else rc = launch_tt<16, 1024, 8>(ctx, a, t0, nt);
         if (rc != SHV_OK) return rc;

@@ -1135,6 +1135,25 @@ std::vector<Stage> Graph::ProfileRows(int rows) {
     return fold_stages(p, per, total, nullptr);
 }
 
+// One headless prompt chunk timed op by op; unlike ProfileRows it is a real Extend: the sequence
+// advances by the chunk.
+std::vector<Stage> Graph::ProfileChunk(const std::vector<int32_t> &ids) {
+    const int n = static_cast<int>(ids.size());
+    Seq &q = seq_[slot_];
+    if (n < 1 || n > o_.MaxTokens) throw Error("llm: Graph.ProfileChunk: " + std::to_string(n) + " rows; 1.." + std::to_string(o_.MaxTokens));
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past + n + 1 > o_.NKV) throw Error("llm: Graph.ProfileChunk: " + std::to_string(q.past + n) + " tokens do not fit " + std::to_string(o_.NKV) + " cells");
+    check_ids(ids);
+    dev_.upload(ids_ + slot_ * ids_stride_ + q.past, ids.data(), static_cast<size_t>(n) * 4);
+    put_pos();
+    Pass &p = pass(slot_, n, kPrefill, false);
+    std::vector<uint64_t> per(p.ops.size());
+    uint64_t total = 0;
+    check(shv_dispatch_multi(dev_.ctx(), p.ops.data(), static_cast<int>(p.ops.size()), 1, &total, per.data()), "profile chunk");
+    q.past += n;
+    return fold_stages(p, per, total, nullptr);
+}
+
 // ------------------------------------------------------------------------------ MTPHead -------
 
 MTPHead::MTPHead(Device &dev, const Model &m, HeadGPU &head, int maxTok, int nKV, int slots)

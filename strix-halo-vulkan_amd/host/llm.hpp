@@ -352,6 +352,7 @@ public:
     std::vector<Stage> ProfileStep();
     // GPU time of one `rows`-row verification pass relative to nothing: nanoseconds per op label.
     std::vector<Stage> ProfileRows(int rows);
+    std::vector<Stage> ProfileChunk(const std::vector<int32_t> &ids);
     GraphStats Stats;
     void ResetStats() { Stats = GraphStats(); }
     int Dispatches();

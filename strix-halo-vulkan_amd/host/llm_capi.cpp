@@ -274,6 +274,10 @@ int shvllm_profile_rows(shvllm *h, int rows, char (*labels)[32], uint64_t *nanos
     return guard([&] { stages_out(graph_of(h).ProfileRows(rows), labels, nanos, max, n); });
 }
 
+int shvllm_profile_chunk(shvllm *h, const int32_t *ids, int rows, char (*labels)[32], uint64_t *nanos, int max, int *n) {
+    return guard([&] { stages_out(graph_of(h).ProfileChunk(std::vector<int32_t>(ids, ids + rows)), labels, nanos, max, n); });
+}
+
 static llm::MTPHead &mtp_of(shvllm *h) {
     if (!h || !h->mtp) throw llm::Error("llm: the draft head has not been staged");
     return *h->mtp;

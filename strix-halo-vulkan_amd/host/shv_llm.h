@@ -67,6 +67,8 @@ int shvllm_ids(shvllm *h, int32_t *dst, int max, int *n);
 int shvllm_dn_state_at(shvllm *h, int layer, int slot, int plane, float *dst);
 int shvllm_kv_at(shvllm *h, int layer, int slot, int cells, uint16_t *k, uint16_t *v);
 int shvllm_profile_rows(shvllm *h, int rows, char (*labels)[32], uint64_t *nanos, int max, int *n);
+/* One headless prompt chunk of `rows` ids (at most max_tokens), timed op by op; the sequence advances. */
+int shvllm_profile_chunk(shvllm *h, const int32_t *ids, int rows, char (*labels)[32], uint64_t *nanos, int max, int *n);
 
 /* the draft head (MTPHead) and the greedy speculative loop (Speculator) over the staged graph */
 int shvllm_mtp_stage(shvllm *h, int max_tok, int vocab_prefix);

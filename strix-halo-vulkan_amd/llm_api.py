@@ -87,6 +87,8 @@ def load():
     L.shvllm_kv_at.argtypes = [vp, C.c_int, C.c_int, C.c_int, u16p, u16p]
     L.shvllm_profile_rows.argtypes = [vp, C.c_int, C.POINTER(C.c_char * 32), C.POINTER(C.c_uint64), C.c_int,
                                       C.POINTER(C.c_int)]
+    L.shvllm_profile_chunk.argtypes = [vp, i32p, C.c_int, C.POINTER(C.c_char * 32), C.POINTER(C.c_uint64), C.c_int,
+                                       C.POINTER(C.c_int)]
     L.shvllm_mtp_stage.argtypes = [vp, C.c_int, C.c_int]
     L.shvllm_mtp_rows.argtypes = [vp, f32p, i32p, C.c_int, C.c_int, C.c_int, f32p, f32p]
     L.shvllm_spec_start.argtypes = [vp, i32p, C.c_int, i32p]
@@ -276,6 +278,15 @@ class LLM:
         ns = (C.c_uint64 * 64)()
         n = C.c_int()
         _check(self.L.shvllm_profile_rows(self.h, rows, labels, ns, 64, C.byref(n)))
+        return [(labels[i].value.decode(), ns[i]) for i in range(n.value)]
+
+    def profile_chunk(self, ids):
+        """One headless prompt chunk timed op by op; the sequence advances by the chunk."""
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        labels = (C.c_char * 32 * 64)()
+        ns = (C.c_uint64 * 64)()
+        n = C.c_int()
+        _check(self.L.shvllm_profile_chunk(self.h, ids.ctypes.data_as(C.POINTER(C.c_int32)), len(ids), labels, ns, 64, C.byref(n)))
         return [(labels[i].value.decode(), ns[i]) for i in range(n.value)]
 
     # ---- draft head and speculative loop ----
