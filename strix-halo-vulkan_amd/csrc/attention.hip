@@ -94,15 +94,19 @@ struct Smem {
     float kv_tmp[2][kD];
 };
 
-// grid: (n_splits, n_head_kv, n_seq); rows row0..row0+R-1 of each sequence.  Query row r of the
+// grid: (n_splits, n_head_kv, n_seq * n_groups); group g of a sequence is its rows row0 + R*g ..
+// row0 + R*g + R-1.  With append the launch also writes its rows' cells (one group only: a later
+// group would read cells another block is still writing); without, the cells are there already
+// and any number of groups go in one launch, each masked to its own positions.  Query row r of the
 // tile is head r%8 of sequence row r/8; with R = 1 rows 8..15 are padding.
 template <int R>
-__global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_args a, int row0) {
+__global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_args a, int row00, int n_groups, int append) {
     __shared__ Smem sm;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+    const int split = blockIdx.x, kvh = blockIdx.y;
+    const int seq = blockIdx.z / n_groups, row0 = row00 + R * (blockIdx.z % n_groups);
     const int slot = a.slot ? a.slot[seq] : seq;
-    const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the launch's first row
+    const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the group's first row
     const int n_cells = p_first + R;                       // cells the last row sees
     // The grid is sized for the cache's capacity; how many of its slices take part depends on how
     // many cells the sequence holds now: about kSliceCells a slice while there are slices to spare.
@@ -172,7 +176,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
             for (int i = 0; i < 2; i++)
                 norm_rope_loaded(qv[i], a.q_norm, rope_row, a.rope_dims, a.eps, qtmp + (8 * j + wave * 2 + i) * kD, lane);
         }
-        if (p >= c0 && p < c1) {
+        if (append && p >= c0 && p < c1) {
             // the new cell of row j lies in this slice: one wave appends its K, all threads its V
             if (wave == ((2 * j) & 3)) {
                 const float *ksrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD;
@@ -320,7 +324,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
         sm.wl[wave][n] = l_run;
     }
     __syncthreads();  // everyone is done with the queries in sm.qf / sm.big
-    float *part_base = a.partial + ((static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits + split) * R * kRec;
+    float *part_base = a.partial + ((static_cast<size_t>(blockIdx.z) * a.n_head_kv + kvh) * a.n_splits + split) * R * kRec;
 #pragma unroll
     for (int j = 0; j < R; j++) {
         // this lane's rows 4q..4q+3 belong to sequence row j when q/2 == j
@@ -358,20 +362,21 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
     }
 }
 
-// grid: (n_head * 4, R, n_seq), one block = 64 dims of one head; its waves share the slices'
+// grid: (n_head * 4, R, n_seq * n_groups), one block = 64 dims of one head; its waves share the slices'
 // records of that (row, head), each folds its share with a running max (all of a batch's loads in
 // flight together), and the first wave folds their results.
 constexpr int kMergeWaves = 8;
 template <int R>
-__global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_decode_args a, int row0) {
+__global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_decode_args a, int row00, int n_groups) {
     __shared__ float red[3][kMergeWaves][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + lane, j = blockIdx.y, seq = blockIdx.z;
+    const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + lane, j = blockIdx.y;
+    const int seq = blockIdx.z / n_groups, row0 = row00 + R * (blockIdx.z % n_groups);
     const int kvh = head / kRep, hh = head % kRep;
     const int n_cells = (a.pos ? a.pos[seq] : 0) + row0 + R;
     int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
     if (n_active > a.n_splits) n_active = a.n_splits;
-    const float *pin = a.partial + (static_cast<size_t>(seq) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
+    const float *pin = a.partial + (static_cast<size_t>(blockIdx.z) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
     constexpr int MB = 16, NW = kMergeWaves;
     float num = 0.f, den = 0.f, M = -INFINITY;
     for (int s0 = wave; s0 < n_active; s0 += NW * MB) {
@@ -413,11 +418,35 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_d
     a.out[static_cast<size_t>(seq * a.seq_len + row0 + j) * a.n_head * kD + static_cast<size_t>(head) * kD + d] = nt / dt;
 }
 
+// grid: (n_head_kv, seq_len, n_seq): the cells of every row of a pass, written before any of
+// them is read: K normed and rotated by the first wave, V transposed into its tile by all threads.
+__global__ __launch_bounds__(kBlock) void attn_append_kernel(shv_attn_decode_args a) {
+    __shared__ float ktmp[kD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.x, row = blockIdx.y, seq = blockIdx.z;
+    const int slot = a.slot ? a.slot[seq] : seq;
+    const int p = (a.pos ? a.pos[seq] : 0) + row;
+    const int kvw = a.n_head_kv * kD;
+    uint16_t *kc = static_cast<uint16_t *>(a.kcache) + static_cast<size_t>(slot) * a.max_cells * kvw + kvh * kD;
+    uint16_t *vt = static_cast<uint16_t *>(a.vcache) + static_cast<size_t>(slot) * a.max_cells * kvw + static_cast<size_t>(kvh) * kD * kTile;
+    const size_t vtile = static_cast<size_t>(kvw) * kTile;
+    const float *qkv = a.qkv + static_cast<size_t>(seq * a.seq_len + row) * a.qkv_stride;
+    if (wave == 0) {
+        const float *ksrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD;
+        norm_rope_head(ksrc, a.k_norm, a.rope + static_cast<size_t>(p) * a.rope_dims, a.rope_dims, a.eps, ktmp, lane);
+        uint16_t *dst = kc + static_cast<size_t>(p) * kvw;
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(ktmp[4 * lane + i]));
+    }
+    const float *vsrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvw + kvh * kD;
+    vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vsrc[tid]));
+}
+
 template <int R>
-int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0) {
-    dim3 grid(a.n_splits, a.n_head_kv, a.n_seq);
-    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, a, row0);
-    SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq), dim3(64 * kMergeWaves), 0, a, row0);
+int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_groups, int append) {
+    dim3 grid(a.n_splits, a.n_head_kv, a.n_seq * n_groups);
+    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, a, row0, n_groups, append);
+    SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, a, row0, n_groups);
     return SHV_OK;
 }
 
@@ -438,10 +467,14 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
     SHV_REQUIRE(shv_aligned16(a.qkv) && shv_aligned16(a.kcache) && shv_aligned16(a.vcache) && shv_aligned16(a.q_norm) &&
                     shv_aligned16(a.k_norm) && shv_aligned16(a.out) && shv_aligned16(a.partial) && a.qkv_stride % 4 == 0,
                 "attn_decode: qkv, caches, norms, partial and out must be 16-byte aligned");
-    // the rows of a sequence go two at a time: both see one pass over the cache
-    for (int i = 0; i < a.seq_len; i += 2) {
-        const int rc = a.seq_len - i >= 2 ? launch_rows<2>(ctx, a, i) : launch_rows<1>(ctx, a, i);
-        if (rc != SHV_OK) return rc;
-    }
-    return SHV_OK;
+    // The rows of a sequence go two at a time: both see one pass over the cache.  One or two rows
+    // write their own cells on the way; more rows have all their cells written first and then go
+    // through as pairs of one launch (and a single last row of another).
+    if (a.seq_len <= 2) return a.seq_len == 2 ? launch_rows<2>(ctx, a, 0, 1, 1) : launch_rows<1>(ctx, a, 0, 1, 1);
+    const int pairs = a.seq_len / 2;
+    SHV_REQUIRE(static_cast<long long>(a.n_seq) * pairs <= 65535, "attn_decode: %d sequences of %d rows in one call", a.n_seq, a.seq_len);
+    SHV_LAUNCH(ctx, attn_append_kernel, dim3(a.n_head_kv, a.seq_len, a.n_seq), dim3(kBlock), 0, a);
+    int rc = launch_rows<2>(ctx, a, 0, pairs, 0);
+    if (rc == SHV_OK && (a.seq_len & 1)) rc = launch_rows<1>(ctx, a, a.seq_len - 1, 1, 0);
+    return rc;
 }

@@ -91,7 +91,7 @@ def v_host(vt):
 
 
 def _part_floats(n_seq, n_splits, seq_len=1):
-    return n_seq * min(seq_len, 2) * NKV * n_splits * (NH // NKV) * (D + 2)
+    return n_seq * (seq_len + (seq_len & 1)) * NKV * n_splits * (NH // NKV) * (D + 2)
 
 
 def test_decode_steps_from_an_empty_cache(ctx):
