@@ -195,7 +195,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mtp", action="store_true")
     ap.add_argument("--mtp-rounds", type=int, default=64)
-    ap.add_argument("--prefill-rows", type=int, default=4,
+    ap.add_argument("--prefill-rows", type=int, default=64,
                     help="prompt rows per pass; 1 (with --no-mtp) sends the prompt through the one-row decode "
                          "step itself, so that a kernel trace of the run holds decode launches only")
     ap.add_argument("--pmc-copy", action="store_true",

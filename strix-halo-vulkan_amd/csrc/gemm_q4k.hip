@@ -20,7 +20,6 @@
 // split along its columns (KS waves a tile), whose partial tiles meet in LDS at the end.
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
-#include <cstdlib>
 
 namespace {
 
@@ -60,6 +59,7 @@ struct Lds {
     // fragment (sub-block s, chunk c, part p) is 4*TT entries of 8 bytes: entry kb*TT + token
     static __host__ __device__ constexpr size_t frag_bytes(int k) { return static_cast<size_t>(k / 32) * 4 * (4 * TT * 8); }
     static __host__ __device__ constexpr size_t sx_bytes(int k) { return static_cast<size_t>(k / 32) * TT * 4; }
+    static __host__ __device__ constexpr size_t region(int k) { return frag_bytes(k) + sx_bytes(k); }  // what a pre-staged pass hands over
     static __host__ __device__ constexpr size_t total(int k, int waves) {
         return frag_bytes(k) + sx_bytes(k) + static_cast<size_t>(waves) * 64 * 16 /* tiles or reductions */ + TT * 8;
     }
@@ -167,8 +167,27 @@ __device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt
 
 // grid: blocks of NTHR/64 waves.  KS consecutive waves share a row tile, each over 1/KS of the
 // columns.  t0: first activation row of this launch, nt: how many (<= TT).
+// The activations of rows blockIdx.x*cap .. +cap-1 transformed once, for a pass of many rows:
+// staged in LDS exactly as a block of the product kernel would, then copied out to `staged`, one
+// region of Lds<TT>::region(k) bytes per group of rows.
 template <int TT, int NTHR, int MAXQ>
-__global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int t0, int nt, int n_tiles, int ks) {
+__global__ __launch_bounds__(NTHR) void gemm_stage_kernel(shv_gemv_q4k_args a, char *staged, int cap) {
+    extern __shared__ __align__(16) char smem[];
+    char *frags = smem;
+    float *sxs = reinterpret_cast<float *>(smem + Lds<TT>::frag_bytes(a.k));
+    float *red = sxs + a.k / 32 * TT;
+    const int t0 = blockIdx.x * cap;
+    const int nt = a.n_tok - t0 < cap ? a.n_tok - t0 : cap;
+    stage<TT, NTHR, MAXQ>(a, t0, nt, frags, sxs, red);
+    __syncthreads();
+    const size_t region = Lds<TT>::region(a.k);
+    uint4 *dst = reinterpret_cast<uint4 *>(staged + blockIdx.x * region);
+    const uint4 *src = reinterpret_cast<const uint4 *>(smem);
+    for (size_t i = threadIdx.x; i < region / 16; i += NTHR) dst[i] = src[i];
+}
+
+template <int TT, int NTHR, int MAXQ>
+__global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int t0, int nt, int n_tiles, int ks, const char *staged) {
     extern __shared__ __align__(16) char smem[];
     constexpr int NW = NTHR / 64;
     char *frags = smem;
@@ -210,7 +229,15 @@ __global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int
         }
         yoffs[tid] = off;
     }
-    stage<TT, NTHR, MAXQ>(a, t0, nt, frags, sxs, ytile);
+    if (staged) {
+        // the operands were made once for the whole pass: every block copies its rows' region
+        const size_t region = Lds<TT>::region(a.k);
+        const uint4 *src = reinterpret_cast<const uint4 *>(staged);
+        uint4 *dst = reinterpret_cast<uint4 *>(smem);
+        for (size_t i = tid; i < region / 16; i += NTHR) dst[i] = src[i];
+    } else {
+        stage<TT, NTHR, MAXQ>(a, t0, nt, frags, sxs, ytile);
+    }
     __syncthreads();
 
     const NibbleConsts nc = nibble_consts();
@@ -310,7 +337,7 @@ __global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int
 }
 
 template <int TT, int NTHR, int MAXQ>
-int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt) {
+int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const char *staged) {
     constexpr int NW = NTHR / 64;
     SHV_REQUIRE(nt * (a.k / 4) <= MAXQ * NTHR, "gemm_q4k: %d rows of %d columns are more than one block stages", nt, a.k);
     const int n_tiles = (a.n + kTileRows - 1) / kTileRows;
@@ -336,7 +363,23 @@ int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt) {
     if (blocks > need) blocks = need;
     const int rounds = (need + blocks - 1) / blocks;
     blocks = (need + rounds - 1) / rounds;
-    SHV_LAUNCH(ctx, (gemm_q4k_kernel<TT, NTHR, MAXQ>), dim3(blocks), dim3(NTHR), lds, a, t0, nt, n_tiles, ks);
+    SHV_LAUNCH(ctx, (gemm_q4k_kernel<TT, NTHR, MAXQ>), dim3(blocks), dim3(NTHR), lds, a, t0, nt, n_tiles, ks, staged);
+    return SHV_OK;
+}
+
+// Every group of `cap` rows of the pass transformed once into ctx->gemm_stage.
+template <int TT, int NTHR, int MAXQ>
+int launch_stage(shv_ctx *ctx, const shv_gemv_q4k_args &a, int cap) {
+    const int groups = (a.n_tok + cap - 1) / cap;
+    const size_t lds = Lds<TT>::total(a.k, NTHR / 64);
+    SHV_REQUIRE(groups * Lds<TT>::region(a.k) <= static_cast<size_t>(shv_ctx::kGemmStageBytes), "gemm_q4k: %d rows of %d columns do not fit the staging buffer", a.n_tok, a.k);
+    static size_t raised = 0;
+    if (lds > 48 * 1024 && lds > raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_stage_kernel<TT, NTHR, MAXQ>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        raised = lds;
+    }
+    SHV_LAUNCH(ctx, (gemm_stage_kernel<TT, NTHR, MAXQ>), dim3(groups), dim3(NTHR), lds, a, ctx->gemm_stage, cap);
     return SHV_OK;
 }
 
@@ -364,12 +407,30 @@ bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a) {
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     // the fragments of 16 rows of 4096 columns do not fit LDS: such a pass goes 8 rows at a time
     const int cap = a.k > 2048 ? 8 : 16;
-    for (int t0 = 0; t0 < a.n_tok; t0 += cap) {
-        const int nt = a.n_tok - t0 < cap ? a.n_tok - t0 : cap;
+    // A pass of several groups of rows, or of wide rows, has its activations transformed once, by
+    // a launch of its own, instead of by every block of the products (hundreds of them): the
+    // groups of `cap` rows are staged with the tile size their product will use.  One group of
+    // narrow rows is cheaper staged by the blocks themselves than by another launch.
+    const bool pre = ctx->gemm_stage && a.n_tok > 4 && (a.n_tok > cap || a.k > 2048);
+    if (pre) {
         int rc;
-        if (nt <= 4) rc = getenv("SHV_TT4_1024") ? launch_tt<4, 1024, 4>(ctx, a, t0, nt) : launch_tt<4, 512, 8>(ctx, a, t0, nt);
-        else if (nt <= 8) rc = launch_tt<8, 512, 16>(ctx, a, t0, nt);
-        else rc = launch_tt<16, 1024, 8>(ctx, a, t0, nt);
+        if (cap == 8 || a.n_tok <= 8) rc = launch_stage<8, 512, 16>(ctx, a, a.n_tok <= 8 ? 8 : cap);
+        else rc = launch_stage<16, 1024, 8>(ctx, a, cap);
+        if (rc != SHV_OK) return rc;
+    }
+    const int gcap = pre && a.n_tok <= 8 ? 8 : cap;
+    for (int t0 = 0; t0 < a.n_tok; t0 += gcap) {
+        const int nt = a.n_tok - t0 < gcap ? a.n_tok - t0 : gcap;
+        int rc;
+        if (!pre) {
+            if (nt <= 4) rc = launch_tt<4, 1024, 4>(ctx, a, t0, nt, nullptr);
+            else if (nt <= 8) rc = launch_tt<8, 512, 16>(ctx, a, t0, nt, nullptr);
+            else rc = launch_tt<16, 1024, 8>(ctx, a, t0, nt, nullptr);
+        } else if (gcap == 8) {
+            rc = launch_tt<8, 512, 16>(ctx, a, t0, nt, ctx->gemm_stage + static_cast<size_t>(t0 / gcap) * Lds<8>::region(a.k));
+        } else {
+            rc = launch_tt<16, 1024, 8>(ctx, a, t0, nt, ctx->gemm_stage + static_cast<size_t>(t0 / gcap) * Lds<16>::region(a.k));
+        }
         if (rc != SHV_OK) return rc;
     }
     return SHV_OK;

@@ -199,16 +199,20 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
     }
 }
 
-// grid: ceil((n_expert+1)/4) blocks of 4 waves, one float32 router row per wave.
+// grid: (ceil((n_expert+1)/4), ceil(n_tok/kRouterTokens)) blocks of 4 waves, one float32 router
+// row per wave, kRouterTokens tokens per block.  Tokens go through in groups of kRouterGroup: one
+// set of block-wide waits per group, not per token.
+constexpr int kRouterGroup = 4;
+constexpr int kRouterTokens = 4;
 template <int H>
 __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args a) {
-    __shared__ float xs[H];
-    __shared__ float red[4];
+    __shared__ __align__(16) float xs[kRouterGroup][H];
+    __shared__ float red[kRouterGroup][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = blockIdx.x * 4 + wave;  // n_expert = the shared-gate row
     const bool has_row = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
-    // the wave's router row is in flight while the first token is being normalised, and stays in
-    // registers for every token
+    // the wave's router row is in flight while the first tokens are being normalised, and stays
+    // in registers for every token
     float4 wrow[H / 256];
     {
         const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
@@ -216,46 +220,74 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
         for (int i = 0; i < H / 256; i++)
             wrow[i] = has_row ? *reinterpret_cast<const float4 *>(w + (i * 64 + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    for (int t = 0; t < a.n_tok; t++) {
-        const float *h = a.h + static_cast<size_t>(t) * a.h_stride;
-        float v[H / kBlock], gm[H / kBlock];  // gamma is asked for before the block-wide sum, not after it
-        float ss = 0.f;
+    float gm[H / kBlock];  // gamma is asked for before the block-wide sums, not after them
 #pragma unroll
-        for (int i = 0; i < H / kBlock; i++) {
-            v[i] = h[tid + i * kBlock];
-            gm[i] = a.gamma ? a.gamma[tid + i * kBlock] : 1.f;
+    for (int i = 0; i < H / kBlock; i++) gm[i] = a.gamma ? a.gamma[tid + i * kBlock] : 1.f;
+
+    const int t_first = blockIdx.y * kRouterTokens;
+    const int t_end = t_first + kRouterTokens < a.n_tok ? t_first + kRouterTokens : a.n_tok;
+    // a group's rows are asked for while the group before it is being multiplied
+    float v[kRouterGroup][H / kBlock];
+    auto fetch = [&](int t0) {
+        const int ng = t_end - t0 < kRouterGroup ? t_end - t0 : kRouterGroup;
+#pragma unroll
+        for (int g = 0; g < kRouterGroup; g++) {
+            if (g >= ng) break;
+            const float *h = a.h + static_cast<size_t>(t0 + g) * a.h_stride;
+#pragma unroll
+            for (int i = 0; i < H / kBlock; i++) v[g][i] = h[tid + i * kBlock];
         }
-#pragma unroll
-        for (int i = 0; i < H / kBlock; i++) ss = fmaf(v[i], v[i], ss);
-        float scale = 1.f;
+    };
+    fetch(t_first);
+    for (int t0 = t_first; t0 < t_end; t0 += kRouterGroup) {
+        const int ng = t_end - t0 < kRouterGroup ? t_end - t0 : kRouterGroup;
         if (a.gamma) {
-            ss = block_sum_256(ss, red);
-            scale = 1.f / sqrtf(ss / static_cast<float>(H) + a.eps);
-        }
 #pragma unroll
-        for (int i = 0; i < H / kBlock; i++) {
-            const int c = tid + i * kBlock;
-            const float x = a.gamma ? v[i] * scale * gm[i] : v[i];
-            xs[c] = x;
-            if (blockIdx.x == 0 && a.xn) a.xn[static_cast<size_t>(t) * H + c] = x;
-        }
-        __syncthreads();
-        if (has_row) {
-            float acc = 0.f;
+            for (int g = 0; g < kRouterGroup; g++) {
+                if (g >= ng) break;
+                float ss = 0.f;
 #pragma unroll
-            for (int i = 0; i < H / 256; i++) {
-                const int c = (i * 64 + lane) * 4;
-                const float4 wv = wrow[i];
-                const float4 xv = *reinterpret_cast<const float4 *>(xs + c);
-                acc = fmaf(wv.x, xv.x, acc);
-                acc = fmaf(wv.y, xv.y, acc);
-                acc = fmaf(wv.z, xv.z, acc);
-                acc = fmaf(wv.w, xv.w, acc);
+                for (int i = 0; i < H / kBlock; i++) ss = fmaf(v[g][i], v[g][i], ss);
+                ss = wave_sum_all(ss);
+                if (lane == 0) red[g][wave] = ss;
             }
-            acc = wave_sum_all(acc);
-            if (lane == 0) a.logits[static_cast<size_t>(t) * (a.n_expert + 1) + row] = acc;
+            __syncthreads();
+        }
+#pragma unroll
+        for (int g = 0; g < kRouterGroup; g++) {
+            if (g >= ng) break;
+            float scale = 1.f;
+            if (a.gamma) scale = 1.f / sqrtf(((red[g][0] + red[g][1]) + (red[g][2] + red[g][3])) / static_cast<float>(H) + a.eps);
+#pragma unroll
+            for (int i = 0; i < H / kBlock; i++) {
+                const int c = tid + i * kBlock;
+                const float x = a.gamma ? v[g][i] * scale * gm[i] : v[g][i];
+                xs[g][c] = x;
+                if (blockIdx.x == 0 && a.xn) a.xn[static_cast<size_t>(t0 + g) * H + c] = x;
+            }
         }
         __syncthreads();
+        if (t0 + kRouterGroup < t_end) fetch(t0 + kRouterGroup);
+        if (has_row) {
+#pragma unroll
+            for (int g = 0; g < kRouterGroup; g++) {
+                if (g >= ng) break;
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < H / 256; i++) {
+                    const int c = (i * 64 + lane) * 4;
+                    const float4 wv = wrow[i];
+                    const float4 xv = *reinterpret_cast<const float4 *>(&xs[g][c]);
+                    acc = fmaf(wv.x, xv.x, acc);
+                    acc = fmaf(wv.y, xv.y, acc);
+                    acc = fmaf(wv.z, xv.z, acc);
+                    acc = fmaf(wv.w, xv.w, acc);
+                }
+                acc = wave_sum_all(acc);
+                if (lane == 0) a.logits[static_cast<size_t>(t0 + g) * (a.n_expert + 1) + row] = acc;
+            }
+        }
+        if (t0 + kRouterGroup < t_end) __syncthreads();
     }
 }
 
@@ -439,11 +471,12 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed && a.n_used <= a.n_expert, "moe_router: n_used %d of %d (at most %d)", a.n_used, a.n_expert, kMaxUsed);
     SHV_REQUIRE(a.h_stride >= a.n_embd, "moe_router: h_stride %d < n_embd %d", a.h_stride, a.n_embd);
     SHV_REQUIRE(shv_aligned16(a.router) && shv_aligned16(a.shared_gate), "moe_router: router and shared_gate must be 16-byte aligned");
-    const unsigned blocks = static_cast<unsigned>((a.n_expert + 1 + 3) / 4);
+    const dim3 blocks((a.n_expert + 1 + 3) / 4, (a.n_tok + kRouterTokens - 1) / kRouterTokens);
+    SHV_REQUIRE(blocks.y <= 65535, "moe_router: n_tok %d", a.n_tok);
     switch (a.n_embd) {
-        case 2048: SHV_LAUNCH(ctx, moe_router_kernel<2048>, dim3(blocks), dim3(kBlock), 0, a); break;
-        case 1024: SHV_LAUNCH(ctx, moe_router_kernel<1024>, dim3(blocks), dim3(kBlock), 0, a); break;
-        case 512: SHV_LAUNCH(ctx, moe_router_kernel<512>, dim3(blocks), dim3(kBlock), 0, a); break;
+        case 2048: SHV_LAUNCH(ctx, moe_router_kernel<2048>, blocks, dim3(kBlock), 0, a); break;
+        case 1024: SHV_LAUNCH(ctx, moe_router_kernel<1024>, blocks, dim3(kBlock), 0, a); break;
+        case 512: SHV_LAUNCH(ctx, moe_router_kernel<512>, blocks, dim3(kBlock), 0, a); break;
         default: return shv_set_error(SHV_E_INVALID, "moe_router: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
     }
     // the selection needs every logit of the token, i.e. the whole grid above: a second, tiny

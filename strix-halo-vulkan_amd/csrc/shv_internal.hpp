@@ -27,6 +27,10 @@ struct shv_ctx {
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
     int32_t *counters = nullptr;
     int n_counters = 0;
+    // activations of a many-row projection, transformed once into matrix-core operand order and
+    // copied from here by every block (kGemmStageBytes covers 64 rows of 4096 columns)
+    char *gemm_stage = nullptr;
+    enum { kGemmStageBytes = 2 << 20 };
     // per-block partial results of the arg-max reduction: (value, index) pairs
     float *argmax_val = nullptr;
     int32_t *argmax_idx = nullptr;
