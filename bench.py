@@ -209,7 +209,7 @@ def main():
         sys.exit("bench.py: --steps and --warmup must be at least 1")
     pkg = importlib.import_module("strix-halo-vulkan_amd")
     LA, A = pkg.llm_api, pkg.hip_api
-    nkv = a.prompt + a.warmup + a.steps + 3 * a.mtp_rounds + 64
+    nkv = a.prompt + a.warmup + a.steps + 3 * a.mtp_rounds + 64 + a.prefill_rows
     # prompt rows go through four at a time; the draft block and the state planes of rewindable
     # 3-row passes are staged for the speculative run and cost the plain decode step nothing
     if a.prefill_rows < 1 or (a.prefill_rows < 4 and not a.no_mtp):
@@ -269,6 +269,21 @@ def main():
         "roofline": roof,
         "gemv": gemv_rates(m, cfg, A, LA),
     }
+    # one prompt chunk timed op by op (on a second sequence slot's worth of cells past the decoded
+    # tokens): where a many-row pass spends its time, and what the expert kernels reach once a
+    # launch carries enough bytes
+    if a.prefill_rows >= 16 and ctx_len + a.prefill_rows + 1 <= cfg.nkv:
+        st = dict(m.profile_chunk(rng.integers(0, cfg.vocab, size=a.prefill_rows).astype(np.int32)))
+        rows = a.prefill_rows
+        per_tok_up = (cfg.n_expert_used + 1) * 2 * cfg.ffn_expert * Q4K_ROW(cfg.n_embd)
+        per_tok_down = (cfg.n_expert_used + 1) * cfg.n_embd * Q4K_ROW(cfg.ffn_expert)
+        chunk_us = sum(v for k, v in st.items() if k != "total") / 1e3
+        rec["prefill_chunk"] = {
+            "rows": rows, "us": round(chunk_us, 1), "tok_s": round(rows / chunk_us * 1e6, 1),
+            "op_us": {k: round(v / 1e3, 1) for k, v in sorted(st.items(), key=lambda kv: -kv[1]) if k != "total"},
+            # every row reads its own experts: rows x (10 routed + shared) x rows of the banks
+            "moe_up_GBps": round(rows * per_tok_up * cfg.n_layer / (st["moe.up"] / 1e9) / 1e9, 1),
+            "moe_down_GBps": round(rows * per_tok_down * cfg.n_layer / (st["moe.down"] / 1e9) / 1e9, 1)}
     if a.pmc_copy:
         import ctypes as C
         H = A.load()
