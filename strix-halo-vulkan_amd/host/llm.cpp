@@ -470,6 +470,38 @@ void DeltaNetGPU::SetState(int l, const std::vector<float> &s, int slot, int pla
     dev_.upload(state_[l] + (static_cast<size_t>(slot) * planes_ + plane) * n, s.data(), n * 4);
 }
 
+size_t DeltaNetGPU::CarriedLen() const {
+    size_t layers = 0;
+    for (int l = 0; l < c_.NLayer; l++) layers += state_[l] ? 1 : 0;
+    return layers * (static_cast<size_t>(c_.SSMHeadV) * c_.SSMHeadDim * c_.SSMHeadDim + 3 * static_cast<size_t>(c_.DNFusedRows()));
+}
+
+void DeltaNetGPU::SaveCarried(float *dst, int slot, int plane, int past) const {
+    if (slot < 0 || slot >= slots_ || plane < 0 || plane >= planes_) throw Error("llm: DeltaNetGPU.SaveCarried: no such slot or plane");
+    const size_t n = static_cast<size_t>(c_.SSMHeadV) * c_.SSMHeadDim * c_.SSMHeadDim, row = c_.DNFusedRows();
+    for (int l = 0; l < c_.NLayer; l++) {
+        if (!state_[l]) continue;
+        dev_.download(dst, state_[l] + (static_cast<size_t>(slot) * planes_ + plane) * n, n * 4);
+        dst += n;
+        for (int j = 3; j >= 1; j--, dst += row) {  // positions past-3, past-2, past-1; zero before the start
+            if (past - j < 0) std::fill(dst, dst + row, 0.f);
+            else dev_.download(dst, ring_[l] + (static_cast<size_t>(slot) * ring_slots_ + (past - j) % ring_slots_) * row, row * 4);
+        }
+    }
+}
+
+void DeltaNetGPU::RestoreCarried(const float *src, int slot, int plane, int past) {
+    if (slot < 0 || slot >= slots_ || plane < 0 || plane >= planes_) throw Error("llm: DeltaNetGPU.RestoreCarried: no such slot or plane");
+    const size_t n = static_cast<size_t>(c_.SSMHeadV) * c_.SSMHeadDim * c_.SSMHeadDim, row = c_.DNFusedRows();
+    for (int l = 0; l < c_.NLayer; l++) {
+        if (!state_[l]) continue;
+        dev_.upload(state_[l] + (static_cast<size_t>(slot) * planes_ + plane) * n, src, n * 4);
+        src += n;
+        for (int j = 3; j >= 1; j--, src += row)
+            if (past - j >= 0) dev_.upload(ring_[l] + (static_cast<size_t>(slot) * ring_slots_ + (past - j) % ring_slots_) * row, src, row * 4);
+    }
+}
+
 std::vector<float> DeltaNetGPU::Result() const { return read_back<float>(dev_, attn_, static_cast<size_t>(n_tok_) * c_.VWidth()); }
 std::vector<float> DeltaNetGPU::Out() const { return read_back<float>(dev_, out_, static_cast<size_t>(n_tok_) * c_.NEmbd); }
 
@@ -1133,6 +1165,32 @@ std::vector<Stage> Graph::ProfileRows(int rows) {
     check(shv_dispatch_multi(dev_.ctx(), p.ops.data(), static_cast<int>(p.ops.size()), 1, &total, per.data()), "profile rows");
     put_pos();  // discarded: the position goes back, the committed plane never moved
     return fold_stages(p, per, total, nullptr);
+}
+
+void Graph::Checkpoint(struct Checkpoint &c) {
+    const Seq &q = seq_[slot_];
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past == 0) throw Error("llm: nothing to checkpoint at position 0");
+    c.past = q.past;
+    c.ids.resize(q.past);
+    dev_.download(c.ids.data(), ids_ + slot_ * ids_stride_, static_cast<size_t>(q.past) * 4);
+    c.dn.resize(dn_->CarriedLen());
+    dn_->SaveCarried(c.dn.data(), slot_, q.plane, q.past);
+}
+
+void Graph::Restore(const struct Checkpoint &c) {
+    Seq &q = seq_[slot_];
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    bool same = c.past > 0 && c.past <= q.past && static_cast<int>(c.ids.size()) == c.past && c.dn.size() == dn_->CarriedLen();
+    if (same) {
+        std::vector<int32_t> have(c.past);
+        dev_.download(have.data(), ids_ + slot_ * ids_stride_, static_cast<size_t>(c.past) * 4);
+        same = have == c.ids;
+    }
+    if (!same) throw Error("llm: this slot no longer holds the checkpoint's tokens");
+    dn_->RestoreCarried(c.dn.data(), slot_, q.plane, c.past);
+    q.past = c.past;
+    put_pos();
 }
 
 // One headless prompt chunk timed op by op; unlike ProfileRows it is a real Extend: the sequence

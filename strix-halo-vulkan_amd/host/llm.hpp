@@ -199,6 +199,12 @@ public:
     void SetState(int layer, const std::vector<float> &s, int slot = 0, int plane = 0);
     int Planes() const { return planes_; }
     int RingSlots() const { return ring_slots_; }
+    // What a sequence carries from one token to the next (DeltaNetGPU.CarriedLen / SaveCarried /
+    // RestoreCarried, llm/gpu_deltanet.go): per DeltaNet layer the committed state plane and the
+    // three projection rows before position `past` that the causal conv will still read.
+    size_t CarriedLen() const;
+    void SaveCarried(float *dst, int slot, int plane, int past) const;
+    void RestoreCarried(const float *src, int slot, int plane, int past);
     std::vector<float> Result() const;  // [T][hv*d] attention output before the gated norm
     std::vector<float> Out() const;     // [T][NEmbd]
     float *InPort() const { return in_; }
@@ -302,6 +308,14 @@ struct Pass {
     shv_prerecorded *rec = nullptr;
 };
 
+// llm.Checkpoint (llm/graph.go:902-1003): a sequence's position, tokens and DeltaNet carry, in host
+// memory; the KV cells need no copy, the ones past the checkpoint are simply written again.
+struct Checkpoint {
+    int past = 0;
+    std::vector<int32_t> ids;
+    std::vector<float> dn;
+};
+
 // llm.Graph (llm/graph.go:184-289, NewGraph :609): the whole model as recorded op sequences, one
 // per (slot, row count, kind of pass), recorded the first time each is needed.
 class Graph {
@@ -347,6 +361,11 @@ public:
     void KeepFirst() { Keep(1); }
     void Commit();
     void Rewind();
+    // Checkpoint saves the live slot's sequence into `into` (llm/graph.go:1004-1031); Restore takes
+    // the slot back to it and refuses unless the slot's sequence still starts with the
+    // checkpoint's tokens (:1037-1062).  Neither may run while a rewindable pass is in flight.
+    void Checkpoint(struct Checkpoint &into);
+    void Restore(const struct Checkpoint &c);
     // One decode step dispatched op by op with a GPU time per op, folded by label
     // (DispatchMultiMarked + recorder.submit, vk/engine.go:913, llm/record.go:217-232).
     std::vector<Stage> ProfileStep();

@@ -240,6 +240,23 @@ int shvllm_keep(shvllm *h, int k) {
 int shvllm_commit(shvllm *h) {
     return guard([&] { graph_of(h).Commit(); });
 }
+int shvllm_checkpoint(shvllm *h, shvllm_checkpoint_t **out) {
+    return guard([&] {
+        auto c = std::make_unique<llm::Checkpoint>();
+        graph_of(h).Checkpoint(*c);
+        *out = reinterpret_cast<shvllm_checkpoint_t *>(c.release());
+    });
+}
+
+int shvllm_restore(shvllm *h, const shvllm_checkpoint_t *c) {
+    return guard([&] {
+        if (!c) throw llm::Error("llm: no checkpoint");
+        graph_of(h).Restore(*reinterpret_cast<const llm::Checkpoint *>(c));
+    });
+}
+
+void shvllm_checkpoint_free(shvllm_checkpoint_t *c) { delete reinterpret_cast<llm::Checkpoint *>(c); }
+
 int shvllm_rewind(shvllm *h) {
     return guard([&] { graph_of(h).Rewind(); });
 }

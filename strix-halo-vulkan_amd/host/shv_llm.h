@@ -61,6 +61,13 @@ int shvllm_speculate(shvllm *h, int on);
 int shvllm_speculate_first(shvllm *h, int on);
 int shvllm_keep(shvllm *h, int k);
 int shvllm_commit(shvllm *h);
+/* Graph.Checkpoint / Restore (llm/graph.go:1004-1062): the live slot's position, tokens and
+ * DeltaNet carry saved to host memory, and the slot taken back to them (refused unless its
+ * sequence still starts with the checkpoint's tokens). */
+typedef struct shvllm_checkpoint shvllm_checkpoint_t;
+int shvllm_checkpoint(shvllm *h, shvllm_checkpoint_t **out);
+int shvllm_restore(shvllm *h, const shvllm_checkpoint_t *c);
+void shvllm_checkpoint_free(shvllm_checkpoint_t *c);
 int shvllm_rewind(shvllm *h);
 int shvllm_plane(shvllm *h);
 int shvllm_ids(shvllm *h, int32_t *dst, int max, int *n);

@@ -87,6 +87,10 @@ def load():
     L.shvllm_kv_at.argtypes = [vp, C.c_int, C.c_int, C.c_int, u16p, u16p]
     L.shvllm_profile_rows.argtypes = [vp, C.c_int, C.POINTER(C.c_char * 32), C.POINTER(C.c_uint64), C.c_int,
                                       C.POINTER(C.c_int)]
+    L.shvllm_checkpoint.argtypes = [vp, C.POINTER(vp)]
+    L.shvllm_restore.argtypes = [vp, vp]
+    L.shvllm_checkpoint_free.argtypes = [vp]
+    L.shvllm_checkpoint_free.restype = None
     L.shvllm_profile_chunk.argtypes = [vp, i32p, C.c_int, C.POINTER(C.c_char * 32), C.POINTER(C.c_uint64), C.c_int,
                                        C.POINTER(C.c_int)]
     L.shvllm_mtp_stage.argtypes = [vp, C.c_int, C.c_int]
@@ -279,6 +283,18 @@ class LLM:
         n = C.c_int()
         _check(self.L.shvllm_profile_rows(self.h, rows, labels, ns, 64, C.byref(n)))
         return [(labels[i].value.decode(), ns[i]) for i in range(n.value)]
+
+    def checkpoint(self):
+        """Graph.Checkpoint: an opaque handle to the live slot's saved sequence (free with checkpoint_free)."""
+        c = C.c_void_p()
+        _check(self.L.shvllm_checkpoint(self.h, C.byref(c)))
+        return c
+
+    def restore(self, c):
+        _check(self.L.shvllm_restore(self.h, c))
+
+    def checkpoint_free(self, c):
+        self.L.shvllm_checkpoint_free(c)
 
     def profile_chunk(self, ids):
         """One headless prompt chunk timed op by op; the sequence advances by the chunk."""

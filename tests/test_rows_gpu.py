@@ -270,3 +270,54 @@ def test_speculative_loop_emits_the_greedy_sequence(rig, mode):
     # the trunk holds exactly the emitted tokens but the pending one
     assert m.past() == len(prompt) + len(out) - 1
     assert list(m.ids()) == list(prompt) + out[:-1]
+
+
+def test_checkpoint_restore_is_the_shorter_sequence(rig):
+    """Graph.Checkpoint / Restore (llm/graph.go:1004-1062): after going on past a checkpoint and
+    coming back, the sequence continues exactly as one that never went on; a slot that no longer
+    starts with the checkpoint's tokens is refused, and so is a pass in flight."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(77)
+    head, tail, other = (rng.integers(0, cfg.vocab, size=n).astype(np.int32) for n in (7, 5, 6))
+    fresh(m)
+    for t in head:
+        m.extend(np.array([t], np.int32), want_logits=False)
+    c = m.checkpoint()
+    for t in other:  # the conversation goes somewhere else ...
+        m.extend(np.array([t], np.int32), want_logits=False)
+    m.restore(c)     # ... and comes back
+    assert m.past() == len(head)
+    got = [m.extend(np.array([t], np.int32))[0] for t in tail]
+    state = m.dn_state(0)
+    fresh(m)
+    for t in head:
+        m.extend(np.array([t], np.int32), want_logits=False)
+    want = [m.extend(np.array([t], np.int32))[0] for t in tail]
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)  # same kernels on the same bytes
+    assert np.array_equal(state, m.dn_state(0))
+    # against the CPU too
+    om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+    lg_cpu, _ = om.extend(np.concatenate([head, tail]))
+    assert O.rel_l2(got[-1], lg_cpu) <= 1e-3
+    # a second restore from the same checkpoint, after a chunked continuation
+    m.extend(other)
+    m.restore(c)
+    lg, _ = m.extend(tail)
+    assert O.rel_l2(lg, lg_cpu) <= 1e-3
+    # refusals
+    fresh(m)
+    m.extend(other)
+    with pytest.raises(shv.api.ShvError, match="no longer holds"):
+        m.restore(c)
+    fresh(m)
+    with pytest.raises(shv.api.ShvError, match="nothing to checkpoint"):
+        m.checkpoint()
+    m.extend(head)
+    m.speculate(True)
+    m.extend_rows(tail[:2])
+    with pytest.raises(shv.api.ShvError, match="in flight"):
+        m.checkpoint()
+    m.rewind()
+    m.speculate(False)
+    m.checkpoint_free(c)
