@@ -203,6 +203,27 @@ def mtp_run(m, cfg, prompt, plain, acc, rounds):
     return out
 
 
+def batched_run(m, cfg, n_slots, rng, prompt_len=256, steps=48):
+    """Several sequences advanced one token each per pass (Graph.DecodeRows): the projections
+    read their weights once for all of them, on the matrix cores from five rows."""
+    m.speculate(False)
+    for s in range(n_slots):
+        m.use_slot(s)
+        m.reset()
+        m.extend(rng.integers(0, cfg.vocab, size=prompt_len).astype(np.int32), want_logits=False)
+    slots = np.arange(n_slots, dtype=np.int32)
+    ids = rng.integers(0, cfg.vocab, size=n_slots).astype(np.int32)
+    for _ in range(4):
+        ids, _ = m.decode_rows(slots, ids)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ids, _ = m.decode_rows(slots, ids)   # each pass: upload ids, run, download the arg-maxes
+    dt = time.perf_counter() - t0
+    m.use_slot(0)
+    return {"slots": n_slots, "context": prompt_len + 4 + steps, "ms_per_pass": round(dt / steps * 1e3, 4),
+            "tok_s": round(n_slots * steps / dt, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -214,6 +235,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mtp", action="store_true")
     ap.add_argument("--mtp-rounds", type=int, default=64)
+    ap.add_argument("--batch-slots", type=int, default=8,
+                    help="sequences of the batched-decode leg (one token each per pass); 0 skips it")
     ap.add_argument("--prefill-rows", type=int, default=64,
                     help="prompt rows per pass; 1 (with --no-mtp) sends the prompt through the one-row decode "
                          "step itself, so that a kernel trace of the run holds decode launches only")
@@ -236,8 +259,8 @@ def main():
     if a.no_mtp:
         cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows)
     else:
-        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows, head_rows=3,
-                        speculative=1, spec_rows=3, nextn=1)
+        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows,
+                        head_rows=max(3, a.batch_slots), slots=max(1, a.batch_slots), speculative=1, spec_rows=3, nextn=1)
     m = LA.LLM(cfg)
     m.init_synthetic(20260101)
     m.stage()
@@ -319,6 +342,8 @@ def main():
         rounds = min(a.mtp_rounds, (len(plain) - 4) // 3)
         if rounds >= 1:
             rec["mtp"] = mtp_run(m, cfg, prompt, plain, acc, rounds)
+    if not a.no_mtp and a.batch_slots >= 2:
+        rec["batched_decode"] = batched_run(m, cfg, a.batch_slots, rng)
     if not a.no_cpu:
         rec["cpu_baseline"] = cpu_baseline(m, cfg, LA, a.cpu_tokens)
     m.close()

@@ -167,23 +167,88 @@ __device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt
 
 // grid: blocks of NTHR/64 waves.  KS consecutive waves share a row tile, each over 1/KS of the
 // columns.  t0: first activation row of this launch, nt: how many (<= TT).
-// The activations of rows blockIdx.x*cap .. +cap-1 transformed once, for a pass of many rows:
-// staged in LDS exactly as a block of the product kernel would, then copied out to `staged`, one
-// region of Lds<TT>::region(k) bytes per group of rows.
-template <int TT, int NTHR, int MAXQ>
-__global__ __launch_bounds__(NTHR) void gemm_stage_kernel(shv_gemv_q4k_args a, char *staged, int cap) {
-    extern __shared__ __align__(16) char smem[];
-    char *frags = smem;
-    float *sxs = reinterpret_cast<float *>(smem + Lds<TT>::frag_bytes(a.k));
-    float *red = sxs + a.k / 32 * TT;
-    const int t0 = blockIdx.x * cap;
+// The activations of a pass of many rows transformed once, for every block of the products to
+// copy.  grid: (k/256, groups of `cap` rows), 256 threads: a block takes one super-block's worth of
+// columns of its group's rows, a wave one row's 64 quads at a time, and writes fragments and sums
+// straight into the group's region of `staged` (Lds<TT>::region(k) bytes, laid out as the product
+// kernel lays out its LDS).  The per-row scale of the RMSNorm prologue needs the whole row: each
+// wave adds up the rows it will serve, in a fixed order.
+template <int TT>
+__global__ __launch_bounds__(256) void gemm_stage_kernel(shv_gemv_q4k_args a, char *staged, int cap) {
+    __shared__ float scale_s[TT];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.k, kp = blockIdx.x, grp = blockIdx.y;
+    const int t0 = grp * cap;
     const int nt = a.n_tok - t0 < cap ? a.n_tok - t0 : cap;
-    stage<TT, NTHR, MAXQ>(a, t0, nt, frags, sxs, red);
-    __syncthreads();
-    const size_t region = Lds<TT>::region(a.k);
-    uint4 *dst = reinterpret_cast<uint4 *>(staged + blockIdx.x * region);
-    const uint4 *src = reinterpret_cast<const uint4 *>(smem);
-    for (size_t i = threadIdx.x; i < region / 16; i += NTHR) dst[i] = src[i];
+    char *frags = staged + static_cast<size_t>(grp) * Lds<TT>::region(K);
+    float *sxs = reinterpret_cast<float *>(frags + Lds<TT>::frag_bytes(K));
+    const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+    if (a.prologue == SHV_PRO_RMSNORM) {
+        for (int tl = wave; tl < nt; tl += 4) {
+            const float *x = a.x + static_cast<size_t>(t0 + tl) * a.x_stride;
+            float ss = 0.f;
+            for (int q = lane; q < K / 4; q += 64) {
+                const float4 v = *reinterpret_cast<const float4 *>(x + 4 * q);
+                ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+            }
+            ss = wave_sum_all(ss);
+            if (lane == 0) scale_s[tl] = 1.f / sqrtf(ss / static_cast<float>(K) + a.eps);
+        }
+        __syncthreads();
+    }
+    for (int tl = wave; tl < nt; tl += 4) {
+        const int t = t0 + tl, c = kp * 256 + 4 * lane;
+        const float4 v = *reinterpret_cast<const float4 *>(a.x + static_cast<size_t>(t) * a.x_stride + c);
+        float x[4] = {v.x, v.y, v.z, v.w};
+        if (a.prologue == SHV_PRO_RMSNORM) {
+            const float scale = scale_s[tl];
+            const float4 g = *reinterpret_cast<const float4 *>(a.gamma + c);
+            x[0] *= scale * g.x; x[1] *= scale * g.y; x[2] *= scale * g.z; x[3] *= scale * g.w;
+        } else if (a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID) {
+            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+            if (a.z_ring) {
+                const int s = t / sl, k = t % sl;
+                const int p = a.pos ? a.pos[s] : 0;
+                const int slot = a.slot ? a.slot[s] : s;
+                z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
+            }
+            const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0 ? (c & ~(a.head_dim - 1)) * 2 + a.head_dim + (c & (a.head_dim - 1)) : c;
+            const float4 zq = *reinterpret_cast<const float4 *>(z + zi);
+            const float zz[4] = {zq.x, zq.y, zq.z, zq.w};
+            if (a.prologue == SHV_PRO_GATED_NORM) {
+                float ss = fmaf(x[0], x[0], fmaf(x[1], x[1], fmaf(x[2], x[2], x[3] * x[3])));
+                const int span = a.head_dim / 4;  // lanes a head spans: a power of two up to 64
+                for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
+                const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
+                const float4 g4 = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
+                const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) x[j] = x[j] * scale * gg[j] * sigmoid_fast(zz[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) x[j] *= sigmoid_fast(zz[j]);
+            }
+        }
+        // the sub-block's sum of x: eight neighbouring lanes
+        float sum = (x[0] + x[1]) + (x[2] + x[3]);
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        sum += __shfl_xor(sum, 4, 64);
+        const int sub = c >> 5, kb = (c & 31) >> 3, chunk = (c & 7) >> 2;
+        if ((c & 31) == 0) sxs[sub * TT + tl] = sum;
+        // k order of levels(): [x0, x2, x1, x3]
+        const float o[4] = {x[0], x[2], x[1], x[3]};
+        half4_t h, l;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const _Float16 hi = static_cast<_Float16>(o[j]);
+            h[j] = hi;
+            l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+        }
+        char *e = frags + (static_cast<size_t>((sub * 2 + chunk) * 2) * (4 * TT) + kb * TT + tl) * 8;
+        *reinterpret_cast<half4_t *>(e) = h;
+        *reinterpret_cast<half4_t *>(e + 4 * TT * 8) = l;
+    }
 }
 
 template <int TT, int NTHR, int MAXQ>
@@ -368,18 +433,11 @@ int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const ch
 }
 
 // Every group of `cap` rows of the pass transformed once into ctx->gemm_stage.
-template <int TT, int NTHR, int MAXQ>
+template <int TT>
 int launch_stage(shv_ctx *ctx, const shv_gemv_q4k_args &a, int cap) {
     const int groups = (a.n_tok + cap - 1) / cap;
-    const size_t lds = Lds<TT>::total(a.k, NTHR / 64);
     SHV_REQUIRE(groups * Lds<TT>::region(a.k) <= static_cast<size_t>(shv_ctx::kGemmStageBytes), "gemm_q4k: %d rows of %d columns do not fit the staging buffer", a.n_tok, a.k);
-    static size_t raised = 0;
-    if (lds > 48 * 1024 && lds > raised) {
-        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_stage_kernel<TT, NTHR, MAXQ>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = lds;
-    }
-    SHV_LAUNCH(ctx, (gemm_stage_kernel<TT, NTHR, MAXQ>), dim3(groups), dim3(NTHR), lds, a, ctx->gemm_stage, cap);
+    SHV_LAUNCH(ctx, (gemm_stage_kernel<TT>), dim3(a.k / 256, groups), dim3(256), 0, a, ctx->gemm_stage, cap);
     return SHV_OK;
 }
 
@@ -410,12 +468,13 @@ int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     // A pass of several groups of rows, or of wide rows, has its activations transformed once, by
     // a launch of its own, instead of by every block of the products (hundreds of them): the
     // groups of `cap` rows are staged with the tile size their product will use.  One group of
-    // narrow rows is cheaper staged by the blocks themselves than by another launch.
-    const bool pre = ctx->gemm_stage && a.n_tok > 4 && (a.n_tok > cap || a.k > 2048);
+    // narrow rows is cheaper staged by the blocks themselves, under their first weight loads.
+    const bool pre = ctx->gemm_stage && a.n_tok > 4 && (a.n_tok > cap || a.k > 2048) &&
+                     (a.prologue != SHV_PRO_GATED_NORM || 256 % a.head_dim == 0);
     if (pre) {
         int rc;
-        if (cap == 8 || a.n_tok <= 8) rc = launch_stage<8, 512, 16>(ctx, a, a.n_tok <= 8 ? 8 : cap);
-        else rc = launch_stage<16, 1024, 8>(ctx, a, cap);
+        if (cap == 8 || a.n_tok <= 8) rc = launch_stage<8>(ctx, a, a.n_tok <= 8 ? 8 : cap);
+        else rc = launch_stage<16>(ctx, a, cap);
         if (rc != SHV_OK) return rc;
     }
     const int gcap = pre && a.n_tok <= 8 ? 8 : cap;
