@@ -267,7 +267,7 @@ typedef struct {
  * contiguous KB).  max_cells is a multiple of 32 and both caches hold finite
  * values in every cell (zeros before a cell is written): the last tile of a sequence reads a few
  * cells past its end and weights them by zero. partial is scratch of
- * n_seq*seq_len*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2) floats.  The rows of a sequence are
+ * n_seq*(seq_len rounded up to even)*n_head_kv*n_splits*(n_head/n_head_kv)*(d+2) floats.  The rows of a sequence are
  * taken two at a time over one pass of the cache; with more than two rows every row's cell is
  * written first and all pairs go in one launch, each masked to its own position. */
 typedef struct {

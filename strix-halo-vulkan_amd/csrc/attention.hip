@@ -107,7 +107,10 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
     const int seq = blockIdx.z / n_groups, row0 = row00 + R * (blockIdx.z % n_groups);
     const int slot = a.slot ? a.slot[seq] : seq;
     const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the group's first row
-    const int n_cells = p_first + R;                       // cells the last row sees
+    // the last group of a sequence with an odd number of rows holds one: its second row repeats
+    // the first and is thrown away
+    const int valid = a.seq_len - row0 < R ? a.seq_len - row0 : R;
+    const int n_cells = p_first + valid;                   // cells the last row sees
     // The grid is sized for the cache's capacity; how many of its slices take part depends on how
     // many cells the sequence holds now: about kSliceCells a slice while there are slices to spare.
     int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
@@ -163,8 +166,9 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
     const float *qkv0 = a.qkv + static_cast<size_t>(seq * a.seq_len + row0) * a.qkv_stride;
 #pragma unroll
     for (int j = 0; j < R; j++) {
-        const float *qkv = qkv0 + static_cast<size_t>(j) * a.qkv_stride;
-        const int p = p_first + j;
+        const int jr = j < valid ? j : valid - 1;
+        const float *qkv = qkv0 + static_cast<size_t>(jr) * a.qkv_stride;
+        const int p = p_first + jr;
         const float *rope_row = a.rope + static_cast<size_t>(p) * a.rope_dims;
         if (nc > 0) {
             // this wave's two heads: both rows of the fused projection are requested before either is used
@@ -373,7 +377,9 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_d
     const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + lane, j = blockIdx.y;
     const int seq = blockIdx.z / n_groups, row0 = row00 + R * (blockIdx.z % n_groups);
     const int kvh = head / kRep, hh = head % kRep;
-    const int n_cells = (a.pos ? a.pos[seq] : 0) + row0 + R;
+    if (row0 + j >= a.seq_len) return;  // the thrown-away second row of a last group of one
+    const int valid = a.seq_len - row0 < R ? a.seq_len - row0 : R;
+    const int n_cells = (a.pos ? a.pos[seq] : 0) + row0 + valid;
     int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
     if (n_active > a.n_splits) n_active = a.n_splits;
     const float *pin = a.partial + (static_cast<size_t>(blockIdx.z) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
@@ -469,12 +475,10 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
                 "attn_decode: qkv, caches, norms, partial and out must be 16-byte aligned");
     // The rows of a sequence go two at a time: both see one pass over the cache.  One or two rows
     // write their own cells on the way; more rows have all their cells written first and then go
-    // through as pairs of one launch (and a single last row of another).
+    // through as pairs of one launch (a last pair of one row repeats it and drops the copy).
     if (a.seq_len <= 2) return a.seq_len == 2 ? launch_rows<2>(ctx, a, 0, 1, 1) : launch_rows<1>(ctx, a, 0, 1, 1);
-    const int pairs = a.seq_len / 2;
+    const int pairs = (a.seq_len + 1) / 2;
     SHV_REQUIRE(static_cast<long long>(a.n_seq) * pairs <= 65535, "attn_decode: %d sequences of %d rows in one call", a.n_seq, a.seq_len);
     SHV_LAUNCH(ctx, attn_append_kernel, dim3(a.n_head_kv, a.seq_len, a.n_seq), dim3(kBlock), 0, a);
-    int rc = launch_rows<2>(ctx, a, 0, pairs, 0);
-    if (rc == SHV_OK && (a.seq_len & 1)) rc = launch_rows<1>(ctx, a, a.seq_len - 1, 1, 0);
-    return rc;
+    return launch_rows<2>(ctx, a, 0, pairs, 0);
 }

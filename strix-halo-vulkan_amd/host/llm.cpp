@@ -539,7 +539,7 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
     qkv_ = static_cast<float *>(dev.alloc(T * c_.AttnFusedRows() * 4));
     ctx_ = static_cast<float *>(dev.alloc(T * c_.NHead * c_.HeadDim * 4));
     // one set of slice records per sequence of a batched pass (an ordinary pass is one sequence)
-    partial_ = static_cast<float *>(dev.alloc(T * c_.NHeadKV * kMaxSplits * 8 * (c_.HeadDim + 2) * 4));
+    partial_ = static_cast<float *>(dev.alloc((T + 1) * c_.NHeadKV * kMaxSplits * 8 * (c_.HeadDim + 2) * 4));  // an odd pass rounds up to whole pairs
     const std::vector<float> rt = rope_table(nKV, c_.RopeDims, c_.RopeBase);
     rope_ = static_cast<float *>(dev.alloc(rt.size() * 4));
     dev.upload(rope_, rt.data(), rt.size() * 4);
