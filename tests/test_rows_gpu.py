@@ -321,3 +321,41 @@ def test_checkpoint_restore_is_the_shorter_sequence(rig):
     m.rewind()
     m.speculate(False)
     m.checkpoint_free(c)
+
+
+def test_chunk_size_does_not_matter_over_4096_tokens():
+    """BASELINE's prefill shape: 4096 tokens through a period of three DeltaNet layers and one
+    attention layer at the full widths, in chunks of 64, of 16, and (the first 192) token by token.
+    Every chunk size runs other kernels (matrix cores from 3 or 5 rows, operands staged once from
+    17, rows walked in groups of eight, pairs of attention rows) over the same arithmetic, so the
+    carried state and the last row must agree to rounding."""
+    cfg = dict(n_layer=4, vocab=8192, nkv=4224, slots=1)
+    rng = np.random.default_rng(4096)
+    prompt = rng.integers(0, 8192, size=4096).astype(np.int32)
+    out = {}
+    for rows in (64, 16):
+        m = LA.LLM(LA.Config(max_tokens=rows, **cfg))
+        m.init_synthetic(99)
+        m.stage()
+        lg, hd = m.extend(prompt, want_hidden=True)
+        out[rows] = (lg, hd, m.dn_state(0), m.dn_state(2), m.kv(3, 4096))
+        if rows == 16:
+            m.reset()
+            m.extend(prompt[:192], want_logits=False)
+            short16 = (m.dn_state(1), m.kv(3, 192))
+            m.reset()
+            for t in prompt[:192]:
+                m.extend(np.array([t], np.int32), want_logits=False)
+            short1 = (m.dn_state(1), m.kv(3, 192))
+        m.close()
+    a, b = out[64], out[16]
+    assert O.rel_l2(a[1], b[1]) <= 1e-3 and O.rel_l2(a[0], b[0]) <= 1e-3, (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]))
+    assert O.rel_l2(a[2], b[2]) <= 1e-3 and O.rel_l2(a[3], b[3]) <= 1e-3
+    f16 = lambda bits: bits.view(np.float16).astype(np.float32)
+    for ka, kb in zip(a[4], b[4]):  # the cache: halves, the last bit of a few percent of them flips
+        assert O.rel_l2(f16(ka), f16(kb)) <= 1e-3 and np.mean(ka != kb) <= 0.1
+    assert O.rel_l2(short16[0], short1[0]) <= 1e-3
+    for ka, kb in zip(short16[1], short1[1]):
+        assert O.rel_l2(f16(ka), f16(kb)) <= 1e-3 and np.mean(ka != kb) <= 0.1
+    print("64 vs 16 rows a chunk over 4096 tokens: hidden %.2e logits %.2e state %.2e" %
+          (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]), O.rel_l2(a[2], b[2])))
