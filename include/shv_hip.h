@@ -88,6 +88,7 @@ enum {
     SHV_OP_EMBED = 10,
     SHV_OP_ARGMAX = 11,
     SHV_OP_ADVANCE = 12,
+    SHV_OP_DEQUANT = 13,
     SHV_OP__COUNT
 };
 
@@ -131,6 +132,22 @@ typedef struct {
     int32_t seq_len, ring_slots, ring_stride;
     int32_t z_ring;
 } shv_gemv_q4k_args;
+
+/* ggml type numbers of the tensor types the reference's loader accepts (Dequantizable,
+ * gguf/dequant.go:103-110) */
+enum {
+    SHV_GGML_F32 = 0, SHV_GGML_F16 = 1, SHV_GGML_Q4_1 = 3, SHV_GGML_Q5_0 = 6, SHV_GGML_Q5_1 = 7, SHV_GGML_Q8_0 = 8,
+    SHV_GGML_Q4_K = 12, SHV_GGML_Q5_K = 13, SHV_GGML_Q6_K = 14, SHV_GGML_IQ4_NL = 20, SHV_GGML_BF16 = 30
+};
+
+/* n elements of any of those types to float32, bit for bit what gguf.Dequantize gives
+ * (gguf/dequant.go:52-98; the arms :128-356).  n must be whole blocks of the type (32 or 256). */
+typedef struct {
+    const void *src;
+    float *dst;
+    int64_t n;
+    int32_t type;
+} shv_dequant_args;
 
 /* dst[i] = d*sc*q - dmin*m for every weight of `rows` rows, the reference's dequantQ4_K
  * expression term for term (gguf/dequant.go:252-276); bit-exact. */
@@ -347,6 +364,7 @@ void shv_prerecorded_destroy(shv_ctx *ctx, shv_prerecorded *p);
 /* Convenience entry points: one op each, enqueued without waiting. */
 int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
 int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
+int shv_dequant(shv_ctx *ctx, const shv_dequant_args *a);
 int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
 int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
 int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);

@@ -132,6 +132,168 @@ void shv_ref_dequant_q4k(const uint8_t *data, int64_t nb, float *dst) {
     }
 }
 
+/* ------------------------------------------- the other GGUF tensor types --- */
+/* What a checkpoint of the UD-Q4_K_XL family mixes with Q4_K, and what the reference's loader
+ * accepts (Dequantizable, gguf/dequant.go:103-110).  Each arm is pinned bit for bit by ggml's own
+ * to_float output in gguf/testdata (gguf/dequant_test.go:40-92). */
+
+static inline float bf16_at(const uint8_t *b, int off) {
+    uint32_t u = ((uint32_t)b[off] | ((uint32_t)b[off + 1] << 8)) << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline uint32_t u32_at(const uint8_t *b, int off) {
+    return (uint32_t)b[off] | ((uint32_t)b[off + 1] << 8) | ((uint32_t)b[off + 2] << 16) | ((uint32_t)b[off + 3] << 24);
+}
+
+/* gguf/dequant.go:44-46 */
+static const int8_t kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+/* gguf/dequant.go:128-137: 32 int8 levels times one half scale */
+static void dequant_q8_0(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 34) {
+        float d = f16_at(data, 0);
+        for (int j = 0; j < 32; j++) *dst++ = (float)(int8_t)data[2 + j] * d;
+    }
+}
+
+/* gguf/dequant.go:146-161: level*d + m, low nibbles are elements 0..15, high nibbles 16..31 */
+static void dequant_q4_1(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 20, dst += 32) {
+        float d = f16_at(data, 0), m = f16_at(data, 2);
+        for (int j = 0; j < 16; j++) {
+            dst[j] = (float)(data[4 + j] & 0x0F) * d + m;
+            dst[j + 16] = (float)(data[4 + j] >> 4) * d + m;
+        }
+    }
+}
+
+/* gguf/dequant.go:171-190: five-bit levels centred by 16; the fifth bit of element j is bit j of qh */
+static void dequant_q5_0(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 22, dst += 32) {
+        float d = f16_at(data, 0);
+        uint32_t qh = u32_at(data, 2);
+        for (int j = 0; j < 16; j++) {
+            int x0 = (int)((data[6 + j] & 0x0F) | (((qh >> j) << 4) & 0x10)) - 16;
+            int x1 = (int)((data[6 + j] >> 4) | ((qh >> (j + 12)) & 0x10)) - 16;
+            dst[j] = (float)x0 * d;
+            dst[j + 16] = (float)x1 * d;
+        }
+    }
+}
+
+/* gguf/dequant.go:197-217 */
+static void dequant_q5_1(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 24, dst += 32) {
+        float d = f16_at(data, 0), m = f16_at(data, 2);
+        uint32_t qh = u32_at(data, 4);
+        for (int j = 0; j < 16; j++) {
+            uint8_t x0 = (uint8_t)((data[8 + j] & 0x0F) | (((qh >> j) << 4) & 0x10));
+            uint8_t x1 = (uint8_t)((data[8 + j] >> 4) | ((qh >> (j + 12)) & 0x10));
+            dst[j] = (float)x0 * d + m;
+            dst[j + 16] = (float)x1 * d + m;
+        }
+    }
+}
+
+/* gguf/dequant.go:222-234: nibbles index the non-linear codebook */
+static void dequant_iq4_nl(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 18, dst += 32) {
+        float d = f16_at(data, 0);
+        for (int j = 0; j < 16; j++) {
+            dst[j] = d * (float)kvalues_iq4nl[data[2 + j] & 0xF];
+            dst[j + 16] = d * (float)kvalues_iq4nl[data[2 + j] >> 4];
+        }
+    }
+}
+
+/* gguf/dequant.go:282-317: Q4_K with a 32-byte plane of fifth bits; one byte of qh serves the
+ * same position of all eight sub-blocks, two bits per 64 elements */
+static void dequant_q5_k(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 176) {
+        float d = f16_at(data, 0), dmin = f16_at(data, 2);
+        const uint8_t *scales = data + 4, *qh = data + 16, *ql = data + 48;
+        int is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 256; j += 64) {
+            uint8_t sc, m;
+            shv_ref_scale_min_k4(is, scales, &sc, &m);
+            float d1 = d * (float)sc, m1 = dmin * (float)m;
+            shv_ref_scale_min_k4(is + 1, scales, &sc, &m);
+            float d2 = d * (float)sc, m2 = dmin * (float)m;
+            for (int l = 0; l < 32; l++) *dst++ = d1 * (float)((ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0)) - m1;
+            for (int l = 0; l < 32; l++) *dst++ = d2 * (float)((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
+            ql += 32;
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
+        }
+    }
+}
+
+/* gguf/dequant.go:331-356: six-bit levels centred by 32, sixteen signed int8 group scales, the
+ * half super-scale last; d*scale is formed first, then times the level */
+static void dequant_q6_k(const uint8_t *data, int64_t nb, float *dst) {
+    for (int64_t b = 0; b < nb; b++, data += 210, dst += 256) {
+        const uint8_t *ql = data, *qh = data + 128, *sc = data + 192;
+        float d = f16_at(data, 208);
+        for (int n = 0; n < 256; n += 128) {
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                uint8_t h = qh[n / 4 + l];
+                int q1 = (int)((ql[n / 2 + l] & 0xF) | (((h >> 0) & 3) << 4)) - 32;
+                int q2 = (int)((ql[n / 2 + l + 32] & 0xF) | (((h >> 2) & 3) << 4)) - 32;
+                int q3 = (int)((ql[n / 2 + l] >> 4) | (((h >> 4) & 3) << 4)) - 32;
+                int q4 = (int)((ql[n / 2 + l + 32] >> 4) | (((h >> 6) & 3) << 4)) - 32;
+                const uint8_t *g = sc + n / 16 + is;
+                dst[n + l] = d * (float)(int8_t)g[0] * (float)q1;
+                dst[n + l + 32] = d * (float)(int8_t)g[2] * (float)q2;
+                dst[n + l + 64] = d * (float)(int8_t)g[4] * (float)q3;
+                dst[n + l + 96] = d * (float)(int8_t)g[6] * (float)q4;
+            }
+        }
+    }
+}
+
+/* Bytes of n elements of a ggml type, or -1 (TypeSize/BlockSize, gguf/gguf.go). */
+int64_t shv_ref_type_bytes(int type, int64_t n) {
+    switch (type) {
+        case SHV_GGML_F32: return n * 4;
+        case SHV_GGML_F16: case SHV_GGML_BF16: return n * 2;
+        case SHV_GGML_Q8_0: return n % 32 ? -1 : n / 32 * 34;
+        case SHV_GGML_Q4_1: return n % 32 ? -1 : n / 32 * 20;
+        case SHV_GGML_Q5_0: return n % 32 ? -1 : n / 32 * 22;
+        case SHV_GGML_Q5_1: return n % 32 ? -1 : n / 32 * 24;
+        case SHV_GGML_IQ4_NL: return n % 32 ? -1 : n / 32 * 18;
+        case SHV_GGML_Q4_K: return n % 256 ? -1 : n / 256 * 144;
+        case SHV_GGML_Q5_K: return n % 256 ? -1 : n / 256 * 176;
+        case SHV_GGML_Q6_K: return n % 256 ? -1 : n / 256 * 210;
+    }
+    return -1;
+}
+
+/* Dequantize (gguf/dequant.go:52-98): n elements of a type to float32; 0 on success, -1 for a
+ * type the loader refuses or a count that is not whole blocks. */
+int shv_ref_dequant(int type, const uint8_t *data, int64_t n, float *dst) {
+    if (shv_ref_type_bytes(type, n) < 0) return -1;
+    switch (type) {
+        case SHV_GGML_F32: memcpy(dst, data, (size_t)n * 4); return 0;
+        case SHV_GGML_F16: for (int64_t i = 0; i < n; i++) dst[i] = f16_at(data + 2 * i, 0); return 0;
+        case SHV_GGML_BF16: for (int64_t i = 0; i < n; i++) dst[i] = bf16_at(data + 2 * i, 0); return 0;
+        case SHV_GGML_Q8_0: dequant_q8_0(data, n / 32, dst); return 0;
+        case SHV_GGML_Q4_1: dequant_q4_1(data, n / 32, dst); return 0;
+        case SHV_GGML_Q5_0: dequant_q5_0(data, n / 32, dst); return 0;
+        case SHV_GGML_Q5_1: dequant_q5_1(data, n / 32, dst); return 0;
+        case SHV_GGML_IQ4_NL: dequant_iq4_nl(data, n / 32, dst); return 0;
+        case SHV_GGML_Q4_K: shv_ref_dequant_q4k(data, n / 256, dst); return 0;
+        case SHV_GGML_Q5_K: dequant_q5_k(data, n / 256, dst); return 0;
+        case SHV_GGML_Q6_K: dequant_q6_k(data, n / 256, dst); return 0;
+    }
+    return -1;
+}
+
 /* --------------------------------------------------------- Q4_K quantiser --- */
 
 /* llm/sim.go:1172-1180: ggml nearest_int is round-half-to-even. */

@@ -50,6 +50,13 @@ float    shv_ref_f16_round(float x);
 /* ---- Q4_K, gguf/dequant.go:238-276 ---- */
 void shv_ref_scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m);
 void shv_ref_dequant_q4k(const uint8_t *data, int64_t nblocks, float *dst);
+/* ggml type numbers of the tensor types the loader accepts (gguf/gguf.go, gguf/dequant.go:103-110) */
+enum {
+    SHV_GGML_F32 = 0, SHV_GGML_F16 = 1, SHV_GGML_Q4_1 = 3, SHV_GGML_Q5_0 = 6, SHV_GGML_Q5_1 = 7, SHV_GGML_Q8_0 = 8,
+    SHV_GGML_Q4_K = 12, SHV_GGML_Q5_K = 13, SHV_GGML_Q6_K = 14, SHV_GGML_IQ4_NL = 20, SHV_GGML_BF16 = 30
+};
+int64_t shv_ref_type_bytes(int type, int64_t n);
+int shv_ref_dequant(int type, const uint8_t *data, int64_t n, float *dst);
 
 /* ---- Q4_K quantiser (round-to-nearest arm), llm/quantk.go:115-179, llm/sim.go:982-1060,
  *      llm/quantk.go:211-226, llm/moebank.go:489-532 ---- */

@@ -10,7 +10,7 @@ Q4K_BYTES = 144
 
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
-OP_EMBED, OP_ARGMAX, OP_ADVANCE = 10, 11, 12
+OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT = 10, 11, 12, 13
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 
@@ -41,6 +41,10 @@ class GemvQ4KArgs(C.Structure):
 
 class DequantQ4KArgs(C.Structure):
     _fields_ = [("w", C.c_void_p), ("dst", C.c_void_p), ("rows", C.c_int64), ("k", C.c_int32)]
+
+
+class DequantArgs(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("n", C.c_int64), ("type", C.c_int32)]
 
 
 class QuantizeQ4KArgs(C.Structure):
@@ -131,7 +135,7 @@ SYMBOLS = [
     "shv_submits", "shv_alloc", "shv_free", "shv_upload", "shv_download", "shv_copy", "shv_zero",
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
-    "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_quantize_q4k",
+    "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
 ]
 
@@ -175,6 +179,7 @@ def load():
     L.shv_prerecorded_destroy.restype = None
     L.shv_gemv_q4k.argtypes = [vp, C.POINTER(GemvQ4KArgs)]
     L.shv_dequant_q4k.argtypes = [vp, C.POINTER(DequantQ4KArgs)]
+    L.shv_dequant.argtypes = [vp, C.POINTER(DequantArgs)]
     L.shv_quantize_q4k.argtypes = [vp, C.POINTER(QuantizeQ4KArgs)]
     L.shv_fill_normal.argtypes = [vp, C.POINTER(FillNormalArgs)]
     L.shv_moe_router.argtypes = [vp, C.POINTER(MoeRouterArgs)]
@@ -304,6 +309,11 @@ class Context:
             self.h = None
 
     # ---- convenience wrappers over single ops ----
+    def dequant(self, typ, src, dst, n):
+        """n elements of ggml tensor type `typ` at src to float32 at dst."""
+        a = DequantArgs(_ptr(src), _ptr(dst), n, typ)
+        check(self.L.shv_dequant(self.h, C.byref(a)))
+
     def gemv_q4k(self, w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None,
                  eps=1e-6, head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None,
                  ring_slots=0, ring_stride=0, slot=None, seq_len=0, z_ring=0):

@@ -10,6 +10,9 @@ Writes, next to this script:
   f32_to_f16.txt        the whole 10 575-pair table (safetensors/testdata/f32_to_f16.txt)
   dequant_q4k_in.bin    record 0 (ggml type 12 = Q4_K, 4 blocks, 576 B) of gguf/testdata/dequant_in.bin
   dequant_q4k_ref.bin   its 1024 float32 from ggml's to_float (gguf/testdata/dequant_ref.bin)
+  dequant_in.bin        all eleven records of gguf/testdata/dequant_in.bin (Q4_K, Q5_K, Q5_1, Q8_0, IQ4_NL,
+                        F32, F16, BF16, Q4_1, Q5_0, Q6_K; 3.7 KB)
+  dequant_ref.bin       ggml's to_float of each (18 KB)
   quant_q4k_in.bin      Q4_K round-to-nearest records of llm/testdata/quant_in.bin:
                         all 16 rows of k=2560 and the first 4 rows of k=10240
   quant_q4k_ref.bin     ggml quantize_chunk -> to_float of the same rows (llm/testdata/quant_ref.bin)
@@ -47,6 +50,8 @@ def dequant_record(path, want_type):
     raise SystemExit(f"no record of type {want_type} in {path}")
 
 
+out("dequant_in.bin", open(os.path.join(ref, "gguf/testdata/dequant_in.bin"), "rb").read())
+out("dequant_ref.bin", open(os.path.join(ref, "gguf/testdata/dequant_ref.bin"), "rb").read())
 out("dequant_q4k_in.bin", dequant_record(os.path.join(ref, "gguf/testdata/dequant_in.bin"), 12))
 out("dequant_q4k_ref.bin", dequant_record(os.path.join(ref, "gguf/testdata/dequant_ref.bin"), 12))
 

@@ -97,6 +97,10 @@ def lib():
     L.shv_ref_f16_round.argtypes = [C.c_float]
     L.shv_ref_scale_min_k4.argtypes = [C.c_int, u8p, u8p, u8p]
     L.shv_ref_dequant_q4k.argtypes = [u8p, C.c_int64, f32p]
+    L.shv_ref_dequant.argtypes = [C.c_int, u8p, C.c_int64, f32p]
+    L.shv_ref_dequant.restype = C.c_int
+    L.shv_ref_type_bytes.argtypes = [C.c_int, C.c_int64]
+    L.shv_ref_type_bytes.restype = C.c_int64
     L.shv_ref_make_qkx_quants.restype = C.c_float
     L.shv_ref_make_qkx_quants.argtypes = [f32p, C.c_int, C.c_int, f32p, u8p, u8p, C.c_float,
                                           C.c_float, C.c_int, f32p]
@@ -180,6 +184,24 @@ def dequant_q4k(q, k=None):
     out = np.empty(nblocks * Q4K_BLOCK, dtype=np.float32)
     lib().shv_ref_dequant_q4k(B(q), nblocks, F(out))
     return out if k is None else out.reshape(-1, k)
+
+
+GGML_TYPES = {"F32": 0, "F16": 1, "Q4_1": 3, "Q5_0": 6, "Q5_1": 7, "Q8_0": 8, "Q4_K": 12, "Q5_K": 13, "Q6_K": 14,
+              "IQ4_NL": 20, "BF16": 30}
+
+
+def type_bytes(typ, n):
+    return int(lib().shv_ref_type_bytes(typ, n))
+
+
+def dequant(typ, data, n):
+    """n elements of a ggml tensor type to float32 (the reference's gguf.Dequantize)."""
+    data = np.ascontiguousarray(data, dtype=np.uint8)
+    assert data.size == type_bytes(typ, n), (typ, n, data.size)
+    out = np.empty(n, dtype=np.float32)
+    if lib().shv_ref_dequant(typ, B(data), n, F(out)) != 0:
+        raise ValueError("type %d is not dequantisable" % typ)
+    return out
 
 
 def gemv_q4k(wq, x, n, k, threads=1):

@@ -5,6 +5,7 @@ import os
 import struct
 
 import numpy as np
+import pytest
 
 import oracle_lib as O
 
@@ -58,6 +59,37 @@ def _dequant_record(path):
     b = open(path, "rb").read()
     typ, n, nbytes = struct.unpack_from("<IIQ", b, 0)
     return typ, n, b[16:16 + nbytes]
+
+
+def _records(path):
+    b = open(path, "rb").read()
+    o, out = 0, []
+    while o < len(b):
+        typ, n, nbytes = struct.unpack_from("<IIQ", b, o)
+        out.append((typ, n, b[o + 16:o + 16 + nbytes]))
+        o += 16 + nbytes
+    return out
+
+
+def test_every_tensor_type_matches_ggml_bit_for_bit(golden_dir):
+    """All eleven types the reference's loader accepts (gguf/dequant.go:103-110), each against
+    ggml's own to_float of the same bytes (gguf/dequant_test.go:40-92)."""
+    ins = _records(os.path.join(golden_dir, "dequant_in.bin"))
+    refs = _records(os.path.join(golden_dir, "dequant_ref.bin"))
+    assert len(ins) == len(refs) == 11
+    assert {t for t, _, _ in ins} == set(O.GGML_TYPES.values())
+    for (typ, n, payload), (rtyp, rn, rpayload) in zip(ins, refs):
+        assert (typ, n) == (rtyp, rn) and len(payload) == O.type_bytes(typ, n)
+        got = O.dequant(typ, np.frombuffer(payload, dtype=np.uint8), n)
+        want = np.frombuffer(rpayload, dtype=np.float32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), typ
+
+
+def test_dequant_refuses_what_the_loader_refuses():
+    assert O.type_bytes(2, 32) == -1        # Q4_0 is not among the loader's types
+    assert O.type_bytes(12, 100) == -1      # not whole super-blocks
+    with pytest.raises((ValueError, AssertionError)):
+        O.dequant(12, np.zeros(10, np.uint8), 100)
 
 
 def test_dequant_q4k_matches_ggml_bit_for_bit(golden_dir):
