@@ -89,6 +89,7 @@ enum {
     SHV_OP_ARGMAX = 11,
     SHV_OP_ADVANCE = 12,
     SHV_OP_DEQUANT = 13,
+    SHV_OP_GEMV = 14,
     SHV_OP__COUNT
 };
 
@@ -148,6 +149,19 @@ typedef struct {
     int64_t n;
     int32_t type;
 } shv_dequant_args;
+
+/* y[r] = sum_i W[r][i] * x[i] (+ residual[r]) for W [n][k] row-major in any of those types: the
+ * CPU path's matvec over Tensor.DequantizeRow (llm/hc.go:255-264, gguf/dequant.go:119-124) for the
+ * tensors of a checkpoint that are not Q4_K.  One row of activations, no prologue; Q4_K weights
+ * on the token path go through shv_gemv_q4k. */
+typedef struct {
+    const void *w;
+    const float *x;
+    float *y;
+    const float *residual;
+    int32_t n, k;
+    int32_t type;
+} shv_gemv_args;
 
 /* dst[i] = d*sc*q - dmin*m for every weight of `rows` rows, the reference's dequantQ4_K
  * expression term for term (gguf/dequant.go:252-276); bit-exact. */
@@ -365,6 +379,7 @@ void shv_prerecorded_destroy(shv_ctx *ctx, shv_prerecorded *p);
 int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
 int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
 int shv_dequant(shv_ctx *ctx, const shv_dequant_args *a);
+int shv_gemv(shv_ctx *ctx, const shv_gemv_args *a);
 int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
 int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
 int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);

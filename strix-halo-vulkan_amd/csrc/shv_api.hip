@@ -193,6 +193,7 @@ static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t by
         case SHV_OP_ARGMAX: return run_as<shv_argmax_args>(ctx, args, bytes, shv_launch_argmax, "argmax");
         case SHV_OP_ADVANCE: return run_as<shv_advance_args>(ctx, args, bytes, shv_launch_advance, "advance");
         case SHV_OP_DEQUANT: return run_as<shv_dequant_args>(ctx, args, bytes, shv_launch_dequant, "dequant");
+        case SHV_OP_GEMV: return run_as<shv_gemv_args>(ctx, args, bytes, shv_launch_gemv, "gemv");
         default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
     }
 }
@@ -322,6 +323,7 @@ void shv_prerecorded_destroy(shv_ctx *ctx, shv_prerecorded *p) {
 int shv_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a) { return dispatch_one(ctx, SHV_OP_GEMV_Q4K, a, sizeof(*a)); }
 int shv_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a) { return dispatch_one(ctx, SHV_OP_DEQUANT_Q4K, a, sizeof(*a)); }
 int shv_dequant(shv_ctx *ctx, const shv_dequant_args *a) { return dispatch_one(ctx, SHV_OP_DEQUANT, a, sizeof(*a)); }
+int shv_gemv(shv_ctx *ctx, const shv_gemv_args *a) { return dispatch_one(ctx, SHV_OP_GEMV, a, sizeof(*a)); }
 int shv_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a) { return dispatch_one(ctx, SHV_OP_QUANTIZE_Q4K, a, sizeof(*a)); }
 int shv_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a) { return dispatch_one(ctx, SHV_OP_FILL_NORMAL, a, sizeof(*a)); }
 int shv_moe_router(shv_ctx *ctx, const shv_moe_router_args *a) { return dispatch_one(ctx, SHV_OP_MOE_ROUTER, a, sizeof(*a)); }

@@ -103,6 +103,7 @@ bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a);
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a);
 int shv_launch_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
 int shv_launch_dequant(shv_ctx *ctx, const shv_dequant_args *a);
+int shv_launch_gemv(shv_ctx *ctx, const shv_gemv_args *a);
 int shv_launch_quantize_q4k(shv_ctx *ctx, const shv_quantize_q4k_args *a);
 int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
 int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);

@@ -10,7 +10,7 @@ Q4K_BYTES = 144
 
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
-OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT = 10, 11, 12, 13
+OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV = 10, 11, 12, 13, 14
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 
@@ -45,6 +45,11 @@ class DequantQ4KArgs(C.Structure):
 
 class DequantArgs(C.Structure):
     _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("n", C.c_int64), ("type", C.c_int32)]
+
+
+class GemvArgs(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("x", C.c_void_p), ("y", C.c_void_p), ("residual", C.c_void_p),
+                ("n", C.c_int32), ("k", C.c_int32), ("type", C.c_int32)]
 
 
 class QuantizeQ4KArgs(C.Structure):
@@ -135,7 +140,7 @@ SYMBOLS = [
     "shv_submits", "shv_alloc", "shv_free", "shv_upload", "shv_download", "shv_copy", "shv_zero",
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
-    "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_quantize_q4k",
+    "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
 ]
 
@@ -180,6 +185,7 @@ def load():
     L.shv_gemv_q4k.argtypes = [vp, C.POINTER(GemvQ4KArgs)]
     L.shv_dequant_q4k.argtypes = [vp, C.POINTER(DequantQ4KArgs)]
     L.shv_dequant.argtypes = [vp, C.POINTER(DequantArgs)]
+    L.shv_gemv.argtypes = [vp, C.POINTER(GemvArgs)]
     L.shv_quantize_q4k.argtypes = [vp, C.POINTER(QuantizeQ4KArgs)]
     L.shv_fill_normal.argtypes = [vp, C.POINTER(FillNormalArgs)]
     L.shv_moe_router.argtypes = [vp, C.POINTER(MoeRouterArgs)]
@@ -313,6 +319,11 @@ class Context:
         """n elements of ggml tensor type `typ` at src to float32 at dst."""
         a = DequantArgs(_ptr(src), _ptr(dst), n, typ)
         check(self.L.shv_dequant(self.h, C.byref(a)))
+
+    def gemv(self, typ, w, x, y, n, k, residual=None):
+        """y = W x (+ residual) for W [n][k] of ggml tensor type `typ`."""
+        a = GemvArgs(_ptr(w), _ptr(x), _ptr(y), _ptr(residual), n, k, typ)
+        check(self.L.shv_gemv(self.h, C.byref(a)))
 
     def gemv_q4k(self, w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None,
                  eps=1e-6, head_dim=0, x_stride=None, y_stride=None, z_stride=None, pos=None,

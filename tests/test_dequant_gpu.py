@@ -38,32 +38,64 @@ def test_ggml_vectors_bit_for_bit(ctx, golden_dir):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), typ
 
 
+def random_tensor(name, n, seed=None):
+    """`n` elements of tensor type `name`: random bytes with finite half scales, so every bit pattern of
+    levels, fifth/sixth-bit planes and packed scales occurs."""
+    typ = O.GGML_TYPES[name]
+    rng = np.random.default_rng(typ if seed is None else seed)
+    raw = rng.integers(0, 256, size=O.type_bytes(typ, n), dtype=np.uint8)
+    if name in ("F32", "F16", "BF16"):
+        vals = rng.standard_normal(n).astype(np.float32)
+        return {"F32": vals.view(np.uint8), "F16": vals.astype(np.float16).view(np.uint8),
+                "BF16": (vals.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)}[name].copy()
+    # put finite halves where the formats keep their scales
+    blk = {"Q8_0": (34, [0]), "Q4_1": (20, [0, 2]), "Q5_0": (22, [0]), "Q5_1": (24, [0, 2]), "IQ4_NL": (18, [0]),
+           "Q4_K": (144, [0, 2]), "Q5_K": (176, [0, 2]), "Q6_K": (210, [208])}[name]
+    rows = raw.reshape(-1, blk[0])
+    for off in blk[1]:
+        h = (rng.standard_normal(rows.shape[0]) * 0.05).astype(np.float16).view(np.uint16)
+        rows[:, off] = h & 0xFF
+        rows[:, off + 1] = h >> 8
+    return raw
+
+
 @pytest.mark.parametrize("name", sorted(O.GGML_TYPES))
 def test_random_blocks_match_the_cpu(ctx, name):
-    """Random bytes with finite half scales: every bit pattern of levels, fifth/sixth-bit planes and
-    packed scales, 64 Ki elements a type."""
     typ, n = O.GGML_TYPES[name], 65536
-    rng = np.random.default_rng(typ)
-    nbytes = O.type_bytes(typ, n)
-    raw = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
-    if name in ("F32", "F16", "BF16"):
-        width = {"F32": 4, "F16": 2, "BF16": 2}[name]
-        vals = rng.standard_normal(n).astype(np.float32)
-        raw = {"F32": vals.view(np.uint8), "F16": vals.astype(np.float16).view(np.uint8),
-               "BF16": (vals.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)}[name].copy()
-        assert raw.size == n * width
-    else:
-        # put finite halves where the formats keep their scales
-        blk = {"Q8_0": (34, [0]), "Q4_1": (20, [0, 2]), "Q5_0": (22, [0]), "Q5_1": (24, [0, 2]), "IQ4_NL": (18, [0]),
-               "Q4_K": (144, [0, 2]), "Q5_K": (176, [0, 2]), "Q6_K": (210, [208])}[name]
-        rows = raw.reshape(-1, blk[0])
-        for off in blk[1]:
-            h = (rng.standard_normal(rows.shape[0]) * 0.05).astype(np.float16).view(np.uint16)
-            rows[:, off] = h & 0xFF
-            rows[:, off + 1] = h >> 8
+    raw = random_tensor(name, n)
     want = O.dequant(typ, raw, n)
     got = _device(ctx, typ, raw.tobytes(), n)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("k", [256, 2048, 4096])
+@pytest.mark.parametrize("name", sorted(O.GGML_TYPES))
+def test_gemv_of_every_type_matches_matvec_over_dequantised_rows(ctx, name, k):
+    """y = W x as the CPU path forms it (llm/hc.go:255-264 over gguf/dequant.go:119-124): rows
+    dequantised by the fixture-pinned restatement, dotted in float64.  fp32 accumulation, so 1e-5
+    relative L2 (the path's bar is 1e-3); 37 rows leave the last block ragged."""
+    typ, n = O.GGML_TYPES[name], 37
+    raw = random_tensor(name, n * k, seed=1000 + typ + k)
+    rng = np.random.default_rng(k)
+    x = rng.standard_normal(k).astype(np.float32)
+    res = rng.standard_normal(n).astype(np.float32)
+    w = O.dequant(typ, raw, n * k).reshape(n, k).astype(np.float64)
+    y = ctx.alloc(n * 4)
+    ctx.gemv(typ, ctx.upload(raw), ctx.upload(x), y, n, k)
+    assert O.rel_l2(y.read(np.float32, n), w @ x) <= 1e-5
+    ctx.gemv(typ, ctx.upload(raw), ctx.upload(x), y, n, k, residual=ctx.upload(res))
+    assert O.rel_l2(y.read(np.float32, n), w @ x + res) <= 1e-5
+
+
+def test_gemv_at_vocabulary_height_agrees_with_the_q4k_kernel(ctx):
+    """151936 x 2048 Q4_K through both kernels: same weights, same x, results equal to rounding."""
+    n, k = 151936, 2048
+    raw = random_tensor("Q4_K", n * k, seed=5)
+    x = np.random.default_rng(6).standard_normal(k).astype(np.float32)
+    w, xd, y0, y1 = ctx.upload(raw), ctx.upload(x), ctx.alloc(n * 4), ctx.alloc(n * 4)
+    ctx.gemv(O.GGML_TYPES["Q4_K"], w, xd, y0, n, k)
+    ctx.gemv_q4k(w, xd, y1, n, k)
+    assert O.rel_l2(y0.read(np.float32, n), y1.read(np.float32, n)) <= 1e-5
 
 
 def test_refusals(ctx):
@@ -72,3 +104,9 @@ def test_refusals(ctx):
         ctx.dequant(2, src, dst, 32)      # Q4_0: not a type the loader accepts
     with pytest.raises(shv.api.ShvError):
         ctx.dequant(12, src, dst, 100)    # not whole super-blocks
+    with pytest.raises(shv.api.ShvError):
+        ctx.gemv(2, src, src, dst, 4, 32)     # Q4_0
+    with pytest.raises(shv.api.ShvError):
+        ctx.gemv(14, src, src, dst, 1, 128)   # Q6_K rows are whole super-blocks
+    with pytest.raises(shv.api.ShvError):
+        ctx.gemv(8, src, src, dst, 1, 32768)  # x would not fit its staging
