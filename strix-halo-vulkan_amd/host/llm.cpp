@@ -192,6 +192,152 @@ void Model::InitSynthetic(uint64_t seed) {
     shv_free(dev_.ctx(), stage);
 }
 
+// The fused tensor a window of rows belongs to, by address.
+const std::string *Model::base_of(const TensorView &alias) const {
+    for (const auto &kv : tensors_) {
+        const TensorView &b = kv.second;
+        if (b.init_std < 0.f) continue;
+        const char *p = static_cast<const char *>(alias.ptr), *lo = static_cast<const char *>(b.ptr);
+        if (p >= lo && p < lo + b.bytes) return &kv.first;
+    }
+    return nullptr;
+}
+
+Config Model::ConfigFromGGUF(const gguf::Set &s) {
+    const std::string arch = s.Arch();
+    if (arch.empty()) throw Error("llm: checkpoint states no general.architecture");
+    Config c;
+    auto want = [&](const char *k, int *dst) {
+        uint64_t v;
+        if (!s.Uint(arch + "." + k, &v)) throw Error("llm: the checkpoint states no " + arch + "." + k);
+        *dst = static_cast<int>(v);
+    };
+    auto may = [&](const char *k, int *dst) {
+        uint64_t v;
+        if (s.Uint(arch + "." + k, &v)) *dst = static_cast<int>(v);
+    };
+    int blocks = 0;
+    want("block_count", &blocks);
+    want("embedding_length", &c.NEmbd);
+    want("attention.head_count", &c.NHead);
+    want("attention.head_count_kv", &c.NHeadKV);
+    want("attention.key_length", &c.HeadDim);
+    want("rope.dimension_count", &c.RopeDims);
+    want("expert_count", &c.NExpert);
+    want("expert_used_count", &c.NExpertUsed);
+    want("expert_feed_forward_length", &c.FFNExpert);
+    want("ssm.state_size", &c.SSMHeadDim);
+    want("ssm.group_count", &c.SSMHeadK);
+    want("ssm.time_step_rank", &c.SSMHeadV);
+    want("ssm.conv_kernel", &c.SSMConv);
+    may("full_attention_interval", &c.AttnEvery);
+    c.NextN = 0;
+    may("nextn_predict_layers", &c.NextN);
+    c.NLayer = blocks - c.NextN;  // block_count counts the draft block (llm/mtp.go:137)
+    double f;
+    if (s.Float(arch + ".attention.layer_norm_rms_epsilon", &f)) c.RMSEps = static_cast<float>(f);
+    if (s.Float(arch + ".rope.freq_base", &f)) c.RopeBase = static_cast<float>(f);
+    if (!s.Has("token_embd.weight") || s.Get("token_embd.weight").Dims.size() < 2) throw Error("llm: the checkpoint has no 2-D token_embd.weight to read the vocabulary from");
+    c.VocabSize = static_cast<int>(s.Get("token_embd.weight").Dims[1]);
+    return c;
+}
+
+void Model::LoadGGUF(const gguf::Set &s) {
+    std::map<std::string, int64_t> covered;  // rows of each whole tensor that came from the file
+    for (const auto &kv : tensors_) {
+        const std::string &name = kv.first;
+        const TensorView &v = kv.second;
+        if (!s.Has(name)) continue;
+        const gguf::Tensor &t = s.Get(name);
+        const std::string shape = "[" + std::to_string(t.Dims[0]) + " x " + std::to_string(t.Rows()) + "] " + gguf::TypeName(t.Type);
+        if (t.Dims[0] != v.cols || t.Rows() != v.rows)
+            throw Error("llm: " + name + " is " + shape + " in the checkpoint, the metadata makes it [" + std::to_string(v.cols) + " x " + std::to_string(v.rows) + "]");
+        const uint32_t same = v.kind == TensorView::Q4K ? gguf::Q4_K : v.kind == TensorView::F16 ? gguf::F16 : gguf::F32;
+        if (t.Type == same) {
+            if (t.Bytes != v.bytes) throw Error("llm: " + name + ": " + std::to_string(t.Bytes) + " bytes in the checkpoint, " + std::to_string(v.bytes) + " staged");
+            dev_.upload(v.ptr, t.Data, t.Bytes);
+        } else if (v.kind == TensorView::F32) {
+            // small float tensors (norms, routers, conv taps) in whatever the converter chose: expanded on the device
+            void *raw = nullptr;
+            check(shv_alloc(dev_.ctx(), t.Bytes, &raw), "staging");
+            try {
+                dev_.upload(raw, t.Data, t.Bytes);
+                shv_dequant_args d{raw, static_cast<float *>(v.ptr), t.Elems(), static_cast<int32_t>(t.Type)};
+                check(shv_dequant(dev_.ctx(), &d), name.c_str());
+                dev_.sync();
+            } catch (...) {
+                shv_free(dev_.ctx(), raw);
+                throw;
+            }
+            shv_free(dev_.ctx(), raw);
+        } else {
+            throw Error("llm: " + name + " is " + gguf::TypeName(t.Type) + " in the checkpoint; the kernels stream it as " + gguf::TypeName(same));
+        }
+        const std::string *base = v.init_std < 0.f ? base_of(v) : &name;
+        if (base) covered[*base] += v.rows;
+    }
+    for (const auto &kv : tensors_) {
+        if (kv.second.init_std < 0.f) continue;
+        const int64_t got = covered.count(kv.first) ? covered[kv.first] : 0;
+        if (got < kv.second.rows)
+            throw Error("llm: the checkpoint fills " + std::to_string(got) + " of " + std::to_string(kv.second.rows) + " rows of " + kv.first + " (the tensor or its constituents are missing)");
+    }
+    dev_.sync();
+}
+
+void Model::SaveGGUF(const std::string &path, const std::string &arch) const {
+    const Config &c = cfg_;
+    gguf::Writer w;
+    w.PutStr(gguf::kKeyArchitecture, arch);
+    auto u32 = [&](const char *k, int v) { w.PutU32(arch + "." + k, static_cast<uint32_t>(v)); };
+    u32("block_count", c.Blocks());
+    u32("embedding_length", c.NEmbd);
+    u32("attention.head_count", c.NHead);
+    u32("attention.head_count_kv", c.NHeadKV);
+    u32("attention.key_length", c.HeadDim);
+    u32("rope.dimension_count", c.RopeDims);
+    w.PutF32(arch + ".rope.freq_base", c.RopeBase);
+    u32("expert_count", c.NExpert);
+    u32("expert_used_count", c.NExpertUsed);
+    u32("expert_feed_forward_length", c.FFNExpert);
+    w.PutF32(arch + ".attention.layer_norm_rms_epsilon", c.RMSEps);
+    u32("ssm.state_size", c.SSMHeadDim);
+    u32("ssm.group_count", c.SSMHeadK);
+    u32("ssm.time_step_rank", c.SSMHeadV);
+    u32("ssm.conv_kernel", c.SSMConv);
+    u32("full_attention_interval", c.AttnEvery);
+    u32("nextn_predict_layers", c.NextN);
+
+    // constituents stand in for a fused tensor when they tile it
+    std::map<std::string, std::vector<std::string>> parts;
+    for (const auto &kv : tensors_)
+        if (kv.second.init_std < 0.f)
+            if (const std::string *b = base_of(kv.second)) parts[*b].push_back(kv.first);
+    auto emit = [&](const std::string &name, const TensorView &v) {
+        std::vector<int64_t> dims;
+        if (v.rows == 1) dims = {v.cols};
+        else if (name.find("_exps.") != std::string::npos) dims = {v.cols, v.rows / c.NExpert, c.NExpert};
+        else dims = {v.cols, v.rows};
+        const uint32_t type = v.kind == TensorView::Q4K ? gguf::Q4_K : v.kind == TensorView::F16 ? gguf::F16 : gguf::F32;
+        Device *dev = &dev_;
+        const void *src = v.ptr;
+        w.AddTensor(name, type, dims, [dev, src](uint8_t *dst, uint64_t bytes) { dev->download(dst, src, bytes); });
+    };
+    for (const auto &kv : tensors_) {
+        if (kv.second.init_std < 0.f) continue;
+        int64_t rows = 0;
+        auto it = parts.find(kv.first);
+        if (it != parts.end())
+            for (const std::string &p : it->second) rows += tensors_.at(p).rows;
+        if (rows == kv.second.rows)
+            for (const std::string &p : it->second) emit(p, tensors_.at(p));
+        else
+            emit(kv.first, kv.second);
+    }
+    dev_.sync();
+    w.Write(path);
+}
+
 // ---------------------------------------------------------------------------------- MoE -------
 
 MoEGPU::MoEGPU(Device &dev, const Model &m, int maxTokens) : dev_(dev), m_(m), c_(m.config()), max_tok_(maxTokens) {

@@ -16,6 +16,7 @@
 #include <string>
 #include <vector>
 
+#include "gguf.hpp"
 #include "shv_hip.h"
 
 namespace llm {
@@ -113,9 +114,25 @@ public:
     uint64_t WeightBytes() const;
     static std::string Blk(int layer, const char *name);
 
+    // llm.Open's readConfig (llm/model.go:66-99): the model's shape from the checkpoint's own
+    // metadata, keys under its general.architecture; the vocabulary is token_embd's row count.
+    static Config ConfigFromGGUF(const gguf::Set &s);
+    // Every tensor of this model from a mapped checkpoint into its device buffer, straight from
+    // the mapping.  A fused projection is filled from its constituents (attn_q / attn_k / attn_v,
+    // attn_qkv / attn_gate / ssm_alpha / ssm_beta, nextn.enorm / hnorm) when the file carries
+    // those, as llama.cpp's converter writes them.  Types must be the ones the kernels stream
+    // (Q4_K matrices, F16 embedding); an F32 tensor of the model takes any type the dequantiser
+    // knows and is expanded on the device.  Throws, naming the tensor, on a missing tensor, a
+    // shape that disagrees with the metadata, or a type the kernels do not read.
+    void LoadGGUF(const gguf::Set &s);
+    // This model as one version-3 file the above reads back bit for bit: metadata keys as
+    // ConfigFromGGUF reads them, constituents in place of fused tensors, expert banks 3-D.
+    void SaveGGUF(const std::string &path, const std::string &arch = "qwen3next") const;
+
 private:
     void add(const std::string &name, TensorView::Kind kind, int64_t rows, int64_t cols, float mean, float std);
     void alias(const std::string &name, const std::string &of, int64_t row0, int64_t rows);
+    const std::string *base_of(const TensorView &alias) const;
     Device &dev_;
     Config cfg_;
     std::map<std::string, TensorView> tensors_;

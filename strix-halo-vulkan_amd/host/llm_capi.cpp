@@ -1,6 +1,7 @@
 // Flat C entry points over llm::Graph for ctypes callers: see shv_llm.h.
 #include "shv_llm.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <memory>
@@ -35,6 +36,27 @@ static llm::Graph &graph_of(shvllm *h) {
     return *h->graph;
 }
 
+static void graph_opts(shvllm &hh, const shvllm_config &cc) {
+    shvllm *h = &hh;
+    const shvllm_config *c = &cc;
+    h->opts.NKV = c->nkv;
+    h->opts.Layers = c->layers;
+    h->opts.NoHead = c->no_head != 0;
+    h->opts.AttnSplits = c->attn_splits;
+    h->opts.MaxTokens = c->max_tokens > 0 ? c->max_tokens : 1;
+    h->opts.Slots = c->slots > 0 ? c->slots : 1;
+    h->opts.HeadRows = c->head_rows;
+    h->opts.Speculative = c->speculative != 0;
+    if (c->spec_rows > 0) h->opts.SpecRows = c->spec_rows;
+}
+
+template <typename T>
+static int copy_out(const std::vector<T> *v, T *dst, uint64_t max) {
+    if (!v || !dst) return 0;
+    std::copy(v->begin(), v->begin() + std::min<uint64_t>(max, v->size()), dst);
+    return 1;
+}
+
 extern "C" {
 
 const char *shvllm_last_error(void) { return g_err; }
@@ -63,15 +85,7 @@ int shvllm_open(int device, const shvllm_config *c, shvllm **out) {
         cfg.SSMConv = c->ssm_conv;
         cfg.AttnEvery = c->attn_every;
         cfg.NextN = c->nextn;
-        h->opts.NKV = c->nkv;
-        h->opts.Layers = c->layers;
-        h->opts.NoHead = c->no_head != 0;
-        h->opts.AttnSplits = c->attn_splits;
-        h->opts.MaxTokens = c->max_tokens > 0 ? c->max_tokens : 1;
-        h->opts.Slots = c->slots > 0 ? c->slots : 1;
-        h->opts.HeadRows = c->head_rows;
-        h->opts.Speculative = c->speculative != 0;
-        if (c->spec_rows > 0) h->opts.SpecRows = c->spec_rows;
+        graph_opts(*h, *c);
         h->model = std::make_unique<llm::Model>(*h->dev, cfg);
         for (const auto &kv : h->model->Tensors()) h->names.push_back(kv.first);
         *out = h.release();
@@ -92,6 +106,41 @@ shv_ctx *shvllm_ctx(shvllm *h) { return h && h->dev ? h->dev->ctx() : nullptr; }
 
 int shvllm_init_synthetic(shvllm *h, uint64_t seed) {
     return guard([&] { h->model->InitSynthetic(seed); });
+}
+
+int shvllm_open_gguf(int device, const char *path, const shvllm_config *c, shvllm **out) {
+    return guard([&] {
+        if (!path || !c || !out) throw llm::Error("llm: shvllm_open_gguf: NULL argument");
+        std::unique_ptr<gguf::Set> set = gguf::Set::Open(path);
+        auto h = std::make_unique<shvllm>();
+        h->dev = std::make_unique<llm::Device>(device);
+        graph_opts(*h, *c);
+        h->model = std::make_unique<llm::Model>(*h->dev, llm::Model::ConfigFromGGUF(*set));
+        h->model->LoadGGUF(*set);
+        for (const auto &kv : h->model->Tensors()) h->names.push_back(kv.first);
+        *out = h.release();
+    });
+}
+
+int shvllm_get_config(shvllm *h, shvllm_config *o) {
+    return guard([&] {
+        if (!h || !h->model || !o) throw llm::Error("llm: shvllm_get_config: NULL argument");
+        const llm::Config &c = h->model->config();
+        o->n_layer = c.NLayer, o->n_embd = c.NEmbd, o->n_head = c.NHead, o->n_head_kv = c.NHeadKV, o->head_dim = c.HeadDim;
+        o->rope_dims = c.RopeDims, o->rope_base = c.RopeBase, o->n_expert = c.NExpert, o->n_expert_used = c.NExpertUsed;
+        o->ffn_expert = c.FFNExpert, o->vocab = c.VocabSize, o->rms_eps = c.RMSEps, o->ssm_head_dim = c.SSMHeadDim;
+        o->ssm_head_k = c.SSMHeadK, o->ssm_head_v = c.SSMHeadV, o->ssm_conv = c.SSMConv, o->attn_every = c.AttnEvery, o->nextn = c.NextN;
+        o->nkv = h->opts.NKV, o->layers = h->opts.Layers, o->no_head = h->opts.NoHead, o->attn_splits = h->opts.AttnSplits;
+        o->max_tokens = h->opts.MaxTokens, o->slots = h->opts.Slots, o->head_rows = h->opts.HeadRows;
+        o->speculative = h->opts.Speculative, o->spec_rows = h->opts.SpecRows;
+    });
+}
+
+int shvllm_save_gguf(shvllm *h, const char *path) {
+    return guard([&] {
+        if (!h || !h->model || !path) throw llm::Error("llm: shvllm_save_gguf: NULL argument");
+        h->model->SaveGGUF(path);
+    });
 }
 
 int shvllm_tensor_count(shvllm *h) { return h ? static_cast<int>(h->names.size()) : 0; }
@@ -372,6 +421,167 @@ int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos) {
             nanos[1] = s.VerifyNanos;
         }
     });
+}
+
+// ---- the GGUF container by itself ---------------------------------------------------------------
+
+struct shvgguf {
+    std::unique_ptr<gguf::Set> set;    // OpenSet
+    std::unique_ptr<gguf::File> file;  // Open: one file, shards not joined
+    std::vector<const gguf::Tensor *> tensors;
+    const gguf::KV *kv = nullptr;
+    const std::vector<std::string> *keys = nullptr;
+};
+
+static shvgguf &gg(shvgguf *g) {
+    if (!g) throw gguf::Error("gguf: NULL handle");
+    return *g;
+}
+static const gguf::Value *value_of(shvgguf *g, const char *key) { return g && key ? g->kv->Find(key) : nullptr; }
+
+int shvgguf_open(const char *path, shvgguf **out) {
+    return guard([&] {
+        if (!path || !out) throw gguf::Error("gguf: NULL argument");
+        auto g = std::make_unique<shvgguf>();
+        g->set = gguf::Set::Open(path);
+        g->tensors = g->set->Tensors;
+        g->kv = g->set.get();
+        g->keys = &g->set->Keys();
+        *out = g.release();
+    });
+}
+
+int shvgguf_open_file(const char *path, shvgguf **out) {
+    return guard([&] {
+        if (!path || !out) throw gguf::Error("gguf: NULL argument");
+        auto g = std::make_unique<shvgguf>();
+        g->file = gguf::File::Open(path);
+        for (const gguf::Tensor &t : g->file->Tensors) g->tensors.push_back(&t);
+        g->kv = g->file.get();
+        g->keys = &g->file->Keys();
+        *out = g.release();
+    });
+}
+
+void shvgguf_close(shvgguf *g) { delete g; }
+int shvgguf_files(shvgguf *g) { return !g ? 0 : g->set ? static_cast<int>(g->set->Files.size()) : 1; }
+
+int shvgguf_file_info(shvgguf *g, int i, const char **path, uint32_t *version, uint64_t *alignment, int64_t *data_start) {
+    return guard([&] {
+        if (i < 0 || i >= shvgguf_files(g)) throw gguf::Error("gguf: file index out of range");
+        const gguf::File &f = gg(g).set ? *g->set->Files[i] : *g->file;
+        if (path) *path = f.Path.c_str();
+        if (version) *version = f.Version;
+        if (alignment) *alignment = f.Alignment;
+        if (data_start) *data_start = f.DataStart;
+    });
+}
+
+int shvgguf_len(shvgguf *g) { return g ? static_cast<int>(g->tensors.size()) : 0; }
+int64_t shvgguf_params(shvgguf *g) {
+    int64_t n = 0;
+    if (g)
+        for (const gguf::Tensor *t : g->tensors) n += t->Elems();
+    return n;
+}
+int64_t shvgguf_bytes(shvgguf *g) {
+    int64_t n = 0;
+    if (g)
+        for (const gguf::Tensor *t : g->tensors) n += static_cast<int64_t>(t->Bytes);
+    return n;
+}
+const char *shvgguf_arch(shvgguf *g) {
+    const gguf::Value *v = value_of(g, gguf::kKeyArchitecture);
+    return v && v->kind == gguf::Value::Str ? v->s.c_str() : "";
+}
+
+int shvgguf_tensor_at(shvgguf *g, int i, const char **name, uint32_t *type, int32_t *n_dims, int64_t *dims, const void **data,
+                      uint64_t *bytes, int32_t *shard, int64_t *rows, int64_t *row_bytes) {
+    return guard([&] {
+        if (i < 0 || i >= shvgguf_len(g)) throw gguf::Error("gguf: tensor index out of range");
+        const gguf::Tensor &t = *gg(g).tensors[i];
+        if (name) *name = t.Name.c_str();
+        if (type) *type = t.Type;
+        if (n_dims) *n_dims = static_cast<int32_t>(t.Dims.size());
+        if (dims)
+            for (size_t j = 0; j < t.Dims.size(); j++) dims[j] = t.Dims[j];
+        if (data) *data = t.Data;
+        if (bytes) *bytes = t.Bytes;
+        if (shard) *shard = t.Shard;
+        if (rows) *rows = t.Rows();
+        if (row_bytes) *row_bytes = t.RowBytes();
+    });
+}
+
+int shvgguf_find(shvgguf *g, const char *name) {
+    if (!g || !name) return -1;
+    for (size_t i = 0; i < g->tensors.size(); i++)
+        if (g->tensors[i]->Name == name) return static_cast<int>(i);
+    return -1;
+}
+
+int shvgguf_advise_random(shvgguf *g, int i) {
+    return guard([&] {
+        if (i < 0 || i >= shvgguf_len(g)) throw gguf::Error("gguf: tensor index out of range");
+        gg(g).tensors[i]->AdviseRandom();
+    });
+}
+
+int shvgguf_key_count(shvgguf *g) { return g ? static_cast<int>(g->keys->size()) : 0; }
+const char *shvgguf_key_at(shvgguf *g, int i) { return g && i >= 0 && i < shvgguf_key_count(g) ? (*g->keys)[i].c_str() : nullptr; }
+int shvgguf_kind(shvgguf *g, const char *key) {
+    const gguf::Value *v = value_of(g, key);
+    return v ? static_cast<int>(v->kind) : 0;
+}
+int shvgguf_uint(shvgguf *g, const char *key, uint64_t *out) { return g && key && out && g->kv->Uint(key, out); }
+int shvgguf_int(shvgguf *g, const char *key, int64_t *out) { return g && key && out && g->kv->Int(key, out); }
+int shvgguf_float(shvgguf *g, const char *key, double *out) { return g && key && out && g->kv->Float(key, out); }
+int shvgguf_bool(shvgguf *g, const char *key, int32_t *out) {
+    bool b = false;
+    if (!g || !key || !out || !g->kv->Bool(key, &b)) return 0;
+    *out = b;
+    return 1;
+}
+int shvgguf_str(shvgguf *g, const char *key, const char **out, uint64_t *len) {
+    const gguf::Value *v = value_of(g, key);
+    if (!v || v->kind != gguf::Value::Str) return 0;
+    if (out) *out = v->s.data();
+    if (len) *len = v->s.size();
+    return 1;
+}
+int shvgguf_array_len(shvgguf *g, const char *key, uint64_t *n) {
+    const gguf::Value *v = value_of(g, key);
+    if (!v || v->kind < gguf::Value::Uints) return 0;
+    if (n) *n = v->Len();
+    return 1;
+}
+int shvgguf_uints(shvgguf *g, const char *key, uint64_t *dst, uint64_t max) { return g && key ? copy_out(g->kv->Uints(key), dst, max) : 0; }
+int shvgguf_ints(shvgguf *g, const char *key, int64_t *dst, uint64_t max) { return g && key ? copy_out(g->kv->Ints(key), dst, max) : 0; }
+int shvgguf_floats(shvgguf *g, const char *key, double *dst, uint64_t max) { return g && key ? copy_out(g->kv->Floats(key), dst, max) : 0; }
+int shvgguf_string_at(shvgguf *g, const char *key, uint64_t i, const char **out, uint64_t *len) {
+    const std::vector<std::string> *v = g && key ? g->kv->Strings(key) : nullptr;
+    if (!v || i >= v->size()) return 0;
+    if (out) *out = (*v)[i].data();
+    if (len) *len = (*v)[i].size();
+    return 1;
+}
+
+const char *shvgguf_type_name(uint32_t type) {
+    static thread_local std::string name;
+    name = gguf::TypeName(type);
+    return name.c_str();
+}
+int shvgguf_type_block(uint32_t type, int32_t *elems, int32_t *nbytes) {
+    const gguf::TypeInfo *i = gguf::Info(type);
+    if (!i) return 0;
+    if (elems) *elems = i->elems;
+    if (nbytes) *nbytes = i->nbytes;
+    return 1;
+}
+int64_t shvgguf_size_of(uint32_t type, int64_t n) {
+    int64_t out = -1;
+    guard([&] { out = gguf::SizeOf(type, n); });
+    return out;
 }
 
 }  // extern "C"

@@ -34,6 +34,13 @@ int shvllm_open(int device, const shvllm_config *cfg, shvllm **out);  /* device 
 void shvllm_close(shvllm *h);
 shv_ctx *shvllm_ctx(shvllm *h);
 int shvllm_init_synthetic(shvllm *h, uint64_t seed);
+/* llm.Open (llm/model.go:52-64): a checkpoint (a .gguf, any shard of a split one, or a directory
+ * holding one) mapped, its shape read from its metadata and every tensor staged in device memory.
+ * The model fields of *opts are ignored; its graph fields (nkv ... spec_rows) are kept. */
+int shvllm_open_gguf(int device, const char *path, const shvllm_config *opts, shvllm **out);
+int shvllm_get_config(shvllm *h, shvllm_config *out);
+/* this model written as one GGUF file that shvllm_open_gguf reads back bit for bit */
+int shvllm_save_gguf(shvllm *h, const char *path);
 int shvllm_tensor_count(shvllm *h);
 int shvllm_tensor_at(shvllm *h, int i, const char **name, void **dptr, uint64_t *bytes, int32_t *kind,
                      int64_t *rows, int64_t *cols, int32_t *is_alias);
@@ -89,6 +96,42 @@ int shvllm_spec_round(shvllm *h, const int32_t *forced, int n_forced, int32_t *o
 /* counts: rounds, drafted, accepted, tokens, passes[5], drafted_at[4], accepted_at[4] (17 values);
  * nanos: draft, verify */
 int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos);
+
+/* ---- the GGUF container by itself (package gguf, gguf/gguf.go): no device involved ---------- */
+typedef struct shvgguf shvgguf;
+int shvgguf_open(const char *path, shvgguf **out);   /* OpenSet: a file, any shard, or a directory */
+int shvgguf_open_file(const char *path, shvgguf **out); /* Open: this one file, no sibling shards */
+void shvgguf_close(shvgguf *g);
+int shvgguf_files(shvgguf *g);
+int shvgguf_file_info(shvgguf *g, int i, const char **path, uint32_t *version, uint64_t *alignment, int64_t *data_start);
+int shvgguf_len(shvgguf *g);
+int64_t shvgguf_params(shvgguf *g);
+int64_t shvgguf_bytes(shvgguf *g);
+const char *shvgguf_arch(shvgguf *g);
+/* tensor i of the joined table; dims has room for 4 */
+int shvgguf_tensor_at(shvgguf *g, int i, const char **name, uint32_t *type, int32_t *n_dims, int64_t *dims,
+                      const void **data, uint64_t *bytes, int32_t *shard, int64_t *rows, int64_t *row_bytes);
+int shvgguf_find(shvgguf *g, const char *name);      /* index, or -1 */
+int shvgguf_advise_random(shvgguf *g, int i);
+int shvgguf_key_count(shvgguf *g);
+const char *shvgguf_key_at(shvgguf *g, int i);
+/* metadata: 1 = found and of a kind the getter answers, 0 = not.  kind: 0 none, 1 uint, 2 int, 3 float,
+ * 4 bool, 5 string, 6 uints, 7 ints, 8 floats, 9 bools, 10 strings (widths widen as File.Uint/Int/Float do) */
+int shvgguf_kind(shvgguf *g, const char *key);
+int shvgguf_uint(shvgguf *g, const char *key, uint64_t *out);
+int shvgguf_int(shvgguf *g, const char *key, int64_t *out);
+int shvgguf_float(shvgguf *g, const char *key, double *out);
+int shvgguf_bool(shvgguf *g, const char *key, int32_t *out);
+int shvgguf_str(shvgguf *g, const char *key, const char **out, uint64_t *len);
+int shvgguf_array_len(shvgguf *g, const char *key, uint64_t *n);
+int shvgguf_uints(shvgguf *g, const char *key, uint64_t *dst, uint64_t max);
+int shvgguf_ints(shvgguf *g, const char *key, int64_t *dst, uint64_t max);
+int shvgguf_floats(shvgguf *g, const char *key, double *dst, uint64_t max);
+int shvgguf_string_at(shvgguf *g, const char *key, uint64_t i, const char **out, uint64_t *len);
+/* block geometry of a ggml type: name ("?<n>" when unknown; valid until the next call on this thread) */
+const char *shvgguf_type_name(uint32_t type);
+int shvgguf_type_block(uint32_t type, int32_t *elems, int32_t *nbytes);   /* 0 when unknown */
+int64_t shvgguf_size_of(uint32_t type, int64_t n);                        /* -1 with the error set */
 
 #ifdef __cplusplus
 }

@@ -56,6 +56,9 @@ def load():
     L.shvllm_ctx.argtypes = [vp]
     L.shvllm_ctx.restype = vp
     L.shvllm_init_synthetic.argtypes = [vp, C.c_uint64]
+    L.shvllm_open_gguf.argtypes = [C.c_int, C.c_char_p, C.POINTER(Config), C.POINTER(vp)]
+    L.shvllm_get_config.argtypes = [vp, C.POINTER(Config)]
+    L.shvllm_save_gguf.argtypes = [vp, C.c_char_p]
     L.shvllm_tensor_count.argtypes = [vp]
     L.shvllm_tensor_at.argtypes = [vp, C.c_int, C.POINTER(C.c_char_p), C.POINTER(vp), C.POINTER(C.c_uint64),
                                    C.POINTER(C.c_int32), C.POINTER(C.c_int64), C.POINTER(C.c_int64),
@@ -113,14 +116,24 @@ KIND_DTYPE = {0: np.float32, 1: np.uint16, 2: np.uint8}  # F32, F16 (bit pattern
 class LLM:
     """llm.Model + llm.Graph behind one handle."""
 
-    def __init__(self, cfg, device=0):
+    def __init__(self, cfg, device=0, gguf=None):
+        """With gguf=path the model's shape and weights come from that checkpoint (llm.Open) and
+        only the graph fields of cfg (nkv, max_tokens, slots ...) are used."""
         self.L = load()
         self.H = hip_api.load()
-        self.cfg = cfg
         h = C.c_void_p()
-        _check(self.L.shvllm_open(device, C.byref(cfg), C.byref(h)))
+        if gguf is None:
+            _check(self.L.shvllm_open(device, C.byref(cfg), C.byref(h)))
+        else:
+            _check(self.L.shvllm_open_gguf(device, str(gguf).encode(), C.byref(cfg), C.byref(h)))
+            cfg = Config()
+            _check(self.L.shvllm_get_config(h, C.byref(cfg)))
+        self.cfg = cfg
         self.h = h
         self.ctx = self.L.shvllm_ctx(h)
+
+    def save_gguf(self, path):
+        _check(self.L.shvllm_save_gguf(self.h, str(path).encode()))
 
     def close(self):
         if self.h:

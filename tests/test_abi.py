@@ -21,9 +21,18 @@ def test_every_declared_symbol_is_exported():
     assert declared == set(shv.api.SYMBOLS), declared ^ set(shv.api.SYMBOLS)
 
 
+def test_host_library_exports_what_its_header_declares():
+    hdr = open(os.path.join(shv.ROOT, "strix-halo-vulkan_amd", "host", "shv_llm.h")).read()
+    declared = set(re.findall(r"\b(shv(?:llm|gguf)_[a-z0-9_]+)\s*\(", hdr))
+    assert len(declared) > 60
+    L = ctypes.CDLL(shv.pkg.llm_api.lib_path())
+    missing = sorted(s for s in declared if not hasattr(L, s))
+    assert not missing, missing
+
+
 def test_struct_sizes_fit_the_op_record():
     for t in (shv.api.GemvQ4KArgs, shv.api.DequantQ4KArgs, shv.api.QuantizeQ4KArgs,
-              shv.api.FillNormalArgs):
+              shv.api.FillNormalArgs, shv.api.DequantArgs, shv.api.GemvArgs):
         assert ctypes.sizeof(t) <= 248, t
     assert ctypes.sizeof(shv.api.Op) == 256
 

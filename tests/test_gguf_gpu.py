@@ -1,0 +1,190 @@
+"""Checkpoints through the GGUF container onto the device: a model written out and read back
+(llm.Open, llm/model.go:52-99) is the same bytes in HBM and decodes the same tokens; constituents
+fill fused projections; float tensors in other types are expanded by the device dequantiser; a
+split checkpoint loads like a whole one; a tensor of any accepted type goes from the mapping
+through the any-type GEMV."""
+import numpy as np
+import pytest
+
+import gguf_file as GF
+import oracle_lib as O
+import shv
+from test_dequant_gpu import random_tensor
+
+pytestmark = pytest.mark.gpu
+LA = shv.pkg.llm_api
+G = shv.pkg.gguf_api
+ShvError = shv.api.ShvError
+
+
+def small_cfg(**kw):
+    d = dict(n_layer=4, n_expert=16, n_expert_used=4, vocab=4096, nkv=128)
+    d.update(kw)
+    return LA.Config(**d)
+
+
+@pytest.fixture(scope="module")
+def saved(tmp_path_factory):
+    cfg = small_cfg(nextn=1)
+    m = LA.LLM(cfg)
+    m.init_synthetic(77)
+    m.stage()
+    path = tmp_path_factory.mktemp("gguf") / "model.gguf"
+    m.save_gguf(path)
+    yield m, cfg, str(path)
+    m.close()
+
+
+def _greedy(m, prompt, n):
+    m.reset()
+    lg, _ = m.extend(prompt)
+    ids, _ = m.generate(n)
+    return lg, ids
+
+
+def _rewrite(parsed, path, tensors=None, drop=(), extra_kv=()):
+    """The parsed file written again by the tests' own writer, with some tensors replaced or left out."""
+    w = GF.Writer()
+    for k, v in list(parsed["kv"].items()) + list(extra_kv):
+        w.put(k, GF.STR if isinstance(v, str) else GF.F32 if isinstance(v, float) else GF.U32, v)
+    for name, (typ, dims, data) in parsed["tensors"].items():
+        if name in drop:
+            continue
+        if tensors and name in tensors:
+            typ, dims, data = tensors[name]
+        w.tensor(name, typ, dims, data)
+    return w.write(path)
+
+
+def test_saved_file_is_a_plain_gguf_of_constituents(saved):
+    m, cfg, path = saved
+    p = GF.parse(path)
+    assert p["version"] == 3 and p["kv"]["general.architecture"] == "qwen3next"
+    kv = p["kv"]
+    assert kv["qwen3next.block_count"] == 5 and kv["qwen3next.nextn_predict_layers"] == 1
+    assert kv["qwen3next.embedding_length"] == cfg.n_embd and kv["qwen3next.expert_count"] == 16
+    assert kv["qwen3next.ssm.state_size"] == cfg.ssm_head_dim and kv["qwen3next.full_attention_interval"] == 4
+    names = set(p["tensors"])
+    assert not [n for n in names if "fused" in n]
+    for n in ("blk.3.attn_q.weight", "blk.3.attn_k.weight", "blk.3.attn_v.weight", "blk.0.attn_qkv.weight",
+              "blk.0.attn_gate.weight", "blk.0.ssm_alpha.weight", "blk.0.ssm_beta.weight", "blk.4.nextn.enorm.weight",
+              "blk.4.nextn.hnorm.weight", "token_embd.weight", "output.weight"):
+        assert n in names, n
+    typ, dims, data = p["tensors"]["blk.1.ffn_down_exps.weight"]
+    assert typ == 12 and dims == [cfg.ffn_expert, cfg.n_embd, cfg.n_expert]
+    assert p["tensors"]["output_norm.weight"][1] == [cfg.n_embd]
+    assert p["tensors"]["token_embd.weight"][:2] == (1, [cfg.n_embd, cfg.vocab])
+    for n, (typ, dims, data) in p["tensors"].items():
+        assert np.array_equal(np.frombuffer(data, np.uint8), m.download(n).view(np.uint8)), n
+
+
+def test_checkpoint_reads_back_bit_for_bit_and_decodes_the_same_tokens(saved):
+    m, cfg, path = saved
+    r = LA.LLM(small_cfg(n_layer=1, n_expert=2, vocab=7), gguf=path)   # the shape comes from the file
+    try:
+        for f, _ in LA.Config._fields_:
+            if f not in ("layers", "no_head", "attn_splits", "max_tokens", "slots", "head_rows", "speculative", "spec_rows"):
+                assert getattr(r.cfg, f) == getattr(cfg, f), f
+        a, b = m.tensors(), r.tensors()
+        assert [t[0] for t in a] == [t[0] for t in b]
+        for t in a:
+            assert np.array_equal(m.download(t[0]).view(np.uint8), r.download(t[0]).view(np.uint8)), t[0]
+        r.stage()
+        prompt = np.random.default_rng(3).integers(0, cfg.vocab, size=9).astype(np.int32)
+        lg0, ids0 = _greedy(m, prompt, 16)
+        lg1, ids1 = _greedy(r, prompt, 16)
+        assert np.array_equal(lg0.view(np.uint32), lg1.view(np.uint32))
+        assert np.array_equal(ids0, ids1)
+    finally:
+        r.close()
+
+
+def test_split_checkpoint_loads_like_a_whole_one(saved, tmp_path):
+    m, cfg, path = saved
+    p = GF.parse(path)
+    names = list(p["tensors"])
+    cut = [names[:len(names) // 3], names[len(names) // 3:2 * len(names) // 3], names[2 * len(names) // 3:]]
+    for i, part in enumerate(cut):
+        extra = [("split.no", i), ("split.count", 3), ("split.tensors.count", len(names))]
+        q = dict(p, kv=p["kv"] if i == 0 else {})
+        _rewrite(q, tmp_path / ("m-%05d-of-00003.gguf" % (i + 1)), drop=set(names) - set(part), extra_kv=extra)
+    r = LA.LLM(small_cfg(), gguf=tmp_path / "m-00002-of-00003.gguf")
+    try:
+        for t in m.tensors():
+            assert np.array_equal(m.download(t[0]).view(np.uint8), r.download(t[0]).view(np.uint8)), t[0]
+    finally:
+        r.close()
+
+
+def test_float_tensors_of_other_types_are_expanded_on_the_device(saved, tmp_path):
+    m, cfg, path = saved
+    p = GF.parse(path)
+    swap = {}
+
+    def as_type(name, typ):
+        _, dims, data = p["tensors"][name]
+        v = np.frombuffer(data, np.float32)
+        if typ == 1:
+            raw = v.astype(np.float16).view(np.uint8)
+        elif typ == 30:
+            raw = (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+        else:       # Q8_0 blocks of 32: d = max|x| / 127
+            blk = v.reshape(-1, 32)
+            d = (np.abs(blk).max(axis=1) / 127).astype(np.float16)
+            q = np.round(blk / np.maximum(d.astype(np.float32), 1e-30)[:, None]).clip(-127, 127).astype(np.int8)
+            raw = np.concatenate([d.view(np.uint8).reshape(-1, 2), q.view(np.uint8)], axis=1).reshape(-1)
+        swap[name] = (typ, dims, raw.tobytes())
+
+    as_type("output_norm.weight", 30)
+    as_type("blk.0.attn_norm.weight", 1)
+    as_type("blk.2.ffn_gate_inp.weight", 8)
+    as_type("blk.1.ssm_conv1d.weight", 1)
+    r = LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "mixed.gguf", tensors=swap))
+    try:
+        for name, (typ, dims, raw) in swap.items():
+            want = O.dequant(typ, np.frombuffer(raw, np.uint8), int(np.prod(dims)))
+            assert np.array_equal(r.download(name).view(np.uint32), want.view(np.uint32)), name
+        assert np.array_equal(r.download("blk.1.attn_norm.weight"), m.download("blk.1.attn_norm.weight"))
+    finally:
+        r.close()
+
+
+def test_load_refuses_what_it_cannot_stage(saved, tmp_path):
+    m, cfg, path = saved
+    p = GF.parse(path)
+    with pytest.raises(ShvError, match=r"rows of blk\.3\.attn_qkv_fused"):
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "nok.gguf", drop={"blk.3.attn_k.weight"}))
+    with pytest.raises(ShvError, match=r"0 of 1 rows of output_norm"):
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "nonorm.gguf", drop={"output_norm.weight"}))
+    _, dims, data = p["tensors"]["blk.0.ffn_up_shexp.weight"]
+    n = int(np.prod(dims))
+    q8 = (8, dims, bytes(n // 32 * 34))
+    with pytest.raises(ShvError, match="Q8_0 in the checkpoint; the kernels stream it as Q4_K"):
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "q8.gguf", tensors={"blk.0.ffn_up_shexp.weight": q8}))
+    short = (0, [cfg.n_embd // 2], bytes(cfg.n_embd * 2))
+    with pytest.raises(ShvError, match="the metadata makes it"):
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "shape.gguf", tensors={"output_norm.weight": short}))
+    q = dict(p, kv={k: v for k, v in p["kv"].items() if k != "qwen3next.ssm.state_size"})
+    with pytest.raises(ShvError, match="states no qwen3next.ssm.state_size"):
+        LA.LLM(small_cfg(), gguf=_rewrite(q, tmp_path / "nokey.gguf"))
+    q = dict(p, kv={k: v for k, v in p["kv"].items() if k != "general.architecture"})
+    with pytest.raises(ShvError, match="no general.architecture"):
+        LA.LLM(small_cfg(), gguf=_rewrite(q, tmp_path / "noarch.gguf"))
+
+
+@pytest.mark.parametrize("name", ["Q8_0", "Q6_K", "Q5_K", "IQ4_NL", "BF16"])
+def test_gemv_over_a_mapped_tensor(ctx, tmp_path, name):
+    """A tensor's bytes straight from the mapping into HBM and through the any-type GEMV, against
+    matvec over the CPU's dequantised rows (llm/hc.go:255-264)."""
+    typ, n, k = O.GGML_TYPES[name], 96, 1024
+    w = GF.Writer()
+    w.tensor("pad", 0, [3], bytes(12))                   # pushes the next tensor off the file's natural alignment
+    w.tensor("w", typ, [k, n], random_tensor(name, n * k, seed=typ + 9).tobytes())
+    with G.GGUF(w.write(tmp_path / "w.gguf")) as f:
+        t = f.get("w")
+        assert t.type == typ and t.rows == n and t.dims[0] == k
+        x = np.random.default_rng(1).standard_normal(k).astype(np.float32)
+        y = ctx.alloc(n * 4)
+        ctx.gemv(t.type, ctx.upload(np.array(t.data())), ctx.upload(x), y, n, k)
+        want = O.dequant(typ, np.array(t.data()), n * k).reshape(n, k).astype(np.float64) @ x
+        assert O.rel_l2(y.read(np.float32, n), want) <= 1e-5
