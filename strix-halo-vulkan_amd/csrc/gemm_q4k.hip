@@ -18,6 +18,9 @@
 //                   any exchange:  y += d*sc*acc - (64*d*sc + dmin*m)*sum(x).
 // Waves do not talk to one another while they stream, except that a matrix with few rows is also
 // split along its columns (KS waves a tile), whose partial tiles meet in LDS at the end.
+#include <algorithm>
+#include <cstdlib>
+
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
 
@@ -26,6 +29,7 @@ namespace {
 using namespace shv;
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kTileRows = 16;
@@ -165,8 +169,42 @@ __device__ __forceinline__ void stage(const shv_gemv_q4k_args &a, int t0, int nt
     }
 }
 
-// grid: blocks of NTHR/64 waves.  KS consecutive waves share a row tile, each over 1/KS of the
-// columns.  t0: first activation row of this launch, nt: how many (<= TT).
+// pro(x) of the four columns c..c+3 of activation row t; `scale` is the row's RMSNorm factor.
+// Every lane of a wave calls it for the same row (the gated norm adds up across lanes).
+__device__ __forceinline__ void pro_quad(const shv_gemv_q4k_args &a, int t, int c, float scale, float (&x)[4]) {
+    const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+    const float4 v = *reinterpret_cast<const float4 *>(a.x + static_cast<size_t>(t) * a.x_stride + c);
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    if (a.prologue == SHV_PRO_RMSNORM) {
+        const float4 g = *reinterpret_cast<const float4 *>(a.gamma + c);
+        x[0] *= scale * g.x; x[1] *= scale * g.y; x[2] *= scale * g.z; x[3] *= scale * g.w;
+    } else if (a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID) {
+        const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
+        if (a.z_ring) {
+            const int s = t / sl, k = t % sl;
+            const int p = a.pos ? a.pos[s] : 0;
+            const int slot = a.slot ? a.slot[s] : s;
+            z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
+        }
+        const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0 ? (c & ~(a.head_dim - 1)) * 2 + a.head_dim + (c & (a.head_dim - 1)) : c;
+        const float4 zq = *reinterpret_cast<const float4 *>(z + zi);
+        const float zz[4] = {zq.x, zq.y, zq.z, zq.w};
+        if (a.prologue == SHV_PRO_GATED_NORM) {
+            float ss = fmaf(x[0], x[0], fmaf(x[1], x[1], fmaf(x[2], x[2], x[3] * x[3])));
+            const int span = a.head_dim / 4;  // lanes a head spans: a power of two up to 64
+            for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
+            const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
+            const float4 g4 = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
+            const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) x[j] = x[j] * scale * gg[j] * sigmoid_fast(zz[j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) x[j] *= sigmoid_fast(zz[j]);
+        }
+    }
+}
+
 // The activations of a pass of many rows transformed once, for every block of the products to
 // copy.  grid: (k/256, groups of `cap` rows), 256 threads: a block takes one super-block's worth of
 // columns of its group's rows, a wave one row's 64 quads at a time, and writes fragments and sums
@@ -182,7 +220,6 @@ __global__ __launch_bounds__(256) void gemm_stage_kernel(shv_gemv_q4k_args a, ch
     const int nt = a.n_tok - t0 < cap ? a.n_tok - t0 : cap;
     char *frags = staged + static_cast<size_t>(grp) * Lds<TT>::region(K);
     float *sxs = reinterpret_cast<float *>(frags + Lds<TT>::frag_bytes(K));
-    const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
     if (a.prologue == SHV_PRO_RMSNORM) {
         for (int tl = wave; tl < nt; tl += 4) {
             const float *x = a.x + static_cast<size_t>(t0 + tl) * a.x_stride;
@@ -198,37 +235,8 @@ __global__ __launch_bounds__(256) void gemm_stage_kernel(shv_gemv_q4k_args a, ch
     }
     for (int tl = wave; tl < nt; tl += 4) {
         const int t = t0 + tl, c = kp * 256 + 4 * lane;
-        const float4 v = *reinterpret_cast<const float4 *>(a.x + static_cast<size_t>(t) * a.x_stride + c);
-        float x[4] = {v.x, v.y, v.z, v.w};
-        if (a.prologue == SHV_PRO_RMSNORM) {
-            const float scale = scale_s[tl];
-            const float4 g = *reinterpret_cast<const float4 *>(a.gamma + c);
-            x[0] *= scale * g.x; x[1] *= scale * g.y; x[2] *= scale * g.z; x[3] *= scale * g.w;
-        } else if (a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID) {
-            const float *z = a.z + static_cast<size_t>(t) * a.z_stride;
-            if (a.z_ring) {
-                const int s = t / sl, k = t % sl;
-                const int p = a.pos ? a.pos[s] : 0;
-                const int slot = a.slot ? a.slot[s] : s;
-                z = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
-            }
-            const int zi = a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim > 0 ? (c & ~(a.head_dim - 1)) * 2 + a.head_dim + (c & (a.head_dim - 1)) : c;
-            const float4 zq = *reinterpret_cast<const float4 *>(z + zi);
-            const float zz[4] = {zq.x, zq.y, zq.z, zq.w};
-            if (a.prologue == SHV_PRO_GATED_NORM) {
-                float ss = fmaf(x[0], x[0], fmaf(x[1], x[1], fmaf(x[2], x[2], x[3] * x[3])));
-                const int span = a.head_dim / 4;  // lanes a head spans: a power of two up to 64
-                for (int off = 1; off < span; off <<= 1) ss += __shfl_xor(ss, off, 64);
-                const float scale = 1.f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
-                const float4 g4 = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
-                const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
-#pragma unroll
-                for (int j = 0; j < 4; j++) x[j] = x[j] * scale * gg[j] * sigmoid_fast(zz[j]);
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; j++) x[j] *= sigmoid_fast(zz[j]);
-            }
-        }
+        float x[4];
+        pro_quad(a, t, c, a.prologue == SHV_PRO_RMSNORM ? scale_s[tl] : 1.f, x);
         // the sub-block's sum of x: eight neighbouring lanes
         float sum = (x[0] + x[1]) + (x[2] + x[3]);
         sum += __shfl_xor(sum, 1, 64);
@@ -251,6 +259,8 @@ __global__ __launch_bounds__(256) void gemm_stage_kernel(shv_gemv_q4k_args a, ch
     }
 }
 
+// grid: blocks of NTHR/64 waves.  KS consecutive waves share a row tile, each over 1/KS of the
+// columns.  t0: first activation row of this launch, nt: how many (<= TT).
 template <int TT, int NTHR, int MAXQ>
 __global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int t0, int nt, int n_tiles, int ks, const char *staged) {
     extern __shared__ __align__(16) char smem[];
@@ -401,6 +411,267 @@ __global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int
     }
 }
 
+// ---------------------------------------------------------------- passes of 17 to 64 rows -------
+// A prompt chunk has more rows than one block can keep in LDS for the whole width of the matrix,
+// so its operands stream: the activations of 64 rows are made once into `staged` as slabs of 128
+// columns (four sub-blocks), each slab in the order the products read it, and every block of the
+// product walks the slabs through two LDS buffers while its waves stream their own weight rows.
+// A wave owns 32 weight rows (two tiles) and all 64 activation rows (four tiles): one
+// v_mfma_f32_16x16x32_f16 per (tile, tile, half of x) covers a whole 32-column sub-block, whose
+// eight levels a lane already holds in the 8 payload bytes it loaded.  A matrix with few rows is
+// also split along its columns over blockIdx.y; the parts meet in a second small launch.
+constexpr int kWideTok = 64;                                 // activation rows of a launch
+constexpr int kWideFrag = 64 * 16;                           // one operand: a lane's eight halves
+constexpr int kWideSlabA = 4 * 4 * 2 * kWideFrag;            // [sub-block 4][token tile 4][hi, lo]
+constexpr int kWideSlab = kWideSlabA + 4 * kWideTok * 4;     // + the sub-blocks' sums of x
+
+__host__ __device__ constexpr size_t wide_region(int k) { return static_cast<size_t>(k / 128) * kWideSlab; }
+
+// Where activation row t of the pass writes its outputs: the DeltaNet projection ring, or plain rows.
+__device__ __forceinline__ size_t out_offset(const shv_gemv_q4k_args &a, int t) {
+    if (a.ring_slots > 0 && !a.z_ring) {
+        const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+        const int s = t / sl, i = t % sl;
+        const int p = a.pos ? a.pos[s] : 0;
+        const int slot = a.slot ? a.slot[s] : s;
+        return (static_cast<size_t>(slot) * a.ring_slots + (p + i) % a.ring_slots) * a.ring_stride;
+    }
+    return static_cast<size_t>(t) * a.y_stride;
+}
+
+// The same for a pass of up to 64 rows a group, in the slab order gemm_wide_kernel streams.
+// grid: (k/256, 16 quartets of rows, groups of 64 rows), 256 threads: a wave takes one row's 64
+// quads of one super-block's columns; rows a group does not have are written as zeros.
+__global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args a, char *staged) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = a.k, kp = blockIdx.x, grp = blockIdx.z;
+    const int t0 = grp * kWideTok;
+    const int nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;
+    const int tl = blockIdx.y * 4 + wave;
+    char *region = staged + static_cast<size_t>(grp) * wide_region(K);
+    float scale = 1.f;
+    if (a.prologue == SHV_PRO_RMSNORM && tl < nt) {
+        // the row's factor needs the whole row: every wave adds up its own, in a fixed order
+        const float *x = a.x + static_cast<size_t>(t0 + tl) * a.x_stride;
+        float ss = 0.f;
+        for (int q = lane; q < K / 4; q += 64) {
+            const float4 v = *reinterpret_cast<const float4 *>(x + 4 * q);
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+        }
+        ss = wave_sum_all(ss);
+        scale = 1.f / sqrtf(ss / static_cast<float>(K) + a.eps);
+    }
+    const int c = kp * 256 + 4 * lane;
+    // the quad's place: slab of 128 columns, sub-block of it, k block of 8 columns, which half of those
+    char *slab = region + static_cast<size_t>(c >> 7) * kWideSlab;
+    const int sub = (c & 127) >> 5, kb = (c & 31) >> 3, qh = (c & 7) >> 2;
+    float x[4] = {0.f, 0.f, 0.f, 0.f};
+    if (tl < nt) pro_quad(a, t0 + tl, c, scale, x);
+    float sum = (x[0] + x[1]) + (x[2] + x[3]);
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    sum += __shfl_xor(sum, 4, 64);
+    if ((c & 31) == 0) reinterpret_cast<float *>(slab + kWideSlabA)[sub * kWideTok + tl] = sum;
+    // slot order of a lane's eight columns: [0, 2, 1, 3, 4, 6, 5, 7]
+    const float o[4] = {x[0], x[2], x[1], x[3]};
+    half4_t h, l;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const _Float16 hi = static_cast<_Float16>(o[j]);
+        h[j] = hi;
+        l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+    }
+    char *e = slab + static_cast<size_t>((sub * 4 + (tl >> 4)) * 2) * kWideFrag + (kb * 16 + (tl & 15)) * 16 + qh * 8;
+    *reinterpret_cast<half4_t *>(e) = h;
+    *reinterpret_cast<half4_t *>(e + kWideFrag) = l;
+}
+
+struct WideLoads {
+    uint4 hdr;
+    uint2 q[2];
+    // step: which 128 columns of the row; the two 64-weight groups of that half of a super-block
+    __device__ __forceinline__ void load(const char *row, int step, int kb) {
+        const char *sb = row + static_cast<size_t>(step >> 1) * SHV_Q4K_BYTES;
+        hdr = *reinterpret_cast<const uint4 *>(sb);
+#pragma unroll
+        for (int g = 0; g < 2; g++) q[g] = *reinterpret_cast<const uint2 *>(sb + 16 + ((step & 1) * 2 + g) * 32 + kb * 8);
+    }
+};
+
+// grid: (row groups of NW * R * 16 rows, column parts); NW waves, each owning R row tiles.
+// part: [parts][64][n] partial products when the columns are split, else unused.
+template <int NW, int kWideR>
+__global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a, int t0, int nt, const char *staged, float *part, int steps_per) {
+    extern __shared__ __align__(16) char smem[];
+    size_t *yoffs = reinterpret_cast<size_t *>(smem + 2 * kWideSlab);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, kb = lane >> 4;
+    const int sbs = a.k / SHV_Q4K_BLOCK;
+    const size_t row_bytes = static_cast<size_t>(sbs) * SHV_Q4K_BYTES;
+    const int s0 = blockIdx.y * steps_per, s1 = s0 + steps_per;
+    constexpr int NTHR = NW * 64;
+    const int row0 = (blockIdx.x * NW + wave) * (kWideR * kTileRows);
+    const int ntt = (nt + kTileRows - 1) / kTileRows;
+
+    const char *rp[kWideR];
+    WideLoads w[kWideR];
+#pragma unroll
+    for (int r = 0; r < kWideR; r++) {
+        const int row = row0 + r * kTileRows + n;
+        rp[r] = static_cast<const char *>(a.w) + static_cast<size_t>(row < a.n ? row : a.n - 1) * row_bytes;
+        w[r].load(rp[r], s0, kb);
+    }
+    if (tid < nt) yoffs[tid] = out_offset(a, t0 + tid);
+    constexpr int kVec = kWideSlab / 16;  // 16-byte pieces of a slab
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(staged + static_cast<size_t>(s0) * kWideSlab);
+        uint4 *dst = reinterpret_cast<uint4 *>(smem);
+        for (int i = tid; i < kVec; i += NTHR) dst[i] = src[i];
+    }
+    __syncthreads();
+
+    const NibbleConsts nc = nibble_consts();
+    float4_t y[kWideR][4];
+#pragma unroll
+    for (int r = 0; r < kWideR; r++)
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) y[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int s = s0; s < s1; s++) {
+        const int cur = (s - s0) & 1;
+        const bool more = s + 1 < s1;
+        // the next slab and the next weights are requested before this step's products
+        // a slab is kPer pieces of 16 bytes a thread, and the sums one more for the first 64 threads
+        constexpr int kPer = kWideSlabA / 16 / NTHR;
+        static_assert(kPer * NTHR * 16 == kWideSlabA && kVec - kPer * NTHR == 64, "slab copy layout");
+        // (the last step asks for its own slab again, so that the loads are unconditional)
+        uint4 an[kPer], asx;
+        WideLoads wn[kWideR];
+        {
+            const int sn = more ? s + 1 : s;
+            const uint4 *src = reinterpret_cast<const uint4 *>(staged + static_cast<size_t>(sn) * kWideSlab);
+#pragma unroll
+            for (int i = 0; i < kPer; i++) an[i] = src[tid + i * NTHR];
+            asx = src[kPer * NTHR + (tid & 63)];
+#pragma unroll
+            for (int r = 0; r < kWideR; r++) wn[r].load(rp[r], sn, kb);
+        }
+        const char *A = smem + cur * kWideSlab;
+        const float *sxs = reinterpret_cast<const float *>(A + kWideSlabA);
+        float dd[kWideR], dmin[kWideR];
+#pragma unroll
+        for (int r = 0; r < kWideR; r++) {
+            dd[r] = f16_bits_to_f32(w[r].hdr.x);
+            dmin[r] = f16_bits_to_f32(w[r].hdr.x >> 16);
+        }
+#pragma unroll
+        for (int sub = 0; sub < 4; sub++) {
+            const int g = sub >> 1, hi = sub & 1;
+            half8_t b[kWideR];
+            float ds[kWideR], e[kWideR];
+#pragma unroll
+            for (int r = 0; r < kWideR; r++) {
+                uint32_t sc, mn;
+                q4k_group_scale_min(w[r].hdr, (s & 1) * 2 + g, sc, mn);
+                const uint32_t q0 = w[r].q[g].x, q1 = w[r].q[g].y;
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                u32x4 v;
+                // slot order of the eight columns: bytes [0, 2, 1, 3, 4, 6, 5, 7]
+                if (hi == 0) {
+                    v.x = ((q0 << 4) & nc.mask) | nc.one; v.y = ((q0 >> 4) & nc.mask) | nc.one;
+                    v.z = ((q1 << 4) & nc.mask) | nc.one; v.w = ((q1 >> 4) & nc.mask) | nc.one;
+                } else {
+                    v.x = (q0 & nc.mask) | nc.one; v.y = ((q0 >> 8) & nc.mask) | nc.one;
+                    v.z = (q1 & nc.mask) | nc.one; v.w = ((q1 >> 8) & nc.mask) | nc.one;
+                }
+                b[r] = __builtin_bit_cast(half8_t, v);
+                ds[r] = dd[r] * static_cast<float>(hi ? sc >> 8 : sc & 0xFFu);
+                e[r] = fmaf(64.f, ds[r], dmin[r] * static_cast<float>(hi ? mn >> 8 : mn & 0xFFu));
+            }
+#pragma unroll
+            for (int tt = 0; tt < 4; tt++) {
+                if (tt < ntt) {
+                    const char *f = A + static_cast<size_t>((sub * 4 + tt) * 2) * kWideFrag + lane * 16;
+                    const half8_t xh = *reinterpret_cast<const half8_t *>(f);
+                    const half8_t xl = *reinterpret_cast<const half8_t *>(f + kWideFrag);
+                    const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * kWideTok + tt * kTileRows + 4 * kb);
+                    const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
+#pragma unroll
+                    for (int r = 0; r < kWideR; r++) {
+                        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc, 0, 0, 0);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(-e[r], sxv[j], fmaf(ds[r], acc[j], y[r][tt][j]));
+                    }
+                }
+            }
+        }
+        if (more) {
+            // the other buffer was last read a step ago, before the barrier that ended that step
+            uint4 *dst = reinterpret_cast<uint4 *>(smem + (cur ^ 1) * kWideSlab);
+#pragma unroll
+            for (int i = 0; i < kPer; i++) dst[tid + i * NTHR] = an[i];
+            if (tid < 64) dst[kPer * NTHR + tid] = asx;
+#pragma unroll
+            for (int r = 0; r < kWideR; r++) w[r] = wn[r];
+        }
+        __syncthreads();
+    }
+
+    // C[token 16 tt + 4 kb + j][row n] of each tile
+#pragma unroll
+    for (int r = 0; r < kWideR; r++) {
+        const int row = row0 + r * kTileRows + n;
+        if (row >= a.n) continue;
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int tok = tt * kTileRows + 4 * kb + j;
+                if (tok >= nt) continue;
+                float v = y[r][tt][j];
+                if (gridDim.y > 1) {
+                    part[(static_cast<size_t>(blockIdx.y) * kWideTok + tok) * a.n + row] = v;
+                } else {
+                    if (a.residual) v += a.residual[static_cast<size_t>(t0 + tok) * a.y_stride + row];
+                    a.y[yoffs[tok] + row] = v;
+                }
+            }
+        }
+    }
+}
+
+// The column parts of a split product added up in a fixed order.  grid: (ceil(n/256), nt), one
+// wave a block; a thread takes four neighbouring outputs, with 16-byte moves when the row count
+// and the addresses allow them.
+__global__ __launch_bounds__(64) void gemm_wide_join_kernel(shv_gemv_q4k_args a, int t0, const float *part, int parts, int vec) {
+    const int tok = blockIdx.y;
+    const size_t yo = out_offset(a, t0 + tok);
+    const int row = (blockIdx.x * 64 + threadIdx.x) * 4;
+    if (row >= a.n) return;
+    if (vec) {
+        float4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (int p = 0; p < parts; p++) {
+            const float4 o = *reinterpret_cast<const float4 *>(part + (static_cast<size_t>(p) * kWideTok + tok) * a.n + row);
+            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+        }
+        if (a.residual) {
+            const float4 r = *reinterpret_cast<const float4 *>(a.residual + static_cast<size_t>(t0 + tok) * a.y_stride + row);
+            v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
+        }
+        *reinterpret_cast<float4 *>(a.y + yo + row) = v;
+        return;
+    }
+    for (int i = 0; i < 4 && row + i < a.n; i++) {
+        float v = 0.f;
+        for (int p = 0; p < parts; p++) v += part[(static_cast<size_t>(p) * kWideTok + tok) * a.n + row + i];
+        if (a.residual) v += a.residual[static_cast<size_t>(t0 + tok) * a.y_stride + row + i];
+        a.y[yo + row + i] = v;
+    }
+}
+
 template <int TT, int NTHR, int MAXQ>
 int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const char *staged) {
     constexpr int NW = NTHR / 64;
@@ -441,6 +712,43 @@ int launch_stage(shv_ctx *ctx, const shv_gemv_q4k_args &a, int cap) {
     return SHV_OK;
 }
 
+// One group of up to 64 rows whose operands are already in `staged`.
+template <int NW, int R>
+int launch_wide(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const char *staged) {
+    constexpr int kRows = NW * R * kTileRows;
+    const int bx = (a.n + kRows - 1) / kRows;
+    const int steps = a.k / 128;
+    // few row groups: the columns are split too, as far as every part keeps two steps, the launch
+    // stays within one round of the chip (a block a compute unit, see below), and the parts fit
+    int ks = 1;
+    const int cus = ctx->prop.multiProcessorCount;
+    while (steps % (ks * 2) == 0 && steps / (ks * 2) >= 2 && bx * ks * 2 <= cus &&
+           static_cast<size_t>(ks * 2) * kWideTok * a.n * 4 <= static_cast<size_t>(shv_ctx::kGemmPartBytes))
+        ks *= 2;
+    if (const char *e = std::getenv("SHV_WIDE_KS")) {
+        const int want = std::atoi(e);
+        if (want >= 1 && steps % want == 0 && static_cast<size_t>(want) * kWideTok * a.n * 4 <= static_cast<size_t>(shv_ctx::kGemmPartBytes)) ks = want;
+    }
+    SHV_REQUIRE(ks == 1 || ctx->gemm_part, "gemm_q4k: no buffer for the parts of a split product");
+    // More than half a compute unit's LDS, so that two blocks never share one: a launch of fewer
+    // blocks than compute units would otherwise double up on some and leave others idle.
+    const size_t lds = std::max<size_t>(2 * kWideSlab + kWideTok * sizeof(size_t), 84 * 1024);
+    static bool raised = false;
+    if (!raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        raised = true;
+    }
+    SHV_LAUNCH(ctx, (gemm_wide_kernel<NW, R>), dim3(bx, ks), dim3(NW * 64), lds, a, t0, nt, staged, ctx->gemm_part, steps / ks);
+    if (ks > 1) {
+        // 16-byte moves need whole quads of outputs at 16-byte addresses in every row
+        const bool ring = a.ring_slots > 0 && !a.z_ring;
+        const int vec = a.n % 4 == 0 && shv_aligned16(a.y) && (ring ? a.ring_stride % 4 == 0 : a.y_stride % 4 == 0) &&
+                        (!a.residual || (shv_aligned16(a.residual) && a.y_stride % 4 == 0));
+        SHV_LAUNCH(ctx, gemm_wide_join_kernel, dim3((a.n + 255) / 256, nt), dim3(64), 0, a, t0, ctx->gemm_part, ks, vec);
+    }
+    return SHV_OK;
+}
+
 }  // namespace
 
 // Whether the matrix-core kernel takes this call: arguments are already validated by the GEMV's
@@ -465,6 +773,22 @@ bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a) {
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     // the fragments of 16 rows of 4096 columns do not fit LDS: such a pass goes 8 rows at a time
     const int cap = a.k > 2048 ? 8 : 16;
+    // more rows than one block keeps in LDS: groups of 64 stream their operands
+    if (a.n_tok > cap && ctx->gemm_stage && (a.prologue != SHV_PRO_GATED_NORM || 256 % a.head_dim == 0)) {
+        const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
+        SHV_REQUIRE(groups * wide_region(a.k) <= static_cast<size_t>(shv_ctx::kGemmStageBytes), "gemm_q4k: %d rows of %d columns do not fit the staging buffer", a.n_tok, a.k);
+        SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(a.k / 256, kWideTok / 4, groups), dim3(256), 0, a, ctx->gemm_stage);
+        for (int g = 0; g < groups; g++) {
+            const int t0 = g * kWideTok;
+            const int nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;
+            const char *st = ctx->gemm_stage + static_cast<size_t>(g) * wide_region(a.k);
+            // many rows: sixteen waves a block keep a compute unit's matrix cores and vector units
+            // both busy; a matrix of few rows needs smaller blocks to spread over the chip
+            const int rc = a.n >= 8192 ? launch_wide<16, 1>(ctx, a, t0, nt, st) : launch_wide<8, 1>(ctx, a, t0, nt, st);
+            if (rc != SHV_OK) return rc;
+        }
+        return SHV_OK;
+    }
     // A pass of several groups of rows, or of wide rows, has its activations transformed once, by
     // a launch of its own, instead of by every block of the products (hundreds of them): the
     // groups of `cap` rows are staged with the tile size their product will use.  One group of

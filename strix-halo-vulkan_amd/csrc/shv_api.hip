@@ -50,6 +50,7 @@ int shv_init(int device, shv_ctx **out) {
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->counters), ctx->n_counters * sizeof(int32_t));
     if (e == hipSuccess) e = hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->gemm_stage), shv_ctx::kGemmStageBytes);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->gemm_part), shv_ctx::kGemmPartBytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_val), shv_ctx::kArgmaxBlocks * sizeof(float));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_idx), shv_ctx::kArgmaxBlocks * sizeof(int32_t));
     if (e != hipSuccess) {
@@ -72,6 +73,7 @@ void shv_destroy(shv_ctx *ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->gemm_stage) (void)hipFree(ctx->gemm_stage);
+    if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
     if (ctx->argmax_val) (void)hipFree(ctx->argmax_val);
     if (ctx->argmax_idx) (void)hipFree(ctx->argmax_idx);
     for (hipEvent_t ev : ctx->mark_pool) (void)hipEventDestroy(ev);

@@ -30,7 +30,10 @@ struct shv_ctx {
     // activations of a many-row projection, transformed once into matrix-core operand order and
     // copied from here by every block (kGemmStageBytes covers 64 rows of 4096 columns)
     char *gemm_stage = nullptr;
-    enum { kGemmStageBytes = 2 << 20 };
+    enum { kGemmStageBytes = 4 << 20 };
+    // partial products of a pass whose columns are split over blocks: [parts][64 rows][n] floats
+    float *gemm_part = nullptr;
+    enum { kGemmPartBytes = 16 << 20 };
     // per-block partial results of the arg-max reduction: (value, index) pairs
     float *argmax_val = nullptr;
     int32_t *argmax_idx = nullptr;

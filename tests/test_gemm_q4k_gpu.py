@@ -47,7 +47,11 @@ def row_ctx():
 
 @pytest.mark.parametrize("n,k,rows", [(1024, 2048, 2), (4096, 2048, 3), (2048, 4096, 4), (2048, 512, 16),
                                       (48, 1024, 5), (7, 2048, 2), (33, 256, 9), (12352, 2048, 16),
-                                      (2048, 4096, 17), (512, 2048, 40)])
+                                      (2048, 4096, 17), (512, 2048, 40),
+                                      # passes of more rows than a block keeps in LDS stream their operands:
+                                      # whole and ragged groups of 64, split columns, rows not a multiple of 128
+                                      (12352, 2048, 64), (2048, 4096, 64), (9216, 2048, 33), (1000, 1024, 50),
+                                      (512, 2048, 57), (2048, 4096, 9), (40, 256, 20)])
 def test_rows_match_oracle_and_float64(ctx, row_ctx, n, k, rows):
     rng = np.random.default_rng(n + k + rows)
     wq = _weights(rng, n, k)
@@ -71,11 +75,12 @@ def test_rows_match_oracle_and_float64(ctx, row_ctx, n, k, rows):
     print(f"gemm {n}x{k} x{rows}: worst rel-L2 vs float64 {worst:.2e}")
 
 
-def test_rmsnorm_prologue_residual_in_place(ctx):
+@pytest.mark.parametrize("rows", [3, 64])
+def test_rmsnorm_prologue_residual_in_place(ctx, rows):
     """The residual stream's own rows are the residual and the destination (dn.out, attn.out, the
     MoE down projection write x in place)."""
     rng = np.random.default_rng(31)
-    n, k, rows, eps = 2048, 2048, 3, 1e-6
+    n, k, eps = 2048, 2048, 1e-6
     wq = _weights(rng, n, k)
     h = (rng.standard_normal((rows, k)) * 3).astype(np.float32)
     gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
@@ -89,11 +94,12 @@ def test_rmsnorm_prologue_residual_in_place(ctx):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx):
+@pytest.mark.parametrize("rows,slots", [(4, 8), (37, 64)])
+def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx, rows, slots):
     """DeltaNet's output projection at its real shape: 4096 columns (two column ranges), per-head
     norm, the gate z read from the projection ring at each row's position, residual in place."""
     rng = np.random.default_rng(32)
-    n, k, d, eps, rows, slots = 2048, 4096, 128, 1e-6, 4, 8
+    n, k, d, eps = 2048, 4096, 128, 1e-6
     ring_stride, z_col = 12352, 8192
     wq = _weights(rng, n, k)
     o = rng.standard_normal((rows, k)).astype(np.float32)
@@ -116,11 +122,12 @@ def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-def test_sigmoid_gate_prologue_with_fused_query_rows(ctx):
+@pytest.mark.parametrize("rows", [3, 64])
+def test_sigmoid_gate_prologue_with_fused_query_rows(ctx, rows):
     """Attention's output projection: x * sigmoid(gate), the gate being the second half of each
     head's [q | gate] rows in the fused projection (llm/attn.go:162-166,198-205)."""
     rng = np.random.default_rng(33)
-    n, k, d, rows = 2048, 4096, 256, 3
+    n, k, d = 2048, 4096, 256
     heads, zw = k // d, 2 * k + 1024
     wq = _weights(rng, n, k)
     c = rng.standard_normal((rows, k)).astype(np.float32)
@@ -137,11 +144,12 @@ def test_sigmoid_gate_prologue_with_fused_query_rows(ctx):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-def test_ring_output_for_sequences_and_slots(ctx):
+@pytest.mark.parametrize("seq_len,slots", [(3, 8), (20, 32)])
+def test_ring_output_for_sequences_and_slots(ctx, seq_len, slots):
     """The DeltaNet input projection writes each row into its sequence's ring at its position:
     here two sequences of three rows each, on slots 2 and 0, wrapping around an 8-row ring."""
     rng = np.random.default_rng(34)
-    n, k, slots, n_slots, seq_len = 528, 2048, 8, 3, 3
+    n, k, n_slots = 528, 2048, 3
     wq = _weights(rng, n, k)
     x = rng.standard_normal((2 * seq_len, k)).astype(np.float32)
     pos, slot = np.array([6, 17], np.int32), np.array([2, 0], np.int32)
