@@ -289,7 +289,7 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "moe_up_hbm_traffic.json")
     if os.path.exists(tpath) and (cfg.n_embd, cfg.n_expert_used, cfg.ffn_expert) == (2048, 10, 512):
         traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
-    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048> (expert-gathered Q4_K gate/up GEMV + SwiGLU)",
+    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048, 1> (expert-gathered Q4_K gate/up GEMV + SwiGLU)",
             "achieved": round(up_bytes / (up_ns / 1e9) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": round(up_bytes / (up_ns / 1e9) / HBM_PEAK, 4), "traffic": traffic,
             "bytes_per_launch": up_bytes, "avg_launch_us": round(up_ns / 1e3, 3), "launches_per_step": cfg.n_layer}

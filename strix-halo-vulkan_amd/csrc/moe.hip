@@ -303,9 +303,11 @@ __global__ __launch_bounds__(64) void moe_route_kernel(shv_moe_router_args a) {
 
 // ------------------------------------------------------------------------------- up ----------
 
-// grid: (ffn/RPP/4 row groups, n_used+1 slots, n_tok).  One pass per wave: RPP gate rows and the
-// same RPP up rows of one expert, six 16-byte loads per lane in flight together.
-template <int K>
+// grid: (ffn/RPP/4/P row groups, n_used+1 slots, n_tok).  A pass of a wave is RPP gate rows and the
+// same RPP up rows of one expert, six 16-byte loads per lane in flight together.  P: passes a wave
+// makes over the staged activation row; a launch of many tokens has blocks to spare and uses
+// them to stage the row an eighth as often (64-row chunk: 148 to 119 us a layer).
+template <int K, int P>
 __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
@@ -316,8 +318,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int slot = blockIdx.y, t = blockIdx.z;
     const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
-    const int row = (blockIdx.x * 4 + wave) * RPP + rsub;  // row within the expert
-    const bool live = row < a.ffn;
+    const int row0 = (blockIdx.x * 4 + wave) * P * RPP + rsub;  // row within the expert, first pass
 
     // the activation row is requested before anything else and staged further down
     const float *x = a.xn + static_cast<size_t>(t) * K;
@@ -349,10 +350,12 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
         gbase = static_cast<const char *>(a.gate_sh);
         ubase = static_cast<const char *>(a.up_sh);
     }
-    const size_t roff = static_cast<size_t>(live ? row : 0) * ROWB + sb * SHV_Q4K_BYTES;
-    Q4kLane wg, wu;
-    wg.load(gbase + roff, g);
-    wu.load(ubase + roff, g);
+    Q4kLane wg[2], wu[2];
+    {
+        const size_t roff = static_cast<size_t>(row0 < a.ffn ? row0 : 0) * ROWB + sb * SHV_Q4K_BYTES;
+        wg[0].load(gbase + roff, g);
+        wu[0].load(ubase + roff, g);
+    }
 
 #pragma unroll
     for (int i = 0; i < K / kBlock; i++) xs[lds_slot(tid + i * kBlock)] = xv[i];
@@ -360,54 +363,62 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     float xr[64], xs_lo, xs_hi;
     load_x_slice(xs, gi, xr, xs_lo, xs_hi);
     const NibbleConsts nc = nibble_consts();
-    float gv = wg.dot(g, nc, xr, xs_lo, xs_hi);
-    float uv = wu.dot(g, nc, xr, xs_lo, xs_hi);
-    gv = group_sum<LPR>(gv);
-    uv = group_sum<LPR>(uv);
-    if (live && group_sum_owner<LPR>(lane)) {
-        const float s = gv * sigmoid_exact(gv);
-        a.act[(static_cast<size_t>(t) * (a.n_used + 1) + slot) * a.ffn + row] = s * uv;
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        const int row = row0 + p * RPP;
+        if (p + 1 < P) {
+            // the next pass's weights are on their way while this pass multiplies
+            const size_t roff = static_cast<size_t>(row + RPP < a.ffn ? row + RPP : 0) * ROWB + sb * SHV_Q4K_BYTES;
+            wg[(p + 1) & 1].load(gbase + roff, g);
+            wu[(p + 1) & 1].load(ubase + roff, g);
+        }
+        float gv = wg[p & 1].dot(g, nc, xr, xs_lo, xs_hi);
+        float uv = wu[p & 1].dot(g, nc, xr, xs_lo, xs_hi);
+        gv = group_sum<LPR>(gv);
+        uv = group_sum<LPR>(uv);
+        if (row < a.ffn && group_sum_owner<LPR>(lane)) {
+            const float s = gv * sigmoid_exact(gv);
+            a.act[(static_cast<size_t>(t) * (a.n_used + 1) + slot) * a.ffn + row] = s * uv;
+        }
     }
 }
 
 // ------------------------------------------------------------------------------ down ---------
 
-// grid: (n_embd/RPP row groups, n_tok).  A block owns RPP output rows of one token; its four
+// grid: (n_embd/RPP/P row groups, n_tok).  A block owns P * RPP output rows of one token; its four
 // waves split the n_used+1 slots, each lane scales its partial dot by the slot's weight, and the
-// block adds the four waves' sums (and the residual) at the end.
-template <int K, int MAXS>
+// block adds the four waves' sums (and the residual) at the end.  P: passes over the staged
+// activation rows, as in the up projection (two for many tokens; more costs registers and is slower).
+template <int K, int MAXS, int P>
 __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int SPW = (MAXS + 3) / 4;  // slots per wave
     __shared__ __align__(16) float xs[MAXS][lds_padded(K)];
-    __shared__ float part[4][RPP];
+    __shared__ float part[4][P * RPP];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t = blockIdx.y;
     const int ns = a.n_used + 1;
     const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
-    const int row = blockIdx.x * RPP + rsub;
-    const bool live = row < a.n_embd;
-    const size_t roff = static_cast<size_t>(live ? row : 0) * ROWB + sb * SHV_Q4K_BYTES;
+    const int row0 = blockIdx.x * P * RPP + rsub;
     // the residual of the row this thread will write at the end is asked for now
     float res = 0.f;
-    if (a.residual && tid < RPP && blockIdx.x * RPP + tid < a.n_embd) res = a.residual[static_cast<size_t>(t) * a.res_stride + blockIdx.x * RPP + tid];
+    if (a.residual && tid < P * RPP && blockIdx.x * P * RPP + tid < a.n_embd) res = a.residual[static_cast<size_t>(t) * a.res_stride + blockIdx.x * P * RPP + tid];
 
-    Q4kLane w[SPW];
+    Q4kLane w[2][SPW];
     float wt[SPW];
+    const char *base[SPW];
 #pragma unroll
     for (int i = 0; i < SPW; i++) {
         const int s = wave + 4 * i;
         wt[i] = 0.f;
+        base[i] = static_cast<const char *>(a.down_sh);
         if (s < ns) {
-            const char *base;
             if (s < a.n_used) {
                 const int e = a.topk[static_cast<size_t>(t) * a.n_used + s];
-                base = static_cast<const char *>(a.down_exps) + static_cast<size_t>(e) * a.n_embd * ROWB;
-            } else {
-                base = static_cast<const char *>(a.down_sh);
+                base[i] = static_cast<const char *>(a.down_exps) + static_cast<size_t>(e) * a.n_embd * ROWB;
             }
-            w[i].load(base + roff, g);
+            w[0][i].load(base[i] + static_cast<size_t>(row0 < a.n_embd ? row0 : 0) * ROWB + sb * SHV_Q4K_BYTES, g);
             wt[i] = a.weights[static_cast<size_t>(t) * ns + s];
         }
     }
@@ -438,21 +449,32 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
     __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
 
     const NibbleConsts nc = nibble_consts();
-    float acc = 0.f;
 #pragma unroll
-    for (int i = 0; i < SPW; i++) {
-        const int s = wave + 4 * i;
-        if (s < ns) {
-            float xr[64], xs_lo, xs_hi;
-            load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
-            acc = fmaf(wt[i], w[i].dot(g, nc, xr, xs_lo, xs_hi), acc);
+    for (int p = 0; p < P; p++) {
+        const int row = row0 + p * RPP;
+        if (p + 1 < P) {
+            // the next pass's weights are on their way while this pass multiplies
+            const size_t roff = static_cast<size_t>(row + RPP < a.n_embd ? row + RPP : 0) * ROWB + sb * SHV_Q4K_BYTES;
+#pragma unroll
+            for (int i = 0; i < SPW; i++)
+                if (wave + 4 * i < ns) w[(p + 1) & 1][i].load(base[i] + roff, g);
         }
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < SPW; i++) {
+            const int s = wave + 4 * i;
+            if (s < ns) {
+                float xr[64], xs_lo, xs_hi;
+                load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
+                acc = fmaf(wt[i], w[p & 1][i].dot(g, nc, xr, xs_lo, xs_hi), acc);
+            }
+        }
+        acc = group_sum<LPR>(acc);
+        if (group_sum_owner<LPR>(lane)) part[wave][p * RPP + rsub] = acc;
     }
-    acc = group_sum<LPR>(acc);
-    if (group_sum_owner<LPR>(lane)) part[wave][rsub] = acc;
     __syncthreads();
-    if (tid < RPP) {
-        const int r = blockIdx.x * RPP + tid;
+    if (tid < P * RPP) {
+        const int r = blockIdx.x * P * RPP + tid;
         if (r < a.n_embd) {
             float v = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
             a.out[static_cast<size_t>(t) * a.out_stride + r] = v + res;
@@ -498,23 +520,41 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
                 "moe_up: weight banks must be 16-byte aligned");
     dim3 block(kBlock);
+    // enough tokens to fill the chip with blocks eight passes tall; not when the blocks route
+    // for themselves, which they do once per block
+    const bool many = a.n_tok >= ctx->moe_tall_min && !a.logits;
     switch (a.n_embd) {
         case 2048: {
             constexpr int RPP = 64 / (2048 / 64);
-            dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            SHV_LAUNCH(ctx, moe_up_kernel<2048>, grid, block, 0, a);
+            if (many) {
+                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), a.n_used + 1, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 8>), grid, block, 0, a);
+            } else {
+                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 1>), grid, block, 0, a);
+            }
             break;
         }
         case 1024: {
             constexpr int RPP = 64 / (1024 / 64);
-            dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            SHV_LAUNCH(ctx, moe_up_kernel<1024>, grid, block, 0, a);
+            if (many) {
+                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), a.n_used + 1, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<1024, 8>), grid, block, 0, a);
+            } else {
+                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<1024, 1>), grid, block, 0, a);
+            }
             break;
         }
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
-            dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-            SHV_LAUNCH(ctx, moe_up_kernel<512>, grid, block, 0, a);
+            if (many) {
+                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), a.n_used + 1, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<512, 8>), grid, block, 0, a);
+            } else {
+                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<512, 1>), grid, block, 0, a);
+            }
             break;
         }
         default: return shv_set_error(SHV_E_INVALID, "moe_up: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
@@ -533,12 +573,14 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     switch (a.ffn) {
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
-            SHV_LAUNCH(ctx, (moe_down_kernel<512, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
+            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 2>), dim3((a.n_embd + RPP * 2 - 1) / (RPP * 2), a.n_tok), block, 0, a);
+            else SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
             break;
         }
         case 256: {
             constexpr int RPP = 64 / (256 / 64);
-            SHV_LAUNCH(ctx, (moe_down_kernel<256, 12>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
+            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 2>), dim3((a.n_embd + RPP * 2 - 1) / (RPP * 2), a.n_tok), block, 0, a);
+            else SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
             break;
         }
         default: return shv_set_error(SHV_E_INVALID, "moe_down: ffn = %d; built for 256 and 512", a.ffn);

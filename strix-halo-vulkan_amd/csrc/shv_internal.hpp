@@ -23,6 +23,7 @@ struct shv_ctx {
     // operands).  SHV_MFMA_MIN_ROWS in the environment sets both; a large value keeps every pass
     // on the row kernel.
     int mfma_min_rows = 3, mfma_min_rows_wide = 5;
+    int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
     int32_t *counters = nullptr;
