@@ -97,6 +97,29 @@ int shvllm_spec_round(shvllm *h, const int32_t *forced, int n_forced, int32_t *o
  * nanos: draft, verify */
 int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos);
 
+/* ---- the host sampler (llm.Sampler, llm/sample.go): penalties -> top_k -> top_p -> min_p -> temp -> draw,
+ * and speculative sampling's Verify.  No device involved; rows are host floats and come back unchanged. ---- */
+typedef struct shvsampler shvsampler;
+shvsampler *shvsampler_new(float temp, int top_k, float top_p, int64_t seed);   /* NewSampler */
+void shvsampler_free(shvsampler *s);
+void shvsampler_set(shvsampler *s, float min_p, float repeat_penalty, float presence_penalty);
+int shvsampler_greedy(shvsampler *s);
+void shvsampler_accept(shvsampler *s, const int32_t *ids, int n);
+int32_t shvsampler_sample(shvsampler *s, float *logits, int n);
+/* the distribution Sample draws from, most likely first; returns its length (ids/p take up to max) */
+int shvsampler_dist(shvsampler *s, float *logits, int n, int32_t *ids, float *p, int max);
+shvsampler *shvsampler_draft(shvsampler *s, int64_t seed);                       /* DraftSampler; NULL when greedy */
+int32_t shvsampler_propose(shvsampler *s, float *logits, int n);                 /* keeps its distribution in s */
+int shvsampler_last_dist(shvsampler *s, int32_t *ids, float *p, int max);
+/* Verify against the distribution of proposer's last propose; proposer NULL (or greedy) is Sample */
+int32_t shvsampler_verify(shvsampler *s, float *logits, int n, int32_t draft, shvsampler *proposer);
+/* loops for the distribution tests: counts[id]++ per draw; speculate_many returns how often the draft was kept */
+void shvsampler_sample_many(shvsampler *s, float *logits, int n, int draws, int32_t *counts);
+int64_t shvsampler_speculate_many(shvsampler *s, shvsampler *ds, float *pl, float *ql, int n, int draws, int32_t *counts);
+int32_t shvsampler_argmax(const float *logits, int n);
+int shvsampler_top_n(const float *logits, int n, int k, int32_t *dst);
+int shvsampler_top_k_of(const float *logits, int n, int k, int32_t *dst);
+
 /* ---- the GGUF container by itself (package gguf, gguf/gguf.go): no device involved ---------- */
 typedef struct shvgguf shvgguf;
 int shvgguf_open(const char *path, shvgguf **out);   /* OpenSet: a file, any shard, or a directory */
