@@ -301,6 +301,120 @@ __global__ __launch_bounds__(64) void moe_route_kernel(shv_moe_router_args a) {
     if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(lg[a.n_expert]) : 0.f;
 }
 
+// The same selection with a thread per expert (grid: n_tok blocks of 512 threads): the one wave
+// above spends most of its 4 us in dependent instructions (eight exponentials, eight ballots, the
+// candidates' ranks), which eight waves do side by side.  Same rule: probabilities as the
+// reference forms them, the n_used largest in descending order with ties to the lower index,
+// their sum in slot order clamped at 2^-14.  The threshold is the n_used-th largest of the 16
+// half-wave maxima; the few keys at or above it are compacted and ranked by the first wave.
+// Rows with more than 64 candidates (many equal probabilities) take the one-wave road.
+constexpr int kRouteBlock = 512;
+__global__ __launch_bounds__(kRouteBlock) void moe_route_block_kernel(shv_moe_router_args a) {
+    __shared__ __align__(16) float probs[192];  // the one-wave road's scratch
+    __shared__ float s_max[8], s_sum[8];
+    __shared__ uint32_t s_gm[16];
+    __shared__ uint32_t s_thr;
+    __shared__ int s_cnt[8];
+    __shared__ uint32_t cand_p[64];
+    __shared__ int32_t cand_e[64];
+    __shared__ int32_t sel_e[kMaxUsed];
+    __shared__ float sel_w[kMaxUsed];
+    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
+    float *wt = a.weights + static_cast<size_t>(t) * (a.n_used + 1);
+    int32_t *topk = a.topk + static_cast<size_t>(t) * a.n_used;
+    const int e = tid;
+    const bool has = e < a.n_expert;
+    const float l = has ? lg[e] : -INFINITY;
+    // the shared gate's logit is asked for with the rest
+    const float lsh = (tid == kRouteBlock - 1 && a.shared_gate) ? lg[a.n_expert] : 0.f;
+    float mx = wave_max_all(l);
+    if (lane == 0) s_max[wave] = mx;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < 8; w++) mx = fmaxf(mx, s_max[w]);
+    const float ex = has ? expf(l - mx) : 0.f;
+    const float ws = wave_sum_all(ex);
+    if (lane == 0) s_sum[wave] = ws;
+    // half-wave maxima of the unnormalised exponentials give the same threshold as the
+    // probabilities' would (one common positive factor), but the keys compared below are the
+    // probabilities themselves, as the reference's are
+    __syncthreads();
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) sum += s_sum[w];
+    const float inv = 1.f / sum;
+    const uint32_t kh = has ? __float_as_uint(ex * inv) : 0u;
+    uint32_t gm = kh;
+#pragma unroll
+    for (int off = 1; off < 32; off <<= 1) {
+        const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(gm), off, 64));
+        gm = o > gm ? o : gm;
+    }
+    if ((lane & 31) == 0) s_gm[tid >> 5] = gm;
+    if (tid == 0) s_thr = 0u;
+    __syncthreads();
+    if (tid < 16) {
+        const uint32_t mine = s_gm[tid];
+        int rank = 0;
+#pragma unroll
+        for (int j = 0; j < 16; j++) rank += (s_gm[j] > mine || (s_gm[j] == mine && j < tid)) ? 1 : 0;
+        if (rank == a.n_used - 1) s_thr = mine;
+    }
+    __syncthreads();
+    const uint32_t thr = s_thr;
+    const bool pred = has && kh >= thr;
+    const unsigned long long mask = __ballot(pred);
+    if (lane == 0) s_cnt[wave] = __popcll(mask);
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        before += w < wave ? s_cnt[w] : 0;
+        total += s_cnt[w];
+    }
+    if (total > 64 || a.n_expert < 64 || a.n_used > 16) {
+        // uniform over the block: many equal probabilities, or a shape the threshold does not cover
+        if (wave == 0) {
+            route_token<8, false>(lg, a.n_expert, a.n_used, topk, wt, probs);
+            if (lane == 0) wt[a.n_used] = a.shared_gate ? sigmoid_exact(lg[a.n_expert]) : 0.f;
+        }
+        return;
+    }
+    if (pred) {
+        const int pos = before + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)));
+        cand_p[pos] = kh;
+        cand_e[pos] = e;
+    }
+    if (tid == kRouteBlock - 1) wt[a.n_used] = a.shared_gate ? sigmoid_exact(lsh) : 0.f;
+    __syncthreads();
+    if (wave != 0) return;
+    // candidates are in expert order; rank of candidate j = how many come before it (as in route_token)
+    const uint32_t my_p = lane < total ? cand_p[lane] : 0u;
+    const int my_e = lane < total ? cand_e[lane] : 0x7FFFFFFF;
+    int rank = 0;
+    for (int j = 0; j < total; j++) {
+        const uint32_t pj = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_p), j));
+        const int ej = __builtin_amdgcn_readlane(my_e, j);
+        const int bef = __popcll(__ballot(my_p > pj || (my_p == pj && my_e < ej)));
+        rank = lane == j ? bef : rank;
+    }
+    if (lane < total && rank < a.n_used) {
+        sel_e[rank] = my_e;
+        sel_w[rank] = __uint_as_float(my_p);
+    }
+    __builtin_amdgcn_wave_barrier();
+    const float w_mine = lane < a.n_used ? sel_w[lane] : 0.f;
+    const int32_t e_mine = lane < a.n_used ? sel_e[lane] : 0;
+    float wsum = 0.f;
+    for (int k = 0; k < a.n_used; k++) wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_mine), k));
+    if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
+    if (lane < a.n_used) {
+        topk[lane] = e_mine;
+        wt[lane] = w_mine / wsum;
+    }
+}
+
 // ------------------------------------------------------------------------------- up ----------
 
 // grid: (ffn/RPP/4/P row groups, n_used+1 slots, n_tok).  A pass of a wave is RPP gate rows and the
@@ -503,7 +617,10 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     }
     // the selection needs every logit of the token, i.e. the whole grid above: a second, tiny
     // launch is cheaper than handing the logits to one block inside the first
-    if (!a.defer_route) SHV_LAUNCH(ctx, moe_route_kernel, dim3(a.n_tok), dim3(64), 0, a);
+    if (!a.defer_route) {
+        if (a.n_expert > 64 && a.n_expert <= kRouteBlock) SHV_LAUNCH(ctx, moe_route_block_kernel, dim3(a.n_tok), dim3(kRouteBlock), 0, a);
+        else SHV_LAUNCH(ctx, moe_route_kernel, dim3(a.n_tok), dim3(64), 0, a);
+    }
     return SHV_OK;
 }
 
