@@ -19,7 +19,6 @@
 // Waves do not talk to one another while they stream, except that a matrix with few rows is also
 // split along its columns (KS waves a tile), whose partial tiles meet in LDS at the end.
 #include <algorithm>
-#include <cstdlib>
 
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
@@ -725,10 +724,6 @@ int launch_wide(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const 
     while (steps % (ks * 2) == 0 && steps / (ks * 2) >= 2 && bx * ks * 2 <= cus &&
            static_cast<size_t>(ks * 2) * kWideTok * a.n * 4 <= static_cast<size_t>(shv_ctx::kGemmPartBytes))
         ks *= 2;
-    if (const char *e = std::getenv("SHV_WIDE_KS")) {
-        const int want = std::atoi(e);
-        if (want >= 1 && steps % want == 0 && static_cast<size_t>(want) * kWideTok * a.n * 4 <= static_cast<size_t>(shv_ctx::kGemmPartBytes)) ks = want;
-    }
     SHV_REQUIRE(ks == 1 || ctx->gemm_part, "gemm_q4k: no buffer for the parts of a split product");
     // More than half a compute unit's LDS, so that two blocks never share one: a launch of fewer
     // blocks than compute units would otherwise double up on some and leave others idle.
