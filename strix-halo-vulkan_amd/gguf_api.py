@@ -121,7 +121,7 @@ class GGUF:
         for i in range(self.L.shvgguf_files(self.h)):
             p, v, a, d = C.c_char_p(), C.c_uint32(), C.c_uint64(), C.c_int64()
             llm_api._check(self.L.shvgguf_file_info(self.h, i, C.byref(p), C.byref(v), C.byref(a), C.byref(d)))
-            out.append(dict(path=p.value.decode(), version=v.value, alignment=a.value, data_start=d.value))
+            out.append(dict(path=p.value.decode("utf-8", "replace"), version=v.value, alignment=a.value, data_start=d.value))
         return out
 
     def __len__(self):
@@ -134,14 +134,14 @@ class GGUF:
         return self.L.shvgguf_bytes(self.h)
 
     def arch(self):
-        return self.L.shvgguf_arch(self.h).decode()
+        return self.L.shvgguf_arch(self.h).decode("utf-8", "replace")
 
     def tensor_at(self, i):
         name, typ, nd, dims = C.c_char_p(), C.c_uint32(), C.c_int32(), (C.c_int64 * 4)()
         data, nb, shard, rows, rb = C.c_void_p(), C.c_uint64(), C.c_int32(), C.c_int64(), C.c_int64()
         llm_api._check(self.L.shvgguf_tensor_at(self.h, i, C.byref(name), C.byref(typ), C.byref(nd), dims, C.byref(data),
                                                 C.byref(nb), C.byref(shard), C.byref(rows), C.byref(rb)))
-        return Tensor(name.value.decode(), typ.value, list(dims[:nd.value]), data.value, nb.value, shard.value,
+        return Tensor(name.value.decode("utf-8", "replace"), typ.value, list(dims[:nd.value]), data.value, nb.value, shard.value,
                       rows.value, rb.value)
 
     def tensors(self):
@@ -157,7 +157,7 @@ class GGUF:
         return self.tensor_at(i)
 
     def keys(self):
-        return [self.L.shvgguf_key_at(self.h, i).decode() for i in range(self.L.shvgguf_key_count(self.h))]
+        return [self.L.shvgguf_key_at(self.h, i).decode("utf-8", "replace") for i in range(self.L.shvgguf_key_count(self.h))]
 
     def kind(self, key):
         return self.L.shvgguf_kind(self.h, key.encode())

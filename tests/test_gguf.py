@@ -282,3 +282,42 @@ def test_rows_of_a_mapped_tensor_dequantise_like_the_fixture(tmp_path, golden_di
             cols = t.dims[0]
             got = np.concatenate([O.dequant(t.type, np.array(t.row(i)), cols) for i in range(t.rows)])
             assert np.array_equal(got.view(np.uint32), want[t.name].view(np.uint32)), t.name
+
+
+def test_damaged_headers_are_refused_not_followed(tmp_path):
+    """A checkpoint is an untrusted file: whatever a header claims, the reader stays inside the
+    mapping.  2 000 files made from a good one by overwriting bytes of the header or cutting it
+    short either open (and then every tensor's span lies inside the file) or are refused."""
+    w = GF.Writer()
+    _sample(w)
+    good = bytearray(w.bytes())
+    header = good.index(b"\x11" * 64)          # the data section starts with token_embd's fill
+    rng = np.random.default_rng(99)
+    opened = refused = 0
+    for trial in range(2000):
+        b = bytearray(good)
+        for _ in range(int(rng.integers(1, 4))):
+            at = int(rng.integers(4, header))
+            b[at] = int(rng.integers(0, 256)) if trial % 3 else 0xFF
+        if trial % 5 == 0:
+            b = b[:int(rng.integers(24, len(b)))]
+        p = tmp_path / "f.gguf"
+        p.write_bytes(bytes(b))
+        try:
+            f = G.GGUF(p, single=True)
+        except ShvError:
+            refused += 1
+            continue
+        opened += 1
+        size = len(b)
+        start = f.files()[0]["data_start"]
+        for t in f.tensors():
+            d = t.data()
+            assert t.nbytes == G.size_of(t.type, t.elems()) and len(d) == t.nbytes
+            if t.nbytes:
+                int(d[0]), int(d[-1])          # both ends are readable
+        for k in f.keys():
+            f.kind(k), f.uint(k), f.str(k), f.strings(k)
+        assert 0 <= start <= size
+        f.close()
+    assert opened > 100 and refused > 100, (opened, refused)
