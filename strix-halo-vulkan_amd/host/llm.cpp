@@ -1497,6 +1497,11 @@ void MTPHead::RowsHost(const std::vector<float> &hs, const std::vector<int32_t> 
     }
 }
 
+void MTPHead::LastLogits(std::vector<float> *out) {
+    out->resize(vocab_ > 0 ? vocab_ : c_.VocabSize);
+    dev_.download(out->data(), logits_, out->size() * 4);
+}
+
 // --------------------------------------------------------------------------- Speculator -------
 
 Speculator::Speculator(Graph &g, MTPHead &d, int depth) : Depth(depth), g_(g), d_(d) {
@@ -1512,7 +1517,8 @@ int32_t Speculator::Start(const std::vector<int32_t> &prompt) {
     if (T < 1) throw Error("llm: Speculator.Start: no prompt");
     const size_t E = g_.GetModel().config().NEmbd;
     g_.Speculate(false);  // the prompt is committed as it runs
-    const float *res = g_.ForwardResidual(prompt, nullptr);
+    std::vector<float> logits;  // the prompt's last row, when a sampler will want it
+    const float *res = g_.ForwardResidual(prompt, sampler_ ? &logits : nullptr);
     // Prime (llm/spec.go:286-326): the draft's cell at position p is written from the trunk's
     // residual at p-1 and the token at p; cell 0 has nothing behind it and takes a zero residual.
     d_.Reset();
@@ -1526,8 +1532,15 @@ int32_t Speculator::Start(const std::vector<int32_t> &prompt) {
     // the trunk's residual after the last prompt row seeds the first round
     check(shv_copy(g_.Dev().ctx(), h_, res + static_cast<size_t>(T - 1) * E, E * 4), "seed");
     owe_x_.clear();
-    // the token the prompt's last row sampled sits one past the sequence's end
-    pend_ = g_.Generate(1, nullptr)[0];
+    if (sampler_) {
+        // the prompt enters the penalties' window, then its last row is sampled on the host
+        sampler_->Accept(prompt.data(), T);
+        pend_ = sampler_->Sample(logits.data(), static_cast<int>(logits.size()));
+        sampler_->Accept(&pend_, 1);
+    } else {
+        // the token the prompt's last row sampled sits one past the sequence's end
+        pend_ = g_.Generate(1, nullptr)[0];
+    }
     g_.Speculate(true);
     g_.SpeculateFirst(true);
     Stats = SpecStats();
@@ -1535,8 +1548,83 @@ int32_t Speculator::Start(const std::vector<int32_t> &prompt) {
     return pend_;
 }
 
+void Speculator::UseSampler(Sampler *s, int64_t draft_seed) {
+    if (!s || s->Greedy()) {
+        sampler_ = nullptr;
+        draft_sampler_.reset();
+        return;
+    }
+    sampler_ = s;
+    draft_sampler_ = s->DraftSampler(draft_seed);
+}
+
+// A round under a sampler (llm/spec.go:703-857 with llm/sample.go:183-250).  The passes are the
+// greedy round's; what differs is who names the tokens: each draft is a draw from the draft
+// sampler's distribution over the draft head's logits, each verified row goes through Verify.
+std::vector<int32_t> Speculator::sampled_round(const std::vector<int32_t> &forced) {
+    const size_t E = g_.GetModel().config().NEmbd;
+    const int V = g_.GetModel().config().VocabSize;
+    const int at = g_.Past();
+    const int owed = static_cast<int>(owe_x_.size());
+    const uint64_t d0 = d_.GPUNanos;
+    std::vector<int32_t> rows{pend_};
+    std::vector<int32_t> xs(owe_x_);
+    xs.push_back(pend_);
+    std::vector<Dist> q(Depth);
+    std::vector<bool> drawn(Depth, false);
+    std::vector<float> ql;
+    d_.Rows(h_, xs, at - owed, true);
+    for (int k = 0; k < Depth; k++) {
+        if (k > 0) {
+            std::vector<int32_t> one{rows[k]};
+            d_.Rows(d_.ResPort() + (k == 1 ? static_cast<size_t>(owed) * E : 0), one, at + k, true);
+        }
+        if (k < static_cast<int>(forced.size())) {
+            rows.push_back(forced[k]);  // not a draw from q: verified as a plain sample
+        } else {
+            d_.LastLogits(&ql);
+            rows.push_back(draft_sampler_->Propose(ql.data(), static_cast<int>(ql.size()), &q[k]));
+            drawn[k] = true;
+        }
+    }
+    Stats.DraftNanos += d_.GPUNanos - d0;
+
+    const uint64_t v0 = g_.Stats.GPUNanos;
+    std::vector<float> logits;
+    g_.ExtendRows(rows, &logits, nullptr);
+    Stats.VerifyNanos += g_.Stats.GPUNanos - v0;
+    const int n = static_cast<int>(rows.size());
+    Stats.Passes[std::min(n, 4)]++;
+    Stats.Rounds++;
+    if (n > 1) Stats.Drafted++;
+
+    std::vector<int32_t> out;
+    for (int i = 0; i < n; i++) {
+        float *row = logits.data() + static_cast<size_t>(i) * V;
+        int32_t tok;
+        if (i + 1 < n) tok = sampler_->Verify(row, V, rows[i + 1], drawn[i] ? &q[i] : nullptr);
+        else tok = sampler_->Sample(row, V);
+        sampler_->Accept(&tok, 1);
+        out.push_back(tok);
+        if (i + 1 == n) break;
+        Stats.DraftedAt[std::min(i, 3)]++;
+        if (rows[i + 1] != tok) break;
+        Stats.AcceptedAt[std::min(i, 3)]++;
+    }
+    const int keep = static_cast<int>(out.size());
+    if (keep > 1) Stats.Accepted++;
+    g_.Keep(keep);
+    check(shv_copy(g_.Dev().ctx(), h_, g_.ResPort(), static_cast<size_t>(keep) * E * 4), "seed");
+    owe_x_.assign(rows.begin() + 1, rows.begin() + keep);
+    d_.Rewind(std::min(d_.Past(), at + 1));
+    pend_ = out[keep - 1];
+    Stats.Tokens += keep;
+    return out;
+}
+
 std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced) {
     if (pend_ < 0) throw Error("llm: Speculator.Round before Start");
+    if (sampler_) return sampled_round(forced);
     const size_t E = g_.GetModel().config().NEmbd;
     const int at = g_.Past();
     const int owed = static_cast<int>(owe_x_.size());

@@ -12,11 +12,13 @@
 #include <cstdint>
 #include <functional>
 #include <map>
+#include <memory>
 #include <stdexcept>
 #include <string>
 #include <vector>
 
 #include "gguf.hpp"
+#include "sample.hpp"
 #include "shv_hip.h"
 
 namespace llm {
@@ -453,6 +455,7 @@ public:
     void RowsHost(const std::vector<float> &hs, const std::vector<int32_t> &ids, int pos, bool head,
                   std::vector<float> *logits, std::vector<float> *res);
     const float *ResPort() const { return x_; }  // [n][NEmbd] of the last call
+    void LastLogits(std::vector<float> *out);     // the last head call's logits, over the drafted prefix of the vocabulary
     int Past() const { return pasts_[slot_]; }
     void Rewind(int n);
     void Reset() { pasts_[slot_] = 0; }
@@ -485,9 +488,13 @@ struct SpecStats {
     uint64_t DraftNanos = 0, VerifyNanos = 0;
 };
 
-// llm.Speculator (llm/spec.go:221-857), greedy: the draft head proposes Depth tokens, one
-// verification pass of Depth+1 rows checks them, the longest agreeing prefix is kept.  Every token
-// it emits is the trunk's own arg-max over the trunk's own sequence.
+// llm.Speculator (llm/spec.go:221-857): the draft head proposes Depth tokens, one verification
+// pass of Depth+1 rows checks them, the longest agreeing prefix is kept.  Greedy by default: every
+// token it emits is the trunk's own arg-max over the trunk's own sequence.  With a sampler
+// (UseSampler) the draft draws its proposals from its own sampler's distribution q and the trunk
+// keeps each with probability min(1, p/q), else redraws from max(0, p - q) (Sampler::Verify), so
+// the tokens are distributed as the trunk's sampler's whatever the draft proposes; the rows'
+// logits then come to the host, where the reference keeps its sampler too.
 class Speculator {
 public:
     Speculator(Graph &g, MTPHead &d, int depth);
@@ -498,6 +505,9 @@ public:
     // not empty, replaces the draft head's proposals (the draft still runs): the reference's
     // `propose` hook, which tests use to drive every acceptance length.
     std::vector<int32_t> Round(const std::vector<int32_t> &forced = {});
+    // s == nullptr or a greedy sampler: back to arg-max.  The sampler is borrowed; the draft's is made
+    // from it (Sampler::DraftSampler) with its own seed.  Takes effect at the next Start.
+    void UseSampler(Sampler *s, int64_t draft_seed);
     void Stop() { g_.Speculate(false); }
     SpecStats Stats;
     int Depth;
@@ -508,6 +518,9 @@ private:
     int32_t pend_ = -1;
     float *h_ = nullptr;  // [Depth+1][NEmbd]: the owed rows' residuals, then the trunk's last one
     std::vector<int32_t> owe_x_;
+    Sampler *sampler_ = nullptr;
+    std::unique_ptr<Sampler> draft_sampler_;
+    std::vector<int32_t> sampled_round(const std::vector<int32_t> &forced);
 };
 
 }  // namespace llm

@@ -14,6 +14,7 @@ struct shvllm {
     std::unique_ptr<llm::Graph> graph;
     std::unique_ptr<llm::MTPHead> mtp;
     std::unique_ptr<llm::Speculator> spec;
+    std::unique_ptr<llm::Sampler> sampler;
     llm::GraphOpts opts;
     std::vector<std::string> names;
 };
@@ -382,6 +383,18 @@ int shvllm_mtp_past(shvllm *h) { return h && h->mtp ? h->mtp->Past() : -1; }
 
 int shvllm_spec_open(shvllm *h, int depth) {
     return guard([&] { h->spec = std::make_unique<llm::Speculator>(graph_of(h), mtp_of(h), depth); });
+}
+
+int shvllm_spec_sampler(shvllm *h, float temp, int top_k, float top_p, float min_p, float repeat_penalty, float presence_penalty,
+                        int64_t seed, int64_t draft_seed) {
+    return guard([&] {
+        llm::Speculator &sp = spec_of(h);
+        h->sampler = std::make_unique<llm::Sampler>(temp, top_k, top_p, seed);
+        h->sampler->MinP = min_p;
+        h->sampler->RepeatPenalty = repeat_penalty;
+        h->sampler->PresencePenalty = presence_penalty;
+        sp.UseSampler(h->sampler.get(), draft_seed);
+    });
 }
 
 int shvllm_spec_start(shvllm *h, const int32_t *prompt, int n, int32_t *first) {

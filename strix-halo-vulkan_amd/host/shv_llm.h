@@ -90,6 +90,10 @@ int shvllm_mtp_rows(shvllm *h, const float *hs, const int32_t *ids, int n, int p
 int shvllm_mtp_rewind(shvllm *h, int n);
 int shvllm_mtp_past(shvllm *h);
 int shvllm_spec_open(shvllm *h, int depth);
+/* the sampler the loop's tokens are drawn with (Sampler + DraftSampler + Verify); temp <= 0: greedy again.
+ * Call before shvllm_spec_start. */
+int shvllm_spec_sampler(shvllm *h, float temp, int top_k, float top_p, float min_p, float repeat_penalty, float presence_penalty,
+                        int64_t seed, int64_t draft_seed);
 int shvllm_spec_start(shvllm *h, const int32_t *prompt, int n, int32_t *first);
 /* one round; forced (n_forced of them, may be 0) replaces the draft head's proposals */
 int shvllm_spec_round(shvllm *h, const int32_t *forced, int n_forced, int32_t *out, int max, int *n_out);

@@ -99,6 +99,7 @@ def load():
     L.shvllm_mtp_stage.argtypes = [vp, C.c_int, C.c_int]
     L.shvllm_mtp_rows.argtypes = [vp, f32p, i32p, C.c_int, C.c_int, C.c_int, f32p, f32p]
     L.shvllm_spec_start.argtypes = [vp, i32p, C.c_int, i32p]
+    L.shvllm_spec_sampler.argtypes = [vp, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int64, C.c_int64]
     L.shvllm_spec_round.argtypes = [vp, i32p, C.c_int, i32p, C.c_int, C.POINTER(C.c_int)]
     L.shvllm_spec_stats.argtypes = [vp, i32p, C.POINTER(C.c_uint64)]
     _lib = L
@@ -344,6 +345,10 @@ class LLM:
 
     def spec_open(self, depth):
         _check(self.L.shvllm_spec_open(self.h, depth))
+
+    def spec_sampler(self, temp, top_k=0, top_p=0.0, min_p=0.0, repeat_penalty=1.0, presence_penalty=0.0, seed=0, draft_seed=1):
+        """Speculator.UseSampler: the loop's tokens are drawn (temp <= 0: arg-max again)."""
+        _check(self.L.shvllm_spec_sampler(self.h, temp, top_k, top_p, min_p, repeat_penalty, presence_penalty, seed, draft_seed))
 
     def spec_start(self, prompt):
         prompt = np.ascontiguousarray(prompt, dtype=np.int32)

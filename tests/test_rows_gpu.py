@@ -272,6 +272,55 @@ def test_speculative_loop_emits_the_greedy_sequence(rig, mode):
     assert list(m.ids()) == list(prompt) + out[:-1]
 
 
+def test_sampled_speculation(rig):
+    """The loop under a sampler (Speculator.UseSampler; llm/spec.go:703-857 with llm/sample.go:183-250):
+    drafts are draws from the draft sampler's distribution, rows go through Verify on the host.
+    top-k 1 at any temperature is the arg-max, so that loop is the greedy loop token for token,
+    round for round; at temperature 1 the run is a function of its seeds, and every token it emits is
+    one the trunk's own cuts allow at its position."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(23)
+    prompt = rng.integers(0, cfg.vocab, size=9).astype(np.int32)
+    n_new, depth = 20, ROWS - 1
+
+    def run(sampler):
+        fresh(m)
+        m.mtp_stage(max_tok=ROWS)
+        m.spec_open(depth)
+        if sampler:
+            m.spec_sampler(**sampler)
+        out = [m.spec_start(prompt)]
+        while len(out) < n_new:
+            out += list(m.spec_round())
+        st = m.spec_stats()
+        assert st["tokens"] == len(out) and m.past() == len(prompt) + len(out) - 1
+        assert list(m.ids()) == list(prompt) + out[:-1]
+        return out, st
+
+    greedy, st_g = run(None)
+    wall, st_w = run(dict(temp=0.8, top_k=1, seed=3, draft_seed=4))
+    assert wall == greedy and st_w["accepted_at"] == st_g["accepted_at"] and st_w["rounds"] == st_g["rounds"]
+    cold, _ = run(dict(temp=0.0, top_k=40, top_p=0.9))
+    assert cold == greedy
+
+    warm = dict(temp=1.0, top_k=6, seed=11, draft_seed=12)
+    a, _ = run(warm)
+    b, _ = run(warm)
+    c, _ = run(dict(warm, seed=13))
+    assert a == b and a != c and a != greedy
+    # each emitted token is among the trunk's most likely at its position (ten allowed for the six
+    # kept: a pass of other shape rounds a little differently)
+    for i in (0, 1, 5, 12, n_new - 1):
+        fresh(m)
+        lg, _ = m.extend(np.concatenate([prompt, np.array(a[:i], np.int32)]))
+        assert a[i] in np.argsort(-lg)[:10], i
+    # penalties reach the loop: a large presence penalty keeps a token from repeating inside the window
+    pen, _ = run(dict(temp=1.0, top_k=6, presence_penalty=50.0, seed=11, draft_seed=12))
+    assert len(set(pen)) == len(pen)
+    for t in prompt:
+        assert t not in pen
+
+
 def test_checkpoint_restore_is_the_shorter_sequence(rig):
     """Graph.Checkpoint / Restore (llm/graph.go:1004-1062): after going on past a checkpoint and
     coming back, the sequence continues exactly as one that never went on; a slot that no longer
