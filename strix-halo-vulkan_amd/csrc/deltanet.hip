@@ -157,6 +157,127 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
     if (!a.spec) *reinterpret_cast<float4 *>(srow) = s;
 }
 
+// The same step for calls of many rows (prompt chunks), where the groups' preparation - not the
+// rule - is most of the time of the kernel above: here four more waves prepare group g+1 into a
+// second set of LDS buffers while the four waves that hold the state walk group g, with one
+// block-wide barrier a group.  A preparing wave owns whole vectors (the 128 q or k channels of a
+// key head, two a lane), so the norms need no exchange between waves: waves 0/1 take q of rows
+// 0-3 / 4-7 of the group, waves 2/3 take k; wave 0 also makes the block's eight v channels of
+// every row, wave 1 the rows' decay and write strength.
+// grid: (128/8 row chunks, n_head_v, n_seq), 512 threads.
+__global__ __launch_bounds__(2 * kBlock) void dn_step_pipe_kernel(shv_dn_step_args a) {
+    __shared__ __align__(16) float qs[2][kPrep][kD];
+    __shared__ __align__(16) float ks[2][kPrep][kD];
+    __shared__ float vs[2][kPrep][kRowsPerBlock];
+    __shared__ float gb[2][kPrep][2];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;
+    const bool producer = tid >= kBlock;
+    const int chunk = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
+    const int slot = a.slot ? a.slot[seq] : seq;
+    const int pos0 = a.pos ? a.pos[seq] : 0;
+    const int hk = h % a.n_head_k;
+    const int qk = a.n_head_k * kD, vw = a.n_head_v * kD;
+    const int alpha_off = 2 * qk + 2 * vw, beta_off = alpha_off + a.n_head_v;
+    const float *ring = a.ring + static_cast<size_t>(slot) * a.ring_slots * a.ring_stride;
+    const int groups = (a.seq_len + kPrep - 1) / kPrep;
+
+    // ---- the preparing waves' constants ----
+    const int kind = wave >> 1, r0 = (wave & 1) * 4;       // q or k; first of the wave's four rows of a group
+    const int ch0 = (kind ? qk : 0) + hk * kD + lane, ch1 = ch0 + 64;
+    float4 tp0 = {0.f, 0.f, 0.f, 0.f}, tp1 = tp0;
+    if (producer) {
+        tp0 = *reinterpret_cast<const float4 *>(a.conv1d + static_cast<size_t>(ch0) * 4);
+        tp1 = *reinterpret_cast<const float4 *>(a.conv1d + static_cast<size_t>(ch1) * 4);
+    }
+    auto prepare = [&](int g) {
+        const int b = g & 1, i0 = g * kPrep;
+        const int nr = a.seq_len - i0 < kPrep ? a.seq_len - i0 : kPrep;
+        const int p0 = pos0 + i0;
+        // sliding window of the wave's four rows: positions p0 + r0 - 3 .. p0 + r0 + 3
+        float x0[7], x1[7];
+        int rs = (p0 + r0 + a.ring_slots - 3) % a.ring_slots;
+#pragma unroll
+        for (int jj = 0; jj < 7; jj++) {
+            const bool on = r0 + jj - 3 < nr && p0 + r0 + jj - 3 >= 0;
+            x0[jj] = on ? ring[static_cast<size_t>(rs) * a.ring_stride + ch0] : 0.f;
+            x1[jj] = on ? ring[static_cast<size_t>(rs) * a.ring_stride + ch1] : 0.f;
+            rs = rs + 1 == a.ring_slots ? 0 : rs + 1;
+        }
+        // the v channels and the gates are asked for before the q/k arithmetic
+        float cv = 0.f, g_alpha = 0.f, g_beta = 0.f;
+        const int vr_row = lane / kRowsPerBlock, vr = lane % kRowsPerBlock;
+        if (wave == 0 && vr_row < nr) cv = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, 2 * qk + h * kD + chunk * kRowsPerBlock + vr, p0 + vr_row);
+        if (wave == 1 && lane < nr) {
+            const float *row = ring + static_cast<size_t>((p0 + lane) % a.ring_slots) * a.ring_stride;
+            g_alpha = row[alpha_off + h];
+            g_beta = row[beta_off + h];
+        }
+        float (*dst)[kD] = kind ? ks[b] : qs[b];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            if (r0 + r >= nr) break;
+            float c0 = 0.f, c1 = 0.f;
+            c0 += x0[r] * tp0.x; c0 += x0[r + 1] * tp0.y; c0 += x0[r + 2] * tp0.z; c0 += x0[r + 3] * tp0.w;
+            c1 += x1[r] * tp1.x; c1 += x1[r + 1] * tp1.y; c1 += x1[r + 2] * tp1.z; c1 += x1[r + 3] * tp1.w;
+            const float a0 = c0 * sigmoid_exact(c0), a1 = c1 * sigmoid_exact(c1);
+            const float ssq = wave_sum_all(fmaf(a0, a0, a1 * a1));
+            const float nrm = a.qk_norm_max ? 1.f / fmaxf(sqrtf(ssq), a.eps) : 1.f / sqrtf(ssq + a.eps);
+            dst[r0 + r][lane] = a0 * nrm;
+            dst[r0 + r][lane + 64] = a1 * nrm;
+        }
+        if (wave == 0 && vr_row < nr) vs[b][vr_row][vr] = cv * sigmoid_exact(cv);
+        if (wave == 1 && lane < nr) {
+            const float asp = softplus_ref(g_alpha + a.dt_bias[h]);
+            gb[b][lane][0] = expf(asp * a.a[h]);
+            gb[b][lane][1] = sigmoid_exact(g_beta);
+        }
+    };
+
+    // ---- the state-holding waves' constants ----
+    const int rsub = lane >> 5, li = lane & 31;
+    const int jl = wave * 2 + rsub;
+    const int j = chunk * kRowsPerBlock + jl;
+    const int planes = a.n_planes > 1 ? a.n_planes : 1;
+    const int cur = a.plane ? static_cast<int>(static_cast<unsigned>(a.plane[slot]) % static_cast<unsigned>(planes)) : 0;
+    const size_t plane_floats = static_cast<size_t>(a.n_head_v) * kD * kD;
+    float *sslot = a.state + static_cast<size_t>(slot) * planes * plane_floats + (static_cast<size_t>(h) * kD + j) * kD + li * 4;
+    float *srow = sslot + cur * plane_floats;
+    float4 s = {0.f, 0.f, 0.f, 0.f};
+    if (!producer) s = *reinterpret_cast<const float4 *>(srow);
+    const float scale = 1.f / sqrtf(static_cast<float>(kD));
+
+    if (producer) prepare(0);
+    __syncthreads();
+    for (int g = 0; g < groups; g++) {
+        if (producer) {
+            if (g + 1 < groups) prepare(g + 1);
+        } else {
+            const int b = g & 1, i0 = g * kPrep;
+            const int nr = a.seq_len - i0 < kPrep ? a.seq_len - i0 : kPrep;
+            for (int r = 0; r < nr; r++) {
+                const int i = i0 + r;
+                const float4 k4 = *reinterpret_cast<const float4 *>(&ks[b][r][li * 4]);
+                const float4 q4 = *reinterpret_cast<const float4 *>(&qs[b][r][li * 4]);
+                const float gg = gb[b][r][0], beta = gb[b][r][1], vj = vs[b][r][jl];
+                s.x *= gg; s.y *= gg; s.z *= gg; s.w *= gg;
+                const float dk = sum32_all(fmaf(s.x, k4.x, fmaf(s.y, k4.y, fmaf(s.z, k4.z, s.w * k4.w))));
+                const float delta = (vj - dk) * beta;
+                s.x = fmaf(delta, k4.x, s.x);
+                s.y = fmaf(delta, k4.y, s.y);
+                s.z = fmaf(delta, k4.z, s.z);
+                s.w = fmaf(delta, k4.w, s.w);
+                const float oq = sum32_all(fmaf(s.x, q4.x, fmaf(s.y, q4.y, fmaf(s.z, q4.z, s.w * q4.w))));
+                if (li == 0)
+                    a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j] = oq * scale;
+                if (a.spec) *reinterpret_cast<float4 *>(sslot + ((cur + 1 + i) % planes) * plane_floats) = s;
+            }
+        }
+        __syncthreads();  // group g has been read, group g+1 is ready
+    }
+    if (!producer && !a.spec) *reinterpret_cast<float4 *>(srow) = s;
+}
+
 }  // namespace
 
 int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
@@ -175,6 +296,8 @@ int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
     SHV_REQUIRE(!a.spec || (a.n_planes > 1 && a.seq_len < a.n_planes), "dn_step: a rewindable pass of %d rows needs more than %d state planes",
                 a.seq_len, a.n_planes);
     dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
-    SHV_LAUNCH(ctx, dn_step_kernel, grid, dim3(kBlock), 0, a);
+    // more than one group of rows: preparation and rule overlap
+    if (a.seq_len > kPrep) SHV_LAUNCH(ctx, dn_step_pipe_kernel, grid, dim3(2 * kBlock), 0, a);
+    else SHV_LAUNCH(ctx, dn_step_kernel, grid, dim3(kBlock), 0, a);
     return SHV_OK;
 }

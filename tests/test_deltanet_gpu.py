@@ -138,24 +138,35 @@ def test_decode_step_with_random_state(ctx, B):
         assert O.rel_l2(got_state[b], s_state) <= TOL, b
 
 
-def test_three_rows_in_one_call_equal_three_calls(ctx):
-    """A multi-row pass over one sequence (the verify pass's shape) must walk the rows in order on
-    one state: same answer as three single steps."""
-    case = DnCase(ctx, seed=21)
+@pytest.mark.parametrize("T,slots,pos0", [(3, 8, 0), (8, 16, 0), (9, 16, 0), (37, 48, 0), (64, 80, 0), (21, 32, 27)])
+def test_rows_in_one_call_equal_single_steps(ctx, T, slots, pos0):
+    """A multi-row pass over one sequence (a verify pass, a prompt chunk) walks its rows in order
+    on one state: the CPU's answer row by row.  Up to eight rows go through the decode kernel, more
+    through the one whose extra waves prepare the next group of eight while the rule runs on this
+    one: whole and ragged groups, and a start in mid-sequence with the ring wrapping (history rows
+    at pos0-3..pos0-1, the state of a sequence that has already run)."""
+    case = DnCase(ctx, seed=21 + T)
     case.upload()
-    T, slots = 3, 8
-    xn = case.rng.standard_normal((T, case.H)).astype(np.float32)
-    conv_state = np.zeros((case.cw, 3), np.float32)
-    s_state = np.zeros((case.hv, case.d, case.d), np.float32)
+    rng = case.rng
+    xn = rng.standard_normal((T, case.H)).astype(np.float32)
+    hist = rng.standard_normal((3, case.width)).astype(np.float32) if pos0 else np.zeros((3, case.width), np.float32)
+    s0 = (rng.standard_normal((case.hv, case.d, case.d)) * 0.1).astype(np.float32) if pos0 else np.zeros((case.hv, case.d, case.d), np.float32)
+    conv_state = np.ascontiguousarray(hist[:, :case.cw].T)       # [cw][3], column 0 oldest
+    s_state = s0.copy()
     _, want_attn = case.oracle(xn, conv_state, s_state)
+    ring = np.zeros((slots, case.width), np.float32)
+    for i in range(3):
+        if pos0:
+            ring[(pos0 - 3 + i) % slots] = hist[i]
     c = ctx
-    d_ring = c.alloc(slots * case.width * 4).zero()
-    d_state = c.alloc(s_state.nbytes).zero()
+    d_ring, d_state = c.upload(ring), c.upload(s0)
     d_attn, d_res = c.alloc(T * case.vw * 4), c.alloc(T * case.H * 4)
-    ops = case.step_ops(c.upload(xn), d_ring, d_state, d_attn, d_res, c.upload(np.array([0], np.int32)),
+    ops = case.step_ops(c.upload(xn), d_ring, d_state, d_attn, d_res, c.upload(np.array([pos0], np.int32)),
                         None, 1, T, slots)[:2]
     c.dispatch_multi(ops)
-    assert O.rel_l2(d_attn.read(np.float32, T * case.vw).reshape(T, -1), want_attn) <= TOL
+    got = d_attn.read(np.float32, T * case.vw).reshape(T, -1)
+    for t in range(T):
+        assert O.rel_l2(got[t], want_attn[t]) <= TOL, t
     assert O.rel_l2(d_state.read(np.float32, s_state.size), s_state) <= TOL
 
 
