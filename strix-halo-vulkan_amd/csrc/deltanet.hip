@@ -158,21 +158,24 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
 }
 
 // The same step for calls of many rows (prompt chunks), where the groups' preparation - not the
-// rule - is most of the time of the kernel above: here four more waves prepare group g+1 into a
+// rule - is most of the time of the kernel above: here eight more waves prepare group g+1 into a
 // second set of LDS buffers while the four waves that hold the state walk group g, with one
 // block-wide barrier a group.  A preparing wave owns whole vectors (the 128 q or k channels of a
-// key head, two a lane), so the norms need no exchange between waves: waves 0/1 take q of rows
-// 0-3 / 4-7 of the group, waves 2/3 take k; wave 0 also makes the block's eight v channels of
-// every row, wave 1 the rows' decay and write strength.
-// grid: (128/8 row chunks, n_head_v, n_seq), 512 threads.
-__global__ __launch_bounds__(2 * kBlock) void dn_step_pipe_kernel(shv_dn_step_args a) {
+// key head, two a lane), so the norms need no exchange between waves: the first half of them
+// take q, two rows of the group each, the second half k; wave 0 also makes the block's eight v
+// channels of every row, wave 1 the rows' decay and write strength.
+// grid: (128/8 row chunks, n_head_v, n_seq), 256 + 64 * kPrepWaves threads.
+constexpr int kPrepWaves = 8;                       // half of them for q, half for k
+constexpr int kPrepRows = kPrep / (kPrepWaves / 2); // rows of a group a preparing wave takes
+__global__ __launch_bounds__(kBlock + 64 * kPrepWaves) void dn_step_pipe_kernel(shv_dn_step_args a) {
     __shared__ __align__(16) float qs[2][kPrep][kD];
     __shared__ __align__(16) float ks[2][kPrep][kD];
     __shared__ float vs[2][kPrep][kRowsPerBlock];
     __shared__ float gb[2][kPrep][2];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;
+    const int tid = threadIdx.x, lane = tid & 63;
     const bool producer = tid >= kBlock;
+    const int wave = producer ? (tid - kBlock) >> 6 : tid >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
     const int slot = a.slot ? a.slot[seq] : seq;
     const int pos0 = a.pos ? a.pos[seq] : 0;
@@ -183,7 +186,7 @@ __global__ __launch_bounds__(2 * kBlock) void dn_step_pipe_kernel(shv_dn_step_ar
     const int groups = (a.seq_len + kPrep - 1) / kPrep;
 
     // ---- the preparing waves' constants ----
-    const int kind = wave >> 1, r0 = (wave & 1) * 4;       // q or k; first of the wave's four rows of a group
+    const int kind = wave / (kPrepWaves / 2), r0 = (wave % (kPrepWaves / 2)) * kPrepRows;  // q or k; first of the wave's rows of a group
     const int ch0 = (kind ? qk : 0) + hk * kD + lane, ch1 = ch0 + 64;
     float4 tp0 = {0.f, 0.f, 0.f, 0.f}, tp1 = tp0;
     if (producer) {
@@ -194,11 +197,11 @@ __global__ __launch_bounds__(2 * kBlock) void dn_step_pipe_kernel(shv_dn_step_ar
         const int b = g & 1, i0 = g * kPrep;
         const int nr = a.seq_len - i0 < kPrep ? a.seq_len - i0 : kPrep;
         const int p0 = pos0 + i0;
-        // sliding window of the wave's four rows: positions p0 + r0 - 3 .. p0 + r0 + 3
-        float x0[7], x1[7];
+        // sliding window of the wave's rows: positions p0 + r0 - 3 .. p0 + r0 + kPrepRows - 1
+        float x0[kPrepRows + 3], x1[kPrepRows + 3];
         int rs = (p0 + r0 + a.ring_slots - 3) % a.ring_slots;
 #pragma unroll
-        for (int jj = 0; jj < 7; jj++) {
+        for (int jj = 0; jj < kPrepRows + 3; jj++) {
             const bool on = r0 + jj - 3 < nr && p0 + r0 + jj - 3 >= 0;
             x0[jj] = on ? ring[static_cast<size_t>(rs) * a.ring_stride + ch0] : 0.f;
             x1[jj] = on ? ring[static_cast<size_t>(rs) * a.ring_stride + ch1] : 0.f;
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(2 * kBlock) void dn_step_pipe_kernel(shv_dn_step_ar
         }
         float (*dst)[kD] = kind ? ks[b] : qs[b];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
+        for (int r = 0; r < kPrepRows; r++) {
             if (r0 + r >= nr) break;
             float c0 = 0.f, c1 = 0.f;
             c0 += x0[r] * tp0.x; c0 += x0[r + 1] * tp0.y; c0 += x0[r + 2] * tp0.z; c0 += x0[r + 3] * tp0.w;
@@ -297,7 +300,7 @@ int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
                 a.seq_len, a.n_planes);
     dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
     // more than one group of rows: preparation and rule overlap
-    if (a.seq_len > kPrep) SHV_LAUNCH(ctx, dn_step_pipe_kernel, grid, dim3(2 * kBlock), 0, a);
+    if (a.seq_len > kPrep) SHV_LAUNCH(ctx, dn_step_pipe_kernel, grid, dim3(kBlock + 64 * kPrepWaves), 0, a);
     else SHV_LAUNCH(ctx, dn_step_kernel, grid, dim3(kBlock), 0, a);
     return SHV_OK;
 }
