@@ -138,6 +138,49 @@ def gemv_rates(m, cfg, A, LA):
     out["config1_4096x2048"] = {"us": round(per * 1e6, 3), "GBps": round(alg / per / 1e9, 1),
                                 "frac_hbm_peak": round(alg / per / HBM_PEAK, 4),
                                 "distinct_matrices": int(copies), "rotating_MB": round(copies * mat_bytes / 1e6, 1)}
+    if not eager:
+        # The same GEMVs as four independent in-order streams (one context each, a quarter of the
+        # matrices each, replayed together): launches of different streams overlap, so this is the
+        # rate the kernel streams at when the 3.7 us of a dependent launch is not between every
+        # two of them - the token loop, whose launches do depend on one another, sees the figure above.
+        n_streams = 4
+        extra, pres, dys = [], [], []
+        try:
+            for s in range(n_streams):
+                c = ctx
+                if s > 0:
+                    cp = C.c_void_p()
+                    A.check(H.shv_init(0, C.byref(cp)))
+                    c = cp
+                    extra.append(cp)
+                dys_s = alloc(n * 4)
+                dys.append(dys_s)
+                sops = [A.make_op(A.OP_GEMV_Q4K, A.gemv_args(w, dx, dys_s, n, k)) for w in mats[s::n_streams]]
+                sarr = (A.Op * len(sops))(*sops)
+                pre = C.c_void_p()
+                A.check(H.shv_prerecord(c, sarr, len(sops), C.byref(pre)))
+                pres.append((c, pre))
+            reps = 10
+            for timed in (False, True):
+                for c, _ in pres:
+                    A.check(H.shv_sync(c))
+                t0 = time.perf_counter()
+                for _ in range(reps if timed else 2):
+                    for c, pre in pres:
+                        A.check(H.shv_prerecorded_launch(c, pre))
+                for c, _ in pres:
+                    A.check(H.shv_sync(c))
+                dt = time.perf_counter() - t0
+            per4 = dt / (reps * copies)
+            out["config1_4096x2048"]["four_streams"] = {"us_per_gemv": round(per4 * 1e6, 3), "GBps": round(alg / per4 / 1e9, 1),
+                                                        "frac_hbm_peak": round(alg / per4 / HBM_PEAK, 4)}
+        finally:
+            for c, pre in pres:
+                H.shv_prerecorded_destroy(c, pre)
+            for p in dys:
+                H.shv_free(ctx, p)
+            for c in extra:
+                H.shv_destroy(c)
     # the vocabulary projection as the token step sees it: cold.  Between two runs of it, 128 of
     # the 4.7 MB matrices above (600 MB, more than twice the Infinity Cache) go through.
     head = next(t for t in m.tensors() if t[0] == "output.weight")
