@@ -103,8 +103,11 @@ template <int R>
 __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_args a, int row00, int n_groups, int append) {
     __shared__ Smem sm;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int split = blockIdx.x, kvh = blockIdx.y;
-    const int seq = blockIdx.z / n_groups, row0 = row00 + R * (blockIdx.z % n_groups);
+    // the groups of a pass run over blockIdx.x, the fastest-varying index: the blocks that read one
+    // slice of the cache for different row pairs are dispatched next to one another (and so land
+    // a few on each die), and all but the first of a die find the slice in its L2
+    const int gz = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+    const int seq = gz / n_groups, row0 = row00 + R * (gz % n_groups);
     const int slot = a.slot ? a.slot[seq] : seq;
     const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the group's first row
     // the last group of a sequence with an odd number of rows holds one: its second row repeats
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
         sm.wl[wave][n] = l_run;
     }
     __syncthreads();  // everyone is done with the queries in sm.qf / sm.big
-    float *part_base = a.partial + ((static_cast<size_t>(blockIdx.z) * a.n_head_kv + kvh) * a.n_splits + split) * R * kRec;
+    float *part_base = a.partial + ((static_cast<size_t>(gz) * a.n_head_kv + kvh) * a.n_splits + split) * R * kRec;
 #pragma unroll
     for (int j = 0; j < R; j++) {
         // this lane's rows 4q..4q+3 belong to sequence row j when q/2 == j
@@ -450,7 +453,7 @@ __global__ __launch_bounds__(kBlock) void attn_append_kernel(shv_attn_decode_arg
 
 template <int R>
 int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_groups, int append) {
-    dim3 grid(a.n_splits, a.n_head_kv, a.n_seq * n_groups);
+    dim3 grid(a.n_seq * n_groups, a.n_head_kv, a.n_splits);
     SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, a, row0, n_groups, append);
     SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, a, row0, n_groups);
     return SHV_OK;
