@@ -96,9 +96,12 @@ struct Reader {
         }
         const uint32_t et = le<uint32_t>();
         const uint64_t cnt = le<uint64_t>();
-        if (cnt > n) throw Error(fmt("array of %llu elements exceeds the file", static_cast<unsigned long long>(cnt)));
         if (et == vtArray) throw Error("nested arrays are not in the GGUF grammar");
         if (et > vtF64) throw Error(fmt("unknown array element type %u", et));
+        // every element takes at least its fixed size of the bytes that are left, so a count the
+        // file cannot hold is refused before anything is reserved for it
+        static const uint8_t kSize[] = {1, 1, 2, 2, 4, 4, 4, 1, 8, 0, 8, 8, 8};
+        if (cnt > (n - o) / kSize[et]) throw Error(fmt("array of %llu elements exceeds the file", static_cast<unsigned long long>(cnt)));
         Value e;
         switch (et) {
             case vtStr: v.kind = Value::Strs; v.ss.reserve(cnt); break;

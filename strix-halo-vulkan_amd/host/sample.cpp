@@ -28,6 +28,7 @@ int32_t Argmax(const float *logits, int n) {
 
 void TopKOf(const float *logits, int n, int k, std::vector<int32_t> *dst) {
     dst->clear();
+    if (k <= 0) return;
     float thr = -std::numeric_limits<float>::infinity();
     for (int i = 0; i < n; i++) {
         const float v = logits[i];
@@ -44,6 +45,7 @@ void TopKOf(const float *logits, int n, int k, std::vector<int32_t> *dst) {
 }
 
 std::vector<int32_t> TopN(const float *logits, int n, int k) {
+    if (n <= 0 || k <= 0) return {};
     std::vector<int32_t> idx(n);
     std::iota(idx.begin(), idx.end(), 0);
     if (k > n) k = n;
@@ -92,6 +94,7 @@ void Sampler::restore(float *logits, const std::vector<Saved> &saved) {
 }
 
 int32_t Sampler::Sample(float *logits, int n) {
+    if (n <= 0) return -1;  // no row, no token
     std::vector<Saved> saved;
     penalise(logits, n, &saved);
     const int32_t id = Greedy() ? Argmax(logits, n) : draw(dist(logits, n));
@@ -100,6 +103,7 @@ int32_t Sampler::Sample(float *logits, int n) {
 }
 
 Dist Sampler::DistOf(float *logits, int n) {
+    if (n <= 0) return Dist{};
     std::vector<Saved> saved;
     penalise(logits, n, &saved);
     Dist d = dist(logits, n);
@@ -108,6 +112,10 @@ Dist Sampler::DistOf(float *logits, int n) {
 }
 
 int32_t Sampler::Propose(float *logits, int n, Dist *q) {
+    if (n <= 0) {
+        if (q) *q = Dist{};
+        return -1;
+    }
     if (Greedy()) {
         if (q) *q = Dist{};
         return Argmax(logits, n);
@@ -119,6 +127,7 @@ int32_t Sampler::Propose(float *logits, int n, Dist *q) {
 }
 
 int32_t Sampler::Verify(float *logits, int n, int32_t draft, const Dist *q) {
+    if (n <= 0) return -1;
     if (!q || Greedy()) return Sample(logits, n);
     std::vector<Saved> saved;
     penalise(logits, n, &saved);

@@ -56,13 +56,13 @@ def argmax(row):
 
 
 def top_n(row, k):
-    out = np.empty(min(k, len(row)), np.int32)
+    out = np.empty(max(0, min(k, len(row))), np.int32)
     n = _lib().shvsampler_top_n(_f(row), len(row), k, _i(out))
     return out[:n]
 
 
 def top_k_of(row, k):
-    out = np.empty(k, np.int32)
+    out = np.empty(max(0, k), np.int32)
     n = _lib().shvsampler_top_k_of(_f(row), len(row), k, _i(out))
     return out[:n]
 

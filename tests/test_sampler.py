@@ -172,6 +172,15 @@ def test_verify_of_a_token_outside_the_draft_distribution_is_a_plain_draw():
         assert s.verify(pl, outside, ds) in allowed
 
 
+def test_empty_rows_and_counts_are_answered_not_read():
+    empty = np.zeros(0, np.float32)
+    s = S.Sampler(1, 5, 0.9, 1)
+    assert s.sample(empty) == -1 and s.propose(empty) == -1 and s.verify(empty, 3, None) == -1
+    assert len(s.dist(empty)[0]) == 0
+    v = np.arange(5, dtype=np.float32)
+    assert len(S.top_n(v, 0)) == 0 and len(S.top_k_of(v, 0)) == 0
+
+
 def test_seeds_name_streams():
     v = np.random.default_rng(1).standard_normal(100).astype(np.float32)
     a = [S.Sampler(1, 0, 0, 42).sample(v) for _ in range(1)]
