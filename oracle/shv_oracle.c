@@ -980,6 +980,7 @@ void shv_ref_model_extend(const shv_ref_model_cfg *c, const shv_ref_model_w *w, 
 void shv_ref_mtp_rows(const shv_ref_model_cfg *c, const shv_ref_model_w *w, const shv_ref_mtp_w *mw,
                       uint16_t *kcache, uint16_t *vcache, const float *hs, const int32_t *ids, int n_tok,
                       int pos, float *logits, float *res, int threads) {
+    if (n_tok <= 0) return;
     int H = c->n_embd;
     size_t T = (size_t)n_tok;
     float *x = (float *)malloc(sizeof(float) * T * H);
