@@ -502,7 +502,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
 // grid: (n_embd/RPP/P row groups, n_tok).  A block owns P * RPP output rows of one token; its four
 // waves split the n_used+1 slots, each lane scales its partial dot by the slot's weight, and the
 // block adds the four waves' sums (and the residual) at the end.  P: passes over the staged
-// activation rows, as in the up projection (two for many tokens; more costs registers and is slower).
+// activation rows, as in the up projection (eight for many tokens, taken slot after slot).
 template <int K, int MAXS, int P>
 __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
@@ -563,28 +563,58 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
     __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
 
     const NibbleConsts nc = nibble_consts();
+    if constexpr (P <= 2) {
 #pragma unroll
-    for (int p = 0; p < P; p++) {
-        const int row = row0 + p * RPP;
-        if (p + 1 < P) {
-            // the next pass's weights are on their way while this pass multiplies
-            const size_t roff = static_cast<size_t>(row + RPP < a.n_embd ? row + RPP : 0) * ROWB + sb * SHV_Q4K_BYTES;
+        for (int p = 0; p < P; p++) {
+            const int row = row0 + p * RPP;
+            if (p + 1 < P) {
+                // the next pass's weights are on their way while this pass multiplies
+                const size_t roff = static_cast<size_t>(row + RPP < a.n_embd ? row + RPP : 0) * ROWB + sb * SHV_Q4K_BYTES;
 #pragma unroll
-            for (int i = 0; i < SPW; i++)
-                if (wave + 4 * i < ns) w[(p + 1) & 1][i].load(base[i] + roff, g);
+                for (int i = 0; i < SPW; i++)
+                    if (wave + 4 * i < ns) w[(p + 1) & 1][i].load(base[i] + roff, g);
+            }
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < SPW; i++) {
+                const int s = wave + 4 * i;
+                if (s < ns) {
+                    float xr[64], xs_lo, xs_hi;
+                    load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
+                    acc = fmaf(wt[i], w[p & 1][i].dot(g, nc, xr, xs_lo, xs_hi), acc);
+                }
+            }
+            acc = group_sum<LPR>(acc);
+            if (group_sum_owner<LPR>(lane)) part[wave][p * RPP + rsub] = acc;
         }
-        float acc = 0.f;
+    } else {
+        // Many passes: slot after slot, so that a slot's 64 activations come out of LDS once for all
+        // of the block's rows instead of once per pass (that re-reading was a third of the kernel at
+        // 64 tokens).  Each output row still adds its slots up in slot order.
+        float acc[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) acc[p] = 0.f;
 #pragma unroll
         for (int i = 0; i < SPW; i++) {
             const int s = wave + 4 * i;
             if (s < ns) {
                 float xr[64], xs_lo, xs_hi;
                 load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
-                acc = fmaf(wt[i], w[p & 1][i].dot(g, nc, xr, xs_lo, xs_hi), acc);
+                Q4kLane ww[2];
+                ww[0] = w[0][i];
+#pragma unroll
+                for (int p = 0; p < P; p++) {
+                    const int row = row0 + p * RPP;
+                    if (p + 1 < P) ww[(p + 1) & 1].load(base[i] + static_cast<size_t>(row + RPP < a.n_embd ? row + RPP : 0) * ROWB + sb * SHV_Q4K_BYTES, g);
+                    acc[p] = fmaf(wt[i], ww[p & 1].dot(g, nc, xr, xs_lo, xs_hi), acc[p]);
+                }
             }
         }
-        acc = group_sum<LPR>(acc);
-        if (group_sum_owner<LPR>(lane)) part[wave][p * RPP + rsub] = acc;
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const float v = group_sum<LPR>(acc[p]);
+            if (group_sum_owner<LPR>(lane)) part[wave][p * RPP + rsub] = v;
+        }
     }
     __syncthreads();
     if (tid < P * RPP) {
@@ -690,13 +720,13 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     switch (a.ffn) {
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
-            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 2>), dim3((a.n_embd + RPP * 2 - 1) / (RPP * 2), a.n_tok), block, 0, a);
+            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a);
             else SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
             break;
         }
         case 256: {
             constexpr int RPP = 64 / (256 / 64);
-            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 2>), dim3((a.n_embd + RPP * 2 - 1) / (RPP * 2), a.n_tok), block, 0, a);
+            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a);
             else SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
             break;
         }
