@@ -299,7 +299,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs the token loop on ONE GPU (one process, one stream); "
-                 "--gpus %d is not supported. How the path would shard is described in DESIGN.md." % a.gpus)
+                 "--gpus %d is not supported (experts and heads would shard across GPUs; none of that is built)." % a.gpus)
     if a.steps < 1 or a.warmup < 1:
         sys.exit("bench.py: --steps and --warmup must be at least 1")
     pkg = importlib.import_module("strix-halo-vulkan_amd")
