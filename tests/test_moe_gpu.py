@@ -98,7 +98,7 @@ def _check(case, residual=False, defer=False):
 
 
 @pytest.mark.parametrize("defer", [False, True])
-@pytest.mark.parametrize("T", [1, 4, 16])
+@pytest.mark.parametrize("T", [1, 4, 9, 16])
 def test_moe_block_matches_oracle(ctx, T, defer):
     """defer: the selection is made by the expert kernel from the router's logits instead of by
     the router's last block; both must give the reference's selection."""
