@@ -50,12 +50,16 @@ __device__ __forceinline__ float conv4(const float *ring, int ring_slots, int ri
 
 constexpr int kPrep = 8;  // rows of a sequence whose conv, norms and gates are prepared together
 
-// grid: (128/8 row chunks, n_head_v, n_seq).  The rows of a call go in groups of kPrep: first
+// grid: (128/(4*RW) row chunks, n_head_v, n_seq); RW state rows a wave (two, 32 lanes x float4 each;
+// or four, two to a lane, for calls of several sequences, whose many small blocks would otherwise
+// queue for the chip and prepare their heads twice as often).  The rows of a call go in groups of kPrep: first
 // everything that does not depend on the state is worked out for the whole group, all threads
 // busy (a thread keeps the sliding window of its channel's ring values, so a row costs one load);
 // then the waves walk the group's rows with nothing between two rows but their own two
 // reductions.
+template <int RW>
 __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
+    constexpr int kRowsPerBlock = 4 * RW, NS = RW / 2;  // NS: state rows a lane holds four values of
     __shared__ __align__(16) float qs[kPrep][kD];
     __shared__ __align__(16) float ks[kPrep][kD];
     __shared__ float vs[kPrep][kRowsPerBlock];
@@ -70,7 +74,7 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
     const int qk = a.n_head_k * kD, vw = a.n_head_v * kD;
     const int alpha_off = 2 * qk + 2 * vw, beta_off = alpha_off + a.n_head_v;
     const int rsub = lane >> 5, li = lane & 31;
-    const int jl = wave * 2 + rsub;           // row within the block
+    const int jl = wave * RW + rsub;          // first row of the lane within the block; its others follow two apart
     const int j = chunk * kRowsPerBlock + jl; // row of the head's state
     // a slot holds n_planes copies of the state; the committed one is read
     const int planes = a.n_planes > 1 ? a.n_planes : 1;
@@ -78,7 +82,9 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
     const size_t plane_floats = static_cast<size_t>(a.n_head_v) * kD * kD;
     float *sslot = a.state + static_cast<size_t>(slot) * planes * plane_floats + (static_cast<size_t>(h) * kD + j) * kD + li * 4;
     float *srow = sslot + cur * plane_floats;
-    float4 s = *reinterpret_cast<const float4 *>(srow);  // in flight while the first group is prepared
+    float4 s[NS];  // in flight while the first group is prepared
+#pragma unroll
+    for (int u = 0; u < NS; u++) s[u] = *reinterpret_cast<const float4 *>(srow + static_cast<size_t>(2 * u) * kD);
 
     const float *ring = a.ring + static_cast<size_t>(slot) * a.ring_slots * a.ring_stride;
     const float scale = 1.f / sqrtf(static_cast<float>(kD));
@@ -117,8 +123,8 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
             const int vch = 2 * qk + h * kD + chunk * kRowsPerBlock + vr;
             const float cv = conv4(ring, a.ring_slots, a.ring_stride, a.conv1d, vch, p0 + r);
             vs[r][vr] = cv * sigmoid_exact(cv);
-        } else if (tid >= 64 && tid < 64 + nr) {
-            const int r = tid - 64;
+        } else if (tid >= kBlock - kPrep && tid - (kBlock - kPrep) < nr) {
+            const int r = tid - (kBlock - kPrep);
             const float *row = ring + static_cast<size_t>((p0 + r) % a.ring_slots) * a.ring_stride;
             const float asp = softplus_ref(row[alpha_off + h] + a.dt_bias[h]);
             gb[r][0] = expf(asp * a.a[h]);
@@ -138,23 +144,31 @@ __global__ __launch_bounds__(kBlock) void dn_step_kernel(shv_dn_step_args a) {
             const int i = i0 + r;
             const float4 k4 = *reinterpret_cast<const float4 *>(&ks[r][li * 4]);
             const float4 q4 = *reinterpret_cast<const float4 *>(&qs[r][li * 4]);
-            const float g = gb[r][0], beta = gb[r][1], vj = vs[r][jl];
-            s.x *= g; s.y *= g; s.z *= g; s.w *= g;
-            const float dk = sum32_all(fmaf(s.x, k4.x, fmaf(s.y, k4.y, fmaf(s.z, k4.z, s.w * k4.w))));
-            const float delta = (vj - dk) * beta;
-            s.x = fmaf(delta, k4.x, s.x);
-            s.y = fmaf(delta, k4.y, s.y);
-            s.z = fmaf(delta, k4.z, s.z);
-            s.w = fmaf(delta, k4.w, s.w);
-            const float oq = sum32_all(fmaf(s.x, q4.x, fmaf(s.y, q4.y, fmaf(s.z, q4.z, s.w * q4.w))));
-            if (li == 0)
-                a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j] = oq * scale;
-            // a rewindable pass keeps every prefix: the state after row i goes to its own plane
-            if (a.spec) *reinterpret_cast<float4 *>(sslot + ((cur + 1 + i) % planes) * plane_floats) = s;
+            const float g = gb[r][0], beta = gb[r][1];
+#pragma unroll
+            for (int u = 0; u < NS; u++) {
+                float4 &su = s[u];
+                const float vj = vs[r][jl + 2 * u];
+                su.x *= g; su.y *= g; su.z *= g; su.w *= g;
+                const float dk = sum32_all(fmaf(su.x, k4.x, fmaf(su.y, k4.y, fmaf(su.z, k4.z, su.w * k4.w))));
+                const float delta = (vj - dk) * beta;
+                su.x = fmaf(delta, k4.x, su.x);
+                su.y = fmaf(delta, k4.y, su.y);
+                su.z = fmaf(delta, k4.z, su.z);
+                su.w = fmaf(delta, k4.w, su.w);
+                const float oq = sum32_all(fmaf(su.x, q4.x, fmaf(su.y, q4.y, fmaf(su.z, q4.z, su.w * q4.w))));
+                if (li == 0)
+                    a.out[(static_cast<size_t>(seq) * a.seq_len + i) * vw + static_cast<size_t>(h) * kD + j + 2 * u] = oq * scale;
+                // a rewindable pass keeps every prefix: the state after row i goes to its own plane
+                if (a.spec) *reinterpret_cast<float4 *>(sslot + ((cur + 1 + i) % planes) * plane_floats + static_cast<size_t>(2 * u) * kD) = su;
+            }
         }
         if (i0 + kPrep < a.seq_len) __syncthreads();  // the next group overwrites what the waves just read
     }
-    if (!a.spec) *reinterpret_cast<float4 *>(srow) = s;
+    if (!a.spec) {
+#pragma unroll
+        for (int u = 0; u < NS; u++) *reinterpret_cast<float4 *>(srow + static_cast<size_t>(2 * u) * kD) = s[u];
+    }
 }
 
 // The same step for calls of many rows (prompt chunks), where the groups' preparation - not the
@@ -301,6 +315,7 @@ int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
     dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
     // more than one group of rows: preparation and rule overlap
     if (a.seq_len > kPrep) SHV_LAUNCH(ctx, dn_step_pipe_kernel, grid, dim3(kBlock + 64 * kPrepWaves), 0, a);
-    else SHV_LAUNCH(ctx, dn_step_kernel, grid, dim3(kBlock), 0, a);
+    else if (a.n_seq >= 4) SHV_LAUNCH(ctx, dn_step_kernel<4>, dim3(kD / 16, a.n_head_v, a.n_seq), dim3(kBlock), 0, a);
+    else SHV_LAUNCH(ctx, dn_step_kernel<2>, grid, dim3(kBlock), 0, a);
     return SHV_OK;
 }

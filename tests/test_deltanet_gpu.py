@@ -106,15 +106,16 @@ def test_decode_steps_from_a_fresh_state(ctx):
         assert O.rel_l2(got_res[t], want_res[t]) <= TOL, t
 
 
-@pytest.mark.parametrize("B", [1, 8])
-def test_decode_step_with_random_state(ctx, B):
+@pytest.mark.parametrize("B,R", [(1, 1), (8, 1), (5, 6)])
+def test_decode_step_with_random_state(ctx, B, R):
     """BASELINE config 3, decode mode: batch 1 and 8 sequences, each with its own state ~N(0,0.1)
-    and its own three rows of conv history, at different positions."""
+    and its own three rows of conv history, at different positions; and five sequences of six rows
+    each in one call (from four sequences on a wave holds four state rows instead of two)."""
     case = DnCase(ctx, seed=10 + B)
     case.upload()
     rng = case.rng
-    slots = 4
-    xn = rng.standard_normal((B, case.H)).astype(np.float32)
+    slots = 4 if R == 1 else 12
+    xn = rng.standard_normal((B, R, case.H)).astype(np.float32)
     s0 = (rng.standard_normal((B, case.hv, case.d, case.d)) * 0.1).astype(np.float32)
     hist = rng.standard_normal((B, 3, case.width)).astype(np.float32)  # rows at positions p-3..p-1
     pos = (3 + 5 * np.arange(B)).astype(np.int32)
@@ -124,17 +125,18 @@ def test_decode_step_with_random_state(ctx, B):
             ring[b, (pos[b] - 3 + i) % slots] = hist[b, i]
     c = ctx
     d_ring, d_state = c.upload(ring), c.upload(s0)
-    d_attn, d_res = c.alloc(B * case.vw * 4), c.alloc(B * case.H * 4)
-    d_pos, d_x = c.upload(pos), c.upload(xn)
-    ops = case.step_ops(d_x, d_ring, d_state, d_attn, d_res, d_pos, None, B, 1, slots)[:2]
+    d_attn, d_res = c.alloc(B * R * case.vw * 4), c.alloc(B * R * case.H * 4)
+    d_pos, d_x = c.upload(pos), c.upload(xn.reshape(B * R, case.H))
+    ops = case.step_ops(d_x, d_ring, d_state, d_attn, d_res, d_pos, None, B, R, slots)[:2]
     c.dispatch_multi(ops)
-    got_attn = d_attn.read(np.float32, B * case.vw).reshape(B, case.vw)
+    got_attn = d_attn.read(np.float32, B * R * case.vw).reshape(B, R, case.vw)
     got_state = d_state.read(np.float32, s0.size).reshape(s0.shape)
     for b in range(B):
         conv_state = np.ascontiguousarray(hist[b, :, :case.cw].T)  # [cw][3], column 0 oldest
         s_state = s0[b].copy()
-        _, want_attn = case.oracle(xn[b:b + 1], conv_state, s_state)
-        assert O.rel_l2(got_attn[b], want_attn[0]) <= TOL, b
+        _, want_attn = case.oracle(xn[b], conv_state, s_state)
+        for r in range(R):
+            assert O.rel_l2(got_attn[b, r], want_attn[r]) <= TOL, (b, r)
         assert O.rel_l2(got_state[b], s_state) <= TOL, b
 
 
