@@ -320,13 +320,16 @@ typedef struct {
 
 /* Token embedding gather (Model.Embeddings, llm/model.go:134; hc.UploadInit, llm/graph.go:1815):
  * x[t] = float32(table[id_t]) for n_tok rows, id_t = ids[pos[0]+t] when pos is given, else ids[t].
- * table is binary16 [vocab][n_embd].  An id outside [0, vocab) yields a row of NaN. */
+ * table is [vocab][n_embd] in ggml type `type` (SHV_GGML_*): binary16 is the fast path, any other
+ * accepted type is expanded as Tensor.DequantizeRow does (llm/model.go:125-131), bit for bit.
+ * An id outside [0, vocab) yields a row of NaN. */
 typedef struct {
     const void *table;
     const int32_t *ids;
     const int32_t *pos;
     float *x;
     int32_t n_tok, n_embd, vocab, x_stride;
+    int32_t type;
 } shv_embed_args;
 
 /* Greedy sampler (Argmax, llm/sample.go:359-367): the index of the first maximum of each row of

@@ -28,10 +28,8 @@ __device__ __forceinline__ void scale_min_k4(int j, const uint8_t *q, uint32_t &
 
 __device__ const int8_t kValuesIQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
-__global__ __launch_bounds__(256) void dequant_kernel(int type, const uint8_t *src, float *dst, long long n) {
-    const long long g = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;  // group of 32 outputs
-    if (g * 32 >= n) return;
-    float *o = dst + g * 32;
+// Group g (32 outputs) of a run of n elements starting at src, written to o.
+__device__ __forceinline__ void dequant_group(int type, const uint8_t *src, long long g, long long n, float *o) {
     switch (type) {
         case SHV_GGML_F32: {
             const int m = n - g * 32 < 32 ? static_cast<int>(n - g * 32) : 32;
@@ -136,10 +134,32 @@ __global__ __launch_bounds__(256) void dequant_kernel(int type, const uint8_t *s
     }
 }
 
+__global__ __launch_bounds__(256) void dequant_kernel(int type, const uint8_t *src, float *dst, long long n) {
+    const long long g = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;  // group of 32 outputs
+    if (g * 32 >= n) return;
+    dequant_group(type, src, g, n, dst + g * 32);
+}
+
+// Embedding rows out of a table kept in the checkpoint's own type: row id_t expanded as
+// Tensor.DequantizeRow does (llm/model.go:125-131, gguf/dequant.go:119-124).  grid (groups/64, n_tok).
+__global__ __launch_bounds__(64) void embed_typed_kernel(shv_embed_args a, long long row_bytes) {
+    const int t = blockIdx.y;
+    const int g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g * 32 >= a.n_embd) return;
+    const int id = a.ids[(a.pos ? a.pos[0] : 0) + t];
+    float *o = a.x + static_cast<size_t>(t) * a.x_stride + g * 32;
+    if (id < 0 || id >= a.vocab) {
+        const int m = a.n_embd - g * 32 < 32 ? a.n_embd - g * 32 : 32;
+        for (int j = 0; j < m; j++) o[j] = __int_as_float(0x7fc00000);
+        return;
+    }
+    dequant_group(a.type, static_cast<const uint8_t *>(a.table) + static_cast<long long>(id) * row_bytes, g, a.n_embd, o);
+}
+
 }  // namespace
 
 // Bytes of n elements of a type, or -1 for a type the loader refuses / a count that is not whole blocks.
-static long long type_bytes(int type, long long n) {
+long long shv_type_bytes(int type, long long n) {
     switch (type) {
         case SHV_GGML_F32: return n * 4;
         case SHV_GGML_F16: case SHV_GGML_BF16: return n * 2;
@@ -157,11 +177,18 @@ static long long type_bytes(int type, long long n) {
 
 int shv_launch_dequant(shv_ctx *ctx, const shv_dequant_args *a) {
     SHV_REQUIRE(a->src && a->dst, "dequant: NULL src or dst");
-    SHV_REQUIRE(a->n > 0 && type_bytes(a->type, a->n) > 0, "dequant: %lld elements of ggml type %d (not a type the loader accepts, or not whole blocks)",
+    SHV_REQUIRE(a->n > 0 && shv_type_bytes(a->type, a->n) > 0, "dequant: %lld elements of ggml type %d (not a type the loader accepts, or not whole blocks)",
                 static_cast<long long>(a->n), a->type);
     const long long groups = (a->n + 31) / 32, blocks = (groups + 255) / 256;
     SHV_REQUIRE(blocks < (1ll << 31), "dequant: %lld elements is too many for one launch", static_cast<long long>(a->n));
     SHV_LAUNCH(ctx, dequant_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, a->type, static_cast<const uint8_t *>(a->src), a->dst,
                static_cast<long long>(a->n));
+    return SHV_OK;
+}
+
+int shv_launch_embed_typed(shv_ctx *ctx, const shv_embed_args *a) {
+    const long long row_bytes = shv_type_bytes(a->type, a->n_embd);
+    SHV_REQUIRE(row_bytes > 0, "embed: a row of %d elements of ggml type %d (not a type the loader accepts, or not whole blocks)", a->n_embd, a->type);
+    SHV_LAUNCH(ctx, embed_typed_kernel, dim3((a->n_embd / 32 + 63) / 64, a->n_tok), dim3(64), 0, *a, row_bytes);
     return SHV_OK;
 }

@@ -170,6 +170,7 @@ int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a) {
     SHV_REQUIRE(a->table && a->ids && a->x, "embed: NULL argument");
     SHV_REQUIRE(a->n_tok >= 1 && a->n_tok <= 65535 && a->n_embd >= 1 && a->vocab >= 1 && a->x_stride >= a->n_embd,
                 "embed: n_tok %d, n_embd %d, vocab %d, x_stride %d", a->n_tok, a->n_embd, a->vocab, a->x_stride);
+    if (a->type != SHV_GGML_F16) return shv_launch_embed_typed(ctx, a);
     const int bx = (a->n_embd + 255) / 256;
     SHV_LAUNCH(ctx, embed_kernel, dim3(bx < 8 ? bx : 8, a->n_tok), dim3(256), 0, *a);
     return SHV_OK;

@@ -108,7 +108,7 @@ class AttnDecodeArgs(C.Structure):
 class EmbedArgs(C.Structure):
     _fields_ = [("table", C.c_void_p), ("ids", C.c_void_p), ("pos", C.c_void_p), ("x", C.c_void_p),
                 ("n_tok", C.c_int32), ("n_embd", C.c_int32), ("vocab", C.c_int32),
-                ("x_stride", C.c_int32)]
+                ("x_stride", C.c_int32), ("type", C.c_int32)]
 
 
 class ArgmaxArgs(C.Structure):

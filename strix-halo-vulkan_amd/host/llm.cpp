@@ -35,6 +35,15 @@ void *Device::alloc(size_t bytes) {
     return p;
 }
 
+void Device::release(void *p, size_t bytes) {
+    auto it = std::find(owned_.begin(), owned_.end(), p);
+    if (it == owned_.end()) throw Error("llm: release of memory this device did not hand out");
+    sync();
+    check(shv_free(ctx_, p), "free");
+    owned_.erase(it);
+    allocated_ -= bytes;
+}
+
 void *Device::alloc_zero(size_t bytes) {
     void *p = alloc(bytes);
     zero(p, bytes < 256 ? 256 : bytes);
@@ -72,6 +81,7 @@ void Model::add(const std::string &name, TensorView::Kind kind, int64_t rows, in
     } else {
         t.bytes = static_cast<uint64_t>(rows) * cols * (kind == TensorView::F16 ? 2 : 4);
     }
+    t.ggml = kind == TensorView::Q4K ? gguf::Q4_K : kind == TensorView::F16 ? gguf::F16 : gguf::F32;
     t.ptr = dev_.alloc(t.bytes);
     tensors_[name] = t;
 }
@@ -242,34 +252,83 @@ Config Model::ConfigFromGGUF(const gguf::Set &s) {
     return c;
 }
 
-void Model::LoadGGUF(const gguf::Set &s) {
+// The ggml types shv_dequant, shv_gemv and the typed embedding gather read (gguf/dequant.go:52-98).
+static bool device_expands(uint32_t t) {
+    switch (t) {
+        case gguf::F32: case gguf::F16: case gguf::BF16: case gguf::Q8_0: case gguf::Q4_1: case gguf::Q5_0: case gguf::Q5_1:
+        case gguf::IQ4_NL: case gguf::Q4_K: case gguf::Q5_K: case gguf::Q6_K: return true;
+    }
+    return false;
+}
+
+void Model::LoadGGUF(const gguf::Set &s, bool transcode) {
     std::map<std::string, int64_t> covered;  // rows of each whole tensor that came from the file
-    for (const auto &kv : tensors_) {
+    transcoded_.clear();
+    // a tensor's bytes as the file holds them, in HBM for the length of one call
+    struct Raw {
+        Device &dev;
+        void *p = nullptr;
+        Raw(Device &d, const gguf::Tensor &t) : dev(d) {
+            check(shv_alloc(dev.ctx(), t.Bytes, &p), "staging");
+            try {
+                dev.upload(p, t.Data, t.Bytes);
+            } catch (...) {
+                shv_free(dev.ctx(), p);
+                throw;
+            }
+        }
+        ~Raw() { shv_free(dev.ctx(), p); }
+    };
+    for (auto &kv : tensors_) {
         const std::string &name = kv.first;
-        const TensorView &v = kv.second;
+        TensorView &v = kv.second;
         if (!s.Has(name)) continue;
         const gguf::Tensor &t = s.Get(name);
         const std::string shape = "[" + std::to_string(t.Dims[0]) + " x " + std::to_string(t.Rows()) + "] " + gguf::TypeName(t.Type);
         if (t.Dims[0] != v.cols || t.Rows() != v.rows)
             throw Error("llm: " + name + " is " + shape + " in the checkpoint, the metadata makes it [" + std::to_string(v.cols) + " x " + std::to_string(v.rows) + "]");
-        const uint32_t same = v.kind == TensorView::Q4K ? gguf::Q4_K : v.kind == TensorView::F16 ? gguf::F16 : gguf::F32;
-        if (t.Type == same) {
+        const uint32_t same = v.kind == TensorView::Q4K ? gguf::Q4_K : v.kind == TensorView::F32 ? gguf::F32 : v.ggml;
+        if (name == "token_embd.weight" && t.Type != v.ggml) {
+            // the table in the checkpoint's own type: the gather expands the rows it reads
+            if (!device_expands(t.Type)) throw Error("llm: " + name + " is " + shape + ": not a type the device expands");
+            if (t.RowBytes() == 0) throw Error("llm: " + name + " is " + shape + ": rows are not whole blocks of the type");
+            dev_.release(v.ptr, v.bytes);
+            v.ptr = dev_.alloc(t.Bytes);
+            v.bytes = t.Bytes;
+            v.kind = t.Type == gguf::F16 ? TensorView::F16 : TensorView::RAW;
+            v.ggml = t.Type;
+            dev_.upload(v.ptr, t.Data, t.Bytes);
+        } else if (t.Type == same) {
             if (t.Bytes != v.bytes) throw Error("llm: " + name + ": " + std::to_string(t.Bytes) + " bytes in the checkpoint, " + std::to_string(v.bytes) + " staged");
             dev_.upload(v.ptr, t.Data, t.Bytes);
         } else if (v.kind == TensorView::F32) {
             // small float tensors (norms, routers, conv taps) in whatever the converter chose: expanded on the device
-            void *raw = nullptr;
-            check(shv_alloc(dev_.ctx(), t.Bytes, &raw), "staging");
+            Raw raw(dev_, t);
+            shv_dequant_args d{raw.p, static_cast<float *>(v.ptr), t.Elems(), static_cast<int32_t>(t.Type)};
+            check(shv_dequant(dev_.ctx(), &d), name.c_str());
+            dev_.sync();
+        } else if (v.kind == TensorView::Q4K && transcode) {
+            // expanded and fitted again, a bounded number of rows at a time
+            const uint64_t row_in = t.RowBytes(), row_out = v.bytes / v.rows;
+            const int64_t step = std::max<int64_t>(1, std::min<int64_t>(v.rows, (64ll << 20) / v.cols));
+            Raw raw(dev_, t);
+            void *f32 = nullptr;
+            check(shv_alloc(dev_.ctx(), static_cast<size_t>(step) * v.cols * 4, &f32), "staging");
             try {
-                dev_.upload(raw, t.Data, t.Bytes);
-                shv_dequant_args d{raw, static_cast<float *>(v.ptr), t.Elems(), static_cast<int32_t>(t.Type)};
-                check(shv_dequant(dev_.ctx(), &d), name.c_str());
+                for (int64_t r0 = 0; r0 < v.rows; r0 += step) {
+                    const int64_t nr = std::min<int64_t>(step, v.rows - r0);
+                    shv_dequant_args d{static_cast<const char *>(raw.p) + r0 * row_in, static_cast<float *>(f32), nr * v.cols, static_cast<int32_t>(t.Type)};
+                    check(shv_dequant(dev_.ctx(), &d), name.c_str());
+                    shv_quantize_q4k_args q{static_cast<const float *>(f32), static_cast<char *>(v.ptr) + r0 * row_out, nr, static_cast<int32_t>(v.cols)};
+                    check(shv_quantize_q4k(dev_.ctx(), &q), name.c_str());
+                }
                 dev_.sync();
             } catch (...) {
-                shv_free(dev_.ctx(), raw);
+                shv_free(dev_.ctx(), f32);
                 throw;
             }
-            shv_free(dev_.ctx(), raw);
+            shv_free(dev_.ctx(), f32);
+            transcoded_.push_back(name);
         } else {
             throw Error("llm: " + name + " is " + gguf::TypeName(t.Type) + " in the checkpoint; the kernels stream it as " + gguf::TypeName(same));
         }
@@ -318,7 +377,7 @@ void Model::SaveGGUF(const std::string &path, const std::string &arch) const {
         if (v.rows == 1) dims = {v.cols};
         else if (name.find("_exps.") != std::string::npos) dims = {v.cols, v.rows / c.NExpert, c.NExpert};
         else dims = {v.cols, v.rows};
-        const uint32_t type = v.kind == TensorView::Q4K ? gguf::Q4_K : v.kind == TensorView::F16 ? gguf::F16 : gguf::F32;
+        const uint32_t type = v.ggml;
         Device *dev = &dev_;
         const void *src = v.ptr;
         w.AddTensor(name, type, dims, [dev, src](uint8_t *dst, uint64_t bytes) { dev->download(dst, src, bytes); });
@@ -951,6 +1010,7 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     r.spec = spec;
     shv_embed_args e{};
     e.table = m_.Tensor("token_embd.weight").ptr;
+    e.type = static_cast<int32_t>(m_.Tensor("token_embd.weight").ggml);
     e.x = x_;
     e.n_tok = rows;
     e.n_embd = c_.NEmbd;
@@ -1420,6 +1480,7 @@ int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos,
         const int E = c_.NEmbd;
         shv_embed_args e{};
         e.table = m_.Tensor("token_embd.weight").ptr;
+        e.type = static_cast<int32_t>(m_.Tensor("token_embd.weight").ggml);
         e.ids = ids_;
         e.x = e_;
         e.n_tok = n;

@@ -37,6 +37,7 @@ public:
     shv_ctx *ctx() const { return ctx_; }
     void *alloc(size_t bytes);  // tracked; released with the device
     void *alloc_zero(size_t bytes);
+    void release(void *p, size_t bytes);  // an alloc() handed back early; bytes as asked for
     void upload(void *dst, const void *src, size_t bytes);
     void download(void *dst, const void *src, size_t bytes);
     void zero(void *dst, size_t bytes);
@@ -97,7 +98,8 @@ struct Config {
 struct TensorView {
     void *ptr = nullptr;
     uint64_t bytes = 0;
-    enum Kind { F32, F16, Q4K } kind = F32;
+    enum Kind { F32, F16, Q4K, RAW } kind = F32;  // RAW: rows in the ggml type `ggml`, as the checkpoint holds them
+    uint32_t ggml = 0;           // the ggml type of the bytes at ptr
     int64_t rows = 0, cols = 0;  // Q4K / F16 / F32 matrices: rows x cols; vectors: rows = 1
     float init_mean = 0.f, init_std = 0.02f;
 };
@@ -122,11 +124,17 @@ public:
     // Every tensor of this model from a mapped checkpoint into its device buffer, straight from
     // the mapping.  A fused projection is filled from its constituents (attn_q / attn_k / attn_v,
     // attn_qkv / attn_gate / ssm_alpha / ssm_beta, nextn.enorm / hnorm) when the file carries
-    // those, as llama.cpp's converter writes them.  Types must be the ones the kernels stream
-    // (Q4_K matrices, F16 embedding); an F32 tensor of the model takes any type the dequantiser
-    // knows and is expanded on the device.  Throws, naming the tensor, on a missing tensor, a
-    // shape that disagrees with the metadata, or a type the kernels do not read.
-    void LoadGGUF(const gguf::Set &s);
+    // those, as llama.cpp's converter writes them.  A tensor in the type the kernels stream
+    // (Q4_K matrices, F32 vectors) is copied byte for byte.  An F32 tensor of the model in any
+    // other type the dequantiser knows is expanded on the device.  The embedding table stays in
+    // the checkpoint's own type (rows are expanded as they are gathered, llm/model.go:125-131).
+    // A matrix the kernels stream as Q4_K that the checkpoint holds in another type is expanded
+    // and fitted again by the round-to-nearest quantiser on the device — the reference's
+    // transcode (llm/moebank.go:288-400, rtn arm), a loss on top of a loss — when `transcode`
+    // allows it; Transcoded() names those tensors.  Throws, naming the tensor, on a missing
+    // tensor, a shape that disagrees with the metadata, or a type that cannot be staged.
+    void LoadGGUF(const gguf::Set &s, bool transcode = true);
+    const std::vector<std::string> &Transcoded() const { return transcoded_; }
     // This model as one version-3 file the above reads back bit for bit: metadata keys as
     // ConfigFromGGUF reads them, constituents in place of fused tensors, expert banks 3-D.
     void SaveGGUF(const std::string &path, const std::string &arch = "qwen3next") const;
@@ -138,6 +146,7 @@ private:
     Device &dev_;
     Config cfg_;
     std::map<std::string, TensorView> tensors_;
+    std::vector<std::string> transcoded_;
 };
 
 // llm.Stage (llm/gpu.go:1578-1581)

@@ -3,6 +3,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 
@@ -117,7 +118,8 @@ int shvllm_open_gguf(int device, const char *path, const shvllm_config *c, shvll
         h->dev = std::make_unique<llm::Device>(device);
         graph_opts(*h, *c);
         h->model = std::make_unique<llm::Model>(*h->dev, llm::Model::ConfigFromGGUF(*set));
-        h->model->LoadGGUF(*set);
+        const char *tc = std::getenv("LLM_TRANSCODE");  // 0: refuse a matrix that is not Q4_K instead of fitting it again
+        h->model->LoadGGUF(*set, !(tc && tc[0] == '0'));
         for (const auto &kv : h->model->Tensors()) h->names.push_back(kv.first);
         *out = h.release();
     });
@@ -167,6 +169,23 @@ int shvllm_tensor(shvllm *h, const char *name, void **dptr, uint64_t *bytes) {
         if (dptr) *dptr = t.ptr;
         if (bytes) *bytes = t.bytes;
     });
+}
+
+int shvllm_tensor_type(shvllm *h, const char *name, int32_t *ggml_type) {
+    return guard([&] {
+        if (!h || !h->model || !name || !ggml_type) throw llm::Error("llm: shvllm_tensor_type: NULL argument");
+        *ggml_type = static_cast<int32_t>(h->model->Tensor(name).ggml);
+    });
+}
+
+int shvllm_transcoded(shvllm *h, char *buf, size_t cap) {
+    if (!h || !h->model) return 0;
+    const std::vector<std::string> &v = h->model->Transcoded();
+    size_t at = 0;
+    for (const std::string &n : v)
+        for (size_t i = 0; i <= n.size() && buf && at + 1 < cap; i++) buf[at++] = i < n.size() ? n[i] : '\n';
+    if (buf && cap) buf[at] = 0;
+    return static_cast<int>(v.size());
 }
 
 uint64_t shvllm_weight_bytes(shvllm *h) { return h && h->model ? h->model->WeightBytes() : 0; }

@@ -45,6 +45,11 @@ int shvllm_tensor_count(shvllm *h);
 int shvllm_tensor_at(shvllm *h, int i, const char **name, void **dptr, uint64_t *bytes, int32_t *kind,
                      int64_t *rows, int64_t *cols, int32_t *is_alias);
 int shvllm_tensor(shvllm *h, const char *name, void **dptr, uint64_t *bytes);
+int shvllm_tensor_type(shvllm *h, const char *name, int32_t *ggml_type);  /* the ggml type of the bytes in device memory */
+/* Matrices the checkpoint held in a type other than Q4_K, expanded and fitted again as Q4_K when the
+ * model was opened (TranscodeMoE's round-to-nearest arm, llm/moebank.go:288-400): their count, and
+ * their names, one a line, into buf when it is given.  LLM_TRANSCODE=0 makes the open refuse them. */
+int shvllm_transcoded(shvllm *h, char *buf, size_t cap);
 uint64_t shvllm_weight_bytes(shvllm *h);
 int shvllm_stage(shvllm *h);   /* NewGraph: allocate state, record the decode step */
 int shvllm_reset(shvllm *h);

@@ -59,6 +59,8 @@ def load():
     L.shvllm_open_gguf.argtypes = [C.c_int, C.c_char_p, C.POINTER(Config), C.POINTER(vp)]
     L.shvllm_get_config.argtypes = [vp, C.POINTER(Config)]
     L.shvllm_save_gguf.argtypes = [vp, C.c_char_p]
+    L.shvllm_tensor_type.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int32)]
+    L.shvllm_transcoded.argtypes = [vp, C.c_char_p, C.c_size_t]
     L.shvllm_tensor_count.argtypes = [vp]
     L.shvllm_tensor_at.argtypes = [vp, C.c_int, C.POINTER(C.c_char_p), C.POINTER(vp), C.POINTER(C.c_uint64),
                                    C.POINTER(C.c_int32), C.POINTER(C.c_int64), C.POINTER(C.c_int64),
@@ -111,7 +113,7 @@ def _check(rc):
         raise hip_api.ShvError(rc, load().shvllm_last_error().decode("utf-8", "replace"))
 
 
-KIND_DTYPE = {0: np.float32, 1: np.uint16, 2: np.uint8}  # F32, F16 (bit patterns), Q4K (bytes)
+KIND_DTYPE = {0: np.float32, 1: np.uint16, 2: np.uint8, 3: np.uint8}  # F32, F16 (bit patterns), Q4K (bytes), RAW (bytes of another ggml type)
 
 
 class LLM:
@@ -163,6 +165,19 @@ class LLM:
         a = np.empty(nb.value // dt.itemsize, dtype=dt)
         hip_api.check(self.H.shv_download(self.ctx, a.ctypes.data, ptr, nb.value))
         return a
+
+    def tensor_type(self, name):
+        t = C.c_int32()
+        _check(self.L.shvllm_tensor_type(self.h, name.encode(), C.byref(t)))
+        return t.value
+
+    def transcoded(self):
+        """Names of the matrices that were fitted again as Q4_K when the checkpoint was opened."""
+        buf = C.create_string_buffer(1 << 16)
+        n = self.L.shvllm_transcoded(self.h, buf, len(buf))
+        names = [x for x in buf.value.decode().split("\n") if x]
+        assert len(names) == n, (n, names)
+        return names
 
     def upload(self, name, arr):
         ptr, nb = C.c_void_p(), C.c_uint64()

@@ -8,7 +8,8 @@ import numpy as np
 U8, I8, U16, I16, U32, I32, F32, BOOL, STR, ARRAY, U64, I64, F64 = range(13)
 _FMT = {U8: "<B", I8: "<b", U16: "<H", I16: "<h", U32: "<I", I32: "<i", F32: "<f", BOOL: "<B", U64: "<Q", I64: "<q", F64: "<d"}
 BLOCK = {0: (1, 4), 1: (1, 2), 30: (1, 2), 3: (32, 20), 6: (32, 22), 7: (32, 24), 8: (32, 34), 20: (32, 18),
-         12: (256, 144), 13: (256, 176), 14: (256, 210)}
+         12: (256, 144), 13: (256, 176), 14: (256, 210),
+         10: (256, 84)}     # Q2_K: a type the loader knows the geometry of and the device does not expand
 
 
 def _str(s):

@@ -38,9 +38,9 @@ def test_ggml_vectors_bit_for_bit(ctx, golden_dir):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), typ
 
 
-def random_tensor(name, n, seed=None):
-    """`n` elements of tensor type `name`: random bytes with finite half scales, so every bit pattern of
-    levels, fifth/sixth-bit planes and packed scales occurs."""
+def random_tensor(name, n, seed=None, scale=0.05):
+    """`n` elements of tensor type `name`: random bytes with finite half scales (normal, sigma `scale`), so
+    every bit pattern of levels, fifth/sixth-bit planes and packed scales occurs."""
     typ = O.GGML_TYPES[name]
     rng = np.random.default_rng(typ if seed is None else seed)
     raw = rng.integers(0, 256, size=O.type_bytes(typ, n), dtype=np.uint8)
@@ -53,7 +53,7 @@ def random_tensor(name, n, seed=None):
            "Q4_K": (144, [0, 2]), "Q5_K": (176, [0, 2]), "Q6_K": (210, [208])}[name]
     rows = raw.reshape(-1, blk[0])
     for off in blk[1]:
-        h = (rng.standard_normal(rows.shape[0]) * 0.05).astype(np.float16).view(np.uint16)
+        h = (rng.standard_normal(rows.shape[0]) * scale).astype(np.float16).view(np.uint16)
         rows[:, off] = h & 0xFF
         rows[:, off + 1] = h >> 8
     return raw

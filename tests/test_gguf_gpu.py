@@ -149,7 +149,7 @@ def test_float_tensors_of_other_types_are_expanded_on_the_device(saved, tmp_path
         r.close()
 
 
-def test_load_refuses_what_it_cannot_stage(saved, tmp_path):
+def test_load_refuses_what_it_cannot_stage(saved, tmp_path, monkeypatch):
     m, cfg, path = saved
     p = GF.parse(path)
     with pytest.raises(ShvError, match=r"rows of blk\.3\.attn_qkv_fused"):
@@ -159,8 +159,16 @@ def test_load_refuses_what_it_cannot_stage(saved, tmp_path):
     _, dims, data = p["tensors"]["blk.0.ffn_up_shexp.weight"]
     n = int(np.prod(dims))
     q8 = (8, dims, bytes(n // 32 * 34))
+    monkeypatch.setenv("LLM_TRANSCODE", "0")
     with pytest.raises(ShvError, match="Q8_0 in the checkpoint; the kernels stream it as Q4_K"):
         LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "q8.gguf", tensors={"blk.0.ffn_up_shexp.weight": q8}))
+    monkeypatch.delenv("LLM_TRANSCODE")
+    q2 = (10, dims, bytes(n // 256 * 84))
+    with pytest.raises(ShvError, match="blk.0.ffn_up_shexp.weight"):
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "q2.gguf", tensors={"blk.0.ffn_up_shexp.weight": q2}))
+    _, edims, _ = p["tensors"]["token_embd.weight"]
+    with pytest.raises(ShvError, match="not a type the device expands"):
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "e2.gguf", tensors={"token_embd.weight": (10, edims, bytes(int(np.prod(edims)) // 256 * 84))}))
     short = (0, [cfg.n_embd // 2], bytes(cfg.n_embd * 2))
     with pytest.raises(ShvError, match="the metadata makes it"):
         LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "shape.gguf", tensors={"output_norm.weight": short}))
@@ -170,6 +178,72 @@ def test_load_refuses_what_it_cannot_stage(saved, tmp_path):
     q = dict(p, kv={k: v for k, v in p["kv"].items() if k != "general.architecture"})
     with pytest.raises(ShvError, match="no general.architecture"):
         LA.LLM(small_cfg(), gguf=_rewrite(q, tmp_path / "noarch.gguf"))
+
+
+def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, tmp_path):
+    """What a converter's mixed recipe looks like: the embedding table and the head in Q6_K, expert
+    banks in Q5_K / Q8_0 / IQ4_NL / Q5_1, one constituent of a fused projection in Q5_0, another in
+    F16.  The table stays in its own type (rows expanded by the gather, llm/model.go:125-131); every
+    such matrix is expanded and fitted again as Q4_K, bit for bit what the CPU's dequantiser
+    (gguf/dequant.go:52-98) followed by the CPU's quantiser (llm/quantk.go:115-179) gives; the model
+    then decodes the tokens the CPU model decodes from those weights."""
+    m, cfg, path = saved
+    p = GF.parse(path)
+    recipe = {"token_embd.weight": "Q8_0", "output.weight": "Q6_K", "blk.0.ffn_down_exps.weight": "Q5_K",
+              "blk.1.ffn_gate_exps.weight": "Q8_0", "blk.2.ffn_down_exps.weight": "IQ4_NL", "blk.1.ffn_up_shexp.weight": "Q5_1",
+              "blk.3.attn_k.weight": "Q5_0", "blk.0.attn_gate.weight": "F16", "blk.2.ssm_out.weight": "Q4_1",
+              "blk.4.nextn.eh_proj.weight": "BF16"}
+    swap, f32 = {}, {}
+    for i, (name, tname) in enumerate(recipe.items()):
+        typ = O.GGML_TYPES[tname]
+        _, dims, _ = p["tensors"][name]
+        n = int(np.prod(dims))
+        if tname in ("F16", "BF16"):
+            v = (np.random.default_rng(50 + i).standard_normal(n) * 0.02).astype(np.float32)
+            raw = v.astype(np.float16).view(np.uint8) if tname == "F16" else (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+        else:
+            raw = random_tensor(tname, n, seed=60 + i, scale=2e-4)
+        if name == "token_embd.weight":
+            # scales of 2^-6: every expanded value is a binary16 too, so the CPU model's binary16 table holds the same rows
+            blocks = raw.reshape(-1, 34)
+            blocks[:, 0], blocks[:, 1] = 0x00, 0x24
+        swap[name] = (typ, dims, raw.tobytes())
+        f32[name] = O.dequant(typ, raw, n)
+    r = LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "recipe.gguf", tensors=swap))
+    try:
+        assert sorted(r.transcoded()) == sorted(n for n in recipe if n != "token_embd.weight")
+        assert r.tensor_type("token_embd.weight") == 8 and r.tensor_type("output.weight") == 12
+        assert np.array_equal(r.download("token_embd.weight"), np.frombuffer(swap["token_embd.weight"][2], np.uint8))
+        for name in recipe:
+            if name == "token_embd.weight":
+                continue
+            k = swap[name][1][0]
+            want = O.quantize_q4k(f32[name].reshape(-1, k))
+            assert np.array_equal(r.download(name).view(np.uint8), want.reshape(-1)), name
+        assert np.array_equal(r.download("blk.3.attn_q.weight"), m.download("blk.3.attn_q.weight"))
+        # saved again, the file names the types now in memory and reads back the same table
+        r.save_gguf(tmp_path / "again.gguf")
+        again = GF.parse(tmp_path / "again.gguf")
+        assert again["tensors"]["token_embd.weight"][0] == 8 and again["tensors"]["output.weight"][0] == 12
+        assert again["tensors"]["token_embd.weight"][2] == swap["token_embd.weight"][2]
+        # the token loop against the CPU loop over the weights as staged
+        r.stage()
+        tensors = {t[0]: r.download(t[0]) for t in r.tensors()}
+        table = f32["token_embd.weight"].astype(np.float16)
+        assert np.array_equal(table.astype(np.float32), f32["token_embd.weight"])
+        tensors["token_embd.weight"] = table.view(np.uint16)
+        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+        prompt = np.random.default_rng(5).integers(0, cfg.vocab, size=7).astype(np.int32)
+        r.reset()
+        lg_gpu, hd_gpu = r.extend(prompt, want_hidden=True)
+        lg_cpu, hd_cpu = om.extend(prompt)
+        assert O.rel_l2(hd_gpu, hd_cpu) <= 1e-3 and O.rel_l2(lg_gpu, lg_cpu) <= 1e-3
+        tok = int(O.lib().shv_ref_argmax(O.F(lg_cpu), cfg.vocab))
+        ids, _ = r.generate(1)
+        top2 = np.sort(lg_cpu)[-2:]
+        assert ids[0] == tok or top2[1] - top2[0] < 1e-4
+    finally:
+        r.close()
 
 
 @pytest.mark.parametrize("name", ["Q8_0", "Q6_K", "Q5_K", "IQ4_NL", "BF16"])

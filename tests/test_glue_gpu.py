@@ -4,6 +4,7 @@ import pytest
 
 import oracle_lib as O
 import shv
+from test_dequant_gpu import random_tensor
 
 pytestmark = pytest.mark.gpu
 A = shv.api
@@ -59,11 +60,33 @@ def test_embedding_gather(ctx):
     ids = np.array([3, 999, 0, 17, 5000], np.int32)
     d_x = ctx.alloc(4 * H * 4)
     d_t, d_ids = ctx.upload(table), ctx.upload(ids)
-    ctx.enqueue(A.OP_EMBED, A.EmbedArgs(d_t.ptr, d_ids.ptr, None, d_x.ptr, 4, H, vocab, H))
+    ctx.enqueue(A.OP_EMBED, A.EmbedArgs(d_t.ptr, d_ids.ptr, None, d_x.ptr, 4, H, vocab, H, 1))
     got = d_x.read(np.float32, 4 * H).reshape(4, H)
     assert np.array_equal(got, table[ids[:4]].astype(np.float32))
     # position-relative read, and an id outside the vocabulary is NaN rather than a wild read
     ctx.enqueue(A.OP_EMBED, A.EmbedArgs(d_t.ptr, d_ids.ptr, ctx.upload(np.array([3], np.int32)).ptr, d_x.ptr,
-                                        2, H, vocab, H))
+                                        2, H, vocab, H, 1))
     got = d_x.read(np.float32, 2 * H).reshape(2, H)
     assert np.array_equal(got[0], table[17].astype(np.float32)) and np.isnan(got[1]).all()
+
+
+@pytest.mark.parametrize("name", ["F32", "BF16", "Q8_0", "Q4_1", "Q5_0", "Q5_1", "IQ4_NL", "Q4_K", "Q5_K", "Q6_K"])
+def test_embedding_gather_from_a_table_of_any_type(ctx, name):
+    """Rows of a table kept in the checkpoint's own type, against Tensor.DequantizeRow
+    (llm/model.go:125-131): bit for bit, the row stride of the output honoured."""
+    typ, vocab, H = O.GGML_TYPES[name], 300, 768
+    raw = random_tensor(name, vocab * H, seed=typ + 40)
+    want = O.dequant(typ, raw, vocab * H).reshape(vocab, H)
+    ids = np.array([7, 299, 0, -1, 123, 300], np.int32)
+    stride = H + 64
+    d_x = ctx.upload(np.full(len(ids) * stride, 5.0, np.float32))
+    ctx.enqueue(A.OP_EMBED, A.EmbedArgs(ctx.upload(raw).ptr, ctx.upload(ids).ptr, None, d_x.ptr, len(ids), H, vocab, stride, typ))
+    got = d_x.read(np.float32, len(ids) * stride).reshape(len(ids), stride)
+    assert np.all(got[:, H:] == 5.0)
+    for t, i in enumerate(ids):
+        if 0 <= i < vocab:
+            assert np.array_equal(got[t, :H].view(np.uint32), want[i].view(np.uint32)), (t, i)
+        else:
+            assert np.isnan(got[t, :H]).all()
+    with pytest.raises(A.ShvError, match="embed: a row of 100 elements"):
+        ctx.enqueue(A.OP_EMBED, A.EmbedArgs(ctx.upload(raw).ptr, ctx.upload(ids).ptr, None, d_x.ptr, 1, 100, vocab, 100, 12))
