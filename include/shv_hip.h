@@ -230,6 +230,11 @@ typedef struct {
     const float *logits;
     float *weights;
     int32_t n_expert;
+    /* ggml type (SHV_GGML_*) of each bank; 0 or SHV_GGML_Q4_K is Q4_K, the tuned path.  A bank in
+     * another accepted type (Q8_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q5_K, Q6_K, F16, BF16) is read as the
+     * checkpoint holds it (llm_moe_gemv.comp's other arms; llm/gpu_moe.go:673-688), rows as
+     * Tensor.DequantizeRow forms them; the selection then comes from the router (logits NULL). */
+    int32_t gate_type, up_type, gate_sh_type, up_sh_type;
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +
@@ -244,6 +249,7 @@ typedef struct {
     float *out;
     int32_t n_tok, n_embd, n_used, ffn;
     int32_t res_stride, out_stride;
+    int32_t down_type, down_sh_type;  /* as in shv_moe_up_args: 0 or SHV_GGML_Q4_K, or the bank's own type */
 } shv_moe_down_args;
 
 /* Gated DeltaNet step(s) after the fused projection (DeltaNetLayer, llm/deltanet.go:266-327 and

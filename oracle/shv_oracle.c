@@ -504,6 +504,37 @@ void shv_ref_gemv_q4k(float *y, const uint8_t *w, const float *x, int n, int k, 
     }
 }
 
+/* The same matvec over rows of any accepted tensor type: each row through Tensor.DequantizeRow
+ * (gguf/dequant.go:119-124), then llm/hc.go:255-264.  type 0 stands for Q4_K here (no bank is
+ * stored as float32).  Returns -1 for rows the type cannot hold. */
+int shv_ref_gemv_any(float *y, int type, const uint8_t *w, const float *x, int n, int k, int threads) {
+    if (type == 0) type = SHV_GGML_Q4_K;
+    if (type == SHV_GGML_Q4_K && k % SHV_Q4K_BLOCK == 0) {
+        shv_ref_gemv_q4k(y, w, x, n, k, threads);
+        return 0;
+    }
+    int64_t row_bytes = shv_ref_type_bytes(type, k);
+    if (row_bytes < 0) return -1;
+    if (threads < 1) threads = 1;
+    if (threads > n) threads = n;
+    int chunk = (n + threads - 1) / threads;
+#pragma omp parallel for num_threads(threads) schedule(static, 1)
+    for (int t = 0; t < threads; t++) {
+        int lo = t * chunk, hi = lo + chunk;
+        if (hi > n) hi = n;
+        if (lo >= hi) continue;
+        float *buf = (float *)malloc(sizeof(float) * (size_t)k);
+        for (int r = lo; r < hi; r++) {
+            shv_ref_dequant(type, w + (size_t)r * (size_t)row_bytes, k, buf);
+            float s = 0;
+            for (int i = 0; i < k; i++) s += buf[i] * x[i];
+            y[r] = s;
+        }
+        free(buf);
+    }
+    return 0;
+}
+
 /* llm/hc.go:266-268 */
 float shv_ref_sigmoid(float x) { return (float)(1 / (1 + exp(-(double)x))); }
 float shv_ref_silu(float x) { return x * shv_ref_sigmoid(x); }
@@ -611,8 +642,11 @@ void shv_ref_moe_block(const shv_ref_moe_cfg *c, const shv_ref_moe_w *w, const f
     float *wn = weights_norm ? weights_norm : (float *)malloc(sizeof(float) * (size_t)n_tok * used);
     shv_ref_moe_route(c, w, x, n_tok, lg, pr, tk, wn);
 
-    size_t up_row = (size_t)H / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
-    size_t dn_row = (size_t)ff / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+    /* banks in the checkpoint's own types (llm/moe.go walks them through Dequantize whatever they are) */
+    const int tg = w->types[0] ? w->types[0] : SHV_GGML_Q4_K, tu = w->types[1] ? w->types[1] : SHV_GGML_Q4_K;
+    const int td = w->types[2] ? w->types[2] : SHV_GGML_Q4_K, tgs = w->types[3], tus = w->types[4], tds = w->types[5];
+    size_t g_row = (size_t)shv_ref_type_bytes(tg, H), u_row = (size_t)shv_ref_type_bytes(tu, H);
+    size_t dn_row = (size_t)shv_ref_type_bytes(td, ff);
     int big = ff > ffs ? ff : ffs;
     float *gate = (float *)malloc(sizeof(float) * big);
     float *up = (float *)malloc(sizeof(float) * big);
@@ -626,11 +660,11 @@ void shv_ref_moe_block(const shv_ref_moe_cfg *c, const shv_ref_moe_w *w, const f
         /* routed experts, llm/moe.go:289-359 */
         for (int k = 0; k < used; k++) {
             int e = tk[(size_t)i * used + k];
-            shv_ref_gemv_q4k(gate, w->gate_exps + (size_t)e * ff * up_row, xi, ff, H, threads);
-            shv_ref_gemv_q4k(up, w->up_exps + (size_t)e * ff * up_row, xi, ff, H, threads);
+            shv_ref_gemv_any(gate, tg, w->gate_exps + (size_t)e * ff * g_row, xi, ff, H, threads);
+            shv_ref_gemv_any(up, tu, w->up_exps + (size_t)e * ff * u_row, xi, ff, H, threads);
             for (int j = 0; j < ff; j++) sw[j] = shv_ref_silu(gate[j]) * up[j];
             if (swiglu) memcpy(swiglu + ((size_t)i * used + k) * ff, sw, sizeof(float) * ff);
-            shv_ref_gemv_q4k(down, w->down_exps + (size_t)e * H * dn_row, sw, H, ff, threads);
+            shv_ref_gemv_any(down, td, w->down_exps + (size_t)e * H * dn_row, sw, H, ff, threads);
             float wt = wn[(size_t)i * used + k];
             for (int j = 0; j < H; j++) weighted[(size_t)k * H + j] = down[j] * wt;
         }
@@ -640,10 +674,10 @@ void shv_ref_moe_block(const shv_ref_moe_cfg *c, const shv_ref_moe_w *w, const f
             for (int j = 0; j < H; j++) o[j] += weighted[(size_t)k * H + j];
         if (moe_out) memcpy(moe_out + (size_t)i * H, o, sizeof(float) * H);
         /* shared expert, llm/moe.go:363-409 */
-        shv_ref_gemv_q4k(gate, w->gate_sh, xi, ffs, H, threads);
-        shv_ref_gemv_q4k(up, w->up_sh, xi, ffs, H, threads);
+        shv_ref_gemv_any(gate, tgs, w->gate_sh, xi, ffs, H, threads);
+        shv_ref_gemv_any(up, tus, w->up_sh, xi, ffs, H, threads);
         for (int j = 0; j < ffs; j++) sw[j] = shv_ref_silu(gate[j]) * up[j];
-        shv_ref_gemv_q4k(down, w->down_sh, sw, H, ffs, threads);
+        shv_ref_gemv_any(down, tds, w->down_sh, sw, H, ffs, threads);
         float g = 0;
         for (int j = 0; j < H; j++) g += w->shared_gate[j] * xi[j];
         float s = shv_ref_sigmoid(g);

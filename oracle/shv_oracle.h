@@ -56,6 +56,8 @@ enum {
     SHV_GGML_Q4_K = 12, SHV_GGML_Q5_K = 13, SHV_GGML_Q6_K = 14, SHV_GGML_IQ4_NL = 20, SHV_GGML_BF16 = 30
 };
 int64_t shv_ref_type_bytes(int type, int64_t n);
+/* y = W x, rows of W in any accepted type (0 = Q4_K): DequantizeRow then llm/hc.go:255-264 */
+int shv_ref_gemv_any(float *y, int type, const uint8_t *w, const float *x, int n, int k, int threads);
 int shv_ref_dequant(int type, const uint8_t *data, int64_t n, float *dst);
 
 /* ---- Q4_K quantiser (round-to-nearest arm), llm/quantk.go:115-179, llm/sim.go:982-1060,
@@ -91,6 +93,7 @@ typedef struct {
     const uint8_t *up_exps;      /* same */
     const uint8_t *down_exps;    /* Q4_K rows: e*n_embd + j, ffn_expert long */
     const uint8_t *gate_sh, *up_sh, *down_sh;  /* shared expert, same shapes for one expert */
+    int types[6];                /* ggml type of gate_exps, up_exps, down_exps, gate_sh, up_sh, down_sh; 0 = Q4_K */
 } shv_ref_moe_w;
 
 void shv_ref_softmax(float *dst, const float *src, int n);

@@ -664,6 +664,7 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
+    if (shv_moe_up_typed(pa)) return shv_launch_moe_up_any(ctx, pa);
     SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
                 "moe_up: weight banks must be 16-byte aligned");
     dim3 block(kBlock);
@@ -715,6 +716,10 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_down: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used + 1 <= 12, "moe_down: n_used %d; built for up to 11 routed experts", a.n_used);
     SHV_REQUIRE(a.n_embd >= 1 && a.out_stride >= a.n_embd && (!a.residual || a.res_stride >= a.n_embd), "moe_down: strides");
+    if (shv_moe_down_typed(pa)) {
+        SHV_REQUIRE(a.ffn >= 1, "moe_down: ffn %d", a.ffn);
+        return shv_launch_moe_down_any(ctx, pa);
+    }
     SHV_REQUIRE(shv_aligned16(a.down_exps) && shv_aligned16(a.down_sh), "moe_down: weight banks must be 16-byte aligned");
     dim3 block(kBlock);
     switch (a.ffn) {

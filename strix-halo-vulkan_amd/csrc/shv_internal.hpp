@@ -115,6 +115,10 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
 int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
+bool shv_moe_up_typed(const shv_moe_up_args *a);      // any of its banks in a type other than Q4_K
+bool shv_moe_down_typed(const shv_moe_down_args *a);
+int shv_launch_moe_up_any(shv_ctx *ctx, const shv_moe_up_args *a);
+int shv_launch_moe_down_any(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a);
 int shv_launch_embed_typed(shv_ctx *ctx, const shv_embed_args *a);  // a table in a type other than binary16
 long long shv_type_bytes(int type, long long n);                    // bytes of n elements of a ggml type, -1 if refused

@@ -261,7 +261,38 @@ static bool device_expands(uint32_t t) {
     return false;
 }
 
-void Model::LoadGGUF(const gguf::Set &s, bool transcode) {
+// ParseMoEBankPlan (llm/moebank.go:165-215) for the one target this build fits banks to: the
+// families a plan narrows to Q4_K, by the tensor suffix each selects.
+static std::vector<std::string> moe_plan_families(const std::string &spec) {
+    static const char *const fam[6] = {"gate_exps", "up_exps", "down_exps", "gate_shexp", "up_shexp", "down_shexp"};
+    std::vector<std::string> out;
+    size_t at = 0;
+    while (at < spec.size()) {
+        size_t end = spec.find(',', at);
+        if (end == std::string::npos) end = spec.size();
+        const std::string part = spec.substr(at, end - at);
+        at = end + 1;
+        if (part.empty()) continue;
+        const size_t eq = part.find('=');
+        if (eq == std::string::npos) throw Error("llm: LLM_MOE_BANK entry \"" + part + "\" is not family=format");
+        const std::string f = part.substr(0, eq), to = part.substr(eq + 1);
+        if (std::find_if(fam, fam + 6, [&](const char *n) { return f == n; }) == fam + 6)
+            throw Error("llm: LLM_MOE_BANK names family \"" + f + "\"; the six are gate_exps, up_exps, down_exps, gate_shexp, up_shexp, down_shexp");
+        if (to != "q4_k") throw Error("llm: LLM_MOE_BANK " + f + "=" + to + ": q4_k is the format banks are fitted to here");
+        out.push_back("ffn_" + f + ".");
+    }
+    return out;
+}
+
+void Model::LoadGGUF(const gguf::Set &s, const LoadOpts &opts) {
+    const bool transcode = opts.transcode;
+    const std::vector<std::string> narrowed = moe_plan_families(opts.moe_plan);
+    auto is_bank = [](const std::string &n) { return n.find("_exps.") != std::string::npos || n.find("_shexp.") != std::string::npos; };
+    auto plan_narrows = [&](const std::string &n) {
+        for (const std::string &f : narrowed)
+            if (n.find(f) != std::string::npos) return true;
+        return false;
+    };
     std::map<std::string, int64_t> covered;  // rows of each whole tensor that came from the file
     transcoded_.clear();
     // a tensor's bytes as the file holds them, in HBM for the length of one call
@@ -296,6 +327,18 @@ void Model::LoadGGUF(const gguf::Set &s, bool transcode) {
             v.ptr = dev_.alloc(t.Bytes);
             v.bytes = t.Bytes;
             v.kind = t.Type == gguf::F16 ? TensorView::F16 : TensorView::RAW;
+            v.ggml = t.Type;
+            dev_.upload(v.ptr, t.Data, t.Bytes);
+        } else if (v.kind != TensorView::F32 && is_bank(name) && t.Type != gguf::Q4_K && t.Type != gguf::F32 && device_expands(t.Type) &&
+                   !(plan_narrows(name) && t.Bytes > v.bytes)) {
+            // an expert bank in the checkpoint's own type: the expert kernels read it through that type's arm
+            if (t.RowBytes() == 0) throw Error("llm: " + name + " is " + shape + ": rows are not whole blocks of the type");
+            if (v.kind == TensorView::Q4K || v.bytes != t.Bytes) {
+                dev_.release(v.ptr, v.bytes);
+                v.ptr = dev_.alloc(t.Bytes);
+                v.bytes = t.Bytes;
+            }
+            v.kind = TensorView::RAW;
             v.ggml = t.Type;
             dev_.upload(v.ptr, t.Data, t.Bytes);
         } else if (t.Type == same) {
@@ -443,15 +486,22 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     r.n_used = c_.NExpertUsed;
     r.eps = c_.RMSEps;
     r.h_stride = c_.NEmbd;
-    const bool fused = FusedRouter(nTok);
+    const TensorView &ge = m_.Tensor(Model::Blk(l, "ffn_gate_exps")), &ue = m_.Tensor(Model::Blk(l, "ffn_up_exps"));
+    const TensorView &gs = m_.Tensor(Model::Blk(l, "ffn_gate_shexp")), &us = m_.Tensor(Model::Blk(l, "ffn_up_shexp"));
+    const TensorView &de = m_.Tensor(Model::Blk(l, "ffn_down_exps")), &ds = m_.Tensor(Model::Blk(l, "ffn_down_shexp"));
+    // banks in another type than Q4_K take the selection from the router kernel
+    const bool up_q4k = ge.ggml == gguf::Q4_K && ue.ggml == gguf::Q4_K && gs.ggml == gguf::Q4_K && us.ggml == gguf::Q4_K;
+    const bool fused = FusedRouter(nTok) && up_q4k;
     r.defer_route = fused ? 1 : 0;
     shv_moe_up_args u{};
     u.xn = xn_;
     u.topk = topk_;
-    u.gate_exps = m_.Tensor(Model::Blk(l, "ffn_gate_exps")).ptr;
-    u.up_exps = m_.Tensor(Model::Blk(l, "ffn_up_exps")).ptr;
-    u.gate_sh = m_.Tensor(Model::Blk(l, "ffn_gate_shexp")).ptr;
-    u.up_sh = m_.Tensor(Model::Blk(l, "ffn_up_shexp")).ptr;
+    u.gate_exps = ge.ptr;
+    u.up_exps = ue.ptr;
+    u.gate_sh = gs.ptr;
+    u.up_sh = us.ptr;
+    u.gate_type = static_cast<int32_t>(ge.ggml), u.up_type = static_cast<int32_t>(ue.ggml);
+    u.gate_sh_type = static_cast<int32_t>(gs.ggml), u.up_sh_type = static_cast<int32_t>(us.ggml);
     u.act = act_;
     u.n_tok = nTok;
     u.n_embd = c_.NEmbd;
@@ -466,8 +516,9 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     d.act = act_;
     d.topk = topk_;
     d.weights = weights_;
-    d.down_exps = m_.Tensor(Model::Blk(l, "ffn_down_exps")).ptr;
-    d.down_sh = m_.Tensor(Model::Blk(l, "ffn_down_shexp")).ptr;
+    d.down_exps = de.ptr;
+    d.down_sh = ds.ptr;
+    d.down_type = static_cast<int32_t>(de.ggml), d.down_sh_type = static_cast<int32_t>(ds.ggml);
     d.residual = in;
     d.out = out;
     d.n_tok = nTok;

@@ -133,7 +133,21 @@ public:
     // transcode (llm/moebank.go:288-400, rtn arm), a loss on top of a loss — when `transcode`
     // allows it; Transcoded() names those tensors.  Throws, naming the tensor, on a missing
     // tensor, a shape that disagrees with the metadata, or a type that cannot be staged.
-    void LoadGGUF(const gguf::Set &s, bool transcode = true);
+    // Expert banks (ffn_{gate,up,down}_{exps,shexp}) are the exception: the reference stages them in
+    // the checkpoint's own type (llm/gpu_moe.go:673-688) and so does this — a bank in any type the
+    // device expands stays as it is and the expert kernels read it through that type's arm —
+    // unless `moe_plan` (the grammar of LLM_MOE_BANK, llm/moebank.go:55-63: family=q4_k,... with
+    // a family naming a ceiling) narrows that family, which refits the banks wider than Q4_K.
+    struct LoadOpts {
+        bool transcode = true;
+        std::string moe_plan;
+    };
+    void LoadGGUF(const gguf::Set &s, const LoadOpts &o);
+    void LoadGGUF(const gguf::Set &s, bool transcode = true) {
+        LoadOpts o;
+        o.transcode = transcode;
+        LoadGGUF(s, o);
+    }
     const std::vector<std::string> &Transcoded() const { return transcoded_; }
     // This model as one version-3 file the above reads back bit for bit: metadata keys as
     // ConfigFromGGUF reads them, constituents in place of fused tensors, expert banks 3-D.

@@ -119,7 +119,12 @@ int shvllm_open_gguf(int device, const char *path, const shvllm_config *c, shvll
         graph_opts(*h, *c);
         h->model = std::make_unique<llm::Model>(*h->dev, llm::Model::ConfigFromGGUF(*set));
         const char *tc = std::getenv("LLM_TRANSCODE");  // 0: refuse a matrix that is not Q4_K instead of fitting it again
-        h->model->LoadGGUF(*set, !(tc && tc[0] == '0'));
+        llm::Model::LoadOpts lo;
+        lo.transcode = !(tc && tc[0] == '0');
+        if (const char *plan = std::getenv("LLM_MOE_BANK")) lo.moe_plan = plan;  // family=q4_k,...: expert banks refitted instead of read natively
+        if (const char *mode = std::getenv("LLM_MOE_BANK_QUANT"))
+            if (std::strcmp(mode, "rtn") != 0) throw llm::Error(std::string("llm: LLM_MOE_BANK_QUANT=") + mode + "; banks are refitted round-to-nearest here (rtn), no importance matrix is read");
+        h->model->LoadGGUF(*set, lo);
         for (const auto &kv : h->model->Tensors()) h->names.push_back(kv.first);
         *out = h.release();
     });

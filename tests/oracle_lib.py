@@ -34,7 +34,7 @@ class MoeCfg(C.Structure):
 
 class MoeW(C.Structure):
     _fields_ = [("router", f32p), ("shared_gate", f32p), ("gate_exps", u8p), ("up_exps", u8p),
-                ("down_exps", u8p), ("gate_sh", u8p), ("up_sh", u8p), ("down_sh", u8p)]
+                ("down_exps", u8p), ("gate_sh", u8p), ("up_sh", u8p), ("down_sh", u8p), ("types", C.c_int * 6)]
 
 
 class DnCfg(C.Structure):
@@ -230,8 +230,9 @@ class OracleModel:
     """The CPU token loop over a model whose tensors are given by GGUF-style name (numpy arrays):
     Q4_K tensors as bytes, the embedding as binary16 bit patterns, the rest float32."""
 
-    def __init__(self, cfg, tensors, max_cells, sections=(11, 11, 10, 0)):
-        """cfg: any object with the fields of the host layer's config."""
+    def __init__(self, cfg, tensors, max_cells, sections=(11, 11, 10, 0), bank_types=None):
+        """cfg: any object with the fields of the host layer's config.  bank_types: {tensor name:
+        ggml type} for expert banks held in another type than Q4_K."""
         self.cfg, self.t, self.keep = cfg, tensors, []
         ne, d = cfg.n_embd, cfg.ssm_head_dim
         self.mcfg = ModelCfg(
@@ -254,7 +255,9 @@ class OracleModel:
                             F(blk(l, "ssm_a")), F(blk(l, "ssm_dt")), F(blk(l, "ssm_norm")))
             lw.moe = MoeW(F(blk(l, "ffn_gate_inp")), F(blk(l, "ffn_gate_inp_shexp")), B(blk(l, "ffn_gate_exps")),
                           B(blk(l, "ffn_up_exps")), B(blk(l, "ffn_down_exps")), B(blk(l, "ffn_gate_shexp")),
-                          B(blk(l, "ffn_up_shexp")), B(blk(l, "ffn_down_shexp")))
+                          B(blk(l, "ffn_up_shexp")), B(blk(l, "ffn_down_shexp")),
+                          (C.c_int * 6)(*[(bank_types or {}).get("blk.%d.ffn_%s.weight" % (l, n), 0) for n in
+                                          ("gate_exps", "up_exps", "down_exps", "gate_shexp", "up_shexp", "down_shexp")]))
         self.layers = layers
         self.w = ModelW(H(tensors["token_embd.weight"]), F(tensors["output_norm.weight"]),
                         B(tensors["output.weight"]), layers)

@@ -156,13 +156,15 @@ def test_load_refuses_what_it_cannot_stage(saved, tmp_path, monkeypatch):
         LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "nok.gguf", drop={"blk.3.attn_k.weight"}))
     with pytest.raises(ShvError, match=r"0 of 1 rows of output_norm"):
         LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "nonorm.gguf", drop={"output_norm.weight"}))
-    _, dims, data = p["tensors"]["blk.0.ffn_up_shexp.weight"]
+    _, dims, data = p["tensors"]["blk.0.ssm_out.weight"]
     n = int(np.prod(dims))
     q8 = (8, dims, bytes(n // 32 * 34))
     monkeypatch.setenv("LLM_TRANSCODE", "0")
     with pytest.raises(ShvError, match="Q8_0 in the checkpoint; the kernels stream it as Q4_K"):
-        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "q8.gguf", tensors={"blk.0.ffn_up_shexp.weight": q8}))
+        LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "q8.gguf", tensors={"blk.0.ssm_out.weight": q8}))
     monkeypatch.delenv("LLM_TRANSCODE")
+    _, dims, data = p["tensors"]["blk.0.ffn_up_shexp.weight"]
+    n = int(np.prod(dims))
     q2 = (10, dims, bytes(n // 256 * 84))
     with pytest.raises(ShvError, match="blk.0.ffn_up_shexp.weight"):
         LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "q2.gguf", tensors={"blk.0.ffn_up_shexp.weight": q2}))
@@ -180,13 +182,20 @@ def test_load_refuses_what_it_cannot_stage(saved, tmp_path, monkeypatch):
         LA.LLM(small_cfg(), gguf=_rewrite(q, tmp_path / "noarch.gguf"))
 
 
-def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, tmp_path):
-    """What a converter's mixed recipe looks like: the embedding table and the head in Q6_K, expert
-    banks in Q5_K / Q8_0 / IQ4_NL / Q5_1, one constituent of a fused projection in Q5_0, another in
-    F16.  The table stays in its own type (rows expanded by the gather, llm/model.go:125-131); every
-    such matrix is expanded and fitted again as Q4_K, bit for bit what the CPU's dequantiser
-    (gguf/dequant.go:52-98) followed by the CPU's quantiser (llm/quantk.go:115-179) gives; the model
-    then decodes the tokens the CPU model decodes from those weights."""
+BANK_WORDS = ("_exps.", "_shexp.")
+
+
+@pytest.mark.parametrize("plan", ["", "down_exps=q4_k,gate_exps=q4_k,up_shexp=q4_k"])
+def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, tmp_path, monkeypatch, plan):
+    """What a converter's mixed recipe looks like: the embedding table in Q8_0, the head in Q6_K,
+    expert banks in Q5_K / Q8_0 / IQ4_NL / Q5_1, one constituent of a fused projection in Q5_0, others
+    in F16 and Q4_1.  The table stays in its own type (rows expanded by the gather,
+    llm/model.go:125-131) and so do the expert banks (llm/gpu_moe.go:673-688), read through their
+    types' arms; every other such matrix is expanded and fitted again as Q4_K, bit for bit what the
+    CPU's dequantiser (gguf/dequant.go:52-98) followed by the CPU's quantiser
+    (llm/quantk.go:115-179) gives.  Under a plan (LLM_MOE_BANK, llm/moebank.go:55-63) the families
+    it names are refitted too, where they are wider than Q4_K.  Either way the model decodes what
+    the CPU model decodes from the weights as staged."""
     m, cfg, path = saved
     p = GF.parse(path)
     recipe = {"token_embd.weight": "Q8_0", "output.weight": "Q6_K", "blk.0.ffn_down_exps.weight": "Q5_K",
@@ -209,30 +218,38 @@ def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, 
             blocks[:, 0], blocks[:, 1] = 0x00, 0x24
         swap[name] = (typ, dims, raw.tobytes())
         f32[name] = O.dequant(typ, raw, n)
+    if plan:
+        monkeypatch.setenv("LLM_MOE_BANK", plan)
+    # a family's ceiling leaves a bank no wider than Q4_K alone: IQ4_NL stays whatever the plan says
+    refit_banks = {"blk.0.ffn_down_exps.weight", "blk.1.ffn_gate_exps.weight", "blk.1.ffn_up_shexp.weight"} if plan else set()
+    native = {n for n in recipe if any(w in n for w in BANK_WORDS)} - refit_banks
     r = LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "recipe.gguf", tensors=swap))
     try:
-        assert sorted(r.transcoded()) == sorted(n for n in recipe if n != "token_embd.weight")
+        assert sorted(r.transcoded()) == sorted(n for n in recipe if n != "token_embd.weight" and n not in native)
         assert r.tensor_type("token_embd.weight") == 8 and r.tensor_type("output.weight") == 12
-        assert np.array_equal(r.download("token_embd.weight"), np.frombuffer(swap["token_embd.weight"][2], np.uint8))
         for name in recipe:
-            if name == "token_embd.weight":
+            if name == "token_embd.weight" or name in native:
+                assert r.tensor_type(name) == swap[name][0], name
+                assert np.array_equal(r.download(name), np.frombuffer(swap[name][2], np.uint8)), name
                 continue
             k = swap[name][1][0]
             want = O.quantize_q4k(f32[name].reshape(-1, k))
+            assert r.tensor_type(name) == 12
             assert np.array_equal(r.download(name).view(np.uint8), want.reshape(-1)), name
         assert np.array_equal(r.download("blk.3.attn_q.weight"), m.download("blk.3.attn_q.weight"))
-        # saved again, the file names the types now in memory and reads back the same table
+        # saved again, the file names the types now in memory and holds the same bytes
         r.save_gguf(tmp_path / "again.gguf")
         again = GF.parse(tmp_path / "again.gguf")
-        assert again["tensors"]["token_embd.weight"][0] == 8 and again["tensors"]["output.weight"][0] == 12
-        assert again["tensors"]["token_embd.weight"][2] == swap["token_embd.weight"][2]
+        assert again["tensors"]["output.weight"][0] == 12
+        for name in native | {"token_embd.weight"}:
+            assert again["tensors"][name][0] == swap[name][0] and again["tensors"][name][2] == swap[name][2], name
         # the token loop against the CPU loop over the weights as staged
         r.stage()
         tensors = {t[0]: r.download(t[0]) for t in r.tensors()}
         table = f32["token_embd.weight"].astype(np.float16)
         assert np.array_equal(table.astype(np.float32), f32["token_embd.weight"])
         tensors["token_embd.weight"] = table.view(np.uint16)
-        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv, bank_types={n: swap[n][0] for n in native})
         prompt = np.random.default_rng(5).integers(0, cfg.vocab, size=7).astype(np.int32)
         r.reset()
         lg_gpu, hd_gpu = r.extend(prompt, want_hidden=True)
@@ -244,6 +261,18 @@ def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, 
         assert ids[0] == tok or top2[1] - top2[0] < 1e-4
     finally:
         r.close()
+
+
+def test_a_bank_plan_is_held_to_the_grammar(saved, monkeypatch):
+    m, cfg, path = saved
+    for plan, msg in (("down_exps", "is not family=format"), ("ffn_down=q4_k", "names family"), ("down_exps=q5_1", "q4_k is the format")):
+        monkeypatch.setenv("LLM_MOE_BANK", plan)
+        with pytest.raises(ShvError, match=msg):
+            LA.LLM(small_cfg(), gguf=path)
+    monkeypatch.delenv("LLM_MOE_BANK")
+    monkeypatch.setenv("LLM_MOE_BANK_QUANT", "imatrix")
+    with pytest.raises(ShvError, match="no importance matrix"):
+        LA.LLM(small_cfg(), gguf=path)
 
 
 @pytest.mark.parametrize("name", ["Q8_0", "Q6_K", "Q5_K", "IQ4_NL", "BF16"])

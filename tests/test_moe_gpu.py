@@ -4,6 +4,7 @@ import pytest
 
 import oracle_lib as O
 import shv
+from test_dequant_gpu import random_tensor
 
 pytestmark = pytest.mark.gpu
 A = shv.api
@@ -15,7 +16,12 @@ class MoeCase:
     """Seeded synthetic block: router f32 ~N(0,0.02), experts ~N(0,0.02) -> Q4_K by the
     reference quantiser, gamma ~ 1+N(0,0.1), tokens ~N(0,1)."""
 
-    def __init__(self, ctx, seed, H=2048, E=32, used=4, ffn=512, T=1, tie_router=False):
+    BANKS = ("gate_exps", "up_exps", "down_exps", "gate_sh", "up_sh", "down_sh")
+    types = (0,) * 6    # every bank Q4_K unless a case says otherwise
+
+    def __init__(self, ctx, seed, H=2048, E=32, used=4, ffn=512, T=1, tie_router=False, types=None):
+        """types: {bank: tensor type name} for banks held in another type than Q4_K (random blocks
+        of that type with small scales)."""
         rng = np.random.default_rng(seed)
         self.ctx, self.H, self.E, self.used, self.ffn, self.T = ctx, H, E, used, ffn, T
         self.router = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
@@ -26,6 +32,18 @@ class MoeCase:
         self.gate_exps, self.up_exps = q(E * ffn, H), q(E * ffn, H)
         self.down_exps = q(E * H, ffn)
         self.gate_sh, self.up_sh, self.down_sh = q(ffn, H), q(ffn, H), q(H, ffn)
+        self.types = [0] * 6
+        for i, bank in enumerate(self.BANKS):
+            if types and bank in types:
+                name = types[bank]
+                self.types[i] = O.GGML_TYPES[name]
+                n = getattr(self, bank).size // O.q4k_row_bytes(256) * 256
+                if name in ("F16", "BF16"):
+                    v = (rng.standard_normal(n) * 0.02).astype(np.float32)
+                    raw = v.astype(np.float16).view(np.uint8) if name == "F16" else (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+                else:
+                    raw = random_tensor(name, n, seed=seed + i, scale={"Q8_0": 3e-4, "IQ4_NL": 3e-4}.get(name, 1e-4 if name.endswith("_K") else 2e-3))
+                setattr(self, bank, np.ascontiguousarray(raw))
         self.gamma = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
         self.h = rng.standard_normal((T, H)).astype(np.float32)
         self.res = rng.standard_normal((T, H)).astype(np.float32)
@@ -34,7 +52,7 @@ class MoeCase:
         xn = O.rmsnorm(self.h, self.gamma, EPS)
         cfg = O.MoeCfg(self.H, self.E, self.used, self.ffn, self.ffn)
         w = O.MoeW(O.F(self.router), O.F(self.shared_gate), O.B(self.gate_exps), O.B(self.up_exps),
-                   O.B(self.down_exps), O.B(self.gate_sh), O.B(self.up_sh), O.B(self.down_sh))
+                   O.B(self.down_exps), O.B(self.gate_sh), O.B(self.up_sh), O.B(self.down_sh), (O.C.c_int * 6)(*self.types))
         T = self.T
         r = dict(out=np.empty((T, self.H), np.float32), logits=np.empty((T, self.E), np.float32),
                  topk=np.empty((T, self.used), np.int32), weights=np.empty((T, self.used), np.float32),
@@ -58,9 +76,9 @@ class MoeCase:
                              logits.ptr, topk.ptr, weights.ptr, T, H, E, used, EPS, H, 1 if defer else 0)
         ua = A.MoeUpArgs(xn.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr,
                          d["up_sh"].ptr, act.ptr, T, H, used, ffn, logits.ptr if defer else None,
-                         weights.ptr if defer else None, E)
+                         weights.ptr if defer else None, E, self.types[0], self.types[1], self.types[3], self.types[4])
         da = A.MoeDownArgs(act.ptr, topk.ptr, weights.ptr, d["down_exps"].ptr, d["down_sh"].ptr,
-                           d["res"].ptr if residual else None, out.ptr, T, H, used, ffn, H, H)
+                           d["res"].ptr if residual else None, out.ptr, T, H, used, ffn, H, H, self.types[2], self.types[5])
         ops = [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
         c.dispatch_multi(ops)
         return dict(xn=xn.read(np.float32, T * H).reshape(T, H),
@@ -103,6 +121,27 @@ def test_moe_block_matches_oracle(ctx, T, defer):
     """defer: the selection is made by the expert kernel from the router's logits instead of by
     the router's last block; both must give the reference's selection."""
     _check(MoeCase(ctx, seed=100 + T, E=64, used=10, T=T), defer=defer)
+
+
+@pytest.mark.parametrize("types", [
+    dict(gate_exps="Q8_0", up_exps="Q8_0", down_exps="Q8_0", gate_sh="Q8_0", up_sh="Q8_0", down_sh="Q8_0"),
+    dict(down_exps="Q5_K", down_sh="Q6_K"),
+    dict(gate_exps="Q5_K", up_exps="Q6_K", gate_sh="Q5_1", up_sh="Q4_1"),
+    dict(gate_exps="IQ4_NL", down_exps="IQ4_NL", up_sh="Q5_0", down_sh="Q5_1"),
+    dict(up_exps="F16", down_exps="BF16", gate_sh="Q4_K"),
+], ids=lambda d: "+".join(sorted(set(d.values()))))
+@pytest.mark.parametrize("T", [1, 5])
+def test_moe_block_over_banks_in_other_types(ctx, types, T):
+    """Banks read as the checkpoint holds them (llm/gpu_moe.go:673-688, llm_moe_gemv.comp's arms beside
+    Q4_K), routed and shared ones of different types in one block, against the CPU block walking
+    the same banks through Dequantize (llm/moe.go:289-409)."""
+    _check(MoeCase(ctx, seed=300 + T, E=32, used=6, T=T, types=types), residual=True)
+    with pytest.raises(A.ShvError, match="take the selection from the router"):
+        MoeCase(ctx, seed=1, E=16, used=2, T=1, types=dict(gate_exps="Q8_0")).gpu(defer=True)
+    bad = MoeCase(ctx, seed=1, E=16, used=2, T=1)
+    bad.types[2] = 10
+    with pytest.raises(A.ShvError, match="moe_down: rows of 512 elements of ggml type 10"):
+        bad.gpu()
 
 
 def test_moe_block_with_residual_and_few_experts(ctx):
