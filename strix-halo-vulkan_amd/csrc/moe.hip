@@ -10,6 +10,7 @@ using namespace shv;
 
 constexpr int kBlock = 256;
 constexpr int kMaxUsed = 16;
+inline bool is_q4k(int ggml_type) { return ggml_type == 0 || ggml_type == SHV_GGML_Q4_K; }  // 0: the type field left unset
 constexpr float kWeightsSumFloor = 6.103515625e-5f;  // 2^-14
 
 // ---------------------------------------------------------------------------- router ---------
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(kRouteBlock) void moe_route_block_kernel(shv_moe_ro
 // makes over the staged activation row; a launch of many tokens has blocks to spare and uses
 // them to stage the row an eighth as often (64-row chunk: 148 to 119 us a layer).
 template <int K, int P>
-__global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
+__global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int slot0) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     __shared__ float xs[lds_padded(K)];
@@ -430,7 +431,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
     __shared__ int32_t s_topk[kMaxUsed];
     __shared__ float s_w[kMaxUsed + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int slot = blockIdx.y, t = blockIdx.z;
+    const int slot = blockIdx.y + slot0, t = blockIdx.z;  // slot0: a launch over a part of the slots only
     const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
     const int row0 = (blockIdx.x * 4 + wave) * P * RPP + rsub;  // row within the expert, first pass
 
@@ -504,7 +505,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a) {
 // block adds the four waves' sums (and the residual) at the end.  P: passes over the staged
 // activation rows, as in the up projection (eight for many tokens, taken slot after slot).
 template <int K, int MAXS, int P>
-__global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
+__global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a, int s_lo, int s_hi) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int SPW = (MAXS + 3) / 4;  // slots per wave
@@ -527,7 +528,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
         const int s = wave + 4 * i;
         wt[i] = 0.f;
         base[i] = static_cast<const char *>(a.down_sh);
-        if (s < ns) {
+        if (s >= s_lo && s < s_hi) {  // [s_lo, s_hi): the slots this launch adds up
             if (s < a.n_used) {
                 const int e = a.topk[static_cast<size_t>(t) * a.n_used + s];
                 base[i] = static_cast<const char *>(a.down_exps) + static_cast<size_t>(e) * a.n_embd * ROWB;
@@ -546,13 +547,13 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
         const int s = wave + 4 * i;
 #pragma unroll
         for (int j = 0; j < F4; j++)
-            stage[i][j] = s < ns ? *reinterpret_cast<const float4 *>(act + static_cast<size_t>(s) * K + (j * 64 + lane) * 4)
+            stage[i][j] = s >= s_lo && s < s_hi ? *reinterpret_cast<const float4 *>(act + static_cast<size_t>(s) * K + (j * 64 + lane) * 4)
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int i = 0; i < SPW; i++) {
         const int s = wave + 4 * i;
-        if (s < ns) {
+        if (s >= s_lo && s < s_hi) {
 #pragma unroll
             for (int j = 0; j < F4; j++) {
                 const int c = (j * 64 + lane) * 4;  // four consecutive columns never straddle a 64-slice
@@ -572,13 +573,13 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
                 const size_t roff = static_cast<size_t>(row + RPP < a.n_embd ? row + RPP : 0) * ROWB + sb * SHV_Q4K_BYTES;
 #pragma unroll
                 for (int i = 0; i < SPW; i++)
-                    if (wave + 4 * i < ns) w[(p + 1) & 1][i].load(base[i] + roff, g);
+                    if (wave + 4 * i >= s_lo && wave + 4 * i < s_hi) w[(p + 1) & 1][i].load(base[i] + roff, g);
             }
             float acc = 0.f;
 #pragma unroll
             for (int i = 0; i < SPW; i++) {
                 const int s = wave + 4 * i;
-                if (s < ns) {
+                if (s >= s_lo && s < s_hi) {
                     float xr[64], xs_lo, xs_hi;
                     load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
                     acc = fmaf(wt[i], w[p & 1][i].dot(g, nc, xr, xs_lo, xs_hi), acc);
@@ -597,7 +598,7 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a) {
 #pragma unroll
         for (int i = 0; i < SPW; i++) {
             const int s = wave + 4 * i;
-            if (s < ns) {
+            if (s >= s_lo && s < s_hi) {
                 float xr[64], xs_lo, xs_hi;
                 load_x_slice(xs[s], gi, xr, xs_lo, xs_hi);
                 Q4kLane ww[2];
@@ -664,7 +665,12 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
-    if (shv_moe_up_typed(pa)) return shv_launch_moe_up_any(ctx, pa);
+    // Banks of other types than Q4_K go through their own arms; a block whose routed banks and
+    // shared expert differ in that takes one launch each, over its part of the slots.
+    const bool r_other = !is_q4k(a.gate_type) || !is_q4k(a.up_type), s_other = !is_q4k(a.gate_sh_type) || !is_q4k(a.up_sh_type);
+    if (r_other && s_other) return shv_launch_moe_up_any(ctx, pa, 0, a.n_used + 1);
+    if (r_other || s_other) SHV_REQUIRE(!a.logits, "moe_up: banks of other types than Q4_K take the selection from the router, not from logits");
+    const int slot0 = r_other ? a.n_used : 0, slots = r_other ? 1 : s_other ? a.n_used : a.n_used + 1;  // the Q4_K part
     SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
                 "moe_up: weight banks must be 16-byte aligned");
     dim3 block(kBlock);
@@ -675,38 +681,40 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
         case 2048: {
             constexpr int RPP = 64 / (2048 / 64);
             if (many) {
-                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), a.n_used + 1, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 8>), grid, block, 0, a);
+                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), slots, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 8>), grid, block, 0, a, slot0);
             } else {
-                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 1>), grid, block, 0, a);
+                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), slots, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 1>), grid, block, 0, a, slot0);
             }
             break;
         }
         case 1024: {
             constexpr int RPP = 64 / (1024 / 64);
             if (many) {
-                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), a.n_used + 1, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<1024, 8>), grid, block, 0, a);
+                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), slots, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<1024, 8>), grid, block, 0, a, slot0);
             } else {
-                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<1024, 1>), grid, block, 0, a);
+                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), slots, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<1024, 1>), grid, block, 0, a, slot0);
             }
             break;
         }
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
             if (many) {
-                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), a.n_used + 1, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<512, 8>), grid, block, 0, a);
+                dim3 grid((a.ffn + RPP * 32 - 1) / (RPP * 32), slots, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<512, 8>), grid, block, 0, a, slot0);
             } else {
-                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), a.n_used + 1, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<512, 1>), grid, block, 0, a);
+                dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), slots, a.n_tok);
+                SHV_LAUNCH(ctx, (moe_up_kernel<512, 1>), grid, block, 0, a, slot0);
             }
             break;
         }
         default: return shv_set_error(SHV_E_INVALID, "moe_up: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
     }
+    if (r_other) return shv_launch_moe_up_any(ctx, pa, 0, a.n_used);
+    if (s_other) return shv_launch_moe_up_any(ctx, pa, a.n_used, 1);
     return SHV_OK;
 }
 
@@ -716,28 +724,32 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_down: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used + 1 <= 12, "moe_down: n_used %d; built for up to 11 routed experts", a.n_used);
     SHV_REQUIRE(a.n_embd >= 1 && a.out_stride >= a.n_embd && (!a.residual || a.res_stride >= a.n_embd), "moe_down: strides");
-    if (shv_moe_down_typed(pa)) {
-        SHV_REQUIRE(a.ffn >= 1, "moe_down: ffn %d", a.ffn);
-        return shv_launch_moe_down_any(ctx, pa);
-    }
+    SHV_REQUIRE(a.ffn >= 1, "moe_down: ffn %d", a.ffn);
+    // as in the up projection: the Q4_K part of the slots here, the rest through the other arms,
+    // which then add to what this launch has written
+    const bool r_other = !is_q4k(a.down_type), s_other = !is_q4k(a.down_sh_type);
+    if (r_other && s_other) return shv_launch_moe_down_any(ctx, pa, 0, a.n_used + 1, 0);
+    const int s_lo = r_other ? a.n_used : 0, s_hi = s_other ? a.n_used : a.n_used + 1;
     SHV_REQUIRE(shv_aligned16(a.down_exps) && shv_aligned16(a.down_sh), "moe_down: weight banks must be 16-byte aligned");
     dim3 block(kBlock);
     switch (a.ffn) {
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
-            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a);
+            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a, s_lo, s_hi);
             else if (a.n_tok >= 8) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 4>),  // eight sequences decoded together: 5.31 to 5.19 ms a pass
-                dim3((a.n_embd + RPP * 4 - 1) / (RPP * 4), a.n_tok), block, 0, a);
-            else SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
+                dim3((a.n_embd + RPP * 4 - 1) / (RPP * 4), a.n_tok), block, 0, a, s_lo, s_hi);
+            else SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a, s_lo, s_hi);
             break;
         }
         case 256: {
             constexpr int RPP = 64 / (256 / 64);
-            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a);
-            else SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a);
+            if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a, s_lo, s_hi);
+            else SHV_LAUNCH(ctx, (moe_down_kernel<256, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a, s_lo, s_hi);
             break;
         }
         default: return shv_set_error(SHV_E_INVALID, "moe_down: ffn = %d; built for 256 and 512", a.ffn);
     }
+    if (r_other) return shv_launch_moe_down_any(ctx, pa, 0, a.n_used, 1);
+    if (s_other) return shv_launch_moe_down_any(ctx, pa, a.n_used, a.n_used + 1, 1);
     return SHV_OK;
 }

@@ -17,11 +17,11 @@ constexpr int kRowsPerBlock = 4 * kRowsPerWave;
 
 __host__ __device__ inline int bank_type(int t) { return t == 0 ? SHV_GGML_Q4_K : t; }
 
-// grid (ceil(ffn / 16), n_used + 1, n_tok): act[t][slot][row] = silu(Wg row . xn[t]) * (Wu row . xn[t])
-__global__ __launch_bounds__(kBlock) void moe_up_any_kernel(shv_moe_up_args a) {
+// grid (ceil(ffn / 16), slots, n_tok), slot = blockIdx.y + slot0: act[t][slot][row] = silu(Wg row . xn[t]) * (Wu row . xn[t])
+__global__ __launch_bounds__(kBlock) void moe_up_any_kernel(shv_moe_up_args a, int slot0, int rpw) {
     extern __shared__ __align__(16) float xs[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int slot = blockIdx.y, t = blockIdx.z;
+    const int slot = blockIdx.y + slot0, t = blockIdx.z;
     const float *x = a.xn + static_cast<size_t>(t) * a.n_embd;
     for (int c = tid; c < a.n_embd; c += kBlock) xs[c] = x[c];
     __syncthreads();
@@ -33,8 +33,8 @@ __global__ __launch_bounds__(kBlock) void moe_up_any_kernel(shv_moe_up_args a) {
     const uint8_t *ub = static_cast<const uint8_t *>(routed ? a.up_exps : a.up_sh) + e * a.ffn * urb;
     float *act = a.act + (static_cast<size_t>(t) * (a.n_used + 1) + slot) * a.ffn;
     const int groups = a.n_embd / 32;
-    for (int r = 0; r < kRowsPerWave; r++) {
-        const int row = (blockIdx.x * 4 + wave) * kRowsPerWave + r;
+    for (int r = 0; r < rpw; r++) {  // rpw rows a wave: fewer when the launch would otherwise leave CUs idle
+        const int row = (blockIdx.x * 4 + wave) * rpw + r;
         if (row >= a.ffn) break;  // uniform over the wave
         float g = 0.f, u = 0.f;
         for (int q = lane; q < groups; q += 64) {
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kBlock) void moe_up_any_kernel(shv_moe_up_args a) {
 // grid (ceil(n_embd / 4), n_tok), a wave per output row: out[t][row] = residual + sum_slot weights[t][slot] *
 // (Wd_slot row . act[t][slot]).  The lanes of a wave share out the (slot, group) pairs of the row; the
 // activations (a few KB a token, shared by every block) are read where they lie.
-__global__ __launch_bounds__(kBlock) void moe_down_any_kernel(shv_moe_down_args a) {
+__global__ __launch_bounds__(kBlock) void moe_down_any_kernel(shv_moe_down_args a, int s_lo, int s_hi, int add) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t = blockIdx.y, ns = a.n_used + 1;
     const int row = blockIdx.x * 4 + wave;
@@ -60,47 +60,47 @@ __global__ __launch_bounds__(kBlock) void moe_down_any_kernel(shv_moe_down_args 
     const float *wt = a.weights + static_cast<size_t>(t) * ns;
     const int rt = bank_type(a.down_type), st = bank_type(a.down_sh_type);
     const long long rrb = row_bytes(rt, a.ffn), srb = row_bytes(st, a.ffn);
-    const int gpr = a.ffn / 32, routed = a.n_used * gpr;
+    // slots [s_lo, s_hi) only; add: on top of what out already holds (another launch wrote the other slots)
+    const int gpr = a.ffn / 32, r_hi = s_hi < a.n_used ? s_hi : a.n_used, routed = (r_hi - s_lo) * gpr;
     float acc = 0.f;
     for (int p = lane; p < routed; p += 64) {
-        const int slot = p / gpr, q = p - slot * gpr;
+        const int slot = s_lo + p / gpr, q = p - (slot - s_lo) * gpr;
         const uint8_t *rp = static_cast<const uint8_t *>(a.down_exps) + (static_cast<long long>(tk[slot]) * a.n_embd + row) * rrb;
         acc = fmaf(wt[slot], group_dot_rt(rt, rp, q, acts + slot * a.ffn + q * 32), acc);
     }
-    for (int q = lane; q < gpr; q += 64)
+    for (int q = lane; q < gpr && s_hi > a.n_used; q += 64)
         acc = fmaf(wt[a.n_used], group_dot_rt(st, static_cast<const uint8_t *>(a.down_sh) + row * srb, q, acts + a.n_used * a.ffn + q * 32), acc);
     acc = wave_sum_all(acc);
     if (lane == 0) {
-        const float res = a.residual ? a.residual[static_cast<size_t>(t) * a.res_stride + row] : 0.f;
-        a.out[static_cast<size_t>(t) * a.out_stride + row] = res + acc;
+        float *o = a.out + static_cast<size_t>(t) * a.out_stride + row;
+        const float res = add ? *o : a.residual ? a.residual[static_cast<size_t>(t) * a.res_stride + row] : 0.f;
+        *o = res + acc;
     }
 }
 
 }  // namespace
 
-bool shv_moe_up_typed(const shv_moe_up_args *a) {
-    return bank_type(a->gate_type) != SHV_GGML_Q4_K || bank_type(a->up_type) != SHV_GGML_Q4_K || bank_type(a->gate_sh_type) != SHV_GGML_Q4_K ||
-           bank_type(a->up_sh_type) != SHV_GGML_Q4_K;
-}
-bool shv_moe_down_typed(const shv_moe_down_args *a) { return bank_type(a->down_type) != SHV_GGML_Q4_K || bank_type(a->down_sh_type) != SHV_GGML_Q4_K; }
-
-int shv_launch_moe_up_any(shv_ctx *ctx, const shv_moe_up_args *pa) {
+int shv_launch_moe_up_any(shv_ctx *ctx, const shv_moe_up_args *pa, int slot0, int slots) {
     const shv_moe_up_args &a = *pa;
     SHV_REQUIRE(!a.logits, "moe_up: banks of other types than Q4_K take the selection from the router, not from logits");
-    const int types[4] = {bank_type(a.gate_type), bank_type(a.up_type), bank_type(a.gate_sh_type), bank_type(a.up_sh_type)};
+    const bool routed = slot0 < a.n_used, shared = slot0 + slots > a.n_used;
+    const int types[4] = {routed ? bank_type(a.gate_type) : SHV_GGML_Q4_K, routed ? bank_type(a.up_type) : SHV_GGML_Q4_K,
+                          shared ? bank_type(a.gate_sh_type) : SHV_GGML_Q4_K, shared ? bank_type(a.up_sh_type) : SHV_GGML_Q4_K};
     for (int t : types)
         SHV_REQUIRE(t != SHV_GGML_F32 && whole_rows(t, a.n_embd), "moe_up: rows of %d elements of ggml type %d (not a type a bank can be, or not whole blocks)", a.n_embd, t);
     const size_t lds = static_cast<size_t>(a.n_embd) * 4;
     SHV_REQUIRE(lds <= 48 * 1024, "moe_up: n_embd %d does not fit the staging of a row", a.n_embd);
-    SHV_LAUNCH(ctx, moe_up_any_kernel, dim3((a.ffn + kRowsPerBlock - 1) / kRowsPerBlock, a.n_used + 1, a.n_tok), dim3(kBlock), lds, a);
+    const long long tall = static_cast<long long>((a.ffn + kRowsPerBlock - 1) / kRowsPerBlock) * slots * a.n_tok;
+    const int rpw = tall >= 2 * ctx->prop.multiProcessorCount ? kRowsPerWave : 1;
+    SHV_LAUNCH(ctx, moe_up_any_kernel, dim3((a.ffn + 4 * rpw - 1) / (4 * rpw), slots, a.n_tok), dim3(kBlock), lds, a, slot0, rpw);
     return SHV_OK;
 }
 
-int shv_launch_moe_down_any(shv_ctx *ctx, const shv_moe_down_args *pa) {
+int shv_launch_moe_down_any(shv_ctx *ctx, const shv_moe_down_args *pa, int s_lo, int s_hi, int add) {
     const shv_moe_down_args &a = *pa;
-    const int types[2] = {bank_type(a.down_type), bank_type(a.down_sh_type)};
+    const int types[2] = {s_lo < a.n_used ? bank_type(a.down_type) : SHV_GGML_Q4_K, s_hi > a.n_used ? bank_type(a.down_sh_type) : SHV_GGML_Q4_K};
     for (int t : types)
         SHV_REQUIRE(t != SHV_GGML_F32 && whole_rows(t, a.ffn), "moe_down: rows of %d elements of ggml type %d (not a type a bank can be, or not whole blocks)", a.ffn, t);
-    SHV_LAUNCH(ctx, moe_down_any_kernel, dim3((a.n_embd + 3) / 4, a.n_tok), dim3(kBlock), 0, a);
+    SHV_LAUNCH(ctx, moe_down_any_kernel, dim3((a.n_embd + 3) / 4, a.n_tok), dim3(kBlock), 0, a, s_lo, s_hi, add);
     return SHV_OK;
 }

@@ -115,10 +115,10 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
 int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
 int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
-bool shv_moe_up_typed(const shv_moe_up_args *a);      // any of its banks in a type other than Q4_K
-bool shv_moe_down_typed(const shv_moe_down_args *a);
-int shv_launch_moe_up_any(shv_ctx *ctx, const shv_moe_up_args *a);
-int shv_launch_moe_down_any(shv_ctx *ctx, const shv_moe_down_args *a);
+// expert banks in other types than Q4_K: slots [slot0, slot0 + slots) of the up projection; slots
+// [s_lo, s_hi) of the down projection, added to out when `add` (another launch wrote the rest)
+int shv_launch_moe_up_any(shv_ctx *ctx, const shv_moe_up_args *a, int slot0, int slots);
+int shv_launch_moe_down_any(shv_ctx *ctx, const shv_moe_down_args *a, int s_lo, int s_hi, int add);
 int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a);
 int shv_launch_embed_typed(shv_ctx *ctx, const shv_embed_args *a);  // a table in a type other than binary16
 long long shv_type_bytes(int type, long long n);                    // bytes of n elements of a ggml type, -1 if refused

@@ -128,9 +128,10 @@ def test_moe_block_matches_oracle(ctx, T, defer):
     dict(down_exps="Q5_K", down_sh="Q6_K"),
     dict(gate_exps="Q5_K", up_exps="Q6_K", gate_sh="Q5_1", up_sh="Q4_1"),
     dict(gate_exps="IQ4_NL", down_exps="IQ4_NL", up_sh="Q5_0", down_sh="Q5_1"),
-    dict(up_exps="F16", down_exps="BF16", gate_sh="Q4_K"),
-], ids=lambda d: "+".join(sorted(set(d.values()))))
-@pytest.mark.parametrize("T", [1, 5])
+    dict(up_exps="F16", down_exps="BF16", gate_sh="Q4_K"),        # routed slots on the other arms, the shared expert on the Q4_K kernels
+    dict(gate_sh="Q8_0", up_sh="Q8_0", down_sh="Q8_0"),           # and the other way round: what a converter's 8-bit shared expert gives
+], ids=lambda d: "+".join(sorted(set(d.values()))) + "-" + str(len(d)))
+@pytest.mark.parametrize("T", [1, 5, 17])
 def test_moe_block_over_banks_in_other_types(ctx, types, T):
     """Banks read as the checkpoint holds them (llm/gpu_moe.go:673-688, llm_moe_gemv.comp's arms beside
     Q4_K), routed and shared ones of different types in one block, against the CPU block walking
