@@ -58,6 +58,7 @@ int shv_launch_gemv(shv_ctx *ctx, const shv_gemv_args *pa) {
     const shv_gemv_args &a = *pa;
     SHV_REQUIRE(a.w && a.x && a.y, "gemv: NULL w, x or y");
     SHV_REQUIRE(a.n > 0 && a.k > 0, "gemv: %d x %d", a.n, a.k);
+    SHV_REQUIRE(shv_aligned16(a.w), "gemv: the weight matrix must be 16-byte aligned");
     const int blk = a.type == SHV_GGML_Q4_K || a.type == SHV_GGML_Q5_K || a.type == SHV_GGML_Q6_K ? 256 : 32;
     SHV_REQUIRE(row_bytes(a.type, a.k) > 0 && a.k % blk == 0, "gemv: rows of %d elements of ggml type %d (not a type the loader accepts, or not whole blocks)", a.k, a.type);
     switch (a.type) {

@@ -88,6 +88,8 @@ int shv_launch_moe_up_any(shv_ctx *ctx, const shv_moe_up_args *pa, int slot0, in
                           shared ? bank_type(a.gate_sh_type) : SHV_GGML_Q4_K, shared ? bank_type(a.up_sh_type) : SHV_GGML_Q4_K};
     for (int t : types)
         SHV_REQUIRE(t != SHV_GGML_F32 && whole_rows(t, a.n_embd), "moe_up: rows of %d elements of ggml type %d (not a type a bank can be, or not whole blocks)", a.n_embd, t);
+    SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
+                "moe_up: weight banks must be 16-byte aligned");
     const size_t lds = static_cast<size_t>(a.n_embd) * 4;
     SHV_REQUIRE(lds <= 48 * 1024, "moe_up: n_embd %d does not fit the staging of a row", a.n_embd);
     const long long tall = static_cast<long long>((a.ffn + kRowsPerBlock - 1) / kRowsPerBlock) * slots * a.n_tok;
@@ -101,6 +103,7 @@ int shv_launch_moe_down_any(shv_ctx *ctx, const shv_moe_down_args *pa, int s_lo,
     const int types[2] = {s_lo < a.n_used ? bank_type(a.down_type) : SHV_GGML_Q4_K, s_hi > a.n_used ? bank_type(a.down_sh_type) : SHV_GGML_Q4_K};
     for (int t : types)
         SHV_REQUIRE(t != SHV_GGML_F32 && whole_rows(t, a.ffn), "moe_down: rows of %d elements of ggml type %d (not a type a bank can be, or not whole blocks)", a.ffn, t);
+    SHV_REQUIRE(shv_aligned16(a.down_exps) && shv_aligned16(a.down_sh) && shv_aligned16(a.act), "moe_down: weight banks and activations must be 16-byte aligned");
     SHV_LAUNCH(ctx, moe_down_any_kernel, dim3((a.n_embd + 3) / 4, a.n_tok), dim3(kBlock), 0, a, s_lo, s_hi, add);
     return SHV_OK;
 }
