@@ -219,7 +219,11 @@ typedef struct {
  * read.  Banks are GGUF Q4_K: expert e's row j is row e*ffn + j, n_embd long.
  * When logits is given ([T][n_expert+1] from a router run with defer_route) every block first
  * routes its token from them exactly as the router would, and the selection is also stored to
- * topk [T][n_used] and weights [T][n_used+1] for the down projection; otherwise topk is read. */
+ * topk [T][n_used] and weights [T][n_used+1] for the down projection; otherwise topk is read.
+ * A pass of many rows (128 and more; SHV_MOE_GROUP_MIN) whose topk is given, with n_expert stated
+ * and a `group` workspace of n_expert + 1 + T * n_used ints, is grouped by expert on the matrix
+ * cores: an expert's weights are read once per 16 tokens that chose it (the prompt arm of
+ * llm_moe_gemv.comp). */
 typedef struct {
     const float *xn;
     int32_t *topk;
@@ -235,11 +239,15 @@ typedef struct {
      * checkpoint holds it (llm_moe_gemv.comp's other arms; llm/gpu_moe.go:673-688), rows as
      * Tensor.DequantizeRow forms them; the selection then comes from the router (logits NULL). */
     int32_t gate_type, up_type, gate_sh_type, up_sh_type;
+    int32_t *group;          /* workspace of the grouped path, or NULL */
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +
  * llm_moe_combine.comp): out[t] = residual[t] + sum_s weights[t][s] * (Wd_e act[t][s])
- * + weights[t][n_used] * (Wd_shared act[t][n_used]).  residual may be NULL. */
+ * + weights[t][n_used] * (Wd_shared act[t][n_used]).  residual may be NULL.
+ * Grouped by expert as shv_moe_up is when the caller gives n_expert, a `group` workspace of the
+ * same size and `pairs`, [T][n_used+1][n_embd] floats for the products of every (token, slot)
+ * before they are weighted and summed in slot order. */
 typedef struct {
     const float *act;
     const int32_t *topk;
@@ -250,6 +258,9 @@ typedef struct {
     int32_t n_tok, n_embd, n_used, ffn;
     int32_t res_stride, out_stride;
     int32_t down_type, down_sh_type;  /* as in shv_moe_up_args: 0 or SHV_GGML_Q4_K, or the bank's own type */
+    int32_t n_expert;        /* the grouped path: experts in the bank, */
+    int32_t *group;          /* its workspace */
+    float *pairs;            /* and the per-pair products; NULL keeps the per-(token, slot) kernels */
 } shv_moe_down_args;
 
 /* Gated DeltaNet step(s) after the fused projection (DeltaNetLayer, llm/deltanet.go:266-327 and

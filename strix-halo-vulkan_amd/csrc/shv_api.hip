@@ -42,6 +42,10 @@ int shv_init(int device, shv_ctx **out) {
         const int v = std::atoi(e);
         if (v >= 2) ctx->mfma_min_rows = ctx->mfma_min_rows_wide = v;
     }
+    if (const char *e = std::getenv("SHV_MOE_GROUP_MIN")) {
+        const int v = std::atoi(e);
+        if (v >= 1) ctx->moe_group_min = v;
+    }
     if (const char *e = std::getenv("SHV_MOE_TALL_MIN")) {
         const int v = std::atoi(e);
         if (v >= 1) ctx->moe_tall_min = v;

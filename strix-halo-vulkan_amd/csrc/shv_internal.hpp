@@ -23,6 +23,7 @@ struct shv_ctx {
     // operands).  SHV_MFMA_MIN_ROWS in the environment sets both; a large value keeps every pass
     // on the row kernel.
     int mfma_min_rows = 3, mfma_min_rows_wide = 5;
+    int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)
     int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     // scratch the library's own kernels need (arrival counters for last-block epilogues)
@@ -113,6 +114,11 @@ int shv_launch_fill_normal(shv_ctx *ctx, const shv_fill_normal_args *a);
 int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *a);
 int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *a);
 int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *a);
+// passes of many rows grouped by expert on the matrix cores (moe_grouped.hip)
+bool shv_moe_up_grouped_covers(const shv_ctx *ctx, const shv_moe_up_args &a);
+int shv_launch_moe_up_grouped(shv_ctx *ctx, const shv_moe_up_args &a);
+bool shv_moe_down_grouped_covers(const shv_ctx *ctx, const shv_moe_down_args &a);
+int shv_launch_moe_down_grouped(shv_ctx *ctx, const shv_moe_down_args &a);
 int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *a);
 int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
 // expert banks in other types than Q4_K: slots [slot0, slot0 + slots) of the up projection; slots

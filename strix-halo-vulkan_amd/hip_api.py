@@ -75,7 +75,8 @@ class MoeUpArgs(C.Structure):
                 ("act", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("logits", C.c_void_p),
                 ("weights", C.c_void_p), ("n_expert", C.c_int32), ("gate_type", C.c_int32),
-                ("up_type", C.c_int32), ("gate_sh_type", C.c_int32), ("up_sh_type", C.c_int32)]
+                ("up_type", C.c_int32), ("gate_sh_type", C.c_int32), ("up_sh_type", C.c_int32),
+                ("group", C.c_void_p)]
 
 
 class MoeDownArgs(C.Structure):
@@ -83,7 +84,8 @@ class MoeDownArgs(C.Structure):
                 ("down_exps", C.c_void_p), ("down_sh", C.c_void_p), ("residual", C.c_void_p),
                 ("out", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("res_stride", C.c_int32),
-                ("out_stride", C.c_int32), ("down_type", C.c_int32), ("down_sh_type", C.c_int32)]
+                ("out_stride", C.c_int32), ("down_type", C.c_int32), ("down_sh_type", C.c_int32),
+                ("n_expert", C.c_int32), ("group", C.c_void_p), ("pairs", C.c_void_p)]
 
 
 class DnStepArgs(C.Structure):

@@ -455,6 +455,12 @@ MoEGPU::MoEGPU(Device &dev, const Model &m, int maxTokens) : dev_(dev), m_(m), c
     topk_ = static_cast<int32_t *>(dev.alloc(T * c_.NExpertUsed * 4));
     weights_ = static_cast<float *>(dev.alloc(T * (c_.NExpertUsed + 1) * 4));
     act_ = static_cast<float *>(dev.alloc(T * (c_.NExpertUsed + 1) * c_.FFNExpert * 4));
+    // passes of many rows go grouped by expert on the matrix cores and need the per-expert lists
+    // and every (token, slot)'s down products before they are summed
+    if (maxTokens > kBlockRows) {
+        group_ = static_cast<int32_t *>(dev.alloc((c_.NExpert + 1 + T * c_.NExpertUsed) * 4));
+        pairs_ = static_cast<float *>(dev.alloc(T * (c_.NExpertUsed + 1) * c_.NEmbd * 4));
+    }
     act_bytes_ = T * (3ull * c_.NEmbd + c_.NExpert + 1 + 2 * c_.NExpertUsed + 1 + (c_.NExpertUsed + 1ull) * c_.FFNExpert) * 4;
 }
 
@@ -507,12 +513,17 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     u.n_embd = c_.NEmbd;
     u.n_used = c_.NExpertUsed;
     u.ffn = c_.FFNExpert;
+    u.n_expert = c_.NExpert;
     if (fused) {
         u.logits = logits_;
         u.weights = weights_;
-        u.n_expert = c_.NExpert;
+    } else {
+        u.group = group_;
     }
     shv_moe_down_args d{};
+    d.n_expert = c_.NExpert;
+    d.group = group_;
+    d.pairs = pairs_;
     d.act = act_;
     d.topk = topk_;
     d.weights = weights_;
@@ -1000,7 +1011,7 @@ static void drop_passes(Device &dev, std::map<std::vector<int>, Pass> &passes) {
 Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_(m), c_(m.config()), o_(opts) {
     layers_ = opts.Layers > 0 ? opts.Layers : c_.NLayer;
     if (layers_ > c_.NLayer) throw Error("llm: NewGraph: " + std::to_string(layers_) + " layers of a " + std::to_string(c_.NLayer) + "-layer model");
-    if (o_.MaxTokens < 1 || o_.MaxTokens > 64) throw Error("llm: NewGraph: MaxTokens " + std::to_string(o_.MaxTokens) + "; a pass carries 1..64 rows");
+    if (o_.MaxTokens < 1 || o_.MaxTokens > 4096) throw Error("llm: NewGraph: MaxTokens " + std::to_string(o_.MaxTokens) + "; a pass carries 1..4096 rows");
     if (o_.Slots < 1 || o_.Slots > 32) throw Error("llm: NewGraph: Slots " + std::to_string(o_.Slots) + "; 1..32");
     if (o_.NKV < 2) throw Error("llm: NewGraph: NKV " + std::to_string(o_.NKV));
     if (o_.Speculative && (o_.SpecRows < 2 || o_.SpecRows > 8)) throw Error("llm: NewGraph: SpecRows " + std::to_string(o_.SpecRows) + "; 2..8");
@@ -1025,9 +1036,12 @@ Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_
     for (size_t i = 0; i < S; i++) ix[i] = static_cast<int32_t>(i);
     dev.upload(slot_ix_, ix.data(), S * 4);
     best_ = static_cast<int32_t *>(dev.alloc_zero(64 * 4));
+    // a pass of more rows than a block takes goes through the attention / DeltaNet blocks in
+    // groups of kBlockRows, layer by layer, and through the experts whole
+    block_rows_ = std::min(rows_max_, kBlockRows);
     moe_ = new MoEGPU(dev, m, rows_max_);
-    dn_ = new DeltaNetGPU(dev, m, rows_max_, o_.Slots, pos_, planes, plane_);
-    attn_ = new AttnGPU(dev, m, rows_max_, o_.NKV, o_.Slots, pos_);
+    dn_ = new DeltaNetGPU(dev, m, block_rows_, o_.Slots, pos_, planes, plane_);
+    attn_ = new AttnGPU(dev, m, block_rows_, o_.NKV, o_.Slots, pos_);
     if (o_.AttnSplits > 0) attn_->SetSplits(o_.AttnSplits);
     if (!o_.NoHead) head_ = new HeadGPU(dev, m, head_rows);
     // the decode step of slot 0 is recorded up front, as NewGraph does (llm/graph.go:609)
@@ -1083,9 +1097,26 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     }
     p.ops.push_back(make_op(SHV_OP_EMBED, e));
     p.labels.push_back("embed");
+    if (rows > block_rows_ && (kind == kBatch || spec)) throw Error("llm: a pass of " + std::to_string(rows) + " rows is a plain prompt pass; batched and rewindable passes carry up to " + std::to_string(block_rows_));
     for (int l = 0; l < layers_; l++) {
-        auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, r, &p.labels) : dn_->Dispatches(l, x_, x_, r, &p.labels);
-        p.ops.insert(p.ops.end(), sub.begin(), sub.end());
+        if (rows <= block_rows_) {
+            auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, r, &p.labels) : dn_->Dispatches(l, x_, x_, r, &p.labels);
+            p.ops.insert(p.ops.end(), sub.begin(), sub.end());
+        } else {
+            // The sequence's position on the device moves on group by group, so that every group
+            // finds its cells, ring rows and rotary angles where a pass of its own would; after
+            // the last group it goes back for the next layer.
+            for (int r0 = 0; r0 < rows; r0 += block_rows_) {
+                PassRows g = r;
+                g.seq_len = std::min(block_rows_, rows - r0);
+                float *xg = x_ + static_cast<size_t>(r0) * c_.NEmbd;
+                auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, xg, xg, g, &p.labels) : dn_->Dispatches(l, xg, xg, g, &p.labels);
+                p.ops.insert(p.ops.end(), sub.begin(), sub.end());
+                shv_advance_args step{pos_ + slot, 1, r0 + g.seq_len < rows ? g.seq_len : -r0};
+                p.ops.push_back(make_op(SHV_OP_ADVANCE, step));
+                p.labels.push_back("advance");
+            }
+        }
         auto ffn = moe_->Dispatches(l, x_, x_, rows, &p.labels);
         p.ops.insert(p.ops.end(), ffn.begin(), ffn.end());
     }

@@ -216,8 +216,8 @@ private:
     const Model &m_;
     Config c_;
     int max_tok_, n_tok_ = 0;
-    float *in_, *out_, *xn_, *logits_, *weights_, *act_;
-    int32_t *topk_;
+    float *in_, *out_, *xn_, *logits_, *weights_, *act_, *pairs_ = nullptr;
+    int32_t *topk_, *group_ = nullptr;
     uint64_t act_bytes_ = 0;
     int route_mode_ = 0;  // 0 own dispatch, 1 fused, 2 fused for one-row passes
 };
@@ -323,8 +323,11 @@ private:
 };
 
 // llm.GraphOpts (llm/graph.go:58-126), the fields that apply here.
+// Rows an attention or DeltaNet block takes in one go; a pass of more rows walks them in groups.
+constexpr int kBlockRows = 64;
+
 struct GraphOpts {
-    int MaxTokens = 1;  // rows a pass may carry (a longer prompt goes through in chunks of this)
+    int MaxTokens = 1;  // rows a pass may carry, up to 4096 (a longer prompt goes through in chunks of this)
     int NKV = 4096;     // attention cache cells per slot
     int Layers = 0;     // 0: all of the model's layers
     bool NoHead = false;
@@ -439,7 +442,7 @@ private:
     const Model &m_;
     Config c_;
     GraphOpts o_;
-    int layers_, rows_max_, slot_ = 0;
+    int layers_, rows_max_, block_rows_ = 1, slot_ = 0;
     std::vector<Seq> seq_;
     bool spec_ = false, spec_first_ = false, spec_armed_ = false;
     int spec_past_ = 0, spec_rows_ = 0;

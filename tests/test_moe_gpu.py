@@ -64,7 +64,9 @@ class MoeCase:
         r["xn"] = xn
         return r
 
-    def gpu(self, residual=False, defer=False):
+    def gpu(self, residual=False, defer=False, grouped=False):
+        """grouped: hand the expert kernels the workspaces that let a pass of many rows go grouped by
+        expert on the matrix cores."""
         c, T, H, E, used, ffn = self.ctx, self.T, self.H, self.E, self.used, self.ffn
         d = {k: c.upload(getattr(self, k)) for k in
              ("router", "shared_gate", "gate_exps", "up_exps", "down_exps", "gate_sh", "up_sh",
@@ -76,9 +78,15 @@ class MoeCase:
                              logits.ptr, topk.ptr, weights.ptr, T, H, E, used, EPS, H, 1 if defer else 0)
         ua = A.MoeUpArgs(xn.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr,
                          d["up_sh"].ptr, act.ptr, T, H, used, ffn, logits.ptr if defer else None,
-                         weights.ptr if defer else None, E, self.types[0], self.types[1], self.types[3], self.types[4])
+                         weights.ptr if defer else None, E, self.types[0], self.types[1], self.types[3], self.types[4],
+                         None)
         da = A.MoeDownArgs(act.ptr, topk.ptr, weights.ptr, d["down_exps"].ptr, d["down_sh"].ptr,
-                           d["res"].ptr if residual else None, out.ptr, T, H, used, ffn, H, H, self.types[2], self.types[5])
+                           d["res"].ptr if residual else None, out.ptr, T, H, used, ffn, H, H, self.types[2], self.types[5],
+                           E, None, None)
+        if grouped:
+            group, pairs = c.alloc((E + 1 + T * used) * 4), c.alloc(T * (used + 1) * H * 4)
+            ua.group = da.group = group.ptr
+            da.pairs = pairs.ptr
         ops = [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
         c.dispatch_multi(ops)
         return dict(xn=xn.read(np.float32, T * H).reshape(T, H),
@@ -143,6 +151,28 @@ def test_moe_block_over_banks_in_other_types(ctx, types, T):
     bad.types[2] = 10
     with pytest.raises(A.ShvError, match="moe_down: rows of 512 elements of ggml type 10"):
         bad.gpu()
+
+
+@pytest.mark.parametrize("T,E,used,seed", [(160, 64, 10, 165), (131, 16, 4, 137), (128, 64, 1, 264)])
+def test_many_rows_grouped_by_expert_match_oracle(ctx, T, E, used, seed):
+    """Passes of 128 rows and more, given workspaces, run the experts grouped on the matrix cores:
+    whole and ragged token tiles, experts wanted by several tiles of 16 tokens and by none, with
+    the residual (seeds chosen clear of near-ties in the routing).  The grouped products also
+    agree with the per-(token, slot) kernels' to rounding."""
+    case = MoeCase(ctx, seed=seed, E=E, used=used, T=T)
+    want = case.oracle()
+    for t in range(T):
+        p = np.exp(want["logits"][t].astype(np.float64) - want["logits"][t].max())
+        if _margin(p / p.sum(), used) <= 1e-4:
+            pytest.skip("seed sits on a near-tie; pick another")
+    got = case.gpu(residual=True, grouped=True)
+    ref = case.gpu(residual=True)
+    assert np.array_equal(got["topk"], want["topk"]) and np.array_equal(ref["topk"], want["topk"])
+    assert O.rel_l2(got["act"][:, :used], want["swiglu"]) <= TOL
+    assert O.rel_l2(got["out"], want["out"] + case.res) <= TOL
+    assert O.rel_l2(got["act"], ref["act"]) <= 1e-5
+    assert O.rel_l2(got["out"], ref["out"]) <= 1e-5
+    assert not np.array_equal(got["out"], ref["out"]), "the workspaces were given: the grouped kernels should have run"
 
 
 def test_moe_block_with_residual_and_few_experts(ctx):

@@ -63,6 +63,40 @@ def test_chunked_prompt_matches_the_cpu(rig):
     assert O.rel_l2(kf(k), kf(om.kc[3][:11])) <= 2e-3 and O.rel_l2(kf(v), kf(om.vc[3][:11])) <= 2e-3
 
 
+def test_long_pass_matches_the_cpu():
+    """A pass of more rows than an attention or DeltaNet block takes (64): 150 prompt rows go through
+    as one pass of 136 — the blocks in groups of 64 + 64 + 8 rows layer by layer, the experts over all
+    136 rows grouped by expert on the matrix cores — and one of 14.  Last row, carried state and cache
+    are the CPU's, and the same rows in passes of 64 agree to rounding."""
+    rng = np.random.default_rng(150)
+    out = {}
+    for rows in (136, 64):
+        cfg = cfg_rows(max_tokens=rows, nkv=256, slots=1, head_rows=1, speculative=0, nextn=0)
+        prompt = rng.integers(0, cfg.vocab, size=150).astype(np.int32) if rows == 136 else prompt
+        m = LA.LLM(cfg)
+        m.init_synthetic(4321)
+        m.stage()
+        lg, hd = m.extend(prompt, want_hidden=True)
+        assert m.past() == 150
+        if rows == 136:
+            tensors = {t[0]: m.download(t[0]) for t in m.tensors()}
+        out[rows] = (lg, hd, m.dn_state(0), m.dn_state(2), m.kv(3, 150))
+        nxt = m.generate(4)
+        out[rows] += (nxt,)
+        m.close()
+    om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+    lg_cpu, hd_cpu = om.extend(prompt)
+    a, b = out[136], out[64]
+    assert O.rel_l2(a[1], hd_cpu) <= 1e-3 and O.rel_l2(a[0], lg_cpu) <= 1e-3, (O.rel_l2(a[1], hd_cpu), O.rel_l2(a[0], lg_cpu))
+    assert O.rel_l2(a[2], om.dn_s[0]) <= 1e-3 and O.rel_l2(a[3], om.dn_s[2]) <= 1e-3
+    kf = lambda x: x.view(np.float16).astype(np.float32)
+    assert O.rel_l2(kf(a[4][0]), kf(om.kc[3][:150])) <= 2e-3 and O.rel_l2(kf(a[4][1]), kf(om.vc[3][:150])) <= 2e-3
+    assert O.rel_l2(a[1], b[1]) <= 1e-4 and O.rel_l2(a[0], b[0]) <= 1e-4 and O.rel_l2(a[2], b[2]) <= 1e-4
+    assert int(np.argmax(a[0])) == int(np.argmax(lg_cpu))
+    print("136-row pass vs CPU: hidden %.2e logits %.2e; vs 64-row passes: logits %.2e; next tokens %s / %s" %
+          (O.rel_l2(a[1], hd_cpu), O.rel_l2(a[0], lg_cpu), O.rel_l2(a[0], b[0]), a[5], b[5]))
+
+
 def test_extend_rows_is_every_rows_logits(rig):
     m, cfg, tensors = rig
     rng = np.random.default_rng(12)
@@ -374,7 +408,9 @@ def test_checkpoint_restore_is_the_shorter_sequence(rig):
 
 def test_chunk_size_does_not_matter_over_4096_tokens():
     """BASELINE's prefill shape: 4096 tokens through a period of three DeltaNet layers and one
-    attention layer at the full widths, in chunks of 64, of 16, and (the first 192) token by token.
+    attention layer at the full widths, in chunks of 2048 (the blocks in groups of 64 rows layer by
+    layer, the experts over all rows of the pass grouped by expert on the matrix cores), of 64, of 16,
+    and (the first 192) token by token.
     Every chunk size runs other kernels (matrix cores from 3 or 5 rows, operands staged once from
     17, rows walked in groups of eight, pairs of attention rows) over the same arithmetic, so the
     carried state and the last row must agree to rounding."""
@@ -382,7 +418,7 @@ def test_chunk_size_does_not_matter_over_4096_tokens():
     rng = np.random.default_rng(4096)
     prompt = rng.integers(0, 8192, size=4096).astype(np.int32)
     out = {}
-    for rows in (64, 16):
+    for rows in (2048, 64, 16):
         m = LA.LLM(LA.Config(max_tokens=rows, **cfg))
         m.init_synthetic(99)
         m.stage()
@@ -397,6 +433,11 @@ def test_chunk_size_does_not_matter_over_4096_tokens():
                 m.extend(np.array([t], np.int32), want_logits=False)
             short1 = (m.dn_state(1), m.kv(3, 192))
         m.close()
+    a, b = out[64], out[2048]
+    assert O.rel_l2(a[1], b[1]) <= 1e-3 and O.rel_l2(a[0], b[0]) <= 1e-3, (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]))
+    assert O.rel_l2(a[2], b[2]) <= 1e-3 and O.rel_l2(a[3], b[3]) <= 1e-3
+    print("64 vs 2048 rows a chunk over 4096 tokens: hidden %.2e logits %.2e state %.2e" %
+          (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]), O.rel_l2(a[2], b[2])))
     a, b = out[64], out[16]
     assert O.rel_l2(a[1], b[1]) <= 1e-3 and O.rel_l2(a[0], b[0]) <= 1e-3, (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]))
     assert O.rel_l2(a[2], b[2]) <= 1e-3 and O.rel_l2(a[3], b[3]) <= 1e-3
