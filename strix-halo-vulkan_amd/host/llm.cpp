@@ -1039,6 +1039,10 @@ Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_
     // a pass of more rows than a block takes goes through the attention / DeltaNet blocks in
     // groups of kBlockRows, layer by layer, and through the experts whole
     block_rows_ = std::min(rows_max_, kBlockRows);
+    // where each group of such a pass stands: [slot][group] positions, written with the
+    // sequences' own before a prompt goes through and moved on by the long passes themselves
+    groups_ = (rows_max_ + block_rows_ - 1) / block_rows_;
+    if (groups_ > 1) grp_pos_ = static_cast<int32_t *>(dev.alloc_zero(static_cast<size_t>(o_.Slots) * groups_ * 4));
     moe_ = new MoEGPU(dev, m, rows_max_);
     dn_ = new DeltaNetGPU(dev, m, block_rows_, o_.Slots, pos_, planes, plane_);
     attn_ = new AttnGPU(dev, m, block_rows_, o_.NKV, o_.Slots, pos_);
@@ -1103,18 +1107,15 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
             auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, r, &p.labels) : dn_->Dispatches(l, x_, x_, r, &p.labels);
             p.ops.insert(p.ops.end(), sub.begin(), sub.end());
         } else {
-            // The sequence's position on the device moves on group by group, so that every group
-            // finds its cells, ring rows and rotary angles where a pass of its own would; after
-            // the last group it goes back for the next layer.
-            for (int r0 = 0; r0 < rows; r0 += block_rows_) {
+            // every group reads its own position word, so it finds its cells, ring rows and
+            // rotary angles where a pass of its own would
+            for (int r0 = 0, j = 0; r0 < rows; r0 += block_rows_, j++) {
                 PassRows g = r;
+                g.pos = grp_pos_ + static_cast<size_t>(slot) * groups_ + j;
                 g.seq_len = std::min(block_rows_, rows - r0);
                 float *xg = x_ + static_cast<size_t>(r0) * c_.NEmbd;
                 auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, xg, xg, g, &p.labels) : dn_->Dispatches(l, xg, xg, g, &p.labels);
                 p.ops.insert(p.ops.end(), sub.begin(), sub.end());
-                shv_advance_args step{pos_ + slot, 1, r0 + g.seq_len < rows ? g.seq_len : -r0};
-                p.ops.push_back(make_op(SHV_OP_ADVANCE, step));
-                p.labels.push_back("advance");
             }
         }
         auto ffn = moe_->Dispatches(l, x_, x_, rows, &p.labels);
@@ -1128,6 +1129,11 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
         am.logits_stride = c_.VocabSize;
     }
     shv_advance_args adv{pos_ + (slot < 0 ? 0 : slot), 1, rows};
+    if (rows > block_rows_) {
+        shv_advance_args ga{grp_pos_ + static_cast<size_t>(slot) * groups_, groups_, rows};
+        p.ops.push_back(make_op(SHV_OP_ADVANCE, ga));
+        p.labels.push_back("advance");
+    }
     switch (kind) {
         case kPrefill:
             p.ops.push_back(make_op(SHV_OP_ADVANCE, adv));
@@ -1180,6 +1186,12 @@ void Graph::put_pos() {
         v[o_.Slots + s] = seq_[s].plane;
     }
     dev_.upload(ctl_, v.data(), v.size() * 4);
+    if (groups_ > 1) {
+        std::vector<int32_t> g(static_cast<size_t>(o_.Slots) * groups_);
+        for (int s = 0; s < o_.Slots; s++)
+            for (int j = 0; j < groups_; j++) g[static_cast<size_t>(s) * groups_ + j] = seq_[s].past + j * block_rows_;
+        dev_.upload(grp_pos_, g.data(), g.size() * 4);
+    }
 }
 
 void Graph::Reset() {

@@ -442,7 +442,8 @@ private:
     const Model &m_;
     Config c_;
     GraphOpts o_;
-    int layers_, rows_max_, block_rows_ = 1, slot_ = 0;
+    int layers_, rows_max_, block_rows_ = 1, groups_ = 1, slot_ = 0;
+    int32_t *grp_pos_ = nullptr;
     std::vector<Seq> seq_;
     bool spec_ = false, spec_first_ = false, spec_armed_ = false;
     int spec_past_ = 0, spec_rows_ = 0;
