@@ -1,19 +1,21 @@
 // The experts of a pass of many rows, grouped by expert on the matrix cores (the prompt side of
 // MoETrace.Experts, llm/moe.go:289-409; the reference batches a chunk's tokens per expert in
 // llm_moe_gemv.comp's multi-row arm).  The per-(token, expert) GEMV reads and unpacks an expert's
-// weights once per token that chose it, this path once per 16 such tokens: it pays when tokens
+// weights once per token that chose it, this path once per 48 such tokens: it pays when tokens
 // outnumber experts (2048 rows choosing 10 of 512: 40 tokens an expert), not at 64 rows (1.9).
 //
-//   moe_group_kernel          per-expert lists of (token, slot) pairs from topk, tokens ascending
-//   moe_up_grouped_kernel     a block = (expert, half of its ffn rows): the listed tokens' xn rows
-//                             are gathered into LDS as matrix-core operands (two halves hi + lo,
-//                             as the projections do), each wave streams one gate tile and the
-//                             matching up tile of 16 rows, SwiGLU in registers, act[pair] out
-//   moe_down_grouped_kernel   a block = (expert, quarter of n_embd rows): act rows gathered the
-//                             same way, each wave two tiles, raw products to pairout[pair]
-//   moe_combine_kernel        out[t] = residual[t] + sum over slots of weights[t][s]*pairout[t][s],
+//   moe_group_kernel          per-expert lists of (token, slot) pairs from topk
+//   moe_up_grouped_kernel     a block = (expert, half of its ffn rows) and up to 48 of its tokens
+//                             at a time: their xn rows go through LDS as matrix-core operands
+//                             (two halves hi + lo, as the projections do) in slabs of 512 columns,
+//                             each wave streams two gate tiles of 16 rows and the matching up
+//                             tiles, forms a sub-block's weights once for all three token tiles,
+//                             SwiGLU in registers, act[pair] out
+//   moe_down_grouped_kernel   a block = (expert, quarter of n_embd rows): act rows staged the
+//                             same way (one slab), each wave four tiles, raw products to pairs[pair]
+//   moe_combine_kernel        out[t] = residual[t] + sum over slots of weights[t][s]*pairs[t][s],
 //                             slots in order
-// The shared expert is an expert every token lists: its blocks take 16 tokens each.
+// The shared expert is an expert every token lists: its blocks take 48 tokens each.
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
 
@@ -25,9 +27,13 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 16;
+constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int kTok = 16;          // tokens a block multiplies at a time: one matrix-core tile
+constexpr int kTT = 3;            // matrix-core tiles of 16 tokens a block multiplies per pass over the weights
+constexpr int kTok = 16 * kTT;    // tokens of such a pass
+constexpr int kTiles = 4;         // weight row tiles of 16 a wave owns
+constexpr int kSlab = 512;        // columns of the tokens' rows staged at a time
+constexpr int kSlabSubs = kSlab / 32;
 constexpr int kFrag = 64 * 16;    // one operand: a lane's eight halves
 constexpr int kMaxExperts = 1024;
 
@@ -64,12 +70,12 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
     }
 }
 
-// Rows src[i] (each K floats) of up to 16 listed rows into operand order: fragment (sub-block, part)
-// is 64 lanes x 16 bytes, lane = row + 16 * (k block of 8 columns), the eight columns in slot order
-// [0, 2, 1, 3, 4, 6, 5, 7]; sxs[sub][row] is the sub-block's sum of x.
-template <int K>
-__device__ __forceinline__ void gather_rows(const float *const *rows_s, int m, char *frags, float *sxs) {
-    constexpr int QPR = K / 4;                 // quads a row
+// Columns [col0, col0 + kSlab) of up to kTok listed rows (each a row of floats at rows_s[i]) into
+// operand order: the fragment of (sub-block, part hi / lo, token tile) is 64 lanes x 16 bytes,
+// lane = token in the tile + 16 * (k block of 8 columns), the eight columns in slot order
+// [0, 2, 1, 3, 4, 6, 5, 7]; sxs[sub][token] is the sub-block's sum of x.
+__device__ __forceinline__ void gather_slab(const float *const *rows_s, int m, int col0, char *frags, float *sxs) {
+    constexpr int QPR = kSlab / 4;             // quads a row's slab
     constexpr int RPI = kThreads / QPR;        // rows an iteration of the block covers
     const int tid = threadIdx.x;
     const int c = 4 * (tid % QPR);
@@ -78,7 +84,7 @@ __device__ __forceinline__ void gather_rows(const float *const *rows_s, int m, c
         const int i = i0 + tid / QPR;
         const bool on = i < m;
         float4 v = {0.f, 0.f, 0.f, 0.f};
-        if (on) v = *reinterpret_cast<const float4 *>(rows_s[i] + c);
+        if (on) v = *reinterpret_cast<const float4 *>(rows_s[i] + col0 + c);
         float sum = (v.x + v.y) + (v.z + v.w);
         sum += __shfl_xor(sum, 1, 64);
         sum += __shfl_xor(sum, 2, 64);
@@ -93,79 +99,128 @@ __device__ __forceinline__ void gather_rows(const float *const *rows_s, int m, c
                 h[j] = hi;
                 l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
             }
-            char *e = frags + static_cast<size_t>(sub * 2) * kFrag + (kb * 16 + i) * 16 + qh * 8;
+            char *e = frags + static_cast<size_t>((sub * 2) * kTT + (i >> 4)) * kFrag + (kb * 16 + (i & 15)) * 16 + qh * 8;
             *reinterpret_cast<half4_t *>(e) = h;
-            *reinterpret_cast<half4_t *>(e + kFrag) = l;
+            *reinterpret_cast<half4_t *>(e + kTT * kFrag) = l;
         }
     }
 }
 
-struct SbLoads {
-    uint4 hdr;
-    uint2 q[4];
-    __device__ __forceinline__ void load(const char *sb, int kb) {
-        hdr = *reinterpret_cast<const uint4 *>(sb);
+// A wave's place in its R weight rows' streams: the header of the super-block it is in, the next
+// super-block's header and the payload of the next 64-weight group, both on their way.
+template <int R>
+struct RowStream {
+    uint4 hdr[R], hdr_next[R];
+    uint2 q_next[R];
+    // group G = 4 * super-block + g, clamped to the last one so that the loads are unconditional
+    __device__ __forceinline__ void ask_group(const char *const (&rp)[R], int G, int G_last, int kb) {
+        const int Gc = G < G_last ? G : G_last;
 #pragma unroll
-        for (int g = 0; g < 4; g++) q[g] = *reinterpret_cast<const uint2 *>(sb + 16 + g * 32 + kb * 8);
+        for (int r = 0; r < R; r++)
+            q_next[r] = *reinterpret_cast<const uint2 *>(rp[r] + static_cast<size_t>(Gc >> 2) * SHV_Q4K_BYTES + 16 + (Gc & 3) * 32 + kb * 8);
+    }
+    __device__ __forceinline__ void ask_header(const char *const (&rp)[R], int sb, int sb_last) {
+        const int sc = sb < sb_last ? sb : sb_last;
+#pragma unroll
+        for (int r = 0; r < R; r++) hdr_next[r] = *reinterpret_cast<const uint4 *>(rp[r] + static_cast<size_t>(sc) * SHV_Q4K_BYTES);
     }
 };
 
-// y[r][j] += sum over the row's K columns of W[row of tile r][.] * x[token 4 kb + j][.] for R row
-// tiles whose lane rows start at rp[r]; the operands of the 16 tokens are in LDS.
-template <int K, int R>
-__device__ __forceinline__ void tiles_times_rows(const char *const (&rp)[R], const char *frags, const float *sxs, int lane, float4_t (&y)[R]) {
-    constexpr int SBS = K / SHV_Q4K_BLOCK;
+// The 64-weight groups [G0, G0 + NG) of R row tiles (lane rows at rp[r]) against the staged slab,
+// whose first sub-block is the first of group G0:
+// y[r][tt][j] += sum over those columns of W[row of tile r][.] * x[token 16 tt + 4 kb + j][.].
+// A sub-block's eight weights per lane are formed once and multiplied with every token tile:
+// forming them is most of the vector work of such a kernel.
+template <int NG, int R>
+__device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], RowStream<R> &st, int G0, int G_last, const char *frags,
+                                                 const float *sxs, int lane, int n_tt, float4_t (&y)[R][kTT]) {
     const int kb = lane >> 4;
     const NibbleConsts nc = nibble_consts();
-    SbLoads ld[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) ld[r].load(rp[r], kb);
 #pragma unroll 1
-    for (int sb = 0; sb < SBS; sb++) {
-        SbLoads cur[R];
+    for (int gi = 0; gi < NG; gi++) {
+        const int G = G0 + gi, g = G & 3;
+        uint2 q[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) q[r] = st.q_next[r];
+        st.ask_group(rp, G + 1, G_last, kb);
+        if (g == 0) st.ask_header(rp, (G >> 2) + 1, G_last >> 2);
+        uint32_t sc[R], mn[R];
+        float dd[R], dmin[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            cur[r] = ld[r];
-            // the last super-block asks for itself again, so that the loads are unconditional
-            ld[r].load(rp[r] + static_cast<size_t>(sb + 1 < SBS ? sb + 1 : sb) * SHV_Q4K_BYTES, kb);
+            q4k_group_scale_min(st.hdr[r], g, sc[r], mn[r]);
+            dd[r] = f16_bits_to_f32(st.hdr[r].x);
+            dmin[r] = f16_bits_to_f32(st.hdr[r].x >> 16);
         }
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            uint32_t sc[R], mn[R];
+        for (int hi = 0; hi < 2; hi++) {
+            const int sub = gi * 2 + hi;
+            half8_t b[R];
+            float ds[R], e[R];
 #pragma unroll
-            for (int r = 0; r < R; r++) q4k_group_scale_min(cur[r].hdr, g, sc[r], mn[r]);
+            for (int r = 0; r < R; r++) {
+                const uint32_t q0 = q[r].x, q1 = q[r].y;
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                u32x4 v;
+                if (hi == 0) {
+                    v.x = ((q0 << 4) & nc.mask) | nc.one; v.y = ((q0 >> 4) & nc.mask) | nc.one;
+                    v.z = ((q1 << 4) & nc.mask) | nc.one; v.w = ((q1 >> 4) & nc.mask) | nc.one;
+                } else {
+                    v.x = (q0 & nc.mask) | nc.one; v.y = ((q0 >> 8) & nc.mask) | nc.one;
+                    v.z = (q1 & nc.mask) | nc.one; v.w = ((q1 >> 8) & nc.mask) | nc.one;
+                }
+                b[r] = __builtin_bit_cast(half8_t, v);
+                ds[r] = dd[r] * static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu);
+                e[r] = fmaf(64.f, ds[r], dmin[r] * static_cast<float>(hi ? mn[r] >> 8 : mn[r] & 0xFFu));
+            }
 #pragma unroll
-            for (int hi = 0; hi < 2; hi++) {
-                const int sub = sb * 8 + g * 2 + hi;
-                const char *f = frags + static_cast<size_t>(sub * 2) * kFrag + lane * 16;
+            for (int tt = 0; tt < kTT; tt++) {
+                if (tt >= n_tt) break;
+                const char *f = frags + static_cast<size_t>((sub * 2) * kTT + tt) * kFrag + lane * 16;
                 const half8_t xh = *reinterpret_cast<const half8_t *>(f);
-                const half8_t xl = *reinterpret_cast<const half8_t *>(f + kFrag);
-                const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * kTok + 4 * kb);
+                const half8_t xl = *reinterpret_cast<const half8_t *>(f + kTT * kFrag);
+                const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * kTok + 16 * tt + 4 * kb);
                 const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
 #pragma unroll
                 for (int r = 0; r < R; r++) {
-                    const uint32_t q0 = cur[r].q[g].x, q1 = cur[r].q[g].y;
-                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                    u32x4 v;
-                    if (hi == 0) {
-                        v.x = ((q0 << 4) & nc.mask) | nc.one; v.y = ((q0 >> 4) & nc.mask) | nc.one;
-                        v.z = ((q1 << 4) & nc.mask) | nc.one; v.w = ((q1 >> 4) & nc.mask) | nc.one;
-                    } else {
-                        v.x = (q0 & nc.mask) | nc.one; v.y = ((q0 >> 8) & nc.mask) | nc.one;
-                        v.z = (q1 & nc.mask) | nc.one; v.w = ((q1 >> 8) & nc.mask) | nc.one;
-                    }
-                    const half8_t b = __builtin_bit_cast(half8_t, v);
-                    const float dd = f16_bits_to_f32(cur[r].hdr.x), dmin = f16_bits_to_f32(cur[r].hdr.x >> 16);
-                    const float ds = dd * static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu);
-                    const float e = fmaf(64.f, ds, dmin * static_cast<float>(hi ? mn[r] >> 8 : mn[r] & 0xFFu));
                     float4_t acc = {0.f, 0.f, 0.f, 0.f};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b, acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc, 0, 0, 0);
 #pragma unroll
-                    for (int j = 0; j < 4; j++) y[r][j] = fmaf(-e, sxv[j], fmaf(ds, acc[j], y[r][j]));
+                    for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(-e[r], sxv[j], fmaf(ds[r], acc[j], y[r][tt][j]));
                 }
             }
         }
+        if (g == 3) {
+#pragma unroll
+            for (int r = 0; r < R; r++) st.hdr[r] = st.hdr_next[r];
+        }
+    }
+}
+
+// All K columns of up to kTok listed rows against a wave's kTiles row tiles: the rows go through
+// LDS a slab at a time, the weights of the next super-block are on their way while a slab is staged.
+template <int K>
+__device__ __forceinline__ void rows_times_tiles(const char *const (&rp)[kTiles], const float *const *rows_s, int m, char *frags, float *sxs,
+                                                 int lane, float4_t (&y)[kTiles][kTT]) {
+    constexpr int GROUPS = K / 64, NG = kSlab / 64;
+    static_assert(K % kSlab == 0, "whole slabs");
+    const int n_tt = (m + 15) >> 4;
+#pragma unroll
+    for (int r = 0; r < kTiles; r++)
+#pragma unroll
+        for (int tt = 0; tt < kTT; tt++) y[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    RowStream<kTiles> st;
+    st.ask_header(rp, 0, GROUPS / 4 - 1);
+#pragma unroll
+    for (int r = 0; r < kTiles; r++) st.hdr[r] = st.hdr_next[r];
+    st.ask_group(rp, 0, GROUPS - 1, lane >> 4);
+#pragma unroll 1
+    for (int sl = 0; sl < K / kSlab; sl++) {
+        __syncthreads();   // the list is written / the slab before this one has been multiplied
+        gather_slab(rows_s, m, sl * kSlab, frags, sxs);
+        __syncthreads();
+        slab_times_tiles<NG, kTiles>(rp, st, sl * NG, GROUPS - 1, frags, sxs, lane, n_tt, y);
     }
 }
 
@@ -195,91 +250,103 @@ __device__ __forceinline__ Unit unit_of(int b, int parts, int n_expert, int n_to
     return u;
 }
 
-// grid: n_expert * 2 + 2 * ceil(n_tok / 16) blocks of 16 waves; K = n_embd; ffn = 512: a half is
-// 256 rows = 16 tiles, wave w takes gate tile w and up tile w.
+struct Staging {
+    char *frags;
+    float *sxs;
+    const float **rows_s;
+    int32_t *pair_s;
+    __device__ __forceinline__ explicit Staging(char *smem) {
+        frags = smem;
+        sxs = reinterpret_cast<float *>(smem + static_cast<size_t>(kSlabSubs) * 2 * kTT * kFrag);
+        rows_s = reinterpret_cast<const float **>(sxs + kSlabSubs * kTok);
+        pair_s = reinterpret_cast<int32_t *>(rows_s + kTok);
+    }
+};
+constexpr size_t kGroupedLds = static_cast<size_t>(kSlabSubs) * 2 * kTT * kFrag + static_cast<size_t>(kSlabSubs) * kTok * 4 + kTok * sizeof(float *) + kTok * 4;
+
+// grid: n_expert * parts + parts * ceil(n_tok / 48) blocks of 8 waves, parts = ffn / 256; K = n_embd.
+// A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tiles 2w and
+// 2w + 1 and the up tiles of the same rows, so SwiGLU stays in registers.
 template <int K>
 __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_args a) {
-    const int32_t *group = a.group;
     extern __shared__ __align__(16) char smem[];
-    constexpr int SUBS = K / 32;
-    char *frags = smem;
-    float *sxs = reinterpret_cast<float *>(smem + static_cast<size_t>(SUBS) * 2 * kFrag);
-    const float **rows_s = reinterpret_cast<const float **>(sxs + SUBS * kTok);
-    int32_t *pair_s = reinterpret_cast<int32_t *>(rows_s + kTok);
+    const Staging st(smem);
+    const int32_t *group = a.group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int parts = a.ffn / 256;
     const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row = u.part * 256 + wave * 16 + n;   // this lane's row of the expert, gate and up alike
+    const int row = u.part * 256 + wave * 32 + n;   // this lane's row in the wave's first tile, gate and up alike
     const size_t wrow = static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.ffn + row;
-    const char *rp[2] = {static_cast<const char *>(u.expert < 0 ? a.gate_sh : a.gate_exps) + wrow * row_bytes,
-                         static_cast<const char *>(u.expert < 0 ? a.up_sh : a.up_exps) + wrow * row_bytes};
+    const char *gp = static_cast<const char *>(u.expert < 0 ? a.gate_sh : a.gate_exps) + wrow * row_bytes;
+    const char *up = static_cast<const char *>(u.expert < 0 ? a.up_sh : a.up_exps) + wrow * row_bytes;
+    const char *rp[kTiles] = {gp, gp + 16 * row_bytes, up, up + 16 * row_bytes};
     for (int t0 = 0; t0 < u.count; t0 += kTok) {
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {
             const int pair = u.expert < 0 ? (u.first + t0 + tid) * (a.n_used + 1) + a.n_used : group[a.n_expert + 1 + u.first + t0 + tid];
-            pair_s[tid] = pair;
-            rows_s[tid] = a.xn + static_cast<size_t>(pair / (a.n_used + 1)) * K;
+            st.pair_s[tid] = pair;
+            st.rows_s[tid] = a.xn + static_cast<size_t>(pair / (a.n_used + 1)) * K;
         }
-        __syncthreads();
-        gather_rows<K>(rows_s, m, frags, sxs);
-        __syncthreads();
-        float4_t y[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-        tiles_times_rows<K, 2>(rp, frags, sxs, lane, y);
+        float4_t y[kTiles][kTT];
+        rows_times_tiles<K>(rp, st.rows_s, m, st.frags, st.sxs, lane, y);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int i = 4 * kb + j;
-            if (i < m) {
-                const float gv = y[0][j];
-                a.act[static_cast<size_t>(pair_s[i]) * a.ffn + row] = gv * sigmoid_exact(gv) * y[1][j];
+        for (int tt = 0; tt < kTT; tt++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int i = 16 * tt + 4 * kb + j;
+                if (i < m) {
+                    float *dst = a.act + static_cast<size_t>(st.pair_s[i]) * a.ffn + row;
+#pragma unroll
+                    for (int q = 0; q < 2; q++) {
+                        const float gv = y[q][tt][j];
+                        dst[16 * q] = gv * sigmoid_exact(gv) * y[2 + q][tt][j];
+                    }
+                }
             }
-        }
-        __syncthreads();
+        __syncthreads();   // the list is read to the end before the next one replaces it
     }
 }
 
-// grid: n_expert * parts + parts * ceil(n_tok / 16) blocks, parts = n_embd / 512: a part is 512
-// output rows = 32 tiles, wave w takes tiles 2w and 2w + 1.  K = ffn.
+// grid: n_expert * parts + parts * ceil(n_tok / 48) blocks, parts = n_embd / 512: a part is 512
+// output rows = 32 tiles, wave w takes tiles 4w .. 4w + 3.  K = ffn.
 template <int K>
 __global__ __launch_bounds__(kThreads) void moe_down_grouped_kernel(shv_moe_down_args a) {
+    extern __shared__ __align__(16) char smem[];
+    const Staging st(smem);
     const int32_t *group = a.group;
     float *pairout = a.pairs;
-    extern __shared__ __align__(16) char smem[];
-    constexpr int SUBS = K / 32;
-    char *frags = smem;
-    float *sxs = reinterpret_cast<float *>(smem + static_cast<size_t>(SUBS) * 2 * kFrag);
-    const float **rows_s = reinterpret_cast<const float **>(sxs + SUBS * kTok);
-    int32_t *pair_s = reinterpret_cast<int32_t *>(rows_s + kTok);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int parts = a.n_embd / 512;
     const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row0 = u.part * 512 + wave * 32 + n;
+    const int row0 = u.part * 512 + wave * 64 + n;
     const char *base = static_cast<const char *>(u.expert < 0 ? a.down_sh : a.down_exps) +
                        (static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.n_embd + row0) * row_bytes;
-    const char *rp[2] = {base, base + 16 * row_bytes};
+    const char *rp[kTiles] = {base, base + 16 * row_bytes, base + 32 * row_bytes, base + 48 * row_bytes};
     for (int t0 = 0; t0 < u.count; t0 += kTok) {
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {
             const int pair = u.expert < 0 ? (u.first + t0 + tid) * (a.n_used + 1) + a.n_used : group[a.n_expert + 1 + u.first + t0 + tid];
-            pair_s[tid] = pair;
-            rows_s[tid] = a.act + static_cast<size_t>(pair) * K;
+            st.pair_s[tid] = pair;
+            st.rows_s[tid] = a.act + static_cast<size_t>(pair) * K;
         }
-        __syncthreads();
-        gather_rows<K>(rows_s, m, frags, sxs);
-        __syncthreads();
-        float4_t y[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-        tiles_times_rows<K, 2>(rp, frags, sxs, lane, y);
+        float4_t y[kTiles][kTT];
+        rows_times_tiles<K>(rp, st.rows_s, m, st.frags, st.sxs, lane, y);
 #pragma unroll
-        for (int r = 0; r < 2; r++)
+        for (int tt = 0; tt < kTT; tt++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int i = 4 * kb + j;
-                if (i < m) pairout[static_cast<size_t>(pair_s[i]) * a.n_embd + row0 + r * 16] = y[r][j];
+                const int i = 16 * tt + 4 * kb + j;
+                if (i < m) {
+                    float *dst = pairout + static_cast<size_t>(st.pair_s[i]) * a.n_embd + row0;
+#pragma unroll
+                    for (int r = 0; r < kTiles; r++) dst[16 * r] = y[r][tt][j];
+                }
             }
         __syncthreads();
     }
@@ -299,11 +366,6 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(shv_moe_down_args a) {
         v.x = fmaf(ws, p.x, v.x); v.y = fmaf(ws, p.y, v.y); v.z = fmaf(ws, p.z, v.z); v.w = fmaf(ws, p.w, v.w);
     }
     *reinterpret_cast<float4 *>(a.out + static_cast<size_t>(t) * a.out_stride + c) = v;
-}
-
-template <int K>
-constexpr size_t grouped_lds() {
-    return static_cast<size_t>(K / 32) * 2 * kFrag + static_cast<size_t>(K / 32) * kTok * 4 + kTok * sizeof(float *) + kTok * 4;
 }
 
 template <typename Kern>
@@ -333,7 +395,7 @@ bool shv_moe_down_grouped_covers(const shv_ctx *ctx, const shv_moe_down_args &a)
 // Lists, then the grouped gate/up products.
 int shv_launch_moe_up_grouped(shv_ctx *ctx, const shv_moe_up_args &a) {
     SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, a.group);
-    constexpr size_t lds = grouped_lds<2048>();
+    constexpr size_t lds = kGroupedLds;
     static const int raised = raise_lds(&moe_up_grouped_kernel<2048>, lds);
     if (raised != SHV_OK) return raised;
     const int parts = a.ffn / 256, tiles = (a.n_tok + kTok - 1) / kTok;
@@ -349,7 +411,7 @@ int shv_launch_moe_down_grouped(shv_ctx *ctx, const shv_moe_down_args &a) {
                     (!a.residual || (a.res_stride % 4 == 0 && shv_aligned16(a.residual))),
                 "moe_down: the grouped path moves 16 bytes at a time");
     SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
-    constexpr size_t lds = grouped_lds<512>();
+    constexpr size_t lds = kGroupedLds;
     static const int raised = raise_lds(&moe_down_grouped_kernel<512>, lds);
     if (raised != SHV_OK) return raised;
     const int parts = a.n_embd / 512, tiles = (a.n_tok + kTok - 1) / kTok;
