@@ -200,33 +200,39 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
     }
 }
 
-// grid: (ceil((n_expert+1)/4), ceil(n_tok/kRouterTokens)) blocks of 4 waves, one float32 router
-// row per wave, kRouterTokens tokens per block.  Tokens go through in groups of kRouterGroup: one
-// set of block-wide waits per group, not per token.
+// grid: (ceil((n_expert+1)/(4 RW)), ceil(n_tok/tpb)) blocks of 4 waves, RW float32 router rows per
+// wave, tpb tokens per block.  Tokens go through in groups of kRouterGroup: one set of block-wide
+// waits per group, not per token.  A pass of few tokens spreads the router over many small
+// blocks (RW = 1, 4 tokens a block); a prompt pass, where every block reads every token's row and
+// every token's block reads the router, takes RW = 4 and 8 to 32 tokens a block.
 constexpr int kRouterGroup = 4;
 constexpr int kRouterTokens = 4;
-template <int H>
-__global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args a) {
+constexpr int kRouterTokensMany = 32;
+template <int H, int RW>
+__global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args a, int tpb) {
     __shared__ __align__(16) float xs[kRouterGroup][H];
     __shared__ float red[kRouterGroup][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row = blockIdx.x * 4 + wave;  // n_expert = the shared-gate row
-    const bool has_row = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
-    // the wave's router row is in flight while the first tokens are being normalised, and stays
+    const int row0 = (blockIdx.x * 4 + wave) * RW;  // n_expert = the shared-gate row
+    // the wave's router rows are in flight while the first tokens are being normalised, and stay
     // in registers for every token
-    float4 wrow[H / 256];
-    {
+    float4 wrow[RW][H / 256];
+    bool has_row[RW];
+#pragma unroll
+    for (int j = 0; j < RW; j++) {
+        const int row = row0 + j;
+        has_row[j] = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
         const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
 #pragma unroll
         for (int i = 0; i < H / 256; i++)
-            wrow[i] = has_row ? *reinterpret_cast<const float4 *>(w + (i * 64 + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            wrow[j][i] = has_row[j] ? *reinterpret_cast<const float4 *>(w + (i * 64 + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     float gm[H / kBlock];  // gamma is asked for before the block-wide sums, not after them
 #pragma unroll
     for (int i = 0; i < H / kBlock; i++) gm[i] = a.gamma ? a.gamma[tid + i * kBlock] : 1.f;
 
-    const int t_first = blockIdx.y * kRouterTokens;
-    const int t_end = t_first + kRouterTokens < a.n_tok ? t_first + kRouterTokens : a.n_tok;
+    const int t_first = blockIdx.y * tpb;
+    const int t_end = t_first + tpb < a.n_tok ? t_first + tpb : a.n_tok;
     // a group's rows are asked for while the group before it is being multiplied
     float v[kRouterGroup][H / kBlock];
     auto fetch = [&](int t0) {
@@ -269,23 +275,29 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
         }
         __syncthreads();
         if (t0 + kRouterGroup < t_end) fetch(t0 + kRouterGroup);
-        if (has_row) {
 #pragma unroll
-            for (int g = 0; g < kRouterGroup; g++) {
-                if (g >= ng) break;
-                float acc = 0.f;
+        for (int g = 0; g < kRouterGroup; g++) {
+            if (g >= ng) break;
+            float acc[RW];
 #pragma unroll
-                for (int i = 0; i < H / 256; i++) {
-                    const int c = (i * 64 + lane) * 4;
-                    const float4 wv = wrow[i];
-                    const float4 xv = *reinterpret_cast<const float4 *>(&xs[g][c]);
-                    acc = fmaf(wv.x, xv.x, acc);
-                    acc = fmaf(wv.y, xv.y, acc);
-                    acc = fmaf(wv.z, xv.z, acc);
-                    acc = fmaf(wv.w, xv.w, acc);
+            for (int j = 0; j < RW; j++) acc[j] = 0.f;
+#pragma unroll
+            for (int i = 0; i < H / 256; i++) {
+                const int c = (i * 64 + lane) * 4;
+                const float4 xv = *reinterpret_cast<const float4 *>(&xs[g][c]);
+#pragma unroll
+                for (int j = 0; j < RW; j++) {
+                    const float4 wv = wrow[j][i];
+                    acc[j] = fmaf(wv.x, xv.x, acc[j]);
+                    acc[j] = fmaf(wv.y, xv.y, acc[j]);
+                    acc[j] = fmaf(wv.z, xv.z, acc[j]);
+                    acc[j] = fmaf(wv.w, xv.w, acc[j]);
                 }
-                acc = wave_sum_all(acc);
-                if (lane == 0) a.logits[static_cast<size_t>(t0 + g) * (a.n_expert + 1) + row] = acc;
+            }
+#pragma unroll
+            for (int j = 0; j < RW; j++) {
+                const float sum = wave_sum_all(acc[j]);
+                if (lane == 0 && has_row[j]) a.logits[static_cast<size_t>(t0 + g) * (a.n_expert + 1) + row0 + j] = sum;
             }
         }
         if (t0 + kRouterGroup < t_end) __syncthreads();
@@ -638,12 +650,24 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed && a.n_used <= a.n_expert, "moe_router: n_used %d of %d (at most %d)", a.n_used, a.n_expert, kMaxUsed);
     SHV_REQUIRE(a.h_stride >= a.n_embd, "moe_router: h_stride %d < n_embd %d", a.h_stride, a.n_embd);
     SHV_REQUIRE(shv_aligned16(a.router) && shv_aligned16(a.shared_gate), "moe_router: router and shared_gate must be 16-byte aligned");
-    const dim3 blocks((a.n_expert + 1 + 3) / 4, (a.n_tok + kRouterTokens - 1) / kRouterTokens);
+    // four rows a wave only where that still leaves a few hundred blocks
+    const bool many = a.n_tok >= 128;
+    const int rw = many ? 4 : 1, tpb = a.n_tok >= 512 ? kRouterTokensMany : many ? 8 : kRouterTokens;
+    const dim3 blocks((a.n_expert + 1 + 4 * rw - 1) / (4 * rw), (a.n_tok + tpb - 1) / tpb);
     SHV_REQUIRE(blocks.y <= 65535, "moe_router: n_tok %d", a.n_tok);
     switch (a.n_embd) {
-        case 2048: SHV_LAUNCH(ctx, moe_router_kernel<2048>, blocks, dim3(kBlock), 0, a); break;
-        case 1024: SHV_LAUNCH(ctx, moe_router_kernel<1024>, blocks, dim3(kBlock), 0, a); break;
-        case 512: SHV_LAUNCH(ctx, moe_router_kernel<512>, blocks, dim3(kBlock), 0, a); break;
+        case 2048:
+            if (many) SHV_LAUNCH(ctx, (moe_router_kernel<2048, 4>), blocks, dim3(kBlock), 0, a, tpb);
+            else SHV_LAUNCH(ctx, (moe_router_kernel<2048, 1>), blocks, dim3(kBlock), 0, a, tpb);
+            break;
+        case 1024:
+            if (many) SHV_LAUNCH(ctx, (moe_router_kernel<1024, 4>), blocks, dim3(kBlock), 0, a, tpb);
+            else SHV_LAUNCH(ctx, (moe_router_kernel<1024, 1>), blocks, dim3(kBlock), 0, a, tpb);
+            break;
+        case 512:
+            if (many) SHV_LAUNCH(ctx, (moe_router_kernel<512, 4>), blocks, dim3(kBlock), 0, a, tpb);
+            else SHV_LAUNCH(ctx, (moe_router_kernel<512, 1>), blocks, dim3(kBlock), 0, a, tpb);
+            break;
         default: return shv_set_error(SHV_E_INVALID, "moe_router: n_embd = %d; built for 512, 1024 and 2048", a.n_embd);
     }
     // the selection needs every logit of the token, i.e. the whole grid above: a second, tiny
