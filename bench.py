@@ -290,8 +290,9 @@ def main():
     ap.add_argument("--mtp-rounds", type=int, default=64)
     ap.add_argument("--batch-slots", type=int, default=8,
                     help="sequences of the batched-decode leg (one token each per pass); 0 skips it")
-    ap.add_argument("--prefill-rows", type=int, default=64,
-                    help="prompt rows per pass; 1 (with --no-mtp) sends the prompt through the one-row decode "
+    ap.add_argument("--prefill-rows", type=int, default=2048,
+                    help="prompt rows per pass (up to 4096; the default sends the 2048-token prompt through as one "
+                         "chunk); 1 (with --no-mtp) sends the prompt through the one-row decode "
                          "step itself, so that a kernel trace of the run holds decode launches only")
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
@@ -376,9 +377,13 @@ def main():
         rec["prefill_chunk"] = {
             "rows": rows, "us": round(chunk_us, 1), "tok_s": round(rows / chunk_us * 1e6, 1),
             "op_us": {k: round(v / 1e3, 1) for k, v in sorted(st.items(), key=lambda kv: -kv[1]) if k != "total"},
-            # every row reads its own experts: rows x (10 routed + shared) x rows of the banks
-            "moe_up_GBps": round(rows * per_tok_up * cfg.n_layer / (st["moe.up"] / 1e9) / 1e9, 1),
-            "moe_down_GBps": round(rows * per_tok_down * cfg.n_layer / (st["moe.down"] / 1e9) / 1e9, 1)}
+            # multiply-adds of the rows' (10 routed + shared) experts, two flops each
+            "moe_up_TFLOPs": round(rows * per_tok_up / 0.5625 * 2 * cfg.n_layer / (st["moe.up"] / 1e9) / 1e12, 1),
+            "moe_down_TFLOPs": round(rows * per_tok_down / 0.5625 * 2 * cfg.n_layer / (st["moe.down"] / 1e9) / 1e12, 1)}
+        if rows < 128:
+            # below 128 rows every row reads its own experts: rows x (10 routed + shared) x rows of the banks
+            rec["prefill_chunk"]["moe_up_GBps"] = round(rows * per_tok_up * cfg.n_layer / (st["moe.up"] / 1e9) / 1e9, 1)
+            rec["prefill_chunk"]["moe_down_GBps"] = round(rows * per_tok_down * cfg.n_layer / (st["moe.down"] / 1e9) / 1e9, 1)
     if a.pmc_copy:
         import ctypes as C
         H = A.load()
