@@ -11,8 +11,9 @@ resident in HBM before it starts.  Prints ONE JSON line.
 
 Beside the headline it reports
   roofline      the dominant kernel of the step (the expert-gathered gate/up GEMV, 48 launches a
-                token): algorithmic bytes per launch over the kernel's own measured duration
-                (timestamps on the kernel's dispatch, taken live), against 8 TB/s
+                token, which on one-row passes also makes the token's top-10 selection first):
+                algorithmic bytes per launch over the kernel's own measured duration (timestamps on
+                the kernel's dispatch, taken live), against 8 TB/s
   cpu_baseline  the CPU restatement of the reference's Go path (oracle/), timed on this host on a
                 bounded sample of the same model: layers 0..3 (one DeltaNet x3 + attention period)
                 plus the head, a few decode tokens, scaled by 12 periods to a 48-layer token
@@ -343,7 +344,11 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "moe_up_hbm_traffic.json")
     if os.path.exists(tpath) and (cfg.n_embd, cfg.n_expert_used, cfg.ffn_expert) == (2048, 10, 512):
         traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
-    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048, 1> (expert-gathered Q4_K gate/up GEMV + SwiGLU)",
+    # one-row passes route in the expert kernel itself unless LLM_MOE_ROUTE=kernel keeps the selection a launch of its own
+    fused = os.environ.get("LLM_MOE_ROUTE", "rows") in ("rows", "fused")
+    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048, 1> (%sexpert-gathered Q4_K gate/up GEMV + SwiGLU)" %
+                      ("softmax and top-10 of the token's 512 router logits, then the " if fused else ""),
+            "routing": "in this launch" if fused else "a launch of its own",
             "achieved": round(up_bytes / (up_ns / 1e9) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": round(up_bytes / (up_ns / 1e9) / HBM_PEAK, 4), "traffic": traffic,
             "bytes_per_launch": up_bytes, "avg_launch_us": round(up_ns / 1e3, 3), "launches_per_step": cfg.n_layer}

@@ -428,6 +428,124 @@ __global__ __launch_bounds__(kRouteBlock) void moe_route_block_kernel(shv_moe_ro
     }
 }
 
+// The same selection by a block of 256 threads, two experts a thread (tid and tid + 256), for a
+// kernel that routes its own token before it can ask for its expert's rows: every block of the
+// launch repeats it, side by side.  The probabilities are formed exactly as
+// moe_route_block_kernel forms them (the same partial sums over the same 64 experts, added in
+// the same order).  sel_e [kMaxUsed] / sel_w [kMaxUsed + 1] receive experts, weights and the
+// shared expert's gate; probs is the one-wave road's scratch.  Ends with a block-wide wait.
+__device__ __forceinline__ void route_block256(const float *lg, int n_expert, int n_used, bool shared_gate, int32_t *sel_e, float *sel_w, float *probs) {
+    __shared__ float s_max[4], s_sum[8];
+    __shared__ uint32_t s_gm[16];
+    __shared__ uint32_t s_thr;
+    __shared__ int s_cnt[8];
+    __shared__ uint32_t cand_p[64];
+    __shared__ int32_t cand_e[64];
+    __shared__ int32_t r_e[kMaxUsed];
+    __shared__ float r_w[kMaxUsed];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int e0 = tid, e1 = tid + 256;
+    const bool has0 = e0 < n_expert, has1 = e1 < n_expert;
+    const float l0 = has0 ? lg[e0] : -INFINITY, l1 = has1 ? lg[e1] : -INFINITY;
+    const float lsh = (tid == 255 && shared_gate) ? lg[n_expert] : 0.f;
+    float mx = wave_max_all(fmaxf(l0, l1));
+    if (lane == 0) s_max[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    const float ex0 = has0 ? expf(l0 - mx) : 0.f, ex1 = has1 ? expf(l1 - mx) : 0.f;
+    const float ws0 = wave_sum_all(ex0), ws1 = wave_sum_all(ex1);
+    if (lane == 0) {
+        s_sum[wave] = ws0;
+        s_sum[4 + wave] = ws1;
+    }
+    if (tid == 0) s_thr = 0u;
+    __syncthreads();
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) sum += s_sum[w];
+    const float inv = 1.f / sum;
+    const uint32_t kh0 = has0 ? __float_as_uint(ex0 * inv) : 0u, kh1 = has1 ? __float_as_uint(ex1 * inv) : 0u;
+    // 16 groups of 16 threads: n_used of them hold a key at or above the n_used-th largest group maximum
+    uint32_t gm = kh0 > kh1 ? kh0 : kh1;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(gm), off, 64));
+        gm = o > gm ? o : gm;
+    }
+    if ((lane & 15) == 0) s_gm[tid >> 4] = gm;
+    __syncthreads();
+    if (tid < 16) {
+        const uint32_t mine = s_gm[tid];
+        int rank = 0;
+#pragma unroll
+        for (int j = 0; j < 16; j++) rank += (s_gm[j] > mine || (s_gm[j] == mine && j < tid)) ? 1 : 0;
+        if (rank == n_used - 1) s_thr = mine;
+    }
+    __syncthreads();
+    const uint32_t thr = s_thr;
+    const bool p0 = has0 && kh0 >= thr, p1 = has1 && kh1 >= thr;
+    const unsigned long long m0 = __ballot(p0), m1 = __ballot(p1);
+    if (lane == 0) {
+        s_cnt[wave] = __popcll(m0);
+        s_cnt[4 + wave] = __popcll(m1);
+    }
+    __syncthreads();
+    int before0 = 0, before1 = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        before0 += w < wave ? s_cnt[w] : 0;
+        before1 += w < 4 + wave ? s_cnt[w] : 0;
+        total += s_cnt[w];
+    }
+    if (total > 64 || n_expert < 64 || n_used > 16) {
+        // uniform over the block: many equal probabilities, or a shape the threshold does not cover
+        if (wave == 0) {
+            route_token<8, false>(lg, n_expert, n_used, sel_e, sel_w, probs);
+            if (lane == 0) sel_w[n_used] = shared_gate ? sigmoid_exact(lg[n_expert]) : 0.f;
+        }
+        __syncthreads();
+        return;
+    }
+    if (p0) {
+        const int pos = before0 + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m0 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m0), 0u)));
+        cand_p[pos] = kh0;
+        cand_e[pos] = e0;
+    }
+    if (p1) {
+        const int pos = before1 + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m1 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m1), 0u)));
+        cand_p[pos] = kh1;
+        cand_e[pos] = e1;
+    }
+    if (tid == 255) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh) : 0.f;
+    __syncthreads();
+    if (wave == 0) {
+        const uint32_t my_p = lane < total ? cand_p[lane] : 0u;
+        const int my_e = lane < total ? cand_e[lane] : 0x7FFFFFFF;
+        int rank = 0;
+        for (int j = 0; j < total; j++) {
+            const uint32_t pj = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_p), j));
+            const int ej = __builtin_amdgcn_readlane(my_e, j);
+            const int bef = __popcll(__ballot(my_p > pj || (my_p == pj && my_e < ej)));
+            rank = lane == j ? bef : rank;
+        }
+        if (lane < total && rank < n_used) {
+            r_e[rank] = my_e;
+            r_w[rank] = __uint_as_float(my_p);
+        }
+        __builtin_amdgcn_wave_barrier();
+        const float w_mine = lane < n_used ? r_w[lane] : 0.f;
+        const int32_t e_mine = lane < n_used ? r_e[lane] : 0;
+        float wsum = 0.f;
+        for (int k = 0; k < n_used; k++) wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_mine), k));
+        if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
+        if (lane < n_used) {
+            sel_e[lane] = e_mine;
+            sel_w[lane] = w_mine / wsum;
+        }
+    }
+    __syncthreads();
+}
+
 // ------------------------------------------------------------------------------- up ----------
 
 // grid: (ffn/RPP/4/P row groups, n_used+1 slots, n_tok).  A pass of a wave is RPP gate rows and the
@@ -454,13 +572,9 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
     for (int i = 0; i < K / kBlock; i++) xv[i] = x[tid + i * kBlock];
 
     if (a.logits) {
-        // route this block's token from the router's logits (one wave), share the result
-        if (wave == 0) {
-            const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
-            route_token<8, false>(lg, a.n_expert, a.n_used, s_topk, s_w, probs);
-            if (lane == 0) s_w[a.n_used] = sigmoid_exact(lg[a.n_expert]);
-        }
-        __syncthreads();
+        // route this block's token from the router's logits, all four waves together
+        const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
+        route_block256(lg, a.n_expert, a.n_used, true, s_topk, s_w, probs);
         if (blockIdx.x == 0 && blockIdx.y == 0) {
             if (tid < a.n_used) a.topk[static_cast<size_t>(t) * a.n_used + tid] = s_topk[tid];
             if (tid <= a.n_used) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + tid] = s_w[tid];

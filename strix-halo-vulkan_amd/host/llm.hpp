@@ -205,9 +205,9 @@ public:
     uint64_t ActivationBytes() const { return act_bytes_; }
     // Where the top-k selection runs (MoEGPU.SetRouter, llm/gpu_moe.go:307): fused, in the prologue
     // of the gate/up kernel from the router's logits, or as a dispatch of its own after the router.
-    // Its own dispatch unless asked otherwise: fused measures about 1% faster on one-row passes
-    // (one launch fewer on the step's critical path, the selection repeated by every workgroup)
-    // and far slower on passes of several rows; mode 2 fuses one-row passes only.
+    // Fused on one-row passes unless asked otherwise (mode 2): one launch fewer on the step's
+    // critical path, the selection repeated by every workgroup with all four of its waves (482 to
+    // 495 tok/s); on passes of several rows it is far slower than a dispatch of its own.
     void SetRouter(bool fused) { route_mode_ = fused ? 1 : 0; }
     bool FusedRouter(int rows = 1) const { return route_mode_ == 1 || (route_mode_ == 2 && rows == 1); }
 
@@ -219,7 +219,7 @@ private:
     float *in_, *out_, *xn_, *logits_, *weights_, *act_, *pairs_ = nullptr;
     int32_t *topk_, *group_ = nullptr;
     uint64_t act_bytes_ = 0;
-    int route_mode_ = 0;  // 0 own dispatch, 1 fused, 2 fused for one-row passes
+    int route_mode_ = 2;  // 0 own dispatch, 1 fused, 2 fused for one-row passes
 };
 
 // llm.DeltaNetGPU (llm/gpu_deltanet.go:207-322, NewDeltaNetGPUBank :421)
