@@ -439,8 +439,9 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     __shared__ uint32_t s_gm[16];
     __shared__ uint32_t s_thr;
     __shared__ int s_cnt[8];
-    __shared__ uint32_t cand_p[64];
-    __shared__ int32_t cand_e[64];
+    __shared__ __align__(16) uint32_t cand_p[64];
+    __shared__ __align__(16) int32_t cand_e[64];
+    __shared__ int s_before[4][64];
     __shared__ int32_t r_e[kMaxUsed];
     __shared__ float r_w[kMaxUsed];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -448,6 +449,10 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     const bool has0 = e0 < n_expert, has1 = e1 < n_expert;
     const float l0 = has0 ? lg[e0] : -INFINITY, l1 = has1 ? lg[e1] : -INFINITY;
     const float lsh = (tid == 255 && shared_gate) ? lg[n_expert] : 0.f;
+    if (tid < 64) {  // an empty candidate comes before nobody
+        cand_p[tid] = 0u;
+        cand_e[tid] = 0x7FFFFFFF;
+    }
     float mx = wave_max_all(fmaxf(l0, l1));
     if (lane == 0) s_max[wave] = mx;
     __syncthreads();
@@ -467,9 +472,14 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     const uint32_t kh0 = has0 ? __float_as_uint(ex0 * inv) : 0u, kh1 = has1 ? __float_as_uint(ex1 * inv) : 0u;
     // 16 groups of 16 threads: n_used of them hold a key at or above the n_used-th largest group maximum
     uint32_t gm = kh0 > kh1 ? kh0 : kh1;
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(gm), off, 64));
+    {
+        uint32_t o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppXor1, 0xF, 0xF, false));
+        gm = o > gm ? o : gm;
+        o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppXor2, 0xF, 0xF, false));
+        gm = o > gm ? o : gm;
+        o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppHalfMirror, 0xF, 0xF, false));
+        gm = o > gm ? o : gm;
+        o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppMirror, 0xF, 0xF, false));
         gm = o > gm ? o : gm;
     }
     if ((lane & 15) == 0) s_gm[tid >> 4] = gm;
@@ -518,16 +528,26 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     }
     if (tid == 255) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh) : 0.f;
     __syncthreads();
-    if (wave == 0) {
-        const uint32_t my_p = lane < total ? cand_p[lane] : 0u;
-        const int my_e = lane < total ? cand_e[lane] : 0x7FFFFFFF;
-        int rank = 0;
-        for (int j = 0; j < total; j++) {
-            const uint32_t pj = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(my_p), j));
-            const int ej = __builtin_amdgcn_readlane(my_e, j);
-            const int bef = __popcll(__ballot(my_p > pj || (my_p == pj && my_e < ej)));
-            rank = lane == j ? bef : rank;
+    // rank of candidate i = how many candidates come before it: the four waves each compare it
+    // with a quarter of the table
+    const uint32_t my_p = cand_p[lane];
+    const int my_e = cand_e[lane];
+    {
+        int before = 0;
+#pragma unroll
+        for (int j4 = 0; j4 < 4; j4++) {
+            const uint4 pj = *reinterpret_cast<const uint4 *>(&cand_p[wave * 16 + j4 * 4]);
+            const int4 ej = *reinterpret_cast<const int4 *>(&cand_e[wave * 16 + j4 * 4]);
+            before += (pj.x > my_p || (pj.x == my_p && ej.x < my_e)) ? 1 : 0;
+            before += (pj.y > my_p || (pj.y == my_p && ej.y < my_e)) ? 1 : 0;
+            before += (pj.z > my_p || (pj.z == my_p && ej.z < my_e)) ? 1 : 0;
+            before += (pj.w > my_p || (pj.w == my_p && ej.w < my_e)) ? 1 : 0;
         }
+        s_before[wave][lane] = before;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int rank = (s_before[0][lane] + s_before[1][lane]) + (s_before[2][lane] + s_before[3][lane]);
         if (lane < total && rank < n_used) {
             r_e[rank] = my_e;
             r_w[rank] = __uint_as_float(my_p);
