@@ -207,7 +207,7 @@ public:
     // of the gate/up kernel from the router's logits, or as a dispatch of its own after the router.
     // Fused on one-row passes unless asked otherwise (mode 2): one launch fewer on the step's
     // critical path, the selection repeated by every workgroup with all four of its waves (482 to
-    // 495 tok/s); on passes of several rows it is far slower than a dispatch of its own.
+    // 509 tok/s); on passes of several rows it is far slower than a dispatch of its own.
     void SetRouter(bool fused) { route_mode_ = fused ? 1 : 0; }
     bool FusedRouter(int rows = 1) const { return route_mode_ == 1 || (route_mode_ == 2 && rows == 1); }
 
