@@ -97,6 +97,35 @@ def test_long_pass_matches_the_cpu():
           (O.rel_l2(a[1], hd_cpu), O.rel_l2(a[0], lg_cpu), O.rel_l2(a[0], b[0]), a[5], b[5]))
 
 
+def test_long_passes_on_another_slot_and_with_a_one_row_group():
+    """195 prompt rows as passes of 130 (groups of 64 + 64 + 2) and 65 (a group of 64 and a group of one row),
+    on sequence slot 1 and on slot 0: the same bits on both (every group reads its own slot's position
+    words), and the rows in passes of 64 to rounding."""
+    rng = np.random.default_rng(195)
+    prompt = None
+    out = {}
+    for rows in (130, 64):
+        cfg = cfg_rows(max_tokens=rows, nkv=256, slots=2, head_rows=1, speculative=0, nextn=0)
+        if prompt is None:
+            prompt = rng.integers(0, cfg.vocab, size=195).astype(np.int32)
+        m = LA.LLM(cfg)
+        m.init_synthetic(4321)
+        m.stage()
+        got = []
+        for slot in (1, 0):
+            m.use_slot(slot)
+            m.reset()
+            lg, hd = m.extend(prompt, want_hidden=True)
+            assert m.past() == 195
+            got.append((lg, hd, m.generate(3)[0]))
+        assert np.array_equal(got[0][0], got[1][0]) and np.array_equal(got[0][1], got[1][1])
+        assert np.array_equal(got[0][2], got[1][2])
+        out[rows] = got[0]
+        m.close()
+    assert O.rel_l2(out[130][0], out[64][0]) <= 1e-4 and O.rel_l2(out[130][1], out[64][1]) <= 1e-4
+    assert np.array_equal(out[130][2], out[64][2])
+
+
 def test_extend_rows_is_every_rows_logits(rig):
     m, cfg, tensors = rig
     rng = np.random.default_rng(12)
