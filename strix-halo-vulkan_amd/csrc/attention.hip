@@ -372,10 +372,12 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
 // grid: (n_head * 4, R, n_seq * n_groups), one block = 64 dims of one head; its waves share the slices'
 // records of that (row, head), each folds its share with a running max (all of a batch's loads in
 // flight together), and the first wave folds their results.
+// NW waves a block: eight for a decode step, whose one row pair has a slice per 128 cells of context to fold;
+// one for a pass of many row pairs, which takes few slices a pair and would launch eight times the waves for nothing.
 constexpr int kMergeWaves = 8;
-template <int R>
-__global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_decode_args a, int row00, int n_groups) {
-    __shared__ float red[3][kMergeWaves][64];
+template <int R, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_merge_kernel(shv_attn_decode_args a, int row00, int n_groups) {
+    __shared__ float red[3][NW][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + lane, j = blockIdx.y;
     const int seq = blockIdx.z / n_groups, row0 = row00 + R * (blockIdx.z % n_groups);
@@ -386,7 +388,7 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attn_merge_kernel(shv_attn_d
     int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
     if (n_active > a.n_splits) n_active = a.n_splits;
     const float *pin = a.partial + (static_cast<size_t>(blockIdx.z) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
-    constexpr int MB = 16, NW = kMergeWaves;
+    constexpr int MB = 16;
     float num = 0.f, den = 0.f, M = -INFINITY;
     for (int s0 = wave; s0 < n_active; s0 += NW * MB) {
         float v[MB];
@@ -463,7 +465,8 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
     if (b.n_splits > want) b.n_splits = want < 1 ? 1 : want;
     dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
     SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append);
-    SHV_LAUNCH(ctx, (attn_merge_kernel<R>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, b, row0, n_groups);
+    if (a.n_seq * n_groups >= 8 && b.n_splits <= 16) SHV_LAUNCH(ctx, (attn_merge_kernel<R, 1>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64), 0, b, row0, n_groups);
+    else SHV_LAUNCH(ctx, (attn_merge_kernel<R, kMergeWaves>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, b, row0, n_groups);
     return SHV_OK;
 }
 
