@@ -8,11 +8,12 @@
 //   moe_up_grouped_kernel     a block = (expert, half of its ffn rows) and up to 48 of its tokens
 //                             at a time: their xn rows go through LDS as matrix-core operands
 //                             (two halves hi + lo, as the projections do) in slabs of 512 columns,
-//                             each wave streams two gate tiles of 16 rows and the matching up
-//                             tiles, forms a sub-block's weights once for all three token tiles,
-//                             SwiGLU in registers, act[pair] out
+//                             each wave streams one gate tile of 16 rows and the matching up
+//                             tile, forms a sub-block's weights once (as the whole numbers n * sc,
+//                             exact in binary16) for all three token tiles, keeps one matrix
+//                             accumulator per super-block, SwiGLU in registers, act[pair] out
 //   moe_down_grouped_kernel   a block = (expert, quarter of n_embd rows): act rows staged the
-//                             same way (one slab), each wave four tiles, raw products to pairs[pair]
+//                             same way (one slab), each wave two tiles, raw products to pairs[pair]
 //   moe_combine_kernel        out[t] = residual[t] + sum over slots of weights[t][s]*pairs[t][s],
 //                             slots in order
 // The shared expert is an expert every token lists: its blocks take 48 tokens each.
@@ -27,11 +28,11 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 8;
+constexpr int kWaves = 16;
 constexpr int kThreads = kWaves * 64;
 constexpr int kTT = 3;            // matrix-core tiles of 16 tokens a block multiplies per pass over the weights
 constexpr int kTok = 16 * kTT;    // tokens of such a pass
-constexpr int kTiles = 4;         // weight row tiles of 16 a wave owns
+constexpr int kTiles = 2;         // weight row tiles of 16 a wave owns
 constexpr int kSlab = 512;        // columns of the tokens' rows staged at a time
 constexpr int kSlabSubs = kSlab / 32;
 constexpr int kFrag = 64 * 16;    // one operand: a lane's eight halves
@@ -129,11 +130,12 @@ struct RowStream {
 // The 64-weight groups [G0, G0 + NG) of R row tiles (lane rows at rp[r]) against the staged slab,
 // whose first sub-block is the first of group G0:
 // y[r][tt][j] += sum over those columns of W[row of tile r][.] * x[token 16 tt + 4 kb + j][.].
-// A sub-block's eight weights per lane are formed once and multiplied with every token tile:
-// forming them is most of the vector work of such a kernel.
+// A sub-block's eight weights per lane are formed once, as the whole numbers n * sc, and multiplied
+// with every token tile; the matrix accumulators run over a super-block and take its d at its end,
+// the min term is subtracted per sub-block: y = sum_sb d * (sum x * n * sc) - sum_sub dmin * m * sum(x).
 template <int NG, int R>
 __device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], RowStream<R> &st, int G0, int G_last, const char *frags,
-                                                 const float *sxs, int lane, int n_tt, float4_t (&y)[R][kTT]) {
+                                                 const float *sxs, int lane, int n_tt, float4_t (&acc)[R][kTT], float4_t (&y)[R][kTT]) {
     const int kb = lane >> 4;
     const NibbleConsts nc = nibble_consts();
 #pragma unroll 1
@@ -143,20 +145,18 @@ __device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], Row
 #pragma unroll
         for (int r = 0; r < R; r++) q[r] = st.q_next[r];
         st.ask_group(rp, G + 1, G_last, kb);
-        if (g == 0) st.ask_header(rp, (G >> 2) + 1, G_last >> 2);
         uint32_t sc[R], mn[R];
-        float dd[R], dmin[R];
+        float dmin[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
             q4k_group_scale_min(st.hdr[r], g, sc[r], mn[r]);
-            dd[r] = f16_bits_to_f32(st.hdr[r].x);
             dmin[r] = f16_bits_to_f32(st.hdr[r].x >> 16);
         }
 #pragma unroll
         for (int hi = 0; hi < 2; hi++) {
             const int sub = gi * 2 + hi;
             half8_t b[R];
-            float ds[R], e[R];
+            float dm[R];
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 const uint32_t q0 = q[r].x, q1 = q[r].y;
@@ -169,9 +169,11 @@ __device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], Row
                     v.x = (q0 & nc.mask) | nc.one; v.y = ((q0 >> 8) & nc.mask) | nc.one;
                     v.z = (q1 & nc.mask) | nc.one; v.w = ((q1 >> 8) & nc.mask) | nc.one;
                 }
-                b[r] = __builtin_bit_cast(half8_t, v);
-                ds[r] = dd[r] * static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu);
-                e[r] = fmaf(64.f, ds[r], dmin[r] * static_cast<float>(hi ? mn[r] >> 8 : mn[r] & 0xFFu));
+                // the halves 64 + n become n * sc: whole numbers up to 15 * 63, exact in binary16 (as is
+                // 64 * sc, should the two steps be fused), so one accumulator runs over the super-block
+                const _Float16 s16 = static_cast<_Float16>(static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu));
+                b[r] = (__builtin_bit_cast(half8_t, v) - static_cast<half8_t>(static_cast<_Float16>(64.f))) * static_cast<half8_t>(s16);
+                dm[r] = dmin[r] * static_cast<float>(hi ? mn[r] >> 8 : mn[r] & 0xFFu);
             }
 #pragma unroll
             for (int tt = 0; tt < kTT; tt++) {
@@ -183,15 +185,27 @@ __device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], Row
                 const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
 #pragma unroll
                 for (int r = 0; r < R; r++) {
-                    float4_t acc = {0.f, 0.f, 0.f, 0.f};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc, 0, 0, 0);
+                    acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc[r][tt], 0, 0, 0);
+                    acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc[r][tt], 0, 0, 0);
 #pragma unroll
-                    for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(-e[r], sxv[j], fmaf(ds[r], acc[j], y[r][tt][j]));
+                    for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(-dm[r], sxv[j], y[r][tt][j]);
                 }
             }
         }
         if (g == 3) {
+            // the super-block ends: its sums take its d, the next one's header moves in
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const float dd = f16_bits_to_f32(st.hdr[r].x);
+#pragma unroll
+                for (int tt = 0; tt < kTT; tt++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(dd, acc[r][tt][j], y[r][tt][j]);
+                    acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            // asked for only now: a header a super-block ahead costs sixteen registers these kernels do not have
+            st.ask_header(rp, (G >> 2) + 1, G_last >> 2);
 #pragma unroll
             for (int r = 0; r < R; r++) st.hdr[r] = st.hdr_next[r];
         }
@@ -210,6 +224,11 @@ __device__ __forceinline__ void rows_times_tiles(const char *const (&rp)[kTiles]
     for (int r = 0; r < kTiles; r++)
 #pragma unroll
         for (int tt = 0; tt < kTT; tt++) y[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float4_t acc[kTiles][kTT];
+#pragma unroll
+    for (int r = 0; r < kTiles; r++)
+#pragma unroll
+        for (int tt = 0; tt < kTT; tt++) acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
     RowStream<kTiles> st;
     st.ask_header(rp, 0, GROUPS / 4 - 1);
 #pragma unroll
@@ -220,7 +239,7 @@ __device__ __forceinline__ void rows_times_tiles(const char *const (&rp)[kTiles]
         __syncthreads();   // the list is written / the slab before this one has been multiplied
         gather_slab(rows_s, m, sl * kSlab, frags, sxs);
         __syncthreads();
-        slab_times_tiles<NG, kTiles>(rp, st, sl * NG, GROUPS - 1, frags, sxs, lane, n_tt, y);
+        slab_times_tiles<NG, kTiles>(rp, st, sl * NG, GROUPS - 1, frags, sxs, lane, n_tt, acc, y);
     }
 }
 
@@ -264,9 +283,9 @@ struct Staging {
 };
 constexpr size_t kGroupedLds = static_cast<size_t>(kSlabSubs) * 2 * kTT * kFrag + static_cast<size_t>(kSlabSubs) * kTok * 4 + kTok * sizeof(float *) + kTok * 4;
 
-// grid: n_expert * parts + parts * ceil(n_tok / 48) blocks of 8 waves, parts = ffn / 256; K = n_embd.
-// A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tiles 2w and
-// 2w + 1 and the up tiles of the same rows, so SwiGLU stays in registers.
+// grid: n_expert * parts + parts * ceil(n_tok / 48) blocks of 16 waves, parts = ffn / 256; K = n_embd.
+// A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tile w and
+// the up tile of the same rows, so SwiGLU stays in registers.
 template <int K>
 __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_args a) {
     extern __shared__ __align__(16) char smem[];
@@ -278,11 +297,11 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
     const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row = u.part * 256 + wave * 32 + n;   // this lane's row in the wave's first tile, gate and up alike
+    const int row = u.part * 256 + wave * 16 + n;   // this lane's row of the expert, gate and up alike
     const size_t wrow = static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.ffn + row;
     const char *gp = static_cast<const char *>(u.expert < 0 ? a.gate_sh : a.gate_exps) + wrow * row_bytes;
     const char *up = static_cast<const char *>(u.expert < 0 ? a.up_sh : a.up_exps) + wrow * row_bytes;
-    const char *rp[kTiles] = {gp, gp + 16 * row_bytes, up, up + 16 * row_bytes};
+    const char *rp[kTiles] = {gp, up};
     for (int t0 = 0; t0 < u.count; t0 += kTok) {
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {
@@ -298,12 +317,8 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
             for (int j = 0; j < 4; j++) {
                 const int i = 16 * tt + 4 * kb + j;
                 if (i < m) {
-                    float *dst = a.act + static_cast<size_t>(st.pair_s[i]) * a.ffn + row;
-#pragma unroll
-                    for (int q = 0; q < 2; q++) {
-                        const float gv = y[q][tt][j];
-                        dst[16 * q] = gv * sigmoid_exact(gv) * y[2 + q][tt][j];
-                    }
+                    const float gv = y[0][tt][j];
+                    a.act[static_cast<size_t>(st.pair_s[i]) * a.ffn + row] = gv * sigmoid_exact(gv) * y[1][tt][j];
                 }
             }
         __syncthreads();   // the list is read to the end before the next one replaces it
@@ -311,7 +326,7 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
 }
 
 // grid: n_expert * parts + parts * ceil(n_tok / 48) blocks, parts = n_embd / 512: a part is 512
-// output rows = 32 tiles, wave w takes tiles 4w .. 4w + 3.  K = ffn.
+// output rows = 32 tiles, wave w takes tiles 2w and 2w + 1.  K = ffn.
 template <int K>
 __global__ __launch_bounds__(kThreads) void moe_down_grouped_kernel(shv_moe_down_args a) {
     extern __shared__ __align__(16) char smem[];
@@ -324,10 +339,10 @@ __global__ __launch_bounds__(kThreads) void moe_down_grouped_kernel(shv_moe_down
     const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row0 = u.part * 512 + wave * 64 + n;
+    const int row0 = u.part * 512 + wave * 32 + n;
     const char *base = static_cast<const char *>(u.expert < 0 ? a.down_sh : a.down_exps) +
                        (static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.n_embd + row0) * row_bytes;
-    const char *rp[kTiles] = {base, base + 16 * row_bytes, base + 32 * row_bytes, base + 48 * row_bytes};
+    const char *rp[kTiles] = {base, base + 16 * row_bytes};
     for (int t0 = 0; t0 < u.count; t0 += kTok) {
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {
