@@ -831,7 +831,7 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     const int slot0 = r_other ? a.n_used : 0, slots = r_other ? 1 : s_other ? a.n_used : a.n_used + 1;  // the Q4_K part
     SHV_REQUIRE(shv_aligned16(a.gate_exps) && shv_aligned16(a.up_exps) && shv_aligned16(a.gate_sh) && shv_aligned16(a.up_sh),
                 "moe_up: weight banks must be 16-byte aligned");
-    // a pass of many rows whose selection is made: the experts' weights once per 16 tokens
+    // a pass of many rows whose selection is made: the experts' weights once per 48 tokens
     if (!r_other && !s_other && shv_moe_up_grouped_covers(ctx, a)) return shv_launch_moe_up_grouped(ctx, a);
     dim3 block(kBlock);
     // enough tokens to fill the chip with blocks eight passes tall; not when the blocks route
