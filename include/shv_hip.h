@@ -411,6 +411,16 @@ int shv_embed(shv_ctx *ctx, const shv_embed_args *a);
 int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_advance(shv_ctx *ctx, const shv_advance_args *a);
 
+/* shv_argmax for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * results as shv_argmax; the per-block winners and arrival counters live in a static device
+ * array of the library (under 8 KB on each GPU, bound at shv_init) instead of in memory the
+ * context allocated, and the call allocates and frees nothing.  At most
+ * SHV_ARGMAX_STATIC_MAX_ROWS rows a call; more is refused with SHV_E_INVALID.  All calls on one
+ * GPU share the array: calls that overlap on one GPU (two contexts, two streams) race. */
+#define SHV_ARGMAX_STATIC_MAX_ROWS 14
+int shv_argmax_static(shv_ctx *ctx, const shv_argmax_args *a);
+
 #ifdef __cplusplus
 }
 #endif

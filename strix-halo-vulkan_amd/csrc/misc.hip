@@ -164,7 +164,34 @@ __global__ void advance_kernel(shv_advance_args a) {
     if (s < a.n_seq) a.pos[s] += a.delta;
 }
 
+// ---- the arg-max that allocates nothing ------------------------------------------------------
+// Its per-block winners and arrival counters live in this array instead of in memory the context
+// allocated: kArgmaxBlocks values, kArgmaxBlocks indices, then kStaticCounters arrival counters.
+// Every GPU holds its own copy until the process ends; in host code the name is only a handle, the
+// device address comes from hipGetSymbolAddress (shv_static_scratch_bind, once per device).
+constexpr int kStaticCounters = 16;
+constexpr size_t kStaticScratchBytes = shv_ctx::kArgmaxBlocks * (sizeof(float) + sizeof(int32_t)) + kStaticCounters * sizeof(int32_t);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+__global__ void clear_counters_kernel(int32_t *c, int n) {
+    if (static_cast<int>(threadIdx.x) < n) c[threadIdx.x] = 0;
+}
+
 }  // namespace
+
+int shv_static_scratch_bind(shv_ctx *ctx) {
+    SHV_REQUIRE(ctx->device >= 0 && ctx->device < kMaxDevices, "shv_init: device %d; the static scratch table covers %d devices", ctx->device, kMaxDevices);
+    if (!g_scratch_ptr[ctx->device]) {
+        void *p = nullptr;
+        SHV_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));  // the calling thread's current device is ctx->device
+        g_scratch_ptr[ctx->device] = p;
+    }
+    ctx->static_scratch = g_scratch_ptr[ctx->device];
+    return SHV_OK;
+}
 
 int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a) {
     SHV_REQUIRE(a->table && a->ids && a->x, "embed: NULL argument");
@@ -176,19 +203,41 @@ int shv_launch_embed(shv_ctx *ctx, const shv_embed_args *a) {
     return SHV_OK;
 }
 
+static int argmax_blocks(const shv_argmax_args *a) {
+    int nb = (a->n + 1023) / 1024;
+    const int cap = shv_ctx::kArgmaxBlocks / a->n_rows;
+    if (nb > cap) nb = cap;
+    return nb > 256 ? 256 : nb;
+}
+
 int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a) {
     SHV_REQUIRE(a->logits && a->best, "argmax: NULL logits or best");
     SHV_REQUIRE(a->n_rows >= 1 && a->n >= 1 && a->logits_stride >= a->n, "argmax: %d rows of %d, stride %d", a->n_rows, a->n, a->logits_stride);
     SHV_REQUIRE((a->ids == nullptr) == (a->pos == nullptr), "argmax: ids and pos go together");
     SHV_REQUIRE(!a->ids || a->n_rows == 1, "argmax: storing the next token needs exactly one row");
     SHV_REQUIRE(a->advance >= 0, "argmax: advance %d", a->advance);
-    int nb = (a->n + 1023) / 1024;
-    const int cap = shv_ctx::kArgmaxBlocks / a->n_rows;
-    SHV_REQUIRE(cap >= 1 && a->n_rows <= 14, "argmax: %d rows is more than one launch covers", a->n_rows);
-    if (nb > cap) nb = cap;
-    if (nb > 256) nb = 256;
-    SHV_LAUNCH(ctx, argmax_kernel, dim3(nb, a->n_rows), dim3(256), 0, *a, ctx->argmax_val, ctx->argmax_idx,
+    SHV_REQUIRE(a->n_rows <= 14, "argmax: %d rows is more than one launch covers", a->n_rows);
+    SHV_LAUNCH(ctx, argmax_kernel, dim3(argmax_blocks(a), a->n_rows), dim3(256), 0, *a, ctx->argmax_val, ctx->argmax_idx,
                        ctx->counters + shv_ctx::kCounterArgmax);
+    return SHV_OK;
+}
+
+int shv_launch_argmax_static(shv_ctx *ctx, const shv_argmax_args *a) {
+    SHV_REQUIRE(a->logits && a->best, "argmax_static: NULL logits or best");
+    SHV_REQUIRE(a->n_rows >= 1 && a->n >= 1 && a->logits_stride >= a->n, "argmax_static: %d rows of %d, stride %d", a->n_rows, a->n, a->logits_stride);
+    SHV_REQUIRE(a->n_rows <= SHV_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows; the static scratch holds the partial results of at most %d rows a call",
+                a->n_rows, SHV_ARGMAX_STATIC_MAX_ROWS);
+    SHV_REQUIRE((a->ids == nullptr) == (a->pos == nullptr), "argmax_static: ids and pos go together");
+    SHV_REQUIRE(!a->ids || a->n_rows == 1, "argmax_static: storing the next token needs exactly one row");
+    SHV_REQUIRE(a->advance >= 0, "argmax_static: advance %d", a->advance);
+    SHV_REQUIRE(ctx->static_scratch, "argmax_static: the static scratch of device %d was not bound at shv_init", ctx->device);
+    float *pval = static_cast<float *>(ctx->static_scratch);
+    int32_t *pidx = reinterpret_cast<int32_t *>(pval + shv_ctx::kArgmaxBlocks);
+    int32_t *counters = pidx + shv_ctx::kArgmaxBlocks;
+    // the array keeps what the last call left: the arrival counters must start at zero (a fill
+    // kernel, not a memset node, so that a caller may record this call into a graph)
+    SHV_LAUNCH(ctx, clear_counters_kernel, dim3(1), dim3(64), 0, counters, kStaticCounters);
+    SHV_LAUNCH(ctx, argmax_kernel, dim3(argmax_blocks(a), a->n_rows), dim3(256), 0, *a, pval, pidx, counters);
     return SHV_OK;
 }
 

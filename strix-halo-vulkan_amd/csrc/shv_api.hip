@@ -65,6 +65,13 @@ int shv_init(int device, shv_ctx **out) {
         shv_destroy(ctx);
         return shv_set_error(SHV_E_HIP, "shv_init: %s", hipGetErrorString(e));
     }
+    if (std::strncmp(ctx->prop.gcnArchName, "gfx950", 6) == 0) {
+        const int rc = shv_static_scratch_bind(ctx);
+        if (rc != SHV_OK) {
+            shv_destroy(ctx);
+            return rc;
+        }
+    }
     if (std::strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0) {
         char arch[64];
         std::snprintf(arch, sizeof(arch), "%s", ctx->prop.gcnArchName);
@@ -344,5 +351,10 @@ int shv_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a) { return dispat
 int shv_embed(shv_ctx *ctx, const shv_embed_args *a) { return dispatch_one(ctx, SHV_OP_EMBED, a, sizeof(*a)); }
 int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a) { return dispatch_one(ctx, SHV_OP_ARGMAX, a, sizeof(*a)); }
 int shv_advance(shv_ctx *ctx, const shv_advance_args *a) { return dispatch_one(ctx, SHV_OP_ADVANCE, a, sizeof(*a)); }
+
+int shv_argmax_static(shv_ctx *ctx, const shv_argmax_args *a) {
+    SHV_REQUIRE(ctx && a, "shv_argmax_static: NULL argument");
+    return shv_launch_argmax_static(ctx, a);
+}
 
 }  // extern "C"

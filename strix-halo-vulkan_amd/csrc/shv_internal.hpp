@@ -40,6 +40,9 @@ struct shv_ctx {
     float *argmax_val = nullptr;
     int32_t *argmax_idx = nullptr;
     enum { kArgmaxBlocks = 512 };
+    // device address of this GPU's copy of the library's static scratch array (misc.hip), for the
+    // entry point that allocates nothing
+    void *static_scratch = nullptr;
     // Per-kernel GPU timestamps for a marked dispatch: while `marking` is set every launch is
     // bracketed by a pair of events taken from the dispatch packet itself, so an op's time is the
     // time its kernels ran and holds no launch gap.
@@ -130,3 +133,5 @@ int shv_launch_embed_typed(shv_ctx *ctx, const shv_embed_args *a);  // a table i
 long long shv_type_bytes(int type, long long n);                    // bytes of n elements of a ggml type, -1 if refused
 int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_launch_advance(shv_ctx *ctx, const shv_advance_args *a);
+int shv_static_scratch_bind(shv_ctx *ctx);  // at shv_init, with ctx->device current
+int shv_launch_argmax_static(shv_ctx *ctx, const shv_argmax_args *a);

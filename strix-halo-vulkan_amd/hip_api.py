@@ -145,6 +145,7 @@ SYMBOLS = [
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
+    "shv_argmax_static",
 ]
 
 _lib = None
@@ -199,6 +200,7 @@ def load():
     L.shv_embed.argtypes = [vp, C.POINTER(EmbedArgs)]
     L.shv_argmax.argtypes = [vp, C.POINTER(ArgmaxArgs)]
     L.shv_advance.argtypes = [vp, C.POINTER(AdvanceArgs)]
+    L.shv_argmax_static.argtypes = [vp, C.POINTER(ArgmaxArgs)]
     _lib = L
     return L
 
