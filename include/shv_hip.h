@@ -132,6 +132,10 @@ typedef struct {
     int32_t x_stride, y_stride, z_stride;
     int32_t seq_len, ring_slots, ring_stride;
     int32_t z_ring;
+    float *y_flat;           /* with ring output, one row (n_tok == 1): the row is also stored here, at an
+                                address that does not depend on the position, for a consumer that would
+                                otherwise wait for the position word before it can ask for the row (the
+                                DeltaNet output projection's gate z); NULL: not stored */
 } shv_gemv_q4k_args;
 
 /* ggml type numbers of the tensor types the reference's loader accepts (Dequantizable,
@@ -240,6 +244,9 @@ typedef struct {
      * Tensor.DequantizeRow forms them; the selection then comes from the router (logits NULL). */
     int32_t gate_type, up_type, gate_sh_type, up_sh_type;
     int32_t *group;          /* workspace of the grouped path, or NULL */
+    int32_t no_shared_gate;  /* with logits: nonzero says the router ran without a shared_gate (it then
+                                left logits[n_expert] unwritten), and weights[t][n_used] is stored as 0,
+                                as the router's own selection stores it */
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +

@@ -37,21 +37,18 @@ constexpr int kMaxSplits = 512;
 constexpr int kRec = kRep * (kD + 2);  // floats of one (slice, row) record: per head d values, max, sum
 
 // RMS norm over the 256 dims of one head by one wave (4 dims per lane), then NeoX rotary on the
-// first rope_dims dims through LDS.  dst is 256 floats of LDS.
-__device__ __forceinline__ void norm_rope_loaded(const float4 v, const float *gamma, const float *rope_row, int rope_dims, float eps,
+// first rope_dims dims through LDS.  dst is 256 floats of LDS.  The head's values, gamma and the
+// rotary factors of lane < rope_dims/2 (cs, sn) are in registers already: a caller asks for
+// everything it will need before it waits for any of it.
+__device__ __forceinline__ void norm_rope_loaded(const float4 v, const float4 g, float cs, float sn, int rope_dims, float eps,
                                                  float *dst, int lane) {
     const float ss = wave_sum_all(fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w))));
     const float sc = 1.f / sqrtf(ss / static_cast<float>(kD) + eps);
-    const float4 g = *reinterpret_cast<const float4 *>(gamma + 4 * lane);
-    dst[4 * lane + 0] = v.x * sc * g.x;
-    dst[4 * lane + 1] = v.y * sc * g.y;
-    dst[4 * lane + 2] = v.z * sc * g.z;
-    dst[4 * lane + 3] = v.w * sc * g.w;
+    *reinterpret_cast<float4 *>(dst + 4 * lane) = make_float4(v.x * sc * g.x, v.y * sc * g.y, v.z * sc * g.z, v.w * sc * g.w);
     __builtin_amdgcn_wave_barrier();
     const int half = rope_dims / 2;
     if (lane < half) {
         const float x0 = dst[lane], x1 = dst[lane + half];
-        const float cs = rope_row[lane], sn = rope_row[half + lane];
         dst[lane] = x0 * cs - x1 * sn;
         dst[lane + half] = x0 * sn + x1 * cs;
     }
@@ -60,7 +57,9 @@ __device__ __forceinline__ void norm_rope_loaded(const float4 v, const float *ga
 
 __device__ __forceinline__ void norm_rope_head(const float *src, const float *gamma, const float *rope_row, int rope_dims,
                                                float eps, float *dst, int lane) {
-    norm_rope_loaded(*reinterpret_cast<const float4 *>(src + 4 * lane), gamma, rope_row, rope_dims, eps, dst, lane);
+    const int half = rope_dims / 2;
+    const float cs = lane < half ? rope_row[lane] : 0.f, sn = lane < half ? rope_row[half + lane] : 0.f;
+    norm_rope_loaded(*reinterpret_cast<const float4 *>(src + 4 * lane), *reinterpret_cast<const float4 *>(gamma + 4 * lane), cs, sn, rope_dims, eps, dst, lane);
 }
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
@@ -108,8 +107,31 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
     // a few on each die), and all but the first of a die find the slice in its L2
     const int gz = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
     const int seq = gz / n_groups, row0 = row00 + R * (gz % n_groups);
+    // The sequence's slot and position come from device memory.  Asked for first; what does not
+    // depend on them (the rows' q heads of this wave, the new cells' k and v, the norms' gammas) is
+    // asked for right behind, before either is waited for: loads come back in the order they
+    // were issued, and a chain of dependent round trips is what this kernel's prologue costs.
     const int slot = a.slot ? a.slot[seq] : seq;
-    const int p_first = (a.pos ? a.pos[seq] : 0) + row0;  // position of the group's first row
+    const int pos_first = a.pos ? a.pos[seq] : 0;
+    const int tid_ = threadIdx.x, lane_ = tid_ & 63, wave_ = tid_ >> 6;
+    const int valid_ = a.seq_len - row0 < R ? a.seq_len - row0 : R;
+    const float *qkv0 = a.qkv + static_cast<size_t>(seq * a.seq_len + row0) * a.qkv_stride;
+    float4 qv[R][2], kv[R];
+    float vv[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const int jr = j < valid_ ? j : valid_ - 1;
+        const float *qkv = qkv0 + static_cast<size_t>(jr) * a.qkv_stride;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            qv[j][i] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(kvh * kRep + wave_ * 2 + i) * 2 * kD + 4 * lane_);
+        // every wave asks for the row's k (one of them will append it): straight-line code, so that
+        // the compiler's count of outstanding loads stays exact and nothing waits for the tile early
+        kv[j] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD + 4 * lane_);
+        vv[j] = qkv[static_cast<size_t>(a.n_head) * 2 * kD + a.n_head_kv * kD + kvh * kD + tid_];
+    }
+    const float4 gq = *reinterpret_cast<const float4 *>(a.q_norm + 4 * lane_), gk = *reinterpret_cast<const float4 *>(a.k_norm + 4 * lane_);
+    const int p_first = pos_first + row0;  // position of the group's first row
     // the last group of a sequence with an odd number of rows holds one: its second row repeats
     // the first and is thrown away
     const int valid = a.seq_len - row0 < R ? a.seq_len - row0 : R;
@@ -158,42 +180,49 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
         for (int db = 0; db < 16; db++)
             vreg[db] = *reinterpret_cast<const uint4 *>(vt + static_cast<size_t>(t0 / kTile) * vtile + (16 * db + n) * kTile + 8 * q);
     };
-    // the wave's first tile is requested before anything else, unless this launch is about to
-    // append cells inside it
-    const int t_first = c0 + kTile * wave;
-    const bool early = t_first < c1 && t_first + kTile <= p_first;
-    if (early) load_tile(ta, t_first);
-
-    // ---- prologue: queries (float32, into sm.big), new cells ----
+    // ---- prologue: queries (float32, into sm.big), new cells.  The rows' values were asked for at
+    //      the top; the rotary factors (whose row the position names) and the wave's first tile of
+    //      the cache go out together now ----
     float *qtmp = &sm.big[0][0][0];  // [8*R][kD]
-    const float *qkv0 = a.qkv + static_cast<size_t>(seq * a.seq_len + row0) * a.qkv_stride;
+    const int half_rope = a.rope_dims / 2;
+    float cs[R], sn[R];
+    bool app[R];
 #pragma unroll
     for (int j = 0; j < R; j++) {
         const int jr = j < valid ? j : valid - 1;
-        const float *qkv = qkv0 + static_cast<size_t>(jr) * a.qkv_stride;
         const int p = p_first + jr;
-        const float *rope_row = a.rope + static_cast<size_t>(p) * a.rope_dims;
+        const float *rope_row = a.rope_dims > 0 ? a.rope + static_cast<size_t>(p) * a.rope_dims : a.q_norm;  // no rotary: any readable words
+        app[j] = append && p >= c0 && p < c1;  // the new cell of row j lies in this slice
+        const int rl = lane < half_rope ? lane : 0;  // a select, not a branch around the loads
+        cs[j] = rope_row[rl];
+        sn[j] = rope_row[half_rope + rl];
+    }
+    // the wave's first tile, unless this launch is about to append cells inside it
+    // (asked for by every wave, without a branch around the loads, so that the compiler's count of
+    // outstanding loads stays exact and the norms below wait for their own inputs only, not for the
+    // tile: a wave with no tile of its own in a short slice asks for the slice's first one)
+    const int t_first = c0 + kTile * wave;
+    const bool early = t_first < c1 && t_first + kTile <= p_first;
+    load_tile(ta, t_first < c1 ? t_first : c0);
+
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+        const int jr = j < valid ? j : valid - 1;
+        const int p = p_first + jr;
         if (nc > 0) {
-            // this wave's two heads: both rows of the fused projection are requested before either is used
-            float4 qv[2];
 #pragma unroll
             for (int i = 0; i < 2; i++)
-                qv[i] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(kvh * kRep + wave * 2 + i) * 2 * kD + 4 * lane);
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-                norm_rope_loaded(qv[i], a.q_norm, rope_row, a.rope_dims, a.eps, qtmp + (8 * j + wave * 2 + i) * kD, lane);
+                norm_rope_loaded(qv[j][i], gq, cs[j], sn[j], a.rope_dims, a.eps, qtmp + (8 * j + wave * 2 + i) * kD, lane);
         }
-        if (append && p >= c0 && p < c1) {
-            // the new cell of row j lies in this slice: one wave appends its K, all threads its V
+        if (app[j]) {
+            // one wave appends the new cell's K, all threads its V
             if (wave == ((2 * j) & 3)) {
-                const float *ksrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD;
-                norm_rope_head(ksrc, a.k_norm, rope_row, a.rope_dims, a.eps, sm.kv_tmp[j], lane);
+                norm_rope_loaded(kv[j], gk, cs[j], sn[j], a.rope_dims, a.eps, sm.kv_tmp[j], lane);
                 uint16_t *dst = kc + static_cast<size_t>(p) * kvw;
 #pragma unroll
                 for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(sm.kv_tmp[j][4 * lane + i]));
             }
-            const float *vsrc = qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvw + kvh * kD;
-            vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vsrc[tid]));
+            vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vv[j]));
         }
     }
     __threadfence_block();

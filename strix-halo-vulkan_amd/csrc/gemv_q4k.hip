@@ -66,6 +66,7 @@ struct GemvBatch {
                     float r = acc;
                     if (a.residual) r += res[u][t];
                     a.y[y_off[t] + row[u]] = r;
+                    if (a.y_flat) a.y_flat[row[u]] = r;  // one row (the launcher checks)
                 }
             }
         }
@@ -238,6 +239,164 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
     }
 }
 
+
+// ---- one activation row (the decode step) ------------------------------------------------------
+// A short launch is a chain of latencies, so this kernel keeps the chain short: the weights of all
+// of a wave's passes are requested first; the input row is staged by all threads, four consecutive
+// columns each (128-bit loads and LDS stores), together with the sums of every 32 columns, which
+// the lanes would otherwise each add up again; there is ONE block-wide wait; and an RMS norm's
+// scale, a scalar, is applied to the finished dot products instead of to the staged vector, so
+// that the sum of squares does not stand between the loads and the staging.
+// WAVES waves a block, P passes a wave (pass = 64/(K/64) rows); grid = ceil(passes / (WAVES*P)).
+template <int K, int WAVES, int P, int PRO>
+__global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args a) {
+    constexpr int T = WAVES * 64, LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+    constexpr int NV = K / 4 / T;  // float4 a thread stages
+    static_assert(NV >= 1 && K % (4 * T) == 0, "threads of a block each stage whole float4s");
+    __shared__ __align__(16) float xs[lds_padded(K)];
+    __shared__ __align__(16) float xsum[K / 32];
+    __shared__ float red[WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
+    const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
+    const long long pass0 = (static_cast<long long>(blockIdx.x) * WAVES + wave) * P;
+
+    // Loads return in the order they were asked for, so the input row goes first: it comes from
+    // cache in a fraction of the weights' latency, and the staging below (and the block-wide wait)
+    // is over by the time the first weights arrive, instead of queueing behind all of them.
+    int ring_row = 0;  // the ring slot of the row (its sequence's position and slot)
+    if (a.ring_slots > 0) {
+        const int p = a.pos ? a.pos[0] : 0;
+        const int slot = a.slot ? a.slot[0] : 0;
+        ring_row = slot * a.ring_slots + p % a.ring_slots;
+    }
+    float4 xv[NV], gv[NV], zv[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = 4 * (tid + T * j);
+        xv[j] = *reinterpret_cast<const float4 *>(a.x + c);
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            gv[j] = *reinterpret_cast<const float4 *>(a.gamma + c);
+        } else if constexpr (PRO == SHV_PRO_GATED_NORM) {
+            const float *z = a.z_ring ? a.z + static_cast<size_t>(ring_row) * a.ring_stride : a.z;
+            zv[j] = *reinterpret_cast<const float4 *>(z + c);
+            gv[j] = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
+        } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+            // head_dim > 0: z rows are [q (head_dim) | gate (head_dim)] per head and the gate half is
+            // the one wanted (the fused query projection, llm/attn.go:162-166)
+            const HeadSplit hs(a.head_dim > 0 ? a.head_dim : 1);
+            const int zi = a.head_dim > 0 ? hs.head(c) * 2 * a.head_dim + a.head_dim + hs.dim(c) : c;
+            zv[j] = *reinterpret_cast<const float4 *>(a.z + zi);
+        }
+    }
+    Q4kLane w[P];
+    int row[P];
+#pragma unroll
+    for (int u = 0; u < P; u++) {
+        const long long r = (pass0 + u) * RPP + rsub;
+        row[u] = r < a.n ? static_cast<int>(r) : -1;
+        w[u].load(wbase + static_cast<size_t>(row[u] < 0 ? 0 : row[u]) * ROWB, g);
+    }
+    float res[P];
+#pragma unroll
+    for (int u = 0; u < P; u++) res[u] = (a.residual && row[u] >= 0 && group_sum_owner<LPR>(lane)) ? a.residual[row[u]] : 0.f;
+
+    // ---- stage pro(x): thread i of the block takes columns 4*(i + T*j) .. +3 ----
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = 4 * (tid + T * j);
+        float4 v = xv[j];
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            const float4 gm = gv[j];
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+            v = make_float4(v.x * gm.x, v.y * gm.y, v.z * gm.z, v.w * gm.w);
+        } else if constexpr (PRO == SHV_PRO_GATED_NORM) {
+            // a head of head_dim columns is head_dim/4 consecutive threads (a power of two, 8..64)
+            const float4 gm = gv[j], z4 = zv[j];
+            float hs = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
+            const int span = a.head_dim >> 2;
+            hs = sum8_all(hs);
+            if (span >= 16) hs += dpp_f32<kDppMirror>(hs);
+            if (span >= 32) hs += __shfl_xor(hs, 16, 64);
+            if (span >= 64) hs += __shfl_xor(hs, 32, 64);
+            const float sc = 1.f / sqrtf(hs / static_cast<float>(a.head_dim) + a.eps);
+            v = make_float4(v.x * sc * gm.x * sigmoid_fast(z4.x), v.y * sc * gm.y * sigmoid_fast(z4.y),
+                            v.z * sc * gm.z * sigmoid_fast(z4.z), v.w * sc * gm.w * sigmoid_fast(z4.w));
+        } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+            const float4 z4 = zv[j];
+            v = make_float4(v.x * sigmoid_fast(z4.x), v.y * sigmoid_fast(z4.y), v.z * sigmoid_fast(z4.z), v.w * sigmoid_fast(z4.w));
+        }
+        *reinterpret_cast<float4 *>(&xs[lds_slot(c)]) = v;
+        const float s8 = sum8_all((v.x + v.y) + (v.z + v.w));
+        if ((lane & 7) == 0) xsum[c >> 5] = s8;
+    }
+    if constexpr (PRO == SHV_PRO_RMSNORM) {
+        ss = wave_sum_all(ss);
+        if (lane == 0) red[wave] = ss;
+    }
+    __syncthreads();
+    float scale = 1.f;
+    if constexpr (PRO == SHV_PRO_RMSNORM) {
+        float tot = 0.f;
+#pragma unroll
+        for (int i = 0; i < WAVES; i++) tot += red[i];
+        scale = 1.f / sqrtf(tot / static_cast<float>(K) + a.eps);
+    }
+
+    float xr[64], xs_lo, xs_hi;
+    load_x_slice_presummed(xs, xsum, gi, xr, xs_lo, xs_hi);
+    float *y = a.y;
+    if (a.ring_slots > 0 && !a.z_ring) y += static_cast<size_t>(ring_row) * a.ring_stride;
+    const NibbleConsts nc = nibble_consts();
+#pragma unroll
+    for (int u = 0; u < P; u++) {
+        float acc = w[u].dot(g, nc, xr, xs_lo, xs_hi);
+        acc = group_sum<LPR>(acc);
+        if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
+            const float v = fmaf(acc, scale, res[u]);
+            y[row[u]] = v;
+            if (a.y_flat) a.y_flat[row[u]] = v;
+        }
+    }
+}
+
+// Which one-row launches the kernel above takes: the decode step's projections (2048- and
+// 4096-wide inputs).  A matrix of very many rows (the vocabulary projection) is a stream, not a
+// latency, and stays on the looping kernel; so do the other widths and the pair-norm prologue.
+template <int K, int WAVES, int P>
+int launch_row_kp(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    constexpr int RPP = 64 / (K / 64);
+    const long long passes = (static_cast<long long>(a.n) + RPP - 1) / RPP;
+    const dim3 grid(static_cast<unsigned>((passes + WAVES * P - 1) / (WAVES * P))), block(WAVES * 64);
+    switch (a.prologue) {
+        case SHV_PRO_NONE: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_NONE>), grid, block, 0, a); break;
+        case SHV_PRO_RMSNORM: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_RMSNORM>), grid, block, 0, a); break;
+        case SHV_PRO_GATED_NORM: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_GATED_NORM>), grid, block, 0, a); break;
+        default: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_MUL_SIGMOID>), grid, block, 0, a); break;
+    }
+    return SHV_OK;
+}
+
+bool row_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (a.n_tok != 1 || a.prologue == SHV_PRO_RMSNORM_PAIR) return false;
+    if (a.k != 2048 && a.k != 4096) return false;
+    if (!shv_aligned16(a.x) || (a.gamma && !shv_aligned16(a.gamma)) || (a.z && !shv_aligned16(a.z))) return false;
+    if (a.prologue == SHV_PRO_GATED_NORM && (a.head_dim < 32 || a.head_dim > 256 || (a.z_ring && a.ring_stride % 4 != 0))) return false;
+    if (a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim != 0 && a.head_dim < 4) return false;
+    // more rounds of the chip than a few: a stream
+    const long long passes = static_cast<long long>(a.n) / (64 / (a.k / 64));
+    return passes <= static_cast<long long>(ctx->prop.multiProcessorCount) * 4 * 8;
+}
+
+int launch_row(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (a.k == 4096) return launch_row_kp<4096, 8, 1>(ctx, a);
+    // two rows a pass at this width: one pass a wave up to a block a compute unit's worth of
+    // rows, two above that
+    if (a.n <= 2 * 4 * 2 * ctx->prop.multiProcessorCount) return launch_row_kp<2048, 4, 1>(ctx, a);
+    return launch_row_kp<2048, 4, 2>(ctx, a);
+}
+
 template <int K, int NT, int U>
 int launch_ntu(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw, int t0) {
     if (lds > 48 * 1024) {
@@ -336,12 +495,14 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
     if (a.prologue == SHV_PRO_MUL_SIGMOID)
         SHV_REQUIRE(a.z && a.head_dim >= 0 && (a.head_dim & (a.head_dim - 1)) == 0, "gemv_q4k: sigmoid-gate prologue needs z and a head_dim that is 0 or a power of two (%d)", a.head_dim);
     if (a.z_ring) SHV_REQUIRE(a.prologue == SHV_PRO_GATED_NORM && a.ring_slots > 0, "gemv_q4k: z_ring needs the gated-norm prologue and a ring");
+    SHV_REQUIRE(!a.y_flat || (a.n_tok == 1 && a.ring_slots > 0 && !a.z_ring), "gemv_q4k: y_flat goes with ring output of one row");
     if (a.ring_slots > 0) {
         const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
         SHV_REQUIRE((a.z_ring || (a.ring_stride >= a.n && !a.residual)) && sl <= a.ring_slots && a.n_tok % sl == 0,
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
     if (a.n_tok >= (a.k > 2048 ? ctx->mfma_min_rows_wide : ctx->mfma_min_rows) && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
+    if (row_kernel_covers(ctx, a)) return launch_row(ctx, a);
     switch (a.k) {
         case 512: return launch_k<512>(ctx, a);
         case 1024: return launch_k<1024>(ctx, a);

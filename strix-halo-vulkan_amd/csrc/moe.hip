@@ -214,26 +214,12 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
     __shared__ float red[kRouterGroup][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * 4 + wave) * RW;  // n_expert = the shared-gate row
-    // the wave's router rows are in flight while the first tokens are being normalised, and stay
-    // in registers for every token
-    float4 wrow[RW][H / 256];
-    bool has_row[RW];
-#pragma unroll
-    for (int j = 0; j < RW; j++) {
-        const int row = row0 + j;
-        has_row[j] = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
-        const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
-#pragma unroll
-        for (int i = 0; i < H / 256; i++)
-            wrow[j][i] = has_row[j] ? *reinterpret_cast<const float4 *>(w + (i * 64 + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    float gm[H / kBlock];  // gamma is asked for before the block-wide sums, not after them
-#pragma unroll
-    for (int i = 0; i < H / kBlock; i++) gm[i] = a.gamma ? a.gamma[tid + i * kBlock] : 1.f;
-
     const int t_first = blockIdx.y * tpb;
     const int t_end = t_first + tpb < a.n_tok ? t_first + tpb : a.n_tok;
-    // a group's rows are asked for while the group before it is being multiplied
+    // Loads come back in the order they were asked for: the first tokens' rows and gamma go first
+    // (they come from cache, and the normalising below is over by the time the router rows arrive
+    // instead of queueing behind them); a later group's rows are asked for while the group before
+    // it is being multiplied.
     float v[kRouterGroup][H / kBlock];
     auto fetch = [&](int t0) {
         const int ng = t_end - t0 < kRouterGroup ? t_end - t0 : kRouterGroup;
@@ -246,6 +232,21 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
         }
     };
     fetch(t_first);
+    float gm[H / kBlock];
+#pragma unroll
+    for (int i = 0; i < H / kBlock; i++) gm[i] = a.gamma ? a.gamma[tid + i * kBlock] : 1.f;
+    // the wave's router rows stay in registers for every token
+    float4 wrow[RW][H / 256];
+    bool has_row[RW];
+#pragma unroll
+    for (int j = 0; j < RW; j++) {
+        const int row = row0 + j;
+        has_row[j] = row <= a.n_expert && (row < a.n_expert || a.shared_gate);
+        const float *w = row < a.n_expert ? a.router + static_cast<size_t>(row) * H : a.shared_gate;
+#pragma unroll
+        for (int i = 0; i < H / 256; i++)
+            wrow[j][i] = has_row[j] ? *reinterpret_cast<const float4 *>(w + (i * 64 + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     for (int t0 = t_first; t0 < t_end; t0 += kRouterGroup) {
         const int ng = t_end - t0 < kRouterGroup ? t_end - t0 : kRouterGroup;
         if (a.gamma) {
@@ -428,86 +429,107 @@ __global__ __launch_bounds__(kRouteBlock) void moe_route_block_kernel(shv_moe_ro
     }
 }
 
-// The same selection by a block of 256 threads, two experts a thread (tid and tid + 256), for a
-// kernel that routes its own token before it can ask for its expert's rows: every block of the
-// launch repeats it, side by side.  The probabilities are formed exactly as
-// moe_route_block_kernel forms them (the same partial sums over the same 64 experts, added in
-// the same order).  sel_e [kMaxUsed] / sel_w [kMaxUsed + 1] receive experts, weights and the
-// shared expert's gate; probs is the one-wave road's scratch.  Ends with a block-wide wait.
+// The same selection inside a kernel that routes its own token before it can ask for its expert's
+// rows.  Every block of the launch repeats it, so it is kept short: the block's first 256 threads
+// take two experts each (tid and tid + 256); any further waves only keep the block-wide waits
+// (three) and, like the first four, rank the candidates for themselves at the end, so that no
+// wave waits for another's result.  The probabilities are formed exactly as
+// moe_route_block_kernel forms them (the same partial sums over the same 64 experts, added in the
+// same order).  Candidates are the keys whose LOGIT is at or just below the n_used-th largest of
+// the 16 group maxima (a margin of 1e-4 takes in every key whose probability could round to the
+// threshold's), compacted in expert order.  sel_e [kMaxUsed] / sel_w [kMaxUsed + 1] receive
+// experts, weights and the shared expert's gate; probs is the one-wave road's scratch.  On return
+// every wave can read sel_e / sel_w (each has written the same values there itself).
+constexpr int kCandMax = 64;
+
+// A float's bits as an unsigned integer that orders as the float does.
+__device__ __forceinline__ uint32_t ordered_bits(float v) {
+    const uint32_t b = __float_as_uint(v);
+    return b ^ (static_cast<uint32_t>(static_cast<int32_t>(b) >> 31) | 0x80000000u);
+}
+__device__ __forceinline__ float from_ordered_bits(uint32_t u) {
+    return __uint_as_float(u ^ ((u >> 31) ? 0x80000000u : 0xFFFFFFFFu));
+}
+
+// rank += (key of the lane k to the right in the row of 16, cyclically) > own key
+template <int K>
+__device__ __forceinline__ void count_greater_ror(uint32_t key, int &rank) {
+    const uint32_t o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(key), 0x120 + K, 0xF, 0xF, false));
+    rank += o > key ? 1 : 0;
+}
+
 __device__ __forceinline__ void route_block256(const float *lg, int n_expert, int n_used, bool shared_gate, int32_t *sel_e, float *sel_w, float *probs) {
     __shared__ float s_max[4], s_sum[8];
-    __shared__ uint32_t s_gm[16];
-    __shared__ uint32_t s_thr;
-    __shared__ int s_cnt[8];
-    __shared__ __align__(16) uint32_t cand_p[64];
-    __shared__ __align__(16) int32_t cand_e[64];
-    __shared__ int s_before[4][64];
-    __shared__ int32_t r_e[kMaxUsed];
-    __shared__ float r_w[kMaxUsed];
+    __shared__ __align__(16) float s_gm[16];
+    __shared__ int s_cnt[4];
+    __shared__ __align__(16) unsigned long long cand[kCandMax];  // (probability bits << 32) | (0x7FFFFFFF - expert); 0 = empty
+    __shared__ unsigned long long s_sel[16][kMaxUsed];            // per wave: the selected keys in slot order
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool routing = tid < 256;
     const int e0 = tid, e1 = tid + 256;
-    const bool has0 = e0 < n_expert, has1 = e1 < n_expert;
+    const bool has0 = routing && e0 < n_expert, has1 = routing && e1 < n_expert;
     const float l0 = has0 ? lg[e0] : -INFINITY, l1 = has1 ? lg[e1] : -INFINITY;
-    const float lsh = (tid == 255 && shared_gate) ? lg[n_expert] : 0.f;
-    if (tid < 64) {  // an empty candidate comes before nobody
-        cand_p[tid] = 0u;
-        cand_e[tid] = 0x7FFFFFFF;
-    }
-    float mx = wave_max_all(fmaxf(l0, l1));
-    if (lane == 0) s_max[wave] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
-    const float ex0 = has0 ? expf(l0 - mx) : 0.f, ex1 = has1 ? expf(l1 - mx) : 0.f;
-    const float ws0 = wave_sum_all(ex0), ws1 = wave_sum_all(ex1);
-    if (lane == 0) {
-        s_sum[wave] = ws0;
-        s_sum[4 + wave] = ws1;
-    }
-    if (tid == 0) s_thr = 0u;
-    __syncthreads();
-    float sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < 8; w++) sum += s_sum[w];
-    const float inv = 1.f / sum;
-    const uint32_t kh0 = has0 ? __float_as_uint(ex0 * inv) : 0u, kh1 = has1 ? __float_as_uint(ex1 * inv) : 0u;
-    // 16 groups of 16 threads: n_used of them hold a key at or above the n_used-th largest group maximum
-    uint32_t gm = kh0 > kh1 ? kh0 : kh1;
-    {
-        uint32_t o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppXor1, 0xF, 0xF, false));
-        gm = o > gm ? o : gm;
-        o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppXor2, 0xF, 0xF, false));
-        gm = o > gm ? o : gm;
-        o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppHalfMirror, 0xF, 0xF, false));
-        gm = o > gm ? o : gm;
-        o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(gm), kDppMirror, 0xF, 0xF, false));
-        gm = o > gm ? o : gm;
-    }
-    if ((lane & 15) == 0) s_gm[tid >> 4] = gm;
-    __syncthreads();
-    if (tid < 16) {
-        const uint32_t mine = s_gm[tid];
-        int rank = 0;
-#pragma unroll
-        for (int j = 0; j < 16; j++) rank += (s_gm[j] > mine || (s_gm[j] == mine && j < tid)) ? 1 : 0;
-        if (rank == n_used - 1) s_thr = mine;
+    const float lsh = (lane == 63 && shared_gate) ? lg[n_expert] : 0.f;  // every wave keeps the shared gate for itself
+    const float m = fmaxf(l0, l1);
+    if (routing) {  // the block's maximum and the maxima of 16 groups of 16 threads
+        float gm = m;
+        gm = fmaxf(gm, dpp_f32<kDppXor1>(gm));
+        gm = fmaxf(gm, dpp_f32<kDppXor2>(gm));
+        gm = fmaxf(gm, dpp_f32<kDppHalfMirror>(gm));
+        gm = fmaxf(gm, dpp_f32<kDppMirror>(gm));
+        if ((lane & 15) == 0) s_gm[tid >> 4] = gm;
+        // the wave's maximum from its four rows' (no exchange through LDS)
+        const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 16));
+        const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 48));
+        if (lane == 0) s_max[wave] = fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+        if (wave == 0) cand[lane] = 0ull;
     }
     __syncthreads();
-    const uint32_t thr = s_thr;
-    const bool p0 = has0 && kh0 >= thr, p1 = has1 && kh1 >= thr;
-    const unsigned long long m0 = __ballot(p0), m1 = __ballot(p1);
-    if (lane == 0) {
-        s_cnt[wave] = __popcll(m0);
-        s_cnt[4 + wave] = __popcll(m1);
+    const float mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    unsigned long long m0 = 0ull, m1 = 0ull;
+    float ex0 = 0.f, ex1 = 0.f;
+    bool p0 = false, p1 = false;
+    int n0 = 0;
+    if (routing) {
+        // A lower bound of the n_used-th largest key: the n_used-th largest group maximum.  Every
+        // routing wave finds it for itself: the 16 maxima in the lanes of a row, as integers that
+        // order as the floats do with the group's number in the low four bits (which makes them
+        // distinct and rounds the bound down, never up); a lane's rank is how many of the other
+        // fifteen are greater, counted over the row's rotations.
+        const uint32_t key = (ordered_bits(s_gm[lane & 15]) & ~15u) | static_cast<uint32_t>(15 - (lane & 15));
+        int ra = 0, rb = 0, rc = 0;  // three chains, so that the adds do not wait for one another
+        count_greater_ror<1>(key, ra);  count_greater_ror<2>(key, rb);  count_greater_ror<3>(key, rc);
+        count_greater_ror<4>(key, ra);  count_greater_ror<5>(key, rb);  count_greater_ror<6>(key, rc);
+        count_greater_ror<7>(key, ra);  count_greater_ror<8>(key, rb);  count_greater_ror<9>(key, rc);
+        count_greater_ror<10>(key, ra); count_greater_ror<11>(key, rb); count_greater_ror<12>(key, rc);
+        count_greater_ror<13>(key, ra); count_greater_ror<14>(key, rb); count_greater_ror<15>(key, rc);
+        const int rank = ra + rb + rc;
+        const unsigned long long hit = __ballot(lane < 16 && rank == n_used - 1);
+        float thr_l = -INFINITY;
+        if (hit) thr_l = from_ordered_bits(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key & ~15u), __ffsll(static_cast<long long>(hit)) - 1)));
+        // a margin takes in every key whose probability could round to the threshold's
+        // (a bound of -inf, fewer than n_used groups holding anything, rounds down to a NaN pattern)
+        if (!(thr_l == thr_l)) thr_l = -INFINITY;
+        thr_l -= 1e-4f + 1e-6f * fabsf(thr_l - mx);
+        if (!(thr_l == thr_l)) thr_l = -INFINITY;
+        ex0 = has0 ? expf(l0 - mx) : 0.f;
+        ex1 = has1 ? expf(l1 - mx) : 0.f;
+        const float ws0 = wave_sum_all(ex0), ws1 = wave_sum_all(ex1);
+        p0 = has0 && l0 >= thr_l;
+        p1 = has1 && l1 >= thr_l;
+        m0 = __ballot(p0);
+        m1 = __ballot(p1);
+        n0 = __popcll(m0);
+        if (lane == 0) {
+            s_sum[wave] = ws0;
+            s_sum[4 + wave] = ws1;
+            s_cnt[wave] = n0 + __popcll(m1);
+        }
     }
     __syncthreads();
-    int before0 = 0, before1 = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < 8; w++) {
-        before0 += w < wave ? s_cnt[w] : 0;
-        before1 += w < 4 + wave ? s_cnt[w] : 0;
-        total += s_cnt[w];
-    }
-    if (total > 64 || n_expert < 64 || n_used > 16) {
+    const int c0 = s_cnt[0], c1 = s_cnt[1], c2 = s_cnt[2], c3 = s_cnt[3];
+    const int total = c0 + c1 + c2 + c3;
+    if (total > kCandMax || total < n_used || n_expert < 64 || n_used > 16) {
         // uniform over the block: many equal probabilities, or a shape the threshold does not cover
         if (wave == 0) {
             route_token<8, false>(lg, n_expert, n_used, sel_e, sel_w, probs);
@@ -516,54 +538,62 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
         __syncthreads();
         return;
     }
-    if (p0) {
-        const int pos = before0 + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m0 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m0), 0u)));
-        cand_p[pos] = kh0;
-        cand_e[pos] = e0;
-    }
-    if (p1) {
-        const int pos = before1 + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m1 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m1), 0u)));
-        cand_p[pos] = kh1;
-        cand_e[pos] = e1;
-    }
-    if (tid == 255) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh) : 0.f;
-    __syncthreads();
-    // rank of candidate i = how many candidates come before it: the four waves each compare it
-    // with a quarter of the table
-    const uint32_t my_p = cand_p[lane];
-    const int my_e = cand_e[lane];
-    {
-        int before = 0;
+    if (routing) {
+        float sum = 0.f;
 #pragma unroll
-        for (int j4 = 0; j4 < 4; j4++) {
-            const uint4 pj = *reinterpret_cast<const uint4 *>(&cand_p[wave * 16 + j4 * 4]);
-            const int4 ej = *reinterpret_cast<const int4 *>(&cand_e[wave * 16 + j4 * 4]);
-            before += (pj.x > my_p || (pj.x == my_p && ej.x < my_e)) ? 1 : 0;
-            before += (pj.y > my_p || (pj.y == my_p && ej.y < my_e)) ? 1 : 0;
-            before += (pj.z > my_p || (pj.z == my_p && ej.z < my_e)) ? 1 : 0;
-            before += (pj.w > my_p || (pj.w == my_p && ej.w < my_e)) ? 1 : 0;
+        for (int w = 0; w < 8; w++) sum += s_sum[w];
+        const float inv = 1.f / sum;
+        // the table's order does not matter to the ranks: each wave writes its candidates after
+        // those of the waves before it
+        const int before = (wave > 0 ? c0 : 0) + (wave > 1 ? c1 : 0) + (wave > 2 ? c2 : 0);
+        if (p0) {
+            const int pos = before + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m0 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m0), 0u)));
+            cand[pos] = (static_cast<unsigned long long>(__float_as_uint(ex0 * inv)) << 32) | static_cast<uint32_t>(0x7FFFFFFF - e0);
         }
-        s_before[wave][lane] = before;
-    }
-    __syncthreads();
-    if (wave == 0) {
-        const int rank = (s_before[0][lane] + s_before[1][lane]) + (s_before[2][lane] + s_before[3][lane]);
-        if (lane < total && rank < n_used) {
-            r_e[rank] = my_e;
-            r_w[rank] = __uint_as_float(my_p);
-        }
-        __builtin_amdgcn_wave_barrier();
-        const float w_mine = lane < n_used ? r_w[lane] : 0.f;
-        const int32_t e_mine = lane < n_used ? r_e[lane] : 0;
-        float wsum = 0.f;
-        for (int k = 0; k < n_used; k++) wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_mine), k));
-        if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
-        if (lane < n_used) {
-            sel_e[lane] = e_mine;
-            sel_w[lane] = w_mine / wsum;
+        if (p1) {
+            const int pos = before + n0 + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m1 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m1), 0u)));
+            cand[pos] = (static_cast<unsigned long long>(__float_as_uint(ex1 * inv)) << 32) | static_cast<uint32_t>(0x7FFFFFFF - e1);
         }
     }
     __syncthreads();
+    // every wave: lane i owns table entry i; its rank is how many entries are larger (the keys are
+    // distinct: the expert is part of them; empty entries are 0 and larger than nothing).  The
+    // table is read in two halves, every read of a half in flight together.
+    const unsigned long long mine = cand[lane];
+    int r4[4] = {0, 0, 0, 0};  // four chains of counts
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        if (half * (kCandMax / 2) >= total) break;
+        ulonglong2 o[kCandMax / 4];
+#pragma unroll
+        for (int j2 = 0; j2 < kCandMax / 4; j2++) o[j2] = *reinterpret_cast<const ulonglong2 *>(&cand[half * (kCandMax / 2) + 2 * j2]);
+#pragma unroll
+        for (int j2 = 0; j2 < kCandMax / 4; j2++) {
+            r4[(2 * j2) & 3] += o[j2].x > mine ? 1 : 0;
+            r4[(2 * j2 + 1) & 3] += o[j2].y > mine ? 1 : 0;
+        }
+    }
+    const int rank = (r4[0] + r4[1]) + (r4[2] + r4[3]);
+    // slot k's key goes to lane k through the wave's own table, then the sum over the slots in
+    // order, in float32: the reference's sum
+    if (mine != 0ull && rank < n_used) s_sel[wave][rank] = mine;
+    __builtin_amdgcn_wave_barrier();
+    const unsigned long long sk = lane < n_used ? s_sel[wave][lane] : 0ull;
+    const float w_k = __uint_as_float(static_cast<uint32_t>(sk >> 32));
+    const int e_k = 0x7FFFFFFF - static_cast<int>(static_cast<uint32_t>(sk));
+    float wsum = 0.f;
+#pragma unroll
+    for (int k = 0; k < kMaxUsed; k++) {
+        if (k >= n_used) break;
+        wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_k), k));
+    }
+    if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
+    if (lane < n_used) {
+        sel_e[lane] = e_k;
+        sel_w[lane] = w_k / wsum;
+    }
+    if (lane == 63) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh) : 0.f;
+    __builtin_amdgcn_wave_barrier();  // the wave reads what it has written itself (all waves write the same)
 }
 
 // ------------------------------------------------------------------------------- up ----------
@@ -576,7 +606,10 @@ template <int K, int P>
 __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int slot0) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
-    __shared__ float xs[lds_padded(K)];
+    constexpr int NV = K / 4 / kBlock;
+    static_assert(NV >= 1 || K == 512, "a thread stages whole float4s");
+    __shared__ __align__(16) float xs[lds_padded(K)];
+    __shared__ __align__(16) float xsum[K / 32];
     __shared__ __align__(16) float probs[192];
     __shared__ int32_t s_topk[kMaxUsed];
     __shared__ float s_w[kMaxUsed + 1];
@@ -587,14 +620,19 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
 
     // the activation row is requested before anything else and staged further down
     const float *x = a.xn + static_cast<size_t>(t) * K;
-    float xv[K / kBlock];
+    constexpr int NVr = NV >= 1 ? NV : 1;
+    float4 xv[NVr];
 #pragma unroll
-    for (int i = 0; i < K / kBlock; i++) xv[i] = x[tid + i * kBlock];
+    for (int j = 0; j < NVr; j++) {
+        const int c = 4 * (tid + kBlock * j);
+        xv[j] = c < K ? *reinterpret_cast<const float4 *>(x + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 
-    if (a.logits) {
+    // the shared expert's blocks need no selection (the block that stores it is a routed slot's)
+    if (a.logits && slot < a.n_used) {
         // route this block's token from the router's logits, all four waves together
         const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
-        route_block256(lg, a.n_expert, a.n_used, true, s_topk, s_w, probs);
+        route_block256(lg, a.n_expert, a.n_used, a.no_shared_gate == 0, s_topk, s_w, probs);
         if (blockIdx.x == 0 && blockIdx.y == 0) {
             if (tid < a.n_used) a.topk[static_cast<size_t>(t) * a.n_used + tid] = s_topk[tid];
             if (tid <= a.n_used) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + tid] = s_w[tid];
@@ -604,7 +642,9 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
     // the weight loads go out next: they do not depend on the staged vector
     const char *gbase, *ubase;
     if (slot < a.n_used) {
-        const int e = a.logits ? s_topk[slot] : a.topk[static_cast<size_t>(t) * a.n_used + slot];
+        int e;
+        if (a.logits) e = min(max(s_topk[slot], 0), a.n_expert - 1);  // whatever the selection gave, the address stays inside the bank
+        else e = a.topk[static_cast<size_t>(t) * a.n_used + slot];
         gbase = static_cast<const char *>(a.gate_exps) + static_cast<size_t>(e) * a.ffn * ROWB;
         ubase = static_cast<const char *>(a.up_exps) + static_cast<size_t>(e) * a.ffn * ROWB;
     } else {
@@ -619,10 +659,17 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
     }
 
 #pragma unroll
-    for (int i = 0; i < K / kBlock; i++) xs[lds_slot(tid + i * kBlock)] = xv[i];
+    for (int j = 0; j < NVr; j++) {
+        const int c = 4 * (tid + kBlock * j);
+        if (c < K) {
+            *reinterpret_cast<float4 *>(&xs[lds_slot(c)]) = xv[j];
+            const float s8 = sum8_all((xv[j].x + xv[j].y) + (xv[j].z + xv[j].w));
+            if ((lane & 7) == 0) xsum[c >> 5] = s8;
+        }
+    }
     __syncthreads();
     float xr[64], xs_lo, xs_hi;
-    load_x_slice(xs, gi, xr, xs_lo, xs_hi);
+    load_x_slice_presummed(xs, xsum, gi, xr, xs_lo, xs_hi);
     const NibbleConsts nc = nibble_consts();
 #pragma unroll
     for (int p = 0; p < P; p++) {
@@ -773,6 +820,67 @@ __global__ __launch_bounds__(kBlock) void moe_down_kernel(shv_moe_down_args a, i
     }
 }
 
+
+// The down projection of a pass of few tokens (the decode step): a chain of latencies, so every
+// slot gets a wave of its own (a block is n_used+1 waves over P passes of RPP output rows) instead
+// of four waves walking three slots each, the slot's activations are asked for first (loads come
+// back in the order they were issued, and the weights take longest), and the sums of every 32
+// activations the min term needs are made once at staging, not by every lane.  The waves' products
+// are added in slot order by the block's first threads, with the residual.
+// grid: (n_embd / (P * RPP), n_tok), (s_hi - s_lo) * 64 threads.
+template <int K, int P>
+__global__ __launch_bounds__(768) void moe_down_slots_kernel(shv_moe_down_args a, int s_lo, int s_hi) {
+    constexpr int LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES, NV = K / 4 / 64;
+    constexpr int kMaxSlots = 12;
+    __shared__ __align__(16) float xs[kMaxSlots][lds_padded(K)];
+    __shared__ __align__(16) float xsum[kMaxSlots][K / 32];
+    __shared__ float part[kMaxSlots][P * RPP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.y, s = s_lo + wave, ns = a.n_used + 1;
+    const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
+    const int row0 = blockIdx.x * P * RPP + rsub;
+    // this slot's activations, then its expert and weight (scalar loads), then the weights
+    const float *act = a.act + (static_cast<size_t>(t) * ns + s) * K;
+    float4 av[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) av[j] = *reinterpret_cast<const float4 *>(act + 4 * (lane + 64 * j));
+    const char *base = static_cast<const char *>(a.down_sh);
+    if (s < a.n_used) base = static_cast<const char *>(a.down_exps) + static_cast<size_t>(a.topk[static_cast<size_t>(t) * a.n_used + s]) * a.n_embd * ROWB;
+    const float wt = a.weights[static_cast<size_t>(t) * ns + s];
+    Q4kLane w[P];
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        const int row = row0 + p * RPP;
+        w[p].load(base + static_cast<size_t>(row < a.n_embd ? row : 0) * ROWB + sb * SHV_Q4K_BYTES, g);
+    }
+    float res = 0.f;
+    const int out_row = blockIdx.x * P * RPP + tid;
+    if (a.residual && tid < P * RPP && out_row < a.n_embd) res = a.residual[static_cast<size_t>(t) * a.res_stride + out_row];
+    // the wave stages its own slot: no block-wide wait before the products
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = 4 * (lane + 64 * j);
+        *reinterpret_cast<float4 *>(&xs[wave][lds_slot(c)]) = av[j];
+        const float s8 = sum8_all((av[j].x + av[j].y) + (av[j].z + av[j].w));
+        if ((lane & 7) == 0) xsum[wave][c >> 5] = s8;
+    }
+    __builtin_amdgcn_wave_barrier();  // LDS operations of one wave complete in order
+    float xr[64], xs_lo, xs_hi;
+    load_x_slice_presummed(xs[wave], xsum[wave], gi, xr, xs_lo, xs_hi);
+    const NibbleConsts nc = nibble_consts();
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+        float acc = group_sum<LPR>(w[p].dot(g, nc, xr, xs_lo, xs_hi));
+        if (group_sum_owner<LPR>(lane)) part[wave][p * RPP + rsub] = wt * acc;
+    }
+    __syncthreads();
+    if (tid < P * RPP && out_row < a.n_embd) {
+        float v = 0.f;
+        for (int i = 0; i < s_hi - s_lo; i++) v += part[i][tid];  // slot order
+        a.out[static_cast<size_t>(t) * a.out_stride + out_row] = v + res;
+    }
+}
+
 }  // namespace
 
 int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
@@ -897,6 +1005,8 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
         case 512: {
             constexpr int RPP = 64 / (512 / 64);
             if (a.n_tok >= ctx->moe_tall_min) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 8>), dim3((a.n_embd + RPP * 8 - 1) / (RPP * 8), a.n_tok), block, 0, a, s_lo, s_hi);
+            else if (a.n_tok < 8 && a.n_embd % (1 * RPP) == 0 && shv_aligned16(a.act)) SHV_LAUNCH(ctx, (moe_down_slots_kernel<512, 1>),  // the decode step and verification passes
+                dim3(a.n_embd / (1 * RPP), a.n_tok), dim3((s_hi - s_lo) * 64), 0, a, s_lo, s_hi);
             else if (a.n_tok >= 8) SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 4>),  // eight sequences decoded together: 5.31 to 5.19 ms a pass
                 dim3((a.n_embd + RPP * 4 - 1) / (RPP * 4), a.n_tok), block, 0, a, s_lo, s_hi);
             else SHV_LAUNCH(ctx, (moe_down_kernel<512, 12, 1>), dim3((a.n_embd + RPP - 1) / RPP, a.n_tok), block, 0, a, s_lo, s_hi);

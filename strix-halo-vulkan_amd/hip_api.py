@@ -36,7 +36,8 @@ class GemvQ4KArgs(C.Structure):
                 ("n", C.c_int32), ("k", C.c_int32), ("n_tok", C.c_int32), ("prologue", C.c_int32),
                 ("head_dim", C.c_int32), ("eps", C.c_float), ("x_stride", C.c_int32),
                 ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("seq_len", C.c_int32),
-                ("ring_slots", C.c_int32), ("ring_stride", C.c_int32), ("z_ring", C.c_int32)]
+                ("ring_slots", C.c_int32), ("ring_stride", C.c_int32), ("z_ring", C.c_int32),
+                ("y_flat", C.c_void_p)]
 
 
 class DequantQ4KArgs(C.Structure):
@@ -76,7 +77,7 @@ class MoeUpArgs(C.Structure):
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("logits", C.c_void_p),
                 ("weights", C.c_void_p), ("n_expert", C.c_int32), ("gate_type", C.c_int32),
                 ("up_type", C.c_int32), ("gate_sh_type", C.c_int32), ("up_sh_type", C.c_int32),
-                ("group", C.c_void_p)]
+                ("group", C.c_void_p), ("no_shared_gate", C.c_int32)]
 
 
 class MoeDownArgs(C.Structure):

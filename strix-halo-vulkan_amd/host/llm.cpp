@@ -593,6 +593,7 @@ DeltaNetGPU::DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, 
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     attn_ = static_cast<float *>(dev.alloc(T * c_.VWidth() * 4));
+    row_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.DNFusedRows()) * 4));
     ring_.assign(c_.NLayer, nullptr);
     state_.assign(c_.NLayer, nullptr);
     const size_t ring_bytes = static_cast<size_t>(slots) * ring_slots_ * c_.DNFusedRows() * 4;
@@ -655,13 +656,19 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
         throw Error("llm: DeltaNetGPU: a rewindable pass of " + std::to_string(r.seq_len) + " rows needs " + std::to_string(r.seq_len + 1) +
                     " state planes, " + std::to_string(planes_) + " are staged (GraphOpts.Speculative, SpecRows)");
     const int width = c_.DNFusedRows();
+    // A pass of one sequence whose slot is known now: its ring rows, state planes and plane word
+    // are addressed here, and the kernels take no slot table (a dependent load less on their way).
+    const bool own_slot = r.n_seq == 1 && r.host_slot >= 0 && r.host_slot < slots_;
+    const size_t slot_off = own_slot ? static_cast<size_t>(r.host_slot) : 0;
+    const int32_t *slot_tab = own_slot ? nullptr : r.slot;
+    float *ring = ring_[l] + slot_off * ring_slots_ * width;
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor(Model::Blk(l, "ssm_in_fused")).ptr;
     p.x = in;
-    p.y = ring_[l];
+    p.y = ring;
     p.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "attn_norm")).ptr);
     p.pos = r.pos;
-    p.slot = r.slot;
+    p.slot = slot_tab;
     p.n = width;
     p.k = c_.NEmbd;
     p.n_tok = nTok;
@@ -672,18 +679,22 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     p.seq_len = r.seq_len;
     p.ring_slots = ring_slots_;
     p.ring_stride = width;
+    // one row: the projection also leaves the row where the out projection finds its gate
+    // without waiting for the position word
+    const bool flat = nTok == 1;
+    if (flat) p.y_flat = row_;
     shv_dn_step_args s{};
-    s.ring = ring_[l];
+    s.ring = ring;
     s.conv1d = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ssm_conv1d")).ptr);
     s.a = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ssm_a")).ptr);
     s.dt_bias = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ssm_dt")).ptr);
-    s.state = state_[l];
+    s.state = state_[l] + slot_off * planes_ * c_.SSMHeadV * c_.SSMHeadDim * c_.SSMHeadDim;
     s.out = attn_;
     s.pos = r.pos;
-    s.slot = r.slot;
+    s.slot = slot_tab;
     s.n_seq = r.n_seq;
     s.seq_len = r.seq_len;
-    s.plane = plane_;
+    s.plane = plane_ ? plane_ + slot_off : nullptr;
     s.n_planes = planes_;
     s.spec = r.spec ? 1 : 0;
     s.n_head_k = c_.SSMHeadK;
@@ -699,9 +710,6 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     o.y = out;
     o.residual = in;
     o.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ssm_norm")).ptr);
-    o.z = ring_[l] + c_.ConvWidth();  // the z columns of a projection row
-    o.pos = r.pos;
-    o.slot = r.slot;
     o.n = c_.NEmbd;
     o.k = c_.VWidth();
     o.n_tok = nTok;
@@ -710,10 +718,18 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     o.eps = c_.RMSEps;
     o.x_stride = c_.VWidth();
     o.y_stride = c_.NEmbd;
-    o.seq_len = r.seq_len;
-    o.ring_slots = ring_slots_;
-    o.ring_stride = width;
-    o.z_ring = 1;
+    if (flat) {
+        o.z = row_ + c_.ConvWidth();  // the z columns of the projection row
+        o.z_stride = width;
+    } else {
+        o.z = ring + c_.ConvWidth();
+        o.pos = r.pos;
+        o.slot = slot_tab;
+        o.seq_len = r.seq_len;
+        o.ring_slots = ring_slots_;
+        o.ring_stride = width;
+        o.z_ring = 1;
+    }
     if (labels) labels->insert(labels->end(), {"dn.qkv", "dn.step", "dn.out"});
     return {make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_DN_STEP, s), make_op(SHV_OP_GEMV_Q4K, o)};
 }
@@ -872,12 +888,15 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, cons
     a.q_norm = static_cast<const float *>(m_.Tensor(Model::Blk(l, "attn_q_norm")).ptr);
     a.k_norm = static_cast<const float *>(m_.Tensor(Model::Blk(l, "attn_k_norm")).ptr);
     a.rope = rope_;
-    a.kcache = kc_[l];
-    a.vcache = vc_[l];
+    // a pass of one sequence whose slot is known now: its cells are addressed here
+    const bool own_slot = r.n_seq == 1 && r.host_slot >= 0 && r.host_slot < slots_;
+    const size_t slot_bytes = own_slot ? static_cast<size_t>(r.host_slot) * n_kv_ * c_.NHeadKV * c_.HeadDim * 2 : 0;
+    a.kcache = static_cast<char *>(kc_[l]) + slot_bytes;
+    a.vcache = static_cast<char *>(vc_[l]) + slot_bytes;
     a.partial = partial_;
     a.out = ctx_;
     a.pos = r.pos;
-    a.slot = r.slot;
+    a.slot = own_slot ? nullptr : r.slot;
     a.n_seq = r.n_seq;
     a.seq_len = r.seq_len;
     a.n_head = c_.NHead;
@@ -1094,6 +1113,7 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     } else {
         r.pos = pos_ + slot;
         r.slot = slot_ix_ + slot;
+        r.host_slot = slot;
         r.n_seq = 1;
         r.seq_len = rows;
         e.ids = ids_ + slot * ids_stride_;
@@ -1600,6 +1620,7 @@ int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos,
         PassRows r;
         r.pos = pos_ + slot_;
         r.slot = slot_ix_ + slot_;
+        r.host_slot = slot_;
         r.seq_len = n;
         auto a = attn_->Dispatches(layer_, x_, x_, r, &p.labels);
         p.ops.insert(p.ops.end(), a.begin(), a.end());

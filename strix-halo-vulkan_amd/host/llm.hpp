@@ -176,6 +176,9 @@ struct Stage {
 struct PassRows {
     const int32_t *pos = nullptr;
     const int32_t *slot = nullptr;  // nullptr: sequence s is slot s
+    int host_slot = -1;             // a pass of one sequence whose slot the host knows when it records the pass: the
+                                    // blocks then offset their per-slot memory themselves and the kernels are spared
+                                    // a dependent load of the slot word
     int n_seq = 1, seq_len = 1;
     bool spec = false;              // DeltaNet: a rewindable pass (state goes to the other planes)
     int rows() const { return n_seq * seq_len; }
@@ -260,6 +263,7 @@ private:
     int max_tok_, slots_, planes_, ring_slots_, n_tok_ = 0;
     int32_t *pos_, *plane_;
     float *in_, *out_, *attn_;
+    float *row_ = nullptr;               // the projection row of a one-row pass, also kept outside the ring (the out projection's gate)
     std::vector<float *> ring_, state_;  // per layer (nullptr on attention layers)
     uint64_t state_bytes_ = 0;
 };

@@ -210,11 +210,12 @@ def test_moe_refuses_unsupported_shapes(ctx):
                                                  2048, 10, 640, 2048, 2048))
 
 
-def test_moe_full_config_bank(ctx):
+@pytest.fixture(scope="module")
+def full_bank(ctx):
     """BASELINE shape: 512 experts, top-10, ffn 512, H 2048.  The 906 MB bank is drawn and quantised
-    on the device (the device quantiser is bit-exact with the reference's), downloaded, and the
-    oracle runs on the same bytes."""
-    H, E, used, ffn, T = 2048, 512, 10, 512, 4
+    on the device (the device quantiser is bit-exact with the reference's) and downloaded once, so
+    that the oracle runs on the same bytes."""
+    H, E, used, ffn = 2048, 512, 10, 512
     c = ctx
     rng = np.random.default_rng(77)
 
@@ -228,17 +229,86 @@ def test_moe_full_config_bank(ctx):
         return q
 
     case = MoeCase.__new__(MoeCase)
-    case.ctx, case.H, case.E, case.used, case.ffn, case.T = c, H, E, used, ffn, T
+    case.ctx, case.H, case.E, case.used, case.ffn = c, H, E, used, ffn
+    case.types = [0] * 6
     dev = dict(gate_exps=bank(E * ffn, H, 1), up_exps=bank(E * ffn, H, 2), down_exps=bank(E * H, ffn, 3))
     for k, b in dev.items():
         setattr(case, k, b.read(np.uint8, b.nbytes))
+    for b in dev.values():
+        b.free()
     case.router = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
     case.shared_gate = (rng.standard_normal(H) * 0.02).astype(np.float32)
     q = lambda rows, k: O.quantize_q4k((rng.standard_normal((rows, k)) * 0.02).astype(np.float32))
     case.gate_sh, case.up_sh, case.down_sh = q(ffn, H), q(ffn, H), q(H, ffn)
     case.gamma = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
-    case.h = rng.standard_normal((T, H)).astype(np.float32)
-    case.res = rng.standard_normal((T, H)).astype(np.float32)
-    for b in dev.values():
-        b.free()
-    _check(case, residual=True, defer=True)
+    return case
+
+
+def _full_case(full_bank, T, seed):
+    """The bank with T token rows of its own; a seed whose rows sit on a near-tie is stepped past."""
+    import copy
+    case = copy.copy(full_bank)
+    case.T = T
+    for s in range(seed, seed + 50):
+        rng = np.random.default_rng(s)
+        case.h = rng.standard_normal((T, case.H)).astype(np.float32)
+        case.res = rng.standard_normal((T, case.H)).astype(np.float32)
+        xn = case.h * (1.0 / np.sqrt((case.h.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + EPS)) * case.gamma
+        lg = xn.astype(np.float64) @ case.router.astype(np.float64).T
+        p = np.exp(lg - lg.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+        if all(_margin(p[t], case.used) > 2e-4 for t in range(T)):
+            return case
+    raise AssertionError("no seed clear of near-ties")
+
+
+@pytest.mark.parametrize("defer", [False, True])
+@pytest.mark.parametrize("T", [1, 4, 16])
+def test_moe_full_config_bank(ctx, full_bank, T, defer):
+    """BASELINE config 2 at its three batch sizes over the full 512-expert bank, with the selection
+    made by the routing launch (the block-wide routing kernel that every pass of several rows at
+    this shape takes) and by the expert kernel from the logits."""
+    _check(_full_case(full_bank, T, 1000 + T), residual=True, defer=defer)
+
+
+@pytest.mark.parametrize("defer", [False, True])
+def test_route_with_many_equal_probabilities_at_512_experts(ctx, full_bank, defer):
+    """More than 64 experts share the largest probability: the candidates do not fit the ranking
+    table and the selection falls back to rounds of arg-max; ties still go to the lower index
+    (sort.SliceStable, llm/moe.go:249-252)."""
+    import copy
+    case = copy.copy(full_bank)
+    case.T = 2
+    rng = np.random.default_rng(5)
+    case.h = rng.standard_normal((2, case.H)).astype(np.float32)
+    case.res = rng.standard_normal((2, case.H)).astype(np.float32)
+    case.router = case.router.copy()
+    tied = np.arange(37, 37 + 150)
+    case.router[tied] = case.router[300]          # 151 equal logits ...
+    case.router[[3, 490]] = 4.0 * case.router[300]  # ... and two rows that may or may not lie above them
+    want, got = case.oracle(), case.gpu(residual=True, defer=defer)
+    assert np.array_equal(got["topk"], want["topk"])
+    assert O.rel_l2(got["weights"][:, :case.used], want["weights"]) <= 1e-5
+    assert O.rel_l2(got["out"], want["out"] + case.res) <= TOL
+
+
+def test_expert_kernel_routing_without_a_shared_gate(ctx, full_bank):
+    """A router run without a shared gate leaves its logit unwritten; the expert kernel, told so,
+    stores 0 for the shared expert's weight, as the routing launch does."""
+    case = _full_case(full_bank, 1, 2000)
+    c, T, H, E, used, ffn = ctx, 1, case.H, case.E, case.used, case.ffn
+    d = {k: c.upload(getattr(case, k)) for k in ("router", "gate_exps", "up_exps", "gate_sh", "up_sh", "gamma", "h")}
+    xn, logits = c.alloc(T * H * 4), c.upload(np.full(T * (E + 1), 77.0, np.float32))
+    topk, weights = c.alloc(T * used * 4), c.upload(np.full(T * (used + 1), 5.0, np.float32))
+    act = c.alloc(T * (used + 1) * ffn * 4)
+    out = {}
+    for defer in (0, 1):
+        ra = A.MoeRouterArgs(d["h"].ptr, d["gamma"].ptr, d["router"].ptr, None, xn.ptr, logits.ptr, topk.ptr, weights.ptr,
+                             T, H, E, used, EPS, H, defer)
+        ua = A.MoeUpArgs(xn.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr, d["up_sh"].ptr, act.ptr,
+                         T, H, used, ffn, logits.ptr if defer else None, weights.ptr if defer else None, E, 0, 0, 0, 0, None, 1)
+        c.dispatch_multi([A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua)])
+        out[defer] = (topk.read(np.int32, used), weights.read(np.float32, used + 1))
+    assert np.array_equal(out[0][0], out[1][0])
+    assert out[0][1][used] == 0.0 and out[1][1][used] == 0.0
+    assert np.allclose(out[0][1], out[1][1], rtol=1e-6)
