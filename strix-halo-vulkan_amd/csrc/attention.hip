@@ -36,10 +36,38 @@ constexpr int kSliceCells = 128;  // cells a slice gets while there are slices t
 constexpr int kMaxSplits = 512;
 constexpr int kRec = kRep * (kD + 2);  // floats of one (slice, row) record: per head d values, max, sum
 
-// RMS norm over the 256 dims of one head by one wave (4 dims per lane), then NeoX rotary on the
-// first rope_dims dims through LDS.  dst is 256 floats of LDS.  The head's values, gamma and the
-// rotary factors of lane < rope_dims/2 (cs, sn) are in registers already: a caller asks for
-// everything it will need before it waits for any of it.
+// RMS norm over the 256 dims of one head by one wave (4 dims per lane: lane l holds dims 4l..4l+3),
+// then NeoX rotary on the first rope_dims dims, all in registers: dims i and i + rope_dims/2 turn
+// together and sit rope_dims/8 lanes apart, which the launcher requires to be a power of two, so
+// the partner is lane ^ (rope_dims/8).  cs4 / sn4: the rotary factors of this lane's four dims,
+// i.e. entries 4*(lane mod rope_dims/8) .. +3 of the position's cos and sin rows.
+__device__ __forceinline__ float rope_turn(float x, float o, float c, float sn, bool first, bool turns) {
+    // first of the pair: x0' = x0*cos - x1*sin ; second: x1' = x0*sin + x1*cos  (o is the partner's value)
+    const float r = first ? x * c - o * sn : o * sn + x * c;
+    return turns ? r : x;
+}
+
+__device__ __forceinline__ void norm_rope_regs(const float4 v, const float4 g, const float4 cs4, const float4 sn4, int rope_dims, float eps, int lane,
+                                               float &x0, float &x1, float &x2, float &x3) {
+    const float ss = wave_sum_all(fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w))));
+    const float sc = __builtin_amdgcn_rsqf(ss / static_cast<float>(kD) + eps);
+    x0 = v.x * sc * g.x;
+    x1 = v.y * sc * g.y;
+    x2 = v.z * sc * g.z;
+    x3 = v.w * sc * g.w;
+    const int step = rope_dims >> 3;  // lanes between the two dims of a pair
+    if (step > 0) {
+        const float o0 = __shfl_xor(x0, step, 64), o1 = __shfl_xor(x1, step, 64), o2 = __shfl_xor(x2, step, 64), o3 = __shfl_xor(x3, step, 64);
+        const bool first = (lane & step) == 0;  // holds the pair's first dim
+        const bool turns = lane < 2 * step;     // inside the rotated dims
+        x0 = rope_turn(x0, o0, cs4.x, sn4.x, first, turns);
+        x1 = rope_turn(x1, o1, cs4.y, sn4.y, first, turns);
+        x2 = rope_turn(x2, o2, cs4.z, sn4.z, first, turns);
+        x3 = rope_turn(x3, o3, cs4.w, sn4.w, first, turns);
+    }
+}
+
+// The same through LDS, for the kernel that only appends cells (dst is 256 floats of LDS).
 __device__ __forceinline__ void norm_rope_loaded(const float4 v, const float4 g, float cs, float sn, int rope_dims, float eps,
                                                  float *dst, int lane) {
     const float ss = wave_sum_all(fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w))));
@@ -83,6 +111,12 @@ __device__ __forceinline__ void split4(const float *x, half4_t &h, half4_t &l) {
     }
 }
 
+__device__ __forceinline__ void split1(float x, half4_t &h, half4_t &l, int t) {
+    const _Float16 hi = static_cast<_Float16>(x);
+    h[t] = hi;
+    l[t] = static_cast<_Float16>(x - static_cast<float>(hi));
+}
+
 // LDS of one block.  The queries are kept as matrix-core operands: entry [i][h][part][lane] is the
 // four dims 8*(kb + 4*i) + 4*h .. +3 of query row lane%16 (kb = lane/16), as hi or lo halves.
 struct Smem {
@@ -90,7 +124,6 @@ struct Smem {
     float big[4][kRep][kD];        // 32 KB: queries in float32 first; later the waves' accumulators of one row
     float al[4][16];               // per wave: the factor each query row's running sums shrink by
     float wm[4][16], wl[4][16];    // per wave: running max and sum of each query row
-    float kv_tmp[2][kD];
 };
 
 // grid: (n_splits, n_head_kv, n_seq * n_groups); group g of a sequence is its rows row0 + R*g ..
@@ -99,7 +132,7 @@ struct Smem {
 // and any number of groups go in one launch, each masked to its own positions.  Query row r of the
 // tile is head r%8 of sequence row r/8; with R = 1 rows 8..15 are padding.
 template <int R>
-__global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_args a, int row00, int n_groups, int append) {
+__global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_args a, int row00, int n_groups, int append, int slice_cells) {
     __shared__ Smem sm;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // the groups of a pass run over blockIdx.x, the fastest-varying index: the blocks that read one
@@ -116,17 +149,25 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
     const int tid_ = threadIdx.x, lane_ = tid_ & 63, wave_ = tid_ >> 6;
     const int valid_ = a.seq_len - row0 < R ? a.seq_len - row0 : R;
     const float *qkv0 = a.qkv + static_cast<size_t>(seq * a.seq_len + row0) * a.qkv_stride;
-    float4 qv[R][2], kv[R];
+    // Which of the KV head's 8 query heads this wave prepares.  A slice of one tile (a decode
+    // step: slices are made small so that many compute units pull the cache, each at the rate one
+    // unit issues loads) is loaded by the first wave alone, which prepares nothing; the other
+    // three share the heads 3, 3 and 2 and the last appends.  Otherwise every wave takes two heads
+    // and its own tiles.
+    const bool single = slice_cells <= kTile;
+    const int h0 = single ? 3 * (wave_ - 1) : 2 * wave_;
+    const int nh = single ? (wave_ == 0 ? 0 : wave_ == 3 ? 2 : 3) : 2;
+    float4 qv[R][3], kv[R];
     float vv[R];
 #pragma unroll
     for (int j = 0; j < R; j++) {
         const int jr = j < valid_ ? j : valid_ - 1;
         const float *qkv = qkv0 + static_cast<size_t>(jr) * a.qkv_stride;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
-            qv[j][i] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(kvh * kRep + wave_ * 2 + i) * 2 * kD + 4 * lane_);
-        // every wave asks for the row's k (one of them will append it): straight-line code, so that
-        // the compiler's count of outstanding loads stays exact and nothing waits for the tile early
+        for (int i = 0; i < 3; i++) {
+            const int hh = min(max(h0 + i, 0), kRep - 1);  // a head it will not use is asked for all the same: no branch around loads
+            qv[j][i] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(kvh * kRep + hh) * 2 * kD + 4 * lane_);
+        }
         kv[j] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD + 4 * lane_);
         vv[j] = qkv[static_cast<size_t>(a.n_head) * 2 * kD + a.n_head_kv * kD + kvh * kD + tid_];
     }
@@ -138,7 +179,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
     const int n_cells = p_first + valid;                   // cells the last row sees
     // The grid is sized for the cache's capacity; how many of its slices take part depends on how
     // many cells the sequence holds now: about kSliceCells a slice while there are slices to spare.
-    int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
+    int n_active = (n_cells + slice_cells - 1) / slice_cells;
     if (n_active > a.n_splits) n_active = a.n_splits;
     if (split >= n_active) return;
     int cps = (n_cells + n_active - 1) / n_active;
@@ -180,12 +221,12 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
         for (int db = 0; db < 16; db++)
             vreg[db] = *reinterpret_cast<const uint4 *>(vt + static_cast<size_t>(t0 / kTile) * vtile + (16 * db + n) * kTile + 8 * q);
     };
-    // ---- prologue: queries (float32, into sm.big), new cells.  The rows' values were asked for at
-    //      the top; the rotary factors (whose row the position names) and the wave's first tile of
-    //      the cache go out together now ----
-    float *qtmp = &sm.big[0][0][0];  // [8*R][kD]
-    const int half_rope = a.rope_dims / 2;
-    float cs[R], sn[R];
+    // ---- prologue: queries, new cells.  The rows' values were asked for at the top; the rotary
+    //      factors (whose row the position names) and the wave's first tile of the cache go out
+    //      together now.  Norms and rotation stay in registers and every wave writes its heads'
+    //      queries straight into the operand table, so there is one block-wide wait ----
+    const int rstep = a.rope_dims >> 3;
+    float4 cs4[R], sn4[R];
     bool app[R];
 #pragma unroll
     for (int j = 0; j < R; j++) {
@@ -193,59 +234,73 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
         const int p = p_first + jr;
         const float *rope_row = a.rope_dims > 0 ? a.rope + static_cast<size_t>(p) * a.rope_dims : a.q_norm;  // no rotary: any readable words
         app[j] = append && p >= c0 && p < c1;  // the new cell of row j lies in this slice
-        const int rl = lane < half_rope ? lane : 0;  // a select, not a branch around the loads
-        cs[j] = rope_row[rl];
-        sn[j] = rope_row[half_rope + rl];
+        const int rl = rstep > 0 ? 4 * (lane & (rstep - 1)) : 0;
+        cs4[j] = *reinterpret_cast<const float4 *>(rope_row + rl);
+        sn4[j] = *reinterpret_cast<const float4 *>(rope_row + (a.rope_dims >> 1) + rl);
     }
-    // the wave's first tile, unless this launch is about to append cells inside it
-    // (asked for by every wave, without a branch around the loads, so that the compiler's count of
-    // outstanding loads stays exact and the norms below wait for their own inputs only, not for the
-    // tile: a wave with no tile of its own in a short slice asks for the slice's first one)
+    // the wave's first tile, unless this launch is about to append cells inside it.  (After this
+    // branch the compiler no longer knows how many loads are in flight and waits for all of them
+    // where it needs an earlier one: a wave that has both a tile and heads to prepare waits for
+    // the tile before it prepares them.  In a slice of one tile no wave has both.)
     const int t_first = c0 + kTile * wave;
     const bool early = t_first < c1 && t_first + kTile <= p_first;
-    load_tile(ta, t_first < c1 ? t_first : c0);
+    if (early) load_tile(ta, t_first);
 
+    // operand table entry [i][h][part][16*kb + row] holds dims 8*(kb + 4*i) + 4*h .. +3 of query row
+    // `row`: lane l's four dims 4l..4l+3 are h = l&1, kb = (l>>1)&3, i = l>>3
+    const float scale = 1.f / sqrtf(static_cast<float>(kD));
+    const int op_h = lane & 1, op_kb = (lane >> 1) & 3, op_i = lane >> 3;
 #pragma unroll
     for (int j = 0; j < R; j++) {
         const int jr = j < valid ? j : valid - 1;
         const int p = p_first + jr;
-        if (nc > 0) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-                norm_rope_loaded(qv[j][i], gq, cs[j], sn[j], a.rope_dims, a.eps, qtmp + (8 * j + wave * 2 + i) * kD, lane);
+        for (int i = 0; i < 3; i++) {
+            if (i >= nh) break;
+            float q0, q1, q2, q3;
+            norm_rope_regs(qv[j][i], gq, cs4[j], sn4[j], a.rope_dims, a.eps, lane, q0, q1, q2, q3);
+            half4_t hi, lo;
+            split1(q0 * scale, hi, lo, 0);
+            split1(q1 * scale, hi, lo, 1);
+            split1(q2 * scale, hi, lo, 2);
+            split1(q3 * scale, hi, lo, 3);
+            const int row = 8 * j + h0 + i;
+            sm.qf[op_i][op_h][0][16 * op_kb + row] = hi;
+            sm.qf[op_i][op_h][1][16 * op_kb + row] = lo;
         }
         if (app[j]) {
             // one wave appends the new cell's K, all threads its V
-            if (wave == ((2 * j) & 3)) {
-                norm_rope_loaded(kv[j], gk, cs[j], sn[j], a.rope_dims, a.eps, sm.kv_tmp[j], lane);
-                uint16_t *dst = kc + static_cast<size_t>(p) * kvw;
-#pragma unroll
-                for (int i = 0; i < 4; i++) dst[4 * lane + i] = __half_as_ushort(__float2half_rn(sm.kv_tmp[j][4 * lane + i]));
+            if (wave == (single ? 3 : ((2 * j) & 3))) {
+                float k0, k1, k2, k3;
+                norm_rope_regs(kv[j], gk, cs4[j], sn4[j], a.rope_dims, a.eps, lane, k0, k1, k2, k3);
+                const __half2 k01 = __floats2half2_rn(k0, k1), k23 = __floats2half2_rn(k2, k3);
+                uint2 packed;
+                packed.x = *reinterpret_cast<const uint32_t *>(&k01);
+                packed.y = *reinterpret_cast<const uint32_t *>(&k23);
+                *reinterpret_cast<uint2 *>(kc + static_cast<size_t>(p) * kvw + 4 * lane) = packed;
             }
             vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vv[j]));
         }
     }
-    __threadfence_block();
-    __syncthreads();
-    if (nc > 0) {
-        // queries as operands: 8*2*64 entries, four a thread; the score scale goes in here
-        const float scale = 1.f / sqrtf(static_cast<float>(kD));
+    if (R == 1) {
+        // rows 8..15 of the tile are padding: zero operands (entries of lane ln with ln%16 >= 8)
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const int idx = tid + e * kBlock;  // [i][h][lane]
+            const int idx = tid + e * kBlock;  // [i][h][ln]
             const int ln = idx & 63, h = (idx >> 6) & 1, i = idx >> 7;
-            const int row = ln & 15, kb = ln >> 4;
-            float x[4] = {0.f, 0.f, 0.f, 0.f};
-            if (row < 8 * R) {
-                const float4 f = *reinterpret_cast<const float4 *>(qtmp + row * kD + 8 * (kb + 4 * i) + 4 * h);
-                x[0] = f.x * scale; x[1] = f.y * scale; x[2] = f.z * scale; x[3] = f.w * scale;
+            if ((ln & 15) >= 8) {
+                sm.qf[i][h][0][ln] = half4_t{0, 0, 0, 0};
+                sm.qf[i][h][1][ln] = half4_t{0, 0, 0, 0};
             }
-            half4_t hi, lo;
-            split4(x, hi, lo);
-            sm.qf[i][h][0][ln] = hi;
-            sm.qf[i][h][1][ln] = lo;
         }
     }
+    // Only a block that appended cells reads its own stores back (its waves' tiles are asked for
+    // again after the wait).  The fence would also wait for every load in flight, i.e. for the
+    // first tile, before the block-wide wait instead of after it: the other blocks skip it.
+    bool appended = false;
+#pragma unroll
+    for (int j = 0; j < R; j++) appended = appended || app[j];
+    if (appended) __threadfence_block();
     __syncthreads();
 
     // per lane: O[row 4q+i][dim 16*db + n] for the 16 dim blocks; the running max and sum of query
@@ -405,7 +460,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_decode_kernel(shv_attn_decode_
 // one for a pass of many row pairs, which takes few slices a pair and would launch eight times the waves for nothing.
 constexpr int kMergeWaves = 8;
 template <int R, int NW>
-__global__ __launch_bounds__(64 * NW) void attn_merge_kernel(shv_attn_decode_args a, int row00, int n_groups) {
+__global__ __launch_bounds__(64 * NW) void attn_merge_kernel(shv_attn_decode_args a, int row00, int n_groups, int slice_cells) {
     __shared__ float red[3][NW][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int head = blockIdx.x >> 2, d = (blockIdx.x & 3) * 64 + lane, j = blockIdx.y;
@@ -414,7 +469,7 @@ __global__ __launch_bounds__(64 * NW) void attn_merge_kernel(shv_attn_decode_arg
     if (row0 + j >= a.seq_len) return;  // the thrown-away second row of a last group of one
     const int valid = a.seq_len - row0 < R ? a.seq_len - row0 : R;
     const int n_cells = (a.pos ? a.pos[seq] : 0) + row0 + valid;
-    int n_active = (n_cells + kSliceCells - 1) / kSliceCells;
+    int n_active = (n_cells + slice_cells - 1) / slice_cells;
     if (n_active > a.n_splits) n_active = a.n_splits;
     const float *pin = a.partial + (static_cast<size_t>(blockIdx.z) * a.n_head_kv + kvh) * a.n_splits * R * kRec + j * kRec + hh * (kD + 2);
     constexpr int MB = 16;
@@ -492,10 +547,14 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
     const int lanes = a.n_seq * n_groups * a.n_head_kv;
     const int want = (2 * ctx->prop.multiProcessorCount + lanes - 1) / lanes;
     if (b.n_splits > want) b.n_splits = want < 1 ? 1 : want;
+    // one row pair: slices of one tile while there are slices to spare, so that as many compute
+    // units as possible pull the cache (a unit issues a wave's 16-byte loads at about 25 B a clock;
+    // 36 units over 2 300 cells took 2.2 us to ask for them, 144 take a quarter of that)
+    const int slice_cells = a.n_seq * n_groups == 1 ? kTile : kSliceCells;
     dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
-    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append);
-    if (a.n_seq * n_groups >= 8 && b.n_splits <= 16) SHV_LAUNCH(ctx, (attn_merge_kernel<R, 1>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64), 0, b, row0, n_groups);
-    else SHV_LAUNCH(ctx, (attn_merge_kernel<R, kMergeWaves>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, b, row0, n_groups);
+    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
+    if (a.n_seq * n_groups >= 8 && b.n_splits <= 16) SHV_LAUNCH(ctx, (attn_merge_kernel<R, 1>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64), 0, b, row0, n_groups, slice_cells);
+    else SHV_LAUNCH(ctx, (attn_merge_kernel<R, kMergeWaves>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, b, row0, n_groups, slice_cells);
     return SHV_OK;
 }
 
@@ -507,7 +566,9 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
     SHV_REQUIRE(a.head_dim == kD, "attn_decode: head_dim %d; built for %d", a.head_dim, kD);
     SHV_REQUIRE(a.n_head_kv >= 1 && a.n_head == a.n_head_kv * kRep, "attn_decode: %d query heads over %d KV heads; built for %d per KV head",
                 a.n_head, a.n_head_kv, kRep);
-    SHV_REQUIRE(a.rope_dims >= 0 && a.rope_dims <= 128 && a.rope_dims % 2 == 0, "attn_decode: rope_dims %d", a.rope_dims);
+    SHV_REQUIRE(a.rope_dims >= 0 && a.rope_dims <= 128 && (a.rope_dims == 0 || (a.rope_dims >= 8 && (a.rope_dims & (a.rope_dims - 1)) == 0)),
+                "attn_decode: rope_dims %d; 0 or a power of two from 8 to 128 (the rotation pairs dims rope_dims/8 lanes apart)", a.rope_dims);
+    SHV_REQUIRE(shv_aligned16(a.rope), "attn_decode: the rotary table must be 16-byte aligned");
     SHV_REQUIRE(a.n_seq >= 1 && a.seq_len >= 1, "attn_decode: %d sequences of %d rows", a.n_seq, a.seq_len);
     SHV_REQUIRE(a.n_seq <= 65535, "attn_decode: %d sequences", a.n_seq);
     SHV_REQUIRE(a.n_splits >= 1 && a.n_splits <= kMaxSplits, "attn_decode: %d slices; 1..%d", a.n_splits, kMaxSplits);

@@ -320,7 +320,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
             if (span >= 16) hs += dpp_f32<kDppMirror>(hs);
             if (span >= 32) hs += __shfl_xor(hs, 16, 64);
             if (span >= 64) hs += __shfl_xor(hs, 32, 64);
-            const float sc = 1.f / sqrtf(hs / static_cast<float>(a.head_dim) + a.eps);
+            const float sc = __builtin_amdgcn_rsqf(hs / static_cast<float>(a.head_dim) + a.eps);  // one instruction, one unit in the last place: this sits between the loads and the staging
             v = make_float4(v.x * sc * gm.x * sigmoid_fast(z4.x), v.y * sc * gm.y * sigmoid_fast(z4.y),
                             v.z * sc * gm.z * sigmoid_fast(z4.z), v.w * sc * gm.w * sigmoid_fast(z4.w));
         } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
         float tot = 0.f;
 #pragma unroll
         for (int i = 0; i < WAVES; i++) tot += red[i];
-        scale = 1.f / sqrtf(tot / static_cast<float>(K) + a.eps);
+        scale = __builtin_amdgcn_rsqf(tot / static_cast<float>(K) + a.eps);
     }
 
     float xr[64], xs_lo, xs_hi;

@@ -265,7 +265,7 @@ __global__ __launch_bounds__(kBlock) void moe_router_kernel(shv_moe_router_args 
         for (int g = 0; g < kRouterGroup; g++) {
             if (g >= ng) break;
             float scale = 1.f;
-            if (a.gamma) scale = 1.f / sqrtf(((red[g][0] + red[g][1]) + (red[g][2] + red[g][3])) / static_cast<float>(H) + a.eps);
+            if (a.gamma) scale = __builtin_amdgcn_rsqf(((red[g][0] + red[g][1]) + (red[g][2] + red[g][3])) / static_cast<float>(H) + a.eps);
 #pragma unroll
             for (int i = 0; i < H / kBlock; i++) {
                 const int c = tid + i * kBlock;

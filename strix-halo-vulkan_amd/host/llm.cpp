@@ -822,7 +822,11 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
     qkv_ = static_cast<float *>(dev.alloc(T * c_.AttnFusedRows() * 4));
     ctx_ = static_cast<float *>(dev.alloc(T * c_.NHead * c_.HeadDim * 4));
     // one set of slice records per sequence of a batched pass (an ordinary pass is one sequence)
-    partial_ = static_cast<float *>(dev.alloc((T + 1) * c_.NHeadKV * kMaxSplits * 8 * (c_.HeadDim + 2) * 4));  // an odd pass rounds up to whole pairs
+    // Slice records: a pass of P row pairs over all its sequences takes min(splits, ceil(2 CUs / (P kv)))
+    // slices a pair, two rows of 8 heads a record.  One pair can take every slice; many pairs
+    // take at most 2 CUs + P kv records in all, and P is at most the pass's rows.
+    partial_records_ = static_cast<size_t>(c_.NHeadKV) * kMaxSplits + 2 * 512 + (T + 1) * c_.NHeadKV;
+    partial_ = static_cast<float *>(dev.alloc(partial_records_ * 2 * 8 * (c_.HeadDim + 2) * 4));
     const std::vector<float> rt = rope_table(nKV, c_.RopeDims, c_.RopeBase);
     rope_ = static_cast<float *>(dev.alloc(rt.size() * 4));
     dev.upload(rope_, rt.data(), rt.size() * 4);
@@ -840,9 +844,9 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
 }
 
 void AttnGPU::SetSplits(int n) {
-    // slices for the cache's capacity: 128 cells each, up to one block a compute unit over the KV
-    // heads (the kernel engages only as many as the sequence's current length fills)
-    if (n <= 0) n = std::min(128, std::max(8, (n_kv_ + 127) / 128));
+    // slices for the cache's capacity: a tile of 32 cells each while there are slices to spare (the
+    // kernel engages only as many as the sequence's current length fills)
+    if (n <= 0) n = std::min(kMaxSplits, std::max(8, (n_kv_ + 31) / 32));
     if (n > kMaxSplits) throw Error("llm: AttnGPU.SetSplits: at most " + std::to_string(kMaxSplits) + " slices");
     splits_ = n;
 }
@@ -870,6 +874,13 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, cons
     const int nTok = r.rows();
     if (nTok < 1 || nTok > max_tok_) throw Error("llm: AttnGPU: " + std::to_string(nTok) + " rows, staged for " + std::to_string(max_tok_));
     if (r.n_seq > slots_) throw Error("llm: AttnGPU: this block was staged with " + std::to_string(slots_) + " sequence slot(s) (GraphOpts.Slots)");
+    {
+        // the slice records this pass writes (the launcher's own arithmetic) against what was staged
+        const size_t pairs = static_cast<size_t>(r.n_seq) * ((r.seq_len + 1) / 2);
+        const size_t per_pair = std::min<size_t>(splits_, (2 * 512 + pairs * c_.NHeadKV - 1) / (pairs * c_.NHeadKV));
+        if (pairs * c_.NHeadKV * per_pair > partial_records_)
+            throw Error("llm: AttnGPU: " + std::to_string(r.n_seq) + " sequences of " + std::to_string(r.seq_len) + " rows need more slice records than were staged");
+    }
     const int width = c_.AttnFusedRows();
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor(Model::Blk(l, "attn_qkv_fused")).ptr;

@@ -277,6 +277,7 @@ public:
     void Resize(int nTok);
     void Run(int layer);
     static constexpr int kMaxSplits = 512;  // what the decode kernel's merge has room for
+    size_t partial_records_ = 0;            // slice records (two rows of 8 heads each) the scratch holds
     void SetSplits(int n);
     int Splits() const { return splits_; }
     std::vector<shv_op> Dispatches(int layer, const float *in, float *out, int nTok, std::vector<std::string> *labels) const;
