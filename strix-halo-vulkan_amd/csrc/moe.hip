@@ -430,16 +430,21 @@ __global__ __launch_bounds__(kRouteBlock) void moe_route_block_kernel(shv_moe_ro
 }
 
 // The same selection inside a kernel that routes its own token before it can ask for its expert's
-// rows.  Every block of the launch repeats it, so it is kept short: the block's first 256 threads
-// take two experts each (tid and tid + 256); any further waves only keep the block-wide waits
-// (three) and, like the first four, rank the candidates for themselves at the end, so that no
-// wave waits for another's result.  The probabilities are formed exactly as
-// moe_route_block_kernel forms them (the same partial sums over the same 64 experts, added in the
-// same order).  Candidates are the keys whose LOGIT is at or just below the n_used-th largest of
-// the 16 group maxima (a margin of 1e-4 takes in every key whose probability could round to the
-// threshold's), compacted in expert order.  sel_e [kMaxUsed] / sel_w [kMaxUsed + 1] receive
-// experts, weights and the shared expert's gate; probs is the one-wave road's scratch.  On return
-// every wave can read sel_e / sel_w (each has written the same values there itself).
+// rows.  Every block of the launch repeats it and all of them at once, so what counts is how few
+// instructions it takes: the block's first 256 threads take two experts each (tid and tid + 256);
+// any further waves only keep the block-wide waits (three) and, like the first four, rank the
+// candidates for themselves at the end, so that no wave waits for another's result.
+// Candidates are the keys whose logit is at or just below the n_used-th largest of the 16 group
+// maxima, compacted into a table and ranked by (logit, lower index first).  The softmax sum is not
+// formed: a routing weight is p_k / sum over the selected p_j, in which the sum over all experts
+// cancels, so the weights are exp(l_k - max) / sum over the selected exp(l_j - max) (to rounding
+// what the routing kernel's p_k / sum p_j gives), and the reference's floor of 2^-14 on the sum of
+// the selected probabilities cannot engage with at most 512 experts (the largest probability is
+// at least 1/512).  Two different logits whose probabilities round to the same float would be
+// ordered by index in the reference and are ordered by logit here: a tie of the last bit.
+// sel_e [kMaxUsed] / sel_w [kMaxUsed + 1] receive experts, weights and the shared expert's gate;
+// probs is the one-wave road's scratch.  On return every wave can read sel_e / sel_w (each has
+// written the same values there itself).
 constexpr int kCandMax = 64;
 
 // A float's bits as an unsigned integer that orders as the float does.
@@ -459,10 +464,10 @@ __device__ __forceinline__ void count_greater_ror(uint32_t key, int &rank) {
 }
 
 __device__ __forceinline__ void route_block256(const float *lg, int n_expert, int n_used, bool shared_gate, int32_t *sel_e, float *sel_w, float *probs) {
-    __shared__ float s_max[4], s_sum[8];
+    __shared__ float s_max[4];
     __shared__ __align__(16) float s_gm[16];
     __shared__ int s_cnt[4];
-    __shared__ __align__(16) unsigned long long cand[kCandMax];  // (probability bits << 32) | (0x7FFFFFFF - expert); 0 = empty
+    __shared__ __align__(16) unsigned long long cand[kCandMax];  // (logit as ordered bits << 32) | (0x7FFFFFFF - expert)
     __shared__ unsigned long long s_sel[16][kMaxUsed];            // per wave: the selected keys in slot order
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool routing = tid < 256;
@@ -470,9 +475,8 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     const bool has0 = routing && e0 < n_expert, has1 = routing && e1 < n_expert;
     const float l0 = has0 ? lg[e0] : -INFINITY, l1 = has1 ? lg[e1] : -INFINITY;
     const float lsh = (lane == 63 && shared_gate) ? lg[n_expert] : 0.f;  // every wave keeps the shared gate for itself
-    const float m = fmaxf(l0, l1);
     if (routing) {  // the block's maximum and the maxima of 16 groups of 16 threads
-        float gm = m;
+        float gm = fmaxf(l0, l1);
         gm = fmaxf(gm, dpp_f32<kDppXor1>(gm));
         gm = fmaxf(gm, dpp_f32<kDppXor2>(gm));
         gm = fmaxf(gm, dpp_f32<kDppHalfMirror>(gm));
@@ -482,12 +486,10 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
         const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 16));
         const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gm), 48));
         if (lane == 0) s_max[wave] = fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
-        if (wave == 0) cand[lane] = 0ull;
     }
     __syncthreads();
     const float mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
     unsigned long long m0 = 0ull, m1 = 0ull;
-    float ex0 = 0.f, ex1 = 0.f;
     bool p0 = false, p1 = false;
     int n0 = 0;
     if (routing) {
@@ -507,30 +509,20 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
         const unsigned long long hit = __ballot(lane < 16 && rank == n_used - 1);
         float thr_l = -INFINITY;
         if (hit) thr_l = from_ordered_bits(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key & ~15u), __ffsll(static_cast<long long>(hit)) - 1)));
-        // a margin takes in every key whose probability could round to the threshold's
         // (a bound of -inf, fewer than n_used groups holding anything, rounds down to a NaN pattern)
         if (!(thr_l == thr_l)) thr_l = -INFINITY;
-        thr_l -= 1e-4f + 1e-6f * fabsf(thr_l - mx);
-        if (!(thr_l == thr_l)) thr_l = -INFINITY;
-        ex0 = has0 ? expf(l0 - mx) : 0.f;
-        ex1 = has1 ? expf(l1 - mx) : 0.f;
-        const float ws0 = wave_sum_all(ex0), ws1 = wave_sum_all(ex1);
         p0 = has0 && l0 >= thr_l;
         p1 = has1 && l1 >= thr_l;
         m0 = __ballot(p0);
         m1 = __ballot(p1);
         n0 = __popcll(m0);
-        if (lane == 0) {
-            s_sum[wave] = ws0;
-            s_sum[4 + wave] = ws1;
-            s_cnt[wave] = n0 + __popcll(m1);
-        }
+        if (lane == 0) s_cnt[wave] = n0 + __popcll(m1);
     }
     __syncthreads();
     const int c0 = s_cnt[0], c1 = s_cnt[1], c2 = s_cnt[2], c3 = s_cnt[3];
     const int total = c0 + c1 + c2 + c3;
     if (total > kCandMax || total < n_used || n_expert < 64 || n_used > 16) {
-        // uniform over the block: many equal probabilities, or a shape the threshold does not cover
+        // uniform over the block: many equal logits, or a shape the threshold does not cover
         if (wave == 0) {
             route_token<8, false>(lg, n_expert, n_used, sel_e, sel_w, probs);
             if (lane == 0) sel_w[n_used] = shared_gate ? sigmoid_exact(lg[n_expert]) : 0.f;
@@ -539,58 +531,47 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
         return;
     }
     if (routing) {
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < 8; w++) sum += s_sum[w];
-        const float inv = 1.f / sum;
         // the table's order does not matter to the ranks: each wave writes its candidates after
         // those of the waves before it
         const int before = (wave > 0 ? c0 : 0) + (wave > 1 ? c1 : 0) + (wave > 2 ? c2 : 0);
         if (p0) {
             const int pos = before + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m0 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m0), 0u)));
-            cand[pos] = (static_cast<unsigned long long>(__float_as_uint(ex0 * inv)) << 32) | static_cast<uint32_t>(0x7FFFFFFF - e0);
+            cand[pos] = (static_cast<unsigned long long>(ordered_bits(l0)) << 32) | static_cast<uint32_t>(0x7FFFFFFF - e0);
         }
         if (p1) {
             const int pos = before + n0 + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m1 >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m1), 0u)));
-            cand[pos] = (static_cast<unsigned long long>(__float_as_uint(ex1 * inv)) << 32) | static_cast<uint32_t>(0x7FFFFFFF - e1);
+            cand[pos] = (static_cast<unsigned long long>(ordered_bits(l1)) << 32) | static_cast<uint32_t>(0x7FFFFFFF - e1);
         }
     }
     __syncthreads();
-    // every wave: lane i owns table entry i; its rank is how many entries are larger (the keys are
-    // distinct: the expert is part of them; empty entries are 0 and larger than nothing).  The
-    // table is read in two halves, every read of a half in flight together.
-    const unsigned long long mine = cand[lane];
+    // every wave: lane i owns candidate i; its rank is how many candidates are larger (the keys are
+    // distinct: the expert is part of them).  The table is read sixteen entries at a time, all of a
+    // batch's reads in flight together; entries past `total` hold old keys and are masked out.
+    const unsigned long long mine = lane < total ? cand[lane] : 0ull;
     int r4[4] = {0, 0, 0, 0};  // four chains of counts
+    for (int c = 0; c < total; c += 16) {
+        ulonglong2 o[8];
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
-        if (half * (kCandMax / 2) >= total) break;
-        ulonglong2 o[kCandMax / 4];
+        for (int j2 = 0; j2 < 8; j2++) o[j2] = *reinterpret_cast<const ulonglong2 *>(&cand[c + 2 * j2]);
 #pragma unroll
-        for (int j2 = 0; j2 < kCandMax / 4; j2++) o[j2] = *reinterpret_cast<const ulonglong2 *>(&cand[half * (kCandMax / 2) + 2 * j2]);
-#pragma unroll
-        for (int j2 = 0; j2 < kCandMax / 4; j2++) {
-            r4[(2 * j2) & 3] += o[j2].x > mine ? 1 : 0;
-            r4[(2 * j2 + 1) & 3] += o[j2].y > mine ? 1 : 0;
+        for (int j2 = 0; j2 < 8; j2++) {
+            r4[(2 * j2) & 3] += (c + 2 * j2 < total && o[j2].x > mine) ? 1 : 0;
+            r4[(2 * j2 + 1) & 3] += (c + 2 * j2 + 1 < total && o[j2].y > mine) ? 1 : 0;
         }
     }
     const int rank = (r4[0] + r4[1]) + (r4[2] + r4[3]);
-    // slot k's key goes to lane k through the wave's own table, then the sum over the slots in
-    // order, in float32: the reference's sum
-    if (mine != 0ull && rank < n_used) s_sel[wave][rank] = mine;
+    // slot k's key goes to lane k through the wave's own table; the selected experts' exponentials,
+    // then their sum over the slots in order, in float32: the reference's order of additions
+    if (lane < total && rank < n_used) s_sel[wave][rank] = mine;
     __builtin_amdgcn_wave_barrier();
     const unsigned long long sk = lane < n_used ? s_sel[wave][lane] : 0ull;
-    const float w_k = __uint_as_float(static_cast<uint32_t>(sk >> 32));
+    const float ex_k = lane < n_used ? expf(from_ordered_bits(static_cast<uint32_t>(sk >> 32)) - mx) : 0.f;
     const int e_k = 0x7FFFFFFF - static_cast<int>(static_cast<uint32_t>(sk));
     float wsum = 0.f;
-#pragma unroll
-    for (int k = 0; k < kMaxUsed; k++) {
-        if (k >= n_used) break;
-        wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w_k), k));
-    }
-    if (wsum < kWeightsSumFloor) wsum = kWeightsSumFloor;
+    for (int k = 0; k < n_used; k++) wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ex_k), k));
     if (lane < n_used) {
         sel_e[lane] = e_k;
-        sel_w[lane] = w_k / wsum;
+        sel_w[lane] = ex_k / wsum;
     }
     if (lane == 63) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh) : 0.f;
     __builtin_amdgcn_wave_barrier();  // the wave reads what it has written itself (all waves write the same)
