@@ -65,23 +65,30 @@ def token_bytes(cfg, ctx_len):
     return (cfg.n_layer - n_attn) * dn + n_attn * at + cfg.n_layer * moe + head
 
 
-def cpu_baseline(m, cfg, LA, n_tokens):
-    """Time the oracle's token loop on a 4-layer slice of the same weights."""
+def first_period_tensors(m, cfg):
+    """Host copies of the tensors of layers 0..attn_every-1 and of the head (what the CPU legs read)."""
+    per = cfg.attn_every
+    names = [t[0] for t in m.tensors()]
+    keep = [n for n in names if not n.startswith("blk.") or int(n.split(".")[1]) < per]
+    return {n: m.download(n) for n in keep}
+
+
+def cpu_baseline(m, cfg, LA, A, tensors, n_tokens, cores):
+    """Time the oracle's token loop on a 4-layer slice of the same weights, and hold the GPU's
+    4-layer result against the oracle's on the same tokens."""
+    import ctypes as C
     import oracle_lib as O
     per = cfg.attn_every
     sub = LA.Config(**{f: getattr(cfg, f) for f, _ in cfg._fields_})
-    sub.n_layer = per
-    names = [t[0] for t in m.tensors()]
-    keep = [n for n in names if not n.startswith("blk.") or int(n.split(".")[1]) < per]
-    tensors = {n: m.download(n) for n in keep}
-    cores = min(os.cpu_count() or 1, 16)
+    sub.n_layer, sub.nkv, sub.max_tokens, sub.slots, sub.speculative, sub.nextn, sub.head_rows = per, 128, 4, 1, 0, 0, 1
     om = O.OracleModel(sub, tensors, max_cells=64)
     rng = np.random.default_rng(1)
-    om.extend(rng.integers(0, cfg.vocab, size=1).astype(np.int32), threads=cores)  # touch everything once
+    ids = rng.integers(0, cfg.vocab, size=n_tokens + 1).astype(np.int32)
+    om.extend(ids[:1], threads=cores)  # touch everything once
     t0 = time.perf_counter()
     head_s = 0.0
-    for _ in range(n_tokens):
-        om.extend(rng.integers(0, cfg.vocab, size=1).astype(np.int32), threads=cores)
+    for i in range(n_tokens):
+        _, hidden = om.extend(ids[1 + i:2 + i], threads=cores)
     dt = (time.perf_counter() - t0) / n_tokens
     # the head runs once per token, the 4-layer period 12 times: time the head alone to split them
     x = rng.standard_normal(cfg.n_embd).astype(np.float32)
@@ -90,10 +97,29 @@ def cpu_baseline(m, cfg, LA, n_tokens):
     head_s = time.perf_counter() - t0
     periods = cfg.n_layer // per
     per_token = (dt - head_s) * periods + head_s
+    # the same tokens through the GPU path on a model of those four layers (the tensors copied on the
+    # device from the 48-layer model): the residual stream after layer 3, outside every timed region
+    m4 = LA.LLM(sub)
+    try:
+        src = {t[0]: t for t in m.tensors()}
+        for t in m4.tensors():
+            if not t[6]:
+                A.check(A.load().shv_copy(m4.ctx, C.c_void_p(t[1]), C.c_void_p(src[t[0]][1]), t[2]))
+        m4.stage()
+        for i in range(n_tokens + 1):
+            _, got = m4.extend(ids[i:i + 1], want_logits=False, want_hidden=True)
+    finally:
+        m4.close()
+    err = O.rel_l2(got, hidden)
+    if not err <= 1e-3:
+        raise SystemExit("bench.py: the GPU's residual stream after layer %d differs from the oracle's by rel-L2 %.3e (> 1e-3)" % (per - 1, err))
     return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "hidden_rel_l2_vs_gpu": float("%.3e" % err),
             "sample": "C restatement of the reference's Go CPU path (oracle/), layers 0-%d + lm_head of the same "
                       "weights, %d decode tokens at context <= %d; period time x%d + head time; rows of each matvec "
-                      "split over %d threads" % (per - 1, n_tokens, n_tokens + 1, periods, cores)}
+                      "split over %d threads; the GPU path over the same four layers and tokens leaves a residual "
+                      "stream within rel-L2 %.1e of the oracle's (checked here, bound 1e-3)"
+                      % (per - 1, n_tokens, n_tokens + 1, periods, cores, err)}
 
 
 def gemv_rates(m, cfg, A, LA):
@@ -215,6 +241,217 @@ def gemv_rates(m, cfg, A, LA):
     return out
 
 
+class _Borrowed:
+    """hip_api.Context's buffer helpers over the model's own context (which the model destroys)."""
+
+    def __init__(self, A, handle):
+        self.c = A.Context.__new__(A.Context)
+        self.c.L, self.c.h, self.c._bufs = A.load(), handle, []
+
+    def __enter__(self):
+        return self.c
+
+    def __exit__(self, *exc):
+        for b in self.c._bufs:
+            if b.ptr:
+                b.free()
+        self.c._bufs = []
+
+
+def _timed(c, ops, labels, reps=6):
+    """Average ns per label over reps timed runs of the op list (each op has its own timestamps)."""
+    c.dispatch_multi(ops)
+    acc = {}
+    for _ in range(reps):
+        _, per = c.dispatch_multi(ops, per_op=True)
+        for k, v in zip(labels, per):
+            acc[k] = acc.get(k, 0.0) + v / reps
+    return acc
+
+
+def config_blocks(m, cfg, A, tensors, cores, want_cpu):
+    """BASELINE configs 2, 3 (decode) and 4 as blocks of their own, each over all the layers of the
+    model that hold such a block, one after the other, so that every launch finds its weights, state
+    and cache cold as in the token loop.  GPU times are the kernels' own dispatch timestamps; the CPU
+    times beside them are the oracle's block over layer 0's (DeltaNet, experts) or layer 3's
+    (attention) tensors on this host."""
+    import oracle_lib as O
+    out = {}
+    H, E, U, F = cfg.n_embd, cfg.n_expert, cfg.n_expert_used, cfg.ffn_expert
+    tmap = {t[0]: t[1] for t in m.tensors()}
+    blk = lambda l, n: tmap["blk.%d.%s.weight" % (l, n)]
+    rng = np.random.default_rng(7)
+    is_attn = lambda l: (l + 1) % cfg.attn_every == 0
+    eps = cfg.rms_eps
+
+    # ---- config 2: the MoE FFN step ----
+    with _Borrowed(A, m.ctx) as c:
+        res = {}
+        for T in (1, 4, 16):
+            h = rng.standard_normal((T, H)).astype(np.float32)
+            d_h, xn, logits = c.upload(h), c.alloc(T * H * 4), c.alloc(T * (E + 1) * 4)
+            topk, weights = c.alloc(cfg.n_layer * T * U * 4), c.alloc(T * (U + 1) * 4)
+            act, o = c.alloc(T * (U + 1) * F * 4), c.alloc(T * H * 4)
+            defer = 1 if T == 1 else 0   # a one-row pass makes its selection in the expert kernel
+            ops, labels = [], []
+            for l in range(cfg.n_layer):
+                tk = topk.at(l * T * U * 4)
+                ra = A.MoeRouterArgs(d_h.ptr, blk(l, "post_attention_norm"), blk(l, "ffn_gate_inp"), blk(l, "ffn_gate_inp_shexp"),
+                                     xn.ptr, logits.ptr, tk, weights.ptr, T, H, E, U, eps, H, defer)
+                ua = A.MoeUpArgs(xn.ptr, tk, blk(l, "ffn_gate_exps"), blk(l, "ffn_up_exps"), blk(l, "ffn_gate_shexp"),
+                                 blk(l, "ffn_up_shexp"), act.ptr, T, H, U, F, logits.ptr if defer else None,
+                                 weights.ptr if defer else None, E, 0, 0, 0, 0, None, 0)
+                da = A.MoeDownArgs(act.ptr, tk, weights.ptr, blk(l, "ffn_down_exps"), blk(l, "ffn_down_shexp"), d_h.ptr, o.ptr,
+                                   T, H, U, F, H, H, 0, 0, E, None, None)
+                ops += [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
+                labels += ["router", "up", "down"]
+            t = _timed(c, ops, labels)
+            sel = topk.read(np.int32, cfg.n_layer * T * U).reshape(cfg.n_layer, T * U)
+            distinct = float(np.mean([len(np.unique(r)) for r in sel]))
+            per_expert = 2 * F * Q4K_ROW(H) + H * Q4K_ROW(F)
+            alg = (distinct + 1) * per_expert + E * H * 4 + T * (2 * H + 2 * (U + 1) * F + H) * 4
+            us = sum(t.values()) / cfg.n_layer / 1e3
+            r = {"gpu_us": round(us, 2), "router_us": round(t["router"] / cfg.n_layer / 1e3, 2),
+                 "up_us": round(t["up"] / cfg.n_layer / 1e3, 2), "down_us": round(t["down"] / cfg.n_layer / 1e3, 2),
+                 "distinct_routed_experts": round(distinct, 2), "bytes": int(alg),
+                 "GBps": round(alg / us / 1e3, 1), "frac_hbm_peak": round(alg / (us * 1e-6) / HBM_PEAK, 4)}
+            if want_cpu:
+                w = O.MoeW(*[O.F(tensors["blk.0.%s.weight" % n]) for n in ("ffn_gate_inp", "ffn_gate_inp_shexp")],
+                           *[O.B(tensors["blk.0.%s.weight" % n]) for n in ("ffn_gate_exps", "ffn_up_exps", "ffn_down_exps",
+                                                                            "ffn_gate_shexp", "ffn_up_shexp", "ffn_down_shexp")],
+                           (O.C.c_int * 6)(0, 0, 0, 0, 0, 0))
+                mc = O.MoeCfg(H, E, U, F, F)
+                xn_h = O.rmsnorm(h, tensors["blk.0.post_attention_norm.weight"], eps)
+                y = np.empty((T, H), np.float32)
+                best = 1e9
+                for _ in range(3):
+                    t0 = time.perf_counter()
+                    O.lib().shv_ref_moe_block(O.C.byref(mc), O.C.byref(w), O.F(xn_h), T, O.F(y), None, None, None, None, None, None, cores)
+                    best = min(best, time.perf_counter() - t0)
+                r["cpu_us"], r["cpu_cores"] = round(best * 1e6, 1), cores
+            res["T%d" % T] = r
+        out["config2_moe_ffn_step"] = res
+
+    # ---- config 3: one gated-DeltaNet layer at decode, 1 and 8 sequences ----
+    hk, hv, d, conv = cfg.ssm_head_k, cfg.ssm_head_v, cfg.ssm_head_dim, cfg.ssm_conv
+    qk, vw = hk * d, hv * d
+    cw, width = 2 * qk + vw, 2 * qk + 2 * vw + 2 * hv
+    dn_layers = [l for l in range(cfg.n_layer) if not is_attn(l)]
+    with _Borrowed(A, m.ctx) as c:
+        res = {}
+        ring_slots = 8
+        for B in (1, 8):
+            x = rng.standard_normal((B, H)).astype(np.float32)
+            d_x, d_attn, d_o = c.upload(x), c.alloc(B * vw * 4), c.alloc(B * H * 4)
+            d_pos = c.upload(np.full(B, 100, np.int32))
+            d_slot = c.upload(np.arange(B, dtype=np.int32))
+            d_row = c.alloc(width * 4)
+            ops, labels, keep = [], [], []
+            for l in dn_layers:
+                ring = c.alloc(B * ring_slots * width * 4).zero()
+                state = c.alloc(B * hv * d * d * 4).zero()
+                p = A.gemv_args(blk(l, "ssm_in_fused"), d_x, ring, width, H, B, prologue=A.PRO_RMSNORM, gamma=blk(l, "attn_norm"),
+                                eps=eps, pos=d_pos, slot=d_slot if B > 1 else None, seq_len=1, ring_slots=ring_slots, ring_stride=width)
+                s = A.DnStepArgs(ring.ptr, blk(l, "ssm_conv1d"), blk(l, "ssm_a"), blk(l, "ssm_dt"), state.ptr, d_attn.ptr, d_pos.ptr,
+                                 d_slot.ptr if B > 1 else None, B, 1, hk, hv, d, conv, ring_slots, width, eps, 0, None, 1, 0)
+                o = A.gemv_args(blk(l, "ssm_out"), d_attn, d_o, H, vw, B, prologue=A.PRO_GATED_NORM, gamma=blk(l, "ssm_norm"),
+                                residual=d_x, eps=eps, head_dim=d)
+                if B == 1:
+                    p.y_flat = d_row.ptr
+                    o.z, o.z_stride = d_row.at(cw * 4), width
+                else:
+                    o.z, o.pos, o.slot, o.seq_len = ring.at(cw * 4), d_pos.ptr, d_slot.ptr, 1
+                    o.ring_slots, o.ring_stride, o.z_ring = ring_slots, width, 1
+                ops += [A.make_op(A.OP_GEMV_Q4K, p), A.make_op(A.OP_DN_STEP, s), A.make_op(A.OP_GEMV_Q4K, o)]
+                labels += ["qkv", "step", "out"]
+            t = _timed(c, ops, labels)
+            n = len(dn_layers)
+            alg = width * Q4K_ROW(H) + H * Q4K_ROW(vw) + B * (2 * hv * d * d * 4 + (H + width + conv * cw + vw + 2 * H) * 4)
+            us = sum(t.values()) / n / 1e3
+            r = {"gpu_us": round(us, 2), "qkv_us": round(t["qkv"] / n / 1e3, 2), "step_us": round(t["step"] / n / 1e3, 2),
+                 "out_us": round(t["out"] / n / 1e3, 2), "bytes": int(alg), "GBps": round(alg / us / 1e3, 1),
+                 "frac_hbm_peak": round(alg / (us * 1e-6) / HBM_PEAK, 4)}
+            if want_cpu:
+                g = lambda n_: tensors["blk.0.%s.weight" % n_]
+                w = O.DnW(O.B(g("attn_qkv")), O.B(g("attn_gate")), O.B(g("ssm_alpha")), O.B(g("ssm_beta")), O.B(g("ssm_out")),
+                          O.F(g("ssm_conv1d")), O.F(g("ssm_a")), O.F(g("ssm_dt")), O.F(g("ssm_norm")))
+                dc = O.DnCfg(H, d, hk, hv, conv, eps, 0)
+                xn_h = O.rmsnorm(x[:1], g("attn_norm"), eps)
+                cs, ss = np.zeros((cw, conv - 1), np.float32), np.zeros((hv, d, d), np.float32)
+                y, at = np.empty((1, H), np.float32), np.empty((1, vw), np.float32)
+                best = 1e9
+                for _ in range(3):
+                    t0 = time.perf_counter()
+                    O.lib().shv_ref_deltanet_layer(O.C.byref(dc), O.C.byref(w), O.F(xn_h), 1, O.F(cs), O.F(ss), O.F(y),
+                                                   None, None, None, None, None, O.F(at), None, 0, cores)
+                    best = min(best, time.perf_counter() - t0)
+                # the CPU path takes its sequences one after the other
+                r["cpu_us"], r["cpu_cores"] = round(best * 1e6 * B, 1), cores
+            res["decode_B%d" % B] = r
+        out["config3_deltanet_layer"] = res
+
+    # ---- config 4: gated attention decode over a long fp16 cache ----
+    NH, NKV, D, ROPE = cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.rope_dims
+    awidth = NH * 2 * D + 2 * NKV * D
+    at_layers = [l for l in range(cfg.n_layer) if is_attn(l)]
+    with _Borrowed(A, m.ctx) as c:
+        res = {}
+        max_cells = 131072
+        n_slots = 3
+        # one cache pair per attention layer would be 9.7 GB at three slots; four pairs in rotation
+        # (3.2 GB, far more than every cache level) keep each launch's cells cold
+        n_rot = 4
+        caches = [(c.alloc(n_slots * max_cells * NKV * D * 2), c.alloc(n_slots * max_cells * NKV * D * 2)) for _ in range(n_rot)]
+        fill = A.FillNormalArgs
+        for kc, vc in caches:
+            for buf in (kc, vc):
+                f = fill(buf.ptr, n_slots * max_cells * NKV * D, 11, 0.0, 1.0, 1)
+                A.check(c.L.shv_fill_normal(c.h, O.C.byref(f)))
+        d_rope = c.upload(np.ones((max_cells, ROPE), np.float32) * np.float32(0.70710678))
+        for cells in (4096, 32768, 131072):
+            for S in (1, 3):
+                x = rng.standard_normal((S, H)).astype(np.float32)
+                d_x, d_qkv, d_ctx, d_o = c.upload(x), c.alloc(S * awidth * 4), c.alloc(S * NH * D * 4), c.alloc(S * H * 4)
+                d_pos = c.upload(np.full(S, cells - 1, np.int32))
+                d_slot = c.upload(np.arange(S, dtype=np.int32))
+                n_splits = min(512, max(8, (cells + 31) // 32))
+                d_part = c.alloc((S * 2 * NKV * n_splits * (NH // NKV) * (D + 2) + 8192) * 4)
+                ops, labels = [], []
+                for i, l in enumerate(at_layers):
+                    kc, vc = caches[i % n_rot]
+                    p = A.gemv_args(blk(l, "attn_qkv_fused"), d_x, d_qkv, awidth, H, S, prologue=A.PRO_RMSNORM, gamma=blk(l, "attn_norm"), eps=eps)
+                    a = A.AttnDecodeArgs(d_qkv.ptr, blk(l, "attn_q_norm"), blk(l, "attn_k_norm"), d_rope.ptr, kc.ptr, vc.ptr, d_part.ptr,
+                                         d_ctx.ptr, d_pos.ptr, d_slot.ptr if S > 1 else None, S, 1, NH, NKV, D, ROPE, max_cells, awidth, n_splits, eps)
+                    o = A.gemv_args(blk(l, "attn_output"), d_ctx, d_o, H, NH * D, S, prologue=A.PRO_MUL_SIGMOID, z=d_qkv, head_dim=D,
+                                    z_stride=awidth, residual=d_x)
+                    ops += [A.make_op(A.OP_GEMV_Q4K, p), A.make_op(A.OP_ATTN_DECODE, a), A.make_op(A.OP_GEMV_Q4K, o)]
+                    labels += ["qkv", "attn", "out"]
+                t = _timed(c, ops, labels, reps=4)
+                n = len(at_layers)
+                cache_bytes = S * cells * NKV * D * 2 * 2
+                alg = awidth * Q4K_ROW(H) + H * Q4K_ROW(NH * D) + cache_bytes + S * (2 * H + awidth + NH * D) * 4
+                us = sum(t.values()) / n / 1e3
+                r = {"gpu_us": round(us, 2), "qkv_us": round(t["qkv"] / n / 1e3, 2), "attn_us": round(t["attn"] / n / 1e3, 2),
+                     "out_us": round(t["out"] / n / 1e3, 2), "bytes": int(alg), "GBps": round(alg / us / 1e3, 1),
+                     "frac_hbm_peak": round(alg / (us * 1e-6) / HBM_PEAK, 4),
+                     "cache_GBps": round(cache_bytes / (t["attn"] / n) , 1)}
+                if want_cpu and S == 1:
+                    g = lambda n_: tensors["blk.%d.%s.weight" % (cfg.attn_every - 1, n_)]
+                    w = O.AttnW(O.B(g("attn_q")), O.B(g("attn_k")), O.B(g("attn_v")), O.B(g("attn_output")), O.F(g("attn_q_norm")), O.F(g("attn_k_norm")))
+                    ac = O.AttnCfg(H, NH, NKV, D, ROPE, cfg.rope_base, (O.C.c_int * 4)(11, 11, 10, 0), eps)
+                    kh = rng.standard_normal((cells, NKV, D)).astype(np.float16).view(np.uint16)
+                    vh = kh.copy()
+                    xn_h = O.rmsnorm(x[:1], g("attn_norm"), eps)
+                    y = np.empty((1, H), np.float32)
+                    t0 = time.perf_counter()
+                    O.lib().shv_ref_attn_layer(O.C.byref(ac), O.C.byref(w), O.F(xn_h), 1, cells - 1, O.H(kh), O.H(vh), O.F(y), None, None, cores)
+                    res_cpu = time.perf_counter() - t0
+                    r["cpu_us"], r["cpu_cores"] = round(res_cpu * 1e6, 1), cores
+                res["ctx%d_slots%d" % (cells, S)] = r
+        out["config4_attention_decode"] = res
+    return out
+
+
 def mtp_run(m, cfg, prompt, plain, acc, rounds):
     """Pass costs in decode steps and the speculative loop at depth 2 (3-row verification)."""
     kernels = lambda st: sum(v for k, v in st if k != "total")
@@ -288,6 +525,7 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mtp", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-config blocks (configs 1-4 each on its own)")
     ap.add_argument("--mtp-rounds", type=int, default=64)
     ap.add_argument("--batch-slots", type=int, default=8,
                     help="sequences of the batched-decode leg (one token each per pass); 0 skips it")
@@ -407,8 +645,23 @@ def main():
             rec["mtp"] = mtp_run(m, cfg, prompt, plain, acc, rounds)
     if not a.no_mtp and a.batch_slots >= 2:
         rec["batched_decode"] = batched_run(m, cfg, a.batch_slots, rng)
+    cores = min(os.cpu_count() or 1, 16)
+    tensors = first_period_tensors(m, cfg) if not a.no_cpu else None
+    if not a.no_configs:
+        rec["configs"] = config_blocks(m, cfg, A, tensors, cores, not a.no_cpu)
+        rec["configs"]["config1_gemv_4096x2048"] = dict(rec["gemv"]["config1_4096x2048"])
+        if not a.no_cpu:
+            x = rng.standard_normal(cfg.n_embd).astype(np.float32)
+            import oracle_lib as O
+            wq = tensors["blk.0.ffn_gate_exps.weight"][:4096 * Q4K_ROW(cfg.n_embd)]
+            best = 1e9
+            for _ in range(5):
+                t0 = time.perf_counter()
+                O.gemv_q4k(wq, x, 4096, cfg.n_embd, threads=cores)
+                best = min(best, time.perf_counter() - t0)
+            rec["configs"]["config1_gemv_4096x2048"].update(cpu_us=round(best * 1e6, 1), cpu_cores=cores)
     if not a.no_cpu:
-        rec["cpu_baseline"] = cpu_baseline(m, cfg, LA, a.cpu_tokens)
+        rec["cpu_baseline"] = cpu_baseline(m, cfg, LA, A, tensors, a.cpu_tokens, cores)
     m.close()
     print(json.dumps(rec))
 
