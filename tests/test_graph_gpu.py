@@ -137,3 +137,113 @@ def test_profile_step_labels(small):
               "moe.up", "moe.down", "head", "argmax", "total"):
         assert k in st and st[k] > 0, k
     assert m.dispatches() == 1 + 4 * 6 + 2
+
+
+def _oracle_rows_with_gaps(om, tensors, cfg, ids, threads=16):
+    """The oracle's pass over rows `ids` (its block functions in the order of its own token loop,
+    oracle/shv_oracle.c shv_ref_model_extend_rows), which also returns, per row, the smallest gap
+    over all layers between the 10th and the 11th router logit: where that gap is of the size of
+    float32 rounding, which expert is selected is not a statement about the kernels."""
+    C, L, mc = O.C, O.lib(), om.mcfg
+    T, H, E, U = len(ids), cfg.n_embd, cfg.n_expert, cfg.n_expert_used
+    x = tensors["token_embd.weight"].view(np.float16).reshape(cfg.vocab, H)[ids].astype(np.float32)
+    gaps = np.full(T, np.inf)
+    y, lg = np.empty((T, H), np.float32), np.empty((T, E), np.float32)
+    for l in range(cfg.n_layer):
+        lw = om.layers[l]
+        xn = O.rmsnorm(x, tensors["blk.%d.attn_norm.weight" % l], cfg.rms_eps)
+        if (l + 1) % cfg.attn_every == 0:
+            L.shv_ref_attn_layer(C.byref(mc.attn), C.byref(lw.attn), O.F(xn), T, om.state.past, O.H(om.kc[l]), O.H(om.vc[l]),
+                                 O.F(y), None, None, threads)
+        else:
+            L.shv_ref_deltanet_layer(C.byref(mc.dn), C.byref(lw.dn), O.F(xn), T, O.F(om.dn_conv[l]), O.F(om.dn_s[l]), O.F(y),
+                                     None, None, None, None, None, None, None, 0, threads)
+        x = x + y
+        xn = O.rmsnorm(x, tensors["blk.%d.post_attention_norm.weight" % l], cfg.rms_eps)
+        L.shv_ref_moe_block(C.byref(mc.moe), C.byref(lw.moe), O.F(xn), T, O.F(y), O.F(lg), None, None, None, None, None, threads)
+        x = x + y
+        top = np.sort(lg.astype(np.float64), axis=1)[:, ::-1]
+        gaps = np.minimum(gaps, top[:, U - 1] - top[:, U])
+    om.state.past += T
+    xn = O.rmsnorm(x[-1:], tensors["output_norm.weight"], cfg.rms_eps)
+    logits = O.gemv_q4k(tensors["output.weight"], xn[0], cfg.vocab, H, threads=threads)
+    return x, logits, gaps
+
+
+@pytest.mark.timeout(900)
+def test_full_size_model_matches_the_cpu_loop():
+    """The benchmark's own model (48 layers, 512 experts top-10, vocab 151 936) rather than a reduced
+    one: a prompt of 6 ids through the multi-row pass, then 4 greedy tokens through the recorded
+    one-row step, against the oracle over the very same tensors (downloaded, 46 GB on the host).
+    Every row's residual stream within 1e-3 rel-L2, logits too; ids equal unless the oracle's own
+    best two logits sit closer than twice the two paths' largest logit difference.  With 288 top-10 selections among 512 nearly level logits
+    a pass, now and then one sits on a near-tie (a gap of 1e-5 where the logits themselves agree to
+    1e-5): such a row may take the other expert, as the reference's own routing tests exclude
+    near-ties (llm/moe_test.go:59-66); it is left out of the comparison, and most rows must remain."""
+    cfg = LA.Config(nkv=128, max_tokens=8)
+    assert (cfg.n_layer, cfg.n_expert, cfg.n_expert_used, cfg.vocab) == (48, 512, 10, 151936)
+    GAP = 1e-3   # router logits are O(1) and agree to about 2e-4 by the last layers
+    m = LA.LLM(cfg)
+    try:
+        m.init_synthetic(20260101)
+        m.stage()
+        tensors = {t[0]: m.download(t[0]) for t in m.tensors()}
+        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+        check = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+        greedy_done = False
+        for seed in (17, 18, 19, 20, 21):   # until a prompt without a flipped row lets the greedy steps be compared
+            m.reset()
+            om.reset()
+            check.reset()
+            rng = np.random.default_rng(seed)
+            prompt = rng.integers(0, cfg.vocab, size=6).astype(np.int32)
+            rows_cpu, lg_cpu, gaps = _oracle_rows_with_gaps(om, tensors, cfg, prompt)
+            # the walk above is the oracle's own loop: same hidden state, bit for bit
+            _, hd_loop = check.extend(prompt, threads=16)
+            assert np.array_equal(hd_loop, rows_cpu[-1])
+            _, lg_rows, rows_gpu = m.extend_rows(prompt, want_logits=True, want_res=True)
+            errs = [O.rel_l2(rows_gpu[t], rows_cpu[t]) for t in range(len(prompt))]
+            print("full size: prompt rows rel-L2", ["%.2e" % e for e in errs], "gaps", ["%.1e" % g for g in gaps], flush=True)
+            # a row past a near-tie (its own, or an earlier row's, whose state it reads) may hold
+            # another expert's output; every other row must agree
+            so_far = np.minimum.accumulate(gaps)
+            within = [e <= 1e-3 for e in errs]
+            assert all(w or g < GAP for w, g in zip(within, so_far)), (errs, list(so_far))
+            assert sum(within) >= 4
+            compared = 0
+            if all(within):
+                assert O.rel_l2(lg_rows[-1], lg_cpu) <= 1e-3
+                lg, lg_gpu = lg_cpu, lg_rows[-1]
+                for i in range(4):
+                    tok_cpu = int(O.lib().shv_ref_argmax(O.F(lg), cfg.vocab))
+                    tok_gpu = int(np.argmax(lg_gpu))
+                    top2 = np.sort(lg)[-2:]
+                    margin = float(top2[1] - top2[0])
+                    if tok_gpu != tok_cpu:
+                        # only logits closer than twice their own disagreement can swap places
+                        assert margin < 2 * float(np.max(np.abs(lg_gpu - lg))), f"token {i}: gpu {tok_gpu} cpu {tok_cpu} at margin {margin:.3e}"
+                        break
+                    hd_cpu, lg, gap = _oracle_rows_with_gaps(om, tensors, cfg, np.array([tok_cpu], np.int32))
+                    # the recorded one-row step (the decode path proper), fed the same id
+                    lg_gpu, hd_gpu = m.extend(np.array([tok_cpu], np.int32), want_hidden=True)
+                    e_h, e_l = O.rel_l2(hd_gpu, hd_cpu[0]), O.rel_l2(lg_gpu, lg)
+                    print("full size: token %d id %d margin %.3e gap %.1e hidden rel-L2 %.3e logits rel-L2 %.3e"
+                          % (i, tok_cpu, margin, gap[0], e_h, e_l), flush=True)
+                    if e_h > 1e-3 or e_l > 1e-3:
+                        assert min(gap[0], so_far[-1]) < GAP, (e_h, e_l, gap[0])
+                        break
+                    compared += 1
+                if compared == 4:
+                    # carried state of the last DeltaNet layer and the last attention layer's cache
+                    assert O.rel_l2(m.dn_state(46), om.dn_s[46]) <= 1e-3
+                    k, v = m.kv(47, om.past)
+                    kf = lambda a: a.view(np.float16).astype(np.float32)
+                    assert O.rel_l2(kf(k), kf(om.kc[47][:om.past])) <= 2e-3
+                    assert O.rel_l2(kf(v), kf(om.vc[47][:om.past])) <= 2e-3
+            print("full size: seed %d: %d of %d prompt rows within 1e-3, %d greedy steps compared" % (seed, sum(within), len(prompt), compared), flush=True)
+            if compared >= 2:
+                greedy_done = True
+                break
+        assert greedy_done, "no prompt of five left the greedy steps comparable"
+    finally:
+        m.close()
