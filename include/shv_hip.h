@@ -90,6 +90,7 @@ enum {
     SHV_OP_ADVANCE = 12,
     SHV_OP_DEQUANT = 13,
     SHV_OP_GEMV = 14,
+    SHV_OP_RING_ROWS = 15,
     SHV_OP__COUNT
 };
 
@@ -287,7 +288,14 @@ typedef struct {
  * spec != 0 leaves it untouched and stores the state after row i of the pass into plane
  * (plane[slot] + 1 + i) % n_planes, so that accepting the first k rows of the pass is
  * plane[slot] = (plane[slot] + k) % n_planes and discarding it is doing nothing; seq_len must then
- * be below n_planes.  plane NULL reads plane 0. */
+ * be below n_planes.  plane NULL reads plane 0.
+ * work (optional): work_floats floats of scratch, 16-byte aligned.  With at least n_seq*seq_len*
+ * (2*hk*d + hv*d + 2*hv) of them a plain pass (spec == 0) of more than 16 rows goes 64 rows at a
+ * time on the matrix cores (the chunked form of the same rule: q^, k^, v, log g and beta of every
+ * row are prepared into work first, then each chunk is a few 64-row products and one triangular
+ * solve against the state, which is read and written once per pass); results agree with the
+ * row-by-row rule to float32 rounding.  The reference scans row by row at every pass length
+ * (shaders/llm_dn_scan.comp; llm/gpu_deltanet.go:48-52 names the chunked form as not built there). */
 typedef struct {
     const float *ring;
     const float *conv1d;
@@ -304,6 +312,8 @@ typedef struct {
     int32_t qk_norm_max;
     const int32_t *plane;
     int32_t n_planes, spec;
+    float *work;
+    int64_t work_floats;
 } shv_dn_step_args;
 
 /* Gated full-attention decode over an fp16 KV cache (AttnLayerAt, llm/attn.go:162-205, and
@@ -376,6 +386,21 @@ typedef struct {
     int32_t n_seq, delta;
 } shv_advance_args;
 
+/* Rows of one ring of projection rows copied into another: positions pos[0]+first ..
+ * pos[0]+first+count-1 (those below zero are skipped), row p from src[(p % src_slots) * stride] to
+ * dst[(p % dst_slots) * stride], n floats each.  A prompt pass of many rows keeps its DeltaNet
+ * projection rows in a ring of its own, sized for the pass: the conv's three rows of history are
+ * brought into it before the step, and the pass's last three rows are left in the sequence's small
+ * ring after it.  (No counterpart in the reference, whose conv window lives in the layer's own
+ * activation buffer, llm/gpu_deltanet.go:1046-1052.) */
+typedef struct {
+    const float *src;
+    float *dst;
+    const int32_t *pos;
+    int32_t src_slots, dst_slots, stride, n;
+    int32_t first, count;
+} shv_ring_rows_args;
+
 typedef struct {
     uint32_t kind;
     uint32_t flags;          /* bit 0: may overlap the previous op (MultiDispatch.Overlap) */
@@ -417,6 +442,7 @@ int shv_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *a);
 int shv_embed(shv_ctx *ctx, const shv_embed_args *a);
 int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_advance(shv_ctx *ctx, const shv_advance_args *a);
+int shv_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *a);
 
 /* shv_argmax for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and

@@ -312,6 +312,8 @@ int shv_launch_dn_step(shv_ctx *ctx, const shv_dn_step_args *pa) {
     SHV_REQUIRE(a.n_planes >= 0 && a.n_planes <= 64, "dn_step: %d state planes", a.n_planes);
     SHV_REQUIRE(!a.spec || (a.n_planes > 1 && a.seq_len < a.n_planes), "dn_step: a rewindable pass of %d rows needs more than %d state planes",
                 a.seq_len, a.n_planes);
+    SHV_REQUIRE(!a.work || a.work_floats >= 0, "dn_step: work_floats %lld", static_cast<long long>(a.work_floats));
+    if (shv_dn_chunk_covers(a)) return shv_launch_dn_chunk(ctx, a);
     dim3 grid(kD / kRowsPerBlock, a.n_head_v, a.n_seq);
     // more than one group of rows: preparation and rule overlap
     if (a.seq_len > kPrep) SHV_LAUNCH(ctx, dn_step_pipe_kernel, grid, dim3(kBlock + 64 * kPrepWaves), 0, a);

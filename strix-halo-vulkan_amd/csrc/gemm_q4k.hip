@@ -500,7 +500,7 @@ struct WideLoads {
 // grid: (row groups of NW * R * 16 rows, column parts); NW waves, each owning R row tiles.
 // part: [parts][64][n] partial products when the columns are split, else unused.
 template <int NW, int kWideR>
-__global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a, int t0, int nt, const char *staged, float *part, int steps_per) {
+__global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a, int t0, int nt, const char *staged, float *part, int steps_per, int groups) {
     extern __shared__ __align__(16) char smem[];
     size_t *yoffs = reinterpret_cast<size_t *>(smem + 2 * kWideSlab);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -509,7 +509,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a,
     const size_t row_bytes = static_cast<size_t>(sbs) * SHV_Q4K_BYTES;
     const int s0 = blockIdx.y * steps_per, s1 = s0 + steps_per;
     constexpr int NTHR = NW * 64;
-    const int row0 = (blockIdx.x * NW + wave) * (kWideR * kTileRows);
+    // A pass of many groups of 64 rows in one launch: neighbouring blocks take the same weight rows
+    // for different groups, so that a row block's weights come from HBM once and from L2 after.
+    int xb = blockIdx.x;
+    if (groups > 1) {
+        const int grp = xb % groups;
+        xb /= groups;
+        t0 = grp * kWideTok;
+        nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;
+        staged += static_cast<size_t>(grp) * wide_region(a.k);
+    }
+    const int row0 = (xb * NW + wave) * (kWideR * kTileRows);
     const int ntt = (nt + kTileRows - 1) / kTileRows;
 
     const char *rp[kWideR];
@@ -733,7 +743,7 @@ int launch_wide(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const 
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
         raised = true;
     }
-    SHV_LAUNCH(ctx, (gemm_wide_kernel<NW, R>), dim3(bx, ks), dim3(NW * 64), lds, a, t0, nt, staged, ctx->gemm_part, steps / ks);
+    SHV_LAUNCH(ctx, (gemm_wide_kernel<NW, R>), dim3(bx, ks), dim3(NW * 64), lds, a, t0, nt, staged, ctx->gemm_part, steps / ks, 1);
     if (ks > 1) {
         // 16-byte moves need whole quads of outputs at 16-byte addresses in every row
         const bool ring = a.ring_slots > 0 && !a.z_ring;
@@ -741,6 +751,23 @@ int launch_wide(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const 
                         (!a.residual || (shv_aligned16(a.residual) && a.y_stride % 4 == 0));
         SHV_LAUNCH(ctx, gemm_wide_join_kernel, dim3((a.n + 255) / 256, nt), dim3(64), 0, a, t0, ctx->gemm_part, ks, vec);
     }
+    return SHV_OK;
+}
+
+// Every group of 64 rows of a long pass in one launch (the operands of all of them are in
+// ctx->gemm_stage): no split along the columns, the groups themselves fill the chip.
+template <int NW, int R>
+int launch_wide_all(shv_ctx *ctx, const shv_gemv_q4k_args &a, int groups) {
+    constexpr int kRows = NW * R * kTileRows;
+    const int bx = (a.n + kRows - 1) / kRows;
+    const size_t lds = 2 * kWideSlab + kWideTok * sizeof(size_t);
+    static bool raised = false;
+    if (!raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(84 * 1024)));
+        raised = true;
+    }
+    SHV_REQUIRE(static_cast<long long>(bx) * groups <= 0x7fffffffll, "gemm_q4k: %d row blocks of %d groups", bx, groups);
+    SHV_LAUNCH(ctx, (gemm_wide_kernel<NW, R>), dim3(bx * groups, 1), dim3(NW * 64), lds, a, 0, 0, ctx->gemm_stage, ctx->gemm_part, a.k / 128, groups);
     return SHV_OK;
 }
 
@@ -773,6 +800,7 @@ int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
         const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
         SHV_REQUIRE(groups * wide_region(a.k) <= static_cast<size_t>(shv_ctx::kGemmStageBytes), "gemm_q4k: %d rows of %d columns do not fit the staging buffer", a.n_tok, a.k);
         SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(a.k / 256, kWideTok / 4, groups), dim3(256), 0, a, ctx->gemm_stage);
+        if (groups >= 4) return launch_wide_all<8, 1>(ctx, a, groups);
         for (int g = 0; g < groups; g++) {
             const int t0 = g * kWideTok;
             const int nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;

@@ -476,7 +476,7 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
     const shv_gemv_q4k_args &a = *pa;
     SHV_REQUIRE(a.w && a.x && a.y, "gemv_q4k: NULL w, x or y");
     SHV_REQUIRE(a.n > 0, "gemv_q4k: n = %d", a.n);
-    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 64, "gemv_q4k: n_tok %d, the GEMV covers 1..64 rows", a.n_tok);
+    SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 4096, "gemv_q4k: n_tok %d; a pass carries 1..4096 rows", a.n_tok);
     SHV_REQUIRE(shv_aligned16(a.w), "gemv_q4k: w must be 16-byte aligned");
     const int x_width = a.prologue == SHV_PRO_RMSNORM_PAIR ? a.k / 2 : a.k;
     SHV_REQUIRE(a.x_stride >= x_width || a.n_tok == 1, "gemv_q4k: x_stride %d < %d", a.x_stride, x_width);
@@ -502,6 +502,8 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
     if (a.n_tok >= (a.k > 2048 ? ctx->mfma_min_rows_wide : ctx->mfma_min_rows) && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
+    SHV_REQUIRE(a.n_tok <= 64, "gemv_q4k: %d rows: more than 64 go through the matrix-core kernel, which does not take this shape (k %d, prologue %d)",
+                a.n_tok, a.k, a.prologue);
     if (row_kernel_covers(ctx, a)) return launch_row(ctx, a);
     switch (a.k) {
         case 512: return launch_k<512>(ctx, a);

@@ -164,6 +164,17 @@ __global__ void advance_kernel(shv_advance_args a) {
     if (s < a.n_seq) a.pos[s] += a.delta;
 }
 
+// grid: (column chunks of 1024 floats, count); one block a piece of a row
+__global__ __launch_bounds__(256) void ring_rows_kernel(shv_ring_rows_args a) {
+    const int p = (a.pos ? a.pos[0] : 0) + a.first + static_cast<int>(blockIdx.y);
+    if (p < 0) return;
+    const float *src = a.src + static_cast<size_t>(p % a.src_slots) * a.stride;
+    float *dst = a.dst + static_cast<size_t>(p % a.dst_slots) * a.stride;
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (c + 4 <= a.n) *reinterpret_cast<float4 *>(dst + c) = *reinterpret_cast<const float4 *>(src + c);
+    else for (int i = c; i < a.n; i++) dst[i] = src[i];
+}
+
 // ---- the arg-max that allocates nothing ------------------------------------------------------
 // Its per-block winners and arrival counters live in this array instead of in memory the context
 // allocated: kArgmaxBlocks values, kArgmaxBlocks indices, then kStaticCounters arrival counters.
@@ -181,6 +192,16 @@ __global__ void clear_counters_kernel(int32_t *c, int n) {
 }
 
 }  // namespace
+
+int shv_launch_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *pa) {
+    const shv_ring_rows_args &a = *pa;
+    SHV_REQUIRE(a.src && a.dst, "ring_rows: NULL argument");
+    SHV_REQUIRE(a.src_slots >= 1 && a.dst_slots >= 1 && a.n >= 1 && a.stride >= a.n && a.count >= 1 && a.count <= 65535,
+                "ring_rows: %d rows of %d floats between rings of %d and %d slots", a.count, a.n, a.src_slots, a.dst_slots);
+    SHV_REQUIRE(shv_aligned16(a.src) && shv_aligned16(a.dst) && a.stride % 4 == 0, "ring_rows: rings must be 16-byte aligned, rows a multiple of 4 floats apart");
+    SHV_LAUNCH(ctx, ring_rows_kernel, dim3((a.n + 1023) / 1024, a.count), dim3(256), 0, a);
+    return SHV_OK;
+}
 
 int shv_static_scratch_bind(shv_ctx *ctx) {
     SHV_REQUIRE(ctx->device >= 0 && ctx->device < kMaxDevices, "shv_init: device %d; the static scratch table covers %d devices", ctx->device, kMaxDevices);

@@ -30,9 +30,9 @@ struct shv_ctx {
     int32_t *counters = nullptr;
     int n_counters = 0;
     // activations of a many-row projection, transformed once into matrix-core operand order and
-    // copied from here by every block (kGemmStageBytes covers 64 rows of 4096 columns)
+    // copied from here by every block (kGemmStageBytes covers 4096 rows of 4096 columns)
     char *gemm_stage = nullptr;
-    enum { kGemmStageBytes = 4 << 20 };
+    enum { kGemmStageBytes = 72 << 20 };
     // partial products of a pass whose columns are split over blocks: [parts][64 rows][n] floats
     float *gemm_part = nullptr;
     enum { kGemmPartBytes = 16 << 20 };
@@ -133,5 +133,8 @@ int shv_launch_embed_typed(shv_ctx *ctx, const shv_embed_args *a);  // a table i
 long long shv_type_bytes(int type, long long n);                    // bytes of n elements of a ggml type, -1 if refused
 int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_launch_advance(shv_ctx *ctx, const shv_advance_args *a);
+int shv_launch_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *a);
+bool shv_dn_chunk_covers(const shv_dn_step_args &a);
+int shv_launch_dn_chunk(shv_ctx *ctx, const shv_dn_step_args &a);
 int shv_static_scratch_bind(shv_ctx *ctx);  // at shv_init, with ctx->device current
 int shv_launch_argmax_static(shv_ctx *ctx, const shv_argmax_args *a);

@@ -10,7 +10,7 @@ Q4K_BYTES = 144
 
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
-OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV = 10, 11, 12, 13, 14
+OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV, OP_RING_ROWS = 10, 11, 12, 13, 14, 15
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 
@@ -96,7 +96,8 @@ class DnStepArgs(C.Structure):
                 ("seq_len", C.c_int32), ("n_head_k", C.c_int32), ("n_head_v", C.c_int32),
                 ("head_dim", C.c_int32), ("conv", C.c_int32), ("ring_slots", C.c_int32),
                 ("ring_stride", C.c_int32), ("eps", C.c_float), ("qk_norm_max", C.c_int32),
-                ("plane", C.c_void_p), ("n_planes", C.c_int32), ("spec", C.c_int32)]
+                ("plane", C.c_void_p), ("n_planes", C.c_int32), ("spec", C.c_int32),
+                ("work", C.c_void_p), ("work_floats", C.c_int64)]
 
 
 class AttnDecodeArgs(C.Structure):
@@ -125,6 +126,12 @@ class AdvanceArgs(C.Structure):
     _fields_ = [("pos", C.c_void_p), ("n_seq", C.c_int32), ("delta", C.c_int32)]
 
 
+class RingRowsArgs(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("pos", C.c_void_p), ("src_slots", C.c_int32),
+                ("dst_slots", C.c_int32), ("stride", C.c_int32), ("n", C.c_int32), ("first", C.c_int32),
+                ("count", C.c_int32)]
+
+
 class Op(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("flags", C.c_uint32), ("args", C.c_uint8 * 248)]
 
@@ -146,7 +153,7 @@ SYMBOLS = [
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
-    "shv_argmax_static",
+    "shv_argmax_static", "shv_ring_rows",
 ]
 
 _lib = None
@@ -202,6 +209,7 @@ def load():
     L.shv_argmax.argtypes = [vp, C.POINTER(ArgmaxArgs)]
     L.shv_advance.argtypes = [vp, C.POINTER(AdvanceArgs)]
     L.shv_argmax_static.argtypes = [vp, C.POINTER(ArgmaxArgs)]
+    L.shv_ring_rows.argtypes = [vp, C.POINTER(RingRowsArgs)]
     _lib = L
     return L
 

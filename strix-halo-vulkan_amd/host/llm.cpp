@@ -584,12 +584,20 @@ DeltaNetGPU::DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, 
     // refusals at construction, never at run (llm/gpu_deltanet.go:423-447)
     if (c_.SSMHeadDim != 128) throw Error("llm: DeltaNetGPU: head dimension " + std::to_string(c_.SSMHeadDim) + ", the step kernel is built for 128");
     if (c_.SSMConv != 4) throw Error("llm: DeltaNetGPU: conv kernel " + std::to_string(c_.SSMConv) + ", built for 4");
-    if (maxTokens < 1 || maxTokens > 64) throw Error("llm: DeltaNetGPU: a pass of " + std::to_string(maxTokens) + " rows; 1..64");
+    if (maxTokens < 1 || maxTokens > 4096) throw Error("llm: DeltaNetGPU: a pass of " + std::to_string(maxTokens) + " rows; 1..4096");
     if (slots < 1) throw Error("llm: DeltaNetGPU: no slots");
     if (planes < 1 || planes > 64 || (planes > 1 && !plane)) throw Error("llm: DeltaNetGPU: " + std::to_string(planes) + " state planes");
     // the ring holds a pass's rows and the conv's history behind them
-    ring_slots_ = std::max(kRing, maxTokens + c_.SSMConv - 1);
+    ring_slots_ = std::max(kRing, std::min(maxTokens, kSmallPass) + c_.SSMConv - 1);
+    if (maxTokens > kSmallPass) {
+        big_slots_ = maxTokens + c_.SSMConv - 1;
+        big_ring_ = static_cast<float *>(dev.alloc_zero(static_cast<size_t>(big_slots_) * c_.DNFusedRows() * 4));
+    }
     const size_t T = maxTokens;
+    if (maxTokens > 16) {
+        work_floats_ = static_cast<int64_t>(T) * (c_.ConvWidth() + 2 * c_.SSMHeadV);
+        work_ = static_cast<float *>(dev.alloc(static_cast<size_t>(work_floats_) * 4));
+    }
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     out_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));
     attn_ = static_cast<float *>(dev.alloc(T * c_.VWidth() * 4));
@@ -661,7 +669,12 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     const bool own_slot = r.n_seq == 1 && r.host_slot >= 0 && r.host_slot < slots_;
     const size_t slot_off = own_slot ? static_cast<size_t>(r.host_slot) : 0;
     const int32_t *slot_tab = own_slot ? nullptr : r.slot;
-    float *ring = ring_[l] + slot_off * ring_slots_ * width;
+    float *slot_ring = ring_[l] + slot_off * ring_slots_ * width;
+    const bool big = nTok > kSmallPass;
+    if (big && (!own_slot || r.spec || !big_ring_))
+        throw Error("llm: DeltaNetGPU: a pass of " + std::to_string(nTok) + " rows is one sequence's plain prompt chunk (no slot table, not rewindable)");
+    float *ring = big ? big_ring_ : slot_ring;
+    const int ring_slots = big ? big_slots_ : ring_slots_;
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor(Model::Blk(l, "ssm_in_fused")).ptr;
     p.x = in;
@@ -677,7 +690,7 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     p.x_stride = c_.NEmbd;
     p.y_stride = width;
     p.seq_len = r.seq_len;
-    p.ring_slots = ring_slots_;
+    p.ring_slots = ring_slots;
     p.ring_stride = width;
     // one row: the projection also leaves the row where the out projection finds its gate
     // without waiting for the position word
@@ -701,9 +714,11 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     s.n_head_v = c_.SSMHeadV;
     s.head_dim = c_.SSMHeadDim;
     s.conv = c_.SSMConv;
-    s.ring_slots = ring_slots_;
+    s.ring_slots = ring_slots;
     s.ring_stride = width;
     s.eps = c_.RMSEps;
+    s.work = work_;   // passes of more than 16 rows of one or more sequences go chunked
+    s.work_floats = work_floats_;
     shv_gemv_q4k_args o{};
     o.w = m_.Tensor(Model::Blk(l, "ssm_out")).ptr;
     o.x = attn_;
@@ -726,9 +741,18 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
         o.pos = r.pos;
         o.slot = slot_tab;
         o.seq_len = r.seq_len;
-        o.ring_slots = ring_slots_;
+        o.ring_slots = ring_slots;
         o.ring_stride = width;
         o.z_ring = 1;
+    }
+    if (big) {
+        // history in, the pass, history out: only the conv's channels (q, k, v) are read back later
+        const int hist = c_.SSMConv - 1;
+        shv_ring_rows_args hin{slot_ring, big_ring_, r.pos, ring_slots_, big_slots_, width, c_.ConvWidth(), -hist, hist};
+        shv_ring_rows_args hout{big_ring_, slot_ring, r.pos, big_slots_, ring_slots_, width, c_.ConvWidth(), nTok - hist, hist};
+        if (labels) labels->insert(labels->end(), {"dn.hist", "dn.qkv", "dn.step", "dn.hist", "dn.out"});
+        return {make_op(SHV_OP_RING_ROWS, hin), make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_DN_STEP, s), make_op(SHV_OP_RING_ROWS, hout),
+                make_op(SHV_OP_GEMV_Q4K, o)};
     }
     if (labels) labels->insert(labels->end(), {"dn.qkv", "dn.step", "dn.out"});
     return {make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_DN_STEP, s), make_op(SHV_OP_GEMV_Q4K, o)};
@@ -1066,9 +1090,12 @@ Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_
     for (size_t i = 0; i < S; i++) ix[i] = static_cast<int32_t>(i);
     dev.upload(slot_ix_, ix.data(), S * 4);
     best_ = static_cast<int32_t *>(dev.alloc_zero(64 * 4));
-    // a pass of more rows than a block takes goes through the attention / DeltaNet blocks in
-    // groups of kBlockRows, layer by layer, and through the experts whole
-    block_rows_ = std::min(rows_max_, kBlockRows);
+    // A long pass goes through every block whole: one projection over all its rows, one walk of
+    // the recurrence, one launch of the attention.  LLM_PASS_GROUPS=1 keeps the older order
+    // instead, groups of kBlockRows rows through the attention / DeltaNet blocks one after the
+    // other (the experts whole either way), for comparison.
+    const char *pg = std::getenv("LLM_PASS_GROUPS");
+    block_rows_ = pg && pg[0] == '1' ? std::min(rows_max_, kBlockRows) : rows_max_;
     // where each group of such a pass stands: [slot][group] positions, written with the
     // sequences' own before a prompt goes through and moved on by the long passes themselves
     groups_ = (rows_max_ + block_rows_ - 1) / block_rows_;
@@ -1132,7 +1159,7 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     }
     p.ops.push_back(make_op(SHV_OP_EMBED, e));
     p.labels.push_back("embed");
-    if (rows > block_rows_ && (kind == kBatch || spec)) throw Error("llm: a pass of " + std::to_string(rows) + " rows is a plain prompt pass; batched and rewindable passes carry up to " + std::to_string(block_rows_));
+    if (rows > kBlockRows && (kind == kBatch || spec)) throw Error("llm: a pass of " + std::to_string(rows) + " rows is a plain prompt pass; batched and rewindable passes carry up to " + std::to_string(kBlockRows));
     for (int l = 0; l < layers_; l++) {
         if (rows <= block_rows_) {
             auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, r, &p.labels) : dn_->Dispatches(l, x_, x_, r, &p.labels);

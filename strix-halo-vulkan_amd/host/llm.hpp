@@ -229,6 +229,10 @@ private:
 class DeltaNetGPU {
 public:
     static constexpr int kRing = 8;  // least projection rows kept per slot: up to 5 rows a pass + 3 of history
+    // A pass of more rows than this (one sequence's prompt chunk) keeps its projection rows in one
+    // ring sized for the whole pass and shared by all layers and slots; the conv's three rows of
+    // history come from the slot's own ring before the step, and the pass's last three go back after.
+    static constexpr int kSmallPass = 64;
     // planes > 1 stages the state copies a rewindable pass needs (WithDNSpecSlots,
     // llm/gpu_deltanet.go:380); plane is the device array naming each slot's committed copy.
     DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, int32_t *pos, int planes = 1, int32_t *plane = nullptr);
@@ -264,6 +268,10 @@ private:
     int32_t *pos_, *plane_;
     float *in_, *out_, *attn_;
     float *row_ = nullptr;               // the projection row of a one-row pass, also kept outside the ring (the out projection's gate)
+    float *big_ring_ = nullptr;          // the long pass's ring, [big_slots_][DNFusedRows]
+    int big_slots_ = 0;
+    float *work_ = nullptr;              // what the chunked step prepares of a pass's rows (q^, k^, v, log g, beta)
+    int64_t work_floats_ = 0;
     std::vector<float *> ring_, state_;  // per layer (nullptr on attention layers)
     uint64_t state_bytes_ = 0;
 };

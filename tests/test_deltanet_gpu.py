@@ -52,7 +52,8 @@ class DnCase:
         self.d_conv, self.d_a, self.d_dt = c.upload(self.conv1d), c.upload(self.a), c.upload(self.dt_bias)
         self.d_norm = c.upload(self.norm)
 
-    def step_ops(self, d_x, d_ring, d_state, d_attn, d_res, d_pos, d_slot, n_seq, seq_len, ring_slots):
+    def step_ops(self, d_x, d_ring, d_state, d_attn, d_res, d_pos, d_slot, n_seq, seq_len, ring_slots, work=None):
+        """work: a scratch buffer; with it a pass of more than 16 rows takes the chunked kernels."""
         n_tok = n_seq * seq_len
         return [
             A.make_op(A.OP_GEMV_Q4K, A.gemv_args(self.d_fused, d_x, d_ring, self.width, self.H, n_tok,
@@ -61,7 +62,8 @@ class DnCase:
             A.make_op(A.OP_DN_STEP, A.DnStepArgs(d_ring.ptr, self.d_conv.ptr, self.d_a.ptr, self.d_dt.ptr,
                                                  d_state.ptr, d_attn.ptr, d_pos.ptr,
                                                  A.ptr(d_slot), n_seq, seq_len, self.hk, self.hv,
-                                                 self.d, self.conv, ring_slots, self.width, EPS, 0)),
+                                                 self.d, self.conv, ring_slots, self.width, EPS, 0, None, 0, 0,
+                                                 A.ptr(work), work.nbytes // 4 if work is not None else 0)),
             A.make_op(A.OP_GEMV_Q4K, A.gemv_args(self.d_out, d_attn, d_res, self.H, self.vw, n_tok,
                                                  prologue=A.PRO_GATED_NORM, gamma=self.d_norm,
                                                  z=d_ring.at(0), head_dim=self.d, eps=EPS)),
@@ -170,6 +172,64 @@ def test_rows_in_one_call_equal_single_steps(ctx, T, slots, pos0):
     for t in range(T):
         assert O.rel_l2(got[t], want_attn[t]) <= TOL, t
     assert O.rel_l2(d_state.read(np.float32, s_state.size), s_state) <= TOL
+
+
+@pytest.mark.parametrize("T,pos0,n_seq", [(17, 0, 1), (64, 0, 1), (150, 0, 1), (257, 41, 1), (64, 27, 1), (100, 5, 3), (2048, 3, 1)])
+def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
+    """With a workspace a pass of more than 16 rows goes 64 rows at a time on the matrix cores (the
+    delta rule's closed form over a chunk).  Against the oracle's row-by-row rule (every row's
+    output and the final state within 1e-3), and against this library's own row-by-row kernel on
+    the same inputs, which it must match far closer than that: whole chunks, ragged ones, several
+    chunks, a start in mid-sequence (history rows, a state that has already run), several sequences
+    in one call, and a 2048-row pass."""
+    case = DnCase(ctx, seed=300 + T + n_seq)
+    case.upload()
+    rng = case.rng
+    slots = T + 3
+    xn = rng.standard_normal((n_seq, T, case.H)).astype(np.float32)
+    started = pos0 > 0
+    hist = rng.standard_normal((n_seq, 3, case.width)).astype(np.float32) if started else np.zeros((n_seq, 3, case.width), np.float32)
+    s0 = (rng.standard_normal((n_seq, case.hv, case.d, case.d)) * 0.1).astype(np.float32) if started else np.zeros((n_seq, case.hv, case.d, case.d), np.float32)
+    pos = (pos0 + 7 * np.arange(n_seq)).astype(np.int32) if started else np.zeros(n_seq, np.int32)
+    ring = np.zeros((n_seq, slots, case.width), np.float32)
+    for b in range(n_seq):
+        for i in range(3):
+            if started:
+                ring[b, (pos[b] - 3 + i) % slots] = hist[b, i]
+    c = ctx
+    d_x, d_pos = c.upload(xn.reshape(n_seq * T, case.H)), c.upload(pos)
+    results = []
+    for chunked in (True, False):
+        d_ring, d_state = c.upload(ring), c.upload(s0)
+        d_attn, d_res = c.alloc(n_seq * T * case.vw * 4), c.alloc(n_seq * T * case.H * 4)
+        work = c.alloc(n_seq * T * (case.cw + 2 * case.hv) * 4) if chunked else None
+        ops = case.step_ops(d_x, d_ring, d_state, d_attn, d_res, d_pos, None, n_seq, T, slots, work=work)[:2]
+        c.dispatch_multi(ops)
+        results.append((d_attn.read(np.float32, n_seq * T * case.vw).reshape(n_seq, T, case.vw),
+                        d_state.read(np.float32, s0.size).reshape(s0.shape)))
+        for b in (d_ring, d_state, d_attn, d_res):
+            b.free()
+        if work is not None:
+            work.free()
+    (got_attn, got_state), (seq_attn, seq_state) = results
+    e_a, e_s = O.rel_l2(got_attn, seq_attn), O.rel_l2(got_state, seq_state)
+    print(f"deltanet chunked T={T} x{n_seq}: against the row-by-row kernel: rows {e_a:.3e} state {e_s:.3e}")
+    assert e_a <= 2e-5 and e_s <= 2e-5
+    for b in range(n_seq if T <= 300 else 0):
+        conv_state = np.ascontiguousarray(hist[b, :, :case.cw].T)
+        s_state = s0[b].copy()
+        _, want_attn = case.oracle(xn[b], conv_state, s_state)
+        worst = max(O.rel_l2(got_attn[b, t], want_attn[t]) for t in range(T))
+        assert worst <= TOL, (b, worst)
+        assert O.rel_l2(got_state[b], s_state) <= TOL, b
+    if T > 300:
+        # the long pass against the oracle too (a few seconds of CPU)
+        conv_state = np.ascontiguousarray(hist[0, :, :case.cw].T)
+        s_state = s0[0].copy()
+        _, want_attn = case.oracle(xn[0], conv_state, s_state)
+        assert O.rel_l2(got_attn[0], want_attn) <= TOL
+        assert max(O.rel_l2(got_attn[0, t], want_attn[t]) for t in range(0, T, 97)) <= TOL
+        assert O.rel_l2(got_state[0], s_state) <= TOL
 
 
 def test_dn_step_refuses_unsupported_shapes(ctx):
