@@ -226,7 +226,7 @@ typedef struct {
  * routes its token from them exactly as the router would, and the selection is also stored to
  * topk [T][n_used] and weights [T][n_used+1] for the down projection; otherwise topk is read.
  * A pass of many rows (128 and more; SHV_MOE_GROUP_MIN) whose topk is given, with n_expert stated
- * and a `group` workspace of n_expert + 1 + T * n_used ints, is grouped by expert on the matrix
+ * and a `group` workspace of 2 * n_expert + 1 + T * n_used ints, is grouped by expert on the matrix
  * cores: an expert's weights are read once per 48 tokens that chose it (the prompt arm of
  * llm_moe_gemv.comp). */
 typedef struct {

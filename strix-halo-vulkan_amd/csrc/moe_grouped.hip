@@ -8,8 +8,8 @@
 //   moe_up_grouped_kernel     a block = (expert, half of its ffn rows) and up to 48 of its tokens
 //                             at a time: their xn rows go through LDS as matrix-core operands
 //                             (two halves hi + lo, as the projections do) in slabs of 512 columns,
-//                             each wave streams one gate tile of 16 rows and the matching up
-//                             tile, forms a sub-block's weights once (as the whole numbers n * sc,
+//                             each wave streams two gate tiles of 16 rows and the matching up
+//                             tiles, forms a sub-block's weights once (as the whole numbers n * sc,
 //                             exact in binary16) for all three token tiles, keeps one matrix
 //                             accumulator per super-block, SwiGLU in registers, act[pair] out
 //   moe_down_grouped_kernel   a block = (expert, quarter of n_embd rows): act rows staged the
@@ -28,18 +28,20 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 16;
+constexpr int kWaves = 8;       // 256 registers a lane: the streams, the accumulators of four row tiles and the operands fit without spilling
 constexpr int kThreads = kWaves * 64;
 constexpr int kTT = 3;            // matrix-core tiles of 16 tokens a block multiplies per pass over the weights
 constexpr int kTok = 16 * kTT;    // tokens of such a pass
-constexpr int kTiles = 2;         // weight row tiles of 16 a wave owns
+constexpr int kTiles = 4;         // weight row tiles of 16 a wave owns
 constexpr int kSlab = 512;        // columns of the tokens' rows staged at a time
 constexpr int kSlabSubs = kSlab / 32;
 constexpr int kFrag = 64 * 16;    // one operand: a lane's eight halves
 constexpr int kMaxExperts = 1024;
 
 // The caller's `group` workspace: [0, n_expert] start of each expert's list (one more: the total),
-// then n_tok * n_used pair ids (token * (n_used + 1) + slot).  A list's order is whatever the
+// then n_tok * n_used pair ids (token * (n_used + 1) + slot), then the experts in the order their
+// blocks are launched: longest list first, so that the blocks which walk their weights two or
+// three times start early and the launch does not end on them.  A list's order is whatever the
 // arrivals made it; every pair's products are formed in a matrix-core column of their own, so no
 // value depends on it.
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, int n_tok, int n_used, int n_expert, int32_t *group) {
@@ -63,6 +65,17 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
     }
     __syncthreads();
     for (int e = tid; e <= n_expert; e += blockDim.x) group[e] = s_cnt[e];
+    // rank by list length, longer first, equal lengths by index: an expert's place in the launch
+    int32_t *order = group + n_expert + 1 + n_pairs;
+    for (int e = tid; e < n_expert; e += blockDim.x) {
+        const int ce = s_cnt[e + 1] - s_cnt[e];
+        int rank = 0;
+        for (int o = 0; o < n_expert; o++) {
+            const int co = s_cnt[o + 1] - s_cnt[o];
+            rank += (co > ce || (co == ce && o < e)) ? 1 : 0;
+        }
+        order[rank] = e;
+    }
     __syncthreads();
     int32_t *list = group + n_expert + 1;
     for (int i = tid; i < n_pairs; i += blockDim.x) {
@@ -81,28 +94,42 @@ __device__ __forceinline__ void gather_slab(const float *const *rows_s, int m, i
     const int tid = threadIdx.x;
     const int c = 4 * (tid % QPR);
     const int sub = c >> 5, kb = (c & 31) >> 3, qh = (c & 7) >> 2;
-    for (int i0 = 0; i0 < m; i0 += RPI) {
-        const int i = i0 + tid / QPR;
-        const bool on = i < m;
-        float4 v = {0.f, 0.f, 0.f, 0.f};
-        if (on) v = *reinterpret_cast<const float4 *>(rows_s[i] + col0 + c);
-        float sum = (v.x + v.y) + (v.z + v.w);
-        sum += __shfl_xor(sum, 1, 64);
-        sum += __shfl_xor(sum, 2, 64);
-        sum += __shfl_xor(sum, 4, 64);
-        if (on) {
-            if ((c & 31) == 0) sxs[sub * kTok + i] = sum;
-            const float o[4] = {v.x, v.z, v.y, v.w};
-            half4_t h, l;
+    // six rows' quads are asked for before the first is used: two memory latencies a slab, not one a row
+    constexpr int NI = kTok / RPI, NB = 6;
+    static_assert(kTok % RPI == 0 && NI % NB == 0, "whole batches");
+#pragma unroll 1
+    for (int b0 = 0; b0 < NI; b0 += NB) {
+        if (b0 * RPI >= m) break;
+        float4 vv[NB];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const _Float16 hi = static_cast<_Float16>(o[j]);
-                h[j] = hi;
-                l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+        for (int it = 0; it < NB; it++) {
+            const int i = (b0 + it) * RPI + tid / QPR;
+            vv[it] = *reinterpret_cast<const float4 *>(rows_s[i < m ? i : 0] + col0 + c);
+        }
+#pragma unroll
+        for (int it = 0; it < NB; it++) {
+            const int i = (b0 + it) * RPI + tid / QPR;
+            const bool on = i < m;
+            float4 v = vv[it];
+            if (!on) v = float4{0.f, 0.f, 0.f, 0.f};
+            float sum = (v.x + v.y) + (v.z + v.w);
+            sum += __shfl_xor(sum, 1, 64);
+            sum += __shfl_xor(sum, 2, 64);
+            sum += __shfl_xor(sum, 4, 64);
+            if (on) {
+                if ((c & 31) == 0) sxs[sub * kTok + i] = sum;
+                const float o[4] = {v.x, v.z, v.y, v.w};
+                half4_t h, l;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const _Float16 hi = static_cast<_Float16>(o[j]);
+                    h[j] = hi;
+                    l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+                }
+                char *e = frags + static_cast<size_t>((sub * 2) * kTT + (i >> 4)) * kFrag + (kb * 16 + (i & 15)) * 16 + qh * 8;
+                *reinterpret_cast<half4_t *>(e) = h;
+                *reinterpret_cast<half4_t *>(e + kTT * kFrag) = l;
             }
-            char *e = frags + static_cast<size_t>((sub * 2) * kTT + (i >> 4)) * kFrag + (kb * 16 + (i & 15)) * 16 + qh * 8;
-            *reinterpret_cast<half4_t *>(e) = h;
-            *reinterpret_cast<half4_t *>(e + kTT * kFrag) = l;
         }
     }
 }
@@ -251,12 +278,12 @@ struct Unit {
     int part;
     int first, count;  // positions in the expert's list (routed) or token numbers (shared)
 };
-__device__ __forceinline__ Unit unit_of(int b, int parts, int n_expert, int n_tok, const int32_t *group) {
+__device__ __forceinline__ Unit unit_of(int b, int parts, int n_expert, int n_tok, int n_used, const int32_t *group) {
     Unit u;
     const int shared = parts * ((n_tok + kTok - 1) / kTok);  // the shared expert's blocks come first: all of them have work
     if (b >= shared) {
         b -= shared;
-        u.expert = b / parts;
+        u.expert = group[n_expert + 1 + n_tok * n_used + b / parts];
         u.part = b % parts;
         u.first = group[u.expert];
         u.count = group[u.expert + 1] - u.first;
@@ -283,9 +310,9 @@ struct Staging {
 };
 constexpr size_t kGroupedLds = static_cast<size_t>(kSlabSubs) * 2 * kTT * kFrag + static_cast<size_t>(kSlabSubs) * kTok * 4 + kTok * sizeof(float *) + kTok * 4;
 
-// grid: n_expert * parts + parts * ceil(n_tok / 48) blocks of 16 waves, parts = ffn / 256; K = n_embd.
-// A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tile w and
-// the up tile of the same rows, so SwiGLU stays in registers.
+// grid: n_expert * parts + parts * ceil(n_tok / 48) blocks of 8 waves, parts = ffn / 256; K = n_embd.
+// A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tiles 2w and
+// 2w + 1 and the up tiles of the same rows, so SwiGLU stays in registers.
 template <int K>
 __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_args a) {
     extern __shared__ __align__(16) char smem[];
@@ -294,14 +321,14 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int parts = a.ffn / 256;
-    const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, group);
+    const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, a.n_used, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row = u.part * 256 + wave * 16 + n;   // this lane's row of the expert, gate and up alike
+    const int row = u.part * 256 + wave * 32 + n;   // this lane's first row of the expert, gate and up alike; its second is 16 on
     const size_t wrow = static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.ffn + row;
     const char *gp = static_cast<const char *>(u.expert < 0 ? a.gate_sh : a.gate_exps) + wrow * row_bytes;
     const char *up = static_cast<const char *>(u.expert < 0 ? a.up_sh : a.up_exps) + wrow * row_bytes;
-    const char *rp[kTiles] = {gp, up};
+    const char *rp[kTiles] = {gp, gp + 16 * row_bytes, up, up + 16 * row_bytes};
     for (int t0 = 0; t0 < u.count; t0 += kTok) {
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {
@@ -317,8 +344,11 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
             for (int j = 0; j < 4; j++) {
                 const int i = 16 * tt + 4 * kb + j;
                 if (i < m) {
-                    const float gv = y[0][tt][j];
-                    a.act[static_cast<size_t>(st.pair_s[i]) * a.ffn + row] = gv * sigmoid_exact(gv) * y[1][tt][j];
+#pragma unroll
+                    for (int r = 0; r < 2; r++) {
+                        const float gv = y[r][tt][j];
+                        a.act[static_cast<size_t>(st.pair_s[i]) * a.ffn + row + 16 * r] = gv * sigmoid_exact(gv) * y[2 + r][tt][j];
+                    }
                 }
             }
         __syncthreads();   // the list is read to the end before the next one replaces it
@@ -326,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
 }
 
 // grid: n_expert * parts + parts * ceil(n_tok / 48) blocks, parts = n_embd / 512: a part is 512
-// output rows = 32 tiles, wave w takes tiles 2w and 2w + 1.  K = ffn.
+// output rows = 32 tiles, wave w takes tiles 4w .. 4w + 3.  K = ffn.
 template <int K>
 __global__ __launch_bounds__(kThreads) void moe_down_grouped_kernel(shv_moe_down_args a) {
     extern __shared__ __align__(16) char smem[];
@@ -336,13 +366,13 @@ __global__ __launch_bounds__(kThreads) void moe_down_grouped_kernel(shv_moe_down
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int parts = a.n_embd / 512;
-    const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, group);
+    const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, a.n_used, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row0 = u.part * 512 + wave * 32 + n;
+    const int row0 = u.part * 512 + wave * 64 + n;
     const char *base = static_cast<const char *>(u.expert < 0 ? a.down_sh : a.down_exps) +
                        (static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.n_embd + row0) * row_bytes;
-    const char *rp[kTiles] = {base, base + 16 * row_bytes};
+    const char *rp[kTiles] = {base, base + 16 * row_bytes, base + 32 * row_bytes, base + 48 * row_bytes};
     for (int t0 = 0; t0 < u.count; t0 += kTok) {
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {

@@ -458,7 +458,7 @@ MoEGPU::MoEGPU(Device &dev, const Model &m, int maxTokens) : dev_(dev), m_(m), c
     // passes of many rows go grouped by expert on the matrix cores and need the per-expert lists
     // and every (token, slot)'s down products before they are summed
     if (maxTokens > kBlockRows) {
-        group_ = static_cast<int32_t *>(dev.alloc((c_.NExpert + 1 + T * c_.NExpertUsed) * 4));
+        group_ = static_cast<int32_t *>(dev.alloc((2 * c_.NExpert + 1 + T * c_.NExpertUsed) * 4));
         pairs_ = static_cast<float *>(dev.alloc(T * (c_.NExpertUsed + 1) * c_.NEmbd * 4));
     }
     act_bytes_ = T * (3ull * c_.NEmbd + c_.NExpert + 1 + 2 * c_.NExpertUsed + 1 + (c_.NExpertUsed + 1ull) * c_.FFNExpert) * 4;

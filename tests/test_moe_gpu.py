@@ -84,7 +84,7 @@ class MoeCase:
                            d["res"].ptr if residual else None, out.ptr, T, H, used, ffn, H, H, self.types[2], self.types[5],
                            E, None, None)
         if grouped:
-            group, pairs = c.alloc((E + 1 + T * used) * 4), c.alloc(T * (used + 1) * H * 4)
+            group, pairs = c.alloc((2 * E + 1 + T * used) * 4), c.alloc(T * (used + 1) * H * 4)
             ua.group = da.group = group.ptr
             da.pairs = pairs.ptr
         ops = [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
