@@ -441,7 +441,7 @@ __device__ __forceinline__ size_t out_offset(const shv_gemv_q4k_args &a, int t) 
 // The same for a pass of up to 64 rows a group, in the slab order gemm_wide_kernel streams.
 // grid: (k/256, 16 quartets of rows, groups of 64 rows), 256 threads: a wave takes one row's 64
 // quads of one super-block's columns; rows a group does not have are written as zeros.
-__global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args a, char *staged) {
+__global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args a, char *staged, float *x_out) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = a.k, kp = blockIdx.x, grp = blockIdx.z;
     const int t0 = grp * kWideTok;
@@ -466,6 +466,8 @@ __global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args 
     const int sub = (c & 127) >> 5, kb = (c & 31) >> 3, qh = (c & 7) >> 2;
     float x[4] = {0.f, 0.f, 0.f, 0.f};
     if (tl < nt) pro_quad(a, t0 + tl, c, scale, x);
+    // the transformed row itself, for a caller that also needs it as plain float32 (the router's xn)
+    if (x_out && tl < nt) *reinterpret_cast<float4 *>(x_out + static_cast<size_t>(t0 + tl) * K + c) = float4{x[0], x[1], x[2], x[3]};
     float sum = (x[0] + x[1]) + (x[2] + x[3]);
     sum += __shfl_xor(sum, 1, 64);
     sum += __shfl_xor(sum, 2, 64);
@@ -651,6 +653,110 @@ __global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a,
     }
 }
 
+// ------------------------------------------------------------ the router of a long pass -------
+// logits[t][e] = xn[t] . W[e] for float32 rows W (the router's experts and, as one more row, the
+// shared expert's gate) against the staged rows of a pass: the same streaming of slabs as above,
+// the second operand formed from 32 bytes of float32 a lane instead of from nibbles.  A float32
+// weight enters as two binary16 values (hi, and the remainder scaled by 2^11 so that it stays a
+// normal number); x_hi*w_hi + x_lo*w_hi run in one accumulator, x_hi*w_lo in a second one that
+// carries the 2^11: about 22 bits of either operand, float32 sums.
+// grid: (row blocks of NW*16 rows) x groups, NW waves; wave w owns one tile of 16 rows.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void router_wide_kernel(const float *W, const float *extra_row, int n_rows, int K, int n_tok, const char *staged_all,
+                                                              float *logits, int logits_stride, int groups) {
+    extern __shared__ __align__(16) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, kb = lane >> 4;
+    constexpr int NTHR = NW * 64;
+    const int grp = blockIdx.x % groups, xb = blockIdx.x / groups;
+    const int t0 = grp * kWideTok;
+    const int nt = n_tok - t0 < kWideTok ? n_tok - t0 : kWideTok;
+    const char *staged = staged_all + static_cast<size_t>(grp) * wide_region(K);
+    const int row = (xb * NW + wave) * kTileRows + n;
+    // rows past the end read the last row (their results are dropped); row n_rows - 1 may live apart
+    const int rr = row < n_rows ? row : n_rows - 1;
+    const float *wp = (extra_row && rr == n_rows - 1) ? extra_row : W + static_cast<size_t>(rr) * K;
+    const int steps = K / 128;
+    constexpr int kVec = kWideSlab / 16;
+    constexpr int kPer = kWideSlabA / 16 / NTHR;
+    static_assert(kPer * NTHR * 16 == kWideSlabA && kVec - kPer * NTHR == 64, "slab copy layout");
+    float4 w[4][2], wn[4][2];
+    auto load_w = [&](int s, float4 (&dst)[4][2]) {
+#pragma unroll
+        for (int sub = 0; sub < 4; sub++) {
+            const float *p = wp + s * 128 + sub * 32 + kb * 8;
+            dst[sub][0] = *reinterpret_cast<const float4 *>(p);
+            dst[sub][1] = *reinterpret_cast<const float4 *>(p + 4);
+        }
+    };
+    load_w(0, w);
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(staged);
+        uint4 *dst = reinterpret_cast<uint4 *>(smem);
+        for (int i = tid; i < kVec; i += NTHR) dst[i] = src[i];
+    }
+    __syncthreads();
+    float4_t ym[4], yl[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++) ym[tt] = yl[tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < steps; s++) {
+        const int cur = s & 1;
+        const bool more = s + 1 < steps;
+        uint4 an[kPer], asx;
+        {
+            const int sn = more ? s + 1 : s;
+            const uint4 *src = reinterpret_cast<const uint4 *>(staged + static_cast<size_t>(sn) * kWideSlab);
+#pragma unroll
+            for (int i = 0; i < kPer; i++) an[i] = src[tid + i * NTHR];
+            asx = src[kPer * NTHR + (tid & 63)];
+            load_w(sn, wn);
+        }
+        const char *A = smem + cur * kWideSlab;
+#pragma unroll
+        for (int sub = 0; sub < 4; sub++) {
+            // slot order of the eight columns, as the rows were staged: [0, 2, 1, 3, 4, 6, 5, 7]
+            const float o[8] = {w[sub][0].x, w[sub][0].z, w[sub][0].y, w[sub][0].w, w[sub][1].x, w[sub][1].z, w[sub][1].y, w[sub][1].w};
+            half8_t bh, bl;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const _Float16 hi = static_cast<_Float16>(o[j]);
+                bh[j] = hi;
+                bl[j] = static_cast<_Float16>((o[j] - static_cast<float>(hi)) * 2048.f);
+            }
+            // all four token tiles, whatever the group holds: rows it does not have were staged as zeros
+#pragma unroll
+            for (int tt = 0; tt < 4; tt++) {
+                const char *f = A + static_cast<size_t>((sub * 4 + tt) * 2) * kWideFrag + lane * 16;
+                const half8_t xh = *reinterpret_cast<const half8_t *>(f);
+                const half8_t xl = *reinterpret_cast<const half8_t *>(f + kWideFrag);
+                ym[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, bh, ym[tt], 0, 0, 0);
+                ym[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, bh, ym[tt], 0, 0, 0);
+                yl[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, bl, yl[tt], 0, 0, 0);
+            }
+        }
+        if (more) {
+            uint4 *dst = reinterpret_cast<uint4 *>(smem + (cur ^ 1) * kWideSlab);
+#pragma unroll
+            for (int i = 0; i < kPer; i++) dst[tid + i * NTHR] = an[i];
+            if (tid < 64) dst[kPer * NTHR + tid] = asx;
+#pragma unroll
+            for (int sub = 0; sub < 4; sub++) {
+                w[sub][0] = wn[sub][0];
+                w[sub][1] = wn[sub][1];
+            }
+        }
+        __syncthreads();
+    }
+    if (row >= n_rows) return;
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int tok = tt * kTileRows + 4 * kb + j;
+            if (tok < nt) logits[static_cast<size_t>(t0 + tok) * logits_stride + row] = fmaf(yl[tt][j], 1.f / 2048.f, ym[tt][j]);
+        }
+}
+
 // The column parts of a split product added up in a fixed order.  grid: (ceil(n/256), nt), one
 // wave a block; a thread takes four neighbouring outputs, with 16-byte moves when the row count
 // and the addresses allow them.
@@ -773,6 +879,41 @@ int launch_wide_all(shv_ctx *ctx, const shv_gemv_q4k_args &a, int groups) {
 
 }  // namespace
 
+// The router of a pass of many rows: xn = rmsnorm(h) * gamma staged (and written out as float32),
+// then every token's n_expert (+ 1, the shared expert's gate) logits on the matrix cores.
+bool shv_router_wide_covers(const shv_ctx *ctx, const shv_moe_router_args &a) {
+    if (!ctx->gemm_stage || a.n_tok < 128 || !a.gamma || !a.xn) return false;
+    if (a.n_embd % 256 != 0 || a.n_embd < 256 || a.h_stride % 4 != 0) return false;
+    if (!shv_aligned16(a.h) || !shv_aligned16(a.gamma) || !shv_aligned16(a.xn) || !shv_aligned16(a.router) || (a.shared_gate && !shv_aligned16(a.shared_gate))) return false;
+    const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
+    return groups * wide_region(a.n_embd) <= static_cast<size_t>(shv_ctx::kGemmStageBytes);
+}
+
+int shv_launch_router_wide(shv_ctx *ctx, const shv_moe_router_args &a) {
+    shv_gemv_q4k_args g{};
+    g.x = a.h;
+    g.gamma = a.gamma;
+    g.k = a.n_embd;
+    g.n_tok = a.n_tok;
+    g.prologue = SHV_PRO_RMSNORM;
+    g.eps = a.eps;
+    g.x_stride = a.h_stride;
+    const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
+    SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(g.k / 256, kWideTok / 4, groups), dim3(256), 0, g, ctx->gemm_stage, a.xn);
+    constexpr int NW = 4;
+    const int n_rows = a.n_expert + (a.shared_gate ? 1 : 0);
+    const int bx = (n_rows + NW * kTileRows - 1) / (NW * kTileRows);
+    const size_t lds = 2 * kWideSlab;
+    static bool raised = false;
+    if (!raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&router_wide_kernel<NW>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        raised = true;
+    }
+    SHV_LAUNCH(ctx, (router_wide_kernel<NW>), dim3(bx * groups), dim3(NW * 64), lds, a.router, a.shared_gate, n_rows, a.n_embd, a.n_tok,
+               static_cast<const char *>(ctx->gemm_stage), a.logits, a.n_expert + 1, groups);
+    return SHV_OK;
+}
+
 // Whether the matrix-core kernel takes this call: arguments are already validated by the GEMV's
 // launcher, which falls back to its own multi-row kernel otherwise.
 bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a) {
@@ -799,7 +940,7 @@ int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     if (a.n_tok > cap && ctx->gemm_stage && (a.prologue != SHV_PRO_GATED_NORM || 256 % a.head_dim == 0)) {
         const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
         SHV_REQUIRE(groups * wide_region(a.k) <= static_cast<size_t>(shv_ctx::kGemmStageBytes), "gemm_q4k: %d rows of %d columns do not fit the staging buffer", a.n_tok, a.k);
-        SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(a.k / 256, kWideTok / 4, groups), dim3(256), 0, a, ctx->gemm_stage);
+        SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(a.k / 256, kWideTok / 4, groups), dim3(256), 0, a, ctx->gemm_stage, static_cast<float *>(nullptr));
         if (groups >= 4) return launch_wide_all<8, 1>(ctx, a, groups);
         for (int g = 0; g < groups; g++) {
             const int t0 = g * kWideTok;

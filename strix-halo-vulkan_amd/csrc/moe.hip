@@ -873,6 +873,16 @@ int shv_launch_moe_router(shv_ctx *ctx, const shv_moe_router_args *pa) {
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed && a.n_used <= a.n_expert, "moe_router: n_used %d of %d (at most %d)", a.n_used, a.n_expert, kMaxUsed);
     SHV_REQUIRE(a.h_stride >= a.n_embd, "moe_router: h_stride %d < n_embd %d", a.h_stride, a.n_embd);
     SHV_REQUIRE(shv_aligned16(a.router) && shv_aligned16(a.shared_gate), "moe_router: router and shared_gate must be 16-byte aligned");
+    // a pass of many rows: the logits on the matrix cores
+    if (shv_router_wide_covers(ctx, a)) {
+        const int rc = shv_launch_router_wide(ctx, a);
+        if (rc != SHV_OK) return rc;
+        if (!a.defer_route) {
+            if (a.n_expert > 64 && a.n_expert <= kRouteBlock) SHV_LAUNCH(ctx, moe_route_block_kernel, dim3(a.n_tok), dim3(kRouteBlock), 0, a);
+            else SHV_LAUNCH(ctx, moe_route_kernel, dim3(a.n_tok), dim3(64), 0, a);
+        }
+        return SHV_OK;
+    }
     // four rows a wave only where that still leaves a few hundred blocks
     const bool many = a.n_tok >= 128;
     const int rw = many ? 4 : 1, tpb = a.n_tok >= 512 ? kRouterTokensMany : many ? 8 : kRouterTokens;

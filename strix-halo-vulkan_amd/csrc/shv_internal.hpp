@@ -109,6 +109,8 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
 // the matrix-core kernel for passes of two rows and more (gemm_q4k.hip)
 bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a);
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a);
+bool shv_router_wide_covers(const shv_ctx *ctx, const shv_moe_router_args &a);
+int shv_launch_router_wide(shv_ctx *ctx, const shv_moe_router_args &a);
 int shv_launch_dequant_q4k(shv_ctx *ctx, const shv_dequant_q4k_args *a);
 int shv_launch_dequant(shv_ctx *ctx, const shv_dequant_args *a);
 int shv_launch_gemv(shv_ctx *ctx, const shv_gemv_args *a);
