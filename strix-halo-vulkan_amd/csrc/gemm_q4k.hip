@@ -653,6 +653,178 @@ __global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a,
     }
 }
 
+// The same product for a pass of many groups, every group in one launch, with the second operand
+// formed as the experts' grouped kernels form theirs: a sub-block's eight weights a lane become the
+// whole numbers n * sc (exact in binary16), one matrix accumulator runs over a super-block and takes
+// its d at the end, and the min term is the only per-sub-block vector work: half the vector
+// instructions per matrix instruction of the kernel above, and no branch inside a step.
+// grid: (row blocks of NW*R*16 rows) x groups; all four token tiles are multiplied whatever the
+// group holds (rows it does not have were staged as zeros).
+template <int NW, int R>
+__global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a, const char *staged_all, int groups) {
+    extern __shared__ __align__(16) char smem[];
+    size_t *yoffs = reinterpret_cast<size_t *>(smem + 2 * kWideSlab);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, kb = lane >> 4;
+    const int sbs = a.k / SHV_Q4K_BLOCK;
+    const size_t row_bytes = static_cast<size_t>(sbs) * SHV_Q4K_BYTES;
+    constexpr int NTHR = NW * 64;
+    const int grp = blockIdx.x % groups, xb = blockIdx.x / groups;
+    const int t0 = grp * kWideTok;
+    const int nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;
+    const char *staged = staged_all + static_cast<size_t>(grp) * wide_region(a.k);
+    const int row0 = (xb * NW + wave) * (R * kTileRows);
+    const int steps = a.k / 128;
+
+    const char *rp[R];
+    uint4 hdr[R], hdrn[R];
+    uint2 q[R][2], qn[R][2];
+    // step s: the 128 columns s*128.. of the row = groups 2(s&1), 2(s&1)+1 of super-block s>>1
+    auto load_q = [&](int s, uint2 (&dst)[R][2]) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int g = 0; g < 2; g++)
+                dst[r][g] = *reinterpret_cast<const uint2 *>(rp[r] + static_cast<size_t>(s >> 1) * SHV_Q4K_BYTES + 16 + ((s & 1) * 2 + g) * 32 + kb * 8);
+    };
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r * kTileRows + n;
+        rp[r] = static_cast<const char *>(a.w) + static_cast<size_t>(row < a.n ? row : a.n - 1) * row_bytes;
+        hdr[r] = *reinterpret_cast<const uint4 *>(rp[r]);
+    }
+    load_q(0, q);
+    if (tid < nt) yoffs[tid] = out_offset(a, t0 + tid);
+    constexpr int kVec = kWideSlab / 16;
+    constexpr int kPer = kWideSlabA / 16 / NTHR;
+    static_assert(kPer * NTHR * 16 == kWideSlabA && kVec - kPer * NTHR == 64, "slab copy layout");
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(staged);
+        uint4 *dst = reinterpret_cast<uint4 *>(smem);
+        for (int i = tid; i < kVec; i += NTHR) dst[i] = src[i];
+    }
+    __syncthreads();
+
+    const NibbleConsts nc = nibble_consts();
+    float4_t y[R][4], acc[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) y[r][tt] = acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int s = 0; s < steps; s++) {
+        const int cur = s & 1;
+        const bool more = s + 1 < steps;
+        uint4 an[kPer], asx;
+        {
+            const int sn = more ? s + 1 : s;
+            const uint4 *src = reinterpret_cast<const uint4 *>(staged + static_cast<size_t>(sn) * kWideSlab);
+#pragma unroll
+            for (int i = 0; i < kPer; i++) an[i] = src[tid + i * NTHR];
+            asx = src[kPer * NTHR + (tid & 63)];
+            load_q(sn, qn);
+            if (s & 1) {
+#pragma unroll
+                for (int r = 0; r < R; r++) hdrn[r] = *reinterpret_cast<const uint4 *>(rp[r] + static_cast<size_t>(sn >> 1) * SHV_Q4K_BYTES);
+            }
+        }
+        const char *A = smem + cur * kWideSlab;
+        const float *sxs = reinterpret_cast<const float *>(A + kWideSlabA);
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            uint32_t sc[R], mn[R];
+            float dmin[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                q4k_group_scale_min(hdr[r], (s & 1) * 2 + g, sc[r], mn[r]);
+                dmin[r] = f16_bits_to_f32(hdr[r].x >> 16);
+            }
+#pragma unroll
+            for (int hi = 0; hi < 2; hi++) {
+                const int sub = g * 2 + hi;
+                half8_t b[R];
+                float dm[R];
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const uint32_t q0 = q[r][g].x, q1 = q[r][g].y;
+                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                    u32x4 v;
+                    // slot order of the eight columns: bytes [0, 2, 1, 3, 4, 6, 5, 7]
+                    if (hi == 0) {
+                        v.x = ((q0 << 4) & nc.mask) | nc.one; v.y = ((q0 >> 4) & nc.mask) | nc.one;
+                        v.z = ((q1 << 4) & nc.mask) | nc.one; v.w = ((q1 >> 4) & nc.mask) | nc.one;
+                    } else {
+                        v.x = (q0 & nc.mask) | nc.one; v.y = ((q0 >> 8) & nc.mask) | nc.one;
+                        v.z = (q1 & nc.mask) | nc.one; v.w = ((q1 >> 8) & nc.mask) | nc.one;
+                    }
+                    const _Float16 s16 = static_cast<_Float16>(static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu));
+                    b[r] = (__builtin_bit_cast(half8_t, v) - static_cast<half8_t>(static_cast<_Float16>(64.f))) * static_cast<half8_t>(s16);
+                    dm[r] = dmin[r] * static_cast<float>(hi ? mn[r] >> 8 : mn[r] & 0xFFu);
+                }
+#pragma unroll
+                for (int tt = 0; tt < 4; tt++) {
+                    const char *f = A + static_cast<size_t>((sub * 4 + tt) * 2) * kWideFrag + lane * 16;
+                    const half8_t xh = *reinterpret_cast<const half8_t *>(f);
+                    const half8_t xl = *reinterpret_cast<const half8_t *>(f + kWideFrag);
+                    const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * kWideTok + tt * kTileRows + 4 * kb);
+                    const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc[r][tt], 0, 0, 0);
+                        acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc[r][tt], 0, 0, 0);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(-dm[r], sxv[j], y[r][tt][j]);
+                    }
+                }
+            }
+        }
+        if (s & 1) {
+            // the super-block ends: its sums take its d, the next one's header moves in
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const float dd = f16_bits_to_f32(hdr[r].x);
+#pragma unroll
+                for (int tt = 0; tt < 4; tt++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(dd, acc[r][tt][j], y[r][tt][j]);
+                    acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+                hdr[r] = hdrn[r];
+            }
+        }
+        {
+            // (the last step copies its own slab again: no branch around the stores)
+            uint4 *dst = reinterpret_cast<uint4 *>(smem + (cur ^ 1) * kWideSlab);
+#pragma unroll
+            for (int i = 0; i < kPer; i++) dst[tid + i * NTHR] = an[i];
+            if (tid < 64) dst[kPer * NTHR + tid] = asx;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int g = 0; g < 2; g++) q[r][g] = qn[r][g];
+        }
+        __syncthreads();
+    }
+
+    // C[token 16 tt + 4 kb + j][row n] of each tile
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r * kTileRows + n;
+        if (row >= a.n) continue;
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int tok = tt * kTileRows + 4 * kb + j;
+                if (tok >= nt) continue;
+                float v = y[r][tt][j];
+                if (a.residual) v += a.residual[static_cast<size_t>(t0 + tok) * a.y_stride + row];
+                a.y[yoffs[tok] + row] = v;
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------ the router of a long pass -------
 // logits[t][e] = xn[t] . W[e] for float32 rows W (the router's experts and, as one more row, the
 // shared expert's gate) against the staged rows of a pass: the same streaming of slabs as above,
@@ -869,11 +1041,11 @@ int launch_wide_all(shv_ctx *ctx, const shv_gemv_q4k_args &a, int groups) {
     const size_t lds = 2 * kWideSlab + kWideTok * sizeof(size_t);
     static bool raised = false;
     if (!raised) {
-        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(84 * 1024)));
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_pass_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
         raised = true;
     }
     SHV_REQUIRE(static_cast<long long>(bx) * groups <= 0x7fffffffll, "gemm_q4k: %d row blocks of %d groups", bx, groups);
-    SHV_LAUNCH(ctx, (gemm_wide_kernel<NW, R>), dim3(bx * groups, 1), dim3(NW * 64), lds, a, 0, 0, ctx->gemm_stage, ctx->gemm_part, a.k / 128, groups);
+    SHV_LAUNCH(ctx, (gemm_pass_kernel<NW, R>), dim3(bx * groups), dim3(NW * 64), lds, a, static_cast<const char *>(ctx->gemm_stage), groups);
     return SHV_OK;
 }
 
