@@ -537,6 +537,271 @@ __global__ __launch_bounds__(kBlock) void attn_append_kernel(shv_attn_decode_arg
     vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vsrc[tid]));
 }
 
+// ---- prompt passes: four row pairs a block, every tile of the cache through LDS once ----------
+// The kernel above lets each row pair pull the whole cache for itself, which a pass of a thousand
+// pairs pays in L2 bandwidth.  Here a block is four pairs (64 query rows of one KV head), one a
+// wave: the block copies each 32-cell tile of K and V into LDS once (the next tile's loads are in
+// flight while this one is multiplied) and every wave forms its products from there, as
+// v_mfma_f32_16x16x32_f16 (eight dims or eight cells a lane).  A wave slices the cache and writes
+// its records exactly as a block of the kernel above would for that pair, so the same merge follows.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+constexpr int kKRow = kD * 2 + 16;     // bytes from one cell of the K tile to the next (16 rows cover all banks)
+constexpr int kVRow = kTile * 2 + 16;  // bytes from one dim of the V tile to the next
+struct PrefillTiles {
+    char kt[2][kTile * kKRow];         // K tile, rows in operand order (score tile T, slot s at row 16 T + s)
+    char vt[2][kD * kVRow];            // V tile, [dim][cell % 32]
+};
+struct PrefillSmem {
+    // the queries pass through here once, on their way from the lanes that normalised them to the
+    // lanes that hold them as operands (per wave: [32-dim step][hi, lo][16 * (dim group) + query
+    // row]); after that the same bytes are the tiles, so that two blocks fit a compute unit
+    union {
+        half8_t qf[4][8][2][64];
+        PrefillTiles t;
+    } u;
+    float al[4][16];
+};
+
+// grid: (n_seq * ceil(n_groups / 4), n_head_kv, n_splits); the cells of the pass are in the cache already.
+__global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode_args a, int n_groups, int slice_cells) {
+    extern __shared__ __align__(16) char praw[];
+    PrefillSmem &sm = *reinterpret_cast<PrefillSmem *>(praw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, q = lane >> 4;
+    const int kvh = blockIdx.y, split = blockIdx.z;
+    const int bps = (n_groups + 3) / 4;
+    const int seq = blockIdx.x / bps, g0 = (blockIdx.x % bps) * 4;
+    const int slot = a.slot ? a.slot[seq] : seq;
+    const int pos_first = a.pos ? a.pos[seq] : 0;
+    // pair gg of the sequence: its rows, what it sees, its slice of that
+    struct Slice { int c0, c1, p_first, valid; bool mine; };
+    auto slice_of = [&](int gg) {
+        Slice s;
+        const bool live = gg < n_groups;
+        const int g = live ? gg : n_groups - 1;
+        const int row0 = 2 * g;
+        s.valid = a.seq_len - row0 < 2 ? a.seq_len - row0 : 2;
+        s.p_first = pos_first + row0;
+        const int n_cells = s.p_first + s.valid;
+        int n_active = (n_cells + slice_cells - 1) / slice_cells;
+        if (n_active > a.n_splits) n_active = a.n_splits;
+        int cps = (n_cells + n_active - 1) / n_active;
+        cps = (cps + kTile - 1) & ~(kTile - 1);
+        s.c0 = split * cps;
+        s.c1 = s.c0 + cps < n_cells ? s.c0 + cps : n_cells;
+        s.mine = live && split < n_active && s.c1 > s.c0;
+        return s;
+    };
+    const Slice me = slice_of(g0 + wave);
+    int lo = 0x7fffffff, hi = 0;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const Slice o = slice_of(g0 + w);
+        if (o.mine) {
+            lo = o.c0 < lo ? o.c0 : lo;
+            hi = o.c1 > hi ? o.c1 : hi;
+        }
+    }
+    if (hi <= lo) return;  // no pair of the block has cells in this slice (the same for every wave)
+    const int g = g0 + wave < n_groups ? g0 + wave : n_groups - 1;
+    const int row0 = 2 * g, gz = seq * n_groups + g;
+
+    const int kvw = a.n_head_kv * kD;
+    const uint16_t *kc = static_cast<const uint16_t *>(a.kcache) + static_cast<size_t>(slot) * a.max_cells * kvw + kvh * kD;
+    const uint16_t *vtg = static_cast<const uint16_t *>(a.vcache) + static_cast<size_t>(slot) * a.max_cells * kvw + static_cast<size_t>(kvh) * kD * kTile;
+    const size_t vtile = static_cast<size_t>(kvw) * kTile;
+
+    // ---- the tile copy: 4 + 4 pieces of 16 bytes a thread ----
+    uint4 kr[4], vr[4];
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int e = tid + kBlock * u;
+            int c = t0 + (e >> 5);
+            c = c < hi ? c : hi - 1;
+            kr[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c) * kvw + (e & 31) * 8);
+            vr[u] = *reinterpret_cast<const uint4 *>(vtg + static_cast<size_t>(t0 / kTile) * vtile + (e >> 2) * kTile + (e & 3) * 8);
+        }
+    };
+    auto stash = [&](int b) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int e = tid + kBlock * u;
+            const int cl = e >> 5;                                         // cell of the tile
+            const int rho = 16 * ((cl >> 2) & 1) + 4 * (cl >> 3) + (cl & 3);  // its row in operand order
+            *reinterpret_cast<uint4 *>(sm.u.t.kt[b] + rho * kKRow + (e & 31) * 16) = kr[u];
+            *reinterpret_cast<uint4 *>(sm.u.t.vt[b] + (e >> 2) * kVRow + (e & 3) * 16) = vr[u];
+        }
+    };
+    fetch(lo);
+
+    // ---- the wave's 16 query rows: norm, rotation, scale, operand order ----
+    {
+        const float4 gq = *reinterpret_cast<const float4 *>(a.q_norm + 4 * lane);
+        const int rstep = a.rope_dims >> 3;
+        const float scale = 1.f / sqrtf(static_cast<float>(kD));
+        const int op_h = lane & 1, op_kb = (lane >> 1) & 3, op_i = lane >> 3;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int jr = j < me.valid ? j : me.valid - 1;
+            const int p = me.p_first + jr;
+            const float *rope_row = a.rope_dims > 0 ? a.rope + static_cast<size_t>(p) * a.rope_dims : a.q_norm;
+            const int rl = rstep > 0 ? 4 * (lane & (rstep - 1)) : 0;
+            const float4 cs4 = *reinterpret_cast<const float4 *>(rope_row + rl);
+            const float4 sn4 = *reinterpret_cast<const float4 *>(rope_row + (a.rope_dims >> 1) + rl);
+            const float *qkv = a.qkv + static_cast<size_t>(seq * a.seq_len + row0 + jr) * a.qkv_stride;
+            float4 qv[kRep];
+#pragma unroll
+            for (int hh = 0; hh < kRep; hh++) qv[hh] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(kvh * kRep + hh) * 2 * kD + 4 * lane);
+#pragma unroll
+            for (int hh = 0; hh < kRep; hh++) {
+                float q0, q1, q2, q3;
+                norm_rope_regs(qv[hh], gq, cs4, sn4, a.rope_dims, a.eps, lane, q0, q1, q2, q3);
+                half4_t h4, l4;
+                split1(q0 * scale, h4, l4, 0);
+                split1(q1 * scale, h4, l4, 1);
+                split1(q2 * scale, h4, l4, 2);
+                split1(q3 * scale, h4, l4, 3);
+                const int row = 8 * j + hh;
+                half4_t *dh = reinterpret_cast<half4_t *>(&sm.u.qf[wave][op_i][0][16 * op_kb + row]) + op_h;
+                half4_t *dl = reinterpret_cast<half4_t *>(&sm.u.qf[wave][op_i][1][16 * op_kb + row]) + op_h;
+                *dh = h4;
+                *dl = l4;
+            }
+        }
+    }
+    __builtin_amdgcn_wave_barrier();   // a wave reads back only what it wrote itself
+    half8_t qh[8], ql[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        qh[i] = sm.u.qf[wave][i][0][lane];
+        ql[i] = sm.u.qf[wave][i][1][lane];
+    }
+    __syncthreads();   // every wave holds its queries: the bytes become the tiles
+    stash(0);
+    __syncthreads();
+
+    float4_t o[16];
+#pragma unroll
+    for (int db = 0; db < 16; db++) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const int my_row_pos = me.p_first + (n >> 3);
+
+    int b = 0;
+    for (int t0 = lo; t0 < hi; t0 += kTile, b ^= 1) {
+        const bool more = t0 + kTile < hi;
+        if (more) fetch(t0 + kTile);
+        // tiles wholly outside the wave's slice or beyond what its rows see are skipped
+        if (me.mine && t0 < me.c1 && t0 + kTile > me.c0 && t0 <= me.p_first + 1) {
+            const char *kt = sm.u.t.kt[b], *vt = sm.u.t.vt[b];
+            // operands come from LDS four reads ahead of the products that use them: a read's
+            // latency is about what eight products take, and asked for one at a time it is paid 32 times a tile
+            float4_t st[2];
+            half8_t vb[2][4];
+            {
+                float4_t acc[2][2];
+#pragma unroll
+                for (int T = 0; T < 2; T++)
+#pragma unroll
+                    for (int e = 0; e < 2; e++) acc[T][e] = float4_t{0.f, 0.f, 0.f, 0.f};
+                half8_t kb[2][4];
+                auto read_k = [&](half8_t (&dst)[4], int g4) {   // batch g4: dim steps 2 g4, 2 g4 + 1 of both score tiles
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int i = 2 * g4 + (e >> 1), T = e & 1;
+                        dst[e] = *reinterpret_cast<const half8_t *>(kt + (16 * T + n) * kKRow + (32 * i + 8 * q) * 2);
+                    }
+                };
+                read_k(kb[0], 0);
+#pragma unroll
+                for (int g4 = 0; g4 < 4; g4++) {
+                    if (g4 + 1 < 4) read_k(kb[(g4 + 1) & 1], g4 + 1);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int i = 2 * g4 + (e >> 1), T = e & 1;
+                        acc[T][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb[g4 & 1][e], qh[i], acc[T][0], 0, 0, 0);
+                        acc[T][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb[g4 & 1][e], ql[i], acc[T][1], 0, 0, 0);
+                    }
+                }
+                // the first values go out now, under the softmax arithmetic
+#pragma unroll
+                for (int e = 0; e < 4; e++) vb[0][e] = *reinterpret_cast<const half8_t *>(vt + (16 * e + n) * kVRow + 16 * q);
+                st[0] = acc[0][0] + acc[0][1];
+                st[1] = acc[1][0] + acc[1][1];
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int T = 0; T < 2; T++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int c = t0 + 8 * q + 4 * T + i;
+                    st[T][i] = (c >= me.c0 && c < me.c1 && c <= my_row_pos) ? st[T][i] : -INFINITY;
+                    mx = fmaxf(mx, st[T][i]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            float sum = 0.f;
+            half8_t ph, pl;
+#pragma unroll
+            for (int T = 0; T < 2; T++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float pv = __expf(st[T][i] - m_use);
+                    sum += pv;
+                    const _Float16 hi16 = static_cast<_Float16>(pv);
+                    ph[4 * T + i] = hi16;
+                    pl[4 * T + i] = static_cast<_Float16>(pv - static_cast<float>(hi16));
+                }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            const float alpha = __expf(m_run - m_use);
+            l_run = l_run * alpha + sum;
+            m_run = m_new;
+            if (__ballot(alpha != 1.f) != 0ull) {
+                if (q == 0) sm.al[wave][n] = alpha;
+                __builtin_amdgcn_wave_barrier();
+                const float4 af = *reinterpret_cast<const float4 *>(&sm.al[wave][4 * q]);
+                const float av[4] = {af.x, af.y, af.z, af.w};
+#pragma unroll
+                for (int db = 0; db < 16; db++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) o[db][i] *= av[i];
+                __builtin_amdgcn_wave_barrier();
+            }
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                if (g4 + 1 < 4) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) vb[(g4 + 1) & 1][e] = *reinterpret_cast<const half8_t *>(vt + (16 * (4 * (g4 + 1) + e) + n) * kVRow + 16 * q);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int db = 4 * g4 + e;
+                    float4_t acc = o[db];
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph, vb[g4 & 1][e], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl, vb[g4 & 1][e], acc, 0, 0, 0);
+                    o[db] = acc;
+                }
+            }
+        }
+        if (more) stash(b ^ 1);   // the other buffer was last read a tile ago, before the wait that ended that tile
+        __syncthreads();
+    }
+    if (!me.mine) return;
+    // the wave's record of this slice: per row and head the unnormalised sums, then (max, sum)
+    float *rec = a.partial + ((static_cast<size_t>(gz) * a.n_head_kv + kvh) * a.n_splits + split) * 2 * kRec;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = 4 * q + i;  // query row: sequence row r / 8, head r % 8
+        float *dst = rec + (r >> 3) * kRec + (r & 7) * (kD + 2);
+#pragma unroll
+        for (int db = 0; db < 16; db++) dst[16 * db + n] = o[db][i];
+    }
+    if (q == 0) *reinterpret_cast<float2 *>(rec + (n >> 3) * kRec + (n & 7) * (kD + 2) + kD) = make_float2(m_run, l_run);
+}
+
 template <int R>
 int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_groups, int append) {
     // The slices are there to spread ONE row pair's cache over the chip.  A pass of many pairs (or
@@ -551,8 +816,18 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
     // units as possible pull the cache (a unit issues a wave's 16-byte loads at about 25 B a clock;
     // 36 units over 2 300 cells took 2.2 us to ask for them, 144 take a quarter of that)
     const int slice_cells = a.n_seq * n_groups == 1 ? kTile : kSliceCells;
-    dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
-    SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
+    if (R == 2 && !append && row0 == 0 && n_groups >= 8) {
+        // a prompt pass: four pairs a block share the cache's tiles
+        static bool raised = false;
+        if (!raised) {
+            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
+            raised = true;
+        }
+        SHV_LAUNCH(ctx, attn_prefill_kernel, dim3(a.n_seq * ((n_groups + 3) / 4), a.n_head_kv, b.n_splits), dim3(kBlock), sizeof(PrefillSmem), b, n_groups, slice_cells);
+    } else {
+        dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
+        SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
+    }
     if (a.n_seq * n_groups >= 8 && b.n_splits <= 16) SHV_LAUNCH(ctx, (attn_merge_kernel<R, 1>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64), 0, b, row0, n_groups, slice_cells);
     else SHV_LAUNCH(ctx, (attn_merge_kernel<R, kMergeWaves>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, b, row0, n_groups, slice_cells);
     return SHV_OK;
