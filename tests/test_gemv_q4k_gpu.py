@@ -119,7 +119,7 @@ def test_gemv_refuses_shapes_it_does_not_cover(ctx):
     with pytest.raises(shv.pkg.ShvError):
         ctx.gemv_q4k(d, d, d, 16, 768)
     with pytest.raises(shv.pkg.ShvError):
-        ctx.gemv_q4k(d, d, d, 16, 2048, n_tok=65)
+        ctx.gemv_q4k(d, d, d, 16, 2048, n_tok=4097)   # a pass carries up to 4096 rows
     with pytest.raises(shv.pkg.ShvError):
         ctx.gemv_q4k(d.at(4), d, d, 16, 2048)
 
