@@ -174,14 +174,14 @@ def test_rows_in_one_call_equal_single_steps(ctx, T, slots, pos0):
     assert O.rel_l2(d_state.read(np.float32, s_state.size), s_state) <= TOL
 
 
-@pytest.mark.parametrize("T,pos0,n_seq", [(17, 0, 1), (64, 0, 1), (150, 0, 1), (257, 41, 1), (64, 27, 1), (100, 5, 3), (2048, 3, 1)])
+@pytest.mark.parametrize("T,pos0,n_seq", [(17, 0, 1), (64, 0, 1), (150, 0, 1), (257, 41, 1), (64, 27, 1), (100, 5, 3), (2048, 3, 1), (4096, 0, 1)])
 def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
     """With a workspace a pass of more than 16 rows goes 64 rows at a time on the matrix cores (the
     delta rule's closed form over a chunk).  Against the oracle's row-by-row rule (every row's
     output and the final state within 1e-3), and against this library's own row-by-row kernel on
     the same inputs, which it must match far closer than that: whole chunks, ragged ones, several
     chunks, a start in mid-sequence (history rows, a state that has already run), several sequences
-    in one call, and a 2048-row pass."""
+    in one call, and passes of 2048 and 4096 rows."""
     case = DnCase(ctx, seed=300 + T + n_seq)
     case.upload()
     rng = case.rng

@@ -64,10 +64,11 @@ def test_chunked_prompt_matches_the_cpu(rig):
 
 
 def test_long_pass_matches_the_cpu():
-    """A pass of more rows than an attention or DeltaNet block takes (64): 150 prompt rows go through
-    as one pass of 136 — the blocks in groups of 64 + 64 + 8 rows layer by layer, the experts over all
-    136 rows grouped by expert on the matrix cores — and one of 14.  Last row, carried state and cache
-    are the CPU's, and the same rows in passes of 64 agree to rounding."""
+    """A long pass: 150 prompt rows go through as one pass of 136 and one of 14.  The 136 rows take
+    every block whole: one matrix-core launch per projection, the DeltaNet recurrence in chunks of
+    64 rows in closed form (64 + 64 + 8), the attention four row pairs a block over tiles shared
+    through LDS, the experts grouped by expert on the matrix cores.  Last row, carried state and
+    cache are the CPU's, and the same rows in passes of 64 agree to rounding."""
     rng = np.random.default_rng(150)
     out = {}
     for rows in (136, 64):
@@ -98,9 +99,10 @@ def test_long_pass_matches_the_cpu():
 
 
 def test_long_passes_on_another_slot_and_with_a_one_row_group():
-    """195 prompt rows as passes of 130 (groups of 64 + 64 + 2) and 65 (a group of 64 and a group of one row),
-    on sequence slot 1 and on slot 0: the same bits on both (every group reads its own slot's position
-    words), and the rows in passes of 64 to rounding."""
+    """195 prompt rows as passes of 130 (DeltaNet chunks of 64 + 64 + 2) and 65 (a chunk of 64 and one of a
+    single row), on sequence slot 1 and on slot 0: the same bits on both (the pass's ring takes its
+    conv history from the slot's own ring and hands the last rows back to it), and the rows in passes
+    of 64 to rounding."""
     rng = np.random.default_rng(195)
     prompt = None
     out = {}
@@ -437,17 +439,18 @@ def test_checkpoint_restore_is_the_shorter_sequence(rig):
 
 def test_chunk_size_does_not_matter_over_4096_tokens():
     """BASELINE's prefill shape: 4096 tokens through a period of three DeltaNet layers and one
-    attention layer at the full widths, in chunks of 2048 (the blocks in groups of 64 rows layer by
-    layer, the experts over all rows of the pass grouped by expert on the matrix cores), of 64, of 16,
-    and (the first 192) token by token.
+    attention layer at the full widths, as one pass of 4096, in chunks of 2048 (either way every
+    block whole: whole-pass projections, the recurrence in closed form 64 rows at a time, attention
+    tiles shared by four row pairs, experts grouped on the matrix cores), of 64, of 16, and (the
+    first 192) token by token.
     Every chunk size runs other kernels (matrix cores from 3 or 5 rows, operands staged once from
-    17, rows walked in groups of eight, pairs of attention rows) over the same arithmetic, so the
-    carried state and the last row must agree to rounding."""
+    17, the row-by-row recurrence up to 16 rows and the chunked one above, pairs of attention rows)
+    over the same arithmetic, so the carried state and the last row must agree to rounding."""
     cfg = dict(n_layer=4, vocab=8192, nkv=4224, slots=1)
     rng = np.random.default_rng(4096)
     prompt = rng.integers(0, 8192, size=4096).astype(np.int32)
     out = {}
-    for rows in (2048, 64, 16):
+    for rows in (4096, 2048, 64, 16):
         m = LA.LLM(LA.Config(max_tokens=rows, **cfg))
         m.init_synthetic(99)
         m.stage()
@@ -466,6 +469,11 @@ def test_chunk_size_does_not_matter_over_4096_tokens():
     assert O.rel_l2(a[1], b[1]) <= 1e-3 and O.rel_l2(a[0], b[0]) <= 1e-3, (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]))
     assert O.rel_l2(a[2], b[2]) <= 1e-3 and O.rel_l2(a[3], b[3]) <= 1e-3
     print("64 vs 2048 rows a chunk over 4096 tokens: hidden %.2e logits %.2e state %.2e" %
+          (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]), O.rel_l2(a[2], b[2])))
+    a, b = out[64], out[4096]
+    assert O.rel_l2(a[1], b[1]) <= 1e-3 and O.rel_l2(a[0], b[0]) <= 1e-3, (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]))
+    assert O.rel_l2(a[2], b[2]) <= 1e-3 and O.rel_l2(a[3], b[3]) <= 1e-3
+    print("64 vs 4096 rows a chunk over 4096 tokens: hidden %.2e logits %.2e state %.2e" %
           (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]), O.rel_l2(a[2], b[2])))
     a, b = out[64], out[16]
     assert O.rel_l2(a[1], b[1]) <= 1e-3 and O.rel_l2(a[0], b[0]) <= 1e-3, (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]))
