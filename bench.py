@@ -388,6 +388,20 @@ def config_blocks(m, cfg, A, tensors, cores, want_cpu):
                 # the CPU path takes its sequences one after the other
                 r["cpu_us"], r["cpu_cores"] = round(best * 1e6 * B, 1), cores
             res["decode_B%d" % B] = r
+        if want_cpu:
+            # the prefill side on the CPU: 256 rows through the oracle's layer (it walks them one by one), per row
+            g = lambda n_: tensors["blk.0.%s.weight" % n_]
+            w = O.DnW(O.B(g("attn_qkv")), O.B(g("attn_gate")), O.B(g("ssm_alpha")), O.B(g("ssm_beta")), O.B(g("ssm_out")),
+                      O.F(g("ssm_conv1d")), O.F(g("ssm_a")), O.F(g("ssm_dt")), O.F(g("ssm_norm")))
+            dc = O.DnCfg(H, d, hk, hv, conv, eps, 0)
+            n_s = 256
+            xs = rng.standard_normal((n_s, H)).astype(np.float32)
+            cs, ss = np.zeros((cw, conv - 1), np.float32), np.zeros((hv, d, d), np.float32)
+            y, at = np.empty((n_s, H), np.float32), np.empty((n_s, vw), np.float32)
+            t0 = time.perf_counter()
+            O.lib().shv_ref_deltanet_layer(O.C.byref(dc), O.C.byref(w), O.F(xs), n_s, O.F(cs), O.F(ss), O.F(y),
+                                           None, None, None, None, None, O.F(at), None, 0, cores)
+            res["prefill_cpu"] = {"rows": n_s, "us_per_row": round((time.perf_counter() - t0) / n_s * 1e6, 1), "cpu_cores": cores}
         out["config3_deltanet_layer"] = res
 
     # ---- config 4: gated attention decode over a long fp16 cache ----
@@ -544,15 +558,16 @@ def main():
         sys.exit("bench.py: --steps and --warmup must be at least 1")
     pkg = importlib.import_module("strix-halo-vulkan_amd")
     LA, A = pkg.llm_api, pkg.hip_api
-    nkv = a.prompt + a.warmup + a.steps + 3 * a.mtp_rounds + 64 + a.prefill_rows
+    big = 4096 if a.prefill_rows >= 64 else 0   # a 4096-row chunk is also timed op by op (config 3's prefill shape)
+    nkv = a.prompt + a.warmup + a.steps + 3 * a.mtp_rounds + 64 + a.prefill_rows + big
     # prompt rows go through four at a time; the draft block and the state planes of rewindable
     # 3-row passes are staged for the speculative run and cost the plain decode step nothing
     if a.prefill_rows < 1 or (a.prefill_rows < 4 and not a.no_mtp):
         sys.exit("bench.py: --prefill-rows below 4 needs --no-mtp (the speculative leg stages 3-row passes)")
     if a.no_mtp:
-        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows)
+        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=max(a.prefill_rows, big))
     else:
-        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=a.prefill_rows,
+        cfg = LA.Config(n_layer=a.layers, nkv=(nkv + 127) // 128 * 128, max_tokens=max(a.prefill_rows, big),
                         head_rows=max(3, a.batch_slots), slots=max(1, a.batch_slots), speculative=1, spec_rows=3, nextn=1)
     m = LA.LLM(cfg)
     m.init_synthetic(20260101)
@@ -600,7 +615,7 @@ def main():
                                "drawn N(0,0.02) and quantised on the device by the reference's quantiser, fp16 KV "
                                "cache, vocab 151936; prompt %d random ids then greedy decode at batch 1"
                                % (cfg.n_layer, a.prompt),
-                   "context_at_end": ctx_len, "prefill": "%d rows a pass (%.1f tok/s, untimed)" % (a.prefill_rows, a.prompt / prefill_s),
+                   "context_at_end": ctx_len, "prefill": "%d rows a pass (%.1f tok/s by the host's clock, upload and first-use set-up included, untimed)" % (a.prefill_rows, a.prompt / prefill_s),
                    "weights_GB": round(m.weight_bytes() / 1e9, 2), "dispatches_per_step": m.dispatches()},
         "gpu_ms_per_step": round(gpu_ns / a.steps / 1e6, 4),
         "token_bytes": tb, "token_roofline_tok_s": round(HBM_PEAK / tb, 1), "frac_of_token_roofline": round(tok_s * tb / HBM_PEAK, 4),
@@ -627,6 +642,18 @@ def main():
             # below 128 rows every row reads its own experts: rows x (10 routed + shared) x rows of the banks
             rec["prefill_chunk"]["moe_up_GBps"] = round(rows * per_tok_up * cfg.n_layer / (st["moe.up"] / 1e9) / 1e9, 1)
             rec["prefill_chunk"]["moe_down_GBps"] = round(rows * per_tok_down * cfg.n_layer / (st["moe.down"] / 1e9) / 1e9, 1)
+        if big and m.past() + big + 1 <= cfg.nkv:
+            # BASELINE config 3's prefill shape and config 4's long-pass side: one chunk of 4096 rows
+            st4 = dict(m.profile_chunk(rng.integers(0, cfg.vocab, size=big).astype(np.int32)))
+            us4 = sum(v for k, v in st4.items() if k != "total") / 1e3
+            n_dn = cfg.n_layer - cfg.n_layer // cfg.attn_every
+            dn_us = sum(st4.get(k, 0) for k in ("dn.hist", "dn.qkv", "dn.step", "dn.out")) / 1e3
+            at_us = sum(st4.get(k, 0) for k in ("attn.qkv", "attn.attn", "attn.out")) / 1e3
+            rec["prefill_chunk_4096"] = {
+                "rows": big, "context_before": m.past() - big, "us": round(us4, 1), "tok_s": round(big / us4 * 1e6, 1),
+                "op_us": {k: round(v / 1e3, 1) for k, v in sorted(st4.items(), key=lambda kv: -kv[1]) if k != "total"},
+                "deltanet_layer_us": round(dn_us / n_dn, 1), "deltanet_step_us_per_layer": round(st4.get("dn.step", 0) / 1e3 / n_dn, 1),
+                "attention_layer_us": round(at_us / (cfg.n_layer // cfg.attn_every), 1)}
     if a.pmc_copy:
         import ctypes as C
         H = A.load()
@@ -650,6 +677,13 @@ def main():
     if not a.no_configs:
         rec["configs"] = config_blocks(m, cfg, A, tensors, cores, not a.no_cpu)
         rec["configs"]["config1_gemv_4096x2048"] = dict(rec["gemv"]["config1_4096x2048"])
+        if "prefill_chunk_4096" in rec:
+            pc = rec["prefill_chunk_4096"]
+            rec["configs"]["config3_deltanet_layer"]["prefill_4096_rows"] = {
+                "gpu_us_per_layer": pc["deltanet_layer_us"], "gpu_us_per_row": round(pc["deltanet_layer_us"] / pc["rows"], 4),
+                "step_us_per_layer": pc["deltanet_step_us_per_layer"], "recurrence": "closed form over chunks of 64 rows"}
+            rec["configs"]["config4_attention_decode"]["prefill_4096_rows"] = {
+                "gpu_us_per_layer": pc["attention_layer_us"], "context_before": pc["context_before"]}
         if not a.no_cpu:
             x = rng.standard_normal(cfg.n_embd).astype(np.float32)
             import oracle_lib as O

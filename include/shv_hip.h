@@ -255,7 +255,9 @@ typedef struct {
  * + weights[t][n_used] * (Wd_shared act[t][n_used]).  residual may be NULL.
  * Grouped by expert as shv_moe_up is when the caller gives n_expert, a `group` workspace of the
  * same size and `pairs`, [T][n_used+1][n_embd] floats for the products of every (token, slot)
- * before they are weighted and summed in slot order. */
+ * before they are weighted and summed in slot order.  group_ready != 0 says that `group` already
+ * holds this pass's lists (the grouped shv_moe_up of the same topk and n_tok filled it just before)
+ * and spares the launch that would build them again. */
 typedef struct {
     const float *act;
     const int32_t *topk;
@@ -269,6 +271,7 @@ typedef struct {
     int32_t n_expert;        /* the grouped path: experts in the bank, */
     int32_t *group;          /* its workspace */
     float *pairs;            /* and the per-pair products; NULL keeps the per-(token, slot) kernels */
+    int32_t group_ready;     /* the lists in `group` are this pass's already */
 } shv_moe_down_args;
 
 /* Gated DeltaNet step(s) after the fused projection (DeltaNetLayer, llm/deltanet.go:266-327 and

@@ -54,14 +54,23 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
         if (e >= 0 && e < n_expert) atomicAdd(&s_cnt[e], 1);
     }
     __syncthreads();
-    if (tid == 0) {
-        int at = 0;
-        for (int e = 0; e < n_expert; e++) {
-            const int c = s_cnt[e];
-            s_cnt[e] = at;
-            at += c;
+    {
+        // starts = running sum of the counts: thread e takes expert e (the block has a thread for each)
+        __shared__ int32_t s_wsum[16];
+        const int lane = tid & 63, wave = tid >> 6;
+        const int c = tid < n_expert ? s_cnt[tid] : 0;
+        int incl = c;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
         }
-        s_cnt[n_expert] = at;
+        if (lane == 63) s_wsum[wave] = incl;
+        __syncthreads();
+        int base = 0;
+        for (int w = 0; w < wave; w++) base += s_wsum[w];
+        if (tid < n_expert) s_cnt[tid] = base + incl - c;
+        if (tid == n_expert - 1) s_cnt[n_expert] = base + incl;
     }
     __syncthreads();
     for (int e = tid; e <= n_expert; e += blockDim.x) group[e] = s_cnt[e];
@@ -455,7 +464,7 @@ int shv_launch_moe_down_grouped(shv_ctx *ctx, const shv_moe_down_args &a) {
     SHV_REQUIRE(a.n_embd % 4 == 0 && a.out_stride % 4 == 0 && shv_aligned16(a.out) &&
                     (!a.residual || (a.res_stride % 4 == 0 && shv_aligned16(a.residual))),
                 "moe_down: the grouped path moves 16 bytes at a time");
-    SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
+    if (!a.group_ready) SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
     constexpr size_t lds = kGroupedLds;
     static const int raised = raise_lds(&moe_down_grouped_kernel<512>, lds);
     if (raised != SHV_OK) return raised;

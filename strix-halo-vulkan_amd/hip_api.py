@@ -86,7 +86,7 @@ class MoeDownArgs(C.Structure):
                 ("out", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("res_stride", C.c_int32),
                 ("out_stride", C.c_int32), ("down_type", C.c_int32), ("down_sh_type", C.c_int32),
-                ("n_expert", C.c_int32), ("group", C.c_void_p), ("pairs", C.c_void_p)]
+                ("n_expert", C.c_int32), ("group", C.c_void_p), ("pairs", C.c_void_p), ("group_ready", C.c_int32)]
 
 
 class DnStepArgs(C.Structure):

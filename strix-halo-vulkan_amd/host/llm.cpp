@@ -524,6 +524,7 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     d.n_expert = c_.NExpert;
     d.group = group_;
     d.pairs = pairs_;
+    d.group_ready = (!fused && up_q4k && group_) ? 1 : 0;  // the up projection of this pass has grouped its rows (or neither takes that road)
     d.act = act_;
     d.topk = topk_;
     d.weights = weights_;
