@@ -248,7 +248,10 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 // scale, a scalar, is applied to the finished dot products instead of to the staged vector, so
 // that the sum of squares does not stand between the loads and the staging.
 // WAVES waves a block, P passes a wave (pass = 64/(K/64) rows); grid = ceil(passes / (WAVES*P)).
-template <int K, int WAVES, int P, int PRO>
+// STAGED (a variant kept for comparison): the lane of a super-block's first group decodes all
+// eight (d*sc, dmin*m) pairs of the header and leaves them in LDS for the four lanes of the
+// super-block, instead of every lane decoding its own group's from the header it holds anyway.
+template <int K, int WAVES, int P, int PRO, bool STAGED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args a) {
     constexpr int T = WAVES * 64, LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int NV = K / 4 / T;  // float4 a thread stages
@@ -349,9 +352,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
     float *y = a.y;
     if (a.ring_slots > 0 && !a.z_ring) y += static_cast<size_t>(ring_row) * a.ring_stride;
     const NibbleConsts nc = nibble_consts();
+    __shared__ float4 staged_sc[STAGED ? WAVES * P * 64 : 1];
+    if constexpr (STAGED) {
+#pragma unroll
+        for (int u = 0; u < P; u++) {
+            if (g == 0) {
+                const float d = f16_bits_to_f32(w[u].hdr.x), dmin = f16_bits_to_f32(w[u].hdr.x >> 16);
+#pragma unroll
+                for (int gg = 0; gg < 4; gg++) {
+                    uint32_t sc, mn;
+                    q4k_group_scale_min(w[u].hdr, gg, sc, mn);
+                    staged_sc[(wave * P + u) * 64 + lane + gg] = make_float4(d * static_cast<float>(sc & 0xFFu), d * static_cast<float>(sc >> 8),
+                                                                              dmin * static_cast<float>(mn & 0xFFu), dmin * static_cast<float>(mn >> 8));
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
 #pragma unroll
     for (int u = 0; u < P; u++) {
-        float acc = w[u].dot(g, nc, xr, xs_lo, xs_hi);
+        float acc;
+        if constexpr (STAGED) acc = q4k_group_dot_scaled(w[u].q0, w[u].q1, staged_sc[(wave * P + u) * 64 + lane], nc, xr, xs_lo, xs_hi);
+        else acc = w[u].dot(g, nc, xr, xs_lo, xs_hi);
         acc = group_sum<LPR>(acc);
         if (row[u] >= 0 && group_sum_owner<LPR>(lane)) {
             const float v = fmaf(acc, scale, res[u]);
@@ -369,6 +391,15 @@ int launch_row_kp(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     constexpr int RPP = 64 / (K / 64);
     const long long passes = (static_cast<long long>(a.n) + RPP - 1) / RPP;
     const dim3 grid(static_cast<unsigned>((passes + WAVES * P - 1) / (WAVES * P))), block(WAVES * 64);
+    if (ctx->gemv_scales_lds) {
+        switch (a.prologue) {
+            case SHV_PRO_NONE: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_NONE, true>), grid, block, 0, a); break;
+            case SHV_PRO_RMSNORM: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_RMSNORM, true>), grid, block, 0, a); break;
+            case SHV_PRO_GATED_NORM: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_GATED_NORM, true>), grid, block, 0, a); break;
+            default: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_MUL_SIGMOID, true>), grid, block, 0, a); break;
+        }
+        return SHV_OK;
+    }
     switch (a.prologue) {
         case SHV_PRO_NONE: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_NONE>), grid, block, 0, a); break;
         case SHV_PRO_RMSNORM: SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, P, SHV_PRO_RMSNORM>), grid, block, 0, a); break;

@@ -42,6 +42,7 @@ int shv_init(int device, shv_ctx **out) {
         const int v = std::atoi(e);
         if (v >= 2) ctx->mfma_min_rows = ctx->mfma_min_rows_wide = v;
     }
+    if (const char *e = std::getenv("SHV_GEMV_SCALES")) ctx->gemv_scales_lds = std::strcmp(e, "lds") == 0;
     if (const char *e = std::getenv("SHV_MOE_GROUP_MIN")) {
         const int v = std::atoi(e);
         if (v >= 1) ctx->moe_group_min = v;

@@ -152,6 +152,23 @@ __device__ __forceinline__ float q4k_group_dot(const uint4 &hdr, const uint4 &p0
     return ds0 * lo - dm0 * xs_lo + ds1 * hi - dm1 * xs_hi;
 }
 
+// The same with the group's scales already multiplied out: sc = (d*sc_lo, d*sc_hi, dmin*m_lo, dmin*m_hi).
+__device__ __forceinline__ float q4k_group_dot_scaled(const uint4 &p0, const uint4 &p1, const float4 sc, const NibbleConsts &c,
+                                                      const float *xr, float xs_lo, float xs_hi) {
+    float lo = 0.f, hi = 0.f;
+    q4k_dot8(p0.x, c, xr + 0, xr + 32, lo, hi);
+    q4k_dot8(p0.y, c, xr + 4, xr + 36, lo, hi);
+    q4k_dot8(p0.z, c, xr + 8, xr + 40, lo, hi);
+    q4k_dot8(p0.w, c, xr + 12, xr + 44, lo, hi);
+    q4k_dot8(p1.x, c, xr + 16, xr + 48, lo, hi);
+    q4k_dot8(p1.y, c, xr + 20, xr + 52, lo, hi);
+    q4k_dot8(p1.z, c, xr + 24, xr + 56, lo, hi);
+    q4k_dot8(p1.w, c, xr + 28, xr + 60, lo, hi);
+    lo = fmaf(-64.f, xs_lo, lo);
+    hi = fmaf(-64.f, xs_hi, hi);
+    return sc.x * lo - sc.z * xs_lo + sc.y * hi - sc.w * xs_hi;
+}
+
 typedef uint32_t u32x4_native __attribute__((ext_vector_type(4)));
 
 // 128-bit load of weight bytes.  A plain load on purpose: the lanes of a super-block share its

@@ -23,6 +23,9 @@ struct shv_ctx {
     // operands).  SHV_MFMA_MIN_ROWS in the environment sets both; a large value keeps every pass
     // on the row kernel.
     int mfma_min_rows = 3, mfma_min_rows_wide = 5;
+    // SHV_GEMV_SCALES=lds: the one-row GEMV hands each super-block's eight (d*sc, dmin*m) pairs from one lane to
+    // the four that use them through LDS instead of letting every lane decode its own (for comparison; slower)
+    bool gemv_scales_lds = false;
     int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)
     int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
