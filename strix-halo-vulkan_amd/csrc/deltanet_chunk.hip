@@ -19,7 +19,8 @@
 //                    of the other rows) and walks the chunks of the pass with that slab in
 //                    registers as float32; the solve is blocked 4 x 16: the four 16x16 diagonal
 //                    blocks of (I + A) are inverted by substitution on the vector units (each lane
-//                    a column), everything else is v_mfma_f32_16x16x16/32_f16
+//                    a column, one wave, while the other three form the tiles of A below the
+//                    diagonal), everything else is v_mfma_f32_16x16x16/32_f16
 //
 // float32 operands enter the matrix cores as a sum of two binary16 values (the low part scaled
 // by 2^11 so that it stays normal), three products per term (hi*hi, hi*lo, lo*hi): about 22 bits
@@ -250,51 +251,44 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
             L.beta[tid] = bt;
         }
         __syncthreads();
-        if (c + 1 < n_chunks) fetch(c + 1);  // in flight under the whole chunk
 
-        // ---- 2: P = K K^T and R = Q K^T, rows of wave w against row tiles 0..w; A and M from them ----
-        half8_t akh[4], akl[4], aqh[4], aql[4];  // the wave's own rows as first operands, kept for step 3
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            akh[ks] = *reinterpret_cast<const half8_t *>(&L.kh[16 * w + n][32 * ks + 8 * g]);
-            akl[ks] = *reinterpret_cast<const half8_t *>(&L.kl[16 * w + n][32 * ks + 8 * g]);
-            aqh[ks] = *reinterpret_cast<const half8_t *>(&L.qh[16 * w + n][32 * ks + 8 * g]);
-            aql[ks] = *reinterpret_cast<const half8_t *>(&L.ql[16 * w + n][32 * ks + 8 * g]);
-        }
-        float Gt[4], bt4[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            Gt[r] = L.G[16 * w + 4 * g + r];
-            bt4[r] = L.beta[16 * w + 4 * g + r];
-        }
-        for (int st = 0; st <= w; st++) {
+        // ---- 2: P = K K^T and R = Q K^T over the lower triangle of 4 x 4 tiles of 16 rows; A and M from them.
+        //      First every wave its own diagonal tile; then, while wave 0 inverts the four diagonal
+        //      blocks of I + A on the vector units, the other three take two of the six tiles below
+        //      the diagonal each ----
+        auto tile = [&](int tt, int st) {
             float4_t pm = {0.f, 0.f, 0.f, 0.f}, pl = pm, rm = pm, rl = pm;
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
+                const half8_t xkh = *reinterpret_cast<const half8_t *>(&L.kh[16 * tt + n][32 * ks + 8 * g]);
+                const half8_t xkl = *reinterpret_cast<const half8_t *>(&L.kl[16 * tt + n][32 * ks + 8 * g]);
+                const half8_t xqh = *reinterpret_cast<const half8_t *>(&L.qh[16 * tt + n][32 * ks + 8 * g]);
+                const half8_t xql = *reinterpret_cast<const half8_t *>(&L.ql[16 * tt + n][32 * ks + 8 * g]);
                 const half8_t bh = *reinterpret_cast<const half8_t *>(&L.kh[16 * st + n][32 * ks + 8 * g]);
                 const half8_t bl = *reinterpret_cast<const half8_t *>(&L.kl[16 * st + n][32 * ks + 8 * g]);
-                mma32(akh[ks], akl[ks], bh, bl, pm, pl);
-                mma32(aqh[ks], aql[ks], bh, bl, rm, rl);
+                mma32(xkh, xkl, bh, bl, pm, pl);
+                mma32(xqh, xql, bh, bl, rm, rl);
             }
             const float Gs = L.G[16 * st + n];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int t = 16 * w + 4 * g + r, s = 16 * st + n;
-                const float dec = __expf(Gt[r] - Gs);
+                const int t = 16 * tt + 4 * g + r, s = 16 * st + n;
+                const float Gtr = L.G[t], btr = L.beta[t];
+                const float dec = __expf(Gtr - Gs);
                 const float P = fmaf(pl[r], kLoInv, pm[r]), R = fmaf(rl[r], kLoInv, rm[r]);
-                const float av = s < t ? bt4[r] * dec * P : 0.f;
+                const float av = s < t ? btr * dec * P : 0.f;
                 const float mv = s <= t ? dec * R : 0.f;
                 _Float16 hi, lo;
                 split(-av, hi, lo);
                 L.ah[t][s] = hi; L.al[t][s] = lo;
                 split(mv, hi, lo);
                 L.mh[t][s] = hi; L.ml[t][s] = lo;
-                if (st == w) L.adiag[w][4 * g + r][n] = av;
+                if (st == tt) L.adiag[tt][4 * g + r][n] = av;
             }
-        }
+        };
+        tile(w, w);
         __syncthreads();
-
-        // ---- 3: wave 0 inverts the four diagonal blocks; every wave's rows against the state ----
+        if (c + 1 < n_chunks) fetch(c + 1);  // in flight under the rest of the chunk (the stores that read these registers have drained)
         if (w == 0) {
             // lane (b = g, column n): T = (I + A_bb)^-1 by forward substitution, the column in registers
             float T[16];
@@ -312,6 +306,31 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 L.th[g][t][n] = hi;
                 L.tl[g][t][n] = lo;
             }
+        } else if (w == 1) {
+            tile(3, 0);
+            tile(1, 0);
+        } else if (w == 2) {
+            tile(3, 1);
+            tile(2, 0);
+        } else {
+            tile(3, 2);
+            tile(2, 1);
+        }
+
+        // ---- 3: every wave's rows against the state ----
+        half8_t akh[4], akl[4], aqh[4], aql[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            akh[ks] = *reinterpret_cast<const half8_t *>(&L.kh[16 * w + n][32 * ks + 8 * g]);
+            akl[ks] = *reinterpret_cast<const half8_t *>(&L.kl[16 * w + n][32 * ks + 8 * g]);
+            aqh[ks] = *reinterpret_cast<const half8_t *>(&L.qh[16 * w + n][32 * ks + 8 * g]);
+            aql[ks] = *reinterpret_cast<const half8_t *>(&L.ql[16 * w + n][32 * ks + 8 * g]);
+        }
+        float Gt[4], bt4[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            Gt[r] = L.G[16 * w + 4 * g + r];
+            bt4[r] = L.beta[16 * w + 4 * g + r];
         }
         float4_t acc, accl = {0.f, 0.f, 0.f, 0.f}, w2;
         {
