@@ -568,9 +568,21 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
     PrefillSmem &sm = *reinterpret_cast<PrefillSmem *>(praw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, q = lane >> 4;
-    const int kvh = blockIdx.y, split = blockIdx.z;
+    // Workgroups are handed to the chip's eight dies in turn (workgroup i to die i % 8), and each die has its
+    // own L2: the blocks of one die all take the same KV head, so that a die's L2 holds one head's K and V
+    // (half the cells' bytes) and the blocks that walk it side by side find each other's tiles there.
+    int kvh = blockIdx.y, bx = blockIdx.x;
+    {
+        const int per = 8 / a.n_head_kv;  // dies a KV head gets
+        if (a.n_head_kv <= 8 && per * a.n_head_kv == 8 && gridDim.x % per == 0) {
+            const int id = blockIdx.x + gridDim.x * blockIdx.y, die = id & 7;
+            kvh = die % a.n_head_kv;
+            bx = (id >> 3) * per + die / a.n_head_kv;
+        }
+    }
+    const int split = blockIdx.z;
     const int bps = (n_groups + 3) / 4;
-    const int seq = blockIdx.x / bps, g0 = (blockIdx.x % bps) * 4;
+    const int seq = bx / bps, g0 = (bx % bps) * 4;
     const int slot = a.slot ? a.slot[seq] : seq;
     const int pos_first = a.pos ? a.pos[seq] : 0;
     // pair gg of the sequence: its rows, what it sees, its slice of that
