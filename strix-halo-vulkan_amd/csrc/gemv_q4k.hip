@@ -383,6 +383,143 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
     }
 }
 
+// ---- two to four activation rows of one sequence (a verification pass, a short prompt tail) ------
+// The one-row kernel's shape with the rows side by side: every row's inputs first, the weights of
+// the wave's passes once, each row staged with its sums, one block-wide wait, then the lane walks
+// the rows with its weights in registers (a row's 64 activations come from LDS when its turn comes).
+template <int K, int WAVES, int P, int PRO, int NT>
+__global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_args a) {
+    constexpr int T = WAVES * 64, LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
+    constexpr int NV = K / 4 / T;
+    static_assert(NV >= 1 && K % (4 * T) == 0, "threads of a block each stage whole float4s");
+    __shared__ __align__(16) float xs[NT][lds_padded(K)];
+    __shared__ __align__(16) float xsum[NT][K / 32];
+    __shared__ float red[NT][WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
+    const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
+    const long long pass0 = (static_cast<long long>(blockIdx.x) * WAVES + wave) * P;
+    // the rows are rows 0..NT-1 of ONE sequence: ring rows follow its position
+    int p0 = 0, ring_base = 0;
+    if (a.ring_slots > 0) {
+        p0 = a.pos ? a.pos[0] : 0;
+        ring_base = (a.slot ? a.slot[0] : 0) * a.ring_slots;
+    }
+    float4 xv[NT][NV], gv[NV], zv[NT][NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int c = 4 * (tid + T * j);
+        if constexpr (PRO == SHV_PRO_RMSNORM) gv[j] = *reinterpret_cast<const float4 *>(a.gamma + c);
+        else if constexpr (PRO == SHV_PRO_GATED_NORM) gv[j] = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            xv[t][j] = *reinterpret_cast<const float4 *>(a.x + static_cast<size_t>(t) * a.x_stride + c);
+            if constexpr (PRO == SHV_PRO_GATED_NORM) {
+                const float *z = a.z_ring ? a.z + static_cast<size_t>(ring_base + (p0 + t) % a.ring_slots) * a.ring_stride
+                                          : a.z + static_cast<size_t>(t) * a.z_stride;
+                zv[t][j] = *reinterpret_cast<const float4 *>(z + c);
+            } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+                const HeadSplit hs(a.head_dim > 0 ? a.head_dim : 1);
+                const int zi = a.head_dim > 0 ? hs.head(c) * 2 * a.head_dim + a.head_dim + hs.dim(c) : c;
+                zv[t][j] = *reinterpret_cast<const float4 *>(a.z + static_cast<size_t>(t) * a.z_stride + zi);
+            }
+        }
+    }
+    Q4kLane w[P];
+    int row[P];
+#pragma unroll
+    for (int u = 0; u < P; u++) {
+        const long long r = (pass0 + u) * RPP + rsub;
+        row[u] = r < a.n ? static_cast<int>(r) : -1;
+        w[u].load(wbase + static_cast<size_t>(row[u] < 0 ? 0 : row[u]) * ROWB, g);
+    }
+    float res[NT][P];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int u = 0; u < P; u++)
+            res[t][u] = (a.residual && row[u] >= 0 && group_sum_owner<LPR>(lane)) ? a.residual[static_cast<size_t>(t) * a.y_stride + row[u]] : 0.f;
+
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int c = 4 * (tid + T * j);
+            float4 v = xv[t][j];
+            if constexpr (PRO == SHV_PRO_RMSNORM) {
+                const float4 gm = gv[j];
+                ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+                v = make_float4(v.x * gm.x, v.y * gm.y, v.z * gm.z, v.w * gm.w);
+            } else if constexpr (PRO == SHV_PRO_GATED_NORM) {
+                const float4 gm = gv[j], z4 = zv[t][j];
+                float hs = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
+                const int span = a.head_dim >> 2;
+                hs = sum8_all(hs);
+                if (span >= 16) hs += dpp_f32<kDppMirror>(hs);
+                if (span >= 32) hs += __shfl_xor(hs, 16, 64);
+                if (span >= 64) hs += __shfl_xor(hs, 32, 64);
+                const float sc = __builtin_amdgcn_rsqf(hs / static_cast<float>(a.head_dim) + a.eps);
+                v = make_float4(v.x * sc * gm.x * sigmoid_fast(z4.x), v.y * sc * gm.y * sigmoid_fast(z4.y),
+                                v.z * sc * gm.z * sigmoid_fast(z4.z), v.w * sc * gm.w * sigmoid_fast(z4.w));
+            } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+                const float4 z4 = zv[t][j];
+                v = make_float4(v.x * sigmoid_fast(z4.x), v.y * sigmoid_fast(z4.y), v.z * sigmoid_fast(z4.z), v.w * sigmoid_fast(z4.w));
+            }
+            *reinterpret_cast<float4 *>(&xs[t][lds_slot(c)]) = v;
+            const float s8 = sum8_all((v.x + v.y) + (v.z + v.w));
+            if ((lane & 7) == 0) xsum[t][c >> 5] = s8;
+        }
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            ss = wave_sum_all(ss);
+            if (lane == 0) red[t][wave] = ss;
+        }
+    }
+    __syncthreads();
+    const NibbleConsts nc = nibble_consts();
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        float scale = 1.f;
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            float tot = 0.f;
+#pragma unroll
+            for (int i = 0; i < WAVES; i++) tot += red[t][i];
+            scale = __builtin_amdgcn_rsqf(tot / static_cast<float>(K) + a.eps);
+        }
+        float xr[64], xs_lo, xs_hi;
+        load_x_slice_presummed(xs[t], xsum[t], gi, xr, xs_lo, xs_hi);
+        float *y = a.y + static_cast<size_t>(t) * a.y_stride;
+        if (a.ring_slots > 0 && !a.z_ring) y = a.y + static_cast<size_t>(ring_base + (p0 + t) % a.ring_slots) * a.ring_stride;
+#pragma unroll
+        for (int u = 0; u < P; u++) {
+            float acc = w[u].dot(g, nc, xr, xs_lo, xs_hi);
+            acc = group_sum<LPR>(acc);
+            if (row[u] >= 0 && group_sum_owner<LPR>(lane)) y[row[u]] = fmaf(acc, scale, res[t][u]);
+        }
+    }
+}
+
+template <int K, int WAVES, int P, int NT>
+int launch_fewrows_kpn(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    constexpr int RPP = 64 / (K / 64);
+    const long long passes = (static_cast<long long>(a.n) + RPP - 1) / RPP;
+    const dim3 grid(static_cast<unsigned>((passes + WAVES * P - 1) / (WAVES * P))), block(WAVES * 64);
+    switch (a.prologue) {
+        case SHV_PRO_NONE: SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, P, SHV_PRO_NONE, NT>), grid, block, 0, a); break;
+        case SHV_PRO_RMSNORM: SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, P, SHV_PRO_RMSNORM, NT>), grid, block, 0, a); break;
+        case SHV_PRO_GATED_NORM: SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, P, SHV_PRO_GATED_NORM, NT>), grid, block, 0, a); break;
+        default: SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, P, SHV_PRO_MUL_SIGMOID, NT>), grid, block, 0, a); break;
+    }
+    return SHV_OK;
+}
+
+template <int NT>
+int launch_fewrows(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (a.k == 4096) return launch_fewrows_kpn<4096, 8, 1, NT>(ctx, a);
+    if (a.n <= 2 * 4 * 2 * ctx->prop.multiProcessorCount) return launch_fewrows_kpn<2048, 4, 1, NT>(ctx, a);
+    return launch_fewrows_kpn<2048, 4, 2, NT>(ctx, a);
+}
+
 // Which one-row launches the kernel above takes: the decode step's projections (2048- and
 // 4096-wide inputs).  A matrix of very many rows (the vocabulary projection) is a stream, not a
 // latency, and stays on the looping kernel; so do the other widths and the pair-norm prologue.
@@ -409,6 +546,9 @@ int launch_row_kp(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     return SHV_OK;
 }
 
+// Two to four rows of one sequence take the rows-side-by-side form of the same kernel.
+bool fewrows_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a);
+
 bool row_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     if (a.n_tok != 1 || a.prologue == SHV_PRO_RMSNORM_PAIR) return false;
     if (a.k != 2048 && a.k != 4096) return false;
@@ -418,6 +558,17 @@ bool row_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     // more rounds of the chip than a few: a stream
     const long long passes = static_cast<long long>(a.n) / (64 / (a.k / 64));
     return passes <= static_cast<long long>(ctx->prop.multiProcessorCount) * 4 * 8;
+}
+
+bool fewrows_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (a.n_tok < 2 || a.n_tok > 4 || a.y_flat) return false;
+    // one sequence: its rows share a position word and a slot
+    const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+    if (sl != a.n_tok) return false;
+    if (a.x_stride % 4 != 0 || ((a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID) && !a.z_ring && a.z_stride % 4 != 0)) return false;
+    shv_gemv_q4k_args one = a;
+    one.n_tok = 1;
+    return row_kernel_covers(ctx, one);
 }
 
 int launch_row(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
@@ -532,6 +683,10 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
         SHV_REQUIRE((a.z_ring || (a.ring_stride >= a.n && !a.residual)) && sl <= a.ring_slots && a.n_tok % sl == 0,
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
+    // two to four rows of one sequence: the one-row kernel's shape with the rows side by side (SHV_MFMA_MIN_ROWS
+    // at or below the row count sends them to the matrix cores instead, as before)
+    if (fewrows_kernel_covers(ctx, a) && !ctx->mfma_rows_forced)
+        return a.n_tok == 2 ? launch_fewrows<2>(ctx, a) : a.n_tok == 3 ? launch_fewrows<3>(ctx, a) : launch_fewrows<4>(ctx, a);
     if (a.n_tok >= (a.k > 2048 ? ctx->mfma_min_rows_wide : ctx->mfma_min_rows) && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
     SHV_REQUIRE(a.n_tok <= 64, "gemv_q4k: %d rows: more than 64 go through the matrix-core kernel, which does not take this shape (k %d, prologue %d)",
                 a.n_tok, a.k, a.prologue);

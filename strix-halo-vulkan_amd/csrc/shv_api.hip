@@ -40,7 +40,10 @@ int shv_init(int device, shv_ctx **out) {
     ctx->device = device;
     if (const char *e = std::getenv("SHV_MFMA_MIN_ROWS")) {
         const int v = std::atoi(e);
-        if (v >= 2) ctx->mfma_min_rows = ctx->mfma_min_rows_wide = v;
+        if (v >= 2) {
+            ctx->mfma_min_rows = ctx->mfma_min_rows_wide = v;
+            ctx->mfma_rows_forced = true;
+        }
     }
     if (const char *e = std::getenv("SHV_GEMV_SCALES")) ctx->gemv_scales_lds = std::strcmp(e, "lds") == 0;
     if (const char *e = std::getenv("SHV_MOE_GROUP_MIN")) {

@@ -23,6 +23,7 @@ struct shv_ctx {
     // operands).  SHV_MFMA_MIN_ROWS in the environment sets both; a large value keeps every pass
     // on the row kernel.
     int mfma_min_rows = 3, mfma_min_rows_wide = 5;
+    bool mfma_rows_forced = false;  // SHV_MFMA_MIN_ROWS was given: the few-rows GEMV steps aside for the caller's threshold
     // SHV_GEMV_SCALES=lds: the one-row GEMV hands each super-block's eight (d*sc, dmin*m) pairs from one lane to
     // the four that use them through LDS instead of letting every lane decode its own (for comparison; slower)
     bool gemv_scales_lds = false;
