@@ -1309,6 +1309,8 @@ void Graph::extend(const std::vector<int32_t> &ids, float *res_all) {
     last_rows_ = last;
 }
 
+int Graph::StepRows() const { return head_ ? std::min(head_->MaxRows(), o_.Slots) : 0; }
+
 void Graph::Extend(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *hidden) {
     if (logits && !head_) throw Error("llm: Graph.Extend: the graph was staged without a head");
     extend(ids, nullptr);

@@ -407,6 +407,7 @@ public:
     int Plane() const { return seq_[slot_].plane; }  // the live slot's committed DeltaNet state plane
     int NKV() const { return o_.NKV; }
     int MaxRows() const { return rows_max_; }
+    int StepRows() const;  // rows one DecodeRows pass may carry: 0 without a head
     std::vector<int32_t> Ids() const;
     // Rewindable passes (llm/graph.go:1122-1267).  While Speculate is on, ExtendRows leaves the
     // committed DeltaNet state alone and stores the state after each of its rows apart; exactly

@@ -8,6 +8,7 @@
 #include <memory>
 
 #include "llm.hpp"
+#include "sched.hpp"
 
 struct shvllm {
     std::unique_ptr<llm::Device> dev;
@@ -457,6 +458,150 @@ int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos) {
             nanos[0] = s.DraftNanos;
             nanos[1] = s.VerifyNanos;
         }
+    });
+}
+
+// ---- the scheduler ------------------------------------------------------------------------------
+
+struct shvllm_sched {
+    std::unique_ptr<llm::Sched> s;
+    llm::SchedPass last;  // what shvllm_sched_next handed out and shvllm_sched_finish books
+};
+
+static llm::Sched &sched_of(shvllm_sched *s) {
+    if (!s || !s->s) throw llm::Error("llm: NULL scheduler");
+    return *s->s;
+}
+
+static void pass_out(const llm::SchedPass &p, shvllm_sched_pass *o) {
+    if (!o) return;
+    std::memset(o, 0, sizeof(*o));
+    o->kind = p.kind, o->unit = p.unit, o->slot = p.slot, o->pos = p.pos, o->n = p.n;
+    o->fresh = p.fresh, o->restore = p.restore, o->take = p.take, o->step = p.step;
+    o->wait_ms = p.wait_ms;
+    o->n_units = static_cast<int32_t>(std::min<size_t>(p.units.size(), SHVLLM_SCHED_MAX_ROWS));
+    for (int i = 0; i < o->n_units; i++) o->units[i] = p.units[i], o->slots[i] = p.slots[i];
+}
+
+int shvllm_sched_open(shvllm *h, int slots, const shvllm_sched_opts *opts, shvllm_sched **out) {
+    return guard([&] {
+        if (!out) throw llm::Error("llm: shvllm_sched_open: NULL argument");
+        llm::SchedOpts o;
+        if (opts) {
+            if (opts->batch > 0) o.Batch = opts->batch;
+            o.PreemptChunk = opts->preempt_chunk;
+            o.Reserve = opts->reserve;
+            o.NoBatchDecode = opts->no_batch_decode != 0;
+            if (opts->coalesce_ms >= 0) o.CoalesceMs = opts->coalesce_ms;
+        }
+        llm::Graph *g = h ? &graph_of(h) : nullptr;
+        if ((g ? g->Slots() : slots) > SHVLLM_SCHED_MAX_ROWS) throw llm::Error("llm: a scheduler covers at most " + std::to_string(SHVLLM_SCHED_MAX_ROWS) + " slots");
+        auto s = std::make_unique<shvllm_sched>();
+        s->s = std::make_unique<llm::Sched>(g, slots, o);
+        *out = s.release();
+    });
+}
+
+void shvllm_sched_close(shvllm_sched *s) { delete s; }
+
+int shvllm_sched_acquire(shvllm_sched *s, int cls, const int32_t *prompt, int n, int mark, double now_ms, int *job) {
+    return guard([&] {
+        if (!prompt || n < 1 || !job) throw llm::Error("llm: shvllm_sched_acquire: an empty prompt or NULL argument");
+        *job = sched_of(s).Acquire(cls, std::vector<int32_t>(prompt, prompt + n), mark, now_ms);
+    });
+}
+
+int shvllm_sched_release(shvllm_sched *s, int job, double now_ms) {
+    return guard([&] { sched_of(s).Release(job, now_ms); });
+}
+
+int shvllm_sched_job_info(shvllm_sched *s, int job, shvllm_sched_job *out) {
+    return guard([&] {
+        if (!out) throw llm::Error("llm: shvllm_sched_job_info: NULL argument");
+        const llm::SchedJobInfo j = sched_of(s).Job(job);
+        out->cls = j.cls, out->slot = j.slot, out->reused = j.reused, out->restored = j.restored, out->stepping = j.stepping;
+        out->served_ms = j.served_ms, out->arrival = j.arrival;
+    });
+}
+
+int shvllm_sched_run(shvllm_sched *s, int job, const int32_t *ids, int n, int fresh, int *unit) {
+    return guard([&] {
+        if (!ids || n < 1 || !unit) throw llm::Error("llm: shvllm_sched_run: no ids or NULL argument");
+        *unit = sched_of(s).Run(job, std::vector<int32_t>(ids, ids + n), fresh != 0);
+    });
+}
+
+int shvllm_sched_step(shvllm_sched *s, int job, int32_t id, int *unit) {
+    return guard([&] {
+        if (!unit) throw llm::Error("llm: shvllm_sched_step: NULL argument");
+        *unit = sched_of(s).Step(job, id);
+    });
+}
+
+int shvllm_sched_withdraw(shvllm_sched *s, int unit) {
+    return guard([&] { sched_of(s).Withdraw(unit); });
+}
+
+int shvllm_sched_next(shvllm_sched *s, double now_ms, shvllm_sched_pass *out) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        if (s->last.kind != llm::SchedPass::kNone) throw llm::Error("llm: the last pass has not been finished");
+        s->last = sc.Next(now_ms);
+        pass_out(s->last, out);
+    });
+}
+
+int shvllm_sched_finish(shvllm_sched *s, double took_ms, int ok, double now_ms) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        if (s->last.kind == llm::SchedPass::kNone) throw llm::Error("llm: no pass is out");
+        const llm::SchedPass p = s->last;
+        s->last = llm::SchedPass();
+        sc.Finish(p, took_ms, ok != 0, now_ms, nullptr, ok ? "" : "the caller's pass failed");
+    });
+}
+
+int shvllm_sched_pump(shvllm_sched *s, shvllm_sched_pass *out) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        if (s->last.kind != llm::SchedPass::kNone) throw llm::Error("llm: the last pass has not been finished");
+        pass_out(sc.Pump(), out);
+    });
+}
+
+int shvllm_sched_unit(shvllm_sched *s, int unit, int *state, int *left, double *busy_ms, float *logits, int max) {
+    return guard([&] {
+        const llm::Sched::UnitState u = sched_of(s).Unit(unit);
+        if (!u.known) throw llm::Error("llm: no such unit " + std::to_string(unit));
+        if (state) *state = !u.done ? 0 : (u.failed ? 2 : 1);
+        if (left) *left = u.left;
+        if (busy_ms) *busy_ms = u.busy_ms;
+        if (u.failed) std::snprintf(g_err, sizeof(g_err), "%s", u.err.c_str());
+        if (logits && u.done && !u.failed) std::copy(u.logits.begin(), u.logits.begin() + std::min<size_t>(max, u.logits.size()), logits);
+    });
+}
+
+int shvllm_sched_forget(shvllm_sched *s, int unit) {
+    return guard([&] { sched_of(s).Forget(unit); });
+}
+
+int shvllm_sched_counts(shvllm_sched *s, int32_t counts[6]) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        const llm::SchedCounts c = sc.Counts();
+        counts[0] = c.restores, counts[1] = c.batches, counts[2] = c.batch_rows, counts[3] = c.passes;
+        counts[4] = sc.Waiting(), counts[5] = sc.Pending();
+    });
+}
+
+int shvllm_sched_held(shvllm_sched *s, int slot, int32_t *dst, int max, int *n, int *ckpt_len) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        if (slot < 0 || slot >= sc.Slots()) throw llm::Error("llm: slot " + std::to_string(slot));
+        const std::vector<int32_t> &h = sc.Held(slot);
+        if (n) *n = static_cast<int>(h.size());
+        if (dst) std::copy(h.begin(), h.begin() + std::min<size_t>(max, h.size()), dst);
+        if (ckpt_len) *ckpt_len = sc.CheckpointLen(slot);
     });
 }
 

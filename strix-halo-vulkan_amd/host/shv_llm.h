@@ -106,6 +106,51 @@ int shvllm_spec_round(shvllm *h, const int32_t *forced, int n_forced, int32_t *o
  * nanos: draft, verify */
 int shvllm_spec_stats(shvllm *h, int32_t *counts, uint64_t *nanos);
 
+/* ---- the scheduler (backend/llm_sched.go:201-898): several conversations interleaved on one graph.
+ * A request acquires a slot, queues a prefill and then decode steps; the caller's one device thread
+ * calls shvllm_sched_pump, which picks the next pass by the policy (interactive strictly before
+ * background, then least device time, background prefill in preempt chunks, pending decode steps
+ * of one class in one pass), runs it on the graph and books it.  With h NULL the object is the
+ * policy alone over `slots` slots: shvllm_sched_next says what would run, shvllm_sched_finish books
+ * a duration the caller supplies, and no device is touched.  Times are milliseconds on a clock of
+ * the caller's choosing; pump uses the steady clock.  Not thread-safe: one caller at a time. ---- */
+typedef struct shvllm_sched shvllm_sched;
+typedef struct shvllm_sched_opts {
+    int32_t batch, preempt_chunk, reserve, no_batch_decode;
+    double coalesce_ms;
+} shvllm_sched_opts;
+#define SHVLLM_SCHED_MAX_ROWS 64
+typedef struct shvllm_sched_pass {
+    int32_t kind;      /* 0 nothing, 1 one chunk of one unit, 2 a batched decode pass */
+    int32_t unit, slot, pos, n, fresh, restore, take, step; /* kind 1 */
+    int32_t n_units;   /* kind 2 */
+    int32_t units[SHVLLM_SCHED_MAX_ROWS], slots[SHVLLM_SCHED_MAX_ROWS];
+    double wait_ms;    /* kind 0: > 0 while a batch waits for conversations still sampling */
+} shvllm_sched_pass;
+typedef struct shvllm_sched_job {
+    int32_t cls, slot, reused, restored, stepping;
+    double served_ms;
+    uint64_t arrival;
+} shvllm_sched_job;
+int shvllm_sched_open(shvllm *h, int slots, const shvllm_sched_opts *opts, shvllm_sched **out);
+void shvllm_sched_close(shvllm_sched *s);
+/* cls 0 interactive, 1 background; mark: prompt position of the slot's checkpoint, 0 for none */
+int shvllm_sched_acquire(shvllm_sched *s, int cls, const int32_t *prompt, int n, int mark, double now_ms, int *job);
+int shvllm_sched_release(shvllm_sched *s, int job, double now_ms);
+int shvllm_sched_job_info(shvllm_sched *s, int job, shvllm_sched_job *out);
+int shvllm_sched_run(shvllm_sched *s, int job, const int32_t *ids, int n, int fresh, int *unit);
+int shvllm_sched_step(shvllm_sched *s, int job, int32_t id, int *unit);
+int shvllm_sched_withdraw(shvllm_sched *s, int unit);
+int shvllm_sched_next(shvllm_sched *s, double now_ms, shvllm_sched_pass *out);
+int shvllm_sched_finish(shvllm_sched *s, double took_ms, int ok, double now_ms);  /* books the pass shvllm_sched_next handed out last */
+int shvllm_sched_pump(shvllm_sched *s, shvllm_sched_pass *out);
+/* state: 0 queued, 1 done, 2 failed; logits [vocab] when done and given; left: ids not yet run */
+int shvllm_sched_unit(shvllm_sched *s, int unit, int *state, int *left, double *busy_ms, float *logits, int max);
+int shvllm_sched_forget(shvllm_sched *s, int unit);
+/* counts: restores, batched passes, rows in them, passes, jobs waiting for a slot, units queued */
+int shvllm_sched_counts(shvllm_sched *s, int32_t counts[6]);
+int shvllm_sched_held(shvllm_sched *s, int slot, int32_t *dst, int max, int *n, int *ckpt_len);
+
 /* ---- the host sampler (llm.Sampler, llm/sample.go): penalties -> top_k -> top_p -> min_p -> temp -> draw,
  * and speculative sampling's Verify.  No device involved; rows are host floats and come back unchanged. ---- */
 typedef struct shvsampler shvsampler;

@@ -35,6 +35,26 @@ class Config(C.Structure):
 _lib = None
 
 
+SCHED_MAX_ROWS = 64
+INTERACTIVE, BACKGROUND = 0, 1  # backend/llm_sched.go:77-80
+
+
+class SchedOpts(C.Structure):
+    _fields_ = [("batch", C.c_int32), ("preempt_chunk", C.c_int32), ("reserve", C.c_int32), ("no_batch_decode", C.c_int32),
+                ("coalesce_ms", C.c_double)]
+
+
+class SchedPass(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("unit", C.c_int32), ("slot", C.c_int32), ("pos", C.c_int32), ("n", C.c_int32),
+                ("fresh", C.c_int32), ("restore", C.c_int32), ("take", C.c_int32), ("step", C.c_int32), ("n_units", C.c_int32),
+                ("units", C.c_int32 * SCHED_MAX_ROWS), ("slots", C.c_int32 * SCHED_MAX_ROWS), ("wait_ms", C.c_double)]
+
+
+class SchedJob(C.Structure):
+    _fields_ = [("cls", C.c_int32), ("slot", C.c_int32), ("reused", C.c_int32), ("restored", C.c_int32), ("stepping", C.c_int32),
+                ("served_ms", C.c_double), ("arrival", C.c_uint64)]
+
+
 def lib_path():
     return os.path.join(HERE, "libshv_llm.so")
 
@@ -104,6 +124,24 @@ def load():
     L.shvllm_spec_sampler.argtypes = [vp, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int64, C.c_int64]
     L.shvllm_spec_round.argtypes = [vp, i32p, C.c_int, i32p, C.c_int, C.POINTER(C.c_int)]
     L.shvllm_spec_stats.argtypes = [vp, i32p, C.POINTER(C.c_uint64)]
+    dp = C.POINTER(C.c_double)
+    ip = C.POINTER(C.c_int)
+    L.shvllm_sched_open.argtypes = [vp, C.c_int, C.POINTER(SchedOpts), C.POINTER(vp)]
+    L.shvllm_sched_close.argtypes = [vp]
+    L.shvllm_sched_close.restype = None
+    L.shvllm_sched_acquire.argtypes = [vp, C.c_int, i32p, C.c_int, C.c_int, C.c_double, ip]
+    L.shvllm_sched_release.argtypes = [vp, C.c_int, C.c_double]
+    L.shvllm_sched_job_info.argtypes = [vp, C.c_int, C.POINTER(SchedJob)]
+    L.shvllm_sched_run.argtypes = [vp, C.c_int, i32p, C.c_int, C.c_int, ip]
+    L.shvllm_sched_step.argtypes = [vp, C.c_int, C.c_int32, ip]
+    L.shvllm_sched_withdraw.argtypes = [vp, C.c_int]
+    L.shvllm_sched_next.argtypes = [vp, C.c_double, C.POINTER(SchedPass)]
+    L.shvllm_sched_finish.argtypes = [vp, C.c_double, C.c_int, C.c_double]
+    L.shvllm_sched_pump.argtypes = [vp, C.POINTER(SchedPass)]
+    L.shvllm_sched_unit.argtypes = [vp, C.c_int, ip, ip, dp, f32p, C.c_int]
+    L.shvllm_sched_forget.argtypes = [vp, C.c_int]
+    L.shvllm_sched_counts.argtypes = [vp, i32p]
+    L.shvllm_sched_held.argtypes = [vp, C.c_int, i32p, C.c_int, ip, ip]
     _lib = L
     return L
 
@@ -388,3 +426,88 @@ class LLM:
         return dict(rounds=int(counts[0]), drafted=int(counts[1]), accepted=int(counts[2]), tokens=int(counts[3]),
                     passes=counts[4:9].tolist(), drafted_at=counts[9:13].tolist(), accepted_at=counts[13:17].tolist(),
                     draft_ns=int(nanos[0]), verify_ns=int(nanos[1]))
+
+
+class Sched:
+    """The scheduler over one staged graph (backend/llm_sched.go), or, with llm=None, its policy
+    alone over `slots` slots: next() says which pass would run and finish() books a duration the
+    caller names, with no device involved."""
+
+    def __init__(self, llm=None, slots=1, batch=2048, preempt_chunk=0, reserve=1, no_batch_decode=False, coalesce_ms=5.0):
+        self.L = load()
+        self.llm = llm
+        o = SchedOpts(batch, preempt_chunk, reserve, int(no_batch_decode), coalesce_ms)
+        s = C.c_void_p()
+        _check(self.L.shvllm_sched_open(llm.h if llm is not None else None, slots, C.byref(o), C.byref(s)))
+        self.s = s
+
+    def close(self):
+        if self.s:
+            self.L.shvllm_sched_close(self.s)
+            self.s = None
+
+    def acquire(self, cls, prompt, mark=0, now_ms=0.0):
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        job = C.c_int()
+        _check(self.L.shvllm_sched_acquire(self.s, cls, prompt.ctypes.data_as(C.POINTER(C.c_int32)), len(prompt), mark, now_ms, C.byref(job)))
+        return job.value
+
+    def release(self, job, now_ms=0.0):
+        _check(self.L.shvllm_sched_release(self.s, job, now_ms))
+
+    def job(self, job):
+        j = SchedJob()
+        _check(self.L.shvllm_sched_job_info(self.s, job, C.byref(j)))
+        return j
+
+    def run(self, job, ids, fresh):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        u = C.c_int()
+        _check(self.L.shvllm_sched_run(self.s, job, ids.ctypes.data_as(C.POINTER(C.c_int32)), len(ids), int(fresh), C.byref(u)))
+        return u.value
+
+    def step(self, job, tok):
+        u = C.c_int()
+        _check(self.L.shvllm_sched_step(self.s, job, int(tok), C.byref(u)))
+        return u.value
+
+    def withdraw(self, unit):
+        _check(self.L.shvllm_sched_withdraw(self.s, unit))
+
+    def next(self, now_ms=0.0):
+        p = SchedPass()
+        _check(self.L.shvllm_sched_next(self.s, now_ms, C.byref(p)))
+        return p
+
+    def finish(self, took_ms, ok=True, now_ms=0.0):
+        _check(self.L.shvllm_sched_finish(self.s, took_ms, int(ok), now_ms))
+
+    def pump(self):
+        p = SchedPass()
+        _check(self.L.shvllm_sched_pump(self.s, C.byref(p)))
+        return p
+
+    def unit(self, unit, want_logits=False):
+        """(state, ids left, device ms, logits): state 0 queued, 1 done, 2 failed (self.error then says why)."""
+        st, left, busy = C.c_int(), C.c_int(), C.c_double()
+        logits = np.empty(self.llm.cfg.vocab, np.float32) if want_logits and self.llm is not None else None
+        rc = self.L.shvllm_sched_unit(self.s, unit, C.byref(st), C.byref(left), C.byref(busy),
+                                      logits.ctypes.data_as(C.POINTER(C.c_float)) if logits is not None else None,
+                                      len(logits) if logits is not None else 0)
+        _check(rc)
+        self.error = self.L.shvllm_last_error().decode("utf-8", "replace") if st.value == 2 else ""
+        return st.value, left.value, busy.value, logits
+
+    def forget(self, unit):
+        _check(self.L.shvllm_sched_forget(self.s, unit))
+
+    def counts(self):
+        c = np.zeros(6, np.int32)
+        _check(self.L.shvllm_sched_counts(self.s, c.ctypes.data_as(C.POINTER(C.c_int32))))
+        return dict(restores=int(c[0]), batches=int(c[1]), batch_rows=int(c[2]), passes=int(c[3]), waiting=int(c[4]), pending=int(c[5]))
+
+    def held(self, slot, max_ids=1 << 16):
+        dst = np.empty(max_ids, np.int32)
+        n, ck = C.c_int(), C.c_int()
+        _check(self.L.shvllm_sched_held(self.s, slot, dst.ctypes.data_as(C.POINTER(C.c_int32)), max_ids, C.byref(n), C.byref(ck)))
+        return dst[:min(n.value, max_ids)].copy(), ck.value

@@ -1,0 +1,183 @@
+"""The scheduler running conversations on the GPU: the reference's three gates of this kind,
+TestLLMConcurrentIsSolo, TestLLMInteractiveGoesFirst and TestLLMCheckpointIsTheSystemPrompt
+(backend/llm_sched_test.go:82, :147, :253), on a synthetic model with greedy sampling.
+
+A conversation here is what backend/llm.go:472-606 does around the scheduler: acquire a slot,
+queue the prompt past what the slot saves, then one decode step per sampled token.  The test's
+one thread pumps the scheduler, so the order of passes is the policy's alone."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+import shv
+
+pytestmark = pytest.mark.gpu
+LA = shv.pkg.llm_api
+I, B = LA.INTERACTIVE, LA.BACKGROUND
+
+
+@pytest.fixture(scope="module")
+def rig():
+    cfg = LA.Config(n_layer=4, n_expert=16, n_expert_used=4, vocab=4096, nkv=512, max_tokens=64, slots=3,
+                    head_rows=3, speculative=0, nextn=0)
+    m = LA.LLM(cfg)
+    m.init_synthetic(2468)
+    m.stage()
+    yield m, cfg
+    m.close()
+
+
+class Conv:
+    """One greedy request."""
+
+    def __init__(self, s, cls, prompt, n, mark=0):
+        self.s, self.n = s, n
+        self.prompt = np.asarray(prompt, np.int32)
+        self.job = s.acquire(cls, self.prompt, mark)
+        self.unit = None
+        self.toks, self.logits, self.at_pass = [], [], []
+        self.done = False
+        self.reused = self.restored = self.born = None
+
+    def poll(self, passes):
+        """Moves the request on as far as it goes without the device; True while it is live."""
+        if self.done:
+            return False
+        if self.born is None:
+            self.born = passes
+        if self.unit is None:
+            j = self.s.job(self.job)
+            if j.slot < 0:
+                return True
+            self.reused, self.restored = j.reused, bool(j.restored)
+            self.unit = self.s.run(self.job, self.prompt[j.reused:], j.reused == 0)
+            return True
+        st, _, _, lg = self.s.unit(self.unit, want_logits=True)
+        if st == 0:
+            return True
+        assert st == 1, self.s.error
+        self.s.forget(self.unit)
+        self.logits.append(lg)
+        self.toks.append(int(np.argmax(lg)))
+        self.at_pass.append(passes)
+        if len(self.toks) == self.n:
+            self.s.release(self.job)
+            self.done = True
+            return False
+        self.unit = self.s.step(self.job, self.toks[-1])
+        return True
+
+
+def drive(s, convs, arrivals=()):
+    """Pumps until every conversation is through.  arrivals: (condition, factory) pairs; a factory is
+    called, once, at the first moment its condition holds, and the conversation it makes joins."""
+    convs = list(convs)
+    arrivals = list(arrivals)
+    passes = 0
+    for _ in range(100000):
+        for k in range(len(arrivals) - 1, -1, -1):
+            if arrivals[k][0]():
+                convs.append(arrivals.pop(k)[1]())
+        live = [c.poll(passes) for c in convs]
+        if not any(live) and not arrivals:
+            return convs
+        p = s.pump()
+        if p.kind:
+            passes += 1
+        else:
+            assert p.wait_ms > 0 or any(c.unit is None for c in convs if not c.done), "nothing to run and nobody sampling"
+    raise AssertionError("the conversations never finished")
+
+
+def same_until_a_tie(got, want):
+    """Greedy tokens of two runs that went through different kernels (a row of a batched pass, a
+    pass of its own) agree until a step whose two best logits are closer than the runs differ."""
+    for t, (a, b) in enumerate(zip(got.toks, want.toks)):
+        diff = float(np.max(np.abs(got.logits[t] - want.logits[t])))
+        assert O.rel_l2(got.logits[t], want.logits[t]) <= 1e-4, t
+        if a != b:
+            top = np.sort(want.logits[t])[-2:]
+            assert top[1] - top[0] < 2 * diff, (t, a, b, top, diff)
+            return t
+    return len(want.toks)
+
+
+def test_concurrent_is_solo(rig):
+    m, cfg = rig
+    rng = np.random.default_rng(5)
+    prompts = [rng.integers(0, cfg.vocab, size=k).astype(np.int32) for k in (9, 150, 23)]
+    n = 24
+    s = LA.Sched(m, reserve=0, preempt_chunk=16)
+    try:
+        solo = []
+        for p in prompts:
+            solo += drive(s, [Conv(s, B, p, n)])
+        assert s.counts()["batches"] == 0
+        both = drive(s, [Conv(s, B, p, n) for p in prompts])
+        c = s.counts()
+        assert c["batches"] > 0, "no decode step shared a pass, so the comparison says nothing about batching"
+        assert c["batch_rows"] / c["batches"] > 2.0
+        for k in range(3):
+            assert both[k].reused == 0
+            agreed = same_until_a_tie(both[k], solo[k])
+            assert agreed >= n // 2, (k, agreed)
+        # the long prompt went in chunks of 16 between the others' work and still is the one sequence
+        assert both[1].at_pass[0] > both[0].at_pass[0]
+    finally:
+        s.close()
+
+
+@pytest.mark.parametrize("cls", [I, B])
+def test_interactive_goes_first(rig, cls):
+    m, cfg = rig
+    rng = np.random.default_rng(6)
+    s = LA.Sched(m, reserve=0, preempt_chunk=16)
+    try:
+        bg = [Conv(s, B, rng.integers(0, cfg.vocab, size=12).astype(np.int32), 60) for _ in range(2)]
+        made = []
+
+        def arrive():
+            made.append(Conv(s, cls, rng.integers(0, cfg.vocab, size=40).astype(np.int32), 16))
+            return made[0]
+
+        drive(s, bg, [(lambda: all(len(c.toks) >= 4 for c in bg), arrive)])
+        fg = made[0]
+        first, last = fg.at_pass[0], fg.at_pass[-1]
+        during = [sum(1 for t in c.at_pass if first < t <= last) for c in bg]
+        after = [sum(1 for t in c.at_pass if t > last) for c in bg]
+        assert all(a > 0 for a in after), "the background requests finished first, so the run shows nothing"
+        if cls == I:
+            assert max(during) <= 1, during
+            # nor did it wait behind their steps: its prompt was the very next pass, in one chunk
+            assert fg.at_pass[0] - fg.born == 1
+        else:
+            assert min(during) > 1, during
+            assert fg.at_pass[0] - fg.born > 3, "a background prompt of 40 goes in three chunks between the others' steps"
+    finally:
+        s.close()
+
+
+def test_checkpoint_is_the_system_prompt(rig):
+    m, cfg = rig
+    rng = np.random.default_rng(7)
+    sysp, other = (rng.integers(0, cfg.vocab, size=k).astype(np.int32) for k in (140, 120))
+    ask, ask2, q = (rng.integers(0, cfg.vocab, size=k).astype(np.int32) for k in (11, 9, 6))
+    s = LA.Sched(m, reserve=0)
+    try:
+        def run(system, turn, n):
+            c = Conv(s, I, np.concatenate([system, turn]), n, mark=len(system))
+            return drive(s, [c])[0]
+
+        run(other, q, 8)
+        want = run(sysp, ask, 24)
+        assert s.counts()["restores"] == 0 and want.reused == 0
+        mid = run(sysp, ask2, 8)     # restores the system prompt and runs on past it
+        assert (mid.reused, mid.restored) == (len(sysp), True)
+        got = run(sysp, ask, 24)      # so this restore has a detour to undo
+        assert (got.reused, got.restored) == (len(sysp), True)
+        assert s.counts()["restores"] == 2
+        assert got.toks == want.toks
+        for a, b in zip(got.logits, want.logits):
+            assert np.array_equal(a, b)  # the same chunks over the same bytes
+    finally:
+        s.close()
