@@ -169,7 +169,7 @@ struct RowStream {
 // A sub-block's eight weights per lane are formed once, as the whole numbers n * sc, and multiplied
 // with every token tile; the matrix accumulators run over a super-block and take its d at its end,
 // the min term is subtracted per sub-block: y = sum_sb d * (sum x * n * sc) - sum_sub dmin * m * sum(x).
-template <int NG, int R>
+template <int NG, int R, int SXS = kTok>
 __device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], RowStream<R> &st, int G0, int G_last, const char *frags,
                                                  const float *sxs, int lane, int n_tt, float4_t (&acc)[R][kTT], float4_t (&y)[R][kTT]) {
     const int kb = lane >> 4;
@@ -217,8 +217,18 @@ __device__ __forceinline__ void slab_times_tiles(const char *const (&rp)[R], Row
                 const char *f = frags + static_cast<size_t>((sub * 2) * kTT + tt) * kFrag + lane * 16;
                 const half8_t xh = *reinterpret_cast<const half8_t *>(f);
                 const half8_t xl = *reinterpret_cast<const half8_t *>(f + kTT * kFrag);
-                const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * kTok + 16 * tt + 4 * kb);
-                const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
+                float sxv[4];
+                if constexpr (SXS > 0) {
+                    const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * SXS + 16 * tt + 4 * kb);
+                    sxv[0] = sx.x, sxv[1] = sx.y, sxv[2] = sx.z, sxv[3] = sx.w;
+                } else {
+                    // the sub-block's sum of x per token, from the operands themselves: a product
+                    // with ones leaves token 4 kb + j's sum in register j of every lane
+                    const half8_t ones = static_cast<half8_t>(static_cast<_Float16>(1.f));
+                    float4_t s4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, ones, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    s4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, ones, s4, 0, 0, 0);
+                    sxv[0] = s4[0], sxv[1] = s4[1], sxv[2] = s4[2], sxv[3] = s4[3];
+                }
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc[r][tt], 0, 0, 0);
@@ -279,6 +289,297 @@ __device__ __forceinline__ void rows_times_tiles(const char *const (&rp)[kTiles]
     }
 }
 
+// The same product over rows that a launch before this one has made into operands, a row's
+// own bytes together (moe_stage_kernel): [row][sub-block][part hi, lo][block of 8 columns] x 16
+// bytes, 128 bytes a sub-block, the eight columns in slot order.  A slab of 256 columns is 48
+// fragments which the loads place in LDS themselves, a lane's 16 bytes each from the listed row it
+// stands for (the four lanes of a row read 64 bytes in a line, the other part the line's other
+// half), so staging costs no vector work and no registers, and the next slab is on its way while
+// this one is multiplied.  Wave w asks for sub-block w of the slab: its two parts for every token
+// tile.  The sub-blocks' sums of x come from the operands (slab_times_tiles with SXS 0).
+// tok_s: the listed rows' numbers in the staged array.
+// The masks and exponents of the two nibble positions a weight is read from.
+struct NibbleMasks {
+    uint32_t m0, m4;  // bits 0..3, 4..7 of both halves
+    uint32_t o0, o4;  // the halves 1024, 64
+};
+__device__ __forceinline__ NibbleMasks nibble_masks() {
+    NibbleMasks c;
+    c.m0 = 0x000F000Fu, c.m4 = 0x00F000F0u;
+    c.o0 = 0x64006400u, c.o4 = 0x54005400u;
+    // opaque to the optimiser: a mask in a scalar register and an exponent in a vector one make (q & m) | o one instruction
+    asm volatile("" : "+s"(c.m0), "+s"(c.m4));
+    asm volatile("" : "+v"(c.o0), "+v"(c.o4));
+    return c;
+}
+
+typedef const __attribute__((address_space(1))) void *global_ptr_t;
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+constexpr int kStWaves = kWaves;                 // waves of a block of the staged kernels: two such blocks share a compute unit, one's waits under the other's work
+constexpr int kStThreads = kStWaves * 64;
+constexpr int kStSubs = kStWaves;             // sub-blocks of a staged slab: one a wave
+constexpr int kStQuarter = 1024 / (32 * kStSubs);  // slabs in the 1024 columns one min-term product covers
+constexpr int kStSlab = 32 * kStSubs;
+constexpr int kStFrags = kStSubs * 2 * kTT * kFrag;
+constexpr int kStSubBytes = 128;              // a row's sub-block: 2 parts x 4 column blocks x 16 bytes
+constexpr int kStSumFrags = kTT * 2 * kFrag;   // the sums of a quarter of the columns (four super-blocks): [token tile][part]
+constexpr int kStMinHdrs = kStWaves * kTiles * kFrag;   // every lane's row header of its super-block of the quarter, a wave's own
+constexpr size_t kStagedLds = 2 * static_cast<size_t>(kStFrags) + 2 * kStSumFrags + kStMinHdrs + 2 * kTok * 4;
+
+// After the rows, every row's sums of x over its sub-blocks, as operands too: [row][super-block]
+// x 32 bytes, the eight sums' binary16 values and then what those leave.
+__host__ __device__ constexpr size_t staged_sums_offset(int rows, int k) { return static_cast<size_t>(rows) * (k / 32) * 128; }
+__host__ __device__ constexpr size_t staged_bytes(int rows, int k) { return staged_sums_offset(rows, k) + static_cast<size_t>(rows) * (k / 256) * 32; }
+
+// grid: (k / 1024, rows), 256 threads, a quad of columns each.
+__global__ __launch_bounds__(256) void moe_stage_kernel(const float *x, int x_stride, int k, int rows, char *staged) {
+    const int t = blockIdx.y, c = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (c >= k) return;
+    const float4 v = *reinterpret_cast<const float4 *>(x + static_cast<size_t>(t) * x_stride + c);
+    const float o[4] = {v.x, v.z, v.y, v.w};
+    half4_t h, l;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const _Float16 hi = static_cast<_Float16>(o[j]);
+        h[j] = hi;
+        l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+    }
+    char *e = staged + (static_cast<size_t>(t) * (k / 32) + (c >> 5)) * kStSubBytes + ((c & 31) >> 3) * 16 + ((c & 7) >> 2) * 8;
+    *reinterpret_cast<half4_t *>(e) = h;
+    *reinterpret_cast<half4_t *>(e + 64) = l;
+    // the sub-block's sum: eight neighbouring lanes (k is a multiple of 32, so they are all here)
+    float sum = (v.x + v.y) + (v.z + v.w);
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    sum += __shfl_xor(sum, 4, 64);
+    if ((c & 31) == 0) {
+        const _Float16 hi = static_cast<_Float16>(sum);
+        _Float16 *sp = reinterpret_cast<_Float16 *>(staged + staged_sums_offset(rows, k) + (static_cast<size_t>(t) * (k / 256) + (c >> 8)) * 32) + ((c >> 5) & 7);
+        sp[0] = hi;
+        sp[8] = static_cast<_Float16>(sum - static_cast<float>(hi));
+    }
+}
+
+template <int K>
+__device__ __forceinline__ void ask_staged_slab(const char *staged, const int32_t *tok_s, int m, int n_tt, int sl, char *buf, int lane, int wave) {
+    const int sg = sl * kStSubs + wave;  // this wave's sub-block of the row
+    const int n = lane & 15, kb = lane >> 4;
+#pragma unroll
+    for (int tt = 0; tt < kTT; tt++) {
+        if (tt >= n_tt) break;
+        const int i = 16 * tt + n;
+        const int t = tok_s[i < m ? i : 0];  // a column past the list repeats the first row; nobody reads its products
+        const char *g = staged + (static_cast<size_t>(t) * (K / 32) + sg) * kStSubBytes + kb * 16;
+        char *f = buf + ((wave * 2) * kTT + tt) * kFrag;
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(g), (lds_ptr_t)(f), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(g + 64), (lds_ptr_t)(f + kTT * kFrag), 16, 0, 0);
+    }
+}
+
+// The sums of x of columns [1024 q, 1024 q + 1024), four super-blocks, as the operands of the
+// min term: fragment (token tile, part), lane = token in the tile + 16 * (super-block of the four).
+// The waves share the fragments out.
+template <int K>
+__device__ __forceinline__ void ask_staged_sums(const char *sums, const int32_t *tok_s, int m, int n_tt, int q, char *buf, int lane, int wave) {
+    const int n = lane & 15, kb = lane >> 4;
+    const int sb = 4 * q + kb < K / 256 ? 4 * q + kb : K / 256 - 1;  // past the row: a real sum against a zero weight
+    for (int f = wave; f < 2 * n_tt; f += kStWaves) {
+        const int tt = f >> 1, part = f & 1;
+        const int i = 16 * tt + n;
+        const int t = tok_s[i < m ? i : 0];
+        const char *g = sums + (static_cast<size_t>(t) * (K / 256) + sb) * 32 + part * 16;
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(g), (lds_ptr_t)(buf + f * kFrag), 16, 0, 0);
+    }
+}
+
+// The headers min_terms reads, on their way a slab ahead: lane (row, kb) asks for its R rows'
+// headers of super-block 4 q + kb, into the wave's own kTiles fragments at hbuf.
+template <int K, int R>
+__device__ __forceinline__ void ask_min_headers(const char *const (&rp)[R], int q, char *hbuf, int lane) {
+    const int sb = 4 * q + (lane >> 4) < K / 256 ? 4 * q + (lane >> 4) : 0;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(rp[r] + static_cast<size_t>(sb) * SHV_Q4K_BYTES), (lds_ptr_t)(hbuf + r * kFrag), 16, 0, 0);
+}
+
+// y -= sum over the quarter's sub-blocks of dmin * m * sum(x), on the matrix cores: lane (row,
+// kb) forms its row's eight -dmin * m of super-block 4 q + kb as two halves each (the product has
+// 17 significant bits), the tokens' sums come as two halves too, and three products (the small
+// halves' one is below float32's last bit) add to the accumulators what the vector units would
+// subtract sub-block by sub-block.
+template <int K, int R, int NTT>
+__device__ __forceinline__ void min_terms(int q, const char *sfr, const char *hbuf, int lane, float4_t (&y)[R][NTT]) {
+    const int kb = lane >> 4;
+    const bool on = 4 * q + kb < K / 256;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint4 h = *reinterpret_cast<const uint4 *>(hbuf + r * kFrag + lane * 16);
+        const float nd = on ? -f16_bits_to_f32(h.x >> 16) : 0.f;
+        const uint32_t m03 = h.z & 0x3F3F3F3Fu, m47 = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+        half8_t bh, bl;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float p = nd * static_cast<float>(((j < 4 ? m03 : m47) >> (8 * (j & 3))) & 0xFFu);
+            const _Float16 hi = static_cast<_Float16>(p);
+            bh[j] = hi;
+            bl[j] = static_cast<_Float16>(p - static_cast<float>(hi));
+        }
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) {
+            const half8_t sh = *reinterpret_cast<const half8_t *>(sfr + (tt * 2) * kFrag + lane * 16);
+            const half8_t sl = *reinterpret_cast<const half8_t *>(sfr + (tt * 2 + 1) * kFrag + lane * 16);
+            y[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sh, bh, y[r][tt], 0, 0, 0);
+            y[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sl, bh, y[r][tt], 0, 0, 0);
+            y[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sh, bl, y[r][tt], 0, 0, 0);
+        }
+    }
+}
+
+// slab_times_tiles for staged rows and NTT token tiles, without the min term (min_terms has it):
+// the (sub-block, token tile) steps of a 64-weight group run as one pipeline in which the
+// fragments of the step after this one are read from LDS before this step's products are issued,
+// so no product waits for an LDS read.
+template <int NG, int R, int NTT, typename Ask>
+__device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[R], RowStream<R> &st, int G0, int G_last, const char *frags,
+                                                        int lane, float4_t (&acc)[R][NTT], float4_t (&y)[R][NTT], Ask &&ask_next) {
+    const int kb = lane >> 4;
+    const NibbleMasks nc = nibble_masks();
+    // LDS addresses are 32 bits wide: kept as such, a fragment's place costs no 64-bit arithmetic
+    typedef const __attribute__((address_space(3))) char *lds_bytes_t;
+    typedef const __attribute__((address_space(3))) half8_t *lds_half8_t;
+    const lds_bytes_t fl = (lds_bytes_t)(frags) + lane * 16;
+    half8_t nh = *(lds_half8_t)(fl), nl = *(lds_half8_t)(fl + kTT * kFrag);
+#pragma unroll 1
+    for (int gi = 0; gi < NG; gi++) {
+        const int G = G0 + gi, g = G & 3;
+        const lds_bytes_t fg = fl + gi * (4 * kTT * kFrag);                     // this group's two sub-blocks
+        const lds_bytes_t fn = gi + 1 < NG ? fg + 4 * kTT * kFrag : fl;        // the group after it (the slab's first again past its last, unused)
+        uint2 q[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) q[r] = st.q_next[r];
+        // the group's bytes are here: only now the loads that nothing in this slab waits for (a
+        // wait for loaded registers also waits for every load issued before them)
+        asm volatile("" : "+v"(q[0].x), "+v"(q[1].x), "+v"(q[2].x), "+v"(q[3].x));
+        if (gi == 0) ask_next();
+        st.ask_group(rp, G + 1, G_last, kb);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay up here, a group ahead of their use
+        uint32_t sc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint32_t mn;
+            q4k_group_scale_min(st.hdr[r], g, sc[r], mn);
+        }
+#pragma unroll
+        for (int hi = 0; hi < 2; hi++) {
+            half8_t b[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const uint32_t q0 = q[r].x, q1 = q[r].y;
+                typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                // A nibble in the low bits of a half's mantissa reads, under the right exponent, as
+                // C + n: bits 0..3 under 1024's, bits 4..7 under 64's (the odd bytes' nibbles take
+                // one shift down there).  One fused multiply-add then makes (C + n) * sc - C * sc =
+                // n * sc: a whole number up to 15 * 63, exact in binary16, as are C * sc.
+                const _Float16 s1 = static_cast<_Float16>(static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu));
+                const half2_t s2 = {s1, s1};
+                half2_t w[4], c[4];
+                if (hi == 0) {
+                    w[0] = __builtin_bit_cast(half2_t, (q0 & nc.m0) | nc.o0); w[1] = __builtin_bit_cast(half2_t, ((q0 >> 4) & nc.m4) | nc.o4);
+                    w[2] = __builtin_bit_cast(half2_t, (q1 & nc.m0) | nc.o0); w[3] = __builtin_bit_cast(half2_t, ((q1 >> 4) & nc.m4) | nc.o4);
+                    c[0] = c[2] = s2 * static_cast<half2_t>(static_cast<_Float16>(-1024.f));
+                    c[1] = c[3] = s2 * static_cast<half2_t>(static_cast<_Float16>(-64.f));
+                } else {
+                    w[0] = __builtin_bit_cast(half2_t, (q0 & nc.m4) | nc.o4); w[1] = __builtin_bit_cast(half2_t, ((q0 >> 8) & nc.m4) | nc.o4);
+                    w[2] = __builtin_bit_cast(half2_t, (q1 & nc.m4) | nc.o4); w[3] = __builtin_bit_cast(half2_t, ((q1 >> 8) & nc.m4) | nc.o4);
+                    c[0] = c[1] = c[2] = c[3] = s2 * static_cast<half2_t>(static_cast<_Float16>(-64.f));
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const half2_t p = __builtin_elementwise_fma(w[i], s2, c[i]);
+                    b[r][2 * i] = p[0];
+                    b[r][2 * i + 1] = p[1];
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < NTT; tt++) {
+                const half8_t xh = nh, xl = nl;
+                // the step after this one: the next token tile, the next sub-block's first, or (past
+                // the slab's last) the first again, unused
+                const int ntt = tt + 1 < NTT ? tt + 1 : 0;
+                const lds_bytes_t f = tt + 1 < NTT ? fg + ((hi * 2) * kTT + ntt) * kFrag : (hi == 0 ? fg + 2 * kTT * kFrag : fn);
+                nh = *(lds_half8_t)(f);
+                nl = *(lds_half8_t)(f + kTT * kFrag);
+#pragma unroll
+                for (int r = 0; r < R; r++) acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc[r][tt], 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < R; r++) acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc[r][tt], 0, 0, 0);
+            }
+        }
+        if (g == 3) {
+            // the super-block ends: its sums take its d, the next one's header moves in
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const float dd = f16_bits_to_f32(st.hdr[r].x);
+#pragma unroll
+                for (int tt = 0; tt < NTT; tt++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(dd, acc[r][tt][j], y[r][tt][j]);
+                    acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            st.ask_header(rp, (G >> 2) + 1, G_last >> 2);
+#pragma unroll
+            for (int r = 0; r < R; r++) st.hdr[r] = st.hdr_next[r];
+        }
+    }
+}
+
+template <int K, int NTT>
+__device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTiles], const char *staged, size_t sums_offset, const int32_t *tok_s, int m,
+                                                   char *bufs, int lane, int wave, float4_t (&y)[kTiles][NTT]) {
+    constexpr int GROUPS = K / 64, NG = kStSlab / 64, SLABS = K / kStSlab;
+    static_assert(K % kStSlab == 0, "whole slabs");
+#pragma unroll
+    for (int r = 0; r < kTiles; r++)
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) y[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float4_t acc[kTiles][NTT];
+#pragma unroll
+    for (int r = 0; r < kTiles; r++)
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const char *sums = staged + sums_offset;
+    char *sum_bufs = bufs + 2 * kStFrags;
+    char *hbuf = sum_bufs + 2 * kStSumFrags + wave * (kTiles * kFrag);
+    ask_staged_slab<K>(staged, tok_s, m, NTT, 0, bufs, lane, wave);
+    ask_staged_sums<K>(sums, tok_s, m, NTT, 0, sum_bufs, lane, wave);
+    ask_min_headers<K, kTiles>(rp, 0, hbuf, lane);
+    RowStream<kTiles> st;
+    st.ask_header(rp, 0, GROUPS / 4 - 1);
+#pragma unroll
+    for (int r = 0; r < kTiles; r++) st.hdr[r] = st.hdr_next[r];
+    st.ask_group(rp, 0, GROUPS - 1, lane >> 4);
+#pragma unroll 1
+    for (int sl = 0; sl < SLABS; sl++) {
+        char *buf = bufs + (sl & 1) * kStFrags;
+        // this wave's loads have landed, then everybody's: the slab is whole, and the buffer the
+        // next one goes to has been read to its end
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        if (sl % kStQuarter == 0) min_terms<K, kTiles, NTT>(sl / kStQuarter, sum_bufs + ((sl / kStQuarter) & 1) * kStSumFrags, hbuf, lane, y);
+        staged_slab_times_tiles<NG, kTiles, NTT>(rp, st, sl * NG, GROUPS - 1, buf, lane, acc, y, [&] {
+            if (sl + 1 < SLABS) {
+                ask_staged_slab<K>(staged, tok_s, m, NTT, sl + 1, bufs + ((sl + 1) & 1) * kStFrags, lane, wave);
+                if ((sl + 1) % kStQuarter == 0) {
+                    const int q = (sl + 1) / kStQuarter;
+                    ask_staged_sums<K>(sums, tok_s, m, NTT, q, sum_bufs + (q & 1) * kStSumFrags, lane, wave);
+                    ask_min_headers<K, kTiles>(rp, q, hbuf, lane);
+                }
+            }
+        });
+    }
+}
+
 // Which expert, which part of its rows and which of its tokens a block takes.  The first
 // parts * ceil(n_tok / 16) blocks are the shared expert, one per (part, tile of 16 tokens); the
 // rest are the routed experts (every token tile of the expert's list in turn).
@@ -319,21 +620,45 @@ struct Staging {
 };
 constexpr size_t kGroupedLds = static_cast<size_t>(kSlabSubs) * 2 * kTT * kFrag + static_cast<size_t>(kSlabSubs) * kTok * 4 + kTok * sizeof(float *) + kTok * 4;
 
+// One pass of a block of the gate/up kernel over up to 16 NTT of its tokens: the products, SwiGLU, act out.
+template <int K, int NTT>
+__device__ __forceinline__ void up_pass(const shv_moe_up_args &a, const char *const (&rp)[kTiles], const char *staged, const int32_t *tok_s,
+                                        const int32_t *pair_s, int m, char *smem, int row) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, kb = lane >> 4;
+    float4_t y[kTiles][NTT];
+    staged_times_tiles<K, NTT>(rp, staged, staged_sums_offset(a.n_tok, K), tok_s, m, smem, lane, wave, y);
+#pragma unroll
+    for (int tt = 0; tt < NTT; tt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = 16 * tt + 4 * kb + j;
+            if (i < m) {
+#pragma unroll
+                for (int r = 0; r < 2; r++) {
+                    const float gv = y[r][tt][j];
+                    a.act[static_cast<size_t>(pair_s[i]) * a.ffn + row + 16 * r] = gv * sigmoid_exact(gv) * y[2 + r][tt][j];
+                }
+            }
+        }
+}
+
 // grid: n_expert * parts + parts * ceil(n_tok / 48) blocks of 8 waves, parts = ffn / 256; K = n_embd.
 // A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tiles 2w and
 // 2w + 1 and the up tiles of the same rows, so SwiGLU stays in registers.
 template <int K>
-__global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_args a) {
+__global__ __launch_bounds__(kStThreads, 2) void moe_up_grouped_kernel(shv_moe_up_args a, const char *staged) {
     extern __shared__ __align__(16) char smem[];
-    const Staging st(smem);
+    // the two slab buffers, then the listed rows' pair and token numbers
+    int32_t *pair_s = reinterpret_cast<int32_t *>(smem + 2 * kStFrags + 2 * kStSumFrags + kStMinHdrs);
+    int32_t *tok_s = pair_s + kTok;
     const int32_t *group = a.group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
-    const int parts = a.ffn / 256;
+    const int parts = a.ffn / (32 * kStWaves);
     const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, a.n_used, group);
     if (u.count <= 0) return;
     const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
-    const int row = u.part * 256 + wave * 32 + n;   // this lane's first row of the expert, gate and up alike; its second is 16 on
+    const int row = u.part * (32 * kStWaves) + wave * 32 + n;   // this lane's first row of the expert, gate and up alike; its second is 16 on
     const size_t wrow = static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.ffn + row;
     const char *gp = static_cast<const char *>(u.expert < 0 ? a.gate_sh : a.gate_exps) + wrow * row_bytes;
     const char *up = static_cast<const char *>(u.expert < 0 ? a.up_sh : a.up_exps) + wrow * row_bytes;
@@ -342,24 +667,14 @@ __global__ __launch_bounds__(kThreads) void moe_up_grouped_kernel(shv_moe_up_arg
         const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
         if (tid < m) {
             const int pair = u.expert < 0 ? (u.first + t0 + tid) * (a.n_used + 1) + a.n_used : group[a.n_expert + 1 + u.first + t0 + tid];
-            st.pair_s[tid] = pair;
-            st.rows_s[tid] = a.xn + static_cast<size_t>(pair / (a.n_used + 1)) * K;
+            pair_s[tid] = pair;
+            tok_s[tid] = pair / (a.n_used + 1);
         }
-        float4_t y[kTiles][kTT];
-        rows_times_tiles<K>(rp, st.rows_s, m, st.frags, st.sxs, lane, y);
-#pragma unroll
-        for (int tt = 0; tt < kTT; tt++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int i = 16 * tt + 4 * kb + j;
-                if (i < m) {
-#pragma unroll
-                    for (int r = 0; r < 2; r++) {
-                        const float gv = y[r][tt][j];
-                        a.act[static_cast<size_t>(st.pair_s[i]) * a.ffn + row + 16 * r] = gv * sigmoid_exact(gv) * y[2 + r][tt][j];
-                    }
-                }
-            }
+        __syncthreads();   // the list is written; the pass before this one has read its last slab
+        const int n_tt = (m + 15) >> 4;
+        if (n_tt == 3) up_pass<K, 3>(a, rp, staged, tok_s, pair_s, m, smem, row);
+        else if (n_tt == 2) up_pass<K, 2>(a, rp, staged, tok_s, pair_s, m, smem, row);
+        else up_pass<K, 1>(a, rp, staged, tok_s, pair_s, m, smem, row);
         __syncthreads();   // the list is read to the end before the next one replaces it
     }
 }
@@ -439,21 +754,23 @@ bool shapes_covered(const shv_ctx *ctx, int n_tok, int n_embd, int ffn, int n_us
 // repeat, the shapes the kernels are built for, and a selection that is already made (topk from
 // the router).  The launchers in moe.hip have checked that every bank is Q4_K.
 bool shv_moe_up_grouped_covers(const shv_ctx *ctx, const shv_moe_up_args &a) {
-    return a.group && !a.logits && shv_aligned16(a.xn) && shapes_covered(ctx, a.n_tok, a.n_embd, a.ffn, a.n_used, a.n_expert);
+    return a.group && !a.logits && shv_aligned16(a.xn) && shapes_covered(ctx, a.n_tok, a.n_embd, a.ffn, a.n_used, a.n_expert) && ctx->gemm_stage &&
+           staged_bytes(a.n_tok, a.n_embd) <= static_cast<size_t>(shv_ctx::kGemmStageBytes);
 }
 
 bool shv_moe_down_grouped_covers(const shv_ctx *ctx, const shv_moe_down_args &a) {
     return a.group && a.pairs && shv_aligned16(a.act) && shv_aligned16(a.pairs) && shapes_covered(ctx, a.n_tok, a.n_embd, a.ffn, a.n_used, a.n_expert);
 }
 
-// Lists, then the grouped gate/up products.
+// Lists, the rows as operands, then the grouped gate/up products.
 int shv_launch_moe_up_grouped(shv_ctx *ctx, const shv_moe_up_args &a) {
     SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, a.group);
-    constexpr size_t lds = kGroupedLds;
+    SHV_LAUNCH(ctx, moe_stage_kernel, dim3((a.n_embd + 1023) / 1024, a.n_tok), dim3(256), 0, a.xn, a.n_embd, a.n_embd, a.n_tok, ctx->gemm_stage);
+    constexpr size_t lds = kStagedLds;
     static const int raised = raise_lds(&moe_up_grouped_kernel<2048>, lds);
     if (raised != SHV_OK) return raised;
-    const int parts = a.ffn / 256, tiles = (a.n_tok + kTok - 1) / kTok;
-    SHV_LAUNCH(ctx, moe_up_grouped_kernel<2048>, dim3(a.n_expert * parts + parts * tiles), dim3(kThreads), lds, a);
+    const int parts = a.ffn / (32 * kStWaves), tiles = (a.n_tok + kTok - 1) / kTok;
+    SHV_LAUNCH(ctx, moe_up_grouped_kernel<2048>, dim3(a.n_expert * parts + parts * tiles), dim3(kStThreads), lds, a, static_cast<const char *>(ctx->gemm_stage));
     return SHV_OK;
 }
 
