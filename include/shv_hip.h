@@ -248,6 +248,10 @@ typedef struct {
     int32_t no_shared_gate;  /* with logits: nonzero says the router ran without a shared_gate (it then
                                 left logits[n_expert] unwritten), and weights[t][n_used] is stored as 0,
                                 as the router's own selection stores it */
+    int32_t act_packed;      /* grouped path only: act is left as the matrix-core operands the grouped
+                                shv_moe_down reads (two binary16 parts of every value, same bytes a row)
+                                instead of floats; the shv_moe_down of this pass must be the library's
+                                next call on the stream, with act_packed and group_ready set too */
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +
@@ -272,6 +276,7 @@ typedef struct {
     int32_t *group;          /* its workspace */
     float *pairs;            /* and the per-pair products; NULL keeps the per-(token, slot) kernels */
     int32_t group_ready;     /* the lists in `group` are this pass's already */
+    int32_t act_packed;      /* act is what the grouped shv_moe_up left with its act_packed set (needs group_ready) */
 } shv_moe_down_args;
 
 /* Gated DeltaNet step(s) after the fused projection (DeltaNetLayer, llm/deltanet.go:266-327 and

@@ -535,7 +535,7 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
 }
 
 template <int K, int NTT>
-__device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTiles], const char *staged, size_t sums_offset, const int32_t *tok_s, int m,
+__device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTiles], const char *staged, const char *sums, const int32_t *tok_s, int m,
                                                    char *bufs, int lane, int wave, float4_t (&y)[kTiles][NTT]) {
     constexpr int GROUPS = K / 64, NG = kStSlab / 64, SLABS = K / kStSlab;
     static_assert(K % kStSlab == 0, "whole slabs");
@@ -548,7 +548,6 @@ __device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTile
     for (int r = 0; r < kTiles; r++)
 #pragma unroll
         for (int tt = 0; tt < NTT; tt++) acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
-    const char *sums = staged + sums_offset;
     char *sum_bufs = bufs + 2 * kStFrags;
     char *hbuf = sum_bufs + 2 * kStSumFrags + wave * (kTiles * kFrag);
     ask_staged_slab<K>(staged, tok_s, m, NTT, 0, bufs, lane, wave);
@@ -620,23 +619,60 @@ struct Staging {
 };
 constexpr size_t kGroupedLds = static_cast<size_t>(kSlabSubs) * 2 * kTT * kFrag + static_cast<size_t>(kSlabSubs) * kTok * 4 + kTok * sizeof(float *) + kTok * 4;
 
-// One pass of a block of the gate/up kernel over up to 16 NTT of its tokens: the products, SwiGLU, act out.
+// Where the grouped down projection finds a pair's act row when it comes as operands: the row's
+// own 4 * ffn bytes of act in the staged layout, and its sub-blocks' sums in the library's scratch.
+__host__ __device__ constexpr size_t packed_sums_bytes(long long pairs, int ffn) { return static_cast<size_t>(pairs) * (ffn / 256) * 32; }
+
+// One pass of a block of the gate/up kernel over up to 16 NTT of its tokens: the products, SwiGLU, act out
+// (as floats, or, packed, as the operands the grouped down projection stages from).
 template <int K, int NTT>
 __device__ __forceinline__ void up_pass(const shv_moe_up_args &a, const char *const (&rp)[kTiles], const char *staged, const int32_t *tok_s,
-                                        const int32_t *pair_s, int m, char *smem, int row) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, kb = lane >> 4;
+                                        const int32_t *pair_s, int m, char *smem, int row, char *act_sums) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, kb = lane >> 4, n = lane & 15;
     float4_t y[kTiles][NTT];
-    staged_times_tiles<K, NTT>(rp, staged, staged_sums_offset(a.n_tok, K), tok_s, m, smem, lane, wave, y);
+    staged_times_tiles<K, NTT>(rp, staged, staged + staged_sums_offset(a.n_tok, K), tok_s, m, smem, lane, wave, y);
+    // this wave's 32 columns are one sub-block of the down projection's rows
+    const int sub = row >> 5;   // row = 32 * sub + n
+    // column 16 r + n of the sub-block: block of 8 columns 2 r + n / 8, slot of [0, 2, 1, 3, 4, 6, 5, 7]
+    const int p8 = n & 7, slot = (p8 & 4) | ((p8 & 1) << 1) | ((p8 & 2) >> 1);
 #pragma unroll
     for (int tt = 0; tt < NTT; tt++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = 16 * tt + 4 * kb + j;
-            if (i < m) {
+            float v[2];
 #pragma unroll
-                for (int r = 0; r < 2; r++) {
-                    const float gv = y[r][tt][j];
-                    a.act[static_cast<size_t>(pair_s[i]) * a.ffn + row + 16 * r] = gv * sigmoid_exact(gv) * y[2 + r][tt][j];
+            for (int r = 0; r < 2; r++) {
+                const float gv = y[r][tt][j];
+                v[r] = gv * sigmoid_exact(gv) * y[2 + r][tt][j];
+            }
+            if (!a.act_packed) {
+                if (i < m) {
+#pragma unroll
+                    for (int r = 0; r < 2; r++) a.act[static_cast<size_t>(pair_s[i]) * a.ffn + row + 16 * r] = v[r];
+                }
+            } else {
+                // the sub-block's sum: both tiles, the 16 lanes of the token
+                float sum = v[0] + v[1];
+                sum += __shfl_xor(sum, 1, 64);
+                sum += __shfl_xor(sum, 2, 64);
+                sum += __shfl_xor(sum, 4, 64);
+                sum += __shfl_xor(sum, 8, 64);
+                if (i < m) {
+                    const size_t pair = static_cast<size_t>(pair_s[i]);
+                    char *e = reinterpret_cast<char *>(a.act) + (pair * (a.ffn / 32) + sub) * kStSubBytes + (n >> 3) * 16 + slot * 2;
+#pragma unroll
+                    for (int r = 0; r < 2; r++) {
+                        const _Float16 hi = static_cast<_Float16>(v[r]);
+                        *reinterpret_cast<_Float16 *>(e + r * 32) = hi;
+                        *reinterpret_cast<_Float16 *>(e + r * 32 + 64) = static_cast<_Float16>(v[r] - static_cast<float>(hi));
+                    }
+                    if (n == 0) {
+                        const _Float16 hi = static_cast<_Float16>(sum);
+                        _Float16 *sp = reinterpret_cast<_Float16 *>(act_sums + (pair * (a.ffn / 256) + (sub >> 3)) * 32) + (sub & 7);
+                        sp[0] = hi;
+                        sp[8] = static_cast<_Float16>(sum - static_cast<float>(hi));
+                    }
                 }
             }
         }
@@ -646,7 +682,7 @@ __device__ __forceinline__ void up_pass(const shv_moe_up_args &a, const char *co
 // A part is 256 gate rows and the same 256 up rows = 16 + 16 tiles; wave w takes gate tiles 2w and
 // 2w + 1 and the up tiles of the same rows, so SwiGLU stays in registers.
 template <int K>
-__global__ __launch_bounds__(kStThreads, 2) void moe_up_grouped_kernel(shv_moe_up_args a, const char *staged) {
+__global__ __launch_bounds__(kStThreads, 2) void moe_up_grouped_kernel(shv_moe_up_args a, const char *staged, char *act_sums) {
     extern __shared__ __align__(16) char smem[];
     // the two slab buffers, then the listed rows' pair and token numbers
     int32_t *pair_s = reinterpret_cast<int32_t *>(smem + 2 * kStFrags + 2 * kStSumFrags + kStMinHdrs);
@@ -672,9 +708,9 @@ __global__ __launch_bounds__(kStThreads, 2) void moe_up_grouped_kernel(shv_moe_u
         }
         __syncthreads();   // the list is written; the pass before this one has read its last slab
         const int n_tt = (m + 15) >> 4;
-        if (n_tt == 3) up_pass<K, 3>(a, rp, staged, tok_s, pair_s, m, smem, row);
-        else if (n_tt == 2) up_pass<K, 2>(a, rp, staged, tok_s, pair_s, m, smem, row);
-        else up_pass<K, 1>(a, rp, staged, tok_s, pair_s, m, smem, row);
+        if (n_tt == 3) up_pass<K, 3>(a, rp, staged, tok_s, pair_s, m, smem, row, act_sums);
+        else if (n_tt == 2) up_pass<K, 2>(a, rp, staged, tok_s, pair_s, m, smem, row, act_sums);
+        else up_pass<K, 1>(a, rp, staged, tok_s, pair_s, m, smem, row, act_sums);
         __syncthreads();   // the list is read to the end before the next one replaces it
     }
 }
@@ -718,6 +754,55 @@ __global__ __launch_bounds__(kThreads) void moe_down_grouped_kernel(shv_moe_down
                 }
             }
         __syncthreads();
+    }
+}
+
+// One pass of a block of the staged down kernel: the products of up to 16 NTT listed pairs, raw, to pairs[pair].
+template <int K, int NTT>
+__device__ __forceinline__ void down_pass(const shv_moe_down_args &a, const char *const (&rp)[kTiles], const char *act_sums, const int32_t *pair_s,
+                                          int m, char *smem, int row0) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, kb = lane >> 4;
+    float4_t y[kTiles][NTT];
+    staged_times_tiles<K, NTT>(rp, reinterpret_cast<const char *>(a.act), act_sums, pair_s, m, smem, lane, wave, y);
+#pragma unroll
+    for (int tt = 0; tt < NTT; tt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = 16 * tt + 4 * kb + j;
+            if (i < m) {
+                float *dst = a.pairs + static_cast<size_t>(pair_s[i]) * a.n_embd + row0;
+#pragma unroll
+                for (int r = 0; r < kTiles; r++) dst[16 * r] = y[r][tt][j];
+            }
+        }
+}
+
+// The down projection over act rows that the gate/up kernel left as operands (act_packed): the
+// same blocks and tiles as moe_down_grouped_kernel, the rows staged by the loads themselves.
+template <int K>
+__global__ __launch_bounds__(kStThreads, 2) void moe_down_staged_kernel(shv_moe_down_args a, const char *act_sums) {
+    extern __shared__ __align__(16) char smem[];
+    int32_t *pair_s = reinterpret_cast<int32_t *>(smem + 2 * kStFrags + 2 * kStSumFrags + kStMinHdrs);
+    const int32_t *group = a.group;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15;
+    const int parts = a.n_embd / (64 * kStWaves);
+    const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, a.n_used, group);
+    if (u.count <= 0) return;
+    const size_t row_bytes = static_cast<size_t>(K / SHV_Q4K_BLOCK) * SHV_Q4K_BYTES;
+    const int row0 = u.part * (64 * kStWaves) + wave * 64 + n;
+    const char *base = static_cast<const char *>(u.expert < 0 ? a.down_sh : a.down_exps) +
+                       (static_cast<size_t>(u.expert < 0 ? 0 : u.expert) * a.n_embd + row0) * row_bytes;
+    const char *rp[kTiles] = {base, base + 16 * row_bytes, base + 32 * row_bytes, base + 48 * row_bytes};
+    for (int t0 = 0; t0 < u.count; t0 += kTok) {
+        const int m = u.count - t0 < kTok ? u.count - t0 : kTok;
+        if (tid < m) pair_s[tid] = u.expert < 0 ? (u.first + t0 + tid) * (a.n_used + 1) + a.n_used : group[a.n_expert + 1 + u.first + t0 + tid];
+        __syncthreads();   // the list is written; the pass before this one has read its last slab
+        const int n_tt = (m + 15) >> 4;
+        if (n_tt == 3) down_pass<K, 3>(a, rp, act_sums, pair_s, m, smem, row0);
+        else if (n_tt == 2) down_pass<K, 2>(a, rp, act_sums, pair_s, m, smem, row0);
+        else down_pass<K, 1>(a, rp, act_sums, pair_s, m, smem, row0);
+        __syncthreads();   // the list is read to the end before the next one replaces it
     }
 }
 
@@ -770,7 +855,10 @@ int shv_launch_moe_up_grouped(shv_ctx *ctx, const shv_moe_up_args &a) {
     static const int raised = raise_lds(&moe_up_grouped_kernel<2048>, lds);
     if (raised != SHV_OK) return raised;
     const int parts = a.ffn / (32 * kStWaves), tiles = (a.n_tok + kTok - 1) / kTok;
-    SHV_LAUNCH(ctx, moe_up_grouped_kernel<2048>, dim3(a.n_expert * parts + parts * tiles), dim3(kStThreads), lds, a, static_cast<const char *>(ctx->gemm_stage));
+    SHV_REQUIRE(!a.act_packed || (ctx->gemm_part && packed_sums_bytes(static_cast<long long>(a.n_tok) * (a.n_used + 1), a.ffn) <= static_cast<size_t>(shv_ctx::kGemmPartBytes)),
+                "moe_up: %d rows are too many for act_packed", a.n_tok);
+    SHV_LAUNCH(ctx, moe_up_grouped_kernel<2048>, dim3(a.n_expert * parts + parts * tiles), dim3(kStThreads), lds, a, static_cast<const char *>(ctx->gemm_stage),
+               reinterpret_cast<char *>(ctx->gemm_part));
     return SHV_OK;
 }
 
@@ -782,11 +870,20 @@ int shv_launch_moe_down_grouped(shv_ctx *ctx, const shv_moe_down_args &a) {
                     (!a.residual || (a.res_stride % 4 == 0 && shv_aligned16(a.residual))),
                 "moe_down: the grouped path moves 16 bytes at a time");
     if (!a.group_ready) SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
-    constexpr size_t lds = kGroupedLds;
-    static const int raised = raise_lds(&moe_down_grouped_kernel<512>, lds);
-    if (raised != SHV_OK) return raised;
     const int parts = a.n_embd / 512, tiles = (a.n_tok + kTok - 1) / kTok;
-    SHV_LAUNCH(ctx, moe_down_grouped_kernel<512>, dim3(a.n_expert * parts + parts * tiles), dim3(kThreads), lds, a);
+    if (a.act_packed) {
+        SHV_REQUIRE(a.group_ready && ctx->gemm_part, "moe_down: act_packed needs the grouped moe_up of this pass right before (group_ready)");
+        constexpr size_t lds = kStagedLds;
+        static const int raised = raise_lds(&moe_down_staged_kernel<512>, lds);
+        if (raised != SHV_OK) return raised;
+        static_assert(64 * kStWaves == 512, "a part is 512 rows");
+        SHV_LAUNCH(ctx, moe_down_staged_kernel<512>, dim3(a.n_expert * parts + parts * tiles), dim3(kStThreads), lds, a, reinterpret_cast<const char *>(ctx->gemm_part));
+    } else {
+        constexpr size_t lds = kGroupedLds;
+        static const int raised = raise_lds(&moe_down_grouped_kernel<512>, lds);
+        if (raised != SHV_OK) return raised;
+        SHV_LAUNCH(ctx, moe_down_grouped_kernel<512>, dim3(a.n_expert * parts + parts * tiles), dim3(kThreads), lds, a);
+    }
     SHV_LAUNCH(ctx, moe_combine_kernel, dim3((a.n_embd + 1023) / 1024, a.n_tok), dim3(256), 0, a);
     return SHV_OK;
 }

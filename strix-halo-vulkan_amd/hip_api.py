@@ -77,7 +77,7 @@ class MoeUpArgs(C.Structure):
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("logits", C.c_void_p),
                 ("weights", C.c_void_p), ("n_expert", C.c_int32), ("gate_type", C.c_int32),
                 ("up_type", C.c_int32), ("gate_sh_type", C.c_int32), ("up_sh_type", C.c_int32),
-                ("group", C.c_void_p), ("no_shared_gate", C.c_int32)]
+                ("group", C.c_void_p), ("no_shared_gate", C.c_int32), ("act_packed", C.c_int32)]
 
 
 class MoeDownArgs(C.Structure):
@@ -86,7 +86,7 @@ class MoeDownArgs(C.Structure):
                 ("out", C.c_void_p), ("n_tok", C.c_int32), ("n_embd", C.c_int32),
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("res_stride", C.c_int32),
                 ("out_stride", C.c_int32), ("down_type", C.c_int32), ("down_sh_type", C.c_int32),
-                ("n_expert", C.c_int32), ("group", C.c_void_p), ("pairs", C.c_void_p), ("group_ready", C.c_int32)]
+                ("n_expert", C.c_int32), ("group", C.c_void_p), ("pairs", C.c_void_p), ("group_ready", C.c_int32), ("act_packed", C.c_int32)]
 
 
 class DnStepArgs(C.Structure):

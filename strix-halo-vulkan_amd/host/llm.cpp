@@ -525,6 +525,9 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     d.group = group_;
     d.pairs = pairs_;
     d.group_ready = (!fused && up_q4k && group_) ? 1 : 0;  // the up projection of this pass has grouped its rows (or neither takes that road)
+    // both projections in Q4_K, one right after the other: when they group their rows, act goes from one to the other as operands
+    const bool down_q4k = de.ggml == gguf::Q4_K && ds.ggml == gguf::Q4_K;
+    u.act_packed = d.act_packed = (d.group_ready && down_q4k && pairs_) ? 1 : 0;
     d.act = act_;
     d.topk = topk_;
     d.weights = weights_;

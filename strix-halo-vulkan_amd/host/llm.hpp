@@ -201,7 +201,7 @@ public:
     std::vector<float> Logits() const;    // [T][NExpert+1]
     std::vector<int32_t> TopK() const;    // [T][used]
     std::vector<float> Weights() const;   // [T][used+1]
-    std::vector<float> Swiglu() const;    // [T][used+1][ffn]
+    std::vector<float> Swiglu() const;    // [T][used+1][ffn]; of a pass short enough not to be grouped by expert (a grouped pass leaves operands there, not floats)
     std::vector<float> Out() const;       // [T][NEmbd]
     float *InPort() const { return in_; }
     float *OutPort() const { return out_; }

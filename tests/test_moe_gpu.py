@@ -64,9 +64,10 @@ class MoeCase:
         r["xn"] = xn
         return r
 
-    def gpu(self, residual=False, defer=False, grouped=False):
+    def gpu(self, residual=False, defer=False, grouped=False, packed=False, group_ready=None):
         """grouped: hand the expert kernels the workspaces that let a pass of many rows go grouped by
-        expert on the matrix cores."""
+        expert on the matrix cores.  packed: act goes from the gate/up kernel to the down kernel
+        as matrix-core operands instead of floats."""
         c, T, H, E, used, ffn = self.ctx, self.T, self.H, self.E, self.used, self.ffn
         d = {k: c.upload(getattr(self, k)) for k in
              ("router", "shared_gate", "gate_exps", "up_exps", "down_exps", "gate_sh", "up_sh",
@@ -87,6 +88,9 @@ class MoeCase:
             group, pairs = c.alloc((2 * E + 1 + T * used) * 4), c.alloc(T * (used + 1) * H * 4)
             ua.group = da.group = group.ptr
             da.pairs = pairs.ptr
+        if packed:
+            ua.act_packed = da.act_packed = 1
+            da.group_ready = 1 if group_ready is None else group_ready
         ops = [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
         c.dispatch_multi(ops)
         return dict(xn=xn.read(np.float32, T * H).reshape(T, H),
@@ -173,6 +177,14 @@ def test_many_rows_grouped_by_expert_match_oracle(ctx, T, E, used, seed):
     assert O.rel_l2(got["act"], ref["act"]) <= 1e-5
     assert O.rel_l2(got["out"], ref["out"]) <= 1e-5
     assert not np.array_equal(got["out"], ref["out"]), "the workspaces were given: the grouped kernels should have run"
+    # act handed over as operands: the same products, the down projection's rows staged by its loads
+    pk = case.gpu(residual=True, grouped=True, packed=True)
+    assert np.array_equal(pk["topk"], want["topk"])
+    assert O.rel_l2(pk["out"], want["out"] + case.res) <= TOL
+    assert O.rel_l2(pk["out"], got["out"]) <= 1e-5
+    assert not np.array_equal(pk["act"], got["act"]), "act should hold operands, not floats"
+    with pytest.raises(A.ShvError, match="act_packed needs the grouped moe_up"):
+        case.gpu(residual=True, grouped=True, packed=True, group_ready=0)
 
 
 def test_moe_block_with_residual_and_few_experts(ctx):
