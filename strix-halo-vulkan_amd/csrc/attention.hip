@@ -537,33 +537,45 @@ __global__ __launch_bounds__(kBlock) void attn_append_kernel(shv_attn_decode_arg
     vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vsrc[tid]));
 }
 
-// ---- prompt passes: four row pairs a block, every tile of the cache through LDS once ----------
+// ---- prompt passes: eight row pairs a block, every tile of the cache through LDS once ---------
 // The kernel above lets each row pair pull the whole cache for itself, which a pass of a thousand
-// pairs pays in L2 bandwidth.  Here a block is four pairs (64 query rows of one KV head), one a
-// wave: the block copies each 32-cell tile of K and V into LDS once (the next tile's loads are in
-// flight while this one is multiplied) and every wave forms its products from there, as
-// v_mfma_f32_16x16x32_f16 (eight dims or eight cells a lane).  A wave slices the cache and writes
-// its records exactly as a block of the kernel above would for that pair, so the same merge follows.
+// pairs pays in L2 bandwidth.  Here a block is eight pairs (128 query rows of one KV head), one a
+// wave.  A 32-cell tile of K and V is 32 chunks of 1 KB, each exactly what one LDS read of a wave
+// takes (64 lanes x 16 bytes, in lane order: no bank is asked twice), and the loads put them
+// there themselves: a lane names the 16 bytes of the cache that belong at its place in the chunk
+// and the load writes LDS, so a tile passes through no register and costs no vector work.  Four
+// tiles are in the ring: three on their way while one is multiplied.  Every wave forms its
+// products from there, as v_mfma_f32_16x16x32_f16 (eight dims or eight cells a lane), slices the
+// cache and writes its records exactly as a block of the kernel above would for that pair, so the
+// same merge follows.
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-constexpr int kKRow = kD * 2 + 16;     // bytes from one cell of the K tile to the next (16 rows cover all banks)
-constexpr int kVRow = kTile * 2 + 16;  // bytes from one dim of the V tile to the next
-struct PrefillTiles {
-    char kt[2][kTile * kKRow];         // K tile, rows in operand order (score tile T, slot s at row 16 T + s)
-    char vt[2][kD * kVRow];            // V tile, [dim][cell % 32]
-};
+typedef const __attribute__((address_space(1))) void *global_ptr_t;
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+constexpr int kPfWaves = 8;
+constexpr int kPfThreads = kPfWaves * 64;
+constexpr int kPfStages = 4;
+constexpr int kChunk = 64 * 16;
+constexpr int kTileBytes = 32 * kChunk;   // K: chunk 8 T + i (score tile T, 32-dim step i); V: chunk 16 + db (16 dims)
 struct PrefillSmem {
     // the queries pass through here once, on their way from the lanes that normalised them to the
     // lanes that hold them as operands (per wave: [32-dim step][hi, lo][16 * (dim group) + query
-    // row]); after that the same bytes are the tiles, so that two blocks fit a compute unit
+    // row]); after that the same bytes are the ring of tiles
     union {
-        half8_t qf[4][8][2][64];
-        PrefillTiles t;
+        half8_t qf[kPfWaves][8][2][64];
+        char ring[kPfStages][kTileBytes];
     } u;
-    float al[4][16];
 };
 
-// grid: (n_seq * ceil(n_groups / 4), n_head_kv, n_splits); the cells of the pass are in the cache already.
-__global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode_args a, int n_groups, int slice_cells) {
+// The barrier between two tiles.  A wave's loads complete in order, so "at most eight of mine still
+// out" says that all but its two youngest tiles' loads have written LDS; the LDS reads of the tile
+// just multiplied have returned (their values were used); then the workgroup meets.  Written out
+// because __syncthreads() would first wait for every load in flight, the tiles ahead included.
+__device__ __forceinline__ void tile_barrier() {
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// grid: (n_seq * ceil(n_groups / 8), n_head_kv, n_splits); the cells of the pass are in the cache already.
+__global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decode_args a, int n_groups, int slice_cells) {
     extern __shared__ __align__(16) char praw[];
     PrefillSmem &sm = *reinterpret_cast<PrefillSmem *>(praw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -581,8 +593,8 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
         }
     }
     const int split = blockIdx.z;
-    const int bps = (n_groups + 3) / 4;
-    const int seq = bx / bps, g0 = (bx % bps) * 4;
+    const int bps = (n_groups + kPfWaves - 1) / kPfWaves;
+    const int seq = bx / bps, g0 = (bx % bps) * kPfWaves;
     const int slot = a.slot ? a.slot[seq] : seq;
     const int pos_first = a.pos ? a.pos[seq] : 0;
     // pair gg of the sequence: its rows, what it sees, its slice of that
@@ -607,7 +619,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
     const Slice me = slice_of(g0 + wave);
     int lo = 0x7fffffff, hi = 0;
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
+    for (int w = 0; w < kPfWaves; w++) {
         const Slice o = slice_of(g0 + w);
         if (o.mine) {
             lo = o.c0 < lo ? o.c0 : lo;
@@ -623,29 +635,29 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
     const uint16_t *vtg = static_cast<const uint16_t *>(a.vcache) + static_cast<size_t>(slot) * a.max_cells * kvw + static_cast<size_t>(kvh) * kD * kTile;
     const size_t vtile = static_cast<size_t>(kvw) * kTile;
 
-    // ---- the tile copy: 4 + 4 pieces of 16 bytes a thread ----
-    uint4 kr[4], vr[4];
-    auto fetch = [&](int t0) {
+    // ---- the tile copy: four chunks a wave, waves 0..3 the keys, 4..7 the values ----
+    // K chunk (T, i): lane (n, q) stands for score-tile slot n = cell 8 (n / 4) + 4 T + n % 4 of the tile, dims 32 i + 8 q ..;
+    // V chunk db: lane (n, q) stands for dim 16 db + n, cells 8 q .. of the tile.  A tile past the last repeats it.
+    const int last_tile = (hi - 1) / kTile;
+    auto ask_tile = [&](int t0, int stage) {
+        char *ring = sm.u.ring[stage];
+        const int tile = t0 / kTile < last_tile ? t0 / kTile : last_tile;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int e = tid + kBlock * u;
-            int c = t0 + (e >> 5);
-            c = c < hi ? c : hi - 1;
-            kr[u] = *reinterpret_cast<const uint4 *>(kc + static_cast<size_t>(c) * kvw + (e & 31) * 8);
-            vr[u] = *reinterpret_cast<const uint4 *>(vtg + static_cast<size_t>(t0 / kTile) * vtile + (e >> 2) * kTile + (e & 3) * 8);
+            const int ch = 4 * wave + u;
+            const uint16_t *g;
+            if (wave < 4) {
+                const int T = ch >> 3, i = ch & 7;
+                int c = tile * kTile + 8 * (n >> 2) + 4 * T + (n & 3);
+                c = c < hi ? c : hi - 1;
+                g = kc + static_cast<size_t>(c) * kvw + 32 * i + 8 * q;
+            } else {
+                const int db = ch - 16;
+                g = vtg + static_cast<size_t>(tile) * vtile + (16 * db + n) * kTile + 8 * q;
+            }
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(g), (lds_ptr_t)(ring + ch * kChunk), 16, 0, 0);
         }
     };
-    auto stash = [&](int b) {
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int e = tid + kBlock * u;
-            const int cl = e >> 5;                                         // cell of the tile
-            const int rho = 16 * ((cl >> 2) & 1) + 4 * (cl >> 3) + (cl & 3);  // its row in operand order
-            *reinterpret_cast<uint4 *>(sm.u.t.kt[b] + rho * kKRow + (e & 31) * 16) = kr[u];
-            *reinterpret_cast<uint4 *>(sm.u.t.vt[b] + (e >> 2) * kVRow + (e & 3) * 16) = vr[u];
-        }
-    };
-    fetch(lo);
 
     // ---- the wave's 16 query rows: norm, rotation, scale, operand order ----
     {
@@ -689,9 +701,11 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
         qh[i] = sm.u.qf[wave][i][0][lane];
         ql[i] = sm.u.qf[wave][i][1][lane];
     }
-    __syncthreads();   // every wave holds its queries: the bytes become the tiles
-    stash(0);
-    __syncthreads();
+    __syncthreads();   // every wave holds its queries: the bytes become the ring of tiles
+    ask_tile(lo, 0);
+    ask_tile(lo + kTile, 1);
+    ask_tile(lo + 2 * kTile, 2);
+    tile_barrier();   // the first tile has landed: all but the two youngest tiles' loads of every wave
 
     float4_t o[16];
 #pragma unroll
@@ -700,12 +714,12 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
     const int my_row_pos = me.p_first + (n >> 3);
 
     int b = 0;
-    for (int t0 = lo; t0 < hi; t0 += kTile, b ^= 1) {
-        const bool more = t0 + kTile < hi;
-        if (more) fetch(t0 + kTile);
+    for (int t0 = lo; t0 < hi; t0 += kTile, b = (b + 1) & (kPfStages - 1)) {
+        // three tiles on: into the stage read a tile ago (every wave has passed the barrier that ended that tile)
+        ask_tile(t0 + 3 * kTile, (b + 3) & (kPfStages - 1));
         // tiles wholly outside the wave's slice or beyond what its rows see are skipped
         if (me.mine && t0 < me.c1 && t0 + kTile > me.c0 && t0 <= me.p_first + 1) {
-            const char *kt = sm.u.t.kt[b], *vt = sm.u.t.vt[b];
+            const char *kt = sm.u.ring[b], *vt = sm.u.ring[b] + 16 * kChunk;
             // operands come from LDS four reads ahead of the products that use them: a read's
             // latency is about what eight products take, and asked for one at a time it is paid 32 times a tile
             float4_t st[2];
@@ -721,7 +735,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int i = 2 * g4 + (e >> 1), T = e & 1;
-                        dst[e] = *reinterpret_cast<const half8_t *>(kt + (16 * T + n) * kKRow + (32 * i + 8 * q) * 2);
+                        dst[e] = *reinterpret_cast<const half8_t *>(kt + (8 * T + i) * kChunk + lane * 16);
                     }
                 };
                 read_k(kb[0], 0);
@@ -737,7 +751,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
                 }
                 // the first values go out now, under the softmax arithmetic
 #pragma unroll
-                for (int e = 0; e < 4; e++) vb[0][e] = *reinterpret_cast<const half8_t *>(vt + (16 * e + n) * kVRow + 16 * q);
+                for (int e = 0; e < 4; e++) vb[0][e] = *reinterpret_cast<const half8_t *>(vt + e * kChunk + lane * 16);
                 st[0] = acc[0][0] + acc[0][1];
                 st[1] = acc[1][0] + acc[1][1];
             }
@@ -772,21 +786,20 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
             l_run = l_run * alpha + sum;
             m_run = m_new;
             if (__ballot(alpha != 1.f) != 0ull) {
-                if (q == 0) sm.al[wave][n] = alpha;
-                __builtin_amdgcn_wave_barrier();
-                const float4 af = *reinterpret_cast<const float4 *>(&sm.al[wave][4 * q]);
-                const float av[4] = {af.x, af.y, af.z, af.w};
+                // a lane's four accumulator rows are query rows 4 q + i: their factors sit in lanes 4 q + i
+                float av[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) av[i] = __shfl(alpha, 4 * q + i, 64);
 #pragma unroll
                 for (int db = 0; db < 16; db++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) o[db][i] *= av[i];
-                __builtin_amdgcn_wave_barrier();
             }
 #pragma unroll
             for (int g4 = 0; g4 < 4; g4++) {
                 if (g4 + 1 < 4) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) vb[(g4 + 1) & 1][e] = *reinterpret_cast<const half8_t *>(vt + (16 * (4 * (g4 + 1) + e) + n) * kVRow + 16 * q);
+                    for (int e = 0; e < 4; e++) vb[(g4 + 1) & 1][e] = *reinterpret_cast<const half8_t *>(vt + (4 * (g4 + 1) + e) * kChunk + lane * 16);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -798,8 +811,7 @@ __global__ __launch_bounds__(kBlock, 2) void attn_prefill_kernel(shv_attn_decode
                 }
             }
         }
-        if (more) stash(b ^ 1);   // the other buffer was last read a tile ago, before the wait that ended that tile
-        __syncthreads();
+        tile_barrier();   // the next tile has landed, this one has been read
     }
     if (!me.mine) return;
     // the wave's record of this slice: per row and head the unnormalised sums, then (max, sum)
@@ -829,13 +841,13 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
     // 36 units over 2 300 cells took 2.2 us to ask for them, 144 take a quarter of that)
     const int slice_cells = a.n_seq * n_groups == 1 ? kTile : kSliceCells;
     if (R == 2 && !append && row0 == 0 && n_groups >= 8) {
-        // a prompt pass: four pairs a block share the cache's tiles
+        // a prompt pass: eight pairs a block share the cache's tiles
         static bool raised = false;
         if (!raised) {
             SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
             raised = true;
         }
-        SHV_LAUNCH(ctx, attn_prefill_kernel, dim3(a.n_seq * ((n_groups + 3) / 4), a.n_head_kv, b.n_splits), dim3(kBlock), sizeof(PrefillSmem), b, n_groups, slice_cells);
+        SHV_LAUNCH(ctx, attn_prefill_kernel, dim3(a.n_seq * ((n_groups + kPfWaves - 1) / kPfWaves), a.n_head_kv, b.n_splits), dim3(kPfThreads), sizeof(PrefillSmem), b, n_groups, slice_cells);
     } else {
         dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
         SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
