@@ -813,6 +813,8 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
         }
         tile_barrier();   // the next tile has landed, this one has been read
     }
+    // the loads asked for past the last tile still write LDS: none may be out when the wave ends and its LDS goes to another workgroup
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (!me.mine) return;
     // the wave's record of this slice: per row and head the unnormalised sums, then (max, sum)
     float *rec = a.partial + ((static_cast<size_t>(gz) * a.n_head_kv + kvh) * a.n_splits + split) * 2 * kRec;
