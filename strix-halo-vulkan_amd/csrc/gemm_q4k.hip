@@ -424,7 +424,12 @@ constexpr int kWideFrag = 64 * 16;                           // one operand: a l
 constexpr int kWideSlabA = 4 * 4 * 2 * kWideFrag;            // [sub-block 4][token tile 4][hi, lo]
 constexpr int kWideSlab = kWideSlabA + 4 * kWideTok * 4;     // + the sub-blocks' sums of x
 
-__host__ __device__ constexpr size_t wide_region(int k) { return static_cast<size_t>(k / 128) * kWideSlab; }
+// After a group's slabs, the same sums as operands of the min term: for every 1024 columns (four
+// super-blocks) a fragment per (token tile, part): lane = token in the tile + 16 * (super-block of
+// the four), the super-block's eight sums' binary16 values (part 0) and what those leave (part 1).
+constexpr int kWideSumFrags = 4 * 2 * kWideFrag;
+__host__ __device__ constexpr size_t wide_sums_offset(int k) { return static_cast<size_t>(k / 128) * kWideSlab; }
+__host__ __device__ constexpr size_t wide_region(int k) { return wide_sums_offset(k) + static_cast<size_t>((k + 1023) / 1024) * kWideSumFrags; }
 
 // Where activation row t of the pass writes its outputs: the DeltaNet projection ring, or plain rows.
 __device__ __forceinline__ size_t out_offset(const shv_gemv_q4k_args &a, int t) {
@@ -472,7 +477,14 @@ __global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args 
     sum += __shfl_xor(sum, 1, 64);
     sum += __shfl_xor(sum, 2, 64);
     sum += __shfl_xor(sum, 4, 64);
-    if ((c & 31) == 0) reinterpret_cast<float *>(slab + kWideSlabA)[sub * kWideTok + tl] = sum;
+    if ((c & 31) == 0) {
+        reinterpret_cast<float *>(slab + kWideSlabA)[sub * kWideTok + tl] = sum;
+        const _Float16 hi = static_cast<_Float16>(sum);
+        _Float16 *sp = reinterpret_cast<_Float16 *>(region + wide_sums_offset(K) + static_cast<size_t>(((c >> 10) * 4 + (tl >> 4)) * 2) * kWideFrag +
+                                                    (((c >> 8) & 3) * 16 + (tl & 15)) * 16) + ((c >> 5) & 7);
+        sp[0] = hi;
+        sp[kWideFrag / 2] = static_cast<_Float16>(sum - static_cast<float>(hi));
+    }
     // slot order of a lane's eight columns: [0, 2, 1, 3, 4, 6, 5, 7]
     const float o[4] = {x[0], x[2], x[1], x[3]};
     half4_t h, l;
@@ -663,7 +675,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_wide_kernel(shv_gemv_q4k_args a,
 template <int NW, int R>
 __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a, const char *staged_all, int groups) {
     extern __shared__ __align__(16) char smem[];
-    size_t *yoffs = reinterpret_cast<size_t *>(smem + 2 * kWideSlab);
+    char *sumf = smem + 2 * kWideSlab;   // the sums of the quarter of the columns in hand, as operands
+    size_t *yoffs = reinterpret_cast<size_t *>(sumf + kWideSumFrags);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int sbs = a.k / SHV_Q4K_BLOCK;
@@ -695,17 +708,35 @@ __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a,
     }
     load_q(0, q);
     if (tid < nt) yoffs[tid] = out_offset(a, t0 + tid);
-    constexpr int kVec = kWideSlab / 16;
-    constexpr int kPer = kWideSlabA / 16 / NTHR;
-    static_assert(kPer * NTHR * 16 == kWideSlabA && kVec - kPer * NTHR == 64, "slab copy layout");
-    {
-        const uint4 *src = reinterpret_cast<const uint4 *>(staged);
-        uint4 *dst = reinterpret_cast<uint4 *>(smem);
-        for (int i = tid; i < kVec; i += NTHR) dst[i] = src[i];
-    }
+    // A slab is 33 pieces of 1 KB that lie in `staged` as they will in LDS: the loads place them
+    // there themselves (lane l's 16 bytes at 16 l of the piece), through no register.
+    constexpr int kPieces = kWideSlab / 1024;
+    static_assert(kPieces * 1024 == kWideSlab, "whole pieces");
+    auto ask_slab = [&](int s, char *buf) {
+        const char *src = staged + static_cast<size_t>(s) * kWideSlab + lane * 16;
+        for (int c = wave; c < kPieces; c += NW)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + c * 1024), (__attribute__((address_space(3))) void *)(buf + c * 1024), 16, 0, 0);
+    };
+    // the min term of columns [1024 qt, 1024 qt + 1024): the tokens' sums (wave w asks for fragment w of eight) and this lane's
+    // rows' headers of super-block 4 qt + kb, both a step ahead of their use
+    static_assert(NW == 8, "a fragment of sums a wave");
+    uint4 hq[R];
+    auto ask_quarter = [&](int qt) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(staged + wide_sums_offset(a.k) + static_cast<size_t>(qt * 8 + wave) * kWideFrag + lane * 16),
+                                         (__attribute__((address_space(3))) void *)(sumf + wave * kWideFrag), 16, 0, 0);
+        const int sb = 4 * qt + kb < sbs ? 4 * qt + kb : 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) hq[r] = *reinterpret_cast<const uint4 *>(rp[r] + static_cast<size_t>(sb) * SHV_Q4K_BYTES);
+    };
+    ask_slab(0, smem);
+    ask_quarter(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 
     const NibbleConsts nc = nibble_consts();
+    uint32_t m0 = 0x000F000Fu, o0 = 0x64006400u;   // bits 0..3 of both halves under the exponent of 1024
+    asm volatile("" : "+s"(m0));
+    asm volatile("" : "+v"(o0));
     float4_t y[R][4], acc[R][4];
 #pragma unroll
     for (int r = 0; r < R; r++)
@@ -715,13 +746,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a,
     for (int s = 0; s < steps; s++) {
         const int cur = s & 1;
         const bool more = s + 1 < steps;
-        uint4 an[kPer], asx;
         {
             const int sn = more ? s + 1 : s;
-            const uint4 *src = reinterpret_cast<const uint4 *>(staged + static_cast<size_t>(sn) * kWideSlab);
-#pragma unroll
-            for (int i = 0; i < kPer; i++) an[i] = src[tid + i * NTHR];
-            asx = src[kPer * NTHR + (tid & 63)];
+            if (more) ask_slab(sn, smem + (cur ^ 1) * kWideSlab);   // the other buffer was read to its end before the barrier that ended the last step
+            if (more && (sn & 7) == 0) {
+                // the sums in LDS were read at this quarter's first step, steps ago; every wave is past that
+                ask_quarter(sn >> 3);
+            }
             load_q(sn, qn);
             if (s & 1) {
 #pragma unroll
@@ -729,51 +760,84 @@ __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a,
             }
         }
         const char *A = smem + cur * kWideSlab;
-        const float *sxs = reinterpret_cast<const float *>(A + kWideSlabA);
-#pragma unroll
-        for (int g = 0; g < 2; g++) {
-            uint32_t sc[R], mn[R];
-            float dmin[R];
+        if ((s & 7) == 0) {
+            // y -= sum over the quarter's sub-blocks of dmin * m * sum(x), as three matrix products a token tile:
+            // -dmin * m has 17 significant bits and goes as two halves, the sums come as two halves too
+            // (the small halves' product is below float32's last bit)
+            const bool on = 4 * (s >> 3) + kb < sbs;
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                q4k_group_scale_min(hdr[r], (s & 1) * 2 + g, sc[r], mn[r]);
-                dmin[r] = f16_bits_to_f32(hdr[r].x >> 16);
+                const float nd = on ? -f16_bits_to_f32(hq[r].x >> 16) : 0.f;
+                const uint32_t m03 = hq[r].z & 0x3F3F3F3Fu, m47 = ((hq[r].w >> 4) & 0x0F0F0F0Fu) | ((hq[r].z >> 2) & 0x30303030u);
+                half8_t bh, bl;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float p = nd * static_cast<float>(((j < 4 ? m03 : m47) >> (8 * (j & 3))) & 0xFFu);
+                    const _Float16 hi = static_cast<_Float16>(p);
+                    bh[j] = hi;
+                    bl[j] = static_cast<_Float16>(p - static_cast<float>(hi));
+                }
+#pragma unroll
+                for (int tt = 0; tt < 4; tt++) {
+                    half8_t sh = *reinterpret_cast<const half8_t *>(sumf + (tt * 2) * kWideFrag + lane * 16);
+                    half8_t sl = *reinterpret_cast<const half8_t *>(sumf + (tt * 2 + 1) * kWideFrag + lane * 16);
+                    if (!on) sh = sl = static_cast<half8_t>(static_cast<_Float16>(0.f));   // a super-block past the row: nothing was staged there
+                    y[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sh, bh, y[r][tt], 0, 0, 0);
+                    y[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sl, bh, y[r][tt], 0, 0, 0);
+                    y[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sh, bl, y[r][tt], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            uint32_t sc[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                uint32_t mn;
+                q4k_group_scale_min(hdr[r], (s & 1) * 2 + g, sc[r], mn);
             }
 #pragma unroll
             for (int hi = 0; hi < 2; hi++) {
                 const int sub = g * 2 + hi;
                 half8_t b[R];
-                float dm[R];
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     const uint32_t q0 = q[r][g].x, q1 = q[r][g].y;
-                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                    u32x4 v;
+                    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                    // A nibble in the low bits of a half's mantissa reads, under the right exponent, as
+                    // C + n: bits 0..3 under 1024's, bits 4..7 under 64's (the odd bytes' nibbles take
+                    // one shift down there).  One fused multiply-add then makes (C + n) * sc - C * sc =
+                    // n * sc: a whole number up to 15 * 63, exact in binary16, as are C * sc.
                     // slot order of the eight columns: bytes [0, 2, 1, 3, 4, 6, 5, 7]
+                    const _Float16 s1 = static_cast<_Float16>(static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu));
+                    const half2_t s2 = {s1, s1};
+                    half2_t w[4], c[4];
                     if (hi == 0) {
-                        v.x = ((q0 << 4) & nc.mask) | nc.one; v.y = ((q0 >> 4) & nc.mask) | nc.one;
-                        v.z = ((q1 << 4) & nc.mask) | nc.one; v.w = ((q1 >> 4) & nc.mask) | nc.one;
+                        w[0] = __builtin_bit_cast(half2_t, (q0 & m0) | o0); w[1] = __builtin_bit_cast(half2_t, ((q0 >> 4) & nc.mask) | nc.one);
+                        w[2] = __builtin_bit_cast(half2_t, (q1 & m0) | o0); w[3] = __builtin_bit_cast(half2_t, ((q1 >> 4) & nc.mask) | nc.one);
+                        c[0] = c[2] = s2 * static_cast<half2_t>(static_cast<_Float16>(-1024.f));
+                        c[1] = c[3] = s2 * static_cast<half2_t>(static_cast<_Float16>(-64.f));
                     } else {
-                        v.x = (q0 & nc.mask) | nc.one; v.y = ((q0 >> 8) & nc.mask) | nc.one;
-                        v.z = (q1 & nc.mask) | nc.one; v.w = ((q1 >> 8) & nc.mask) | nc.one;
+                        w[0] = __builtin_bit_cast(half2_t, (q0 & nc.mask) | nc.one); w[1] = __builtin_bit_cast(half2_t, ((q0 >> 8) & nc.mask) | nc.one);
+                        w[2] = __builtin_bit_cast(half2_t, (q1 & nc.mask) | nc.one); w[3] = __builtin_bit_cast(half2_t, ((q1 >> 8) & nc.mask) | nc.one);
+                        c[0] = c[1] = c[2] = c[3] = s2 * static_cast<half2_t>(static_cast<_Float16>(-64.f));
                     }
-                    const _Float16 s16 = static_cast<_Float16>(static_cast<float>(hi ? sc[r] >> 8 : sc[r] & 0xFFu));
-                    b[r] = (__builtin_bit_cast(half8_t, v) - static_cast<half8_t>(static_cast<_Float16>(64.f))) * static_cast<half8_t>(s16);
-                    dm[r] = dmin[r] * static_cast<float>(hi ? mn[r] >> 8 : mn[r] & 0xFFu);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const half2_t p = __builtin_elementwise_fma(w[i], s2, c[i]);
+                        b[r][2 * i] = p[0];
+                        b[r][2 * i + 1] = p[1];
+                    }
                 }
 #pragma unroll
                 for (int tt = 0; tt < 4; tt++) {
                     const char *f = A + static_cast<size_t>((sub * 4 + tt) * 2) * kWideFrag + lane * 16;
                     const half8_t xh = *reinterpret_cast<const half8_t *>(f);
                     const half8_t xl = *reinterpret_cast<const half8_t *>(f + kWideFrag);
-                    const float4 sx = *reinterpret_cast<const float4 *>(sxs + sub * kWideTok + tt * kTileRows + 4 * kb);
-                    const float sxv[4] = {sx.x, sx.y, sx.z, sx.w};
 #pragma unroll
                     for (int r = 0; r < R; r++) {
                         acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b[r], acc[r][tt], 0, 0, 0);
                         acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc[r][tt], 0, 0, 0);
-#pragma unroll
-                        for (int j = 0; j < 4; j++) y[r][tt][j] = fmaf(-dm[r], sxv[j], y[r][tt][j]);
                     }
                 }
             }
@@ -792,17 +856,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a,
                 hdr[r] = hdrn[r];
             }
         }
-        {
-            // (the last step copies its own slab again: no branch around the stores)
-            uint4 *dst = reinterpret_cast<uint4 *>(smem + (cur ^ 1) * kWideSlab);
 #pragma unroll
-            for (int i = 0; i < kPer; i++) dst[tid + i * NTHR] = an[i];
-            if (tid < 64) dst[kPer * NTHR + tid] = asx;
+        for (int r = 0; r < R; r++)
 #pragma unroll
-            for (int r = 0; r < R; r++)
-#pragma unroll
-                for (int g = 0; g < 2; g++) q[r][g] = qn[r][g];
-        }
+            for (int g = 0; g < 2; g++) q[r][g] = qn[r][g];
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the next slab have landed, then everybody's
         __syncthreads();
     }
 
@@ -1038,7 +1096,7 @@ template <int NW, int R>
 int launch_wide_all(shv_ctx *ctx, const shv_gemv_q4k_args &a, int groups) {
     constexpr int kRows = NW * R * kTileRows;
     const int bx = (a.n + kRows - 1) / kRows;
-    const size_t lds = 2 * kWideSlab + kWideTok * sizeof(size_t);
+    const size_t lds = 2 * kWideSlab + kWideSumFrags + kWideTok * sizeof(size_t);
     static bool raised = false;
     if (!raised) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_pass_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
