@@ -719,11 +719,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a,
     };
     // the min term of columns [1024 qt, 1024 qt + 1024): the tokens' sums (wave w asks for fragment w of eight) and this lane's
     // rows' headers of super-block 4 qt + kb, both a step ahead of their use
-    static_assert(NW == 8, "a fragment of sums a wave");
+    static_assert(NW >= 8, "a fragment of sums a wave");
     uint4 hq[R];
     auto ask_quarter = [&](int qt) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(staged + wide_sums_offset(a.k) + static_cast<size_t>(qt * 8 + wave) * kWideFrag + lane * 16),
-                                         (__attribute__((address_space(3))) void *)(sumf + wave * kWideFrag), 16, 0, 0);
+        if (wave < 8)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(staged + wide_sums_offset(a.k) + static_cast<size_t>(qt * 8 + wave) * kWideFrag + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(sumf + wave * kWideFrag), 16, 0, 0);
         const int sb = 4 * qt + kb < sbs ? 4 * qt + kb : 0;
 #pragma unroll
         for (int r = 0; r < R; r++) hq[r] = *reinterpret_cast<const uint4 *>(rp[r] + static_cast<size_t>(sb) * SHV_Q4K_BYTES);
