@@ -444,11 +444,11 @@ __device__ __forceinline__ size_t out_offset(const shv_gemv_q4k_args &a, int t) 
 }
 
 // The same for a pass of up to 64 rows a group, in the slab order gemm_wide_kernel streams.
-// grid: (k/256, 16 quartets of rows, groups of 64 rows), 256 threads: a wave takes one row's 64
-// quads of one super-block's columns; rows a group does not have are written as zeros.
+// grid: (parts of the k/256 column blocks, 16 quartets of rows, groups of 64 rows), 256 threads: a wave takes one row's 64
+// quads of one super-block's columns at a time; rows a group does not have are written as zeros.
 __global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args a, char *staged, float *x_out) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int K = a.k, kp = blockIdx.x, grp = blockIdx.z;
+    const int K = a.k, grp = blockIdx.z;
     const int t0 = grp * kWideTok;
     const int nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;
     const int tl = blockIdx.y * 4 + wave;
@@ -465,38 +465,51 @@ __global__ __launch_bounds__(256) void gemm_wide_stage_kernel(shv_gemv_q4k_args 
         ss = wave_sum_all(ss);
         scale = 1.f / sqrtf(ss / static_cast<float>(K) + a.eps);
     }
-    const int c = kp * 256 + 4 * lane;
-    // the quad's place: slab of 128 columns, sub-block of it, k block of 8 columns, which half of those
-    char *slab = region + static_cast<size_t>(c >> 7) * kWideSlab;
-    const int sub = (c & 127) >> 5, kb = (c & 31) >> 3, qh = (c & 7) >> 2;
-    float x[4] = {0.f, 0.f, 0.f, 0.f};
-    if (tl < nt) pro_quad(a, t0 + tl, c, scale, x);
-    // the transformed row itself, for a caller that also needs it as plain float32 (the router's xn)
-    if (x_out && tl < nt) *reinterpret_cast<float4 *>(x_out + static_cast<size_t>(t0 + tl) * K + c) = float4{x[0], x[1], x[2], x[3]};
-    float sum = (x[0] + x[1]) + (x[2] + x[3]);
-    sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
-    sum += __shfl_xor(sum, 4, 64);
-    if ((c & 31) == 0) {
-        reinterpret_cast<float *>(slab + kWideSlabA)[sub * kWideTok + tl] = sum;
-        const _Float16 hi = static_cast<_Float16>(sum);
-        _Float16 *sp = reinterpret_cast<_Float16 *>(region + wide_sums_offset(K) + static_cast<size_t>(((c >> 10) * 4 + (tl >> 4)) * 2) * kWideFrag +
-                                                    (((c >> 8) & 3) * 16 + (tl & 15)) * 16) + ((c >> 5) & 7);
-        sp[0] = hi;
-        sp[kWideFrag / 2] = static_cast<_Float16>(sum - static_cast<float>(hi));
-    }
-    // slot order of a lane's eight columns: [0, 2, 1, 3, 4, 6, 5, 7]
-    const float o[4] = {x[0], x[2], x[1], x[3]};
-    half4_t h, l;
+    // the block's waves take their rows' column blocks of 256 in turn, blockIdx.x first: a row's factor is formed once for all of them
+    for (int kp = blockIdx.x; kp < K / 256; kp += gridDim.x) {
+        const int c = kp * 256 + 4 * lane;
+        // the quad's place: slab of 128 columns, sub-block of it, k block of 8 columns, which half of those
+        char *slab = region + static_cast<size_t>(c >> 7) * kWideSlab;
+        const int sub = (c & 127) >> 5, kb = (c & 31) >> 3, qh = (c & 7) >> 2;
+        float x[4] = {0.f, 0.f, 0.f, 0.f};
+        if (tl < nt) pro_quad(a, t0 + tl, c, scale, x);
+        // the transformed row itself, for a caller that also needs it as plain float32 (the router's xn)
+        if (x_out && tl < nt) *reinterpret_cast<float4 *>(x_out + static_cast<size_t>(t0 + tl) * K + c) = float4{x[0], x[1], x[2], x[3]};
+        float sum = (x[0] + x[1]) + (x[2] + x[3]);
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        sum += __shfl_xor(sum, 4, 64);
+        if ((c & 31) == 0) {
+            reinterpret_cast<float *>(slab + kWideSlabA)[sub * kWideTok + tl] = sum;
+            const _Float16 hi = static_cast<_Float16>(sum);
+            _Float16 *sp = reinterpret_cast<_Float16 *>(region + wide_sums_offset(K) + static_cast<size_t>(((c >> 10) * 4 + (tl >> 4)) * 2) * kWideFrag +
+                                                        (((c >> 8) & 3) * 16 + (tl & 15)) * 16) + ((c >> 5) & 7);
+            sp[0] = hi;
+            sp[kWideFrag / 2] = static_cast<_Float16>(sum - static_cast<float>(hi));
+        }
+        // slot order of a lane's eight columns: [0, 2, 1, 3, 4, 6, 5, 7]
+        const float o[4] = {x[0], x[2], x[1], x[3]};
+        half4_t h, l;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const _Float16 hi = static_cast<_Float16>(o[j]);
-        h[j] = hi;
-        l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+        for (int j = 0; j < 4; j++) {
+            const _Float16 hi = static_cast<_Float16>(o[j]);
+            h[j] = hi;
+            l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+        }
+        char *e = slab + static_cast<size_t>((sub * 4 + (tl >> 4)) * 2) * kWideFrag + (kb * 16 + (tl & 15)) * 16 + qh * 8;
+        *reinterpret_cast<half4_t *>(e) = h;
+        *reinterpret_cast<half4_t *>(e + kWideFrag) = l;
     }
-    char *e = slab + static_cast<size_t>((sub * 4 + (tl >> 4)) * 2) * kWideFrag + (kb * 16 + (tl & 15)) * 16 + qh * 8;
-    *reinterpret_cast<half4_t *>(e) = h;
-    *reinterpret_cast<half4_t *>(e + kWideFrag) = l;
+}
+
+// How many blocks share a row's column blocks: under the RMSNorm prologue every one of them reads the whole row for
+// its factor, so as few as still fill the chip.
+static inline int stage_parts(const shv_gemv_q4k_args &a, int groups) {
+    const int all = a.k / 256;
+    if (a.prologue != SHV_PRO_RMSNORM) return all;
+    int parts = 1;
+    while (parts < all && parts * (kWideTok / 4) * groups < 1024) parts *= 2;
+    return parts;
 }
 
 struct WideLoads {
@@ -1130,7 +1143,7 @@ int shv_launch_router_wide(shv_ctx *ctx, const shv_moe_router_args &a) {
     g.eps = a.eps;
     g.x_stride = a.h_stride;
     const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
-    SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(g.k / 256, kWideTok / 4, groups), dim3(256), 0, g, ctx->gemm_stage, a.xn);
+    SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(stage_parts(g, groups), kWideTok / 4, groups), dim3(256), 0, g, ctx->gemm_stage, a.xn);
     constexpr int NW = 4;
     const int n_rows = a.n_expert + (a.shared_gate ? 1 : 0);
     const int bx = (n_rows + NW * kTileRows - 1) / (NW * kTileRows);
@@ -1171,7 +1184,7 @@ int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     if (a.n_tok > cap && ctx->gemm_stage && (a.prologue != SHV_PRO_GATED_NORM || 256 % a.head_dim == 0)) {
         const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
         SHV_REQUIRE(groups * wide_region(a.k) <= static_cast<size_t>(shv_ctx::kGemmStageBytes), "gemm_q4k: %d rows of %d columns do not fit the staging buffer", a.n_tok, a.k);
-        SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(a.k / 256, kWideTok / 4, groups), dim3(256), 0, a, ctx->gemm_stage, static_cast<float *>(nullptr));
+        SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(stage_parts(a, groups), kWideTok / 4, groups), dim3(256), 0, a, ctx->gemm_stage, static_cast<float *>(nullptr));
         if (groups >= 4) return launch_wide_all<8, 1>(ctx, a, groups);
         for (int g = 0; g < groups; g++) {
             const int t0 = g * kWideTok;
