@@ -575,7 +575,7 @@ __device__ __forceinline__ void tile_barrier() {
 }
 
 // grid: (n_seq * ceil(n_groups / 8), n_head_kv, n_splits); the cells of the pass are in the cache already.
-__global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decode_args a, int n_groups, int slice_cells) {
+__global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decode_args a, int n_groups, int slice_cells, int direct) {
     extern __shared__ __align__(16) char praw[];
     PrefillSmem &sm = *reinterpret_cast<PrefillSmem *>(praw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -816,6 +816,21 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
     // the loads asked for past the last tile still write LDS: none may be out when the wave ends and its LDS goes to another workgroup
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (!me.mine) return;
+    if (direct) {
+        // one slice a pair: what the merge would make of its single record, sums / sum, goes straight out
+        float lr[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * q + i, 64);   // query row 4 q + i keeps its sum in lane 4 q + i
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = 4 * q + i;  // query row: sequence row r / 8, head r % 8
+            if ((r >> 3) >= me.valid) continue;
+            float *dst = a.out + (static_cast<size_t>(seq * a.seq_len + row0 + (r >> 3)) * a.n_head + kvh * kRep + (r & 7)) * kD;
+#pragma unroll
+            for (int db = 0; db < 16; db++) dst[16 * db + n] = o[db][i] / lr[i];
+        }
+        return;
+    }
     // the wave's record of this slice: per row and head the unnormalised sums, then (max, sum)
     float *rec = a.partial + ((static_cast<size_t>(gz) * a.n_head_kv + kvh) * a.n_splits + split) * 2 * kRec;
 #pragma unroll
@@ -849,7 +864,10 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
             SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
             raised = true;
         }
-        SHV_LAUNCH(ctx, attn_prefill_kernel, dim3(a.n_seq * ((n_groups + kPfWaves - 1) / kPfWaves), a.n_head_kv, b.n_splits), dim3(kPfThreads), sizeof(PrefillSmem), b, n_groups, slice_cells);
+        // with one slice a pair there is nothing to merge: the kernel writes the rows themselves
+        const int direct = b.n_splits == 1 ? 1 : 0;
+        SHV_LAUNCH(ctx, attn_prefill_kernel, dim3(a.n_seq * ((n_groups + kPfWaves - 1) / kPfWaves), a.n_head_kv, b.n_splits), dim3(kPfThreads), sizeof(PrefillSmem), b, n_groups, slice_cells, direct);
+        if (direct) return SHV_OK;
     } else {
         dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
         SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);

@@ -49,9 +49,18 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
     const int tid = threadIdx.x, n_pairs = n_tok * n_used;
     for (int e = tid; e <= n_expert; e += blockDim.x) s_cnt[e] = 0;
     __syncthreads();
-    for (int i = tid; i < n_pairs; i += blockDim.x) {
-        const int e = topk[i];
-        if (e >= 0 && e < n_expert) atomicAdd(&s_cnt[e], 1);
+    // eight of a thread's selections are asked for before the first is counted: the passes over topk cost its latency once a batch, not once a pair
+    constexpr int NB = 8;
+    for (int i0 = tid; i0 < n_pairs; i0 += NB * blockDim.x) {
+        int e[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const int i = i0 + b * blockDim.x;
+            e[b] = i < n_pairs ? topk[i] : -1;
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+            if (e[b] >= 0 && e[b] < n_expert) atomicAdd(&s_cnt[e[b]], 1);
     }
     __syncthreads();
     {
@@ -87,9 +96,18 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
     }
     __syncthreads();
     int32_t *list = group + n_expert + 1;
-    for (int i = tid; i < n_pairs; i += blockDim.x) {
-        const int e = topk[i];
-        if (e >= 0 && e < n_expert) list[atomicAdd(&s_cnt[e], 1)] = (i / n_used) * (n_used + 1) + i % n_used;
+    for (int i0 = tid; i0 < n_pairs; i0 += NB * blockDim.x) {
+        int e[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const int i = i0 + b * blockDim.x;
+            e[b] = i < n_pairs ? topk[i] : -1;
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const int i = i0 + b * blockDim.x;
+            if (e[b] >= 0 && e[b] < n_expert) list[atomicAdd(&s_cnt[e[b]], 1)] = (i / n_used) * (n_used + 1) + i % n_used;
+        }
     }
 }
 
