@@ -190,8 +190,9 @@ type MoEBanks struct {
 // MoEUp is llm_moe_gemv.comp MODE 0 + llm_moe_act.comp: act[t][s] = silu(Wg x) * (Wu x) for the
 // token's experts and the shared one.  logits/weights non-nil: every block routes its token first.
 // group non-nil (2*nExpert + 1 + rows*nUsed ints): a pass of 128 rows and more goes grouped by
-// expert on the matrix cores.
-func MoEUp(xn, topk *Buffer, b MoEBanks, act *Buffer, rows, nEmbd, nUsed, ffn, nExpert int, logits, weights, group *Buffer) Op {
+// expert on the matrix cores.  packed: such a pass leaves act as the operands the grouped MoEDown
+// reads instead of floats (MoEDown must follow at once, with groupReady and packed too).
+func MoEUp(xn, topk *Buffer, b MoEBanks, act *Buffer, rows, nEmbd, nUsed, ffn, nExpert int, logits, weights, group *Buffer, packed bool) Op {
 	var a C.shv_moe_up_args
 	a.xn, a.topk = fp(xn), ip(topk)
 	a.gate_exps, a.up_exps, a.gate_sh, a.up_sh = vp(b.GateExps), vp(b.UpExps), vp(b.GateSh), vp(b.UpSh)
@@ -199,11 +200,14 @@ func MoEUp(xn, topk *Buffer, b MoEBanks, act *Buffer, rows, nEmbd, nUsed, ffn, n
 	a.n_tok, a.n_embd, a.n_used, a.ffn, a.n_expert = C.int32_t(rows), C.int32_t(nEmbd), C.int32_t(nUsed), C.int32_t(ffn), C.int32_t(nExpert)
 	a.logits, a.weights, a.group = fp(logits), fp(weights), ip(group)
 	a.gate_type, a.up_type, a.gate_sh_type, a.up_sh_type = C.int32_t(b.Types[0]), C.int32_t(b.Types[1]), C.int32_t(b.Types[3]), C.int32_t(b.Types[4])
+	if packed {
+		a.act_packed = 1
+	}
 	return mk(C.SHV_OP_MOE_UP, unsafe.Pointer(&a), C.sizeof_shv_moe_up_args)
 }
 
 // MoEDown is llm_moe_gemv.comp MODE 1 + llm_moe_combine.comp (+ the residual add).
-func MoEDown(act, topk, weights *Buffer, b MoEBanks, residual, out *Buffer, rows, nEmbd, nUsed, ffn, nExpert int, group, pairs *Buffer, groupReady bool) Op {
+func MoEDown(act, topk, weights *Buffer, b MoEBanks, residual, out *Buffer, rows, nEmbd, nUsed, ffn, nExpert int, group, pairs *Buffer, groupReady, packed bool) Op {
 	var a C.shv_moe_down_args
 	a.act, a.topk, a.weights = fp(act), ip(topk), fp(weights)
 	a.down_exps, a.down_sh = vp(b.DownExps), vp(b.DownSh)
@@ -214,6 +218,9 @@ func MoEDown(act, topk, weights *Buffer, b MoEBanks, residual, out *Buffer, rows
 	a.group, a.pairs = ip(group), fp(pairs)
 	if groupReady {
 		a.group_ready = 1
+	}
+	if packed {
+		a.act_packed = 1
 	}
 	return mk(C.SHV_OP_MOE_DOWN, unsafe.Pointer(&a), C.sizeof_shv_moe_down_args)
 }

@@ -49,12 +49,14 @@ func (g *moeHIP) graph(layer int, in, out *hip.Buffer) ([]hip.Op, []string, erro
 	} else {
 		grp = g.group
 	}
+	ready := !fused && q4k && g.group != nil
+	packed := ready && g.pairs != nil // both projections Q4_K, one right after the other: act goes over as operands
 	ops := []hip.Op{
 		hip.MoERouter(in, g.norm[layer], g.router[layer], g.sharedGate[layer], g.xn, g.logits, g.topk, g.weights,
 			g.rows, c.NEmbd, c.NExpert, c.NExpertUsed, c.RMSEps, fused),
-		hip.MoEUp(g.xn, g.topk, g.banks[layer], g.act, g.rows, c.NEmbd, c.NExpertUsed, c.FFNExpert, c.NExpert, lg, wt, grp),
+		hip.MoEUp(g.xn, g.topk, g.banks[layer], g.act, g.rows, c.NEmbd, c.NExpertUsed, c.FFNExpert, c.NExpert, lg, wt, grp, packed),
 		hip.MoEDown(g.act, g.topk, g.weights, g.banks[layer], in, out, g.rows, c.NEmbd, c.NExpertUsed, c.FFNExpert, c.NExpert,
-			g.group, g.pairs, !fused && q4k && g.group != nil),
+			g.group, g.pairs, ready, packed),
 	}
 	return ops, []string{"moe.router", "moe.up", "moe.down"}, nil
 }
