@@ -75,6 +75,49 @@ def test_rows_match_oracle_and_float64(ctx, row_ctx, n, k, rows):
     print(f"gemm {n}x{k} x{rows}: worst rel-L2 vs float64 {worst:.2e}")
 
 
+@pytest.mark.parametrize("n,k,rows", [(1000, 256, 256), (513, 512, 300), (2048, 1024, 193), (12352, 2048, 257),
+                                      (2048, 4096, 320), (2048, 2048, 2048)])
+def test_long_pass_matches_float64_and_oracle(ctx, n, k, rows):
+    """A pass of four groups of 64 rows and more goes to the kernel that walks every group in one
+    launch and takes Q4_K's min term on the matrix cores as well; here whole and ragged groups, every
+    width of a super-block count that kernel has a case for, and columns not a multiple of 128.  Every
+    row is held to a float64 product; the oracle's GEMV (llm/hc.go:255-264) takes a sample of rows, the
+    first and last of each group among them."""
+    rng = np.random.default_rng(n + k + rows)
+    wq = _weights(rng, n, k)
+    x = (rng.standard_normal((rows, k)) * rng.uniform(0.01, 30.0, size=(rows, 1))).astype(np.float32)
+    w64 = O.dequant_q4k(wq, k).astype(np.float64)
+    dy = ctx.alloc(rows * n * 4)
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(x), dy, n, k, n_tok=rows)
+    got = dy.read(np.float32, rows * n).reshape(rows, n)
+    want = x.astype(np.float64) @ w64.T
+    err = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert err.max() <= TOL64, (int(err.argmax()), float(err.max()))
+    sample = sorted({t for g in range(0, rows, 64) for t in (g, min(g + 63, rows - 1))} | {rows // 2})[:24]
+    for t in sample:
+        assert O.rel_l2(got[t], O.gemv_q4k(wq, x[t], n, k, threads=8)) <= TOL, t
+    print(f"gemm {n}x{k} x{rows}: worst rel-L2 vs float64 {err.max():.2e}")
+
+
+@pytest.mark.parametrize("rows", [256, 333])
+def test_long_pass_rmsnorm_prologue_residual_in_place(ctx, rows):
+    """The long pass with the norm folded in and the residual stream updated in place (the MoE block's
+    shared expert and the output projections of a prompt chunk run this way)."""
+    rng = np.random.default_rng(310 + rows)
+    n, k, eps = 2048, 2048, 1e-6
+    wq = _weights(rng, n, k)
+    h = (rng.standard_normal((rows, k)) * 3).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    res = rng.standard_normal((rows, n)).astype(np.float32)
+    dy = ctx.upload(res)
+    ctx.gemv_q4k(ctx.upload(wq), ctx.upload(h), dy, n, k, n_tok=rows, prologue=A.PRO_RMSNORM,
+                 gamma=ctx.upload(gamma), residual=dy, eps=eps)
+    got = dy.read(np.float32, rows * n).reshape(rows, n)
+    for t in list(range(0, rows, 17)) + [rows - 1]:
+        want = O.gemv_q4k(wq, O.rmsnorm(h[t], gamma, eps), n, k, threads=8) + res[t]
+        assert O.rel_l2(got[t], want) <= TOL, t
+
+
 @pytest.mark.parametrize("rows", [3, 64])
 def test_rmsnorm_prologue_residual_in_place(ctx, rows):
     """The residual stream's own rows are the residual and the destination (dn.out, attn.out, the
@@ -94,7 +137,7 @@ def test_rmsnorm_prologue_residual_in_place(ctx, rows):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-@pytest.mark.parametrize("rows,slots", [(4, 8), (37, 64)])
+@pytest.mark.parametrize("rows,slots", [(4, 8), (37, 64), (260, 512)])
 def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx, rows, slots):
     """DeltaNet's output projection at its real shape: 4096 columns (two column ranges), per-head
     norm, the gate z read from the projection ring at each row's position, residual in place."""
@@ -114,7 +157,7 @@ def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx, rows, slots):
                  pos=ctx.upload(np.array([pos], np.int32)), slot=ctx.upload(np.array([slot], np.int32)),
                  seq_len=rows, ring_slots=slots, ring_stride=ring_stride, z_ring=1)
     got = dy.read(np.float32, rows * n).reshape(rows, n)
-    for t in range(rows):
+    for t in (range(rows) if rows <= 64 else list(range(0, rows, 13)) + [rows - 1]):
         z = ring[slot, (pos + t) % slots, z_col:z_col + k]
         xn = O.rmsnorm(o[t].reshape(-1, d), gamma, eps).ravel()
         sig = np.array([L.shv_ref_sigmoid(float(v)) for v in z], dtype=np.float32)
