@@ -598,7 +598,7 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
     const int slot = a.slot ? a.slot[seq] : seq;
     const int pos_first = a.pos ? a.pos[seq] : 0;
     // pair gg of the sequence: its rows, what it sees, its slice of that
-    struct Slice { int c0, c1, p_first, valid; bool mine; };
+    struct Slice { int c0, c1, p_first, valid; bool mine, empty; };
     auto slice_of = [&](int gg) {
         Slice s;
         const bool live = gg < n_groups;
@@ -614,9 +614,17 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
         s.c0 = split * cps;
         s.c1 = s.c0 + cps < n_cells ? s.c0 + cps : n_cells;
         s.mine = live && split < n_active && s.c1 > s.c0;
+        // slices start on a tile of V: rounded up, the last of a pair's slices can start past its cells
+        s.empty = live && split < n_active && s.c1 <= s.c0;
         return s;
     };
     const Slice me = slice_of(g0 + wave);
+    if (me.empty && lane < 2 * kRep) {
+        // the merge reads every slice the pair counts as taking part: this one says it holds nothing
+        const int gz = seq * n_groups + g0 + wave;
+        float *rec = a.partial + ((static_cast<size_t>(gz) * a.n_head_kv + kvh) * a.n_splits + split) * 2 * kRec;
+        *reinterpret_cast<float2 *>(rec + (lane >> 3) * kRec + (lane & 7) * (kD + 2) + kD) = make_float2(-INFINITY, 0.f);
+    }
     int lo = 0x7fffffff, hi = 0;
 #pragma unroll
     for (int w = 0; w < kPfWaves; w++) {

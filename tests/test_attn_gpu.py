@@ -155,6 +155,34 @@ def test_rows_of_one_sequence_in_one_call(ctx, past, rows, n_splits):
     assert (np.abs(g - w) <= np.abs(w) * 2.0 ** -10 + 1e-5).all()
 
 
+@pytest.mark.parametrize("past,rows,n_splits", [(1030, 64, 64), (1500, 48, 64), (2100, 32, 16), (4200, 16, 64), (700, 40, 6)])
+def test_prompt_chunk_with_a_slice_left_empty(ctx, past, rows, n_splits):
+    """A prompt chunk of 15 rows and more over a cache that holds more cells than its slices were
+    cut for: slices start on whole tiles of V, so the last of a row pair's slices can start past the
+    pair's cells and hold nothing.  The merge must take such a slice for empty whatever its record
+    held before (here noise: the records of an earlier layer's pass in real use)."""
+    case = AttnCase(ctx, seed=50 + past)
+    max_cells = ((past + rows + 63) // 64) * 64
+    case.upload(max_cells)
+    rng = case.rng
+    kc = np.zeros((max_cells, NKV, D), np.uint16)
+    vc = np.zeros_like(kc)
+    kc[:past] = rng.standard_normal((past, NKV, D)).astype(np.float16).view(np.uint16)
+    vc[:past] = rng.standard_normal((past, NKV, D)).astype(np.float16).view(np.uint16)
+    xn = rng.standard_normal((rows, H)).astype(np.float32)
+    c = ctx
+    d_kc, d_vc = c.upload(kc), c.upload(v_dev(vc))
+    want_out, want_pre = case.oracle(xn, past, kc, vc)
+    d_qkv, d_ctx, d_out = c.alloc(rows * case.width * 4), c.alloc(rows * NH * D * 4), c.alloc(rows * H * 4)
+    d_part = c.upload((rng.standard_normal(_part_floats(1, n_splits, rows)) * 8).astype(np.float32))
+    c.dispatch_multi(case.ops(c.upload(xn), d_qkv, d_kc, d_vc, d_part, d_ctx, d_out,
+                              c.upload(np.array([past], np.int32)), 1, rows, max_cells, n_splits))
+    got_pre = d_ctx.read(np.float32, rows * NH * D).reshape(rows, -1)
+    got_out = d_out.read(np.float32, rows * H).reshape(rows, -1)
+    for t in range(rows):
+        assert O.rel_l2(got_pre[t], want_pre[t]) <= TOL and O.rel_l2(got_out[t], want_out[t]) <= TOL, t
+
+
 @pytest.mark.parametrize("past,n_seq,n_splits", [(4096, 1, 16), (4096, 3, 16), (32768, 1, 64),
                                                  (32768, 3, 64), (131071, 1, 256), (131071, 3, 128),
                                                  (1000, 1, 7), (5, 1, 64)])

@@ -486,3 +486,28 @@ def test_chunk_size_does_not_matter_over_4096_tokens():
         assert O.rel_l2(f16(ka), f16(kb)) <= 1e-3 and np.mean(ka != kb) <= 0.1
     print("64 vs 16 rows a chunk over 4096 tokens: hidden %.2e logits %.2e state %.2e" %
           (O.rel_l2(a[1], b[1]), O.rel_l2(a[0], b[0]), O.rel_l2(a[2], b[2])))
+
+
+def test_chunk_size_does_not_matter_to_a_second_attention_layer():
+    """What a chunk's rows leave an attention layer with is only seen by the layers after it: two
+    attention layers in a row, 2560 tokens in chunks of 64, 48, 32 and 16 rows.  The second
+    layer's keys are made of every row the first one put out, so they hold the first layer's
+    attention to account at every row and cache length, where the last row's logits hold one."""
+    cfg = dict(n_layer=2, attn_every=1, vocab=8192, nkv=2688, slots=1)
+    prompt = np.random.default_rng(2560).integers(0, 8192, size=2560).astype(np.int32)
+    out = {}
+    for rows in (64, 48, 32, 16):
+        m = LA.LLM(LA.Config(max_tokens=rows, **cfg))
+        m.init_synthetic(7)
+        m.stage()
+        _, hd = m.extend(prompt, want_hidden=True)
+        k, v = m.kv(1, 2560)
+        out[rows] = (hd, k.view(np.float16).astype(np.float32).reshape(2560, -1), v.view(np.float16).astype(np.float32).reshape(2560, -1))
+        m.close()
+    for rows in (64, 48, 32):
+        a, b = out[rows], out[16]
+        assert O.rel_l2(a[0], b[0]) <= 1e-4, (rows, O.rel_l2(a[0], b[0]))
+        for x, y in ((a[1], b[1]), (a[2], b[2])):
+            # halves: a cell here and there rounds the other way, none is off by more than that
+            e = np.linalg.norm(x - y, axis=1) / np.linalg.norm(y, axis=1)
+            assert e.max() <= 2e-3, (rows, int(e.argmax()), float(e.max()))
