@@ -490,13 +490,14 @@ def test_chunk_size_does_not_matter_over_4096_tokens():
 
 def test_chunk_size_does_not_matter_to_a_second_attention_layer():
     """What a chunk's rows leave an attention layer with is only seen by the layers after it: two
-    attention layers in a row, 2560 tokens in chunks of 64, 48, 32 and 16 rows.  The second
+    attention layers in a row, 2560 tokens as one chunk and in chunks of 512 down to 16 rows.  The second
     layer's keys are made of every row the first one put out, so they hold the first layer's
     attention to account at every row and cache length, where the last row's logits hold one."""
     cfg = dict(n_layer=2, attn_every=1, vocab=8192, nkv=2688, slots=1)
     prompt = np.random.default_rng(2560).integers(0, 8192, size=2560).astype(np.int32)
     out = {}
-    for rows in (64, 48, 32, 16):
+    sizes = (2560, 512, 256, 128, 100, 64, 48, 32, 16)
+    for rows in sizes:
         m = LA.LLM(LA.Config(max_tokens=rows, **cfg))
         m.init_synthetic(7)
         m.stage()
@@ -504,7 +505,7 @@ def test_chunk_size_does_not_matter_to_a_second_attention_layer():
         k, v = m.kv(1, 2560)
         out[rows] = (hd, k.view(np.float16).astype(np.float32).reshape(2560, -1), v.view(np.float16).astype(np.float32).reshape(2560, -1))
         m.close()
-    for rows in (64, 48, 32):
+    for rows in sizes[:-1]:
         a, b = out[rows], out[16]
         assert O.rel_l2(a[0], b[0]) <= 1e-4, (rows, O.rel_l2(a[0], b[0]))
         for x, y in ((a[1], b[1]), (a[2], b[2])):
