@@ -410,6 +410,268 @@ __global__ __launch_bounds__(NTHR) void gemm_q4k_kernel(shv_gemv_q4k_args a, int
     }
 }
 
+// ---------------------------------------------------------------- passes of 3 to 16 rows -------
+// Several sequences decoded together, or the rows of a verification pass, against matrices of the
+// decode step's widths: the weights are what the launch moves, the rest is what it waits for.  One
+// block of sixteen waves a compute unit; every thread asks for its share of the activation rows,
+// the gates and gammas that go with them and its wave's first super-blocks before anything is
+// computed, the rows become matrix operands under those loads, and one block-wide wait later every
+// wave multiplies: v_mfma_f32_16x16x32_f16 with the eight rows as A (binary16 pairs hi + lo, the
+// tokens of the upper half of the tile repeat the lower) and a sub-block's weights as B, formed as
+// the whole numbers n * sc by one fused multiply-add on halves, one accumulator a super-block
+// (y += d * acc), the min term from the sub-blocks' sums of x.  The RMSNorm factor of a row is
+// applied to its outputs, so nothing waits for a row's sum of squares.
+// Operand order in LDS: fragment (sub-block, part) is 32 entries of 16 bytes, entry 8 kb + token
+// holding columns 8 kb .. 8 kb + 7 of the sub-block in the order [0, 2, 1, 3, 4, 6, 5, 7]; a wave
+// stages whole sub-blocks (lane = token + 8 * quad of the sub-block), so its writes fill a
+// fragment's 512 bytes side by side.
+__device__ __forceinline__ size_t out_offset(const shv_gemv_q4k_args &a, int t);
+constexpr int kRowsTok = 8, kRowsWaves = 16, kRowsThreads = kRowsWaves * 64;
+constexpr int kRowsFrag = 4 * kRowsTok * 16;  // bytes of one (sub-block, part) fragment
+
+template <int K>
+struct RowsLds {
+    static constexpr size_t frags = static_cast<size_t>(K / 32) * 2 * kRowsFrag;
+    static constexpr size_t sums = static_cast<size_t>(K / 32) * kRowsTok * 4;
+    static constexpr size_t red = static_cast<size_t>(kRowsTok) * kRowsWaves * 4;
+    static constexpr size_t ytile = static_cast<size_t>(kRowsWaves) * 64 * 16;
+    static constexpr size_t total = frags + sums + red + ytile + kRowsTok * sizeof(size_t);
+};
+
+// grid: blocks of sixteen waves; KS consecutive waves share a 16-row tile of the matrix, each over
+// 1/KS of its super-blocks.  t0: first activation row of this launch, nt: how many (<= 8).
+template <int K, int PRO, int RD>
+__global__ __launch_bounds__(kRowsThreads) void gemm_rows_kernel(shv_gemv_q4k_args a, int t0, int nt, int n_tiles, int ks_log2) {
+    extern __shared__ __align__(16) char smem[];
+    constexpr int SBS = K / SHV_Q4K_BLOCK;
+    constexpr int WCOLS = K / kRowsWaves;   // columns a wave stages: 128 or 256
+    constexpr int NQ = WCOLS / 32;          // sub-blocks a wave stages, one a step: a lane's quads
+    char *frags = smem;
+    float *sxs = reinterpret_cast<float *>(smem + RowsLds<K>::frags);
+    float *red = reinterpret_cast<float *>(smem + RowsLds<K>::frags + RowsLds<K>::sums);          // [token][wave]
+    float *ytile = red + kRowsTok * kRowsWaves;                                                 // [wave][64] float4
+    size_t *yoffs = reinterpret_cast<size_t *>(ytile + kRowsWaves * 64 * 4);                    // [token]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, kb = lane >> 4;  // B: weight row of the tile, k block; C: row n, tokens 4 kb .. 4 kb + 3
+    constexpr size_t row_bytes = static_cast<size_t>(SBS) * SHV_Q4K_BYTES;
+    const int ks = 1 << ks_log2, steps_log2 = __builtin_ctz(SBS) - ks_log2, steps = 1 << steps_log2;
+    const int part = wave & (ks - 1), tpb = kRowsWaves >> ks_log2;
+    const int tl0 = blockIdx.x * tpb + (wave >> ks_log2), stride = gridDim.x * tpb;
+    const int iters = (n_tiles + stride - 1) / stride;
+    const int total = iters << steps_log2;  // (tile, super-block) steps of this wave, the same count for every wave
+    const char *wbase = static_cast<const char *>(a.w) + static_cast<size_t>(part << steps_log2) * SHV_Q4K_BYTES;
+    auto sb_of = [&](int idx) {
+        const int tile = tl0 + (idx >> steps_log2) * stride, r = tile * kTileRows + n;
+        return wbase + static_cast<size_t>(r < a.n ? r : a.n - 1) * row_bytes + static_cast<size_t>(idx & (steps - 1)) * SHV_Q4K_BYTES;
+    };
+
+    // ---- everything this thread will need, asked for at once: its quads of the rows first ----
+    const int st_tok = lane & (kRowsTok - 1), st_quad = lane >> 3;  // token, quad of the sub-block
+    const int t_ld = t0 + (st_tok < nt ? st_tok : nt - 1);          // rows past the pass repeat its last (their outputs are dropped)
+    const int c0 = wave * WCOLS + 4 * st_quad;                      // step i: columns c0 + 32 i ..
+    float4 xv[NQ], zv[NQ], gv[PRO == SHV_PRO_GATED_NORM ? 4 : NQ];
+    {
+        const float *xrow = a.x + static_cast<size_t>(t_ld) * a.x_stride;
+        const float *zrow = a.z;
+        if constexpr (PRO == SHV_PRO_GATED_NORM || PRO == SHV_PRO_MUL_SIGMOID) {
+            zrow = a.z + static_cast<size_t>(t_ld) * a.z_stride;
+            if (a.z_ring) {
+                const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
+                const int s = t_ld / sl, k = t_ld % sl;
+                const int p = a.pos ? a.pos[s] : 0;
+                const int slot = a.slot ? a.slot[s] : s;
+                zrow = a.z + (static_cast<size_t>(slot) * a.ring_slots + (p + k) % a.ring_slots) * a.ring_stride;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NQ; i++) {
+            const int c = c0 + 32 * i;
+            xv[i] = *reinterpret_cast<const float4 *>(xrow + c);
+            if constexpr (PRO == SHV_PRO_RMSNORM) gv[i] = *reinterpret_cast<const float4 *>(a.gamma + c);
+            if constexpr (PRO == SHV_PRO_GATED_NORM) {
+                // heads of 128 columns: the gammas of step i are those of step i + 4
+                if (i < 4) gv[i] = *reinterpret_cast<const float4 *>(a.gamma + (c & 127));
+                zv[i] = *reinterpret_cast<const float4 *>(zrow + c);
+            }
+            if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+                // z rows are [q | gate] per head and the gate half is wanted (head_dim 0: plain rows)
+                const int zi = a.head_dim > 0 ? (c & ~(a.head_dim - 1)) * 2 + a.head_dim + (c & (a.head_dim - 1)) : c;
+                zv[i] = *reinterpret_cast<const float4 *>(zrow + zi);
+            }
+        }
+    }
+    SbLoads ld[RD];
+#pragma unroll
+    for (int d = 0; d < RD; d++)
+        if (d < total) ld[d].load(sb_of(d), kb);
+    if (tid < nt) yoffs[tid] = out_offset(a, t0 + tid);
+
+    // ---- the rows become operands ----
+    {
+        float ss = 0.f;
+        float hs[NQ];
+        if constexpr (PRO == SHV_PRO_GATED_NORM) {
+            // a head is four steps of this lane and the eight lanes of its token
+#pragma unroll
+            for (int i = 0; i < NQ; i++) hs[i] = fmaf(xv[i].x, xv[i].x, fmaf(xv[i].y, xv[i].y, fmaf(xv[i].z, xv[i].z, xv[i].w * xv[i].w)));
+#pragma unroll
+            for (int h = 0; h < NQ; h += 4) {
+                float t = (hs[h] + hs[h + 1]) + (hs[h + 2] + hs[h + 3]);
+                t += __shfl_xor(t, 8, 64);
+                t += __shfl_xor(t, 16, 64);
+                t += __shfl_xor(t, 32, 64);
+                hs[h] = __builtin_amdgcn_rsqf(t * (1.f / 128.f) + a.eps);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NQ; i++) {
+            float4 v = xv[i];
+            if constexpr (PRO == SHV_PRO_RMSNORM) {
+                ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+                v = make_float4(v.x * gv[i].x, v.y * gv[i].y, v.z * gv[i].z, v.w * gv[i].w);
+            } else if constexpr (PRO == SHV_PRO_GATED_NORM) {
+                const float sc = hs[i & ~3];
+                const float4 g = gv[i & 3], z = zv[i];
+                v = make_float4(v.x * sc * g.x * sigmoid_fast(z.x), v.y * sc * g.y * sigmoid_fast(z.y),
+                                v.z * sc * g.z * sigmoid_fast(z.z), v.w * sc * g.w * sigmoid_fast(z.w));
+            } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+                const float4 z = zv[i];
+                v = make_float4(v.x * sigmoid_fast(z.x), v.y * sigmoid_fast(z.y), v.z * sigmoid_fast(z.z), v.w * sigmoid_fast(z.w));
+            }
+            // the sub-block's sum of x: the eight lanes of this token
+            float sum = (v.x + v.y) + (v.z + v.w);
+            sum += __shfl_xor(sum, 8, 64);
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            const int sub = wave * NQ + i;
+            if (st_quad == 0) sxs[sub * kRowsTok + st_tok] = sum;
+            const float o[4] = {v.x, v.z, v.y, v.w};
+            half4_t h, l;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const _Float16 hi = static_cast<_Float16>(o[j]);
+                h[j] = hi;
+                l[j] = static_cast<_Float16>(o[j] - static_cast<float>(hi));
+            }
+            char *e = frags + static_cast<size_t>(sub) * 2 * kRowsFrag + ((st_quad >> 1) * kRowsTok + st_tok) * 16 + (st_quad & 1) * 8;
+            *reinterpret_cast<half4_t *>(e) = h;
+            *reinterpret_cast<half4_t *>(e + kRowsFrag) = l;
+        }
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            ss += __shfl_xor(ss, 8, 64);
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            if (st_quad == 0) red[st_tok * kRowsWaves + wave] = ss;
+        }
+    }
+    // LDS writes only: the super-blocks asked for above stay on their way
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // this lane's four tokens (those of the tile's upper half repeat the lower): their RMSNorm factors
+    const int tk0 = (4 * kb) & (kRowsTok - 1);
+    float scale[4] = {1.f, 1.f, 1.f, 1.f};
+    if constexpr (PRO == SHV_PRO_RMSNORM) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float4 *r4 = reinterpret_cast<const float4 *>(red + (tk0 + j) * kRowsWaves);
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < kRowsWaves / 4; w++) {
+                const float4 r = r4[w];
+                tot += (r.x + r.y) + (r.z + r.w);
+            }
+            scale[j] = __builtin_amdgcn_rsqf(tot * (1.f / static_cast<float>(K)) + a.eps);
+        }
+    }
+    const char *my_frag = frags + (kb * kRowsTok + (n & (kRowsTok - 1))) * 16;
+    const float *my_sx = sxs + tk0;
+    uint32_t m0 = 0x000F000Fu, o0 = 0x64006400u, m4 = 0x00F000F0u, o4 = 0x54005400u;
+    asm volatile("" : "+s"(m0), "+s"(m4));
+    asm volatile("" : "+v"(o0), "+v"(o4));
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+    float4_t y = {0.f, 0.f, 0.f, 0.f};
+    for (int base = 0; base < total; base += RD) {
+#pragma unroll
+        for (int d = 0; d < RD; d++) {
+            const int idx = base + d;
+            if (idx >= total) break;
+            const SbLoads cur = ld[d];
+            if (idx + RD < total) ld[d].load(sb_of(idx + RD), kb);
+            const int sb = (part << steps_log2) + (idx & (steps - 1));
+            const float dd = f16_bits_to_f32(cur.hdr.x), dmin = f16_bits_to_f32(cur.hdr.x >> 16);
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint32_t sc, mn;
+                q4k_group_scale_min(cur.hdr, g, sc, mn);
+                const uint32_t q0 = cur.q[g].x, q1 = cur.q[g].y;
+#pragma unroll
+                for (int hi = 0; hi < 2; hi++) {
+                    const int sub = sb * 8 + g * 2 + hi;
+                    // (C + n) * sc - C * sc = n * sc, a whole number up to 945: bits 0..3 of a half read as
+                    // 1024 + n under 1024's exponent, bits 4..7 as 64 + n under 64's
+                    const _Float16 s1 = static_cast<_Float16>(static_cast<float>(hi ? sc >> 8 : sc & 0xFFu));
+                    const half2_t s2 = {s1, s1};
+                    half2_t w[4], c[4];
+                    if (hi == 0) {
+                        w[0] = __builtin_bit_cast(half2_t, (q0 & m0) | o0); w[1] = __builtin_bit_cast(half2_t, ((q0 >> 4) & m4) | o4);
+                        w[2] = __builtin_bit_cast(half2_t, (q1 & m0) | o0); w[3] = __builtin_bit_cast(half2_t, ((q1 >> 4) & m4) | o4);
+                        c[0] = c[2] = s2 * static_cast<half2_t>(static_cast<_Float16>(-1024.f));
+                        c[1] = c[3] = s2 * static_cast<half2_t>(static_cast<_Float16>(-64.f));
+                    } else {
+                        w[0] = __builtin_bit_cast(half2_t, (q0 & m4) | o4); w[1] = __builtin_bit_cast(half2_t, ((q0 >> 8) & m4) | o4);
+                        w[2] = __builtin_bit_cast(half2_t, (q1 & m4) | o4); w[3] = __builtin_bit_cast(half2_t, ((q1 >> 8) & m4) | o4);
+                        c[0] = c[1] = c[2] = c[3] = s2 * static_cast<half2_t>(static_cast<_Float16>(-64.f));
+                    }
+                    half8_t b;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const half2_t p = __builtin_elementwise_fma(w[i], s2, c[i]);
+                        b[2 * i] = p[0];
+                        b[2 * i + 1] = p[1];
+                    }
+                    const char *f = my_frag + static_cast<size_t>(sub) * 2 * kRowsFrag;
+                    const half8_t xh = *reinterpret_cast<const half8_t *>(f);
+                    const half8_t xl = *reinterpret_cast<const half8_t *>(f + kRowsFrag);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, b, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b, acc, 0, 0, 0);
+                    const float e = dmin * static_cast<float>(hi ? mn >> 8 : mn & 0xFFu);
+                    const float4 sx = *reinterpret_cast<const float4 *>(my_sx + sub * kRowsTok);
+                    y[0] = fmaf(-e, sx.x, y[0]); y[1] = fmaf(-e, sx.y, y[1]);
+                    y[2] = fmaf(-e, sx.z, y[2]); y[3] = fmaf(-e, sx.w, y[3]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) y[j] = fmaf(dd, acc[j], y[j]);
+            if ((idx & (steps - 1)) != steps - 1) continue;
+            // ---- the tile's last super-block: the column parts meet in LDS, then C[4 kb + j][n] goes out ----
+            const int tile = tl0 + (idx >> steps_log2) * stride, r = tile * kTileRows + n;
+            if (ks > 1) {
+                *reinterpret_cast<float4_t *>(ytile + (wave * 64 + lane) * 4) = y;
+                __syncthreads();
+                if (part == 0) {
+                    for (int p = 1; p < ks; p++) y += *reinterpret_cast<const float4_t *>(ytile + ((wave + p) * 64 + lane) * 4);
+                }
+            }
+            if (part == 0 && tile < n_tiles && r < a.n && kb < kRowsTok / 4) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int tok = 4 * kb + j;
+                    if (tok < nt) {
+                        float v = y[j] * scale[j];
+                        if (a.residual) v += a.residual[static_cast<size_t>(t0 + tok) * a.y_stride + r];
+                        a.y[yoffs[tok] + r] = v;
+                    }
+                }
+            }
+            if (ks > 1) __syncthreads();
+            y = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+}
+
 // ---------------------------------------------------------------- passes of 17 to 64 rows -------
 // A prompt chunk has more rows than one block can keep in LDS for the whole width of the matrix,
 // so its operands stream: the activations of 64 rows are made once into `staged` as slabs of 128
@@ -1104,6 +1366,51 @@ int launch_wide(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const 
     return SHV_OK;
 }
 
+// Eight rows a launch on the sixteen-wave kernel: a matrix of few row tiles is split along its
+// columns over the waves of a block as far as that fills the chip's wave slots.
+template <int K, int PRO, int RD>
+int launch_rows_kp(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    constexpr int SBS = K / SHV_Q4K_BLOCK;
+    const int n_tiles = (a.n + kTileRows - 1) / kTileRows;
+    const long long slots = static_cast<long long>(ctx->prop.multiProcessorCount) * kRowsWaves;
+    int ks_log2 = 0;
+    while ((2 << ks_log2) <= kRowsWaves && (2 << ks_log2) <= SBS && static_cast<long long>(n_tiles) * (2 << ks_log2) <= slots) ks_log2++;
+    const int tpb = kRowsWaves >> ks_log2;
+    int blocks = (n_tiles + tpb - 1) / tpb;
+    if (blocks > ctx->prop.multiProcessorCount) blocks = ctx->prop.multiProcessorCount;
+    constexpr size_t lds = RowsLds<K>::total;
+    static bool raised = false;
+    if (!raised) {
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<K, PRO, RD>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        raised = true;
+    }
+    for (int t0 = 0; t0 < a.n_tok; t0 += kRowsTok) {
+        const int nt = a.n_tok - t0 < kRowsTok ? a.n_tok - t0 : kRowsTok;
+        SHV_LAUNCH(ctx, (gemm_rows_kernel<K, PRO, RD>), dim3(blocks), dim3(kRowsThreads), lds, a, t0, nt, n_tiles, ks_log2);
+    }
+    return SHV_OK;
+}
+
+template <int K, int RD>
+int launch_rows_k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    switch (a.prologue) {
+        case SHV_PRO_NONE: return launch_rows_kp<K, SHV_PRO_NONE, RD>(ctx, a);
+        case SHV_PRO_RMSNORM: return launch_rows_kp<K, SHV_PRO_RMSNORM, RD>(ctx, a);
+        case SHV_PRO_GATED_NORM: return launch_rows_kp<K, SHV_PRO_GATED_NORM, RD>(ctx, a);
+        default: return launch_rows_kp<K, SHV_PRO_MUL_SIGMOID, RD>(ctx, a);
+    }
+}
+
+// Which passes the sixteen-wave kernel takes (the arguments have passed shv_gemm_q4k_covers).
+bool rows_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (ctx->gemm_rows_min <= 0 || a.n_tok < ctx->gemm_rows_min) return false;
+    if (a.k != 2048 && a.k != 4096) return false;
+    if (a.n_tok > kRowsTok) return false;  // more rows would read the weights once per eight
+    if (a.prologue == SHV_PRO_GATED_NORM && a.head_dim != 128) return false;  // a head is four staging steps of a lane
+    if (a.prologue == SHV_PRO_MUL_SIGMOID && a.head_dim != 0 && (a.head_dim < 4 || (a.head_dim & (a.head_dim - 1)) != 0)) return false;
+    return true;
+}
+
 // Every group of 64 rows of a long pass in one launch (the operands of all of them are in
 // ctx->gemm_stage): no split along the columns, the groups themselves fill the chip.
 template <int NW, int R>
@@ -1178,6 +1485,7 @@ bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a) {
 }
 
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (rows_kernel_covers(ctx, a)) return a.k == 2048 ? launch_rows_k<2048, 3>(ctx, a) : launch_rows_k<4096, 1>(ctx, a);
     // the fragments of 16 rows of 4096 columns do not fit LDS: such a pass goes 8 rows at a time
     const int cap = a.k > 2048 ? 8 : 16;
     // more rows than one block keeps in LDS: groups of 64 stream their operands

@@ -46,6 +46,10 @@ int shv_init(int device, shv_ctx **out) {
         }
     }
     if (const char *e = std::getenv("SHV_GEMV_SCALES")) ctx->gemv_scales_lds = std::strcmp(e, "lds") == 0;
+    if (const char *e = std::getenv("SHV_GEMM_ROWS_MIN")) {
+        const int v = std::atoi(e);
+        if (v >= 0) ctx->gemm_rows_min = v;
+    }
     if (const char *e = std::getenv("SHV_MOE_GROUP_MIN")) {
         const int v = std::atoi(e);
         if (v >= 1) ctx->moe_group_min = v;

@@ -27,6 +27,9 @@ struct shv_ctx {
     // SHV_GEMV_SCALES=lds: the one-row GEMV hands each super-block's eight (d*sc, dmin*m) pairs from one lane to
     // the four that use them through LDS instead of letting every lane decode its own (for comparison; slower)
     bool gemv_scales_lds = false;
+    // passes of this many rows up to 16 (8 where rows are 4096 wide) take the sixteen-wave matrix-core kernel that
+    // stages its rows under the weight loads (SHV_GEMM_ROWS_MIN; 0: never)
+    int gemm_rows_min = 5;
     int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)
     int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;

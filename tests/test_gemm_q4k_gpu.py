@@ -51,7 +51,11 @@ def row_ctx():
                                       # passes of more rows than a block keeps in LDS stream their operands:
                                       # whole and ragged groups of 64, split columns, rows not a multiple of 128
                                       (12352, 2048, 64), (2048, 4096, 64), (9216, 2048, 33), (1000, 1024, 50),
-                                      (512, 2048, 57), (2048, 4096, 9), (40, 256, 20)])
+                                      (512, 2048, 57), (2048, 4096, 9), (40, 256, 20),
+                                      # 5..16 rows of the decode step's widths (8 where rows are 4096 wide): sixteen waves
+                                      # a block, the rows staged under the weight loads; ragged tiles, one to three rounds
+                                      (4096, 2048, 5), (12352, 2048, 8), (1000, 2048, 7), (7, 2048, 6), (2048, 2048, 13),
+                                      (2048, 4096, 8), (2048, 4096, 5), (33, 4096, 6), (9216, 2048, 16), (70000, 2048, 8)])
 def test_rows_match_oracle_and_float64(ctx, row_ctx, n, k, rows):
     rng = np.random.default_rng(n + k + rows)
     wq = _weights(rng, n, k)
@@ -118,7 +122,7 @@ def test_long_pass_rmsnorm_prologue_residual_in_place(ctx, rows):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-@pytest.mark.parametrize("rows", [3, 64])
+@pytest.mark.parametrize("rows", [3, 6, 8, 11, 64])
 def test_rmsnorm_prologue_residual_in_place(ctx, rows):
     """The residual stream's own rows are the residual and the destination (dn.out, attn.out, the
     MoE down projection write x in place)."""
@@ -137,7 +141,7 @@ def test_rmsnorm_prologue_residual_in_place(ctx, rows):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-@pytest.mark.parametrize("rows,slots", [(4, 8), (37, 64), (260, 512)])
+@pytest.mark.parametrize("rows,slots", [(4, 8), (5, 8), (8, 8), (37, 64), (260, 512)])
 def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx, rows, slots):
     """DeltaNet's output projection at its real shape: 4096 columns (two column ranges), per-head
     norm, the gate z read from the projection ring at each row's position, residual in place."""
@@ -165,7 +169,7 @@ def test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx, rows, slots):
         assert O.rel_l2(got[t], want) <= TOL, t
 
 
-@pytest.mark.parametrize("rows", [3, 64])
+@pytest.mark.parametrize("rows", [3, 7, 8, 64])
 def test_sigmoid_gate_prologue_with_fused_query_rows(ctx, rows):
     """Attention's output projection: x * sigmoid(gate), the gate being the second half of each
     head's [q | gate] rows in the fused projection (llm/attn.go:162-166,198-205)."""
@@ -207,3 +211,45 @@ def test_ring_output_for_sequences_and_slots(ctx, seq_len, slots):
             assert O.rel_l2(row, O.gemv_q4k(wq, x[s * seq_len + i], n, k, threads=8)) <= TOL, (s, i)
             written[slot[s], (pos[s] + i) % slots] = True
     assert (got[~written] == -7.0).all()
+
+
+@pytest.mark.parametrize("n_seq", [5, 8, 12])
+def test_one_row_each_of_several_sequences(ctx, n_seq):
+    """Several sequences decoded together: a row each, every sequence at its own position on its own slot.  The DeltaNet
+    input projection (norm folded in) writes each row into its sequence's ring; the output projection takes each row's
+    gate from that ring at the sequence's position, norms per head and adds the residual in place."""
+    rng = np.random.default_rng(35 + n_seq)
+    H, W, d, eps, slots, n_slots = 2048, 12352, 128, 1e-6, 8, 13
+    z_col, k2 = 8192, 4096
+    w_in, w_out = _weights(rng, W, H), _weights(rng, H, k2)
+    x = (rng.standard_normal((n_seq, H)) * 2).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    pos = rng.integers(0, 40, size=n_seq).astype(np.int32)
+    slot = rng.permutation(n_slots)[:n_seq].astype(np.int32)
+    ring0 = rng.standard_normal((n_slots, slots, W)).astype(np.float32)
+    dring = ctx.upload(ring0)
+    dpos, dslot = ctx.upload(pos), ctx.upload(slot)
+    ctx.gemv_q4k(ctx.upload(w_in), ctx.upload(x), dring, W, H, n_tok=n_seq, prologue=A.PRO_RMSNORM, gamma=ctx.upload(gamma),
+                 eps=eps, pos=dpos, slot=dslot, seq_len=1, ring_slots=slots, ring_stride=W)
+    ring = dring.read(np.float32, ring0.size).reshape(ring0.shape)
+    written = np.zeros((n_slots, slots), bool)
+    for s in range(n_seq):
+        want = O.gemv_q4k(w_in, O.rmsnorm(x[s], gamma, eps), W, H, threads=8)
+        assert O.rel_l2(ring[slot[s], pos[s] % slots], want) <= TOL, s
+        written[slot[s], pos[s] % slots] = True
+    assert (ring[~written] == ring0[~written]).all()
+    o = rng.standard_normal((n_seq, k2)).astype(np.float32)
+    g2 = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    res = rng.standard_normal((n_seq, H)).astype(np.float32)
+    dy = ctx.upload(res)
+    ctx.gemv_q4k(ctx.upload(w_out), ctx.upload(o), dy, H, k2, n_tok=n_seq, prologue=A.PRO_GATED_NORM, gamma=ctx.upload(g2),
+                 z=dring.at(z_col * 4), head_dim=d, eps=eps, residual=dy, pos=dpos, slot=dslot, seq_len=1, ring_slots=slots,
+                 ring_stride=W, z_ring=1)
+    got = dy.read(np.float32, n_seq * H).reshape(n_seq, H)
+    L = O.lib()
+    for s in range(n_seq):
+        z = ring[slot[s], pos[s] % slots, z_col:z_col + k2]
+        xn = O.rmsnorm(o[s].reshape(-1, d), g2, eps).ravel()
+        sig = np.array([L.shv_ref_sigmoid(float(v)) for v in z], dtype=np.float32)
+        want = O.gemv_q4k(w_out, (xn * sig).astype(np.float32), H, k2, threads=8) + res[s]
+        assert O.rel_l2(got[s], want) <= TOL, s
