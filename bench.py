@@ -80,8 +80,9 @@ def cpu_baseline(m, cfg, LA, A, tensors, n_tokens, cores):
     import oracle_lib as O
     per = cfg.attn_every
     sub = LA.Config(**{f: getattr(cfg, f) for f, _ in cfg._fields_})
-    sub.n_layer, sub.nkv, sub.max_tokens, sub.slots, sub.speculative, sub.nextn, sub.head_rows = per, 128, 4, 1, 0, 0, 1
-    om = O.OracleModel(sub, tensors, max_cells=64)
+    cells = (n_tokens + 2 + 127) // 128 * 128
+    sub.n_layer, sub.nkv, sub.max_tokens, sub.slots, sub.speculative, sub.nextn, sub.head_rows = per, cells, 4, 1, 0, 0, 1
+    om = O.OracleModel(sub, tensors, max_cells=cells)
     rng = np.random.default_rng(1)
     ids = rng.integers(0, cfg.vocab, size=n_tokens + 1).astype(np.int32)
     om.extend(ids[:1], threads=cores)  # touch everything once
@@ -113,7 +114,7 @@ def cpu_baseline(m, cfg, LA, A, tensors, n_tokens, cores):
     err = O.rel_l2(got, hidden)
     if not err <= 1e-3:
         raise SystemExit("bench.py: the GPU's residual stream after layer %d differs from the oracle's by rel-L2 %.3e (> 1e-3)" % (per - 1, err))
-    return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+    return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "kind": "port", "sample_seconds": round(dt * n_tokens, 2),
             "hidden_rel_l2_vs_gpu": float("%.3e" % err),
             "sample": "C restatement of the reference's Go CPU path (oracle/), layers 0-%d + lm_head of the same "
                       "weights, %d decode tokens at context <= %d; period time x%d + head time; rows of each matvec "
@@ -536,7 +537,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=48)
-    ap.add_argument("--cpu-tokens", type=int, default=4)
+    ap.add_argument("--cpu-tokens", type=int, default=384,
+                    help="decode tokens of the CPU leg (four layers and the head each; about ten seconds of host work at the default)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-mtp", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-config blocks (configs 1-4 each on its own)")
