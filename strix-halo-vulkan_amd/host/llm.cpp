@@ -1343,6 +1343,20 @@ const float *Graph::ForwardResidual(const std::vector<int32_t> &ids, std::vector
     return res_all_;
 }
 
+const float *Graph::ExtendResidual(const std::vector<int32_t> &ids, std::vector<float> *logits) {
+    if (logits && !head_) throw Error("llm: Graph.ExtendResidual: the graph was staged without a head");
+    if (ids.size() > res_all_rows_) {
+        res_all_rows_ = std::max<size_t>(ids.size(), 256);
+        res_all_ = static_cast<float *>(dev_.alloc(res_all_rows_ * c_.NEmbd * 4));
+    }
+    extend(ids, res_all_);
+    if (logits) {
+        logits->resize(c_.VocabSize);
+        dev_.download(logits->data(), head_->LogitsPort(), static_cast<size_t>(c_.VocabSize) * 4);
+    }
+    return res_all_;
+}
+
 void Graph::ExtendRows(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *res) {
     if (!head_) throw Error("llm: this graph was staged without a head");
     const int n = static_cast<int>(ids.size());
@@ -1724,12 +1738,105 @@ void MTPHead::LastLogits(std::vector<float> *out) {
 
 // --------------------------------------------------------------------------- Speculator -------
 
-Speculator::Speculator(Graph &g, MTPHead &d, int depth) : Depth(depth), g_(g), d_(d) {
+Speculator::Speculator(Graph &g, MTPHead &d, int depth, int slot) : Depth(depth), g_(g), d_(d), slot_(slot) {
     if (depth < 1 || depth + 1 > g.MaxRows()) throw Error("llm: a draft depth of " + std::to_string(depth) + " needs passes of " + std::to_string(depth + 1) + " rows — GraphOpts.SpecRows");
     if (d.MaxRows() < depth + 1) throw Error("llm: the draft head is staged for " + std::to_string(d.MaxRows()) + " rows; a round owes up to " + std::to_string(depth + 1));
-    h_ = static_cast<float *>(g.Dev().alloc(static_cast<size_t>(depth + 1) * g.GetModel().config().NEmbd * 4));
-    g.Speculate(true);
-    g.SpeculateFirst(true);
+    if (slot >= g.Slots() || slot >= d.Slots())
+        throw Error("llm: speculator slot " + std::to_string(slot) + "; the trunk holds " + std::to_string(g.Slots()) + " and the draft " + std::to_string(d.Slots()));
+    // the owed rows (fewer than one draft call's worth: Owe settles at that) and the seed after them
+    cap_rows_ = std::max(depth + 1, d.MaxRows()) + 2;
+    h_ = static_cast<float *>(g.Dev().alloc(static_cast<size_t>(cap_rows_) * g.GetModel().config().NEmbd * 4));
+    if (slot < 0) {
+        g.Speculate(true);
+        g.SpeculateFirst(true);
+    }
+}
+
+void Speculator::use_slot() {
+    if (slot_ >= 0) d_.UseSlot(slot_);
+}
+
+void Speculator::Prime(const std::vector<int32_t> &ids, int at, const float *res) {
+    const int n = static_cast<int>(ids.size());
+    const size_t E = g_.GetModel().config().NEmbd;
+    if (n < 1 || !res) throw Error("llm: Speculator.Prime: no rows");
+    use_slot();
+    if (at == 0) owe_x_.clear();  // the slot's sequence starts over, and what its draft owed went with it
+    if (at > 0 && !seeded_) throw Error("llm: priming from position " + std::to_string(at) + " without the residual before it");
+    if (!owe_x_.empty()) throw Error("llm: priming the draft while it owes " + std::to_string(owe_x_.size()) + " rows; settle first");
+    if (at > 0 && at != d_.Past()) throw Error("llm: priming the draft at " + std::to_string(at) + "; its cache holds " + std::to_string(d_.Past()));
+    if (at == 0) {
+        d_.Reset();
+        g_.Dev().zero(h_, E * 4);
+    }
+    d_.Rows(h_, {ids[0]}, at, false);
+    const int M = d_.MaxRows();
+    for (int a = 1; a < n; a += M) {
+        const int k = std::min(M, n - a);
+        d_.Rows(res + static_cast<size_t>(a - 1) * E, std::vector<int32_t>(ids.begin() + a, ids.begin() + a + k), at + a, false);
+    }
+    check(shv_copy(g_.Dev().ctx(), h_, res + static_cast<size_t>(n - 1) * E, E * 4), "seed");
+    seeded_ = true;
+    pend_ = -1;
+}
+
+void Speculator::Owe(int32_t x, const float *h) {
+    if (!seeded_) throw Error("llm: Speculator.Owe without the residual before the row");
+    const size_t E = g_.GetModel().config().NEmbd;
+    // the seed becomes the residual before x's position, h the new seed
+    owe_x_.push_back(x);
+    check(shv_copy(g_.Dev().ctx(), h_ + owe_x_.size() * E, h, E * 4), "owed row");
+    // a round's first draft call carries the owed rows and the pending token: a long run of
+    // plain steps is written as it fills a call (llm/spec.go:366-371)
+    if (static_cast<int>(owe_x_.size()) >= d_.MaxRows()) settle_owed();
+}
+
+void Speculator::settle_owed() {
+    const int n = static_cast<int>(owe_x_.size());
+    if (n == 0) return;
+    const size_t E = g_.GetModel().config().NEmbd;
+    use_slot();
+    const int at = past() - n, M = d_.MaxRows();
+    for (int p0 = 0; p0 < n; p0 += M) {
+        const int k = std::min(M, n - p0);
+        d_.Rows(h_ + static_cast<size_t>(p0) * E, std::vector<int32_t>(owe_x_.begin() + p0, owe_x_.begin() + p0 + k), at + p0, false);
+    }
+    check(shv_copy(g_.Dev().ctx(), h_, h_ + static_cast<size_t>(n) * E, E * 4), "seed");
+    owe_x_.clear();
+}
+
+void Speculator::Settle() {
+    pend_ = -1;
+    use_slot();
+    settle_owed();
+    // a deeper draft wrote cells past the trunk: they are masked once the position says so
+    if (d_.Past() > past()) d_.Rewind(past());
+}
+
+std::vector<float> Speculator::Residual() const {
+    const size_t E = g_.GetModel().config().NEmbd;
+    std::vector<float> h(E);
+    g_.Dev().download(h.data(), h_ + owe_x_.size() * E, E * 4);
+    return h;
+}
+
+void Speculator::Rewind(int past, const std::vector<float> &h) {
+    const size_t E = g_.GetModel().config().NEmbd;
+    if (h.size() != E) throw Error("llm: rewinding the draft without the residual before " + std::to_string(past));
+    use_slot();
+    d_.Rewind(past);
+    g_.Dev().upload(h_, h.data(), E * 4);
+    seeded_ = true;
+    pend_ = -1;
+    owe_x_.clear();
+}
+
+std::vector<int32_t> Speculator::RoundFrom(int32_t first, const std::vector<int32_t> &forced, int limit) {
+    if (!seeded_) throw Error("llm: a round without the trunk's residual");
+    use_slot();
+    if (static_cast<int>(owe_x_.size()) + 1 > d_.MaxRows()) settle_owed();
+    pend_ = first;
+    return Round(forced, limit);
 }
 
 int32_t Speculator::Start(const std::vector<int32_t> &prompt) {
@@ -1752,6 +1859,7 @@ int32_t Speculator::Start(const std::vector<int32_t> &prompt) {
     // the trunk's residual after the last prompt row seeds the first round
     check(shv_copy(g_.Dev().ctx(), h_, res + static_cast<size_t>(T - 1) * E, E * 4), "seed");
     owe_x_.clear();
+    seeded_ = true;
     if (sampler_) {
         // the prompt enters the penalties' window, then its last row is sampled on the host
         sampler_->Accept(prompt.data(), T);
@@ -1781,7 +1889,7 @@ void Speculator::UseSampler(Sampler *s, int64_t draft_seed) {
 // A round under a sampler (llm/spec.go:703-857 with llm/sample.go:183-250).  The passes are the
 // greedy round's; what differs is who names the tokens: each draft is a draw from the draft
 // sampler's distribution over the draft head's logits, each verified row goes through Verify.
-std::vector<int32_t> Speculator::sampled_round(const std::vector<int32_t> &forced) {
+std::vector<int32_t> Speculator::sampled_round(const std::vector<int32_t> &forced, int limit) {
     const size_t E = g_.GetModel().config().NEmbd;
     const int V = g_.GetModel().config().VocabSize;
     const int at = g_.Past();
@@ -1820,6 +1928,7 @@ std::vector<int32_t> Speculator::sampled_round(const std::vector<int32_t> &force
 
     std::vector<int32_t> out;
     for (int i = 0; i < n; i++) {
+        if (limit > 0 && static_cast<int>(out.size()) >= limit) break;
         float *row = logits.data() + static_cast<size_t>(i) * V;
         int32_t tok;
         if (i + 1 < n) tok = sampler_->Verify(row, V, rows[i + 1], drawn[i] ? &q[i] : nullptr);
@@ -1842,9 +1951,10 @@ std::vector<int32_t> Speculator::sampled_round(const std::vector<int32_t> &force
     return out;
 }
 
-std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced) {
+std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced, int limit) {
     if (pend_ < 0) throw Error("llm: Speculator.Round before Start");
-    if (sampler_) return sampled_round(forced);
+    use_slot();
+    if (sampler_) return sampled_round(forced, limit);
     const size_t E = g_.GetModel().config().NEmbd;
     const int at = g_.Past();
     const int owed = static_cast<int>(owe_x_.size());
@@ -1879,6 +1989,7 @@ std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced) {
     //    draft it disagrees with
     std::vector<int32_t> out;
     for (int i = 0; i < n; i++) {
+        if (limit > 0 && static_cast<int>(out.size()) >= limit) break;
         out.push_back(best[i]);
         if (i + 1 == n) break;
         Stats.DraftedAt[std::min(i, 3)]++;

@@ -387,6 +387,9 @@ public:
     // ForwardResidual is Forward that also keeps the residual of EVERY prompt row on the device,
     // [T][NEmbd], which is what primes the draft head (llm/graph.go:1441-1450).
     const float *ForwardResidual(const std::vector<int32_t> &ids, std::vector<float> *logits);
+    // ExtendResidual is the same for a sequence that goes on: ids appended, every row's residual kept
+    // (llm/graph.go ExtendResidual, as backend/llm_sched.go:672 calls it for a chunk that primes a draft).
+    const float *ExtendResidual(const std::vector<int32_t> &ids, std::vector<float> *logits);
     // ExtendRows appends ids and computes every row's logits: the verification pass
     // (llm/graph.go:1383-1429).  logits [n][vocab] and res [n][NEmbd] (the residual before the
     // final norm) are copied out when asked for; Argmaxes() and ResPort() serve a caller that
@@ -404,6 +407,8 @@ public:
     int Slots() const { return o_.Slots; }
     int Slot() const { return slot_; }
     int Past() const { return seq_[slot_].past; }
+    int PastOf(int s) const { return seq_.at(s).past; }
+    bool InFlight() const { return spec_armed_; }  // a rewindable pass has run and is neither kept nor committed
     int Plane() const { return seq_[slot_].plane; }  // the live slot's committed DeltaNet state plane
     int NKV() const { return o_.NKV; }
     int MaxRows() const { return rows_max_; }
@@ -538,18 +543,40 @@ struct SpecStats {
 // logits then come to the host, where the reference keeps its sampler too.
 class Speculator {
 public:
-    Speculator(Graph &g, MTPHead &d, int depth);
+    // slot >= 0: the speculator of one sequence slot of a served graph (NewSlotSpeculator,
+    // llm/spec.go:258): it drafts in that slot of the draft's cache and leaves Graph.Speculate to
+    // its caller, who also runs plain and batched passes on the same graph.
+    Speculator(Graph &g, MTPHead &d, int depth, int slot = -1);
     // Prefill the prompt through the trunk and the draft (Start + Prime, llm/spec.go:300-420);
     // returns the first generated token.
     int32_t Start(const std::vector<int32_t> &prompt);
     // One round (llm/spec.go:703-857): the tokens it emitted, 1..Depth+1 of them.  `forced`, when
     // not empty, replaces the draft head's proposals (the draft still runs): the reference's
     // `propose` hook, which tests use to drive every acceptance length.
-    std::vector<int32_t> Round(const std::vector<int32_t> &forced = {});
+    // limit > 0: the round keeps at most that many tokens (a request's remaining budget).
+    std::vector<int32_t> Round(const std::vector<int32_t> &forced = {}, int limit = 0);
     // s == nullptr or a greedy sampler: back to arg-max.  The sampler is borrowed; the draft's is made
     // from it (Sampler::DraftSampler) with its own seed.  Takes effect at the next Start.
     void UseSampler(Sampler *s, int64_t draft_seed);
     void Stop() { g_.Speculate(false); }
+    // ---- the served loop's pieces (llm/spec.go:285-456) ----
+    // Prime writes the draft's cells at positions at .. at+n-1 from a chunk the trunk has just run:
+    // res is ExtendResidual's, row r the trunk's residual at at+r, on the device.  Position `at`
+    // is seeded from the residual this speculator holds, or zeros at position 0.
+    void Prime(const std::vector<int32_t> &ids, int at, const float *res);
+    // Owe records a plain decode step the trunk ran on this slot, token x and the trunk's residual
+    // at that row (on the device): the draft catches up at the next round or at Settle.
+    void Owe(int32_t x, const float *h);
+    // Settle writes the draft's cells for the rows it owes; nothing is pending after it.
+    void Settle();
+    // The trunk's residual one row before its position, which a checkpoint keeps beside the
+    // trunk's state so that Rewind can resume from it.
+    std::vector<float> Residual() const;
+    void Rewind(int past, const std::vector<float> &h);
+    // One round from `first`, the token named last and not yet run (Round, llm/spec.go:349).
+    std::vector<int32_t> RoundFrom(int32_t first, const std::vector<int32_t> &forced = {}, int limit = 0);
+    bool Seeded() const { return seeded_; }
+    int Owed() const { return static_cast<int>(owe_x_.size()); }
     SpecStats Stats;
     int Depth;
 
@@ -557,11 +584,16 @@ private:
     Graph &g_;
     MTPHead &d_;
     int32_t pend_ = -1;
-    float *h_ = nullptr;  // [Depth+1][NEmbd]: the owed rows' residuals, then the trunk's last one
+    int slot_ = -1, cap_rows_ = 0;
+    bool seeded_ = false;
+    float *h_ = nullptr;  // [cap_rows_][NEmbd]: the owed rows' residuals, then the trunk's last one
     std::vector<int32_t> owe_x_;
+    void use_slot();
+    int past() const { return slot_ >= 0 ? g_.PastOf(slot_) : g_.Past(); }
+    void settle_owed();
     Sampler *sampler_ = nullptr;
     std::unique_ptr<Sampler> draft_sampler_;
-    std::vector<int32_t> sampled_round(const std::vector<int32_t> &forced);
+    std::vector<int32_t> sampled_round(const std::vector<int32_t> &forced, int limit);
 };
 
 }  // namespace llm

@@ -479,6 +479,7 @@ static void pass_out(const llm::SchedPass &p, shvllm_sched_pass *o) {
     o->kind = p.kind, o->unit = p.unit, o->slot = p.slot, o->pos = p.pos, o->n = p.n;
     o->fresh = p.fresh, o->restore = p.restore, o->take = p.take, o->step = p.step;
     o->wait_ms = p.wait_ms;
+    o->prime = p.prime, o->tracked = p.tracked;
     o->n_units = static_cast<int32_t>(std::min<size_t>(p.units.size(), SHVLLM_SCHED_MAX_ROWS));
     for (int i = 0; i < o->n_units; i++) o->units[i] = p.units[i], o->slots[i] = p.slots[i];
 }
@@ -493,11 +494,12 @@ int shvllm_sched_open(shvllm *h, int slots, const shvllm_sched_opts *opts, shvll
             o.Reserve = opts->reserve;
             o.NoBatchDecode = opts->no_batch_decode != 0;
             if (opts->coalesce_ms >= 0) o.CoalesceMs = opts->coalesce_ms;
+            o.SpecDepth = opts->spec_depth;
         }
         llm::Graph *g = h ? &graph_of(h) : nullptr;
         if ((g ? g->Slots() : slots) > SHVLLM_SCHED_MAX_ROWS) throw llm::Error("llm: a scheduler covers at most " + std::to_string(SHVLLM_SCHED_MAX_ROWS) + " slots");
         auto s = std::make_unique<shvllm_sched>();
-        s->s = std::make_unique<llm::Sched>(g, slots, o);
+        s->s = std::make_unique<llm::Sched>(g, slots, o, h && o.SpecDepth > 0 ? &mtp_of(h) : nullptr);
         *out = s.release();
     });
 }
@@ -538,6 +540,13 @@ int shvllm_sched_step(shvllm_sched *s, int job, int32_t id, int *unit) {
     });
 }
 
+int shvllm_sched_decode(shvllm_sched *s, int job, int32_t id, int room, int *unit) {
+    return guard([&] {
+        if (!unit) throw llm::Error("llm: shvllm_sched_decode: NULL argument");
+        *unit = sched_of(s).Decode(job, id, room);
+    });
+}
+
 int shvllm_sched_withdraw(shvllm_sched *s, int unit) {
     return guard([&] { sched_of(s).Withdraw(unit); });
 }
@@ -555,9 +564,22 @@ int shvllm_sched_finish(shvllm_sched *s, double took_ms, int ok, double now_ms) 
     return guard([&] {
         llm::Sched &sc = sched_of(s);
         if (s->last.kind == llm::SchedPass::kNone) throw llm::Error("llm: no pass is out");
+        if (s->last.kind == llm::SchedPass::kRound && ok) throw llm::Error("llm: a round is finished with its tokens (shvllm_sched_finish_round)");
         const llm::SchedPass p = s->last;
         s->last = llm::SchedPass();
         sc.Finish(p, took_ms, ok != 0, now_ms, nullptr, ok ? "" : "the caller's pass failed");
+    });
+}
+
+int shvllm_sched_finish_round(shvllm_sched *s, double took_ms, int ok, double now_ms, const int32_t *toks, int n) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        if (s->last.kind != llm::SchedPass::kRound) throw llm::Error("llm: no round is out");
+        if (ok && (!toks || n < 1)) throw llm::Error("llm: a finished round names its tokens");
+        const llm::SchedPass p = s->last;
+        s->last = llm::SchedPass();
+        const std::vector<int32_t> t(toks, toks + (ok ? n : 0));
+        sc.Finish(p, took_ms, ok != 0, now_ms, nullptr, ok ? "" : "the caller's round failed", &t);
     });
 }
 
@@ -578,6 +600,15 @@ int shvllm_sched_unit(shvllm_sched *s, int unit, int *state, int *left, double *
         if (busy_ms) *busy_ms = u.busy_ms;
         if (u.failed) std::snprintf(g_err, sizeof(g_err), "%s", u.err.c_str());
         if (logits && u.done && !u.failed) std::copy(u.logits.begin(), u.logits.begin() + std::min<size_t>(max, u.logits.size()), logits);
+    });
+}
+
+int shvllm_sched_unit_tokens(shvllm_sched *s, int unit, int32_t *dst, int max, int *n) {
+    return guard([&] {
+        const llm::Sched::UnitState u = sched_of(s).Unit(unit);
+        if (!u.known) throw llm::Error("llm: no such unit " + std::to_string(unit));
+        if (n) *n = static_cast<int>(u.toks.size());
+        if (dst) std::copy(u.toks.begin(), u.toks.begin() + std::min<size_t>(max, u.toks.size()), dst);
     });
 }
 
@@ -602,6 +633,21 @@ int shvllm_sched_held(shvllm_sched *s, int slot, int32_t *dst, int max, int *n, 
         if (n) *n = static_cast<int>(h.size());
         if (dst) std::copy(h.begin(), h.begin() + std::min<size_t>(max, h.size()), dst);
         if (ckpt_len) *ckpt_len = sc.CheckpointLen(slot);
+    });
+}
+
+int shvllm_sched_round_counts(shvllm_sched *s, int32_t counts[2]) {
+    return guard([&] {
+        const llm::SchedCounts c = sched_of(s).Counts();
+        counts[0] = c.rounds, counts[1] = c.round_tokens;
+    });
+}
+
+int shvllm_sched_tracked(shvllm_sched *s, int slot, int *tracked) {
+    return guard([&] {
+        llm::Sched &sc = sched_of(s);
+        if (slot < 0 || slot >= sc.Slots() || !tracked) throw llm::Error("llm: slot " + std::to_string(slot));
+        *tracked = sc.Tracked(slot) ? 1 : 0;
     });
 }
 

@@ -23,7 +23,7 @@ int Sched::UsablePrefix(const std::vector<int32_t> &held, const std::vector<int3
     return 0;
 }
 
-Sched::Sched(Graph *g, int slots, const SchedOpts &o) : g_(g), o_(o) {
+Sched::Sched(Graph *g, int slots, const SchedOpts &o, MTPHead *draft) : g_(g), o_(o) {
     if (g) slots = g->Slots();
     if (slots < 1) throw Error("llm: a scheduler needs at least one slot");
     if (o_.Batch < 1) throw Error("llm: scheduler batch " + std::to_string(o_.Batch));
@@ -34,6 +34,15 @@ Sched::Sched(Graph *g, int slots, const SchedOpts &o) : g_(g), o_(o) {
     // a batched decode pass carries as many rows as the graph's head was staged for
     step_rows_ = g ? g->StepRows() : slots;
     if (step_rows_ < 1) throw Error("llm: the scheduler needs a graph staged with its head");
+    if (o_.SpecDepth < 0) throw Error("llm: scheduler: negative draft depth");
+    if (o_.SpecDepth > 0 && g) {
+        if (!draft) throw Error("llm: speculative rounds need the draft head staged");
+        if (g->DeltaNet().Planes() < o_.SpecDepth + 2)
+            throw Error("llm: rounds of " + std::to_string(o_.SpecDepth + 1) + " rows need a graph staged for them (GraphOpts.Speculative, SpecRows)");
+        for (int i = 0; i < slots; i++) specs_.push_back(std::make_unique<Speculator>(*g, *draft, o_.SpecDepth, i));
+    }
+    // without a graph the policy alone says when a round would run
+    spec_on_ = o_.SpecDepth > 0;
 }
 
 Sched::~Sched() = default;
@@ -207,6 +216,34 @@ int Sched::Step(int job, int32_t tok) {
     return id;
 }
 
+int Sched::Decode(int job, int32_t tok, int room) {
+    const int id = Step(job, tok);
+    UnitRec &u = units_.at(id);
+    u.round = spec_on_;
+    u.room = room;
+    return id;
+}
+
+// speculates: whether a picked decode unit runs as a speculative round: it asked to, its slot's
+// draft is caught up, the round's rows fit the cache and the request's budget, and no other
+// conversation of its class is decoding (backend/llm_sched.go:936-953).
+bool Sched::speculates(int unit) const {
+    const UnitRec &u = units_.at(unit);
+    if (!u.round || u.room < 2 || !spec_on_) return false;
+    const JobRec &j = jobs_.at(u.job);
+    const Slot &sl = slots_[j.slot];
+    if (!sl.track) return false;
+    if (g_ && static_cast<int>(sl.held.size()) + o_.SpecDepth + 1 > g_->NKV()) return false;
+    for (const Slot &o : slots_)
+        if (o.job >= 0 && o.job != u.job && jobs_.at(o.job).cls == j.cls && jobs_.at(o.job).stepping) return false;
+    return true;
+}
+
+void Sched::wipe(Slot &sl, int slot) {
+    sl.held.clear(), sl.ckpt_len = 0, sl.ckpt_keys.clear(), ckpts_[slot].reset();
+    sl.track = false, sl.ckpt_primed = false, sl.ckpt_res.clear();
+}
+
 void Sched::drop_pending(int unit) {
     auto it = std::find(pending_.begin(), pending_.end(), unit);
     if (it != pending_.end()) pending_.erase(it);
@@ -296,6 +333,14 @@ SchedPass Sched::Next(double now_ms) {
     if (id < 0) return p;
     UnitRec &u = units_.at(id);
     const JobRec &j = jobs_.at(u.job);
+    if (u.step && speculates(id)) {
+        p.kind = SchedPass::kRound;
+        p.unit = id, p.slot = j.slot, p.pos = static_cast<int>(slots_[j.slot].held.size()), p.n = 1, p.step = true;
+        p.ids.assign(1, u.ids[u.at]);
+        p.room = u.room;
+        u.on_device = true;
+        return p;
+    }
     if (u.step) {
         const std::vector<int> b = steps(id);
         const double wait = coalesce_wait(id, static_cast<int>(b.size()), now_ms);
@@ -333,14 +378,44 @@ SchedPass Sched::Next(double now_ms) {
     p.unit = id, p.slot = j.slot, p.pos = pos, p.n = n;
     p.fresh = u.fresh, p.restore = u.restore && !u.fresh, p.step = u.step;
     p.take = j.mark > 0 && pos + n == j.mark;
+    // the draft's cells below a restored checkpoint are still its tokens' if the draft covered what
+    // the slot held and the checkpoint kept the residual to resume from (backend/llm_sched.go:625-637)
+    p.tracked = sl.track && (!p.restore || sl.ckpt_primed);
+    p.prime = spec_on_ && !u.step && (p.fresh || p.tracked);
     p.ids.assign(u.ids.begin() + u.at, u.ids.begin() + u.at + n);
     u.on_device = true;
     return p;
 }
 
-void Sched::Finish(const SchedPass &p, double took_ms, bool ok, double now_ms, const std::vector<float> *logits, const std::string &err) {
+void Sched::Finish(const SchedPass &p, double took_ms, bool ok, double now_ms, const std::vector<float> *logits, const std::string &err,
+                   const std::vector<int32_t> *toks) {
     if (p.kind == SchedPass::kNone) return;
     counts_.passes++;
+    if (p.kind == SchedPass::kRound) {
+        // the rows the round kept: its input and every token it drew but the last, which is pending
+        // like a sampled token (backend/llm_sched.go:994-1003)
+        UnitRec &u = units_.at(p.unit);
+        JobRec &j = jobs_.at(u.job);
+        Slot &sl = slots_[p.slot];
+        u.on_device = false;
+        if (ok && (!toks || toks->empty())) throw Error("llm: a finished round names its tokens");
+        if (!ok) {
+            wipe(sl, p.slot);
+        } else {
+            sl.held.push_back(p.ids[0]);
+            sl.held.insert(sl.held.end(), toks->begin(), toks->end() - 1);
+            counts_.rounds++;
+            counts_.round_tokens += static_cast<int>(toks->size());
+            u.st.toks = *toks;
+        }
+        last_step_ms_ = now_ms;
+        u.st.busy_ms += took_ms;
+        j.served_ms += took_ms;
+        u.at = u.ids.size(), u.st.left = 0;
+        u.st.done = true, u.st.failed = !ok, u.st.err = ok ? std::string() : err;
+        drop_pending(p.unit);
+        return;
+    }
     if (p.kind == SchedPass::kSteps) {
         // each row had the whole pass's latency and a share of its cost (backend/llm_sched.go:845-870)
         const size_t rows = p.units.size();
@@ -351,7 +426,7 @@ void Sched::Finish(const SchedPass &p, double took_ms, bool ok, double now_ms, c
             Slot &sl = slots_[j.slot];
             if (!ok) {
                 // which rows' states moved is not something this can say
-                sl.held.clear(), sl.ckpt_len = 0, sl.ckpt_keys.clear(), ckpts_[j.slot].reset();
+                wipe(sl, j.slot);
             } else {
                 sl.held.push_back(u.ids[u.at]);
                 if (vocab) u.st.logits.assign(logits->begin() + i * vocab, logits->begin() + (i + 1) * vocab);
@@ -371,7 +446,7 @@ void Sched::Finish(const SchedPass &p, double took_ms, bool ok, double now_ms, c
     u.on_device = false;
     if (!ok) {
         // whatever the slot held is no longer something this can describe (backend/llm_sched.go:714-717)
-        sl.held.clear(), sl.ckpt_len = 0, sl.ckpt_keys.clear(), ckpts_[p.slot].reset();
+        wipe(sl, p.slot);
     } else if (p.fresh) {
         sl.held = p.ids;
     } else if (p.restore) {
@@ -382,9 +457,16 @@ void Sched::Finish(const SchedPass &p, double took_ms, bool ok, double now_ms, c
     } else {
         sl.held.insert(sl.held.end(), p.ids.begin(), p.ids.end());
     }
+    if (ok) {
+        // a priming chunk leaves the draft caught up; a plain step is owed to a draft that was; any
+        // other pass leaves the draft behind for good (backend/llm_sched.go:664-690,707-709)
+        sl.track = p.prime || (p.step && p.tracked);
+    }
     if (ok && p.take) {
         sl.ckpt_len = static_cast<int>(sl.held.size());
         sl.ckpt_keys = sl.held;
+        sl.ckpt_primed = p.prime;
+        if (!p.prime) sl.ckpt_res.clear();
     }
     if (p.step) last_step_ms_ = now_ms;
     u.st.busy_ms += took_ms;
@@ -403,24 +485,60 @@ SchedPass Sched::Pump() {
     SchedPass p = Next(clock_ms());
     if (p.kind == SchedPass::kNone) return p;
     std::vector<float> logits;
+    std::vector<int32_t> toks;
     std::string err;
     bool ok = true;
+    const size_t E = g_->GetModel().config().NEmbd;
     const double t0 = clock_ms();
     try {
-        if (g_->Speculating()) g_->Speculate(false);
-        if (p.kind == SchedPass::kSteps) {
+        if (p.kind == SchedPass::kRound) {
+            // backend/llm_sched.go:957-992
+            Speculator &sp = *specs_.at(p.slot);
+            g_->UseSlot(p.slot);
+            if (!g_->Speculating()) g_->Speculate(true);
+            g_->SpeculateFirst(true);
+            try {
+                toks = sp.RoundFrom(p.ids[0], {}, p.room);
+            } catch (const std::exception &) {
+                // a pass may be left in flight, which would refuse every later UseSlot; the slot's
+                // sequence is lost either way
+                try {
+                    if (g_->InFlight()) g_->Commit();
+                    g_->Reset();
+                } catch (const std::exception &) {
+                }
+                throw;
+            }
+        } else if (p.kind == SchedPass::kSteps) {
+            if (g_->Speculating()) g_->Speculate(false);
             g_->DecodeRows(p.slots, p.ids, &logits);
+            // each row a slot's draft did not see: owed to it (backend/llm_sched.go:834-840)
+            for (size_t i = 0; i < p.slots.size(); i++)
+                if (!specs_.empty() && slots_[p.slots[i]].track) specs_[p.slots[i]]->Owe(p.ids[i], g_->ResPort() + i * E);
         } else {
+            Speculator *sp = specs_.empty() ? nullptr : specs_[p.slot].get();
+            if (g_->Speculating()) g_->Speculate(false);
             g_->UseSlot(p.slot);
             if (p.restore) {
                 if (!ckpts_[p.slot]) throw Error("llm: slot " + std::to_string(p.slot) + " has no checkpoint to restore");
                 g_->Restore(*ckpts_[p.slot]);
+                if (sp && p.tracked) sp->Rewind(ckpts_[p.slot]->past, slots_[p.slot].ckpt_res);
             }
-            if (p.fresh) g_->Reset();
             // only the unit's last chunk's logits are anyone's: the ones between are not read back
             const UnitRec &u = units_.at(p.unit);
             const bool last = u.at + p.n == u.ids.size();
-            g_->Extend(p.ids, last ? &logits : nullptr, nullptr);
+            const bool prime = sp && p.prime;
+            if (prime && !p.fresh) sp->Settle();  // a continuation primes from where the draft is, once its owed rows are written
+            if (p.fresh) g_->Reset();
+            if (prime) {
+                const float *res = g_->ExtendResidual(p.ids, last ? &logits : nullptr);
+                sp->Prime(p.ids, p.pos, res);
+            } else {
+                g_->Extend(p.ids, last ? &logits : nullptr, nullptr);
+                // a plain step the draft did not see: owed to it
+                if (sp && p.step && p.tracked) sp->Owe(p.ids[0], g_->ResPort());
+            }
+            if (p.take && prime) slots_[p.slot].ckpt_res = sp->Residual();
             if (p.take) {
                 // a checkpoint that cannot be taken costs the next request its prefix, not this one its answer
                 try {
@@ -429,6 +547,7 @@ SchedPass Sched::Pump() {
                 } catch (const std::exception &) {
                     ckpts_[p.slot].reset();
                     slots_[p.slot].ckpt_len = 0, slots_[p.slot].ckpt_keys.clear();
+                    slots_[p.slot].ckpt_primed = false, slots_[p.slot].ckpt_res.clear();
                     p.take = false;
                 }
             }
@@ -438,7 +557,7 @@ SchedPass Sched::Pump() {
         err = e.what();
     }
     const double t1 = clock_ms();
-    Finish(p, t1 - t0, ok, t1, &logits, err);
+    Finish(p, t1 - t0, ok, t1, &logits, err, &toks);
     return p;
 }
 

@@ -118,14 +118,17 @@ typedef struct shvllm_sched shvllm_sched;
 typedef struct shvllm_sched_opts {
     int32_t batch, preempt_chunk, reserve, no_batch_decode;
     double coalesce_ms;
+    int32_t spec_depth;  /* tokens a speculative round drafts (needs shvllm_mtp_stage and a graph staged for rewindable
+                            passes of spec_depth + 1 rows); 0: decode by plain steps only */
 } shvllm_sched_opts;
 #define SHVLLM_SCHED_MAX_ROWS 64
 typedef struct shvllm_sched_pass {
-    int32_t kind;      /* 0 nothing, 1 one chunk of one unit, 2 a batched decode pass */
+    int32_t kind;      /* 0 nothing, 1 one chunk of one unit, 2 a batched decode pass, 3 a speculative round of `unit` on `slot` */
     int32_t unit, slot, pos, n, fresh, restore, take, step; /* kind 1 */
     int32_t n_units;   /* kind 2 */
     int32_t units[SHVLLM_SCHED_MAX_ROWS], slots[SHVLLM_SCHED_MAX_ROWS];
     double wait_ms;    /* kind 0: > 0 while a batch waits for conversations still sampling */
+    int32_t prime, tracked; /* kind 1 with spec_depth: the chunk primes the slot's draft; the draft was caught up when handed out */
 } shvllm_sched_pass;
 typedef struct shvllm_sched_job {
     int32_t cls, slot, reused, restored, stepping;
@@ -140,16 +143,26 @@ int shvllm_sched_release(shvllm_sched *s, int job, double now_ms);
 int shvllm_sched_job_info(shvllm_sched *s, int job, shvllm_sched_job *out);
 int shvllm_sched_run(shvllm_sched *s, int job, const int32_t *ids, int n, int fresh, int *unit);
 int shvllm_sched_step(shvllm_sched *s, int job, int32_t id, int *unit);
+/* a decode step that may run as a speculative round (backend/llm_sched.go:455-464): the unit ends with the round's
+ * tokens (shvllm_sched_unit_tokens; the last is pending like a sampled one) or, run as a plain step, with logits.
+ * room: tokens the request may still take.  Rounds name tokens by arg-max. */
+int shvllm_sched_decode(shvllm_sched *s, int job, int32_t id, int room, int *unit);
 int shvllm_sched_withdraw(shvllm_sched *s, int unit);
 int shvllm_sched_next(shvllm_sched *s, double now_ms, shvllm_sched_pass *out);
 int shvllm_sched_finish(shvllm_sched *s, double took_ms, int ok, double now_ms);  /* books the pass shvllm_sched_next handed out last */
+/* the same for a round (kind 3) the caller ran itself: the tokens it drew */
+int shvllm_sched_finish_round(shvllm_sched *s, double took_ms, int ok, double now_ms, const int32_t *toks, int n);
 int shvllm_sched_pump(shvllm_sched *s, shvllm_sched_pass *out);
 /* state: 0 queued, 1 done, 2 failed; logits [vocab] when done and given; left: ids not yet run */
 int shvllm_sched_unit(shvllm_sched *s, int unit, int *state, int *left, double *busy_ms, float *logits, int max);
+int shvllm_sched_unit_tokens(shvllm_sched *s, int unit, int32_t *dst, int max, int *n);  /* a round's tokens; n 0 for a unit that ran as a step */
 int shvllm_sched_forget(shvllm_sched *s, int unit);
 /* counts: restores, batched passes, rows in them, passes, jobs waiting for a slot, units queued */
 int shvllm_sched_counts(shvllm_sched *s, int32_t counts[6]);
 int shvllm_sched_held(shvllm_sched *s, int slot, int32_t *dst, int max, int *n, int *ckpt_len);
+/* counts: speculative rounds, tokens they drew; tracked: whether the slot's draft covers what the slot holds */
+int shvllm_sched_round_counts(shvllm_sched *s, int32_t counts[2]);
+int shvllm_sched_tracked(shvllm_sched *s, int slot, int *tracked);
 
 /* ---- the host sampler (llm.Sampler, llm/sample.go): penalties -> top_k -> top_p -> min_p -> temp -> draw,
  * and speculative sampling's Verify.  No device involved; rows are host floats and come back unchanged. ---- */

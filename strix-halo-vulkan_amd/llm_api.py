@@ -41,13 +41,14 @@ INTERACTIVE, BACKGROUND = 0, 1  # backend/llm_sched.go:77-80
 
 class SchedOpts(C.Structure):
     _fields_ = [("batch", C.c_int32), ("preempt_chunk", C.c_int32), ("reserve", C.c_int32), ("no_batch_decode", C.c_int32),
-                ("coalesce_ms", C.c_double)]
+                ("coalesce_ms", C.c_double), ("spec_depth", C.c_int32)]
 
 
 class SchedPass(C.Structure):
     _fields_ = [("kind", C.c_int32), ("unit", C.c_int32), ("slot", C.c_int32), ("pos", C.c_int32), ("n", C.c_int32),
                 ("fresh", C.c_int32), ("restore", C.c_int32), ("take", C.c_int32), ("step", C.c_int32), ("n_units", C.c_int32),
-                ("units", C.c_int32 * SCHED_MAX_ROWS), ("slots", C.c_int32 * SCHED_MAX_ROWS), ("wait_ms", C.c_double)]
+                ("units", C.c_int32 * SCHED_MAX_ROWS), ("slots", C.c_int32 * SCHED_MAX_ROWS), ("wait_ms", C.c_double),
+                ("prime", C.c_int32), ("tracked", C.c_int32)]
 
 
 class SchedJob(C.Structure):
@@ -142,6 +143,11 @@ def load():
     L.shvllm_sched_forget.argtypes = [vp, C.c_int]
     L.shvllm_sched_counts.argtypes = [vp, i32p]
     L.shvllm_sched_held.argtypes = [vp, C.c_int, i32p, C.c_int, ip, ip]
+    L.shvllm_sched_decode.argtypes = [vp, C.c_int, C.c_int32, C.c_int, ip]
+    L.shvllm_sched_unit_tokens.argtypes = [vp, C.c_int, i32p, C.c_int, ip]
+    L.shvllm_sched_finish_round.argtypes = [vp, C.c_double, C.c_int, C.c_double, i32p, C.c_int]
+    L.shvllm_sched_round_counts.argtypes = [vp, i32p]
+    L.shvllm_sched_tracked.argtypes = [vp, C.c_int, ip]
     _lib = L
     return L
 
@@ -433,10 +439,13 @@ class Sched:
     alone over `slots` slots: next() says which pass would run and finish() books a duration the
     caller names, with no device involved."""
 
-    def __init__(self, llm=None, slots=1, batch=2048, preempt_chunk=0, reserve=1, no_batch_decode=False, coalesce_ms=5.0):
+    def __init__(self, llm=None, slots=1, batch=2048, preempt_chunk=0, reserve=1, no_batch_decode=False, coalesce_ms=5.0,
+                 spec_depth=0):
+        """spec_depth > 0: decode() units may run as speculative rounds (the model needs mtp_stage() first and a
+        configuration with speculative=1, spec_rows >= spec_depth + 1)."""
         self.L = load()
         self.llm = llm
-        o = SchedOpts(batch, preempt_chunk, reserve, int(no_batch_decode), coalesce_ms)
+        o = SchedOpts(batch, preempt_chunk, reserve, int(no_batch_decode), coalesce_ms, spec_depth)
         s = C.c_void_p()
         _check(self.L.shvllm_sched_open(llm.h if llm is not None else None, slots, C.byref(o), C.byref(s)))
         self.s = s
@@ -470,6 +479,33 @@ class Sched:
         u = C.c_int()
         _check(self.L.shvllm_sched_step(self.s, job, int(tok), C.byref(u)))
         return u.value
+
+    def decode(self, job, tok, room):
+        """A decode step that may run as a speculative round (Sched::Decode)."""
+        u = C.c_int()
+        _check(self.L.shvllm_sched_decode(self.s, job, int(tok), int(room), C.byref(u)))
+        return u.value
+
+    def unit_tokens(self, unit, max_ids=16):
+        """The tokens a round drew for `unit`; empty for a unit that ran as a plain step."""
+        dst = np.empty(max_ids, np.int32)
+        n = C.c_int()
+        _check(self.L.shvllm_sched_unit_tokens(self.s, unit, dst.ctypes.data_as(C.POINTER(C.c_int32)), max_ids, C.byref(n)))
+        return dst[:min(n.value, max_ids)].copy()
+
+    def finish_round(self, took_ms, toks, ok=True, now_ms=0.0):
+        toks = np.ascontiguousarray(toks, dtype=np.int32)
+        _check(self.L.shvllm_sched_finish_round(self.s, took_ms, int(ok), now_ms, toks.ctypes.data_as(C.POINTER(C.c_int32)), len(toks)))
+
+    def round_counts(self):
+        c = np.zeros(2, np.int32)
+        _check(self.L.shvllm_sched_round_counts(self.s, c.ctypes.data_as(C.POINTER(C.c_int32))))
+        return dict(rounds=int(c[0]), round_tokens=int(c[1]))
+
+    def tracked(self, slot):
+        t = C.c_int()
+        _check(self.L.shvllm_sched_tracked(self.s, slot, C.byref(t)))
+        return bool(t.value)
 
     def withdraw(self, unit):
         _check(self.L.shvllm_sched_withdraw(self.s, unit))

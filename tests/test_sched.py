@@ -347,3 +347,86 @@ def test_bad_arguments_are_refused(sched):
         s.finish(1.0)  # no pass is out
     with pytest.raises(shv.pkg.hip_api.ShvError):
         api.Sched(None, slots=0)
+
+
+ROUND = 3
+
+
+def test_a_decode_runs_as_a_round_only_while_its_draft_is_caught_up_and_it_decodes_alone(sched):
+    # backend/llm_sched.go:936-953: asked to, draft caught up, room for two tokens, no other conversation of its class decoding
+    s = sched(slots=2, reserve=0, spec_depth=2)
+    a = s.acquire(I, ids(8))
+    p = prefill_plans = None
+    u = s.run(a, ids(8), True)
+    p = s.next()
+    assert p.kind == CHUNK and p.prime and not p.tracked   # a fresh text chunk primes the slot's draft
+    s.finish(1.0)
+    assert s.tracked(0)
+    # a plain step() never speculates; a decode() with room for one token does not either
+    u1 = s.step(a, 1)
+    p = s.next()
+    assert p.kind == CHUNK and p.step and p.tracked and not p.prime   # owed to the draft, which stays caught up
+    s.finish(1.0)
+    assert s.tracked(0)
+    u2 = s.decode(a, 2, room=1)
+    assert s.next().kind == CHUNK
+    s.finish(1.0)
+    # room for two: a round; it keeps its input and all but the last token it drew
+    u3 = s.decode(a, 3, room=8)
+    p = s.next()
+    assert p.kind == ROUND and p.unit == u3 and p.slot == 0 and p.pos == 10
+    s.finish_round(2.0, [40, 41, 42])
+    assert s.unit(u3)[0] == 1 and s.unit_tokens(u3).tolist() == [40, 41, 42]
+    assert s.held(0)[0].tolist() == list(range(8)) + [1, 2, 3, 40, 41]
+    assert s.round_counts() == dict(rounds=1, round_tokens=3)
+    # a second conversation of the class starts decoding: both go as plain rows of one pass instead
+    b = s.acquire(I, ids(8, 100))
+    prefill(s, b, ids(8, 100))
+    ub, ua = s.decode(b, 7, room=8), s.decode(a, 42, room=8)
+    p = s.next()
+    assert p.kind == STEPS and p.n_units == 2
+    s.finish(1.0)
+    assert s.unit_tokens(ua).size == 0 and s.tracked(0) and s.tracked(1)
+    # alone again once the other is released
+    s.release(b)
+    ua = s.decode(a, 50, room=8)
+    assert s.next().kind == ROUND
+    s.finish_round(2.0, [60])
+    assert s.held(0)[0].tolist()[-2:] == [42, 50]
+
+
+def test_a_failed_round_costs_the_slot_its_sequence(sched):
+    s = sched(slots=1, reserve=0, spec_depth=1)
+    a = s.acquire(I, ids(8))
+    prefill(s, a, ids(8))
+    u = s.decode(a, 1, room=4)
+    assert s.next().kind == ROUND
+    s.finish_round(1.0, [], ok=False)
+    assert s.unit(u)[0] == 2 and s.held(0)[0].size == 0 and not s.tracked(0)
+
+
+def test_a_checkpoint_keeps_the_draft_only_when_a_priming_chunk_took_it(sched):
+    # backend/llm_sched.go:625-637,696-703: a restore keeps the draft's cells below the mark when the checkpoint holds the
+    # residual to resume from, which a chunk that primed the draft leaves; otherwise the draft is behind for good
+    s = sched(slots=1, reserve=0, spec_depth=2)
+    sysp = ids(50)
+    a = s.acquire(I, np.concatenate([sysp, ids(10, 100)]), mark=50)
+    plans = prefill(s, a, np.concatenate([sysp, ids(10, 100)]))
+    assert plans[0][:2] == (0, 50) and plans[0][4]
+    assert s.tracked(0)
+    s.release(a)
+    b = s.acquire(I, np.concatenate([sysp, ids(12, 200)]), mark=50)
+    assert s.job(b).restored and s.job(b).reused == 50
+    u = s.run(b, ids(12, 200), False)
+    p = s.next()
+    assert p.kind == CHUNK and p.restore and p.tracked and p.prime
+    s.finish(1.0)
+    assert s.tracked(0)
+    s.release(b)
+    # without a draft (spec_depth 0) nothing primes and no decode is a round
+    t = sched(slots=1, reserve=0)
+    c = t.acquire(I, ids(8))
+    prefill(t, c, ids(8))
+    assert not t.tracked(0)
+    t.decode(c, 1, room=8)
+    assert t.next().kind == CHUNK

@@ -181,3 +181,101 @@ def test_checkpoint_is_the_system_prompt(rig):
             assert np.array_equal(a, b)  # the same chunks over the same bytes
     finally:
         s.close()
+
+
+# ---- speculative rounds under the scheduler (TestLLMSpeculationIsPlain, backend/llm_spec_test.go:36) ----
+
+@pytest.fixture(scope="module")
+def spec_rig():
+    cfg = LA.Config(n_layer=4, n_expert=16, n_expert_used=4, vocab=4096, nkv=512, max_tokens=64, slots=2,
+                    head_rows=3, speculative=1, spec_rows=3, nextn=1)
+    m = LA.LLM(cfg)
+    m.init_synthetic(1357)
+    m.stage()
+    m.mtp_stage(max_tok=4)
+    yield m, cfg
+    m.close()
+
+
+class SpecConv(Conv):
+    """A greedy request that decodes through decode(): a unit ends with a round's tokens or with a step's logits."""
+
+    def poll(self, passes):
+        if self.done:
+            return False
+        if self.born is None:
+            self.born = passes
+        if self.unit is None:
+            j = self.s.job(self.job)
+            if j.slot < 0:
+                return True
+            self.reused, self.restored = j.reused, bool(j.restored)
+            self.unit = self.s.run(self.job, self.prompt[j.reused:], j.reused == 0)
+            return True
+        st, _, _, lg = self.s.unit(self.unit, want_logits=True)
+        if st == 0:
+            return True
+        assert st == 1, self.s.error
+        drew = self.s.unit_tokens(self.unit)
+        self.s.forget(self.unit)
+        if drew.size:
+            assert drew.size <= self.n - len(self.toks), "a round kept more tokens than the request had room for"
+            self.toks += [int(t) for t in drew]
+            self.logits += [None] * drew.size
+        else:
+            self.logits.append(lg)
+            self.toks.append(int(np.argmax(lg)))
+        if len(self.toks) >= self.n:
+            self.s.release(self.job)
+            self.done = True
+            return False
+        self.unit = self.s.decode(self.job, self.toks[-1], self.n - len(self.toks))
+        return True
+
+
+def test_speculation_is_plain(spec_rig):
+    """A scheduler with the draft head emits exactly what one without it emits: a single request, a second turn
+    that continues the first, two conversations at once and then one of them alone (its draft owes the batched
+    rows), and a request restored from a checkpoint; and it speculated to do it."""
+    m, cfg = spec_rig
+    rng = np.random.default_rng(11)
+    P = lambda k: rng.integers(0, cfg.vocab, size=k).astype(np.int32)
+    p_one, p_turn, p_a, p_b = P(20), P(14), P(9), P(17)
+    more, sysp, ask1, ask2 = P(6), P(50), P(7), P(9)
+
+    def scenarios(s, mk):
+        out = {}
+        out["greedy"] = [drive(s, [mk(s, I, p_one, 24)])[0].toks]
+        first = drive(s, [mk(s, I, p_turn, 12)])[0]
+        second = drive(s, [mk(s, I, np.concatenate([p_turn, np.asarray(first.toks, np.int32), more]), 12)])[0]
+        out["two turns"] = [first.toks, second.toks]
+        out["reused"] = second.reused
+        both = drive(s, [mk(s, I, p_a, 10), mk(s, I, p_b, 30)])
+        again = drive(s, [mk(s, I, np.concatenate([p_b, np.asarray(both[1].toks, np.int32), more]), 10)])[0]
+        out["concurrent, then alone"] = [both[0].toks, both[1].toks, again.toks]
+        a = drive(s, [mk(s, I, np.concatenate([sysp, ask1]), 10, 50)])[0]
+        b = drive(s, [mk(s, I, np.concatenate([sysp, ask2]), 10, 50)])[0]
+        out["checkpoint restored"] = [a.toks, b.toks]
+        out["restored"] = b.restored
+        return out
+
+    s = LA.Sched(m, reserve=0)
+    try:
+        want = scenarios(s, Conv)
+        assert s.counts()["batches"] > 0
+    finally:
+        s.close()
+    s = LA.Sched(m, reserve=0, spec_depth=2)
+    try:
+        got = scenarios(s, SpecConv)
+        rc, c = s.round_counts(), s.counts()
+    finally:
+        s.close()
+    assert rc["rounds"] > 0, "no speculative round ran"
+    assert c["batches"] > 0 and c["restores"] > 0 and got["restored"] and want["restored"]
+    assert got["reused"] > 0 and want["reused"] > 0, "the second turn did not continue the first"
+    for name in ("greedy", "two turns", "concurrent, then alone", "checkpoint restored"):
+        for k, (g, w) in enumerate(zip(got[name], want[name])):
+            assert len(g) == len(w) and len(w) > 0
+            assert g == w, (name, k, g, w)
+    print("speculative rounds %d, %.2f tokens a round, %d batched passes" % (rc["rounds"], rc["round_tokens"] / rc["rounds"], c["batches"]))
