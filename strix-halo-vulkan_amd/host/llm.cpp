@@ -1886,6 +1886,18 @@ void Speculator::UseSampler(Sampler *s, int64_t draft_seed) {
     draft_sampler_ = s->DraftSampler(draft_seed);
 }
 
+void Speculator::SetSampler(Sampler *s, bool exact, int64_t draft_seed) {
+    if (!s || s->Greedy()) {
+        sampler_ = nullptr, exact_ = false;
+        draft_sampler_.reset();
+        return;
+    }
+    // a request keeps its draft sampler from round to round
+    if (!exact && (s != sampler_ || exact_ || !draft_sampler_)) draft_sampler_ = s->DraftSampler(draft_seed);
+    if (exact) draft_sampler_.reset();
+    sampler_ = s, exact_ = exact;
+}
+
 // A round under a sampler (llm/spec.go:703-857 with llm/sample.go:183-250).  The passes are the
 // greedy round's; what differs is who names the tokens: each draft is a draw from the draft
 // sampler's distribution over the draft head's logits, each verified row goes through Verify.
@@ -1901,14 +1913,16 @@ std::vector<int32_t> Speculator::sampled_round(const std::vector<int32_t> &force
     std::vector<Dist> q(Depth);
     std::vector<bool> drawn(Depth, false);
     std::vector<float> ql;
-    d_.Rows(h_, xs, at - owed, true);
+    int32_t dtok = d_.Rows(h_, xs, at - owed, true);
     for (int k = 0; k < Depth; k++) {
         if (k > 0) {
             std::vector<int32_t> one{rows[k]};
-            d_.Rows(d_.ResPort() + (k == 1 ? static_cast<size_t>(owed) * E : 0), one, at + k, true);
+            dtok = d_.Rows(d_.ResPort() + (k == 1 ? static_cast<size_t>(owed) * E : 0), one, at + k, true);
         }
         if (k < static_cast<int>(forced.size())) {
             rows.push_back(forced[k]);  // not a draw from q: verified as a plain sample
+        } else if (exact_) {
+            rows.push_back(dtok);       // the draft head's arg-max: likewise
         } else {
             d_.LastLogits(&ql);
             rows.push_back(draft_sampler_->Propose(ql.data(), static_cast<int>(ql.size()), &q[k]));

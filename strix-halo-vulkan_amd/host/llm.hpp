@@ -558,6 +558,12 @@ public:
     // s == nullptr or a greedy sampler: back to arg-max.  The sampler is borrowed; the draft's is made
     // from it (Sampler::DraftSampler) with its own seed.  Takes effect at the next Start.
     void UseSampler(Sampler *s, int64_t draft_seed);
+    // The sampler of the rounds from here on, for a caller that serves several requests (nullptr or a
+    // greedy one: arg-max).  exact: the drafts are the draft head's arg-max and every verified row
+    // is ONE plain draw of s, kept while it equals the draft after it, so a seeded request consumes
+    // its random stream exactly as a loop of plain steps does (backend/llm_spec_test.go:24-31);
+    // otherwise the drafts are drawn and verified by speculative sampling, as UseSampler arranges.
+    void SetSampler(Sampler *s, bool exact, int64_t draft_seed);
     void Stop() { g_.Speculate(false); }
     // ---- the served loop's pieces (llm/spec.go:285-456) ----
     // Prime writes the draft's cells at positions at .. at+n-1 from a chunk the trunk has just run:
@@ -592,6 +598,7 @@ private:
     int past() const { return slot_ >= 0 ? g_.PastOf(slot_) : g_.Past(); }
     void settle_owed();
     Sampler *sampler_ = nullptr;
+    bool exact_ = false;
     std::unique_ptr<Sampler> draft_sampler_;
     std::vector<int32_t> sampled_round(const std::vector<int32_t> &forced, int limit);
 };

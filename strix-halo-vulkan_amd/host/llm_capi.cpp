@@ -8,6 +8,7 @@
 #include <memory>
 
 #include "llm.hpp"
+#include "sampler_handle.hpp"
 #include "sched.hpp"
 
 struct shvllm {
@@ -544,6 +545,13 @@ int shvllm_sched_decode(shvllm_sched *s, int job, int32_t id, int room, int *uni
     return guard([&] {
         if (!unit) throw llm::Error("llm: shvllm_sched_decode: NULL argument");
         *unit = sched_of(s).Decode(job, id, room);
+    });
+}
+
+int shvllm_sched_decode_sampled(shvllm_sched *s, int job, int32_t id, int room, shvsampler *sampler, int exact, int64_t draft_seed, int *unit) {
+    return guard([&] {
+        if (!unit) throw llm::Error("llm: shvllm_sched_decode_sampled: NULL argument");
+        *unit = sched_of(s).Decode(job, id, room, sampler ? &sampler->s : nullptr, exact != 0, draft_seed);
     });
 }
 

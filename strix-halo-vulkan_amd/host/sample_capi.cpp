@@ -2,15 +2,8 @@
 #include <algorithm>
 #include <cstring>
 
-#include "sample.hpp"
+#include "sampler_handle.hpp"
 #include "shv_llm.h"
-
-struct shvsampler {
-    llm::Sampler s;
-    llm::Dist last;  // the distribution of the last propose
-    bool has_last = false;
-    shvsampler(float t, int k, float p, int64_t seed) : s(t, k, p, seed) {}
-};
 
 static int copy_dist(const llm::Dist &d, int32_t *ids, float *p, int max) {
     const int n = static_cast<int>(std::min<size_t>(d.IDs.size(), max < 0 ? 0 : max));

@@ -216,11 +216,12 @@ int Sched::Step(int job, int32_t tok) {
     return id;
 }
 
-int Sched::Decode(int job, int32_t tok, int room) {
+int Sched::Decode(int job, int32_t tok, int room, Sampler *sampler, bool exact, int64_t draft_seed) {
     const int id = Step(job, tok);
     UnitRec &u = units_.at(id);
     u.round = spec_on_;
     u.room = room;
+    u.sampler = sampler, u.exact = exact, u.draft_seed = draft_seed;
     return id;
 }
 
@@ -498,6 +499,8 @@ SchedPass Sched::Pump() {
             if (!g_->Speculating()) g_->Speculate(true);
             g_->SpeculateFirst(true);
             try {
+                const UnitRec &u = units_.at(p.unit);
+                sp.SetSampler(u.sampler, u.exact, u.draft_seed);
                 toks = sp.RoundFrom(p.ids[0], {}, p.room);
             } catch (const std::exception &) {
                 // a pass may be left in flight, which would refuse every later UseSlot; the slot's

@@ -15,7 +15,7 @@
 // asked for it runs as a speculative round while no other conversation of its class is decoding
 // (two decoding together batch as plain rows instead), a text prefill chunk primes the slot's draft,
 // plain and batched steps are owed to it, and a checkpoint keeps the residual the draft resumes from.
-// Rounds here name their tokens by arg-max; a request that samples decodes by plain steps.
+// A round names its tokens by arg-max or, handed the request's sampler, by that sampler.
 //
 // The reference runs this as a goroutine that blocks on a condition variable.  Here the policy
 // is a plain state machine with no thread and no clock of its own: Next() says what the device
@@ -35,6 +35,7 @@ namespace llm {
 class Graph;
 class MTPHead;
 class Speculator;
+class Sampler;
 struct Checkpoint;
 
 enum SchedClass { kInteractive = 0, kBackground = 1 };  // backend/llm_sched.go:77-80
@@ -107,7 +108,9 @@ public:
     // ends either with the tokens a round drew (Unit().toks, the last of them pending like a
     // sampled one) or, when it ran as a plain step, with that step's logits.  room: how many
     // tokens the request may still take.
-    int Decode(int job, int32_t id, int room);
+    // sampler: the request's own (borrowed until the unit is done), which then names the round's
+    // tokens; exact as Speculator::SetSampler has it (a seeded request).
+    int Decode(int job, int32_t id, int room, Sampler *sampler = nullptr, bool exact = false, int64_t draft_seed = 1);
     // Withdraw takes a unit that is not on the device out of the queue (:483-495).
     void Withdraw(int unit);
 
@@ -165,8 +168,10 @@ private:
         std::vector<int32_t> ids;
         size_t at = 0;  // ids[at..] are still to run
         bool fresh = false, restore = false, step = false, on_device = false;
-        bool round = false;
+        bool round = false, exact = false;
         int room = 0;
+        Sampler *sampler = nullptr;
+        int64_t draft_seed = 1;
         UnitState st;
     };
     int reuse(const Slot &sl, const std::vector<int32_t> &prompt, bool *restore) const;

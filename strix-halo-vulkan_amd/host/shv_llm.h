@@ -145,8 +145,14 @@ int shvllm_sched_run(shvllm_sched *s, int job, const int32_t *ids, int n, int fr
 int shvllm_sched_step(shvllm_sched *s, int job, int32_t id, int *unit);
 /* a decode step that may run as a speculative round (backend/llm_sched.go:455-464): the unit ends with the round's
  * tokens (shvllm_sched_unit_tokens; the last is pending like a sampled one) or, run as a plain step, with logits.
- * room: tokens the request may still take.  Rounds name tokens by arg-max. */
+ * room: tokens the request may still take.  The round names its tokens by arg-max. */
 int shvllm_sched_decode(shvllm_sched *s, int job, int32_t id, int room, int *unit);
+/* the same with the request's sampler (borrowed until the unit is done), which names the round's tokens and takes
+ * them into its window itself: exact != 0 for a seeded request (every verified row is one plain draw, so the random
+ * stream is consumed as plain steps consume it), else the drafts are drawn with a sampler seeded by draft_seed and
+ * verified by speculative sampling.  A unit that ran as a plain step returns logits as ever. */
+struct shvsampler;
+int shvllm_sched_decode_sampled(shvllm_sched *s, int job, int32_t id, int room, struct shvsampler *sampler, int exact, int64_t draft_seed, int *unit);
 int shvllm_sched_withdraw(shvllm_sched *s, int unit);
 int shvllm_sched_next(shvllm_sched *s, double now_ms, shvllm_sched_pass *out);
 int shvllm_sched_finish(shvllm_sched *s, double took_ms, int ok, double now_ms);  /* books the pass shvllm_sched_next handed out last */

@@ -144,6 +144,7 @@ def load():
     L.shvllm_sched_counts.argtypes = [vp, i32p]
     L.shvllm_sched_held.argtypes = [vp, C.c_int, i32p, C.c_int, ip, ip]
     L.shvllm_sched_decode.argtypes = [vp, C.c_int, C.c_int32, C.c_int, ip]
+    L.shvllm_sched_decode_sampled.argtypes = [vp, C.c_int, C.c_int32, C.c_int, vp, C.c_int, C.c_int64, ip]
     L.shvllm_sched_unit_tokens.argtypes = [vp, C.c_int, i32p, C.c_int, ip]
     L.shvllm_sched_finish_round.argtypes = [vp, C.c_double, C.c_int, C.c_double, i32p, C.c_int]
     L.shvllm_sched_round_counts.argtypes = [vp, i32p]
@@ -480,10 +481,15 @@ class Sched:
         _check(self.L.shvllm_sched_step(self.s, job, int(tok), C.byref(u)))
         return u.value
 
-    def decode(self, job, tok, room):
-        """A decode step that may run as a speculative round (Sched::Decode)."""
+    def decode(self, job, tok, room, sampler=None, exact=False, draft_seed=1):
+        """A decode step that may run as a speculative round (Sched::Decode).  sampler: a sample_api.Sampler, which
+        then names a round's tokens and takes them into its window itself (a unit that ran as a plain step leaves
+        sampling to the caller, as ever); exact: a seeded request, every verified row one plain draw."""
         u = C.c_int()
-        _check(self.L.shvllm_sched_decode(self.s, job, int(tok), int(room), C.byref(u)))
+        if sampler is None:
+            _check(self.L.shvllm_sched_decode(self.s, job, int(tok), int(room), C.byref(u)))
+        else:
+            _check(self.L.shvllm_sched_decode_sampled(self.s, job, int(tok), int(room), sampler.h, int(exact), int(draft_seed), C.byref(u)))
         return u.value
 
     def unit_tokens(self, unit, max_ids=16):

@@ -279,3 +279,66 @@ def test_speculation_is_plain(spec_rig):
             assert len(g) == len(w) and len(w) > 0
             assert g == w, (name, k, g, w)
     print("speculative rounds %d, %.2f tokens a round, %d batched passes" % (rc["rounds"], rc["round_tokens"] / rc["rounds"], c["batches"]))
+
+
+class SampledConv:
+    """A request with its own sampler: plain steps are sampled here, rounds by the sampler inside the scheduler."""
+
+    def __init__(self, s, prompt, n, sampler, spec, exact):
+        self.s, self.n, self.sampler, self.spec, self.exact = s, n, sampler, spec, exact
+        self.prompt = np.asarray(prompt, np.int32)
+        self.job = s.acquire(I, self.prompt, 0)
+        self.unit, self.toks, self.done = None, [], False
+        sampler.accept(*[int(t) for t in self.prompt])
+
+    def poll(self, passes):
+        if self.done:
+            return False
+        if self.unit is None:
+            j = self.s.job(self.job)
+            if j.slot < 0:
+                return True
+            self.unit = self.s.run(self.job, self.prompt[j.reused:], j.reused == 0)
+            return True
+        st, _, _, lg = self.s.unit(self.unit, want_logits=True)
+        if st == 0:
+            return True
+        assert st == 1, self.s.error
+        drew = self.s.unit_tokens(self.unit)
+        self.s.forget(self.unit)
+        if drew.size:
+            self.toks += [int(t) for t in drew]   # the round's sampler has taken them into its window
+        else:
+            t = self.sampler.sample(lg)
+            self.sampler.accept(t)
+            self.toks.append(int(t))
+        if len(self.toks) >= self.n:
+            self.s.release(self.job)
+            self.done = True
+            return False
+        room = self.n - len(self.toks)
+        self.unit = self.s.decode(self.job, self.toks[-1], room, self.sampler, self.exact) if self.spec else self.s.step(self.job, self.toks[-1])
+        return True
+
+
+def test_sampled_rounds(spec_rig):
+    """A seeded request under the draft head draws what it draws by plain steps (a round spends one draw a verified
+    row, in order); an unseeded one verifies by speculative sampling, whose stream is another, so it is held to
+    running, speculating and staying inside the sampler's support."""
+    m, cfg = spec_rig
+    SA = shv.pkg.sample_api
+    prompt = np.random.default_rng(21).integers(0, cfg.vocab, size=18).astype(np.int32)
+    mk = lambda: SA.Sampler(0.8, 40, 0.95, 7, repeat_penalty=1.1)
+    out = {}
+    for name, spec, exact in (("plain", False, False), ("seeded", True, True), ("unseeded", True, False)):
+        s = LA.Sched(m, reserve=0, spec_depth=2 if spec else 0)
+        smp = mk()
+        try:
+            c = drive(s, [SampledConv(s, prompt, 32, smp, spec, exact)])[0]
+            out[name] = (c.toks, s.round_counts()["rounds"])
+        finally:
+            s.close()
+            smp.close()
+    assert out["plain"][1] == 0 and out["seeded"][1] > 0 and out["unseeded"][1] > 0
+    assert out["seeded"][0] == out["plain"][0]
+    assert len(out["unseeded"][0]) == 32 and all(0 <= t < cfg.vocab for t in out["unseeded"][0])
