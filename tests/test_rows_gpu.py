@@ -512,3 +512,50 @@ def test_chunk_size_does_not_matter_to_a_second_attention_layer():
             # halves: a cell here and there rounds the other way, none is off by more than that
             e = np.linalg.norm(x - y, axis=1) / np.linalg.norm(y, axis=1)
             assert e.max() <= 2e-3, (rows, int(e.argmax()), float(e.max()))
+
+
+def test_sequences_of_very_different_lengths_decode_together():
+    """Eight sequences of 5 to 5000 tokens advanced together for twenty steps against each of them advanced alone on
+    the same tokens, over two periods of layers (so that what a batched pass leaves an attention layer with is read by
+    the layers after it), at the full widths; then a three-row pass at 5020 cells against three steps."""
+    S, steps = 8, 20
+    cfg = LA.Config(n_layer=8, nkv=6144, max_tokens=256, head_rows=S, slots=S, vocab=32768)
+    m = LA.LLM(cfg)
+    m.init_synthetic(20260101)
+    m.stage()
+    try:
+        rng = np.random.default_rng(3)
+        lens = [5, 100, 700, 1023, 1500, 2049, 3000, 5000]
+        prompts = [rng.integers(0, cfg.vocab, size=n).astype(np.int32) for n in lens]
+
+        def prefill():
+            for s in range(S):
+                m.use_slot(s)
+                m.reset()
+                m.extend(prompts[s], want_logits=False)
+
+        prefill()
+        slots = np.arange(S, dtype=np.int32)
+        ids = rng.integers(0, cfg.vocab, size=S).astype(np.int32)
+        fed, batched = [], []
+        for _ in range(steps):
+            fed.append(ids.copy())
+            ids, lg = m.decode_rows(slots, ids, want_logits=True)
+            batched.append(lg.copy())
+        prefill()
+        for s in range(S):
+            m.use_slot(s)
+            for t in range(steps):
+                lg, _ = m.extend(np.array([fed[t][s]], np.int32))
+                assert O.rel_l2(batched[t][s], lg) <= 1e-3, (lens[s], t)
+        three = rng.integers(0, cfg.vocab, size=3).astype(np.int32)
+        m.use_slot(7)
+        _, lg3, _ = m.extend_rows(three, want_logits=True)
+        m.use_slot(6)
+        m.reset()
+        m.extend(np.concatenate([prompts[7], np.array([fed[t][7] for t in range(steps)], np.int32)]), want_logits=False)
+        for i in range(3):
+            lg, _ = m.extend(three[i:i + 1])
+            assert O.rel_l2(lg3[i], lg) <= 1e-3, i
+    finally:
+        m.close()
