@@ -956,7 +956,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_pass_kernel(shv_gemv_q4k_args a,
     const int n = lane & 15, kb = lane >> 4;
     const int sbs = a.k / SHV_Q4K_BLOCK;
     const size_t row_bytes = static_cast<size_t>(sbs) * SHV_Q4K_BYTES;
-    constexpr int NTHR = NW * 64;
     const int grp = blockIdx.x % groups, xb = blockIdx.x / groups;
     const int t0 = grp * kWideTok;
     const int nt = a.n_tok - t0 < kWideTok ? a.n_tok - t0 : kWideTok;
