@@ -922,6 +922,7 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
+    ctx->moe_stamp = {};  // only the grouped launch leaves lists or operands behind, and says so itself
     // Banks of other types than Q4_K go through their own arms; a block whose routed banks and
     // shared expert differ in that takes one launch each, over its part of the slots.
     const bool r_other = !is_q4k(a.gate_type) || !is_q4k(a.up_type), s_other = !is_q4k(a.gate_sh_type) || !is_q4k(a.up_sh_type);
@@ -984,6 +985,14 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     SHV_REQUIRE(a.n_used >= 1 && a.n_used + 1 <= 12, "moe_down: n_used %d; built for up to 11 routed experts", a.n_used);
     SHV_REQUIRE(a.n_embd >= 1 && a.out_stride >= a.n_embd && (!a.residual || a.res_stride >= a.n_embd), "moe_down: strides");
     SHV_REQUIRE(a.ffn >= 1, "moe_down: ffn %d", a.ffn);
+    // act as matrix-core operands is read by the grouped Q4_K launch alone: every other road below
+    // takes floats, so the flag and what the gate/up launch really left must agree with the road
+    {
+        const bool packed_here = ctx->moe_stamp.packed && ctx->moe_stamp.act == a.act;
+        const bool grouped_road = is_q4k(a.down_type) && is_q4k(a.down_sh_type) && shv_moe_down_grouped_covers(ctx, a);
+        SHV_REQUIRE(!a.act_packed || grouped_road, "moe_down: act_packed is set, but this call does not take the grouped Q4_K path (bank types, workspaces or %d rows)", a.n_tok);
+        SHV_REQUIRE(a.act_packed || !packed_here, "moe_down: the shv_moe_up before this call left act as matrix-core operands (its act_packed); this call reads floats");
+    }
     // as in the up projection: the Q4_K part of the slots here, the rest through the other arms,
     // which then add to what this launch has written
     const bool r_other = !is_q4k(a.down_type), s_other = !is_q4k(a.down_sh_type);

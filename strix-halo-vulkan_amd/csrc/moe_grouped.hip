@@ -867,16 +867,18 @@ bool shv_moe_down_grouped_covers(const shv_ctx *ctx, const shv_moe_down_args &a)
 
 // Lists, the rows as operands, then the grouped gate/up products.
 int shv_launch_moe_up_grouped(shv_ctx *ctx, const shv_moe_up_args &a) {
+    // refused before anything is enqueued: an error return leaves no half pass on the stream
+    SHV_REQUIRE(!a.act_packed || (ctx->gemm_part && packed_sums_bytes(static_cast<long long>(a.n_tok) * (a.n_used + 1), a.ffn) <= static_cast<size_t>(shv_ctx::kGemmPartBytes)),
+                "moe_up: %d rows are too many for act_packed", a.n_tok);
     SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, a.group);
     SHV_LAUNCH(ctx, moe_stage_kernel, dim3((a.n_embd + 1023) / 1024, a.n_tok), dim3(256), 0, a.xn, a.n_embd, a.n_embd, a.n_tok, ctx->gemm_stage);
     constexpr size_t lds = kStagedLds;
     static const int raised = raise_lds(&moe_up_grouped_kernel<2048>, lds);
     if (raised != SHV_OK) return raised;
     const int parts = a.ffn / (32 * kStWaves), tiles = (a.n_tok + kTok - 1) / kTok;
-    SHV_REQUIRE(!a.act_packed || (ctx->gemm_part && packed_sums_bytes(static_cast<long long>(a.n_tok) * (a.n_used + 1), a.ffn) <= static_cast<size_t>(shv_ctx::kGemmPartBytes)),
-                "moe_up: %d rows are too many for act_packed", a.n_tok);
     SHV_LAUNCH(ctx, moe_up_grouped_kernel<2048>, dim3(a.n_expert * parts + parts * tiles), dim3(kStThreads), lds, a, static_cast<const char *>(ctx->gemm_stage),
                reinterpret_cast<char *>(ctx->gemm_part));
+    ctx->moe_stamp = {a.topk, a.group, a.act, a.n_tok, a.n_used, true, a.act_packed != 0};
     return SHV_OK;
 }
 
@@ -887,10 +889,14 @@ int shv_launch_moe_down_grouped(shv_ctx *ctx, const shv_moe_down_args &a) {
     SHV_REQUIRE(a.n_embd % 4 == 0 && a.out_stride % 4 == 0 && shv_aligned16(a.out) &&
                     (!a.residual || (a.res_stride % 4 == 0 && shv_aligned16(a.residual))),
                 "moe_down: the grouped path moves 16 bytes at a time");
-    if (!a.group_ready) SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
+    // the lists are this pass's only if the grouped gate/up launch of this very pass made them
+    const shv_ctx::MoeStamp &st = ctx->moe_stamp;
+    const bool lists = a.group_ready && st.grouped && st.topk == a.topk && st.group == a.group && st.n_tok == a.n_tok && st.n_used == a.n_used;
+    SHV_REQUIRE(!a.act_packed || (lists && st.packed && st.act == a.act && ctx->gemm_part),
+                "moe_down: act_packed, but the shv_moe_up before this call did not leave act as operands for this pass");
+    if (!lists) SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
     const int parts = a.n_embd / 512, tiles = (a.n_tok + kTok - 1) / kTok;
     if (a.act_packed) {
-        SHV_REQUIRE(a.group_ready && ctx->gemm_part, "moe_down: act_packed needs the grouped moe_up of this pass right before (group_ready)");
         constexpr size_t lds = kStagedLds;
         static const int raised = raise_lds(&moe_down_staged_kernel<512>, lds);
         if (raised != SHV_OK) return raised;

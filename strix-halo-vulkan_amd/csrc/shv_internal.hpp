@@ -73,6 +73,15 @@ struct shv_ctx {
         return hipSuccess;
     }
     enum { kCounterRouter = 0, kCounterArgmax = 1, kCounterAttn = 16 };
+    // What the last shv_moe_up on this context left behind for the shv_moe_down that follows it:
+    // the pass its per-expert lists in `group` belong to, and whether act holds matrix-core
+    // operands instead of floats.  shv_moe_down believes its group_ready / act_packed flags only
+    // when they agree with this.
+    struct MoeStamp {
+        const void *topk = nullptr, *group = nullptr, *act = nullptr;
+        int n_tok = 0, n_used = 0;
+        bool grouped = false, packed = false;
+    } moe_stamp;
 };
 
 struct shv_prerecorded {

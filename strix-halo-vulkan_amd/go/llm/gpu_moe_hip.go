@@ -37,10 +37,11 @@ func (g *moeHIP) graph(layer int, in, out *hip.Buffer) ([]hip.Op, []string, erro
 		return nil, nil, fmt.Errorf("llm: layer %d of %d", layer, len(g.banks))
 	}
 	c := g.cfg
-	q4k := true
-	for _, t := range g.banks[layer].Types[:2] {
-		q4k = q4k && t == ggmlQ4K
-	}
+	// Types is (gate, up, down, shared gate, shared up, shared down): the gate/up launch goes its
+	// Q4_K road only when all four of its banks are Q4_K, the down launch only when both of its are
+	ty := g.banks[layer].Types
+	q4k := ty[0] == ggmlQ4K && ty[1] == ggmlQ4K && ty[3] == ggmlQ4K && ty[4] == ggmlQ4K
+	downQ4K := ty[2] == ggmlQ4K && ty[5] == ggmlQ4K
 	// a one-row pass routes in the expert kernel itself; banks of another type take the router's selection
 	fused := g.routeInUp && g.rows == 1 && q4k
 	var lg, wt, grp *hip.Buffer
@@ -50,7 +51,7 @@ func (g *moeHIP) graph(layer int, in, out *hip.Buffer) ([]hip.Op, []string, erro
 		grp = g.group
 	}
 	ready := !fused && q4k && g.group != nil
-	packed := ready && g.pairs != nil // both projections Q4_K, one right after the other: act goes over as operands
+	packed := ready && downQ4K && g.pairs != nil // both projections Q4_K, one right after the other: act goes over as operands
 	ops := []hip.Op{
 		hip.MoERouter(in, g.norm[layer], g.router[layer], g.sharedGate[layer], g.xn, g.logits, g.topk, g.weights,
 			g.rows, c.NEmbd, c.NExpert, c.NExpertUsed, c.RMSEps, fused),
