@@ -91,6 +91,7 @@ enum {
     SHV_OP_DEQUANT = 13,
     SHV_OP_GEMV = 14,
     SHV_OP_RING_ROWS = 15,
+    SHV_OP_ROUTER_FOLD = 16,
     SHV_OP__COUNT
 };
 
@@ -137,7 +138,32 @@ typedef struct {
                                 address that does not depend on the position, for a consumer that would
                                 otherwise wait for the position word before it can ask for the row (the
                                 DeltaNet output projection's gate z); NULL: not stored */
+    /* The router's logits in the same launch (one row, k = 4096, n = 2048, a residual): the
+     * projection feeds y = residual + W pro(x) to an RMSNorm and a float32 router R (llm/moe.go:
+     * 219-232), and R (gamma * y) is linear in y: it is fold[e] . [pro(x) | residual] with
+     * fold [fold_rows][k + n] = [R diag(gamma) W | R diag(gamma)] made once by shv_router_fold.
+     * fold_out[e] receives that product WITHOUT the norm's factor rsqrt(mean(y^2) + eps), which
+     * shv_moe_up applies (its gamma argument).  residual must not alias y then.  NULL: no logits. */
+    const float *fold;
+    float *fold_out;
+    int32_t fold_rows;
 } shv_gemv_q4k_args;
+
+/* The table shv_gemv_q4k's `fold` reads, for one layer: out [rows][k + n_embd] float32,
+ * rows = n_expert + (shared_gate ? 1 : 0); out[e][k + i] = R[e][i] * gamma[i] and
+ * out[e][j] = sum_i R[e][i] * gamma[i] * W[i][j] accumulated in float64, W [n_embd][k] the Q4_K
+ * output projection as dequantQ4_K expands it (gguf/dequant.go:252-276), R the router's rows with
+ * the shared gate as the last.  scratch: n_embd * k floats.  Made once when a graph is staged,
+ * as the reference makes its dense banks then (llm/bank_q4.go:172-266). */
+typedef struct {
+    const float *router;
+    const float *shared_gate;
+    const float *gamma;
+    const void *w_out;
+    float *out;
+    float *scratch;
+    int32_t n_expert, n_embd, k;
+} shv_router_fold_args;
 
 /* ggml type numbers of the tensor types the reference's loader accepts (Dequantizable,
  * gguf/dequant.go:103-110) */
@@ -252,6 +278,12 @@ typedef struct {
                                 shv_moe_down reads (two binary16 parts of every value, same bytes a row)
                                 instead of floats; the shv_moe_down of this pass must be the library's
                                 next call on the stream, with act_packed and group_ready set too */
+    const float *gamma;      /* with logits, one row: xn is the row BEFORE its RMSNorm and logits are the
+                                router's products without the norm's factor (shv_gemv_q4k's fold_out);
+                                the kernel forms the factor from the row it stages, multiplies the row
+                                by gamma and applies the factor to its own products and to the logits
+                                (llm/hc.go:176-190).  NULL: xn is normalised already */
+    float eps;
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +
@@ -451,6 +483,7 @@ int shv_embed(shv_ctx *ctx, const shv_embed_args *a);
 int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_advance(shv_ctx *ctx, const shv_advance_args *a);
 int shv_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *a);
+int shv_router_fold(shv_ctx *ctx, const shv_router_fold_args *a);
 
 /* shv_argmax for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and

@@ -251,12 +251,20 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 // STAGED (a variant kept for comparison): the lane of a super-block's first group decodes all
 // eight (d*sc, dmin*m) pairs of the header and leaves them in LDS for the four lanes of the
 // super-block, instead of every lane decoding its own group's from the header it holds anyway.
-template <int K, int WAVES, int P, int PRO, bool STAGED = false>
+// FOLD: the launch also forms the router's logits of the MoE block that follows (a.fold: rows of
+// k + n floats, [R diag(gamma) W | R diag(gamma)], against [pro(x) | residual]; see router_fold.hip).
+// Every block takes two of those rows beside its own, four waves a row and a quarter of the row a
+// wave; the residual row (n = 4 T floats) is staged behind pro(x), so y must be another buffer.
+template <int K, int WAVES, int P, int PRO, bool STAGED = false, bool FOLD = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args a) {
     constexpr int T = WAVES * 64, LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int NV = K / 4 / T;  // float4 a thread stages
     static_assert(NV >= 1 && K % (4 * T) == 0, "threads of a block each stage whole float4s");
-    __shared__ __align__(16) float xs[lds_padded(K)];
+    constexpr int FN = 4 * T;               // FOLD: the residual row's length (one float4 a thread)
+    constexpr int FQ = (K + FN) / 4;        // a wave's quarter of a fold row
+    constexpr int FV = FQ / 256;            // float4 a lane loads of it
+    static_assert(!FOLD || (WAVES == 8 && FQ % 256 == 0), "a fold row is split over four waves");
+    __shared__ __align__(16) float xs[lds_padded(FOLD ? K + FN : K)];
     __shared__ __align__(16) float xsum[K / 32];
     __shared__ float red[WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -292,6 +300,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
             zv[j] = *reinterpret_cast<const float4 *>(a.z + zi);
         }
     }
+    float4 fres = make_float4(0.f, 0.f, 0.f, 0.f);
+    if constexpr (FOLD) fres = *reinterpret_cast<const float4 *>(a.residual + 4 * tid);
     Q4kLane w[P];
     int row[P];
 #pragma unroll
@@ -303,6 +313,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
     float res[P];
 #pragma unroll
     for (int u = 0; u < P; u++) res[u] = (a.residual && row[u] >= 0 && group_sum_owner<LPR>(lane)) ? a.residual[row[u]] : 0.f;
+    // the wave's quarter of its fold row, behind the weights
+    float4 fw[FOLD ? FV : 1];
+    const int fold_row = static_cast<int>(blockIdx.x) * 2 + (wave >> 2), fold_q = wave & 3;
+    if constexpr (FOLD) {
+        const float *fr = a.fold + static_cast<size_t>(fold_row < a.fold_rows ? fold_row : 0) * (K + FN) + fold_q * FQ;
+#pragma unroll
+        for (int j = 0; j < FV; j++) fw[j] = *reinterpret_cast<const float4 *>(fr + (j * 64 + lane) * 4);
+    }
 
     // ---- stage pro(x): thread i of the block takes columns 4*(i + T*j) .. +3 ----
     float ss = 0.f;
@@ -338,6 +356,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
         ss = wave_sum_all(ss);
         if (lane == 0) red[wave] = ss;
     }
+    if constexpr (FOLD) *reinterpret_cast<float4 *>(&xs[lds_slot(K + 4 * tid)]) = fres;
     __syncthreads();
     float scale = 1.f;
     if constexpr (PRO == SHV_PRO_RMSNORM) {
@@ -380,6 +399,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
             y[row[u]] = v;
             if (a.y_flat) a.y_flat[row[u]] = v;
         }
+    }
+    if constexpr (FOLD) {
+        // the quarter row against the same columns of [pro(x) | residual]; the four quarters meet in
+        // LDS and are added in a fixed order
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < FV; j++) {
+            const float4 xv4 = *reinterpret_cast<const float4 *>(&xs[lds_slot(fold_q * FQ + (j * 64 + lane) * 4)]);
+            acc = fmaf(fw[j].x, xv4.x, fmaf(fw[j].y, xv4.y, fmaf(fw[j].z, xv4.z, fmaf(fw[j].w, xv4.w, acc))));
+        }
+        acc = wave_sum_all(acc);
+        __syncthreads();  // red is free again: every wave has its scale
+        if (lane == 0) red[wave] = acc;
+        __syncthreads();
+        if ((tid & 255) == 0 && fold_row < a.fold_rows) a.fold_out[fold_row] = (red[wave] + red[wave + 1]) + (red[wave + 2] + red[wave + 3]);
     }
 }
 
@@ -571,7 +605,19 @@ bool fewrows_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     return row_kernel_covers(ctx, one);
 }
 
+// The output projection of a decode step with the router's rows of the MoE block behind it.
+int launch_row_fold(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    constexpr int K = 4096, WAVES = 8;
+    const int rows_blocks = (a.n + WAVES - 1) / WAVES, fold_blocks = (a.fold_rows + 1) / 2;
+    const dim3 grid(static_cast<unsigned>(rows_blocks > fold_blocks ? rows_blocks : fold_blocks)), block(WAVES * 64);
+    if (a.prologue == SHV_PRO_GATED_NORM) SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, 1, SHV_PRO_GATED_NORM, false, true>), grid, block, 0, a);
+    else if (a.prologue == SHV_PRO_MUL_SIGMOID) SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, 1, SHV_PRO_MUL_SIGMOID, false, true>), grid, block, 0, a);
+    else SHV_LAUNCH(ctx, (gemv_row_kernel<K, WAVES, 1, SHV_PRO_NONE, false, true>), grid, block, 0, a);
+    return SHV_OK;
+}
+
 int launch_row(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (a.fold) return launch_row_fold(ctx, a);
     if (a.k == 4096) return launch_row_kp<4096, 8, 1>(ctx, a);
     // two rows a pass at this width: one pass a wave up to a block a compute unit's worth of
     // rows, two above that
@@ -682,6 +728,13 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
         const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
         SHV_REQUIRE((a.z_ring || (a.ring_stride >= a.n && !a.residual)) && sl <= a.ring_slots && a.n_tok % sl == 0,
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
+    }
+    if (a.fold) {
+        SHV_REQUIRE(a.n_tok == 1 && a.k == 4096 && a.n == 2048 && a.residual && a.fold_out && a.fold_rows >= 1 && (a.ring_slots == 0 || a.z_ring),
+                    "gemv_q4k: the router's rows ride on a one-row 2048 x 4096 projection with a residual (n_tok %d, n %d, k %d)", a.n_tok, a.n, a.k);
+        SHV_REQUIRE(a.prologue == SHV_PRO_NONE || a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID, "gemv_q4k: fold with prologue %d", a.prologue);
+        SHV_REQUIRE(a.residual != a.y && shv_aligned16(a.residual) && shv_aligned16(a.fold), "gemv_q4k: fold reads the whole residual row while y is written: they must be different, 16-byte aligned buffers");
+        SHV_REQUIRE(row_kernel_covers(ctx, a) && !ctx->gemv_scales_lds, "gemv_q4k: fold needs the one-row kernel's alignment of x, gamma and z");
     }
     // two to four rows of one sequence: the one-row kernel's shape with the rows side by side (SHV_MFMA_MIN_ROWS
     // at or below the row count sends them to the matrix cores instead, as before)

@@ -88,7 +88,7 @@ __device__ void select_by_rounds(uint32_t *kh, uint32_t *kl, int n_used, int32_t
 // search with wave ballots) are compacted into LDS and ranked against each other.
 // lds: scratch of at least 192 floats.
 template <int PER, bool AGENT>
-__device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *lds) {
+__device__ void route_token(const float *logits, int n_expert, int n_used, int32_t *topk, float *weights, float *lds, float scale = 1.f) {
     const int lane = threadIdx.x & 63;
     uint32_t *cand_p = reinterpret_cast<uint32_t *>(lds);       // [64]
     int32_t *cand_e = reinterpret_cast<int32_t *>(lds + 64);    // [64]
@@ -99,7 +99,7 @@ __device__ void route_token(const float *logits, int n_expert, int n_used, int32
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int e = lane + i * 64;
-        l[i] = e < n_expert ? (AGENT ? load_agent(logits + e) : logits[e]) : -INFINITY;
+        l[i] = e < n_expert ? (AGENT ? load_agent(logits + e) : logits[e]) * scale : -INFINITY;  // scale: a factor the logits still lack
         mx = fmaxf(mx, l[i]);
     }
     mx = wave_max_all(mx);
@@ -463,7 +463,12 @@ __device__ __forceinline__ void count_greater_ror(uint32_t key, int &rank) {
     rank += o > key ? 1 : 0;
 }
 
-__device__ __forceinline__ void route_block256(const float *lg, int n_expert, int n_used, bool shared_gate, int32_t *sel_e, float *sel_w, float *probs) {
+// NORM: the logits still lack the RMSNorm's factor of the token row (they came with the output
+// projection's launch); the block's waves have left their sums of squares of the row's k columns in
+// `red` before the call, and the factor, which changes no order, goes into the weights alone.
+template <bool NORM>
+__device__ __forceinline__ void route_block256(const float *lg, int n_expert, int n_used, bool shared_gate, int32_t *sel_e, float *sel_w, float *probs,
+                                               const float *red = nullptr, float mean_div = 1.f, float eps = 0.f) {
     __shared__ float s_max[4];
     __shared__ __align__(16) float s_gm[16];
     __shared__ int s_cnt[4];
@@ -489,6 +494,8 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     }
     __syncthreads();
     const float mx = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    float scale = 1.f;
+    if constexpr (NORM) scale = __builtin_amdgcn_rsqf(((red[0] + red[1]) + (red[2] + red[3])) * mean_div + eps);
     unsigned long long m0 = 0ull, m1 = 0ull;
     bool p0 = false, p1 = false;
     int n0 = 0;
@@ -524,8 +531,8 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     if (total > kCandMax || total < n_used || n_expert < 64 || n_used > 16) {
         // uniform over the block: many equal logits, or a shape the threshold does not cover
         if (wave == 0) {
-            route_token<8, false>(lg, n_expert, n_used, sel_e, sel_w, probs);
-            if (lane == 0) sel_w[n_used] = shared_gate ? sigmoid_exact(lg[n_expert]) : 0.f;
+            route_token<8, false>(lg, n_expert, n_used, sel_e, sel_w, probs, scale);
+            if (lane == 0) sel_w[n_used] = shared_gate ? sigmoid_exact(lg[n_expert] * scale) : 0.f;
         }
         __syncthreads();
         return;
@@ -565,7 +572,7 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
     if (lane < total && rank < n_used) s_sel[wave][rank] = mine;
     __builtin_amdgcn_wave_barrier();
     const unsigned long long sk = lane < n_used ? s_sel[wave][lane] : 0ull;
-    const float ex_k = lane < n_used ? expf(from_ordered_bits(static_cast<uint32_t>(sk >> 32)) - mx) : 0.f;
+    const float ex_k = lane < n_used ? expf(from_ordered_bits(static_cast<uint32_t>(sk >> 32)) * scale - mx * scale) : 0.f;
     const int e_k = 0x7FFFFFFF - static_cast<int>(static_cast<uint32_t>(sk));
     float wsum = 0.f;
     for (int k = 0; k < n_used; k++) wsum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ex_k), k));
@@ -573,7 +580,7 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
         sel_e[lane] = e_k;
         sel_w[lane] = ex_k / wsum;
     }
-    if (lane == 63) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh) : 0.f;
+    if (lane == 63) sel_w[n_used] = shared_gate ? sigmoid_exact(lsh * scale) : 0.f;
     __builtin_amdgcn_wave_barrier();  // the wave reads what it has written itself (all waves write the same)
 }
 
@@ -583,7 +590,10 @@ __device__ __forceinline__ void route_block256(const float *lg, int n_expert, in
 // same RPP up rows of one expert, six 16-byte loads per lane in flight together.  P: passes a wave
 // makes over the staged activation row; a launch of many tokens has blocks to spare and uses
 // them to stage the row an eighth as often (64-row chunk: 148 to 119 us a layer).
-template <int K, int P>
+// NORM: a.xn is the row before its RMSNorm and a.logits lack the norm's factor (see route_block256):
+// the row is staged as x * gamma, the factor comes from the block's own sum of squares and goes
+// onto the finished gate and up products.
+template <int K, int P, bool NORM = false>
 __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int slot0) {
     constexpr int LPR = K / 64, RPP = 64 / LPR;
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
@@ -603,17 +613,35 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
     const float *x = a.xn + static_cast<size_t>(t) * K;
     constexpr int NVr = NV >= 1 ? NV : 1;
     float4 xv[NVr];
+    __shared__ float red[4];
 #pragma unroll
     for (int j = 0; j < NVr; j++) {
         const int c = 4 * (tid + kBlock * j);
         xv[j] = c < K ? *reinterpret_cast<const float4 *>(x + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if constexpr (NORM) {
+        float4 gm[NVr];
+#pragma unroll
+        for (int j = 0; j < NVr; j++) {
+            const int c = 4 * (tid + kBlock * j);
+            gm[j] = c < K ? *reinterpret_cast<const float4 *>(a.gamma + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NVr; j++) {
+            const float4 v = xv[j];
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+            xv[j] = make_float4(v.x * gm[j].x, v.y * gm[j].y, v.z * gm[j].z, v.w * gm[j].w);
+        }
+        ss = wave_sum_all(ss);
+        if (lane == 0) red[wave] = ss;  // read behind the next block-wide wait, wherever that is
     }
 
     // the shared expert's blocks need no selection (the block that stores it is a routed slot's)
     if (a.logits && slot < a.n_used) {
         // route this block's token from the router's logits, all four waves together
         const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
-        route_block256(lg, a.n_expert, a.n_used, a.no_shared_gate == 0, s_topk, s_w, probs);
+        route_block256<NORM>(lg, a.n_expert, a.n_used, a.no_shared_gate == 0, s_topk, s_w, probs, red, 1.f / static_cast<float>(K), a.eps);
         if (blockIdx.x == 0 && blockIdx.y == 0) {
             if (tid < a.n_used) a.topk[static_cast<size_t>(t) * a.n_used + tid] = s_topk[tid];
             if (tid <= a.n_used) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + tid] = s_w[tid];
@@ -649,6 +677,8 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
         }
     }
     __syncthreads();
+    float scale = 1.f;
+    if constexpr (NORM) scale = __builtin_amdgcn_rsqf(((red[0] + red[1]) + (red[2] + red[3])) / static_cast<float>(K) + a.eps);
     float xr[64], xs_lo, xs_hi;
     load_x_slice_presummed(xs, xsum, gi, xr, xs_lo, xs_hi);
     const NibbleConsts nc = nibble_consts();
@@ -663,8 +693,8 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
         }
         float gv = wg[p & 1].dot(g, nc, xr, xs_lo, xs_hi);
         float uv = wu[p & 1].dot(g, nc, xr, xs_lo, xs_hi);
-        gv = group_sum<LPR>(gv);
-        uv = group_sum<LPR>(uv);
+        gv = group_sum<LPR>(gv) * scale;
+        uv = group_sum<LPR>(uv) * scale;
         if (row < a.ffn && group_sum_owner<LPR>(lane)) {
             const float s = gv * sigmoid_exact(gv);
             a.act[(static_cast<size_t>(t) * (a.n_used + 1) + slot) * a.ffn + row] = s * uv;
@@ -922,6 +952,10 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
+    if (a.gamma)
+        SHV_REQUIRE(a.logits && a.n_tok == 1 && a.n_embd == 2048 && shv_aligned16(a.gamma) && shv_aligned16(a.xn) && is_q4k(a.gate_type) && is_q4k(a.up_type) &&
+                        is_q4k(a.gate_sh_type) && is_q4k(a.up_sh_type),
+                    "moe_up: the RMSNorm of the row inside the launch (gamma) goes with logits, one row of 2048 and Q4_K banks");
     ctx->moe_stamp = {};  // only the grouped launch leaves lists or operands behind, and says so itself
     // Banks of other types than Q4_K go through their own arms; a block whose routed banks and
     // shared expert differ in that takes one launch each, over its part of the slots.
@@ -945,7 +979,8 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
                 SHV_LAUNCH(ctx, (moe_up_kernel<2048, 8>), grid, block, 0, a, slot0);
             } else {
                 dim3 grid((a.ffn + RPP * 4 - 1) / (RPP * 4), slots, a.n_tok);
-                SHV_LAUNCH(ctx, (moe_up_kernel<2048, 1>), grid, block, 0, a, slot0);
+                if (a.gamma) SHV_LAUNCH(ctx, (moe_up_kernel<2048, 1, true>), grid, block, 0, a, slot0);
+                else SHV_LAUNCH(ctx, (moe_up_kernel<2048, 1>), grid, block, 0, a, slot0);
             }
             break;
         }
@@ -990,8 +1025,10 @@ int shv_launch_moe_down(shv_ctx *ctx, const shv_moe_down_args *pa) {
     {
         const bool packed_here = ctx->moe_stamp.packed && ctx->moe_stamp.act == a.act;
         const bool grouped_road = is_q4k(a.down_type) && is_q4k(a.down_sh_type) && shv_moe_down_grouped_covers(ctx, a);
-        SHV_REQUIRE(!a.act_packed || grouped_road, "moe_down: act_packed is set, but this call does not take the grouped Q4_K path (bank types, workspaces or %d rows)", a.n_tok);
-        SHV_REQUIRE(a.act_packed || !packed_here, "moe_down: the shv_moe_up before this call left act as matrix-core operands (its act_packed); this call reads floats");
+        // (a pass too short to be grouped ignores the flag in both launches: act is floats then)
+        SHV_REQUIRE(!packed_here || (a.act_packed && grouped_road),
+                    "moe_down: the shv_moe_up before this call left act as matrix-core operands (its act_packed); this call %s",
+                    a.act_packed ? "does not take the grouped Q4_K path that reads them (bank types, workspaces)" : "reads floats (act_packed is not set)");
     }
     // as in the up projection: the Q4_K part of the slots here, the rest through the other arms,
     // which then add to what this launch has written

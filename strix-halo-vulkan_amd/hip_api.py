@@ -10,7 +10,7 @@ Q4K_BYTES = 144
 
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
-OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV, OP_RING_ROWS = 10, 11, 12, 13, 14, 15
+OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV, OP_RING_ROWS, OP_ROUTER_FOLD = 10, 11, 12, 13, 14, 15, 16
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 
@@ -37,7 +37,13 @@ class GemvQ4KArgs(C.Structure):
                 ("head_dim", C.c_int32), ("eps", C.c_float), ("x_stride", C.c_int32),
                 ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("seq_len", C.c_int32),
                 ("ring_slots", C.c_int32), ("ring_stride", C.c_int32), ("z_ring", C.c_int32),
-                ("y_flat", C.c_void_p)]
+                ("y_flat", C.c_void_p), ("fold", C.c_void_p), ("fold_out", C.c_void_p), ("fold_rows", C.c_int32)]
+
+
+class RouterFoldArgs(C.Structure):
+    _fields_ = [("router", C.c_void_p), ("shared_gate", C.c_void_p), ("gamma", C.c_void_p), ("w_out", C.c_void_p),
+                ("out", C.c_void_p), ("scratch", C.c_void_p), ("n_expert", C.c_int32), ("n_embd", C.c_int32),
+                ("k", C.c_int32)]
 
 
 class DequantQ4KArgs(C.Structure):
@@ -77,7 +83,8 @@ class MoeUpArgs(C.Structure):
                 ("n_used", C.c_int32), ("ffn", C.c_int32), ("logits", C.c_void_p),
                 ("weights", C.c_void_p), ("n_expert", C.c_int32), ("gate_type", C.c_int32),
                 ("up_type", C.c_int32), ("gate_sh_type", C.c_int32), ("up_sh_type", C.c_int32),
-                ("group", C.c_void_p), ("no_shared_gate", C.c_int32), ("act_packed", C.c_int32)]
+                ("group", C.c_void_p), ("no_shared_gate", C.c_int32), ("act_packed", C.c_int32),
+                ("gamma", C.c_void_p), ("eps", C.c_float)]
 
 
 class MoeDownArgs(C.Structure):
@@ -153,7 +160,7 @@ SYMBOLS = [
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
-    "shv_argmax_static", "shv_ring_rows",
+    "shv_argmax_static", "shv_ring_rows", "shv_router_fold",
 ]
 
 _lib = None
@@ -210,6 +217,7 @@ def load():
     L.shv_advance.argtypes = [vp, C.POINTER(AdvanceArgs)]
     L.shv_argmax_static.argtypes = [vp, C.POINTER(ArgmaxArgs)]
     L.shv_ring_rows.argtypes = [vp, C.POINTER(RingRowsArgs)]
+    L.shv_router_fold.argtypes = [vp, C.POINTER(RouterFoldArgs)]
     _lib = L
     return L
 

@@ -545,6 +545,57 @@ std::vector<shv_op> MoEGPU::Dispatches(int l, const float *in, float *out, int n
     return {make_op(SHV_OP_MOE_ROUTER, r), make_op(SHV_OP_MOE_UP, u), make_op(SHV_OP_MOE_DOWN, d)};
 }
 
+bool MoEGPU::Fold(int l, const TensorView &w_out) {
+    if (fold_.empty()) fold_.assign(c_.NLayer + 1, nullptr);
+    if (l < 0 || l >= static_cast<int>(fold_.size())) return false;
+    const TensorView &ge = m_.Tensor(Model::Blk(l, "ffn_gate_exps")), &ue = m_.Tensor(Model::Blk(l, "ffn_up_exps"));
+    const TensorView &gs = m_.Tensor(Model::Blk(l, "ffn_gate_shexp")), &us = m_.Tensor(Model::Blk(l, "ffn_up_shexp"));
+    const bool up_q4k = ge.ggml == gguf::Q4_K && ue.ggml == gguf::Q4_K && gs.ggml == gguf::Q4_K && us.ggml == gguf::Q4_K;
+    // what the fused launches are built for: a 2048-wide stream, a 4096-wide mixer output, the
+    // selection inside the gate/up kernel, everything it touches in the types the kernels stream
+    if (!up_q4k || !FusedRouter(1) || c_.NEmbd != 2048 || w_out.rows != c_.NEmbd || w_out.cols != 4096 || w_out.ggml != gguf::Q4_K || c_.NExpert > 512)
+        return false;
+    const size_t rows = c_.NExpert + 1, width = static_cast<size_t>(w_out.cols) + c_.NEmbd;
+    if (!fold_[l]) fold_[l] = static_cast<float *>(dev_.alloc(rows * width * 4));
+    const size_t scratch_bytes = static_cast<size_t>(c_.NEmbd) * w_out.cols * 4;
+    float *scratch = static_cast<float *>(dev_.alloc(scratch_bytes));
+    shv_router_fold_args f{};
+    f.router = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ffn_gate_inp")).ptr);
+    f.shared_gate = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ffn_gate_inp_shexp")).ptr);
+    f.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "post_attention_norm")).ptr);
+    f.w_out = w_out.ptr;
+    f.out = fold_[l];
+    f.scratch = scratch;
+    f.n_expert = c_.NExpert;
+    f.n_embd = c_.NEmbd;
+    f.k = static_cast<int32_t>(w_out.cols);
+    check(shv_router_fold(dev_.ctx(), &f), "MoEGPU.Fold");
+    dev_.sync();
+    dev_.release(scratch, scratch_bytes);
+    fold_k_ = static_cast<int>(w_out.cols);
+    return true;
+}
+
+void MoEGPU::FoldInto(int l, PassRows &r) const {
+    if (!Folded(l)) throw Error("llm: MoEGPU: layer " + std::to_string(l) + " has no folded router");
+    r.fold = fold_[l];
+    r.fold_rows = c_.NExpert + 1;
+    r.fold_out = logits_;
+}
+
+std::vector<shv_op> MoEGPU::DispatchesFolded(int l, const float *in, float *out, std::vector<std::string> *labels) const {
+    if (!Folded(l)) throw Error("llm: MoEGPU: layer " + std::to_string(l) + " has no folded router");
+    auto ops = Dispatches(l, in, out, 1, nullptr);
+    // the router's launch goes; gate/up takes the row as it is and normalises it itself
+    shv_moe_up_args u{};
+    std::memcpy(&u, ops[1].args, sizeof u);
+    u.xn = in;
+    u.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "post_attention_norm")).ptr);
+    u.eps = c_.RMSEps;
+    if (labels) labels->insert(labels->end(), {"moe.up", "moe.down"});
+    return {make_op(SHV_OP_MOE_UP, u), ops[2]};
+}
+
 void MoEGPU::Run(int layer) {
     if (n_tok_ < 1) throw Error("llm: MoEGPU.Run before Upload");
     dev_.run(Dispatches(layer, in_, out_, n_tok_, nullptr));
@@ -737,6 +788,9 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     o.eps = c_.RMSEps;
     o.x_stride = c_.VWidth();
     o.y_stride = c_.NEmbd;
+    o.fold = r.fold;
+    o.fold_rows = r.fold_rows;
+    o.fold_out = r.fold_out;
     if (flat) {
         o.z = row_ + c_.ConvWidth();  // the z columns of the projection row
         o.z_stride = width;
@@ -960,6 +1014,9 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, cons
     o.x_stride = c_.NHead * c_.HeadDim;
     o.y_stride = c_.NEmbd;
     o.z_stride = width;
+    o.fold = r.fold;
+    o.fold_rows = r.fold_rows;
+    o.fold_out = r.fold_out;
     if (labels) labels->insert(labels->end(), {"attn.qkv", "attn.attn", "attn.out"});
     return {make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_ATTN_DECODE, a), make_op(SHV_OP_GEMV_Q4K, o)};
 }
@@ -1109,6 +1166,15 @@ Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_
     attn_ = new AttnGPU(dev, m, block_rows_, o_.NKV, o_.Slots, pos_);
     if (o_.AttnSplits > 0) attn_->SetSplits(o_.AttnSplits);
     if (!o_.NoHead) head_ = new HeadGPU(dev, m, head_rows);
+    // One-row passes take the router's logits from the launch of the mixer's output projection
+    // (48 launches fewer a step at 48 layers): the tables are made here, once, from the weights
+    // as they stand, as the reference makes its banks when it stages a graph (llm/graph.go:635);
+    // LLM_ROUTER_FOLD=0 keeps the router's own launch.
+    const char *rf = std::getenv("LLM_ROUTER_FOLD");
+    if (!(rf && rf[0] == '0')) {
+        x2_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.NEmbd) * 4));
+        for (int l = 0; l < layers_; l++) moe_->Fold(l, m.Tensor(Model::Blk(l, c_.IsAttn(l) ? "attn_output" : "ssm_out")));
+    }
     // the decode step of slot 0 is recorded up front, as NewGraph does (llm/graph.go:609)
     pass(0, 1, head_ ? kSample : kPrefill, false);
 }
@@ -1165,6 +1231,17 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     p.labels.push_back("embed");
     if (rows > kBlockRows && (kind == kBatch || spec)) throw Error("llm: a pass of " + std::to_string(rows) + " rows is a plain prompt pass; batched and rewindable passes carry up to " + std::to_string(kBlockRows));
     for (int l = 0; l < layers_; l++) {
+        if (rows == 1 && x2_ && moe_->Folded(l)) {
+            // the mixer writes the row beside the stream (its output projection reads the whole
+            // residual row for the router's products while it writes), the MoE block brings it back
+            PassRows rf = r;
+            moe_->FoldInto(l, rf);
+            auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x2_, rf, &p.labels) : dn_->Dispatches(l, x_, x2_, rf, &p.labels);
+            p.ops.insert(p.ops.end(), sub.begin(), sub.end());
+            auto ffn = moe_->DispatchesFolded(l, x2_, x_, &p.labels);
+            p.ops.insert(p.ops.end(), ffn.begin(), ffn.end());
+            continue;
+        }
         if (rows <= block_rows_) {
             auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x_, r, &p.labels) : dn_->Dispatches(l, x_, x_, r, &p.labels);
             p.ops.insert(p.ops.end(), sub.begin(), sub.end());

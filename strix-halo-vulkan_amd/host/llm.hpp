@@ -181,6 +181,12 @@ struct PassRows {
                                     // a dependent load of the slot word
     int n_seq = 1, seq_len = 1;
     bool spec = false;              // DeltaNet: a rewindable pass (state goes to the other planes)
+    // A one-row pass whose mixer's output projection also forms the logits of the layer's router
+    // (MoEGPU::Fold): the table's rows, how many, and where the products go.  out must then be
+    // another buffer than in.
+    const float *fold = nullptr;
+    int fold_rows = 0;
+    float *fold_out = nullptr;
     int rows() const { return n_seq * seq_len; }
 };
 
@@ -198,6 +204,16 @@ public:
     void Run(int layer);
     std::vector<Stage> Profile(int layer, int iters);
     std::vector<shv_op> Dispatches(int layer, const float *in, float *out, int nTok, std::vector<std::string> *labels) const;
+    // The router's rows of `layer` carried through the output projection `w_out` (Q4_K [NEmbd][k])
+    // that feeds the block: made once, when a graph is staged.  False (and nothing made) where the
+    // shapes or types are not the ones the fused launch is built for.
+    bool Fold(int layer, const TensorView &w_out);
+    bool Folded(int layer) const { return layer >= 0 && layer < static_cast<int>(fold_.size()) && fold_[layer] != nullptr; }
+    // What the mixer's output projection needs to form the logits (fields of PassRows)
+    void FoldInto(int layer, PassRows &r) const;
+    // The block on a one-row pass whose logits came with the output projection: gate/up (which
+    // normalises the row itself) and down.  `in` is the row before its RMSNorm.
+    std::vector<shv_op> DispatchesFolded(int layer, const float *in, float *out, std::vector<std::string> *labels) const;
     std::vector<float> Logits() const;    // [T][NExpert+1]
     std::vector<int32_t> TopK() const;    // [T][used]
     std::vector<float> Weights() const;   // [T][used+1]
@@ -224,6 +240,8 @@ private:
     int32_t *topk_, *group_ = nullptr;
     uint64_t act_bytes_ = 0;
     int route_mode_ = 2;  // 0 own dispatch, 1 fused, 2 fused for passes of up to three rows
+    std::vector<float *> fold_;  // per layer [NExpert+1][k + NEmbd], or nullptr
+    int fold_k_ = 0;
 };
 
 // llm.DeltaNetGPU (llm/gpu_deltanet.go:207-322, NewDeltaNetGPUBank :421)
@@ -469,6 +487,7 @@ private:
     int spec_past_ = 0, spec_rows_ = 0;
     int last_rows_ = 0;
     float *x_ = nullptr;       // residual stream, [rows_max][NEmbd]
+    float *x2_ = nullptr;      // a one-row pass's row between a layer's mixer and its MoE block (router fold)
     float *res_all_ = nullptr; // ForwardResidual's rows
     size_t res_all_rows_ = 0;
     int32_t *ids_ = nullptr;   // [Slots][NKV+2] the sequences' tokens by position

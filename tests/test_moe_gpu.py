@@ -201,8 +201,14 @@ def test_flags_that_do_not_fit_the_road_taken_are_refused(ctx, types):
     block is the CPU's."""
     case = MoeCase(ctx, seed=411, E=32, used=4, T=128, types=types)
     want = case.oracle()
-    with pytest.raises(A.ShvError, match="act_packed"):
-        case.gpu(residual=True, grouped=True, packed=True)
+    if "gate_sh" in types:
+        # gate/up did not go grouped and left floats; the grouped down launch would read them as operands
+        with pytest.raises(A.ShvError, match="did not leave act as operands"):
+            case.gpu(residual=True, grouped=True, packed=True)
+    else:
+        # gate/up went grouped and packed act; the down launch goes another road, which reads floats
+        with pytest.raises(A.ShvError, match="left act as matrix-core operands"):
+            case.gpu(residual=True, grouped=True, packed=True)
     got = case.gpu(residual=True, grouped=True)
     ok = [t for t in range(case.T) if np.array_equal(got["topk"][t], want["topk"][t])]
     assert len(ok) >= case.T - 2
@@ -396,3 +402,99 @@ def test_expert_kernel_routing_without_a_shared_gate(ctx, full_bank):
     assert np.array_equal(out[0][0], out[1][0])
     assert out[0][1][used] == 0.0 and out[1][1][used] == 0.0
     assert np.allclose(out[0][1], out[1][1], rtol=1e-6)
+
+
+# ---- the router's logits formed by the launch of the output projection that feeds the block ----
+
+def _fold_case(ctx, case, seed, prologue):
+    """A 2048 x 4096 Q4_K output projection W, its input v (with what the prologue needs) and the
+    residual row x in front of the MoE block `case`: h = x + W pro(v) is the block's input."""
+    rng = np.random.default_rng(seed)
+    H, K = case.H, 4096
+    w = O.quantize_q4k((rng.standard_normal((H, K)) * 0.02).astype(np.float32))
+    v = rng.standard_normal(K).astype(np.float32)
+    x = rng.standard_normal(H).astype(np.float32)
+    z = rng.standard_normal(K).astype(np.float32)
+    gn = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32)
+    if prologue == A.PRO_GATED_NORM:
+        vh = v.reshape(-1, 128).astype(np.float64)
+        pv = vh / np.sqrt((vh ** 2).mean(axis=1, keepdims=True) + EPS) * gn * (1 / (1 + np.exp(-z.reshape(-1, 128).astype(np.float64))))
+        pv = pv.reshape(-1)
+    elif prologue == A.PRO_MUL_SIGMOID:
+        pv = v.astype(np.float64) / (1 + np.exp(-z.astype(np.float64)))
+    else:
+        pv = v.astype(np.float64)
+    wf = O.dequant_q4k(w, K).astype(np.float64)
+    h = (x.astype(np.float64) + wf @ pv).astype(np.float32)
+    return dict(w=w, v=v, x=x, z=z, gn=gn, h=h)
+
+
+@pytest.mark.parametrize("prologue", [A.PRO_NONE, A.PRO_GATED_NORM, A.PRO_MUL_SIGMOID], ids=["plain", "gated-norm", "sigmoid-gate"])
+@pytest.mark.parametrize("E,used", [(512, 10), (16, 4)])
+def test_router_rows_ride_on_the_output_projection(ctx, full_bank, prologue, E, used):
+    """One row: the output projection's launch also forms R diag(gamma) h from the table
+    shv_router_fold makes, and the gate/up kernel applies the RMSNorm's factor to those products,
+    to the row it stages and to its own products.  Held to the CPU block on h = x + W pro(v)
+    (float64), and to the launches it replaces (projection in place, router, gate/up, down)."""
+    import copy
+    if E == 512:
+        case = copy.copy(full_bank)
+        case.T = 1
+    else:
+        case = MoeCase(ctx, seed=77, E=E, used=used, T=1)
+    H, K, ffn, c = case.H, 4096, case.ffn, ctx
+    for seed in range(500, 540):
+        f = _fold_case(ctx, case, seed, prologue)
+        case.h = f["h"].reshape(1, H)
+        case.res = np.zeros((1, H), np.float32)
+        want = case.oracle()
+        lg = want["logits"][0].astype(np.float64)
+        p = np.exp(lg - lg.max())
+        if _margin(p / p.sum(), used) > 2e-4:
+            break
+    else:
+        raise AssertionError("no seed clear of near-ties")
+    d = {k: c.upload(getattr(case, k)) for k in ("router", "shared_gate", "gate_exps", "up_exps", "down_exps", "gate_sh", "up_sh", "down_sh", "gamma")}
+    dw, dv, dx, dz, dgn = (c.upload(f[k]) for k in ("w", "v", "x", "z", "gn"))
+    table, scratch = c.alloc((E + 1) * (K + H) * 4), c.alloc(H * K * 4)
+    c.enqueue(A.OP_ROUTER_FOLD, A.RouterFoldArgs(d["router"].ptr, d["shared_gate"].ptr, d["gamma"].ptr, dw.ptr, table.ptr, scratch.ptr, E, H, K))
+    # the table against its definition in float64
+    tb = table.read(np.float32, (E + 1) * (K + H)).reshape(E + 1, K + H)
+    rg = np.vstack([case.router, case.shared_gate[None]]).astype(np.float64) * case.gamma.astype(np.float64)
+    wf = O.dequant_q4k(f["w"], K).astype(np.float64)
+    assert O.rel_l2(tb[:, K:], rg) <= 1e-7
+    assert O.rel_l2(tb[:, :K], rg @ wf) <= 1e-7
+    y, raw = c.alloc(H * 4), c.alloc((E + 1) * 4)
+    topk, weights, act, out = c.alloc(used * 4), c.alloc((used + 1) * 4), c.alloc((used + 1) * ffn * 4), c.alloc(H * 4)
+    g = A.gemv_args(dw, dv, y, H, K, 1, prologue, dgn if prologue == A.PRO_GATED_NORM else None, dz if prologue != A.PRO_NONE else None,
+                    dx, EPS, 128 if prologue == A.PRO_GATED_NORM else 0)
+    g.fold, g.fold_out, g.fold_rows = table.ptr, raw.ptr, E + 1
+    ua = A.MoeUpArgs(y.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr, d["up_sh"].ptr, act.ptr, 1, H, used, ffn,
+                     raw.ptr, weights.ptr, E, 0, 0, 0, 0, None, 0, 0, d["gamma"].ptr, EPS)
+    da = A.MoeDownArgs(act.ptr, topk.ptr, weights.ptr, d["down_exps"].ptr, d["down_sh"].ptr, y.ptr, out.ptr, 1, H, used, ffn, H, H, 0, 0, E, None, None)
+    c.dispatch_multi([A.make_op(A.OP_GEMV_Q4K, g), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)])
+    got_h = y.read(np.float32, H)
+    assert O.rel_l2(got_h, f["h"]) <= 1e-5
+    scale = 1.0 / np.sqrt((f["h"].astype(np.float64) ** 2).mean() + EPS)
+    got_lg = raw.read(np.float32, E + 1).astype(np.float64) * scale
+    assert O.rel_l2(got_lg[:E], want["logits"][0]) <= 2e-5
+    assert np.array_equal(topk.read(np.int32, used), want["topk"][0])
+    wt = weights.read(np.float32, used + 1)
+    assert O.rel_l2(wt[:used], want["weights"][0]) <= 1e-5
+    assert abs(wt[used] - want["sig"][0]) <= 1e-5
+    assert O.rel_l2(act.read(np.float32, (used + 1) * ffn).reshape(used + 1, ffn)[:used], want["swiglu"][0]) <= TOL
+    got_out = out.read(np.float32, H)
+    assert O.rel_l2(got_out, want["out"][0] + f["h"]) <= TOL
+    # the launches it replaces, on the same inputs
+    case.h = got_h.reshape(1, H)
+    case.res = got_h.reshape(1, H)
+    ref = case.gpu(residual=True, defer=True)
+    assert np.array_equal(ref["topk"][0], topk.read(np.int32, used))
+    assert O.rel_l2(got_out, ref["out"][0]) <= 1e-5
+    # refusals: y aliasing the residual the fold reads; more than one row
+    g.y = dx.ptr
+    with pytest.raises(A.ShvError, match="different"):
+        c.enqueue(A.OP_GEMV_Q4K, g)
+    ua.n_tok = 2
+    with pytest.raises(A.ShvError, match="one row"):
+        c.enqueue(A.OP_MOE_UP, ua)
