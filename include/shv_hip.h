@@ -284,6 +284,9 @@ typedef struct {
                                 by gamma and applies the factor to its own products and to the logits
                                 (llm/hc.go:176-190).  NULL: xn is normalised already */
     float eps;
+    const float *shared_gate; /* with gamma: the shared expert's gate vector (llm/moe.go:396-402); its weight
+                                sigmoid(shared_gate . xn) is then formed here from the staged row instead of
+                                read from logits[n_expert].  NULL: from the logits */
 } shv_moe_up_args;
 
 /* Down projection, weighting and combine (llm/moe.go:331-357,390-407; llm_moe_gemv.comp MODE 1 +

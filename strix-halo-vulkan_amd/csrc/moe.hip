@@ -636,15 +636,31 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
         ss = wave_sum_all(ss);
         if (lane == 0) red[wave] = ss;  // read behind the next block-wide wait, wherever that is
     }
+    // the shared expert's gate from the staged row, by the first of the shared expert's blocks
+    const bool gate_here = NORM && a.shared_gate && slot == a.n_used && blockIdx.x == 0;
+    __shared__ float red_sg[4];
+    if constexpr (NORM) {
+        if (gate_here) {
+            float dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < NVr; j++) {
+                const int c = 4 * (tid + kBlock * j);
+                const float4 sg = c < K ? *reinterpret_cast<const float4 *>(a.shared_gate + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+                dot = fmaf(sg.x, xv[j].x, fmaf(sg.y, xv[j].y, fmaf(sg.z, xv[j].z, fmaf(sg.w, xv[j].w, dot))));
+            }
+            dot = wave_sum_all(dot);
+            if (lane == 0) red_sg[wave] = dot;
+        }
+    }
 
     // the shared expert's blocks need no selection (the block that stores it is a routed slot's)
     if (a.logits && slot < a.n_used) {
         // route this block's token from the router's logits, all four waves together
         const float *lg = a.logits + static_cast<size_t>(t) * (a.n_expert + 1);
-        route_block256<NORM>(lg, a.n_expert, a.n_used, a.no_shared_gate == 0, s_topk, s_w, probs, red, 1.f / static_cast<float>(K), a.eps);
+        route_block256<NORM>(lg, a.n_expert, a.n_used, a.no_shared_gate == 0 && !(NORM && a.shared_gate), s_topk, s_w, probs, red, 1.f / static_cast<float>(K), a.eps);
         if (blockIdx.x == 0 && blockIdx.y == 0) {
             if (tid < a.n_used) a.topk[static_cast<size_t>(t) * a.n_used + tid] = s_topk[tid];
-            if (tid <= a.n_used) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + tid] = s_w[tid];
+            if (tid < a.n_used + ((NORM && a.shared_gate) ? 0 : 1)) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + tid] = s_w[tid];
         }
     }
 
@@ -678,7 +694,10 @@ __global__ __launch_bounds__(kBlock) void moe_up_kernel(shv_moe_up_args a, int s
     }
     __syncthreads();
     float scale = 1.f;
-    if constexpr (NORM) scale = __builtin_amdgcn_rsqf(((red[0] + red[1]) + (red[2] + red[3])) / static_cast<float>(K) + a.eps);
+    if constexpr (NORM) {
+        scale = __builtin_amdgcn_rsqf(((red[0] + red[1]) + (red[2] + red[3])) / static_cast<float>(K) + a.eps);
+        if (gate_here && tid == 0) a.weights[static_cast<size_t>(t) * (a.n_used + 1) + a.n_used] = sigmoid_exact(((red_sg[0] + red_sg[1]) + (red_sg[2] + red_sg[3])) * scale);
+    }
     float xr[64], xs_lo, xs_hi;
     load_x_slice_presummed(xs, xsum, gi, xr, xs_lo, xs_hi);
     const NibbleConsts nc = nibble_consts();
@@ -952,6 +971,7 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 65535, "moe_up: n_tok %d", a.n_tok);
     SHV_REQUIRE(a.n_used >= 1 && a.n_used <= kMaxUsed, "moe_up: n_used %d", a.n_used);
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
+    SHV_REQUIRE(!a.shared_gate || (a.gamma && shv_aligned16(a.shared_gate)), "moe_up: shared_gate goes with gamma (the row normalised inside the launch), 16-byte aligned");
     if (a.gamma)
         SHV_REQUIRE(a.logits && a.n_tok == 1 && a.n_embd == 2048 && shv_aligned16(a.gamma) && shv_aligned16(a.xn) && is_q4k(a.gate_type) && is_q4k(a.up_type) &&
                         is_q4k(a.gate_sh_type) && is_q4k(a.up_sh_type),

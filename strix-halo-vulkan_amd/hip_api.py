@@ -84,7 +84,7 @@ class MoeUpArgs(C.Structure):
                 ("weights", C.c_void_p), ("n_expert", C.c_int32), ("gate_type", C.c_int32),
                 ("up_type", C.c_int32), ("gate_sh_type", C.c_int32), ("up_sh_type", C.c_int32),
                 ("group", C.c_void_p), ("no_shared_gate", C.c_int32), ("act_packed", C.c_int32),
-                ("gamma", C.c_void_p), ("eps", C.c_float)]
+                ("gamma", C.c_void_p), ("eps", C.c_float), ("shared_gate", C.c_void_p)]
 
 
 class MoeDownArgs(C.Structure):

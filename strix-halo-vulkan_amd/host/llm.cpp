@@ -555,13 +555,13 @@ bool MoEGPU::Fold(int l, const TensorView &w_out) {
     // selection inside the gate/up kernel, everything it touches in the types the kernels stream
     if (!up_q4k || !FusedRouter(1) || c_.NEmbd != 2048 || w_out.rows != c_.NEmbd || w_out.cols != 4096 || w_out.ggml != gguf::Q4_K || c_.NExpert > 512)
         return false;
-    const size_t rows = c_.NExpert + 1, width = static_cast<size_t>(w_out.cols) + c_.NEmbd;
+    const size_t rows = c_.NExpert, width = static_cast<size_t>(w_out.cols) + c_.NEmbd;  // the shared gate's product is formed by gate/up
     if (!fold_[l]) fold_[l] = static_cast<float *>(dev_.alloc(rows * width * 4));
     const size_t scratch_bytes = static_cast<size_t>(c_.NEmbd) * w_out.cols * 4;
     float *scratch = static_cast<float *>(dev_.alloc(scratch_bytes));
     shv_router_fold_args f{};
     f.router = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ffn_gate_inp")).ptr);
-    f.shared_gate = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ffn_gate_inp_shexp")).ptr);
+    f.shared_gate = nullptr;
     f.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "post_attention_norm")).ptr);
     f.w_out = w_out.ptr;
     f.out = fold_[l];
@@ -579,7 +579,7 @@ bool MoEGPU::Fold(int l, const TensorView &w_out) {
 void MoEGPU::FoldInto(int l, PassRows &r) const {
     if (!Folded(l)) throw Error("llm: MoEGPU: layer " + std::to_string(l) + " has no folded router");
     r.fold = fold_[l];
-    r.fold_rows = c_.NExpert + 1;
+    r.fold_rows = c_.NExpert;  // the shared gate's row stays behind: gate/up forms that product from the row it stages
     r.fold_out = logits_;
 }
 
@@ -592,6 +592,7 @@ std::vector<shv_op> MoEGPU::DispatchesFolded(int l, const float *in, float *out,
     u.xn = in;
     u.gamma = static_cast<const float *>(m_.Tensor(Model::Blk(l, "post_attention_norm")).ptr);
     u.eps = c_.RMSEps;
+    u.shared_gate = static_cast<const float *>(m_.Tensor(Model::Blk(l, "ffn_gate_inp_shexp")).ptr);
     if (labels) labels->insert(labels->end(), {"moe.up", "moe.down"});
     return {make_op(SHV_OP_MOE_UP, u), ops[2]};
 }

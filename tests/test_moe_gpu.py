@@ -468,9 +468,12 @@ def test_router_rows_ride_on_the_output_projection(ctx, full_bank, prologue, E, 
     topk, weights, act, out = c.alloc(used * 4), c.alloc((used + 1) * 4), c.alloc((used + 1) * ffn * 4), c.alloc(H * 4)
     g = A.gemv_args(dw, dv, y, H, K, 1, prologue, dgn if prologue == A.PRO_GATED_NORM else None, dz if prologue != A.PRO_NONE else None,
                     dx, EPS, 128 if prologue == A.PRO_GATED_NORM else 0)
-    g.fold, g.fold_out, g.fold_rows = table.ptr, raw.ptr, E + 1
+    # the shared gate's product either as the table's last row (few experts here) or formed by the
+    # gate/up kernel from the row it stages (what the token loop does: 512 rows fill 256 blocks evenly)
+    sg_in_up = E == 512
+    g.fold, g.fold_out, g.fold_rows = table.ptr, raw.ptr, E if sg_in_up else E + 1
     ua = A.MoeUpArgs(y.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr, d["up_sh"].ptr, act.ptr, 1, H, used, ffn,
-                     raw.ptr, weights.ptr, E, 0, 0, 0, 0, None, 0, 0, d["gamma"].ptr, EPS)
+                     raw.ptr, weights.ptr, E, 0, 0, 0, 0, None, 0, 0, d["gamma"].ptr, EPS, d["shared_gate"].ptr if sg_in_up else None)
     da = A.MoeDownArgs(act.ptr, topk.ptr, weights.ptr, d["down_exps"].ptr, d["down_sh"].ptr, y.ptr, out.ptr, 1, H, used, ffn, H, H, 0, 0, E, None, None)
     c.dispatch_multi([A.make_op(A.OP_GEMV_Q4K, g), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)])
     got_h = y.read(np.float32, H)
