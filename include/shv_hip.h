@@ -138,7 +138,7 @@ typedef struct {
                                 address that does not depend on the position, for a consumer that would
                                 otherwise wait for the position word before it can ask for the row (the
                                 DeltaNet output projection's gate z); NULL: not stored */
-    /* The router's logits in the same launch (one row, k = 4096, n = 2048, a residual): the
+    /* The router's logits in the same launch (one to four rows of one sequence, k = 4096, n = 2048, a residual): the
      * projection feeds y = residual + W pro(x) to an RMSNorm and a float32 router R (llm/moe.go:
      * 219-232), and R (gamma * y) is linear in y: it is fold[e] . [pro(x) | residual] with
      * fold [fold_rows][k + n] = [R diag(gamma) W | R diag(gamma)] made once by shv_router_fold.
@@ -147,6 +147,7 @@ typedef struct {
     const float *fold;
     float *fold_out;
     int32_t fold_rows;
+    int32_t fold_stride;     /* two to four rows of one sequence: row t's products go to fold_out + t * fold_stride */
 } shv_gemv_q4k_args;
 
 /* The table shv_gemv_q4k's `fold` reads, for one layer: out [rows][k + n_embd] float32,
@@ -278,7 +279,7 @@ typedef struct {
                                 shv_moe_down reads (two binary16 parts of every value, same bytes a row)
                                 instead of floats; the shv_moe_down of this pass must be the library's
                                 next call on the stream, with act_packed and group_ready set too */
-    const float *gamma;      /* with logits, one row: xn is the row BEFORE its RMSNorm and logits are the
+    const float *gamma;      /* with logits, up to four rows: xn is the row BEFORE its RMSNorm and logits are the
                                 router's products without the norm's factor (shv_gemv_q4k's fold_out);
                                 the kernel forms the factor from the row it stages, multiplies the row
                                 by gamma and applies the factor to its own products and to the logits

@@ -253,18 +253,18 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 // super-block, instead of every lane decoding its own group's from the header it holds anyway.
 // FOLD: the launch also forms the router's logits of the MoE block that follows (a.fold: rows of
 // k + n floats, [R diag(gamma) W | R diag(gamma)], against [pro(x) | residual]; see router_fold.hip).
-// Every block takes two of those rows beside its own, four waves a row and a quarter of the row a
-// wave; the residual row (n = 4 T floats) is staged behind pro(x), so y must be another buffer.
+// Every block takes two of those rows beside its own, four waves a row: a wave takes a quarter of
+// the row's first k entries against the staged pro(x) and a quarter of its last n against the
+// residual row, which it reads from memory itself (so y must be another buffer).
 template <int K, int WAVES, int P, int PRO, bool STAGED = false, bool FOLD = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args a) {
     constexpr int T = WAVES * 64, LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int NV = K / 4 / T;  // float4 a thread stages
     static_assert(NV >= 1 && K % (4 * T) == 0, "threads of a block each stage whole float4s");
-    constexpr int FN = 4 * T;               // FOLD: the residual row's length (one float4 a thread)
-    constexpr int FQ = (K + FN) / 4;        // a wave's quarter of a fold row
-    constexpr int FV = FQ / 256;            // float4 a lane loads of it
-    static_assert(!FOLD || (WAVES == 8 && FQ % 256 == 0), "a fold row is split over four waves");
-    __shared__ __align__(16) float xs[lds_padded(FOLD ? K + FN : K)];
+    constexpr int FN = 2048;                         // FOLD: the residual row's length
+    constexpr int FA = K / 4 / 256, FB = FN / 4 / 256;  // float4 a lane loads of a wave's quarter: against pro(x), against the residual
+    static_assert(!FOLD || (WAVES == 8 && K % 1024 == 0), "a fold row is split over four waves");
+    __shared__ __align__(16) float xs[lds_padded(K)];
     __shared__ __align__(16) float xsum[K / 32];
     __shared__ float red[WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -300,8 +300,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
             zv[j] = *reinterpret_cast<const float4 *>(a.z + zi);
         }
     }
-    float4 fres = make_float4(0.f, 0.f, 0.f, 0.f);
-    if constexpr (FOLD) fres = *reinterpret_cast<const float4 *>(a.residual + 4 * tid);
+    // FOLD: the wave's quarter of the residual row, asked for with the other inputs
+    const int fold_row = static_cast<int>(blockIdx.x) * 2 + (wave >> 2), fold_q = wave & 3;
+    float4 fx[FOLD ? FB : 1];
+    if constexpr (FOLD) {
+#pragma unroll
+        for (int j = 0; j < FB; j++) fx[j] = *reinterpret_cast<const float4 *>(a.residual + fold_q * (FN / 4) + (j * 64 + lane) * 4);
+    }
     Q4kLane w[P];
     int row[P];
 #pragma unroll
@@ -314,12 +319,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
 #pragma unroll
     for (int u = 0; u < P; u++) res[u] = (a.residual && row[u] >= 0 && group_sum_owner<LPR>(lane)) ? a.residual[row[u]] : 0.f;
     // the wave's quarter of its fold row, behind the weights
-    float4 fw[FOLD ? FV : 1];
-    const int fold_row = static_cast<int>(blockIdx.x) * 2 + (wave >> 2), fold_q = wave & 3;
+    float4 fw[FOLD ? FA + FB : 1];
     if constexpr (FOLD) {
-        const float *fr = a.fold + static_cast<size_t>(fold_row < a.fold_rows ? fold_row : 0) * (K + FN) + fold_q * FQ;
+        const float *fr = a.fold + static_cast<size_t>(fold_row < a.fold_rows ? fold_row : 0) * (K + FN);
 #pragma unroll
-        for (int j = 0; j < FV; j++) fw[j] = *reinterpret_cast<const float4 *>(fr + (j * 64 + lane) * 4);
+        for (int j = 0; j < FA; j++) fw[j] = *reinterpret_cast<const float4 *>(fr + fold_q * (K / 4) + (j * 64 + lane) * 4);
+#pragma unroll
+        for (int j = 0; j < FB; j++) fw[FA + j] = *reinterpret_cast<const float4 *>(fr + K + fold_q * (FN / 4) + (j * 64 + lane) * 4);
     }
 
     // ---- stage pro(x): thread i of the block takes columns 4*(i + T*j) .. +3 ----
@@ -356,7 +362,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
         ss = wave_sum_all(ss);
         if (lane == 0) red[wave] = ss;
     }
-    if constexpr (FOLD) *reinterpret_cast<float4 *>(&xs[lds_slot(K + 4 * tid)]) = fres;
     __syncthreads();
     float scale = 1.f;
     if constexpr (PRO == SHV_PRO_RMSNORM) {
@@ -405,10 +410,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
         // LDS and are added in a fixed order
         float acc = 0.f;
 #pragma unroll
-        for (int j = 0; j < FV; j++) {
-            const float4 xv4 = *reinterpret_cast<const float4 *>(&xs[lds_slot(fold_q * FQ + (j * 64 + lane) * 4)]);
+        for (int j = 0; j < FA; j++) {
+            const float4 xv4 = *reinterpret_cast<const float4 *>(&xs[lds_slot(fold_q * (K / 4) + (j * 64 + lane) * 4)]);
             acc = fmaf(fw[j].x, xv4.x, fmaf(fw[j].y, xv4.y, fmaf(fw[j].z, xv4.z, fmaf(fw[j].w, xv4.w, acc))));
         }
+#pragma unroll
+        for (int j = 0; j < FB; j++) acc = fmaf(fw[FA + j].x, fx[j].x, fmaf(fw[FA + j].y, fx[j].y, fmaf(fw[FA + j].z, fx[j].z, fmaf(fw[FA + j].w, fx[j].w, acc))));
         acc = wave_sum_all(acc);
         __syncthreads();  // red is free again: every wave has its scale
         if (lane == 0) red[wave] = acc;
@@ -421,11 +428,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
 // The one-row kernel's shape with the rows side by side: every row's inputs first, the weights of
 // the wave's passes once, each row staged with its sums, one block-wide wait, then the lane walks
 // the rows with its weights in registers (a row's 64 activations come from LDS when its turn comes).
-template <int K, int WAVES, int P, int PRO, int NT>
+template <int K, int WAVES, int P, int PRO, int NT, bool FOLD = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_args a) {
     constexpr int T = WAVES * 64, LPR = K / 64, RPP = 64 / LPR, ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     constexpr int NV = K / 4 / T;
     static_assert(NV >= 1 && K % (4 * T) == 0, "threads of a block each stage whole float4s");
+    // FOLD: the router's rows beside the block's own, as in the one-row kernel, against every row
+    constexpr int FN = 2048, FA = K / 4 / 256, FB = FN / 4 / 256;
+    static_assert(!FOLD || (WAVES == 8 && K % 1024 == 0), "a fold row is split over four waves");
     __shared__ __align__(16) float xs[NT][lds_padded(K)];
     __shared__ __align__(16) float xsum[NT][K / 32];
     __shared__ float red[NT][WAVES];
@@ -459,6 +469,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_a
             }
         }
     }
+    const int fold_row = static_cast<int>(blockIdx.x) * 2 + (wave >> 2), fold_q = wave & 3;
+    float4 fx[FOLD ? NT : 1][FOLD ? FB : 1];
+    if constexpr (FOLD) {
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int j = 0; j < FB; j++) fx[t][j] = *reinterpret_cast<const float4 *>(a.residual + static_cast<size_t>(t) * a.y_stride + fold_q * (FN / 4) + (j * 64 + lane) * 4);
+    }
     Q4kLane w[P];
     int row[P];
 #pragma unroll
@@ -473,6 +491,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_a
 #pragma unroll
         for (int u = 0; u < P; u++)
             res[t][u] = (a.residual && row[u] >= 0 && group_sum_owner<LPR>(lane)) ? a.residual[static_cast<size_t>(t) * a.y_stride + row[u]] : 0.f;
+    float4 fw[FOLD ? FA + FB : 1];
+    if constexpr (FOLD) {
+        const float *fr = a.fold + static_cast<size_t>(fold_row < a.fold_rows ? fold_row : 0) * (K + FN);
+#pragma unroll
+        for (int j = 0; j < FA; j++) fw[j] = *reinterpret_cast<const float4 *>(fr + fold_q * (K / 4) + (j * 64 + lane) * 4);
+#pragma unroll
+        for (int j = 0; j < FB; j++) fw[FA + j] = *reinterpret_cast<const float4 *>(fr + K + fold_q * (FN / 4) + (j * 64 + lane) * 4);
+    }
 
 #pragma unroll
     for (int t = 0; t < NT; t++) {
@@ -531,6 +557,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_a
             if (row[u] >= 0 && group_sum_owner<LPR>(lane)) y[row[u]] = fmaf(acc, scale, res[t][u]);
         }
     }
+    if constexpr (FOLD) {
+        float facc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < FA; j++) {
+                const float4 xv4 = *reinterpret_cast<const float4 *>(&xs[t][lds_slot(fold_q * (K / 4) + (j * 64 + lane) * 4)]);
+                acc = fmaf(fw[j].x, xv4.x, fmaf(fw[j].y, xv4.y, fmaf(fw[j].z, xv4.z, fmaf(fw[j].w, xv4.w, acc))));
+            }
+#pragma unroll
+            for (int j = 0; j < FB; j++) acc = fmaf(fw[FA + j].x, fx[t][j].x, fmaf(fw[FA + j].y, fx[t][j].y, fmaf(fw[FA + j].z, fx[t][j].z, fmaf(fw[FA + j].w, fx[t][j].w, acc))));
+            facc[t] = wave_sum_all(acc);
+        }
+        __syncthreads();  // red is free again: every wave has its scales
+        if (lane == 0) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) red[t][wave] = facc[t];
+        }
+        __syncthreads();
+        // a.fold_stride floats from one row's products to the next
+        if ((tid & 255) < NT && fold_row < a.fold_rows) {
+            const int t = tid & 255;
+            a.fold_out[static_cast<size_t>(t) * a.fold_stride + fold_row] = (red[t][wave] + red[t][wave + 1]) + (red[t][wave + 2] + red[t][wave + 3]);
+        }
+    }
 }
 
 template <int K, int WAVES, int P, int NT>
@@ -548,7 +600,19 @@ int launch_fewrows_kpn(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
 }
 
 template <int NT>
+int launch_fewrows_fold(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    constexpr int K = 4096, WAVES = 8;
+    const int rows_blocks = (a.n + WAVES - 1) / WAVES, fold_blocks = (a.fold_rows + 1) / 2;
+    const dim3 grid(static_cast<unsigned>(rows_blocks > fold_blocks ? rows_blocks : fold_blocks)), block(WAVES * 64);
+    if (a.prologue == SHV_PRO_GATED_NORM) SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, 1, SHV_PRO_GATED_NORM, NT, true>), grid, block, 0, a);
+    else if (a.prologue == SHV_PRO_MUL_SIGMOID) SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, 1, SHV_PRO_MUL_SIGMOID, NT, true>), grid, block, 0, a);
+    else SHV_LAUNCH(ctx, (gemv_fewrows_kernel<K, WAVES, 1, SHV_PRO_NONE, NT, true>), grid, block, 0, a);
+    return SHV_OK;
+}
+
+template <int NT>
 int launch_fewrows(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
+    if (a.fold) return launch_fewrows_fold<NT>(ctx, a);
     if (a.k == 4096) return launch_fewrows_kpn<4096, 8, 1, NT>(ctx, a);
     if (a.n <= 2 * 4 * 2 * ctx->prop.multiProcessorCount) return launch_fewrows_kpn<2048, 4, 1, NT>(ctx, a);
     return launch_fewrows_kpn<2048, 4, 2, NT>(ctx, a);
@@ -730,11 +794,14 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
                     "gemv_q4k: ring of %d slots, stride %d, sequences of %d in %d rows", a.ring_slots, a.ring_stride, sl, a.n_tok);
     }
     if (a.fold) {
-        SHV_REQUIRE(a.n_tok == 1 && a.k == 4096 && a.n == 2048 && a.residual && a.fold_out && a.fold_rows >= 1 && (a.ring_slots == 0 || a.z_ring),
-                    "gemv_q4k: the router's rows ride on a one-row 2048 x 4096 projection with a residual (n_tok %d, n %d, k %d)", a.n_tok, a.n, a.k);
+        SHV_REQUIRE(a.n_tok >= 1 && a.n_tok <= 4 && a.k == 4096 && a.n == 2048 && a.residual && a.fold_out && a.fold_rows >= 1 && (a.ring_slots == 0 || a.z_ring),
+                    "gemv_q4k: the router's rows ride on a 2048 x 4096 projection of one to four rows with a residual (n_tok %d, n %d, k %d)", a.n_tok, a.n, a.k);
         SHV_REQUIRE(a.prologue == SHV_PRO_NONE || a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID, "gemv_q4k: fold with prologue %d", a.prologue);
-        SHV_REQUIRE(a.residual != a.y && shv_aligned16(a.residual) && shv_aligned16(a.fold), "gemv_q4k: fold reads the whole residual row while y is written: they must be different, 16-byte aligned buffers");
-        SHV_REQUIRE(row_kernel_covers(ctx, a) && !ctx->gemv_scales_lds, "gemv_q4k: fold needs the one-row kernel's alignment of x, gamma and z");
+        SHV_REQUIRE(a.residual != a.y && shv_aligned16(a.residual) && shv_aligned16(a.fold) && a.y_stride % 4 == 0,
+                    "gemv_q4k: fold reads the whole residual row while y is written: they must be different, 16-byte aligned buffers");
+        SHV_REQUIRE(a.n_tok == 1 || a.fold_stride >= a.fold_rows, "gemv_q4k: fold_stride %d < fold_rows %d", a.fold_stride, a.fold_rows);
+        SHV_REQUIRE(!ctx->gemv_scales_lds && !ctx->mfma_rows_forced && (a.n_tok == 1 ? row_kernel_covers(ctx, a) : fewrows_kernel_covers(ctx, a)),
+                    "gemv_q4k: fold needs the row kernels' shapes and alignment of x, gamma and z (rows of one sequence)");
     }
     // two to four rows of one sequence: the one-row kernel's shape with the rows side by side (SHV_MFMA_MIN_ROWS
     // at or below the row count sends them to the matrix cores instead, as before)

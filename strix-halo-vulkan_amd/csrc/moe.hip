@@ -973,9 +973,9 @@ int shv_launch_moe_up(shv_ctx *ctx, const shv_moe_up_args *pa) {
     SHV_REQUIRE(a.ffn >= 1, "moe_up: ffn %d", a.ffn);
     SHV_REQUIRE(!a.shared_gate || (a.gamma && shv_aligned16(a.shared_gate)), "moe_up: shared_gate goes with gamma (the row normalised inside the launch), 16-byte aligned");
     if (a.gamma)
-        SHV_REQUIRE(a.logits && a.n_tok == 1 && a.n_embd == 2048 && shv_aligned16(a.gamma) && shv_aligned16(a.xn) && is_q4k(a.gate_type) && is_q4k(a.up_type) &&
+        SHV_REQUIRE(a.logits && a.n_tok <= 4 && a.n_embd == 2048 && shv_aligned16(a.gamma) && shv_aligned16(a.xn) && is_q4k(a.gate_type) && is_q4k(a.up_type) &&
                         is_q4k(a.gate_sh_type) && is_q4k(a.up_sh_type),
-                    "moe_up: the RMSNorm of the row inside the launch (gamma) goes with logits, one row of 2048 and Q4_K banks");
+                    "moe_up: the RMSNorm of the row inside the launch (gamma) goes with logits, one to four rows of 2048 and Q4_K banks");
     ctx->moe_stamp = {};  // only the grouped launch leaves lists or operands behind, and says so itself
     // Banks of other types than Q4_K go through their own arms; a block whose routed banks and
     // shared expert differ in that takes one launch each, over its part of the slots.

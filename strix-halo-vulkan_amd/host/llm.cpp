@@ -581,11 +581,13 @@ void MoEGPU::FoldInto(int l, PassRows &r) const {
     r.fold = fold_[l];
     r.fold_rows = c_.NExpert;  // the shared gate's row stays behind: gate/up forms that product from the row it stages
     r.fold_out = logits_;
+    r.fold_stride = c_.NExpert + 1;
 }
 
-std::vector<shv_op> MoEGPU::DispatchesFolded(int l, const float *in, float *out, std::vector<std::string> *labels) const {
+std::vector<shv_op> MoEGPU::DispatchesFolded(int l, const float *in, float *out, int nTok, std::vector<std::string> *labels) const {
     if (!Folded(l)) throw Error("llm: MoEGPU: layer " + std::to_string(l) + " has no folded router");
-    auto ops = Dispatches(l, in, out, 1, nullptr);
+    if (nTok < 1 || nTok > kFoldRows || !FusedRouter(nTok)) throw Error("llm: MoEGPU: a pass of " + std::to_string(nTok) + " rows makes its selection in a launch of its own");
+    auto ops = Dispatches(l, in, out, nTok, nullptr);
     // the router's launch goes; gate/up takes the row as it is and normalises it itself
     shv_moe_up_args u{};
     std::memcpy(&u, ops[1].args, sizeof u);
@@ -792,6 +794,7 @@ std::vector<shv_op> DeltaNetGPU::Dispatches(int l, const float *in, float *out, 
     o.fold = r.fold;
     o.fold_rows = r.fold_rows;
     o.fold_out = r.fold_out;
+    o.fold_stride = r.fold_stride;
     if (flat) {
         o.z = row_ + c_.ConvWidth();  // the z columns of the projection row
         o.z_stride = width;
@@ -1018,6 +1021,7 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, cons
     o.fold = r.fold;
     o.fold_rows = r.fold_rows;
     o.fold_out = r.fold_out;
+    o.fold_stride = r.fold_stride;
     if (labels) labels->insert(labels->end(), {"attn.qkv", "attn.attn", "attn.out"});
     return {make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_ATTN_DECODE, a), make_op(SHV_OP_GEMV_Q4K, o)};
 }
@@ -1173,7 +1177,7 @@ Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_
     // LLM_ROUTER_FOLD=0 keeps the router's own launch.
     const char *rf = std::getenv("LLM_ROUTER_FOLD");
     if (!(rf && rf[0] == '0')) {
-        x2_ = static_cast<float *>(dev.alloc(static_cast<size_t>(c_.NEmbd) * 4));
+        x2_ = static_cast<float *>(dev.alloc(static_cast<size_t>(MoEGPU::kFoldRows) * c_.NEmbd * 4));
         for (int l = 0; l < layers_; l++) moe_->Fold(l, m.Tensor(Model::Blk(l, c_.IsAttn(l) ? "attn_output" : "ssm_out")));
     }
     // the decode step of slot 0 is recorded up front, as NewGraph does (llm/graph.go:609)
@@ -1232,14 +1236,15 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     p.labels.push_back("embed");
     if (rows > kBlockRows && (kind == kBatch || spec)) throw Error("llm: a pass of " + std::to_string(rows) + " rows is a plain prompt pass; batched and rewindable passes carry up to " + std::to_string(kBlockRows));
     for (int l = 0; l < layers_; l++) {
-        if (rows == 1 && x2_ && moe_->Folded(l)) {
+        // (rows of one sequence: a batch of several sequences' rows goes through other projection kernels)
+        if (x2_ && moe_->Folded(l) && (rows == 1 || (kind != kBatch && rows <= MoEGPU::kFoldRows && moe_->FusedRouter(rows)))) {
             // the mixer writes the row beside the stream (its output projection reads the whole
             // residual row for the router's products while it writes), the MoE block brings it back
             PassRows rf = r;
             moe_->FoldInto(l, rf);
             auto sub = c_.IsAttn(l) ? attn_->Dispatches(l, x_, x2_, rf, &p.labels) : dn_->Dispatches(l, x_, x2_, rf, &p.labels);
             p.ops.insert(p.ops.end(), sub.begin(), sub.end());
-            auto ffn = moe_->DispatchesFolded(l, x2_, x_, &p.labels);
+            auto ffn = moe_->DispatchesFolded(l, x2_, x_, rows, &p.labels);
             p.ops.insert(p.ops.end(), ffn.begin(), ffn.end());
             continue;
         }

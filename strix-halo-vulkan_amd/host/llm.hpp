@@ -181,11 +181,11 @@ struct PassRows {
                                     // a dependent load of the slot word
     int n_seq = 1, seq_len = 1;
     bool spec = false;              // DeltaNet: a rewindable pass (state goes to the other planes)
-    // A one-row pass whose mixer's output projection also forms the logits of the layer's router
+    // A pass of one to four rows of a sequence whose mixer's output projection also forms the logits of the layer's router
     // (MoEGPU::Fold): the table's rows, how many, and where the products go.  out must then be
     // another buffer than in.
     const float *fold = nullptr;
-    int fold_rows = 0;
+    int fold_rows = 0, fold_stride = 0;
     float *fold_out = nullptr;
     int rows() const { return n_seq * seq_len; }
 };
@@ -213,7 +213,8 @@ public:
     void FoldInto(int layer, PassRows &r) const;
     // The block on a one-row pass whose logits came with the output projection: gate/up (which
     // normalises the row itself) and down.  `in` is the row before its RMSNorm.
-    std::vector<shv_op> DispatchesFolded(int layer, const float *in, float *out, std::vector<std::string> *labels) const;
+    std::vector<shv_op> DispatchesFolded(int layer, const float *in, float *out, int nTok, std::vector<std::string> *labels) const;
+    static constexpr int kFoldRows = 4;  // rows of one sequence the fused launches take
     std::vector<float> Logits() const;    // [T][NExpert+1]
     std::vector<int32_t> TopK() const;    // [T][used]
     std::vector<float> Weights() const;   // [T][used+1]

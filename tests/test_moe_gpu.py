@@ -498,6 +498,50 @@ def test_router_rows_ride_on_the_output_projection(ctx, full_bank, prologue, E, 
     g.y = dx.ptr
     with pytest.raises(A.ShvError, match="different"):
         c.enqueue(A.OP_GEMV_Q4K, g)
-    ua.n_tok = 2
-    with pytest.raises(A.ShvError, match="one row"):
+    ua.n_tok = 5
+    with pytest.raises(A.ShvError, match="four rows"):
         c.enqueue(A.OP_MOE_UP, ua)
+
+
+@pytest.mark.parametrize("T", [2, 3])
+def test_router_rows_ride_on_a_projection_of_a_few_rows(ctx, T):
+    """The same for two and three rows of one sequence (a verification pass): the rows-side-by-side
+    projection kernel forms every row's products, the gate/up kernel normalises each row itself."""
+    E, used = 64, 10
+    case = MoeCase(ctx, seed=91, E=E, used=used, T=T)
+    H, K, ffn, c = case.H, 4096, case.ffn, ctx
+    rng = np.random.default_rng(600 + T)
+    w = O.quantize_q4k((rng.standard_normal((H, K)) * 0.02).astype(np.float32))
+    v = rng.standard_normal((T, K)).astype(np.float32)
+    z = rng.standard_normal((T, K)).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    pv = v.astype(np.float64) / (1 + np.exp(-z.astype(np.float64)))
+    h = (x.astype(np.float64) + pv @ O.dequant_q4k(w, K).astype(np.float64).T).astype(np.float32)
+    case.h, case.res = h, np.zeros((T, H), np.float32)
+    want = case.oracle()
+    d = {k: c.upload(getattr(case, k)) for k in ("router", "shared_gate", "gate_exps", "up_exps", "down_exps", "gate_sh", "up_sh", "down_sh", "gamma")}
+    dw, dv, dx, dz = c.upload(w), c.upload(v), c.upload(x), c.upload(z)
+    table, scratch = c.alloc(E * (K + H) * 4), c.alloc(H * K * 4)
+    c.enqueue(A.OP_ROUTER_FOLD, A.RouterFoldArgs(d["router"].ptr, None, d["gamma"].ptr, dw.ptr, table.ptr, scratch.ptr, E, H, K))
+    y, raw = c.alloc(T * H * 4), c.alloc(T * (E + 1) * 4)
+    topk, weights, act, out = c.alloc(T * used * 4), c.alloc(T * (used + 1) * 4), c.alloc(T * (used + 1) * ffn * 4), c.alloc(T * H * 4)
+    g = A.gemv_args(dw, dv, y, H, K, T, A.PRO_MUL_SIGMOID, None, dz, dx, EPS, 0)
+    g.fold, g.fold_out, g.fold_rows, g.fold_stride = table.ptr, raw.ptr, E, E + 1
+    ua = A.MoeUpArgs(y.ptr, topk.ptr, d["gate_exps"].ptr, d["up_exps"].ptr, d["gate_sh"].ptr, d["up_sh"].ptr, act.ptr, T, H, used, ffn,
+                     raw.ptr, weights.ptr, E, 0, 0, 0, 0, None, 0, 0, d["gamma"].ptr, EPS, d["shared_gate"].ptr)
+    da = A.MoeDownArgs(act.ptr, topk.ptr, weights.ptr, d["down_exps"].ptr, d["down_sh"].ptr, y.ptr, out.ptr, T, H, used, ffn, H, H, 0, 0, E, None, None)
+    c.dispatch_multi([A.make_op(A.OP_GEMV_Q4K, g), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)])
+    got_h = y.read(np.float32, T * H).reshape(T, H)
+    assert O.rel_l2(got_h, h) <= 1e-5
+    scale = 1.0 / np.sqrt((h.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + EPS)
+    got_lg = raw.read(np.float32, T * (E + 1)).reshape(T, E + 1)[:, :E].astype(np.float64) * scale
+    assert O.rel_l2(got_lg, want["logits"]) <= 2e-5
+    tk = topk.read(np.int32, T * used).reshape(T, used)
+    for t in range(T):
+        lg = want["logits"][t].astype(np.float64)
+        p = np.exp(lg - lg.max())
+        assert _margin(p / p.sum(), used) > 1e-4, "seed sits on a near-tie; pick another"
+    assert np.array_equal(tk, want["topk"])
+    wt = weights.read(np.float32, T * (used + 1)).reshape(T, used + 1)
+    assert O.rel_l2(wt[:, :used], want["weights"]) <= 1e-5 and O.rel_l2(wt[:, used], want["sig"]) <= 1e-5
+    assert O.rel_l2(out.read(np.float32, T * H).reshape(T, H), want["out"] + h) <= TOL
