@@ -148,6 +148,14 @@ typedef struct {
     float *fold_out;
     int32_t fold_rows;
     int32_t fold_stride;     /* two to four rows of one sequence: row t's products go to fold_out + t * fold_stride */
+    /* The greedy sampler in the same launch (one row; the vocabulary projection of a decode step):
+     * what shv_argmax does with its best / ids / pos / advance over y[0..n) is done by the block
+     * of this launch that finishes last (Argmax, llm/sample.go:359-367: first maximum, NaN never
+     * wins).  amax_best NULL: no arg-max. */
+    int32_t *amax_best;
+    int32_t *amax_ids;
+    int32_t *amax_pos;
+    int32_t amax_advance;
 } shv_gemv_q4k_args;
 
 /* The table shv_gemv_q4k's `fold` reads, for one layer: out [rows][k + n_embd] float32,

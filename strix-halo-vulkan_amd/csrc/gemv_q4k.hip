@@ -53,9 +53,11 @@ struct GemvBatch {
         }
     }
 
+    // AMAX: the lane also keeps the best (value, row) of what it stores (one row of activations)
+    template <bool AMAX = false>
     __device__ __forceinline__ void compute(const shv_gemv_q4k_args &a, int g, int lane, const NibbleConsts &nc,
                                             const float (*xr)[64], const float *xs_lo, const float *xs_hi,
-                                            const size_t *y_off, int t0) const {
+                                            const size_t *y_off, int t0, float *bv = nullptr, int *bi = nullptr) const {
 #pragma unroll
         for (int u = 0; u < U; u++) {
 #pragma unroll
@@ -67,6 +69,9 @@ struct GemvBatch {
                     if (a.residual) r += res[u][t];
                     a.y[y_off[t] + row[u]] = r;
                     if (a.y_flat) a.y_flat[row[u]] = r;  // one row (the launcher checks)
+                    if constexpr (AMAX) {
+                        if (amax_better(r, row[u], *bv, *bi)) { *bv = r; *bi = row[u]; }
+                    }
                 }
             }
         }
@@ -76,8 +81,11 @@ struct GemvBatch {
 // The grid's waves share the passes round-robin: wave w takes passes w, w + W, w + 2W, ... (W waves
 // in the grid), so at any moment the chip streams one contiguous window of rows and no wave has
 // more than one pass more than another.  U passes are loaded together; n_batches batches a wave.
-template <int K, int NT, int U>
-__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int n_batches, int t0) {
+// AMAX (one row): every block leaves the best (value, row) of the rows it wrote, and the block that
+// arrives last names the row's first maximum as the next token, as the arg-max launch would.
+template <int K, int NT, int U, bool AMAX = false>
+__global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, int n_batches, int t0, float *amax_val = nullptr,
+                                                          int32_t *amax_idx = nullptr, int32_t *amax_counter = nullptr) {
     constexpr int LPR = K / 64;   // lanes per row
     constexpr int XPAD = K + K / 64 * 4;
     extern __shared__ float smem[];
@@ -228,13 +236,55 @@ __global__ __launch_bounds__(kBlock) void gemv_q4k_kernel(shv_gemv_q4k_args a, i
 
     const NibbleConsts nc = nibble_consts();
     const int nb = n_batches;  // double-buffered
+    // "no candidate" is (-inf, n): any real element beats it, including -inf at a lower index
+    float bv = -INFINITY;
+    int bi = n;
     for (int b = 0; b < nb; b += 2) {
         const bool has_b = b + 1 < nb;
         if (has_b) B.load(a, wbase, g, rsub, lane, first_pass + static_cast<long long>(b + 1) * U * stride, stride, n, t0);
-        A.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
+        A.template compute<AMAX>(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0, &bv, &bi);
         if (has_b) {
             if (b + 2 < nb) A.load(a, wbase, g, rsub, lane, first_pass + static_cast<long long>(b + 2) * U * stride, stride, n, t0);
-            B.compute(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0);
+            B.template compute<AMAX>(a, g, lane, nc, xr, xs_lo, xs_hi, y_off, t0, &bv, &bi);
+        }
+    }
+    if constexpr (AMAX) {
+        __shared__ float sv[kWavesPerBlock];
+        __shared__ int si[kWavesPerBlock];
+        __shared__ int is_last;
+        const int nblk = static_cast<int>(gridDim.x);
+        amax_wave(bv, bi);
+        if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+        __syncthreads();
+        if (tid == 0) {
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; w++)
+                if (amax_better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+            store_agent(amax_val + blockIdx.x, bv);
+            store_agent(amax_idx + blockIdx.x, bi);
+        }
+        if (!arrive_last(amax_counter, nblk, &is_last)) return;
+        bv = -INFINITY;
+        bi = n;
+        for (int b = tid; b < nblk; b += kBlock) {
+            const float v = load_agent(amax_val + b);
+            const int i = load_agent(amax_idx + b);
+            if (amax_better(v, i, bv, bi)) { bv = v; bi = i; }
+        }
+        amax_wave(bv, bi);
+        if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+        __syncthreads();
+        if (tid == 0) {
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; w++)
+                if (amax_better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+            if (bi >= n) bi = 0;  // a row of NaN has no element that is `>` -inf: the reference returns 0 there
+            a.amax_best[0] = bi;
+            if (a.amax_ids && a.amax_pos) {
+                const int p = a.amax_pos[0] + (a.amax_advance > 0 ? a.amax_advance : 1);
+                a.amax_ids[p] = bi;
+                a.amax_pos[0] = p;
+            }
         }
     }
 }
@@ -700,7 +750,16 @@ int launch_ntu(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, 
             raised = true;
         }
     }
-    SHV_LAUNCH(ctx, (gemv_q4k_kernel<K, NT, U>), grid, block, lds, a, ppw, t0);
+    if constexpr (NT == 1) {
+        if (a.amax_best) {
+            SHV_REQUIRE(grid.x <= static_cast<unsigned>(shv_ctx::kGemvAmaxBlocks) && ctx->gemv_amax_val && ctx->gemv_amax_idx, "gemv_q4k: arg-max over %u blocks", grid.x);
+            if (lds > 48 * 1024) SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_kernel<K, NT, U, true>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            SHV_LAUNCH(ctx, (gemv_q4k_kernel<K, NT, U, true>), grid, block, lds, a, ppw, t0, ctx->gemv_amax_val, ctx->gemv_amax_idx,
+                       ctx->counters + shv_ctx::kCounterGemvAmax);
+            return SHV_OK;
+        }
+    }
+    SHV_LAUNCH(ctx, (gemv_q4k_kernel<K, NT, U>), grid, block, lds, a, ppw, t0, static_cast<float *>(nullptr), static_cast<int32_t *>(nullptr), static_cast<int32_t *>(nullptr));
     return SHV_OK;
 }
 
@@ -802,6 +861,17 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
         SHV_REQUIRE(a.n_tok == 1 || a.fold_stride >= a.fold_rows, "gemv_q4k: fold_stride %d < fold_rows %d", a.fold_stride, a.fold_rows);
         SHV_REQUIRE(!ctx->gemv_scales_lds && !ctx->mfma_rows_forced && (a.n_tok == 1 ? row_kernel_covers(ctx, a) : fewrows_kernel_covers(ctx, a)),
                     "gemv_q4k: fold needs the row kernels' shapes and alignment of x, gamma and z (rows of one sequence)");
+    }
+    if (a.amax_best) {
+        SHV_REQUIRE(a.n_tok == 1 && a.ring_slots == 0 && !a.fold && !a.residual, "gemv_q4k: the arg-max in the launch goes with one plain row of outputs");
+        SHV_REQUIRE((a.amax_ids == nullptr) == (a.amax_pos == nullptr) && a.amax_advance >= 0, "gemv_q4k: amax_ids and amax_pos go together");
+        switch (a.k) {  // straight to the looping kernel: the short launches' kernel has no arg-max
+            case 512: return launch_k<512>(ctx, a);
+            case 1024: return launch_k<1024>(ctx, a);
+            case 2048: return launch_k<2048>(ctx, a);
+            case 4096: return launch_k<4096>(ctx, a);
+            default: return shv_set_error(SHV_E_INVALID, "gemv_q4k: k = %d; built for 512, 1024, 2048 and 4096", a.k);
+        }
     }
     // two to four rows of one sequence: the one-row kernel's shape with the rows side by side (SHV_MFMA_MIN_ROWS
     // at or below the row count sends them to the matrix cores instead, as before)

@@ -69,6 +69,8 @@ int shv_init(int device, shv_ctx **out) {
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->gemm_part), shv_ctx::kGemmPartBytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_val), shv_ctx::kArgmaxBlocks * sizeof(float));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_idx), shv_ctx::kArgmaxBlocks * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->gemv_amax_val), shv_ctx::kGemvAmaxBlocks * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->gemv_amax_idx), shv_ctx::kGemvAmaxBlocks * sizeof(int32_t));
     if (e != hipSuccess) {
         shv_destroy(ctx);
         return shv_set_error(SHV_E_HIP, "shv_init: %s", hipGetErrorString(e));
@@ -99,6 +101,8 @@ void shv_destroy(shv_ctx *ctx) {
     if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
     if (ctx->argmax_val) (void)hipFree(ctx->argmax_val);
     if (ctx->argmax_idx) (void)hipFree(ctx->argmax_idx);
+    if (ctx->gemv_amax_val) (void)hipFree(ctx->gemv_amax_val);
+    if (ctx->gemv_amax_idx) (void)hipFree(ctx->gemv_amax_idx);
     for (hipEvent_t ev : ctx->mark_pool) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);

@@ -280,6 +280,18 @@ __device__ __forceinline__ bool arrive_last(int32_t *counter, int expected, int 
     return *lds_flag != 0;
 }
 
+// ---- greedy arg-max: (value, index) pairs ordered so that the larger value wins and, between
+// equal values, the lower index; NaN never wins (Argmax, llm/sample.go:359-367) ------------------
+__device__ __forceinline__ bool amax_better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+__device__ __forceinline__ void amax_wave(float &v, int &i) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(v, off, 64);
+        const int oi = __shfl_xor(i, off, 64);
+        if (amax_better(ov, oi, v, i)) { v = ov; i = oi; }
+    }
+}
+
 __device__ __forceinline__ float sigmoid_exact(float x) { return 1.f / (1.f + expf(-x)); }
 
 // Sigmoid through the hardware exp2 and reciprocal, a few units in the last place from the exact

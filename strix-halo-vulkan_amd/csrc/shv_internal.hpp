@@ -47,6 +47,10 @@ struct shv_ctx {
     float *argmax_val = nullptr;
     int32_t *argmax_idx = nullptr;
     enum { kArgmaxBlocks = 512 };
+    // the same for the arg-max a vocabulary projection makes in its own launch: one pair a block
+    float *gemv_amax_val = nullptr;
+    int32_t *gemv_amax_idx = nullptr;
+    enum { kGemvAmaxBlocks = 2048 };
     // device address of this GPU's copy of the library's static scratch array (misc.hip), for the
     // entry point that allocates nothing
     void *static_scratch = nullptr;
@@ -72,7 +76,7 @@ struct shv_ctx {
         *e = mark_pool[i + 1];
         return hipSuccess;
     }
-    enum { kCounterRouter = 0, kCounterArgmax = 1, kCounterAttn = 16 };
+    enum { kCounterRouter = 0, kCounterArgmax = 1, kCounterAttn = 16, kCounterGemvAmax = 15 };
     // What the last shv_moe_up on this context left behind for the shv_moe_down that follows it:
     // the pass its per-expert lists in `group` belong to, and whether act holds matrix-core
     // operands instead of floats.  shv_moe_down believes its group_ready / act_packed flags only

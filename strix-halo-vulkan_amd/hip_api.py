@@ -37,7 +37,8 @@ class GemvQ4KArgs(C.Structure):
                 ("head_dim", C.c_int32), ("eps", C.c_float), ("x_stride", C.c_int32),
                 ("y_stride", C.c_int32), ("z_stride", C.c_int32), ("seq_len", C.c_int32),
                 ("ring_slots", C.c_int32), ("ring_stride", C.c_int32), ("z_ring", C.c_int32),
-                ("y_flat", C.c_void_p), ("fold", C.c_void_p), ("fold_out", C.c_void_p), ("fold_rows", C.c_int32), ("fold_stride", C.c_int32)]
+                ("y_flat", C.c_void_p), ("fold", C.c_void_p), ("fold_out", C.c_void_p), ("fold_rows", C.c_int32), ("fold_stride", C.c_int32),
+                ("amax_best", C.c_void_p), ("amax_ids", C.c_void_p), ("amax_pos", C.c_void_p), ("amax_advance", C.c_int32)]
 
 
 class RouterFoldArgs(C.Structure):

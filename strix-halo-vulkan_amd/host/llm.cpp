@@ -1287,11 +1287,24 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
         case kSample: {
             if (!head_) throw Error("llm: this graph was staged without a head");
             auto h = head_->Dispatches(x_ + static_cast<size_t>(rows - 1) * c_.NEmbd, 1, &p.labels);
-            p.ops.insert(p.ops.end(), h.begin(), h.end());
             am.ids = ids_ + slot * ids_stride_;
             am.pos = pos_ + slot;
             am.n_rows = 1;
             am.advance = rows;
+            // The vocabulary projection names the next token itself: its last block to finish does
+            // what the arg-max launch would (LLM_HEAD_ARGMAX=0 keeps that launch).
+            const char *ha = std::getenv("LLM_HEAD_ARGMAX");
+            if (!(ha && ha[0] == '0') && h.size() == 1 && h[0].kind == SHV_OP_GEMV_Q4K) {
+                shv_gemv_q4k_args g{};
+                std::memcpy(&g, h[0].args, sizeof g);
+                g.amax_best = am.best;
+                g.amax_ids = am.ids;
+                g.amax_pos = am.pos;
+                g.amax_advance = am.advance;
+                p.ops.push_back(make_op(SHV_OP_GEMV_Q4K, g));
+                break;
+            }
+            p.ops.insert(p.ops.end(), h.begin(), h.end());
             p.ops.push_back(make_op(SHV_OP_ARGMAX, am));
             p.labels.push_back("argmax");
             break;

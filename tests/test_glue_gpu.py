@@ -90,3 +90,53 @@ def test_embedding_gather_from_a_table_of_any_type(ctx, name):
             assert np.isnan(got[t, :H]).all()
     with pytest.raises(A.ShvError, match="embed: a row of 100 elements"):
         ctx.enqueue(A.OP_EMBED, A.EmbedArgs(ctx.upload(raw).ptr, ctx.upload(ids).ptr, None, d_x.ptr, 1, 100, vocab, 100, 12))
+
+
+def test_vocabulary_projection_names_the_next_token_itself(ctx):
+    """shv_gemv_q4k with amax_best: the launch's last block does what shv_argmax does over the row
+    the launch wrote — first maximum, ties to the lower id, NaN never wins, the next token stored
+    and the position advanced — and the logits are the plain launch's bit for bit.  Twice in a
+    row, so that the arrival counter is seen to re-arm."""
+    rng = np.random.default_rng(12)
+    n, k = 151936, 2048
+    f = ctx.alloc(n * k * 4)
+    ctx.enqueue(A.OP_FILL_NORMAL, A.FillNormalArgs(f.ptr, n * k, 99, 0.0, 0.02))
+    w = ctx.alloc(n * (k // 256 * 144))
+    ctx.enqueue(A.OP_QUANTIZE_Q4K, A.QuantizeQ4KArgs(f.ptr, w.ptr, n, k))
+    ctx.sync()
+    f.free()
+    # rows 100 and 7000 become copies of row 140000: three equal logits, the lowest id must win if they are the maximum
+    rb = k // 256 * 144
+    wb = w.read(np.uint8, n * rb).reshape(n, rb)
+    wb[100] = wb[140000]
+    wb[7000] = wb[140000]
+    w.write(wb)
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    d_gamma = ctx.upload(gamma)
+    y0, y1, best = ctx.alloc(n * 4), ctx.alloc(n * 4), ctx.alloc(4)
+    ids, pos = ctx.upload(np.full(16, -1, np.int32)), ctx.upload(np.array([3], np.int32))
+    row140k = O.dequant_q4k(wb[140000:140001], k)[0]
+    for trial, x in enumerate((rng.standard_normal(k).astype(np.float32), (row140k / gamma * 50).astype(np.float32))):
+        dx = ctx.upload(x)
+        ctx.gemv_q4k(w, dx, y0, n, k, prologue=A.PRO_RMSNORM, gamma=d_gamma)
+        g = A.gemv_args(w, dx, y1, n, k, 1, A.PRO_RMSNORM, d_gamma)
+        g.amax_best, g.amax_ids, g.amax_pos, g.amax_advance = best.ptr, ids.ptr, pos.ptr, 1 + trial
+        ctx.enqueue(A.OP_GEMV_Q4K, g)
+        lg = y0.read(np.float32, n)
+        assert np.array_equal(lg, y1.read(np.float32, n))
+        want = int(np.argmax(lg))
+        assert best.read(np.int32, 1)[0] == want
+        if trial == 1:
+            assert want == 100, "the row aligned with x should win, at its lowest copy"
+    got_ids = list(ids.read(np.int32, 8))
+    assert got_ids[:4] == [-1] * 4 and got_ids[4] >= 0 and got_ids[5] == -1 and got_ids[6] == 100 and got_ids[7] == -1
+    assert pos.read(np.int32, 1)[0] == 6
+    # NaN in, NaN out everywhere: nothing is `>` -inf and the reference returns 0
+    x = np.full(k, np.nan, np.float32)
+    g = A.gemv_args(w, ctx.upload(x), y1, n, k, 1, A.PRO_RMSNORM, d_gamma)
+    g.amax_best = best.ptr
+    ctx.enqueue(A.OP_GEMV_Q4K, g)
+    assert best.read(np.int32, 1)[0] == 0
+    with pytest.raises(A.ShvError, match="one plain row"):
+        g.n_tok = 2
+        ctx.enqueue(A.OP_GEMV_Q4K, g)
