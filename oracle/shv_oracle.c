@@ -881,9 +881,11 @@ void shv_ref_rope(const shv_ref_attn_cfg *c, float *x, const int32_t *pos, int n
 
 /* llm/attn.go:135-219 (dense arm) + attention :444-496, generalised to a cache that already
  * holds `past` cells: the row at position p sees cells 0..p. */
-void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn,
-                        int n_tok, int past, uint16_t *kcache, uint16_t *vcache, float *out,
-                        float *q_rot, float *pregate_t, int threads) {
+/* allow: NULL (dense), or [n_tok][past + n_tok] bytes, the selection of llm/attn.go:423-443: a
+ * cell it leaves out is unreadable however visible the causal mask says it is. */
+static void attn_layer_core(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn,
+                            int n_tok, int past, uint16_t *kcache, uint16_t *vcache, float *out,
+                            float *q_rot, float *pregate_t, const uint8_t *allow, int threads) {
     int H = c->n_embd, nh = c->n_head, nkv = c->n_head_kv, d = c->head_dim;
     int qw = nh * d * 2, gw = nh * d, kvw = nkv * d;
     size_t T = (size_t)n_tok;
@@ -923,15 +925,18 @@ void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, cons
 #pragma omp parallel for collapse(2) num_threads(threads > 1 ? threads : 1) schedule(dynamic, 1)
     for (int i = 0; i < n_tok; i++) {
         for (int h = 0; h < nh; h++) {
-            int n = past + i + 1;
-            float *scores = (float *)malloc(sizeof(float) * n);
+            int cells = past + i + 1;
+            const uint8_t *al = allow ? allow + (size_t)i * (past + n_tok) : NULL;
+            float *scores = (float *)malloc(sizeof(float) * cells);
             int kvh = h / rep;
             const float *qv = Q + ((size_t)i * nh + h) * d;
-            for (int j = 0; j < n; j++) {
+            int n = 0;
+            for (int j = 0; j < cells; j++) {
+                if (al && !al[j]) continue;
                 const uint16_t *kv = kcache + ((size_t)j * nkv + kvh) * d;
                 float s = 0;
                 for (int x = 0; x < d; x++) s += qv[x] * shv_ref_f16_to_f32(kv[x]);
-                scores[j] = s * scale;
+                scores[n++] = s * scale;
             }
             float max = scores[0];
             for (int j = 1; j < n; j++)
@@ -942,8 +947,10 @@ void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, cons
                 sum += scores[j];
             }
             float *dst = pre + ((size_t)i * nh + h) * d;
-            for (int j = 0; j < n; j++) {
-                float wgt = scores[j] / sum;
+            n = 0;
+            for (int j = 0; j < cells; j++) {
+                if (al && !al[j]) continue;
+                float wgt = scores[n++] / sum;
                 const uint16_t *vv = vcache + ((size_t)j * nkv + kvh) * d;
                 for (int x = 0; x < d; x++) dst[x] += wgt * shv_ref_f16_to_f32(vv[x]);
             }
@@ -956,6 +963,164 @@ void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, cons
     for (int i = 0; i < n_tok; i++)
         shv_ref_gemv_q4k(out + (size_t)i * H, w->o, pre + (size_t)i * gw, H, gw, threads);
     free(pre); free(pos); free(V); free(K); free(G); free(Q); free(qfull);
+}
+
+void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn,
+                        int n_tok, int past, uint16_t *kcache, uint16_t *vcache, float *out,
+                        float *q_rot, float *pregate_t, int threads) {
+    attn_layer_core(c, w, xn, n_tok, past, kcache, vcache, out, q_rot, pregate_t, NULL, threads);
+}
+
+/* ---------------------------------------------------- block-sparse indexer --- */
+
+/* llm/attn.go:672-682 */
+uint32_t shv_ref_f2ui(float v) {
+    uint32_t y = f32_bits(v);
+    if (y & 0x80000000u) return y ^ 0xFFFFFFFFu;
+    return y | 0x80000000u;
+}
+
+/* llm/attn.go:637-670 */
+uint32_t shv_ref_topk_threshold(const float *x, int len, int n) {
+    uint32_t histo[256];
+    uint32_t prefix = 0, desired = (uint32_t)n;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        memset(histo, 0, sizeof histo);
+        uint32_t hi_mask = 0;
+        if (shift + 8 < 32) hi_mask = 0xFFFFFFFFu << (unsigned)(shift + 8);
+        uint32_t prefix_hi = prefix & hi_mask;
+        for (int i = 0; i < len; i++) {
+            uint32_t key = shv_ref_f2ui(x[i]);
+            if ((key & hi_mask) == prefix_hi) histo[(key >> (unsigned)shift) & 255]++;
+        }
+        uint32_t acc = 0, b = 0;
+        for (int bb = 255; bb >= 0; bb--) {
+            uint32_t cnt = histo[bb];
+            if (acc + cnt >= desired) { b = (uint32_t)bb; break; }
+            acc += cnt;
+        }
+        prefix |= b << (unsigned)shift;
+        desired -= acc;
+    }
+    return prefix;
+}
+
+/* llm/attn.go:615-632 */
+int shv_ref_topk(const float *x, int len, int n, int32_t *sel) {
+    uint32_t thr = shv_ref_topk_threshold(x, len, n);
+    int m = 0;
+    for (int i = 0; i < len; i++)
+        if (shv_ref_f2ui(x[i]) > thr) sel[m++] = i;
+    int above = m;
+    for (int i = 0; i < len && m < n; i++)
+        if (shv_ref_f2ui(x[i]) == thr) sel[m++] = i;
+    return above;
+}
+
+/* llm/attn.go:231-421 at cell positions past..past+n_tok-1 of a sequence whose earlier raw keys
+ * are in idxcache; fills allow [n_tok][past+n_tok] (llm/attn.go:423-443). */
+static void qsa_indexer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn, int n_tok, int past,
+                        uint16_t *idxcache, int n_kv, uint8_t *allow, int32_t *topk_t, int32_t *above_t, float *score_t,
+                        int threads) {
+    int H = c->n_embd, D = c->idx_dim, IH = c->idx_heads, R = c->ratio;
+    int N = past + n_tok;                       /* occupied cells after this pass */
+    int n_blocks = (n_kv + R - 1) / R;
+    int n_bid = N / R;                          /* whole blocks only */
+    /* the raw key, cached before the norm and the rotation, rounded to halves by the cache */
+    float *raw = (float *)malloc(sizeof(float) * D);
+    for (int i = 0; i < n_tok; i++) {
+        shv_ref_matvec(raw, w->idx_k, xn + (size_t)i * H, D, H);
+        for (int j = 0; j < D; j++) idxcache[(size_t)(past + i) * D + j] = shv_ref_f32_to_f16(raw[j]);
+    }
+    free(raw);
+    /* pooled keys: a block that does not exist pools cell 0 `ratio` times (the zero fill) */
+    float *pooled = (float *)calloc((size_t)n_blocks * D, sizeof(float));
+    float inv = 1 / (float)R;
+    for (int b = 0; b < n_blocks; b++) {
+        float *dst = pooled + (size_t)b * D;
+        for (int s_ = 0; s_ < R; s_++) {
+            int cell = b < n_bid ? b * R + s_ : 0;
+            for (int j = 0; j < D; j++) dst[j] += shv_ref_f16_to_f32(idxcache[(size_t)cell * D + j]);
+        }
+        for (int j = 0; j < D; j++) dst[j] *= inv;
+    }
+    shv_ref_head_norm(pooled, w->idx_k_norm, D, n_blocks, c->eps);
+    int32_t *blk_pos = (int32_t *)calloc((size_t)n_blocks, sizeof(int32_t));
+    for (int b = 0; b < n_bid && b < n_blocks; b++) blk_pos[b] = b * R;   /* a block's position is its first cell's */
+    shv_ref_rope(c, pooled, blk_pos, 1, D, n_blocks);
+    free(blk_pos);
+    float *idxq = (float *)malloc(sizeof(float) * (size_t)n_tok * IH * D);
+    int32_t *pos = (int32_t *)malloc(sizeof(int32_t) * (size_t)n_tok);
+    for (int i = 0; i < n_tok; i++) {
+        shv_ref_matvec(idxq + (size_t)i * IH * D, w->idx_q, xn + (size_t)i * H, IH * D, H);
+        pos[i] = past + i;
+    }
+    shv_ref_head_norm(idxq, w->idx_q_norm, D, IH * n_tok, c->eps);
+    shv_ref_rope(c, idxq, pos, IH, D, n_tok);
+    free(pos);
+    /* rectified per-head dot products, summed */
+    float *score = (float *)malloc(sizeof(float) * (size_t)n_tok * n_blocks);
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) schedule(static)
+    for (int i = 0; i < n_tok; i++) {
+        for (int b = 0; b < n_blocks; b++) {
+            float s = 0;
+            const float *k = pooled + (size_t)b * D;
+            for (int h = 0; h < IH; h++) {
+                const float *q = idxq + ((size_t)i * IH + h) * D;
+                float d = 0;
+                for (int j = 0; j < D; j++) d += q[j] * k[j];
+                if (d > 0) s += d;
+            }
+            score[(size_t)i * n_blocks + b] = s;
+        }
+    }
+    if (score_t) memcpy(score_t, score, sizeof(float) * (size_t)n_tok * n_blocks);
+    /* bias, expansion to cells, causal mask, selection */
+    int dead_bid = n_bid >= n_blocks ? n_blocks - 1 : n_bid;
+    int width = c->top_k + R - 1;
+    if (width > n_kv) width = n_kv;
+    memset(allow, 0, (size_t)n_tok * N);
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) schedule(static)
+    for (int i = 0; i < n_tok; i++) {
+        int p = past + i;
+        float *bias = (float *)malloc(sizeof(float) * n_blocks);
+        float *cellv = (float *)malloc(sizeof(float) * n_kv);
+        int32_t *sel = (int32_t *)malloc(sizeof(int32_t) * width);
+        int tail_start = (p + 1) / R * R;
+        for (int b = 0; b < n_blocks; b++) {
+            if (b >= n_bid) bias[b] = -INFINITY;
+            else if (b * R >= tail_start) bias[b] = 1e9f;
+            else bias[b] = 0;
+        }
+        if (n_bid < n_blocks) bias[dead_bid] = 1e9f;
+        for (int j = 0; j < n_kv; j++) {
+            int blk = j < n_bid * R ? j / R : dead_bid;
+            float v = score[(size_t)i * n_blocks + blk] + bias[blk];
+            if (j > p || j >= N) v = -INFINITY;
+            cellv[j] = v;
+        }
+        int ab = shv_ref_topk(cellv, n_kv, width, sel);
+        if (topk_t) memcpy(topk_t + (size_t)i * width, sel, sizeof(int32_t) * width);
+        if (above_t) above_t[i] = ab;
+        for (int k = 0; k < width; k++)
+            if (sel[k] < N) allow[(size_t)i * N + sel[k]] = 1;
+        free(sel); free(cellv); free(bias);
+    }
+    free(score); free(idxq); free(pooled);
+}
+
+void shv_ref_attn_layer_qsa(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn,
+                            int n_tok, int past, uint16_t *kcache, uint16_t *vcache, uint16_t *idxcache,
+                            int n_kv, float *out, float *q_rot, float *pregate_t, int32_t *topk_t,
+                            int32_t *above_t, float *score_t, int threads) {
+    if (c->ratio <= 0) {
+        attn_layer_core(c, w, xn, n_tok, past, kcache, vcache, out, q_rot, pregate_t, NULL, threads);
+        return;
+    }
+    uint8_t *allow = (uint8_t *)malloc((size_t)n_tok * (past + n_tok));
+    qsa_indexer(c, w, xn, n_tok, past, idxcache, n_kv, allow, topk_t, above_t, score_t, threads);
+    attn_layer_core(c, w, xn, n_tok, past, kcache, vcache, out, q_rot, pregate_t, allow, threads);
+    free(allow);
 }
 
 /* ------------------------------------------------------------- token loop --- */
@@ -973,7 +1138,9 @@ void shv_ref_model_extend_rows(const shv_ref_model_cfg *c, const shv_ref_model_w
         const shv_ref_layer_w *lw = &w->layers[l];
         for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->attn_norm, H, c->eps);
         if ((l + 1) % c->attn_every == 0)
-            shv_ref_attn_layer(&c->attn, &lw->attn, xn, n_tok, st->past, st->kcache[l], st->vcache[l], y, NULL, NULL, threads);
+            shv_ref_attn_layer_qsa(&c->attn, &lw->attn, xn, n_tok, st->past, st->kcache[l], st->vcache[l],
+                                   (c->attn.ratio > 0 && st->idxcache) ? st->idxcache[l] : NULL, c->max_cells, y, NULL, NULL, NULL, NULL, NULL,
+                                   threads);
         else
             shv_ref_deltanet_layer(&c->dn, &lw->dn, xn, n_tok, st->dn_conv[l], st->dn_s[l], y, NULL, NULL, NULL,
                                    NULL, NULL, NULL, NULL, 0, threads);
@@ -1030,7 +1197,9 @@ void shv_ref_mtp_rows(const shv_ref_model_cfg *c, const shv_ref_model_w *w, cons
     }
     const shv_ref_layer_w *lw = &mw->layer;
     for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->attn_norm, H, c->eps);
-    shv_ref_attn_layer(&c->attn, &lw->attn, xn, n_tok, pos, kcache, vcache, y, NULL, NULL, threads);
+    shv_ref_attn_cfg dense = c->attn;
+    dense.ratio = 0;  /* the draft block is plain attention whatever the trunk's layers are */
+    shv_ref_attn_layer(&dense, &lw->attn, xn, n_tok, pos, kcache, vcache, y, NULL, NULL, threads);
     for (size_t i = 0; i < T * H; i++) x[i] += y[i];
     for (int t = 0; t < n_tok; t++) shv_ref_rmsnorm(xn + (size_t)t * H, x + (size_t)t * H, lw->ffn_norm, H, c->eps);
     shv_ref_moe_block(&c->moe, &lw->moe, xn, n_tok, y, NULL, NULL, NULL, NULL, NULL, NULL, threads);

@@ -146,6 +146,8 @@ typedef struct {
     float rope_base;
     int sections[4];
     float eps;
+    /* the block-sparse indexer beside the layer (llm/attn.go:56-68): ratio 0 is a dense layer */
+    int idx_heads, idx_dim, top_k, ratio;
 } shv_ref_attn_cfg;
 
 typedef struct {
@@ -154,6 +156,10 @@ typedef struct {
     const uint8_t *v;   /* Q4_K [n_head_kv*d][n_embd] */
     const uint8_t *o;   /* Q4_K [n_embd][n_head*d] */
     const float *q_norm, *k_norm;  /* [d] */
+    /* the indexer's tensors (llm/attn.go:90-93), float32: never quantised in the reference either */
+    const float *idx_q;            /* [idx_heads*idx_dim][n_embd] */
+    const float *idx_k;            /* [idx_dim][n_embd] */
+    const float *idx_q_norm, *idx_k_norm;  /* [idx_dim] */
 } shv_ref_attn_w;
 
 /* x is [n_tok][n_heads][head_dim], rotated in place at text positions pos[t]. */
@@ -168,6 +174,31 @@ void shv_ref_rope(const shv_ref_attn_cfg *c, float *x, const int32_t *pos, int n
 void shv_ref_attn_layer(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn,
                         int n_tok, int past, uint16_t *kcache, uint16_t *vcache, float *out,
                         float *q_rot, float *pregate, int threads);
+
+/* ---- the block-sparse indexer, llm/attn.go:221-443 (indexerAt, selected) and :588-682 (topK,
+ * topKThreshold, f2ui) ----
+ * The radix select: the key of the n-th largest of x[0..len) under the order-preserving map f2ui,
+ * by four 8-bit histogram passes (llm/attn.go:637-670). */
+uint32_t shv_ref_f2ui(float v);
+uint32_t shv_ref_topk_threshold(const float *x, int len, int n);
+/* The selection itself (llm/attn.go:615-632): every index strictly above the threshold in
+ * ascending order, then indices equal to it in ascending order until n are taken.  sel receives
+ * min(n, len) indices; returns how many of them are strictly above. */
+int shv_ref_topk(const float *x, int len, int n, int32_t *sel);
+/* The layer with its indexer (cfg.ratio > 0), generalised like shv_ref_attn_layer to a cache that
+ * already holds `past` cells: with past = 0 this is AttnLayerAt with Ratio > 0 under exact
+ * matvecs, the fp16 KV cache and the fp16 indexer-key cache (llm/attn.go:273-285; the reference
+ * couples those roundings and its int8 activations under one switch, which is split here as for
+ * the dense layer; the scores are formed in float32, the Exact arm of :330-356).
+ * idxcache is [n_kv][idx_dim] binary16: the raw indexer keys, appended like K and V.  n_kv is the
+ * padded cell count the block structure, bias and top-k width are cut against (:124-133).
+ * Row i (position p = past + i) sees the cells its selection names among 0..p.
+ * Optional traces: topk [n_tok][width] ascending cell lists (width = min(top_k + ratio - 1, n_kv)),
+ * above [n_tok], score [n_tok][ceil(n_kv/ratio)] the pre-bias block scores. */
+void shv_ref_attn_layer_qsa(const shv_ref_attn_cfg *c, const shv_ref_attn_w *w, const float *xn,
+                            int n_tok, int past, uint16_t *kcache, uint16_t *vcache, uint16_t *idxcache,
+                            int n_kv, float *out, float *q_rot, float *pregate, int32_t *topk,
+                            int32_t *above, float *score, int threads);
 
 /* ---- the token loop over the synthetic Qwen3-Next-shape model ----
  * The reference's loop body is llm/graph.go:2330-2466 (per layer: mix -> DeltaNet or attention ->
@@ -212,6 +243,7 @@ typedef struct {
     uint16_t **kcache;    /* [n_layer] -> [max_cells][n_head_kv][head_dim] */
     uint16_t **vcache;
     int past;             /* tokens already in the sequence */
+    uint16_t **idxcache;  /* [n_layer] -> [max_cells][idx_dim], attention layers of a model with an indexer; else NULL */
 } shv_ref_model_state;
 
 /* Extend the sequence by n_tok tokens (Graph.Extend, llm/graph.go:1709-1777): logits [vocab] and

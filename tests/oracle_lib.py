@@ -51,11 +51,13 @@ class DnW(C.Structure):
 class AttnCfg(C.Structure):
     _fields_ = [("n_embd", C.c_int), ("n_head", C.c_int), ("n_head_kv", C.c_int),
                 ("head_dim", C.c_int), ("rope_dims", C.c_int), ("rope_base", C.c_float),
-                ("sections", C.c_int * 4), ("eps", C.c_float)]
+                ("sections", C.c_int * 4), ("eps", C.c_float),
+                ("idx_heads", C.c_int), ("idx_dim", C.c_int), ("top_k", C.c_int), ("ratio", C.c_int)]
 
 
 class AttnW(C.Structure):
-    _fields_ = [("q", u8p), ("k", u8p), ("v", u8p), ("o", u8p), ("q_norm", f32p), ("k_norm", f32p)]
+    _fields_ = [("q", u8p), ("k", u8p), ("v", u8p), ("o", u8p), ("q_norm", f32p), ("k_norm", f32p),
+                ("idx_q", f32p), ("idx_k", f32p), ("idx_q_norm", f32p), ("idx_k_norm", f32p)]
 
 
 class ModelCfg(C.Structure):
@@ -73,7 +75,7 @@ class ModelW(C.Structure):
 
 class ModelState(C.Structure):
     _fields_ = [("dn_conv", C.POINTER(f32p)), ("dn_s", C.POINTER(f32p)), ("kcache", C.POINTER(u16p)),
-                ("vcache", C.POINTER(u16p)), ("past", C.c_int)]
+                ("vcache", C.POINTER(u16p)), ("past", C.c_int), ("idxcache", C.POINTER(u16p))]
 
 
 class MtpW(C.Structure):
@@ -129,6 +131,14 @@ def lib():
     L.shv_ref_rope.argtypes = [C.POINTER(AttnCfg), f32p, i32p, C.c_int, C.c_int, C.c_int]
     L.shv_ref_attn_layer.argtypes = [C.POINTER(AttnCfg), C.POINTER(AttnW), f32p, C.c_int, C.c_int,
                                      u16p, u16p, f32p, f32p, f32p, C.c_int]
+    L.shv_ref_f2ui.restype = C.c_uint32
+    L.shv_ref_f2ui.argtypes = [C.c_float]
+    L.shv_ref_topk_threshold.restype = C.c_uint32
+    L.shv_ref_topk_threshold.argtypes = [f32p, C.c_int, C.c_int]
+    L.shv_ref_topk.restype = C.c_int
+    L.shv_ref_topk.argtypes = [f32p, C.c_int, C.c_int, i32p]
+    L.shv_ref_attn_layer_qsa.argtypes = [C.POINTER(AttnCfg), C.POINTER(AttnW), f32p, C.c_int, C.c_int, u16p, u16p, u16p,
+                                         C.c_int, f32p, f32p, f32p, i32p, i32p, f32p, C.c_int]
     L.shv_ref_model_extend.argtypes = [C.POINTER(ModelCfg), C.POINTER(ModelW), C.POINTER(ModelState), i32p,
                                        C.c_int, f32p, f32p, C.c_int]
     L.shv_ref_model_extend_rows.argtypes = L.shv_ref_model_extend.argtypes
@@ -240,7 +250,9 @@ class OracleModel:
             MoeCfg(ne, cfg.n_expert, cfg.n_expert_used, cfg.ffn_expert, cfg.ffn_expert),
             DnCfg(ne, d, cfg.ssm_head_k, cfg.ssm_head_v, cfg.ssm_conv, cfg.rms_eps, 0),
             AttnCfg(ne, cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.rope_dims, cfg.rope_base,
-                    (C.c_int * 4)(*sections), cfg.rms_eps))
+                    (C.c_int * 4)(*sections), cfg.rms_eps, getattr(cfg, "idx_heads", 0), getattr(cfg, "idx_dim", 0),
+                    getattr(cfg, "idx_top_k", 0), getattr(cfg, "idx_ratio", 0)))
+        self.qsa = getattr(cfg, "idx_ratio", 0) > 0
         blk = lambda l, n: tensors["blk.%d.%s.weight" % (l, n)]
         layers = (LayerW * cfg.n_layer)()
         for l in range(cfg.n_layer):
@@ -249,6 +261,9 @@ class OracleModel:
             if (l + 1) % cfg.attn_every == 0:
                 lw.attn = AttnW(B(blk(l, "attn_q")), B(blk(l, "attn_k")), B(blk(l, "attn_v")),
                                 B(blk(l, "attn_output")), F(blk(l, "attn_q_norm")), F(blk(l, "attn_k_norm")))
+                if self.qsa:
+                    lw.attn.idx_q, lw.attn.idx_k = F(blk(l, "indexer.q_proj")), F(blk(l, "indexer.k_proj"))
+                    lw.attn.idx_q_norm, lw.attn.idx_k_norm = F(blk(l, "indexer.q_norm")), F(blk(l, "indexer.k_norm"))
             else:
                 lw.dn = DnW(B(blk(l, "attn_qkv")), B(blk(l, "attn_gate")), B(blk(l, "ssm_alpha")),
                             B(blk(l, "ssm_beta")), B(blk(l, "ssm_out")), F(blk(l, "ssm_conv1d")),
@@ -268,18 +283,22 @@ class OracleModel:
         c, n = self.cfg, self.cfg.n_layer
         cw = 2 * c.ssm_head_k * c.ssm_head_dim + c.ssm_head_v * c.ssm_head_dim
         self.dn_conv, self.dn_s, self.kc, self.vc = [None] * n, [None] * n, [None] * n, [None] * n
-        a_conv, a_s, a_k, a_v = (f32p * n)(), (f32p * n)(), (u16p * n)(), (u16p * n)()
+        self.ic = [None] * n   # the indexer's raw keys, attention layers of a model that has one
+        a_conv, a_s, a_k, a_v, a_i = (f32p * n)(), (f32p * n)(), (u16p * n)(), (u16p * n)(), (u16p * n)()
         for l in range(n):
             if (l + 1) % c.attn_every == 0:
                 self.kc[l] = np.zeros((self.max_cells, c.n_head_kv, c.head_dim), np.uint16)
                 self.vc[l] = np.zeros_like(self.kc[l])
                 a_k[l], a_v[l] = H(self.kc[l]), H(self.vc[l])
+                if self.qsa:
+                    self.ic[l] = np.zeros((self.max_cells, c.idx_dim), np.uint16)
+                    a_i[l] = H(self.ic[l])
             else:
                 self.dn_conv[l] = np.zeros((cw, c.ssm_conv - 1), np.float32)
                 self.dn_s[l] = np.zeros((c.ssm_head_v, c.ssm_head_dim, c.ssm_head_dim), np.float32)
                 a_conv[l], a_s[l] = F(self.dn_conv[l]), F(self.dn_s[l])
-        self.arrays = (a_conv, a_s, a_k, a_v)
-        self.state = ModelState(a_conv, a_s, a_k, a_v, 0)
+        self.arrays = (a_conv, a_s, a_k, a_v, a_i)
+        self.state = ModelState(a_conv, a_s, a_k, a_v, 0, a_i if self.qsa else None)
 
     def extend(self, ids, threads=8):
         ids = np.ascontiguousarray(ids, dtype=np.int32)
@@ -305,10 +324,10 @@ class OracleModel:
     def snapshot(self):
         """the carried state, to come back to with restore()"""
         cp = lambda xs: [None if a is None else a.copy() for a in xs]
-        return cp(self.dn_conv), cp(self.dn_s), cp(self.kc), cp(self.vc), self.state.past
+        return cp(self.dn_conv), cp(self.dn_s), cp(self.kc), cp(self.vc), self.state.past, cp(self.ic)
 
     def restore(self, snap):
-        for dst, src in zip((self.dn_conv, self.dn_s, self.kc, self.vc), snap[:4]):
+        for dst, src in zip((self.dn_conv, self.dn_s, self.kc, self.vc, self.ic), snap[:4] + (snap[5],)):
             for d, s_ in zip(dst, src):
                 if d is not None:
                     d[...] = s_

@@ -548,3 +548,225 @@ def test_draft_head_wiring():
     for args in (("nextn.hnorm", "nextn.enorm", False), ("nextn.enorm", "nextn.hnorm", True)):
         x_bad, _ = by_hand(*args)
         assert O.rel_l2(x_bad, res1[0]) > 1e-2
+
+
+# ------------------------------------------------------------ block-sparse indexer -------------
+
+def test_f2ui_keeps_the_order_of_floats():
+    """llm/attn.go:672-682: flip the sign bit of a positive, invert a negative: an unsigned key that
+    orders as the float does, -inf the smallest there is."""
+    rng = np.random.default_rng(30)
+    v = np.concatenate([rng.standard_normal(2000) * 10.0 ** rng.integers(-20, 20, 2000),
+                        [0.0, 1e9, -1e9, np.inf, -np.inf, 1e-45, -1e-45, 3.4e38, -3.4e38]]).astype(np.float32)
+    keys = np.array([L.shv_ref_f2ui(float(x)) for x in v], np.uint64)
+    order = np.argsort(v, kind="stable")
+    vs, ks = v[order], keys[order]
+    assert all(ks[i] < ks[i + 1] for i in range(len(vs) - 1) if vs[i] < vs[i + 1])
+    assert all(ks[i] == ks[i + 1] for i in range(len(vs) - 1) if vs[i] == vs[i + 1] and np.signbit(vs[i]) == np.signbit(vs[i + 1]))
+    assert keys[list(v).index(-np.inf)] == keys.min()
+
+
+def _topk(x, n):
+    x = np.ascontiguousarray(x, np.float32)
+    sel = np.empty(min(n, len(x)), np.int32)
+    above = L.shv_ref_topk(O.F(x), len(x), n, O.I(sel))
+    return sel, above
+
+
+def test_radix_select_is_the_nth_largest_with_ties_filled_in_index_order():
+    """llm/attn.go:588-670 (topK, topKThreshold): the threshold is the n-th largest value; every cell
+    strictly above it is taken, then cells equal to it in ascending index until n are held.  Brute
+    force by sorting, on rows without ties, rows that are mostly ties (a block's cells share one
+    score) and rows that are mostly -inf (the causal mask)."""
+    rng = np.random.default_rng(31)
+    for trial in range(60):
+        n_cells = int(rng.integers(1, 400))
+        n = int(rng.integers(1, n_cells + 1))
+        kind = trial % 3
+        if kind == 0:
+            x = rng.standard_normal(n_cells).astype(np.float32)
+        elif kind == 1:
+            x = np.repeat(rng.integers(-3, 4, (n_cells + 3) // 4).astype(np.float32), 4)[:n_cells]   # blocks of equal scores
+        else:
+            x = rng.standard_normal(n_cells).astype(np.float32)
+            x[rng.random(n_cells) < 0.7] = -np.inf
+        thr_key = L.shv_ref_topk_threshold(O.F(x), n_cells, n)
+        nth = np.sort(x)[::-1][n - 1]
+        assert thr_key == L.shv_ref_f2ui(float(nth))
+        sel, above = _topk(x, n)
+        assert len(sel) == n and len(set(sel)) == n
+        want_above = np.flatnonzero(x > nth)
+        assert above == len(want_above) and list(sel[:above]) == list(want_above)
+        fill = np.flatnonzero(x == nth)[:n - above]
+        assert list(sel[above:]) == list(fill)
+    # the negative control: taking the ties from the top instead is another set
+    x = np.array([1, 1, 1, 1, 5, 1, 1], np.float32)
+    sel, above = _topk(x, 3)
+    assert above == 1 and sorted(sel) == [0, 1, 4]
+
+
+def qsa_cfg(top_k=8, ratio=4, idx_heads=2, idx_dim=32, **kw):
+    c = attn_cfg(**kw)
+    c.idx_heads, c.idx_dim, c.top_k, c.ratio = idx_heads, idx_dim, top_k, ratio
+    return c
+
+
+def qsa_setup(rng, cfg):
+    aw, w = attn_setup(rng, cfg)
+    H, D, IH = cfg.n_embd, cfg.idx_dim, cfg.idx_heads
+    w["iq"] = (rng.standard_normal((IH * D, H)) * 0.05).astype(np.float32)
+    w["ik"] = (rng.standard_normal((D, H)) * 0.05).astype(np.float32)
+    w["iqn"] = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    w["ikn"] = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    aw.idx_q, aw.idx_k, aw.idx_q_norm, aw.idx_k_norm = O.F(w["iq"]), O.F(w["ik"]), O.F(w["iqn"]), O.F(w["ikn"])
+    return aw, w
+
+
+def run_qsa(cfg, aw, x, past, kc, vc, ic, n_kv):
+    T = x.shape[0]
+    width = min(cfg.top_k + cfg.ratio - 1, n_kv)
+    nb = (n_kv + cfg.ratio - 1) // cfg.ratio
+    out, pre = np.empty((T, cfg.n_embd), np.float32), np.empty((T, cfg.n_head * cfg.head_dim), np.float32)
+    topk, above, score = np.empty((T, width), np.int32), np.empty(T, np.int32), np.empty((T, nb), np.float32)
+    L.shv_ref_attn_layer_qsa(O.C.byref(cfg), O.C.byref(aw), O.F(x), T, past, O.H(kc), O.H(vc), O.H(ic), n_kv, O.F(out), None, O.F(pre),
+                             O.I(topk), O.I(above), O.F(score), 1)
+    return dict(out=out, pre=pre, topk=topk, above=above, score=score)
+
+
+def _rope64(x, pos, rot, base):
+    """NeoX rotation in float64: x [..., dim], one position for the whole array."""
+    y = x.copy()
+    half = rot // 2
+    i = np.arange(half)
+    th = pos * base ** (-2.0 * i / rot)
+    c, s = np.cos(th), np.sin(th)
+    y[..., :half] = x[..., :half] * c - x[..., half:rot] * s
+    y[..., half:rot] = x[..., :half] * s + x[..., half:rot] * c
+    return y
+
+
+def _indexer64(cfg, w, xn, n_kv):
+    """The selection re-derived in float64 for a prompt from position 0: visible sets per row and
+    the margin between the last value taken and the first left out."""
+    T, D, IH, R = xn.shape[0], cfg.idx_dim, cfg.idx_heads, cfg.ratio
+    half = lambda a: a.astype(np.float16).astype(np.float64)
+    raw = half((xn.astype(np.float64) @ w["ik"].astype(np.float64).T).astype(np.float32))     # the cache holds halves
+    n_bid = T // R
+    norm = lambda v, g: v / np.sqrt((v ** 2).mean(axis=-1, keepdims=True) + EPS) * g.astype(np.float64)
+    keys = np.stack([_rope64(norm(raw[b * R:(b + 1) * R].mean(axis=0), w["ikn"]), b * R, cfg.rope_dims, 1e7) for b in range(n_bid)]) \
+        if n_bid else np.zeros((0, D))
+    dead = norm(raw[0], w["ikn"])                                           # a block that is not there: cell 0, position 0
+    q = (xn.astype(np.float64) @ w["iq"].astype(np.float64).T).reshape(T, IH, D)
+    q = np.stack([_rope64(norm(q[i], w["iqn"]), i, cfg.rope_dims, 1e7) for i in range(T)])
+    width = min(cfg.top_k + R - 1, n_kv)
+    sets, margins = [], []
+    for i in range(T):
+        sc = np.maximum(q[i] @ keys.T, 0).sum(axis=0) if n_bid else np.zeros(0)       # [n_bid]
+        sd = np.maximum(q[i] @ dead, 0).sum()
+        tail_start = (i + 1) // R * R
+        v = np.full(i + 1, -np.inf)
+        for j in range(i + 1):
+            if j < n_bid * R:
+                b = j // R
+                v[j] = np.float32(np.float32(sc[b]) + np.float32(1e9 if b * R >= tail_start else 0))
+            else:
+                v[j] = np.float32(np.float32(sd) + np.float32(1e9))
+        if i + 1 <= width:
+            sets.append(set(range(i + 1)))
+            margins.append(np.inf)
+            continue
+        order = np.sort(v)[::-1]
+        nth = order[width - 1]
+        take = list(np.flatnonzero(v > nth))
+        take += list(np.flatnonzero(v == nth)[:width - len(take)])
+        sets.append(set(int(t) for t in take))
+        below = order[order < nth]
+        above = order[order > nth]
+        m = min((above.min() - nth) if len(above) else np.inf, (nth - below.max()) if len(below) else np.inf)
+        margins.append(m)
+    return sets, margins
+
+
+def test_indexer_selection_against_independent_float64():
+    """indexerAt (llm/attn.go:231-421) re-derived in numpy float64 — raw keys through a binary16
+    cache, whole blocks pooled, normed and turned at their first cell's position, rectified
+    per-head scores, the 1e9 tail, the causal mask, the top (top_k + ratio - 1) cells with ties
+    filled in index order — must name the same visible cells row for row wherever the value at
+    the cut is clear of its neighbours."""
+    cfg = qsa_cfg(top_k=8, ratio=4)
+    rng = np.random.default_rng(32)
+    aw, w = qsa_setup(rng, cfg)
+    T, n_kv = 45, 64
+    x = rng.standard_normal((T, cfg.n_embd)).astype(np.float32)
+    kc = np.zeros((n_kv, cfg.n_head_kv, cfg.head_dim), np.uint16)
+    vc, ic = np.zeros_like(kc), np.zeros((n_kv, cfg.idx_dim), np.uint16)
+    got = run_qsa(cfg, aw, x, 0, kc, vc, ic, n_kv)
+    sets, margins = _indexer64(cfg, w, x, n_kv)
+    checked = 0
+    for i in range(T):
+        mine = set(int(c) for c in got["topk"][i] if c <= i)
+        if margins[i] > 1e-4:
+            assert mine == sets[i], (i, sorted(mine ^ sets[i]))
+            checked += 1
+        # what every row must hold whatever the scores: its own incomplete tail
+        assert set(range((i + 1) // 4 * 4, i + 1)) <= mine
+    assert checked >= T - 4
+    # selections really cut: late rows see fewer cells than are visible
+    assert len(set(int(c) for c in got["topk"][T - 1] if c <= T - 1)) == 11 < T
+    # the lists are ascending within the strictly-above part and within the fill
+    for i in range(T):
+        a = got["above"][i]
+        assert list(got["topk"][i][:a]) == sorted(got["topk"][i][:a])
+
+
+def test_indexer_at_seven_tokens_in_a_larger_cache():
+    """llm/attn.go:124-133, :221-230: 7 tokens in a 256-cell cache make one block of 4 and leave
+    cells 4..6 unpooled; every block that does not exist pools cell 0, so their scores all equal
+    the score of the spare block that collects the tail; the selection covers every visible cell
+    and the layer is the dense one bit for bit."""
+    cfg = qsa_cfg(top_k=16, ratio=4)
+    rng = np.random.default_rng(33)
+    aw, w = qsa_setup(rng, cfg)
+    T, n_kv = 7, 256
+    x = rng.standard_normal((T, cfg.n_embd)).astype(np.float32)
+    mk = lambda: (np.zeros((n_kv, cfg.n_head_kv, cfg.head_dim), np.uint16), np.zeros((n_kv, cfg.n_head_kv, cfg.head_dim), np.uint16))
+    kc, vc = mk()
+    ic = np.zeros((n_kv, cfg.idx_dim), np.uint16)
+    got = run_qsa(cfg, aw, x, 0, kc, vc, ic, n_kv)
+    assert (got["score"][:, 1:] == got["score"][:, 1:2]).all()       # blocks 1..63 are all cell 0's key
+    assert not (got["score"][:, 0] == got["score"][:, 1]).all()
+    for i in range(T):
+        assert set(range(i + 1)) <= set(int(c) for c in got["topk"][i])
+    dense = attn_cfg()
+    kd, vd = mk()
+    out_d, pre_d = run_attn(dense, aw, x, 0, kd, vd)
+    assert np.array_equal(got["out"], out_d) and np.array_equal(got["pre"], pre_d)
+
+
+def test_indexer_over_a_cache_is_a_chunk_split():
+    """Rows appended over a cache select what the same rows select in one pass from position 0,
+    and the layer's output is the same bit for bit (19 + 13 + 1 = 33 rows)."""
+    cfg = qsa_cfg(top_k=8, ratio=4)
+    rng = np.random.default_rng(34)
+    aw, w = qsa_setup(rng, cfg)
+    T, n_kv = 33, 64
+    x = rng.standard_normal((T, cfg.n_embd)).astype(np.float32)
+    z = lambda: (np.zeros((n_kv, cfg.n_head_kv, cfg.head_dim), np.uint16), np.zeros((n_kv, cfg.n_head_kv, cfg.head_dim), np.uint16),
+                 np.zeros((n_kv, cfg.idx_dim), np.uint16))
+    whole = run_qsa(cfg, aw, x, 0, *z(), n_kv)
+    kc, vc, ic = z()
+    parts, past = [], 0
+    for n in (19, 13, 1):
+        parts.append(run_qsa(cfg, aw, x[past:past + n], past, kc, vc, ic, n_kv))
+        past += n
+    out = np.concatenate([p["out"] for p in parts])
+    vis = lambda tk, i: set(int(c) for c in tk if c <= i)
+    tk = np.concatenate([p["topk"] for p in parts])
+    for i in range(T):
+        assert vis(tk[i], i) == vis(whole["topk"][i], i), i
+    assert np.array_equal(out, whole["out"])
+    # and the selection matters: the dense layer gives other numbers on the late rows
+    dense = attn_cfg()
+    kd, vd, _ = z()
+    out_d, _ = run_attn(dense, aw, x, 0, kd, vd)
+    assert np.array_equal(out_d[:11], whole["out"][:11]) and O.rel_l2(out_d[20:], whole["out"][20:]) > 1e-3
