@@ -92,6 +92,7 @@ enum {
     SHV_OP_GEMV = 14,
     SHV_OP_RING_ROWS = 15,
     SHV_OP_ROUTER_FOLD = 16,
+    SHV_OP_QSA_INDEX = 17,
     SHV_OP__COUNT
 };
 
@@ -402,7 +403,48 @@ typedef struct {
     int32_t n_head, n_head_kv, head_dim, rope_dims;
     int32_t max_cells, qkv_stride, n_splits;
     float eps;
+    /* The block-sparse selection (AttnTrace.selected, llm/attn.go:423-443): row r of the pass may
+     * read cell c only if bit c % 32 of mask[r * mask_stride + c / 32] is set (and c is visible at
+     * all); shv_qsa_index makes it.  NULL: every visible cell. */
+    const uint32_t *mask;
+    int32_t mask_stride;
 } shv_attn_decode_args;
+
+/* The block-sparse indexer beside a full-attention layer (AttnTrace.indexerAt, llm/attn.go:231-421;
+ * topK / topKThreshold / f2ui :588-682; shaders llm_attn_idx / score / select / selblk.comp), for
+ * n_seq sequences of seq_len consecutive rows at positions pos[s]+i on slot[s]:
+ *   [q (idx_heads*idx_dim) | k (idx_dim)] = w . RMSNorm(x)*gamma in float32; the raw key goes to
+ *   idxcache (binary16) at the row's cell; every block of `ratio` cells the pass completes is pooled
+ *   (mean), RMS-normed with k_norm, rotated at its first cell's position and kept in `pooled`; a
+ *   query head is normed with q_norm and rotated at the row's position; a block's score is the sum
+ *   over heads of max(0, q_h . k); a cell's value is its block's score, plus 1e9 for blocks at or
+ *   after the row's own incomplete block, and the score of the block that does not exist (cell 0
+ *   pooled `ratio` times, the reference's zero fill) plus 1e9 for the cells after the last whole
+ *   block; of the row's visible cells the (top_k + ratio - 1) largest are taken by a radix select:
+ *   everything strictly above the threshold, then cells equal to it in ascending index.
+ * mask [rows][mask_stride] receives the selection, a bit a cell, for shv_attn_decode.
+ * idxcache is [n_slots][max_cells][idx_dim] binary16; pooled [n_slots][max_cells/ratio + 1][idx_dim]
+ * float32 (the last row is rewritten by every call); work [rows][idx_heads*idx_dim + idx_dim] and
+ * score [rows][max_cells/ratio + 1] are scratch.  rope is the attention's table. */
+typedef struct {
+    const float *x;
+    const float *gamma;
+    const float *w;
+    const float *q_norm;
+    const float *k_norm;
+    const float *rope;
+    uint16_t *idxcache;
+    float *pooled;
+    const int32_t *pos;
+    const int32_t *slot;
+    float *work;
+    float *score;
+    uint32_t *mask;
+    int32_t n_seq, seq_len, n_embd;
+    int32_t idx_heads, idx_dim, top_k, ratio, rope_dims;
+    int32_t max_cells, mask_stride;
+    float eps;
+} shv_qsa_index_args;
 
 /* Token embedding gather (Model.Embeddings, llm/model.go:134; hc.UploadInit, llm/graph.go:1815):
  * x[t] = float32(table[id_t]) for n_tok rows, id_t = ids[pos[0]+t] when pos is given, else ids[t].
@@ -496,6 +538,7 @@ int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_advance(shv_ctx *ctx, const shv_advance_args *a);
 int shv_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *a);
 int shv_router_fold(shv_ctx *ctx, const shv_router_fold_args *a);
+int shv_qsa_index(shv_ctx *ctx, const shv_qsa_index_args *a);
 
 /* shv_argmax for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and

@@ -131,7 +131,9 @@ struct Smem {
 // group would read cells another block is still writing); without, the cells are there already
 // and any number of groups go in one launch, each masked to its own positions.  Query row r of the
 // tile is head r%8 of sequence row r/8; with R = 1 rows 8..15 are padding.
-template <int R>
+// QSA: a.mask names, a bit a cell, the cells each row may read (the block-sparse indexer's
+// selection, llm/attn.go:423-443); a tile none of the wave's rows may read is not loaded at all.
+template <int R, bool QSA = false>
 __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_args a, int row00, int n_groups, int append, int slice_cells) {
     __shared__ Smem sm;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -243,8 +245,14 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
     // where it needs an earlier one: a wave that has both a tile and heads to prepare waits for
     // the tile before it prepares them.  In a slice of one tile no wave has both.)
     const int t_first = c0 + kTile * wave;
-    const bool early = t_first < c1 && t_first + kTile <= p_first;
+    const bool early = !QSA && t_first < c1 && t_first + kTile <= p_first;
     if (early) load_tile(ta, t_first);
+    // the lane's query row is sequence row n / 8: its mask words
+    const uint32_t *mrow = nullptr;
+    if constexpr (QSA) {
+        const int jr = (n >> 3) < valid ? (n >> 3) : valid - 1;
+        mrow = a.mask + static_cast<size_t>(seq * a.seq_len + row0 + jr) * a.mask_stride;
+    }
 
     // operand table entry [i][h][part][16*kb + row] holds dims 8*(kb + 4*i) + 4*h .. +3 of query row
     // `row`: lane l's four dims 4l..4l+3 are h = l&1, kb = (l>>1)&3, i = l>>3
@@ -311,7 +319,7 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
     float m_run = -INFINITY, l_run = 0.f;
     const int my_row_pos = p_first + (n >> 3);  // the last cell query row n may see
 
-    auto compute = [&](const Tile &tl, int t0) {
+    auto compute = [&](const Tile &tl, int t0, uint32_t mw) {
         const uint4(&kreg)[2][8] = tl.k;
         const uint4(&vreg)[16] = tl.v;
         // ---- S^T = K Q^T: A = K (cells x dims), B = Q^T (dims x rows); four independent chains
@@ -352,7 +360,9 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int c = t0 + 8 * q + 4 * T + i;
-                st[T][i] = (c < c1 && c <= my_row_pos) ? st[T][i] : -INFINITY;
+                bool ok = c < c1 && c <= my_row_pos;
+                if constexpr (QSA) ok = ok && ((mw >> (8 * q + 4 * T + i)) & 1u) != 0u;
+                st[T][i] = ok ? st[T][i] : -INFINITY;
                 mx = fmaxf(mx, st[T][i]);
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -406,8 +416,13 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
     // overlap the other's products
     constexpr int kStep = 4 * kTile;
     for (int t0 = t_first; t0 < c1; t0 += kStep) {
+        uint32_t mw = 0xFFFFFFFFu;
+        if constexpr (QSA) {
+            mw = mrow[t0 >> 5];  // tiles start on multiples of 32 cells: one word a tile and row
+            if (__ballot(mw != 0u) == 0ull) continue;
+        }
         if (!early || t0 != t_first) load_tile(ta, t0);
-        compute(ta, t0);
+        compute(ta, t0, mw);
     }
     // ---- the four waves' results of each sequence row are merged and go to scratch ----
     if (q == 0) {
@@ -573,8 +588,15 @@ struct PrefillSmem {
 __device__ __forceinline__ void tile_barrier() {
     asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
+// The same for the kernel that also loads mask words between the tiles' loads, which the count above
+// does not know of: it waits for everything (the tiles ahead included; that build gives up their
+// head start).
+__device__ __forceinline__ void tile_barrier_all() {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
 // grid: (n_seq * ceil(n_groups / 8), n_head_kv, n_splits); the cells of the pass are in the cache already.
+template <bool QSA>
 __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decode_args a, int n_groups, int slice_cells, int direct) {
     extern __shared__ __align__(16) char praw[];
     PrefillSmem &sm = *reinterpret_cast<PrefillSmem *>(praw);
@@ -713,7 +735,13 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
     ask_tile(lo, 0);
     ask_tile(lo + kTile, 1);
     ask_tile(lo + 2 * kTile, 2);
-    tile_barrier();   // the first tile has landed: all but the two youngest tiles' loads of every wave
+    if constexpr (QSA) tile_barrier_all();
+    else tile_barrier();   // the first tile has landed: all but the two youngest tiles' loads of every wave
+    const uint32_t *mrow = nullptr;
+    if constexpr (QSA) {
+        const int jr = (n >> 3) < me.valid ? (n >> 3) : me.valid - 1;
+        mrow = a.mask + static_cast<size_t>(seq * a.seq_len + row0 + jr) * a.mask_stride;
+    }
 
     float4_t o[16];
 #pragma unroll
@@ -725,8 +753,10 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
     for (int t0 = lo; t0 < hi; t0 += kTile, b = (b + 1) & (kPfStages - 1)) {
         // three tiles on: into the stage read a tile ago (every wave has passed the barrier that ended that tile)
         ask_tile(t0 + 3 * kTile, (b + 3) & (kPfStages - 1));
+        uint32_t mw = 0xFFFFFFFFu;
+        if constexpr (QSA) mw = mrow[t0 >> 5];
         // tiles wholly outside the wave's slice or beyond what its rows see are skipped
-        if (me.mine && t0 < me.c1 && t0 + kTile > me.c0 && t0 <= me.p_first + 1) {
+        if (me.mine && t0 < me.c1 && t0 + kTile > me.c0 && t0 <= me.p_first + 1 && (!QSA || __ballot(mw != 0u) != 0ull)) {
             const char *kt = sm.u.ring[b], *vt = sm.u.ring[b] + 16 * kChunk;
             // operands come from LDS four reads ahead of the products that use them: a read's
             // latency is about what eight products take, and asked for one at a time it is paid 32 times a tile
@@ -769,7 +799,9 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int c = t0 + 8 * q + 4 * T + i;
-                    st[T][i] = (c >= me.c0 && c < me.c1 && c <= my_row_pos) ? st[T][i] : -INFINITY;
+                    bool ok = c >= me.c0 && c < me.c1 && c <= my_row_pos;
+                    if constexpr (QSA) ok = ok && ((mw >> (8 * q + 4 * T + i)) & 1u) != 0u;
+                    st[T][i] = ok ? st[T][i] : -INFINITY;
                     mx = fmaxf(mx, st[T][i]);
                 }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -819,7 +851,8 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(shv_attn_decod
                 }
             }
         }
-        tile_barrier();   // the next tile has landed, this one has been read
+        if constexpr (QSA) tile_barrier_all();
+        else tile_barrier();   // the next tile has landed, this one has been read
     }
     // the loads asked for past the last tile still write LDS: none may be out when the wave ends and its LDS goes to another workgroup
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -869,16 +902,20 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
         // a prompt pass: eight pairs a block share the cache's tiles
         static bool raised = false;
         if (!raised) {
-            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
+            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
+            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
             raised = true;
         }
         // with one slice a pair there is nothing to merge: the kernel writes the rows themselves
         const int direct = b.n_splits == 1 ? 1 : 0;
-        SHV_LAUNCH(ctx, attn_prefill_kernel, dim3(a.n_seq * ((n_groups + kPfWaves - 1) / kPfWaves), a.n_head_kv, b.n_splits), dim3(kPfThreads), sizeof(PrefillSmem), b, n_groups, slice_cells, direct);
+        const dim3 grid(a.n_seq * ((n_groups + kPfWaves - 1) / kPfWaves), a.n_head_kv, b.n_splits);
+        if (a.mask) SHV_LAUNCH(ctx, attn_prefill_kernel<true>, grid, dim3(kPfThreads), sizeof(PrefillSmem), b, n_groups, slice_cells, direct);
+        else SHV_LAUNCH(ctx, attn_prefill_kernel<false>, grid, dim3(kPfThreads), sizeof(PrefillSmem), b, n_groups, slice_cells, direct);
         if (direct) return SHV_OK;
     } else {
         dim3 grid(a.n_seq * n_groups, a.n_head_kv, b.n_splits);
-        SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
+        if (a.mask) SHV_LAUNCH(ctx, (attn_decode_kernel<R, true>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
+        else SHV_LAUNCH(ctx, (attn_decode_kernel<R>), grid, dim3(kBlock), 0, b, row0, n_groups, append, slice_cells);
     }
     if (a.n_seq * n_groups >= 8 && b.n_splits <= 16) SHV_LAUNCH(ctx, (attn_merge_kernel<R, 1>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64), 0, b, row0, n_groups, slice_cells);
     else SHV_LAUNCH(ctx, (attn_merge_kernel<R, kMergeWaves>), dim3(a.n_head * 4, R, a.n_seq * n_groups), dim3(64 * kMergeWaves), 0, b, row0, n_groups, slice_cells);
@@ -901,6 +938,7 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
     SHV_REQUIRE(a.n_splits >= 1 && a.n_splits <= kMaxSplits, "attn_decode: %d slices; 1..%d", a.n_splits, kMaxSplits);
     SHV_REQUIRE(a.qkv_stride >= a.n_head * 2 * kD + 2 * a.n_head_kv * kD, "attn_decode: qkv_stride %d", a.qkv_stride);
     SHV_REQUIRE(a.max_cells >= kTile && a.max_cells % kTile == 0, "attn_decode: max_cells %d; a multiple of %d", a.max_cells, kTile);
+    SHV_REQUIRE(!a.mask || a.mask_stride >= a.max_cells / 32, "attn_decode: mask_stride %d words for %d cells", a.mask_stride, a.max_cells);
     SHV_REQUIRE(shv_aligned16(a.qkv) && shv_aligned16(a.kcache) && shv_aligned16(a.vcache) && shv_aligned16(a.q_norm) &&
                     shv_aligned16(a.k_norm) && shv_aligned16(a.out) && shv_aligned16(a.partial) && a.qkv_stride % 4 == 0,
                 "attn_decode: qkv, caches, norms, partial and out must be 16-byte aligned");

@@ -225,6 +225,7 @@ static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t by
         case SHV_OP_GEMV: return run_as<shv_gemv_args>(ctx, args, bytes, shv_launch_gemv, "gemv");
         case SHV_OP_RING_ROWS: return run_as<shv_ring_rows_args>(ctx, args, bytes, shv_launch_ring_rows, "ring_rows");
         case SHV_OP_ROUTER_FOLD: return run_as<shv_router_fold_args>(ctx, args, bytes, shv_launch_router_fold, "router_fold");
+        case SHV_OP_QSA_INDEX: return run_as<shv_qsa_index_args>(ctx, args, bytes, shv_launch_qsa_index, "qsa_index");
         default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
     }
 }
@@ -367,6 +368,7 @@ int shv_argmax(shv_ctx *ctx, const shv_argmax_args *a) { return dispatch_one(ctx
 int shv_advance(shv_ctx *ctx, const shv_advance_args *a) { return dispatch_one(ctx, SHV_OP_ADVANCE, a, sizeof(*a)); }
 int shv_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *a) { return dispatch_one(ctx, SHV_OP_RING_ROWS, a, sizeof(*a)); }
 int shv_router_fold(shv_ctx *ctx, const shv_router_fold_args *a) { return dispatch_one(ctx, SHV_OP_ROUTER_FOLD, a, sizeof(*a)); }
+int shv_qsa_index(shv_ctx *ctx, const shv_qsa_index_args *a) { return dispatch_one(ctx, SHV_OP_QSA_INDEX, a, sizeof(*a)); }
 
 int shv_argmax_static(shv_ctx *ctx, const shv_argmax_args *a) {
     SHV_REQUIRE(ctx && a, "shv_argmax_static: NULL argument");

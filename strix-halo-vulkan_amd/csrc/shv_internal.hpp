@@ -157,6 +157,7 @@ int shv_launch_argmax(shv_ctx *ctx, const shv_argmax_args *a);
 int shv_launch_advance(shv_ctx *ctx, const shv_advance_args *a);
 int shv_launch_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *a);
 int shv_launch_router_fold(shv_ctx *ctx, const shv_router_fold_args *a);
+int shv_launch_qsa_index(shv_ctx *ctx, const shv_qsa_index_args *a);
 bool shv_dn_chunk_covers(const shv_dn_step_args &a);
 int shv_launch_dn_chunk(shv_ctx *ctx, const shv_dn_step_args &a);
 int shv_static_scratch_bind(shv_ctx *ctx);  // at shv_init, with ctx->device current

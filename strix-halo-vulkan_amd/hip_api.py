@@ -10,7 +10,7 @@ Q4K_BYTES = 144
 
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
-OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV, OP_RING_ROWS, OP_ROUTER_FOLD = 10, 11, 12, 13, 14, 15, 16
+OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV, OP_RING_ROWS, OP_ROUTER_FOLD, OP_QSA_INDEX = 10, 11, 12, 13, 14, 15, 16, 17
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 
@@ -115,7 +115,15 @@ class AttnDecodeArgs(C.Structure):
                 ("slot", C.c_void_p), ("n_seq", C.c_int32), ("seq_len", C.c_int32),
                 ("n_head", C.c_int32), ("n_head_kv", C.c_int32), ("head_dim", C.c_int32),
                 ("rope_dims", C.c_int32), ("max_cells", C.c_int32), ("qkv_stride", C.c_int32),
-                ("n_splits", C.c_int32), ("eps", C.c_float)]
+                ("n_splits", C.c_int32), ("eps", C.c_float), ("mask", C.c_void_p), ("mask_stride", C.c_int32)]
+
+
+class QsaIndexArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("gamma", C.c_void_p), ("w", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
+                ("rope", C.c_void_p), ("idxcache", C.c_void_p), ("pooled", C.c_void_p), ("pos", C.c_void_p), ("slot", C.c_void_p),
+                ("work", C.c_void_p), ("score", C.c_void_p), ("mask", C.c_void_p), ("n_seq", C.c_int32), ("seq_len", C.c_int32),
+                ("n_embd", C.c_int32), ("idx_heads", C.c_int32), ("idx_dim", C.c_int32), ("top_k", C.c_int32), ("ratio", C.c_int32),
+                ("rope_dims", C.c_int32), ("max_cells", C.c_int32), ("mask_stride", C.c_int32), ("eps", C.c_float)]
 
 
 class EmbedArgs(C.Structure):
@@ -161,7 +169,7 @@ SYMBOLS = [
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
-    "shv_argmax_static", "shv_ring_rows", "shv_router_fold",
+    "shv_argmax_static", "shv_ring_rows", "shv_router_fold", "shv_qsa_index",
 ]
 
 _lib = None
@@ -219,6 +227,7 @@ def load():
     L.shv_argmax_static.argtypes = [vp, C.POINTER(ArgmaxArgs)]
     L.shv_ring_rows.argtypes = [vp, C.POINTER(RingRowsArgs)]
     L.shv_router_fold.argtypes = [vp, C.POINTER(RouterFoldArgs)]
+    L.shv_qsa_index.argtypes = [vp, C.POINTER(QsaIndexArgs)]
     _lib = L
     return L
 
