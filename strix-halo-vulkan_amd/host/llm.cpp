@@ -108,6 +108,9 @@ Model::Model(Device &dev, const Config &cfg) : dev_(dev), cfg_(cfg) {
     add("output_norm.weight", TensorView::F32, 1, c.NEmbd, 1.f, 0.1f);
     add("output.weight", TensorView::Q4K, c.VocabSize, c.NEmbd, 0.f, 0.02f);
     if (c.NextN < 0 || c.NextN > 1) throw Error("llm: nextn_predict_layers " + std::to_string(c.NextN) + "; one draft block at most");
+    if (c.IdxRatio < 0 || (c.IdxRatio > 0 && (c.IdxHeads < 1 || c.IdxHeads > 8 || c.IdxDim < 64 || c.IdxDim > 256 || c.IdxDim % 64 || c.IdxTopK < 1 || 32 % c.IdxRatio)))
+        throw Error("llm: indexer of " + std::to_string(c.IdxHeads) + " heads x " + std::to_string(c.IdxDim) + ", top " + std::to_string(c.IdxTopK) + ", ratio " +
+                    std::to_string(c.IdxRatio) + "; 1..8 heads of 64..256 dims, a ratio that divides 32");
     for (int l = 0; l < c.Blocks(); l++) {
         if (l >= c.NLayer) {
             // the draft block's own tensors (llm/mtp.go:36-53): the two input norms side by side
@@ -130,6 +133,15 @@ Model::Model(Device &dev, const Config &cfg) : dev_(dev), cfg_(cfg) {
             add(Blk(l, "attn_output"), TensorView::Q4K, c.NEmbd, c.NHead * c.HeadDim, 0.f, 0.02f);
             add(Blk(l, "attn_q_norm"), TensorView::F32, 1, c.HeadDim, 1.f, 0.1f);
             add(Blk(l, "attn_k_norm"), TensorView::F32, 1, c.HeadDim, 1.f, 0.1f);
+            if (c.QSA(l)) {
+                // the indexer's projections (llm/model.go:409-424), float32 and one matrix: four
+                // query heads, then the key
+                add(Blk(l, "indexer.qk_fused"), TensorView::F32, c.IdxRows(), c.NEmbd, 0.f, 0.02f);
+                alias(Blk(l, "indexer.q_proj"), Blk(l, "indexer.qk_fused"), 0, c.IdxHeads * c.IdxDim);
+                alias(Blk(l, "indexer.k_proj"), Blk(l, "indexer.qk_fused"), c.IdxHeads * c.IdxDim, c.IdxDim);
+                add(Blk(l, "indexer.q_norm"), TensorView::F32, 1, c.IdxDim, 1.f, 0.1f);
+                add(Blk(l, "indexer.k_norm"), TensorView::F32, 1, c.IdxDim, 1.f, 0.1f);
+            }
         } else {
             // fused rows: qkv | z | alpha | beta (llm/deltanet.go:135-154)
             add(Blk(l, "ssm_in_fused"), TensorView::Q4K, c.DNFusedRows(), c.NEmbd, 0.f, 0.02f);
@@ -244,6 +256,21 @@ Config Model::ConfigFromGGUF(const gguf::Set &s) {
     c.NextN = 0;
     may("nextn_predict_layers", &c.NextN);
     c.NLayer = blocks - c.NextN;  // block_count counts the draft block (llm/mtp.go:137)
+    // llm/model.go:385-405: the indexer's shape, and one compress ratio for the layers that have one
+    // (the per-layer array's non-zero entries must agree; a scalar key is read too)
+    may("attention.indexer.head_count", &c.IdxHeads);
+    may("attention.indexer.key_length", &c.IdxDim);
+    may("attention.indexer.top_k", &c.IdxTopK);
+    may("attention.compress_ratio", &c.IdxRatio);
+    if (const std::vector<int64_t> *cr = s.Ints(arch + ".attention.compress_ratios")) {
+        for (size_t l = 0; l < cr->size(); l++) {
+            const int r = static_cast<int>((*cr)[l]);
+            if (r == 0) continue;
+            if (c.IdxRatio != 0 && c.IdxRatio != r) throw Error("llm: attention.compress_ratios names " + std::to_string(c.IdxRatio) + " and " + std::to_string(r) + "; one ratio for all indexed layers is what is built");
+            c.IdxRatio = r;
+        }
+    }
+    if (c.IdxHeads == 0 || c.IdxDim == 0 || c.IdxTopK == 0) c.IdxRatio = 0;
     double f;
     if (s.Float(arch + ".attention.layer_norm_rms_epsilon", &f)) c.RMSEps = static_cast<float>(f);
     if (s.Float(arch + ".rope.freq_base", &f)) c.RopeBase = static_cast<float>(f);
@@ -409,6 +436,14 @@ void Model::SaveGGUF(const std::string &path, const std::string &arch) const {
     u32("ssm.conv_kernel", c.SSMConv);
     u32("full_attention_interval", c.AttnEvery);
     u32("nextn_predict_layers", c.NextN);
+    if (c.IdxRatio > 0) {
+        u32("attention.indexer.head_count", c.IdxHeads);
+        u32("attention.indexer.key_length", c.IdxDim);
+        u32("attention.indexer.top_k", c.IdxTopK);
+        std::vector<int32_t> ratios(c.Blocks(), 0);
+        for (int l = 0; l < c.Blocks(); l++) ratios[l] = c.QSA(l) ? c.IdxRatio : 0;
+        w.PutI32s(arch + ".attention.compress_ratios", ratios);
+    }
 
     // constituents stand in for a fused tensor when they tile it
     std::map<std::string, std::vector<std::string>> parts;
@@ -927,6 +962,22 @@ AttnGPU::AttnGPU(Device &dev, const Model &m, int maxTokens, int nKV, int slots,
         vc_[l] = dev.alloc_zero(cb);
         cache_bytes_ += 2 * cb;
     }
+    idxc_.assign(c_.Blocks(), nullptr);
+    pooled_.assign(c_.Blocks(), nullptr);
+    for (int l = 0; l < c_.Blocks(); l++) {
+        if (!kc_[l] || !c_.QSA(l)) continue;
+        if (nKV % c_.IdxRatio) throw Error("llm: AttnGPU: " + std::to_string(nKV) + " cells are not whole blocks of " + std::to_string(c_.IdxRatio));
+        const size_t ib = static_cast<size_t>(slots) * nKV * c_.IdxDim * 2, pb = static_cast<size_t>(slots) * (nKV / c_.IdxRatio + 1) * c_.IdxDim * 4;
+        idxc_[l] = static_cast<uint16_t *>(dev.alloc_zero(ib));
+        pooled_[l] = static_cast<float *>(dev.alloc_zero(pb));
+        cache_bytes_ += ib + pb;
+        if (!qsa_work_) {
+            mask_stride_ = nKV / 32;
+            qsa_work_ = static_cast<float *>(dev.alloc(T * c_.IdxRows() * 4));
+            qsa_score_ = static_cast<float *>(dev.alloc(T * (nKV / c_.IdxRatio + 1) * 4));
+            qsa_mask_ = static_cast<uint32_t *>(dev.alloc(T * mask_stride_ * 4));
+        }
+    }
 }
 
 void AttnGPU::SetSplits(int n) {
@@ -1004,6 +1055,38 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, cons
     a.qkv_stride = width;
     a.n_splits = splits_;
     a.eps = c_.RMSEps;
+    // a layer with an indexer: which cells each row may read, made beside the projection (both read the block's input)
+    shv_qsa_index_args qi{};
+    const bool qsa = idxc_[l] != nullptr;
+    if (qsa) {
+        qi.x = in;
+        qi.gamma = p.gamma;
+        qi.w = static_cast<const float *>(m_.Tensor(Model::Blk(l, "indexer.qk_fused")).ptr);
+        qi.q_norm = static_cast<const float *>(m_.Tensor(Model::Blk(l, "indexer.q_norm")).ptr);
+        qi.k_norm = static_cast<const float *>(m_.Tensor(Model::Blk(l, "indexer.k_norm")).ptr);
+        qi.rope = rope_;
+        const size_t slot_off = own_slot ? static_cast<size_t>(r.host_slot) : 0;
+        qi.idxcache = idxc_[l] + slot_off * n_kv_ * c_.IdxDim;
+        qi.pooled = pooled_[l] + slot_off * (n_kv_ / c_.IdxRatio + 1) * c_.IdxDim;
+        qi.pos = r.pos;
+        qi.slot = own_slot ? nullptr : r.slot;
+        qi.work = qsa_work_;
+        qi.score = qsa_score_;
+        qi.mask = qsa_mask_;
+        qi.n_seq = r.n_seq;
+        qi.seq_len = r.seq_len;
+        qi.n_embd = c_.NEmbd;
+        qi.idx_heads = c_.IdxHeads;
+        qi.idx_dim = c_.IdxDim;
+        qi.top_k = c_.IdxTopK;
+        qi.ratio = c_.IdxRatio;
+        qi.rope_dims = c_.RopeDims;
+        qi.max_cells = n_kv_;
+        qi.mask_stride = mask_stride_;
+        qi.eps = c_.RMSEps;
+        a.mask = qsa_mask_;
+        a.mask_stride = mask_stride_;
+    }
     shv_gemv_q4k_args o{};
     o.w = m_.Tensor(Model::Blk(l, "attn_output")).ptr;
     o.x = ctx_;
@@ -1022,6 +1105,10 @@ std::vector<shv_op> AttnGPU::Dispatches(int l, const float *in, float *out, cons
     o.fold_rows = r.fold_rows;
     o.fold_out = r.fold_out;
     o.fold_stride = r.fold_stride;
+    if (qsa) {
+        if (labels) labels->insert(labels->end(), {"attn.qkv", "attn.index", "attn.attn", "attn.out"});
+        return {make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_QSA_INDEX, qi), make_op(SHV_OP_ATTN_DECODE, a), make_op(SHV_OP_GEMV_Q4K, o)};
+    }
     if (labels) labels->insert(labels->end(), {"attn.qkv", "attn.attn", "attn.out"});
     return {make_op(SHV_OP_GEMV_Q4K, p), make_op(SHV_OP_ATTN_DECODE, a), make_op(SHV_OP_GEMV_Q4K, o)};
 }

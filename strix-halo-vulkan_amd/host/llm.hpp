@@ -83,6 +83,11 @@ struct Config {
     int SSMConv = 4;       // ssm.conv_kernel
     int AttnEvery = 4;     // every 4th layer is full attention, the rest gated DeltaNet
     int NextN = 0;         // nextn_predict_layers: 1 adds the draft head as block NLayer (llm/mtp.go:137)
+    // The block-sparse indexer beside the trunk's full-attention layers (AttnConfig.IdxHeads /
+    // IdxDim / TopK / Ratio, llm/attn.go:56-68; llm/model.go:385-405).  IdxRatio 0: dense layers.
+    int IdxHeads = 0, IdxDim = 0, IdxTopK = 0, IdxRatio = 0;
+    bool QSA(int layer) const { return IdxRatio > 0 && layer < NLayer && IsAttn(layer); }
+    int IdxRows() const { return IdxHeads * IdxDim + IdxDim; }  // the queries' rows, then the key's
 
     // The draft block is a full-attention layer (llm/mtp.go:17-21).
     bool IsAttn(int layer) const { return layer >= NLayer || (layer + 1) % AttnEvery == 0; }
@@ -327,6 +332,14 @@ private:
     float *in_, *out_, *qkv_, *ctx_, *partial_, *rope_;
     std::vector<void *> kc_, vc_;
     uint64_t cache_bytes_ = 0;
+    // the indexer of layers that have one: raw keys [slots][cells][IdxDim] binary16 and the pooled
+    // blocks' keys [slots][cells/ratio + 1][IdxDim] per layer; projection rows, scores and the
+    // selection's bit mask of one pass, shared by the layers
+    std::vector<uint16_t *> idxc_;
+    std::vector<float *> pooled_;
+    float *qsa_work_ = nullptr, *qsa_score_ = nullptr;
+    uint32_t *qsa_mask_ = nullptr;
+    int mask_stride_ = 0;
 };
 
 // llm.HeadGPU (llm/gpu_head.go:54-100, NewHeadGPUBank :114)

@@ -89,6 +89,7 @@ int shvllm_open(int device, const shvllm_config *c, shvllm **out) {
         cfg.SSMConv = c->ssm_conv;
         cfg.AttnEvery = c->attn_every;
         cfg.NextN = c->nextn;
+        cfg.IdxHeads = c->idx_heads, cfg.IdxDim = c->idx_dim, cfg.IdxTopK = c->idx_top_k, cfg.IdxRatio = c->idx_ratio;
         graph_opts(*h, *c);
         h->model = std::make_unique<llm::Model>(*h->dev, cfg);
         for (const auto &kv : h->model->Tensors()) h->names.push_back(kv.first);
@@ -143,6 +144,7 @@ int shvllm_get_config(shvllm *h, shvllm_config *o) {
         o->nkv = h->opts.NKV, o->layers = h->opts.Layers, o->no_head = h->opts.NoHead, o->attn_splits = h->opts.AttnSplits;
         o->max_tokens = h->opts.MaxTokens, o->slots = h->opts.Slots, o->head_rows = h->opts.HeadRows;
         o->speculative = h->opts.Speculative, o->spec_rows = h->opts.SpecRows;
+        o->idx_heads = c.IdxHeads, o->idx_dim = c.IdxDim, o->idx_top_k = c.IdxTopK, o->idx_ratio = c.IdxRatio;
     });
 }
 

@@ -27,6 +27,7 @@ typedef struct {
     int32_t max_tokens, slots, head_rows;        /* GraphOpts: rows a pass, sequences, rows with logits */
     int32_t speculative, spec_rows;              /* GraphOpts: rewindable passes and their width */
     int32_t nextn;                               /* 1: the model carries the draft block */
+    int32_t idx_heads, idx_dim, idx_top_k, idx_ratio;  /* the block-sparse indexer of the trunk's attention layers; ratio 0: none */
 } shvllm_config;
 
 const char *shvllm_last_error(void);

@@ -20,7 +20,8 @@ class Config(C.Structure):
                 ("ssm_conv", C.c_int32), ("attn_every", C.c_int32), ("nkv", C.c_int32),
                 ("layers", C.c_int32), ("no_head", C.c_int32), ("attn_splits", C.c_int32),
                 ("max_tokens", C.c_int32), ("slots", C.c_int32), ("head_rows", C.c_int32),
-                ("speculative", C.c_int32), ("spec_rows", C.c_int32), ("nextn", C.c_int32)]
+                ("speculative", C.c_int32), ("spec_rows", C.c_int32), ("nextn", C.c_int32),
+                ("idx_heads", C.c_int32), ("idx_dim", C.c_int32), ("idx_top_k", C.c_int32), ("idx_ratio", C.c_int32)]
 
     def __init__(self, **kw):
         d = dict(n_layer=48, n_embd=2048, n_head=16, n_head_kv=2, head_dim=256, rope_dims=64,

@@ -220,3 +220,75 @@ def test_decode_over_a_long_cache_reads_what_the_indexer_names(ctx):
     # and it matters: the dense layer over the same cache gives other numbers
     dense = dev.run(x, past, masked=False)
     assert O.rel_l2(dense["pre"], want["pre"]) > 1e-2
+
+
+# ---- through the op surface: AttnGPU with Ratio > 0 inside the token loop ------------------------
+
+LA = shv.pkg.llm_api
+
+
+def test_token_loop_with_an_indexer_matches_the_cpu_loop(tmp_path):
+    """A four-layer model (three DeltaNet layers and one full-attention layer with an indexer of
+    four heads, top 16, ratio 4): a prompt of 70 in passes of 64 and 6, then greedy steps through
+    the recorded one-row pass, against the CPU loop over the same tensors.  Past 19 cells the
+    attention layer reads a selection; the logits stay the CPU's and the ids equal.  The same
+    model staged without the indexer's cut (top_k as large as the cache) gives other logits: the
+    selection is really applied."""
+    kw = dict(n_layer=4, n_expert=16, n_expert_used=4, vocab=4096, nkv=256, max_tokens=64, idx_heads=4, idx_dim=128, idx_top_k=16, idx_ratio=4)
+    cfg = LA.Config(**kw)
+    m = LA.LLM(cfg)
+    try:
+        m.init_synthetic(99)
+        m.stage()
+        names = [t[0] for t in m.tensors()]
+        assert "blk.3.indexer.q_proj.weight" in names and "blk.3.indexer.k_norm.weight" in names and "blk.0.indexer.q_proj.weight" not in names
+        tensors = {t[0]: m.download(t[0]) for t in m.tensors()}
+        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+        rng = np.random.default_rng(5)
+        prompt = rng.integers(0, cfg.vocab, size=70).astype(np.int32)
+        lg_gpu, hd_gpu = m.extend(prompt, want_hidden=True)
+        lg_cpu, hd_cpu = om.extend(prompt)
+        assert O.rel_l2(hd_gpu, hd_cpu) <= 1e-3 and O.rel_l2(lg_gpu, lg_cpu) <= 1e-3
+        lg = lg_cpu
+        for i in range(6):
+            tok = int(O.lib().shv_ref_argmax(O.F(lg), cfg.vocab))
+            assert int(np.argmax(lg_gpu)) == tok
+            lg, _ = om.extend(np.array([tok], np.int32))
+            lg_gpu, _ = m.extend(np.array([tok], np.int32))
+            assert O.rel_l2(lg_gpu, lg) <= 1e-3, i
+        # the device loop (arg-max in the launch, positions on the device) walks the same ids
+        m.reset()
+        m.extend(prompt)
+        ids_gpu, _ = m.generate(6)
+        om2 = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
+        lg, _ = om2.extend(prompt)
+        want = []
+        for i in range(6):
+            want.append(int(O.lib().shv_ref_argmax(O.F(lg), cfg.vocab)))
+            lg, _ = om2.extend(np.array([want[-1]], np.int32))
+        assert list(ids_gpu) == want
+        # the checkpoint carries the indexer: its shape in the metadata (llm/model.go:385-405), its
+        # projections under their own names, and what is read back decodes bit for bit
+        path = tmp_path / "qsa.gguf"
+        m.save_gguf(path)
+        m.reset()
+        lg_a, _ = m.extend(prompt)
+    finally:
+        m.close()
+    back = LA.LLM(LA.Config(nkv=256, max_tokens=64), gguf=path)
+    try:
+        assert (back.cfg.idx_heads, back.cfg.idx_dim, back.cfg.idx_top_k, back.cfg.idx_ratio) == (4, 128, 16, 4)
+        back.stage()
+        lg_b, _ = back.extend(prompt)
+        assert np.array_equal(lg_a, lg_b)
+    finally:
+        back.close()
+    # without the cut
+    wide = LA.LLM(LA.Config(**dict(kw, idx_top_k=256)))
+    try:
+        wide.init_synthetic(99)
+        wide.stage()
+        lg_wide, _ = wide.extend(prompt)
+        assert O.rel_l2(lg_wide, lg_cpu) > 1e-3
+    finally:
+        wide.close()
