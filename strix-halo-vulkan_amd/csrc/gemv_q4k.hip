@@ -873,9 +873,13 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
             default: return shv_set_error(SHV_E_INVALID, "gemv_q4k: k = %d; built for 512, 1024, 2048 and 4096", a.k);
         }
     }
-    // two to four rows of one sequence: the one-row kernel's shape with the rows side by side (SHV_MFMA_MIN_ROWS
-    // at or below the row count sends them to the matrix cores instead, as before)
-    if (fewrows_kernel_covers(ctx, a) && !ctx->mfma_rows_forced)
+    // two to eight rows: every weight formed once for all of them, the products on the matrix cores; 4096 columns
+    // wide, up to four rows of one sequence are quicker side by side in the one-row kernel's shape (6.7 against
+    // 8.0 us for three rows of a 2048 x 4096 output projection: a block there stages 16 K columns a row)
+    const bool few = fewrows_kernel_covers(ctx, a) && !ctx->mfma_rows_forced;
+    if (!ctx->mfma_rows_forced && !(few && a.k == 4096) && shv_gemv_mrows_covers(ctx, a)) return shv_launch_gemv_mrows(ctx, a);
+    // (SHV_MFMA_MIN_ROWS at or below the row count sends few rows to the tiled matrix-core kernels instead, as before)
+    if (few)
         return a.n_tok == 2 ? launch_fewrows<2>(ctx, a) : a.n_tok == 3 ? launch_fewrows<3>(ctx, a) : launch_fewrows<4>(ctx, a);
     if (a.n_tok >= (a.k > 2048 ? ctx->mfma_min_rows_wide : ctx->mfma_min_rows) && shv_gemm_q4k_covers(a)) return shv_launch_gemm_q4k(ctx, a);
     SHV_REQUIRE(a.n_tok <= 64, "gemv_q4k: %d rows: more than 64 go through the matrix-core kernel, which does not take this shape (k %d, prologue %d)",

@@ -30,6 +30,9 @@ struct shv_ctx {
     // passes of this many rows up to 16 (8 where rows are 4096 wide) take the sixteen-wave matrix-core kernel that
     // stages its rows under the weight loads (SHV_GEMM_ROWS_MIN; 0: never)
     int gemm_rows_min = 5;
+    // SHV_MROWS=0: projections of two to eight rows go the ways they went before the kernel that forms each weight
+    // once for all rows (the side-by-side row kernel up to four rows, the tiled matrix-core kernels above)
+    bool mrows_off = false;
     int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)
     int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
@@ -128,6 +131,8 @@ static inline bool shv_aligned16(const void *p) { return (reinterpret_cast<uintp
 int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *a);
 // the matrix-core kernel for passes of two rows and more (gemm_q4k.hip)
 bool shv_gemm_q4k_covers(const shv_gemv_q4k_args &a);
+bool shv_gemv_mrows_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a);
+int shv_launch_gemv_mrows(shv_ctx *ctx, const shv_gemv_q4k_args &a);
 int shv_launch_gemm_q4k(shv_ctx *ctx, const shv_gemv_q4k_args &a);
 bool shv_router_wide_covers(const shv_ctx *ctx, const shv_moe_router_args &a);
 int shv_launch_router_wide(shv_ctx *ctx, const shv_moe_router_args &a);

@@ -199,7 +199,7 @@ def test_full_size_model_matches_the_cpu_loop():
         tensors = {t[0]: m.download(t[0]) for t in m.tensors()}
         om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
         check = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
-        greedy_done = False
+        greedy_done, lost = False, 0
         for seed in (17, 18, 19, 20, 21):   # until a prompt without a flipped row lets the greedy steps be compared
             m.reset()
             om.reset()
@@ -218,7 +218,13 @@ def test_full_size_model_matches_the_cpu_loop():
             so_far = np.minimum.accumulate(gaps)
             within = [e <= 1e-3 for e in errs]
             assert all(w or g < GAP for w, g in zip(within, so_far)), (errs, list(so_far))
-            assert sum(within) >= 4
+            if sum(within) < 4:
+                # the near-tie sits in one of the first rows and every later row reads its state: this prompt says
+                # nothing further; at most two prompts of the five may go that way
+                lost += 1
+                print("full size: seed %d: a router gap of %.1e in row %d; next prompt" % (seed, so_far[within.index(False)], within.index(False)), flush=True)
+                assert lost <= 2
+                continue
             compared = 0
             if all(within):
                 assert O.rel_l2(lg_rows[-1], lg_cpu) <= 1e-3
@@ -273,19 +279,37 @@ def _full_size_speculative_round(m, cfg, tensors, prompt):
     m.extend(prompt)
     plain = [int(t) for t in m.generate(n_new + depth + 1)[0]]
     # the verification pass itself against the CPU: the pending token and two drafts as three
-    # rewindable rows, every row's logits
+    # rewindable rows, every row's logits.  A row at or behind a router near-tie of the oracle's own
+    # (in the pass or in what was fed before it, as in the prompt pass above) may hold another
+    # expert's output and says nothing; the pass is then taken one token further on, and one of
+    # four such passes must agree in every row.
+    GAP = 4e-4
     om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv)
-    om.extend(prompt, threads=16)
-    m.reset()
-    m.extend(prompt)
-    m.speculate(True)
-    rows = np.array(plain[:depth + 1], np.int32)
-    _, lg_rows, _ = m.extend_rows(rows, want_logits=True, want_res=True)
-    lg_cpu, _ = om.extend_rows(rows, threads=16)
-    errs = [O.rel_l2(lg_rows[t], lg_cpu[t]) for t in range(depth + 1)]
-    print("full size: verification pass rows' logits rel-L2", ["%.2e" % e for e in errs], flush=True)
-    assert max(errs) <= 1e-3
-    m.rewind()
+    gamma = tensors["output_norm.weight"]
+    clean = False
+    for start in range(4):
+        before = np.concatenate([prompt, np.array(plain[:start], np.int32)])
+        rows = np.array(plain[start:start + depth + 1], np.int32)
+        om.reset()
+        _, _, gaps_before = _oracle_rows_with_gaps(om, tensors, cfg, before)
+        x_cpu, _, gaps = _oracle_rows_with_gaps(om, tensors, cfg, rows)
+        lg_cpu = [O.gemv_q4k(tensors["output.weight"], O.rmsnorm(x_cpu[t:t + 1], gamma, cfg.rms_eps)[0], cfg.vocab, cfg.n_embd, threads=16)
+                  for t in range(depth + 1)]
+        m.speculate(False)
+        m.reset()
+        m.extend(before)
+        m.speculate(True)
+        _, lg_rows, _ = m.extend_rows(rows, want_logits=True, want_res=True)
+        m.rewind()
+        errs = [O.rel_l2(lg_rows[t], lg_cpu[t]) for t in range(depth + 1)]
+        print("full size: verification pass after %d tokens: rows' logits rel-L2" % start, ["%.2e" % e for e in errs],
+              "gaps", ["%.1e" % g for g in gaps], flush=True)
+        so_far = np.minimum.accumulate(np.concatenate([gaps_before, gaps]))[-(depth + 1):]
+        assert all(e <= 1e-3 or g < GAP for e, g in zip(errs, so_far)), (errs, list(so_far))
+        if max(errs) <= 1e-3:
+            clean = True
+            break
+    assert clean, "every verification pass of four sat behind a router near-tie"
     m.speculate(False)
     # the loop: true continuations as drafts in even rounds, the draft head's own in odd ones
     m.reset()
