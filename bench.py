@@ -114,13 +114,13 @@ def cpu_baseline(m, cfg, LA, A, tensors, n_tokens, cores):
     err = O.rel_l2(got, hidden)
     if not err <= 1e-3:
         raise SystemExit("bench.py: the GPU's residual stream after layer %d differs from the oracle's by rel-L2 %.3e (> 1e-3)" % (per - 1, err))
-    return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "kind": "port", "sample_seconds": round(dt * n_tokens, 2),
+    return {"value": round(1.0 / per_token, 3), "unit": "tok/s", "cores": cores, "host_cpus": os.cpu_count(), "kind": "port", "sample_seconds": round(dt * n_tokens, 2),
             "hidden_rel_l2_vs_gpu": float("%.3e" % err),
             "sample": "C restatement of the reference's Go CPU path (oracle/), layers 0-%d + lm_head of the same "
                       "weights, %d decode tokens at context <= %d; period time x%d + head time; rows of each matvec "
-                      "split over %d threads; the GPU path over the same four layers and tokens leaves a residual "
-                      "stream within rel-L2 %.1e of the oracle's (checked here, bound 1e-3)"
-                      % (per - 1, n_tokens, n_tokens + 1, periods, cores, err)}
+                      "split over %d threads (os.cpu_count() of this host: %s); the GPU path over the same four layers "
+                      "and tokens leaves a residual stream within rel-L2 %.1e of the oracle's (checked here, bound 1e-3)"
+                      % (per - 1, n_tokens, n_tokens + 1, periods, cores, os.cpu_count(), err)}
 
 
 def gemv_rates(m, cfg, A, LA):
@@ -601,9 +601,13 @@ def main():
         traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
     # one-row passes route in the expert kernel itself unless LLM_MOE_ROUTE=kernel keeps the selection a launch of its own
     fused = os.environ.get("LLM_MOE_ROUTE", "rows") in ("rows", "fused")
-    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048, 1> (%sexpert-gathered Q4_K gate/up GEMV + SwiGLU)" %
-                      ("softmax and top-10 of the token's 512 router logits, then the " if fused else ""),
+    # the router's logits ride on the mixer's output projection unless LLM_ROUTER_FOLD=0; gate/up then also normalises its row
+    folded = fused and os.environ.get("LLM_ROUTER_FOLD", "1") != "0"
+    roof = {"bound": "hbm", "kernel": "moe_up_kernel<2048, 1%s> (%sexpert-gathered Q4_K gate/up GEMV + SwiGLU)" %
+                      (", true" if folded else "", ("RMSNorm of the residual row, " if folded else "") +
+                       ("softmax and top-10 of the token's 512 router logits, then the " if fused else "")),
             "routing": "in this launch" if fused else "a launch of its own",
+            "router_logits": "rows of the mixer's output projection launch" if folded else "a launch of their own",
             "achieved": round(up_bytes / (up_ns / 1e9) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": round(up_bytes / (up_ns / 1e9) / HBM_PEAK, 4), "traffic": traffic,
             "bytes_per_launch": up_bytes, "avg_launch_us": round(up_ns / 1e3, 3), "launches_per_step": cfg.n_layer}
@@ -621,7 +625,10 @@ def main():
                    "weights_GB": round(m.weight_bytes() / 1e9, 2), "dispatches_per_step": m.dispatches()},
         "gpu_ms_per_step": round(gpu_ns / a.steps / 1e6, 4),
         "token_bytes": tb, "token_roofline_tok_s": round(HBM_PEAK / tb, 1), "frac_of_token_roofline": round(tok_s * tb / HBM_PEAK, 4),
-        "step_kernel_us": {k: round(v / 1e3, 1) for k, v in sorted(acc.items(), key=lambda kv: -kv[1])},
+        # each op's own duration in an op-by-op profiled step (events around every op), and their sum; the wall time
+        # of such a step, which the events themselves stretch, is not reported
+        "step_kernel_us": dict([("sum_of_ops", round(sum(v for k, v in acc.items() if k != "total") / 1e3, 1))] +
+                               [(k, round(v / 1e3, 1)) for k, v in sorted(acc.items(), key=lambda kv: -kv[1]) if k != "total"]),
         "roofline": roof,
         "gemv": gemv_rates(m, cfg, A, LA),
     }

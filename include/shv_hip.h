@@ -93,6 +93,7 @@ enum {
     SHV_OP_RING_ROWS = 15,
     SHV_OP_ROUTER_FOLD = 16,
     SHV_OP_QSA_INDEX = 17,
+    SHV_OP_ARGMAX_STATIC = 18, /* shv_argmax_static as an op, so that a recorded sequence can hold it */
     SHV_OP__COUNT
 };
 

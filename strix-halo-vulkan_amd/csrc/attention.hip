@@ -900,11 +900,11 @@ int launch_rows(shv_ctx *ctx, const shv_attn_decode_args &a, int row0, int n_gro
     const int slice_cells = a.n_seq * n_groups == 1 ? kTile : kSliceCells;
     if (R == 2 && !append && row0 == 0 && n_groups >= 8) {
         // a prompt pass: eight pairs a block share the cache's tiles
-        static bool raised = false;
-        if (!raised) {
+        static std::atomic<bool> raised{false};
+        if (!raised.load(std::memory_order_acquire)) {
             SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
             SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_prefill_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(PrefillSmem))));
-            raised = true;
+            raised.store(true, std::memory_order_release);
         }
         // with one slice a pair there is nothing to merge: the kernel writes the rows themselves
         const int direct = b.n_splits == 1 ? 1 : 0;

@@ -461,10 +461,10 @@ int shv_launch_dn_chunk(shv_ctx *ctx, const shv_dn_step_args &a) {
     const int pw = 2 * a.n_head_k * kD + a.n_head_v * kD + 2 * a.n_head_v;
     const int items = 2 * a.n_head_k / 4 + a.n_head_v * kD / kThreads + 1;
     SHV_LAUNCH(ctx, dn_prep_kernel, dim3(items, (a.seq_len + kPrepTok - 1) / kPrepTok, a.n_seq), dim3(kThreads), 0, a, a.work, pw);
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&dn_chunk_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(ChunkLds))));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     SHV_LAUNCH(ctx, dn_chunk_kernel, dim3(a.n_head_v * (kD / kJ), a.n_seq), dim3(kThreads), sizeof(ChunkLds), a, static_cast<const float *>(a.work), pw);
     return SHV_OK;

@@ -1298,11 +1298,11 @@ int launch_tt(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const ch
     SHV_REQUIRE(nt * (a.k / 4) <= MAXQ * NTHR, "gemm_q4k: %d rows of %d columns are more than one block stages", nt, a.k);
     const int n_tiles = (a.n + kTileRows - 1) / kTileRows;
     const size_t lds = Lds<TT>::total(a.k, NW);
-    static size_t raised = 0;
-    if (lds > 48 * 1024 && lds > raised) {
+    static std::atomic<size_t> raised{0};
+    if (lds > 48 * 1024 && lds > raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_kernel<TT, NTHR, MAXQ>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = lds;
+        raised.store(lds, std::memory_order_release);
     }
     int per_cu = 0;
     SHV_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(&gemm_q4k_kernel<TT, NTHR, MAXQ>), NTHR, lds));
@@ -1349,10 +1349,10 @@ int launch_wide(shv_ctx *ctx, const shv_gemv_q4k_args &a, int t0, int nt, const 
     // More than half a compute unit's LDS, so that two blocks never share one: a launch of fewer
     // blocks than compute units would otherwise double up on some and leave others idle.
     const size_t lds = std::max<size_t>(2 * kWideSlab + kWideTok * sizeof(size_t), 84 * 1024);
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wide_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     SHV_LAUNCH(ctx, (gemm_wide_kernel<NW, R>), dim3(bx, ks), dim3(NW * 64), lds, a, t0, nt, staged, ctx->gemm_part, steps / ks, 1);
     if (ks > 1) {
@@ -1378,10 +1378,10 @@ int launch_rows_kp(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     int blocks = (n_tiles + tpb - 1) / tpb;
     if (blocks > ctx->prop.multiProcessorCount) blocks = ctx->prop.multiProcessorCount;
     constexpr size_t lds = RowsLds<K>::total;
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows_kernel<K, PRO, RD>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     for (int t0 = 0; t0 < a.n_tok; t0 += kRowsTok) {
         const int nt = a.n_tok - t0 < kRowsTok ? a.n_tok - t0 : kRowsTok;
@@ -1417,10 +1417,10 @@ int launch_wide_all(shv_ctx *ctx, const shv_gemv_q4k_args &a, int groups) {
     constexpr int kRows = NW * R * kTileRows;
     const int bx = (a.n + kRows - 1) / kRows;
     const size_t lds = 2 * kWideSlab + kWideSumFrags + kWideTok * sizeof(size_t);
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_pass_kernel<NW, R>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     SHV_REQUIRE(static_cast<long long>(bx) * groups <= 0x7fffffffll, "gemm_q4k: %d row blocks of %d groups", bx, groups);
     SHV_LAUNCH(ctx, (gemm_pass_kernel<NW, R>), dim3(bx * groups), dim3(NW * 64), lds, a, static_cast<const char *>(ctx->gemm_stage), groups);
@@ -1454,10 +1454,10 @@ int shv_launch_router_wide(shv_ctx *ctx, const shv_moe_router_args &a) {
     const int n_rows = a.n_expert + (a.shared_gate ? 1 : 0);
     const int bx = (n_rows + NW * kTileRows - 1) / (NW * kTileRows);
     const size_t lds = 2 * kWideSlab;
-    static bool raised = false;
-    if (!raised) {
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&router_wide_kernel<NW>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     SHV_LAUNCH(ctx, (router_wide_kernel<NW>), dim3(bx * groups), dim3(NW * 64), lds, a.router, a.shared_gate, n_rows, a.n_embd, a.n_tok,
                static_cast<const char *>(ctx->gemm_stage), a.logits, a.n_expert + 1, groups);

@@ -43,10 +43,10 @@ int launch_type(shv_ctx *ctx, const shv_gemv_args &a) {
     SHV_REQUIRE(blocks < (1ll << 31), "gemv: %d rows is too many for one launch", a.n);
     const size_t lds = static_cast<size_t>(a.k) * 4;
     SHV_REQUIRE(lds <= 64 * 1024, "gemv: k = %d does not fit the staging of x", a.k);
-    static bool raised = false;
-    if (lds > 48 * 1024 && !raised) {
+    static std::atomic<bool> raised{false};
+    if (lds > 48 * 1024 && !raised.load(std::memory_order_acquire)) {
         SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_any_kernel<TYPE>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
     SHV_LAUNCH(ctx, gemv_any_kernel<TYPE>, dim3(static_cast<unsigned>(blocks)), dim3(kBlock), lds, a);
     return SHV_OK;

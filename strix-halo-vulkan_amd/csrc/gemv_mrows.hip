@@ -344,10 +344,10 @@ template <int K, int PRO, int NT, int TILES>
 int launch_tiles(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     const size_t lds = mrows_lds<K, NT, TILES>();
     if (lds > 48 * 1024) {
-        static bool raised = false;  // above the default allowance the limit is raised once per kernel
-        if (!raised) {
+        static std::atomic<bool> raised{false};  // above the default allowance the limit is raised once per kernel
+        if (!raised.load(std::memory_order_acquire)) {
             SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mrows_kernel<K, PRO, NT, TILES>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            raised = true;
+            raised.store(true, std::memory_order_release);
         }
     }
     SHV_LAUNCH(ctx, (gemv_mrows_kernel<K, PRO, NT, TILES>), dim3((a.n + 16 * TILES - 1) / (16 * TILES)), dim3(256), lds, a);

@@ -743,11 +743,11 @@ template <int K, int NT, int U>
 int launch_ntu(shv_ctx *ctx, const shv_gemv_q4k_args &a, dim3 grid, dim3 block, size_t lds, int ppw, int t0) {
     if (lds > 48 * 1024) {
         // above the default dynamic-LDS allowance the limit has to be raised once per kernel
-        static bool raised = false;
-        if (!raised) {
+        static std::atomic<bool> raised{false};
+        if (!raised.load(std::memory_order_acquire)) {
             SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_kernel<K, NT, U>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            raised = true;
+            raised.store(true, std::memory_order_release);
         }
     }
     if constexpr (NT == 1) {

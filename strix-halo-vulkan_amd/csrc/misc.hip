@@ -1,4 +1,6 @@
 // Format-level kernels: bit-exact Q4_K dequantisation and on-device synthetic fill.
+#include <mutex>
+
 #include "shv_device.hpp"
 #include "shv_internal.hpp"
 
@@ -186,6 +188,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
 void *g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;  // shv_init may run on several threads at once
 
 __global__ void clear_counters_kernel(int32_t *c, int n) {
     if (static_cast<int>(threadIdx.x) < n) c[threadIdx.x] = 0;
@@ -205,6 +208,7 @@ int shv_launch_ring_rows(shv_ctx *ctx, const shv_ring_rows_args *pa) {
 
 int shv_static_scratch_bind(shv_ctx *ctx) {
     SHV_REQUIRE(ctx->device >= 0 && ctx->device < kMaxDevices, "shv_init: device %d; the static scratch table covers %d devices", ctx->device, kMaxDevices);
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
     if (!g_scratch_ptr[ctx->device]) {
         void *p = nullptr;
         SHV_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));  // the calling thread's current device is ctx->device

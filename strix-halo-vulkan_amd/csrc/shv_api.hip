@@ -227,6 +227,7 @@ static int dispatch_one(shv_ctx *ctx, uint32_t kind, const void *args, size_t by
         case SHV_OP_RING_ROWS: return run_as<shv_ring_rows_args>(ctx, args, bytes, shv_launch_ring_rows, "ring_rows");
         case SHV_OP_ROUTER_FOLD: return run_as<shv_router_fold_args>(ctx, args, bytes, shv_launch_router_fold, "router_fold");
         case SHV_OP_QSA_INDEX: return run_as<shv_qsa_index_args>(ctx, args, bytes, shv_launch_qsa_index, "qsa_index");
+        case SHV_OP_ARGMAX_STATIC: return run_as<shv_argmax_args>(ctx, args, bytes, shv_launch_argmax_static, "argmax_static");
         default: return shv_set_error(SHV_E_INVALID, "shv_enqueue: unknown op kind %u", kind);
     }
 }

@@ -11,6 +11,7 @@ Q4K_BYTES = 144
 OP_GEMV_Q4K, OP_DEQUANT_Q4K, OP_QUANTIZE_Q4K, OP_FILL_NORMAL = 1, 2, 3, 4
 OP_MOE_ROUTER, OP_MOE_UP, OP_MOE_DOWN, OP_DN_STEP, OP_ATTN_DECODE = 5, 6, 7, 8, 9
 OP_EMBED, OP_ARGMAX, OP_ADVANCE, OP_DEQUANT, OP_GEMV, OP_RING_ROWS, OP_ROUTER_FOLD, OP_QSA_INDEX = 10, 11, 12, 13, 14, 15, 16, 17
+OP_ARGMAX_STATIC = 18
 PRO_NONE, PRO_RMSNORM, PRO_GATED_NORM, PRO_MUL_SIGMOID, PRO_RMSNORM_PAIR = 0, 1, 2, 3, 4
 
 

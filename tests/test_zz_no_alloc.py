@@ -60,3 +60,28 @@ def test_static_argmax_stores_the_next_token_and_refuses_too_many_rows(ctx):
     args = A.ArgmaxArgs(x.ptr, out.ptr, None, None, rows, 64, 64)
     assert L.shv_argmax_static(ctx.h, C.byref(args)) == -1
     assert b"at most 14 rows" in L.shv_last_error()
+
+
+def test_static_argmax_recorded_into_a_graph_and_replayed(ctx):
+    """Its stated callers record it: the op (counters cleared by a kernel, then the arg-max) goes into a
+    recorded sequence of the library, which replays as a HIP graph; three replays, with other eager
+    work and new logits in the same buffer between them, each against shv_argmax on the same rows."""
+    L = A.load()
+    rng = np.random.default_rng(5)
+    rows, n = 3, 151936
+    dev = ctx.upload(np.zeros((rows, n), np.float32))
+    best = ctx.upload(np.full(rows, -7, np.int32))
+    rec = ctx.prerecord([A.make_op(A.OP_ARGMAX_STATIC, A.ArgmaxArgs(dev.ptr, best.ptr, None, None, rows, n, n))])
+    try:
+        for rep in range(3):
+            logits = rng.standard_normal((rows, n)).astype(np.float32)
+            logits[rep % rows, [rep, n - 1 - rep]] = 7.0        # a tie across blocks: the lower index
+            dev.write(logits)
+            best.write(np.full(rows, -7, np.int32))
+            rec.submit(1)
+            got = list(best.read(np.int32, rows))
+            eager = ctx.upload(np.full(rows, -7, np.int32))
+            A.check(L.shv_argmax(ctx.h, C.byref(A.ArgmaxArgs(dev.ptr, eager.ptr, None, None, rows, n, n))))
+            assert got == list(eager.read(np.int32, rows)) == list(np.argmax(logits, axis=1)), rep
+    finally:
+        rec.destroy()
