@@ -140,6 +140,15 @@ type GemvOpts struct {
 	RingSlots, RingStride int // y (or, with ZRing, z) is a ring of projection rows addressed by position
 	ZRing               bool
 	YFlat               *Buffer // one-row ring output: the row once more at a fixed address
+	// The router's logits in the same launch (the mixer's output projection of a pass of one to
+	// three rows): Fold is the layer's table made by RouterFold, FoldOut receives FoldRows products
+	// a row, FoldStride floats apart; Residual must not be y.
+	Fold, FoldOut        *Buffer
+	FoldRows, FoldStride int
+	// The greedy sampler in the same launch (a one-row vocabulary projection): what Argmax does
+	// with best / ids / pos / advance.
+	AmaxBest, AmaxIds, AmaxPos *Buffer
+	AmaxAdvance                int
 }
 
 // GemvQ4K is llm_gemv_q4k.comp / llm_gemm_q4k.comp: y[t] = W pro(x[t]) (+ residual[t]) for rows
@@ -157,6 +166,10 @@ func GemvQ4K(w, x, y *Buffer, n, k, rows int, o GemvOpts) Op {
 		a.z_ring = 1
 	}
 	a.y_flat = fp(o.YFlat)
+	a.fold, a.fold_out = fp(o.Fold), fp(o.FoldOut)
+	a.fold_rows, a.fold_stride = C.int32_t(o.FoldRows), C.int32_t(o.FoldStride)
+	a.amax_best, a.amax_ids, a.amax_pos = ip(o.AmaxBest), ip(o.AmaxIds), ip(o.AmaxPos)
+	a.amax_advance = C.int32_t(o.AmaxAdvance)
 	return mk(C.SHV_OP_GEMV_Q4K, unsafe.Pointer(&a), C.sizeof_shv_gemv_q4k_args)
 }
 
@@ -179,6 +192,33 @@ func MoERouter(h, gamma, router, sharedGate, xn, logits, topk, weights *Buffer, 
 		a.defer_route = 1
 	}
 	return mk(C.SHV_OP_MOE_ROUTER, unsafe.Pointer(&a), C.sizeof_shv_moe_router_args)
+}
+
+// RouterFold makes a layer's table [R diag(gamma) W | R diag(gamma)] (nExpert rows of k + nEmbd
+// floats) from the float32 router, the post-attention norm's gamma and the Q4_K output projection
+// W [nEmbd][k]; scratch holds nEmbd * k floats and may be freed afterwards.  Run once when the
+// graph is staged, where the reference makes its dense banks (llm/bank_q4.go:172-266).
+func RouterFold(router, gamma, wOut, out, scratch *Buffer, nExpert, nEmbd, k int) Op {
+	var a C.shv_router_fold_args
+	a.router, a.gamma, a.w_out = fp(router), fp(gamma), vp(wOut)
+	a.out, a.scratch = fp(out), fp(scratch)
+	a.n_expert, a.n_embd, a.k = C.int32_t(nExpert), C.int32_t(nEmbd), C.int32_t(k)
+	return mk(C.SHV_OP_ROUTER_FOLD, unsafe.Pointer(&a), C.sizeof_shv_router_fold_args)
+}
+
+// MoENorm is what MoEUp needs when the router's logits came from the output projection (GemvOpts.Fold):
+// xn is then the un-normalised residual row; the kernel normalises it, scales the logits by the same
+// factor and forms the shared expert's gate.
+type MoENorm struct {
+	Gamma, SharedGate *Buffer
+	Eps               float32
+}
+
+// WithNorm sets those fields on an op made by MoEUp.
+func (o Op) WithNorm(n MoENorm) Op {
+	a := (*C.shv_moe_up_args)(unsafe.Pointer(&o.args[0]))
+	a.gamma, a.shared_gate, a.eps = fp(n.Gamma), fp(n.SharedGate), C.float(n.Eps)
+	return o
 }
 
 // MoEBanks names the six expert banks and their ggml types (gguf.Tensor.Type).
