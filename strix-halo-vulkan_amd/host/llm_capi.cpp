@@ -6,10 +6,12 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <set>
 
 #include "llm.hpp"
 #include "sampler_handle.hpp"
 #include "sched.hpp"
+#include "text.hpp"
 
 struct shvllm {
     std::unique_ptr<llm::Device> dev;
@@ -820,6 +822,280 @@ int64_t shvgguf_size_of(uint32_t type, int64_t n) {
     int64_t out = -1;
     guard([&] { out = gguf::SizeOf(type, n); });
     return out;
+}
+
+
+// ---- text: tokenizer, stop set, chat template, completion reader ---------------------------------
+
+struct shvtext_tokenizer {
+    llm::text::Tokenizer tok;
+};
+struct shvtext_decoder {
+    llm::text::ChatDecoder dec;
+    std::string stopped;
+};
+
+static char *dup_bytes(const std::string &s, uint64_t *len) {
+    char *p = static_cast<char *>(std::malloc(s.size() + 1));
+    if (!p) throw std::bad_alloc();
+    std::memcpy(p, s.data(), s.size());
+    p[s.size()] = 0;
+    if (len) *len = s.size();
+    return p;
+}
+static std::string bytes_of(const char *p, uint64_t len) { return p ? std::string(p, static_cast<size_t>(len)) : std::string(); }
+static std::vector<std::string> tools_of(const char *tools_json) {
+    std::vector<std::string> tools;
+    if (tools_json && *tools_json) {
+        const llm::text::JValue v = llm::text::ParseJSON(tools_json);
+        if (v.kind != llm::text::JValue::Array) throw llm::text::Error("llm: tools is not a JSON array");
+        for (const auto &t : v.items) tools.push_back(t.raw);
+    }
+    return tools;
+}
+
+void shvtext_free(void *p) { std::free(p); }
+
+int shvtext_tokenizer_from_vocab(const char *const *tokens, const uint64_t *token_len, int n_tokens, const char *const *merges,
+                                 const uint64_t *merge_len, int n_merges, const int32_t *types, const char *const *specials,
+                                 int n_specials, const char *pre, shvtext_tokenizer **out) {
+    return guard([&] {
+        if (!out || (n_tokens > 0 && (!tokens || !token_len)) || (n_merges > 0 && (!merges || !merge_len))) throw llm::text::Error("tokenizer: NULL argument");
+        llm::text::Vocab v;
+        for (int i = 0; i < n_tokens; i++) v.Tokens.emplace_back(tokens[i], static_cast<size_t>(token_len[i]));
+        for (int i = 0; i < n_merges; i++) v.Merges.emplace_back(merges[i], static_cast<size_t>(merge_len[i]));
+        if (types) v.Types.assign(types, types + n_tokens);
+        for (int i = 0; i < n_specials; i++) v.Specials.emplace_back(specials[i]);
+        if (pre) v.Pre = pre;
+        *out = new shvtext_tokenizer{llm::text::Tokenizer::FromVocab(v)};
+    });
+}
+
+int shvtext_tokenizer_from_gguf(shvgguf *g, shvtext_tokenizer **out, int32_t *eog, int eog_max, int *n_eog) {
+    return guard([&] {
+        if (!out) throw llm::text::Error("tokenizer: NULL argument");
+        auto t = std::make_unique<shvtext_tokenizer>(shvtext_tokenizer{llm::text::Tokenizer::FromGGUF(*gg(g).kv)});
+        const std::set<int32_t> stop = llm::text::EndOfGeneration(*gg(g).kv, t->tok);
+        if (n_eog) *n_eog = static_cast<int>(stop.size());
+        int k = 0;
+        for (int32_t id : stop)
+            if (eog && k < eog_max) eog[k++] = id;
+        *out = t.release();
+    });
+}
+
+void shvtext_tokenizer_free(shvtext_tokenizer *t) { delete t; }
+int shvtext_tokenizer_size(shvtext_tokenizer *t) { return t ? t->tok.Size() : 0; }
+int shvtext_tokenizer_id(shvtext_tokenizer *t, const char *token, int32_t *id) {
+    int32_t v = -1;
+    const bool ok = t && token && t->tok.ID(token, &v);
+    if (id) *id = v;
+    return ok ? 1 : 0;
+}
+
+int shvtext_encode(shvtext_tokenizer *t, const char *text, uint64_t len, int32_t **ids, int *n) {
+    return guard([&] {
+        if (!t || !ids || !n) throw llm::text::Error("tokenizer: NULL argument");
+        const std::vector<int32_t> v = t->tok.Encode(bytes_of(text, len));
+        int32_t *p = static_cast<int32_t *>(std::malloc((v.size() + 1) * sizeof(int32_t)));
+        if (!p) throw std::bad_alloc();
+        std::copy(v.begin(), v.end(), p);
+        *ids = p;
+        *n = static_cast<int>(v.size());
+    });
+}
+
+int shvtext_decode(shvtext_tokenizer *t, const int32_t *ids, int n, char **out, uint64_t *len) {
+    return guard([&] {
+        if (!t || !out || (n > 0 && !ids)) throw llm::text::Error("tokenizer: NULL argument");
+        *out = dup_bytes(t->tok.Decode(std::vector<int32_t>(ids, ids + n)), len);
+    });
+}
+
+int shvtext_split(const char *text, uint64_t len, int marks, char **out, uint64_t *out_len, int32_t **piece_len, int *n) {
+    return guard([&] {
+        if (!out || !piece_len || !n) throw llm::text::Error("tokenizer: NULL argument");
+        const std::vector<std::string> pieces = llm::text::Split(bytes_of(text, len), marks != 0);
+        std::string all;
+        int32_t *lens = static_cast<int32_t *>(std::malloc((pieces.size() + 1) * sizeof(int32_t)));
+        if (!lens) throw std::bad_alloc();
+        for (size_t i = 0; i < pieces.size(); i++) {
+            all += pieces[i];
+            lens[i] = static_cast<int32_t>(pieces[i].size());
+        }
+        *out = dup_bytes(all, out_len);
+        *piece_len = lens;
+        *n = static_cast<int>(pieces.size());
+    });
+}
+
+int shvtext_pyjson(const char *raw, char **out) {
+    return guard([&] {
+        if (!raw || !out) throw llm::text::Error("llm: NULL argument");
+        *out = dup_bytes(llm::text::PyJSON(raw), nullptr);
+    });
+}
+
+int shvtext_parse_tool_arguments(const char *s, char **out_json) {
+    return guard([&] {
+        if (!s || !out_json) throw llm::text::Error("llm: NULL argument");
+        std::string j = "[";
+        bool first = true;
+        for (const llm::text::ChatArg &a : llm::text::ParseToolArguments(s)) {
+            if (!first) j += ',';
+            first = false;
+            j += "{\"name\":" + llm::text::GoJSONString(a.Name) + ",\"value\":" + a.Value + "}";
+        }
+        j += ']';
+        *out_json = dup_bytes(j, nullptr);
+    });
+}
+
+int shvtext_render_chat(const char *request_json, char **out) {
+    return guard([&] {
+        using llm::text::JValue;
+        if (!request_json || !out) throw llm::text::Error("llm: NULL argument");
+        const JValue req = llm::text::ParseJSON(request_json);
+        const auto str = [](const JValue *v) { return v && v->kind == JValue::String ? v->str : std::string(); };
+        const auto flag = [](const JValue *v) { return v && v->kind == JValue::Bool && v->b; };
+        std::vector<llm::text::ChatMessage> msgs;
+        if (const JValue *ms = req.Get("messages"))
+            for (const JValue &m : ms->items) {
+                llm::text::ChatMessage msg;
+                msg.Role = str(m.Get("role"));
+                msg.Content = str(m.Get("content"));
+                msg.Reasoning = str(m.Get("reasoning"));
+                if (const JValue *parts = m.Get("parts"))
+                    if (parts->kind == JValue::Array) {
+                        msg.HasParts = true;
+                        for (const JValue &p : parts->items) msg.Parts.push_back({str(p.Get("text")), flag(p.Get("image"))});
+                    }
+                if (const JValue *calls = m.Get("tool_calls"))
+                    for (const JValue &c : calls->items) {
+                        llm::text::ChatToolCall call;
+                        call.Name = str(c.Get("name"));
+                        if (const JValue *args = c.Get("args"))
+                            for (const JValue &a : args->items) {
+                                const JValue *val = a.Get("value");
+                                call.Args.push_back({str(a.Get("name")), val ? val->raw : std::string()});
+                            }
+                        msg.ToolCalls.push_back(call);
+                    }
+                msgs.push_back(msg);
+            }
+        llm::text::ChatOpts opt;
+        if (const JValue *tools = req.Get("tools"))
+            for (const JValue &t : tools->items) opt.Tools.push_back(t.raw);
+        if (const JValue *o = req.Get("opts")) {
+            opt.Effort = str(o->Get("effort"));
+            opt.NoThinking = flag(o->Get("no_thinking"));
+            opt.DropThinking = flag(o->Get("drop_thinking"));
+            opt.NoGenerationPrompt = flag(o->Get("no_generation_prompt"));
+            opt.AddVisionID = flag(o->Get("add_vision_id"));
+        }
+        *out = dup_bytes(llm::text::RenderChat(msgs, opt), nullptr);
+    });
+}
+
+int shvtext_decoder_new(const char *tools_json, int thinking, shvtext_decoder **out) {
+    return guard([&] {
+        if (!out) throw llm::text::Error("llm: NULL argument");
+        *out = new shvtext_decoder{llm::text::ChatDecoder(tools_of(tools_json), thinking != 0), std::string()};
+    });
+}
+void shvtext_decoder_free(shvtext_decoder *d) { delete d; }
+int shvtext_decoder_stop_at(shvtext_decoder *d, const char *const *seqs, const uint64_t *lens, int n) {
+    return guard([&] {
+        if (!d || (n > 0 && (!seqs || !lens))) throw llm::text::Error("llm: NULL argument");
+        std::vector<std::string> v;
+        for (int i = 0; i < n; i++) v.emplace_back(seqs[i], static_cast<size_t>(lens[i]));
+        d->dec.StopAt(v);
+    });
+}
+const char *shvtext_decoder_stopped(shvtext_decoder *d, uint64_t *len) {
+    if (!d) return "";
+    d->stopped = d->dec.Stopped();
+    if (len) *len = d->stopped.size();
+    return d->stopped.c_str();
+}
+int shvtext_decoder_write(shvtext_decoder *d, const char *piece, uint64_t len, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len) {
+    return guard([&] {
+        if (!d || !reasoning || !content) throw llm::text::Error("llm: NULL argument");
+        std::string r, c;
+        d->dec.Write(bytes_of(piece, len), &r, &c);
+        *reasoning = dup_bytes(r, r_len);
+        *content = dup_bytes(c, c_len);
+    });
+}
+int shvtext_decoder_close(shvtext_decoder *d, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len, char **calls_json) {
+    return guard([&] {
+        if (!d || !reasoning || !content || !calls_json) throw llm::text::Error("llm: NULL argument");
+        std::string r, c;
+        std::vector<llm::text::ChatCall> calls;
+        d->dec.Close(&r, &c, &calls);
+        std::string j = "[";
+        for (size_t i = 0; i < calls.size(); i++) {
+            if (i) j += ',';
+            j += "{\"name\":" + llm::text::GoJSONString(calls[i].Name) + ",\"arguments\":" + llm::text::GoJSONString(calls[i].Arguments) + "}";
+        }
+        j += ']';
+        *reasoning = dup_bytes(r, r_len);
+        *content = dup_bytes(c, c_len);
+        *calls_json = dup_bytes(j, nullptr);
+    });
+}
+
+struct shvtext_stream {
+    llm::text::ChatStream st;
+    std::string stopped;
+};
+
+int shvtext_stream_new(shvtext_tokenizer *t, const int32_t *eog, int n_eog, const char *tools_json, int thinking, shvtext_stream **out) {
+    return guard([&] {
+        if (!t || !out || (n_eog > 0 && !eog)) throw llm::text::Error("llm: NULL argument");
+        *out = new shvtext_stream{llm::text::ChatStream(&t->tok, std::set<int32_t>(eog, eog + n_eog), tools_of(tools_json), thinking != 0), std::string()};
+    });
+}
+void shvtext_stream_free(shvtext_stream *s) { delete s; }
+int shvtext_stream_stop_at(shvtext_stream *s, const char *const *seqs, const uint64_t *lens, int n) {
+    return guard([&] {
+        if (!s || (n > 0 && (!seqs || !lens))) throw llm::text::Error("llm: NULL argument");
+        std::vector<std::string> v;
+        for (int i = 0; i < n; i++) v.emplace_back(seqs[i], static_cast<size_t>(lens[i]));
+        s->st.StopAt(v);
+    });
+}
+int shvtext_stream_push(shvtext_stream *s, int32_t id, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len, int *finish) {
+    return guard([&] {
+        if (!s || !reasoning || !content || !finish) throw llm::text::Error("llm: NULL argument");
+        std::string r, c;
+        *finish = static_cast<int>(s->st.Push(id, &r, &c));
+        *reasoning = dup_bytes(r, r_len);
+        *content = dup_bytes(c, c_len);
+    });
+}
+const char *shvtext_stream_stopped(shvtext_stream *s, uint64_t *len) {
+    if (!s) return "";
+    s->stopped = s->st.Stopped();
+    if (len) *len = s->stopped.size();
+    return s->stopped.c_str();
+}
+int shvtext_stream_close(shvtext_stream *s, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len, char **calls_json) {
+    return guard([&] {
+        if (!s || !reasoning || !content || !calls_json) throw llm::text::Error("llm: NULL argument");
+        std::string r, c;
+        std::vector<llm::text::ChatCall> calls;
+        s->st.Close(&r, &c, &calls);
+        std::string j = "[";
+        for (size_t i = 0; i < calls.size(); i++) {
+            if (i) j += ',';
+            j += "{\"name\":" + llm::text::GoJSONString(calls[i].Name) + ",\"arguments\":" + llm::text::GoJSONString(calls[i].Arguments) + "}";
+        }
+        j += ']';
+        *reasoning = dup_bytes(r, r_len);
+        *content = dup_bytes(c, c_len);
+        *calls_json = dup_bytes(j, nullptr);
+    });
 }
 
 }  // extern "C"

@@ -230,6 +230,56 @@ const char *shvgguf_type_name(uint32_t type);
 int shvgguf_type_block(uint32_t type, int32_t *elems, int32_t *nbytes);   /* 0 when unknown */
 int64_t shvgguf_size_of(uint32_t type, int64_t n);                        /* -1 with the error set */
 
+/* ---- the text on either side of the token loop (host/text.hpp).  Strings the library hands out are malloc'ed, NUL-
+ * terminated copies (with their length where they may hold NUL) and go back through shvtext_free. ---- */
+typedef struct shvtext_tokenizer shvtext_tokenizer;
+typedef struct shvtext_decoder shvtext_decoder;
+void shvtext_free(void *p);
+/* tokenizer.FromVocab (zimage/tokenizer/vocab.go:62): tokens by id over the byte-level alphabet, merges as "left right";
+ * types (llama_token_attr numbering, one an id) or NULL; specials: names to match whole besides the types'; pre: "qwen2",
+ * "" or "qwen35" */
+int shvtext_tokenizer_from_vocab(const char *const *tokens, const uint64_t *token_len, int n_tokens, const char *const *merges,
+                                 const uint64_t *merge_len, int n_merges, const int32_t *types, const char *const *specials,
+                                 int n_specials, const char *pre, shvtext_tokenizer **out);
+/* LoadTokenizer + EndOfGeneration (llm/tokenizer.go:22-68) from an open checkpoint's metadata: the stop set's ids go to
+ * eog (up to eog_max of them), their count to n_eog */
+int shvtext_tokenizer_from_gguf(shvgguf *g, shvtext_tokenizer **out, int32_t *eog, int eog_max, int *n_eog);
+void shvtext_tokenizer_free(shvtext_tokenizer *t);
+int shvtext_tokenizer_size(shvtext_tokenizer *t);
+int shvtext_tokenizer_id(shvtext_tokenizer *t, const char *token, int32_t *id);   /* 1 found, 0 not */
+int shvtext_encode(shvtext_tokenizer *t, const char *text, uint64_t len, int32_t **ids, int *n);
+int shvtext_decode(shvtext_tokenizer *t, const int32_t *ids, int n, char **out, uint64_t *len);
+/* the pre-tokenizer's pieces (zimage/tokenizer/split.go): concatenated in out, their byte lengths in piece_len */
+int shvtext_split(const char *text, uint64_t len, int marks, char **out, uint64_t *out_len, int32_t **piece_len, int *n);
+/* pyJSON (llm/pyjson.go:31): Python's json.dumps(x, ensure_ascii=False) of one JSON value */
+int shvtext_pyjson(const char *raw, char **out);
+/* ParseToolArguments (llm/chat.go:399): [{"name": ..., "value": <the JSON as it arrived>}, ...] in the object's order */
+int shvtext_parse_tool_arguments(const char *s, char **out_json);
+/* RenderChat (llm/chat.go:195).  request_json: {"messages": [{"role", "content" | "parts": [{"text"} | {"image": true}],
+ * "reasoning", "tool_calls": [{"name", "args": [{"name", "value"}]}]}], "tools": [...], "opts": {"effort", "no_thinking",
+ * "drop_thinking", "no_generation_prompt", "add_vision_id"}} -- the shape of the reference's own test cases */
+int shvtext_render_chat(const char *request_json, char **out);
+/* ChatDecoder (llm/chatdecode.go): tools_json is the request's tools array or NULL; thinking: the generation prompt left
+ * <think> open */
+int shvtext_decoder_new(const char *tools_json, int thinking, shvtext_decoder **out);
+void shvtext_decoder_free(shvtext_decoder *d);
+int shvtext_decoder_stop_at(shvtext_decoder *d, const char *const *seqs, const uint64_t *lens, int n);
+const char *shvtext_decoder_stopped(shvtext_decoder *d, uint64_t *len);   /* valid until the next call on d */
+int shvtext_decoder_write(shvtext_decoder *d, const char *piece, uint64_t len, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len);
+/* calls_json: [{"name": ..., "arguments": "<a JSON object as a string>"}, ...] */
+int shvtext_decoder_close(shvtext_decoder *d, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len, char **calls_json);
+
+/* The text side of the emit loop (backend/llm.go:561-590): a sampled id becomes its bytes, whole characters (a
+ * character's bytes come in several tokens routinely) go to the completion reader, and what that releases is the token's
+ * delta.  finish: 0 running, 1 an end-of-generation id, 2 a stop sequence.  The tokenizer must outlive the stream. */
+typedef struct shvtext_stream shvtext_stream;
+int shvtext_stream_new(shvtext_tokenizer *t, const int32_t *eog, int n_eog, const char *tools_json, int thinking, shvtext_stream **out);
+void shvtext_stream_free(shvtext_stream *s);
+int shvtext_stream_stop_at(shvtext_stream *s, const char *const *seqs, const uint64_t *lens, int n);
+int shvtext_stream_push(shvtext_stream *s, int32_t id, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len, int *finish);
+const char *shvtext_stream_stopped(shvtext_stream *s, uint64_t *len);
+int shvtext_stream_close(shvtext_stream *s, char **reasoning, uint64_t *r_len, char **content, uint64_t *c_len, char **calls_json);
+
 #ifdef __cplusplus
 }
 #endif
