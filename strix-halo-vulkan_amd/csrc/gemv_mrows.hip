@@ -5,10 +5,10 @@
 // row.  Here a weight is turned into a binary16 operand once (~2 operations) and the matrix cores
 // multiply it with every row at no further vector cost:
 //   v_mfma_f32_16x16x32_f16   A = 16 weight rows x 32 columns, B = 32 columns x 16, of which
-//                             column 2t holds the high half of row t's activations and 2t+1 the
-//                             remainder times 2048 (hi + lo / 2048 = x to ~2^-22), so
-//                             y[t] = C[.][2t] + C[.][2t+1] / 2048; a wave first scales its part of a
-//                             row by a power of two so that the halves are normal numbers
+//                             column 2t holds the high part of row t's activations (cut to eleven
+//                             bits) and 2t+1 the remainder, so y[t] = C[.][2t] + C[.][2t+1]; a wave
+//                             first scales its part of a row by a power of two that brings the
+//                             largest magnitude to [512, 1024), so that the parts are normal numbers
 //   a weight as an operand    n * sc, a whole number below 946 and exact in binary16: the nibble is
 //                             masked into the mantissa of 1024.0 (low nibbles) or 64.0 (high
 //                             nibbles) and one packed fma takes off 1024 * sc or 64 * sc again;
@@ -34,12 +34,15 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 
-// x -> (hi, lo) halves, hi + lo / 2048 = x to about 2^-22 (the remainder scaled up so that it is a normal
-// number wherever hi is one well inside the range)
-__device__ __forceinline__ void split_half(float x, _Float16 &h, _Float16 &l) {
-    h = static_cast<_Float16>(x);
-    l = static_cast<_Float16>((x - static_cast<float>(h)) * 2048.f);
+// x -> a high part that binary16 holds exactly (x cut to eleven significant bits: one mask) and the exact remainder.
+// For the rows this kernel stages, scaled so that their largest magnitude is in [512, 1024), a remainder too small
+// for a normal binary16 belongs to an entry below 0.125, and what is lost of it is below 2^-33 of the largest.
+__device__ __forceinline__ void split_cut(float x, float &hi, float &lo) {
+    hi = __uint_as_float(__float_as_uint(x) & 0xFFFFE000u);
+    lo = x - hi;
 }
+// two floats to one dword of two halves, rounded toward zero (exact for split_cut's high parts)
+__device__ __forceinline__ uint32_t pack_halves(float a, float b) { return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b)); }
 
 // the largest of a wave's values, none of them negative, in every lane
 __device__ __forceinline__ float wave_max_nonneg(float v) {
@@ -50,11 +53,6 @@ __device__ __forceinline__ float wave_max_nonneg(float v) {
     v = fmaxf(v, dpp_f32<kDppBcast15, 0xA>(v));  // rows the mask leaves out read 0
     v = fmaxf(v, dpp_f32<kDppBcast31, 0xC>(v));
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
-}
-
-// the order in which a payload dword's nibbles come out of the masks below: bytes 0, 2, 1, 3
-__device__ __forceinline__ constexpr int frag_pos(int byte_in_8) {
-    return (byte_in_8 & 4) | ((byte_in_8 & 1) << 1) | ((byte_in_8 >> 1) & 1);
 }
 
 // Eight weights of two payload dwords (bytes 0..7 of the lane's 16 or bytes 8..15) as n * sc:
@@ -213,16 +211,17 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
         unscale[t] = __uint_as_float(static_cast<uint32_t>(ex - 9) << 23);          // its inverse (0 below 2^-118)
 #pragma unroll
         for (int u = 0; u < FPL; u++) {
-            half8_t hi, lo;
-            float s8 = 0.f;
+            float h8[8], l8[8], s8 = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                _Float16 h, l;
-                split_half(v[u][i] * up, h, l);
-                hi[frag_pos(i)] = h;
-                lo[frag_pos(i)] = l;
-                s8 += v[u][i] * up;
+                const float vs = v[u][i] * up;
+                split_cut(vs, h8[i], l8[i]);
+                s8 += vs;
             }
+            // operand order within a fragment: the order a payload dword's nibbles come out of the masks (bytes 0, 2, 1, 3)
+            const uint4 hw = make_uint4(pack_halves(h8[0], h8[2]), pack_halves(h8[1], h8[3]), pack_halves(h8[4], h8[6]), pack_halves(h8[5], h8[7]));
+            const uint4 lw = make_uint4(pack_halves(l8[0], l8[2]), pack_halves(l8[1], l8[3]), pack_halves(l8[4], l8[6]), pack_halves(l8[5], l8[7]));
+            const half8_t hi = __builtin_bit_cast(half8_t, hw), lo = __builtin_bit_cast(half8_t, lw);
             const int f = lane + 64 * u;
             bf[f * FS + 2 * t] = hi;
             bf[f * FS + 2 * t + 1] = lo;
@@ -232,16 +231,13 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
             if ((f & 5) == 0) {
                 const int jj = f & 3, m = (f >> 2) & 3, L = (f >> 4) & 1, s = f >> 5;
                 const int grp = 2 * L + (jj >> 1), odd = m >> 1;  // sub-block 2 grp + odd of the super-block
-                _Float16 h, l;
-                split_half(s32, h, l);
+                float sh, sl;
+                split_cut(s32, sh, sl);
                 // operand (column group grp, column 2t / 2t+1), halves (sub 2 grp, 0, sub 2 grp + 1, 0)
-                half2_t *dst_hi = reinterpret_cast<half2_t *>(&sf[(s * 4 + grp) * NC + 2 * t]) + odd;
-                half2_t *dst_lo = reinterpret_cast<half2_t *>(&sf[(s * 4 + grp) * NC + 2 * t + 1]) + odd;
-                half2_t hh, ll;
-                hh[0] = h; hh[1] = static_cast<_Float16>(0.f);
-                ll[0] = l; ll[1] = static_cast<_Float16>(0.f);
-                *dst_hi = hh;
-                *dst_lo = ll;
+                uint32_t *dst_hi = reinterpret_cast<uint32_t *>(&sf[(s * 4 + grp) * NC + 2 * t]) + odd;
+                uint32_t *dst_lo = reinterpret_cast<uint32_t *>(&sf[(s * 4 + grp) * NC + 2 * t + 1]) + odd;
+                *dst_hi = pack_halves(sh, 0.f);
+                *dst_lo = pack_halves(sl, 0.f);
             }
         }
         if constexpr (PRO == SHV_PRO_RMSNORM) {
@@ -253,11 +249,10 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
 
     // ---- products ----
     const int bc = r < NC ? r : NC - 1;  // columns past the rows' hold whatever: their results are never read
-    // a lane's column: activation row r / 2, the high (even column) or the low halves' products
+    // a lane's column: activation row r / 2 (its high parts in the even column, the remainders in the odd one)
     float back = 0.f;
 #pragma unroll
     for (int t = 0; t < NT; t++) back = (r >> 1) == t ? unscale[t] : back;
-    back *= (r & 1) ? 1.f / 2048.f : 1.f;
 #pragma unroll
     for (int ti = 0; ti < TILES; ti++) {
     float4_t yacc = {0.f, 0.f, 0.f, 0.f};
