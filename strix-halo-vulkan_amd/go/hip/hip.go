@@ -265,6 +265,129 @@ func MoEDown(act, topk, weights *Buffer, b MoEBanks, residual, out *Buffer, rows
 	return mk(C.SHV_OP_MOE_DOWN, unsafe.Pointer(&a), C.sizeof_shv_moe_down_args)
 }
 
+// PassRows says which rows a pass carries (llm::PassRows in host/llm.hpp; the reference's rowSet,
+// llm/graph.go:1383-1429): NSeq sequences of SeqLen consecutive rows, their positions and slots in
+// device memory, and whether the pass is rewindable.
+type PassRows struct {
+	NSeq, SeqLen int
+	Pos, Slot    *Buffer // device int32 per sequence; Slot nil: sequence s is slot s
+	Spec         bool
+}
+
+// DNStepArgs are the fields of shv_dn_step_args a caller sets (llm_dn_conv.comp + llm_dn_scan.comp).
+type DNStepArgs struct {
+	Ring, Conv1D, A, DtBias, State, Out *Buffer
+	Rows                                PassRows
+	HeadK, HeadV, HeadDim, Conv         int
+	RingSlots, RingStride               int
+	Eps                                 float32
+	Plane                               *Buffer // device int32 per slot: the committed state plane
+	Planes                              int
+	Work                                *Buffer // scratch of the chunked form; nil keeps every pass row by row
+}
+
+// DNStep is the gated delta rule over the ring rows of a pass.
+func DNStep(d DNStepArgs) Op {
+	var a C.shv_dn_step_args
+	a.ring, a.conv1d, a.a, a.dt_bias = fp(d.Ring), fp(d.Conv1D), fp(d.A), fp(d.DtBias)
+	a.state, a.out = fp(d.State), fp(d.Out)
+	a.pos, a.slot = ip(d.Rows.Pos), ip(d.Rows.Slot)
+	a.n_seq, a.seq_len = C.int32_t(d.Rows.NSeq), C.int32_t(d.Rows.SeqLen)
+	a.n_head_k, a.n_head_v, a.head_dim, a.conv = C.int32_t(d.HeadK), C.int32_t(d.HeadV), C.int32_t(d.HeadDim), C.int32_t(d.Conv)
+	a.ring_slots, a.ring_stride, a.eps = C.int32_t(d.RingSlots), C.int32_t(d.RingStride), C.float(d.Eps)
+	a.plane, a.n_planes = ip(d.Plane), C.int32_t(d.Planes)
+	if d.Rows.Spec {
+		a.spec = 1
+	}
+	if d.Work != nil {
+		a.work, a.work_floats = fp(d.Work), C.int64_t(d.Work.size/4)
+	}
+	return mk(C.SHV_OP_DN_STEP, unsafe.Pointer(&a), C.sizeof_shv_dn_step_args)
+}
+
+// AttnArgs are the fields of shv_attn_decode_args a caller sets (llm_attn_pack.comp,
+// llm_attn_wmma.comp -DSPLITK, llm_attn_combine.comp in one op).
+type AttnArgs struct {
+	QKV, QNorm, KNorm, Rope      *Buffer
+	KCache, VCache, Partial, Out *Buffer
+	Rows                         PassRows
+	NHead, NHeadKV, HeadDim      int
+	RopeDims, MaxCells           int
+	QKVStride, Splits            int
+	Eps                          float32
+	Mask                         *Buffer // the block-sparse indexer's selection (QSAIndex), or nil
+	MaskStride                   int
+}
+
+// AttnDecode appends the rows' cells and attends over each sequence's cache.
+func AttnDecode(d AttnArgs) Op {
+	var a C.shv_attn_decode_args
+	a.qkv, a.q_norm, a.k_norm, a.rope = fp(d.QKV), fp(d.QNorm), fp(d.KNorm), fp(d.Rope)
+	a.kcache, a.vcache, a.partial, a.out = vp(d.KCache), vp(d.VCache), fp(d.Partial), fp(d.Out)
+	a.pos, a.slot = ip(d.Rows.Pos), ip(d.Rows.Slot)
+	a.n_seq, a.seq_len = C.int32_t(d.Rows.NSeq), C.int32_t(d.Rows.SeqLen)
+	a.n_head, a.n_head_kv, a.head_dim = C.int32_t(d.NHead), C.int32_t(d.NHeadKV), C.int32_t(d.HeadDim)
+	a.rope_dims, a.max_cells = C.int32_t(d.RopeDims), C.int32_t(d.MaxCells)
+	a.qkv_stride, a.n_splits, a.eps = C.int32_t(d.QKVStride), C.int32_t(d.Splits), C.float(d.Eps)
+	if d.Mask != nil {
+		a.mask = (*C.uint32_t)(d.Mask.ptr)
+		a.mask_stride = C.int32_t(d.MaskStride)
+	}
+	return mk(C.SHV_OP_ATTN_DECODE, unsafe.Pointer(&a), C.sizeof_shv_attn_decode_args)
+}
+
+// QSAArgs are the fields of shv_qsa_index_args (indexerAt / selected / topK, llm/attn.go:247-443).
+type QSAArgs struct {
+	X, Gamma, W, QNorm, KNorm, Rope *Buffer
+	IdxCache, Pooled                *Buffer
+	Rows                            PassRows
+	Work, Score, Mask               *Buffer
+	NEmbd, IdxHeads, IdxDim         int
+	TopK, Ratio, RopeDims, MaxCells int
+	MaskStride                      int
+	Eps                             float32
+}
+
+// QSAIndex makes the per-row selection mask of an attention layer with a compression ratio.
+func QSAIndex(d QSAArgs) Op {
+	var a C.shv_qsa_index_args
+	a.x, a.gamma, a.w, a.q_norm, a.k_norm, a.rope = fp(d.X), fp(d.Gamma), fp(d.W), fp(d.QNorm), fp(d.KNorm), fp(d.Rope)
+	a.idxcache, a.pooled = vp(d.IdxCache), fp(d.Pooled)
+	a.pos, a.slot = ip(d.Rows.Pos), ip(d.Rows.Slot)
+	a.work, a.score, a.mask = fp(d.Work), fp(d.Score), (*C.uint32_t)(vp(d.Mask))
+	a.n_seq, a.seq_len, a.n_embd = C.int32_t(d.Rows.NSeq), C.int32_t(d.Rows.SeqLen), C.int32_t(d.NEmbd)
+	a.idx_heads, a.idx_dim, a.top_k, a.ratio = C.int32_t(d.IdxHeads), C.int32_t(d.IdxDim), C.int32_t(d.TopK), C.int32_t(d.Ratio)
+	a.rope_dims, a.max_cells, a.mask_stride, a.eps = C.int32_t(d.RopeDims), C.int32_t(d.MaxCells), C.int32_t(d.MaskStride), C.float(d.Eps)
+	return mk(C.SHV_OP_QSA_INDEX, unsafe.Pointer(&a), C.sizeof_shv_qsa_index_args)
+}
+
+// RingRows copies count rows of n floats between two rings of projection rows addressed by the sequence's
+// position (a long pass's ring and the sequence's own small one).
+func RingRows(src, dst, pos *Buffer, srcSlots, dstSlots, stride, n, first, count int) Op {
+	var a C.shv_ring_rows_args
+	a.src, a.dst, a.pos = fp(src), fp(dst), ip(pos)
+	a.src_slots, a.dst_slots, a.stride, a.n = C.int32_t(srcSlots), C.int32_t(dstSlots), C.int32_t(stride), C.int32_t(n)
+	a.first, a.count = C.int32_t(first), C.int32_t(count)
+	return mk(C.SHV_OP_RING_ROWS, unsafe.Pointer(&a), C.sizeof_shv_ring_rows_args)
+}
+
+// Embed gathers rows of the embedding table (Model.Embedding + HCGPU.UploadInit): ids[pos[0]..] when pos is given.
+func Embed(table, ids, pos, x *Buffer, rows, nEmbd, vocab, typ int) Op {
+	var a C.shv_embed_args
+	a.table, a.ids, a.pos, a.x = vp(table), ip(ids), ip(pos), fp(x)
+	a.n_tok, a.n_embd, a.vocab, a.x_stride, a._type = C.int32_t(rows), C.int32_t(nEmbd), C.int32_t(vocab), C.int32_t(nEmbd), C.int32_t(typ)
+	return mk(C.SHV_OP_EMBED, unsafe.Pointer(&a), C.sizeof_shv_embed_args)
+}
+
+// Argmax is Argmax (llm/sample.go:359-367) over rows of logits; with ids and pos, one row's result is stored
+// as the sequence's next token and its position advanced.
+func Argmax(logits, best, ids, pos *Buffer, rows, n, stride, advance int) Op {
+	var a C.shv_argmax_args
+	a.logits, a.best, a.ids, a.pos = fp(logits), ip(best), ip(ids), ip(pos)
+	a.n_rows, a.n, a.logits_stride, a.advance = C.int32_t(rows), C.int32_t(n), C.int32_t(stride), C.int32_t(advance)
+	return mk(C.SHV_OP_ARGMAX, unsafe.Pointer(&a), C.sizeof_shv_argmax_args)
+}
+
 // Raw wraps an argument block the caller filled itself (shv_dn_step_args, shv_attn_decode_args,
 // shv_embed_args, shv_argmax_args, shv_advance_args, shv_ring_rows_args): llm/gpu_deltanet.go and
 // llm/gpu_attn.go build theirs field by field exactly as the functions above do.
