@@ -192,10 +192,13 @@ typedef struct {
     int32_t type;
 } shv_dequant_args;
 
-/* y[r] = sum_i W[r][i] * x[i] (+ residual[r]) for W [n][k] row-major in any of those types: the
- * CPU path's matvec over Tensor.DequantizeRow (llm/hc.go:255-264, gguf/dequant.go:119-124) for the
- * tensors of a checkpoint that are not Q4_K.  One row of activations, no prologue; Q4_K weights
- * on the token path go through shv_gemv_q4k. */
+/* y[t][r] = sum_i W[r][i] * pro(x[t])[i] (+ residual[t][r]) for W [n][k] row-major in any of those
+ * types: the CPU path's matvec over Tensor.DequantizeRow (llm/hc.go:255-264, gguf/dequant.go:119-124)
+ * for the tensors of a checkpoint that are not Q4_K.  gamma non-NULL: pro is the RMSNorm
+ * x * rsqrt(mean(x^2) + eps) * gamma (llm/hc.go:176-190), which is how a vocabulary projection kept in
+ * the checkpoint's own type (a Q6_K head) takes its rows; NULL: pro(x) = x.  n_tok 0 means one row;
+ * rows are x_stride and y_stride floats apart (0: k and n); the weights are read once for every four
+ * rows.  Q4_K weights on the token path go through shv_gemv_q4k. */
 typedef struct {
     const void *w;
     const float *x;
@@ -203,6 +206,10 @@ typedef struct {
     const float *residual;
     int32_t n, k;
     int32_t type;
+    int32_t n_tok;
+    const float *gamma;
+    float eps;
+    int32_t x_stride, y_stride;
 } shv_gemv_args;
 
 /* dst[i] = d*sc*q - dmin*m for every weight of `rows` rows, the reference's dequantQ4_K

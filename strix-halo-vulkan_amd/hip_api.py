@@ -58,7 +58,8 @@ class DequantArgs(C.Structure):
 
 class GemvArgs(C.Structure):
     _fields_ = [("w", C.c_void_p), ("x", C.c_void_p), ("y", C.c_void_p), ("residual", C.c_void_p),
-                ("n", C.c_int32), ("k", C.c_int32), ("type", C.c_int32)]
+                ("n", C.c_int32), ("k", C.c_int32), ("type", C.c_int32), ("n_tok", C.c_int32), ("gamma", C.c_void_p),
+                ("eps", C.c_float), ("x_stride", C.c_int32), ("y_stride", C.c_int32)]
 
 
 class QuantizeQ4KArgs(C.Structure):
@@ -353,9 +354,9 @@ class Context:
         a = DequantArgs(_ptr(src), _ptr(dst), n, typ)
         check(self.L.shv_dequant(self.h, C.byref(a)))
 
-    def gemv(self, typ, w, x, y, n, k, residual=None):
-        """y = W x (+ residual) for W [n][k] of ggml tensor type `typ`."""
-        a = GemvArgs(_ptr(w), _ptr(x), _ptr(y), _ptr(residual), n, k, typ)
+    def gemv(self, typ, w, x, y, n, k, residual=None, n_tok=0, gamma=None, eps=0.0, x_stride=0, y_stride=0):
+        """y[t] = W pro(x[t]) (+ residual[t]) for W [n][k] of ggml tensor type `typ`; gamma: the RMSNorm prologue."""
+        a = GemvArgs(_ptr(w), _ptr(x), _ptr(y), _ptr(residual), n, k, typ, n_tok, _ptr(gamma), eps, x_stride, y_stride)
         check(self.L.shv_gemv(self.h, C.byref(a)))
 
     def gemv_q4k(self, w, x, y, n, k, n_tok=1, prologue=PRO_NONE, gamma=None, z=None, residual=None,

@@ -368,6 +368,18 @@ void Model::LoadGGUF(const gguf::Set &s, const LoadOpts &opts) {
             v.kind = TensorView::RAW;
             v.ggml = t.Type;
             dev_.upload(v.ptr, t.Data, t.Bytes);
+        } else if (name == "output.weight" && v.kind != TensorView::F32 && t.Type != gguf::Q4_K && opts.head_native && device_expands(t.Type)) {
+            // the vocabulary projection in the checkpoint's own type (converters keep it wider than the rest: Q6_K,
+            // Q8_0): the head's launch reads it through that type's arm (shv_gemv) instead of a Q4_K refit of it
+            if (t.RowBytes() == 0) throw Error("llm: " + name + " is " + shape + ": rows are not whole blocks of the type");
+            if (v.bytes != t.Bytes) {
+                dev_.release(v.ptr, v.bytes);
+                v.ptr = dev_.alloc(t.Bytes);
+                v.bytes = t.Bytes;
+            }
+            v.kind = TensorView::RAW;
+            v.ggml = t.Type;
+            dev_.upload(v.ptr, t.Data, t.Bytes);
         } else if (t.Type == same) {
             if (t.Bytes != v.bytes) throw Error("llm: " + name + ": " + std::to_string(t.Bytes) + " bytes in the checkpoint, " + std::to_string(v.bytes) + " staged");
             dev_.upload(v.ptr, t.Data, t.Bytes);
@@ -1165,6 +1177,24 @@ std::vector<shv_op> HeadGPU::Dispatches(const float *in, int rows, std::vector<s
 std::vector<shv_op> HeadGPU::DispatchesTo(const float *in, int rows, const float *gamma, float *logits, int cols,
                                           std::vector<std::string> *labels) const {
     if (rows < 1 || cols < 1 || cols > c_.VocabSize) throw Error("llm: HeadGPU: " + std::to_string(rows) + " rows over " + std::to_string(cols) + " columns");
+    const TensorView &w = m_.Tensor("output.weight");
+    if (w.kind == TensorView::RAW) {
+        // a head kept in the checkpoint's own type: matvec over rows expanded as Tensor.DequantizeRow expands them
+        shv_gemv_args g{};
+        g.w = w.ptr;
+        g.x = in;
+        g.y = logits;
+        g.n = cols;
+        g.k = c_.NEmbd;
+        g.type = static_cast<int32_t>(w.ggml);
+        g.n_tok = rows;
+        g.gamma = gamma;
+        g.eps = c_.RMSEps;
+        g.x_stride = c_.NEmbd;
+        g.y_stride = c_.VocabSize;
+        if (labels) labels->push_back("head");
+        return {make_op(SHV_OP_GEMV, g)};
+    }
     shv_gemv_q4k_args p{};
     p.w = m_.Tensor("output.weight").ptr;
     p.x = in;

@@ -146,6 +146,7 @@ public:
     struct LoadOpts {
         bool transcode = true;
         std::string moe_plan;
+        bool head_native = true;  // output.weight stays in the checkpoint's own type (LLM_HEAD_TYPE=q4_k refits it like the rest)
     };
     void LoadGGUF(const gguf::Set &s, const LoadOpts &o);
     void LoadGGUF(const gguf::Set &s, bool transcode = true) {

@@ -126,6 +126,10 @@ int shvllm_open_gguf(int device, const char *path, const shvllm_config *c, shvll
         const char *tc = std::getenv("LLM_TRANSCODE");  // 0: refuse a matrix that is not Q4_K instead of fitting it again
         llm::Model::LoadOpts lo;
         lo.transcode = !(tc && tc[0] == '0');
+        if (const char *ht = std::getenv("LLM_HEAD_TYPE")) {  // q4_k: the vocabulary projection refitted like every other dense matrix
+            if (std::strcmp(ht, "q4_k") == 0) lo.head_native = false;
+            else if (std::strcmp(ht, "own") != 0) throw llm::Error(std::string("llm: LLM_HEAD_TYPE=") + ht + "; own (the checkpoint's type, the default) or q4_k");
+        }
         if (const char *plan = std::getenv("LLM_MOE_BANK")) lo.moe_plan = plan;  // family=q4_k,...: expert banks refitted instead of read natively
         if (const char *mode = std::getenv("LLM_MOE_BANK_QUANT"))
             if (std::strcmp(mode, "rtn") != 0) throw llm::Error(std::string("llm: LLM_MOE_BANK_QUANT=") + mode + "; banks are refitted round-to-nearest here (rtn), no importance matrix is read");

@@ -110,3 +110,29 @@ def test_refusals(ctx):
         ctx.gemv(14, src, src, dst, 1, 128)   # Q6_K rows are whole super-blocks
     with pytest.raises(shv.api.ShvError):
         ctx.gemv(8, src, src, dst, 1, 32768)  # x would not fit its staging
+
+
+@pytest.mark.parametrize("name", ["Q6_K", "Q8_0", "F16", "Q5_K"])
+@pytest.mark.parametrize("rows", [1, 3, 6])
+def test_gemv_rows_with_the_rmsnorm_prologue(ctx, name, rows):
+    """The any-type GEMV as a vocabulary projection takes it: rows of a pass, the final RMSNorm as its prologue
+    (llm/hc.go:176-190), strides wider than the rows, a residual in place; the weights read once per four rows."""
+    typ, n, k, eps = O.GGML_TYPES[name], 200, 2048, 1e-6
+    rng = np.random.default_rng(typ + rows)
+    raw = random_tensor(name, n * k, seed=typ + 31)
+    w = O.dequant(typ, raw, n * k).reshape(n, k).astype(np.float64)
+    xs, ys = k + 64, n + 8
+    x = np.zeros((rows, xs), np.float32)
+    x[:, :k] = rng.standard_normal((rows, k)) * 3
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    res = np.zeros((rows, ys), np.float32)
+    res[:, :n] = rng.standard_normal((rows, n))
+    dy = ctx.upload(res)
+    ctx.gemv(typ, ctx.upload(raw), ctx.upload(x), dy, n, k, residual=dy, n_tok=rows, gamma=ctx.upload(gamma), eps=eps, x_stride=xs, y_stride=ys)
+    got = dy.read(np.float32, rows * ys).reshape(rows, ys)
+    x64 = x[:, :k].astype(np.float64)
+    xn = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + eps) * gamma
+    want = xn @ w.T + res[:, :n]
+    for t in range(rows):
+        assert O.rel_l2(got[t, :n], want[t]) <= 1e-5, t
+    assert np.all(got[:, n:] == 0)     # nothing written past a row's n outputs

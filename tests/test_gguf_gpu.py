@@ -222,11 +222,11 @@ def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, 
         monkeypatch.setenv("LLM_MOE_BANK", plan)
     # a family's ceiling leaves a bank no wider than Q4_K alone: IQ4_NL stays whatever the plan says
     refit_banks = {"blk.0.ffn_down_exps.weight", "blk.1.ffn_gate_exps.weight", "blk.1.ffn_up_shexp.weight"} if plan else set()
-    native = {n for n in recipe if any(w in n for w in BANK_WORDS)} - refit_banks
+    native = ({n for n in recipe if any(w in n for w in BANK_WORDS)} - refit_banks) | {"output.weight"}   # the head keeps its type too
     r = LA.LLM(small_cfg(), gguf=_rewrite(p, tmp_path / "recipe.gguf", tensors=swap))
     try:
         assert sorted(r.transcoded()) == sorted(n for n in recipe if n != "token_embd.weight" and n not in native)
-        assert r.tensor_type("token_embd.weight") == 8 and r.tensor_type("output.weight") == 12
+        assert r.tensor_type("token_embd.weight") == 8 and r.tensor_type("output.weight") == 14
         for name in recipe:
             if name == "token_embd.weight" or name in native:
                 assert r.tensor_type(name) == swap[name][0], name
@@ -240,7 +240,6 @@ def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, 
         # saved again, the file names the types now in memory and holds the same bytes
         r.save_gguf(tmp_path / "again.gguf")
         again = GF.parse(tmp_path / "again.gguf")
-        assert again["tensors"]["output.weight"][0] == 12
         for name in native | {"token_embd.weight"}:
             assert again["tensors"][name][0] == swap[name][0] and again["tensors"][name][2] == swap[name][2], name
         # the token loop against the CPU loop over the weights as staged
@@ -249,11 +248,17 @@ def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, 
         table = f32["token_embd.weight"].astype(np.float16)
         assert np.array_equal(table.astype(np.float32), f32["token_embd.weight"])
         tensors["token_embd.weight"] = table.view(np.uint16)
-        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv, bank_types={n: swap[n][0] for n in native})
+        # the CPU model walks its layers with any Q4_K head (its logits are not used): the head in the checkpoint's type
+        # is matvec over the CPU's dequantised rows of it (llm/hc.go:255-264), applied to the CPU's own residual stream
+        head = f32["output.weight"].reshape(cfg.vocab, cfg.n_embd)
+        tensors["output.weight"] = O.quantize_q4k(head)
+        om = O.OracleModel(cfg, tensors, max_cells=cfg.nkv, bank_types={n: swap[n][0] for n in native if n != "output.weight"})
         prompt = np.random.default_rng(5).integers(0, cfg.vocab, size=7).astype(np.int32)
         r.reset()
         lg_gpu, hd_gpu = r.extend(prompt, want_hidden=True)
-        lg_cpu, hd_cpu = om.extend(prompt)
+        _, hd_cpu = om.extend(prompt)
+        xn = O.rmsnorm(hd_cpu.reshape(1, -1), tensors["output_norm.weight"], cfg.rms_eps)[0]
+        lg_cpu = (head.astype(np.float64) @ xn.astype(np.float64)).astype(np.float32)
         assert O.rel_l2(hd_gpu, hd_cpu) <= 1e-3 and O.rel_l2(lg_gpu, lg_cpu) <= 1e-3
         tok = int(O.lib().shv_ref_argmax(O.F(lg_cpu), cfg.vocab))
         ids, _ = r.generate(1)
@@ -261,6 +266,47 @@ def test_checkpoint_of_mixed_types_is_staged_and_decodes_as_the_cpu_does(saved, 
         assert ids[0] == tok or top2[1] - top2[0] < 1e-4
     finally:
         r.close()
+
+
+def test_the_head_in_its_own_type_or_refitted(saved, tmp_path, monkeypatch):
+    """A checkpoint's vocabulary projection in Q8_0 stays Q8_0 in HBM and the head's launch reads it through that type's
+    arm, for one row and for the rows of a pass; LLM_HEAD_TYPE=q4_k refits it like any other dense matrix (and says so)."""
+    m, cfg, path = saved
+    p = GF.parse(path)
+    _, dims, _ = p["tensors"]["output.weight"]
+    raw = random_tensor("Q8_0", int(np.prod(dims)), seed=77, scale=2e-4)
+    head = O.dequant(O.GGML_TYPES["Q8_0"], raw, int(np.prod(dims))).reshape(cfg.vocab, cfg.n_embd)
+    out = _rewrite(p, tmp_path / "head.gguf", tensors={"output.weight": (O.GGML_TYPES["Q8_0"], dims, raw.tobytes())})
+    r = LA.LLM(small_cfg(head_rows=5), gguf=out)
+    try:
+        assert r.tensor_type("output.weight") == 8 and "output.weight" not in r.transcoded()
+        assert np.array_equal(r.download("output.weight"), raw)
+        r.stage()
+        gamma = r.download("output_norm.weight")
+        rows = np.random.default_rng(9).integers(0, cfg.vocab, size=5).astype(np.int32)
+        _, lg_rows, res = r.extend_rows(rows, want_logits=True, want_res=True)
+        for t in range(5):
+            xn = O.rmsnorm(res[t:t + 1], gamma, cfg.rms_eps)[0]
+            assert O.rel_l2(lg_rows[t], head.astype(np.float64) @ xn.astype(np.float64)) <= 1e-4, t
+        # the recorded one-row step: logits of its row, and the token it names is their first maximum
+        lg, hd = r.extend(rows[:1], want_hidden=True)
+        want = head.astype(np.float64) @ O.rmsnorm(hd.reshape(1, -1), gamma, cfg.rms_eps)[0].astype(np.float64)
+        assert O.rel_l2(lg, want) <= 1e-4
+        ids, _ = r.generate(1)
+        top2 = np.sort(lg)[-2:]
+        assert ids[0] == int(np.argmax(lg)) or top2[1] - top2[0] < 1e-5
+    finally:
+        r.close()
+    monkeypatch.setenv("LLM_HEAD_TYPE", "q4_k")
+    r = LA.LLM(small_cfg(), gguf=out)
+    try:
+        assert r.tensor_type("output.weight") == 12 and "output.weight" in r.transcoded()
+        assert np.array_equal(r.download("output.weight").view(np.uint8), O.quantize_q4k(head).reshape(-1))
+    finally:
+        r.close()
+    monkeypatch.setenv("LLM_HEAD_TYPE", "q6_k")
+    with pytest.raises(ShvError, match="LLM_HEAD_TYPE"):
+        LA.LLM(small_cfg(), gguf=out)
 
 
 def test_a_bank_plan_is_held_to_the_grammar(saved, monkeypatch):
