@@ -188,7 +188,6 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
     cps = (cps + kTile - 1) & ~(kTile - 1);  // slices start on a tile of V
     const int c0 = split * cps;
     const int c1 = c0 + cps < n_cells ? c0 + cps : n_cells;
-    const int nc = c1 > c0 ? c1 - c0 : 0;
 
     const int kvw = a.n_head_kv * kD;
     // K is [cell][kv head][dim]; V is kept transposed in tiles of 32 cells,

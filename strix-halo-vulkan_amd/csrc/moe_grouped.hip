@@ -707,7 +707,7 @@ __global__ __launch_bounds__(kStThreads, 2) void moe_up_grouped_kernel(shv_moe_u
     int32_t *tok_s = pair_s + kTok;
     const int32_t *group = a.group;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n = lane & 15, kb = lane >> 4;
+    const int n = lane & 15;
     const int parts = a.ffn / (32 * kStWaves);
     const Unit u = unit_of(blockIdx.x, parts, a.n_expert, a.n_tok, a.n_used, group);
     if (u.count <= 0) return;

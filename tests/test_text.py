@@ -45,11 +45,29 @@ def _random_texts(n, seed):
     return ["".join(rng.choice(pool) for _ in range(rng.randint(1, 40))) for _ in range(n)]
 
 
+def _random_code_points(n, seed):
+    """Strings over the whole code space, every general category drawn equally often (a third ASCII): what decides
+    a piece is the class of each character, and the classes' tables are ranges over all planes."""
+    import unicodedata
+    rng = random.Random(seed)
+    cats = {}
+    for cp in range(0x110000):
+        if not 0xD800 <= cp <= 0xDFFF:
+            cats.setdefault(unicodedata.category(chr(cp)), []).append(cp)
+    names = sorted(cats)
+
+    def one():
+        if rng.random() < 0.35:
+            return rng.choice("abcXYZ 019\t\n\r'.,-sStTrReEvVmMlLdD")
+        return chr(rng.choice(cats[rng.choice(names)]))
+    return ["".join(one() for _ in range(rng.randint(1, 24))) for _ in range(n)]
+
+
 @pytest.mark.parametrize("marks,pattern", [(False, QWEN2), (True, QWEN35)], ids=["qwen2", "qwen35"])
 def test_the_pre_tokenizer_is_the_regex_it_hand_rolls(marks, pattern):
     regex = pytest.importorskip("regex")
     rx = regex.compile(pattern)
-    for text in CORPUS + _random_texts(600, 5 + marks):
+    for text in CORPUS + _random_texts(600, 5 + marks) + _random_code_points(3000, 11 + marks):
         want = [m.group(0).encode("utf-8") for m in rx.finditer(text)]
         got = T.split(text, marks)
         assert got == want, (text, got, want)
