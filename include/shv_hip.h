@@ -68,9 +68,20 @@ int shv_alloc(shv_ctx *ctx, size_t bytes, void **dptr);
 int shv_free(shv_ctx *ctx, void *dptr);
 int shv_upload(shv_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int shv_download(shv_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+/* shv_upload for a pass's control words and token ids (Buffer.WriteU32s on a host-visible buffer,
+ * vk/engine.go:319-634, costs the reference a store; a blocking upload costs 16 us of host time here,
+ * a dozen of them a speculative round): up to SHV_UPLOAD_ASYNC_MAX bytes are copied into pinned
+ * staging of the library's own and handed to the stream; the call returns at once, src_host may
+ * be reused, and the bytes are in place for every later op, copy or download of THIS context (work
+ * elsewhere must follow a shv_sync).  Larger transfers, and all of them with SHV_UPLOAD_SYNC=1 in
+ * the environment, block like shv_upload. */
+#define SHV_UPLOAD_ASYNC_MAX 512
+int shv_upload_async(shv_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int shv_copy(shv_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);  /* async, in order */
 int shv_zero(shv_ctx *ctx, void *dst_dev, size_t bytes);                       /* Buffer.Zero*, async */
-int shv_host_alloc(shv_ctx *ctx, size_t bytes, void **hptr);  /* pinned staging */
+/* Pinned host memory the device can address: staging for transfers, and somewhere an op can leave a
+ * small result (the arg-max's best) that the host reads after the submit's wait without a download. */
+int shv_host_alloc(shv_ctx *ctx, size_t bytes, void **hptr);
 int shv_host_free(shv_ctx *ctx, void *hptr);
 
 /* ---- op argument blocks ---------------------------------------------------------------- */

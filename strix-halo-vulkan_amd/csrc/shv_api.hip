@@ -63,6 +63,9 @@ int shv_init(int device, shv_ctx **out) {
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev_begin);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev_end);
+    const char *up_sync = std::getenv("SHV_UPLOAD_SYNC");
+    if (e == hipSuccess && !(up_sync && std::atoi(up_sync) != 0))
+        e = hipHostMalloc(reinterpret_cast<void **>(&ctx->up_ring), static_cast<size_t>(shv_ctx::kUpSlots) * shv_ctx::kUpSlotBytes, hipHostMallocDefault);
     ctx->n_counters = 4096;
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&ctx->counters), ctx->n_counters * sizeof(int32_t));
     if (e == hipSuccess) e = hipMemset(ctx->counters, 0, ctx->n_counters * sizeof(int32_t));
@@ -104,6 +107,7 @@ void shv_destroy(shv_ctx *ctx) {
     if (ctx->argmax_idx) (void)hipFree(ctx->argmax_idx);
     if (ctx->gemv_amax_val) (void)hipFree(ctx->gemv_amax_val);
     if (ctx->gemv_amax_idx) (void)hipFree(ctx->gemv_amax_idx);
+    if (ctx->up_ring) (void)hipHostFree(ctx->up_ring);
     for (hipEvent_t ev : ctx->mark_pool) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
@@ -126,7 +130,7 @@ int shv_device_props(shv_ctx *ctx, shv_props *out) {
 
 int shv_sync(shv_ctx *ctx) {
     SHV_REQUIRE(ctx, "shv_sync: NULL context");
-    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(ctx->wait_stream());
     return SHV_OK;
 }
 
@@ -152,7 +156,7 @@ int shv_alloc(shv_ctx *ctx, size_t bytes, void **dptr) {
 int shv_free(shv_ctx *ctx, void *dptr) {
     SHV_REQUIRE(ctx, "shv_free: NULL context");
     if (!dptr) return SHV_OK;
-    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(ctx->wait_stream());
     SHV_HIP_CHECK(hipFree(dptr));
     return SHV_OK;
 }
@@ -162,7 +166,22 @@ int shv_upload(shv_ctx *ctx, void *dst, const void *src, size_t bytes) {
     SHV_REQUIRE(!ctx->capturing, "shv_upload: not valid while recording");
     if (bytes == 0) return SHV_OK;
     SHV_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
-    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(ctx->wait_stream());
+    return SHV_OK;
+}
+
+int shv_upload_async(shv_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    SHV_REQUIRE(ctx && dst && src, "shv_upload_async: NULL argument");
+    SHV_REQUIRE(!ctx->capturing, "shv_upload_async: not valid while recording");
+    if (bytes == 0) return SHV_OK;
+    if (!ctx->up_ring || bytes > shv_ctx::kUpSlotBytes) return shv_upload(ctx, dst, src, bytes);
+    // a slot is free again once the stream has been waited for after the copy that read it
+    if (ctx->up_pending == shv_ctx::kUpSlots) SHV_HIP_CHECK(ctx->wait_stream());
+    char *slot = ctx->up_ring + static_cast<size_t>(ctx->up_next) * shv_ctx::kUpSlotBytes;
+    std::memcpy(slot, src, bytes);
+    SHV_HIP_CHECK(hipMemcpyAsync(dst, slot, bytes, hipMemcpyHostToDevice, ctx->stream));
+    ctx->up_next = (ctx->up_next + 1) % shv_ctx::kUpSlots;
+    ctx->up_pending++;
     return SHV_OK;
 }
 
@@ -171,7 +190,7 @@ int shv_download(shv_ctx *ctx, void *dst, const void *src, size_t bytes) {
     SHV_REQUIRE(!ctx->capturing, "shv_download: not valid while recording");
     if (bytes == 0) return SHV_OK;
     SHV_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
-    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(ctx->wait_stream());
     return SHV_OK;
 }
 
@@ -265,7 +284,7 @@ int shv_dispatch_multi(shv_ctx *ctx, const shv_op *ops, int n_ops, int iters, ui
         }
     ctx->marking = false;
     if (e == hipSuccess) e = hipEventRecord(ctx->ev_end, ctx->stream);
-    const hipError_t es = hipStreamSynchronize(ctx->stream);
+    const hipError_t es = ctx->wait_stream();
     if (e == hipSuccess) e = es;
     ctx->submits++;
     if (rc == SHV_OK && e == hipSuccess) {
@@ -292,7 +311,7 @@ int shv_prerecord(shv_ctx *ctx, const shv_op *ops, int n_ops, shv_prerecorded **
     SHV_REQUIRE(n_ops > 0, "shv_prerecord: empty op sequence");
     SHV_REQUIRE(!ctx->capturing, "shv_prerecord: already recording");
     *out = nullptr;
-    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(ctx->wait_stream());
     SHV_HIP_CHECK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
     int rc = SHV_OK;
@@ -336,7 +355,7 @@ int shv_prerecorded_submit(shv_ctx *ctx, shv_prerecorded *p, int iters, uint64_t
     SHV_HIP_CHECK(hipEventRecord(ctx->ev_begin, ctx->stream));
     for (int i = 0; i < iters; i++) SHV_HIP_CHECK(hipGraphLaunch(p->exec, ctx->stream));
     SHV_HIP_CHECK(hipEventRecord(ctx->ev_end, ctx->stream));
-    SHV_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SHV_HIP_CHECK(ctx->wait_stream());
     ctx->submits += static_cast<uint64_t>(iters);
     float ms = 0;
     SHV_HIP_CHECK(hipEventElapsedTime(&ms, ctx->ev_begin, ctx->ev_end));

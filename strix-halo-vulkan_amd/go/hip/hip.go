@@ -78,6 +78,12 @@ func (b *Buffer) Destroy()                      { C.shv_free(b.dev.ctx, b.ptr); 
 func (b *Buffer) Write(src []byte) error {
 	return call(func() C.int { return C.shv_upload(b.dev.ctx, b.ptr, unsafe.Pointer(&src[0]), C.size_t(len(src))) })
 }
+
+// WriteSoon is Write for a pass's control words and ids: up to 512 bytes are copied aside and handed to the
+// stream, and the call does not wait for the device (the reference writes such words into host-visible memory).
+func (b *Buffer) WriteSoon(src []byte) error {
+	return call(func() C.int { return C.shv_upload_async(b.dev.ctx, b.ptr, unsafe.Pointer(&src[0]), C.size_t(len(src))) })
+}
 func (b *Buffer) Read(dst []byte) error {
 	return call(func() C.int { return C.shv_download(b.dev.ctx, unsafe.Pointer(&dst[0]), b.ptr, C.size_t(len(dst))) })
 }

@@ -166,7 +166,7 @@ def make_op(kind, args, flags=0):
 # every symbol include/shv_hip.h declares; the CPU test suite checks the library exports them all
 SYMBOLS = [
     "shv_last_error", "shv_device_count", "shv_init", "shv_destroy", "shv_device_props", "shv_sync",
-    "shv_submits", "shv_alloc", "shv_free", "shv_upload", "shv_download", "shv_copy", "shv_zero",
+    "shv_submits", "shv_alloc", "shv_free", "shv_upload", "shv_upload_async", "shv_download", "shv_copy", "shv_zero",
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
     "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
@@ -198,6 +198,7 @@ def load():
     L.shv_alloc.argtypes = [vp, C.c_size_t, vpp]
     L.shv_free.argtypes = [vp, vp]
     L.shv_upload.argtypes = [vp, vp, vp, C.c_size_t]
+    L.shv_upload_async.argtypes = [vp, vp, vp, C.c_size_t]
     L.shv_download.argtypes = [vp, vp, vp, C.c_size_t]
     L.shv_copy.argtypes = [vp, vp, vp, C.c_size_t]
     L.shv_zero.argtypes = [vp, vp, C.c_size_t]
@@ -256,6 +257,14 @@ class DeviceBuffer:
         arr = np.ascontiguousarray(arr)
         assert byte_offset + arr.nbytes <= self.nbytes, (byte_offset, arr.nbytes, self.nbytes)
         check(self.ctx.L.shv_upload(self.ctx.h, self.ptr + byte_offset, arr.ctypes.data, arr.nbytes))
+        return self
+
+    def write_async(self, arr, byte_offset=0):
+        """write() that does not wait for the device when arr is up to 512 bytes (the array is copied before the
+        call returns); ordered before whatever this context does next."""
+        arr = np.ascontiguousarray(arr)
+        assert byte_offset + arr.nbytes <= self.nbytes, (byte_offset, arr.nbytes, self.nbytes)
+        check(self.ctx.L.shv_upload_async(self.ctx.h, self.ptr + byte_offset, arr.ctypes.data, arr.nbytes))
         return self
 
     def read(self, dtype, count, byte_offset=0):

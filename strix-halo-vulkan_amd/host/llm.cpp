@@ -24,7 +24,16 @@ Device::~Device() {
     if (!ctx_) return;
     shv_sync(ctx_);
     for (void *p : owned_) shv_free(ctx_, p);
+    for (void *p : host_owned_) shv_host_free(ctx_, p);
     shv_destroy(ctx_);
+}
+
+void *Device::host_alloc(size_t bytes) {
+    void *p = nullptr;
+    check(shv_host_alloc(ctx_, bytes, &p), "host_alloc");
+    std::memset(p, 0, bytes);
+    host_owned_.push_back(p);
+    return p;
 }
 
 void *Device::alloc(size_t bytes) {
@@ -50,7 +59,9 @@ void *Device::alloc_zero(size_t bytes) {
     return p;
 }
 
-void Device::upload(void *dst, const void *src, size_t bytes) { check(shv_upload(ctx_, dst, src, bytes), "upload"); }
+// small transfers (a pass's control words and ids) do not wait for the device; everything here runs on this
+// device's one stream, which orders them
+void Device::upload(void *dst, const void *src, size_t bytes) { check(shv_upload_async(ctx_, dst, src, bytes), "upload"); }
 void Device::download(void *dst, const void *src, size_t bytes) { check(shv_download(ctx_, dst, src, bytes), "download"); }
 void Device::zero(void *dst, size_t bytes) { check(shv_zero(ctx_, dst, bytes), "zero"); }
 void Device::sync() { check(shv_sync(ctx_), "sync"); }
@@ -1272,7 +1283,8 @@ Graph::Graph(Device &dev, const Model &m, const GraphOpts &opts) : dev_(dev), m_
     std::vector<int32_t> ix(S);
     for (size_t i = 0; i < S; i++) ix[i] = static_cast<int32_t>(i);
     dev.upload(slot_ix_, ix.data(), S * 4);
-    best_ = static_cast<int32_t *>(dev.alloc_zero(64 * 4));
+    // the rows' arg-maxes land in host memory: read after the pass's wait, no download
+    best_ = static_cast<int32_t *>(dev.host_alloc(64 * 4));
     // A long pass goes through every block whole: one projection over all its rows, one walk of
     // the recurrence, one launch of the attention.  LLM_PASS_GROUPS=1 keeps the older order
     // instead, groups of kBlockRows rows through the attention / DeltaNet blocks one after the
@@ -1635,7 +1647,10 @@ void Graph::DecodeRows(const std::vector<int> &slots, const std::vector<int32_t>
     }
 }
 
-std::vector<int32_t> Graph::Argmaxes() const { return read_back<int32_t>(dev_, best_, last_rows_ > 0 ? last_rows_ : 1); }
+std::vector<int32_t> Graph::Argmaxes() const {
+    dev_.sync();  // every pass is waited for when it is submitted; this costs nothing then
+    return std::vector<int32_t>(best_, best_ + (last_rows_ > 0 ? last_rows_ : 1));
+}
 
 std::vector<int32_t> Graph::Generate(int n, uint64_t *gpu_nanos) {
     Seq &q = seq_[slot_];
@@ -1821,7 +1836,7 @@ MTPHead::MTPHead(Device &dev, const Model &m, HeadGPU &head, int maxTok, int nKV
     pos_ = ctl_;
     slot_ix_ = ctl_ + S;
     ids_ = ctl_ + 2 * S;
-    best_ = ids_ + T;
+    best_ = static_cast<int32_t *>(dev.host_alloc(16 * 4));  // the draft's arg-max, read by the host after the pass's wait
     std::vector<int32_t> ix(S);
     for (size_t i = 0; i < S; i++) ix[i] = static_cast<int32_t>(i);
     dev.upload(slot_ix_, ix.data(), S * 4);
@@ -1922,9 +1937,7 @@ int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos,
     Steps++;
     pasts_[slot_] = pos + n;
     if (!head) return -1;
-    int32_t best = -1;
-    dev_.download(&best, best_, 4);
-    return best;
+    return best_[0];  // submit_pass has waited for the pass
 }
 
 void MTPHead::RowsHost(const std::vector<float> &hs, const std::vector<int32_t> &ids, int pos, bool head, std::vector<float> *logits,

@@ -38,6 +38,7 @@ public:
     void *alloc(size_t bytes);  // tracked; released with the device
     void *alloc_zero(size_t bytes);
     void release(void *p, size_t bytes);  // an alloc() handed back early; bytes as asked for
+    void *host_alloc(size_t bytes);       // pinned host memory the device can write; zeroed, released with the device
     void upload(void *dst, const void *src, size_t bytes);
     void download(void *dst, const void *src, size_t bytes);
     void zero(void *dst, size_t bytes);
@@ -47,7 +48,7 @@ public:
 
 private:
     shv_ctx *ctx_ = nullptr;
-    std::vector<void *> owned_;
+    std::vector<void *> owned_, host_owned_;
     size_t allocated_ = 0;
 };
 

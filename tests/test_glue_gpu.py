@@ -140,3 +140,36 @@ def test_vocabulary_projection_names_the_next_token_itself(ctx):
     with pytest.raises(A.ShvError, match="one plain row"):
         g.n_tok = 2
         ctx.enqueue(A.OP_GEMV_Q4K, g)
+
+
+def test_small_uploads_that_do_not_wait_arrive_in_order(ctx):
+    """shv_upload_async: a pass's control words go through pinned staging and the call returns at once.  What a
+    later download or op of the context sees is what blocking uploads would have left: several hundred of them in a
+    row (more than the staging ring holds, so it wraps and waits), overlapping destinations where the last write
+    wins, a source buffer reused right after each call, and a transfer above the limit taking the blocking road."""
+    rng = np.random.default_rng(3)
+    buf = ctx.alloc(4096 * 4)
+    want = np.zeros(4096, np.int32)
+    buf.write(want)
+    src = np.zeros(128, np.int32)
+    for i in range(700):
+        n = int(rng.integers(1, 129))
+        at = int(rng.integers(0, 4096 - n))
+        src[:n] = rng.integers(-2 ** 31, 2 ** 31 - 1, size=n)
+        buf.write_async(src[:n], byte_offset=at * 4)
+        want[at:at + n] = src[:n]
+        src[:] = -1                                     # the call has copied what it needs
+    assert np.array_equal(buf.read(np.int32, 4096), want)
+    big = rng.integers(0, 100, size=1000).astype(np.int32)   # 4000 bytes: above the limit
+    buf.write_async(big)
+    want[:1000] = big
+    assert np.array_equal(buf.read(np.int32, 4096), want)
+    # an op enqueued right behind an upload sees it: the arg-max of the row just written
+    row = np.zeros(100, np.float32)
+    logits, best = ctx.alloc(400), ctx.alloc(16)
+    for winner in (7, 93, 0, 41):
+        row[:] = 0
+        row[winner] = 1
+        logits.write_async(row)
+        ctx.enqueue(A.OP_ARGMAX, A.ArgmaxArgs(logits.ptr, best.ptr, None, None, 1, 100, 100))
+        assert int(best.read(np.int32, 1)[0]) == winner
