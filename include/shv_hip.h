@@ -537,6 +537,12 @@ int shv_dispatch_multi(shv_ctx *ctx, const shv_op *ops, int n_ops, int iters,
 int shv_prerecord(shv_ctx *ctx, const shv_op *ops, int n_ops, shv_prerecorded **out);
 int shv_prerecorded_submit(shv_ctx *ctx, shv_prerecorded *p, int iters, uint64_t *total_ns);
 int shv_prerecorded_launch(shv_ctx *ctx, shv_prerecorded *p);
+/* GPU time between two points of the stream for work handed over with launch (which does not block):
+ * shv_stamp(i) marks the point the stream has reached, i in 0..SHV_STAMPS-1; after a wait (shv_sync,
+ * a submit, a download) shv_stamp_elapsed gives the nanoseconds from stamp `from` to stamp `to`. */
+#define SHV_STAMPS 4
+int shv_stamp(shv_ctx *ctx, int i);
+int shv_stamp_elapsed(shv_ctx *ctx, int from, int to, uint64_t *ns);
 int shv_prerecorded_count(const shv_prerecorded *p);
 void shv_prerecorded_destroy(shv_ctx *ctx, shv_prerecorded *p);
 

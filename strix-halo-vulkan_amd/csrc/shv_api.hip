@@ -109,6 +109,8 @@ void shv_destroy(shv_ctx *ctx) {
     if (ctx->gemv_amax_idx) (void)hipFree(ctx->gemv_amax_idx);
     if (ctx->up_ring) (void)hipHostFree(ctx->up_ring);
     for (hipEvent_t ev : ctx->mark_pool) (void)hipEventDestroy(ev);
+    for (hipEvent_t ev : ctx->stamps)
+        if (ev) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -346,6 +348,28 @@ int shv_prerecorded_launch(shv_ctx *ctx, shv_prerecorded *p) {
     SHV_REQUIRE(ctx && p && p->exec, "shv_prerecorded_launch: NULL argument");
     SHV_HIP_CHECK(hipGraphLaunch(p->exec, ctx->stream));
     ctx->submits++;
+    return SHV_OK;
+}
+
+int shv_stamp(shv_ctx *ctx, int i) {
+    SHV_REQUIRE(ctx && i >= 0 && i < SHV_STAMPS, "shv_stamp: stamp %d of %d", i, SHV_STAMPS);
+    SHV_REQUIRE(!ctx->capturing, "shv_stamp: not valid while recording");
+    if (!ctx->stamps[i]) SHV_HIP_CHECK(hipEventCreate(&ctx->stamps[i]));
+    SHV_HIP_CHECK(hipEventRecord(ctx->stamps[i], ctx->stream));
+    return SHV_OK;
+}
+
+int shv_stamp_elapsed(shv_ctx *ctx, int from, int to, uint64_t *ns) {
+    SHV_REQUIRE(ctx && ns && from >= 0 && from < SHV_STAMPS && to >= 0 && to < SHV_STAMPS, "shv_stamp_elapsed: bad argument");
+    SHV_REQUIRE(ctx->stamps[from] && ctx->stamps[to], "shv_stamp_elapsed: a stamp that was never made");
+    float ms = 0;
+    const hipError_t e = hipEventElapsedTime(&ms, ctx->stamps[from], ctx->stamps[to]);
+    if (e == hipErrorNotReady) {
+        (void)hipGetLastError();
+        return shv_set_error(SHV_E_STATE, "shv_stamp_elapsed: the stream has not reached the stamps yet; wait for it first");
+    }
+    SHV_HIP_CHECK(e);
+    *ns = static_cast<uint64_t>(static_cast<double>(ms < 0 ? 0 : ms) * 1e6);
     return SHV_OK;
 }
 

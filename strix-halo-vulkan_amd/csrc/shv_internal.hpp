@@ -37,6 +37,7 @@ struct shv_ctx {
     int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)
     int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    hipEvent_t stamps[SHV_STAMPS] = {};  // shv_stamp's, made when first used
     // shv_upload_async copies up to kUpSlotBytes into the next slot of a ring of pinned host memory and hands them
     // to the stream from there: the call returns without waiting for the device (a pass's control words, a few
     // token ids).  up_pending counts the slots written since the stream was last waited for; a full ring waits.

@@ -454,5 +454,14 @@ func (p *Prerecorded) Submit(iters int) (time.Duration, error) {
 func (p *Prerecorded) Launch() error {
 	return call(func() C.int { return C.shv_prerecorded_launch(p.dev.ctx, p.p) })
 }
+
+// Stamp marks the point the stream has reached (i in 0..3); StampElapsed is the GPU time between two stamps once the
+// stream has been waited for: the time of work handed over with Launch.
+func (d *Device) Stamp(i int) error { return call(func() C.int { return C.shv_stamp(d.ctx, C.int(i)) }) }
+func (d *Device) StampElapsed(from, to int) (time.Duration, error) {
+	var ns C.uint64_t
+	err := call(func() C.int { return C.shv_stamp_elapsed(d.ctx, C.int(from), C.int(to), &ns) })
+	return time.Duration(ns), err
+}
 func (p *Prerecorded) Count() int { return int(C.shv_prerecorded_count(p.p)) }
 func (p *Prerecorded) Destroy()   { C.shv_prerecorded_destroy(p.dev.ctx, p.p); p.p = nil }

@@ -168,7 +168,7 @@ SYMBOLS = [
     "shv_last_error", "shv_device_count", "shv_init", "shv_destroy", "shv_device_props", "shv_sync",
     "shv_submits", "shv_alloc", "shv_free", "shv_upload", "shv_upload_async", "shv_download", "shv_copy", "shv_zero",
     "shv_host_alloc", "shv_host_free", "shv_enqueue", "shv_dispatch_multi", "shv_prerecord",
-    "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_prerecorded_count",
+    "shv_prerecorded_submit", "shv_prerecorded_launch", "shv_stamp", "shv_stamp_elapsed", "shv_prerecorded_count",
     "shv_prerecorded_destroy", "shv_gemv_q4k", "shv_dequant_q4k", "shv_dequant", "shv_gemv", "shv_quantize_q4k",
     "shv_fill_normal", "shv_moe_router", "shv_moe_up", "shv_moe_down", "shv_dn_step", "shv_attn_decode", "shv_embed", "shv_argmax", "shv_advance",
     "shv_argmax_static", "shv_ring_rows", "shv_router_fold", "shv_qsa_index",
@@ -210,6 +210,8 @@ def load():
     L.shv_prerecord.argtypes = [vp, C.POINTER(Op), C.c_int, vpp]
     L.shv_prerecorded_submit.argtypes = [vp, vp, C.c_int, C.POINTER(C.c_uint64)]
     L.shv_prerecorded_launch.argtypes = [vp, vp]
+    L.shv_stamp.argtypes = [vp, C.c_int]
+    L.shv_stamp_elapsed.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_uint64)]
     L.shv_prerecorded_count.argtypes = [vp]
     L.shv_prerecorded_destroy.argtypes = [vp, vp]
     L.shv_prerecorded_destroy.restype = None
@@ -334,6 +336,14 @@ class Context:
 
     def sync(self):
         check(self.L.shv_sync(self.h))
+
+    def stamp(self, i):
+        check(self.L.shv_stamp(self.h, i))
+
+    def stamp_elapsed(self, frm, to):
+        ns = C.c_uint64()
+        check(self.L.shv_stamp_elapsed(self.h, frm, to, C.byref(ns)))
+        return ns.value
 
     def enqueue(self, kind, args):
         check(self.L.shv_enqueue(self.h, kind, C.byref(args), C.sizeof(args)))

@@ -1612,6 +1612,31 @@ void Graph::ExtendRows(const std::vector<int32_t> &ids, std::vector<float> *logi
     }
 }
 
+void Graph::StageIds(int at, const std::vector<int32_t> &ids) {
+    if (at < 0 || at + static_cast<int>(ids.size()) > o_.NKV) throw Error("llm: Graph.StageIds: positions " + std::to_string(at) + ".. do not fit " + std::to_string(o_.NKV) + " cells");
+    check_ids(ids);
+    dev_.upload(ids_ + slot_ * ids_stride_ + at, ids.data(), ids.size() * 4);
+}
+
+void Graph::ExtendRowsStaged(int n) {
+    if (!head_) throw Error("llm: this graph was staged without a head");
+    Seq &q = seq_[slot_];
+    if (n <= 0 || n > head_->MaxRows()) throw Error("llm: " + std::to_string(n) + " rows, the head arena holds " + std::to_string(head_->MaxRows()) + " — GraphOpts.HeadRows");
+    if (spec_armed_) throw Error("llm: a speculative pass is in flight; commit or rewind it first");
+    if (q.past + n + 1 > o_.NKV) throw Error("llm: Graph.ExtendRows: " + std::to_string(q.past + n) + " tokens do not fit " + std::to_string(o_.NKV) + " cells");
+    Pass &p = pass(slot_, n, kRows, spec_);
+    put_pos();
+    submit(p, 1, "rows");
+    Stats.Runs++;
+    if (spec_) {
+        spec_armed_ = true;
+        spec_past_ = q.past;
+        spec_rows_ = n;
+    }
+    q.past += n;
+    last_rows_ = n;
+}
+
 void Graph::DecodeRows(const std::vector<int> &slots, const std::vector<int32_t> &ids, std::vector<float> *logits) {
     const int n = static_cast<int>(slots.size());
     if (n == 0 || n != static_cast<int>(ids.size())) throw Error("llm: " + std::to_string(n) + " slots and " + std::to_string(ids.size()) + " tokens");
@@ -1866,22 +1891,24 @@ void MTPHead::SetVocab(int k) {
     vocab_ = k;
 }
 
-int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos, bool head) {
-    const int n = static_cast<int>(ids.size());
-    if (!hs || n < 1 || n > max_tok_) throw Error("llm: MTPHead.Rows: " + std::to_string(n) + " rows, staged for " + std::to_string(max_tok_));
-    if (pos < 0 || pos > pasts_[slot_]) throw Error("llm: MTPHead.Rows: position " + std::to_string(pos) + " leaves a gap after the draft cache's " + std::to_string(pasts_[slot_]) + " cells");
-    if (pos + n + 1 > n_kv_) throw Error("llm: MTPHead.Rows: " + std::to_string(pos + n) + " cells do not fit " + std::to_string(n_kv_));
-    for (int32_t id : ids)
-        if (id < 0 || id >= c_.VocabSize) throw Error("llm: token " + std::to_string(id) + " is outside the vocabulary");
-    const std::vector<int> key{slot_, n, head ? 1 : 0};
+Pass &MTPHead::draft_pass(int n, bool head, int k, int32_t *ring) {
+    // ring: the tokens come from the trunk's id ring at this head's position word, and the arg-max goes back there
+    const std::vector<int> key{slot_, n, head ? 1 : 0, ring ? 1 + k : 0};
     auto it = passes_.find(key);
+    if (it != passes_.end() && it->second.ring != ring) {
+        if (it->second.rec) shv_prerecorded_destroy(dev_.ctx(), it->second.rec);
+        passes_.erase(it);
+        it = passes_.end();
+    }
     if (it == passes_.end()) {
         Pass p;
+        p.ring = ring;
         const int E = c_.NEmbd;
         shv_embed_args e{};
         e.table = m_.Tensor("token_embd.weight").ptr;
         e.type = static_cast<int32_t>(m_.Tensor("token_embd.weight").ggml);
-        e.ids = ids_;
+        e.ids = ring ? ring : ids_;
+        e.pos = ring ? pos_ + slot_ : nullptr;
         e.x = e_;
         e.n_tok = n;
         e.n_embd = E;
@@ -1919,7 +1946,12 @@ int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos,
             p.ops.insert(p.ops.end(), h.begin(), h.end());
             shv_argmax_args am{};
             am.logits = logits_;
-            am.best = best_;
+            am.best = best_ + (ring ? k : 0);
+            if (ring) {
+                am.ids = ring;
+                am.pos = pos_ + slot_;
+                am.advance = n;
+            }
             am.n_rows = 1;
             am.n = cols;
             am.logits_stride = c_.VocabSize;
@@ -1928,12 +1960,41 @@ int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos,
         }
         it = passes_.emplace(key, std::move(p)).first;
     }
+    return it->second;
+}
+
+void MTPHead::RowsChained(const float *hs, int n, int pos, int k, int32_t *ring) {
+    if (!hs || !ring || n < 1 || n > max_tok_) throw Error("llm: MTPHead.RowsChained: " + std::to_string(n) + " rows, staged for " + std::to_string(max_tok_));
+    if (k < 0 || k >= 16) throw Error("llm: MTPHead.RowsChained: draft " + std::to_string(k));
+    const int at = pos >= 0 ? pos : pasts_[slot_];  // the device's position word follows the calls as pasts_ does
+    if (at > pasts_[slot_]) throw Error("llm: MTPHead.Rows: position " + std::to_string(at) + " leaves a gap after the draft cache's " + std::to_string(pasts_[slot_]) + " cells");
+    if (at + n + 1 > n_kv_) throw Error("llm: MTPHead.Rows: " + std::to_string(at + n) + " cells do not fit " + std::to_string(n_kv_));
+    Pass &pass = draft_pass(n, true, k, ring);
+    check(shv_copy(dev_.ctx(), h_, hs, static_cast<size_t>(n) * c_.NEmbd * 4), "draft input");
+    if (pos >= 0) {
+        const int32_t p32 = pos;
+        dev_.upload(pos_ + slot_, &p32, 4);
+    }
+    if (!pass.rec) check(shv_prerecord(dev_.ctx(), pass.ops.data(), static_cast<int>(pass.ops.size()), &pass.rec), "draft");
+    check(shv_prerecorded_launch(dev_.ctx(), pass.rec), "draft");
+    Steps++;
+    pasts_[slot_] = at + n;
+}
+
+int32_t MTPHead::Rows(const float *hs, const std::vector<int32_t> &ids, int pos, bool head) {
+    const int n = static_cast<int>(ids.size());
+    if (!hs || n < 1 || n > max_tok_) throw Error("llm: MTPHead.Rows: " + std::to_string(n) + " rows, staged for " + std::to_string(max_tok_));
+    if (pos < 0 || pos > pasts_[slot_]) throw Error("llm: MTPHead.Rows: position " + std::to_string(pos) + " leaves a gap after the draft cache's " + std::to_string(pasts_[slot_]) + " cells");
+    if (pos + n + 1 > n_kv_) throw Error("llm: MTPHead.Rows: " + std::to_string(pos + n) + " cells do not fit " + std::to_string(n_kv_));
+    for (int32_t id : ids)
+        if (id < 0 || id >= c_.VocabSize) throw Error("llm: token " + std::to_string(id) + " is outside the vocabulary");
+    Pass &pass = draft_pass(n, head, 0, nullptr);
     // the block's input h may be this block's own output rows: it is copied aside first
     check(shv_copy(dev_.ctx(), h_, hs, static_cast<size_t>(n) * c_.NEmbd * 4), "draft input");
     dev_.upload(ids_, ids.data(), static_cast<size_t>(n) * 4);
     const int32_t p32 = pos;
     dev_.upload(pos_ + slot_, &p32, 4);
-    GPUNanos += submit_pass(dev_, it->second, 1, "draft");
+    GPUNanos += submit_pass(dev_, pass, 1, "draft");
     Steps++;
     pasts_[slot_] = pos + n;
     if (!head) return -1;
@@ -1971,6 +2032,7 @@ Speculator::Speculator(Graph &g, MTPHead &d, int depth, int slot) : Depth(depth)
         throw Error("llm: speculator slot " + std::to_string(slot) + "; the trunk holds " + std::to_string(g.Slots()) + " and the draft " + std::to_string(d.Slots()));
     // the owed rows (fewer than one draft call's worth: Owe settles at that) and the seed after them
     cap_rows_ = std::max(depth + 1, d.MaxRows()) + 2;
+    if (const char *e = std::getenv("LLM_SPEC_CHAIN")) chained_ = e[0] != '0';
     h_ = static_cast<float *>(g.Dev().alloc(static_cast<size_t>(cap_rows_) * g.GetModel().config().NEmbd * 4));
     if (slot < 0) {
         g.Speculate(true);
@@ -2195,6 +2257,7 @@ std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced, int l
     if (pend_ < 0) throw Error("llm: Speculator.Round before Start");
     use_slot();
     if (sampler_) return sampled_round(forced, limit);
+    if (chained_ && !no_prerecord()) return chained_round(forced, limit);
     const size_t E = g_.GetModel().config().NEmbd;
     const int at = g_.Past();
     const int owed = static_cast<int>(owe_x_.size());
@@ -2219,14 +2282,17 @@ std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced, int l
     const uint64_t v0 = g_.Stats.GPUNanos;
     g_.ExtendRows(rows, nullptr, nullptr);
     Stats.VerifyNanos += g_.Stats.GPUNanos - v0;
-    const std::vector<int32_t> best = g_.Argmaxes();
+    return finish_round(rows, g_.Argmaxes(), at, limit);
+}
+
+// 3. row i's arg-max is the trunk's token at at+i+1; the pass is the sequence up to the first
+//    draft it disagrees with
+std::vector<int32_t> Speculator::finish_round(const std::vector<int32_t> &rows, const std::vector<int32_t> &best, int at, int limit) {
+    const size_t E = g_.GetModel().config().NEmbd;
     const int n = static_cast<int>(rows.size());
     Stats.Passes[std::min(n, 4)]++;
     Stats.Rounds++;
     if (n > 1) Stats.Drafted++;
-
-    // 3. row i's arg-max is the trunk's token at at+i+1; the pass is the sequence up to the first
-    //    draft it disagrees with
     std::vector<int32_t> out;
     for (int i = 0; i < n; i++) {
         if (limit > 0 && static_cast<int>(out.size()) >= limit) break;
@@ -2247,6 +2313,38 @@ std::vector<int32_t> Speculator::Round(const std::vector<int32_t> &forced, int l
     pend_ = out[keep - 1];
     Stats.Tokens += keep;
     return out;
+}
+
+// The greedy round without a wait between its passes.  Nothing the host decides depends on a draft before the
+// verification pass has run: the draft head reads its tokens from the trunk's id ring, names the next one there
+// itself and moves its own position word, the verification pass reads the same ring, and the host learns drafts and
+// arg-maxes together after the one wait (what each call's wait cost: 25 us of launch and wake-up, three a round).
+std::vector<int32_t> Speculator::chained_round(const std::vector<int32_t> &forced, int limit) {
+    const size_t E = g_.GetModel().config().NEmbd;
+    const int at = g_.Past();
+    const int owed = static_cast<int>(owe_x_.size());
+    int32_t *ring = g_.IdsPort();
+    std::vector<int32_t> xs(owe_x_);
+    xs.push_back(pend_);
+    g_.StageIds(at - owed, xs);
+    check(shv_stamp(g_.Dev().ctx(), 0), "stamp");
+    for (int k = 0; k < Depth; k++) {
+        if (k == 0) d_.RowsChained(h_, owed + 1, at - owed, 0, ring);
+        else d_.RowsChained(d_.ResPort() + (k == 1 ? static_cast<size_t>(owed) * E : 0), 1, -1, k, ring);
+        // a forced draft replaces the head's own in the ring before anything reads it
+        if (k < static_cast<int>(forced.size())) g_.StageIds(at + k + 1, {forced[k]});
+    }
+    check(shv_stamp(g_.Dev().ctx(), 1), "stamp");
+    const uint64_t v0 = g_.Stats.GPUNanos;
+    g_.ExtendRowsStaged(Depth + 1);
+    Stats.VerifyNanos += g_.Stats.GPUNanos - v0;
+    uint64_t dns = 0;
+    check(shv_stamp_elapsed(g_.Dev().ctx(), 0, 1, &dns), "stamp");
+    Stats.DraftNanos += dns;
+    d_.GPUNanos += dns;
+    std::vector<int32_t> rows{pend_};
+    for (int k = 0; k < Depth; k++) rows.push_back(k < static_cast<int>(forced.size()) ? forced[k] : d_.DraftAt(k));
+    return finish_round(rows, g_.Argmaxes(), at, limit);
 }
 
 }  // namespace llm

@@ -399,6 +399,7 @@ struct Pass {
     std::vector<shv_op> ops;
     std::vector<std::string> labels;
     shv_prerecorded *rec = nullptr;
+    int32_t *ring = nullptr;  // a draft pass that reads its tokens from the trunk's id ring: which ring
 };
 
 // llm.Checkpoint (llm/graph.go:902-1003): a sequence's position, tokens and DeltaNet carry, in host
@@ -432,6 +433,12 @@ public:
     void ExtendRows(const std::vector<int32_t> &ids, std::vector<float> *logits, std::vector<float> *res);
     // DecodeRows advances n sequences by one token each in one pass (llm/graph.go:1527-1666).
     void DecodeRows(const std::vector<int> &slots, const std::vector<int32_t> &ids, std::vector<float> *logits);
+    // The same pass over ids that are on the device already: StageIds puts tokens at positions at.. of the live
+    // slot's id ring without waiting for the device, IdsPort() is that ring for an op that names a token itself
+    // (a draft head's arg-max), ExtendRowsStaged runs the n rows at positions past.. that the ring then holds.
+    void StageIds(int at, const std::vector<int32_t> &ids);
+    int32_t *IdsPort() const { return ids_ + slot_ * ids_stride_; }
+    void ExtendRowsStaged(int n);
     std::vector<int32_t> Argmaxes() const;     // the greedy token of each row of the last ExtendRows / DecodeRows
     const float *ResPort() const { return x_; }  // residual rows of the last pass, on the device
     // Greedy continuation (cmd/llm/generate.go:121-165): n replays of the recorded decode step with
@@ -536,6 +543,12 @@ public:
     // the reference's host-side signature: hs from host memory, logits and residual copied back
     void RowsHost(const std::vector<float> &hs, const std::vector<int32_t> &ids, int pos, bool head,
                   std::vector<float> *logits, std::vector<float> *res);
+    // Rows for a caller that does not wait (a greedy round): the n tokens are read from `ring` (the trunk's id ring
+    // of the sequence) at positions pos..pos+n-1, the head's arg-max is stored as the token at pos+n there, kept
+    // for DraftAt(k) and moves this head's position word on, so that the call for draft k+1 (n = 1, pos < 0: the
+    // position the device holds) needs nothing from the host.  Returns without waiting for the device.
+    void RowsChained(const float *hs, int n, int pos, int k, int32_t *ring);
+    int32_t DraftAt(int k) const { return best_[k]; }  // valid once the stream has been waited for
     const float *ResPort() const { return x_; }  // [n][NEmbd] of the last call
     void LastLogits(std::vector<float> *out);     // the last head call's logits, over the drafted prefix of the vocabulary
     int Past() const { return pasts_[slot_]; }
@@ -560,6 +573,7 @@ private:
     float *x_, *h_, *e_, *logits_;
     int32_t *ctl_, *pos_, *slot_ix_, *ids_, *best_;
     std::map<std::vector<int>, Pass> passes_;
+    Pass &draft_pass(int n, bool head, int k, int32_t *ring);
 };
 
 // llm.SpecStats (llm/spec.go:67-112), the counters that exist without a sampler.
@@ -637,6 +651,10 @@ private:
     bool exact_ = false;
     std::unique_ptr<Sampler> draft_sampler_;
     std::vector<int32_t> sampled_round(const std::vector<int32_t> &forced, int limit);
+    // the greedy round handed to the device in one go: drafts and verification back to back, one wait
+    bool chained_ = true;  // LLM_SPEC_CHAIN=0: every draft call and the verification pass waited for in turn
+    std::vector<int32_t> chained_round(const std::vector<int32_t> &forced, int limit);
+    std::vector<int32_t> finish_round(const std::vector<int32_t> &rows, const std::vector<int32_t> &best, int at, int limit);
 };
 
 }  // namespace llm
