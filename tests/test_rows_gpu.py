@@ -337,6 +337,34 @@ def test_speculative_loop_emits_the_greedy_sequence(rig, mode):
     assert list(m.ids()) == list(prompt) + out[:-1]
 
 
+def test_a_round_handed_over_whole_is_the_round_waited_for_call_by_call(rig, monkeypatch):
+    """The greedy round launches its draft calls and the verification pass back to back and waits once (the drafts
+    travel through the trunk's id ring on the device); LLM_SPEC_CHAIN=0 waits after every call and carries the drafts
+    through the host, as the reference's loop does.  Same tokens round by round, same counters, same sequence left
+    in the trunk, with the head's own drafts and with forced ones that end a round early."""
+    m, cfg, tensors = rig
+    rng = np.random.default_rng(23)
+    prompt = rng.integers(0, cfg.vocab, size=9).astype(np.int32)
+    depth = ROWS - 1
+    runs = {}
+    for chain in ("0", "1"):
+        monkeypatch.setenv("LLM_SPEC_CHAIN", chain)
+        fresh(m)
+        m.mtp_stage(max_tok=ROWS)
+        m.spec_open(depth)
+        rounds = [[m.spec_start(prompt)]]
+        for i in range(10):
+            forced = [] if i % 3 else [int(rounds[-1][-1] + 1) % cfg.vocab]   # a wrong first draft: one token kept
+            rounds.append(list(m.spec_round(forced)))
+            if not i % 3:
+                assert len(rounds[-1]) == 1
+        st = m.spec_stats()
+        runs[chain] = (rounds, {k: st[k] for k in ("rounds", "tokens", "drafted", "accepted", "passes", "drafted_at", "accepted_at")},
+                       list(m.ids()), m.past())
+    assert runs["0"] == runs["1"]
+    assert runs["1"][1]["rounds"] == 10
+
+
 def test_sampled_speculation(rig):
     """The loop under a sampler (Speculator.UseSampler; llm/spec.go:703-857 with llm/sample.go:183-250):
     drafts are draws from the draft sampler's distribution, rows go through Verify on the host.
