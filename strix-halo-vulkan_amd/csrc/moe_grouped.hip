@@ -46,22 +46,34 @@ constexpr int kMaxExperts = 1024;
 // value depends on it.
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, int n_tok, int n_used, int n_expert, int32_t *group) {
     __shared__ int32_t s_cnt[kMaxExperts + 1];
+    __shared__ __align__(16) int32_t s_len[kMaxExperts];
     const int tid = threadIdx.x, n_pairs = n_tok * n_used;
     for (int e = tid; e <= n_expert; e += blockDim.x) s_cnt[e] = 0;
-    __syncthreads();
-    // eight of a thread's selections are asked for before the first is counted: the passes over topk cost its latency once a batch, not once a pair
-    constexpr int NB = 8;
-    for (int i0 = tid; i0 < n_pairs; i0 += NB * blockDim.x) {
-        int e[NB];
+    for (int e = tid; e < kMaxExperts; e += blockDim.x) s_len[e] = -1;  // past n_expert: shorter than any list
+    // A thread's selections are asked for once, all together, and stay in registers for both passes (the count and
+    // the placement): up to NQ quads of four a thread, i.e. 4096 * NQ pairs; a longer pass reads the rest again.
+    constexpr int NQ = 8;
+    // whole quads of an aligned table; the tail and what does not fit the registers go one by one
+    const int n_quads = (reinterpret_cast<uintptr_t>(topk) & 15) == 0 ? n_pairs / 4 : 0;
+    int4 q[NQ];
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const int i = i0 + b * blockDim.x;
-            e[b] = i < n_pairs ? topk[i] : -1;
-        }
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-            if (e[b] >= 0 && e[b] < n_expert) atomicAdd(&s_cnt[e[b]], 1);
+    for (int b = 0; b < NQ; b++) {
+        const int i = tid + b * 1024;
+        q[b] = i < n_quads ? reinterpret_cast<const int4 *>(topk)[i] : make_int4(-1, -1, -1, -1);
     }
+    const int rest0 = (n_quads < NQ * 1024 ? n_quads : NQ * 1024) * 4;
+    __syncthreads();
+    auto count = [&](int e) {
+        if (e >= 0 && e < n_expert) atomicAdd(&s_cnt[e], 1);
+    };
+#pragma unroll
+    for (int b = 0; b < NQ; b++) {
+        count(q[b].x);
+        count(q[b].y);
+        count(q[b].z);
+        count(q[b].w);
+    }
+    for (int i = rest0 + tid; i < n_pairs; i += 1024) count(topk[i]);
     __syncthreads();
     {
         // starts = running sum of the counts: thread e takes expert e (the block has a thread for each)
@@ -78,37 +90,46 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
         __syncthreads();
         int base = 0;
         for (int w = 0; w < wave; w++) base += s_wsum[w];
-        if (tid < n_expert) s_cnt[tid] = base + incl - c;
+        if (tid < n_expert) {
+            s_cnt[tid] = base + incl - c;
+            s_len[tid] = c;
+        }
         if (tid == n_expert - 1) s_cnt[n_expert] = base + incl;
     }
     __syncthreads();
     for (int e = tid; e <= n_expert; e += blockDim.x) group[e] = s_cnt[e];
-    // rank by list length, longer first, equal lengths by index: an expert's place in the launch
+    // rank by list length, longer first, equal lengths by index: an expert's place in the launch.  Every thread
+    // walks the same lengths, four a read (one address a wave: a broadcast), sixteen reads in flight.
     int32_t *order = group + n_expert + 1 + n_pairs;
-    for (int e = tid; e < n_expert; e += blockDim.x) {
-        const int ce = s_cnt[e + 1] - s_cnt[e];
+    if (tid < n_expert) {
+        const int e = tid, ce = s_len[e];
         int rank = 0;
-        for (int o = 0; o < n_expert; o++) {
-            const int co = s_cnt[o + 1] - s_cnt[o];
-            rank += (co > ce || (co == ce && o < e)) ? 1 : 0;
+        const int n4 = (n_expert + 3) / 4;
+#pragma unroll 16
+        for (int o4 = 0; o4 < n4; o4++) {
+            const int4 c4 = *reinterpret_cast<const int4 *>(&s_len[4 * o4]);
+            const int o = 4 * o4;
+            rank += (c4.x > ce || (c4.x == ce && o < e)) ? 1 : 0;
+            rank += (c4.y > ce || (c4.y == ce && o + 1 < e)) ? 1 : 0;
+            rank += (c4.z > ce || (c4.z == ce && o + 2 < e)) ? 1 : 0;
+            rank += (c4.w > ce || (c4.w == ce && o + 3 < e)) ? 1 : 0;
         }
         order[rank] = e;
     }
-    __syncthreads();
+    __syncthreads();  // the starts are copied out before the placement moves them
     int32_t *list = group + n_expert + 1;
-    for (int i0 = tid; i0 < n_pairs; i0 += NB * blockDim.x) {
-        int e[NB];
+    auto place = [&](int e, int i) {
+        if (e >= 0 && e < n_expert) list[atomicAdd(&s_cnt[e], 1)] = (i / n_used) * (n_used + 1) + i % n_used;
+    };
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const int i = i0 + b * blockDim.x;
-            e[b] = i < n_pairs ? topk[i] : -1;
-        }
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const int i = i0 + b * blockDim.x;
-            if (e[b] >= 0 && e[b] < n_expert) list[atomicAdd(&s_cnt[e[b]], 1)] = (i / n_used) * (n_used + 1) + i % n_used;
-        }
+    for (int b = 0; b < NQ; b++) {
+        const int i = 4 * (tid + b * 1024);
+        place(q[b].x, i);
+        place(q[b].y, i + 1);
+        place(q[b].z, i + 2);
+        place(q[b].w, i + 3);
     }
+    for (int i = rest0 + tid; i < n_pairs; i += 1024) place(topk[i], i);
 }
 
 // Columns [col0, col0 + kSlab) of up to kTok listed rows (each a row of floats at rows_s[i]) into
