@@ -173,3 +173,27 @@ def test_small_uploads_that_do_not_wait_arrive_in_order(ctx):
         logits.write_async(row)
         ctx.enqueue(A.OP_ARGMAX, A.ArgmaxArgs(logits.ptr, best.ptr, None, None, 1, 100, 100))
         assert int(best.read(np.int32, 1)[0]) == winner
+
+
+def test_stamps_time_work_that_was_launched_without_a_wait(ctx):
+    """shv_stamp / shv_stamp_elapsed: the GPU time between two points of the stream, for passes handed over with
+    shv_prerecorded_launch.  More work between the stamps takes longer; a stamp that was never made, a number out of
+    range and stamps the stream has not reached yet are refused."""
+    pos = ctx.alloc(16).zero()
+    op = A.make_op(A.OP_ADVANCE, A.AdvanceArgs(pos.ptr, 1, 1))
+    one, many = ctx.prerecord([op]), ctx.prerecord([op] * 200)
+    with pytest.raises(A.ShvError):
+        ctx.stamp(4)
+    with pytest.raises(A.ShvError, match="never made"):
+        ctx.stamp_elapsed(2, 3)
+    ctx.stamp(0)
+    one.launch()
+    ctx.stamp(1)
+    many.launch()
+    ctx.stamp(2)
+    ctx.sync()
+    short, long_ = ctx.stamp_elapsed(0, 1), ctx.stamp_elapsed(1, 2)
+    assert 0 < short < long_ and long_ > 100_000, (short, long_)      # 200 dependent launches: hundreds of microseconds
+    assert int(pos.read(np.int32, 1)[0]) == 201
+    one.destroy()
+    many.destroy()
