@@ -499,8 +499,9 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
         // the group's bytes are here: only now the loads that nothing in this slab waits for (a
         // wait for loaded registers also waits for every load issued before them)
         asm volatile("" : "+v"(q[0].x), "+v"(q[1].x), "+v"(q[2].x), "+v"(q[3].x));
-        if (gi == 0) ask_next();
+        // the next group's bytes first: a wait for them then does not wait for the slab's loads behind them
         st.ask_group(rp, G + 1, G_last, kb);
+        if (gi == 0) ask_next();
         __builtin_amdgcn_sched_barrier(0);  // the loads stay up here, a group ahead of their use
         uint32_t sc[R];
 #pragma unroll
