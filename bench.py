@@ -679,6 +679,9 @@ def main():
         rounds = min(a.mtp_rounds, (len(plain) - 4) // 3)
         if rounds >= 1:
             rec["mtp"] = mtp_run(m, cfg, prompt, plain, acc, rounds)
+            # the recorded 3-row verification pass against the recorded one-row step, both as the GPU's clock has them
+            # (pass_N_rows_in_steps above are sums of per-kernel times of passes dispatched op by op)
+            rec["mtp"]["verify_pass_in_steps"] = round(rec["mtp"]["true_continuation_as_drafts"]["verify_gpu_ms_per_round"] / rec["gpu_ms_per_step"], 3)
     if not a.no_mtp and a.batch_slots >= 2:
         rec["batched_decode"] = batched_run(m, cfg, a.batch_slots, rng)
     cores = min(os.cpu_count() or 1, 16)
