@@ -116,7 +116,10 @@ def test_concurrent_is_solo(rig):
         both = drive(s, [Conv(s, B, p, n) for p in prompts])
         c = s.counts()
         assert c["batches"] > 0, "no decode step shared a pass, so the comparison says nothing about batching"
-        assert c["batch_rows"] / c["batches"] > 2.0
+        # (whether the long prompt is through before the short requests end, so that passes of three rows occur, is
+        # the policy's fair share of MEASURED time and changes with what a pass costs: the reference logs the figure,
+        # backend/llm_sched_test.go:124-128; three-row passes are held to the sequences in tests/test_rows_gpu.py)
+        assert c["batch_rows"] / c["batches"] >= 2.0
         for k in range(3):
             assert both[k].reused == 0
             agreed = same_until_a_tie(both[k], solo[k])
