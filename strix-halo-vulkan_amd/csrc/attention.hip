@@ -127,9 +127,12 @@ struct Smem {
 };
 
 // grid: (n_splits, n_head_kv, n_seq * n_groups); group g of a sequence is its rows row0 + R*g ..
-// row0 + R*g + R-1.  With append the launch also writes its rows' cells (one group only: a later
-// group would read cells another block is still writing); without, the cells are there already
-// and any number of groups go in one launch, each masked to its own positions.  Query row r of the
+// row0 + R*g + R-1.  With append the launch also writes its rows' cells; without, the cells are there
+// already and any number of groups go in one launch, each masked to its own positions.  A later group
+// reads the cells of the rows before it, which another block may still be writing: append 1 is for
+// one group; with append 2 (two groups: three or four rows) a block of the second group writes the
+// first group's cells in its slice as well, the same bytes the first group's block writes there, so
+// that it reads only what it has written itself.  Query row r of the
 // tile is head r%8 of sequence row r/8; with R = 1 rows 8..15 are padding.
 // QSA: a.mask names, a bit a cell, the cells each row may read (the block-sparse indexer's
 // selection, llm/attn.go:423-443); a tile none of the wave's rows may read is not loaded at all.
@@ -172,6 +175,17 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
         }
         kv[j] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD + 4 * lane_);
         vv[j] = qkv[static_cast<size_t>(a.n_head) * 2 * kD + a.n_head_kv * kD + kvh * kD + tid_];
+    }
+    // append 2: the rows of the pass before this group's (at most kForeign), whose cells this block writes too
+    constexpr int kForeign = 2;
+    const int n_foreign = append == 2 ? row0 - row00 : 0;
+    float4 kvf[kForeign];
+    float vvf[kForeign];
+#pragma unroll
+    for (int f = 0; f < kForeign; f++) {
+        const float *qkv = a.qkv + static_cast<size_t>(seq * a.seq_len + row00 + (f < n_foreign ? f : 0)) * a.qkv_stride;
+        kvf[f] = *reinterpret_cast<const float4 *>(qkv + static_cast<size_t>(a.n_head) * 2 * kD + kvh * kD + 4 * lane_);
+        vvf[f] = qkv[static_cast<size_t>(a.n_head) * 2 * kD + a.n_head_kv * kD + kvh * kD + tid_];
     }
     const float4 gq = *reinterpret_cast<const float4 *>(a.q_norm + 4 * lane_), gk = *reinterpret_cast<const float4 *>(a.k_norm + 4 * lane_);
     const int p_first = pos_first + row0;  // position of the group's first row
@@ -243,8 +257,20 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
     // branch the compiler no longer knows how many loads are in flight and waits for all of them
     // where it needs an earlier one: a wave that has both a tile and heads to prepare waits for
     // the tile before it prepares them.  In a slice of one tile no wave has both.)
+    float4 csf[kForeign], snf[kForeign];
+    bool appf[kForeign];
+#pragma unroll
+    for (int f = 0; f < kForeign; f++) {
+        const int p = pos_first + row00 + (f < n_foreign ? f : 0);
+        const float *rope_row = a.rope_dims > 0 ? a.rope + static_cast<size_t>(p) * a.rope_dims : a.q_norm;
+        appf[f] = f < n_foreign && p >= c0 && p < c1;
+        const int rl = rstep > 0 ? 4 * (lane & (rstep - 1)) : 0;
+        csf[f] = *reinterpret_cast<const float4 *>(rope_row + rl);
+        snf[f] = *reinterpret_cast<const float4 *>(rope_row + (a.rope_dims >> 1) + rl);
+    }
     const int t_first = c0 + kTile * wave;
-    const bool early = !QSA && t_first < c1 && t_first + kTile <= p_first;
+    // (the first position any block of this pass may be writing is the pass's first row's)
+    const bool early = !QSA && t_first < c1 && t_first + kTile <= p_first - n_foreign;
     if (early) load_tile(ta, t_first);
     // the lane's query row is sequence row n / 8: its mask words
     const uint32_t *mrow = nullptr;
@@ -289,6 +315,22 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
             vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vv[j]));
         }
     }
+#pragma unroll
+    for (int f = 0; f < kForeign; f++) {
+        if (appf[f]) {
+            const int p = pos_first + row00 + f;
+            if (wave == ((2 * f + 1) & 3)) {
+                float k0, k1, k2, k3;
+                norm_rope_regs(kvf[f], gk, csf[f], snf[f], a.rope_dims, a.eps, lane, k0, k1, k2, k3);
+                const __half2 k01 = __floats2half2_rn(k0, k1), k23 = __floats2half2_rn(k2, k3);
+                uint2 packed;
+                packed.x = *reinterpret_cast<const uint32_t *>(&k01);
+                packed.y = *reinterpret_cast<const uint32_t *>(&k23);
+                *reinterpret_cast<uint2 *>(kc + static_cast<size_t>(p) * kvw + 4 * lane) = packed;
+            }
+            vt[static_cast<size_t>(p / kTile) * vtile + tid * kTile + p % kTile] = __half_as_ushort(__float2half_rn(vvf[f]));
+        }
+    }
     if (R == 1) {
         // rows 8..15 of the tile are padding: zero operands (entries of lane ln with ln%16 >= 8)
 #pragma unroll
@@ -307,6 +349,8 @@ __global__ __launch_bounds__(kBlock, 1) void attn_decode_kernel(shv_attn_decode_
     bool appended = false;
 #pragma unroll
     for (int j = 0; j < R; j++) appended = appended || app[j];
+#pragma unroll
+    for (int f = 0; f < kForeign; f++) appended = appended || appf[f];
     if (appended) __threadfence_block();
     __syncthreads();
 
@@ -947,6 +991,8 @@ int shv_launch_attn_decode(shv_ctx *ctx, const shv_attn_decode_args *pa) {
     if (a.seq_len <= 2) return a.seq_len == 2 ? launch_rows<2>(ctx, a, 0, 1, 1) : launch_rows<1>(ctx, a, 0, 1, 1);
     const int pairs = (a.seq_len + 1) / 2;
     SHV_REQUIRE(static_cast<long long>(a.n_seq) * pairs <= 65535, "attn_decode: %d sequences of %d rows in one call", a.n_seq, a.seq_len);
+    // three or four rows (a verification pass): the second pair's blocks write the first pair's cells too, no launch for them
+    if (pairs == 2 && !ctx->attn_append_launch) return launch_rows<2>(ctx, a, 0, pairs, 2);
     SHV_LAUNCH(ctx, attn_append_kernel, dim3(a.n_head_kv, a.seq_len, a.n_seq), dim3(kBlock), 0, a);
     return launch_rows<2>(ctx, a, 0, pairs, 0);
 }

@@ -125,7 +125,11 @@ def test_decode_steps_from_an_empty_cache(ctx):
         assert np.count_nonzero(got != want) <= got.size // 20
 
 
-@pytest.mark.parametrize("past,rows,n_splits", [(0, 2, 4), (0, 5, 4), (61, 4, 8), (300, 3, 16), (4000, 2, 64)])
+@pytest.mark.parametrize("past,rows,n_splits", [(0, 2, 4), (0, 5, 4), (61, 4, 8), (300, 3, 16), (4000, 2, 64),
+                                                # three and four rows write their cells inside the launch, the second pair's
+                                                # blocks the first pair's too: new cells on either side of a slice's and of
+                                                # a tile's boundary, in the first tile, deep in a long cache
+                                                (127, 4, 8), (126, 3, 8), (31, 4, 4), (255, 3, 16), (0, 3, 4), (1, 4, 4), (2046, 4, 64)])
 def test_rows_of_one_sequence_in_one_call(ctx, past, rows, n_splits):
     """A verification pass or a prompt chunk: `rows` consecutive rows appended in one call, each
     seeing the cells up to its own (the cache is walked once for two rows at a time), against the
