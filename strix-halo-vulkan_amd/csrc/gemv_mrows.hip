@@ -70,24 +70,49 @@ __device__ __forceinline__ half8_t weights8(uint32_t d0, uint32_t d1, half2_t sc
     return r;
 }
 
-// K columns, NT activation rows, prologue PRO.  grid: n / 16 blocks of 256 threads.
-// Fragment f of a wave's quarter (KW = K/4 columns, NF = KW/8 fragments) is eight consecutive
-// columns: f = ((s * 2 + L) * 4 + m) * 4 + jj  with s the super-block within the quarter, L the
+// the largest of the values, none negative, of the lane's half of the wave (lanes 0..31, 32..63), in every lane of the half
+__device__ __forceinline__ float half_max_nonneg(float v, int lane) {
+    v = fmaxf(v, dpp_f32<kDppXor1>(v));
+    v = fmaxf(v, dpp_f32<kDppXor2>(v));
+    v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f32<kDppMirror>(v));
+    v = fmaxf(v, dpp_f32<kDppBcast15, 0xA>(v));
+    const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 31)), hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+    return lane < 32 ? lo : hi;
+}
+__device__ __forceinline__ float half_sum(float v, int lane) {
+    v = group_sum<32>(v);
+    const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 31)), hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+    return lane < 32 ? lo : hi;
+}
+
+// K columns, NT activation rows, prologue PRO, W waves a block.  grid: n / (16 TILES) blocks of 64 W threads.
+// Fragment f of a wave's part (KW = K/W columns, NF = KW/8 fragments) is eight consecutive
+// columns: f = ((s * 2 + L) * 4 + m) * 4 + jj  with s the super-block within the part, L the
 // half of the super-block (64-weight groups 2L, 2L+1), m the product within a lane's 16 payload
 // bytes (0, 1: low nibbles of bytes 0..7 / 8..15; 2, 3: the high nibbles) and jj the operand's
 // column group (lane / 16): columns  256 s' + 64 (2L + jj/2) + 32 (m/2) + 16 (jj%2) + 8 (m%2) ..+7.
-template <int K, int PRO, int NT, int TILES>
-__global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
-    constexpr int KW = K / 4, NSB = KW / 256, NF = KW / 8, FPL = NF / 64, NC = 2 * NT, FS = NC | 1;
+// What a block pays per activation row is the staging, which every block repeats: W says over how many waves a row's
+// columns are spread.  Four waves suit two to four rows; with sixteen waves over 4096 columns a wave stages one
+// super-block of each row, 32 fragments, and two rows share the wave's lanes; the launcher says where that pays.
+template <int K, int PRO, int NT, int TILES, int W>
+__global__ __launch_bounds__(64 * W) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
+    constexpr int KW = K / W, NSB = KW / 256, NF = KW / 8, NC = 2 * NT, FS = NC | 1;
+    constexpr bool HALF = NF < 64;                 // two activation rows side by side in a wave's lanes
+    constexpr int FPL = HALF ? 1 : NF / 64;        // fragments of one row a lane stages
+    constexpr int PPL = HALF ? (NT + 1) / 2 : NT * FPL;  // (row, fragment) pairs a lane stages
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
-    static_assert(NSB >= 1 && FPL >= 1 && NT >= 2 && NT <= 8, "shape");
+    static_assert(NSB >= 1 && (NF == 32 || NF % 64 == 0) && NT >= 2 && NT <= 8, "shape");
+    static_assert(W == 4 || TILES == 1, "the tiles' partial results take the operands' place in LDS only when there is one tile");
     extern __shared__ __align__(16) char smem[];
     // a fragment's columns lie FS entries of 16 bytes apart, an odd number: sixteen lanes that store one column of
     // sixteen consecutive fragments then hit sixteen different groups of four banks
-    half8_t *bf_all = reinterpret_cast<half8_t *>(smem);                                  // [4 waves][NF][FS]
-    half4_t *sf_all = reinterpret_cast<half4_t *>(smem + sizeof(half8_t) * 4 * NF * FS);  // [4 waves][NSB][4][NC]
-    float *cpart = reinterpret_cast<float *>(smem + sizeof(half8_t) * 4 * NF * FS + sizeof(half4_t) * 4 * NSB * 4 * NC);  // [TILES][4][64][4]
-    float *red = cpart + TILES * 4 * 64 * 4;                                              // [NT][4]
+    half8_t *bf_all = reinterpret_cast<half8_t *>(smem);                                  // [W waves][NF][FS]
+    half4_t *sf_all = reinterpret_cast<half4_t *>(smem + sizeof(half8_t) * W * NF * FS);  // [W waves][NSB][4][NC]
+    float *red = reinterpret_cast<float *>(smem + sizeof(half8_t) * W * NF * FS + sizeof(half4_t) * W * NSB * 4 * NC);  // [NT][W]
+    float *uns = red + NT * W;                                                            // [W][NT]
+    // the waves' partial tiles: behind everything with four waves, over the operands (read to their end by then) with more
+    float *cpart = W == 4 ? uns + W * NT : reinterpret_cast<float *>(smem);               // [TILES][W][64][4]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, j = lane >> 4;
     half8_t *bf = bf_all + wave * NF * FS;
@@ -106,15 +131,19 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
             ring_row[t] = slot * a.ring_slots + (p + i) % a.ring_slots;
         }
     }
-    // ---- the wave's quarter of every activation row, a fragment (eight columns) a lane ----
-    float4 xv[NT][FPL][2], zv[NT][FPL][2], gv[FPL][2];
-    int fcol[FPL];
+    // ---- the wave's part of every activation row: pair u of a lane is (row pt[u], fragment pf[u]) ----
+    float4 xv[PPL][2], zv[PPL][2], gv[PPL][2];
+    int pt[PPL], pf[PPL];
+    bool pv[PPL];
 #pragma unroll
-    for (int u = 0; u < FPL; u++) {
-        const int f = lane + 64 * u;
+    for (int u = 0; u < PPL; u++) {
+        const int t_raw = HALF ? 2 * u + (lane >> 5) : u / FPL;
+        pv[u] = t_raw < NT;
+        pt[u] = pv[u] ? t_raw : NT - 1;
+        pf[u] = HALF ? (lane & 31) : lane + 64 * (u % FPL);
+        const int f = pf[u], t = pt[u];
         const int jj = f & 3, m = (f >> 2) & 3, L = (f >> 4) & 1, s = f >> 5;
-        fcol[u] = wave * KW + 256 * s + 64 * (2 * L + (jj >> 1)) + 32 * (m >> 1) + 16 * (jj & 1) + 8 * (m & 1);
-        const int c = fcol[u];
+        const int c = wave * KW + 256 * s + 64 * (2 * L + (jj >> 1)) + 32 * (m >> 1) + 16 * (jj & 1) + 8 * (m & 1);
         if constexpr (PRO == SHV_PRO_RMSNORM) {
             gv[u][0] = *reinterpret_cast<const float4 *>(a.gamma + c);
             gv[u][1] = *reinterpret_cast<const float4 *>(a.gamma + c + 4);
@@ -122,22 +151,23 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
             gv[u][0] = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)));
             gv[u][1] = *reinterpret_cast<const float4 *>(a.gamma + (c & (a.head_dim - 1)) + 4);
         }
+        const float *x = a.x + static_cast<size_t>(t) * a.x_stride + c;
+        xv[u][0] = *reinterpret_cast<const float4 *>(x);
+        xv[u][1] = *reinterpret_cast<const float4 *>(x + 4);
+        if constexpr (PRO == SHV_PRO_GATED_NORM) {
+            // the lane's row of the ring, picked without indexing the register array by a variable
+            int rr = 0;
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const float *x = a.x + static_cast<size_t>(t) * a.x_stride + c;
-            xv[t][u][0] = *reinterpret_cast<const float4 *>(x);
-            xv[t][u][1] = *reinterpret_cast<const float4 *>(x + 4);
-            if constexpr (PRO == SHV_PRO_GATED_NORM) {
-                const float *z = a.z_ring ? a.z + static_cast<size_t>(ring_row[t]) * a.ring_stride : a.z + static_cast<size_t>(t) * a.z_stride;
-                zv[t][u][0] = *reinterpret_cast<const float4 *>(z + c);
-                zv[t][u][1] = *reinterpret_cast<const float4 *>(z + c + 4);
-            } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
-                const HeadSplit hs(a.head_dim > 0 ? a.head_dim : 1);
-                const int zi = a.head_dim > 0 ? hs.head(c) * 2 * a.head_dim + a.head_dim + hs.dim(c) : c;
-                const float *z = a.z + static_cast<size_t>(t) * a.z_stride + zi;
-                zv[t][u][0] = *reinterpret_cast<const float4 *>(z);
-                zv[t][u][1] = *reinterpret_cast<const float4 *>(z + 4);
-            }
+            for (int tt = 0; tt < NT; tt++) rr = tt == t ? ring_row[tt] : rr;
+            const float *z = a.z_ring ? a.z + static_cast<size_t>(rr) * a.ring_stride : a.z + static_cast<size_t>(t) * a.z_stride;
+            zv[u][0] = *reinterpret_cast<const float4 *>(z + c);
+            zv[u][1] = *reinterpret_cast<const float4 *>(z + c + 4);
+        } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+            const HeadSplit hs(a.head_dim > 0 ? a.head_dim : 1);
+            const int zi = a.head_dim > 0 ? hs.head(c) * 2 * a.head_dim + a.head_dim + hs.dim(c) : c;
+            const float *z = a.z + static_cast<size_t>(t) * a.z_stride + zi;
+            zv[u][0] = *reinterpret_cast<const float4 *>(z);
+            zv[u][1] = *reinterpret_cast<const float4 *>(z + 4);
         }
     }
     // ---- the wave's weights, of every tile of the block: per super-block the row's header and this lane's 2 x 16
@@ -164,70 +194,88 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
         res[ti] = (a.residual && out_t < NT && out_row < a.n) ? a.residual[static_cast<size_t>(out_t) * a.y_stride + out_row] : 0.f;
     }
 
-    // ---- stage: prologue, a power of two that brings the wave's quarter of the row into binary16's range, operand
+    // ---- stage: prologue, a power of two that brings the wave's part of the row into binary16's range, operand
     // order, the sub-blocks' sums ----
-    float unscale[NT];
+    float v[PPL][8], ssq[PPL], mxp[PPL];
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        float ss = 0.f, mx = 0.f;
-        float v[FPL][8];
+    for (int u = 0; u < PPL; u++) {
+        const float x8[8] = {xv[u][0].x, xv[u][0].y, xv[u][0].z, xv[u][0].w, xv[u][1].x, xv[u][1].y, xv[u][1].z, xv[u][1].w};
 #pragma unroll
-        for (int u = 0; u < FPL; u++) {
-            const float x8[8] = {xv[t][u][0].x, xv[t][u][0].y, xv[t][u][0].z, xv[t][u][0].w, xv[t][u][1].x, xv[t][u][1].y, xv[t][u][1].z, xv[t][u][1].w};
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[u][i] = x8[i];
-            if constexpr (PRO == SHV_PRO_RMSNORM) {
-                const float g[8] = {gv[u][0].x, gv[u][0].y, gv[u][0].z, gv[u][0].w, gv[u][1].x, gv[u][1].y, gv[u][1].z, gv[u][1].w};
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    ss = fmaf(v[u][i], v[u][i], ss);
-                    v[u][i] *= g[i];
-                }
-            } else if constexpr (PRO == SHV_PRO_GATED_NORM) {
-                // a head of 128 columns is sixteen consecutive fragments: the sixteen lanes of a row of the wave
-                const float g[8] = {gv[u][0].x, gv[u][0].y, gv[u][0].z, gv[u][0].w, gv[u][1].x, gv[u][1].y, gv[u][1].z, gv[u][1].w};
-                const float z[8] = {zv[t][u][0].x, zv[t][u][0].y, zv[t][u][0].z, zv[t][u][0].w, zv[t][u][1].x, zv[t][u][1].y, zv[t][u][1].z, zv[t][u][1].w};
-                float hs = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; i++) hs = fmaf(v[u][i], v[u][i], hs);
-                hs = group_sum<16>(hs);
-                const float sc = __builtin_amdgcn_rsqf(hs / 128.f + a.eps);
-#pragma unroll
-                for (int i = 0; i < 8; i++) v[u][i] = v[u][i] * sc * g[i] * sigmoid_fast(z[i]);
-            } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
-                const float z[8] = {zv[t][u][0].x, zv[t][u][0].y, zv[t][u][0].z, zv[t][u][0].w, zv[t][u][1].x, zv[t][u][1].y, zv[t][u][1].z, zv[t][u][1].w};
-#pragma unroll
-                for (int i = 0; i < 8; i++) v[u][i] *= sigmoid_fast(z[i]);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; i++) mx = fmaxf(mx, fabsf(v[u][i]));
-        }
-        // the largest magnitude of the quarter goes to [512, 1024): a sub-block's sum stays below binary16's limit,
-        // and what is smaller than the largest by 2^-23 and more loses bits that the sum would not show anyway
-        mx = wave_max_nonneg(mx);
-        int ex = static_cast<int>((__float_as_uint(mx) >> 23) & 0xFFu);
-        ex = ex < 9 ? 9 : ex > 254 ? 254 : ex;
-        const float up = __uint_as_float(static_cast<uint32_t>(263 - ex) << 23);  // 2^(136 - ex)
-        unscale[t] = __uint_as_float(static_cast<uint32_t>(ex - 9) << 23);          // its inverse (0 below 2^-118)
-#pragma unroll
-        for (int u = 0; u < FPL; u++) {
-            float h8[8], l8[8], s8 = 0.f;
+        for (int i = 0; i < 8; i++) v[u][i] = x8[i];
+        ssq[u] = 0.f;
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            const float g[8] = {gv[u][0].x, gv[u][0].y, gv[u][0].z, gv[u][0].w, gv[u][1].x, gv[u][1].y, gv[u][1].z, gv[u][1].w};
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const float vs = v[u][i] * up;
-                split_cut(vs, h8[i], l8[i]);
-                s8 += vs;
+                ssq[u] = fmaf(v[u][i], v[u][i], ssq[u]);
+                v[u][i] *= g[i];
             }
-            // operand order within a fragment: the order a payload dword's nibbles come out of the masks (bytes 0, 2, 1, 3)
-            const uint4 hw = make_uint4(pack_halves(h8[0], h8[2]), pack_halves(h8[1], h8[3]), pack_halves(h8[4], h8[6]), pack_halves(h8[5], h8[7]));
-            const uint4 lw = make_uint4(pack_halves(l8[0], l8[2]), pack_halves(l8[1], l8[3]), pack_halves(l8[4], l8[6]), pack_halves(l8[5], l8[7]));
-            const half8_t hi = __builtin_bit_cast(half8_t, hw), lo = __builtin_bit_cast(half8_t, lw);
-            const int f = lane + 64 * u;
+        } else if constexpr (PRO == SHV_PRO_GATED_NORM) {
+            // a head of 128 columns is sixteen consecutive fragments: the sixteen lanes of a row of the wave
+            const float g[8] = {gv[u][0].x, gv[u][0].y, gv[u][0].z, gv[u][0].w, gv[u][1].x, gv[u][1].y, gv[u][1].z, gv[u][1].w};
+            const float z[8] = {zv[u][0].x, zv[u][0].y, zv[u][0].z, zv[u][0].w, zv[u][1].x, zv[u][1].y, zv[u][1].z, zv[u][1].w};
+            float hs = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) hs = fmaf(v[u][i], v[u][i], hs);
+            hs = group_sum<16>(hs);
+            const float sc = __builtin_amdgcn_rsqf(hs / 128.f + a.eps);
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[u][i] = v[u][i] * sc * g[i] * sigmoid_fast(z[i]);
+        } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
+            const float z[8] = {zv[u][0].x, zv[u][0].y, zv[u][0].z, zv[u][0].w, zv[u][1].x, zv[u][1].y, zv[u][1].z, zv[u][1].w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[u][i] *= sigmoid_fast(z[i]);
+        }
+        mxp[u] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) mxp[u] = fmaxf(mxp[u], fabsf(v[u][i]));
+    }
+    // per activation row: the largest magnitude of the wave's part goes to [512, 1024): a sub-block's sum stays below
+    // binary16's limit, and what is smaller than the largest by 2^-23 and more loses bits that the sum would not show
+    float up[PPL];
+#pragma unroll
+    for (int g0 = 0; g0 < PPL; g0 += FPL) {
+        // the pairs g0 .. g0 + FPL - 1 are one row's (of each half of the wave, when two rows share it)
+        float mx = 0.f, ss = 0.f;
+#pragma unroll
+        for (int u = g0; u < g0 + FPL; u++) {
+            mx = fmaxf(mx, mxp[u]);
+            ss += ssq[u];
+        }
+        mx = HALF ? half_max_nonneg(mx, lane) : wave_max_nonneg(mx);
+        int ex = static_cast<int>((__float_as_uint(mx) >> 23) & 0xFFu);
+        ex = ex < 9 ? 9 : ex > 254 ? 254 : ex;
+        const float upv = __uint_as_float(static_cast<uint32_t>(263 - ex) << 23);      // 2^(136 - ex)
+        const float unscale = __uint_as_float(static_cast<uint32_t>(ex - 9) << 23);    // its inverse (0 below 2^-118)
+#pragma unroll
+        for (int u = g0; u < g0 + FPL; u++) up[u] = upv;
+        const bool writer = (lane & (HALF ? 31 : 63)) == 0 && pv[g0];
+        if (writer) uns[wave * NT + pt[g0]] = unscale;
+        if constexpr (PRO == SHV_PRO_RMSNORM) {
+            ss = HALF ? half_sum(ss, lane) : wave_sum_all(ss);
+            if (writer) red[pt[g0] * W + wave] = ss;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < PPL; u++) {
+        const int f = pf[u], t = pt[u];
+        float h8[8], l8[8], s8 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float vs = v[u][i] * up[u];
+            split_cut(vs, h8[i], l8[i]);
+            s8 += vs;
+        }
+        // operand order within a fragment: the order a payload dword's nibbles come out of the masks (bytes 0, 2, 1, 3)
+        const uint4 hw = make_uint4(pack_halves(h8[0], h8[2]), pack_halves(h8[1], h8[3]), pack_halves(h8[4], h8[6]), pack_halves(h8[5], h8[7]));
+        const uint4 lw = make_uint4(pack_halves(l8[0], l8[2]), pack_halves(l8[1], l8[3]), pack_halves(l8[4], l8[6]), pack_halves(l8[5], l8[7]));
+        const half8_t hi = __builtin_bit_cast(half8_t, hw), lo = __builtin_bit_cast(half8_t, lw);
+        // the sub-block's 32 columns are the fragments f, f ^ 1 (jj % 2) and f ^ 4, f ^ 5 (m % 2): lanes of one half
+        float s32 = s8 + dpp_f32<kDppXor1>(s8);
+        s32 += __shfl_xor(s32, 4, 64);
+        if (pv[u]) {
             bf[f * FS + 2 * t] = hi;
             bf[f * FS + 2 * t + 1] = lo;
-            // the sub-block's 32 columns are the fragments f, f ^ 1 (jj % 2) and f ^ 4, f ^ 5 (m % 2)
-            float s32 = s8 + dpp_f32<kDppXor1>(s8);
-            s32 += __shfl_xor(s32, 4, 64);
             if ((f & 5) == 0) {
                 const int jj = f & 3, m = (f >> 2) & 3, L = (f >> 4) & 1, s = f >> 5;
                 const int grp = 2 * L + (jj >> 1), odd = m >> 1;  // sub-block 2 grp + odd of the super-block
@@ -240,19 +288,14 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
                 *dst_lo = pack_halves(sl, 0.f);
             }
         }
-        if constexpr (PRO == SHV_PRO_RMSNORM) {
-            ss = wave_sum_all(ss);
-            if (lane == 0) red[t * 4 + wave] = ss;
-        }
     }
     __builtin_amdgcn_wave_barrier();  // a wave reads back only what it staged itself; its LDS operations complete in order
 
     // ---- products ----
     const int bc = r < NC ? r : NC - 1;  // columns past the rows' hold whatever: their results are never read
     // a lane's column: activation row r / 2 (its high parts in the even column, the remainders in the odd one)
-    float back = 0.f;
-#pragma unroll
-    for (int t = 0; t < NT; t++) back = (r >> 1) == t ? unscale[t] : back;
+    const float back = (r >> 1) < NT ? uns[wave * NT + (r >> 1)] : 0.f;
+    float4_t ytile[TILES];
 #pragma unroll
     for (int ti = 0; ti < TILES; ti++) {
     float4_t yacc = {0.f, 0.f, 0.f, 0.f};
@@ -299,15 +342,21 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
             yacc[i] = fmaf(-f16_bits_to_f32(dd >> 16), cmin[i], yacc[i]);
         }
     }
-#pragma unroll
-    for (int i = 0; i < 4; i++) cpart[((ti * 4 + wave) * 64 + lane) * 4 + i] = yacc[i] * back;
+    ytile[ti] = yacc * back;
     }
-    // ---- the four waves' tiles meet; thread (row, activation row) adds its two columns of each ----
+    if constexpr (W != 4) __syncthreads();  // every wave has read its operands to the end: the partial tiles take their place
+#pragma unroll
+    for (int ti = 0; ti < TILES; ti++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) cpart[((ti * W + wave) * 64 + lane) * 4 + i] = ytile[ti][i];
+    // ---- the waves' tiles meet; thread (row, activation row) adds its two columns of each ----
     __syncthreads();
     if (out_t < NT) {
         float scale = 1.f;
         if constexpr (PRO == SHV_PRO_RMSNORM) {
-            const float tot = (red[out_t * 4 + 0] + red[out_t * 4 + 1]) + (red[out_t * 4 + 2] + red[out_t * 4 + 3]);
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < W; w++) tot += red[out_t * W + w];
             scale = __builtin_amdgcn_rsqf(tot / static_cast<float>(K) + a.eps);
         }
         // ring_row of this thread's activation row: picked without indexing the register array by a variable
@@ -320,8 +369,8 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
             const int out_row = (static_cast<int>(blockIdx.x) * TILES + ti) * 16 + out_r;
             float y = 0.f;
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const float *cp = cpart + ((ti * 4 + w) * 64 + 16 * (out_r >> 2)) * 4 + (out_r & 3);
+            for (int w = 0; w < W; w++) {
+                const float *cp = cpart + ((ti * W + w) * 64 + 16 * (out_r >> 2)) * 4 + (out_r & 3);
                 y += cp[(2 * out_t) * 4] + cp[(2 * out_t + 1) * 4];
             }
             if (out_row < a.n) dst[out_row] = fmaf(y, scale, res[ti]);
@@ -329,23 +378,24 @@ __global__ __launch_bounds__(256) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
     }
 }
 
-template <int K, int NT, int TILES>
+template <int K, int NT, int TILES, int W>
 size_t mrows_lds() {
-    constexpr int KW = K / 4, NSB = KW / 256, NF = KW / 8, NC = 2 * NT, FS = NC | 1;
-    return sizeof(half8_t) * 4 * NF * FS + sizeof(half4_t) * 4 * NSB * 4 * NC + sizeof(float) * (TILES * 4 * 64 * 4 + NT * 4);
+    constexpr int KW = K / W, NSB = KW / 256, NF = KW / 8, NC = 2 * NT, FS = NC | 1;
+    return sizeof(half8_t) * W * NF * FS + sizeof(half4_t) * W * NSB * 4 * NC + sizeof(float) * (2 * NT * W + (W == 4 ? TILES * W * 64 * 4 : 0));
 }
 
-template <int K, int PRO, int NT, int TILES>
+template <int K, int PRO, int NT, int TILES, int W = 4>
 int launch_tiles(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
-    const size_t lds = mrows_lds<K, NT, TILES>();
+    const size_t lds = mrows_lds<K, NT, TILES, W>();
+    static_assert(W == 4 || sizeof(half8_t) * (K / 8) * ((2 * NT) | 1) >= sizeof(float) * TILES * W * 64 * 4, "the partial tiles fit where the operands were");
     if (lds > 48 * 1024) {
         static std::atomic<bool> raised{false};  // above the default allowance the limit is raised once per kernel
         if (!raised.load(std::memory_order_acquire)) {
-            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mrows_kernel<K, PRO, NT, TILES>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mrows_kernel<K, PRO, NT, TILES, W>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
             raised.store(true, std::memory_order_release);
         }
     }
-    SHV_LAUNCH(ctx, (gemv_mrows_kernel<K, PRO, NT, TILES>), dim3((a.n + 16 * TILES - 1) / (16 * TILES)), dim3(256), lds, a);
+    SHV_LAUNCH(ctx, (gemv_mrows_kernel<K, PRO, NT, TILES, W>), dim3((a.n + 16 * TILES - 1) / (16 * TILES)), dim3(64 * W), lds, a);
     return SHV_OK;
 }
 
@@ -354,9 +404,17 @@ int launch_tiles(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
 // over chains of distinct matrices (us a launch, tiles a block 1 / 2 / 4):
 //   12352 x 2048, 772 tiles   3 rows 9.2 / 9.3 / 10.1    6 rows 13.0 / 11.2 / 11.9    8 rows 15.5 / 16.0 / 12.8
 //   151936 x 2048, 9496 tiles 2 rows 56 / 48 / 52        3 rows 74 / 59 / 59          4 rows 81 / 63 / 60
+// From five rows on the staging is what a launch takes, and a row's columns go over more waves (SHV_MROWS_WAVES=4
+// keeps four).
 template <int K, int PRO, int NT>
 int launch_pro(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     const int tiles = (a.n + 15) / 16, cus = ctx->prop.multiProcessorCount;
+    if constexpr (NT >= 5 && K == 4096) {
+        // 2048 x 4096 at eight rows: 13.7 us on four waves, 10.2 on sixteen (a gated norm in front), 12.5 and 9.2 (a sigmoid
+        // gate).  2048 columns over eight waves, one super-block a wave there too, gained nothing: 12352 rows at eight
+        // rows 12.3 -> 13.3 us, 9216 rows 11.6 -> 10.9, and stay on four.
+        if (!ctx->mrows_four_waves && tiles < 8 * cus) return launch_tiles<K, PRO, NT, 1, 16>(ctx, a);
+    }
     if constexpr (K == 2048) {
         if (tiles >= 8 * cus) return NT >= 4 ? launch_tiles<K, PRO, NT, 4>(ctx, a) : launch_tiles<K, PRO, NT, 2>(ctx, a);
         if (NT >= 6 && tiles >= 2 * cus) return launch_tiles<K, PRO, NT, 4>(ctx, a);

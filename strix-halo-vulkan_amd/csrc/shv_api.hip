@@ -51,6 +51,7 @@ int shv_init(int device, shv_ctx **out) {
         if (v >= 0) ctx->gemm_rows_min = v;
     }
     if (const char *e = std::getenv("SHV_MROWS")) ctx->mrows_off = std::atoi(e) == 0;
+    if (const char *e = std::getenv("SHV_MROWS_WAVES")) ctx->mrows_four_waves = std::atoi(e) == 4;
     if (const char *e = std::getenv("SHV_ATTN_APPEND")) ctx->attn_append_launch = std::strcmp(e, "launch") == 0;
     if (const char *e = std::getenv("SHV_MOE_GROUP_MIN")) {
         const int v = std::atoi(e);

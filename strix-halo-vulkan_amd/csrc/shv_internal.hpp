@@ -34,6 +34,7 @@ struct shv_ctx {
     // SHV_MROWS=0: projections of two to eight rows go the ways they went before the kernel that forms each weight
     // once for all rows (the side-by-side row kernel up to four rows, the tiled matrix-core kernels above)
     bool mrows_off = false;
+    bool mrows_four_waves = false;  // SHV_MROWS_WAVES=4: five to eight rows stay on blocks of four waves
     // SHV_ATTN_APPEND=launch: passes of three and four rows write their new cells in a launch of their own, as longer ones do
     bool attn_append_launch = false;
     int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)

@@ -141,3 +141,50 @@ def test_two_sequences_and_more_write_their_own_ring_rows(ctx, rows):
     for t in range(rows):
         assert O.rel_l2(got[4, (6 + t) % slots_ring], want[t]) <= 1e-3, t
     assert np.count_nonzero(got.any(axis=2)) == rows
+
+
+# The output projections' prologues through this kernel (the library's own context; the tests of these names in
+# test_gemm_q4k_gpu.py run on a context that sends every pass to the tiled matrix-core kernels): five rows and more
+# of 4096 columns spread a row over sixteen waves, two rows to a wave's lanes.
+import test_gemm_q4k_gpu as G
+
+
+@pytest.mark.parametrize("rows,slots", [(2, 8), (5, 8), (6, 8), (7, 8), (8, 8)])
+def test_gated_norm_prologue_with_the_gate_from_the_ring(ctx, rows, slots):
+    G.test_gated_norm_prologue_with_ring_gate_and_wide_rows(ctx, rows, slots)
+
+
+@pytest.mark.parametrize("rows", [2, 5, 6, 7, 8])
+def test_sigmoid_gate_prologue(ctx, rows):
+    G.test_sigmoid_gate_prologue_with_fused_query_rows(ctx, rows)
+
+
+@pytest.mark.parametrize("rows", [5, 7, 8])
+def test_sixteen_waves_equal_four(ctx, rows):
+    """2048 x 4096 with the RMSNorm in front and a residual behind: the block of sixteen waves against the block of
+    four (SHV_MROWS_WAVES=4) to rounding, both against float64."""
+    os.environ["SHV_MROWS_WAVES"] = "4"
+    try:
+        four = A.Context(0)
+    finally:
+        del os.environ["SHV_MROWS_WAVES"]
+    try:
+        rng = np.random.default_rng(900 + rows)
+        n, k = 2048, 4096
+        wq = _weights(rng, n, k)
+        w64 = O.dequant_q4k(wq, k).astype(np.float64)
+        gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+        x = (rng.standard_normal((rows, k)) * 3).astype(np.float32)
+        res = rng.standard_normal((rows, n)).astype(np.float32)
+        outs = []
+        for c in (ctx, four):
+            dy = c.upload(res)
+            c.gemv_q4k(c.upload(wq), c.upload(x), dy, n, k, n_tok=rows, prologue=A.PRO_RMSNORM, gamma=c.upload(gamma), eps=1e-6, residual=dy)
+            outs.append(dy.read(np.float32, rows * n).reshape(rows, n))
+        x64 = x.astype(np.float64)
+        want = (x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-6) * gamma) @ w64.T + res
+        for t in range(rows):
+            assert O.rel_l2(outs[0][t], want[t]) <= 1e-5 and O.rel_l2(outs[1][t], want[t]) <= 1e-5, t
+            assert O.rel_l2(outs[0][t], outs[1][t]) <= 3e-6, t
+    finally:
+        four.destroy()
