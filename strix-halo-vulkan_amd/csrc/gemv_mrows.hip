@@ -93,8 +93,8 @@ __device__ __forceinline__ float half_sum(float v, int lane) {
 // bytes (0, 1: low nibbles of bytes 0..7 / 8..15; 2, 3: the high nibbles) and jj the operand's
 // column group (lane / 16): columns  256 s' + 64 (2L + jj/2) + 32 (m/2) + 16 (jj%2) + 8 (m%2) ..+7.
 // What a block pays per activation row is the staging, which every block repeats: W says over how many waves a row's
-// columns are spread.  Four waves suit two to four rows; with sixteen waves over 4096 columns a wave stages one
-// super-block of each row, 32 fragments, and two rows share the wave's lanes; the launcher says where that pays.
+// columns are spread.  Four waves suit two to four rows; with sixteen waves over 4096 columns (eight over 2048) a wave
+// stages one super-block of each row, 32 fragments, and two rows share the wave's lanes; the launcher says where that pays.
 template <int K, int PRO, int NT, int TILES, int W>
 __global__ __launch_bounds__(64 * W) void gemv_mrows_kernel(shv_gemv_q4k_args a) {
     constexpr int KW = K / W, NSB = KW / 256, NF = KW / 8, NC = 2 * NT, FS = NC | 1;
@@ -103,7 +103,6 @@ __global__ __launch_bounds__(64 * W) void gemv_mrows_kernel(shv_gemv_q4k_args a)
     constexpr int PPL = HALF ? (NT + 1) / 2 : NT * FPL;  // (row, fragment) pairs a lane stages
     constexpr int ROWB = K / SHV_Q4K_BLOCK * SHV_Q4K_BYTES;
     static_assert(NSB >= 1 && (NF == 32 || NF % 64 == 0) && NT >= 2 && NT <= 8, "shape");
-    static_assert(W == 4 || TILES == 1, "the tiles' partial results take the operands' place in LDS only when there is one tile");
     extern __shared__ __align__(16) char smem[];
     // a fragment's columns lie FS entries of 16 bytes apart, an odd number: sixteen lanes that store one column of
     // sixteen consecutive fragments then hit sixteen different groups of four banks
@@ -111,8 +110,10 @@ __global__ __launch_bounds__(64 * W) void gemv_mrows_kernel(shv_gemv_q4k_args a)
     half4_t *sf_all = reinterpret_cast<half4_t *>(smem + sizeof(half8_t) * W * NF * FS);  // [W waves][NSB][4][NC]
     float *red = reinterpret_cast<float *>(smem + sizeof(half8_t) * W * NF * FS + sizeof(half4_t) * W * NSB * 4 * NC);  // [NT][W]
     float *uns = red + NT * W;                                                            // [W][NT]
-    // the waves' partial tiles: behind everything with four waves, over the operands (read to their end by then) with more
-    float *cpart = W == 4 ? uns + W * NT : reinterpret_cast<float *>(smem);               // [TILES][W][64][4]
+    // the waves' partial tiles: behind everything with four waves, over the operands (read to their end by then) with
+    // more, where they fit there
+    constexpr bool ALIAS = W != 4 && sizeof(half8_t) * W * NF * FS >= sizeof(float) * TILES * W * 64 * 4;
+    float *cpart = ALIAS ? reinterpret_cast<float *>(smem) : uns + W * NT;                // [TILES][W][64][4]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, j = lane >> 4;
     half8_t *bf = bf_all + wave * NF * FS;
@@ -344,7 +345,7 @@ __global__ __launch_bounds__(64 * W) void gemv_mrows_kernel(shv_gemv_q4k_args a)
     }
     ytile[ti] = yacc * back;
     }
-    if constexpr (W != 4) __syncthreads();  // every wave has read its operands to the end: the partial tiles take their place
+    if constexpr (ALIAS) __syncthreads();  // every wave has read its operands to the end: the partial tiles take their place
 #pragma unroll
     for (int ti = 0; ti < TILES; ti++)
 #pragma unroll
@@ -381,13 +382,13 @@ __global__ __launch_bounds__(64 * W) void gemv_mrows_kernel(shv_gemv_q4k_args a)
 template <int K, int NT, int TILES, int W>
 size_t mrows_lds() {
     constexpr int KW = K / W, NSB = KW / 256, NF = KW / 8, NC = 2 * NT, FS = NC | 1;
-    return sizeof(half8_t) * W * NF * FS + sizeof(half4_t) * W * NSB * 4 * NC + sizeof(float) * (2 * NT * W + (W == 4 ? TILES * W * 64 * 4 : 0));
+    constexpr bool ALIAS = W != 4 && sizeof(half8_t) * W * NF * FS >= sizeof(float) * TILES * W * 64 * 4;
+    return sizeof(half8_t) * W * NF * FS + sizeof(half4_t) * W * NSB * 4 * NC + sizeof(float) * (2 * NT * W + (ALIAS ? 0 : TILES * W * 64 * 4));
 }
 
 template <int K, int PRO, int NT, int TILES, int W = 4>
 int launch_tiles(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     const size_t lds = mrows_lds<K, NT, TILES, W>();
-    static_assert(W == 4 || sizeof(half8_t) * (K / 8) * ((2 * NT) | 1) >= sizeof(float) * TILES * W * 64 * 4, "the partial tiles fit where the operands were");
     if (lds > 48 * 1024) {
         static std::atomic<bool> raised{false};  // above the default allowance the limit is raised once per kernel
         if (!raised.load(std::memory_order_acquire)) {
@@ -411,9 +412,19 @@ int launch_pro(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     const int tiles = (a.n + 15) / 16, cus = ctx->prop.multiProcessorCount;
     if constexpr (NT >= 5 && K == 4096) {
         // 2048 x 4096 at eight rows: 13.7 us on four waves, 10.2 on sixteen (a gated norm in front), 12.5 and 9.2 (a sigmoid
-        // gate).  2048 columns over eight waves, one super-block a wave there too, gained nothing: 12352 rows at eight
-        // rows 12.3 -> 13.3 us, 9216 rows 11.6 -> 10.9, and stay on four.
+        // gate).
         if (!ctx->mrows_four_waves && tiles < 8 * cus) return launch_tiles<K, PRO, NT, 1, 16>(ctx, a);
+    }
+    if constexpr (K == 2048 && NT >= 4) {
+        // 2048 columns over eight waves (a super-block of every row a wave) and several tiles a block, us a launch
+        // against the blocks of four waves below: 12352 rows at 8 / 5 / 4 rows 10.2 / 9.5 / 8.5 against 12.3 / 11.3 / 9.8,
+        // 9216 rows at 8 rows 10.0 against 11.6; at two and three rows nothing either way (8.0 and 8.5-8.9 against 8.1
+        // and 8.8) and four waves stay.
+        if (!ctx->mrows_four_waves && tiles < 8 * cus && (NT >= 5 || tiles >= 3 * cus)) {
+            if (tiles >= 2 * cus) return launch_tiles<K, PRO, NT, 4, 8>(ctx, a);
+            if (tiles >= cus) return launch_tiles<K, PRO, NT, 2, 8>(ctx, a);
+            return launch_tiles<K, PRO, NT, 1, 8>(ctx, a);
+        }
     }
     if constexpr (K == 2048) {
         if (tiles >= 8 * cus) return NT >= 4 ? launch_tiles<K, PRO, NT, 4>(ctx, a) : launch_tiles<K, PRO, NT, 2>(ctx, a);

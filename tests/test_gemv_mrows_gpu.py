@@ -85,10 +85,12 @@ def test_rows_of_zeros_and_a_zero_quarter(ctx):
 @pytest.mark.parametrize("n,rows", [(8192 + 16, 6), (8192 + 40, 8), (8200, 5),      # four tiles a block from six rows on, ragged tails
                                     (32768 + 48, 2), (32768 + 48, 3), (32768 + 8, 4),  # a stream: two and four tiles a block
                                     (32768, 7),                                   # a stream of five rows and more stays with the tiled kernel
-                                    (16, 2), (20, 8), (4080, 4)])                 # one tile, a ragged only tile, one tile a block
+                                    (16, 2), (20, 8), (4080, 4),                  # one tile, a ragged only tile, one tile a block
+                                    # eight waves a block from four rows on: four, two and one tile a block, ragged tails
+                                    (12352, 4), (12352, 8), (4096 + 24, 5), (6000, 7), (3000, 6)])
 def test_every_split_of_a_matrix_into_blocks(ctx, old_ctx, n, rows):
-    """The launcher gives a block one, two or four tiles of sixteen weight rows depending on how many
-    tiles there are and how many activation rows; the last block's tiles may be ragged or absent."""
+    """The launcher gives a block one, two or four tiles of sixteen weight rows and four or eight waves depending on
+    how many tiles there are and how many activation rows; the last block's tiles may be ragged or absent."""
     rng = np.random.default_rng(n + rows)
     k = 2048
     wq = _weights(rng, n, k)
