@@ -151,7 +151,7 @@ typedef struct {
                                 address that does not depend on the position, for a consumer that would
                                 otherwise wait for the position word before it can ask for the row (the
                                 DeltaNet output projection's gate z); NULL: not stored */
-    /* The router's logits in the same launch (one to four rows of one sequence, k = 4096, n = 2048, a residual): the
+    /* The router's logits in the same launch (one to four rows, k = 4096, n = 2048, a residual): the
      * projection feeds y = residual + W pro(x) to an RMSNorm and a float32 router R (llm/moe.go:
      * 219-232), and R (gamma * y) is linear in y: it is fold[e] . [pro(x) | residual] with
      * fold [fold_rows][k + n] = [R diag(gamma) W | R diag(gamma)] made once by shv_router_fold.
@@ -160,7 +160,7 @@ typedef struct {
     const float *fold;
     float *fold_out;
     int32_t fold_rows;
-    int32_t fold_stride;     /* two to four rows of one sequence: row t's products go to fold_out + t * fold_stride */
+    int32_t fold_stride;     /* two to four rows: row t's products go to fold_out + t * fold_stride */
     /* The greedy sampler in the same launch (one row; the vocabulary projection of a decode step):
      * what shv_argmax does with its best / ids / pos / advance over y[0..n) is done by the block
      * of this launch that finishes last (Argmax, llm/sample.go:359-367: first maximum, NaN never

@@ -474,7 +474,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_row_kernel(shv_gemv_q4k_args 
     }
 }
 
-// ---- two to four activation rows of one sequence (a verification pass, a short prompt tail) ------
+// ---- two to four activation rows (a verification pass, a short prompt tail, a few sequences' steps) ------
 // The one-row kernel's shape with the rows side by side: every row's inputs first, the weights of
 // the wave's passes once, each row staged with its sums, one block-wide wait, then the lane walks
 // the rows with its weights in registers (a row's 64 activations come from LDS when its turn comes).
@@ -493,11 +493,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_a
     const int gi = lane % LPR, rsub = lane / LPR, sb = gi >> 2, g = gi & 3;
     const char *wbase = static_cast<const char *>(a.w) + sb * SHV_Q4K_BYTES;
     const long long pass0 = (static_cast<long long>(blockIdx.x) * WAVES + wave) * P;
-    // the rows are rows 0..NT-1 of ONE sequence: ring rows follow its position
-    int p0 = 0, ring_base = 0;
-    if (a.ring_slots > 0) {
-        p0 = a.pos ? a.pos[0] : 0;
-        ring_base = (a.slot ? a.slot[0] : 0) * a.ring_slots;
+    // row t is row t % seq_len of sequence t / seq_len: its ring row follows that sequence's position and slot
+    const int seq_rows = a.seq_len > 0 ? a.seq_len : a.n_tok;
+    int ring_row[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        ring_row[t] = 0;
+        if (a.ring_slots > 0) {
+            const int s = t / seq_rows;
+            ring_row[t] = (a.slot ? a.slot[s] : s) * a.ring_slots + ((a.pos ? a.pos[s] : 0) + t % seq_rows) % a.ring_slots;
+        }
     }
     float4 xv[NT][NV], gv[NV], zv[NT][NV];
 #pragma unroll
@@ -509,7 +514,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_a
         for (int t = 0; t < NT; t++) {
             xv[t][j] = *reinterpret_cast<const float4 *>(a.x + static_cast<size_t>(t) * a.x_stride + c);
             if constexpr (PRO == SHV_PRO_GATED_NORM) {
-                const float *z = a.z_ring ? a.z + static_cast<size_t>(ring_base + (p0 + t) % a.ring_slots) * a.ring_stride
+                const float *z = a.z_ring ? a.z + static_cast<size_t>(ring_row[t]) * a.ring_stride
                                           : a.z + static_cast<size_t>(t) * a.z_stride;
                 zv[t][j] = *reinterpret_cast<const float4 *>(z + c);
             } else if constexpr (PRO == SHV_PRO_MUL_SIGMOID) {
@@ -599,7 +604,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_fewrows_kernel(shv_gemv_q4k_a
         float xr[64], xs_lo, xs_hi;
         load_x_slice_presummed(xs[t], xsum[t], gi, xr, xs_lo, xs_hi);
         float *y = a.y + static_cast<size_t>(t) * a.y_stride;
-        if (a.ring_slots > 0 && !a.z_ring) y = a.y + static_cast<size_t>(ring_base + (p0 + t) % a.ring_slots) * a.ring_stride;
+        if (a.ring_slots > 0 && !a.z_ring) y = a.y + static_cast<size_t>(ring_row[t]) * a.ring_stride;
 #pragma unroll
         for (int u = 0; u < P; u++) {
             float acc = w[u].dot(g, nc, xr, xs_lo, xs_hi);
@@ -694,7 +699,7 @@ int launch_row_kp(shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     return SHV_OK;
 }
 
-// Two to four rows of one sequence take the rows-side-by-side form of the same kernel.
+// Two to four rows (of one sequence or of several) take the rows-side-by-side form of the same kernel.
 bool fewrows_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a);
 
 bool row_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
@@ -710,9 +715,9 @@ bool row_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
 
 bool fewrows_kernel_covers(const shv_ctx *ctx, const shv_gemv_q4k_args &a) {
     if (a.n_tok < 2 || a.n_tok > 4 || a.y_flat) return false;
-    // one sequence: its rows share a position word and a slot
+    // whole sequences of equal length (one of n_tok rows, or n_tok of one row each)
     const int sl = a.seq_len > 0 ? a.seq_len : a.n_tok;
-    if (sl != a.n_tok) return false;
+    if (sl < 1 || a.n_tok % sl != 0) return false;
     if (a.x_stride % 4 != 0 || ((a.prologue == SHV_PRO_GATED_NORM || a.prologue == SHV_PRO_MUL_SIGMOID) && !a.z_ring && a.z_stride % 4 != 0)) return false;
     shv_gemv_q4k_args one = a;
     one.n_tok = 1;
@@ -860,7 +865,7 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
                     "gemv_q4k: fold reads the whole residual row while y is written: they must be different, 16-byte aligned buffers");
         SHV_REQUIRE(a.n_tok == 1 || a.fold_stride >= a.fold_rows, "gemv_q4k: fold_stride %d < fold_rows %d", a.fold_stride, a.fold_rows);
         SHV_REQUIRE(!ctx->gemv_scales_lds && !ctx->mfma_rows_forced && (a.n_tok == 1 ? row_kernel_covers(ctx, a) : fewrows_kernel_covers(ctx, a)),
-                    "gemv_q4k: fold needs the row kernels' shapes and alignment of x, gamma and z (rows of one sequence)");
+                    "gemv_q4k: fold needs the row kernels' shapes and alignment of x, gamma and z (whole sequences of equal length)");
     }
     if (a.amax_best) {
         SHV_REQUIRE(a.n_tok == 1 && a.ring_slots == 0 && !a.fold && !a.residual, "gemv_q4k: the arg-max in the launch goes with one plain row of outputs");
@@ -874,7 +879,7 @@ int shv_launch_gemv_q4k(shv_ctx *ctx, const shv_gemv_q4k_args *pa) {
         }
     }
     // two to eight rows: every weight formed once for all of them, the products on the matrix cores; 4096 columns
-    // wide, up to four rows of one sequence are quicker side by side in the one-row kernel's shape (6.7 against
+    // wide, up to four rows are quicker side by side in the one-row kernel's shape (6.7 against
     // 8.0 us for three rows of a 2048 x 4096 output projection: a block there stages 16 K columns a row)
     const bool few = fewrows_kernel_covers(ctx, a) && !ctx->mfma_rows_forced;
     if (!ctx->mfma_rows_forced && !(few && a.k == 4096) && shv_gemv_mrows_covers(ctx, a)) return shv_launch_gemv_mrows(ctx, a);

@@ -1365,8 +1365,9 @@ Pass &Graph::pass(int slot, int rows, Kind kind, bool spec) {
     p.labels.push_back("embed");
     if (rows > kBlockRows && (kind == kBatch || spec)) throw Error("llm: a pass of " + std::to_string(rows) + " rows is a plain prompt pass; batched and rewindable passes carry up to " + std::to_string(kBlockRows));
     for (int l = 0; l < layers_; l++) {
-        // (rows of one sequence: a batch of several sequences' rows goes through other projection kernels)
-        if (x2_ && moe_->Folded(l) && (rows == 1 || (kind != kBatch && rows <= MoEGPU::kFoldRows && moe_->FusedRouter(rows)))) {
+        // (rows of one sequence or one row each of several: LLM_BATCH_FOLD=0 keeps the router's launches in batched passes)
+        static const bool batch_fold = [] { const char *e = std::getenv("LLM_BATCH_FOLD"); return !(e && e[0] == '0'); }();
+        if (x2_ && moe_->Folded(l) && (rows == 1 || ((kind != kBatch || batch_fold) && rows <= MoEGPU::kFoldRows && moe_->FusedRouter(rows)))) {
             // the mixer writes the row beside the stream (its output projection reads the whole
             // residual row for the router's products while it writes), the MoE block brings it back
             PassRows rf = r;

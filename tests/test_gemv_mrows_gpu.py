@@ -190,3 +190,11 @@ def test_sixteen_waves_equal_four(ctx, rows):
             assert O.rel_l2(outs[0][t], outs[1][t]) <= 3e-6, t
     finally:
         four.destroy()
+
+
+@pytest.mark.parametrize("n_seq", [2, 3, 4, 5, 8])
+def test_one_row_each_of_several_sequences(ctx, n_seq):
+    """Several sequences' steps in one pass on the library's own context: two to four go through the side-by-side
+    row kernel at 4096 columns (each row's gate from its own sequence's ring row) and this kernel at 2048, five and
+    eight through the wider blocks."""
+    G.test_one_row_each_of_several_sequences(ctx, n_seq)
