@@ -183,7 +183,7 @@ type graphHIP struct {
 }
 
 // layers is Graph.layers (llm/graph.go:2330) without hyper-connection streams: per layer the mixer on
-// RMSNorm(x) and the MoE block on RMSNorm(x), each adding to x.  One to three rows of one sequence with a
+// RMSNorm(x) and the MoE block on RMSNorm(x), each adding to x.  One to four rows (of one sequence or one each of several) with a
 // folded router take the two-op MoE block; everything else the three-op one.
 func (g *graphHIP) layers(r hip.PassRows) ([]hip.Op, []string, error) {
 	c := g.cfg
@@ -191,7 +191,7 @@ func (g *graphHIP) layers(r hip.PassRows) ([]hip.Op, []string, error) {
 	ops := []hip.Op{hip.Embed(g.embd, g.ids, g.pos, g.x, rows, c.NEmbd, c.VocabSize, g.embdType)}
 	kinds := []string{"embed"}
 	for l := 0; l < c.NLayer; l++ {
-		folded := g.foldTable != nil && g.foldTable[l] != nil && r.NSeq == 1 && rows <= 3
+		folded := g.foldTable != nil && g.foldTable[l] != nil && rows <= 4
 		var f fold
 		mixOut := g.x
 		if folded {

@@ -28,7 +28,7 @@ type moeHIP struct {
 	xn, logits, topk, weights, act *hip.Buffer
 	group, pairs                   *hip.Buffer // workspaces of the grouped path; nil keeps every pass per (token, slot)
 	rows                           int
-	routeInUp                      bool // passes of one to three rows make their selection inside MoEUp (LLM_MOE_ROUTE=rows)
+	routeInUp                      bool // passes of one to four rows make their selection inside MoEUp (LLM_MOE_ROUTE=rows)
 }
 
 // graph is MoEGPU.graph for one layer: in and out are the residual stream's rows (out may be in).
@@ -42,8 +42,8 @@ func (g *moeHIP) graph(layer int, in, out *hip.Buffer) ([]hip.Op, []string, erro
 	ty := g.banks[layer].Types
 	q4k := ty[0] == ggmlQ4K && ty[1] == ggmlQ4K && ty[3] == ggmlQ4K && ty[4] == ggmlQ4K
 	downQ4K := ty[2] == ggmlQ4K && ty[5] == ggmlQ4K
-	// passes of one to three rows route in the expert kernel itself; banks of another type take the router's selection
-	fused := g.routeInUp && g.rows <= 3 && q4k
+	// passes of one to four rows route in the expert kernel itself; banks of another type take the router's selection
+	fused := g.routeInUp && g.rows <= 4 && q4k
 	var lg, wt, grp *hip.Buffer
 	if fused {
 		lg, wt = g.logits, g.weights

@@ -232,12 +232,14 @@ public:
     uint64_t ActivationBytes() const { return act_bytes_; }
     // Where the top-k selection runs (MoEGPU.SetRouter, llm/gpu_moe.go:307): fused, in the prologue
     // of the gate/up kernel from the router's logits, or as a dispatch of its own after the router.
-    // Fused on passes of one to three rows unless asked otherwise (mode 2): one launch fewer on the
+    // Fused on passes of one to four rows unless asked otherwise (mode 2): one launch fewer on the
     // step's critical path, the selection repeated by every workgroup with all four of its waves
-    // (482 to 509 tok/s; a 2-row pass 2.32 to 2.28 ms, a 3-row pass 2.81 to 2.75); level at four
-    // rows, and from there slower than a dispatch of its own (eight rows 4.80 to 5.04 ms).
+    // (482 to 509 tok/s; a 2-row pass 2.32 to 2.28 ms, a 3-row pass 2.81 to 2.75); with the router's
+    // rows on the mixer's output projection (Fold) two launches fewer, which pays at four rows too
+    // (four sequences a pass 3.14 to 2.90 ms); beyond, where there is no such table, slower than a
+    // dispatch of its own (eight rows 4.80 to 5.04 ms).
     void SetRouter(bool fused) { route_mode_ = fused ? 1 : 0; }
-    bool FusedRouter(int rows = 1) const { return route_mode_ == 1 || (route_mode_ == 2 && rows <= 3); }
+    bool FusedRouter(int rows = 1) const { return route_mode_ == 1 || (route_mode_ == 2 && rows <= kFoldRows); }
 
 private:
     Device &dev_;
@@ -247,7 +249,7 @@ private:
     float *in_, *out_, *xn_, *logits_, *weights_, *act_, *pairs_ = nullptr;
     int32_t *topk_, *group_ = nullptr;
     uint64_t act_bytes_ = 0;
-    int route_mode_ = 2;  // 0 own dispatch, 1 fused, 2 fused for passes of up to three rows
+    int route_mode_ = 2;  // 0 own dispatch, 1 fused, 2 fused for passes of up to four rows
     std::vector<float *> fold_;  // per layer [NExpert+1][k + NEmbd], or nullptr
     int fold_k_ = 0;
 };

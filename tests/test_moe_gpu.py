@@ -503,9 +503,9 @@ def test_router_rows_ride_on_the_output_projection(ctx, full_bank, prologue, E, 
         c.enqueue(A.OP_MOE_UP, ua)
 
 
-@pytest.mark.parametrize("T", [2, 3])
+@pytest.mark.parametrize("T", [2, 3, 4])
 def test_router_rows_ride_on_a_projection_of_a_few_rows(ctx, T):
-    """The same for two and three rows of one sequence (a verification pass): the rows-side-by-side
+    """The same for two to four rows (a verification pass, a few sequences' steps): the rows-side-by-side
     projection kernel forms every row's products, the gate/up kernel normalises each row itself."""
     E, used = 64, 10
     case = MoeCase(ctx, seed=91, E=E, used=used, T=T)
