@@ -684,6 +684,8 @@ def main():
             rec["mtp"]["verify_pass_in_steps"] = round(rec["mtp"]["true_continuation_as_drafts"]["verify_gpu_ms_per_round"] / rec["gpu_ms_per_step"], 3)
     if not a.no_mtp and a.batch_slots >= 2:
         rec["batched_decode"] = batched_run(m, cfg, a.batch_slots, rng)
+        # fewer sequences a pass, on the same staged slots: what a lightly loaded server runs
+        rec["batched_decode_few"] = {str(n): batched_run(m, cfg, n, rng, steps=24) for n in (2, 3, 4) if n < a.batch_slots}
     cores = min(os.cpu_count() or 1, 16)
     tensors = first_period_tensors(m, cfg) if not a.no_cpu else None
     if not a.no_configs:
