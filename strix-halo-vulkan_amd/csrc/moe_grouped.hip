@@ -479,10 +479,24 @@ __device__ __forceinline__ void min_terms(int q, const char *sfr, const char *hb
 // fragments of the step after this one are read from LDS before this step's products are issued,
 // so no product waits for an LDS read.
 template <int NG, int R, int NTT, typename Ask>
-__device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[R], RowStream<R> &st, int G0, int G_last, const char *frags,
+__device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[R], RowStream<R> &st, int G0, int G_last, const char *frags, const char *hbuf,
                                                         int lane, float4_t (&acc)[R][NTT], float4_t (&y)[R][NTT], Ask &&ask_next) {
+    static_assert(NG == 4, "a slab is one super-block: its header is read once, where the slab begins");
     const int kb = lane >> 4;
     const NibbleMasks nc = nibble_masks();
+    // The rows' headers of this super-block are in LDS already: min_terms' loads brought the quarter's (lane (row, kb)
+    // holds super-block 4 q + kb's), a slab and more ahead.  Asked for from memory where a super-block ends they were
+    // waited for where the next begins, and kept a super-block ahead they cost sixteen registers.
+    typedef uint32_t u32x4_lds __attribute__((ext_vector_type(4)));
+    uint4 hdr[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const u32x4_lds h = *reinterpret_cast<const __attribute__((address_space(3))) u32x4_lds *>(
+            (const __attribute__((address_space(3))) char *)(hbuf) + r * kFrag + ((lane & 15) + 16 * ((G0 >> 2) & 3)) * 16);
+        hdr[r] = make_uint4(h.x, h.y, h.z, h.w);
+    }
+    // read to the end before the loads of the quarter after this one may be asked for (they land in the same place)
+    asm volatile("" : "+v"(hdr[0].x), "+v"(hdr[1].x), "+v"(hdr[2].x), "+v"(hdr[3].x));
     // LDS addresses are 32 bits wide: kept as such, a fragment's place costs no 64-bit arithmetic
     typedef const __attribute__((address_space(3))) char *lds_bytes_t;
     typedef const __attribute__((address_space(3))) half8_t *lds_half8_t;
@@ -507,7 +521,7 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
 #pragma unroll
         for (int r = 0; r < R; r++) {
             uint32_t mn;
-            q4k_group_scale_min(st.hdr[r], g, sc[r], mn);
+            q4k_group_scale_min(hdr[r], g, sc[r], mn);
         }
 #pragma unroll
         for (int hi = 0; hi < 2; hi++) {
@@ -559,7 +573,7 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
             // the super-block ends: its sums take its d, the next one's header moves in
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const float dd = f16_bits_to_f32(st.hdr[r].x);
+                const float dd = f16_bits_to_f32(hdr[r].x);
 #pragma unroll
                 for (int tt = 0; tt < NTT; tt++) {
 #pragma unroll
@@ -567,9 +581,6 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
                     acc[r][tt] = float4_t{0.f, 0.f, 0.f, 0.f};
                 }
             }
-            st.ask_header(rp, (G >> 2) + 1, G_last >> 2);
-#pragma unroll
-            for (int r = 0; r < R; r++) st.hdr[r] = st.hdr_next[r];
         }
     }
 }
@@ -594,9 +605,6 @@ __device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTile
     ask_staged_sums<K>(sums, tok_s, m, NTT, 0, sum_bufs, lane, wave);
     ask_min_headers<K, kTiles>(rp, 0, hbuf, lane);
     RowStream<kTiles> st;
-    st.ask_header(rp, 0, GROUPS / 4 - 1);
-#pragma unroll
-    for (int r = 0; r < kTiles; r++) st.hdr[r] = st.hdr_next[r];
     st.ask_group(rp, 0, GROUPS - 1, lane >> 4);
 #pragma unroll 1
     for (int sl = 0; sl < SLABS; sl++) {
@@ -606,7 +614,7 @@ __device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTile
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         if (sl % kStQuarter == 0) min_terms<K, kTiles, NTT>(sl / kStQuarter, sum_bufs + ((sl / kStQuarter) & 1) * kStSumFrags, hbuf, lane, y);
-        staged_slab_times_tiles<NG, kTiles, NTT>(rp, st, sl * NG, GROUPS - 1, buf, lane, acc, y, [&] {
+        staged_slab_times_tiles<NG, kTiles, NTT>(rp, st, sl * NG, GROUPS - 1, buf, hbuf, lane, acc, y, [&] {
             if (sl + 1 < SLABS) {
                 ask_staged_slab<K>(staged, tok_s, m, NTT, sl + 1, bufs + ((sl + 1) & 1) * kStFrags, lane, wave);
                 if ((sl + 1) % kStQuarter == 0) {
