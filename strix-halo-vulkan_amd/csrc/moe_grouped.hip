@@ -195,6 +195,16 @@ struct RowStream {
         for (int r = 0; r < R; r++)
             q_next[r] = *reinterpret_cast<const uint2 *>(rp[r] + static_cast<size_t>(Gc >> 2) * SHV_Q4K_BYTES + 16 + (Gc & 3) * 32 + kb * 8);
     }
+    // A lane's 16 bytes of a PAIR of groups (pair Pg = groups 2 Pg, 2 Pg + 1: 64 payload bytes a row, one line's
+    // worth in one load where two 8-byte loads of a group each took a half line apiece): lane (row, kb) holds bytes
+    // 16 kb .. 16 kb + 15 of the pair, i.e. columns 16 (kb & 1) .. + 15 of group 2 Pg + (kb >> 1), low and high nibbles.
+    uint4 pair_next[R];
+    __device__ __forceinline__ void ask_pair(const char *const (&rp)[R], int Pg, int P_last, int kb) {
+        const int Pc = Pg < P_last ? Pg : P_last;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            pair_next[r] = *reinterpret_cast<const uint4 *>(rp[r] + static_cast<size_t>(Pc >> 1) * SHV_Q4K_BYTES + 16 + (Pc & 1) * 64 + kb * 16);
+    }
     __device__ __forceinline__ void ask_header(const char *const (&rp)[R], int sb, int sb_last) {
         const int sc = sb < sb_last ? sb : sb_last;
 #pragma unroll
@@ -401,14 +411,19 @@ __global__ __launch_bounds__(256) void moe_stage_kernel(const float *x, int x_st
 
 template <int K>
 __device__ __forceinline__ void ask_staged_slab(const char *staged, const int32_t *tok_s, int m, int n_tt, int sl, char *buf, int lane, int wave) {
-    const int sg = sl * kStSubs + wave;  // this wave's sub-block of the row
+    // Wave w asks for product w of the slab's eight: pair w / 4 of its groups, the pair's low (0) or high (1) nibbles,
+    // the first or second eight of a lane's sixteen bytes.  Its lane (token, kb) stands where the weights' lane
+    // (row, kb) does: sub-block 2 (group of the lane) + nibble, columns 16 (kb & 1) + 8 (half) .. + 7 of it.
     const int n = lane & 15, kb = lane >> 4;
+    const int pr = wave >> 2, hi = (wave >> 1) & 1, half = wave & 1;
+    const int sg = sl * kStSubs + 4 * pr + 2 * (kb >> 1) + hi;  // the sub-block this lane's eight columns lie in
+    const int cb = 2 * (kb & 1) + half;                          // and which eight of its 32
 #pragma unroll
     for (int tt = 0; tt < kTT; tt++) {
         if (tt >= n_tt) break;
         const int i = 16 * tt + n;
         const int t = tok_s[i < m ? i : 0];  // a column past the list repeats the first row; nobody reads its products
-        const char *g = staged + (static_cast<size_t>(t) * (K / 32) + sg) * kStSubBytes + kb * 16;
+        const char *g = staged + (static_cast<size_t>(t) * (K / 32) + sg) * kStSubBytes + cb * 16;
         char *f = buf + ((wave * 2) * kTT + tt) * kFrag;
         __builtin_amdgcn_global_load_lds((global_ptr_t)(g), (lds_ptr_t)(f), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((global_ptr_t)(g + 64), (lds_ptr_t)(f + kTT * kFrag), 16, 0, 0);
@@ -486,49 +501,48 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
     const NibbleMasks nc = nibble_masks();
     // The rows' headers of this super-block are in LDS already: min_terms' loads brought the quarter's (lane (row, kb)
     // holds super-block 4 q + kb's), a slab and more ahead.  Asked for from memory where a super-block ends they were
-    // waited for where the next begins, and kept a super-block ahead they cost sixteen registers.
+    // waited for where the next begins; kept in registers they cost sixteen, so each pair of groups reads them again.
     typedef uint32_t u32x4_lds __attribute__((ext_vector_type(4)));
-    uint4 hdr[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        const u32x4_lds h = *reinterpret_cast<const __attribute__((address_space(3))) u32x4_lds *>(
-            (const __attribute__((address_space(3))) char *)(hbuf) + r * kFrag + ((lane & 15) + 16 * ((G0 >> 2) & 3)) * 16);
-        hdr[r] = make_uint4(h.x, h.y, h.z, h.w);
-    }
-    // read to the end before the loads of the quarter after this one may be asked for (they land in the same place)
-    asm volatile("" : "+v"(hdr[0].x), "+v"(hdr[1].x), "+v"(hdr[2].x), "+v"(hdr[3].x));
+    const __attribute__((address_space(3))) char *hl = (const __attribute__((address_space(3))) char *)(hbuf) + ((lane & 15) + 16 * ((G0 >> 2) & 3)) * 16;
     // LDS addresses are 32 bits wide: kept as such, a fragment's place costs no 64-bit arithmetic
     typedef const __attribute__((address_space(3))) char *lds_bytes_t;
     typedef const __attribute__((address_space(3))) half8_t *lds_half8_t;
     const lds_bytes_t fl = (lds_bytes_t)(frags) + lane * 16;
     half8_t nh = *(lds_half8_t)(fl), nl = *(lds_half8_t)(fl + kTT * kFrag);
 #pragma unroll 1
-    for (int gi = 0; gi < NG; gi++) {
-        const int G = G0 + gi, g = G & 3;
-        const lds_bytes_t fg = fl + gi * (4 * kTT * kFrag);                     // this group's two sub-blocks
-        const lds_bytes_t fn = gi + 1 < NG ? fg + 4 * kTT * kFrag : fl;        // the group after it (the slab's first again past its last, unused)
-        uint2 q[R];
+    for (int pi = 0; pi < NG / 2; pi++) {
+        const int Pg = (G0 >> 1) + pi;                                          // the pair of groups: 2 Pg, 2 Pg + 1
+        const lds_bytes_t fp = fl + pi * (8 * kTT * kFrag);                     // this pair's four products
+        const lds_bytes_t fn = pi + 1 < NG / 2 ? fp + 8 * kTT * kFrag : fl;    // the pair after it (the slab's first again past its last, unused)
+        uint4 q[R];
 #pragma unroll
-        for (int r = 0; r < R; r++) q[r] = st.q_next[r];
-        // the group's bytes are here: only now the loads that nothing in this slab waits for (a
+        for (int r = 0; r < R; r++) q[r] = st.pair_next[r];
+        // the pair's bytes are here: only now the loads that nothing in this slab waits for (a
         // wait for loaded registers also waits for every load issued before them)
         asm volatile("" : "+v"(q[0].x), "+v"(q[1].x), "+v"(q[2].x), "+v"(q[3].x));
-        // the next group's bytes first: a wait for them then does not wait for the slab's loads behind them
-        st.ask_group(rp, G + 1, G_last, kb);
-        if (gi == 0) ask_next();
-        __builtin_amdgcn_sched_barrier(0);  // the loads stay up here, a group ahead of their use
-        uint32_t sc[R];
+        // this lane's group of the pair, within the super-block: its scales, and the rows' d
+        const int g = (2 * Pg + (kb >> 1)) & 3;
+        uint32_t sc[R], dd16[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
+            const u32x4_lds h = *reinterpret_cast<const __attribute__((address_space(3))) u32x4_lds *>(hl + r * kFrag);
             uint32_t mn;
-            q4k_group_scale_min(hdr[r], g, sc[r], mn);
+            q4k_group_scale_min(make_uint4(h.x, h.y, h.z, h.w), g, sc[r], mn);
+            dd16[r] = h.x;
         }
+        // read to the end before the loads of the quarter after this one may be asked for (they land in the same place)
+        asm volatile("" : "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]), "+v"(dd16[0]), "+v"(dd16[1]), "+v"(dd16[2]), "+v"(dd16[3]));
+        // the next pair's bytes first: a wait for them then does not wait for the slab's loads behind them
+        st.ask_pair(rp, Pg + 1, G_last >> 1, kb);
+        ask_next(pi);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay up here, a pair ahead of their use
 #pragma unroll
-        for (int hi = 0; hi < 2; hi++) {
+        for (int u = 0; u < 4; u++) {
+            const int hi = u >> 1;  // products 0, 1: the low nibbles of bytes 0..7 and 8..15; 2, 3: the high nibbles
             half8_t b[R];
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const uint32_t q0 = q[r].x, q1 = q[r].y;
+                const uint32_t q0 = (u & 1) ? q[r].z : q[r].x, q1 = (u & 1) ? q[r].w : q[r].y;
                 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
                 // A nibble in the low bits of a half's mantissa reads, under the right exponent, as
                 // C + n: bits 0..3 under 1024's, bits 4..7 under 64's (the odd bytes' nibbles take
@@ -557,10 +571,10 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
 #pragma unroll
             for (int tt = 0; tt < NTT; tt++) {
                 const half8_t xh = nh, xl = nl;
-                // the step after this one: the next token tile, the next sub-block's first, or (past
+                // the step after this one: the next token tile, the next product's first, or (past
                 // the slab's last) the first again, unused
                 const int ntt = tt + 1 < NTT ? tt + 1 : 0;
-                const lds_bytes_t f = tt + 1 < NTT ? fg + ((hi * 2) * kTT + ntt) * kFrag : (hi == 0 ? fg + 2 * kTT * kFrag : fn);
+                const lds_bytes_t f = tt + 1 < NTT ? fp + ((u * 2) * kTT + ntt) * kFrag : (u < 3 ? fp + ((u + 1) * 2) * kTT * kFrag : fn);
                 nh = *(lds_half8_t)(f);
                 nl = *(lds_half8_t)(f + kTT * kFrag);
 #pragma unroll
@@ -569,11 +583,11 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
                 for (int r = 0; r < R; r++) acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc[r][tt], 0, 0, 0);
             }
         }
-        if (g == 3) {
-            // the super-block ends: its sums take its d, the next one's header moves in
+        if (Pg & 1) {
+            // the super-block ends: its sums take its d
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const float dd = f16_bits_to_f32(hdr[r].x);
+                const float dd = f16_bits_to_f32(dd16[r]);
 #pragma unroll
                 for (int tt = 0; tt < NTT; tt++) {
 #pragma unroll
@@ -605,7 +619,7 @@ __device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTile
     ask_staged_sums<K>(sums, tok_s, m, NTT, 0, sum_bufs, lane, wave);
     ask_min_headers<K, kTiles>(rp, 0, hbuf, lane);
     RowStream<kTiles> st;
-    st.ask_group(rp, 0, GROUPS - 1, lane >> 4);
+    st.ask_pair(rp, 0, GROUPS / 2 - 1, lane >> 4);
 #pragma unroll 1
     for (int sl = 0; sl < SLABS; sl++) {
         char *buf = bufs + (sl & 1) * kStFrags;
@@ -614,10 +628,12 @@ __device__ __forceinline__ void staged_times_tiles(const char *const (&rp)[kTile
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         if (sl % kStQuarter == 0) min_terms<K, kTiles, NTT>(sl / kStQuarter, sum_bufs + ((sl / kStQuarter) & 1) * kStSumFrags, hbuf, lane, y);
-        staged_slab_times_tiles<NG, kTiles, NTT>(rp, st, sl * NG, GROUPS - 1, buf, hbuf, lane, acc, y, [&] {
+        staged_slab_times_tiles<NG, kTiles, NTT>(rp, st, sl * NG, GROUPS - 1, buf, hbuf, lane, acc, y, [&](int pi) {
+            // the next slab at the slab's first pair of groups; the next quarter's sums and headers at its second, behind
+            // the last reading of this quarter's headers
             if (sl + 1 < SLABS) {
-                ask_staged_slab<K>(staged, tok_s, m, NTT, sl + 1, bufs + ((sl + 1) & 1) * kStFrags, lane, wave);
-                if ((sl + 1) % kStQuarter == 0) {
+                if (pi == 0) ask_staged_slab<K>(staged, tok_s, m, NTT, sl + 1, bufs + ((sl + 1) & 1) * kStFrags, lane, wave);
+                if (pi == 1 && (sl + 1) % kStQuarter == 0) {
                     const int q = (sl + 1) / kStQuarter;
                     ask_staged_sums<K>(sums, tok_s, m, NTT, q, sum_bufs + (q & 1) * kStSumFrags, lane, wave);
                     ask_min_headers<K, kTiles>(rp, q, hbuf, lane);
