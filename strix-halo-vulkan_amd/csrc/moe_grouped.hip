@@ -568,6 +568,9 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
                     b[r][2 * i + 1] = p[1];
                 }
             }
+            // the matrix instructions of a step win the SIMD's issue slot over the other wave's vector
+            // instructions, which then run under them instead of between them
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int tt = 0; tt < NTT; tt++) {
                 const half8_t xh = nh, xl = nl;
@@ -582,6 +585,7 @@ __device__ __forceinline__ void staged_slab_times_tiles(const char *const (&rp)[
 #pragma unroll
                 for (int r = 0; r < R; r++) acc[r][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xl, b[r], acc[r][tt], 0, 0, 0);
             }
+            __builtin_amdgcn_s_setprio(0);
         }
         if (Pg & 1) {
             // the super-block ends: its sums take its d
