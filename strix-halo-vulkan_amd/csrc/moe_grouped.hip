@@ -4,7 +4,8 @@
 // weights once per token that chose it, this path once per 48 such tokens: it pays when tokens
 // outnumber experts (2048 rows choosing 10 of 512: 40 tokens an expert), not at 64 rows (1.9).
 //
-//   moe_group_kernel          per-expert lists of (token, slot) pairs from topk
+//   moe_group_kernel          per-expert lists of (token, slot) pairs from topk (one block; long passes:
+//                             moe_group_count_kernel + moe_group_place_kernel, sixteen blocks)
 //   moe_up_grouped_kernel     a block = (expert, half of its ffn rows) and up to 48 of its tokens
 //                             at a time: their xn rows go through LDS as matrix-core operands
 //                             (two halves hi + lo, as the projections do) in slabs of 512 columns,
@@ -130,6 +131,83 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
         place(q[b].w, i + 3);
     }
     for (int i = rest0 + tid; i < n_pairs; i += 1024) place(topk[i], i);
+}
+
+// The same lists by several blocks in two launches, for passes long enough that one block's count and placement
+// (one compute unit's scattered stores) are most of the grouping: block b takes pairs [b * chunk, (b + 1) * chunk).
+// First launch: every block's count of its pairs per expert, to counts[b][e].  Second: every block adds up the
+// counts (an expert's total, and what the blocks before it hold of it), forms the starts, and places its own pairs
+// behind those of the blocks before it; block 0 also writes the starts and the experts' launch order.
+constexpr int kGroupBlocks = 16;
+__global__ __launch_bounds__(1024) void moe_group_count_kernel(const int32_t *topk, int n_pairs, int chunk, int n_expert, int32_t *counts) {
+    __shared__ int32_t s_cnt[kMaxExperts];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < n_expert; e += 1024) s_cnt[e] = 0;
+    __syncthreads();
+    const int lo = blockIdx.x * chunk, hi = lo + chunk < n_pairs ? lo + chunk : n_pairs;
+    for (int i = lo + tid; i < hi; i += 1024) {
+        const int e = topk[i];
+        if (e >= 0 && e < n_expert) atomicAdd(&s_cnt[e], 1);
+    }
+    __syncthreads();
+    for (int e = tid; e < n_expert; e += 1024) counts[blockIdx.x * n_expert + e] = s_cnt[e];
+}
+
+__global__ __launch_bounds__(1024) void moe_group_place_kernel(const int32_t *topk, int n_pairs, int chunk, int n_used, int n_expert, const int32_t *counts,
+                                                               int32_t *group) {
+    __shared__ int32_t s_cnt[kMaxExperts + 1];
+    __shared__ __align__(16) int32_t s_len[kMaxExperts];
+    __shared__ int32_t s_wsum[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nb = gridDim.x, b = blockIdx.x;
+    // thread e: expert e's total, and the pairs of it the blocks before this one hold
+    int c = 0, before = 0;
+    if (tid < n_expert) {
+        for (int o = 0; o < nb; o++) {
+            const int v = counts[o * n_expert + tid];
+            c += v;
+            before += o < b ? v : 0;
+        }
+    }
+    int incl = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    if (lane == 63) s_wsum[wave] = incl;
+    s_len[tid] = tid < n_expert ? c : -1;   // past n_expert: shorter than any list
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; w++) base += s_wsum[w];
+    const int start = base + incl - c;
+    if (tid < n_expert) s_cnt[tid] = start + before;
+    if (b == 0) {
+        if (tid < n_expert) group[tid] = start;
+        if (tid == n_expert - 1) group[n_expert] = start + c;
+        // an expert's place in the launch: longer lists first, equal lengths by index
+        if (tid < n_expert) {
+            const int e = tid;
+            int rank = 0;
+            const int n4 = (n_expert + 3) / 4;
+#pragma unroll 16
+            for (int o4 = 0; o4 < n4; o4++) {
+                const int4 c4 = *reinterpret_cast<const int4 *>(&s_len[4 * o4]);
+                const int o = 4 * o4;
+                rank += (c4.x > c || (c4.x == c && o < e)) ? 1 : 0;
+                rank += (c4.y > c || (c4.y == c && o + 1 < e)) ? 1 : 0;
+                rank += (c4.z > c || (c4.z == c && o + 2 < e)) ? 1 : 0;
+                rank += (c4.w > c || (c4.w == c && o + 3 < e)) ? 1 : 0;
+            }
+            group[n_expert + 1 + n_pairs + rank] = e;
+        }
+    }
+    __syncthreads();
+    int32_t *list = group + n_expert + 1;
+    const int lo = b * chunk, hi = lo + chunk < n_pairs ? lo + chunk : n_pairs;
+    for (int i = lo + tid; i < hi; i += 1024) {
+        const int e = topk[i];
+        if (e >= 0 && e < n_expert) list[atomicAdd(&s_cnt[e], 1)] = (i / n_used) * (n_used + 1) + i % n_used;
+    }
 }
 
 // Columns [col0, col0 + kSlab) of up to kTok listed rows (each a row of floats at rows_s[i]) into
@@ -890,6 +968,22 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(shv_moe_down_args a) {
     *reinterpret_cast<float4 *>(a.out + static_cast<size_t>(t) * a.out_stride + c) = v;
 }
 
+// The per-expert lists of a pass: one block for short passes, kGroupBlocks in two launches from 2048 pairs on
+// (their counts meet in the library's scratch, which nothing else on the stream is using between the two).
+int launch_group(shv_ctx *ctx, const int32_t *topk, int n_tok, int n_used, int n_expert, int32_t *group) {
+    const int n_pairs = n_tok * n_used;
+    if (n_pairs < 2048 || !ctx->gemm_part || ctx->moe_group_one_block) {
+        SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, topk, n_tok, n_used, n_expert, group);
+        return SHV_OK;
+    }
+    static_assert(static_cast<size_t>(kGroupBlocks) * kMaxExperts * 4 <= static_cast<size_t>(shv_ctx::kGemmPartBytes), "the blocks' counts fit the scratch");
+    int32_t *counts = reinterpret_cast<int32_t *>(ctx->gemm_part);
+    const int chunk = (n_pairs + kGroupBlocks - 1) / kGroupBlocks;
+    SHV_LAUNCH(ctx, moe_group_count_kernel, dim3(kGroupBlocks), dim3(1024), 0, topk, n_pairs, chunk, n_expert, counts);
+    SHV_LAUNCH(ctx, moe_group_place_kernel, dim3(kGroupBlocks), dim3(1024), 0, topk, n_pairs, chunk, n_used, n_expert, counts, group);
+    return SHV_OK;
+}
+
 template <typename Kern>
 int raise_lds(Kern kern, size_t lds) {
     SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
@@ -920,7 +1014,7 @@ int shv_launch_moe_up_grouped(shv_ctx *ctx, const shv_moe_up_args &a) {
     // refused before anything is enqueued: an error return leaves no half pass on the stream
     SHV_REQUIRE(!a.act_packed || (ctx->gemm_part && packed_sums_bytes(static_cast<long long>(a.n_tok) * (a.n_used + 1), a.ffn) <= static_cast<size_t>(shv_ctx::kGemmPartBytes)),
                 "moe_up: %d rows are too many for act_packed", a.n_tok);
-    SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, a.group);
+    if (const int rc = launch_group(ctx, a.topk, a.n_tok, a.n_used, a.n_expert, a.group); rc != SHV_OK) return rc;
     SHV_LAUNCH(ctx, moe_stage_kernel, dim3((a.n_embd + 1023) / 1024, a.n_tok), dim3(256), 0, a.xn, a.n_embd, a.n_embd, a.n_tok, ctx->gemm_stage);
     constexpr size_t lds = kStagedLds;
     static const int raised = raise_lds(&moe_up_grouped_kernel<2048>, lds);
@@ -944,7 +1038,9 @@ int shv_launch_moe_down_grouped(shv_ctx *ctx, const shv_moe_down_args &a) {
     const bool lists = a.group_ready && st.grouped && st.topk == a.topk && st.group == a.group && st.n_tok == a.n_tok && st.n_used == a.n_used;
     SHV_REQUIRE(!a.act_packed || (lists && st.packed && st.act == a.act && ctx->gemm_part),
                 "moe_down: act_packed, but the shv_moe_up before this call did not leave act as operands for this pass");
-    if (!lists) SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group));
+    if (!lists) {
+        if (const int rc = launch_group(ctx, a.topk, a.n_tok, a.n_used, a.n_expert, const_cast<int32_t *>(a.group)); rc != SHV_OK) return rc;
+    }
     const int parts = a.n_embd / 512, tiles = (a.n_tok + kTok - 1) / kTok;
     if (a.act_packed) {
         constexpr size_t lds = kStagedLds;

@@ -98,7 +98,8 @@ class MoeCase:
             da.group_ready = 1 if group_ready is None else group_ready
         ops = [A.make_op(A.OP_MOE_ROUTER, ra), A.make_op(A.OP_MOE_UP, ua), A.make_op(A.OP_MOE_DOWN, da)]
         c.dispatch_multi(ops)
-        return dict(xn=xn.read(np.float32, T * H).reshape(T, H),
+        return dict(group=group.read(np.int32, 2 * E + 1 + T * used) if grouped else None,
+                    xn=xn.read(np.float32, T * H).reshape(T, H),
                     logits=logits.read(np.float32, T * (E + 1)).reshape(T, E + 1),
                     topk=topk.read(np.int32, T * used).reshape(T, used),
                     weights=weights.read(np.float32, T * (used + 1)).reshape(T, used + 1),
@@ -160,6 +161,24 @@ def test_moe_block_over_banks_in_other_types(ctx, types, T):
     bad.types[2] = 10
     with pytest.raises(A.ShvError, match="moe_down: rows of 512 elements of ggml type 10"):
         bad.gpu()
+
+
+@pytest.mark.parametrize("T,E,used", [(160, 64, 10), (300, 64, 10), (517, 128, 8), (1030, 512, 2)])
+def test_lists_by_expert_hold_every_pair_once(ctx, T, E, used):
+    """The workspace the grouped kernels walk (llm/moe.go:289-409 batches a chunk's tokens per expert): starts that
+    add up, under every expert exactly the (token, slot) pairs that chose it, in any order, and the experts' launch
+    order by list length, longer first, equal lengths by index.  Passes below 2048 pairs are listed by one block,
+    longer ones by sixteen in two launches: both roads are here."""
+    case = MoeCase(ctx, seed=T, E=E, used=used, T=T)
+    got = case.gpu(residual=True, grouped=True)
+    g, topk = got["group"], got["topk"]
+    starts, lists, order = g[:E + 1], g[E + 1:E + 1 + T * used], g[E + 1 + T * used:]
+    counts = np.bincount(topk.ravel(), minlength=E)
+    assert starts[0] == 0 and np.array_equal(np.diff(starts), counts)
+    for e in range(E):
+        want = sorted(t * (used + 1) + s for t, s in zip(*np.nonzero(topk == e)))
+        assert sorted(lists[starts[e]:starts[e + 1]]) == want, e
+    assert list(order) == sorted(range(E), key=lambda e: (-counts[e], e))
 
 
 @pytest.mark.parametrize("T,E,used,seed", [(160, 64, 10, 165), (131, 16, 4, 137), (128, 64, 1, 264)])
