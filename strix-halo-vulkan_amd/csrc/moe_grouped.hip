@@ -99,23 +99,26 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *topk, in
     }
     __syncthreads();
     for (int e = tid; e <= n_expert; e += blockDim.x) group[e] = s_cnt[e];
-    // rank by list length, longer first, equal lengths by index: an expert's place in the launch.  Every thread
-    // walks the same lengths, four a read (one address a wave: a broadcast), sixteen reads in flight.
+    // rank by list length, longer first, equal lengths by index: an expert's place in the launch.  32 threads an
+    // expert, each against every 32nd length, 32 experts a round: with a thread an expert half the block idles
+    // through E comparisons each.
     int32_t *order = group + n_expert + 1 + n_pairs;
-    if (tid < n_expert) {
-        const int e = tid, ce = s_len[e];
-        int rank = 0;
-        const int n4 = (n_expert + 3) / 4;
-#pragma unroll 16
-        for (int o4 = 0; o4 < n4; o4++) {
-            const int4 c4 = *reinterpret_cast<const int4 *>(&s_len[4 * o4]);
-            const int o = 4 * o4;
-            rank += (c4.x > ce || (c4.x == ce && o < e)) ? 1 : 0;
-            rank += (c4.y > ce || (c4.y == ce && o + 1 < e)) ? 1 : 0;
-            rank += (c4.z > ce || (c4.z == ce && o + 2 < e)) ? 1 : 0;
-            rank += (c4.w > ce || (c4.w == ce && o + 3 < e)) ? 1 : 0;
+    {
+        const int part = tid & 31;
+        for (int e = tid >> 5; e < n_expert; e += 32) {
+            const int ce = s_len[e];
+            int rank = 0;
+            for (int o = part; o < n_expert; o += 32) {
+                const int co = s_len[o];
+                rank += (co > ce || (co == ce && o < e)) ? 1 : 0;
+            }
+            rank += __shfl_xor(rank, 16, 64);
+            rank += __shfl_xor(rank, 8, 64);
+            rank += __shfl_xor(rank, 4, 64);
+            rank += __shfl_xor(rank, 2, 64);
+            rank += __shfl_xor(rank, 1, 64);
+            if (part == 0) order[rank] = e;
         }
-        order[rank] = e;
     }
     __syncthreads();  // the starts are copied out before the placement moves them
     int32_t *list = group + n_expert + 1;
@@ -162,10 +165,14 @@ __global__ __launch_bounds__(1024) void moe_group_place_kernel(const int32_t *to
     // thread e: expert e's total, and the pairs of it the blocks before this one hold
     int c = 0, before = 0;
     if (tid < n_expert) {
-        for (int o = 0; o < nb; o++) {
-            const int v = counts[o * n_expert + tid];
-            c += v;
-            before += o < b ? v : 0;
+        // all of them asked for together: one after the other they are sixteen trips to memory
+        int v[kGroupBlocks];
+#pragma unroll
+        for (int o = 0; o < kGroupBlocks; o++) v[o] = o < nb ? counts[o * n_expert + tid] : 0;
+#pragma unroll
+        for (int o = 0; o < kGroupBlocks; o++) {
+            c += v[o];
+            before += o < b ? v[o] : 0;
         }
     }
     int incl = c;
@@ -184,21 +191,28 @@ __global__ __launch_bounds__(1024) void moe_group_place_kernel(const int32_t *to
     if (b == 0) {
         if (tid < n_expert) group[tid] = start;
         if (tid == n_expert - 1) group[n_expert] = start + c;
-        // an expert's place in the launch: longer lists first, equal lengths by index
-        if (tid < n_expert) {
-            const int e = tid;
+    }
+    // An expert's place in the launch: longer lists first, equal lengths by index.  Each block ranks its share of
+    // the experts, 32 threads an expert (each against every 32nd length), instead of one block all of them with a
+    // thread an expert: E^2 comparisons are most of what one block would spend on a pass's lists.
+    {
+        const int per = (n_expert + nb - 1) / nb, e0 = b * per;
+        const int part = tid & 31;
+        for (int eb = tid >> 5; eb < per; eb += 32) {
+            const int e = e0 + eb;
+            const bool live = e < n_expert;
+            const int ce = live ? s_len[e] : 0;
             int rank = 0;
-            const int n4 = (n_expert + 3) / 4;
-#pragma unroll 16
-            for (int o4 = 0; o4 < n4; o4++) {
-                const int4 c4 = *reinterpret_cast<const int4 *>(&s_len[4 * o4]);
-                const int o = 4 * o4;
-                rank += (c4.x > c || (c4.x == c && o < e)) ? 1 : 0;
-                rank += (c4.y > c || (c4.y == c && o + 1 < e)) ? 1 : 0;
-                rank += (c4.z > c || (c4.z == c && o + 2 < e)) ? 1 : 0;
-                rank += (c4.w > c || (c4.w == c && o + 3 < e)) ? 1 : 0;
+            for (int o = part; o < n_expert; o += 32) {
+                const int co = s_len[o];
+                rank += (co > ce || (co == ce && o < e)) ? 1 : 0;
             }
-            group[n_expert + 1 + n_pairs + rank] = e;
+            rank += __shfl_xor(rank, 16, 64);
+            rank += __shfl_xor(rank, 8, 64);
+            rank += __shfl_xor(rank, 4, 64);
+            rank += __shfl_xor(rank, 2, 64);
+            rank += __shfl_xor(rank, 1, 64);
+            if (live && part == 0) group[n_expert + 1 + n_pairs + rank] = e;
         }
     }
     __syncthreads();
@@ -968,11 +982,12 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(shv_moe_down_args a) {
     *reinterpret_cast<float4 *>(a.out + static_cast<size_t>(t) * a.out_stride + c) = v;
 }
 
-// The per-expert lists of a pass: one block for short passes, kGroupBlocks in two launches from 2048 pairs on
+// The per-expert lists of a pass: one block for short passes of few experts, kGroupBlocks in two launches from 2048
+// pairs or 128 experts on (ranking the experts by length is E^2 comparisons, a block's share of them a sixteenth)
 // (their counts meet in the library's scratch, which nothing else on the stream is using between the two).
 int launch_group(shv_ctx *ctx, const int32_t *topk, int n_tok, int n_used, int n_expert, int32_t *group) {
     const int n_pairs = n_tok * n_used;
-    if (n_pairs < 2048 || !ctx->gemm_part || ctx->moe_group_one_block) {
+    if ((n_pairs < 2048 && n_expert < 128) || !ctx->gemm_part || ctx->moe_group_one_block) {
         SHV_LAUNCH(ctx, moe_group_kernel, dim3(1), dim3(1024), 0, topk, n_tok, n_used, n_expert, group);
         return SHV_OK;
     }

@@ -163,12 +163,12 @@ def test_moe_block_over_banks_in_other_types(ctx, types, T):
         bad.gpu()
 
 
-@pytest.mark.parametrize("T,E,used", [(160, 64, 10), (300, 64, 10), (517, 128, 8), (1030, 512, 2)])
+@pytest.mark.parametrize("T,E,used", [(160, 64, 10), (300, 64, 10), (130, 128, 8), (517, 128, 8), (1030, 512, 2)])
 def test_lists_by_expert_hold_every_pair_once(ctx, T, E, used):
     """The workspace the grouped kernels walk (llm/moe.go:289-409 batches a chunk's tokens per expert): starts that
     add up, under every expert exactly the (token, slot) pairs that chose it, in any order, and the experts' launch
-    order by list length, longer first, equal lengths by index.  Passes below 2048 pairs are listed by one block,
-    longer ones by sixteen in two launches: both roads are here."""
+    order by list length, longer first, equal lengths by index.  Passes below 2048 pairs over fewer than 128 experts
+    are listed by one block, the others by sixteen in two launches: both roads are here."""
     case = MoeCase(ctx, seed=T, E=E, used=used, T=T)
     got = case.gpu(residual=True, grouped=True)
     g, topk = got["group"], got["topk"]
