@@ -366,7 +366,11 @@ typedef struct {
  * time on the matrix cores (the chunked form of the same rule: q^, k^, v, log g and beta of every
  * row are prepared into work first, then each chunk is a few 64-row products and one triangular
  * solve against the state, which is read and written once per pass); results agree with the
- * row-by-row rule to float32 rounding.  The reference scans row by row at every pass length
+ * row-by-row rule to float32 rounding.  With room behind those rows (their count rounded up to a
+ * multiple of 4 floats) for 10 880 more floats per (sequence, chunk of 64 rows, value head), what a
+ * chunk needs that does not depend on the state is formed for every chunk of the pass at once, by a
+ * launch of its own, instead of inside the walk over the chunks by each of a head's eight blocks:
+ * the same values bit for bit, the walk a quarter shorter.  The reference scans row by row at every pass length
  * (shaders/llm_dn_scan.comp; llm/gpu_deltanet.go:48-52 names the chunked form as not built there). */
 typedef struct {
     const float *ring;

@@ -15,6 +15,10 @@
 //
 //   dn_prep_kernel   everything that does not depend on the state, once per pass: causal conv +
 //                    SiLU of q, k, v, the L2 norm of q and k per key head, log g and beta
+//   dn_chunk_kernel  (as producer, when the workspace has room) what a chunk needs that does not
+//                    depend on the state either — A, M, the inverses of the diagonal blocks of I + A,
+//                    G, beta — for every (value head, chunk) of the pass at once: the walk below is a
+//                    chain, this part of it need not be, nor be repeated by a head's eight blocks
 //   dn_chunk_kernel  a block owns 16 of a value head's 128 state rows (they evolve independently
 //                    of the other rows) and walks the chunks of the pass with that slab in
 //                    registers as float32; the solve is blocked 4 x 16: the four 16x16 diagonal
@@ -119,17 +123,25 @@ constexpr int kKS = kD + 8;    // halves between rows of the [64][128] operands 
 constexpr int kAS = kC + 8;    // halves between rows of the [64][64] and [16][64] operands
 constexpr int kTS = 24;        // halves between rows of a 16x16 inverse
 
+// What a chunk's solve and outputs need besides the state, q^ and k^: a function of the chunk's k^, q^, g and beta
+// alone, so it can be formed for all chunks of a pass at once and handed over as one image of these bytes.
+struct PreRec {
+    _Float16 ah[kC][kAS], al[kC][kAS];                            // -A[t][s], s < t
+    _Float16 mh[kC][kAS], ml[kC][kAS];                            // M[t][s] = e^(G_t - G_s) (q_t . k_s), s <= t
+    _Float16 th[4][16][kTS], tl[4][16][kTS];                      // the inverses of the diagonal blocks of I + A
+    float G[kC], beta[kC];
+};
+static_assert(sizeof(PreRec) % 16 == 0, "moved 16 bytes at a time");
+constexpr int kPreVecs = sizeof(PreRec) / 16, kPrePerThread = (kPreVecs + kThreads - 1) / kThreads;
+
 struct ChunkLds {
     _Float16 kh[kC][kKS], kl[kC][kKS], qh[kC][kKS], ql[kC][kKS];  // k^ and q^ of the chunk, hi and scaled lo
     _Float16 sh[kJ][kKS], sl[kJ][kKS];                            // the state slab S[j][i]
-    _Float16 ah[kC][kAS], al[kC][kAS];                            // -A[t][s], s < t
-    _Float16 mh[kC][kAS], ml[kC][kAS];                            // M[t][s] = e^(G_t - G_s) (q_t . k_s), s <= t
+    alignas(16) PreRec pre;
     _Float16 uh[kJ][kAS], ul[kJ][kAS];                            // U transposed, [j][s]
     _Float16 dh[kJ][kAS], dl[kJ][kAS];                            // U e^(G_C - G_s) transposed
-    _Float16 th[4][16][kTS], tl[4][16][kTS];                      // the inverses of the diagonal blocks of I + A
-    float adiag[4][16][16];                                       // those blocks of A in float32
+    float adiag[4][16][16];                                       // the diagonal blocks of A in float32
     float v[kC][kJ];                                              // v of the chunk, the block's 16 columns
-    float glog[kC], G[kC], beta[kC];
 };
 
 __device__ __forceinline__ float4_t mfma32(half8_t x, half8_t y, float4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, c, 0, 0, 0); }
@@ -150,15 +162,21 @@ __device__ __forceinline__ void mma16(half4_t xh, half4_t xl, half4_t yh, half4_
 // grid: (n_head_v * 8, n_seq): blocks that share a key head are neighbours (they read the same q^
 // and k^); 256 threads.  Wave w owns rows 16w..16w+15 of the chunk in every [64][..] product and
 // the state's columns 32w..32w+31.
-__global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args a, const float *prep, int pw) {
+// ROLE 0: the walk, every chunk's operands formed on the way.  ROLE 1: the walk with the chunks' records (PreRec)
+// read from recs.  ROLE 2: the producer of those records, grid (n_head_v, ceil(chunks / per), n_seq): the block forms
+// the records of `per` chunks in a row of its head by the very steps 1 and 2 of the walk (the next chunk's rows on
+// their way meanwhile) and stores them; nothing of the state is touched.
+constexpr int kWalk = 0, kWalkRecs = 1, kMakeRecs = 2;
+template <int ROLE>
+__global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args a, const float *prep, int pw, char *recs, int per) {
     extern __shared__ __align__(16) char smem_raw[];
     ChunkLds &L = *reinterpret_cast<ChunkLds *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
-    const int seq = blockIdx.y;
+    const int seq = ROLE == kMakeRecs ? blockIdx.z : blockIdx.y;
     const int rep = a.n_head_v / a.n_head_k;
     const int hk = blockIdx.x % a.n_head_k, rest = blockIdx.x / a.n_head_k;
-    const int h = hk + a.n_head_k * (rest % rep), slab = rest / rep;
+    const int h = ROLE == kMakeRecs ? static_cast<int>(blockIdx.x) : hk + a.n_head_k * (rest % rep), slab = ROLE == kMakeRecs ? 0 : rest / rep;
     const int slot = a.slot ? a.slot[seq] : seq;
     const int qk = a.n_head_k * kD, vw = a.n_head_v * kD;
     const int planes = a.n_planes > 1 ? a.n_planes : 1;
@@ -169,11 +187,13 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
     const float scale = 1.f / sqrtf(static_cast<float>(kD));
 
     // the slab in float32: tiles of 16 columns i, tile 2w and 2w+1; element [r] is S[j = 4g + r][i = 16 tile + n]
-    float4_t S[2];
+    float4_t S[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if constexpr (ROLE != kMakeRecs) {
 #pragma unroll
-    for (int u = 0; u < 2; u++)
+        for (int u = 0; u < 2; u++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) S[u][r] = state[static_cast<size_t>(4 * g + r) * kD + 16 * (2 * w + u) + n];
+            for (int r = 0; r < 4; r++) S[u][r] = state[static_cast<size_t>(4 * g + r) * kD + 16 * (2 * w + u) + n];
+    }
     auto publish_state = [&]() {
 #pragma unroll
         for (int u = 0; u < 2; u++)
@@ -185,9 +205,14 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 L.sl[4 * g + r][16 * (2 * w + u) + n] = lo;
             }
     };
-    publish_state();
+    if constexpr (ROLE != kMakeRecs) publish_state();
 
     const int n_chunks = (a.seq_len + kC - 1) / kC;
+    const int c_first = ROLE == kMakeRecs ? static_cast<int>(blockIdx.y) * per : 0;
+    const int c_end = ROLE == kMakeRecs ? (c_first + per < n_chunks ? c_first + per : n_chunks) : n_chunks;
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    u32x4_t pr[ROLE == kWalkRecs ? kPrePerThread : 1];
+    auto rec_of = [&](int c) { return recs + (static_cast<size_t>(seq * n_chunks + c) * a.n_head_v + h) * sizeof(PreRec); };
     // a thread's share of a chunk's q^ and k^: float4 f = tid + 256 u of the [64][32] float4s
     float4 kf[8], qf[8], vf;
     float gl = 0.f, bt = 0.f;
@@ -208,16 +233,25 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
             vf = *reinterpret_cast<const float4 *>(rows + static_cast<size_t>(on ? t0 + row : 0) * pw + 2 * qk + h * kD + slab * kJ + c4);
             if (!on) vf = float4{0.f, 0.f, 0.f, 0.f};
         }
-        if (tid < kC) {
+        if (ROLE != kWalkRecs && tid < kC) {
             const bool on = t0 + tid < a.seq_len;
             const float *src = rows + static_cast<size_t>(on ? t0 + tid : 0) * pw + 2 * qk + vw;
             gl = on ? src[h] : 0.f;
             bt = on ? src[a.n_head_v + h] : 0.f;
         }
     };
-    fetch(0);
+    // the record of chunk c, this thread's sixteen-byte pieces of it (the last piece of the last threads repeats the first)
+    const int last_piece = tid + kThreads * (kPrePerThread - 1) < kPreVecs ? kThreads * (kPrePerThread - 1) : -tid;
+#define SHV_DN_FETCH_REC(c_)                                                                  \
+    if constexpr (ROLE == kWalkRecs) {                                                        \
+        const u32x4_t *src_ = reinterpret_cast<const u32x4_t *>(rec_of(c_)) + tid;                \
+        _Pragma("unroll") for (int u = 0; u + 1 < kPrePerThread; u++) pr[u] = src_[kThreads * u]; \
+        pr[kPrePerThread - 1] = src_[last_piece];                                             \
+    }
+    fetch(c_first);
+    SHV_DN_FETCH_REC(c_first)
 
-    for (int c = 0; c < n_chunks; c++) {
+    for (int c = c_first; c < c_end; c++) {
         const int t0 = c * kC;
         // ---- 1: the chunk's operands into LDS ----
 #pragma unroll
@@ -239,7 +273,12 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
             *reinterpret_cast<half4_t *>(&L.ql[row][c4]) = ql4;
         }
         *reinterpret_cast<float4 *>(&L.v[tid >> 2][(tid & 3) * 4]) = vf;
-        if (tid < kC) {
+        if constexpr (ROLE == kWalkRecs) {
+            u32x4_t *dst = reinterpret_cast<u32x4_t *>(&L.pre) + tid;
+#pragma unroll
+            for (int u = 0; u + 1 < kPrePerThread; u++) dst[kThreads * u] = pr[u];
+            if (last_piece > 0) dst[last_piece] = pr[kPrePerThread - 1];
+        } else if (tid < kC) {
             // running sum of log g over the chunk: one wave, a prefix sum by shuffles
             float s = gl;
 #pragma unroll
@@ -247,8 +286,8 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 const float up = __shfl_up(s, o, 64);
                 if (lane >= o) s += up;
             }
-            L.G[tid] = s;
-            L.beta[tid] = bt;
+            L.pre.G[tid] = s;
+            L.pre.beta[tid] = bt;
         }
         __syncthreads();
 
@@ -269,27 +308,34 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 mma32(xkh, xkl, bh, bl, pm, pl);
                 mma32(xqh, xql, bh, bl, rm, rl);
             }
-            const float Gs = L.G[16 * st + n];
+            const float Gs = L.pre.G[16 * st + n];
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int t = 16 * tt + 4 * g + r, s = 16 * st + n;
-                const float Gtr = L.G[t], btr = L.beta[t];
+                const float Gtr = L.pre.G[t], btr = L.pre.beta[t];
                 const float dec = __expf(Gtr - Gs);
                 const float P = fmaf(pl[r], kLoInv, pm[r]), R = fmaf(rl[r], kLoInv, rm[r]);
                 const float av = s < t ? btr * dec * P : 0.f;
                 const float mv = s <= t ? dec * R : 0.f;
                 _Float16 hi, lo;
                 split(-av, hi, lo);
-                L.ah[t][s] = hi; L.al[t][s] = lo;
+                L.pre.ah[t][s] = hi; L.pre.al[t][s] = lo;
                 split(mv, hi, lo);
-                L.mh[t][s] = hi; L.ml[t][s] = lo;
+                L.pre.mh[t][s] = hi; L.pre.ml[t][s] = lo;
                 if (st == tt) L.adiag[tt][4 * g + r][n] = av;
             }
         };
-        tile(w, w);
-        __syncthreads();
-        if (c + 1 < n_chunks) fetch(c + 1);  // in flight under the rest of the chunk (the stores that read these registers have drained)
-        if (w == 0) {
+        if constexpr (ROLE != kWalkRecs) {
+            tile(w, w);
+            __syncthreads();
+        }
+        if (c + 1 < c_end) {
+            fetch(c + 1);  // in flight under the rest of the chunk (the stores that read these registers have drained)
+            SHV_DN_FETCH_REC(c + 1)
+        }
+        if (ROLE == kWalkRecs) {
+            // the record holds it all
+        } else if (w == 0) {
             // lane (b = g, column n): T = (I + A_bb)^-1 by forward substitution, the column in registers
             float T[16];
 #pragma unroll
@@ -303,8 +349,8 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 T[t] = s0 + s1;
                 _Float16 hi, lo;
                 split(T[t], hi, lo);
-                L.th[g][t][n] = hi;
-                L.tl[g][t][n] = lo;
+                L.pre.th[g][t][n] = hi;
+                L.pre.tl[g][t][n] = lo;
             }
         } else if (w == 1) {
             tile(3, 0);
@@ -315,6 +361,15 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
         } else {
             tile(3, 2);
             tile(2, 1);
+        }
+
+        if constexpr (ROLE == kMakeRecs) {
+            __syncthreads();
+            const uint4 *src = reinterpret_cast<const uint4 *>(&L.pre);
+            uint4 *dst = reinterpret_cast<uint4 *>(rec_of(c));
+            for (int i = tid; i < kPreVecs; i += kThreads) dst[i] = src[i];
+            __syncthreads();   // stored before the next chunk's gates and tiles overwrite it
+            continue;
         }
 
         // ---- 3: every wave's rows against the state ----
@@ -329,8 +384,8 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
         float Gt[4], bt4[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            Gt[r] = L.G[16 * w + 4 * g + r];
-            bt4[r] = L.beta[16 * w + 4 * g + r];
+            Gt[r] = L.pre.G[16 * w + 4 * g + r];
+            bt4[r] = L.pre.beta[16 * w + 4 * g + r];
         }
         float4_t acc, accl = {0.f, 0.f, 0.f, 0.f}, w2;
         {
@@ -353,7 +408,7 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
         __syncthreads();
 
         // ---- 4: the solve, block row after block row ----
-        const float GC = L.G[kC - 1];
+        const float GC = L.pre.G[kC - 1];
 #pragma unroll
         for (int cb = 0; cb < 4; cb++) {
             if (w == cb) {
@@ -365,8 +420,8 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                     split(fmaf(accl[r], kLoInv, acc[r]), hi, lo);
                     bh[r] = hi; bl[r] = lo;
                 }
-                const half4_t th = *reinterpret_cast<const half4_t *>(&L.th[cb][n][4 * g]);
-                const half4_t tl = *reinterpret_cast<const half4_t *>(&L.tl[cb][n][4 * g]);
+                const half4_t th = *reinterpret_cast<const half4_t *>(&L.pre.th[cb][n][4 * g]);
+                const half4_t tl = *reinterpret_cast<const half4_t *>(&L.pre.tl[cb][n][4 * g]);
                 float4_t um = {0.f, 0.f, 0.f, 0.f}, ul = um;
                 mma16(th, tl, bh, bl, um, ul);
                 half4_t uh4, ul4, dh4, dl4;
@@ -386,8 +441,8 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
             }
             __syncthreads();
             if (w > cb) {
-                const half4_t xh = *reinterpret_cast<const half4_t *>(&L.ah[16 * w + n][16 * cb + 4 * g]);
-                const half4_t xl = *reinterpret_cast<const half4_t *>(&L.al[16 * w + n][16 * cb + 4 * g]);
+                const half4_t xh = *reinterpret_cast<const half4_t *>(&L.pre.ah[16 * w + n][16 * cb + 4 * g]);
+                const half4_t xl = *reinterpret_cast<const half4_t *>(&L.pre.al[16 * w + n][16 * cb + 4 * g]);
                 const half4_t yh = *reinterpret_cast<const half4_t *>(&L.uh[n][16 * cb + 4 * g]);
                 const half4_t yl = *reinterpret_cast<const half4_t *>(&L.ul[n][16 * cb + 4 * g]);
                 mma16(xh, xl, yh, yl, acc, accl);
@@ -398,8 +453,8 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
         {
             float4_t om = {0.f, 0.f, 0.f, 0.f}, ol = om;
             for (int cb = 0; cb <= w; cb++) {
-                const half4_t xh = *reinterpret_cast<const half4_t *>(&L.mh[16 * w + n][16 * cb + 4 * g]);
-                const half4_t xl = *reinterpret_cast<const half4_t *>(&L.ml[16 * w + n][16 * cb + 4 * g]);
+                const half4_t xh = *reinterpret_cast<const half4_t *>(&L.pre.mh[16 * w + n][16 * cb + 4 * g]);
+                const half4_t xl = *reinterpret_cast<const half4_t *>(&L.pre.ml[16 * w + n][16 * cb + 4 * g]);
                 const half4_t yh = *reinterpret_cast<const half4_t *>(&L.uh[n][16 * cb + 4 * g]);
                 const half4_t yl = *reinterpret_cast<const half4_t *>(&L.ul[n][16 * cb + 4 * g]);
                 mma16(xh, xl, yh, yl, om, ol);
@@ -439,10 +494,12 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
         }
         __syncthreads();
     }
+    if constexpr (ROLE != kMakeRecs) {
 #pragma unroll
-    for (int u = 0; u < 2; u++)
+        for (int u = 0; u < 2; u++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) state[static_cast<size_t>(4 * g + r) * kD + 16 * (2 * w + u) + n] = S[u][r];
+            for (int r = 0; r < 4; r++) state[static_cast<size_t>(4 * g + r) * kD + 16 * (2 * w + u) + n] = S[u][r];
+    }
 }
 
 }  // namespace
@@ -463,9 +520,28 @@ int shv_launch_dn_chunk(shv_ctx *ctx, const shv_dn_step_args &a) {
     SHV_LAUNCH(ctx, dn_prep_kernel, dim3(items, (a.seq_len + kPrepTok - 1) / kPrepTok, a.n_seq), dim3(kThreads), 0, a, a.work, pw);
     static std::atomic<bool> raised{false};
     if (!raised.load(std::memory_order_acquire)) {
-        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&dn_chunk_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(ChunkLds))));
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&dn_chunk_kernel<kWalk>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(ChunkLds))));
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&dn_chunk_kernel<kWalkRecs>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(ChunkLds))));
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&dn_chunk_kernel<kMakeRecs>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(sizeof(ChunkLds))));
         raised.store(true, std::memory_order_release);
     }
-    SHV_LAUNCH(ctx, dn_chunk_kernel, dim3(a.n_head_v * (kD / kJ), a.n_seq), dim3(kThreads), sizeof(ChunkLds), a, static_cast<const float *>(a.work), pw);
+    // Room behind the prepared rows for a record per (sequence, chunk, value head): the chunks' state-independent
+    // part is then formed for all of them at once, and the walk over the chunks only reads it.
+    const long long prep_floats = (static_cast<long long>(a.n_seq) * a.seq_len * pw + 3) & ~3ll;
+    const int n_chunks = (a.seq_len + kC - 1) / kC;
+    const long long rec_floats = static_cast<long long>(a.n_seq) * n_chunks * a.n_head_v * static_cast<long long>(sizeof(PreRec) / 4);
+    const dim3 grid(a.n_head_v * (kD / kJ), a.n_seq);
+    if (n_chunks >= 2 && n_chunks <= 65535 && a.n_seq <= 65535 && prep_floats + rec_floats <= a.work_floats && !ctx->dn_chunk_no_recs) {
+        char *recs = reinterpret_cast<char *>(a.work + prep_floats);
+        // chunks a producer block takes in a row: as many as still leave a block for every compute unit (a block that
+        // takes several has the next one's rows on their way while it works)
+        int per = static_cast<int>(static_cast<long long>(a.n_head_v) * n_chunks * a.n_seq / ctx->prop.multiProcessorCount);
+        per = per < 1 ? 1 : per > 8 ? 8 : per;
+        SHV_LAUNCH(ctx, dn_chunk_kernel<kMakeRecs>, dim3(a.n_head_v, (n_chunks + per - 1) / per, a.n_seq), dim3(kThreads), sizeof(ChunkLds), a,
+                   static_cast<const float *>(a.work), pw, recs, per);
+        SHV_LAUNCH(ctx, dn_chunk_kernel<kWalkRecs>, grid, dim3(kThreads), sizeof(ChunkLds), a, static_cast<const float *>(a.work), pw, recs, 0);
+    } else {
+        SHV_LAUNCH(ctx, dn_chunk_kernel<kWalk>, grid, dim3(kThreads), sizeof(ChunkLds), a, static_cast<const float *>(a.work), pw, static_cast<char *>(nullptr), 0);
+    }
     return SHV_OK;
 }

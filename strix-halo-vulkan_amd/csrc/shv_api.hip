@@ -57,6 +57,7 @@ int shv_init(int device, shv_ctx **out) {
         const int v = std::atoi(e);
         if (v >= 1) ctx->moe_group_min = v;
     }
+    if (const char *e = std::getenv("SHV_DN_RECS")) ctx->dn_chunk_no_recs = std::atoi(e) == 0;
     if (const char *e = std::getenv("SHV_MOE_GROUP_BLOCKS")) ctx->moe_group_one_block = std::atoi(e) == 1;
     if (const char *e = std::getenv("SHV_MOE_TALL_MIN")) {
         const int v = std::atoi(e);

@@ -38,6 +38,7 @@ struct shv_ctx {
     // SHV_ATTN_APPEND=launch: passes of three and four rows write their new cells in a launch of their own, as longer ones do
     bool attn_append_launch = false;
     int moe_group_min = 128;  // rows from which a MoE pass with a workspace is grouped by expert on the matrix cores (SHV_MOE_GROUP_MIN)
+    bool dn_chunk_no_recs = false;  // SHV_DN_RECS=0: the chunked delta rule forms every chunk's state-independent part inside the walk, whatever the workspace holds
     bool moe_group_one_block = false;  // SHV_MOE_GROUP_BLOCKS=1: the per-expert lists of a long pass by one block in one launch
     int moe_tall_min = 16;  // tokens from which the MoE kernels' blocks make several passes over their staged rows (SHV_MOE_TALL_MIN)
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;

@@ -711,7 +711,10 @@ DeltaNetGPU::DeltaNetGPU(Device &dev, const Model &m, int maxTokens, int slots, 
     }
     const size_t T = maxTokens;
     if (maxTokens > 16) {
-        work_floats_ = static_cast<int64_t>(T) * (c_.ConvWidth() + 2 * c_.SSMHeadV);
+        // the prepared rows of a pass, and behind them a record of 43 520 bytes per (chunk of 64 rows, value head):
+        // with that much room the chunks' state-independent part is formed for all of them at once (shv_dn_step)
+        work_floats_ = ((static_cast<int64_t>(T) * (c_.ConvWidth() + 2 * c_.SSMHeadV) + 3) & ~int64_t{3}) +
+                       static_cast<int64_t>((T + 63) / 64 + 1) * c_.SSMHeadV * (43520 / 4);
         work_ = static_cast<float *>(dev.alloc(static_cast<size_t>(work_floats_) * 4));
     }
     in_ = static_cast<float *>(dev.alloc(T * c_.NEmbd * 4));

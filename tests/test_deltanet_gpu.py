@@ -181,7 +181,10 @@ def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
     output and the final state within 1e-3), and against this library's own row-by-row kernel on
     the same inputs, which it must match far closer than that: whole chunks, ragged ones, several
     chunks, a start in mid-sequence (history rows, a state that has already run), several sequences
-    in one call, and passes of 2048 and 4096 rows."""
+    in one call, and passes of 2048 and 4096 rows.  With room in the workspace for a record per chunk
+    and value head, what a chunk needs that does not depend on the state is formed for all chunks at
+    once by a launch of its own: the same arithmetic in another place, so the two chunked roads must
+    agree bit for bit."""
     case = DnCase(ctx, seed=300 + T + n_seq)
     case.upload()
     rng = case.rng
@@ -199,10 +202,12 @@ def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
     c = ctx
     d_x, d_pos = c.upload(xn.reshape(n_seq * T, case.H)), c.upload(pos)
     results = []
-    for chunked in (True, False):
+    prep_floats = (n_seq * T * (case.cw + 2 * case.hv) + 3) & ~3
+    rec_floats = n_seq * ((T + 63) // 64) * case.hv * 10880
+    for chunked in ("records", "in the walk", None):
         d_ring, d_state = c.upload(ring), c.upload(s0)
         d_attn, d_res = c.alloc(n_seq * T * case.vw * 4), c.alloc(n_seq * T * case.H * 4)
-        work = c.alloc(n_seq * T * (case.cw + 2 * case.hv) * 4) if chunked else None
+        work = c.alloc((prep_floats + (rec_floats if chunked == "records" else 0)) * 4) if chunked else None
         ops = case.step_ops(d_x, d_ring, d_state, d_attn, d_res, d_pos, None, n_seq, T, slots, work=work)[:2]
         c.dispatch_multi(ops)
         results.append((d_attn.read(np.float32, n_seq * T * case.vw).reshape(n_seq, T, case.vw),
@@ -211,7 +216,8 @@ def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
             b.free()
         if work is not None:
             work.free()
-    (got_attn, got_state), (seq_attn, seq_state) = results
+    (got_attn, got_state), (walk_attn, walk_state), (seq_attn, seq_state) = results
+    assert np.array_equal(got_attn.view(np.uint32), walk_attn.view(np.uint32)) and np.array_equal(got_state.view(np.uint32), walk_state.view(np.uint32))
     e_a, e_s = O.rel_l2(got_attn, seq_attn), O.rel_l2(got_state, seq_state)
     print(f"deltanet chunked T={T} x{n_seq}: against the row-by-row kernel: rows {e_a:.3e} state {e_s:.3e}")
     assert e_a <= 2e-5 and e_s <= 2e-5
