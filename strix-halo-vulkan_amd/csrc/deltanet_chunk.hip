@@ -57,7 +57,8 @@ __device__ __forceinline__ void split(float x, _Float16 &hi, _Float16 &lo) {
 }
 
 // ------------------------------------------------------------------------------- prep --------
-// One row of the result per pass row: [q^ (hk*d) | k^ (hk*d) | v (hv*d) | log g (hv) | beta (hv)].
+// One row of the result per pass row: [q^ (hk*d) | k^ (hk*d) | v (hv*d) | log g (hv) | beta (hv)]; q^ and k^ as
+// binary16 pairs (value = hi + lo / 2048), every four columns' sixteen bytes holding their four hi, then their four lo.
 // grid: (items, ceil(seq_len / 4), n_seq), 256 threads; an item is four (q or k, key head) vectors
 // (a wave each), or 256 v channels, or the gates; a thread keeps the sliding window of its
 // channel over the block's four rows.
@@ -102,8 +103,18 @@ __global__ __launch_bounds__(kThreads) void dn_prep_kernel(shv_dn_step_args a, f
             if (is_qk) {
                 const float ssq = wave_sum_all(fmaf(a0, a0, a1 * a1));
                 const float nrm = a.qk_norm_max ? 1.f / fmaxf(sqrtf(ssq), a.eps) : 1.f / sqrtf(ssq + a.eps);
-                dst[static_cast<size_t>(r) * pw + ch0] = a0 * nrm;
-                dst[static_cast<size_t>(r) * pw + ch1] = a1 * nrm;
+                // as the two halves the matrix cores take, split here once instead of by every block that stages the
+                // row: four columns' large halves, then their small ones, in the sixteen bytes the four floats had
+                char *seg = reinterpret_cast<char *>(dst + static_cast<size_t>(r) * pw + vec * kD);
+                const float val[2] = {a0 * nrm, a1 * nrm};
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const int cc = lane + 64 * e;
+                    _Float16 hi, lo;
+                    split(val[e], hi, lo);
+                    *reinterpret_cast<_Float16 *>(seg + (cc >> 2) * 16 + (cc & 3) * 2) = hi;
+                    *reinterpret_cast<_Float16 *>(seg + (cc >> 2) * 16 + 8 + (cc & 3) * 2) = lo;
+                }
             } else {
                 dst[static_cast<size_t>(r) * pw + ch0] = a0;
             }
@@ -257,20 +268,13 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const int f = tid + kThreads * u, row = f >> 5, c4 = (f & 31) * 4;
-            const float kv[4] = {kf[u].x, kf[u].y, kf[u].z, kf[u].w}, qv[4] = {qf[u].x, qf[u].y, qf[u].z, qf[u].w};
-            half4_t h4, l4, qh4, ql4;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                _Float16 hi, lo;
-                split(kv[e], hi, lo);
-                h4[e] = hi; l4[e] = lo;
-                split(qv[e], hi, lo);
-                qh4[e] = hi; ql4[e] = lo;
-            }
-            *reinterpret_cast<half4_t *>(&L.kh[row][c4]) = h4;
-            *reinterpret_cast<half4_t *>(&L.kl[row][c4]) = l4;
-            *reinterpret_cast<half4_t *>(&L.qh[row][c4]) = qh4;
-            *reinterpret_cast<half4_t *>(&L.ql[row][c4]) = ql4;
+            // the prepared rows hold q^ and k^ as halves already: four hi, four lo
+            struct Halves { half4_t hi, lo; };
+            const Halves kk = __builtin_bit_cast(Halves, kf[u]), qq = __builtin_bit_cast(Halves, qf[u]);
+            *reinterpret_cast<half4_t *>(&L.kh[row][c4]) = kk.hi;
+            *reinterpret_cast<half4_t *>(&L.kl[row][c4]) = kk.lo;
+            *reinterpret_cast<half4_t *>(&L.qh[row][c4]) = qq.hi;
+            *reinterpret_cast<half4_t *>(&L.ql[row][c4]) = qq.lo;
         }
         *reinterpret_cast<float4 *>(&L.v[tid >> 2][(tid & 3) * 4]) = vf;
         if constexpr (ROLE == kWalkRecs) {
