@@ -1450,17 +1450,28 @@ int shv_launch_router_wide(shv_ctx *ctx, const shv_moe_router_args &a) {
     g.x_stride = a.h_stride;
     const int groups = (a.n_tok + kWideTok - 1) / kWideTok;
     SHV_LAUNCH(ctx, gemm_wide_stage_kernel, dim3(stage_parts(g, groups), kWideTok / 4, groups), dim3(256), 0, g, ctx->gemm_stage, a.xn);
-    constexpr int NW = 4;
     const int n_rows = a.n_expert + (a.shared_gate ? 1 : 0);
-    const int bx = (n_rows + NW * kTileRows - 1) / (NW * kTileRows);
     const size_t lds = 2 * kWideSlab;
     static std::atomic<bool> raised{false};
     if (!raised.load(std::memory_order_acquire)) {
-        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&router_wide_kernel<NW>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&router_wide_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        SHV_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&router_wide_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
         raised.store(true, std::memory_order_release);
     }
-    SHV_LAUNCH(ctx, (router_wide_kernel<NW>), dim3(bx * groups), dim3(NW * 64), lds, a.router, a.shared_gate, n_rows, a.n_embd, a.n_tok,
-               static_cast<const char *>(ctx->gemm_stage), a.logits, a.n_expert + 1, groups);
+    // Every block reads its group's slabs whole: blocks of eight waves (128 router rows) halve that traffic, and from 64 groups
+    // on there are still blocks enough for the chip (4096 rows, 513 router rows: 320 blocks; the 2048-row pass is 1.7 % faster
+    // with four waves a block and 288 of them)
+    if (groups >= 64) {
+        constexpr int NW = 8;
+        const int bx = (n_rows + NW * kTileRows - 1) / (NW * kTileRows);
+        SHV_LAUNCH(ctx, (router_wide_kernel<NW>), dim3(bx * groups), dim3(NW * 64), lds, a.router, a.shared_gate, n_rows, a.n_embd, a.n_tok,
+                   static_cast<const char *>(ctx->gemm_stage), a.logits, a.n_expert + 1, groups);
+    } else {
+        constexpr int NW = 4;
+        const int bx = (n_rows + NW * kTileRows - 1) / (NW * kTileRows);
+        SHV_LAUNCH(ctx, (router_wide_kernel<NW>), dim3(bx * groups), dim3(NW * 64), lds, a.router, a.shared_gate, n_rows, a.n_embd, a.n_tok,
+                   static_cast<const char *>(ctx->gemm_stage), a.logits, a.n_expert + 1, groups);
+    }
     return SHV_OK;
 }
 

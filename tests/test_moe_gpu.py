@@ -380,6 +380,38 @@ def test_long_pass_over_the_full_bank_matches_oracle(ctx, full_bank, T):
     assert O.rel_l2(flt["out"], got["out"]) <= 1e-5
 
 
+@pytest.mark.parametrize("T,E", [(200, 512), (2048, 130), (4100, 130), (4099, 512)])
+def test_router_of_a_long_pass_alone(ctx, T, E):
+    """shv_moe_router over passes long enough for the matrix cores (llm/moe.go:219-243: xn = rmsnorm(h) * gamma, logits
+    = W xn in float32): xn and every logit against a float64 product of the same rows, with four waves a block below
+    4096 rows and eight from there on, row counts that leave a ragged last group of 64 and router rows (E + the shared
+    gate's) that leave a ragged last block."""
+    rng = np.random.default_rng(T + E)
+    H, used = 2048, 4
+    h = rng.standard_normal((T, H)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    W = (rng.standard_normal((E, H)) * 0.05).astype(np.float32)
+    sg = (rng.standard_normal(H) * 0.05).astype(np.float32)
+    c = ctx
+    d = {k: c.upload(v) for k, v in dict(h=h, gamma=gamma, W=W, sg=sg).items()}
+    xn, logits = c.alloc(T * H * 4), c.alloc(T * (E + 1) * 4)
+    topk, weights = c.alloc(T * used * 4), c.alloc(T * (used + 1) * 4)
+    c.enqueue(A.OP_MOE_ROUTER, A.MoeRouterArgs(d["h"].ptr, d["gamma"].ptr, d["W"].ptr, d["sg"].ptr, xn.ptr, logits.ptr, topk.ptr, weights.ptr,
+                                               T, H, E, used, EPS, H, 0))
+    h64 = h.astype(np.float64)
+    want_xn = h64 / np.sqrt((h64 * h64).mean(axis=1, keepdims=True) + EPS) * gamma
+    got_xn = xn.read(np.float32, T * H).reshape(T, H)
+    assert O.rel_l2(got_xn, want_xn) <= 1e-6
+    got = logits.read(np.float32, T * (E + 1)).reshape(T, E + 1)
+    want = want_xn @ np.vstack([W, sg]).astype(np.float64).T
+    err = max(O.rel_l2(got[t], want[t]) for t in range(0, T, 37))
+    assert O.rel_l2(got, want) <= 1e-5 and err <= 1e-5, err
+    # the selection from those logits: each row's ids are its largest logits, in descending order
+    ids = topk.read(np.int32, T * used).reshape(T, used)
+    for t in (0, 63, 64, T // 2, T - 1):
+        assert list(ids[t]) == list(np.argsort(-got[t, :E], kind="stable")[:used])
+
+
 @pytest.mark.parametrize("defer", [False, True])
 def test_route_with_many_equal_probabilities_at_512_experts(ctx, full_bank, defer):
     """More than 64 experts share the largest probability: the candidates do not fit the ranking
