@@ -137,7 +137,7 @@ constexpr int kTS = 24;        // halves between rows of a 16x16 inverse
 // What a chunk's solve and outputs need besides the state, q^ and k^: a function of the chunk's k^, q^, g and beta
 // alone, so it can be formed for all chunks of a pass at once and handed over as one image of these bytes.
 struct PreRec {
-    _Float16 ah[kC][kAS], al[kC][kAS];                            // -A[t][s], s < t
+    _Float16 ah[kC][kAS], al[kC][kAS];                            // -A[t][s], s < t; in a stored record (I + A)^-1 [t][s], s <= t
     _Float16 mh[kC][kAS], ml[kC][kAS];                            // M[t][s] = e^(G_t - G_s) (q_t . k_s), s <= t
     _Float16 th[4][16][kTS], tl[4][16][kTS];                      // the inverses of the diagonal blocks of I + A
     float G[kC], beta[kC];
@@ -151,6 +151,7 @@ struct ChunkLds {
     alignas(16) PreRec pre;
     _Float16 uh[kJ][kAS], ul[kJ][kAS];                            // U transposed, [j][s]
     _Float16 dh[kJ][kAS], dl[kJ][kAS];                            // U e^(G_C - G_s) transposed
+    _Float16 bth[kJ][kAS], btl[kJ][kAS];                          // B transposed, [j][t] (the walk over records)
     float adiag[4][16][16];                                       // the diagonal blocks of A in float32
     float v[kC][kJ];                                              // v of the chunk, the block's 16 columns
 };
@@ -369,6 +370,55 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
 
         if constexpr (ROLE == kMakeRecs) {
             __syncthreads();
+            // The record carries (I + A)^-1 whole, so that the walk's solve is one product, U = (I + A)^-1 B, with one
+            // wait before it instead of one per block row.  Wave w forms block column w of it, block rows w..3, by the
+            // walk's own recurrence on the identity, X_c = T_cc (I_c - sum_{w <= b < c} A_cb X_b): a product's result is
+            // already laid out as the next product's second operand, so the column never leaves the wave's registers.
+            float4_t X[4];
+            half4_t xbh[4], xbl[4];
+#pragma unroll
+            for (int cr = 0; cr < 4; cr++) {
+                X[cr] = float4_t{0.f, 0.f, 0.f, 0.f};
+                if (cr < w) continue;
+                float4_t am = {0.f, 0.f, 0.f, 0.f}, alo = am;
+#pragma unroll
+                for (int b = 0; b < cr; b++) {
+                    if (b < w) continue;
+                    const half4_t xh = *reinterpret_cast<const half4_t *>(&L.pre.ah[16 * cr + n][16 * b + 4 * g]);
+                    const half4_t xl = *reinterpret_cast<const half4_t *>(&L.pre.al[16 * cr + n][16 * b + 4 * g]);
+                    mma16(xh, xl, xbh[b], xbl[b], am, alo);
+                }
+                half4_t bh, bl;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float e = (cr == w && 4 * g + r == n ? 1.f : 0.f) + fmaf(alo[r], kLoInv, am[r]);
+                    _Float16 hi, lo;
+                    split(e, hi, lo);
+                    bh[r] = hi; bl[r] = lo;
+                }
+                const half4_t th = *reinterpret_cast<const half4_t *>(&L.pre.th[cr][n][4 * g]);
+                const half4_t tl = *reinterpret_cast<const half4_t *>(&L.pre.tl[cr][n][4 * g]);
+                float4_t um = {0.f, 0.f, 0.f, 0.f}, ul = um;
+                mma16(th, tl, bh, bl, um, ul);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    X[cr][r] = fmaf(ul[r], kLoInv, um[r]);   // (I + A)^-1 [t = 16 cr + 4g + r][s = 16 w + n]
+                    _Float16 hi, lo;
+                    split(X[cr][r], hi, lo);
+                    xbh[cr][r] = hi; xbl[cr][r] = lo;
+                }
+            }
+            __syncthreads();   // every wave has read the last of -A
+#pragma unroll
+            for (int cr = 0; cr < 4; cr++) {
+                if (cr < w) continue;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    L.pre.ah[16 * cr + 4 * g + r][16 * w + n] = xbh[cr][r];
+                    L.pre.al[16 * cr + 4 * g + r][16 * w + n] = xbl[cr][r];
+                }
+            }
+            __syncthreads();
             const uint4 *src = reinterpret_cast<const uint4 *>(&L.pre);
             uint4 *dst = reinterpret_cast<uint4 *>(rec_of(c));
             for (int i = tid; i < kPreVecs; i += kThreads) dst[i] = src[i];
@@ -409,10 +459,49 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 w2[r] = gam * fmaf(w2l[r], kLoInv, w2m[r]);
             }
         }
+        const float GC = L.pre.G[kC - 1];
+        if constexpr (ROLE == kWalkRecs) {
+            // ---- 4, with (I + A)^-1 in the record: U = (I + A)^-1 B.  Every wave's rows of B as second operands for all,
+            //      one wait, then this wave's rows of U from the block rows up to its own ----
+            {
+                half4_t bh, bl;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    _Float16 hi, lo;
+                    split(acc[r], hi, lo);
+                    bh[r] = hi; bl[r] = lo;
+                }
+                *reinterpret_cast<half4_t *>(&L.bth[n][16 * w + 4 * g]) = bh;
+                *reinterpret_cast<half4_t *>(&L.btl[n][16 * w + 4 * g]) = bl;
+            }
+            __syncthreads();
+            float4_t um = {0.f, 0.f, 0.f, 0.f}, ul = um;
+            for (int cb = 0; cb <= w; cb++) {
+                const half4_t xh = *reinterpret_cast<const half4_t *>(&L.pre.ah[16 * w + n][16 * cb + 4 * g]);
+                const half4_t xl = *reinterpret_cast<const half4_t *>(&L.pre.al[16 * w + n][16 * cb + 4 * g]);
+                const half4_t yh = *reinterpret_cast<const half4_t *>(&L.bth[n][16 * cb + 4 * g]);
+                const half4_t yl = *reinterpret_cast<const half4_t *>(&L.btl[n][16 * cb + 4 * g]);
+                mma16(xh, xl, yh, yl, um, ul);
+            }
+            half4_t uh4, ul4, dh4, dl4;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float u = fmaf(ul[r], kLoInv, um[r]);   // U[s = 16 w + 4g + r][j = n]
+                _Float16 hi, lo;
+                split(u, hi, lo);
+                uh4[r] = hi; ul4[r] = lo;
+                split(u * __expf(GC - Gt[r]), hi, lo);
+                dh4[r] = hi; dl4[r] = lo;
+            }
+            *reinterpret_cast<half4_t *>(&L.uh[n][16 * w + 4 * g]) = uh4;
+            *reinterpret_cast<half4_t *>(&L.ul[n][16 * w + 4 * g]) = ul4;
+            *reinterpret_cast<half4_t *>(&L.dh[n][16 * w + 4 * g]) = dh4;
+            *reinterpret_cast<half4_t *>(&L.dl[n][16 * w + 4 * g]) = dl4;
+            __syncthreads();
+        } else {
         __syncthreads();
 
         // ---- 4: the solve, block row after block row ----
-        const float GC = L.pre.G[kC - 1];
 #pragma unroll
         for (int cb = 0; cb < 4; cb++) {
             if (w == cb) {
@@ -451,6 +540,7 @@ __global__ __launch_bounds__(kThreads, 1) void dn_chunk_kernel(shv_dn_step_args 
                 const half4_t yl = *reinterpret_cast<const half4_t *>(&L.ul[n][16 * cb + 4 * g]);
                 mma16(xh, xl, yh, yl, acc, accl);
             }
+        }
         }
 
         // ---- 5: the rows' outputs ----

@@ -183,8 +183,9 @@ def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
     chunks, a start in mid-sequence (history rows, a state that has already run), several sequences
     in one call, and passes of 2048 and 4096 rows.  With room in the workspace for a record per chunk
     and value head, what a chunk needs that does not depend on the state is formed for all chunks at
-    once by a launch of its own: the same arithmetic in another place, so the two chunked roads must
-    agree bit for bit."""
+    once by a launch of its own, (I + A)^-1 whole among it, so that road's solve is one product
+    where the other walks the block rows: the two chunked roads are held to the same bar against the
+    row-by-row kernel, and to each other."""
     case = DnCase(ctx, seed=300 + T + n_seq)
     case.upload()
     rng = case.rng
@@ -217,7 +218,9 @@ def test_chunked_rows_equal_the_row_by_row_rule(ctx, T, pos0, n_seq):
         if work is not None:
             work.free()
     (got_attn, got_state), (walk_attn, walk_state), (seq_attn, seq_state) = results
-    assert np.array_equal(got_attn.view(np.uint32), walk_attn.view(np.uint32)) and np.array_equal(got_state.view(np.uint32), walk_state.view(np.uint32))
+    e_w = max(O.rel_l2(walk_attn, seq_attn), O.rel_l2(walk_state, seq_state), O.rel_l2(got_attn, walk_attn), O.rel_l2(got_state, walk_state))
+    print(f"deltanet chunked T={T} x{n_seq}: the walk that forms its chunks' operands itself, and the two walks against each other: {e_w:.3e}")
+    assert e_w <= 2e-5
     e_a, e_s = O.rel_l2(got_attn, seq_attn), O.rel_l2(got_state, seq_state)
     print(f"deltanet chunked T={T} x{n_seq}: against the row-by-row kernel: rows {e_a:.3e} state {e_s:.3e}")
     assert e_a <= 2e-5 and e_s <= 2e-5
